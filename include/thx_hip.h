@@ -1,0 +1,164 @@
+/*
+ * thx_hip.h — C ABI of libthx_hip.so: fused Elemwise / CAReduce kernels for one
+ * AMD MI355X (gfx950), compiled at run time with hipRTC.
+ *
+ * The library replaces, for Theano's data-parallel core, what the reference
+ * reaches through pygpu / libgpuarray (citations are relative to the Theano
+ * source tree):
+ *   - GpuElemwise_new / GpuElemwise_call       theano/gpuarray/elemwise.py:240, 376
+ *   - the generated GpuCAReduceCuda kernels and their launch code
+ *                                              theano/gpuarray/elemwise.py:449-2420
+ *   - pygpu_empty / GpuArray_write / GpuArray_read / GpuArray_memset
+ *                                              theano/gpuarray/basic_ops.py:593-633, 708-741
+ * Every function is plain C: pointers, sizes and PODs. All functions return
+ * THX_OK (0) or an error code; thx_last_error() gives the message of the last
+ * failure on the calling thread. One device, one in-order stream, no internal
+ * threads. Device results are deterministic: no atomics are used.
+ */
+#ifndef THX_HIP_H
+#define THX_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define THX_MAX_ND 8
+
+/* Error codes and the Python exception each one maps to (the classes raised by
+ * the reference at theano/gpuarray/elemwise.py:292-315, 376-379, 642-654, 707-713). */
+enum {
+  THX_OK = 0,
+  THX_ERR_HIP = 1,         /* RuntimeError: a HIP / hipRTC runtime call failed        */
+  THX_ERR_SHAPE = 2,       /* ValueError:   input dimension mis-match                  */
+  THX_ERR_TYPE = 3,        /* TypeError:    wrong rank, dtype or unusable strides      */
+  THX_ERR_COMPILE = 4,     /* RuntimeError: hipRTC rejected generated source (log kept)*/
+  THX_ERR_MEMORY = 5,      /* MemoryError:  device allocation failed                   */
+  THX_ERR_UNSUPPORTED = 6, /* NotImplementedError                                     */
+  THX_ERR_ARG = 7          /* ValueError:   malformed argument                         */
+};
+
+/* Element types; values are part of the ABI. */
+enum {
+  THX_BOOL = 0, THX_I8 = 1, THX_U8 = 2, THX_I16 = 3, THX_U16 = 4, THX_I32 = 5,
+  THX_U32 = 6, THX_I64 = 7, THX_U64 = 8, THX_F16 = 9, THX_F32 = 10, THX_F64 = 11,
+  THX_NDTYPES = 12
+};
+
+/* OR-ed into thx_array.dtype of an INPUT: `base + offset_bytes` is HOST memory
+ * holding one element (all extents 1). Its value is copied into the kernel
+ * arguments at call time, so it costs no device memory traffic. The reference
+ * keeps 0-d operands on the host as well (theano/gpuarray/type.py:55-57). */
+#define THX_HOST_SCALAR 0x100
+
+/* A strided view of device memory (counterpart of libgpuarray's GpuArray:
+ * data, offset, nd, dimensions, byte strides, typecode). Strides may be zero
+ * or negative; they must be multiples of the element size. */
+typedef struct thx_array {
+  void* base;
+  int64_t offset_bytes;
+  int32_t nd;
+  int32_t dtype;
+  int64_t shape[THX_MAX_ND];
+  int64_t strides_bytes[THX_MAX_ND];
+} thx_array;
+
+/* ---- device, memory, transfers ------------------------------------------ */
+
+/* Select `device`, create the stream, read device properties. Idempotent. */
+int thx_init(int device);
+/* "gfx950:sramecc+:xnack-"-style architecture string and CU count of the device. */
+int thx_device_info(char* arch, size_t arch_cap, int* compute_units, int64_t* hbm_bytes);
+const char* thx_last_error(void);
+
+/* Pooled device allocation (replaces pygpu_empty). thx_free returns the block
+ * to the pool; thx_pool_trim releases cached blocks to the driver. */
+int thx_alloc(size_t nbytes, void** out);
+int thx_free(void* ptr);
+int thx_pool_trim(void);
+int thx_h2d(void* dst, const void* src, size_t nbytes);      /* GpuArray_write */
+int thx_d2h(void* dst, const void* src, size_t nbytes);      /* GpuArray_read, synchronous */
+int thx_d2d(void* dst, const void* src, size_t nbytes);
+int thx_fill_bytes(void* dst, int value, size_t nbytes);     /* GpuArray_memset, a fill kernel */
+int thx_sync(void);
+
+/* ---- run-time compilation ----------------------------------------------- */
+
+/* Directory of the on-disk code-object cache (default $THX_CACHE_DIR, else
+ * ~/.cache/thx_hip). Pass NULL or "" to disable the disk cache. */
+int thx_set_cache_dir(const char* path);
+/* Counters since thx_init: kernels compiled by hipRTC, loaded from disk, and
+ * served from memory. */
+int thx_cache_stats(int64_t* compiled, int64_t* disk_hits, int64_t* mem_hits);
+
+/* ---- Elemwise ------------------------------------------------------------ */
+
+typedef struct thx_elemwise thx_elemwise;
+
+/* Create an n-ary elementwise operation from generated device source defining
+ * a functor type named `functor_name` (see kernels/thx_elemwise.h for the
+ * functor contract). Operands are the n_in inputs followed by the n_out
+ * outputs; dtypes are THX_* codes in that order. Nothing is compiled yet:
+ * kernels are specialised per access plan at the first call that needs them.
+ * Replaces GpuElemwise_new (theano/gpuarray/elemwise.py:240). */
+int thx_elemwise_new(const char* functor_src, const char* functor_name, int n_in, int n_out,
+                     const int32_t* dtypes, thx_elemwise** out);
+
+#define THX_BROADCAST 1 /* size-1 input dimensions broadcast against larger ones */
+#define THX_DRY_RUN 2   /* validate, plan and compile (into the disk cache) but do not launch;
+                           needs no device: the target is $THX_ARCH, default gfx950 */
+
+/* Run on `ins` (n_in arrays) writing `outs` (n_out arrays, preallocated, every
+ * one of the full result shape; an output may alias an input exactly for
+ * in-place operation). All arrays must have the same rank (<= THX_MAX_ND).
+ * Fails with THX_ERR_SHAPE on a dimension mis-match. Asynchronous.
+ * Replaces GpuElemwise_call(ge, args, GE_BROADCAST) (theano/gpuarray/elemwise.py:376). */
+int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* outs, int flags);
+int thx_elemwise_free(thx_elemwise* e);
+
+/* ---- CAReduce ------------------------------------------------------------ */
+
+typedef struct thx_reduce thx_reduce;
+
+/* Create a (multi-)reduction from generated device source defining a functor
+ * named `functor_name` (contract in kernels/thx_reduce.h): n_in inputs feed a
+ * fused prologue, n_out results of identical shape leave a fused epilogue.
+ * acc_bytes = sizeof of the functor's accumulator struct.
+ * Replaces the kernel generation of GpuCAReduceCuda
+ * (theano/gpuarray/elemwise.py:1756-2420). */
+int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, int n_out,
+                   const int32_t* dtypes, int acc_bytes, thx_reduce** out);
+
+/* Reduce the dimensions d with reduce_mask[d] != 0. `ins` all have rank nd and
+ * broadcast against each other like Elemwise inputs; `outs` are C-contiguous
+ * arrays of the kept dimensions, in order. A zero-length reduce domain yields
+ * the identity (the caller rejects it for max/min, as
+ * theano/tensor/elemwise.py:1489-1506 does). Asynchronous.
+ * Replaces the c_code_reduce_* launch routines (theano/gpuarray/elemwise.py:1095-1723). */
+int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_mask,
+                    const thx_array* outs, int flags);
+int thx_reduce_free(thx_reduce* r);
+
+/* ---- inspection and timing ------------------------------------------------ */
+
+/* Name of the kernel plan used by the last elemwise / reduce call on this
+ * thread (e.g. "ew|nd1|i32|v4|u4|m0,1,1,0"), for tests and profiling. */
+const char* thx_last_plan(void);
+
+/* Per-kernel timing with HIP events on the library's stream. Between
+ * thx_profile_begin and thx_profile_end every launch is bracketed by an event
+ * pair; thx_profile_end synchronises and writes one line per kernel:
+ * "<plan>\t<launches>\t<total_ms>\n". Returns THX_ERR_ARG if `cap` is too small. */
+int thx_profile_begin(void);
+int thx_profile_end(char* buf, size_t cap);
+
+/* Whole-region timing: events recorded on the library's stream. */
+int thx_timer_start(void);
+int thx_timer_stop(float* elapsed_ms); /* synchronises */
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* THX_HIP_H */

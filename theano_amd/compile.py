@@ -1,0 +1,241 @@
+"""``function``: compile a graph into a callable that runs on the GPU.
+
+The counterpart of ``theano.function`` (``theano/compile/function.py:74``,
+``FunctionMaker`` ``theano/compile/function_module.py:1428``) reduced to this
+path: clone the graph, run the HIP rewrite pipeline (lift, fuse), order the
+nodes, and execute them one ``perform`` call each, releasing intermediate
+results after their last use (the loop of ``theano/gof/vm.py:237-305``).
+"""
+import numpy as np
+
+from . import gof
+from .gof import Constant, FunctionGraph, Variable
+from .tensor.type import TensorType, as_tensor_variable
+
+
+class In(object):
+    def __init__(self, variable, name=None, borrow=False, allow_downcast=None):
+        self.variable = variable
+        self.name = name or variable.name
+        self.borrow = borrow
+        self.allow_downcast = allow_downcast
+
+
+class Out(object):
+    """``device=True`` leaves the result in GPU memory (a ``HipArray``)."""
+
+    def __init__(self, variable, borrow=False, device=False):
+        self.variable = variable
+        self.borrow = borrow
+        self.device = device
+
+
+class SharedVariable(Variable):
+    """A variable with persistent device storage, an implicit input of every
+    function that uses it (``theano/compile/sharedvalue.py``)."""
+
+    def __init__(self, type, value, name=None):
+        Variable.__init__(self, type, None, None, name)
+        self.container = [value]
+
+    def get_value(self, borrow=False, return_internal_type=False):
+        v = self.container[0]
+        return v if return_internal_type else v.to_numpy()
+
+    def set_value(self, value, borrow=False):
+        self.container[0] = self.type.filter(value)
+
+    def clone(self):
+        return self  # shared variables are never copied into a function graph
+
+
+def shared(value, name=None, broadcastable=None):
+    """Device-resident shared variable holding ``value``."""
+    from .hip.ops import HipArrayType, HipArrayVariable
+    from .hip.runtime import HipArray
+    if isinstance(value, HipArray):
+        dtype, shape = str(value.dtype), value.shape
+    else:
+        value = np.asarray(value)
+        dtype, shape = str(value.dtype), value.shape
+    if broadcastable is None:
+        broadcastable = (False,) * len(shape)
+    t = HipArrayType(dtype, broadcastable)
+
+    class _Shared(SharedVariable, HipArrayVariable):
+        pass
+    return _Shared(t, t.filter(value), name=name)
+
+
+class Function(object):
+    """Callable produced by ``function``."""
+
+    def __init__(self, fgraph, in_specs, out_specs, single_output, shared_inputs):
+        self.fgraph = fgraph
+        self.maker = self  # so that f.maker.fgraph reads as with the reference
+        self.in_specs = in_specs
+        self.out_specs = out_specs
+        self.single_output = single_output
+        self.shared_inputs = shared_inputs
+        self.nodes = fgraph.toposort()
+        self._prepare()
+
+    def _prepare(self):
+        from .hip.opt import DeviceConstant
+        from .hip.runtime import HipArray
+        # storage cells
+        self.storage = {}
+        for v in self.fgraph.inputs:
+            self.storage[v] = [None]
+        self.constants = []
+        for node in self.nodes:
+            for i in node.inputs:
+                if i not in self.storage:
+                    if isinstance(i, DeviceConstant):
+                        self.storage[i] = [None]
+                        self.constants.append(i)
+                    elif isinstance(i, Constant):
+                        self.storage[i] = [np.asarray(i.data)]
+                    elif isinstance(i, SharedVariable):
+                        self.storage[i] = i.container
+                    else:
+                        raise gof.InconsistencyError("%s is used but never computed" % i)
+            for o in node.outputs:
+                self.storage[o] = [None]
+        for o in self.fgraph.outputs:
+            if o not in self.storage:
+                if isinstance(o, Constant):
+                    self.storage[o] = [np.asarray(o.data)]
+                elif isinstance(o, SharedVariable):
+                    self.storage[o] = o.container
+        # last use of every computed variable, for early release
+        keep = set(id(o) for o in self.fgraph.outputs)
+        last = {}
+        for k, node in enumerate(self.nodes):
+            for i in node.inputs:
+                last[id(i)] = k
+        self.release = [[] for _ in self.nodes]
+        computed = set()
+        for node in self.nodes:
+            for o in node.outputs:
+                computed.add(id(o))
+        by_id = dict((id(v), v) for v in self.storage)
+        for vid, k in last.items():
+            if vid in computed and vid not in keep:
+                self.release[k].append(self.storage[by_id[vid]])
+        for k, node in enumerate(self.nodes):
+            for o in node.outputs:
+                if id(o) not in last and id(o) not in keep:
+                    self.release[k].append(self.storage[o])
+        self.thunks = []
+        for node in self.nodes:
+            node.op.prepare_node(node)
+            self.thunks.append((node.op.perform, node, [self.storage[i] for i in node.inputs],
+                                [self.storage[o] for o in node.outputs]))
+        self._constants_ready = False
+        self._HipArray = HipArray
+
+    def _upload_constants(self):
+        for c in self.constants:
+            self.storage[c][0] = self._HipArray.from_numpy(np.asarray(c.data))
+        self._constants_ready = True
+
+    def __call__(self, *args):
+        if len(args) != len(self.in_specs):
+            raise TypeError("function takes %d arguments, got %d" % (len(self.in_specs), len(args)))
+        if not self._constants_ready:
+            self._upload_constants()
+        HipArray = self._HipArray
+        for spec, var, a in zip(self.in_specs, self.fgraph.inputs, args):
+            if isinstance(a, HipArray) and isinstance(var.type, TensorType):
+                # device-resident argument for a host-typed input: checked like a host value
+                if str(a.dtype) != var.type.dtype or a.ndim != var.type.ndim:
+                    raise TypeError("Bad input argument %s: expected %s, got %s" % (spec.name, var.type, a))
+                for d, b in enumerate(var.type.broadcastable):
+                    if b and a.shape[d] != 1:
+                        raise TypeError("Non-unit value on shape on a broadcastable dimension.", a.shape,
+                                        var.type.broadcastable)
+                self.storage[var][0] = a
+            else:
+                try:
+                    self.storage[var][0] = var.type.filter(a, strict=False, allow_downcast=spec.allow_downcast)
+                except TypeError as e:
+                    raise TypeError("Bad input argument to theano function with name \"%s\": %s" % (spec.name, e))
+        for k, (perform, node, ins, outs) in enumerate(self.thunks):
+            perform(node, [c[0] for c in ins], outs)
+            for cell in self.release[k]:
+                cell[0] = None
+        results = [self.storage[o][0] for o in self.fgraph.outputs]
+        for v in self.fgraph.inputs:
+            self.storage[v][0] = None
+        for o in self.fgraph.outputs:
+            if o.owner is not None:
+                self.storage[o][0] = None
+        if self.single_output:
+            return results[0]
+        return results
+
+    def toposort(self):
+        return list(self.nodes)
+
+
+def function(inputs, outputs, fuse=True, name=None, on_unused_input="raise"):
+    """Compile ``outputs`` as a function of ``inputs``.
+
+    ``inputs``: variables or ``In`` instances.  A host-typed input may be given
+    a ``HipArray`` at call time, which skips the upload.  ``outputs``: a
+    variable, ``Out`` or a list of those; ``Out(v, device=True)`` leaves the
+    result on the GPU.  Every op must have a HIP implementation."""
+    from .hip import opt as hip_opt
+    from .hip.ops import HipArrayType, as_hip_variable
+
+    in_specs = [i if isinstance(i, In) else In(i) for i in inputs]
+    single = not isinstance(outputs, (list, tuple))
+    out_list = [outputs] if single else list(outputs)
+    out_specs = [o if isinstance(o, Out) else Out(o) for o in out_list]
+    out_vars = []
+    for spec in out_specs:
+        v = spec.variable
+        if not isinstance(v, Variable):
+            v = as_tensor_variable(v)
+        if spec.device and isinstance(v.type, TensorType):
+            v = as_hip_variable(v)
+        out_vars.append(v)
+    in_vars = [s.variable for s in in_specs]
+    shared_inputs = [v for v in gof.graph_inputs(out_vars) if isinstance(v, SharedVariable)]
+    used = set(id(v) for v in gof.graph_inputs(out_vars))
+    if on_unused_input == "raise":
+        for v in in_vars:
+            if id(v) not in used:
+                raise ValueError("theano function was asked to create a function computing outputs given certain "
+                                 "inputs, but the provided input variable %s is not part of the computational graph "
+                                 "needed to compute the outputs." % v)
+    # clone everything except shared variables
+    memo = dict((s, s) for s in shared_inputs)
+    memo = gof.clone_get_equiv(in_vars, out_vars, copy_inputs=True, memo=memo)
+    c_in = [memo[v] for v in in_vars]
+    c_out = [memo[v] for v in out_vars]
+    fgraph = _SharedAwareGraph(c_in, c_out, shared_inputs)
+    fgraph = hip_opt.optimize(fgraph, fuse=fuse)
+    return Function(fgraph, in_specs, out_specs, single, shared_inputs)
+
+
+class _SharedAwareGraph(FunctionGraph):
+    """FunctionGraph that accepts shared variables as undeclared inputs."""
+
+    def __init__(self, inputs, outputs, shared_inputs):
+        self._shared = set(id(s) for s in shared_inputs)
+        FunctionGraph.__init__(self, inputs, outputs, clone_graph=False)
+
+    def rebuild(self, outputs):
+        g = _SharedAwareGraph.__new__(_SharedAwareGraph)
+        g._shared = self._shared
+        FunctionGraph.__init__(g, self.inputs, outputs, clone_graph=False)
+        return g
+
+    def _import_var(self, var):
+        if var.owner is None and id(var) in self._shared:
+            self.variables.add(var)
+            self.clients.setdefault(var, [])
+            return
+        FunctionGraph._import_var(self, var)

@@ -1,0 +1,32 @@
+"""Process-wide settings, the counterpart of the few ``theano.config`` flags the
+Elemwise / CAReduce path reads (``theano/configdefaults.py:40-87``).
+
+``floatX`` defaults to float32 here (the reference defaults to float64): Python
+float literals take this dtype, so float32 graphs stay float32.
+"""
+import contextlib
+import os
+
+
+class _Config(object):
+    floatX = os.environ.get("THEANO_AMD_FLOATX", "float32")
+    cast_policy = "custom"          # theano/configdefaults.py:65-76
+    int_division = "int"            # x / y on two integer tensors; 'int', 'floatX' or 'raise'
+    device = int(os.environ.get("THEANO_AMD_DEVICE", "0"))
+    # Largest number of inputs a fused Elemwise may take: the kernel argument
+    # block is 4096 bytes (same budget as theano/gpuarray/elemwise.py:44-83).
+    max_fused_inputs = 32
+
+    @contextlib.contextmanager
+    def change_flags(self, **kw):
+        old = {k: getattr(self, k) for k in kw}
+        try:
+            for k, v in kw.items():
+                setattr(self, k, v)
+            yield self
+        finally:
+            for k, v in old.items():
+                setattr(self, k, v)
+
+
+config = _Config()

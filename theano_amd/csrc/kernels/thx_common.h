@@ -1,0 +1,101 @@
+// Device-side helpers shared by every run-time compiled kernel (gfx950, wave64).
+// This text is compiled by hipRTC together with a generated functor and one
+// `extern "C"` entry point per launch plan; nothing here is host code.
+#pragma once
+
+typedef unsigned char thx_bool;  // numpy bool storage: one byte holding 0 or 1
+typedef signed char thx_i8;
+typedef unsigned char thx_u8;
+typedef short thx_i16;
+typedef unsigned short thx_u16;
+typedef int thx_i32;
+typedef unsigned int thx_u32;
+typedef long long thx_i64;
+typedef unsigned long long thx_u64;
+typedef _Float16 thx_f16;
+typedef float thx_f32;
+typedef double thx_f64;
+
+#define THX_DEV __device__ __forceinline__
+#define THX_WAVE 64
+
+namespace thx {
+
+// How one operand is addressed along the vectorised (innermost) dimension.
+enum { M_VEC = 0,      // unit stride: one wide load/store per thread
+       M_BCAST = 1,    // zero stride: one element shared by the whole vector
+       M_GATHER = 2,   // any other stride: one access per element
+       M_IMM = 3 };    // a single host value passed in the kernel arguments
+
+template <int B> struct AlignFor { enum { value = B >= 16 ? 16 : B }; };
+
+// N consecutive elements, aligned so that a 16-byte pack is one dwordx4 access.
+template <class T, int N>
+struct __attribute__((aligned(AlignFor<sizeof(T) * N>::value))) Vec {
+  T v[N];
+};
+
+// Division by a run-time constant d >= 2 for dividends below 2^31:
+// q = mulhi(n, m) >> s with m = ceil(2^(31+L)/d), s = L-1, L = ceil(log2 d).
+struct FastDiv {
+  unsigned m, s, d, pad;
+};
+
+THX_DEV void divmod(unsigned n, const FastDiv& f, unsigned& q, unsigned& r) {
+  q = __umulhi(n, f.m) >> f.s;
+  r = n - q * f.d;
+}
+THX_DEV void divmod(unsigned long long n, const FastDiv& f, unsigned long long& q,
+                    unsigned long long& r) {
+  q = n / f.d;
+  r = n - q * f.d;
+}
+
+template <class IT> struct UnsignedOf;
+template <> struct UnsignedOf<int> { typedef unsigned type; };
+template <> struct UnsignedOf<long long> { typedef unsigned long long type; };
+
+// ---- shuffles of every accumulator field type -----------------------------
+THX_DEV int shfl_xor_t(int v, int m) { return __shfl_xor(v, m, THX_WAVE); }
+THX_DEV unsigned shfl_xor_t(unsigned v, int m) { return (unsigned)__shfl_xor((int)v, m, THX_WAVE); }
+THX_DEV float shfl_xor_t(float v, int m) { return __shfl_xor(v, m, THX_WAVE); }
+THX_DEV double shfl_xor_t(double v, int m) { return __shfl_xor(v, m, THX_WAVE); }
+THX_DEV long long shfl_xor_t(long long v, int m) { return __shfl_xor(v, m, THX_WAVE); }
+THX_DEV unsigned long long shfl_xor_t(unsigned long long v, int m) {
+  return (unsigned long long)__shfl_xor((long long)v, m, THX_WAVE);
+}
+THX_DEV unsigned char shfl_xor_t(unsigned char v, int m) { return (unsigned char)__shfl_xor((int)v, m, THX_WAVE); }
+THX_DEV signed char shfl_xor_t(signed char v, int m) { return (signed char)__shfl_xor((int)v, m, THX_WAVE); }
+THX_DEV short shfl_xor_t(short v, int m) { return (short)__shfl_xor((int)v, m, THX_WAVE); }
+THX_DEV unsigned short shfl_xor_t(unsigned short v, int m) { return (unsigned short)__shfl_xor((int)v, m, THX_WAVE); }
+THX_DEV _Float16 shfl_xor_t(_Float16 v, int m) { return (_Float16)__shfl_xor((float)v, m, THX_WAVE); }
+
+// Butterfly over W lanes (W a power of two, <= 64): every lane ends with the
+// combination of its W-lane group.
+template <class R, int W>
+THX_DEV typename R::Acc group_reduce(typename R::Acc a) {
+#pragma unroll
+  for (int m = W / 2; m >= 1; m >>= 1) {
+    typename R::Acc b = R::shfl_xor(a, m);
+    R::comb(a, b);
+  }
+  return a;
+}
+
+// Whole-block combine through LDS; `lds` holds NW accumulators. Result valid in
+// every thread. Must be reached by all threads of the block.
+template <class R, int NW>
+THX_DEV typename R::Acc block_reduce(typename R::Acc a, typename R::Acc* lds) {
+  a = group_reduce<R, THX_WAVE>(a);
+  if (NW == 1) return a;
+  const int lane = threadIdx.x & (THX_WAVE - 1), wave = threadIdx.x / THX_WAVE;
+  __syncthreads();
+  if (lane == 0) lds[wave] = a;
+  __syncthreads();
+  typename R::Acc r = lds[0];
+#pragma unroll
+  for (int w = 1; w < NW; ++w) R::comb(r, lds[w]);
+  return r;
+}
+
+}  // namespace thx

@@ -1,0 +1,140 @@
+// N-ary strided/broadcast elementwise kernels.
+//
+// A generated functor F supplies
+//   enum { NIN, NOUT, NOPS = NIN + NOUT };
+//   template <int V> struct Regs;                       // one Vec per operand
+//   template <int V, class A> static void load(const A&, Regs<V>&);
+//   template <int V> static void compute(Regs<V>&);     // the scalar graph, V times
+//   template <int V, class A> static void store(const A&, const Regs<V>&);
+// and a generated plan P supplies
+//   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK };
+//   static constexpr int mode(int operand);             // M_VEC / M_BCAST / M_GATHER
+// The host collapses dimensions, so ND is the rank after merging every pair of
+// neighbouring dimensions that all operands walk with compatible strides.
+#pragma once
+
+namespace thx {
+
+template <int NOPS, int ND, class IT>
+struct EwParams {
+  char* ptr[NOPS];       // operand base addresses (inputs, then outputs)
+  unsigned long long imm[NOPS];  // value bytes of M_IMM operands
+  long long nvec;        // whole vectors to process
+  long long n;           // elements in total
+  FastDiv fd[ND];        // extent of each dimension; the last one counts vectors
+  IT stride[NOPS][ND];   // element strides, 0 where an operand broadcasts
+};
+
+template <class P, int NOPS>
+struct EwAcc {
+  typedef typename P::IT IT;
+  char* const* ptr;
+  const unsigned long long* imm;
+  const IT (*stride)[P::ND];
+  IT off[NOPS];
+
+  template <int I, class T, int N>
+  THX_DEV void ld(Vec<T, N>& r) const {
+    if (P::mode(I) == M_IMM) {
+      const T s = *(const T*)&imm[I];
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = s;
+      return;
+    }
+    const T* b = (const T*)ptr[I] + off[I];
+    if (N == 1) {
+      r.v[0] = *b;
+    } else if (P::mode(I) == M_VEC) {
+      r = *(const Vec<T, N>*)b;
+    } else if (P::mode(I) == M_BCAST) {
+      const T s = *b;
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = s;
+    } else {
+      const IT st = stride[I][P::ND - 1];
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = b[k * st];
+    }
+  }
+
+  template <int I, class T, int N>
+  THX_DEV void st(const Vec<T, N>& r) const {
+    T* b = (T*)ptr[I] + off[I];
+    if (N == 1) {
+      *b = r.v[0];
+    } else if (P::mode(I) == M_VEC) {
+      *(Vec<T, N>*)b = r;
+    } else {
+      const IT st = stride[I][P::ND - 1];
+#pragma unroll
+      for (int k = 0; k < N; ++k) b[k * st] = r.v[k];
+    }
+  }
+};
+
+// One thread handles UNR vectors, BLOCK apart, so a wave's accesses stay
+// contiguous; all loads are issued before any arithmetic or store.
+template <class F, class P>
+__device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename P::IT>& p) {
+  typedef typename P::IT IT;
+  typedef typename UnsignedOf<IT>::type UT;
+  constexpr int VEC = P::VEC, UNR = P::UNR, ND = P::ND, NOPS = F::NOPS;
+
+  typename F::template Regs<VEC> r[UNR];
+  EwAcc<P, NOPS> a[UNR];
+  bool full[UNR];
+  const long long q0 = (long long)blockIdx.x * (P::BLOCK * UNR) + threadIdx.x;
+
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) {
+    const long long q = q0 + (long long)u * P::BLOCK;
+    full[u] = q < p.nvec;
+    a[u].ptr = p.ptr;
+    a[u].imm = p.imm;
+    a[u].stride = p.stride;
+    if (ND == 1) {
+#pragma unroll
+      for (int i = 0; i < NOPS; ++i) a[u].off[i] = (IT)(q * VEC) * p.stride[i][0];
+    } else {
+      UT rem = (UT)(full[u] ? q : 0), c;
+      divmod(rem, p.fd[ND - 1], rem, c);
+#pragma unroll
+      for (int i = 0; i < NOPS; ++i) a[u].off[i] = (IT)(c * VEC) * p.stride[i][ND - 1];
+#pragma unroll
+      for (int d = ND - 2; d >= 1; --d) {
+        divmod(rem, p.fd[d], rem, c);
+#pragma unroll
+        for (int i = 0; i < NOPS; ++i) a[u].off[i] += (IT)c * p.stride[i][d];
+      }
+#pragma unroll
+      for (int i = 0; i < NOPS; ++i) a[u].off[i] += (IT)rem * p.stride[i][0];
+    }
+    if (full[u]) F::template load<VEC>(a[u], r[u]);
+  }
+#pragma unroll
+  for (int u = 0; u < UNR; ++u)
+    if (full[u]) F::template compute<VEC>(r[u]);
+#pragma unroll
+  for (int u = 0; u < UNR; ++u)
+    if (full[u]) F::template store<VEC>(a[u], r[u]);
+
+  // ND == 1 only: the elements after the last whole vector, one per thread.
+  if (ND == 1 && VEC > 1) {
+    const long long tail0 = (p.n / VEC) * VEC;
+    const long long e = tail0 + threadIdx.x;
+    if (blockIdx.x == 0 && e < p.n) {
+      typename F::template Regs<1> r1;
+      EwAcc<P, NOPS> a1;
+      a1.ptr = p.ptr;
+      a1.imm = p.imm;
+      a1.stride = p.stride;
+#pragma unroll
+      for (int i = 0; i < NOPS; ++i) a1.off[i] = (IT)e * p.stride[i][0];
+      F::template load<1>(a1, r1);
+      F::template compute<1>(r1);
+      F::template store<1>(a1, r1);
+    }
+  }
+}
+
+}  // namespace thx

@@ -1,0 +1,397 @@
+// Commutative-associative reductions with a fused per-element prologue and a
+// fused per-result epilogue.
+//
+// A generated functor R supplies
+//   enum { NIN, NOUT };
+//   struct Acc;                                          // one field per reduction
+//   template <int V> struct Regs;                        // one Vec per input
+//   static void init(Acc&);                              // identities
+//   template <int V, class A> static void load(const A&, Regs<V>&);
+//   template <int V> static void accum(Acc&, const Regs<V>&);        // fold V elements into one Acc
+//   template <int V> static void accum_lanes(Acc*, const Regs<V>&);  // element k into acc[k]
+//   static void comb(Acc&, const Acc&);                  // merge two partial results
+//   static Acc shfl_xor(const Acc&, int mask);
+//   template <class O> static void post(const O&, long long index, const Acc&);  // epilogue, casts, stores
+// Results never depend on atomics: long reductions are split into S slices
+// whose partial Acc values go to a scratch array laid out [slice][output] and
+// are merged by red_final in a fixed order.
+#pragma once
+
+namespace thx {
+
+template <int NOUT>
+struct RedOut {
+  char* ptr[NOUT];
+};
+
+// ---------------------------------------------------------------------------
+// "Row" form: every output owns a reduce domain of RA x RC elements, RC being
+// the vectorised dimension. TPR threads cooperate on one output; a block holds
+// BLOCK / TPR outputs. Covers trailing-axis reductions, whole-array reductions
+// (one output, many slices) and outer x kept x inner patterns (RA > 1).
+template <int NIN, int NOUT, int NK, class IT>
+struct RowParams {
+  char* in[NIN];
+  unsigned long long imm[NIN];
+  RedOut<NOUT> out;
+  char* partial;          // Acc[S][n_out] when S > 1
+  long long n_out;
+  long long nvec;         // vectors in one output's reduce domain (RA * RC / VEC)
+  long long chunk;        // vectors per slice
+  int S;                  // slices per output
+  int pad;
+  FastDiv kfd[NK];        // extents of the kept dimensions (slot 0 unused)
+  FastDiv rcv;            // RC / VEC, used when RA > 1
+  IT kstride[NIN][NK];    // input strides along the kept dimensions
+  IT ra_stride[NIN];
+  IT rc_stride[NIN];
+};
+
+template <class P, int NIN>
+struct RedAcc {
+  typedef typename P::IT IT;
+  char* const* ptr;
+  const unsigned long long* imm;
+  const IT* vstride;  // stride along the vectorised dimension, per input
+  IT off[NIN];
+
+  template <int I, class T, int N>
+  THX_DEV void ld(Vec<T, N>& r) const {
+    if (P::mode(I) == M_IMM) {
+      const T s = *(const T*)&imm[I];
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = s;
+      return;
+    }
+    const T* b = (const T*)ptr[I] + off[I];
+    if (N == 1) {
+      r.v[0] = *b;
+    } else if (P::mode(I) == M_VEC) {
+      r = *(const Vec<T, N>*)b;
+    } else if (P::mode(I) == M_BCAST) {
+      const T s = *b;
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = s;
+    } else {
+      const IT st = vstride[I];
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = b[k * st];
+    }
+  }
+};
+
+// Plan members: typedef IT; enum { NK, VEC, UNR, BLOCK, TPR, RA2 (1 when RA > 1) };
+// static constexpr int mode(int input).
+template <class R, class P>
+__device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, P::NK, typename P::IT>& p) {
+  typedef typename P::IT IT;
+  typedef typename UnsignedOf<IT>::type UT;
+  typedef typename R::Acc Acc;
+  constexpr int VEC = P::VEC, UNR = P::UNR, NIN = R::NIN, NK = P::NK, TPR = P::TPR;
+  constexpr int RPB = P::BLOCK / TPR;
+  __shared__ Acc lds[P::BLOCK / THX_WAVE];
+
+  const long long bid = blockIdx.x;
+  const long long ob = bid / p.S;
+  const int s = (int)(bid - ob * p.S);
+  const long long o = ob * RPB + threadIdx.x / TPR;
+  const int t = threadIdx.x % TPR;
+  const bool live = o < p.n_out;
+
+  IT base[NIN];
+  {
+    UT rem = (UT)(live ? o : 0), c;
+#pragma unroll
+    for (int i = 0; i < NIN; ++i) base[i] = 0;
+#pragma unroll
+    for (int d = NK - 1; d >= 1; --d) {
+      divmod(rem, p.kfd[d], rem, c);
+#pragma unroll
+      for (int i = 0; i < NIN; ++i) base[i] += (IT)c * p.kstride[i][d];
+    }
+#pragma unroll
+    for (int i = 0; i < NIN; ++i) base[i] += (IT)rem * p.kstride[i][0];
+  }
+
+  Acc acc[UNR];
+#pragma unroll
+  for (int u = 0; u < UNR; ++u) R::init(acc[u]);
+
+  if (live) {
+    const long long j0 = (long long)s * p.chunk;
+    long long j1 = j0 + p.chunk;
+    if (j1 > p.nvec) j1 = p.nvec;
+    for (long long j = j0 + t; j < j1; j += (long long)TPR * UNR) {
+      typename R::template Regs<VEC> r[UNR];
+      bool ok[UNR];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        const long long q = j + (long long)u * TPR;
+        ok[u] = q < j1;
+        RedAcc<P, NIN> a;
+        a.ptr = p.in;
+      a.imm = p.imm;
+        a.imm = p.imm;
+        a.vstride = p.rc_stride;
+        if (P::RA2) {
+          UT ra, cv;
+          divmod((UT)(ok[u] ? q : j0), p.rcv, ra, cv);
+#pragma unroll
+          for (int i = 0; i < NIN; ++i)
+            a.off[i] = base[i] + (IT)ra * p.ra_stride[i] + (IT)(cv * VEC) * p.rc_stride[i];
+        } else {
+#pragma unroll
+          for (int i = 0; i < NIN; ++i) a.off[i] = base[i] + (IT)(q * VEC) * p.rc_stride[i];
+        }
+        if (ok[u]) R::template load<VEC>(a, r[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < UNR; ++u)
+        if (ok[u]) R::template accum<VEC>(acc[u], r[u]);
+    }
+  }
+#pragma unroll
+  for (int u = 1; u < UNR; ++u) R::comb(acc[0], acc[u]);
+
+  Acc tot;
+  if (TPR > THX_WAVE) {
+    tot = block_reduce<R, P::BLOCK / THX_WAVE>(acc[0], lds);
+  } else {
+    tot = group_reduce<R, TPR>(acc[0]);
+  }
+  if (live && t == 0) {
+    if (p.S == 1) {
+      R::post(p.out, o, tot);
+    } else {
+      ((Acc*)p.partial)[(long long)s * p.n_out + o] = tot;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// "Column" form: outer kept dims x one or two reduced dims (R rows in all) x
+// one kept inner dim (C columns, vectorised). A block is TX x TY threads: TX threads side by
+// side along the columns (VEC columns each, so a wave reads whole row segments)
+// and TY row lanes; per-column partials live in registers and the TY lanes are
+// merged through LDS at the end. Rows are split into S slices.
+template <int NIN, int NOUT, int NK, class IT>
+struct ColParams {
+  char* in[NIN];
+  unsigned long long imm[NIN];
+  RedOut<NOUT> out;
+  char* partial;          // Acc[S][n_out] when S > 1
+  long long n_out;        // A * C
+  long long rows;         // R
+  long long rows_per_slice;
+  int cols;               // C
+  int cblocks;            // blocks along the columns
+  int S;
+  int pad;
+  FastDiv kfd[NK];        // extents of the outer kept dimensions (slot 0 unused)
+  FastDiv r1;             // extent of the inner reduced dimension, used when RR2
+  IT kstride[NIN][NK];
+  IT r0_stride[NIN];      // outer reduced dimension (RR2 only)
+  IT r1_stride[NIN];      // inner (or only) reduced dimension
+  IT c_stride[NIN];
+};
+
+// Plan members: typedef IT; enum { NK, VEC, UNR, BLOCK, TX, RR2 (1 when two
+// reduced dimensions remain after collapsing) }; mode(int).
+template <class R, class P>
+__device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, P::NK, typename P::IT>& p) {
+  typedef typename P::IT IT;
+  typedef typename UnsignedOf<IT>::type UT;
+  typedef typename R::Acc Acc;
+  constexpr int VEC = P::VEC, UNR = P::UNR, NIN = R::NIN, NK = P::NK, TX = P::TX;
+  constexpr int TY = P::BLOCK / TX;
+  __shared__ Acc lds[TY][VEC][TX];
+
+  long long bid = blockIdx.x;
+  const int cb = (int)(bid % p.cblocks);
+  bid /= p.cblocks;
+  const int s = (int)(bid % p.S);
+  const long long a_idx = bid / p.S;
+  const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
+  const int cv = cb * TX + tx;                 // column vector owned by this thread
+  const bool live = (long long)cv * VEC < p.cols;
+
+  IT base[NIN];
+  {
+    UT rem = (UT)a_idx, c;
+#pragma unroll
+    for (int i = 0; i < NIN; ++i) base[i] = (IT)(live ? cv * VEC : 0) * p.c_stride[i];
+#pragma unroll
+    for (int d = NK - 1; d >= 1; --d) {
+      divmod(rem, p.kfd[d], rem, c);
+#pragma unroll
+      for (int i = 0; i < NIN; ++i) base[i] += (IT)c * p.kstride[i][d];
+    }
+#pragma unroll
+    for (int i = 0; i < NIN; ++i) base[i] += (IT)rem * p.kstride[i][0];
+  }
+
+  Acc acc[VEC];
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) R::init(acc[k]);
+
+  if (live) {
+    const long long r0 = (long long)s * p.rows_per_slice;
+    long long r1 = r0 + p.rows_per_slice;
+    if (r1 > p.rows) r1 = p.rows;
+    for (long long rr = r0 + ty; rr < r1; rr += (long long)TY * UNR) {
+      typename R::template Regs<VEC> r[UNR];
+      bool ok[UNR];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        const long long q = rr + (long long)u * TY;
+        ok[u] = q < r1;
+        RedAcc<P, NIN> a;
+        a.ptr = p.in;
+      a.imm = p.imm;
+        a.imm = p.imm;
+        a.vstride = p.c_stride;
+        if (P::RR2) {
+          UT q0, q1;
+          divmod((UT)(ok[u] ? q : r0), p.r1, q0, q1);
+#pragma unroll
+          for (int i = 0; i < NIN; ++i)
+            a.off[i] = base[i] + (IT)q0 * p.r0_stride[i] + (IT)q1 * p.r1_stride[i];
+        } else {
+#pragma unroll
+          for (int i = 0; i < NIN; ++i) a.off[i] = base[i] + (IT)q * p.r1_stride[i];
+        }
+        if (ok[u]) R::template load<VEC>(a, r[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < UNR; ++u)
+        if (ok[u]) R::template accum_lanes<VEC>(acc, r[u]);
+    }
+  }
+
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) lds[ty][k][tx] = acc[k];
+  __syncthreads();
+  for (int c = threadIdx.x; c < TX * VEC; c += P::BLOCK) {
+    const int x = c / VEC, k = c % VEC;
+    const long long col = (long long)cb * (TX * VEC) + c;
+    if (col < p.cols) {
+      Acc tot = lds[0][k][x];
+#pragma unroll
+      for (int y = 1; y < TY; ++y) R::comb(tot, lds[y][k][x]);
+      const long long o = a_idx * p.cols + col;
+      if (p.S == 1) {
+        R::post(p.out, o, tot);
+      } else {
+        ((Acc*)p.partial)[(long long)s * p.n_out + o] = tot;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Second pass: merge the S partial Acc values of every output, slice 0 first.
+// TPO threads per output (1, 64 or BLOCK).
+template <int NOUT>
+struct FinalParams {
+  RedOut<NOUT> out;
+  char* partial;
+  long long n_out;
+  int S;
+  int pad;
+};
+
+template <class R, int BLOCK, int TPO>
+__device__ __forceinline__ void red_final_body(const FinalParams<R::NOUT>& p) {
+  typedef typename R::Acc Acc;
+  __shared__ Acc lds[BLOCK / THX_WAVE];
+  const Acc* part = (const Acc*)p.partial;
+  const long long o = (long long)blockIdx.x * (BLOCK / TPO) + threadIdx.x / TPO;
+  const int t = threadIdx.x % TPO;
+  const bool live = o < p.n_out;
+  Acc acc;
+  R::init(acc);
+  if (live)
+    for (int s = t; s < p.S; s += TPO) R::comb(acc, part[(long long)s * p.n_out + o]);
+  if (TPO > THX_WAVE) {
+    acc = block_reduce<R, BLOCK / THX_WAVE>(acc, lds);
+  } else if (TPO > 1) {
+    acc = group_reduce<R, TPO>(acc);
+  }
+  if (live && t == 0) R::post(p.out, o, acc);
+}
+
+// ---------------------------------------------------------------------------
+// Fallback for any mask that does not collapse to the row or column form: TPR
+// threads per output walk the flattened reduce domain and decompose every
+// index. Correct for every pattern, coalesced only by luck.
+template <int NIN, int NOUT, int NK, int NR, class IT>
+struct GenParams {
+  char* in[NIN];
+  unsigned long long imm[NIN];
+  RedOut<NOUT> out;
+  long long n_out;
+  long long n_red;
+  FastDiv kfd[NK];
+  FastDiv rfd[NR];
+  IT kstride[NIN][NK];
+  IT rstride[NIN][NR];
+};
+
+// Plan members: typedef IT; enum { NK, NR, BLOCK, TPR }.
+template <class R, class P>
+__device__ __forceinline__ void red_gen_body(const GenParams<R::NIN, R::NOUT, P::NK, P::NR, typename P::IT>& p) {
+  typedef typename P::IT IT;
+  typedef typename UnsignedOf<IT>::type UT;
+  typedef typename R::Acc Acc;
+  constexpr int NIN = R::NIN, NK = P::NK, NR = P::NR, TPR = P::TPR;
+  __shared__ Acc lds[P::BLOCK / THX_WAVE];
+  const long long o = (long long)blockIdx.x * (P::BLOCK / TPR) + threadIdx.x / TPR;
+  const int t = threadIdx.x % TPR;
+  const bool live = o < p.n_out;
+  IT base[NIN];
+  {
+    UT rem = (UT)(live ? o : 0), c;
+#pragma unroll
+    for (int i = 0; i < NIN; ++i) base[i] = 0;
+#pragma unroll
+    for (int d = NK - 1; d >= 1; --d) {
+      divmod(rem, p.kfd[d], rem, c);
+#pragma unroll
+      for (int i = 0; i < NIN; ++i) base[i] += (IT)c * p.kstride[i][d];
+    }
+#pragma unroll
+    for (int i = 0; i < NIN; ++i) base[i] += (IT)rem * p.kstride[i][0];
+  }
+  Acc acc;
+  R::init(acc);
+  if (live) {
+    for (long long j = t; j < p.n_red; j += TPR) {
+      UT rem = (UT)j, c;
+      RedAcc<P, NIN> a;
+      a.ptr = p.in;
+      a.imm = p.imm;
+      a.vstride = nullptr;
+#pragma unroll
+      for (int i = 0; i < NIN; ++i) a.off[i] = base[i];
+#pragma unroll
+      for (int d = NR - 1; d >= 1; --d) {
+        divmod(rem, p.rfd[d], rem, c);
+#pragma unroll
+        for (int i = 0; i < NIN; ++i) a.off[i] += (IT)c * p.rstride[i][d];
+      }
+#pragma unroll
+      for (int i = 0; i < NIN; ++i) a.off[i] += (IT)rem * p.rstride[i][0];
+      typename R::template Regs<1> r;
+      R::template load<1>(a, r);
+      R::template accum<1>(acc, r);
+    }
+  }
+  if (TPR > THX_WAVE) {
+    acc = block_reduce<R, P::BLOCK / THX_WAVE>(acc, lds);
+  } else if (TPR > 1) {
+    acc = group_reduce<R, TPR>(acc);
+  }
+  if (live && t == 0) R::post(p.out, o, acc);
+}
+
+}  // namespace thx

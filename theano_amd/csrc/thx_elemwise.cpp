@@ -1,0 +1,238 @@
+// Elementwise planner: validates operands, collapses dimensions, picks an
+// access plan (rank, index width, vector width, per-operand access mode),
+// compiles the matching kernel on first use and launches it.
+#include <cstdlib>
+#include <cstring>
+#include <sstream>
+#include <unordered_map>
+
+#include "thx_internal.h"
+
+struct thx_elemwise {
+  std::string src, name;
+  int n_in = 0, n_out = 0;
+  std::vector<int32_t> dtypes;
+  std::unordered_map<std::string, thx::Kernel> plans;
+};
+
+namespace thx {
+
+enum { M_VEC = 0, M_BCAST = 1, M_GATHER = 2, M_IMM = 3 };
+
+struct Dims {
+  int nd = 0;
+  int64_t shape[THX_MAX_ND];
+  std::vector<std::vector<int64_t>> stride;  // [operand][dim]
+};
+
+// Drop extent-1 dimensions, then merge neighbours (outer d, inner d+1) that
+// every operand walks as one: stride[d] == stride[d+1] * shape[d+1].
+static void collapse(Dims* d) {
+  const size_t nops = d->stride.size();
+  int w = 0;
+  for (int i = 0; i < d->nd; ++i) {
+    if (d->shape[i] == 1) continue;
+    d->shape[w] = d->shape[i];
+    for (size_t o = 0; o < nops; ++o) d->stride[o][w] = d->stride[o][i];
+    ++w;
+  }
+  d->nd = w;
+  if (w == 0) {
+    d->nd = 1;
+    d->shape[0] = 1;
+    for (size_t o = 0; o < nops; ++o) d->stride[o][0] = 0;
+    return;
+  }
+  int out = 0;  // index of the dimension being grown
+  for (int i = 1; i < d->nd; ++i) {
+    bool ok = true;
+    for (size_t o = 0; o < nops && ok; ++o) ok = d->stride[o][out] == d->stride[o][i] * d->shape[i];
+    if (ok) {
+      d->shape[out] *= d->shape[i];
+      for (size_t o = 0; o < nops; ++o) d->stride[o][out] = d->stride[o][i];
+    } else {
+      ++out;
+      d->shape[out] = d->shape[i];
+      for (size_t o = 0; o < nops; ++o) d->stride[o][out] = d->stride[o][i];
+    }
+  }
+  d->nd = out + 1;
+}
+
+static int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : dflt;
+}
+
+}  // namespace thx
+
+using namespace thx;
+
+extern "C" {
+
+int thx_elemwise_new(const char* functor_src, const char* functor_name, int n_in, int n_out, const int32_t* dtypes,
+                     thx_elemwise** out) {
+  if (!functor_src || !functor_name || !dtypes || !out) return fail(THX_ERR_ARG, "thx_elemwise_new: null argument");
+  if (n_in < 1 || n_out < 1) return fail(THX_ERR_ARG, "thx_elemwise_new: needs inputs and outputs");
+  for (int i = 0; i < n_in + n_out; ++i)
+    if (!dtype_size(dtypes[i])) return fail(THX_ERR_TYPE, "thx_elemwise_new: unknown dtype code %d", dtypes[i]);
+  thx_elemwise* e = new thx_elemwise;
+  e->src = functor_src;
+  e->name = functor_name;
+  e->n_in = n_in;
+  e->n_out = n_out;
+  e->dtypes.assign(dtypes, dtypes + n_in + n_out);
+  *out = e;
+  return THX_OK;
+}
+
+int thx_elemwise_free(thx_elemwise* e) {
+  delete e;
+  return THX_OK;
+}
+
+int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* outs, int flags) {
+  if (!e || !ins || !outs) return fail(THX_ERR_ARG, "thx_elemwise_call: null argument");
+  const bool dry = (flags & THX_DRY_RUN) != 0;
+  if (!dry) {
+    int rc = ensure_init();
+    if (rc) return rc;
+  }
+  const int nops = e->n_in + e->n_out;
+  int nd = 0;
+  int64_t shape[THX_MAX_ND];
+  std::vector<View> views;
+  int rc = gather_inputs("elemwise", ins, e->n_in, e->dtypes.data(), flags, &nd, shape, &views);
+  if (rc) return rc;
+  views.resize(nops);
+  for (int o = 0; o < e->n_out; ++o) {
+    const thx_array& a = outs[o];
+    View& v = views[e->n_in + o];
+    if (a.nd != nd) return fail(THX_ERR_TYPE, "elemwise: output %d has rank %d, expected %d", o, a.nd, nd);
+    if (a.dtype != e->dtypes[e->n_in + o])
+      return fail(THX_ERR_TYPE, "elemwise: output %d has dtype code %d, the operation was built for %d", o, a.dtype,
+                  e->dtypes[e->n_in + o]);
+    const int isz = dtype_size(a.dtype);
+    v.ptr = (char*)a.base + a.offset_bytes;
+    v.dtype = a.dtype;
+    if (((uintptr_t)v.ptr) % isz) return fail(THX_ERR_TYPE, "elemwise: output %d is not aligned to its element size", o);
+    for (int d = 0; d < nd; ++d) {
+      if (a.shape[d] != shape[d])
+        return fail(THX_ERR_SHAPE, "elemwise: output %d has extent %lld along dimension %d, the result has %lld", o,
+                    (long long)a.shape[d], d, (long long)shape[d]);
+      if (a.strides_bytes[d] % isz)
+        return fail(THX_ERR_TYPE, "elemwise: output %d stride is not a multiple of its element size", o);
+      v.stride[d] = a.strides_bytes[d] / isz;
+      if (shape[d] > 1 && v.stride[d] == 0)
+        return fail(THX_ERR_TYPE, "elemwise: output %d has a zero stride along dimension %d", o, d);
+    }
+  }
+  int64_t n = 1;
+  for (int d = 0; d < nd; ++d) n *= shape[d];
+  if (n == 0) {
+    set_last_plan("ew|empty");
+    return THX_OK;
+  }
+
+  Dims dm;
+  dm.nd = nd;
+  for (int d = 0; d < nd; ++d) dm.shape[d] = shape[d];
+  dm.stride.resize(nops);
+  for (int o = 0; o < nops; ++o) dm.stride[o].assign(views[o].stride, views[o].stride + THX_MAX_ND);
+  if (nd == 0) {
+    dm.nd = 1;
+    dm.shape[0] = 1;
+    for (int o = 0; o < nops; ++o) dm.stride[o][0] = 0;
+  }
+  collapse(&dm);
+  const int ND = dm.nd;
+  const int64_t inner = dm.shape[ND - 1];
+
+  // index width: every element offset and the flat index must fit in 31 bits
+  bool wide = n >= (int64_t(1) << 31) - 65536;
+  for (int o = 0; o < nops && !wide; ++o) {
+    int64_t span = 0;
+    for (int d = 0; d < ND; ++d) span += (dm.shape[d] - 1) * (dm.stride[o][d] < 0 ? -dm.stride[o][d] : dm.stride[o][d]);
+    if (span >= (int64_t(1) << 31) - 65536) wide = true;
+  }
+
+  // access modes along the innermost dimension
+  std::vector<int> mode(nops);
+  int maxsz = 0;
+  bool any_vec = false;
+  for (int o = 0; o < nops; ++o) {
+    const int64_t st = dm.stride[o][ND - 1];
+    mode[o] = st == 1 ? M_VEC : (st == 0 ? M_BCAST : M_GATHER);
+    if (n == 1) mode[o] = M_BCAST;
+    if (views[o].imm) mode[o] = M_IMM;
+    if (o >= e->n_in && mode[o] == M_BCAST) mode[o] = M_GATHER;
+    if (mode[o] == M_VEC) {
+      any_vec = true;
+      if (dtype_size(views[o].dtype) > maxsz) maxsz = dtype_size(views[o].dtype);
+    }
+  }
+  int vec = any_vec ? 16 / maxsz : 1;
+  const int force_vec = env_int("THX_EW_VEC", 0);
+  if (force_vec > 0 && force_vec < vec) vec = force_vec;
+  auto vec_ok = [&](int v) {
+    if (v == 1) return true;
+    if (ND > 1 && (inner % v != 0 || inner / v < 2)) return false;
+    for (int o = 0; o < nops; ++o) {
+      if (mode[o] != M_VEC) continue;
+      const int isz = dtype_size(views[o].dtype);
+      if (((uintptr_t)views[o].ptr) % (size_t)(isz * v)) return false;
+      for (int d = 0; d < ND - 1; ++d)
+        if (dm.stride[o][d] % v) return false;
+    }
+    return true;
+  };
+  while (!vec_ok(vec)) vec /= 2;
+
+  const int64_t nvec = ND == 1 ? n / vec : n / vec;
+  int unr = nvec >= (int64_t(1) << 20) ? 4 : (nvec >= (int64_t(1) << 18) ? 2 : 1);
+  const int force_unr = env_int("THX_EW_UNR", 0);
+  if (force_unr > 0) unr = force_unr;
+  const int block = 256;
+
+  std::ostringstream key;
+  key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|m";
+  for (int o = 0; o < nops; ++o) key << mode[o] << (o + 1 < nops ? "," : "");
+  const std::string plan = key.str();
+  set_last_plan(e->name + "|" + plan);
+
+  Kernel k;
+  auto it = e->plans.find(plan);
+  if (it != e->plans.end() && (it->second.func || dry)) {
+    k = it->second;
+  } else {
+    std::ostringstream s;
+    s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
+      << " IT;\n  enum { ND = " << ND << ", VEC = " << vec << ", UNR = " << unr << ", BLOCK = " << block
+      << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+    for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
+    s << "};\n    return m[i];\n  }\n};\n"
+      << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::EwParams<" << e->name
+      << "::NOPS, ThxPlan::ND, ThxPlan::IT> p) {\n  thx::ew_body<" << e->name << ", ThxPlan>(p);\n}\n";
+    rc = get_kernel(s.str(), "thx_entry", &k);
+    if (rc) return rc;
+    e->plans[plan] = k;
+  }
+  if (dry) return THX_OK;
+
+  ParamPack pk;
+  for (int o = 0; o < nops; ++o) pk.put<char*>(views[o].ptr);
+  for (int o = 0; o < nops; ++o) pk.put<uint64_t>(views[o].immval);
+  pk.put<int64_t>(nvec);
+  pk.put<int64_t>(n);
+  for (int d = 0; d < ND; ++d) pk.put<FastDivH>(make_fastdiv(d == ND - 1 && ND > 1 ? (uint64_t)(inner / vec) : (uint64_t)dm.shape[d]));
+  for (int o = 0; o < nops; ++o)
+    for (int d = 0; d < ND; ++d) pk.put_index(wide, dm.stride[o][d]);
+  pk.align(8);
+
+  int64_t grid = (nvec + (int64_t)block * unr - 1) / ((int64_t)block * unr);
+  if (grid < 1) grid = 1;
+  if (grid > 0x7fffffffLL) return fail(THX_ERR_UNSUPPORTED, "elemwise: %lld blocks exceed the grid limit", (long long)grid);
+  return launch(k, e->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
+}
+
+}  // extern "C"

@@ -1,0 +1,100 @@
+// Host-side internals of libthx_hip.so shared by the runtime, the elementwise
+// planner and the reduction planner.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "../../include/thx_hip.h"
+
+namespace thx {
+
+// ---- errors ---------------------------------------------------------------
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+void set_last_plan(const std::string& plan);
+
+#define THX_HIP_CHECK(expr)                                                        \
+  do {                                                                             \
+    hipError_t e_ = (expr);                                                        \
+    if (e_ != hipSuccess)                                                          \
+      return ::thx::fail(THX_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+// ---- global state -----------------------------------------------------------
+struct Runtime {
+  bool ready = false;
+  int device = -1;
+  int cus = 0;
+  int64_t hbm = 0;
+  std::string arch;       // as reported, e.g. gfx950:sramecc+:xnack-
+  std::string arch_base;  // gfx950
+  hipStream_t stream = nullptr;
+  char* scratch = nullptr;  // partial results of split reductions
+  size_t scratch_bytes = 0;
+};
+Runtime& rt();
+int ensure_init();
+int ensure_scratch(size_t bytes);
+
+// ---- run-time compilation ---------------------------------------------------
+struct Kernel {
+  hipModule_t module = nullptr;
+  hipFunction_t func = nullptr;
+};
+// Compile (or fetch from the caches) `source`, which must define an
+// extern "C" __global__ function named `entry`.
+int get_kernel(const std::string& source, const std::string& entry, Kernel* out);
+// The embedded device headers (thx_common.h, thx_elemwise.h, thx_reduce.h).
+const std::string& device_prelude();
+
+// Launch with one by-value parameter block.
+int launch(const Kernel& k, const std::string& plan, unsigned grid, unsigned block,
+           const void* params, size_t params_bytes);
+
+// ---- array helpers ----------------------------------------------------------
+int dtype_size(int dtype);
+const char* dtype_ctype(int dtype);
+
+// FastDiv as laid out in kernels/thx_common.h.
+struct FastDivH {
+  uint32_t m, s, d, pad;
+};
+FastDivH make_fastdiv(uint64_t d);
+
+// Byte-wise builder for kernel parameter blocks whose layout depends on
+// template arguments; mirrors the natural alignment rules of the device structs.
+struct ParamPack {
+  std::vector<unsigned char> buf;
+  void align(size_t a) {
+    while (buf.size() % a) buf.push_back(0);
+  }
+  template <class T>
+  void put(const T& v) {
+    align(alignof(T));
+    const unsigned char* p = reinterpret_cast<const unsigned char*>(&v);
+    buf.insert(buf.end(), p, p + sizeof(T));
+  }
+  void put_index(bool wide, int64_t v) {
+    if (wide) put<int64_t>(v);
+    else put<int32_t>(static_cast<int32_t>(v));
+  }
+};
+
+// One operand after validation: element strides over the common shape.
+struct View {
+  char* ptr = nullptr;
+  int dtype = 0;
+  bool imm = false;     // a host scalar travelling in the kernel arguments
+  uint64_t immval = 0;  // its value bytes
+  int64_t stride[THX_MAX_ND] = {0};
+};
+
+// Check ranks/dtypes, compute the broadcast shape of `ins`, convert strides to
+// elements (0 on broadcast dimensions). `what` names the operation in messages.
+int gather_inputs(const char* what, const thx_array* ins, int n_in, const int32_t* dtypes, int flags,
+                  int* nd_out, int64_t* shape, std::vector<View>* views);
+
+}  // namespace thx

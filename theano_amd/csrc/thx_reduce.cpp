@@ -1,0 +1,478 @@
+// Reduction planner: canonicalises (shape, strides, mask) into kept and reduced
+// dimension lists, chooses the row, column or generic kernel form, sizes the
+// slice split for the device, compiles on first use and launches one or two
+// passes.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <sstream>
+#include <unordered_map>
+
+#include "thx_internal.h"
+
+struct thx_reduce {
+  std::string src, name;
+  int n_in = 0, n_out = 0, acc_bytes = 0;
+  std::vector<int32_t> dtypes;
+  std::unordered_map<std::string, thx::Kernel> plans;
+};
+
+namespace thx {
+
+enum { M_VEC = 0, M_BCAST = 1, M_GATHER = 2, M_IMM = 3 };
+
+struct Dim {
+  int64_t extent;
+  std::vector<int64_t> stride;  // per input
+};
+
+static void merge_dims(std::vector<Dim>* v) {
+  std::vector<Dim> out;
+  for (const Dim& d : *v) {
+    if (!out.empty()) {
+      Dim& o = out.back();  // o is the outer neighbour of d
+      bool ok = true;
+      for (size_t i = 0; i < d.stride.size() && ok; ++i) ok = o.stride[i] == d.stride[i] * d.extent;
+      if (ok) {
+        o.extent *= d.extent;
+        o.stride = d.stride;
+        continue;
+      }
+    }
+    out.push_back(d);
+  }
+  v->swap(out);
+}
+
+static int64_t iabs(int64_t x) { return x < 0 ? -x : x; }
+static int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static int64_t round_up(int64_t a, int64_t b) { return ceil_div(a, b) * b; }
+static int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return v ? atoi(v) : dflt;
+}
+
+static std::string plan_struct(bool wide, const std::vector<std::pair<std::string, int64_t>>& consts,
+                               const std::vector<int>& mode) {
+  std::ostringstream s;
+  s << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int") << " IT;\n  enum { ";
+  for (size_t i = 0; i < consts.size(); ++i) s << consts[i].first << " = " << consts[i].second << (i + 1 < consts.size() ? ", " : "");
+  s << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+  for (size_t i = 0; i < mode.size(); ++i) s << mode[i] << (i + 1 < mode.size() ? ", " : "");
+  s << "};\n    return m[i];\n  }\n};\n";
+  return s.str();
+}
+
+static int final_pass(thx_reduce* r, const std::vector<char*>& outp, char* partial, int64_t n_out, int S, bool dry) {
+  const int tpo = n_out >= 1024 ? 1 : (n_out >= 16 ? 64 : 256);
+  const std::string plan = "rf|t" + std::to_string(tpo);
+  Kernel k;
+  auto it = r->plans.find(plan);
+  if (it != r->plans.end() && (it->second.func || dry)) {
+    k = it->second;
+  } else {
+    std::ostringstream s;
+    s << device_prelude() << r->src << "\nextern \"C\" __global__ __launch_bounds__(256) void thx_entry(thx::FinalParams<"
+      << r->name << "::NOUT> p) {\n  thx::red_final_body<" << r->name << ", 256, " << tpo << ">(p);\n}\n";
+    int rc = get_kernel(s.str(), "thx_entry", &k);
+    if (rc) return rc;
+    r->plans[plan] = k;
+  }
+  if (dry) return THX_OK;
+  ParamPack pk;
+  for (char* p : outp) pk.put<char*>(p);
+  pk.put<char*>(partial);
+  pk.put<int64_t>(n_out);
+  pk.put<int32_t>(S);
+  pk.put<int32_t>(0);
+  pk.align(8);
+  const int64_t grid = ceil_div(n_out, 256 / tpo);
+  return launch(k, r->name + "|" + plan, (unsigned)grid, 256, pk.buf.data(), pk.buf.size());
+}
+
+}  // namespace thx
+
+using namespace thx;
+
+extern "C" {
+
+int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, int n_out, const int32_t* dtypes,
+                   int acc_bytes, thx_reduce** out) {
+  if (!functor_src || !functor_name || !dtypes || !out) return fail(THX_ERR_ARG, "thx_reduce_new: null argument");
+  if (n_in < 1 || n_out < 1 || acc_bytes < 1) return fail(THX_ERR_ARG, "thx_reduce_new: needs inputs, outputs and an accumulator");
+  for (int i = 0; i < n_in + n_out; ++i)
+    if (!dtype_size(dtypes[i])) return fail(THX_ERR_TYPE, "thx_reduce_new: unknown dtype code %d", dtypes[i]);
+  thx_reduce* r = new thx_reduce;
+  r->src = functor_src;
+  r->name = functor_name;
+  r->n_in = n_in;
+  r->n_out = n_out;
+  r->acc_bytes = acc_bytes;
+  r->dtypes.assign(dtypes, dtypes + n_in + n_out);
+  *out = r;
+  return THX_OK;
+}
+
+int thx_reduce_free(thx_reduce* r) {
+  delete r;
+  return THX_OK;
+}
+
+int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_mask, const thx_array* outs, int flags) {
+  if (!r || !ins || !outs) return fail(THX_ERR_ARG, "thx_reduce_call: null argument");
+  const bool dry = (flags & THX_DRY_RUN) != 0;
+  if (!dry) {
+    int rc = ensure_init();
+    if (rc) return rc;
+  }
+  const int NIN = r->n_in, NOUT = r->n_out;
+  int nd = 0;
+  int64_t shape[THX_MAX_ND];
+  std::vector<View> views;
+  int rc = gather_inputs("reduce", ins, NIN, r->dtypes.data(), flags, &nd, shape, &views);
+  if (rc) return rc;
+  if (nd > 0 && !reduce_mask) return fail(THX_ERR_ARG, "thx_reduce_call: null mask");
+
+  // outputs: C-contiguous arrays of the kept dimensions
+  int64_t kshape[THX_MAX_ND];
+  int nk_full = 0;
+  int64_t n_out = 1, n_red = 1;
+  for (int d = 0; d < nd; ++d) {
+    if (reduce_mask[d]) {
+      n_red *= shape[d];
+    } else {
+      kshape[nk_full++] = shape[d];
+      n_out *= shape[d];
+    }
+  }
+  std::vector<char*> outp(NOUT);
+  for (int o = 0; o < NOUT; ++o) {
+    const thx_array& a = outs[o];
+    if (a.nd != nk_full) return fail(THX_ERR_TYPE, "reduce: output %d has rank %d, expected %d", o, a.nd, nk_full);
+    if (a.dtype != r->dtypes[NIN + o])
+      return fail(THX_ERR_TYPE, "reduce: output %d has dtype code %d, the operation was built for %d", o, a.dtype,
+                  r->dtypes[NIN + o]);
+    const int isz = dtype_size(a.dtype);
+    int64_t expect = isz;
+    for (int d = nk_full - 1; d >= 0; --d) {
+      if (a.shape[d] != kshape[d])
+        return fail(THX_ERR_SHAPE, "reduce: output %d has extent %lld along dimension %d, the result has %lld", o,
+                    (long long)a.shape[d], d, (long long)kshape[d]);
+      if (a.shape[d] > 1 && a.strides_bytes[d] != expect)
+        return fail(THX_ERR_TYPE, "reduce: output %d is not C-contiguous", o);
+      expect *= a.shape[d];
+    }
+    outp[o] = (char*)a.base + a.offset_bytes;
+    if (((uintptr_t)outp[o]) % isz) return fail(THX_ERR_TYPE, "reduce: output %d is not aligned to its element size", o);
+  }
+  if (n_out == 0) {
+    set_last_plan("red|empty");
+    return THX_OK;
+  }
+  if (n_red == 0) {  // identity through the epilogue
+    set_last_plan(r->name + "|rf|identity");
+    return final_pass(r, outp, nullptr, n_out, 0, dry);
+  }
+
+  // primary input: the one that spans the most memory
+  int primary = 0;
+  {
+    int64_t best = -1;
+    for (int i = 0; i < NIN; ++i) {
+      int64_t foot = 1;
+      for (int d = 0; d < nd; ++d)
+        if (views[i].stride[d] != 0) foot *= shape[d];
+      foot *= dtype_size(views[i].dtype);
+      if (foot > best) {
+        best = foot;
+        primary = i;
+      }
+    }
+  }
+  std::vector<Dim> KD, RD;
+  for (int d = 0; d < nd; ++d) {
+    if (shape[d] == 1) continue;
+    Dim dm;
+    dm.extent = shape[d];
+    for (int i = 0; i < NIN; ++i) dm.stride.push_back(views[i].stride[d]);
+    (reduce_mask[d] ? RD : KD).push_back(dm);
+  }
+  // reduced dimensions commute: walk them from the largest stride to the smallest
+  std::stable_sort(RD.begin(), RD.end(),
+                   [&](const Dim& a, const Dim& b) { return iabs(a.stride[primary]) > iabs(b.stride[primary]); });
+  merge_dims(&KD);
+  merge_dims(&RD);
+  const int NKD = (int)KD.size(), NR = (int)RD.size();
+
+  const int cus = rt().ready ? rt().cus : 256;
+  const int64_t target = (int64_t)cus * env_int("THX_RED_BLOCKS_PER_CU", 8);
+
+  bool wide = n_out >= (int64_t(1) << 31) - 65536 || n_red >= (int64_t(1) << 31) - 65536;
+  for (int i = 0; i < NIN && !wide; ++i) {
+    int64_t span = 0;
+    for (const Dim& d : KD) span += (d.extent - 1) * iabs(d.stride[i]);
+    for (const Dim& d : RD) span += (d.extent - 1) * iabs(d.stride[i]);
+    if (span >= (int64_t(1) << 31) - 65536) wide = true;
+  }
+
+  enum { ROW, COL, GEN } form;
+  if (NR > 2) form = GEN;
+  else if (NR == 0 || NKD == 0) form = ROW;
+  else if (iabs(RD.back().stride[primary]) == 1) form = ROW;
+  else if (KD.back().stride[primary] == 1) form = COL;
+  else form = ROW;
+  const char* force = getenv("THX_RED_FORM");
+  if (force && NR <= 2 && NR > 0) {
+    if (!strcmp(force, "row")) form = ROW;
+    if (!strcmp(force, "col") && NKD > 0) form = COL;
+    if (!strcmp(force, "gen")) form = GEN;
+  }
+
+  auto vec_width = [&](const std::vector<int>& mode) {
+    int maxsz = 0;
+    for (int i = 0; i < NIN; ++i)
+      if (mode[i] == M_VEC) maxsz = std::max(maxsz, dtype_size(views[i].dtype));
+    return maxsz ? 16 / maxsz : 1;
+  };
+
+  const int block = 256;
+  std::string plan;
+  Kernel k;
+  ParamPack pk;
+  int64_t grid = 0;
+  int S = 1;
+
+  if (form == ROW) {
+    const int64_t RC = NR ? RD.back().extent : 1;
+    const int64_t RA = NR == 2 ? RD[0].extent : 1;
+    const int ra2 = NR == 2;
+    std::vector<int> mode(NIN);
+    std::vector<int64_t> rc_stride(NIN), ra_stride(NIN);
+    for (int i = 0; i < NIN; ++i) {
+      rc_stride[i] = NR ? RD.back().stride[i] : 0;
+      ra_stride[i] = ra2 ? RD[0].stride[i] : 0;
+      mode[i] = rc_stride[i] == 1 ? M_VEC : (rc_stride[i] == 0 ? M_BCAST : M_GATHER);
+      if (views[i].imm) mode[i] = M_IMM;
+    }
+    int vec = vec_width(mode);
+    auto vec_ok = [&](int v) {
+      if (v == 1) return true;
+      if (RC % v) return false;
+      if (ra2 && RC / v < 2) return false;
+      for (int i = 0; i < NIN; ++i) {
+        if (mode[i] != M_VEC) continue;
+        if (((uintptr_t)views[i].ptr) % (size_t)(dtype_size(views[i].dtype) * v)) return false;
+        if (ra_stride[i] % v) return false;
+        for (const Dim& d : KD)
+          if (d.stride[i] % v) return false;
+      }
+      return true;
+    };
+    while (!vec_ok(vec)) vec /= 2;
+    const int64_t nvec = RA * RC / vec;
+    int tpr = nvec >= 512 ? 256 : nvec >= 64 ? 64 : nvec >= 16 ? 16 : nvec >= 4 ? 4 : 1;
+    const int force_tpr = env_int("THX_RED_TPR", 0);
+    if (force_tpr > 0) tpr = force_tpr;
+    const int64_t per_thread = ceil_div(nvec, tpr);
+    int unr = per_thread >= 4 ? 4 : per_thread >= 2 ? 2 : 1;
+    const int force_unr = env_int("THX_RED_UNR", 0);
+    if (force_unr > 0) unr = force_unr;
+    const int rpb = block / tpr;
+    const int64_t oblocks = ceil_div(n_out, rpb);
+    int64_t chunk = nvec;
+    if (oblocks * 2 <= target && nvec >= (int64_t)tpr * unr * 4) {
+      int64_t want = std::min(ceil_div(target, oblocks), nvec / ((int64_t)tpr * unr * 2));
+      if (want > 1) {
+        chunk = round_up(ceil_div(nvec, want), (int64_t)tpr * unr);
+        S = (int)ceil_div(nvec, chunk);
+      }
+    }
+    if (ra2 && nvec >= (int64_t(1) << 31) - 65536) wide = true;
+    const int NK = std::max(1, NKD);
+    std::ostringstream key;
+    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|t" << tpr << "|a" << ra2 << "|m";
+    for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
+    plan = key.str();
+    auto it = r->plans.find(plan);
+    if (it != r->plans.end() && (it->second.func || dry)) {
+      k = it->second;
+    } else {
+      std::ostringstream s;
+      s << device_prelude() << r->src
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TPR", tpr}, {"RA2", ra2}}, mode)
+        << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::RowParams<" << r->name
+        << "::NIN, " << r->name << "::NOUT, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
+        << ", ThxPlan>(p);\n}\n";
+      rc = get_kernel(s.str(), "thx_entry", &k);
+      if (rc) return rc;
+      r->plans[plan] = k;
+    }
+    if (!dry && S > 1) {
+      rc = ensure_scratch((size_t)S * n_out * r->acc_bytes);
+      if (rc) return rc;
+    }
+    for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
+    for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
+    for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
+    pk.put<char*>(rt().scratch);
+    pk.put<int64_t>(n_out);
+    pk.put<int64_t>(nvec);
+    pk.put<int64_t>(chunk);
+    pk.put<int32_t>(S);
+    pk.put<int32_t>(0);
+    for (int d = 0; d < NK; ++d) pk.put<FastDivH>(make_fastdiv(d < NKD ? (uint64_t)KD[d].extent : 1));
+    pk.put<FastDivH>(make_fastdiv((uint64_t)(RC / vec)));
+    for (int i = 0; i < NIN; ++i)
+      for (int d = 0; d < NK; ++d) pk.put_index(wide, d < NKD ? KD[d].stride[i] : 0);
+    for (int i = 0; i < NIN; ++i) pk.put_index(wide, ra_stride[i]);
+    for (int i = 0; i < NIN; ++i) pk.put_index(wide, rc_stride[i]);
+    pk.align(8);
+    grid = oblocks * S;
+  } else if (form == COL) {
+    const int64_t C = KD.back().extent;
+    const int ko = NKD - 1;  // outer kept dimensions
+    const int NK = std::max(1, ko);
+    const int rr2 = NR == 2;
+    const int64_t rows = n_red;
+    std::vector<int> mode(NIN);
+    std::vector<int64_t> c_stride(NIN), r0_stride(NIN), r1_stride(NIN);
+    for (int i = 0; i < NIN; ++i) {
+      c_stride[i] = KD.back().stride[i];
+      r1_stride[i] = RD.back().stride[i];
+      r0_stride[i] = rr2 ? RD[0].stride[i] : 0;
+      mode[i] = c_stride[i] == 1 ? M_VEC : (c_stride[i] == 0 ? M_BCAST : M_GATHER);
+      if (views[i].imm) mode[i] = M_IMM;
+    }
+    int vec = vec_width(mode);
+    auto vec_ok = [&](int v) {
+      if (v == 1) return true;
+      if (C % v) return false;
+      if ((int64_t)block * v * r->acc_bytes > 32768) return false;
+      for (int i = 0; i < NIN; ++i) {
+        if (mode[i] != M_VEC) continue;
+        if (((uintptr_t)views[i].ptr) % (size_t)(dtype_size(views[i].dtype) * v)) return false;
+        if (r0_stride[i] % v || r1_stride[i] % v) return false;
+        for (int d = 0; d < ko; ++d)
+          if (KD[d].stride[i] % v) return false;
+      }
+      return true;
+    };
+    while (!vec_ok(vec)) vec /= 2;
+    if ((int64_t)block * vec * r->acc_bytes > 65536)
+      return fail(THX_ERR_UNSUPPORTED, "reduce: accumulator of %d bytes is too large for the column kernel", r->acc_bytes);
+    const int64_t cvecs = C / vec;
+    int tx = 1;
+    while (tx < 64 && tx < cvecs) tx *= 2;
+    const int force_tx = env_int("THX_RED_TX", 0);
+    if (force_tx > 0) tx = force_tx;
+    const int ty = block / tx;
+    const int64_t cblocks = ceil_div(cvecs, tx);
+    int64_t A = 1;
+    for (int d = 0; d < ko; ++d) A *= KD[d].extent;
+    const int64_t per_lane = ceil_div(rows, ty);
+    int unr = per_lane >= 4 ? 4 : per_lane >= 2 ? 2 : 1;
+    const int force_unr = env_int("THX_RED_UNR", 0);
+    if (force_unr > 0) unr = force_unr;
+    const int64_t blocks0 = A * cblocks;
+    int64_t rps = rows;
+    if (blocks0 * 2 <= target && rows >= (int64_t)ty * unr * 2) {
+      int64_t want = std::min(ceil_div(target, blocks0), rows / ((int64_t)ty * unr));
+      if (want > 1) {
+        rps = round_up(ceil_div(rows, want), (int64_t)ty * unr);
+        S = (int)ceil_div(rows, rps);
+      }
+    }
+    std::ostringstream key;
+    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << "|r" << rr2 << "|m";
+    for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
+    plan = key.str();
+    auto it = r->plans.find(plan);
+    if (it != r->plans.end() && (it->second.func || dry)) {
+      k = it->second;
+    } else {
+      std::ostringstream s;
+      s << device_prelude() << r->src
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TX", tx}, {"RR2", rr2}}, mode)
+        << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::ColParams<" << r->name
+        << "::NIN, " << r->name << "::NOUT, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_col_body<" << r->name
+        << ", ThxPlan>(p);\n}\n";
+      rc = get_kernel(s.str(), "thx_entry", &k);
+      if (rc) return rc;
+      r->plans[plan] = k;
+    }
+    if (!dry && S > 1) {
+      rc = ensure_scratch((size_t)S * n_out * r->acc_bytes);
+      if (rc) return rc;
+    }
+    for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
+    for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
+    for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
+    pk.put<char*>(rt().scratch);
+    pk.put<int64_t>(n_out);
+    pk.put<int64_t>(rows);
+    pk.put<int64_t>(rps);
+    pk.put<int32_t>((int32_t)C);
+    pk.put<int32_t>((int32_t)cblocks);
+    pk.put<int32_t>(S);
+    pk.put<int32_t>(0);
+    for (int d = 0; d < NK; ++d) pk.put<FastDivH>(make_fastdiv(d < ko ? (uint64_t)KD[d].extent : 1));
+    pk.put<FastDivH>(make_fastdiv((uint64_t)RD.back().extent));
+    for (int i = 0; i < NIN; ++i)
+      for (int d = 0; d < NK; ++d) pk.put_index(wide, d < ko ? KD[d].stride[i] : 0);
+    for (int i = 0; i < NIN; ++i) pk.put_index(wide, r0_stride[i]);
+    for (int i = 0; i < NIN; ++i) pk.put_index(wide, r1_stride[i]);
+    for (int i = 0; i < NIN; ++i) pk.put_index(wide, c_stride[i]);
+    pk.align(8);
+    if (C >= (int64_t(1) << 31)) return fail(THX_ERR_UNSUPPORTED, "reduce: %lld kept columns", (long long)C);
+    grid = blocks0 * S;
+  } else {
+    const int NK = std::max(1, NKD);
+    const int tpr = n_red >= 512 ? 256 : n_red >= 64 ? 64 : 1;
+    std::vector<int> gmode(NIN, M_GATHER);
+    std::ostringstream key;
+    key << "rg|k" << NK << "|r" << NR << (wide ? "|i64" : "|i32") << "|t" << tpr << "|m";
+    for (int i = 0; i < NIN; ++i) {
+      if (views[i].imm) gmode[i] = M_IMM;
+      key << gmode[i] << (i + 1 < NIN ? "," : "");
+    }
+    plan = key.str();
+    auto it = r->plans.find(plan);
+    if (it != r->plans.end() && (it->second.func || dry)) {
+      k = it->second;
+    } else {
+      std::ostringstream s;
+      s << device_prelude() << r->src
+        << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}}, gmode)
+        << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::GenParams<" << r->name
+        << "::NIN, " << r->name << "::NOUT, ThxPlan::NK, ThxPlan::NR, ThxPlan::IT> p) {\n  thx::red_gen_body<" << r->name
+        << ", ThxPlan>(p);\n}\n";
+      rc = get_kernel(s.str(), "thx_entry", &k);
+      if (rc) return rc;
+      r->plans[plan] = k;
+    }
+    for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
+    for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
+    for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
+    pk.put<int64_t>(n_out);
+    pk.put<int64_t>(n_red);
+    for (int d = 0; d < NK; ++d) pk.put<FastDivH>(make_fastdiv(d < NKD ? (uint64_t)KD[d].extent : 1));
+    for (int d = 0; d < NR; ++d) pk.put<FastDivH>(make_fastdiv((uint64_t)RD[d].extent));
+    for (int i = 0; i < NIN; ++i)
+      for (int d = 0; d < NK; ++d) pk.put_index(wide, d < NKD ? KD[d].stride[i] : 0);
+    for (int i = 0; i < NIN; ++i)
+      for (int d = 0; d < NR; ++d) pk.put_index(wide, RD[d].stride[i]);
+    pk.align(8);
+    grid = ceil_div(n_out, block / tpr);
+  }
+
+  set_last_plan(r->name + "|" + plan + (S > 1 ? "|s" + std::to_string(S) : ""));
+  if (grid > 0x7fffffffLL) return fail(THX_ERR_UNSUPPORTED, "reduce: %lld blocks exceed the grid limit", (long long)grid);
+  if (!dry) {
+    rc = launch(k, r->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
+    if (rc) return rc;
+  }
+  if (S > 1) return final_pass(r, outp, rt().scratch, n_out, S, dry);
+  return THX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,562 @@
+// Runtime of libthx_hip.so: device set-up, pooled memory, transfers, the hipRTC
+// compile path with its two caches, launches and event timing.
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <mutex>
+#include <sstream>
+#include <unordered_map>
+
+#include "thx_internal.h"
+
+namespace thx {
+
+// ---------------------------------------------------------------------------
+// errors
+static thread_local std::string g_error;
+static thread_local std::string g_plan;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[4096];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_error = buf;
+  return code;
+}
+void set_last_plan(const std::string& plan) { g_plan = plan; }
+
+// ---------------------------------------------------------------------------
+// state
+static std::mutex g_mu;
+Runtime& rt() {
+  static Runtime r;
+  return r;
+}
+
+static std::string g_cache_dir;
+static bool g_cache_dir_set = false;
+static int64_t g_n_compiled = 0, g_n_disk = 0, g_n_mem = 0;
+static std::unordered_map<std::string, Kernel> g_kernels;  // by hash of source
+
+// pool
+static std::unordered_map<size_t, std::vector<void*>> g_free;
+static std::unordered_map<void*, size_t> g_live;
+
+// profiling
+struct ProfRec {
+  std::string plan;
+  hipEvent_t a, b;
+};
+static bool g_profiling = false;
+static std::vector<ProfRec> g_prof;
+static hipEvent_t g_t0 = nullptr, g_t1 = nullptr;
+
+static int init_locked(int device) {
+  Runtime& r = rt();
+  if (r.ready) {
+    if (device >= 0 && device != r.device)
+      return fail(THX_ERR_ARG, "thx_init: already bound to device %d, asked for %d", r.device, device);
+    return THX_OK;
+  }
+  if (device < 0) device = 0;
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count == 0)
+    return fail(THX_ERR_HIP, "thx_init: no HIP device is visible (%s)", hipGetErrorString(e));
+  if (device >= count) return fail(THX_ERR_ARG, "thx_init: device %d of %d", device, count);
+  THX_HIP_CHECK(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  THX_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+  r.device = device;
+  r.cus = prop.multiProcessorCount;
+  r.hbm = (int64_t)prop.totalGlobalMem;
+  r.arch = prop.gcnArchName;
+  r.arch_base = r.arch.substr(0, r.arch.find(':'));
+  THX_HIP_CHECK(hipStreamCreateWithFlags(&r.stream, hipStreamNonBlocking));
+  THX_HIP_CHECK(hipEventCreate(&g_t0));
+  THX_HIP_CHECK(hipEventCreate(&g_t1));
+  r.ready = true;
+  return THX_OK;
+}
+
+int ensure_init() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  return init_locked(-1);
+}
+
+int ensure_scratch(size_t bytes) {
+  Runtime& r = rt();
+  if (bytes <= r.scratch_bytes) return THX_OK;
+  if (r.scratch) {
+    THX_HIP_CHECK(hipStreamSynchronize(r.stream));
+    THX_HIP_CHECK(hipFree(r.scratch));
+    r.scratch = nullptr;
+    r.scratch_bytes = 0;
+  }
+  size_t want = bytes < (size_t(8) << 20) ? (size_t(8) << 20) : bytes;
+  void* p = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess)
+    return fail(THX_ERR_MEMORY, "cannot allocate %zu bytes of reduction scratch", want);
+  r.scratch = (char*)p;
+  r.scratch_bytes = want;
+  return THX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// helpers
+int dtype_size(int dtype) {
+  static const int sz[THX_NDTYPES] = {1, 1, 1, 2, 2, 4, 4, 8, 8, 2, 4, 8};
+  return (dtype >= 0 && dtype < THX_NDTYPES) ? sz[dtype] : 0;
+}
+const char* dtype_ctype(int dtype) {
+  static const char* nm[THX_NDTYPES] = {"thx_bool", "thx_i8",  "thx_u8",  "thx_i16", "thx_u16", "thx_i32",
+                                        "thx_u32",  "thx_i64", "thx_u64", "thx_f16", "thx_f32", "thx_f64"};
+  return (dtype >= 0 && dtype < THX_NDTYPES) ? nm[dtype] : "void";
+}
+
+FastDivH make_fastdiv(uint64_t d) {
+  FastDivH f{0, 0, (uint32_t)d, 0};
+  if (d < 2 || d >= (uint64_t(1) << 31)) return f;  // 64-bit plans divide directly; d = 1 slots are never divided by
+  unsigned L = 0;
+  while ((uint64_t(1) << L) < d) ++L;
+  const unsigned __int128 one = 1;
+  const unsigned __int128 num = one << (31 + L);
+  f.m = (uint32_t)((num + d - 1) / d);
+  f.s = L - 1;
+  return f;
+}
+
+int gather_inputs(const char* what, const thx_array* ins, int n_in, const int32_t* dtypes, int flags, int* nd_out,
+                  int64_t* shape, std::vector<View>* views) {
+  if (n_in < 1) return fail(THX_ERR_ARG, "%s: needs at least one input", what);
+  const int nd = ins[0].nd;
+  if (nd < 0 || nd > THX_MAX_ND) return fail(THX_ERR_TYPE, "%s: rank %d is outside 0..%d", what, nd, THX_MAX_ND);
+  for (int d = 0; d < nd; ++d) shape[d] = 1;
+  int owner[THX_MAX_ND];
+  for (int d = 0; d < nd; ++d) owner[d] = -1;
+  for (int i = 0; i < n_in; ++i) {
+    if (ins[i].nd != nd)
+      return fail(THX_ERR_TYPE, "%s: input %d has rank %d, expected %d", what, i, ins[i].nd, nd);
+    if ((ins[i].dtype & ~THX_HOST_SCALAR) != dtypes[i])
+      return fail(THX_ERR_TYPE, "%s: input %d has dtype code %d, the operation was built for %d", what, i,
+                  ins[i].dtype & ~THX_HOST_SCALAR, dtypes[i]);
+    for (int d = 0; d < nd; ++d) {
+      const int64_t s = ins[i].shape[d];
+      if (s < 0) return fail(THX_ERR_ARG, "%s: negative extent", what);
+      if (owner[d] < 0) {
+        shape[d] = s;
+        owner[d] = i;
+      } else if (s != shape[d]) {
+        const bool can = (flags & THX_BROADCAST) != 0;
+        if (can && shape[d] == 1) {
+          shape[d] = s;
+          owner[d] = i;
+        } else if (!(can && s == 1)) {
+          return fail(THX_ERR_SHAPE,
+                      "Input dimension mis-match. (input[%d].shape[%d] = %lld, input[%d].shape[%d] = %lld)",
+                      owner[d], d, (long long)shape[d], i, d, (long long)s);
+        }
+      }
+    }
+  }
+  views->assign(n_in, View());
+  for (int i = 0; i < n_in; ++i) {
+    View& v = (*views)[i];
+    v.ptr = (char*)ins[i].base + ins[i].offset_bytes;
+    v.dtype = ins[i].dtype & ~THX_HOST_SCALAR;
+    const int isz = dtype_size(v.dtype);
+    if (!isz) return fail(THX_ERR_TYPE, "%s: unknown dtype code %d", what, v.dtype);
+    if (ins[i].dtype & THX_HOST_SCALAR) {
+      for (int d = 0; d < nd; ++d)
+        if (ins[i].shape[d] != 1) return fail(THX_ERR_TYPE, "%s: host scalar input %d must have extent 1 everywhere", what, i);
+      if (!v.ptr) return fail(THX_ERR_ARG, "%s: host scalar input %d is null", what, i);
+      v.imm = true;
+      memcpy(&v.immval, v.ptr, (size_t)isz);
+      v.ptr = nullptr;
+      continue;
+    }
+    if (((uintptr_t)v.ptr) % isz)
+      return fail(THX_ERR_TYPE, "%s: input %d is not aligned to its element size", what, i);
+    for (int d = 0; d < nd; ++d) {
+      if (ins[i].shape[d] == 1 && shape[d] != 1) {
+        v.stride[d] = 0;
+      } else {
+        if (ins[i].strides_bytes[d] % isz)
+          return fail(THX_ERR_TYPE, "%s: input %d stride %lld is not a multiple of its element size", what, i,
+                      (long long)ins[i].strides_bytes[d]);
+        v.stride[d] = ins[i].strides_bytes[d] / isz;
+      }
+    }
+  }
+  *nd_out = nd;
+  return THX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// hipRTC
+static uint64_t fnv1a(const std::string& s, uint64_t h) {
+  for (unsigned char c : s) {
+    h ^= c;
+    h *= 1099511628211ULL;
+  }
+  return h;
+}
+
+static std::string source_hash(const std::string& src, const std::string& arch) {
+  int maj = 0, min = 0;
+  hiprtcVersion(&maj, &min);
+  std::string salted = src + "\n//" + arch + "/" + std::to_string(maj) + "." + std::to_string(min);
+  char buf[40];
+  snprintf(buf, sizeof buf, "%016llx%016llx", (unsigned long long)fnv1a(salted, 1469598103934665603ULL),
+           (unsigned long long)fnv1a(salted, 0x9e3779b97f4a7c15ULL));
+  return buf;
+}
+
+static const std::string& cache_dir() {
+  if (!g_cache_dir_set) {
+    const char* env = getenv("THX_CACHE_DIR");
+    if (env) {
+      g_cache_dir = env;
+    } else {
+      const char* home = getenv("HOME");
+      g_cache_dir = std::string(home ? home : "/tmp") + "/.cache/thx_hip";
+    }
+    g_cache_dir_set = true;
+  }
+  return g_cache_dir;
+}
+
+static void mkdirs(const std::string& path) {
+  std::string cur;
+  for (size_t i = 0; i <= path.size(); ++i) {
+    if (i == path.size() || path[i] == '/') {
+      if (!cur.empty()) mkdir(cur.c_str(), 0777);
+    }
+    if (i < path.size()) cur += path[i];
+  }
+}
+
+static std::string target_arch() {
+  if (rt().ready) return rt().arch_base;
+  const char* env = getenv("THX_ARCH");
+  return env ? env : "gfx950";
+}
+
+static int compile_source(const std::string& src, const std::string& arch, std::vector<char>* code) {
+  hiprtcProgram prog;
+  hiprtcResult r = hiprtcCreateProgram(&prog, src.c_str(), "thx_kernel.hip", 0, nullptr, nullptr);
+  if (r != HIPRTC_SUCCESS) return fail(THX_ERR_HIP, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+  const std::string archopt = "--offload-arch=" + arch;
+  // Packed FP32 instructions are disabled for every kernel of this library.
+  const char* opts[] = {archopt.c_str(), "-O3",     "-std=c++17",      "-Xclang",
+                        "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  r = hiprtcCompileProgram(prog, (int)(sizeof opts / sizeof opts[0]), opts);
+  if (r != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, &log[0]);
+    hiprtcDestroyProgram(&prog);
+    if (log.size() > 3500) log.resize(3500);
+    return fail(THX_ERR_COMPILE, "hipRTC compilation failed (%s):\n%s", hiprtcGetErrorString(r), log.c_str());
+  }
+  size_t n = 0;
+  hiprtcGetCodeSize(prog, &n);
+  code->resize(n);
+  hiprtcGetCode(prog, code->data());
+  hiprtcDestroyProgram(&prog);
+  return THX_OK;
+}
+
+int get_kernel(const std::string& source, const std::string& entry, Kernel* out) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  const std::string arch = target_arch();
+  const std::string h = source_hash(source, arch);
+  const bool have_device = rt().ready;
+  if (have_device) {
+    auto it = g_kernels.find(h);
+    if (it != g_kernels.end()) {
+      ++g_n_mem;
+      *out = it->second;
+      return THX_OK;
+    }
+  }
+  std::vector<char> code;
+  const std::string& dir = cache_dir();
+  const std::string path = dir.empty() ? "" : dir + "/" + h + ".hsaco";
+  if (!path.empty()) {
+    std::ifstream f(path, std::ios::binary);
+    if (f) {
+      code.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+      if (!code.empty()) ++g_n_disk;
+    }
+  }
+  if (code.empty()) {
+    int rc = compile_source(source, arch, &code);
+    if (rc) return rc;
+    ++g_n_compiled;
+    if (!path.empty()) {
+      mkdirs(dir);
+      const std::string tmp = path + ".tmp" + std::to_string((long)getpid());
+      std::ofstream f(tmp, std::ios::binary);
+      if (f) {
+        f.write(code.data(), (std::streamsize)code.size());
+        f.close();
+        if (rename(tmp.c_str(), path.c_str()) != 0) unlink(tmp.c_str());
+      }
+    }
+  }
+  if (!have_device) {  // dry run: the code object is compiled and cached only
+    *out = Kernel();
+    return THX_OK;
+  }
+  Kernel k;
+  THX_HIP_CHECK(hipModuleLoadData(&k.module, code.data()));
+  THX_HIP_CHECK(hipModuleGetFunction(&k.func, k.module, entry.c_str()));
+  g_kernels[h] = k;
+  *out = k;
+  return THX_OK;
+}
+
+int launch(const Kernel& k, const std::string& plan, unsigned grid, unsigned block, const void* params,
+           size_t params_bytes) {
+  if (!k.func) return fail(THX_ERR_HIP, "launch of '%s' without a loaded kernel", plan.c_str());
+  if (params_bytes > 4096)
+    return fail(THX_ERR_UNSUPPORTED, "kernel '%s' needs %zu bytes of arguments (limit 4096)", plan.c_str(),
+                params_bytes);
+  void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(params), HIP_LAUNCH_PARAM_BUFFER_SIZE,
+                   &params_bytes, HIP_LAUNCH_PARAM_END};
+  Runtime& r = rt();
+  ProfRec rec;
+  if (g_profiling) {
+    rec.plan = plan;
+    THX_HIP_CHECK(hipEventCreate(&rec.a));
+    THX_HIP_CHECK(hipEventCreate(&rec.b));
+    THX_HIP_CHECK(hipEventRecord(rec.a, r.stream));
+  }
+  THX_HIP_CHECK(hipModuleLaunchKernel(k.func, grid, 1, 1, block, 1, 1, 0, r.stream, nullptr, extra));
+  if (g_profiling) {
+    THX_HIP_CHECK(hipEventRecord(rec.b, r.stream));
+    g_prof.push_back(rec);
+  }
+  return THX_OK;
+}
+
+__global__ void thx_fill_kernel(unsigned char* dst, unsigned char value, size_t n) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x * 16;
+  for (size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 16; i < n; i += stride) {
+    if (i + 16 <= n && (((uintptr_t)(dst + i)) & 15) == 0) {
+      const unsigned w = value * 0x01010101u;
+      *(uint4*)(dst + i) = make_uint4(w, w, w, w);
+    } else {
+      for (size_t j = i; j < n && j < i + 16; ++j) dst[j] = value;
+    }
+  }
+}
+
+}  // namespace thx
+
+using namespace thx;
+
+// ---------------------------------------------------------------------------
+// C ABI
+extern "C" {
+
+const char* thx_last_error(void) { return g_error.c_str(); }
+const char* thx_last_plan(void) { return g_plan.c_str(); }
+
+int thx_init(int device) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  return init_locked(device);
+}
+
+int thx_device_info(char* arch, size_t arch_cap, int* compute_units, int64_t* hbm_bytes) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  if (arch && arch_cap) snprintf(arch, arch_cap, "%s", rt().arch.c_str());
+  if (compute_units) *compute_units = rt().cus;
+  if (hbm_bytes) *hbm_bytes = rt().hbm;
+  return THX_OK;
+}
+
+int thx_alloc(size_t nbytes, void** out) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  std::lock_guard<std::mutex> lk(g_mu);
+  const size_t sz = nbytes ? (nbytes + 511) / 512 * 512 : 512;
+  auto it = g_free.find(sz);
+  if (it != g_free.end() && !it->second.empty()) {
+    *out = it->second.back();
+    it->second.pop_back();
+    g_live[*out] = sz;
+    return THX_OK;
+  }
+  void* p = nullptr;
+  hipError_t e = hipMalloc(&p, sz);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize(rt().stream);
+    for (auto& kv : g_free) {
+      for (void* q : kv.second) (void)hipFree(q);
+      kv.second.clear();
+    }
+    e = hipMalloc(&p, sz);
+  }
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return fail(THX_ERR_MEMORY, "device allocation of %zu bytes failed: %s", sz, hipGetErrorString(e));
+  }
+  g_live[p] = sz;
+  *out = p;
+  return THX_OK;
+}
+
+int thx_free(void* ptr) {
+  if (!ptr) return THX_OK;
+  std::lock_guard<std::mutex> lk(g_mu);
+  auto it = g_live.find(ptr);
+  if (it == g_live.end()) return fail(THX_ERR_ARG, "thx_free: %p was not allocated by thx_alloc", ptr);
+  g_free[it->second].push_back(ptr);
+  g_live.erase(it);
+  return THX_OK;
+}
+
+int thx_pool_trim(void) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (!rt().ready) return THX_OK;
+  THX_HIP_CHECK(hipStreamSynchronize(rt().stream));
+  for (auto& kv : g_free) {
+    for (void* q : kv.second) THX_HIP_CHECK(hipFree(q));
+    kv.second.clear();
+  }
+  return THX_OK;
+}
+
+int thx_h2d(void* dst, const void* src, size_t nbytes) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  if (!nbytes) return THX_OK;
+  THX_HIP_CHECK(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, rt().stream));
+  THX_HIP_CHECK(hipStreamSynchronize(rt().stream));  // the host buffer may be pageable and reused at once
+  return THX_OK;
+}
+
+int thx_d2h(void* dst, const void* src, size_t nbytes) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  if (!nbytes) return THX_OK;
+  THX_HIP_CHECK(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, rt().stream));
+  THX_HIP_CHECK(hipStreamSynchronize(rt().stream));
+  return THX_OK;
+}
+
+int thx_d2d(void* dst, const void* src, size_t nbytes) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  if (!nbytes) return THX_OK;
+  THX_HIP_CHECK(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToDevice, rt().stream));
+  return THX_OK;
+}
+
+int thx_fill_bytes(void* dst, int value, size_t nbytes) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  if (!nbytes) return THX_OK;
+  size_t blocks = (nbytes / 16 + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(thx_fill_kernel, dim3((unsigned)blocks), dim3(256), 0, rt().stream, (unsigned char*)dst,
+                     (unsigned char)value, nbytes);
+  THX_HIP_CHECK(hipGetLastError());
+  return THX_OK;
+}
+
+int thx_sync(void) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  THX_HIP_CHECK(hipStreamSynchronize(rt().stream));
+  return THX_OK;
+}
+
+int thx_set_cache_dir(const char* path) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  g_cache_dir = path ? path : "";
+  g_cache_dir_set = true;
+  return THX_OK;
+}
+
+int thx_cache_stats(int64_t* compiled, int64_t* disk_hits, int64_t* mem_hits) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (compiled) *compiled = g_n_compiled;
+  if (disk_hits) *disk_hits = g_n_disk;
+  if (mem_hits) *mem_hits = g_n_mem;
+  return THX_OK;
+}
+
+int thx_profile_begin(void) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  g_prof.clear();
+  g_profiling = true;
+  return THX_OK;
+}
+
+int thx_profile_end(char* buf, size_t cap) {
+  if (!g_profiling) return fail(THX_ERR_ARG, "thx_profile_end without thx_profile_begin");
+  g_profiling = false;
+  THX_HIP_CHECK(hipStreamSynchronize(rt().stream));
+  std::vector<std::string> order;
+  std::unordered_map<std::string, std::pair<long, double>> agg;
+  for (ProfRec& r : g_prof) {
+    float ms = 0;
+    THX_HIP_CHECK(hipEventElapsedTime(&ms, r.a, r.b));
+    (void)hipEventDestroy(r.a);
+    (void)hipEventDestroy(r.b);
+    auto it = agg.find(r.plan);
+    if (it == agg.end()) {
+      order.push_back(r.plan);
+      agg[r.plan] = {1, ms};
+    } else {
+      it->second.first += 1;
+      it->second.second += ms;
+    }
+  }
+  g_prof.clear();
+  std::ostringstream os;
+  for (const std::string& p : order) {
+    char line[64];
+    snprintf(line, sizeof line, "\t%ld\t%.6f\n", agg[p].first, agg[p].second);
+    os << p << line;
+  }
+  const std::string s = os.str();
+  if (s.size() + 1 > cap) return fail(THX_ERR_ARG, "thx_profile_end: buffer of %zu bytes, need %zu", cap, s.size() + 1);
+  memcpy(buf, s.c_str(), s.size() + 1);
+  return THX_OK;
+}
+
+int thx_timer_start(void) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  THX_HIP_CHECK(hipEventRecord(g_t0, rt().stream));
+  return THX_OK;
+}
+
+int thx_timer_stop(float* elapsed_ms) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  THX_HIP_CHECK(hipEventRecord(g_t1, rt().stream));
+  THX_HIP_CHECK(hipEventSynchronize(g_t1));
+  THX_HIP_CHECK(hipEventElapsedTime(elapsed_ms, g_t0, g_t1));
+  return THX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,175 @@
+"""Device source for the functors the kernel templates are instantiated with.
+
+From a ScalarOp (usually a ``Composite``) and operand dtypes this emits the
+struct described in ``csrc/kernels/thx_elemwise.h`` / ``thx_reduce.h``: operand
+registers, loads, the per-element statements and stores.  The role is that of
+``_generate_op_string`` (``theano/gpuarray/elemwise.py:153-200``) and of the
+kernel bodies assembled in ``GpuCAReduceCuda`` (``:969-1093``): everything
+per-element comes from ``scalar_op.c_code``.
+"""
+import hashlib
+
+import numpy as np
+
+from .. import scalar as scal
+from ..gof import Apply
+from ..scalar import Scalar, c_literal, compute_ctype, storage_ctype
+
+
+def _scalar_node(op, in_dtypes):
+    return op.make_node(*[Scalar(dt)() for dt in in_dtypes])
+
+
+def _indent(text, n):
+    pad = " " * n
+    return "\n".join(pad + l if l.strip() else l for l in text.splitlines())
+
+
+def _name(prefix, text):
+    return prefix + hashlib.sha1(text.encode()).hexdigest()[:16]
+
+
+def _regs(dtypes, names):
+    return "  template <int V> struct Regs { %s };\n" % " ".join(
+        "thx::Vec<%s, V> %s;" % (storage_ctype(dt), nm) for dt, nm in zip(dtypes, names))
+
+
+def elemwise_functor(scalar_op, in_dtypes, out_dtypes=None):
+    """(source, functor name, output dtypes) for an n-ary elementwise op."""
+    node = _scalar_node(scalar_op, in_dtypes)
+    odt = [o.type.dtype for o in node.outputs]
+    if out_dtypes is not None and list(out_dtypes) != odt:
+        raise TypeError("scalar op gives %s, node expects %s" % (odt, list(out_dtypes)))
+    nin, nout = len(in_dtypes), len(odt)
+    ins = ["i%d" % k for k in range(nin)]
+    outs = ["o%d" % k for k in range(nout)]
+    stmt = scalar_op.c_code(node, ins, outs)
+    params = ", ".join(["const %s %s" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)] +
+                       ["%s& %s" % (compute_ctype(dt), nm) for dt, nm in zip(odt, outs)])
+    body = []
+    body.append("  enum { NIN = %d, NOUT = %d, NOPS = %d };" % (nin, nout, nin + nout))
+    body.append(_regs(list(in_dtypes) + odt, ins + outs).rstrip("\n"))
+    body.append("  template <int V, class A> THX_DEV static void load(const A& a, Regs<V>& r) { %s }" % " ".join(
+        "a.template ld<%d>(r.%s);" % (k, nm) for k, nm in enumerate(ins)))
+    body.append("  THX_DEV static void apply(%s) {\n%s\n  }" % (params, _indent(stmt, 4)))
+    call = ", ".join(["(%s)r.%s.v[k]" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)] +
+                     ["t_%s" % nm for nm in outs])
+    decl = " ".join("%s t_%s;" % (compute_ctype(dt), nm) for dt, nm in zip(odt, outs))
+    back = " ".join("r.%s.v[k] = (%s)t_%s;" % (nm, storage_ctype(dt), nm) for dt, nm in zip(odt, outs))
+    body.append("  template <int V> THX_DEV static void compute(Regs<V>& r) {\n#pragma unroll\n"
+                "    for (int k = 0; k < V; ++k) { %s apply(%s); %s }\n  }" % (decl, call, back))
+    body.append("  template <int V, class A> THX_DEV static void store(const A& a, const Regs<V>& r) { %s }" % " ".join(
+        "a.template st<%d>(r.%s);" % (nin + k, nm) for k, nm in enumerate(outs)))
+    text = "\n".join(body)
+    name = _name("F", text)
+    return "struct %s {\n%s\n};\n" % (name, text), name, odt
+
+
+# --------------------------------------------------------------------------
+def reduce_identity(scalar_op, dtype):
+    """Identity element of a reduction op for an accumulator of ``dtype``: the
+    op's own, or the extreme value for max / min
+    (``theano/tensor/elemwise.py:1470-1488``).  None when the op has none."""
+    if isinstance(scalar_op, scal.Minimum):
+        big = True
+    elif isinstance(scalar_op, scal.Maximum):
+        big = False
+    else:
+        if scalar_op.identity is None:
+            return None
+        return c_literal(scalar_op.identity, dtype)
+    if dtype in scal.float_dtypes:
+        return c_literal(np.inf if big else -np.inf, dtype)
+    if dtype == "bool":
+        return c_literal(1 if big else 0, dtype)
+    info = np.iinfo(dtype)
+    return c_literal(info.max if big else info.min, dtype)
+
+
+def acc_struct_bytes(acc_dtypes):
+    """sizeof of a struct holding one field per accumulator dtype."""
+    off, align = 0, 1
+    for dt in acc_dtypes:
+        sz = np.dtype("float32" if dt == "float16" else dt).itemsize
+        off = (off + sz - 1) // sz * sz + sz
+        align = max(align, sz)
+    return (off + align - 1) // align * align
+
+
+def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, post_op=None):
+    """(source, name, sizeof(Acc)) for K simultaneous reductions.
+
+    Per element, ``pre_op`` (nin = len(in_dtypes), nout = K; default: the single
+    input itself) yields K values, each cast to its accumulator dtype and
+    folded with ``scalar_ops[k]``.  ``post_op`` (nin = K) maps the K results to
+    the outputs; the default casts result k to ``out_dtypes[k]``."""
+    K = len(scalar_ops)
+    nin, nout = len(in_dtypes), len(out_dtypes)
+    ins = ["i%d" % k for k in range(nin)]
+    acc_c = [compute_ctype(dt) for dt in acc_dtypes]
+    lines = ["  enum { NIN = %d, NOUT = %d };" % (nin, nout)]
+    lines.append("  struct Acc { %s };" % " ".join("%s a%d;" % (c, k) for k, c in enumerate(acc_c)))
+    lines.append(_regs(in_dtypes, ins).rstrip("\n"))
+    init = []
+    for k, (op, dt) in enumerate(zip(scalar_ops, acc_dtypes)):
+        ident = reduce_identity(op, dt)
+        if ident is None:
+            raise NotImplementedError("reduction with %s has no identity element" % op)
+        init.append("a.a%d = %s;" % (k, ident))
+    lines.append("  THX_DEV static void init(Acc& a) { %s }" % " ".join(init))
+    lines.append("  template <int V, class A> THX_DEV static void load(const A& a, Regs<V>& r) { %s }" % " ".join(
+        "a.template ld<%d>(r.%s);" % (k, nm) for k, nm in enumerate(ins)))
+    # prologue
+    if pre_op is None:
+        if nin != 1 or K != 1:
+            raise ValueError("a reduction without prologue takes one input and one accumulator")
+        pre_stmt = "v.a0 = (%s)i0;" % acc_c[0]
+    else:
+        pnode = _scalar_node(pre_op, in_dtypes)
+        if len(pnode.outputs) != K:
+            raise ValueError("prologue yields %d values for %d reductions" % (len(pnode.outputs), K))
+        tmp = ["p%d" % k for k in range(K)]
+        pre_stmt = " ".join("%s %s;" % (compute_ctype(o.type.dtype), t) for o, t in zip(pnode.outputs, tmp))
+        pre_stmt += "\n" + pre_op.c_code(pnode, ins, tmp) + "\n"
+        pre_stmt += " ".join("v.a%d = (%s)%s;" % (k, acc_c[k], t) for k, t in enumerate(tmp))
+    lines.append("  THX_DEV static void pre(%s, Acc& v) {\n%s\n  }" % (
+        ", ".join("const %s %s" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)), _indent(pre_stmt, 4)))
+    # combine: the reduction op applied to two accumulator-typed values
+    comb = []
+    for k, (op, dt) in enumerate(zip(scalar_ops, acc_dtypes)):
+        cnode = Apply(op, [Scalar(dt)(), Scalar(dt)()], [Scalar(dt)()])
+        comb.append(op.c_code(cnode, ["a.a%d" % k, "b.a%d" % k], ["a.a%d" % k]))
+    lines.append("  THX_DEV static void comb(Acc& a, const Acc& b) {\n%s\n  }" % _indent("\n".join(comb), 4))
+    call = ", ".join("(%s)r.%s.v[k]" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins))
+    lines.append("  template <int V> THX_DEV static void accum(Acc& s, const Regs<V>& r) {\n#pragma unroll\n"
+                 "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s, t); }\n  }" % call)
+    lines.append("  template <int V> THX_DEV static void accum_lanes(Acc* s, const Regs<V>& r) {\n#pragma unroll\n"
+                 "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s[k], t); }\n  }" % call)
+    lines.append("  THX_DEV static Acc shfl_xor(const Acc& a, int m) { Acc r; %s return r; }" % " ".join(
+        "r.a%d = thx::shfl_xor_t(a.a%d, m);" % (k, k) for k in range(K)))
+    # epilogue
+    if post_op is None:
+        if nout != K:
+            raise ValueError("a reduction without epilogue has one output per accumulator")
+        post = []
+        for k, dt in enumerate(out_dtypes):
+            val = "a.a%d" % k
+            if dt == "bool":
+                val = "(%s ? 1 : 0)" % val
+            post.append("((%s*)o.ptr[%d])[idx] = (%s)%s;" % (storage_ctype(dt), k, storage_ctype(dt), val))
+        post_stmt = "\n".join(post)
+    else:
+        qnode = _scalar_node(post_op, acc_dtypes)
+        if [o.type.dtype for o in qnode.outputs] != list(out_dtypes):
+            raise TypeError("epilogue gives %s, node expects %s" % ([o.type.dtype for o in qnode.outputs],
+                                                                      list(out_dtypes)))
+        tmp = ["q%d" % k for k in range(nout)]
+        post_stmt = " ".join("%s %s;" % (compute_ctype(dt), t) for dt, t in zip(out_dtypes, tmp))
+        post_stmt += "\n" + post_op.c_code(qnode, ["a.a%d" % k for k in range(K)], tmp) + "\n"
+        post_stmt += "\n".join("((%s*)o.ptr[%d])[idx] = (%s)%s;" % (storage_ctype(dt), k, storage_ctype(dt), t)
+                               for k, (dt, t) in enumerate(zip(out_dtypes, tmp)))
+    lines.append("  template <class O> THX_DEV static void post(const O& o, long long idx, const Acc& a) {\n%s\n  }"
+                 % _indent(post_stmt, 4))
+    text = "\n".join(lines)
+    name = _name("R", text)
+    return "struct %s {\n%s\n};\n" % (name, text), name, acc_struct_bytes(acc_dtypes)

@@ -1,0 +1,393 @@
+"""The HIP Op family: device type, transfers and the lifted Elemwise /
+DimShuffle / CAReduce ops.
+
+Each op subclasses its host counterpart and overrides ``make_node`` (device
+types) and ``perform`` (one ctypes call), the arrangement the reference uses
+for ``GpuElemwise(HideC, Elemwise)`` (``theano/gpuarray/elemwise.py:86-396``),
+``GpuDimShuffle`` (:406-446) and ``GpuCAReduceCuda`` (:449-2420); the type and
+transfer ops follow ``theano/gpuarray/type.py:129-517`` and
+``theano/gpuarray/basic_ops.py:565-744``.
+"""
+import ctypes
+
+import numpy as np
+
+from .. import scalar as scal
+from ..gof import Apply, Op, Type, Variable
+from ..tensor.elemwise import CAReduce, DimShuffle, Elemwise
+from ..tensor.type import TensorType, _tensor_py_operators
+from . import codegen
+from .runtime import HipArray, call_flags, check, host_scalar_thx, lib, thx_array
+
+
+class HipArrayType(Type):
+    """dtype and broadcast pattern of an array living in device memory."""
+
+    def __init__(self, dtype, broadcastable, name=None):
+        self.dtype = str(dtype)
+        if self.dtype not in scal.all_dtypes:
+            raise TypeError("Unsupported dtype for HipArrayType: %s" % self.dtype)
+        self.broadcastable = tuple(bool(b) for b in broadcastable)
+        self.ndim = len(self.broadcastable)
+        self.name = name
+
+    def clone(self, dtype=None, broadcastable=None):
+        return type(self)(self.dtype if dtype is None else dtype,
+                          self.broadcastable if broadcastable is None else broadcastable)
+
+    def filter(self, data, strict=False, allow_downcast=None):
+        if not isinstance(data, HipArray):
+            if strict:
+                raise TypeError("%s expected a HipArray, got %s" % (self, type(data)))
+            data = HipArray.from_numpy(TensorType(self.dtype, self.broadcastable).filter(
+                data, strict=False, allow_downcast=allow_downcast))
+        if str(data.dtype) != self.dtype:
+            raise TypeError("%s cannot hold a HipArray of dtype %s" % (self, data.dtype))
+        if data.ndim != self.ndim:
+            raise TypeError("Wrong number of dimensions: expected %s, got %s with shape %s." %
+                            (self.ndim, data.ndim, data.shape))
+        for i, b in enumerate(self.broadcastable):
+            if b and data.shape[i] != 1:
+                raise TypeError("Non-unit value on shape on a broadcastable dimension.", data.shape,
+                                self.broadcastable)
+        return data
+
+    def __eq__(self, other):
+        return (type(self) is type(other) and self.dtype == other.dtype and
+                self.broadcastable == other.broadcastable)
+
+    def __hash__(self):
+        return hash((type(self), self.dtype, self.broadcastable))
+
+    def __str__(self):
+        return "HipArrayType(%s, %s)" % (self.dtype, self.broadcastable)
+
+    __repr__ = __str__
+
+    def as_tensor_variable(self, var):
+        return host_from_hip(var)
+
+
+class HipArrayVariable(_tensor_py_operators, Variable):
+    pass
+
+
+HipArrayType.Variable = HipArrayVariable
+
+
+def _is_host_scalar(var):
+    """A host tensor whose every dimension is broadcastable travels as a
+    kernel argument instead of being copied to the device."""
+    return isinstance(var.type, TensorType) and all(var.type.broadcastable)
+
+
+def as_hip_variable(x):
+    """Device version of ``x``; a transfer of a transfer is short-circuited
+    (``theano/gpuarray/basic_ops.py:37-98``)."""
+    if isinstance(x, Variable) and isinstance(x.type, HipArrayType):
+        return x
+    if isinstance(x, Variable) and isinstance(x.type, TensorType):
+        if x.owner is not None and isinstance(x.owner.op, HipToHost):
+            return x.owner.inputs[0]
+        return hip_from_host(x)
+    from ..tensor.type import as_tensor_variable
+    return hip_from_host(as_tensor_variable(x))
+
+
+class HostToHip(Op):
+    __props__ = ()
+
+    def make_node(self, x):
+        if not isinstance(x.type, TensorType):
+            raise TypeError("HostToHip takes a host tensor", x)
+        return Apply(self, [x], [HipArrayType(x.type.dtype, x.type.broadcastable)()])
+
+    def perform(self, node, inputs, output_storage):
+        x = inputs[0]
+        output_storage[0][0] = x if isinstance(x, HipArray) else HipArray.from_numpy(x)
+
+    def infer_shape(self, node, shapes):
+        return shapes
+
+    def grad(self, inputs, grads):
+        return [host_from_hip(as_hip_variable(grads[0]))]
+
+    def __str__(self):
+        return "HostToHip"
+
+
+class HipToHost(Op):
+    __props__ = ()
+
+    def make_node(self, x):
+        if not isinstance(x.type, HipArrayType):
+            raise TypeError("HipToHost takes a device array", x)
+        return Apply(self, [x], [TensorType(x.type.dtype, x.type.broadcastable)()])
+
+    def perform(self, node, inputs, output_storage):
+        output_storage[0][0] = inputs[0].to_numpy()
+
+    def infer_shape(self, node, shapes):
+        return shapes
+
+    def grad(self, inputs, grads):
+        return [as_hip_variable(grads[0])]
+
+    def __str__(self):
+        return "HipToHost"
+
+
+hip_from_host = HostToHip()
+host_from_hip = HipToHost()
+
+
+class HipDimShuffle(DimShuffle):
+    """DimShuffle of a device array: a new (shape, strides) header over the
+    same buffer, computed like ``theano/tensor/c_code/dimshuffle.c:55-98``."""
+
+    def make_node(self, input):
+        input = as_hip_variable(input)
+        host = DimShuffle.make_node(self, TensorType(input.type.dtype, input.type.broadcastable)())
+        ot = host.outputs[0].type
+        return Apply(self, [input], [HipArrayType(ot.dtype, ot.broadcastable)()])
+
+    def __str__(self):
+        return "HipDimShuffle{%s}" % ",".join(str(x) for x in self.new_order)
+
+    def perform(self, node, inputs, output_storage):
+        (x,) = inputs
+        if x.ndim != len(self.input_broadcastable):
+            raise TypeError("input has %d dimensions, DimShuffle was built for %d" %
+                            (x.ndim, len(self.input_broadcastable)))
+        for d in self.drop:
+            if x.shape[d] != 1:
+                raise ValueError("cannot drop dimension %d of extent %d" % (d, x.shape[d]))
+        shape, strides = [], []
+        for v in self.new_order:
+            if v == "x":
+                shape.append(1)
+                strides.append(0)
+            else:
+                shape.append(x.shape[v])
+                strides.append(x.strides[v])
+        # extent-1 dimensions get the stride a C-contiguous array would have
+        for i in range(len(shape) - 1, -1, -1):
+            if shape[i] == 1:
+                strides[i] = x.dtype.itemsize if i == len(shape) - 1 else strides[i + 1] * shape[i + 1]
+        output_storage[0][0] = x.view(shape, strides)
+
+
+def _operand(value, nd, slot):
+    if isinstance(value, HipArray):
+        return value.as_thx(slot)
+    return host_scalar_thx(value, nd, slot)
+
+
+def _check_runtime_broadcast(node_inputs, values, nd):
+    """Non-broadcastable dimensions must agree exactly; an extent of 1 only
+    broadcasts where the type says so (``theano/tensor/elemwise.py:720-740``)."""
+    shape = [1] * nd
+    owner = [None] * nd
+    for k, (var, val) in enumerate(zip(node_inputs, values)):
+        if not isinstance(val, HipArray):
+            if not isinstance(val, np.ndarray) or val.size != 1:
+                raise TypeError("input %d must be a device array or a one-element host array" % k)
+            continue
+        if val.ndim != nd:
+            raise TypeError("input %d has rank %d, expected %d" % (k, val.ndim, nd))
+        vshape = val.shape
+        for d in range(nd):
+            if var.type.broadcastable[d]:
+                if vshape[d] != 1:
+                    raise ValueError("input %d has extent %d on a broadcastable dimension %d" % (k, vshape[d], d))
+                continue
+            if owner[d] is None:
+                owner[d], shape[d] = k, vshape[d]
+            elif vshape[d] != shape[d]:
+                raise ValueError("Input dimension mis-match. (input[%d].shape[%d] = %d, input[%d].shape[%d] = %d)" %
+                                 (owner[d], d, shape[d], k, d, vshape[d]))
+    return tuple(shape)
+
+
+_elemwise_handles = {}
+_reduce_handles = {}
+
+
+class HipElemwise(Elemwise):
+    """Elemwise executed by one fused kernel.  Inputs are device arrays, or host
+    tensors broadcastable in every dimension, which are passed by value."""
+
+    def make_node(self, *inputs):
+        from ..tensor.type import as_tensor_variable
+        ins = []
+        for i in inputs:
+            if not isinstance(i, Variable):
+                i = as_tensor_variable(i)
+            if isinstance(i.type, HipArrayType) or _is_host_scalar(i):
+                ins.append(i)
+            else:
+                ins.append(as_hip_variable(i))
+        shadow = [TensorType(i.type.dtype, i.type.broadcastable)() for i in ins]
+        out_dtypes, out_b, shadow2 = self.get_output_info(DimShuffle, *shadow)
+        # rank alignment, mirrored on the real inputs
+        target = max(i.type.ndim for i in ins)
+        aligned = []
+        for i in ins:
+            diff = target - i.type.ndim
+            if diff and isinstance(i.type, HipArrayType):
+                i = HipDimShuffle(i.type.broadcastable, ["x"] * diff + list(range(i.type.ndim)))(i)
+            aligned.append(i)  # host scalars are passed by value whatever their rank
+        if len(out_dtypes) < 1:
+            raise NotImplementedError("an Elemwise needs at least one output")
+        outputs = [HipArrayType(dt, b)() for dt, b in zip(out_dtypes, out_b)]
+        return Apply(self, aligned, outputs)
+
+    def _handle(self, node):
+        in_dt = tuple(i.type.dtype for i in node.inputs)
+        key = (self.scalar_op, in_dt)
+        h = _elemwise_handles.get(key)
+        if h is None:
+            src, name, out_dt = codegen.elemwise_functor(self.scalar_op, in_dt, [o.type.dtype for o in node.outputs])
+            codes = (ctypes.c_int32 * (len(in_dt) + len(out_dt)))(*[scal.dtype_code(d) for d in in_dt + tuple(out_dt)])
+            handle = ctypes.c_void_p()
+            check(lib.thx_elemwise_new(src.encode(), name.encode(), len(in_dt), len(out_dt), codes,
+                                       ctypes.byref(handle)))
+            h = (handle, len(in_dt), len(out_dt))
+            _elemwise_handles[key] = h
+        return h
+
+    def perform(self, node, inputs, output_storage):
+        flags = call_flags()
+        handle, nin, nout = self._handle(node)
+        nd = node.outputs[0].type.ndim
+        shape = _check_runtime_broadcast(node.inputs, inputs, nd)
+        ins = (thx_array * nin)()
+        for k, v in enumerate(inputs):
+            _operand(v, nd, ins[k])
+        outs = (thx_array * nout)()
+        results = []
+        inplace = dict(self.inplace_pattern)
+        for k, o in enumerate(node.outputs):
+            if k in inplace:
+                arr = inputs[inplace[k]]
+                if arr.shape != shape:
+                    raise ValueError("in-place output %d has shape %s, the result has %s" % (k, arr.shape, shape))
+            else:
+                arr = HipArray.empty(shape, o.type.dtype)
+            arr.as_thx(outs[k])
+            results.append(arr)
+        check(lib.thx_elemwise_call(handle, ins, outs, flags))
+        for k, arr in enumerate(results):
+            output_storage[k][0] = arr
+
+
+class HipCAReduce(CAReduce):
+    """K simultaneous reductions over the same axes in one pass.
+
+    ``scalar_ops[k]`` folds, in ``acc_dtypes[k]``, the k-th value produced per
+    element by ``pre_scalar_op`` applied to the inputs (None: the single input
+    itself).  ``post_scalar_op`` maps the K results to the outputs (None: cast
+    result k to ``out_dtypes[k]``).  A lifted ``CAReduce`` is the K = 1 case
+    without prologue or epilogue; the fusion pass widens it.  The generalisation
+    of ``GpuCAReduceCuda``'s ``pre_scalar_op`` (``theano/gpuarray/elemwise.py:492-493``)."""
+
+    __props__ = ("scalar_ops", "axis", "acc_dtypes", "out_dtypes", "pre_scalar_op", "post_scalar_op")
+
+    def __init__(self, scalar_ops, axis, acc_dtypes, out_dtypes, pre_scalar_op=None, post_scalar_op=None):
+        scalar_ops = tuple(scalar_ops)
+        for op in scalar_ops:
+            if op.nin not in (-1, 2) or op.nout != 1:
+                raise NotImplementedError("CAReduce only supports binary functions with a single output.")
+        self.scalar_ops = scalar_ops
+        self.scalar_op = scalar_ops[0]
+        if axis is None:
+            self.axis = None
+        elif isinstance(axis, (int, np.integer)):
+            self.axis = (int(axis),)
+        else:
+            self.axis = tuple(sorted(set(int(a) for a in axis)))
+        self.acc_dtypes = tuple(acc_dtypes)
+        self.out_dtypes = tuple(out_dtypes)
+        self.pre_scalar_op = pre_scalar_op
+        self.post_scalar_op = post_scalar_op
+        if len(self.acc_dtypes) != len(scalar_ops):
+            raise ValueError("one accumulator dtype per reduction")
+
+    def _props(self):
+        return (self.scalar_ops, self.axis, self.acc_dtypes, self.out_dtypes, self.pre_scalar_op, self.post_scalar_op)
+
+    def __str__(self):
+        ops = ",".join(str(o) for o in self.scalar_ops)
+        ax = "" if self.axis is None else "{%s}" % ", ".join(str(a) for a in self.axis)
+        extra = ""
+        if self.pre_scalar_op is not None:
+            extra += ", pre=%s" % self.pre_scalar_op
+        if self.post_scalar_op is not None:
+            extra += ", post=%s" % self.post_scalar_op
+        return "HipCAReduce{%s}%s{acc=%s%s}" % (ops, ax, ",".join(self.acc_dtypes), extra)
+
+    def make_node(self, *inputs):
+        ins = [i if (isinstance(i.type, HipArrayType) or _is_host_scalar(i)) else as_hip_variable(i) for i in inputs]
+        nd = max(i.type.ndim for i in ins)
+        if any(i.type.ndim != nd for i in ins if isinstance(i.type, HipArrayType)):
+            raise TypeError("HipCAReduce inputs must share one rank")
+        if self.pre_scalar_op is None and len(ins) != 1:
+            raise TypeError("a reduction without prologue takes exactly one input")
+        axis = self.axis if self.axis is not None else tuple(range(nd))
+        for a in axis:
+            if a >= nd or a < 0:
+                raise ValueError("Not enough dimensions on the input to reduce on axis %s" % a)
+        bcast = [all(b) for b in zip(*[i.type.broadcastable for i in ins if i.type.ndim == nd])]
+        ob = [b for d, b in enumerate(bcast) if d not in axis]
+        return Apply(self, ins, [HipArrayType(dt, ob)() for dt in self.out_dtypes])
+
+    def infer_shape(self, node, shapes):
+        nd = max(i.type.ndim for i in node.inputs)
+        axis = self.axis if self.axis is not None else tuple(range(nd))
+        full = [max(s[d] for s in shapes if len(s) == nd) for d in range(nd)]
+        kept = tuple(full[d] for d in range(nd) if d not in axis)
+        return [kept for _ in node.outputs]
+
+    def _handle(self, node):
+        in_dt = tuple(i.type.dtype for i in node.inputs)
+        key = (self.scalar_ops, self.acc_dtypes, self.out_dtypes, self.pre_scalar_op, self.post_scalar_op, in_dt)
+        h = _reduce_handles.get(key)
+        if h is None:
+            src, name, acc_bytes = codegen.reduce_functor(self.scalar_ops, self.acc_dtypes, in_dt, self.out_dtypes,
+                                                          self.pre_scalar_op, self.post_scalar_op)
+            all_dt = in_dt + self.out_dtypes
+            codes = (ctypes.c_int32 * len(all_dt))(*[scal.dtype_code(d) for d in all_dt])
+            handle = ctypes.c_void_p()
+            check(lib.thx_reduce_new(src.encode(), name.encode(), len(in_dt), len(self.out_dtypes), codes, acc_bytes,
+                                     ctypes.byref(handle)))
+            h = (handle, len(in_dt), len(self.out_dtypes))
+            _reduce_handles[key] = h
+        return h
+
+    def perform(self, node, inputs, output_storage):
+        flags = call_flags()
+        handle, nin, nout = self._handle(node)
+        nd = max(i.type.ndim for i in node.inputs)
+        shape = _check_runtime_broadcast(node.inputs, inputs, nd)
+        axis = self.axis if self.axis is not None else tuple(range(nd))
+        n_red = 1
+        for a in axis:
+            n_red *= shape[a]
+        if n_red == 0:
+            for op in self.scalar_ops:
+                if codegen.reduce_identity(op, "float32") is None or isinstance(op, (scal.Maximum, scal.Minimum)):
+                    raise ValueError("Input of CAReduce{%s} has zero-size on axis %s" % (op, axis))
+        mask = (ctypes.c_uint8 * max(nd, 1))(*[1 if d in axis else 0 for d in range(nd)])
+        ins = (thx_array * nin)()
+        for k, v in enumerate(inputs):
+            _operand(v, nd, ins[k])
+        kept = tuple(shape[d] for d in range(nd) if d not in axis)
+        outs = (thx_array * nout)()
+        results = []
+        for k, dt in enumerate(self.out_dtypes):
+            arr = HipArray.empty(kept, dt)
+            arr.as_thx(outs[k])
+            results.append(arr)
+        check(lib.thx_reduce_call(handle, ins, mask, outs, flags))
+        for k, arr in enumerate(results):
+            output_storage[k][0] = arr

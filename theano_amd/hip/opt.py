@@ -1,0 +1,349 @@
+"""Graph rewrites that move a graph onto the HIP ops and fuse it.
+
+Order: lift every Elemwise / DimShuffle / CAReduce node onto the device ops
+(the job of ``GraphToGPU`` with ``local_gpua_elemwise``, ``local_gpua_dimshuffle``
+and ``local_gpua_careduce``, ``theano/gpuarray/opt.py:325-478, 740-866,
+1194-1286``), fuse chains of elementwise nodes into one ``Composite``
+(``local_elemwise_fusion_op``, ``theano/tensor/opt.py:7071-7313``, registered for
+the GPU op at ``theano/gpuarray/opt.py:842-851``), then fold elementwise
+producers into the reductions that consume them (generalising
+``local_gpu_elemwise_careduce``, ``theano/gpuarray/opt.py:2405-2428``) and merge
+sibling reductions that read the same data.
+"""
+import numpy as np
+
+from .. import gof
+from .. import scalar as scal
+from ..config import config
+from ..gof import Constant, FunctionGraph
+from ..tensor import basic as T
+from ..tensor.elemwise import All, Any, CAReduce, CAReduceDtype, DimShuffle, Elemwise
+from ..tensor.type import TensorConstant, TensorType
+from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipToHost, HostToHip, _is_host_scalar,
+                  as_hip_variable, hip_from_host, host_from_hip)
+from .runtime import HipArray
+
+
+class DeviceConstant(Constant):
+    """A non-scalar constant uploaded once when the function is compiled."""
+
+    def signature(self):
+        return (self.type, id(self.data))
+
+
+HipArrayType.Constant = DeviceConstant
+
+
+def _lift_reduce(node, x):
+    op = node.op
+    idt = x.type.dtype
+    if isinstance(op, CAReduceDtype):
+        acc, out = op._acc_dtype(idt), op._output_dtype(idt)
+    else:
+        acc, out = idt, op._output_dtype(idt)
+        if isinstance(op, (All, Any)):
+            acc = "bool"
+    if acc == "float16":
+        raise NotImplementedError("float16 accumulators are not supported (as theano/tensor/elemwise.py:1395-1398)")
+    return HipCAReduce((op.scalar_op,), op.axis if op.axis is not None else tuple(range(x.type.ndim)),
+                       (acc,), (out,))(x)
+
+
+def lift_to_hip(fgraph):
+    """Return a new FunctionGraph computing the same outputs with device ops.
+    Raises NotImplementedError for an op with no device counterpart: there is
+    no host execution to fall back to."""
+    mapping = {}
+    for i in fgraph.inputs:
+        if isinstance(i.type, TensorType) and not all(i.type.broadcastable):
+            mapping[i] = hip_from_host(i)
+        else:
+            mapping[i] = i
+
+    def mapped(v):
+        if v in mapping:
+            return mapping[v]
+        if isinstance(v, Constant):
+            if isinstance(v.type, TensorType) and not all(v.type.broadcastable):
+                mapping[v] = DeviceConstant(HipArrayType(v.type.dtype, v.type.broadcastable), v.data, name=v.name)
+            else:
+                mapping[v] = v
+            return mapping[v]
+        if v.owner is None and hasattr(v, "container"):  # a shared variable
+            mapping[v] = v
+            return v
+        raise gof.InconsistencyError("variable %s is not computed from the function inputs" % v)
+
+    for node in fgraph.toposort():
+        ins = [mapped(i) for i in node.inputs]
+        op = node.op
+        if isinstance(op, (HipElemwise, HipCAReduce, HipDimShuffle, HostToHip, HipToHost, T.ShapeFloat)):
+            if isinstance(op, HostToHip) and isinstance(ins[0].type, HipArrayType):
+                outs = [ins[0]]
+            elif isinstance(op, HipToHost) and isinstance(ins[0].type, TensorType):
+                outs = [ins[0]]
+            else:
+                outs = op.make_node(*ins).outputs
+        elif isinstance(op, Elemwise):
+            if len(node.outputs) != 1:
+                raise NotImplementedError("multi-output Elemwise cannot be lifted: %s" % op)
+            outs = HipElemwise(op.scalar_op, op.inplace_pattern).make_node(*ins).outputs
+        elif isinstance(op, DimShuffle):
+            if isinstance(ins[0].type, HipArrayType):
+                outs = HipDimShuffle(op.input_broadcastable, op.new_order).make_node(ins[0]).outputs
+            else:
+                outs = op.make_node(ins[0]).outputs  # host scalar: a view on the host
+        elif isinstance(op, CAReduce):
+            x = ins[0]
+            if not isinstance(x.type, HipArrayType):
+                x = as_hip_variable(x)
+            outs = [_lift_reduce(node, x)]
+        else:
+            raise NotImplementedError("%s has no HIP implementation and nothing runs on the host" % op)
+        for o, no in zip(node.outputs, outs):
+            mapping[o] = no
+    new_outputs = []
+    for o in fgraph.outputs:
+        m = mapped(o)
+        want_device = isinstance(o.type, HipArrayType)
+        if isinstance(m.type, HipArrayType) and not want_device:
+            m = host_from_hip(m)
+        elif isinstance(m.type, TensorType) and want_device:
+            m = hip_from_host(m)
+        new_outputs.append(m)
+    return fgraph.rebuild(new_outputs)
+
+
+# --------------------------------------------------------------------------
+def _scalar_constant(var):
+    """The scalar Constant standing for an all-broadcastable tensor constant."""
+    if isinstance(var, TensorConstant) and all(var.type.broadcastable):
+        return scal.ScalarConstant(scal.Scalar(var.type.dtype), np.asarray(var.data).reshape(())[()])
+    return None
+
+
+def _fusable(fgraph, var, out_bcast):
+    node = var.owner
+    return (node is not None and isinstance(node.op, HipElemwise) and len(node.outputs) == 1 and
+            not node.op.inplace_pattern and fgraph.n_clients(var) == 1 and
+            tuple(var.type.broadcastable) == tuple(out_bcast))
+
+
+def _fuse_node(fgraph, node):
+    """Splice single-client elementwise producers of ``node`` into it
+    (acceptance rule of ``theano/tensor/opt.py:7168-7218``)."""
+    if not isinstance(node.op, HipElemwise) or len(node.outputs) != 1 or node.op.inplace_pattern:
+        return None
+    out = node.outputs[0]
+    inputs, s_inputs = [], []
+
+    def scalar_for(v):
+        for t, s in zip(inputs, s_inputs):
+            if t is v:
+                return s
+        s = scal.Scalar(v.type.dtype)()
+        inputs.append(v)
+        s_inputs.append(s)
+        return s
+
+    def arg_for(v):
+        c = _scalar_constant(v)
+        return c if c is not None else scalar_for(v)
+
+    s_args, fused = [], False
+    for i in node.inputs:
+        if _fusable(fgraph, i, out.type.broadcastable):
+            p = i.owner
+            before = len(inputs)
+            args = [arg_for(j) for j in p.inputs]
+            if len(inputs) > config.max_fused_inputs:
+                del inputs[before:], s_inputs[before:]
+                s_args.append(scalar_for(i))
+                continue
+            s_args.append(p.op.scalar_op(*args))
+            fused = True
+        else:
+            c = _scalar_constant(i)
+            if c is not None:
+                s_args.append(c)
+                fused = True
+            else:
+                s_args.append(scalar_for(i))
+    if not fused or not inputs:
+        return None
+    s_out = node.op.scalar_op(*s_args)
+    if s_out.type.dtype != out.type.dtype:
+        return None
+    comp = scal.Composite(s_inputs, [s_out])
+    new_out = HipElemwise(comp)(*inputs)
+    if new_out.type != out.type:
+        return None
+    return new_out
+
+
+def fuse_elemwise(fgraph):
+    """Apply ``_fuse_node`` from the outputs towards the inputs until the graph
+    stops changing (``FusionOptimizer``, ``theano/tensor/opt.py:7328-7386``)."""
+    changed = True
+    total = 0
+    while changed:
+        changed = False
+        for node in reversed(fgraph.toposort()):
+            if node not in fgraph.apply_nodes:
+                continue
+            new_out = _fuse_node(fgraph, node)
+            if new_out is not None:
+                fgraph.replace(node.outputs[0], new_out)
+                changed = True
+                total += 1
+    return total
+
+
+# --------------------------------------------------------------------------
+def _as_composite_inputs(node):
+    """Scalar inputs / tensor inputs of an elementwise node with scalar
+    constants turned into literals."""
+    inputs, s_inputs, args = [], [], []
+    for v in node.inputs:
+        c = _scalar_constant(v)
+        if c is not None:
+            args.append(c)
+            continue
+        for t, s in zip(inputs, s_inputs):
+            if t is v:
+                args.append(s)
+                break
+        else:
+            s = scal.Scalar(v.type.dtype)()
+            inputs.append(v)
+            s_inputs.append(s)
+            args.append(s)
+    return inputs, s_inputs, args
+
+
+def fuse_reduce_prologue(fgraph):
+    """``reduce(f(a, b, ...))`` becomes one reduction whose prologue is f, when
+    nothing else uses f's result."""
+    count = 0
+    for node in fgraph.toposort():
+        op = node.op
+        if not isinstance(op, HipCAReduce) or op.pre_scalar_op is not None or len(op.scalar_ops) != 1:
+            continue
+        x = node.inputs[0]
+        p = x.owner
+        if (p is None or not isinstance(p.op, HipElemwise) or len(p.outputs) != 1 or p.op.inplace_pattern or
+                fgraph.n_clients(x) != 1):
+            continue
+        inputs, s_inputs, args = _as_composite_inputs(p)
+        if not inputs or len(inputs) > config.max_fused_inputs:
+            continue
+        # every device input must carry the full rank of the reduced tensor
+        if any(isinstance(i.type, HipArrayType) and i.type.ndim != x.type.ndim for i in inputs):
+            continue
+        pre = scal.Composite(s_inputs, [p.op.scalar_op(*args)])
+        new = HipCAReduce(op.scalar_ops, op.axis, op.acc_dtypes, op.out_dtypes, pre, op.post_scalar_op)(*inputs)
+        if new.type != node.outputs[0].type:
+            continue
+        fgraph.replace(node.outputs[0], new)
+        count += 1
+    return count
+
+
+def _depends_on(var, node, limit=10000):
+    """True when ``var`` is computed (transitively) from an output of ``node``."""
+    stack, seen = [var], set()
+    while stack and len(seen) < limit:
+        v = stack.pop()
+        if id(v) in seen or v.owner is None:
+            continue
+        seen.add(id(v))
+        if v.owner is node:
+            return True
+        stack.extend(v.owner.inputs)
+    return False
+
+
+def merge_sibling_reductions(fgraph):
+    """Two reductions over the same axes whose inputs have the same full shape
+    pattern and share at least one input become one multi-output reduction, so
+    shared operands are read once (e.g. ``sum(g)`` and ``sum(g * xhat)``, or
+    ``any`` and ``all`` of one tensor)."""
+    count = 0
+    changed = True
+    while changed:
+        changed = False
+        reds = [n for n in fgraph.toposort() if isinstance(n.op, HipCAReduce) and n.op.post_scalar_op is None]
+        for ai in range(len(reds)):
+            a = reds[ai]
+            for b in reds[ai + 1:]:
+                if a.op.axis != b.op.axis:
+                    continue
+                if not set(id(i) for i in a.inputs if isinstance(i.type, HipArrayType)) & set(
+                        id(i) for i in b.inputs if isinstance(i.type, HipArrayType)):
+                    continue
+                if a.outputs[0].type.broadcastable != b.outputs[0].type.broadcastable:
+                    continue
+                nd = max(i.type.ndim for i in a.inputs)
+                pa = [all(bb) for bb in zip(*[i.type.broadcastable for i in a.inputs if i.type.ndim == nd])]
+                pb = [all(bb) for bb in zip(*[i.type.broadcastable for i in b.inputs if i.type.ndim == nd])]
+                if pa != pb:
+                    continue
+                if any(_depends_on(i, a) for i in b.inputs) or any(_depends_on(i, b) for i in a.inputs):
+                    continue
+                merged = _merge_two(a, b)
+                if merged is None:
+                    continue
+                outs = merged.outputs
+                ka = len(a.outputs)
+                for o, no in zip(a.outputs, outs[:ka]):
+                    fgraph.replace(o, no)
+                for o, no in zip(b.outputs, outs[ka:]):
+                    fgraph.replace(o, no)
+                count += 1
+                changed = True
+                break
+            if changed:
+                break
+    return count
+
+
+def _merge_two(a, b):
+    inputs, s_inputs = [], []
+
+    def scalar_for(v):
+        for t, s in zip(inputs, s_inputs):
+            if t is v:
+                return s
+        s = scal.Scalar(v.type.dtype)()
+        inputs.append(v)
+        s_inputs.append(s)
+        return s
+
+    outs = []
+    for n in (a, b):
+        args = [scalar_for(v) for v in n.inputs]
+        if n.op.pre_scalar_op is None:
+            outs.extend(scal.identity(x) for x in args)
+        else:
+            res = n.op.pre_scalar_op(*args, return_list=True)
+            outs.extend(res)
+    if len(inputs) > config.max_fused_inputs:
+        return None
+    pre = scal.Composite(s_inputs, outs)
+    op = HipCAReduce(a.op.scalar_ops + b.op.scalar_ops, a.op.axis, a.op.acc_dtypes + b.op.acc_dtypes,
+                     a.op.out_dtypes + b.op.out_dtypes, pre, None)
+    return op.make_node(*inputs)
+
+
+# --------------------------------------------------------------------------
+def optimize(fgraph, fuse=True):
+    """Full pipeline: merge, lift, fuse."""
+    gof.merge_identical(fgraph)
+    fgraph = lift_to_hip(fgraph)
+    gof.merge_identical(fgraph)
+    if fuse:
+        fuse_elemwise(fgraph)
+        fuse_reduce_prologue(fgraph)
+        merge_sibling_reductions(fgraph)
+        gof.merge_identical(fgraph)
+    return fgraph

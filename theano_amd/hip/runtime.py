@@ -1,0 +1,346 @@
+"""ctypes binding of libthx_hip.so and the device array type built on it.
+
+The library is the only execution path: importing this module fails if the
+shared object has not been built, and every call that needs the GPU raises
+when no device is present.  ``HipArray`` plays the role pygpu's ``GpuArray``
+plays for the reference (``theano/gpuarray/type.py:129-517``): a strided view
+(shape, byte strides, offset) over a reference-counted device buffer.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from .. import scalar as scal
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(os.path.dirname(_HERE), "csrc", "libthx_hip.so")
+
+THX_MAX_ND = 8
+THX_BROADCAST = 1
+THX_DRY_RUN = 2
+THX_HOST_SCALAR = 0x100
+
+
+class thx_array(ctypes.Structure):
+    _fields_ = [("base", ctypes.c_void_p), ("offset_bytes", ctypes.c_int64), ("nd", ctypes.c_int32),
+                ("dtype", ctypes.c_int32), ("shape", ctypes.c_int64 * THX_MAX_ND),
+                ("strides_bytes", ctypes.c_int64 * THX_MAX_ND)]
+
+
+class HipRuntimeError(RuntimeError):
+    pass
+
+
+_EXC = {1: HipRuntimeError, 2: ValueError, 3: TypeError, 4: HipRuntimeError, 5: MemoryError,
+        6: NotImplementedError, 7: ValueError}
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        raise ImportError("libthx_hip.so is missing (%s). Build it with `python -m theano_amd.csrc.build`; "
+                          "there is no other execution path." % _LIB_PATH)
+    lib = ctypes.CDLL(_LIB_PATH)
+    vp, sz, i32, i64 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int32, ctypes.c_int64
+    P = ctypes.POINTER
+    sigs = {
+        "thx_init": ([ctypes.c_int], ctypes.c_int),
+        "thx_device_info": ([ctypes.c_char_p, sz, P(ctypes.c_int), P(i64)], ctypes.c_int),
+        "thx_last_error": ([], ctypes.c_char_p),
+        "thx_last_plan": ([], ctypes.c_char_p),
+        "thx_alloc": ([sz, P(vp)], ctypes.c_int),
+        "thx_free": ([vp], ctypes.c_int),
+        "thx_pool_trim": ([], ctypes.c_int),
+        "thx_h2d": ([vp, vp, sz], ctypes.c_int),
+        "thx_d2h": ([vp, vp, sz], ctypes.c_int),
+        "thx_d2d": ([vp, vp, sz], ctypes.c_int),
+        "thx_fill_bytes": ([vp, ctypes.c_int, sz], ctypes.c_int),
+        "thx_sync": ([], ctypes.c_int),
+        "thx_set_cache_dir": ([ctypes.c_char_p], ctypes.c_int),
+        "thx_cache_stats": ([P(i64), P(i64), P(i64)], ctypes.c_int),
+        "thx_elemwise_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, P(i32), P(vp)], ctypes.c_int),
+        "thx_elemwise_call": ([vp, P(thx_array), P(thx_array), ctypes.c_int], ctypes.c_int),
+        "thx_elemwise_free": ([vp], ctypes.c_int),
+        "thx_reduce_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, P(i32), ctypes.c_int, P(vp)],
+                           ctypes.c_int),
+        "thx_reduce_call": ([vp, P(thx_array), P(ctypes.c_uint8), P(thx_array), ctypes.c_int], ctypes.c_int),
+        "thx_reduce_free": ([vp], ctypes.c_int),
+        "thx_rowchain_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, P(i32), ctypes.c_int, P(vp)],
+                             ctypes.c_int),
+        "thx_rowchain_call": ([vp, P(thx_array), P(thx_array), ctypes.c_int], ctypes.c_int),
+        "thx_rowchain_free": ([vp], ctypes.c_int),
+        "thx_profile_begin": ([], ctypes.c_int),
+        "thx_profile_end": ([ctypes.c_char_p, sz], ctypes.c_int),
+        "thx_timer_start": ([], ctypes.c_int),
+        "thx_timer_stop": ([P(ctypes.c_float)], ctypes.c_int),
+    }
+    for name, (argtypes, restype) in sigs.items():
+        fn = getattr(lib, name, None)
+        if fn is None:
+            continue
+        fn.argtypes = argtypes
+        fn.restype = restype
+    return lib
+
+
+lib = _load()
+_default_cache = os.environ.get("THX_CACHE_DIR") or os.path.join(os.path.dirname(_HERE), "_kcache")
+lib.thx_set_cache_dir(_default_cache.encode())
+
+
+def check(rc):
+    if rc != 0:
+        msg = lib.thx_last_error().decode(errors="replace")
+        raise _EXC.get(rc, HipRuntimeError)(msg)
+
+
+_initialised = False
+_dry = False
+_fake_next = [0x7f0000000000]
+
+
+def set_dry_run(flag):
+    """In dry-run mode nothing touches a GPU: arrays get placeholder addresses
+    and every kernel call only validates, plans and compiles (filling the
+    on-disk code-object cache).  Used to check and pre-build kernels on a
+    machine without a device; results are meaningless."""
+    global _dry
+    _dry = bool(flag)
+
+
+def dry_run():
+    return _dry
+
+
+def call_flags():
+    return THX_BROADCAST | (THX_DRY_RUN if _dry else 0)
+
+
+def init(device=None):
+    """Bind the library to a GPU; raises HipRuntimeError when none is visible."""
+    global _initialised
+    if _dry:
+        return
+    if not _initialised:
+        from ..config import config
+        check(lib.thx_init(config.device if device is None else device))
+        _initialised = True
+
+
+def device_info():
+    init()
+    buf = ctypes.create_string_buffer(128)
+    cus, hbm = ctypes.c_int(), ctypes.c_int64()
+    check(lib.thx_device_info(buf, 128, ctypes.byref(cus), ctypes.byref(hbm)))
+    return {"arch": buf.value.decode(), "compute_units": cus.value, "hbm_bytes": hbm.value}
+
+
+def sync():
+    check(lib.thx_sync())
+
+
+def last_plan():
+    return lib.thx_last_plan().decode()
+
+
+def cache_stats():
+    a, b, c = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+    lib.thx_cache_stats(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c))
+    return {"compiled": a.value, "disk_hits": b.value, "mem_hits": c.value}
+
+
+class profile(object):
+    """Context manager collecting per-kernel HIP-event timings:
+    ``with profile() as p: ...`` then ``p.kernels`` maps plan name to
+    (launches, total milliseconds)."""
+
+    def __enter__(self):
+        init()
+        check(lib.thx_profile_begin())
+        self.kernels = {}
+        return self
+
+    def __exit__(self, *exc):
+        buf = ctypes.create_string_buffer(1 << 20)
+        check(lib.thx_profile_end(buf, 1 << 20))
+        for line in buf.value.decode().splitlines():
+            name, n, ms = line.rsplit("\t", 2)
+            self.kernels[name] = (int(n), float(ms))
+        return False
+
+
+def timer_start():
+    check(lib.thx_timer_start())
+
+
+def timer_stop():
+    ms = ctypes.c_float()
+    check(lib.thx_timer_stop(ctypes.byref(ms)))
+    return ms.value
+
+
+# --------------------------------------------------------------------------
+class _Buffer(object):
+    """One pooled device allocation, released when the last view dies."""
+
+    __slots__ = ("ptr", "nbytes", "fake")
+
+    def __init__(self, nbytes):
+        self.nbytes = int(nbytes)
+        self.fake = _dry
+        if _dry:
+            self.ptr = _fake_next[0]
+            _fake_next[0] += (self.nbytes + 4095) // 4096 * 4096 + 4096
+            return
+        init()
+        p = ctypes.c_void_p()
+        check(lib.thx_alloc(max(int(nbytes), 1), ctypes.byref(p)))
+        self.ptr = p.value
+
+    def __del__(self):
+        try:
+            if self.ptr and not self.fake:
+                lib.thx_free(self.ptr)
+                self.ptr = None
+        except Exception:
+            pass
+
+
+def _c_strides(shape, itemsize):
+    strides, acc = [], itemsize
+    for s in reversed(shape):
+        strides.append(acc)
+        acc *= max(int(s), 1)
+    return tuple(reversed(strides))
+
+
+class HipArray(object):
+    """A strided view of device memory."""
+
+    __slots__ = ("buffer", "offset", "shape", "strides", "dtype")
+
+    def __init__(self, buffer, offset, shape, strides, dtype):
+        self.buffer = buffer
+        self.offset = int(offset)
+        self.shape = tuple(int(s) for s in shape)
+        self.strides = tuple(int(s) for s in strides)
+        self.dtype = np.dtype(dtype)
+
+    # -- construction
+    @classmethod
+    def empty(cls, shape, dtype):
+        dtype = np.dtype(dtype)
+        shape = tuple(int(s) for s in shape)
+        if len(shape) > THX_MAX_ND:
+            raise TypeError("arrays of rank %d exceed the limit of %d" % (len(shape), THX_MAX_ND))
+        n = 1
+        for s in shape:
+            n *= s
+        return cls(_Buffer(n * dtype.itemsize), 0, shape, _c_strides(shape, dtype.itemsize), dtype)
+
+    @classmethod
+    def from_numpy(cls, a):
+        a = np.asarray(a)
+        if str(a.dtype) not in scal.all_dtypes:
+            raise TypeError("dtype %s is not supported on the device" % a.dtype)
+        a = np.ascontiguousarray(a)
+        out = cls.empty(a.shape, a.dtype)
+        if a.nbytes and not out.buffer.fake:
+            check(lib.thx_h2d(out.buffer.ptr, a.ctypes.data, a.nbytes))
+        return out
+
+    # -- properties
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    @property
+    def size(self):
+        n = 1
+        for s in self.shape:
+            n *= s
+        return n
+
+    @property
+    def nbytes(self):
+        return self.size * self.dtype.itemsize
+
+    @property
+    def ptr(self):
+        return self.buffer.ptr + self.offset
+
+    @property
+    def c_contiguous(self):
+        expect = self.dtype.itemsize
+        for s, st in zip(reversed(self.shape), reversed(self.strides)):
+            if s > 1 and st != expect:
+                return False
+            expect *= max(s, 1)
+        return True
+
+    def __repr__(self):
+        return "HipArray(shape=%s, dtype=%s, strides=%s)" % (self.shape, self.dtype, self.strides)
+
+    # -- views
+    def view(self, shape, strides, offset=None):
+        return HipArray(self.buffer, self.offset if offset is None else offset, shape, strides, self.dtype)
+
+    def transpose(self, *axes):
+        if not axes:
+            axes = tuple(reversed(range(self.ndim)))
+        return self.view([self.shape[a] for a in axes], [self.strides[a] for a in axes])
+
+    # -- transfers
+    def to_numpy(self):
+        """Copy to host; strided views are copied as the byte span they cover
+        and re-viewed on the host."""
+        out = np.empty(self.shape, self.dtype)
+        if self.buffer.fake:
+            out.fill(0)
+            return out
+        if self.size == 0:
+            return out
+        if self.c_contiguous:
+            check(lib.thx_d2h(out.ctypes.data, self.ptr, out.nbytes))
+            return out
+        lo = hi = 0
+        for s, st in zip(self.shape, self.strides):
+            if st < 0:
+                lo += (s - 1) * st
+            else:
+                hi += (s - 1) * st
+        span = hi - lo + self.dtype.itemsize
+        raw = np.empty(span, np.uint8)
+        check(lib.thx_d2h(raw.ctypes.data, self.ptr + lo, span))
+        view = np.ndarray(self.shape, self.dtype, buffer=raw, offset=-lo, strides=self.strides)
+        out[...] = view
+        return out
+
+    def __array__(self, dtype=None, copy=None):
+        a = self.to_numpy()
+        return a if dtype is None else a.astype(dtype)
+
+    def as_thx(self, out=None):
+        a = out if out is not None else thx_array()
+        a.base = self.buffer.ptr
+        a.offset_bytes = self.offset
+        a.nd = len(self.shape)
+        a.dtype = scal.dtype_code(str(self.dtype))
+        for i, (s, st) in enumerate(zip(self.shape, self.strides)):
+            a.shape[i] = s
+            a.strides_bytes[i] = st
+        return a
+
+
+def host_scalar_thx(value, nd, out=None):
+    """Descriptor of a one-element host array passed by value (as a kernel
+    argument) instead of through device memory."""
+    a = out if out is not None else thx_array()
+    a.base = value.ctypes.data
+    a.offset_bytes = 0
+    a.nd = nd
+    a.dtype = scal.dtype_code(str(value.dtype)) | THX_HOST_SCALAR
+    for i in range(nd):
+        a.shape[i] = 1
+        a.strides_bytes[i] = 0
+    return a

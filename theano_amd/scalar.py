@@ -1,0 +1,1222 @@
+"""Scalar type system and per-element operations.
+
+Mirrors ``theano/scalar/basic.py``: dtype algebra (``upcast`` :59-87, output
+type policies :836-1019), the ScalarOps with their C semantics (:1214-3100),
+``Composite`` (:3764-4127) and the thresholded sigmoid / softplus of
+``theano/tensor/nnet/sigm.py:29-88, 330-372``.  ``c_code`` returns the statement
+executed per element inside a device functor; its text is the normative
+definition of each op here exactly as the C snippets are in the reference.
+float16 values are computed in float32 (what ``Compositef32``
+:4130-4208 arranges for the reference's device code).
+"""
+import math
+
+import numpy as np
+
+from . import gof
+from .config import config
+from .gof import Apply, Constant, MethodNotDefined, Op, Type, Variable
+
+float_dtypes = ("float16", "float32", "float64")
+int_dtypes = ("int8", "int16", "int32", "int64")
+uint_dtypes = ("uint8", "uint16", "uint32", "uint64")
+integer_dtypes = int_dtypes + uint_dtypes
+discrete_dtypes = ("bool",) + integer_dtypes
+continuous_dtypes = float_dtypes
+all_dtypes = discrete_dtypes + float_dtypes
+
+# dtype -> (ABI code, storage C type, compute C type)
+_DTYPE_INFO = {
+    "bool": (0, "thx_bool", "thx_bool"), "int8": (1, "thx_i8", "thx_i8"), "uint8": (2, "thx_u8", "thx_u8"),
+    "int16": (3, "thx_i16", "thx_i16"), "uint16": (4, "thx_u16", "thx_u16"), "int32": (5, "thx_i32", "thx_i32"),
+    "uint32": (6, "thx_u32", "thx_u32"), "int64": (7, "thx_i64", "thx_i64"), "uint64": (8, "thx_u64", "thx_u64"),
+    "float16": (9, "thx_f16", "thx_f32"), "float32": (10, "thx_f32", "thx_f32"), "float64": (11, "thx_f64", "thx_f64"),
+}
+
+
+def dtype_code(dtype):
+    return _DTYPE_INFO[str(dtype)][0]
+
+
+def storage_ctype(dtype):
+    return _DTYPE_INFO[str(dtype)][1]
+
+
+def compute_ctype(dtype):
+    return _DTYPE_INFO[str(dtype)][2]
+
+
+def upcast(dtype, *dtypes):
+    """Result dtype of mixing the given dtypes: NumPy array promotion
+    (``theano/scalar/basic.py:59-87`` with cast_policy 'custom')."""
+    z = np.zeros((), dtype=dtype)
+    for dt in dtypes:
+        z = z + np.zeros((), dtype=dt)
+    return str(z.dtype)
+
+
+class IntegerDivisionError(Exception):
+    pass
+
+
+# --------------------------------------------------------------------------
+class Scalar(Type):
+    """Type of one number of a given dtype (``theano/scalar/basic.py:293-416``)."""
+
+    def __init__(self, dtype):
+        if dtype == "floatX":
+            dtype = config.floatX
+        dtype = str(np.dtype(dtype)) if dtype != "bool" else "bool"
+        if dtype not in _DTYPE_INFO:
+            raise TypeError("unsupported dtype for a Scalar: %s" % dtype)
+        self.dtype = dtype
+
+    def filter(self, data, strict=False, allow_downcast=None):
+        return np.asarray(data, dtype=self.dtype)[()]
+
+    def __eq__(self, other):
+        return type(self) is type(other) and self.dtype == other.dtype
+
+    def __hash__(self):
+        return hash(("Scalar", self.dtype))
+
+    def __str__(self):
+        return self.dtype
+
+    __repr__ = __str__
+
+    @staticmethod
+    def upcast(*types):
+        return upcast(*[getattr(t, "dtype", t) for t in types])
+
+
+def get_scalar_type(dtype):
+    return Scalar(dtype)
+
+
+bool_ = Scalar("bool")
+int8, int16, int32, int64 = Scalar("int8"), Scalar("int16"), Scalar("int32"), Scalar("int64")
+uint8, uint16, uint32, uint64 = Scalar("uint8"), Scalar("uint16"), Scalar("uint32"), Scalar("uint64")
+float16, float32, float64 = Scalar("float16"), Scalar("float32"), Scalar("float64")
+
+
+class _scalar_py_operators(object):
+    """Operator overloads so that gradient formulas read like arithmetic."""
+
+    dtype = property(lambda self: self.type.dtype)
+
+    def __abs__(self): return abs_(self)
+    def __neg__(self): return neg(self)
+    def __invert__(self): return invert(self)
+    def __and__(self, o): return and_(self, o)
+    def __or__(self, o): return or_(self, o)
+    def __xor__(self, o): return xor(self, o)
+    def __rand__(self, o): return and_(o, self)
+    def __ror__(self, o): return or_(o, self)
+    def __rxor__(self, o): return xor(o, self)
+    def __lt__(self, o): return lt(self, o)
+    def __gt__(self, o): return gt(self, o)
+    def __le__(self, o): return le(self, o)
+    def __ge__(self, o): return ge(self, o)
+    def __add__(self, o): return add(self, o)
+    def __sub__(self, o): return sub(self, o)
+    def __mul__(self, o): return mul(self, o)
+    def __truediv__(self, o): return div_proxy(self, o)
+    __div__ = __truediv__
+    def __floordiv__(self, o): return int_div(self, o)
+    def __mod__(self, o): return mod(self, o)
+    def __pow__(self, o): return pow(self, o)
+    def __radd__(self, o): return add(o, self)
+    def __rsub__(self, o): return sub(o, self)
+    def __rmul__(self, o): return mul(o, self)
+    def __rtruediv__(self, o): return div_proxy(o, self)
+    __rdiv__ = __rtruediv__
+    def __rfloordiv__(self, o): return int_div(o, self)
+    def __rmod__(self, o): return mod(o, self)
+    def __rpow__(self, o): return pow(o, self)
+
+    def zeros_like(self, dtype=None):
+        # a zero that still depends on self, as theano/scalar/basic.py:789-799
+        if dtype is None:
+            dtype = self.type.dtype
+        return second(self, ScalarConstant(Scalar(dtype), np.asarray(0, dtype=dtype)[()]))
+
+    def ones_like(self, dtype=None):
+        if dtype is None:
+            dtype = self.type.dtype
+        return second(self, ScalarConstant(Scalar(dtype), np.asarray(1, dtype=dtype)[()]))
+
+    def astype(self, dtype):
+        return cast(self, dtype)
+
+
+class ScalarVariable(_scalar_py_operators, Variable):
+    pass
+
+
+class ScalarConstant(_scalar_py_operators, Constant):
+    def signature(self):
+        return (self.type, np.asarray(self.data).tobytes())
+
+
+Scalar.Variable = ScalarVariable
+Scalar.Constant = ScalarConstant
+
+
+def _autocast(x):
+    """dtype chosen for a Python literal (``NumpyAutocaster``,
+    ``theano/scalar/basic.py:132-214``, cast_policy 'custom')."""
+    if isinstance(x, (bool, np.bool_)):
+        return np.asarray(x, dtype="bool")
+    if isinstance(x, (int, np.integer)) and not hasattr(x, "dtype"):
+        for dt in int_dtypes:
+            try:
+                x_ = np.asarray(x, dtype=dt)
+            except OverflowError:
+                continue
+            if x_ == x:
+                return x_
+        return np.asarray(x, dtype="uint64")
+    if isinstance(x, float):
+        if config.floatX != "float64":
+            return np.asarray(x, dtype=config.floatX)
+        x_ = None
+        for dt in ("float32", "float64"):
+            x_ = np.asarray(x, dtype=dt)
+            if x_ == x or (x != x):
+                break
+        return x_
+    return np.asarray(x)
+
+
+def convert(x, dtype=None):
+    """Typed NumPy value of ``x`` under the casting policy
+    (``theano/scalar/basic.py:252-290``)."""
+    if dtype is not None:
+        return np.asarray(x, dtype=config.floatX if dtype == "floatX" else dtype)
+    if isinstance(x, (bool, int, float, np.bool_)) and not isinstance(x, np.generic):
+        return _autocast(x)
+    if isinstance(x, np.generic):
+        return np.asarray(x)
+    if isinstance(x, np.ndarray):
+        return x
+    x_ = np.asarray(x)
+    if x_.size == 0 and not hasattr(x, "dtype"):
+        x_ = np.asarray(x, dtype=config.floatX)
+    elif x_.dtype == np.float64 and config.floatX != "float64" and not hasattr(x, "dtype"):
+        pass  # lists of Python floats keep NumPy's float64, as in the reference
+    return x_
+
+
+def constant(x, name=None, dtype=None):
+    x = convert(x, dtype=dtype)
+    if x.ndim != 0:
+        raise TypeError("scalar.constant needs a 0-d value")
+    return ScalarConstant(Scalar(str(x.dtype)), x[()], name=name)
+
+
+def as_scalar(x, name=None):
+    if isinstance(x, Apply):
+        x = x.default_output()
+    if isinstance(x, Variable):
+        if isinstance(x.type, Scalar):
+            return x
+        raise TypeError("not a scalar variable: %s" % (x,))
+    return constant(x, name=name)
+
+
+# --------------------------------------------------------------------------
+# output type policies (theano/scalar/basic.py:836-1019)
+def upcast_out(*types):
+    return (Scalar(Scalar.upcast(*types)),)
+
+
+def upcast_out_nobool(*types):
+    t = upcast_out(*types)
+    if t[0] == bool_:
+        raise TypeError("bool output not supported")
+    return t
+
+
+def upcast_out_min8(*types):
+    t = upcast_out(*types)
+    return (int8,) if t[0] == bool_ else t
+
+
+_TO_FLOAT = {"bool": "float32", "int8": "float32", "int16": "float32", "int32": "float64", "int64": "float64",
+             "uint8": "float32", "uint16": "float32", "uint32": "float64", "uint64": "float64"}
+
+
+def upgrade_to_float(*types):
+    return (Scalar(upcast(*[_TO_FLOAT.get(t.dtype, t.dtype) for t in types])),)
+
+
+def same_out(t):
+    return (t,)
+
+
+def same_out_nobool(t):
+    if t == bool_:
+        raise TypeError("bool input not supported")
+    return (t,)
+
+
+def same_out_min8(t):
+    return (int8,) if t == bool_ else (t,)
+
+
+def same_out_float_only(t):
+    if t.dtype not in float_dtypes:
+        raise TypeError("only float type are supported")
+    return (t,)
+
+
+class transfer_type(object):
+    """Output i takes the type of input ``transfer[i]`` (None: the upcast)."""
+
+    def __init__(self, *transfer):
+        self.transfer = transfer
+
+    def __eq__(self, other):
+        return type(self) is type(other) and self.transfer == other.transfer
+
+    def __hash__(self):
+        return hash(("transfer_type", self.transfer))
+
+    def __call__(self, *types):
+        up = upcast_out(*types)[0]
+        return [up if i is None else (Scalar(i) if isinstance(i, str) else types[i]) for i in self.transfer]
+
+
+class specific_out(object):
+    def __init__(self, *spec):
+        self.spec = spec
+
+    def __eq__(self, other):
+        return type(self) is type(other) and self.spec == other.spec
+
+    def __hash__(self):
+        return hash(("specific_out", self.spec))
+
+    def __call__(self, *types):
+        return self.spec
+
+
+# --------------------------------------------------------------------------
+def _fn(name, dtype):
+    """libm-style function name for the compute type of ``dtype``."""
+    return name if compute_ctype(dtype) == "thx_f64" else name + "f"
+
+
+def c_literal(value, dtype):
+    """Device source text of a constant of the given dtype."""
+    dtype = str(dtype)
+    if dtype == "bool":
+        return "((thx_bool)%d)" % (1 if value else 0)
+    if dtype in float_dtypes:
+        v = float(np.asarray(value, dtype=dtype))
+        ct = compute_ctype(dtype)
+        if math.isnan(v):
+            return "((%s)NAN)" % ct
+        if math.isinf(v):
+            return "((%s)%sINFINITY)" % (ct, "-" if v < 0 else "")
+        if ct == "thx_f64":
+            return "(%r)" % v
+        return "(%rf)" % v
+    v = int(value)
+    if dtype == "int64":
+        if v == -(1 << 63):
+            return "(-9223372036854775807LL - 1)"
+        return "(%dLL)" % v
+    if dtype == "uint64":
+        return "(%dULL)" % v
+    if dtype == "uint32":
+        return "(%dU)" % v
+    if dtype == "int32":
+        if v == -(1 << 31):
+            return "(-2147483647 - 1)"
+        return "(%d)" % v
+    return "((%s)%d)" % (storage_ctype(dtype), v)
+
+
+class ScalarOp(Op):
+    """Base of per-element operations (``theano/scalar/basic.py:1022-1198``)."""
+
+    nin = -1
+    nout = 1
+    identity = None
+    commutative = False
+    associative = False
+    __props__ = ("output_types_preference",)
+
+    def __init__(self, output_types_preference=None, name=None):
+        self.name = name
+        if output_types_preference is not None:
+            self.output_types_preference = output_types_preference
+        elif not hasattr(self, "output_types_preference"):
+            self.output_types_preference = None
+
+    def _props(self):
+        return (self.output_types_preference,)
+
+    def __str__(self):
+        return self.name if getattr(self, "name", None) else type(self).__name__
+
+    __repr__ = __str__
+
+    def output_types(self, types):
+        pref = self.output_types_preference
+        if pref is None:
+            raise MethodNotDefined("output_types", type(self))
+        variables = pref(*types)
+        if len(variables) != self.nout:
+            raise TypeError("%s: expected %d outputs, policy gave %d" % (self, self.nout, len(variables)))
+        return list(variables)
+
+    def make_node(self, *inputs):
+        if self.nin >= 0 and len(inputs) != self.nin:
+            raise TypeError("%s takes %d inputs, got %d" % (self, self.nin, len(inputs)))
+        inputs = [as_scalar(i) for i in inputs]
+        outputs = [t() for t in self.output_types([i.type for i in inputs])]
+        if len(outputs) != self.nout:
+            raise TypeError("wrong number of outputs")
+        return Apply(self, inputs, outputs)
+
+    def c_code(self, node, inputs, outputs):
+        """Statement computing ``outputs`` (names) from ``inputs`` (expressions)."""
+        raise MethodNotDefined("c_code", type(self))
+
+    def supports_c_code(self, inputs, outputs):
+        try:
+            node = Apply(self, inputs, [o.clone() for o in outputs])
+            self.c_code(node, ["x"] * len(inputs), ["z"] * len(outputs))
+        except (MethodNotDefined, NotImplementedError):
+            return False
+        return True
+
+    def make_new_inplace(self, output_types_preference=None, name=None):
+        return type(self)(output_types_preference, name)
+
+
+class UnaryScalarOp(ScalarOp):
+    nin = 1
+
+
+class BinaryScalarOp(ScalarOp):
+    nin = 2
+
+
+def _zero_grads(inputs):
+    return [i.zeros_like(dtype=config.floatX) if i.type.dtype in discrete_dtypes else i.zeros_like() for i in inputs]
+
+
+# ---- comparisons (theano/scalar/basic.py:1214-1431) ---------------------------
+class LogicalComparison(BinaryScalarOp):
+    def output_types(self, types):
+        return [bool_]
+
+    def L_op(self, inputs, outputs, gout):
+        return [i.zeros_like(dtype=config.floatX) for i in inputs]
+
+
+def _cmp(name, sym):
+    class _C(LogicalComparison):
+        def c_code(self, node, inputs, outputs):
+            return "%s = (%s %s %s);" % (outputs[0], inputs[0], sym, inputs[1])
+    _C.__name__ = name
+    _C.commutative = sym in ("==", "!=")
+    return _C
+
+
+LT, GT, LE, GE, EQ, NEQ = (_cmp("LT", "<"), _cmp("GT", ">"), _cmp("LE", "<="), _cmp("GE", ">="),
+                           _cmp("EQ", "=="), _cmp("NEQ", "!="))
+lt, gt, le, ge, eq, neq = LT(name="lt"), GT(name="gt"), LE(name="le"), GE(name="ge"), EQ(name="eq"), NEQ(name="neq")
+
+
+class FixedLogicalComparison(UnaryScalarOp):
+    def output_types(self, types):
+        return [bool_]
+
+    def L_op(self, inputs, outputs, gout):
+        return [inputs[0].zeros_like(dtype=config.floatX)]
+
+
+class IsNan(FixedLogicalComparison):
+    def c_code(self, node, inputs, outputs):
+        if node.inputs[0].type.dtype in discrete_dtypes:
+            return "%s = 0;" % outputs[0]
+        return "%s = isnan(%s) ? 1 : 0;" % (outputs[0], inputs[0])
+
+
+class IsInf(FixedLogicalComparison):
+    def c_code(self, node, inputs, outputs):
+        if node.inputs[0].type.dtype in discrete_dtypes:
+            return "%s = 0;" % outputs[0]
+        return "%s = isinf(%s) ? 1 : 0;" % (outputs[0], inputs[0])
+
+
+isnan, isinf = IsNan(name="isnan"), IsInf(name="isinf")
+
+
+class Switch(ScalarOp):
+    nin = 3
+
+    def output_types(self, types):
+        return list(upcast_out(types[1], types[2]))
+
+    def c_code(self, node, inputs, outputs):
+        return "%s = %s ? %s : %s;" % (outputs[0], inputs[0], inputs[1], inputs[2])
+
+    def L_op(self, inputs, outputs, gout):
+        cond, ift, iff = inputs
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            first, secnd = ift.zeros_like(dtype=config.floatX), iff.zeros_like(dtype=config.floatX)
+        else:
+            first, secnd = switch(cond, gz, 0.0), switch(cond, 0.0, gz)
+        return [cond.zeros_like(dtype=config.floatX), first, secnd]
+
+
+switch = Switch(name="switch")
+
+
+# ---- bit operations (theano/scalar/basic.py:1523-1617) ------------------------
+class UnaryBitOp(UnaryScalarOp):
+    def output_types(self, types):
+        for t in types:
+            if t.dtype not in discrete_dtypes:
+                raise TypeError("input to a BitOp must have type (u)int8, (u)int16, (u)int32 or (u)int64 or bool "
+                                "not %s" % t)
+        return list(upcast_out(*types))
+
+    def L_op(self, inputs, outputs, gout):
+        return [inputs[0].zeros_like(dtype=config.floatX)]
+
+
+class BinaryBitOp(BinaryScalarOp):
+    commutative = True
+    associative = True
+
+    def output_types(self, types):
+        t0, t1 = types
+        if t0 == bool_ and t1 == bool_:
+            return [bool_]
+        for t in types:
+            if t.dtype not in integer_dtypes:
+                raise TypeError("input to a BitOp must have type (u)int8, (u)int16, (u)int32 or (u)int64 or be all "
+                                "bools not %s" % t)
+        return list(upcast_out(*types))
+
+    def L_op(self, inputs, outputs, gout):
+        return [i.zeros_like(dtype=config.floatX) for i in inputs]
+
+    def c_code(self, node, inputs, outputs):
+        return "%s = (%s %s %s);" % (outputs[0], inputs[0], self.symbol, inputs[1])
+
+
+class OR(BinaryBitOp):
+    identity = 0
+    symbol = "|"
+
+
+class XOR(BinaryBitOp):
+    identity = 0
+    symbol = "^"
+
+
+class AND(BinaryBitOp):
+    identity = -1
+    symbol = "&"
+
+
+class RightShift(BinaryBitOp):
+    """Arithmetic ``x >> y``.  The reference has no shift op; for signed
+    two's-complement operands this equals ``int_div(x, 2**y)``
+    (``theano/scalar/basic.py:1960-2025``), which is what pins it."""
+    commutative = False
+    associative = False
+    symbol = ">>"
+
+    def output_types(self, types):
+        for t in types:
+            if t.dtype not in integer_dtypes:
+                raise TypeError("shift operands must be integers, not %s" % t)
+        return list(upcast_out(*types))
+
+
+class LeftShift(RightShift):
+    symbol = "<<"
+
+
+class Invert(UnaryBitOp):
+    def c_code(self, node, inputs, outputs):
+        if node.outputs[0].type == bool_:
+            return "%s = (!%s);" % (outputs[0], inputs[0])
+        return "%s = (~%s);" % (outputs[0], inputs[0])
+
+
+or_, xor, and_, invert = OR(name="or_"), XOR(name="xor"), AND(name="and_"), Invert(name="invert")
+right_shift, left_shift = RightShift(name="right_shift"), LeftShift(name="left_shift")
+
+
+# ---- max / min (theano/scalar/basic.py:1623-1696) ------------------------------
+class Maximum(BinaryScalarOp):
+    commutative = True
+    associative = True
+
+    def c_code(self, node, inputs, outputs):
+        x, y = inputs
+        nan = "NAN" if node.outputs[0].type.dtype in float_dtypes else "0"
+        # both comparisons, so that a NaN on either side gives NaN
+        return "%s = ((%s) > (%s) ? (%s) : ((%s) >= (%s) ? (%s) : %s));" % (outputs[0], y, x, y, x, y, x, nan)
+
+    def L_op(self, inputs, outputs, gout):
+        x, y = inputs
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [x.zeros_like(dtype=config.floatX), y.zeros_like(dtype=config.floatX)]
+        e = eq(outputs[0], x)
+        return [e * gz, (constant(1, dtype=gz.type.dtype) - e) * gz]
+
+
+class Minimum(Maximum):
+    def c_code(self, node, inputs, outputs):
+        x, y = inputs
+        nan = "NAN" if node.outputs[0].type.dtype in float_dtypes else "0"
+        return "%s = ((%s) < (%s) ? (%s) : ((%s) <= (%s) ? (%s) : %s));" % (outputs[0], y, x, y, x, y, x, nan)
+
+
+maximum, minimum = Maximum(upcast_out, name="maximum"), Minimum(upcast_out, name="minimum")
+
+
+# ---- arithmetic (theano/scalar/basic.py:1699-2261) ------------------------------
+class Add(ScalarOp):
+    identity = 0
+    commutative = True
+    associative = True
+
+    def c_code(self, node, inputs, outputs):
+        sym = " || " if node.outputs[0].type == bool_ else " + "
+        return "%s = %s;" % (outputs[0], sym.join(inputs) if inputs else "0")
+
+    def L_op(self, inputs, outputs, gout):
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [i.zeros_like(dtype=config.floatX) for i in inputs]
+        return [gz for _ in inputs]
+
+
+class Mul(ScalarOp):
+    identity = 1
+    commutative = True
+    associative = True
+
+    def c_code(self, node, inputs, outputs):
+        sym = " && " if node.outputs[0].type == bool_ else " * "
+        return "%s = %s;" % (outputs[0], sym.join(inputs) if inputs else "1")
+
+    def L_op(self, inputs, outputs, gout):
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [i.zeros_like(dtype=config.floatX) for i in inputs]
+        return [mul(*([gz] + [o for j, o in enumerate(inputs) if j != k])) for k in range(len(inputs))]
+
+
+class Sub(BinaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        return "%s = %s - %s;" % (outputs[0], inputs[0], inputs[1])
+
+    def L_op(self, inputs, outputs, gout):
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [i.zeros_like(dtype=config.floatX) for i in inputs]
+        return [gz, -gz]
+
+
+add, mul, sub = Add(upcast_out, name="add"), Mul(upcast_out, name="mul"), Sub(upcast_out_nobool, name="sub")
+
+
+def int_or_true_div(x_discrete, y_discrete):
+    """Which division ``x / y`` means (``theano/scalar/basic.py:1826-1873``)."""
+    if x_discrete and y_discrete:
+        if config.int_division == "raise":
+            raise IntegerDivisionError("dividing two integer types with '/' is forbidden by config.int_division; "
+                                       "use // or cast one argument to float")
+        if config.int_division == "int":
+            return int_div
+        return true_div
+    return true_div
+
+
+def div_proxy(x, y):
+    x, y = as_scalar(x), as_scalar(y)
+    return int_or_true_div(x.type.dtype in discrete_dtypes, y.type.dtype in discrete_dtypes)(x, y)
+
+
+class TrueDiv(BinaryScalarOp):
+    def output_types(self, types):
+        if all(t.dtype in discrete_dtypes for t in types):
+            return [Scalar(config.floatX)]
+        return BinaryScalarOp.output_types(self, types)
+
+    def c_code(self, node, inputs, outputs):
+        if all(i.type.dtype in discrete_dtypes for i in node.inputs):
+            return "%s = ((double)%s) / %s;" % (outputs[0], inputs[0], inputs[1])
+        return "%s = %s / %s;" % (outputs[0], inputs[0], inputs[1])
+
+    def L_op(self, inputs, outputs, gout):
+        x, y = inputs
+        (gz,) = gout
+        if all(i.type.dtype in discrete_dtypes for i in inputs):
+            return [x.zeros_like(), y.zeros_like()]
+        return [gz / y, -(gz * x) / (y * y)]
+
+
+true_div = TrueDiv(upcast_out, name="true_div")
+
+
+class IntDiv(BinaryScalarOp):
+    """Floor division with Python's sign rule; the four sign cases are spelled
+    out because C division truncates (``theano/scalar/basic.py:1960-2025``).
+    Integer division by zero cannot raise on the device: like the reference's
+    ``#ifdef KERNEL`` branch the hardware result is stored."""
+
+    def c_code(self, node, inputs, outputs):
+        x, y = inputs
+        (z,) = outputs
+        t = upcast(*[i.type.dtype for i in node.inputs])
+        if t in discrete_dtypes:
+            d = lambda a, b: "(%s / %s)" % (a, b)
+            m = lambda a, b: "(%s %% %s)" % (a, b)
+            zero = "%s = 0;" % z
+        else:
+            fl, fm = _fn("floor", t), _fn("fmod", t)
+            d = lambda a, b: "%s(%s / %s)" % (fl, a, b)
+            m = lambda a, b: "%s(%s, %s)" % (fm, a, b)
+            zero = "%s = %s;" % (z, d(x, y))
+        nx, ny = "(-%s)" % x, "(-%s)" % y
+        return ("if (%(y)s == 0) { %(zero)s } "
+                "else if (%(y)s < 0) { if (%(x)s < 0) { %(z)s = %(mm)s; } "
+                "else { %(z)s = -%(pm)s - ((%(mpm)s == 0) ? 0 : 1); } } "
+                "else { if (%(x)s < 0) { %(z)s = -%(mp)s - ((%(mmp)s == 0) ? 0 : 1); } "
+                "else { %(z)s = %(pp)s; } }") % dict(
+                    x=x, y=y, z=z, zero=zero, mm=d(nx, ny), pm=d(x, ny), mpm=m(x, ny), mp=d(nx, y), mmp=m(nx, y),
+                    pp=d(x, y))
+
+    def L_op(self, inputs, outputs, gout):
+        return [i.zeros_like(dtype=config.floatX) for i in inputs]
+
+
+int_div = IntDiv(upcast_out, name="int_div")
+
+
+class Mod(BinaryScalarOp):
+    """Remainder with the sign of the divisor (``theano/scalar/basic.py:2048-2147``)."""
+
+    def c_code(self, node, inputs, outputs):
+        x, y = inputs
+        (z,) = outputs
+        t = upcast(*[i.type.dtype for i in node.inputs])
+        if t in discrete_dtypes:
+            m = lambda a, b: "(%s %% %s)" % (a, b)
+            zero = "%s = 0;" % z
+        else:
+            # the reference calls the double overload whatever the input type
+            m = lambda a, b: "fmod((double)%s, (double)%s)" % (a, b)
+            zero = "%s = %s;" % (z, m(x, y))
+        nx, ny = "(-%s)" % x, "(-%s)" % y
+        return ("if (%(y)s == 0) { %(zero)s } "
+                "else if (%(y)s < 0) { if (%(x)s < 0) { %(z)s = -(%(mm)s); } "
+                "else { %(z)s = (%(pm)s) + (%(pm)s != 0 ? %(y)s : 0); } } "
+                "else { if (%(x)s < 0) { %(z)s = -%(mp)s + (%(mp)s != 0 ? %(y)s : 0); } "
+                "else { %(z)s = %(pp)s; } }") % dict(
+                    x=x, y=y, z=z, zero=zero, mm=m(nx, ny), pm=m(x, ny), mp=m(nx, y), pp=m(x, y))
+
+    def L_op(self, inputs, outputs, gout):
+        x, y = inputs
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [i.zeros_like(dtype=config.floatX) for i in inputs]
+        return [gz, -(x // y) * gz]
+
+
+mod = Mod(upcast_out, name="mod")
+
+
+class Pow(BinaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        # C's pow(): arguments promote to double
+        return "%s = pow((double)%s, (double)%s);" % (outputs[0], inputs[0], inputs[1])
+
+    def L_op(self, inputs, outputs, gout):
+        x, y = inputs
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [i.zeros_like(dtype=config.floatX) for i in inputs]
+        first = gz * y * x ** (y - 1)
+        secnd = switch(eq(x, 0), 0, gz * log(x) * x ** y)
+        return [first, secnd]
+
+
+pow = Pow(upcast_out_min8, name="pow")
+
+
+class Clip(ScalarOp):
+    nin = 3
+
+    def output_types(self, types):
+        return list(upcast_out(*types))
+
+    def c_code(self, node, inputs, outputs):
+        x, lo, hi = inputs
+        return "%s = %s < %s ? %s : %s > %s ? %s : %s;" % (outputs[0], x, lo, lo, x, hi, hi, x)
+
+    def L_op(self, inputs, outputs, gout):
+        x, mn, mx = inputs
+        (gz,) = gout
+        if outputs[0].type.dtype in integer_dtypes:
+            return [i.zeros_like(dtype=config.floatX) for i in inputs]
+        return [((x >= mn) & (x <= mx)) * gz, (x < mn) * gz, (x > mx) * gz]
+
+
+clip = Clip(name="clip")
+
+
+class Second(BinaryScalarOp):
+    """``second(x, y) = y``; only the shape of ``x`` matters at tensor level."""
+
+    def c_code(self, node, inputs, outputs):
+        return "%s = %s;" % (outputs[0], inputs[1])
+
+    def connection_pattern(self, node):
+        return [[False], [True]]
+
+    def L_op(self, inputs, outputs, gout):
+        x, y = inputs
+        (gz,) = gout
+        if y.type.dtype in continuous_dtypes:
+            return [DisconnectedType()(), gz]
+        return [DisconnectedType()(), y.zeros_like()]
+
+
+second = Second(transfer_type(1), name="second")
+
+
+class Identity(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        return "%s = %s;" % (outputs[0], inputs[0])
+
+    def L_op(self, inputs, outputs, gout):
+        if inputs[0].type.dtype in continuous_dtypes:
+            return [gout[0]]
+        return [inputs[0].zeros_like(dtype=config.floatX)]
+
+
+identity = Identity(same_out, name="identity")
+
+
+class Cast(UnaryScalarOp):
+    def __init__(self, o_type, name=None):
+        if not isinstance(o_type, Scalar):
+            raise TypeError(o_type)
+        UnaryScalarOp.__init__(self, specific_out(o_type), name=name)
+        self.o_type = o_type
+
+    def __str__(self):
+        return "Cast{%s}" % self.o_type.dtype
+
+    def make_new_inplace(self, output_types_preference=None, name=None):
+        return type(self)(self.o_type, name)
+
+    def c_code(self, node, inputs, outputs):
+        if node.outputs[0].type == bool_:
+            return "%s = (%s) ? 1 : 0;" % (outputs[0], inputs[0])
+        return "%s = (%s)%s;" % (outputs[0], compute_ctype(node.outputs[0].type.dtype), inputs[0])
+
+    def L_op(self, inputs, outputs, gout):
+        if self.o_type.dtype in continuous_dtypes:
+            return [gout[0]]
+        return [inputs[0].zeros_like(dtype=config.floatX)]
+
+
+_cast_mapping = dict((dt, Cast(Scalar(dt), name="convert_to_" + dt)) for dt in all_dtypes)
+
+
+def cast(x, dtype):
+    if dtype == "floatX":
+        dtype = config.floatX
+    x = as_scalar(x)
+    dtype = str(dtype)
+    if x.type.dtype == dtype:
+        return x
+    return _cast_mapping[dtype](x)
+
+
+class Abs(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        t = node.inputs[0].type.dtype
+        (x,), (z,) = inputs, outputs
+        if t in int_dtypes:
+            return "%s = (%s < 0) ? -%s : %s;" % (z, x, x, x)
+        if t in float_dtypes:
+            return "%s = %s(%s);" % (z, _fn("fabs", t), x)
+        return "%s = %s;" % (z, x)  # bool and unsigned
+
+    def L_op(self, inputs, outputs, gout):
+        (x,) = inputs
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [x.zeros_like(dtype=config.floatX)]
+        return [gout[0] * sgn(x)]
+
+
+abs_ = Abs(same_out, name="abs_")
+
+
+class Sgn(UnaryScalarOp):
+    def output_types(self, types):
+        if types[0] == bool_:
+            raise TypeError(types[0])
+        return [types[0]]
+
+    def c_code(self, node, inputs, outputs):
+        t = node.inputs[0].type.dtype
+        (x,), (z,) = inputs, outputs
+        if t in float_dtypes:
+            return "%s = (%s > 0) ? 1. : ((%s < 0) ? -1. : (isnan(%s) ? NAN : 0.));" % (z, x, x, x)
+        if t in int_dtypes:
+            return "%s = (%s >= 0) ? (%s == 0) ? 0 : 1 : -1;" % (z, x, x)
+        return "%s = (%s == 0) ? 0 : 1;" % (z, x)
+
+    def L_op(self, inputs, outputs, gout):
+        return _zero_grads(inputs)
+
+
+sgn = Sgn(name="sgn")
+
+
+def _unary_math(cname, fname, grad_fn, policy=upgrade_to_float):
+    """A libm call on the input cast to the output type, the shape every unary
+    math op has in the reference (e.g. ``Exp`` ``theano/scalar/basic.py:2919-2952``)."""
+    class _U(UnaryScalarOp):
+        def c_code(self, node, inputs, outputs):
+            ot = node.outputs[0].type.dtype
+            return "%s = %s((%s)%s);" % (outputs[0], _fn(fname, ot), compute_ctype(ot), inputs[0])
+
+        def L_op(self, inputs, outputs, gout):
+            (x,) = inputs
+            if outputs[0].type.dtype in discrete_dtypes:
+                return [x.zeros_like(dtype=config.floatX)]
+            if grad_fn is None:
+                return _zero_grads(inputs)
+            return [grad_fn(x, outputs[0], gout[0])]
+    _U.__name__ = cname
+    return _U(policy, name=fname if fname != "fabs" else "abs")
+
+
+ceil = _unary_math("Ceil", "ceil", None)
+floor = _unary_math("Floor", "floor", None)
+log = _unary_math("Log", "log", lambda x, z, gz: gz / x)
+log2 = _unary_math("Log2", "log2", lambda x, z, gz: gz / (x * math.log(2.0)))
+log10 = _unary_math("Log10", "log10", lambda x, z, gz: gz / (x * math.log(10.0)))
+log1p = _unary_math("Log1p", "log1p", lambda x, z, gz: gz / (1 + x))
+exp = _unary_math("Exp", "exp", lambda x, z, gz: gz * z)
+exp2 = _unary_math("Exp2", "exp2", lambda x, z, gz: gz * z * math.log(2.0))
+expm1 = _unary_math("Expm1", "expm1", lambda x, z, gz: gz * exp(x))
+sqrt = _unary_math("Sqrt", "sqrt", lambda x, z, gz: (gz * 0.5) / z)
+cos = _unary_math("Cos", "cos", lambda x, z, gz: -gz * sin(x))
+sin = _unary_math("Sin", "sin", lambda x, z, gz: gz * cos(x))
+tan = _unary_math("Tan", "tan", lambda x, z, gz: gz / sqr(cos(x)))
+arccos = _unary_math("ArcCos", "acos", lambda x, z, gz: -gz / sqrt(1 - sqr(x)))
+arcsin = _unary_math("ArcSin", "asin", lambda x, z, gz: gz / sqrt(1 - sqr(x)))
+arctan = _unary_math("ArcTan", "atan", lambda x, z, gz: gz / (1 + sqr(x)))
+cosh = _unary_math("Cosh", "cosh", lambda x, z, gz: gz * sinh(x))
+sinh = _unary_math("Sinh", "sinh", lambda x, z, gz: gz * cosh(x))
+tanh = _unary_math("Tanh", "tanh", lambda x, z, gz: gz * (1 - sqr(z)))
+arccosh = _unary_math("ArcCosh", "acosh", lambda x, z, gz: gz / sqrt(sqr(x) - 1))
+arcsinh = _unary_math("ArcSinh", "asinh", lambda x, z, gz: gz / sqrt(sqr(x) + 1))
+arctanh = _unary_math("ArcTanh", "atanh", lambda x, z, gz: gz / (1 - sqr(x)))
+
+
+class Trunc(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        ot = node.outputs[0].type.dtype
+        fl = _fn("floor", ot)
+        (x,) = inputs
+        return "%s = %s >= 0 ? %s(%s) : -%s(-%s);" % (outputs[0], x, fl, x, fl, x)
+
+    def L_op(self, inputs, outputs, gout):
+        return [inputs[0].zeros_like(dtype=config.floatX)]
+
+
+trunc = Trunc(upgrade_to_float, name="trunc")
+
+
+class RoundHalfToEven(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        ot = node.outputs[0].type.dtype
+        return "%s = %s(%s);" % (outputs[0], _fn("rint", ot), inputs[0])
+
+    def L_op(self, inputs, outputs, gout):
+        return _zero_grads(inputs)
+
+
+class RoundHalfAwayFromZero(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        ot = node.outputs[0].type.dtype
+        return "%s = %s(%s);" % (outputs[0], _fn("round", ot), inputs[0])
+
+    def L_op(self, inputs, outputs, gout):
+        return _zero_grads(inputs)
+
+
+round_half_to_even = RoundHalfToEven(same_out_float_only, name="round_half_to_even")
+round_half_away_from_zero = RoundHalfAwayFromZero(same_out_float_only, name="round_half_away_from_zero")
+
+
+class Neg(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        return "%s = -%s;" % (outputs[0], inputs[0])
+
+    def L_op(self, inputs, outputs, gout):
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [inputs[0].zeros_like(dtype=config.floatX)]
+        return [-gout[0]]
+
+
+neg = Neg(same_out_nobool, name="neg")
+
+
+class Inv(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        return "%s = 1.0 / %s;" % (outputs[0], inputs[0])
+
+    def L_op(self, inputs, outputs, gout):
+        (x,) = inputs
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [x.zeros_like(dtype=config.floatX)]
+        return [-gout[0] / (x * x)]
+
+
+inv = Inv(upgrade_to_float, name="inv")
+
+
+class Sqr(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        return "%s = %s * %s;" % (outputs[0], inputs[0], inputs[0])
+
+    def L_op(self, inputs, outputs, gout):
+        (x,) = inputs
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [x.zeros_like(dtype=config.floatX)]
+        return [gout[0] * x * 2]
+
+
+sqr = Sqr(same_out, name="sqr")
+
+
+class ArcTan2(BinaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        ot = node.outputs[0].type.dtype
+        ct = compute_ctype(ot)
+        return "%s = %s((%s)%s, (%s)%s);" % (outputs[0], _fn("atan2", ot), ct, inputs[0], ct, inputs[1])
+
+    def L_op(self, inputs, outputs, gout):
+        y, x = inputs
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [i.zeros_like(dtype=config.floatX) for i in inputs]
+        den = sqr(x) + sqr(y)
+        return [gz * x / den, -gz * y / den]
+
+
+arctan2 = ArcTan2(upgrade_to_float, name="arctan2")
+
+
+# ---- sigmoid / softplus (theano/tensor/nnet/sigm.py:29-88, 330-372) -------------
+class ScalarSigmoid(UnaryScalarOp):
+    """1/(1+exp(-x)) with the reference's saturation thresholds."""
+
+    def c_code(self, node, inputs, outputs):
+        t = node.inputs[0].type.dtype
+        (x,), (z,) = inputs, outputs
+        if t in ("float32", "float16"):
+            return "%s = %s < -88.0f ? 0.0f : %s > 15.0f ? 1.0f : 1.0f / (1.0f + expf(-%s));" % (z, x, x, x)
+        if t == "float64":
+            return "%s = %s < -709.0 ? 0.0 : %s > 19.0 ? 1.0 : 1.0 / (1.0 + exp(-%s));" % (z, x, x, x)
+        raise NotImplementedError("only floating point is implemented")
+
+    def L_op(self, inputs, outputs, gout):
+        y = scalar_sigmoid(inputs[0])
+        return [gout[0] * y * (1.0 - y)]
+
+
+scalar_sigmoid = ScalarSigmoid(upgrade_to_float, name="scalar_sigmoid")
+
+
+class ScalarSoftplus(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        t = node.inputs[0].type.dtype
+        (x,), (z,) = inputs, outputs
+        if t in ("float32", "float16"):
+            return "%s = %s < -103.0f ? 0.0f : %s > 14.0f ? %s : log1pf(expf(%s));" % (z, x, x, x, x)
+        if t == "float64":
+            return "%s = %s < -745.0 ? 0.0 : %s > 16.0 ? %s : log1p(exp(%s));" % (z, x, x, x, x)
+        raise NotImplementedError("only floating point is implemented")
+
+    def L_op(self, inputs, outputs, gout):
+        return [gout[0] * scalar_sigmoid(inputs[0])]
+
+
+scalar_softplus = ScalarSoftplus(upgrade_to_float, name="scalar_softplus")
+
+
+# --------------------------------------------------------------------------
+class DisconnectedType(Type):
+    """Type of the placeholder gradient for an input the cost does not depend
+    on (``theano/gradient.py``)."""
+
+    def filter(self, data, strict=False, allow_downcast=None):
+        raise AssertionError("a disconnected gradient has no value")
+
+    def __eq__(self, other):
+        return type(self) is type(other)
+
+    def __hash__(self):
+        return hash("DisconnectedType")
+
+    def __str__(self):
+        return "DisconnectedType"
+
+
+# --------------------------------------------------------------------------
+class Composite(ScalarOp):
+    """A scalar sub-graph as one op (``theano/scalar/basic.py:3764-4127``).
+
+    The graph is cloned, nested Composites are inlined, constants are kept
+    inside as literals, and the generated code string is the op's identity
+    (eq / hash), as in the reference (:4085-4112)."""
+
+    def __init__(self, inputs, outputs, name=None):
+        for i in inputs:
+            if not isinstance(i.type, Scalar):
+                raise TypeError("Composite inputs must be scalar variables")
+        inputs, outputs = gof.clone(list(inputs), list(outputs))
+        # inline nested composites
+        changed = True
+        while changed:
+            changed = False
+            for node in gof.io_toposort(inputs, outputs):
+                if isinstance(node.op, Composite):
+                    inner = node.op
+                    memo = dict(zip(inner.inputs, node.inputs))
+                    memo = gof.clone_get_equiv([], inner.outputs, copy_inputs=False, memo=memo)
+                    repl = dict(zip(node.outputs, [memo[o] for o in inner.outputs]))
+                    outputs = [repl.get(o, o) for o in outputs]
+                    for n2 in gof.io_toposort(inputs, outputs):
+                        n2.inputs = [repl.get(i, i) for i in n2.inputs]
+                    changed = True
+                    break
+        self.inputs = inputs
+        self.outputs = outputs
+        self.inputs_type = tuple(i.type for i in inputs)
+        self.outputs_type = tuple(o.type for o in outputs)
+        self.nin = len(inputs)
+        self.nout = len(outputs)
+        self.name = name
+        self.output_types_preference = None
+        self._code = None
+
+    # identity ----------------------------------------------------------------
+    def body(self, innames, outnames, prefix="t"):
+        """Statements computing ``outnames`` from ``innames``; temporaries are
+        declared in the compute type of their dtype, in topological order."""
+        names = dict(zip(self.inputs, innames))
+        lines = []
+        nodes = gof.io_toposort(self.inputs, self.outputs)
+        counter = 0
+        for node in nodes:
+            args = []
+            for i in node.inputs:
+                if i in names:
+                    args.append(names[i])
+                elif isinstance(i, Constant):
+                    args.append(c_literal(i.data, i.type.dtype))
+                else:
+                    raise ValueError("Composite graph uses a variable that is not an input: %s" % i)
+            outs = []
+            for o in node.outputs:
+                nm = "%s%d" % (prefix, counter)
+                counter += 1
+                names[o] = nm
+                outs.append(nm)
+                lines.append("%s %s;" % (compute_ctype(o.type.dtype), nm))
+            lines.append(node.op.c_code(node, args, outs))
+        for o, nm in zip(self.outputs, outnames):
+            if o in names:
+                src = names[o]
+            elif isinstance(o, Constant):
+                src = c_literal(o.data, o.type.dtype)
+            else:
+                raise ValueError("Composite output is not computed from its inputs")
+            lines.append("%s = %s;" % (nm, src))
+        return "\n".join(lines)
+
+    def code_signature(self):
+        if self._code is None:
+            self._code = self.body(["i%d" % k for k in range(self.nin)], ["o%d" % k for k in range(self.nout)])
+        return self._code
+
+    def __eq__(self, other):
+        return (type(self) is type(other) and self.inputs_type == other.inputs_type and
+                self.outputs_type == other.outputs_type and self.code_signature() == other.code_signature())
+
+    def __hash__(self):
+        return hash((type(self), self.inputs_type, self.outputs_type, self.code_signature()))
+
+    def __str__(self):
+        if self.name:
+            return self.name
+        names = dict((i, "i%d" % k) for k, i in enumerate(self.inputs))
+
+        def show(v):
+            if v in names:
+                return names[v]
+            if isinstance(v, Constant):
+                return str(v.data)
+            return "%s(%s)" % (v.owner.op, ", ".join(show(i) for i in v.owner.inputs))
+        return "Composite{%s}" % ", ".join(show(o) for o in self.outputs)
+
+    __repr__ = __str__
+
+    # protocol ----------------------------------------------------------------
+    def output_types(self, types):
+        if tuple(types) != self.inputs_type:
+            raise TypeError("Wrong types for Composite. Expected %s, got %s." % (self.inputs_type, tuple(types)))
+        return list(self.outputs_type)
+
+    def make_node(self, *inputs):
+        inputs = [as_scalar(i) for i in inputs]
+        if tuple(i.type for i in inputs) == self.inputs_type:
+            return Apply(self, inputs, [t() for t in self.outputs_type])
+        # rebuild for the new input types (theano/scalar/basic.py:3998-4015)
+        new_ins = [i.type() for i in inputs]
+        memo = dict(zip(self.inputs, new_ins))
+        for node in gof.io_toposort(self.inputs, self.outputs):
+            args = [memo.get(i, i) for i in node.inputs]
+            new_node = node.op.make_node(*args)
+            for o, no in zip(node.outputs, new_node.outputs):
+                memo[o] = no
+        op = Composite(new_ins, [memo.get(o, o) for o in self.outputs])
+        return Apply(op, inputs, [t() for t in op.outputs_type])
+
+    def c_code(self, node, inputs, outputs):
+        # unique temporary prefix per use so that nested emission cannot clash
+        return "{\n" + self.body(list(inputs), list(outputs), prefix="c%x_" % (id(node) & 0xfffff)) + "\n}"
+
+    def L_op(self, inputs, outputs, gout):
+        raise NotImplementedError("grad is not implemented for Composite")
+
+    def __getstate__(self):
+        d = dict(self.__dict__)
+        d["_code"] = None
+        return d

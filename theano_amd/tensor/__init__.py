@@ -1,0 +1,9 @@
+"""Tensor-level API: types, elementwise functions and reductions."""
+from .type import (TensorType, TensorVariable, TensorConstant, as_tensor_variable, constant, tensor, scalar, vector,
+                   matrix, row, col, tensor3, tensor4, bscalar, bvector, bmatrix, wscalar, wvector, wmatrix, iscalar,
+                   ivector, imatrix, itensor3, itensor4, lscalar, lvector, lmatrix, ltensor3, ltensor4, hscalar,
+                   hvector, hmatrix, htensor3, htensor4, fscalar, fvector, fmatrix, frow, fcol, ftensor3, ftensor4,
+                   dscalar, dvector, dmatrix, drow, dcol, dtensor3, dtensor4)
+from .elemwise import DimShuffle, Elemwise, CAReduce, CAReduceDtype, Sum, Prod, All, Any
+from .basic import *  # noqa: F401,F403
+from .basic import Max, Min, ShapeFloat, makeKeepDims, cast, round  # noqa: F401

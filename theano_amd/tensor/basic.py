@@ -1,0 +1,324 @@
+"""User-level tensor functions: one Elemwise instance per ScalarOp, casts,
+fills and the reduction front-ends.
+
+Mirrors the on-path parts of ``theano/tensor/basic.py``: ``_scal_elemwise``
+:975-1020, ``makeKeepDims`` :1613-1647, ``max``/``min`` :1682-1775,
+``sum``/``prod`` :3190-3244, ``mean`` :3291-3382, ``var``/``std`` :3386-3480,
+``any``/``all`` :6353-6366, and ``sigmoid``/``softplus`` of
+``theano/tensor/nnet/sigm.py:167-168, 372``.
+"""
+import numpy as np
+
+from .. import scalar as scal
+from ..config import config
+from ..gof import Apply, Op
+from .elemwise import All, Any, CAReduce, DimShuffle, Elemwise, Prod, Sum
+from .type import TensorType, as_tensor_variable, constant
+
+discrete_dtypes = scal.discrete_dtypes
+continuous_dtypes = scal.continuous_dtypes
+int_dtypes = scal.int_dtypes
+uint_dtypes = scal.uint_dtypes
+
+
+def _elemwise(scalar_op, name):
+    return Elemwise(scalar_op, name="Elemwise{%s}" % name)
+
+
+lt, gt, le, ge = _elemwise(scal.lt, "lt"), _elemwise(scal.gt, "gt"), _elemwise(scal.le, "le"), _elemwise(scal.ge, "ge")
+eq, neq = _elemwise(scal.eq, "eq"), _elemwise(scal.neq, "neq")
+isnan, isinf = _elemwise(scal.isnan, "isnan"), _elemwise(scal.isinf, "isinf")
+switch = _elemwise(scal.switch, "switch")
+where = switch
+and_, or_, xor, invert = (_elemwise(scal.and_, "and_"), _elemwise(scal.or_, "or_"), _elemwise(scal.xor, "xor"),
+                          _elemwise(scal.invert, "invert"))
+bitwise_and, bitwise_or, bitwise_xor, bitwise_not = and_, or_, xor, invert
+right_shift, left_shift = _elemwise(scal.right_shift, "right_shift"), _elemwise(scal.left_shift, "left_shift")
+maximum, minimum = _elemwise(scal.maximum, "maximum"), _elemwise(scal.minimum, "minimum")
+add, mul, sub = _elemwise(scal.add, "add"), _elemwise(scal.mul, "mul"), _elemwise(scal.sub, "sub")
+true_div, int_div, mod = _elemwise(scal.true_div, "true_div"), _elemwise(scal.int_div, "int_div"), _elemwise(scal.mod, "mod")
+pow, clip, second = _elemwise(scal.pow, "pow"), _elemwise(scal.clip, "clip"), _elemwise(scal.second, "second")
+fill = second
+tensor_copy = _elemwise(scal.identity, "identity")
+abs_, sgn, neg, inv = _elemwise(scal.abs_, "abs_"), _elemwise(scal.sgn, "sgn"), _elemwise(scal.neg, "neg"), _elemwise(scal.inv, "inv")
+ceil, floor, trunc = _elemwise(scal.ceil, "ceil"), _elemwise(scal.floor, "floor"), _elemwise(scal.trunc, "trunc")
+round_half_to_even = _elemwise(scal.round_half_to_even, "round_half_to_even")
+round_half_away_from_zero = _elemwise(scal.round_half_away_from_zero, "round_half_away_from_zero")
+log, log2, log10, log1p = _elemwise(scal.log, "log"), _elemwise(scal.log2, "log2"), _elemwise(scal.log10, "log10"), _elemwise(scal.log1p, "log1p")
+exp, exp2, expm1 = _elemwise(scal.exp, "exp"), _elemwise(scal.exp2, "exp2"), _elemwise(scal.expm1, "expm1")
+sqr, sqrt = _elemwise(scal.sqr, "sqr"), _elemwise(scal.sqrt, "sqrt")
+cos, sin, tan = _elemwise(scal.cos, "cos"), _elemwise(scal.sin, "sin"), _elemwise(scal.tan, "tan")
+arccos, arcsin, arctan, arctan2 = (_elemwise(scal.arccos, "arccos"), _elemwise(scal.arcsin, "arcsin"),
+                                   _elemwise(scal.arctan, "arctan"), _elemwise(scal.arctan2, "arctan2"))
+cosh, sinh, tanh = _elemwise(scal.cosh, "cosh"), _elemwise(scal.sinh, "sinh"), _elemwise(scal.tanh, "tanh")
+arccosh, arcsinh, arctanh = _elemwise(scal.arccosh, "arccosh"), _elemwise(scal.arcsinh, "arcsinh"), _elemwise(scal.arctanh, "arctanh")
+sigmoid = _elemwise(scal.scalar_sigmoid, "sigmoid")
+softplus = _elemwise(scal.scalar_softplus, "softplus")
+
+
+def div_proxy(x, y):
+    """``x / y``: integer or true division by operand types
+    (``theano/tensor/basic.py`` ``div_proxy``, ``theano/scalar/basic.py:1826-1885``)."""
+    x, y = as_tensor_variable(x), as_tensor_variable(y)
+    f = scal.int_or_true_div(x.type.dtype in discrete_dtypes, y.type.dtype in discrete_dtypes)
+    return (int_div if f is scal.int_div else true_div)(x, y)
+
+
+_cast_ops = dict((dt, Elemwise(scal._cast_mapping[dt], name="Elemwise{Cast{%s}}" % dt)) for dt in scal.all_dtypes)
+
+
+def cast(x, dtype):
+    if dtype == "floatX":
+        dtype = config.floatX
+    dtype = str(dtype)
+    x = as_tensor_variable(x)
+    if x.type.dtype == dtype:
+        return x
+    return _cast_ops[dtype](x)
+
+
+def zeros_like(model, dtype=None):
+    model = as_tensor_variable(model)
+    if dtype is None:
+        dtype = model.type.dtype
+    return fill(model, constant(0, dtype=dtype))
+
+
+def ones_like(model, dtype=None):
+    model = as_tensor_variable(model)
+    if dtype is None:
+        dtype = model.type.dtype
+    return fill(model, constant(1, dtype=dtype))
+
+
+def round(a, mode="half_away_from_zero"):
+    if mode == "half_away_from_zero":
+        return round_half_away_from_zero(a)
+    if mode == "half_to_even":
+        return round_half_to_even(a)
+    raise Exception("round mode %s is not implemented." % mode)
+
+
+def tensor_from_scalar(s):
+    raise NotImplementedError("scalar variables cannot be turned into tensors here; use a 0-d tensor")
+
+
+# --------------------------------------------------------------------------
+class ShapeFloat(Op):
+    """Extent of dimension ``i`` of the input as a 0-d floating tensor.
+
+    Stands for ``cast(shape(x)[i], dtype)`` in ``mean`` / ``var``
+    (``theano/tensor/basic.py:3352-3373``).  It runs on the host and reads only
+    array metadata, whichever memory the array lives in; fused consumers take
+    its value as a kernel argument."""
+
+    __props__ = ("i", "dtype")
+
+    def __init__(self, i, dtype):
+        self.i = int(i)
+        self.dtype = str(dtype)
+
+    def make_node(self, x):
+        x = x if hasattr(x.type, "ndim") else as_tensor_variable(x)
+        if self.i >= x.type.ndim:
+            raise TypeError("x has too few dimensions for ShapeFloat", (x, self.i))
+        return Apply(self, [x], [TensorType(self.dtype, ())()])
+
+    def perform(self, node, inputs, output_storage):
+        output_storage[0][0] = np.asarray(inputs[0].shape[self.i], dtype=self.dtype)
+
+    def infer_shape(self, node, shapes):
+        return [()]
+
+    def connection_pattern(self, node):
+        return [[False]]
+
+    def grad(self, inp, grads):
+        return [scal.DisconnectedType()()]
+
+
+# --------------------------------------------------------------------------
+def _axis_list(axis, ndim):
+    if axis is None:
+        return list(range(ndim))
+    if isinstance(axis, (int, np.integer)):
+        axis = [int(axis)]
+    elif isinstance(axis, np.ndarray) and axis.ndim == 0:
+        axis = [int(axis)]
+    else:
+        axis = [int(a) for a in axis]
+    return axis
+
+
+def makeKeepDims(x, y, axis):
+    """Re-insert, with length one, the axes of ``x`` that a reduction dropped."""
+    x, y = as_tensor_variable(x), as_tensor_variable(y)
+    newaxis = [a + x.type.ndim if a < 0 else a for a in _axis_list(axis, x.type.ndim)]
+    i, new_dims = 0, []
+    for j in range(x.type.ndim):
+        if j in newaxis:
+            new_dims.append("x")
+        else:
+            new_dims.append(i)
+            i += 1
+    return DimShuffle(y.type.broadcastable, new_dims)(y)
+
+
+def sum(input, axis=None, dtype=None, keepdims=False, acc_dtype=None):
+    out = Sum(axis=axis, dtype=dtype, acc_dtype=acc_dtype)(input)
+    if keepdims:
+        out = makeKeepDims(input, out, axis)
+    return out
+
+
+def prod(input, axis=None, dtype=None, keepdims=False, acc_dtype=None, no_zeros_in_input=False):
+    out = Prod(axis, dtype=dtype, acc_dtype=acc_dtype, no_zeros_in_input=no_zeros_in_input)(input)
+    if keepdims:
+        out = makeKeepDims(input, out, axis)
+    return out
+
+
+class Max(CAReduce):
+    """``CAReduce{maximum}`` carrying the gradient of the reference's
+    ``MaxAndArgmax`` (``theano/tensor/basic.py:1429-1483``), which is what
+    ``tensor.max`` becomes once ``local_max_and_argmax``
+    (``theano/tensor/opt_uncanonicalize.py:51-68``) has run."""
+
+    __props__ = ("axis",)
+
+    def __init__(self, axis=None):
+        CAReduce.__init__(self, scal.maximum, axis)
+
+    def _props(self):
+        return (self.axis,)
+
+    def __str__(self):
+        return "Max" if self.axis is None else "Max{%s}" % ", ".join(map(str, self.axis))
+
+    def L_op(self, inp, out, grads):
+        (x,) = inp
+        (g_max,) = grads
+        if x.type.dtype in discrete_dtypes:
+            return [x.zeros_like(dtype=config.floatX)]
+        axis = self.axis if self.axis is not None else tuple(range(x.type.ndim))
+        pattern, k = [], 0
+        for i in range(x.type.ndim):
+            if i in axis:
+                pattern.append("x")
+            else:
+                pattern.append(k)
+                k += 1
+        g_max_pad = DimShuffle(g_max.type.broadcastable, pattern)(g_max)
+        xmax_pad = DimShuffle(out[0].type.broadcastable, pattern)(out[0])
+        return [eq(xmax_pad, x) * g_max_pad]
+
+
+class Min(CAReduce):
+    """``CAReduce{minimum}`` (what ``local_max_to_min`` produces,
+    ``theano/tensor/opt_uncanonicalize.py:71-94``)."""
+
+    __props__ = ("axis",)
+
+    def __init__(self, axis=None):
+        CAReduce.__init__(self, scal.minimum, axis)
+
+    def _props(self):
+        return (self.axis,)
+
+    def __str__(self):
+        return "Min" if self.axis is None else "Min{%s}" % ", ".join(map(str, self.axis))
+
+    L_op = Max.L_op
+
+
+def max(x, axis=None, keepdims=False):
+    x = as_tensor_variable(x)
+    out = Max(axis)(x)
+    if keepdims:
+        out = makeKeepDims(x, out, axis)
+    return out
+
+
+def min(x, axis=None, keepdims=False):
+    x = as_tensor_variable(x)
+    out = Min(axis)(x)
+    if keepdims:
+        out = makeKeepDims(x, out, axis)
+    return out
+
+
+def mean(input, axis=None, dtype=None, keepdims=False, acc_dtype=None):
+    """Sum divided by the extent of every reduced axis in turn; float16 inputs
+    are summed in float32 and the result is cast back."""
+    input = as_tensor_variable(input)
+    if dtype is not None:
+        sum_dtype = dtype
+    else:
+        sum_dtype = "float32" if input.type.dtype == "float16" else None
+    s = sum(input, axis=axis, dtype=sum_dtype, keepdims=keepdims, acc_dtype=acc_dtype)
+    shp_dtype = "float32" if s.type.dtype in ("float16", "float32") else "float64"
+    for i in _axis_list(axis, input.type.ndim):
+        s = true_div(s, ShapeFloat(i if i >= 0 else i + input.type.ndim, shp_dtype)(input))
+    if s.type.dtype in discrete_dtypes:
+        s = cast(s, shp_dtype)
+    if dtype == "float16" or (dtype is None and input.type.dtype == "float16"):
+        s = cast(s, "float16")
+    s.name = "mean"
+    return s
+
+
+def var(input, axis=None, ddof=0, keepdims=False, corrected=False):
+    """Two-pass variance: mean of the squared deviations from the mean."""
+    if isinstance(ddof, bool):
+        raise ValueError("Parameter keepdims is now at index 3: (input, axis=None, ddof=0, keepdims=False, "
+                         "corrected=False)")
+    input = as_tensor_variable(input)
+    axis = _axis_list(axis, input.type.ndim)
+    mean_input = mean(input, axis, keepdims=True)
+    centered = input - mean_input
+    two = constant(2, dtype=centered.type.dtype)
+    if ddof == 0:
+        v = mean(centered ** two, axis, keepdims=keepdims)
+    else:
+        v = sum(centered ** two, axis=axis, keepdims=keepdims)
+        for i in axis:
+            v = true_div(v, ShapeFloat(i, "float64")(input) - ddof)
+    if corrected:
+        if ddof == 0:
+            error = mean(centered, axis, keepdims=keepdims) ** 2
+        else:
+            error = sum(centered, axis=axis, keepdims=keepdims) ** 2
+            for i in axis:
+                n = ShapeFloat(i, "float64")(input)
+                error = true_div(error, (n - ddof) * n)
+        v = v - error
+    v.name = "var"
+    return v
+
+
+def std(input, axis=None, ddof=0, keepdims=False, corrected=False):
+    ret = sqrt(var(input, axis=axis, ddof=ddof, keepdims=keepdims, corrected=corrected))
+    ret.name = "std"
+    return ret
+
+
+def any(x, axis=None, keepdims=False):
+    out = Any(axis)(x)
+    if keepdims:
+        out = makeKeepDims(x, out, axis)
+    return out
+
+
+def all(x, axis=None, keepdims=False):
+    out = All(axis)(x)
+    if keepdims:
+        out = makeKeepDims(x, out, axis)
+    return out
+
+
+def softmax(x):
+    """Row softmax written with Elemwise and CAReduce nodes, the graph the
+    reference's ``softmax_simplifier`` recognises (``theano/tensor/nnet/nnet.py:888-925``)."""
+    x = as_tensor_variable(x)
+    e = exp(x - max(x, axis=-1, keepdims=True))
+    return e / sum(e, axis=-1, keepdims=True)

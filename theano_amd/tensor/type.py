@@ -1,0 +1,288 @@
+"""TensorType, tensor variables and constants.
+
+Mirrors ``theano/tensor/type.py:15-610`` (dtype + broadcastable pattern,
+``filter``) and the operator overloads of ``theano/tensor/var.py:38-830``.
+"""
+import numpy as np
+
+from .. import scalar as scal
+from ..config import config
+from ..gof import Apply, Constant, Type, Variable
+
+
+class TensorType(Type):
+    """dtype plus, per dimension, whether its extent is known to be 1."""
+
+    def __init__(self, dtype, broadcastable, name=None):
+        if dtype == "floatX":
+            dtype = config.floatX
+        self.dtype = str(dtype)
+        if self.dtype not in scal.all_dtypes:
+            raise TypeError("Unsupported dtype for TensorType: %s" % self.dtype)
+        self.broadcastable = tuple(bool(b) for b in broadcastable)
+        self.ndim = len(self.broadcastable)
+        self.name = name
+        self.numpy_dtype = np.dtype(self.dtype)
+
+    def clone(self, dtype=None, broadcastable=None):
+        return type(self)(self.dtype if dtype is None else dtype,
+                          self.broadcastable if broadcastable is None else broadcastable)
+
+    def filter(self, data, strict=False, allow_downcast=None):
+        """Convert ``data`` to an ndarray of this type or raise TypeError
+        (``theano/tensor/type.py:95-236``)."""
+        if isinstance(data, np.ndarray) and data.dtype == self.numpy_dtype:
+            pass
+        elif strict:
+            raise TypeError("%s expected a ndarray object with dtype = %s (got %s)." %
+                            (self, self.numpy_dtype, getattr(data, "dtype", type(data))))
+        else:
+            arr = np.asarray(data)
+            if allow_downcast or arr.dtype == self.numpy_dtype:
+                data = np.asarray(arr, dtype=self.dtype)
+            else:
+                up = scal.upcast(self.dtype, str(arr.dtype)) if str(arr.dtype) in scal.all_dtypes else None
+                python_number = isinstance(data, (int, float, bool)) or (
+                    isinstance(data, (list, tuple)) and arr.dtype in (np.float64, np.int64))
+                if up == self.dtype or python_number:
+                    data = np.asarray(arr, dtype=self.dtype)
+                else:
+                    raise TypeError("%s cannot store a value of dtype %s without risking loss of precision." %
+                                    (self, arr.dtype))
+        if data.ndim != self.ndim:
+            raise TypeError("Wrong number of dimensions: expected %s, got %s with shape %s." %
+                            (self.ndim, data.ndim, data.shape))
+        for i, b in enumerate(self.broadcastable):
+            if b and data.shape[i] != 1:
+                raise TypeError("Non-unit value on shape on a broadcastable dimension.", data.shape,
+                                self.broadcastable)
+        return data
+
+    def __eq__(self, other):
+        return (type(self) is type(other) and self.dtype == other.dtype and
+                self.broadcastable == other.broadcastable)
+
+    def __hash__(self):
+        return hash((type(self), self.dtype, self.broadcastable))
+
+    def __str__(self):
+        if self.name:
+            return self.name
+        names = {(): "scalar", (False,): "vector", (False, True): "col", (True, False): "row",
+                 (False, False): "matrix"}
+        b = self.broadcastable
+        bcast = names.get(b, "%dD" % len(b) if not any(b) else str(b))
+        return "TensorType(%s, %s)" % (self.dtype, bcast)
+
+    __repr__ = __str__
+
+    @staticmethod
+    def values_eq_approx(a, b, rtol=None, atol=None):
+        if a.shape != b.shape or a.dtype != b.dtype:
+            return False
+        if a.dtype.kind in "biu":
+            return bool(np.array_equal(a, b))
+        tol = {"float16": 1e-3, "float32": 1e-5, "float64": 1e-8}[str(a.dtype)]
+        return bool(np.allclose(a, b, rtol=rtol or 1e-5, atol=atol or tol, equal_nan=True))
+
+
+class _tensor_py_operators(object):
+    """Arithmetic, comparison and reduction sugar on tensor variables."""
+
+    dtype = property(lambda self: self.type.dtype)
+    ndim = property(lambda self: self.type.ndim)
+    broadcastable = property(lambda self: self.type.broadcastable)
+
+    def _b(self):
+        from . import basic
+        return basic
+
+    def __abs__(self): return self._b().abs_(self)
+    def __neg__(self): return self._b().neg(self)
+    def __invert__(self): return self._b().invert(self)
+    def __lt__(self, o): return self._b().lt(self, o)
+    def __le__(self, o): return self._b().le(self, o)
+    def __gt__(self, o): return self._b().gt(self, o)
+    def __ge__(self, o): return self._b().ge(self, o)
+    def __and__(self, o): return self._b().and_(self, o)
+    def __or__(self, o): return self._b().or_(self, o)
+    def __xor__(self, o): return self._b().xor(self, o)
+    def __rand__(self, o): return self._b().and_(o, self)
+    def __ror__(self, o): return self._b().or_(o, self)
+    def __rxor__(self, o): return self._b().xor(o, self)
+    def __rshift__(self, o): return self._b().right_shift(self, o)
+    def __lshift__(self, o): return self._b().left_shift(self, o)
+    def __add__(self, o): return self._b().add(self, o)
+    def __sub__(self, o): return self._b().sub(self, o)
+    def __mul__(self, o): return self._b().mul(self, o)
+    def __truediv__(self, o): return self._b().div_proxy(self, o)
+    __div__ = __truediv__
+    def __floordiv__(self, o): return self._b().int_div(self, o)
+    def __mod__(self, o): return self._b().mod(self, o)
+    def __pow__(self, o): return self._b().pow(self, o)
+    def __radd__(self, o): return self._b().add(o, self)
+    def __rsub__(self, o): return self._b().sub(o, self)
+    def __rmul__(self, o): return self._b().mul(o, self)
+    def __rtruediv__(self, o): return self._b().div_proxy(o, self)
+    __rdiv__ = __rtruediv__
+    def __rfloordiv__(self, o): return self._b().int_div(o, self)
+    def __rmod__(self, o): return self._b().mod(o, self)
+    def __rpow__(self, o): return self._b().pow(o, self)
+
+    # -- views and casts
+    def dimshuffle(self, *pattern):
+        from .elemwise import DimShuffle
+        if len(pattern) == 1 and isinstance(pattern[0], (list, tuple)):
+            pattern = pattern[0]
+        return DimShuffle(self.type.broadcastable, pattern)(self)
+
+    @property
+    def T(self):
+        return self.dimshuffle(*reversed(range(self.ndim)))
+
+    def astype(self, dtype):
+        return self._b().cast(self, dtype)
+
+    def zeros_like(self, dtype=None):
+        return self._b().zeros_like(self, dtype=dtype)
+
+    def ones_like(self, dtype=None):
+        return self._b().ones_like(self, dtype=dtype)
+
+    # -- reductions
+    def sum(self, axis=None, dtype=None, keepdims=False, acc_dtype=None):
+        return self._b().sum(self, axis=axis, dtype=dtype, keepdims=keepdims, acc_dtype=acc_dtype)
+
+    def prod(self, axis=None, dtype=None, keepdims=False, acc_dtype=None):
+        return self._b().prod(self, axis=axis, dtype=dtype, keepdims=keepdims, acc_dtype=acc_dtype)
+
+    def mean(self, axis=None, dtype=None, keepdims=False, acc_dtype=None):
+        return self._b().mean(self, axis=axis, dtype=dtype, keepdims=keepdims, acc_dtype=acc_dtype)
+
+    def var(self, axis=None, ddof=0, keepdims=False, corrected=False):
+        return self._b().var(self, axis=axis, ddof=ddof, keepdims=keepdims, corrected=corrected)
+
+    def std(self, axis=None, ddof=0, keepdims=False, corrected=False):
+        return self._b().std(self, axis=axis, ddof=ddof, keepdims=keepdims, corrected=corrected)
+
+    def max(self, axis=None, keepdims=False):
+        return self._b().max(self, axis=axis, keepdims=keepdims)
+
+    def min(self, axis=None, keepdims=False):
+        return self._b().min(self, axis=axis, keepdims=keepdims)
+
+    def any(self, axis=None, keepdims=False):
+        return self._b().any(self, axis=axis, keepdims=keepdims)
+
+    def all(self, axis=None, keepdims=False):
+        return self._b().all(self, axis=axis, keepdims=keepdims)
+
+
+class TensorVariable(_tensor_py_operators, Variable):
+    pass
+
+
+class TensorConstant(_tensor_py_operators, Constant):
+    def signature(self):
+        a = np.asarray(self.data)
+        return (self.type, a.shape, a.tobytes())
+
+    def __str__(self):
+        if self.name is not None:
+            return self.name
+        a = np.asarray(self.data)
+        return "TensorConstant{%s}" % (a if a.size <= 4 else "shape %s" % (a.shape,))
+
+    __repr__ = __str__
+
+
+TensorType.Variable = TensorVariable
+TensorType.Constant = TensorConstant
+
+
+def constant(x, name=None, ndim=None, dtype=None):
+    """Tensor constant; every extent-1 dimension is broadcastable
+    (``theano/tensor/basic.py:211-262``)."""
+    x_ = scal.convert(x, dtype=dtype)
+    if str(x_.dtype) not in scal.all_dtypes:
+        raise TypeError("cannot make a tensor constant of dtype %s" % x_.dtype)
+    bcast = [s == 1 for s in x_.shape]
+    if ndim is not None:
+        if len(bcast) < ndim:
+            bcast = [True] * (ndim - len(bcast)) + bcast
+            x_ = x_.reshape((1,) * (ndim - x_.ndim) + x_.shape)
+        elif len(bcast) > ndim:
+            raise ValueError("constant has %d dimensions, asked for %d" % (len(bcast), ndim))
+    return TensorConstant(TensorType(str(x_.dtype), bcast), np.ascontiguousarray(x_), name=name)
+
+
+def as_tensor_variable(x, name=None, ndim=None):
+    if isinstance(x, Apply):
+        x = x.default_output()
+    if isinstance(x, Variable):
+        if isinstance(x.type, scal.Scalar):
+            from .basic import tensor_from_scalar
+            x = tensor_from_scalar(x)
+        if not isinstance(x.type, TensorType):
+            to_tensor = getattr(x.type, "as_tensor_variable", None)
+            if to_tensor is None:
+                raise TypeError("Variable type field must be a TensorType.", x, x.type)
+            x = to_tensor(x)
+        if ndim is not None and x.type.ndim != ndim:
+            if x.type.ndim < ndim:
+                x = x.dimshuffle(*(["x"] * (ndim - x.type.ndim) + list(range(x.type.ndim))))
+            else:
+                raise ValueError("TensorType could not be cast to have %i dimensions" % ndim, x.type)
+        return x
+    if isinstance(x, (tuple, list)) and any(isinstance(i, Variable) for i in x):
+        raise TypeError("lists of symbolic variables are not supported here")
+    return constant(x, name=name, ndim=ndim)
+
+
+def _mk(dtype, bcast):
+    def make(name=None):
+        return TensorType(dtype, bcast)(name)
+    return make
+
+
+for _p, _dt in (("b", "int8"), ("w", "int16"), ("i", "int32"), ("l", "int64"), ("h", "float16"),
+                ("f", "float32"), ("d", "float64")):
+    globals()[_p + "scalar"] = _mk(_dt, ())
+    globals()[_p + "vector"] = _mk(_dt, (False,))
+    globals()[_p + "matrix"] = _mk(_dt, (False, False))
+    globals()[_p + "row"] = _mk(_dt, (True, False))
+    globals()[_p + "col"] = _mk(_dt, (False, True))
+    globals()[_p + "tensor3"] = _mk(_dt, (False,) * 3)
+    globals()[_p + "tensor4"] = _mk(_dt, (False,) * 4)
+
+
+def scalar(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, ())(name)
+
+
+def vector(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, (False,))(name)
+
+
+def matrix(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, (False, False))(name)
+
+
+def row(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, (True, False))(name)
+
+
+def col(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, (False, True))(name)
+
+
+def tensor3(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, (False,) * 3)(name)
+
+
+def tensor4(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, (False,) * 4)(name)
+
+
+def tensor(dtype, broadcastable, name=None):
+    return TensorType(dtype, broadcastable)(name)
