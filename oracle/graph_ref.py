@@ -1,0 +1,192 @@
+"""TEST INFRASTRUCTURE - not part of the product.  Only ``tests/``, the
+``cpu_baseline`` leg of ``bench.py`` and ``__graft_entry__.smoke()`` may import
+anything under ``oracle/``.
+
+Evaluates an *unlifted, unfused* theano_amd graph on the CPU the way Theano's
+own backend would node by node:
+
+* ``Elemwise``: broadcast check of ``Elemwise.perform``
+  (``theano/tensor/elemwise.py:720-740``), then the scalar op's C semantics
+  from ``oracle.scalar_ref`` applied to whole arrays; Composite nodes are
+  evaluated op by op.
+* ``CAReduce`` family: dtype tables re-stated here from
+  ``theano/tensor/elemwise.py:1721-1759``, sequential accumulation in the
+  accumulator dtype by ``oracle/careduce.c`` (the loop nest of
+  ``theano/tensor/elemwise_cgen.py:465-527``), then the cast to the output
+  dtype (``elemwise.py:1549-1554``).  Zero-length max / min raise ValueError
+  (``elemwise.py:1489-1506``).
+* ``DimShuffle``: the strided view of ``theano/tensor/c_code/dimshuffle.c:55-98``.
+
+Pinned by tests/test_oracle_graph.py against the reference's literal test
+answers (``theano/tensor/tests/test_elemwise.py:654-748, 953-966``; fusion table
+``theano/tensor/tests/test_opt.py:964-1112``) and NumPy closed forms.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+from . import scalar_ref
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "_build", "liboracle.so")
+_lib = None
+
+_DT_CODE = {"bool": 0, "int8": 1, "uint8": 2, "int16": 3, "uint16": 4, "int32": 5, "uint32": 6, "int64": 7,
+            "uint64": 8, "float16": 9, "float32": 10, "float64": 11}
+_OP_CODE = {"Add": 0, "Mul": 1, "Maximum": 2, "Minimum": 3, "AND": 4, "OR": 5, "XOR": 6}
+
+# theano/tensor/elemwise.py:1733-1741 and :1748-1759
+SUM_OUT_DTYPE = dict(bool="int64", int8="int64", int16="int64", int32="int64", uint8="uint64", uint16="uint64",
+                     uint32="uint64")
+SUM_ACC_DTYPE = dict(bool="int64", int8="int64", int16="int64", int32="int64", uint8="uint64", uint16="uint64",
+                     uint32="uint64", float16="float32", float32="float64")
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            from . import build
+            build.build()
+        _lib = ctypes.CDLL(_LIB)
+        _lib.oracle_careduce.restype = ctypes.c_int
+    return _lib
+
+
+def reduce_identity(op_name, dtype):
+    """theano/tensor/elemwise.py:1470-1488 and the ops' own identities
+    (theano/scalar/basic.py:1554, 1570, 1586, 1700, 1742)."""
+    dt = np.dtype(dtype)
+    if op_name == "Add" or op_name in ("OR", "XOR"):
+        return np.zeros((), dt)
+    if op_name == "Mul":
+        return np.ones((), dt)
+    if op_name == "AND":
+        return np.asarray(True) if dt == np.bool_ else np.asarray(-1).astype(dt)
+    if op_name in ("Maximum", "Minimum"):
+        big = op_name == "Minimum"
+        if dt.kind == "f":
+            return np.asarray(np.inf if big else -np.inf, dt)
+        if dt == np.bool_:
+            return np.asarray(big)
+        info = np.iinfo(dt)
+        return np.asarray(info.max if big else info.min, dt)
+    raise NotImplementedError(op_name)
+
+
+def careduce(x, op_name, axis, acc_dtype, out_dtype):
+    """Sequential CAReduce of a (possibly strided) host array."""
+    x = np.asarray(x)
+    nd = x.ndim
+    axis = tuple(range(nd)) if axis is None else tuple(a + nd if a < 0 else a for a in axis)
+    if op_name in ("Maximum", "Minimum") and any(x.shape[a] == 0 for a in axis):
+        raise ValueError("Input of CAReduce{%s} has zero-size on axis %s" % (op_name.lower(), axis))
+    acc_dtype, out_dtype = str(acc_dtype), str(out_dtype)
+    if x.dtype == np.float16:
+        x = x.astype("float32")  # no float16 C code exists in the reference (elemwise.py:1395-1398)
+    kept = tuple(s for d, s in enumerate(x.shape) if d not in axis)
+    acc = np.empty(kept, dtype=acc_dtype)
+    ident = reduce_identity(op_name, acc_dtype)
+    shape = (ctypes.c_int64 * max(nd, 1))(*x.shape)
+    strides = (ctypes.c_int64 * max(nd, 1))(*x.strides)
+    mask = (ctypes.c_uint8 * max(nd, 1))(*[1 if d in axis else 0 for d in range(nd)])
+    rc = lib().oracle_careduce(_OP_CODE[op_name], _DT_CODE[str(x.dtype)], _DT_CODE[acc_dtype], nd, shape, strides, mask,
+                               ctypes.c_void_p(x.ctypes.data), ctypes.c_void_p(ident.ctypes.data),
+                               ctypes.c_void_p(acc.ctypes.data))
+    if rc != 0:
+        raise NotImplementedError("no C restatement for %s over %s accumulated in %s" % (op_name, x.dtype, acc_dtype))
+    if out_dtype == "bool":
+        return acc != 0
+    return acc.astype(out_dtype)
+
+
+def dimshuffle(x, new_order, drop_check=True):
+    x = np.asarray(x)
+    shuffle = [o for o in new_order if o != "x"]
+    drop = [d for d in range(x.ndim) if d not in shuffle]
+    for d in drop:
+        if x.shape[d] != 1:
+            raise ValueError("cannot drop a dimension of extent %d" % x.shape[d])
+    res = x.transpose(shuffle + drop) if x.ndim else x
+    shape = list(res.shape[:len(shuffle)])
+    for i, o in enumerate(new_order):
+        if o == "x":
+            shape.insert(i, 1)
+    return res.reshape(shape)
+
+
+def _check_broadcast(node, values):
+    nd = node.outputs[0].type.ndim
+    shape, owner = [1] * nd, [None] * nd
+    for k, (var, val) in enumerate(zip(node.inputs, values)):
+        for d in range(nd):
+            if var.type.broadcastable[d]:
+                if val.shape[d] != 1:
+                    raise ValueError("input %d has extent %d on broadcastable dimension %d" % (k, val.shape[d], d))
+                continue
+            if owner[d] is None:
+                owner[d], shape[d] = k, val.shape[d]
+            elif val.shape[d] != shape[d]:
+                raise ValueError("Input dimension mis-match. (input[%d].shape[%d] = %d, input[%d].shape[%d] = %d)"
+                                 % (owner[d], d, shape[d], k, d, val.shape[d]))
+
+
+def eval_scalar_op(op, in_values, out_dtypes):
+    """Evaluate a theano_amd ScalarOp (or Composite) over whole arrays."""
+    name = type(op).__name__
+    if name == "Composite":
+        from theano_amd import gof
+        env = dict(zip(op.inputs, in_values))
+        for node in gof.io_toposort(op.inputs, op.outputs):
+            args = [env[i] if i in env else np.asarray(i.data) for i in node.inputs]
+            outs = eval_scalar_op(node.op, args, [o.type.dtype for o in node.outputs])
+            for o, v in zip(node.outputs, outs):
+                env[o] = v
+        return [env[o] if o in env else np.asarray(o.data) for o in op.outputs]
+    fn = scalar_ref.BY_CLASS.get(name)
+    if fn is None:
+        raise NotImplementedError("no restatement of scalar op %s" % name)
+    return [np.asarray(fn(out_dtypes[0], *[np.asarray(v) for v in in_values]))]
+
+
+def evaluate(inputs, outputs, values):
+    """Values of ``outputs`` (theano_amd variables) given ``values`` for
+    ``inputs``; every Apply node is computed separately, as an unfused graph."""
+    from theano_amd import gof
+    from theano_amd.tensor.elemwise import CAReduce, CAReduceDtype, DimShuffle, Elemwise
+    from theano_amd.tensor.basic import ShapeFloat
+    env = {}
+    for var, val in zip(inputs, values):
+        env[var] = var.type.filter(np.asarray(val), strict=False, allow_downcast=False)
+    for node in gof.io_toposort(inputs, outputs):
+        args = [env[i] if i in env else np.asarray(i.data) for i in node.inputs]
+        op = node.op
+        if isinstance(op, Elemwise):
+            _check_broadcast(node, args)
+            res = eval_scalar_op(op.scalar_op, args, [o.type.dtype for o in node.outputs])
+            shape = np.broadcast_shapes(*[a.shape for a in args])
+            res = [np.broadcast_to(r, shape).astype(o.type.dtype, copy=False) if o.type.dtype != "bool"
+                   else np.broadcast_to(r, shape) != 0 for r, o in zip(res, node.outputs)]
+        elif isinstance(op, DimShuffle):
+            res = [dimshuffle(args[0], op.new_order)]
+        elif isinstance(op, CAReduce):
+            x = args[0]
+            idt = str(x.dtype)
+            sname = type(op.scalar_op).__name__
+            if isinstance(op, CAReduceDtype):
+                out_dt = op.dtype if op.dtype is not None else SUM_OUT_DTYPE.get(idt, idt)
+                acc_dt = op.acc_dtype if op.acc_dtype is not None else SUM_ACC_DTYPE.get(idt, idt)
+            else:
+                out_dt = node.outputs[0].type.dtype
+                acc_dt = "bool" if out_dt == "bool" else idt
+            if acc_dt == "float32" and idt == "float16":
+                x = x.astype("float32")
+            res = [careduce(x, sname, op.axis, acc_dt, out_dt)]
+        elif isinstance(op, ShapeFloat):
+            res = [np.asarray(args[0].shape[op.i], dtype=op.dtype)]
+        else:
+            raise NotImplementedError("oracle cannot evaluate %s" % op)
+        for o, v in zip(node.outputs, res):
+            env[o] = np.asarray(v)
+    return [env[o] if o in env else np.asarray(o.data) for o in outputs]

@@ -1,0 +1,388 @@
+"""TEST INFRASTRUCTURE - not part of the product.  Only ``tests/``, the
+``cpu_baseline`` leg of ``bench.py`` and ``__graft_entry__.smoke()`` may import
+anything under ``oracle/``.
+
+NumPy restatement of the per-element C semantics of Theano's scalar ops
+(``theano/scalar/basic.py``; sigmoid/softplus ``theano/tensor/nnet/sigm.py:60-85,
+344-362``).  Each function takes NumPy arrays and the output dtype decided by
+the graph, and evaluates what the generated C expression evaluates: operands
+are first brought to the type C's usual arithmetic conversions give the
+expression (``c_common_type``), the operation is done in that type, and the
+result is converted to the output dtype as the C assignment does.
+
+Pinning (tests/test_oracle_scalar.py): Mod / IntDiv against Python ``%`` and
+``//`` on the exhaustive int8 grid of ``theano/tensor/tests/test_basic.py:878-896``;
+comparisons and bit ops against the truth tables of
+``theano/scalar/tests/test_basic.py:187-256``; sigmoid against ``1/(1+exp(-x))``
+(``theano/tensor/nnet/tests/test_sigm.py:29-41``); max/min NaN propagation
+(``theano/tensor/tests/test_elemwise.py:525-538``); dtype rules against the
+literal tables of ``theano/scalar/basic.py:855-870`` and
+``theano/scalar/tests/test_basic.py:264-380``; ``right_shift(a, 3) ==
+int_div(a, 8)`` (no shift op exists in the reference).
+"""
+import numpy as np
+
+_RANK = {"bool": 0, "int8": 1, "uint8": 1, "int16": 2, "uint16": 2, "int32": 3, "uint32": 3, "int64": 4, "uint64": 4}
+
+
+def c_common_type(*dtypes):
+    """Type in which C evaluates a binary arithmetic expression over operands
+    of these types (integer promotion, then the usual arithmetic conversions).
+    float16 operands are float here, as in the reference's device code."""
+    dtypes = [str(d) for d in dtypes]
+    if "float64" in dtypes:
+        return "float64"
+    if "float32" in dtypes or "float16" in dtypes:
+        return "float32"
+    cur = "int32"
+    for d in dtypes:
+        if _RANK[d] <= 2:
+            d = "int32"  # integer promotion: every narrower type fits in int
+        if d == cur:
+            continue
+        ud, uc = d.startswith("u"), cur.startswith("u")
+        if ud == uc:
+            cur = d if _RANK[d] > _RANK[cur] else cur
+        else:
+            u, sg = (d, cur) if ud else (cur, d)
+            cur = u if _RANK[u] >= _RANK[sg] else sg
+    return cur
+
+
+def _conv(x, dtype):
+    """C conversion of values to ``dtype`` (bool storage is one byte 0/1)."""
+    x = np.asarray(x)
+    if str(dtype) == "bool":
+        return x != 0
+    with np.errstate(all="ignore"):
+        return x.astype(dtype)
+
+
+def _arith(fn, out_dtype, *xs):
+    ct = c_common_type(*[x.dtype for x in xs])
+    with np.errstate(all="ignore"):
+        r = fn(*[_conv(x, ct) for x in xs])
+    return _conv(r, out_dtype)
+
+
+def add(out_dtype, *xs):
+    if str(out_dtype) == "bool":  # x || y ...
+        r = xs[0] != 0
+        for x in xs[1:]:
+            r = r | (x != 0)
+        return r
+    def f(*a):
+        r = a[0]
+        for b in a[1:]:
+            r = r + b
+        return r
+    return _arith(f, out_dtype, *xs)
+
+
+def mul(out_dtype, *xs):
+    if str(out_dtype) == "bool":  # x && y ...
+        r = xs[0] != 0
+        for x in xs[1:]:
+            r = r & (x != 0)
+        return r
+    def f(*a):
+        r = a[0]
+        for b in a[1:]:
+            r = r * b
+        return r
+    return _arith(f, out_dtype, *xs)
+
+
+def sub(out_dtype, x, y):
+    return _arith(lambda a, b: a - b, out_dtype, x, y)
+
+
+def true_div(out_dtype, x, y):
+    if x.dtype.kind in "biu" and y.dtype.kind in "biu":
+        # ((double)x) / y
+        with np.errstate(all="ignore"):
+            return _conv(x.astype("float64") / y.astype("float64"), out_dtype)
+    return _arith(lambda a, b: a / b, out_dtype, x, y)
+
+
+def _c_div(a, b):
+    """C integer division: truncation toward zero (b != 0)."""
+    q = np.abs(a.astype(object)) // np.abs(b.astype(object))
+    return np.where((a < 0) != (b < 0), -q, q)
+
+
+def _c_mod(a, b):
+    return a.astype(object) - _c_div(a, b) * b.astype(object)
+
+
+def int_div(out_dtype, x, y):
+    """theano/scalar/basic.py:2009-2025: four sign cases over C division."""
+    ct = c_common_type(x.dtype, y.dtype)
+    if np.dtype(ct).kind == "f":
+        with np.errstate(all="ignore"):
+            return _conv(np.floor(_conv(x, ct) / _conv(y, ct)), out_dtype)
+    x, y = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
+    xo, yo = x.astype(object), y.astype(object)
+    res = np.zeros(x.shape, dtype=object)
+    nz = y != 0
+    for idx in np.ndindex(x.shape):
+        if not nz[idx]:
+            continue
+        a, b = int(xo[idx]), int(yo[idx])
+
+        def cdiv(p, q):
+            s = -1 if (p < 0) != (q < 0) else 1
+            return s * (abs(p) // abs(q))
+
+        def cmod(p, q):
+            return p - cdiv(p, q) * q
+        if b < 0:
+            if a < 0:
+                r = cdiv(-a, -b)
+            else:
+                r = -cdiv(a, -b) - (0 if cmod(a, -b) == 0 else 1)
+        else:
+            if a < 0:
+                r = -cdiv(-a, b) - (0 if cmod(-a, b) == 0 else 1)
+            else:
+                r = cdiv(a, b)
+        res[idx] = r
+    return _wrap(res, out_dtype)
+
+
+def mod(out_dtype, x, y):
+    """theano/scalar/basic.py:2119-2135: remainder with the divisor's sign."""
+    ct = c_common_type(x.dtype, y.dtype)
+    if np.dtype(ct).kind == "f":
+        a, b = np.broadcast_arrays(_conv(x, "float64"), _conv(y, "float64"))
+        with np.errstate(all="ignore"):
+            r = np.where(b == 0, np.fmod(a, b),
+                         np.where(b < 0,
+                                  np.where(a < 0, -np.fmod(-a, -b),
+                                           np.fmod(a, -b) + np.where(np.fmod(a, -b) != 0, b, 0)),
+                                  np.where(a < 0, -np.fmod(-a, b) + np.where(np.fmod(-a, b) != 0, b, 0),
+                                           np.fmod(a, b))))
+        return _conv(r, out_dtype)
+    x, y = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
+    xo, yo = x.astype(object), y.astype(object)
+    res = np.zeros(x.shape, dtype=object)
+    for idx in np.ndindex(x.shape):
+        a, b = int(xo[idx]), int(yo[idx])
+        if b == 0:
+            continue
+
+        def cmod(p, q):
+            s = -1 if (p < 0) != (q < 0) else 1
+            return p - s * (abs(p) // abs(q)) * q
+        if b < 0:
+            if a < 0:
+                r = -cmod(-a, -b)
+            else:
+                m = cmod(a, -b)
+                r = m + (b if m != 0 else 0)
+        else:
+            if a < 0:
+                m = cmod(-a, b)
+                r = -m + (b if m != 0 else 0)
+            else:
+                r = cmod(a, b)
+        res[idx] = r
+    return _wrap(res, out_dtype)
+
+
+def _wrap(obj_arr, dtype):
+    """Python ints -> fixed-width integers with two's-complement wrap."""
+    dt = np.dtype(dtype)
+    if dt.kind == "f":
+        return np.array(obj_arr, dtype="float64").astype(dt)
+    bits = dt.itemsize * 8
+    flat = np.array([int(v) & ((1 << bits) - 1) for v in obj_arr.reshape(-1)], dtype=object)
+    if dt.kind == "i":
+        flat = np.array([v - (1 << bits) if v >= (1 << (bits - 1)) else v for v in flat], dtype=object)
+    return flat.astype(dt).reshape(obj_arr.shape)
+
+
+def mod_fast(out_dtype, x, y):
+    """Vectorised equivalent of ``mod`` for integers: NumPy's ``%`` already has
+    the divisor's sign; zero divisors give 0 as on the device."""
+    ct = c_common_type(x.dtype, y.dtype)
+    a, b = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
+    with np.errstate(all="ignore"):
+        r = np.where(b == 0, 0, np.mod(a, np.where(b == 0, 1, b)))
+    return _conv(r, out_dtype)
+
+
+def int_div_fast(out_dtype, x, y):
+    ct = c_common_type(x.dtype, y.dtype)
+    a, b = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
+    with np.errstate(all="ignore"):
+        r = np.where(b == 0, 0, np.floor_divide(a, np.where(b == 0, 1, b)))
+    return _conv(r, out_dtype)
+
+
+def pow_(out_dtype, x, y):
+    with np.errstate(all="ignore"):
+        return _conv(np.power(x.astype("float64"), y.astype("float64")), out_dtype)
+
+
+def maximum(out_dtype, x, y):
+    # (y > x ? y : (x >= y ? x : nan)): NaN on either side gives NaN
+    return _arith(np.maximum, out_dtype, x, y)
+
+
+def minimum(out_dtype, x, y):
+    return _arith(np.minimum, out_dtype, x, y)
+
+
+def _cmp(fn):
+    def f(out_dtype, x, y):
+        ct = c_common_type(x.dtype, y.dtype)
+        return fn(_conv(x, ct), _conv(y, ct))
+    return f
+
+
+lt, gt, le, ge, eq, neq = (_cmp(np.less), _cmp(np.greater), _cmp(np.less_equal), _cmp(np.greater_equal),
+                           _cmp(np.equal), _cmp(np.not_equal))
+
+
+def _bit(fn):
+    def f(out_dtype, x, y):
+        if str(out_dtype) == "bool":
+            return fn(x != 0, y != 0)
+        return _arith(fn, out_dtype, x, y)
+    return f
+
+
+and_, or_, xor = _bit(np.bitwise_and), _bit(np.bitwise_or), _bit(np.bitwise_xor)
+right_shift = _bit(np.right_shift)
+left_shift = _bit(np.left_shift)
+
+
+def invert(out_dtype, x):
+    if str(out_dtype) == "bool":
+        return x == 0
+    return _conv(np.invert(_conv(x, c_common_type(x.dtype))), out_dtype)
+
+
+def isnan(out_dtype, x):
+    return np.isnan(x) if x.dtype.kind == "f" else np.zeros(x.shape, bool)
+
+
+def isinf(out_dtype, x):
+    return np.isinf(x) if x.dtype.kind == "f" else np.zeros(x.shape, bool)
+
+
+def switch(out_dtype, c, a, b):
+    ct = c_common_type(a.dtype, b.dtype)
+    return _conv(np.where(c != 0, _conv(a, ct), _conv(b, ct)), out_dtype)
+
+
+def clip(out_dtype, x, lo, hi):
+    ct = c_common_type(x.dtype, lo.dtype, hi.dtype)
+    x_, lo_, hi_ = _conv(x, ct), _conv(lo, ct), _conv(hi, ct)
+    return _conv(np.where(x_ < lo_, lo_, np.where(x_ > hi_, hi_, x_)), out_dtype)
+
+
+def second(out_dtype, x, y):
+    return _conv(np.broadcast_arrays(x, y)[1], out_dtype)
+
+
+def identity(out_dtype, x):
+    return _conv(x, out_dtype)
+
+
+def cast(out_dtype, x):
+    return _conv(x, out_dtype)
+
+
+def neg(out_dtype, x):
+    return _arith(lambda a: -a, out_dtype, x)
+
+
+def abs_(out_dtype, x):
+    return _conv(np.abs(x), out_dtype)
+
+
+def sgn(out_dtype, x):
+    return _conv(np.sign(x), out_dtype)
+
+
+def inv(out_dtype, x):
+    with np.errstate(all="ignore"):
+        return _conv(1.0 / _conv(x, "float64") if x.dtype != np.float32 and x.dtype != np.float16
+                     else (np.float64(1.0) / x.astype("float64")), out_dtype)
+
+
+def sqr(out_dtype, x):
+    return _arith(lambda a: a * a, out_dtype, x)
+
+
+def _libm(fn):
+    """``z = f((out_t)x)``: the input is cast to the output type first."""
+    def f(out_dtype, x):
+        ct = "float32" if str(out_dtype) == "float16" else out_dtype
+        with np.errstate(all="ignore"):
+            return _conv(fn(_conv(x, ct)), out_dtype)
+    return f
+
+
+exp, exp2, expm1 = _libm(np.exp), _libm(np.exp2), _libm(np.expm1)
+log, log2, log10, log1p = _libm(np.log), _libm(np.log2), _libm(np.log10), _libm(np.log1p)
+sqrt, ceil, floor = _libm(np.sqrt), _libm(np.ceil), _libm(np.floor)
+cos, sin, tan = _libm(np.cos), _libm(np.sin), _libm(np.tan)
+arccos, arcsin, arctan = _libm(np.arccos), _libm(np.arcsin), _libm(np.arctan)
+cosh, sinh, tanh = _libm(np.cosh), _libm(np.sinh), _libm(np.tanh)
+arccosh, arcsinh, arctanh = _libm(np.arccosh), _libm(np.arcsinh), _libm(np.arctanh)
+trunc = _libm(np.trunc)
+round_half_to_even = _libm(np.rint)
+round_half_away_from_zero = _libm(lambda a: np.where(a > 0, np.floor(a + 0.5), np.ceil(a - 0.5)))
+
+
+def arctan2(out_dtype, y, x):
+    ct = "float32" if str(out_dtype) == "float16" else out_dtype
+    return _conv(np.arctan2(_conv(y, ct), _conv(x, ct)), out_dtype)
+
+
+def scalar_sigmoid(out_dtype, x):
+    """theano/tensor/nnet/sigm.py:78-85."""
+    if str(x.dtype) in ("float32", "float16"):
+        xf = x.astype("float32")
+        with np.errstate(all="ignore"):
+            r = np.where(xf < np.float32(-88.0), np.float32(0),
+                         np.where(xf > np.float32(15.0), np.float32(1),
+                                  np.float32(1) / (np.float32(1) + np.exp(-xf))))
+        return _conv(r, out_dtype)
+    xd = x.astype("float64")
+    with np.errstate(all="ignore"):
+        r = np.where(xd < -709.0, 0.0, np.where(xd > 19.0, 1.0, 1.0 / (1.0 + np.exp(-xd))))
+    return _conv(r, out_dtype)
+
+
+def scalar_softplus(out_dtype, x):
+    """theano/tensor/nnet/sigm.py:356-360."""
+    if str(x.dtype) in ("float32", "float16"):
+        xf = x.astype("float32")
+        with np.errstate(all="ignore"):
+            r = np.where(xf < np.float32(-103.0), np.float32(0), np.where(xf > np.float32(14.0), xf,
+                                                                          np.log1p(np.exp(xf))))
+        return _conv(r, out_dtype)
+    xd = x.astype("float64")
+    with np.errstate(all="ignore"):
+        r = np.where(xd < -745.0, 0.0, np.where(xd > 16.0, xd, np.log1p(np.exp(xd))))
+    return _conv(r, out_dtype)
+
+
+# scalar op class name -> restatement
+BY_CLASS = {
+    "Add": add, "Mul": mul, "Sub": sub, "TrueDiv": true_div, "IntDiv": int_div_fast, "Mod": mod_fast, "Pow": pow_,
+    "Maximum": maximum, "Minimum": minimum, "LT": lt, "GT": gt, "LE": le, "GE": ge, "EQ": eq, "NEQ": neq,
+    "AND": and_, "OR": or_, "XOR": xor, "RightShift": right_shift, "LeftShift": left_shift, "Invert": invert,
+    "IsNan": isnan, "IsInf": isinf, "Switch": switch, "Clip": clip, "Second": second, "Identity": identity,
+    "Cast": cast, "Neg": neg, "Abs": abs_, "Sgn": sgn, "Inv": inv, "Sqr": sqr, "Exp": exp, "Exp2": exp2,
+    "Expm1": expm1, "Log": log, "Log2": log2, "Log10": log10, "Log1p": log1p, "Sqrt": sqrt, "Ceil": ceil,
+    "Floor": floor, "Trunc": trunc, "RoundHalfToEven": round_half_to_even,
+    "RoundHalfAwayFromZero": round_half_away_from_zero, "Cos": cos, "Sin": sin, "Tan": tan, "ArcCos": arccos,
+    "ArcSin": arcsin, "ArcTan": arctan, "ArcTan2": arctan2, "Cosh": cosh, "Sinh": sinh, "Tanh": tanh,
+    "ArcCosh": arccosh, "ArcSinh": arcsinh, "ArcTanh": arctanh, "ScalarSigmoid": scalar_sigmoid,
+    "ScalarSoftplus": scalar_softplus,
+}

@@ -1,0 +1,90 @@
+"""The five benchmark configurations: parity against the oracle at reduced
+size, size-independent properties at full size."""
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import hip, tensor as T
+from oracle import graph_ref as G
+from conftest import assert_parity
+import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def parity(graph, vals, what, tol=None):
+    ins, outs = graph
+    got = th.function(ins, outs)(*vals)
+    ref = G.evaluate(ins, outs, vals)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "%s output %d" % (what, k), tol=tol)
+    return got
+
+
+def test_config1_small_and_full():
+    parity(W.c1_graph(), W.c1_inputs("small"), "c1 small")
+    ins, outs = W.c1_graph()
+    x, a, b = W.c1_inputs("full")
+    got = th.function(ins, outs)(x, a, b)[0]
+    t = (a * x + b).astype("float64")
+    ref = (np.where(t < -88, 0.0, np.where(t > 15, 1.0, 1 / (1 + np.exp(-t)))) * x).astype("float32")
+    assert_parity(got, ref, "c1 full")
+
+
+@pytest.mark.parametrize("case", W.C2_CASES)
+def test_config2(case):
+    parity(W.c2_graph(case), W.c2_inputs(case, "small"), "c2 %s small" % case)
+    ins, outs = W.c2_graph(case)
+    (x,) = W.c2_inputs(case, "full")
+    got = th.function(ins, outs)(x)[0]
+    x64 = x.astype("float64")
+    ref = {"sum_axis1": lambda: x64.sum(1), "max_axis1": lambda: x.max(1), "sum_axis0": lambda: x64.sum(0),
+           "sum_all": lambda: x64.sum(), "prod_axis1": lambda: x64.prod(1)}[case]()
+    assert_parity(got, np.asarray(ref).astype("float32"), "c2 %s full" % case)
+
+
+def test_config3_softmax_and_gradient():
+    parity(W.c3_graph(with_grad=False), W.c3_inputs("small", with_grad=False), "c3 fwd small")
+    parity(W.c3_graph(), W.c3_inputs("small"), "c3 fwd+grad small")
+    ins, outs = W.c3_graph()
+    x, y = W.c3_inputs("full")
+    out, dx = th.function(ins, outs)(x, y)
+    # rows of a softmax sum to one, rows of its gradient sum to zero, argmax is preserved
+    assert np.allclose(out.astype("float64").sum(1), 1.0, atol=1e-5)
+    assert np.abs(dx.astype("float64").sum(1)).max() < 1e-5
+    assert np.array_equal(out.argmax(1), x.argmax(1))
+    rows = slice(0, 64)
+    e = np.exp(x[rows].astype("float64") - x[rows].max(1, keepdims=True))
+    sm = e / e.sum(1, keepdims=True)
+    assert_parity(out[rows], sm.astype("float32"), "c3 full rows")
+    assert_parity(dx[rows], (sm * (y[rows] - (sm * y[rows]).sum(1, keepdims=True))).astype("float32"), "c3 grad rows",
+                  tol=dict(rtol=1e-4, atol=1e-6))
+
+
+def test_config4_integer_path():
+    parity(W.c4_graph("all"), W.c4_inputs("small"), "c4 small")
+    ins, outs = W.c4_graph("all")
+    a, b, bias = W.c4_inputs("full")
+    r, s, any_, all_ = th.function(ins, outs)(a, b, bias)
+    ref = (((a & b) ^ (a >> 3)) % 97 + bias).transpose(0, 2, 3, 1)
+    assert r.shape == ref.shape and np.array_equal(r, ref)
+    assert np.array_equal(s, ref.astype("int64").sum((0, 1, 2)))     # checksum of the elementwise result
+    assert np.array_equal(s, r.astype("int64").sum((0, 1, 2)))
+    assert bool(any_) == bool((a > 0).any()) and bool(all_) == bool((a > 0).all())
+
+
+def test_config5_batchnorm_float16():
+    tol = dict(rtol=2e-3, atol=2e-3)
+    parity(W.c5_graph(with_grad=False), W.c5_inputs("small", with_grad=False), "c5 fwd small", tol)
+    parity(W.c5_graph(), W.c5_inputs("small"), "c5 fwd+grad small", tol)
+    ins, outs = W.c5_graph(with_grad=False)
+    x, gamma, beta = W.c5_inputs("full", with_grad=False)
+    y = th.function(ins, outs)(x, gamma, beta)[0]
+    # normalised activations: per-channel mean beta and standard deviation |gamma|
+    yf = y.astype("float64")
+    assert np.allclose(yf.mean((0, 2, 3)), beta.astype("float64").reshape(-1), atol=2e-3)
+    assert np.allclose(yf.std((0, 2, 3)), np.abs(gamma.astype("float64")).reshape(-1), rtol=2e-3, atol=2e-3)
+    ch = 7
+    xc = x[:, ch].astype("float64")
+    ref = gamma.astype("float64")[0, ch] * (xc - xc.mean()) / np.sqrt(xc.var() + 1e-5) + beta.astype("float64")[0, ch]
+    assert_parity(y[:, ch], ref.astype("float16"), "c5 full channel", tol)

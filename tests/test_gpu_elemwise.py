@@ -1,0 +1,168 @@
+"""GPU parity of the elementwise path against the oracle, through the C-ABI."""
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import hip, tensor as T
+from oracle import graph_ref as G
+from conftest import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def run_both(ins, outs, vals):
+    f = th.function(ins, outs)
+    got = f(*vals)
+    ref = G.evaluate(ins, outs, vals)
+    return got, ref
+
+
+def rand(rng, shape, dtype):
+    if dtype == "bool":
+        return rng.integers(0, 2, shape).astype("bool")
+    if np.dtype(dtype).kind in "iu":
+        lo = 0 if np.dtype(dtype).kind == "u" else -100
+        return rng.integers(lo, 100, shape).astype(dtype)
+    return rng.standard_normal(shape).astype(dtype)
+
+
+# the input patterns of _good_broadcast_binary_normal, theano/tensor/tests/test_basic.py:664-684
+BROADCAST_SHAPES = [((2, 3), (2, 3)), ((2, 2), (2,)), ((2, 3), (1, 1)), ((2, 3), (1, 3)), ((2, 3), (2, 1)),
+                    ((3, 5), (1, 5)), ((2, 3, 4, 5), (1, 3, 1, 5)), ((0, 3), (0, 3)), ((5, 1031), (5, 1031)),
+                    ((), ()), ((1,), (1,))]
+
+
+@pytest.mark.parametrize("sa,sb", BROADCAST_SHAPES)
+def test_binary_ops_over_broadcast_patterns(sa, sb):
+    rng = np.random.default_rng(7)
+    a = T.TensorType("float32", [s == 1 for s in sa])("a")
+    b = T.TensorType("float32", [s == 1 for s in sb])("b")
+    av, bv = rand(rng, sa, "float32"), rand(rng, sb, "float32") + 3
+    outs = [a + b, a - b, a * b, a / b, T.maximum(a, b), T.minimum(a, b), a < b, T.eq(a, b), T.switch(a > 0, a, b)]
+    got, ref = run_both([a, b], outs, [av, bv])
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "binary op %d on %s %s" % (k, sa, sb))
+
+
+@pytest.mark.parametrize("dtype", ["int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64"])
+def test_integer_ops_bit_exact(dtype):
+    rng = np.random.default_rng(8)
+    a, b = T.TensorType(dtype, (False, False))("a"), T.TensorType(dtype, (False, False))("b")
+    av = rand(rng, (37, 53), dtype)
+    bv = rand(rng, (37, 53), dtype)
+    bv[bv == 0] = 3
+    outs = [a + b, a * b, a - b, a % b, a // b, a & b, a | b, a ^ b, ~a, abs(a), T.sqr(a), a > b, T.neq(a, b),
+            T.cast(a, "int8"), T.cast(a, "bool"), T.cast(a, "float32"), T.true_div(a, b)]
+    got, ref = run_both([a, b], outs, [av, bv])
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "%s op %d" % (dtype, k))
+
+
+def test_int8_mod_and_intdiv_exhaustive_grid():
+    # theano/tensor/tests/test_basic.py:878-896
+    a, b = T.bcol("a"), T.brow("b")
+    av = np.arange(-127, 128, dtype="int8")[:, None]
+    bv = np.array([v for v in range(-127, 128) if v != 0], dtype="int8")[None, :]
+    f = th.function([a, b], [a % b, a // b])
+    m, d = f(av, bv)
+    assert np.array_equal(m, np.array([[int(x) % int(y) for y in bv[0]] for x in av[:, 0]], dtype="int8"))
+    assert np.array_equal(d, np.array([[int(x) // int(y) for y in bv[0]] for x in av[:, 0]], dtype="int8"))
+
+
+def test_right_shift_equals_int_div():
+    a = T.ivector("a")
+    av = np.arange(-5000, 5000, dtype="int32")
+    s, d = th.function([a], [a >> 3, a // 8])(av)
+    assert np.array_equal(s, d) and np.array_equal(s, av >> 3)
+
+
+def test_bool_ops():
+    rng = np.random.default_rng(9)
+    a, b = T.TensorType("bool", (False,))("a"), T.TensorType("bool", (False,))("b")
+    av, bv = rand(rng, (1000,), "bool"), rand(rng, (1000,), "bool")
+    got, ref = run_both([a, b], [a & b, a | b, a ^ b, ~a, a + b, a * b, T.cast(a, "int32")], [av, bv])
+    for g, r in zip(got, ref):
+        assert_parity(g, r, "bool")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64", "float16"])
+def test_unary_math(dtype):
+    rng = np.random.default_rng(10)
+    x = T.TensorType(dtype, (False, False))("x")
+    xv = (rng.uniform(0.1, 3.0, (61, 130))).astype(dtype)
+    outs = [T.exp(x), T.log(x), T.sqrt(x), T.tanh(x), T.sigmoid(x - 1), T.softplus(x), T.sin(x), T.cos(x), T.sqr(x),
+            T.inv(x), T.neg(x), abs(x - 1), T.sgn(x - 1), T.floor(x), T.ceil(x), T.log1p(x), T.expm1(x), x ** 2,
+            T.clip(x, 0.5, 2.0), T.arctan(x)]
+    got, ref = run_both([x], outs, [xv])
+    tol = {"float64": dict(rtol=1e-12, atol=1e-12)}.get(dtype)
+    if dtype == "float64":  # libm implementations differ in the last ulps for transcendental functions
+        tol = dict(rtol=1e-12, atol=1e-12)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "%s unary %d" % (dtype, k), tol=tol)
+
+
+def test_sigmoid_thresholds_and_nan_handling():
+    x = T.fvector("x")
+    xv = np.array([-100, -88.5, -88, -30, 0, 14.9, 15, 15.1, 100, np.nan, np.inf, -np.inf], "float32")
+    got, ref = run_both([x], [T.sigmoid(x), T.maximum(x, 0), T.minimum(x, 0), T.isnan(x), T.isinf(x)], [xv])
+    for g, r in zip(got, ref):
+        assert_parity(g, r, "special values")
+
+
+def test_weird_strides_five_dims():
+    # theano/tensor/tests/test_elemwise.py:305-318
+    rng = np.random.default_rng(11)
+    x = T.TensorType("float32", (False,) * 5)("x")
+    y = T.TensorType("float32", (False,) * 5)("y")
+    xv = rng.standard_normal((2, 3, 4, 5, 6)).astype("float32")
+    yv = rng.standard_normal((6, 5, 4, 3, 2)).astype("float32")
+    got, ref = run_both([x, y], [x + y.dimshuffle(4, 3, 2, 1, 0), (x * 2).dimshuffle(1, 0, 4, 3, 2)], [xv, yv])
+    for g, r in zip(got, ref):
+        assert_parity(g, r, "5-d transposed")
+
+
+def test_same_input_twice_and_many_inputs():
+    rng = np.random.default_rng(12)
+    x = T.fmatrix("x")
+    xv = rng.standard_normal((17, 33)).astype("float32")
+    got, ref = run_both([x], [x * x + x], [xv])
+    assert_parity(got[0], ref[0], "same input")
+    # theano/gpuarray/tests/test_opt.py:531-572: a sum of many inputs, more than one kernel's argument budget
+    ins = [T.fmatrix("i%d" % k) for k in range(40)]
+    vals = [rng.standard_normal((5, 9)).astype("float32") for _ in ins]
+    out = ins[0]
+    for i in ins[1:]:
+        out = out + i
+    got, ref = run_both(ins, [out], vals)
+    assert_parity(got[0], ref[0], "40 inputs", tol=dict(rtol=1e-5, atol=1e-5))
+
+
+def test_mixed_dtypes_follow_c_promotion():
+    rng = np.random.default_rng(13)
+    i, f, d, h = T.ivector("i"), T.fvector("f"), T.dvector("d"), T.TensorType("float16", (False,))("h")
+    vals = [rand(rng, (300,), "int32"), rand(rng, (300,), "float32"), rand(rng, (300,), "float64"),
+            rand(rng, (300,), "float16")]
+    got, ref = run_both([i, f, d, h], [i * f, i + d, f * d, h * f, h + h, i / 7, T.cast(f, "float16")], vals)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "mixed %d" % k)
+
+
+def test_large_contiguous_and_unaligned_views():
+    rng = np.random.default_rng(14)
+    x = T.fvector("x")
+    xv = rng.standard_normal(3 * 1024 * 1024 + 5).astype("float32")
+    f = th.function([x], T.exp(x) * 0.5)
+    assert_parity(f(xv), G.evaluate([x], [T.exp(x) * 0.5], [xv])[0], "large vector")
+    m = T.fmatrix("m")
+    mv = rng.standard_normal((64, 259)).astype("float32")
+    got, ref = run_both([m], [m.T * 2 + 1], [mv])
+    assert_parity(got[0], ref[0], "transposed output order")
+
+
+def test_host_scalar_operands_travel_by_value():
+    x = T.fmatrix("x")
+    s = T.TensorType("float32", (True, True))("s")
+    f = th.function([x, s], x * s + s)
+    xv = np.arange(12, dtype="float32").reshape(3, 4)
+    assert_parity(f(xv, np.float32([[2.5]])), xv * np.float32(2.5) + np.float32(2.5), "immediate")
+    assert "m0,3,0" in hip.last_plan() or ",3" in hip.last_plan()

@@ -1,0 +1,142 @@
+"""GPU parity of CAReduce against the oracle over shapes, masks, ops and dtypes."""
+import itertools
+
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import hip, tensor as T
+from oracle import graph_ref as G
+from conftest import assert_parity
+from test_oracle_graph import CAREDUCE_CASES
+
+pytestmark = pytest.mark.gpu
+
+REDUCERS = {"sum": lambda v, ax: v.sum(axis=ax), "prod": lambda v, ax: v.prod(axis=ax),
+            "max": lambda v, ax: v.max(axis=ax), "min": lambda v, ax: v.min(axis=ax)}
+
+
+def check(var, out, val, what, tol=None):
+    got = th.function([var], out)(val)
+    ref = G.evaluate([var], [out], [val])[0]
+    assert_parity(got, ref, what + " [" + hip.last_plan() + "]", tol=tol)
+
+
+@pytest.mark.parametrize("shape,axis", CAREDUCE_CASES)
+def test_reference_case_table(shape, axis):
+    rng = np.random.default_rng(21)
+    xf = T.TensorType("float32", (False,) * len(shape))("x")
+    xi = T.TensorType("int32", (False,) * len(shape))("x")
+    vf = rng.standard_normal(shape).astype("float32")
+    vi = rng.integers(-4, 5, shape).astype("int32")
+    zero = any(shape[a] == 0 for a in (range(len(shape)) if axis is None else axis))
+    for name, fn in REDUCERS.items():
+        if zero and name in ("max", "min"):
+            with pytest.raises(ValueError):
+                th.function([xf], fn(xf, axis))(vf)
+            continue
+        check(xf, fn(xf, axis), vf, "%s f32 %s %s" % (name, shape, axis))
+        check(xi, fn(xi, axis), vi, "%s i32 %s %s" % (name, shape, axis))
+    check(xi, T.any(xi > 0, axis=axis), vi, "any")
+    check(xi, T.all(xi > -4, axis=axis), vi, "all")
+
+
+# shape x reduce-mask patterns in the spirit of theano/gpuarray/tests/test_elemwise.py:262-346,
+# including extents above 4096 and degenerate extents
+MASK_CASES = [((4100, 3), [1, 0]), ((3, 4100), [0, 1]), ((4100, 3), [0, 1]), ((3, 4100), [1, 0]), ((5000,), [1]),
+              ((1, 5000), [0, 1]), ((33, 1, 65), [1, 0, 1]), ((33, 65, 17), [0, 1, 0]), ((33, 65, 17), [1, 0, 1]),
+              ((33, 65, 17), [1, 1, 0]), ((33, 65, 17), [0, 1, 1]), ((33, 65, 17), [1, 0, 0]), ((33, 65, 17), [0, 0, 1]),
+              ((5, 7, 9, 11), [1, 0, 1, 0]), ((5, 7, 9, 11), [0, 1, 0, 1]), ((5, 7, 9, 11), [1, 0, 0, 1]),
+              ((5, 7, 9, 11), [0, 1, 1, 0]), ((5, 7, 9, 11), [1, 1, 1, 1]), ((5, 7, 9, 11), [1, 0, 1, 1]),
+              ((3, 4, 5, 6, 7), [1, 0, 1, 0, 1]), ((3, 4, 5, 6, 7, 2), [1, 0, 1, 0, 1, 0]), ((2, 3, 4, 5, 6, 7, 2, 3), [0, 1] * 4),
+              ((1025, 1025), [1, 0]), ((1025, 1025), [0, 1]), ((1025, 1025), [1, 1]), ((70000, 2), [1, 0]),
+              ((2, 70000), [0, 1]), ((300000,), [1]), ((64, 8, 49), [1, 0, 1])]
+
+
+@pytest.mark.parametrize("shape,mask", MASK_CASES)
+def test_shapes_and_masks(shape, mask):
+    rng = np.random.default_rng(22)
+    axis = tuple(d for d, m in enumerate(mask) if m)
+    x = T.TensorType("float32", (False,) * len(shape))("x")
+    v = rng.standard_normal(shape).astype("float32")
+    check(x, x.sum(axis=axis), v, "sum %s %s" % (shape, mask))
+    check(x, x.max(axis=axis), v, "max %s %s" % (shape, mask))
+    xi = T.TensorType("int16", (False,) * len(shape))("xi")
+    vi = rng.integers(-300, 300, shape).astype("int16")
+    check(xi, xi.sum(axis=axis), vi, "int16 sum %s %s" % (shape, mask))
+
+
+@pytest.mark.parametrize("dtype", ["bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64",
+                                   "float16", "float32", "float64"])
+def test_dtype_coverage(dtype):
+    rng = np.random.default_rng(23)
+    x = T.TensorType(dtype, (False, False))("x")
+    if dtype == "bool":
+        v = rng.integers(0, 2, (77, 130)).astype("bool")
+    elif np.dtype(dtype).kind in "iu":
+        v = rng.integers(0 if dtype[0] == "u" else -3, 4, (77, 130)).astype(dtype)
+    else:
+        v = rng.uniform(0.5, 1.5, (77, 130)).astype(dtype)
+    tol = dict(rtol=1e-12, atol=1e-12) if dtype == "float64" else None
+    for axis in ((0,), (1,), None):
+        check(x, x.sum(axis=axis), v, "sum %s %s" % (dtype, axis), tol)
+        check(x, x.max(axis=axis), v, "max %s %s" % (dtype, axis), tol)
+        check(x, x.min(axis=axis), v, "min %s %s" % (dtype, axis), tol)
+        if dtype != "float16":
+            check(x, x.prod(axis=axis), v, "prod %s %s" % (dtype, axis), tol)
+        if dtype != "bool" and np.dtype(dtype).kind != "f":
+            check(x, T.sum(x, axis=axis, dtype="float64"), v, "sum to f64")
+
+
+def test_precision_of_default_accumulator():
+    # theano/tensor/tests/test_elemwise.py:953-966
+    x = T.fvector("x")
+    v = np.asarray([1e8, 1, -1e8], dtype="float32")
+    assert float(th.function([x], x.sum())(v)) == 1.0
+    big = np.ones(1 << 22, "float32") * np.float32(0.1)
+    got = float(th.function([x], x.sum())(big))
+    assert got == np.float32(big.astype("float64").sum())
+
+
+def test_nan_propagation_and_negative_zero():
+    x = T.fmatrix("x")
+    v = np.array([[1.0, np.nan, 3.0], [4.0, 5.0, 6.0], [-np.inf, np.inf, 0.0]], dtype="float32")
+    for axis in ((0,), (1,), None):
+        check(x, x.max(axis=axis), v, "max nan %s" % (axis,))
+        check(x, x.min(axis=axis), v, "min nan %s" % (axis,))
+        check(x, x.sum(axis=axis), v, "sum nan %s" % (axis,))
+
+
+def test_strided_inputs_and_explicit_dtypes():
+    rng = np.random.default_rng(24)
+    x = T.ftensor3("x")
+    v = rng.standard_normal((31, 47, 53)).astype("float32")
+    xt = x.dimshuffle(2, 0, 1)
+    for axis in ((0,), (1,), (2,), (0, 2), (1, 2), None):
+        got = th.function([x], xt.sum(axis=axis))(v)
+        ref = G.evaluate([x], [xt.sum(axis=axis)], [v])[0]
+        assert_parity(got, ref, "transposed view %s" % (axis,))
+    xi = T.imatrix("xi")
+    vi = rng.integers(-2 ** 30, 2 ** 30, (513, 257)).astype("int32")
+    check(xi, T.sum(xi, axis=0, dtype="int64"), vi, "int64 sum")
+    check(xi, T.sum(xi, axis=1, dtype="int32", acc_dtype="int32"), vi, "wrapping int32 sum")
+    check(xi, T.sum(xi, axis=None, dtype="float32", acc_dtype="float64"), vi, "float sum of ints")
+
+
+def test_fused_prologue_and_multi_output():
+    rng = np.random.default_rng(25)
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    r = T.frow("r")
+    xv, yv = rng.standard_normal((301, 515)).astype("float32"), rng.standard_normal((301, 515)).astype("float32")
+    rv = rng.standard_normal((1, 515)).astype("float32")
+    outs = [T.sum(T.sqr(x - y) * r, axis=1), T.sum(abs(x) * y, axis=0), T.max(x * r + y), T.mean(x, axis=0),
+            T.var(x, axis=1), T.std(y, axis=0)]
+    f = th.function([x, y, r], outs)
+    got = f(xv, yv, rv)
+    ref = G.evaluate([x, y, r], outs, [xv, yv, rv])
+    for k, (g, rr) in enumerate(zip(got, ref)):
+        assert_parity(g, rr, "fused reduce %d" % k, tol=dict(rtol=2e-5, atol=2e-6))
+    a = T.imatrix("a")
+    av = rng.integers(-5, 6, (200, 333)).astype("int32")
+    g2 = th.function([a], [T.any(a > 4), T.all(a > -6), T.any(a > 5), T.all(a > 0)])(av)
+    assert [bool(v) for v in g2] == [True, True, False, False]

@@ -1,0 +1,155 @@
+"""Host-side mirror of the reference's Op interface: node construction, type
+inference, error behaviour, gradients' graph structure and what the rewrite
+pipeline (lift + fuse) produces."""
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import scalar as scal
+from theano_amd import tensor as T
+from theano_amd.hip import HipCAReduce, HipDimShuffle, HipElemwise, HipToHost, HostToHip
+from theano_amd.tensor.elemwise import CAReduce, DimShuffle, Elemwise, Sum
+
+
+def ops_of(f, cls):
+    return [n for n in f.toposort() if isinstance(n.op, cls)]
+
+
+def test_elemwise_make_node_pads_ranks_and_ands_broadcast_flags():
+    x, v = T.fmatrix(), T.fvector()
+    z = x + v
+    assert z.type.broadcastable == (False, False) and z.type.dtype == "float32"
+    assert isinstance(z.owner.inputs[1].owner.op, DimShuffle)
+    assert z.owner.inputs[1].owner.op.new_order == ("x", 0)
+    r, c = T.frow(), T.fcol()
+    assert (r * c).type.broadcastable == (False, False)
+    assert (r + r).type.broadcastable == (True, False)
+
+
+def test_props_give_equality_and_hash():
+    assert Elemwise(scal.add) == Elemwise(scal.add) and hash(Elemwise(scal.add)) == hash(Elemwise(scal.add))
+    assert Elemwise(scal.add) != Elemwise(scal.mul)
+    assert Sum(axis=(0,)) == Sum(axis=[0]) and Sum(axis=0) != Sum(axis=1)
+    assert DimShuffle((False, False), (1, 0)) == DimShuffle((False, False), [1, 0])
+    assert HipElemwise(scal.add) != Elemwise(scal.add)
+
+
+def test_python_literals_pick_the_smallest_dtype():
+    x = T.imatrix()
+    assert (x % 97).type.dtype == "int32" and (x % 97).owner.inputs[1].owner.inputs[0].type.dtype == "int8"
+    f = T.fmatrix()
+    assert (f + 1e-5).type.dtype == "float32"  # floatX = float32 keeps float literals narrow
+    assert (f * 2).type.dtype == "float32"
+    assert (x / 2).type.dtype == "int32"       # int / int is integer division under int_division='int'
+    assert T.true_div(x, 2).type.dtype == "float32"
+
+
+def test_dimshuffle_rules():
+    x = T.TensorType("float32", (False, True, False))()
+    assert x.dimshuffle(2, 0).type.broadcastable == (False, False)
+    assert x.dimshuffle(0, "x", 2, 1).type.broadcastable == (False, True, False, True)
+    with pytest.raises(ValueError):
+        x.dimshuffle(1, 2)  # drops a non-broadcastable dimension
+    with pytest.raises(ValueError):
+        x.dimshuffle(0, 0, 2)
+
+
+def test_careduce_axis_normalisation_and_infer_shape():
+    x = T.ftensor3()
+    s = x.sum(axis=(-1, 0))
+    assert s.owner.op.axis == (0, 2) and s.type.ndim == 1
+    assert s.owner.op.infer_shape(s.owner, [(4, 5, 6)]) == ([5],)
+    with pytest.raises(ValueError):
+        x.sum(axis=3)
+    assert T.all(x > 0).type.dtype == "bool" and T.any(x).owner.inputs[0].owner.op.scalar_op == scal.neq
+
+
+def test_bit_ops_reject_floats_and_sub_rejects_bool():
+    with pytest.raises(TypeError):
+        T.fmatrix() & T.fmatrix()
+    b = T.TensorType("bool", (False,))()
+    with pytest.raises(TypeError):
+        b - b
+    assert (b + b).type.dtype == "bool"
+
+
+def test_fusion_collapses_an_elementwise_chain_to_one_composite():
+    x, y, z = T.fmatrix("x"), T.fmatrix("y"), T.fmatrix("z")
+    f = th.function([x, y, z], T.sigmoid(x * y + z) * x + 2.0)
+    ew = ops_of(f, HipElemwise)
+    assert len(ew) == 1 and isinstance(ew[0].op.scalar_op, scal.Composite)
+    assert len(ew[0].inputs) == 3                      # repeated x is one operand, the constant is a literal
+    assert len(ops_of(f, HostToHip)) == 3 and len(ops_of(f, HipToHost)) == 1
+
+
+def test_fusion_respects_broadcast_pattern_and_client_count():
+    x, s = T.fmatrix("x"), T.TensorType("float32", (True, True))("s")
+    # sin(s) has a scalar-shaped output: it is not pulled into the matrix-shaped consumer
+    # (case 71 of theano/tensor/tests/test_opt.py:1107-1111)
+    f = th.function([x, s], x + T.sin(s))
+    assert len(ops_of(f, HipElemwise)) == 2
+    # an expensive producer with two clients is computed once, not duplicated
+    e = T.exp(x)
+    g = th.function([x], [e + 1, e * 2])
+    assert len(ops_of(g, HipElemwise)) == 3
+
+
+def test_config1_is_one_kernel_with_scalars_passed_by_value():
+    import workloads
+    ins, outs = workloads.c1_graph()
+    f = th.function(ins, outs)
+    ew = ops_of(f, HipElemwise)
+    assert len(ew) == 1 and str(ew[0].op.scalar_op) == "Composite{mul(scalar_sigmoid(add(mul(i0, i1), i2)), i1)}"
+    assert len(ops_of(f, HostToHip)) == 1              # a and b stay on the host
+
+
+def test_reduce_prologue_fusion_and_sibling_merge():
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    f = th.function([x, y], T.sum(T.sqr(x - y), axis=1))
+    assert len(ops_of(f, HipElemwise)) == 0
+    (red,) = ops_of(f, HipCAReduce)
+    assert red.op.pre_scalar_op is not None and len(red.inputs) == 2
+    g = th.function([x], [T.any(x > 0), T.all(x > 0)])
+    (red,) = ops_of(g, HipCAReduce)
+    assert len(red.outputs) == 2 and red.op.scalar_ops == (scal.or_, scal.and_)
+
+
+def test_gradient_graph_contains_only_path_ops():
+    x, y = T.fmatrix("x"), T.frow("y")
+    cost = T.sum(T.tanh(x * y))
+    gx, gy = th.grad(cost, [x, y])
+    assert gx.type == x.type and gy.type == y.type   # the broadcast row gets its gradient summed back
+    from theano_amd import gof
+    for node in gof.io_toposort([x, y], [gx, gy]):
+        assert isinstance(node.op, (Elemwise, CAReduce, DimShuffle)), node.op
+    with pytest.raises(TypeError):
+        th.grad(x, x)  # non-scalar cost
+
+
+def test_lifter_refuses_ops_without_a_device_implementation():
+    from theano_amd.gof import Apply, Op
+
+    class HostOnly(Op):
+        def make_node(self, x):
+            return Apply(self, [x], [x.type()])
+    x = T.fmatrix()
+    with pytest.raises(NotImplementedError, match="no HIP implementation"):
+        th.function([x], HostOnly()(x))
+
+
+def test_host_ops_have_no_compute_path():
+    x = T.fmatrix()
+    node = (x + x).owner
+    with pytest.raises(NotImplementedError):
+        node.op.perform(node, [np.zeros((2, 2), "float32")] * 2, [[None]])
+
+
+def test_device_outputs_and_inputs(dry_run):
+    from theano_amd.hip import HipArray
+    x = T.fmatrix()
+    f = th.function([x], th.Out(x * 2, device=True))
+    assert len(ops_of(f, HipToHost)) == 0
+    out = f(np.zeros((3, 4), "float32"))
+    assert isinstance(out, HipArray) and out.shape == (3, 4)
+    out2 = f(out)  # a device array is accepted for a host-typed input
+    assert isinstance(out2, HipArray)

@@ -1,0 +1,199 @@
+"""Pins the graph half of the oracle (Elemwise / CAReduce / DimShuffle
+evaluation) against the reference's literal test answers and against closed
+forms that a dropped term, wrong axis or wrong accumulator would break."""
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import tensor as T
+from oracle import graph_ref as G
+
+# shapes x axes of theano/tensor/tests/test_elemwise.py:352-366
+CAREDUCE_CASES = [((5, 6), None), ((5, 6), (0, 1)), ((5, 6), (0,)), ((5, 6), (1,)), ((5, 6), (-1,)), ((5, 6), (-2,)),
+                  ((5, 6), ()), ((2, 3, 4, 5), (0, 1, 3)), ((2, 3, 4, 5), (-2, -3)), ((5, 0), None), ((5, 0), (0,)),
+                  ((5, 0), (1,)), ((5, 0), ()), ((), None), ((), ())]
+
+
+def _np_reduce(ufunc, x, axis, acc, out):
+    # CAReduce.perform (theano/tensor/elemwise.py:1335-1369): highest axis first, in the accumulator dtype
+    axis = range(x.ndim) if axis is None else [a + x.ndim if a < 0 else a for a in axis]
+    v = x.astype(acc)
+    for a in sorted(axis, reverse=True):
+        v = ufunc.reduce(v, a, dtype=acc)
+    return np.asarray(v).astype(out)
+
+
+@pytest.mark.parametrize("shape,axis", CAREDUCE_CASES)
+def test_careduce_cases_against_numpy(shape, axis):
+    rng = np.random.default_rng(3)
+    x = rng.integers(-5, 6, shape).astype("int32")
+    xf = rng.standard_normal(shape).astype("float32")
+    assert np.array_equal(G.careduce(x, "Add", axis, "int64", "int64"), _np_reduce(np.add, x, axis, "int64", "int64"))
+    assert np.array_equal(G.careduce(x, "Mul", axis, "int64", "int64"),
+                          _np_reduce(np.multiply, x, axis, "int64", "int64"))
+    assert np.allclose(G.careduce(xf, "Add", axis, "float64", "float32"),
+                       _np_reduce(np.add, xf, axis, "float64", "float32"), rtol=1e-6)
+    red = [shape[a] for a in (range(len(shape)) if axis is None else axis)]
+    if 0 in red:
+        with pytest.raises(ValueError):  # theano/tensor/tests/test_elemwise.py:465-472
+            G.careduce(xf, "Maximum", axis, "float32", "float32")
+    else:
+        assert np.array_equal(G.careduce(xf, "Maximum", axis, "float32", "float32"),
+                              _np_reduce(np.maximum, xf, axis, "float32", "float32"))
+        assert np.array_equal(G.careduce(xf, "Minimum", axis, "float32", "float32"),
+                              _np_reduce(np.minimum, xf, axis, "float32", "float32"))
+    b = x > 0
+    assert np.array_equal(G.careduce(b, "OR", axis, "bool", "bool"), _np_reduce(np.logical_or, b, axis, "bool", "bool"))
+    assert np.array_equal(G.careduce(b, "AND", axis, "bool", "bool"),
+                          _np_reduce(np.logical_and, b, axis, "bool", "bool"))
+    assert np.array_equal(G.careduce(x, "XOR", axis, "int32", "int32"),
+                          _np_reduce(np.bitwise_xor, x, axis, "int32", "int32"))
+
+
+def test_reference_literal_answers():
+    # theano/tensor/tests/test_elemwise.py:654 and :680
+    x = np.asarray([[1., 2., 3.], [0., 5., 6.], [0., 0., 9.]], dtype="float32")
+    assert np.allclose(G.careduce(x, "Mul", (1,), "float64", "float32"), [6., 0., 0.])
+    y = np.array([[1, 2, 3], [4, 5, 6], [7, 8, 9]], dtype="float32")
+    assert np.allclose(G.careduce(y, "Mul", (1,), "float64", "float32"), [6, 120, 504])
+    # :953-966  float32 sum of [1e8, 1, -1e8] must be 1: needs the float64 accumulator
+    z = np.asarray([1e8, 1, -1e8], dtype="float32")
+    assert float(G.careduce(z, "Add", None, "float64", "float32")) == 1.0
+    assert float(G.careduce(z, "Add", None, "float32", "float32")) == 0.0  # a float32 accumulator loses it
+
+
+def test_sequential_order_is_observable():
+    # accumulation in float32 from left to right: 1 + 2^-24 * k never leaves 1.0, a pairwise sum would
+    x = np.full(4096, 2.0 ** -24, dtype="float32")
+    x[0] = 1.0
+    assert float(G.careduce(x, "Add", None, "float32", "float32")) == 1.0
+    assert float(G.careduce(x, "Add", None, "float64", "float32")) > 1.0
+
+
+def test_nan_propagates_through_max_min():
+    # theano/tensor/tests/test_elemwise.py:525-538
+    x = np.array([[1.0, np.nan, 3.0], [4.0, 5.0, 6.0]], dtype="float32")
+    mx = G.careduce(x, "Maximum", (1,), "float32", "float32")
+    assert np.isnan(mx[0]) and mx[1] == 6.0
+    mn = G.careduce(x, "Minimum", (0,), "float32", "float32")
+    assert np.isnan(mn[1]) and mn[0] == 1.0
+
+
+def test_strided_and_transposed_inputs():
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((7, 9, 11)).astype("float32")
+    v = x.transpose(2, 0, 1)[::2]
+    assert np.allclose(G.careduce(v, "Add", (0, 2), "float64", "float32"), v.astype("float64").sum((0, 2)), rtol=1e-6)
+
+
+def test_dtype_tables_of_the_product_match_reference_literals():
+    # theano/tensor/tests/test_elemwise.py:828-836 and :854-865
+    out_tbl = dict(bool="int64", int8="int64", int16="int64", int32="int64", uint8="uint64", uint16="uint64",
+                   uint32="uint64")
+    acc_tbl = dict(out_tbl, float16="float32", float32="float64")
+    for dt in ("bool", "int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64", "float16",
+               "float32", "float64"):
+        x = T.TensorType(dt, (False, False))()
+        for method in ("sum", "prod"):
+            s = getattr(x, method)(axis=0)
+            assert s.type.dtype == out_tbl.get(dt, dt)
+            assert s.owner.op.acc_dtype == acc_tbl.get(dt, dt)
+    assert G.SUM_OUT_DTYPE == out_tbl and G.SUM_ACC_DTYPE == acc_tbl
+    with pytest.raises(TypeError):  # precision loss, theano/tensor/elemwise.py:1766-1778
+        T.TensorType("float64", (False,))().sum(acc_dtype="float32")
+
+
+def test_elemwise_graph_closed_forms():
+    # the constant-filled inputs of theano/tensor/tests/test_opt.py:948-961 (1, 2, 3, 4 / 60, 70, 70)
+    shp = (5, 5)
+    fw, fx, fy, fz = [T.TensorType("float32", (False, False))(n) for n in "wxyz"]
+    ix, iy = T.imatrix("ix"), T.imatrix("iy")
+    fwv, fxv, fyv, fzv = [np.zeros(shp, "float32") + k for k in (1, 2, 3, 4)]
+    ixv, iyv = np.zeros(shp, "int32") + 60, np.zeros(shp, "int32") + 70
+    cases = [
+        (fx + fy + fz, [fx, fy, fz], [fxv, fyv, fzv], fxv + fyv + fzv),
+        (fx * fy + fz + fy, [fx, fy, fz], [fxv, fyv, fzv], fxv * fyv + fzv + fyv),
+        ((fw + fx) + (fy + fz) + 2., [fw, fx, fy, fz], [fwv, fxv, fyv, fzv], fwv + fxv + fyv + fzv + 2),
+        (fx - fy + T.tan(fz), [fx, fy, fz], [fxv, fyv, fzv], fxv - fyv + np.tan(fzv)),
+        (fx - fy + T.neg(fz) / T.exp(fw), [fw, fx, fy, fz], [fwv, fxv, fyv, fzv], fxv - fyv - fzv / np.exp(fwv)),
+        (ix + iy + fz, [ix, iy, fz], [ixv, iyv, fzv], (ixv + iyv + fzv.astype("float64"))),
+        (T.true_div(ix, iy) * fx, [ix, iy, fx], [ixv, iyv, fxv], (np.float32(60 / 70) * fxv)),
+        (T.int_div(ix, iy) + iy % ix, [ix, iy], [ixv, iyv], ixv // iyv + iyv % ixv),
+        (T.eq(fx, fy) + T.lt(fx, fy) * T.cast(fz, "int8"), [fx, fy, fz], [fxv, fyv, fzv],
+         ((fxv == fyv) + (fxv < fyv) * fzv.astype("int8")).astype("int8")),
+        (T.switch(fx > fy, fz, fw) + T.sqr(fx), [fw, fx, fy, fz], [fwv, fxv, fyv, fzv],
+         np.where(fxv > fyv, fzv, fwv) + fxv * fxv),
+    ]
+    for out, ins, vals, ref in cases:
+        (got,) = G.evaluate(ins, [out], vals)
+        assert got.dtype == ref.dtype, (out, got.dtype, ref.dtype)
+        assert np.allclose(got, ref, rtol=1e-6)
+
+
+def test_composite_codegen_fixture():
+    # theano/tensor/tests/test_opt.py:1355-1362: [1, 2, 3] -> [6, 12, 18] through x * 2 * 3
+    x = T.fvector("x")
+    (got,) = G.evaluate([x], [x * 2 * 3], [np.array([1, 2, 3], "float32")])
+    assert np.array_equal(got, np.array([6, 12, 18], "float32"))
+
+
+def test_broadcast_mismatch_raises():
+    # theano/tensor/tests/test_basic.py:686-688: (2, 3) + (3, 2) and (2, 3) + (1, 2)
+    x, y = T.fmatrix(), T.fmatrix()
+    with pytest.raises(ValueError):
+        G.evaluate([x, y], [x + y], [np.zeros((2, 3), "float32"), np.zeros((3, 2), "float32")])
+    with pytest.raises(ValueError):
+        G.evaluate([x, y], [x + y], [np.zeros((2, 3), "float32"), np.zeros((1, 2), "float32")])
+
+
+def test_softmax_and_its_gradient_closed_form():
+    rng = np.random.default_rng(11)
+    xv = (3 * rng.standard_normal((6, 17))).astype("float32")
+    yv = rng.uniform(0, 1, (6, 17)).astype("float32")
+    x, y = T.fmatrix(), T.fmatrix()
+    out = T.softmax(x)
+    dx = th.grad(T.sum(out * y), x)
+    sm_ref = np.exp(xv.astype("float64") - xv.max(1, keepdims=True))
+    sm_ref /= sm_ref.sum(1, keepdims=True)
+    got, gdx = G.evaluate([x, y], [out, dx], [xv, yv])
+    assert np.allclose(got, sm_ref, rtol=1e-5, atol=1e-7)
+    assert np.allclose(gdx, sm_ref * (yv - (sm_ref * yv).sum(1, keepdims=True)), rtol=1e-4, atol=1e-7)
+
+
+def test_gradients_against_finite_differences():
+    from theano_amd.gradient import numeric_grad
+    rng = np.random.default_rng(2)
+    x = T.TensorType("float64", (False, False))("x")
+    g = T.TensorType("float64", (True, False))("g")
+    cost = T.sum(T.sigmoid(x * g) * T.sqr(x) + T.log(1 + T.exp(x)) / T.sqrt(T.sqr(g) + 1)) + T.max(x, axis=1).sum()
+    gx, gg = th.grad(cost, [x, g])
+    xv, gv = rng.standard_normal((4, 5)), rng.standard_normal((1, 5))
+
+    def f(a, b):
+        return float(G.evaluate([x, g], [cost], [a, b])[0])
+    nx, ng = numeric_grad(f, [xv, gv])
+    ax, ag = G.evaluate([x, g], [gx, gg], [xv, gv])
+    assert np.allclose(ax, nx, rtol=1e-5, atol=1e-6) and np.allclose(ag, ng, rtol=1e-5, atol=1e-6)
+
+
+def test_batchnorm_gradient_closed_form():
+    # AbstractBatchNormTrainGrad.perform, theano/tensor/nnet/bn.py:659-676
+    rng = np.random.default_rng(4)
+    shape = (5, 3, 4, 2)
+    t4 = T.TensorType("float64", (False,) * 4)
+    pc = T.TensorType("float64", (True, False, True, True))
+    x, dy, gam = t4("x"), t4("dy"), pc("gamma")
+    eps = 1e-5
+    mean = x.mean(axis=(0, 2, 3), keepdims=True)
+    var = x.var(axis=(0, 2, 3), keepdims=True)
+    y = gam * (x - mean) / T.sqrt(var + eps)
+    gx, ggam = th.grad(T.sum(y * dy), [x, gam])
+    xv, dyv, gv = rng.standard_normal(shape), rng.standard_normal(shape), rng.standard_normal((1, 3, 1, 1))
+    ax, ag = G.evaluate([x, dy, gam], [gx, ggam], [xv, dyv, gv])
+    axes = (0, 2, 3)
+    m, v = xv.mean(axes, keepdims=True), xv.var(axes, keepdims=True)
+    invstd = 1 / np.sqrt(v + eps)
+    xmu = xv - m
+    dscale = (dyv * xmu * invstd).sum(axes, keepdims=True)
+    dx = gv * invstd * (dyv - dyv.mean(axes, keepdims=True) - xmu * invstd ** 2 * (dyv * xmu).mean(axes, keepdims=True))
+    assert np.allclose(ag, dscale, rtol=1e-9) and np.allclose(ax, dx, rtol=1e-8, atol=1e-10)

@@ -1,0 +1,114 @@
+"""Pins the scalar half of the oracle against facts that do not come from the
+oracle itself: Python integer arithmetic, truth tables, closed forms and the
+literal dtype tables of the reference."""
+import itertools
+import math
+
+import numpy as np
+import pytest
+
+from oracle import scalar_ref as S
+
+
+def test_mod_intdiv_exhaustive_int8_grid():
+    # the grid of theano/tensor/tests/test_basic.py:878-896: every int8 dividend, every non-zero int8 divisor
+    a = np.arange(-127, 128, dtype="int8")[:, None]
+    b = np.array([v for v in range(-127, 128) if v != 0], dtype="int8")[None, :]
+    py_mod = np.array([[int(x) % int(y) for y in b[0]] for x in a[:, 0]], dtype="int8")
+    py_div = np.array([[int(x) // int(y) for y in b[0]] for x in a[:, 0]], dtype="int8")
+    assert np.array_equal(S.mod("int8", a, b), py_mod)          # literal four-case restatement
+    assert np.array_equal(S.int_div("int8", a, b), py_div)
+    assert np.array_equal(S.mod_fast("int8", a, b), py_mod)      # vectorised form used on large inputs
+    assert np.array_equal(S.int_div_fast("int8", a, b), py_div)
+
+
+def test_mod_sign_table():
+    # theano/scalar/tests/test_basic.py:53-64
+    for x, y in itertools.product((5, -5, 0, 7), (3, -3)):
+        got = S.mod("int32", np.asarray(x, "int32"), np.asarray(y, "int32"))
+        assert int(got) == x % y
+    got = S.mod("float64", np.asarray(-5.5), np.asarray(3.0))
+    assert float(got) == pytest.approx(-5.5 % 3.0)
+
+
+def test_right_shift_is_floor_division_by_power_of_two():
+    a = np.arange(-4096, 4096, dtype="int32")
+    for k in (1, 3, 5):
+        assert np.array_equal(S.right_shift("int32", a, np.asarray(k, "int32")),
+                              S.int_div_fast("int32", a, np.asarray(2 ** k, "int32")))
+        assert np.array_equal(S.right_shift("int32", a, np.asarray(k, "int32")),
+                              np.array([int(v) // (2 ** k) for v in a], dtype="int32"))
+
+
+def test_comparison_and_bit_truth_tables():
+    # theano/scalar/tests/test_basic.py:187-256
+    for x, y in itertools.product((-1, 0, 1, 2), repeat=2):
+        xs, ys = np.asarray(x, "int32"), np.asarray(y, "int32")
+        assert bool(S.lt("bool", xs, ys)) == (x < y)
+        assert bool(S.le("bool", xs, ys)) == (x <= y)
+        assert bool(S.gt("bool", xs, ys)) == (x > y)
+        assert bool(S.ge("bool", xs, ys)) == (x >= y)
+        assert bool(S.eq("bool", xs, ys)) == (x == y)
+        assert bool(S.neq("bool", xs, ys)) == (x != y)
+        assert int(S.and_("int32", xs, ys)) == (x & y)
+        assert int(S.or_("int32", xs, ys)) == (x | y)
+        assert int(S.xor("int32", xs, ys)) == (x ^ y)
+    assert int(S.invert("int8", np.asarray(5, "int8"))) == ~5
+    assert bool(S.invert("bool", np.asarray(True))) is False
+
+
+def test_bool_add_mul_are_logical():
+    # theano/scalar/basic.py:1711-1712, 1753-1754
+    t, f = np.asarray(True), np.asarray(False)
+    assert bool(S.add("bool", t, t)) is True and bool(S.add("bool", f, f)) is False
+    assert bool(S.mul("bool", t, f)) is False and bool(S.mul("bool", t, t)) is True
+
+
+def test_sigmoid_closed_form_and_thresholds():
+    x = np.linspace(-30, 14, 89).astype("float32")
+    ref = 1.0 / (1.0 + np.exp(-x.astype("float64")))
+    assert np.allclose(S.scalar_sigmoid("float32", x), ref, rtol=1e-6)
+    assert float(S.scalar_sigmoid("float32", np.float32(-89.0))) == 0.0
+    assert float(S.scalar_sigmoid("float32", np.float32(15.5))) == 1.0
+    assert float(S.scalar_sigmoid("float64", np.float64(19.5))) == 1.0
+    assert float(S.scalar_sigmoid("float64", np.float64(-710.0))) == 0.0
+
+
+def test_max_min_propagate_nan():
+    a, n = np.float32(1.0), np.float32(np.nan)
+    for fn in (S.maximum, S.minimum):
+        assert math.isnan(float(fn("float32", a, n))) and math.isnan(float(fn("float32", n, a)))
+    assert float(S.maximum("float32", np.float32(-0.5), a)) == 1.0
+    assert float(S.minimum("float32", np.float32(-0.5), a)) == -0.5
+
+
+def test_cast_to_bool_and_integer_wrap():
+    assert np.array_equal(S.cast("bool", np.array([0, 2, -1, 256], "int32")), [False, True, True, True])
+    assert np.array_equal(S.add("int8", np.array([127], "int8"), np.array([1], "int8")), np.array([-128], "int8"))
+    assert np.array_equal(S.mul("int32", np.array([2 ** 30], "int32"), np.array([4], "int32")), np.array([0], "int32"))
+
+
+def test_true_div_of_integers_goes_through_double():
+    got = S.true_div("float32", np.array([1, 7], "int32"), np.array([3, 2], "int32"))
+    assert got.dtype == np.float32 and np.array_equal(got, np.array([1 / 3, 3.5]).astype("float32"))
+
+
+def test_c_common_type_matches_c_rules():
+    c = S.c_common_type
+    assert c("int8", "int8") == "int32" and c("bool", "bool") == "int32"
+    assert c("uint32", "int32") == "uint32" and c("uint32", "int64") == "int64"
+    assert c("uint64", "int64") == "uint64" and c("int32", "float32") == "float32"
+    assert c("int64", "float32", "float64") == "float64"
+
+
+def test_product_dtype_tables_against_reference_literals():
+    # theano/scalar/basic.py:855-870 (upgrade_to_float) through the product's scalar module
+    from theano_amd import scalar as scal
+    table = {"bool": "float32", "int8": "float32", "int16": "float32", "int32": "float64", "int64": "float64",
+             "uint8": "float32", "uint16": "float32", "uint32": "float64", "uint64": "float64",
+             "float32": "float32", "float64": "float64"}
+    for src, dst in table.items():
+        assert scal.exp(scal.Scalar(src)()).type.dtype == dst
+    # upcast follows NumPy array promotion
+    for a, b in itertools.product(scal.all_dtypes, repeat=2):
+        assert scal.upcast(a, b) == str((np.zeros((), a) + np.zeros((), b)).dtype)

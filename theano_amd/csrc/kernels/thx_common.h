@@ -16,6 +16,13 @@ typedef _Float16 thx_f16;
 typedef float thx_f32;
 typedef double thx_f64;
 
+#ifndef INFINITY
+#define INFINITY (__builtin_inff())
+#endif
+#ifndef NAN
+#define NAN (__builtin_nanf(""))
+#endif
+
 #define THX_DEV __device__ __forceinline__
 #define THX_WAVE 64
 

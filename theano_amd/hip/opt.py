@@ -43,7 +43,8 @@ def _lift_reduce(node, x):
         acc, out = idt, op._output_dtype(idt)
         if isinstance(op, (All, Any)):
             acc = "bool"
-    if acc == "float16":
+    if acc == "float16" and not isinstance(op.scalar_op, (scal.Maximum, scal.Minimum)):
+        # max / min are exact in any precision; a float16 running sum or product has no reference C code
         raise NotImplementedError("float16 accumulators are not supported (as theano/tensor/elemwise.py:1395-1398)")
     return HipCAReduce((op.scalar_op,), op.axis if op.axis is not None else tuple(range(x.type.ndim)),
                        (acc,), (out,))(x)
@@ -337,8 +338,9 @@ def _merge_two(a, b):
 
 # --------------------------------------------------------------------------
 def optimize(fgraph, fuse=True):
-    """Full pipeline: merge, lift, fuse."""
-    gof.merge_identical(fgraph)
+    """Full pipeline: clean up, lift, fuse."""
+    from ..tensor.opt import canonicalize
+    canonicalize(fgraph)
     fgraph = lift_to_hip(fgraph)
     gof.merge_identical(fgraph)
     if fuse:

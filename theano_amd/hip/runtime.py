@@ -243,7 +243,7 @@ class HipArray(object):
         a = np.asarray(a)
         if str(a.dtype) not in scal.all_dtypes:
             raise TypeError("dtype %s is not supported on the device" % a.dtype)
-        a = np.ascontiguousarray(a)
+        a = np.asarray(a, order="C")
         out = cls.empty(a.shape, a.dtype)
         if a.nbytes and not out.buffer.fake:
             check(lib.thx_h2d(out.buffer.ptr, a.ctypes.data, a.nbytes))

@@ -81,7 +81,7 @@ class DimShuffle(Op):
         (x,) = inputs
         if not isinstance(x, np.ndarray):
             raise TypeError("DimShuffle.perform takes a host ndarray; device arrays go through HipDimShuffle")
-        res = x.transpose(self.shuffle + self.drop)
+        res = x.transpose(self.shuffle + self.drop) if x.ndim else x
         shape = list(res.shape[:len(self.shuffle)])
         for augm in self.augment:
             shape.insert(augm, 1)

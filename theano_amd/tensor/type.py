@@ -213,7 +213,7 @@ def constant(x, name=None, ndim=None, dtype=None):
             x_ = x_.reshape((1,) * (ndim - x_.ndim) + x_.shape)
         elif len(bcast) > ndim:
             raise ValueError("constant has %d dimensions, asked for %d" % (len(bcast), ndim))
-    return TensorConstant(TensorType(str(x_.dtype), bcast), np.ascontiguousarray(x_), name=name)
+    return TensorConstant(TensorType(str(x_.dtype), bcast), np.asarray(x_, order="C"), name=name)
 
 
 def as_tensor_variable(x, name=None, ndim=None):
