@@ -85,6 +85,8 @@ def careduce(x, op_name, axis, acc_dtype, out_dtype):
     acc_dtype, out_dtype = str(acc_dtype), str(out_dtype)
     if x.dtype == np.float16:
         x = x.astype("float32")  # no float16 C code exists in the reference (elemwise.py:1395-1398)
+        if acc_dtype == "float16":  # max / min: exact in any precision
+            acc_dtype = "float32"
     kept = tuple(s for d, s in enumerate(x.shape) if d not in axis)
     acc = np.empty(kept, dtype=acc_dtype)
     ident = reduce_identity(op_name, acc_dtype)

@@ -134,6 +134,7 @@ class Function(object):
                                 [self.storage[o] for o in node.outputs]))
         self._constants_ready = False
         self._HipArray = HipArray
+        self._last_shape = {}
 
     def _upload_constants(self):
         for c in self.constants:
@@ -147,9 +148,12 @@ class Function(object):
             self._upload_constants()
         HipArray = self._HipArray
         for spec, var, a in zip(self.in_specs, self.fgraph.inputs, args):
+            if type(a) is np.ndarray and a.dtype == var.type.numpy_dtype and a.shape == self._last_shape.get(var):
+                self.storage[var][0] = a  # same dtype and shape as a value that already passed the full check
+                continue
             if isinstance(a, HipArray) and isinstance(var.type, TensorType):
                 # device-resident argument for a host-typed input: checked like a host value
-                if str(a.dtype) != var.type.dtype or a.ndim != var.type.ndim:
+                if a.dtype != var.type.numpy_dtype or len(a.shape) != var.type.ndim:
                     raise TypeError("Bad input argument %s: expected %s, got %s" % (spec.name, var.type, a))
                 for d, b in enumerate(var.type.broadcastable):
                     if b and a.shape[d] != 1:
@@ -158,7 +162,9 @@ class Function(object):
                 self.storage[var][0] = a
             else:
                 try:
-                    self.storage[var][0] = var.type.filter(a, strict=False, allow_downcast=spec.allow_downcast)
+                    v = self.storage[var][0] = var.type.filter(a, strict=False, allow_downcast=spec.allow_downcast)
+                    if type(v) is np.ndarray:
+                        self._last_shape[var] = v.shape
                 except TypeError as e:
                     raise TypeError("Bad input argument to theano function with name \"%s\": %s" % (spec.name, e))
         for k, (perform, node, ins, outs) in enumerate(self.thunks):

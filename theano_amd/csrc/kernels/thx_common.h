@@ -42,6 +42,43 @@ struct __attribute__((aligned(AlignFor<sizeof(T) * N>::value))) Vec {
   T v[N];
 };
 
+// Raw B-byte accesses, optionally with the non-temporal hint (data that is
+// touched once should not displace anything in L2).
+typedef unsigned int thx_u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int thx_u32x2 __attribute__((ext_vector_type(2)));
+
+template <int B> struct RawOf;
+template <> struct RawOf<16> { typedef thx_u32x4 type; };
+template <> struct RawOf<8> { typedef thx_u32x2 type; };
+template <> struct RawOf<4> { typedef unsigned int type; };
+template <> struct RawOf<2> { typedef unsigned short type; };
+template <> struct RawOf<1> { typedef unsigned char type; };
+
+template <class T, int N, bool NT>
+THX_DEV void load_vec(Vec<T, N>& r, const T* b) {
+  constexpr int BYTES = sizeof(T) * N;
+  constexpr int CH = BYTES >= 16 ? 16 : BYTES;  // bytes per access
+  typedef typename RawOf<CH>::type Raw;
+  Raw* dst = (Raw*)&r;
+  const Raw* src = (const Raw*)b;
+#pragma unroll
+  for (int c = 0; c < BYTES / CH; ++c) dst[c] = NT ? __builtin_nontemporal_load(src + c) : src[c];
+}
+
+template <class T, int N, bool NT>
+THX_DEV void store_vec(T* b, const Vec<T, N>& r) {
+  constexpr int BYTES = sizeof(T) * N;
+  constexpr int CH = BYTES >= 16 ? 16 : BYTES;
+  typedef typename RawOf<CH>::type Raw;
+  const Raw* src = (const Raw*)&r;
+  Raw* dst = (Raw*)b;
+#pragma unroll
+  for (int c = 0; c < BYTES / CH; ++c) {
+    if (NT) __builtin_nontemporal_store(src[c], dst + c);
+    else dst[c] = src[c];
+  }
+}
+
 // Division by a run-time constant d >= 2 for dividends below 2^31:
 // q = mulhi(n, m) >> s with m = ceil(2^(31+L)/d), s = L-1, L = ceil(log2 d).
 struct FastDiv {
@@ -49,7 +86,7 @@ struct FastDiv {
 };
 
 THX_DEV void divmod(unsigned n, const FastDiv& f, unsigned& q, unsigned& r) {
-  q = __umulhi(n, f.m) >> f.s;
+  q = f.d == 1 ? n : (__umulhi(n, f.m) >> f.s);
   r = n - q * f.d;
 }
 THX_DEV void divmod(unsigned long long n, const FastDiv& f, unsigned long long& q,

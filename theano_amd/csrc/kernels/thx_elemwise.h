@@ -7,7 +7,7 @@
 //   template <int V> static void compute(Regs<V>&);     // the scalar graph, V times
 //   template <int V, class A> static void store(const A&, const Regs<V>&);
 // and a generated plan P supplies
-//   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK };
+//   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK, NT (non-temporal accesses) };
 //   static constexpr int mode(int operand);             // M_VEC / M_BCAST / M_GATHER
 // The host collapses dimensions, so ND is the rank after merging every pair of
 // neighbouring dimensions that all operands walk with compatible strides.
@@ -45,7 +45,7 @@ struct EwAcc {
     if (N == 1) {
       r.v[0] = *b;
     } else if (P::mode(I) == M_VEC) {
-      r = *(const Vec<T, N>*)b;
+      load_vec<T, N, P::NT != 0>(r, b);
     } else if (P::mode(I) == M_BCAST) {
       const T s = *b;
 #pragma unroll
@@ -63,7 +63,7 @@ struct EwAcc {
     if (N == 1) {
       *b = r.v[0];
     } else if (P::mode(I) == M_VEC) {
-      *(Vec<T, N>*)b = r;
+      store_vec<T, N, P::NT != 0>(b, r);
     } else {
       const IT st = stride[I][P::ND - 1];
 #pragma unroll
@@ -134,6 +134,142 @@ __device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename 
       F::template compute<1>(r1);
       F::template store<1>(a1, r1);
     }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Permuted-read variant. Some inputs are unit-stride along a dimension T that
+// is not the innermost one of the result (a dimshuffled view). A block owns a
+// TILE x TILE patch of (T, innermost): those inputs are read in rows along T
+// - full cache lines - into LDS and read back transposed, while every other
+// operand is accessed along the innermost dimension. Rows of a tile are padded
+// by one element so that the transposed reads hit distinct banks.
+//
+// Extra plan members: enum { TILE, NTR (staged inputs), ESZ (largest staged
+// element) }; static constexpr int slot(int operand): LDS slot or -1.
+template <int NOPS, int ND, class IT>
+struct EwTrParams {
+  char* ptr[NOPS];
+  unsigned long long imm[NOPS];
+  int ext_t, ext_i;         // extents of dimension T and of the innermost dimension
+  FastDiv tiles_i, tiles_t;  // tiles along each of them
+  FastDiv ofd[ND];          // extents of the other (outer) dimensions, ND - 2 of them used
+  IT ostride[NOPS][ND];     // strides along the outer dimensions
+  IT tstride[NOPS];
+  IT istride[NOPS];
+};
+
+template <class P, int NOPS>
+struct TrStageAcc {  // global -> LDS for the staged inputs, nothing for the others
+  typedef typename P::IT IT;
+  char* const* ptr;
+  unsigned char* lds;
+  IT off[NOPS];
+  int cell;
+  template <int I, class T, int N>
+  THX_DEV void ld(Vec<T, N>&) const {
+    if (P::slot(I) >= 0) {
+      T* tile = (T*)(lds + P::slot(I) * (P::TILE * (P::TILE + 1) * P::ESZ));
+      tile[cell] = *((const T*)ptr[I] + off[I]);
+    }
+  }
+};
+
+template <class P, int NOPS>
+struct TrAcc {  // LDS (transposed) or global -> registers, registers -> global
+  typedef typename P::IT IT;
+  char* const* ptr;
+  const unsigned long long* imm;
+  const unsigned char* lds;
+  IT off[NOPS];
+  int cell;
+  template <int I, class T, int N>
+  THX_DEV void ld(Vec<T, N>& r) const {
+    if (P::slot(I) >= 0) {
+      const T* tile = (const T*)(lds + P::slot(I) * (P::TILE * (P::TILE + 1) * P::ESZ));
+      r.v[0] = tile[cell];
+    } else if (P::mode(I) == M_IMM) {
+      r.v[0] = *(const T*)&imm[I];
+    } else {
+      r.v[0] = *((const T*)ptr[I] + off[I]);
+    }
+  }
+  template <int I, class T, int N>
+  THX_DEV void st(const Vec<T, N>& r) const {
+    *((T*)ptr[I] + off[I]) = r.v[0];
+  }
+};
+
+template <class F, class P>
+__device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, typename P::IT>& p) {
+  typedef typename P::IT IT;
+  constexpr int TILE = P::TILE, NOPS = F::NOPS, ND = P::ND, ROWS = P::BLOCK / TILE, UNR = 4;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[P::NTR * TILE * (TILE + 1) * P::ESZ];
+
+  unsigned rem = blockIdx.x, ti, tt, c;
+  divmod(rem, p.tiles_i, rem, ti);
+  divmod(rem, p.tiles_t, rem, tt);
+  IT base[NOPS];
+#pragma unroll
+  for (int i = 0; i < NOPS; ++i) base[i] = 0;
+#pragma unroll
+  for (int d = ND - 3; d >= 1; --d) {
+    divmod(rem, p.ofd[d], rem, c);
+#pragma unroll
+    for (int i = 0; i < NOPS; ++i) base[i] += (IT)c * p.ostride[i][d];
+  }
+  if (ND >= 3) {
+#pragma unroll
+    for (int i = 0; i < NOPS; ++i) base[i] += (IT)rem * p.ostride[i][0];
+  }
+  const int t0 = tt * TILE, i0 = ti * TILE;
+  const int lane = threadIdx.x % TILE, row = threadIdx.x / TILE;
+
+  // stage: lanes run along T
+  {
+    typename F::template Regs<1> dummy;
+    const int t = t0 + lane;
+#pragma unroll
+    for (int k = 0; k < TILE / ROWS; ++k) {
+      const int ii = row + k * ROWS, i = i0 + ii;
+      if (t < p.ext_t && i < p.ext_i) {
+        TrStageAcc<P, NOPS> a;
+        a.ptr = p.ptr;
+        a.lds = lds;
+        a.cell = ii * (TILE + 1) + lane;
+#pragma unroll
+        for (int o = 0; o < NOPS; ++o) a.off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
+        F::template load<1>(a, dummy);
+      }
+    }
+  }
+  __syncthreads();
+
+  // compute: lanes run along the innermost dimension
+  const int i = i0 + lane;
+#pragma unroll
+  for (int k0 = 0; k0 < TILE / ROWS; k0 += UNR) {
+    typename F::template Regs<1> r[UNR];
+    TrAcc<P, NOPS> a[UNR];
+    bool ok[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int tl = row + (k0 + u) * ROWS, t = t0 + tl;
+      ok[u] = t < p.ext_t && i < p.ext_i;
+      a[u].ptr = p.ptr;
+      a[u].imm = p.imm;
+      a[u].lds = lds;
+      a[u].cell = lane * (TILE + 1) + tl;
+#pragma unroll
+      for (int o = 0; o < NOPS; ++o) a[u].off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
+      if (ok[u]) F::template load<1>(a[u], r[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
+      if (ok[u]) F::template compute<1>(r[u]);
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
+      if (ok[u]) F::template store<1>(a[u], r[u]);
   }
 }
 

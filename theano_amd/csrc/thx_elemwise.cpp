@@ -1,6 +1,7 @@
 // Elementwise planner: validates operands, collapses dimensions, picks an
 // access plan (rank, index width, vector width, per-operand access mode),
 // compiles the matching kernel on first use and launches it.
+#include <algorithm>
 #include <cstdlib>
 #include <cstring>
 #include <sstream>
@@ -188,14 +189,100 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   };
   while (!vec_ok(vec)) vec /= 2;
 
+  // permuted-read plan: inputs that are unit-stride along another dimension T go through LDS tiles
+  if (ND >= 2 && !wide && !env_int("THX_EW_NO_TRANSPOSE", 0)) {
+    bool any_gather = false, outs_ok = true;
+    for (int o = 0; o < nops; ++o) {
+      if (o < e->n_in && mode[o] == M_GATHER) any_gather = true;
+      if (o >= e->n_in && mode[o] != M_VEC) outs_ok = false;
+    }
+    int tdim = -1;
+    if (any_gather && outs_ok && inner >= 16) {
+      for (int d = ND - 2; d >= 0 && tdim < 0; --d) {
+        if (dm.shape[d] < 16) continue;
+        bool ok = true;
+        for (int o = 0; o < e->n_in && ok; ++o)
+          if (mode[o] == M_GATHER && dm.stride[o][d] != 1) ok = false;
+        if (ok) tdim = d;
+      }
+    }
+    if (tdim >= 0) {
+      std::vector<int> slot(nops, -1);
+      int ntr = 0, esz = 1;
+      for (int o = 0; o < e->n_in; ++o)
+        if (mode[o] == M_GATHER) {
+          slot[o] = ntr++;
+          esz = std::max(esz, dtype_size(views[o].dtype));
+        }
+      int tile = 64;
+      if ((int64_t)ntr * tile * (tile + 1) * esz > 60000) tile = 32;
+      if ((int64_t)ntr * tile * (tile + 1) * esz <= 60000) {
+        const int block = 256;
+        const int nt = env_int("THX_NT", 0);
+        std::ostringstream key;
+        key << "et|nd" << ND << "|t" << tile << "|n" << ntr << "|e" << esz << (nt ? "|nt" : "") << "|m";
+        for (int o = 0; o < nops; ++o) key << (slot[o] >= 0 ? 9 : mode[o]) << (o + 1 < nops ? "," : "");
+        const std::string plan = key.str();
+        set_last_plan(e->name + "|" + plan);
+        Kernel k;
+        auto it = e->plans.find(plan);
+        if (it != e->plans.end() && (it->second.func || dry)) {
+          k = it->second;
+        } else {
+          std::ostringstream s;
+          s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef int IT;\n  enum { ND = " << ND
+            << ", TILE = " << tile << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz << ", NT = " << nt
+            << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+          for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
+          s << "};\n    return m[i];\n  }\n  static constexpr int slot(int i) {\n    constexpr int m[] = {";
+          for (int o = 0; o < nops; ++o) s << slot[o] << (o + 1 < nops ? ", " : "");
+          s << "};\n    return m[i];\n  }\n};\n"
+            << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::EwTrParams<" << e->name
+            << "::NOPS, ThxPlan::ND, ThxPlan::IT> p) {\n  thx::ew_tr_body<" << e->name << ", ThxPlan>(p);\n}\n";
+          rc = get_kernel(s.str(), "thx_entry", &k);
+          if (rc) return rc;
+          e->plans[plan] = k;
+        }
+        if (dry) return THX_OK;
+        const int64_t ext_t = dm.shape[tdim], ext_i = inner;
+        const int64_t tiles_t = (ext_t + tile - 1) / tile, tiles_i = (ext_i + tile - 1) / tile;
+        int64_t outer = 1;
+        std::vector<int> odims;
+        for (int d = 0; d < ND - 1; ++d)
+          if (d != tdim) {
+            odims.push_back(d);
+            outer *= dm.shape[d];
+          }
+        const int64_t grid = outer * tiles_t * tiles_i;
+        if (grid <= 0x7fffffffLL) {
+          ParamPack pk;
+          for (int o = 0; o < nops; ++o) pk.put<char*>(views[o].ptr);
+          for (int o = 0; o < nops; ++o) pk.put<uint64_t>(views[o].immval);
+          pk.put<int32_t>((int32_t)ext_t);
+          pk.put<int32_t>((int32_t)ext_i);
+          pk.put<FastDivH>(make_fastdiv((uint64_t)tiles_i));
+          pk.put<FastDivH>(make_fastdiv((uint64_t)tiles_t));
+          for (int d = 0; d < ND; ++d) pk.put<FastDivH>(make_fastdiv(d < (int)odims.size() ? (uint64_t)dm.shape[odims[d]] : 1));
+          for (int o = 0; o < nops; ++o)
+            for (int d = 0; d < ND; ++d) pk.put<int32_t>(d < (int)odims.size() ? (int32_t)dm.stride[o][odims[d]] : 0);
+          for (int o = 0; o < nops; ++o) pk.put<int32_t>((int32_t)dm.stride[o][tdim]);
+          for (int o = 0; o < nops; ++o) pk.put<int32_t>((int32_t)dm.stride[o][ND - 1]);
+          pk.align(8);
+          return launch(k, e->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
+        }
+      }
+    }
+  }
+
   const int64_t nvec = ND == 1 ? n / vec : n / vec;
   int unr = nvec >= (int64_t(1) << 20) ? 4 : (nvec >= (int64_t(1) << 18) ? 2 : 1);
   const int force_unr = env_int("THX_EW_UNR", 0);
   if (force_unr > 0) unr = force_unr;
   const int block = 256;
+  const int nt = env_int("THX_NT", 0) && n * 4 >= (int64_t(1) << 24);
 
   std::ostringstream key;
-  key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|m";
+  key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nt ? "|nt" : "") << "|m";
   for (int o = 0; o < nops; ++o) key << mode[o] << (o + 1 < nops ? "," : "");
   const std::string plan = key.str();
   set_last_plan(e->name + "|" + plan);
@@ -208,7 +295,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
     std::ostringstream s;
     s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
       << " IT;\n  enum { ND = " << ND << ", VEC = " << vec << ", UNR = " << unr << ", BLOCK = " << block
-      << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+      << ", NT = " << nt << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
     for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
     s << "};\n    return m[i];\n  }\n};\n"
       << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::EwParams<" << e->name

@@ -236,6 +236,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   };
 
   const int block = 256;
+  const int nt = env_int("THX_NT", 0);
   std::string plan;
   Kernel k;
   ParamPack pk;
@@ -290,7 +291,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     if (ra2 && nvec >= (int64_t(1) << 31) - 65536) wide = true;
     const int NK = std::max(1, NKD);
     std::ostringstream key;
-    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|t" << tpr << "|a" << ra2 << "|m";
+    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|t" << tpr << "|a" << ra2 << (nt ? "|nt" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str();
     auto it = r->plans.find(plan);
@@ -299,7 +300,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     } else {
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TPR", tpr}, {"RA2", ra2}}, mode)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TPR", tpr}, {"RA2", ra2}, {"NT", nt}}, mode)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -383,7 +384,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       }
     }
     std::ostringstream key;
-    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << "|r" << rr2 << "|m";
+    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << "|r" << rr2 << (nt ? "|nt" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str();
     auto it = r->plans.find(plan);
@@ -392,7 +393,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     } else {
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TX", tx}, {"RR2", rr2}}, mode)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TX", tx}, {"RR2", rr2}, {"NT", nt}}, mode)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::ColParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_col_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -442,7 +443,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     } else {
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}}, gmode)
+        << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}, {"NT", 0}}, gmode)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::GenParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, ThxPlan::NK, ThxPlan::NR, ThxPlan::IT> p) {\n  thx::red_gen_body<" << r->name
         << ", ThxPlan>(p);\n}\n";

@@ -186,12 +186,33 @@ def _operand(value, nd, slot):
 def _check_runtime_broadcast(node_inputs, values, nd):
     """Non-broadcastable dimensions must agree exactly; an extent of 1 only
     broadcasts where the type says so (``theano/tensor/elemwise.py:720-740``)."""
+    shape = None
+    for k, (var, val) in enumerate(zip(node_inputs, values)):
+        if type(val) is not HipArray:
+            if not isinstance(val, np.ndarray) or val.size != 1:
+                raise TypeError("input %d must be a device array or a one-element host array" % k)
+            continue
+        if shape is None and not any(var.type.broadcastable):
+            shape = val.shape  # fast path: the first full-shaped input fixes the result shape
+            if len(shape) != nd:
+                raise TypeError("input %d has rank %d, expected %d" % (k, len(shape), nd))
+            first = k
+    if shape is not None:
+        ok = True
+        for k, (var, val) in enumerate(zip(node_inputs, values)):
+            if type(val) is HipArray and val.shape != shape:
+                vs = val.shape
+                if len(vs) != nd or any(v != s and not (b and v == 1)
+                                        for v, s, b in zip(vs, shape, var.type.broadcastable)) or any(
+                                            b and v != 1 for v, b in zip(vs, var.type.broadcastable)):
+                    ok = False
+                    break
+        if ok:
+            return shape
     shape = [1] * nd
     owner = [None] * nd
     for k, (var, val) in enumerate(zip(node_inputs, values)):
         if not isinstance(val, HipArray):
-            if not isinstance(val, np.ndarray) or val.size != 1:
-                raise TypeError("input %d must be a device array or a one-element host array" % k)
             continue
         if val.ndim != nd:
             raise TypeError("input %d has rank %d, expected %d" % (k, val.ndim, nd))
@@ -258,27 +279,36 @@ class HipElemwise(Elemwise):
 
     def perform(self, node, inputs, output_storage):
         flags = call_flags()
-        handle, nin, nout = self._handle(node)
-        nd = node.outputs[0].type.ndim
+        cache = node.tag.get("thx")
+        if cache is None:
+            handle, nin, nout = self._handle(node)
+            cache = node.tag["thx"] = (handle, nin, nout, (thx_array * nin)(), (thx_array * nout)(),
+                                       node.outputs[0].type.ndim, dict(self.inplace_pattern),
+                                       [np.dtype(o.type.dtype) for o in node.outputs])
+        handle, nin, nout, ins, outs, nd, inplace, out_dt = cache
         shape = _check_runtime_broadcast(node.inputs, inputs, nd)
-        ins = (thx_array * nin)()
-        for k, v in enumerate(inputs):
-            _operand(v, nd, ins[k])
-        outs = (thx_array * nout)()
+        k = 0
+        for v in inputs:
+            if type(v) is HipArray:
+                v.as_thx(ins[k])
+            else:
+                host_scalar_thx(v, nd, ins[k])
+            k += 1
         results = []
-        inplace = dict(self.inplace_pattern)
-        for k, o in enumerate(node.outputs):
+        for k in range(nout):
             if k in inplace:
                 arr = inputs[inplace[k]]
                 if arr.shape != shape:
                     raise ValueError("in-place output %d has shape %s, the result has %s" % (k, arr.shape, shape))
             else:
-                arr = HipArray.empty(shape, o.type.dtype)
+                arr = HipArray._new_contiguous(shape, out_dt[k])
             arr.as_thx(outs[k])
             results.append(arr)
-        check(lib.thx_elemwise_call(handle, ins, outs, flags))
-        for k, arr in enumerate(results):
-            output_storage[k][0] = arr
+        rc = lib.thx_elemwise_call(handle, ins, outs, flags)
+        if rc:
+            check(rc)
+        for k in range(nout):
+            output_storage[k][0] = results[k]
 
 
 class HipCAReduce(CAReduce):
@@ -366,10 +396,16 @@ class HipCAReduce(CAReduce):
 
     def perform(self, node, inputs, output_storage):
         flags = call_flags()
-        handle, nin, nout = self._handle(node)
-        nd = max(i.type.ndim for i in node.inputs)
+        cache = node.tag.get("thx")
+        if cache is None:
+            handle, nin, nout = self._handle(node)
+            nd = max(i.type.ndim for i in node.inputs)
+            axis = self.axis if self.axis is not None else tuple(range(nd))
+            mask = (ctypes.c_uint8 * max(nd, 1))(*[1 if d in axis else 0 for d in range(nd)])
+            cache = node.tag["thx"] = (handle, nin, nout, (thx_array * nin)(), (thx_array * nout)(), nd, axis, mask,
+                                       [np.dtype(d) for d in self.out_dtypes])
+        handle, nin, nout, ins, outs, nd, axis, mask, out_dt = cache
         shape = _check_runtime_broadcast(node.inputs, inputs, nd)
-        axis = self.axis if self.axis is not None else tuple(range(nd))
         n_red = 1
         for a in axis:
             n_red *= shape[a]
@@ -377,17 +413,16 @@ class HipCAReduce(CAReduce):
             for op in self.scalar_ops:
                 if codegen.reduce_identity(op, "float32") is None or isinstance(op, (scal.Maximum, scal.Minimum)):
                     raise ValueError("Input of CAReduce{%s} has zero-size on axis %s" % (op, axis))
-        mask = (ctypes.c_uint8 * max(nd, 1))(*[1 if d in axis else 0 for d in range(nd)])
-        ins = (thx_array * nin)()
         for k, v in enumerate(inputs):
             _operand(v, nd, ins[k])
         kept = tuple(shape[d] for d in range(nd) if d not in axis)
-        outs = (thx_array * nout)()
         results = []
-        for k, dt in enumerate(self.out_dtypes):
-            arr = HipArray.empty(kept, dt)
+        for k in range(nout):
+            arr = HipArray._new_contiguous(kept, out_dt[k])
             arr.as_thx(outs[k])
             results.append(arr)
-        check(lib.thx_reduce_call(handle, ins, mask, outs, flags))
+        rc = lib.thx_reduce_call(handle, ins, mask, outs, flags)
+        if rc:
+            check(rc)
         for k, arr in enumerate(results):
             output_storage[k][0] = arr

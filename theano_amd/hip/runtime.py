@@ -214,10 +214,13 @@ def _c_strides(shape, itemsize):
     return tuple(reversed(strides))
 
 
+_CODE_OF = dict((np.dtype(name), scal.dtype_code(name)) for name in scal.all_dtypes)
+
+
 class HipArray(object):
     """A strided view of device memory."""
 
-    __slots__ = ("buffer", "offset", "shape", "strides", "dtype")
+    __slots__ = ("buffer", "offset", "shape", "strides", "dtype", "code")
 
     def __init__(self, buffer, offset, shape, strides, dtype):
         self.buffer = buffer
@@ -225,6 +228,28 @@ class HipArray(object):
         self.shape = tuple(int(s) for s in shape)
         self.strides = tuple(int(s) for s in strides)
         self.dtype = np.dtype(dtype)
+        self.code = _CODE_OF[self.dtype]
+
+    @classmethod
+    def _new_contiguous(cls, shape, dtype):
+        """``empty`` for callers that already hold a tuple of ints and a np.dtype."""
+        self = cls.__new__(cls)
+        n = dtype.itemsize
+        strides = []
+        for s in reversed(shape):
+            strides.append(n)
+            n *= s if s > 1 else 1
+        strides.reverse()
+        total = dtype.itemsize
+        for s in shape:
+            total *= s
+        self.buffer = _Buffer(total)
+        self.offset = 0
+        self.shape = shape
+        self.strides = tuple(strides)
+        self.dtype = dtype
+        self.code = _CODE_OF[dtype]
+        return self
 
     # -- construction
     @classmethod
@@ -241,7 +266,7 @@ class HipArray(object):
     @classmethod
     def from_numpy(cls, a):
         a = np.asarray(a)
-        if str(a.dtype) not in scal.all_dtypes:
+        if a.dtype not in _CODE_OF:
             raise TypeError("dtype %s is not supported on the device" % a.dtype)
         a = np.asarray(a, order="C")
         out = cls.empty(a.shape, a.dtype)
@@ -325,10 +350,16 @@ class HipArray(object):
         a.base = self.buffer.ptr
         a.offset_bytes = self.offset
         a.nd = len(self.shape)
-        a.dtype = scal.dtype_code(str(self.dtype))
-        for i, (s, st) in enumerate(zip(self.shape, self.strides)):
-            a.shape[i] = s
-            a.strides_bytes[i] = st
+        a.dtype = self.code
+        shp, st = a.shape, a.strides_bytes
+        i = 0
+        for s in self.shape:
+            shp[i] = s
+            i += 1
+        i = 0
+        for s in self.strides:
+            st[i] = s
+            i += 1
         return a
 
 
@@ -339,7 +370,7 @@ def host_scalar_thx(value, nd, out=None):
     a.base = value.ctypes.data
     a.offset_bytes = 0
     a.nd = nd
-    a.dtype = scal.dtype_code(str(value.dtype)) | THX_HOST_SCALAR
+    a.dtype = _CODE_OF[value.dtype] | THX_HOST_SCALAR
     for i in range(nd):
         a.shape[i] = 1
         a.strides_bytes[i] = 0

@@ -4,6 +4,10 @@ from .type import (TensorType, TensorVariable, TensorConstant, as_tensor_variabl
                    ivector, imatrix, itensor3, itensor4, lscalar, lvector, lmatrix, ltensor3, ltensor4, hscalar,
                    hvector, hmatrix, htensor3, htensor4, fscalar, fvector, fmatrix, frow, fcol, ftensor3, ftensor4,
                    dscalar, dvector, dmatrix, drow, dcol, dtensor3, dtensor4)
+from . import type as _type
+for _n in dir(_type):  # bscalar ... dtensor4 and friends
+    if _n[0] in "bwilhfd" and _n[1:] in ("scalar", "vector", "matrix", "row", "col", "tensor3", "tensor4"):
+        globals()[_n] = getattr(_type, _n)
 from .elemwise import DimShuffle, Elemwise, CAReduce, CAReduceDtype, Sum, Prod, All, Any
 from .basic import *  # noqa: F401,F403
 from .basic import Max, Min, ShapeFloat, makeKeepDims, cast, round  # noqa: F401
