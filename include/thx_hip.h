@@ -13,7 +13,8 @@
  * Every function is plain C: pointers, sizes and PODs. All functions return
  * THX_OK (0) or an error code; thx_last_error() gives the message of the last
  * failure on the calling thread. One device, one in-order stream, no internal
- * threads. Device results are deterministic: no atomics are used.
+ * threads. Device results are reproducible: data is never accumulated with
+ * atomics (split reductions merge their partial results in a fixed order).
  */
 #ifndef THX_HIP_H
 #define THX_HIP_H
@@ -140,6 +141,30 @@ int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, 
 int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_mask,
                     const thx_array* outs, int flags);
 int thx_reduce_free(thx_reduce* r);
+
+/* ---- Row chains ------------------------------------------------------------ */
+
+typedef struct thx_rowchain thx_rowchain;
+
+/* Operand kinds of a row chain. */
+enum { THX_KIND_FULL = 0, THX_KIND_ROW = 1, THX_KIND_COL = 2, THX_KIND_SCALAR = 3 };
+
+/* Create a fused "elementwise + reductions along the last axis" operation from
+ * generated device source defining a functor named `functor_name` (contract in
+ * kernels/thx_rowchain.h). kinds[i] says how operand i (inputs, then outputs)
+ * relates to the full shape [rows..., C]: FULL = that shape, ROW = one value
+ * per row ([rows..., 1] or [rows...]), COL = one value per column ([1..., C]),
+ * SCALAR = one value (device array or THX_HOST_SCALAR). Outputs are FULL or ROW.
+ * The reference has no such kernel for arbitrary graphs; it covers row softmax
+ * with the dedicated GpuSoftmax kernel (theano/gpuarray/nnet.py) instead. */
+int thx_rowchain_new(const char* functor_src, const char* functor_name, int n_in, int n_out,
+                     const int32_t* dtypes, const int32_t* kinds, thx_rowchain** out);
+/* One launch: each row is read once, kept in registers through every step and
+ * written once. Fails with THX_ERR_UNSUPPORTED - the caller then runs the
+ * unfused nodes - when rows are not unit-stride, leading dimensions do not
+ * collapse to one row stride, or a row exceeds 16384 vector slots. */
+int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* outs, int flags);
+int thx_rowchain_free(thx_rowchain* c);
 
 /* ---- inspection and timing ------------------------------------------------ */
 

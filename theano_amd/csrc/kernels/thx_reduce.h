@@ -12,9 +12,11 @@
 //   static void comb(Acc&, const Acc&);                  // merge two partial results
 //   static Acc shfl_xor(const Acc&, int mask);
 //   template <class O> static void post(const O&, long long index, const Acc&);  // epilogue, casts, stores
-// Results never depend on atomics: long reductions are split into S slices
-// whose partial Acc values go to a scratch array laid out [slice][output] and
-// are merged by red_final in a fixed order.
+// Long reductions are split into S slices whose partial Acc values go to a
+// scratch array laid out [slice][output]; a second, small launch (red_final)
+// merges them in slice order, so results are reproducible run to run. (Merging
+// inside the first launch by the last block to arrive was measured slower on
+// gfx950: the device-scope release each block needs costs more than a launch.)
 #pragma once
 
 namespace thx {
@@ -159,13 +161,12 @@ __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, P:
   } else {
     tot = group_reduce<R, TPR>(acc[0]);
   }
-  if (live && t == 0) {
-    if (p.S == 1) {
-      R::post(p.out, o, tot);
-    } else {
-      ((Acc*)p.partial)[(long long)s * p.n_out + o] = tot;
-    }
+  if (p.S == 1) {
+    if (live && t == 0) R::post(p.out, o, tot);
+    return;
   }
+  Acc* part = (Acc*)p.partial;
+  if (live && t == 0) part[(long long)s * p.n_out + o] = tot;
 }
 
 // ---------------------------------------------------------------------------
@@ -271,6 +272,7 @@ __device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, P:
 #pragma unroll
   for (int k = 0; k < VEC; ++k) lds[ty][k][tx] = acc[k];
   __syncthreads();
+  Acc* part = (Acc*)p.partial;
   for (int c = threadIdx.x; c < TX * VEC; c += P::BLOCK) {
     const int x = c / VEC, k = c % VEC;
     const long long col = (long long)cb * (TX * VEC) + c;
@@ -282,7 +284,7 @@ __device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, P:
       if (p.S == 1) {
         R::post(p.out, o, tot);
       } else {
-        ((Acc*)p.partial)[(long long)s * p.n_out + o] = tot;
+        part[(long long)s * p.n_out + o] = tot;
       }
     }
   }

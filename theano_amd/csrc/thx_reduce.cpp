@@ -205,7 +205,9 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   const int NKD = (int)KD.size(), NR = (int)RD.size();
 
   const int cus = rt().ready ? rt().cus : 256;
-  const int64_t target = (int64_t)cus * env_int("THX_RED_BLOCKS_PER_CU", 8);
+  // blocks wanted when a reduction has to be split to fill the device: few, so that the second pass stays tiny
+  const int bpc = env_int("THX_RED_BLOCKS_PER_CU", 0);
+  const int64_t target_row = (int64_t)cus * (bpc > 0 ? bpc : 2), target_col = (int64_t)cus * (bpc > 0 ? bpc : 1);
 
   bool wide = n_out >= (int64_t(1) << 31) - 65536 || n_red >= (int64_t(1) << 31) - 65536;
   for (int i = 0; i < NIN && !wide; ++i) {
@@ -281,8 +283,8 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     const int rpb = block / tpr;
     const int64_t oblocks = ceil_div(n_out, rpb);
     int64_t chunk = nvec;
-    if (oblocks * 2 <= target && nvec >= (int64_t)tpr * unr * 4) {
-      int64_t want = std::min(ceil_div(target, oblocks), nvec / ((int64_t)tpr * unr * 2));
+    if (oblocks * 2 <= target_row && nvec >= (int64_t)tpr * unr * 4) {
+      int64_t want = std::min(ceil_div(target_row, oblocks), nvec / ((int64_t)tpr * unr * 2));
       if (want > 1) {
         chunk = round_up(ceil_div(nvec, want), (int64_t)tpr * unr);
         S = (int)ceil_div(nvec, chunk);
@@ -376,8 +378,8 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     if (force_unr > 0) unr = force_unr;
     const int64_t blocks0 = A * cblocks;
     int64_t rps = rows;
-    if (blocks0 * 2 <= target && rows >= (int64_t)ty * unr * 2) {
-      int64_t want = std::min(ceil_div(target, blocks0), rows / ((int64_t)ty * unr));
+    if (blocks0 * 2 <= target_col && rows >= (int64_t)ty * unr * 2) {
+      int64_t want = std::min(ceil_div(target_col, blocks0), rows / ((int64_t)ty * unr));
       if (want > 1) {
         rps = round_up(ceil_div(rows, want), (int64_t)ty * unr);
         S = (int)ceil_div(rows, rps);

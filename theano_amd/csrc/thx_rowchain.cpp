@@ -1,0 +1,235 @@
+// Row-chain planner: checks that every operand of an elementwise + row-reduction
+// island can be walked row by row with unit column stride, picks the vector
+// width and the number of threads per row, compiles on first use and launches.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+#include <sstream>
+#include <unordered_map>
+
+#include "thx_internal.h"
+
+struct thx_rowchain {
+  std::string src, name;
+  int n_in = 0, n_out = 0;
+  std::vector<int32_t> dtypes, kinds;
+  std::unordered_map<std::string, thx::Kernel> plans;
+};
+
+namespace thx {
+
+enum { K_FULL = 0, K_ROW = 1, K_COL = 2, K_SCALAR = 3 };
+
+// Stride between consecutive rows when the leading `nlead` dimensions collapse
+// into one row index; false when they do not.
+static bool row_stride(const int64_t* shape, const int64_t* stride, int nlead, int64_t* out) {
+  int64_t st = 0;
+  bool have = false;
+  for (int d = nlead - 1; d >= 0; --d) {
+    if (shape[d] == 1) continue;
+    if (!have) {
+      st = stride[d];
+      have = true;
+      *out = st;
+      st *= shape[d];
+    } else {
+      if (stride[d] != st) return false;
+      st *= shape[d];
+    }
+  }
+  if (!have) *out = 0;
+  return true;
+}
+
+}  // namespace thx
+
+using namespace thx;
+
+extern "C" {
+
+int thx_rowchain_new(const char* functor_src, const char* functor_name, int n_in, int n_out, const int32_t* dtypes,
+                     const int32_t* kinds, thx_rowchain** out) {
+  if (!functor_src || !functor_name || !dtypes || !kinds || !out) return fail(THX_ERR_ARG, "thx_rowchain_new: null argument");
+  if (n_in < 1 || n_out < 1) return fail(THX_ERR_ARG, "thx_rowchain_new: needs inputs and outputs");
+  for (int i = 0; i < n_in + n_out; ++i) {
+    if (!dtype_size(dtypes[i])) return fail(THX_ERR_TYPE, "thx_rowchain_new: unknown dtype code %d", dtypes[i]);
+    if (kinds[i] < K_FULL || kinds[i] > K_SCALAR || (i >= n_in && kinds[i] > K_ROW))
+      return fail(THX_ERR_ARG, "thx_rowchain_new: bad operand kind %d", kinds[i]);
+  }
+  thx_rowchain* c = new thx_rowchain;
+  c->src = functor_src;
+  c->name = functor_name;
+  c->n_in = n_in;
+  c->n_out = n_out;
+  c->dtypes.assign(dtypes, dtypes + n_in + n_out);
+  c->kinds.assign(kinds, kinds + n_in + n_out);
+  *out = c;
+  return THX_OK;
+}
+
+int thx_rowchain_free(thx_rowchain* c) {
+  delete c;
+  return THX_OK;
+}
+
+int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* outs, int flags) {
+  if (!c || !ins || !outs) return fail(THX_ERR_ARG, "thx_rowchain_call: null argument");
+  const bool dry = (flags & THX_DRY_RUN) != 0;
+  if (!dry) {
+    int rc = ensure_init();
+    if (rc) return rc;
+  }
+  const int NIN = c->n_in, NOUT = c->n_out, NOPS = NIN + NOUT;
+  // the full shape comes from the first full operand
+  const thx_array* full = nullptr;
+  for (int i = 0; i < NOPS && !full; ++i)
+    if (c->kinds[i] == K_FULL) full = i < NIN ? &ins[i] : &outs[i - NIN];
+  if (!full) return fail(THX_ERR_ARG, "rowchain: no full-shaped operand");
+  const int nd = full->nd;
+  if (nd < 1 || nd > THX_MAX_ND) return fail(THX_ERR_TYPE, "rowchain: rank %d", nd);
+  int64_t rows = 1;
+  for (int d = 0; d < nd - 1; ++d) rows *= full->shape[d];
+  const int64_t C = full->shape[nd - 1];
+  if (rows == 0 || C == 0) {
+    set_last_plan("rw|empty");
+    return THX_OK;
+  }
+  if (C >= (int64_t(1) << 30)) return fail(THX_ERR_UNSUPPORTED, "rowchain: rows of %lld elements", (long long)C);
+
+  std::vector<char*> ptr(NOPS, nullptr);
+  std::vector<uint64_t> imm(NIN, 0);
+  std::vector<int> is_imm(NIN, 0);
+  std::vector<int64_t> rstride(NOPS, 0);
+  int maxsz = 1;
+  for (int i = 0; i < NOPS; ++i) {
+    const thx_array& a = i < NIN ? ins[i] : outs[i - NIN];
+    const int kind = c->kinds[i];
+    const int dt = a.dtype & ~THX_HOST_SCALAR;
+    if (dt != c->dtypes[i]) return fail(THX_ERR_TYPE, "rowchain: operand %d has dtype code %d, expected %d", i, dt, c->dtypes[i]);
+    const int isz = dtype_size(dt);
+    char* p = (char*)a.base + a.offset_bytes;
+    if (a.dtype & THX_HOST_SCALAR) {
+      if (kind != K_SCALAR || i >= NIN) return fail(THX_ERR_TYPE, "rowchain: operand %d cannot be a host scalar", i);
+      memcpy(&imm[i], p, (size_t)isz);
+      is_imm[i] = 1;
+      continue;
+    }
+    if (((uintptr_t)p) % isz) return fail(THX_ERR_TYPE, "rowchain: operand %d is not aligned to its element size", i);
+    ptr[i] = p;
+    int64_t st[THX_MAX_ND];
+    for (int d = 0; d < a.nd; ++d) {
+      if (a.strides_bytes[d] % isz) return fail(THX_ERR_TYPE, "rowchain: operand %d has a stride that is not a multiple of its element size", i);
+      st[d] = a.strides_bytes[d] / isz;
+    }
+    if (kind == K_FULL) {
+      if (a.nd != nd) return fail(THX_ERR_TYPE, "rowchain: operand %d has rank %d, expected %d", i, a.nd, nd);
+      for (int d = 0; d < nd; ++d)
+        if (a.shape[d] != full->shape[d])
+          return fail(THX_ERR_SHAPE, "Input dimension mis-match. (input[%d].shape[%d] = %lld, expected %lld)", i, d,
+                      (long long)a.shape[d], (long long)full->shape[d]);
+      if (C > 1 && st[nd - 1] != 1) return fail(THX_ERR_UNSUPPORTED, "rowchain: operand %d is not contiguous along its rows", i);
+      if (!row_stride(a.shape, st, nd - 1, &rstride[i]))
+        return fail(THX_ERR_UNSUPPORTED, "rowchain: the leading dimensions of operand %d do not collapse", i);
+      maxsz = std::max(maxsz, isz);
+    } else if (kind == K_ROW) {
+      // rank nd with a trailing extent of 1, or rank nd - 1
+      if (a.nd != nd && a.nd != nd - 1) return fail(THX_ERR_TYPE, "rowchain: per-row operand %d has rank %d", i, a.nd);
+      if (a.nd == nd && a.shape[nd - 1] != 1) return fail(THX_ERR_SHAPE, "rowchain: per-row operand %d has %lld columns", i, (long long)a.shape[nd - 1]);
+      for (int d = 0; d < nd - 1; ++d)
+        if (a.shape[d] != full->shape[d])
+          return fail(THX_ERR_SHAPE, "Input dimension mis-match. (input[%d].shape[%d] = %lld, expected %lld)", i, d,
+                      (long long)a.shape[d], (long long)full->shape[d]);
+      if (!row_stride(a.shape, st, nd - 1, &rstride[i]))
+        return fail(THX_ERR_UNSUPPORTED, "rowchain: the leading dimensions of operand %d do not collapse", i);
+    } else if (kind == K_COL) {
+      if (a.nd != nd || a.shape[nd - 1] != C) return fail(THX_ERR_SHAPE, "rowchain: per-column operand %d has the wrong shape", i);
+      for (int d = 0; d < nd - 1; ++d)
+        if (a.shape[d] != 1) return fail(THX_ERR_SHAPE, "rowchain: per-column operand %d has leading extent %lld", i, (long long)a.shape[d]);
+      if (C > 1 && st[nd - 1] != 1) return fail(THX_ERR_UNSUPPORTED, "rowchain: operand %d is not contiguous", i);
+      rstride[i] = 0;
+      maxsz = std::max(maxsz, isz);
+    } else {
+      for (int d = 0; d < a.nd; ++d)
+        if (a.shape[d] != 1) return fail(THX_ERR_SHAPE, "rowchain: scalar operand %d has extent %lld", i, (long long)a.shape[d]);
+    }
+  }
+
+  int vec = 16 / maxsz;
+  auto vec_ok = [&](int v) {
+    if (v == 1) return true;
+    if (C % v) return false;
+    for (int i = 0; i < NOPS; ++i) {
+      if (c->kinds[i] != K_FULL && c->kinds[i] != K_COL) continue;
+      const int isz = dtype_size(c->dtypes[i]);
+      if (((uintptr_t)ptr[i]) % (size_t)(isz * v)) return false;
+      if (rstride[i] % v) return false;
+    }
+    return true;
+  };
+  while (!vec_ok(vec)) vec /= 2;
+  const int64_t cv = C / vec;
+  int tpr, nch;
+  if (cv <= 8 * 64) {
+    tpr = 64;
+    nch = (int)((cv + 63) / 64);
+  } else if (cv <= 16 * 256) {
+    tpr = 256;
+    nch = (int)((cv + 255) / 256);
+  } else {
+    return fail(THX_ERR_UNSUPPORTED, "rowchain: rows of %lld elements do not fit in registers", (long long)C);
+  }
+  const int force_tpr = getenv("THX_ROW_TPR") ? atoi(getenv("THX_ROW_TPR")) : 0;
+  if (force_tpr == 256 || force_tpr == 64) {
+    tpr = force_tpr;
+    nch = (int)((cv + tpr - 1) / tpr);
+    if (nch > 32) return fail(THX_ERR_UNSUPPORTED, "rowchain: forced threads per row give %d chunks", nch);
+  }
+  bool wide = false;
+  for (int i = 0; i < NOPS; ++i) {
+    int64_t span = (rows - 1) * (rstride[i] < 0 ? -rstride[i] : rstride[i]) + C;
+    if (span >= (int64_t(1) << 31) - 65536) wide = true;
+  }
+  const int block = 256;
+  const int nt = getenv("THX_NT") ? atoi(getenv("THX_NT")) : 0;
+
+  std::ostringstream key;
+  key << "rw|v" << vec << "|n" << nch << "|t" << tpr << (wide ? "|i64" : "|i32") << (nt ? "|nt" : "") << "|i";
+  for (int i = 0; i < NIN; ++i) key << is_imm[i];
+  const std::string plan = key.str();
+  set_last_plan(c->name + "|" + plan);
+  Kernel k;
+  auto it = c->plans.find(plan);
+  if (it != c->plans.end() && (it->second.func || dry)) {
+    k = it->second;
+  } else {
+    std::ostringstream s;
+    s << device_prelude() << c->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
+      << " IT;\n  enum { VEC = " << vec << ", NCH = " << nch << ", TPR = " << tpr << ", BLOCK = " << block
+      << ", NT = " << nt << " };\n  static constexpr int imm(int i) {\n    constexpr int m[] = {";
+    for (int i = 0; i < NIN; ++i) s << is_imm[i] << (i + 1 < NIN ? ", " : "");
+    s << "};\n    return m[i];\n  }\n};\n"
+      << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::RowChainParams<" << c->name
+      << "::NIN, " << c->name << "::NOUT, ThxPlan::IT> p) {\n  thx::rowchain_body<" << c->name << ", ThxPlan>(p);\n}\n";
+    int rc = get_kernel(s.str(), "thx_entry", &k);
+    if (rc) return rc;
+    c->plans[plan] = k;
+  }
+  if (dry) return THX_OK;
+
+  ParamPack pk;
+  for (int i = 0; i < NIN; ++i) pk.put<char*>(ptr[i]);
+  for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(imm[i]);
+  for (int i = 0; i < NOUT; ++i) pk.put<char*>(ptr[NIN + i]);
+  pk.put<int64_t>(rows);
+  pk.put<int32_t>((int32_t)C);
+  pk.put<int32_t>((int32_t)cv);
+  for (int i = 0; i < NIN; ++i) pk.put_index(wide, rstride[i]);
+  for (int i = 0; i < NOUT; ++i) pk.put_index(wide, rstride[NIN + i]);
+  pk.align(8);
+  const int rpb = block / tpr;
+  const int64_t grid = (rows + rpb - 1) / rpb;
+  if (grid > 0x7fffffffLL) return fail(THX_ERR_UNSUPPORTED, "rowchain: %lld blocks exceed the grid limit", (long long)grid);
+  return launch(k, c->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
+}
+
+}  // extern "C"

@@ -4,3 +4,4 @@ from .runtime import (HipArray, HipRuntimeError, cache_stats, device_info, dry_r
 from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipToHost, HostToHip, as_hip_variable,  # noqa: F401
                   hip_from_host, host_from_hip)
 from . import opt  # noqa: F401
+from .rowchain import HipRowChain  # noqa: F401

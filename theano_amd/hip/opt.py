@@ -337,7 +337,7 @@ def _merge_two(a, b):
 
 
 # --------------------------------------------------------------------------
-def optimize(fgraph, fuse=True):
+def optimize(fgraph, fuse=True, rowchain=True):
     """Full pipeline: clean up, lift, fuse."""
     from ..tensor.opt import canonicalize
     canonicalize(fgraph)
@@ -345,6 +345,9 @@ def optimize(fgraph, fuse=True):
     gof.merge_identical(fgraph)
     if fuse:
         fuse_elemwise(fgraph)
+        if rowchain:
+            from .rowchain import fuse_row_chains
+            fuse_row_chains(fgraph)
         fuse_reduce_prologue(fgraph)
         merge_sibling_reductions(fgraph)
         gof.merge_identical(fgraph)

@@ -1,0 +1,398 @@
+"""Row chains: islands of elementwise nodes and last-axis reductions executed by
+one kernel that keeps each row on chip.
+
+The reference never fuses across a reduction (``theano/tensor/opt.py:7071-7313``
+only merges Elemwise nodes); for row softmax it substitutes a hand-written
+``Softmax`` op instead (``theano/tensor/nnet/nnet.py:411-600, 888-925``).  Here the
+same effect is obtained for any such island: the sub-graph is turned into a
+straight-line row program (load, elementwise steps, reductions, store), code is
+generated for it and one launch replaces the whole island.  Results follow the
+per-node semantics: elementwise steps use each scalar op's ``c_code``, every
+reduction accumulates in the accumulator dtype of its node and is cast to the
+node's output dtype before anything consumes it.
+"""
+import ctypes
+import hashlib
+
+import numpy as np
+
+from .. import gof
+from .. import scalar as scal
+from ..gof import Apply, Op
+from ..scalar import Scalar, compute_ctype, storage_ctype
+from ..tensor.type import TensorType
+from . import codegen
+from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, _is_host_scalar)
+from .runtime import HipArray, call_flags, check, host_scalar_thx, lib, thx_array
+
+FULL, ROW, COL, SCALAR = 0, 1, 2, 3
+THX_ERR_UNSUPPORTED = 6
+
+
+def _klass(var, nd):
+    """Operand class of a rank-``nd`` variable by its broadcast pattern."""
+    b = var.type.broadcastable
+    if len(b) != nd:
+        return None
+    if not any(b):
+        return FULL
+    if all(b):
+        return SCALAR
+    if b[-1] and not any(b[:-1]):
+        return ROW
+    if not b[-1] and all(b[:-1]):
+        return COL
+    return None
+
+
+class RowProgram(object):
+    """Straight-line program over per-element values and per-row scalars."""
+
+    def __init__(self):
+        self.in_kinds, self.in_dtypes = [], []
+        self.steps = []        # ("ew", scalar_op, arg ids, out ids) | ("red", scalar_op, acc, out dtype, arg, out)
+        self.var = {}          # id -> (per_element, dtype)
+        self.outputs = []      # (var id, kind, dtype)
+        self._next = 0
+
+    def new_var(self, per_element, dtype):
+        i = self._next
+        self._next += 1
+        self.var[i] = (per_element, dtype)
+        return i
+
+    def add_input(self, kind, dtype):
+        self.in_kinds.append(kind)
+        self.in_dtypes.append(dtype)
+        return self.new_var(kind in (FULL, COL), dtype)
+
+    # -- code generation
+    def source(self):
+        lines, ops = [], []
+        nm = lambda i: ("v%d" if self.var[i][0] else "s%d") % i
+        elem = lambda i: ("v%d[ch][k]" if self.var[i][0] else "s%d") % i
+        loaders = {FULL: "load_full", ROW: "load_row", COL: "load_col", SCALAR: "load_scalar"}
+        for k, (kind, dt) in enumerate(zip(self.in_kinds, self.in_dtypes)):
+            ct = compute_ctype(dt)
+            decl = "%s v%d[X::NCH][X::VEC];" % (ct, k) if kind in (FULL, COL) else "%s s%d;" % (ct, k)
+            lines.append("%s x.template %s<%d, %s, %s>(%s);" % (decl, loaders[kind], k, storage_ctype(dt), ct, nm(k)))
+        for step in self.steps:
+            if step[0] == "ew":
+                _, op, args, outs = step
+                node = op.make_node(*[Scalar(self.var[a][1])() for a in args])
+                per_elem = any(self.var[o][0] for o in outs)
+                for o in outs:
+                    ct = compute_ctype(self.var[o][1])
+                    lines.append("%s v%d[X::NCH][X::VEC];" % (ct, o) if self.var[o][0] else "%s s%d;" % (ct, o))
+                code = op.c_code(node, [elem(a) for a in args], [elem(o) for o in outs])
+                if per_elem:
+                    lines.append("_Pragma(\"unroll\") for (int ch = 0; ch < X::NCH; ++ch) {\n"
+                                 "_Pragma(\"unroll\") for (int k = 0; k < X::VEC; ++k) {\n%s\n}}" % code)
+                else:
+                    lines.append("{\n%s\n}" % code)
+            else:
+                _, op, acc_dt, out_dt, arg, out = step
+                act, oct_ = compute_ctype(acc_dt), compute_ctype(out_dt)
+                ident = codegen.reduce_identity(op, acc_dt)
+                if ident is None:
+                    raise NotImplementedError("reduction with %s has no identity element" % op)
+                cnode = Apply(op, [Scalar(acc_dt)(), Scalar(acc_dt)()], [Scalar(acc_dt)()])
+                ops.append("  struct Op%d { THX_DEV static void comb(%s& a, const %s& b) { %s } };" % (
+                    out, act, act, op.c_code(cnode, ["a", "b"], ["a"])))
+                lines.append("%s a%d = %s;" % (act, out, ident))
+                lines.append("_Pragma(\"unroll\") for (int ch = 0; ch < X::NCH; ++ch) { if (x.valid(ch)) {\n"
+                             "_Pragma(\"unroll\") for (int k = 0; k < X::VEC; ++k) { %s t = (%s)v%d[ch][k]; "
+                             "Op%d::comb(a%d, t); } } }" % (act, act, arg, out, out))
+                lines.append("a%d = x.template allreduce<Op%d, %s>(a%d);" % (out, out, act, out))
+                val = "a%d" % out
+                if out_dt == "bool":
+                    val = "(%s ? 1 : 0)" % val
+                # the result takes the storage precision of the node's output before anything reads it
+                lines.append("%s s%d = (%s)(%s)%s;" % (oct_, out, oct_, storage_ctype(out_dt), val))
+        for k, (vid, kind, dt) in enumerate(self.outputs):
+            ct = compute_ctype(self.var[vid][1])
+            st = "store_full" if kind == FULL else "store_row"
+            lines.append("x.template %s<%d, %s, %s>(%s);" % (st, k, storage_ctype(dt), ct, nm(vid)))
+        body = "\n".join("    " + l for l in "\n".join(lines).splitlines())
+        text = "  enum { NIN = %d, NOUT = %d };\n%s\n  template <class X> THX_DEV static void row(X& x) {\n%s\n  }" % (
+            len(self.in_kinds), len(self.outputs), "\n".join(ops), body)
+        name = "C" + hashlib.sha1((text + repr(self.in_kinds)).encode()).hexdigest()[:16]
+        return "struct %s {\n%s\n};\n" % (name, text), name
+
+
+_handles = {}
+
+
+class HipRowChain(Op):
+    """One launch for a whole elementwise + row-reduction island."""
+
+    __props__ = ("signature",)
+
+    def __init__(self, program, out_types, fallback):
+        self.program = program
+        self.src, self.name = program.source()
+        self.signature = (self.name, tuple(program.in_kinds), tuple(str(t) for t in out_types))
+        self.out_types = list(out_types)
+        self.fallback = fallback   # (inner input variables, inner output variables) of the original island
+
+    def __str__(self):
+        n_red = sum(1 for s in self.program.steps if s[0] == "red")
+        return "HipRowChain{%d steps, %d reductions}" % (len(self.program.steps), n_red)
+
+    def make_node(self, *inputs):
+        return Apply(self, list(inputs), [t() for t in self.out_types])
+
+    def infer_shape(self, node, shapes):
+        full = None
+        for s, k in zip(shapes, self.program.in_kinds):
+            if k == FULL:
+                full = tuple(s)
+        out = []
+        for (vid, kind, dt), t in zip(self.program.outputs, self.out_types):
+            if kind == FULL:
+                out.append(full)
+            elif t.ndim == len(full):
+                out.append(full[:-1] + (1,))
+            else:
+                out.append(full[:-1])
+        return out
+
+    def _handle(self):
+        h = _handles.get(self.signature)
+        if h is None:
+            p = self.program
+            dts = list(p.in_dtypes) + [dt for _, _, dt in p.outputs]
+            kinds = list(p.in_kinds) + [k for _, k, _ in p.outputs]
+            codes = (ctypes.c_int32 * len(dts))(*[scal.dtype_code(d) for d in dts])
+            kk = (ctypes.c_int32 * len(kinds))(*kinds)
+            handle = ctypes.c_void_p()
+            check(lib.thx_rowchain_new(self.src.encode(), self.name.encode(), len(p.in_kinds), len(p.outputs), codes, kk,
+                                       ctypes.byref(handle)))
+            h = _handles[self.signature] = handle
+        return h
+
+    def perform(self, node, inputs, output_storage):
+        p = self.program
+        cache = node.tag.get("thx")
+        if cache is None:
+            cache = node.tag["thx"] = (self._handle(), (thx_array * len(inputs))(), (thx_array * len(p.outputs))(),
+                                       [np.dtype(dt) for _, _, dt in p.outputs])
+        handle, ins, outs, out_dt = cache
+        full = None
+        for v, k in zip(inputs, p.in_kinds):
+            if k == FULL:
+                full = v.shape
+                break
+        nd = len(full)
+        for k, v in enumerate(inputs):
+            if type(v) is HipArray:
+                v.as_thx(ins[k])
+            else:
+                host_scalar_thx(v, nd, ins[k])
+        results = []
+        for k, ((vid, kind, dt), t) in enumerate(zip(p.outputs, self.out_types)):
+            shape = full if kind == FULL else (full[:-1] + (1,) if t.ndim == nd else full[:-1])
+            arr = HipArray._new_contiguous(tuple(shape), out_dt[k])
+            arr.as_thx(outs[k])
+            results.append(arr)
+        rc = lib.thx_rowchain_call(handle, ins, outs, call_flags())
+        if rc == THX_ERR_UNSUPPORTED:
+            results = self._run_fallback(inputs)
+        elif rc:
+            check(rc)
+        for k, arr in enumerate(results):
+            output_storage[k][0] = arr
+
+    def _run_fallback(self, inputs):
+        """Shapes or strides the one-kernel form does not take (very long rows,
+        non-contiguous rows): run the island node by node on the device."""
+        inner_in, inner_out = self.fallback
+        storage = dict((id(v), [val]) for v, val in zip(inner_in, inputs))
+        for n in gof.io_toposort(inner_in, inner_out):
+            args = []
+            for i in n.inputs:
+                cell = storage.get(id(i))
+                if cell is None:
+                    cell = storage[id(i)] = [np.asarray(i.data)]
+                args.append(cell[0])
+            cells = [[None] for _ in n.outputs]
+            n.op.perform(n, args, cells)
+            for o, c in zip(n.outputs, cells):
+                storage[id(o)] = c
+        return [storage[id(o)][0] for o in inner_out]
+
+
+# --------------------------------------------------------------------------
+def _eligible(node, nd):
+    op = node.op
+    if isinstance(op, HipElemwise):
+        if len(node.outputs) != 1 or op.inplace_pattern:
+            return False
+        if _klass(node.outputs[0], nd) not in (FULL, ROW):
+            return False
+        for i in node.inputs:
+            if isinstance(i.type, HipArrayType):
+                if _klass(i, nd) is None:
+                    return False
+            elif not _is_host_scalar(i):
+                return False
+        return True
+    if isinstance(op, HipCAReduce):
+        return (len(op.scalar_ops) == 1 and op.pre_scalar_op is None and op.post_scalar_op is None and
+                len(node.inputs) == 1 and node.inputs[0].type.ndim == nd and op.axis == (nd - 1,) and
+                _klass(node.inputs[0], nd) == FULL and op.acc_dtypes[0] != "float16")
+    if isinstance(op, HipDimShuffle):
+        x = node.inputs[0]
+        return (x.type.ndim == nd - 1 and not any(x.type.broadcastable) and
+                op.new_order == tuple(range(nd - 1)) + ("x",) and x.owner is not None and
+                isinstance(x.owner.op, HipCAReduce))
+    return False
+
+
+def fuse_row_chains(fgraph):
+    """Replace every island that contains a last-axis reduction by one
+    HipRowChain node."""
+    count = 0
+    changed = True
+    while changed:
+        changed = False
+        for seed in fgraph.toposort():
+            if not isinstance(seed.op, HipCAReduce) or seed not in fgraph.apply_nodes:
+                continue
+            nd = seed.inputs[0].type.ndim
+            if nd < 1 or not _eligible(seed, nd):
+                continue
+            island = _grow(fgraph, seed, nd)
+            if island is None:
+                continue
+            if _replace(fgraph, island, nd):
+                count += 1
+                changed = True
+                break
+    return count
+
+
+def _grow(fgraph, seed, nd):
+    island = {seed}
+    frontier = [seed]
+    while frontier:
+        n = frontier.pop()
+        neigh = [i.owner for i in n.inputs if i.owner is not None]
+        for o in n.outputs:
+            neigh.extend(c for c, _ in fgraph.clients.get(o, []) if c != "output")
+        for m in neigh:
+            if m in island or m not in fgraph.apply_nodes or not _eligible(m, nd):
+                continue
+            if isinstance(m.op, HipDimShuffle) and m.inputs[0].owner not in island:
+                continue
+            island.add(m)
+            frontier.append(m)
+    # a DimShuffle only belongs with its reduction; drop strays whose producer never joined
+    for m in list(island):
+        if isinstance(m.op, HipDimShuffle) and m.inputs[0].owner not in island:
+            island.discard(m)
+    n_red = sum(1 for m in island if isinstance(m.op, HipCAReduce))
+    n_ew = sum(1 for m in island if isinstance(m.op, HipElemwise))
+    if n_red == 0 or n_red + n_ew < 2:
+        return None
+    # the island must not feed itself through outside nodes
+    produced = set(id(o) for m in island for o in m.outputs)
+    ext_inputs = [i for m in island for i in m.inputs if id(i) not in produced]
+    stack, seen = [i for i in ext_inputs], set()
+    while stack:
+        v = stack.pop()
+        if id(v) in seen or v.owner is None:
+            continue
+        seen.add(id(v))
+        if v.owner in island:
+            return None
+        stack.extend(v.owner.inputs)
+    return island
+
+
+def _replace(fgraph, island, nd):
+    order = [n for n in fgraph.toposort() if n in island]
+    produced = set(id(o) for m in island for o in m.outputs)
+    prog = RowProgram()
+    ext_inputs, ids = [], {}
+
+    def var_id(v):
+        if id(v) in ids:
+            return ids[id(v)]
+        # an external operand
+        if isinstance(v.type, HipArrayType):
+            k = _klass(v, nd)
+        else:
+            k = SCALAR
+        if k is None:
+            raise ValueError("unsupported operand")
+        ids[id(v)] = prog.add_input(k, v.type.dtype)
+        ext_inputs.append(v)
+        return ids[id(v)]
+
+    # inputs first so that their ids are 0 .. n_in - 1
+    for n in order:
+        for i in n.inputs:
+            if id(i) not in produced and not isinstance(i, gof.Constant):
+                try:
+                    var_id(i)
+                except ValueError:
+                    return False
+    if not any(k == FULL for k in prog.in_kinds):
+        return False
+    from .opt import _scalar_constant
+    for n in order:
+        op = n.op
+        if isinstance(op, HipElemwise):
+            s_in, args = [], []
+            s_args = []
+            for i in n.inputs:
+                c = _scalar_constant(i) if id(i) not in produced else None
+                if c is not None:
+                    s_args.append(c)
+                    continue
+                if isinstance(i, gof.Constant) and id(i) not in ids:
+                    return False
+                s = Scalar(i.type.dtype)()
+                s_in.append(s)
+                s_args.append(s)
+                args.append(var_id(i))
+            sop = scal.Composite(s_in, [op.scalar_op(*s_args)]) if len(s_in) != len(n.inputs) else op.scalar_op
+            per_elem = any(prog.var[a][0] for a in args)
+            if per_elem != (_klass(n.outputs[0], nd) == FULL):
+                return False
+            out = prog.new_var(per_elem, n.outputs[0].type.dtype)
+            ids[id(n.outputs[0])] = out
+            prog.steps.append(("ew", sop, args, [out]))
+        elif isinstance(op, HipCAReduce):
+            arg = var_id(n.inputs[0])
+            out = prog.new_var(False, op.out_dtypes[0])
+            ids[id(n.outputs[0])] = out
+            prog.steps.append(("red", op.scalar_ops[0], op.acc_dtypes[0], op.out_dtypes[0], arg, out))
+        else:  # keepdims DimShuffle: same per-row value
+            ids[id(n.outputs[0])] = ids[id(n.inputs[0])]
+    # outputs: island variables used outside
+    outs = []
+    for n in order:
+        for o in n.outputs:
+            users = fgraph.clients.get(o, [])
+            if any(c == "output" or c not in island for c, _ in users):
+                outs.append(o)
+    if not outs:
+        return False
+    out_types = []
+    for o in outs:
+        kind = FULL if (o.type.ndim == nd and _klass(o, nd) == FULL) else ROW
+        prog.outputs.append((ids[id(o)], kind, o.type.dtype))
+        out_types.append(o.type)
+    if len(ext_inputs) + len(outs) > 48:
+        return False
+    # fallback: a private copy of the island
+    memo = dict((v, v.type()) for v in ext_inputs)
+    inner_in = [memo[v] for v in ext_inputs]
+    memo = gof.clone_get_equiv(ext_inputs, outs, copy_inputs=False, memo=memo)
+    inner_out = [memo[o] for o in outs]
+    new_node = HipRowChain(prog, out_types, (inner_in, inner_out)).make_node(*ext_inputs)
+    for o, no in zip(outs, new_node.outputs):
+        fgraph.replace(o, no)
+    return True
