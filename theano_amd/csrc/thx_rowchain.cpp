@@ -90,10 +90,11 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
   int64_t rows = 1;
   for (int d = 0; d < nd - 1; ++d) rows *= full->shape[d];
   const int64_t C = full->shape[nd - 1];
-  if (rows == 0 || C == 0) {
+  if (rows == 0) {
     set_last_plan("rw|empty");
     return THX_OK;
   }
+  if (C == 0) return fail(THX_ERR_UNSUPPORTED, "rowchain: empty rows are left to the unfused kernels (identity results)");
   if (C >= (int64_t(1) << 30)) return fail(THX_ERR_UNSUPPORTED, "rowchain: rows of %lld elements", (long long)C);
 
   std::vector<char*> ptr(NOPS, nullptr);

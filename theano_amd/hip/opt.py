@@ -123,11 +123,56 @@ def _scalar_constant(var):
     return None
 
 
+_CHEAP_OPS = (scal.Cast, scal.Add, scal.Sub, scal.Mul, scal.Neg, scal.Sqr, scal.Abs, scal.Sgn, scal.Identity,
+              scal.Second, scal.LogicalComparison, scal.Switch, scal.BinaryBitOp, scal.Invert, scal.Maximum,
+              scal.Minimum, scal.Clip, scal.IsNan, scal.IsInf)
+
+
+def _cheap(scalar_op):
+    """True when recomputing the op per consumer costs a few ALU instructions
+    (no division, no transcendental function)."""
+    if isinstance(scalar_op, scal.Composite):
+        return all(isinstance(n.op, _CHEAP_OPS) for n in gof.io_toposort(scalar_op.inputs, scalar_op.outputs))
+    return isinstance(scalar_op, _CHEAP_OPS)
+
+
+def _absorbs(client, var):
+    """Can this consumer take the producer of ``var`` into its own kernel?"""
+    if client == "output":
+        return False
+    op = client.op
+    if isinstance(op, HipElemwise):
+        return (len(client.outputs) == 1 and not op.inplace_pattern and
+                tuple(client.outputs[0].type.broadcastable) == tuple(var.type.broadcastable))
+    if isinstance(op, HipCAReduce):
+        return op.post_scalar_op is None and all(
+            i.type.ndim == var.type.ndim for i in client.inputs if isinstance(i.type, HipArrayType))
+    return False
+
+
+def _duplicable(fgraph, var):
+    """A cheap elementwise result used by several kernels is recomputed inside
+    each of them when that moves fewer bytes than writing it once and reading
+    it back: inputs x consumers <= inputs + output x (1 + consumers)."""
+    node = var.owner
+    clients = fgraph.clients.get(var, [])
+    if len(clients) < 2 or len(clients) > 8 or not _cheap(node.op.scalar_op):
+        return False
+    if not all(_absorbs(c, var) for c, _ in clients):
+        return False
+    out_b = var.type.broadcastable
+    in_bytes = sum(np.dtype(i.type.dtype).itemsize for i in node.inputs
+                   if isinstance(i.type, HipArrayType) and tuple(i.type.broadcastable) == tuple(out_b))
+    out_bytes = np.dtype(var.type.dtype).itemsize
+    n = len(set(id(c) for c, _ in clients))
+    return in_bytes * n <= in_bytes + out_bytes * (1 + n)
+
+
 def _fusable(fgraph, var, out_bcast):
     node = var.owner
     return (node is not None and isinstance(node.op, HipElemwise) and len(node.outputs) == 1 and
-            not node.op.inplace_pattern and fgraph.n_clients(var) == 1 and
-            tuple(var.type.broadcastable) == tuple(out_bcast))
+            not node.op.inplace_pattern and tuple(var.type.broadcastable) == tuple(out_bcast) and
+            (fgraph.n_clients(var) == 1 or _duplicable(fgraph, var)))
 
 
 def _fuse_node(fgraph, node):
@@ -224,29 +269,64 @@ def _as_composite_inputs(node):
 
 def fuse_reduce_prologue(fgraph):
     """``reduce(f(a, b, ...))`` becomes one reduction whose prologue is f, when
-    nothing else uses f's result."""
+    nothing else needs f's result (or f is cheap enough to recompute)."""
     count = 0
-    for node in fgraph.toposort():
-        op = node.op
-        if not isinstance(op, HipCAReduce) or op.pre_scalar_op is not None or len(op.scalar_ops) != 1:
-            continue
-        x = node.inputs[0]
-        p = x.owner
-        if (p is None or not isinstance(p.op, HipElemwise) or len(p.outputs) != 1 or p.op.inplace_pattern or
-                fgraph.n_clients(x) != 1):
-            continue
-        inputs, s_inputs, args = _as_composite_inputs(p)
-        if not inputs or len(inputs) > config.max_fused_inputs:
-            continue
-        # every device input must carry the full rank of the reduced tensor
-        if any(isinstance(i.type, HipArrayType) and i.type.ndim != x.type.ndim for i in inputs):
-            continue
-        pre = scal.Composite(s_inputs, [p.op.scalar_op(*args)])
-        new = HipCAReduce(op.scalar_ops, op.axis, op.acc_dtypes, op.out_dtypes, pre, op.post_scalar_op)(*inputs)
-        if new.type != node.outputs[0].type:
-            continue
-        fgraph.replace(node.outputs[0], new)
-        count += 1
+    changed = True
+    while changed:
+        changed = False
+        for node in fgraph.toposort():
+            op = node.op
+            if not isinstance(op, HipCAReduce) or op.post_scalar_op is not None or node not in fgraph.apply_nodes:
+                continue
+            nd = max(i.type.ndim for i in node.inputs)
+            target = None
+            for x in node.inputs:
+                p = x.owner
+                if (p is None or not isinstance(p.op, HipElemwise) or len(p.outputs) != 1 or p.op.inplace_pattern or
+                        x.type.ndim != nd):
+                    continue
+                if fgraph.n_clients(x) != 1 and not _duplicable(fgraph, x):
+                    continue
+                if any(isinstance(i.type, HipArrayType) and i.type.ndim != nd for i in p.inputs):
+                    continue
+                target = x
+                break
+            if target is None:
+                continue
+            # new operand list: the node's inputs with `target` replaced by its producer's inputs
+            inputs, s_inputs = [], []
+
+            def scalar_for(v):
+                for t, sv in zip(inputs, s_inputs):
+                    if t is v:
+                        return sv
+                sv = scal.Scalar(v.type.dtype)()
+                inputs.append(v)
+                s_inputs.append(sv)
+                return sv
+
+            p = target.owner
+            p_args = []
+            for v in p.inputs:
+                c = _scalar_constant(v)
+                p_args.append(c if c is not None else scalar_for(v))
+            p_out = p.op.scalar_op(*p_args)
+            outer_args = [p_out if v is target else scalar_for(v) for v in node.inputs]
+            if len(inputs) > config.max_fused_inputs or not inputs:
+                continue
+            if op.pre_scalar_op is None:
+                pre_outs = [outer_args[0]]
+            else:
+                pre_outs = op.pre_scalar_op(*outer_args, return_list=True)
+            pre = scal.Composite(s_inputs, pre_outs)
+            new_node = HipCAReduce(op.scalar_ops, op.axis, op.acc_dtypes, op.out_dtypes, pre, None).make_node(*inputs)
+            if [o.type for o in new_node.outputs] != [o.type for o in node.outputs]:
+                continue
+            for o, no in zip(node.outputs, new_node.outputs):
+                fgraph.replace(o, no)
+            count += 1
+            changed = True
+            break
     return count
 
 
@@ -348,7 +428,9 @@ def optimize(fgraph, fuse=True, rowchain=True):
         if rowchain:
             from .rowchain import fuse_row_chains
             fuse_row_chains(fgraph)
+        merge_sibling_reductions(fgraph)
         fuse_reduce_prologue(fgraph)
+        gof.merge_identical(fgraph)
         merge_sibling_reductions(fgraph)
         gof.merge_identical(fgraph)
     return fgraph

@@ -295,6 +295,12 @@ def _grow(fgraph, seed, nd):
     n_ew = sum(1 for m in island if isinstance(m.op, HipElemwise))
     if n_red == 0 or n_red + n_ew < 2:
         return None
+    # worth one kernel only if something inside consumes a reduction result: a lone reduction with
+    # elementwise producers is served (for any row length) by the prologue-fused reduction kernels
+    if not any(isinstance(m.op, HipElemwise) and any(
+            i.owner in island and isinstance(i.owner.op, (HipCAReduce, HipDimShuffle)) for i in m.inputs)
+            for m in island):
+        return None
     # the island must not feed itself through outside nodes
     produced = set(id(o) for m in island for o in m.outputs)
     ext_inputs = [i for m in island for i in m.inputs if id(i) not in produced]

@@ -87,6 +87,16 @@ def local_useless_elemwise(fgraph, node):
             new = rest[0] if len(rest) == 1 else node.op(*rest)
             if new.type == out.type:
                 return [new]
+    if isinstance(sop, scal.Pow):
+        # x ** 2 -> sqr(x), x ** 1 -> x, x ** 0.5 -> sqrt(x), x ** -1 -> inv(x)
+        # (local_pow_specialize, theano/tensor/opt.py:5918-5973)
+        x, y = node.inputs
+        if isinstance(y, TensorConstant) and all(y.type.broadcastable) and x.type.dtype == out.type.dtype:
+            val = float(np.asarray(y.data).reshape(()))
+            new = {2.0: T.sqr, 0.5: T.sqrt, -1.0: T.inv}.get(val)
+            res = x if val == 1.0 else (new(x) if new is not None else None)
+            if res is not None and res.type == out.type:
+                return [res]
     if isinstance(sop, scal.Second):
         x, y = node.inputs
         if y.type == out.type:
@@ -149,7 +159,35 @@ def local_useless_reduce(fgraph, node):
     return False
 
 
-CANONICALIZE = [local_dimshuffle_fold, local_useless_elemwise, local_fill_sink, local_useless_reduce,
+@local_optimizer([T.ShapeFloat])
+def local_shape_lift(fgraph, node):
+    """The extent of an elementwise / DimShuffle / reduction result is the extent
+    of one of its inputs: ask the input, so that shape queries never keep an
+    intermediate result alive (the role of ShapeFeature, theano/tensor/opt.py:970-1500)."""
+    (x,) = node.inputs
+    p = x.owner
+    i = node.op.i
+    if p is None:
+        return False
+    if isinstance(p.op, Elemwise):
+        for v in p.inputs:
+            if v.type.ndim == x.type.ndim and not v.type.broadcastable[i]:
+                return [T.ShapeFloat(i, node.op.dtype)(v)]
+        return False
+    if isinstance(p.op, DimShuffle):
+        src = p.op.new_order[i]
+        if src == "x":
+            return [constant(1, dtype=node.op.dtype)]
+        return [T.ShapeFloat(src, node.op.dtype)(p.inputs[0])]
+    if isinstance(p.op, CAReduce):
+        nd = p.inputs[0].type.ndim
+        axis = tuple(range(nd)) if p.op.axis is None else p.op.axis
+        kept = [d for d in range(nd) if d not in axis]
+        return [T.ShapeFloat(kept[i], node.op.dtype)(p.inputs[0])]
+    return False
+
+
+CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_useless_elemwise, local_fill_sink, local_useless_reduce,
                 local_dimshuffle_lift]
 
 
