@@ -125,15 +125,18 @@ typedef struct thx_reduce thx_reduce;
 
 /* Create a (multi-)reduction from generated device source defining a functor
  * named `functor_name` (contract in kernels/thx_reduce.h): n_in inputs feed a
- * fused prologue, n_out results of identical shape leave a fused epilogue.
- * acc_bytes = sizeof of the functor's accumulator struct.
+ * fused prologue, n_out results of identical shape leave a fused epilogue that
+ * may also read n_extra host scalars (e.g. the divisor of a mean). dtypes lists
+ * inputs, outputs, then those scalars. acc_bytes = sizeof of the functor's
+ * accumulator struct.
  * Replaces the kernel generation of GpuCAReduceCuda
  * (theano/gpuarray/elemwise.py:1756-2420). */
-int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, int n_out,
+int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, int n_out, int n_extra,
                    const int32_t* dtypes, int acc_bytes, thx_reduce** out);
 
-/* Reduce the dimensions d with reduce_mask[d] != 0. `ins` all have rank nd and
- * broadcast against each other like Elemwise inputs; `outs` are C-contiguous
+/* Reduce the dimensions d with reduce_mask[d] != 0. `ins` holds the n_in reduced
+ * inputs, which all have rank nd and broadcast against each other like Elemwise
+ * inputs, followed by the n_extra THX_HOST_SCALAR operands of the epilogue; `outs` are C-contiguous
  * arrays of the kept dimensions, in order. A zero-length reduce domain yields
  * the identity (the caller rejects it for max/min, as
  * theano/tensor/elemwise.py:1489-1506 does). Asynchronous.

@@ -145,8 +145,9 @@ __device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename 
 // operand is accessed along the innermost dimension. Rows of a tile are padded
 // by one element so that the transposed reads hit distinct banks.
 //
-// Extra plan members: enum { TILE, NTR (staged inputs), ESZ (largest staged
-// element) }; static constexpr int slot(int operand): LDS slot or -1.
+// Extra plan members: enum { TILE, TV (elements per access), NTR (staged
+// inputs), ESZ (largest staged element) }; static constexpr int slot(int
+// operand): LDS slot or -1.
 template <int NOPS, int ND, class IT>
 struct EwTrParams {
   char* ptr[NOPS];
@@ -165,12 +166,15 @@ struct TrStageAcc {  // global -> LDS for the staged inputs, nothing for the oth
   char* const* ptr;
   unsigned char* lds;
   IT off[NOPS];
-  int cell;
+  int cell;  // LDS index of the first element: row * (TILE + 1) + position along T
   template <int I, class T, int N>
   THX_DEV void ld(Vec<T, N>&) const {
     if (P::slot(I) >= 0) {
       T* tile = (T*)(lds + P::slot(I) * (P::TILE * (P::TILE + 1) * P::ESZ));
-      tile[cell] = *((const T*)ptr[I] + off[I]);
+      Vec<T, N> r;
+      load_vec<T, N, P::NT != 0>(r, (const T*)ptr[I] + off[I]);
+#pragma unroll
+      for (int k = 0; k < N; ++k) tile[cell + k] = r.v[k];
     }
   }
 };
@@ -182,28 +186,42 @@ struct TrAcc {  // LDS (transposed) or global -> registers, registers -> global
   const unsigned long long* imm;
   const unsigned char* lds;
   IT off[NOPS];
-  int cell;
+  int cell;  // LDS index of the first element: position along the inner dimension * (TILE + 1) + row along T
   template <int I, class T, int N>
   THX_DEV void ld(Vec<T, N>& r) const {
     if (P::slot(I) >= 0) {
       const T* tile = (const T*)(lds + P::slot(I) * (P::TILE * (P::TILE + 1) * P::ESZ));
-      r.v[0] = tile[cell];
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = tile[cell + k * (P::TILE + 1)];
     } else if (P::mode(I) == M_IMM) {
-      r.v[0] = *(const T*)&imm[I];
+      const T s = *(const T*)&imm[I];
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = s;
+    } else if (P::mode(I) == M_BCAST) {
+      const T s = *((const T*)ptr[I] + off[I]);
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = s;
     } else {
-      r.v[0] = *((const T*)ptr[I] + off[I]);
+      load_vec<T, N, P::NT != 0>(r, (const T*)ptr[I] + off[I]);
     }
   }
   template <int I, class T, int N>
   THX_DEV void st(const Vec<T, N>& r) const {
-    *((T*)ptr[I] + off[I]) = r.v[0];
+    store_vec<T, N, P::NT != 0>((T*)ptr[I] + off[I], r);
   }
 };
 
+// TV consecutive elements per access: along T while staging, along the inner
+// dimension while computing. The host guarantees that both extents are
+// multiples of TV and that every vector access is aligned.
 template <class F, class P>
 __device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, typename P::IT>& p) {
   typedef typename P::IT IT;
-  constexpr int TILE = P::TILE, NOPS = F::NOPS, ND = P::ND, ROWS = P::BLOCK / TILE, UNR = 4;
+  constexpr int TILE = P::TILE, TV = P::TV, NOPS = F::NOPS, ND = P::ND;
+  constexpr int LPR = TILE / TV;            // lanes per tile row
+  constexpr int RPP = P::BLOCK / LPR;       // tile rows per pass
+  constexpr int PASSES = TILE / RPP;
+  constexpr int UNR = PASSES < 4 ? PASSES : 4;
   __shared__ __attribute__((aligned(16))) unsigned char lds[P::NTR * TILE * (TILE + 1) * P::ESZ];
 
   unsigned rem = blockIdx.x, ti, tt, c;
@@ -223,53 +241,53 @@ __device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, type
     for (int i = 0; i < NOPS; ++i) base[i] += (IT)rem * p.ostride[i][0];
   }
   const int t0 = tt * TILE, i0 = ti * TILE;
-  const int lane = threadIdx.x % TILE, row = threadIdx.x / TILE;
+  const int lane = threadIdx.x % LPR, row = threadIdx.x / LPR;
 
   // stage: lanes run along T
   {
-    typename F::template Regs<1> dummy;
-    const int t = t0 + lane;
+    typename F::template Regs<TV> dummy;
+    const int t = t0 + lane * TV;
 #pragma unroll
-    for (int k = 0; k < TILE / ROWS; ++k) {
-      const int ii = row + k * ROWS, i = i0 + ii;
+    for (int k = 0; k < PASSES; ++k) {
+      const int ii = row + k * RPP, i = i0 + ii;
       if (t < p.ext_t && i < p.ext_i) {
         TrStageAcc<P, NOPS> a;
         a.ptr = p.ptr;
         a.lds = lds;
-        a.cell = ii * (TILE + 1) + lane;
+        a.cell = ii * (TILE + 1) + lane * TV;
 #pragma unroll
         for (int o = 0; o < NOPS; ++o) a.off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
-        F::template load<1>(a, dummy);
+        F::template load<TV>(a, dummy);
       }
     }
   }
   __syncthreads();
 
   // compute: lanes run along the innermost dimension
-  const int i = i0 + lane;
+  const int i = i0 + lane * TV;
 #pragma unroll
-  for (int k0 = 0; k0 < TILE / ROWS; k0 += UNR) {
-    typename F::template Regs<1> r[UNR];
+  for (int k0 = 0; k0 < PASSES; k0 += UNR) {
+    typename F::template Regs<TV> r[UNR];
     TrAcc<P, NOPS> a[UNR];
     bool ok[UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      const int tl = row + (k0 + u) * ROWS, t = t0 + tl;
+      const int tl = row + (k0 + u) * RPP, t = t0 + tl;
       ok[u] = t < p.ext_t && i < p.ext_i;
       a[u].ptr = p.ptr;
       a[u].imm = p.imm;
       a[u].lds = lds;
-      a[u].cell = lane * (TILE + 1) + tl;
+      a[u].cell = lane * TV * (TILE + 1) + tl;
 #pragma unroll
       for (int o = 0; o < NOPS; ++o) a[u].off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
-      if (ok[u]) F::template load<1>(a[u], r[u]);
+      if (ok[u]) F::template load<TV>(a[u], r[u]);
     }
 #pragma unroll
     for (int u = 0; u < UNR; ++u)
-      if (ok[u]) F::template compute<1>(r[u]);
+      if (ok[u]) F::template compute<TV>(r[u]);
 #pragma unroll
     for (int u = 0; u < UNR; ++u)
-      if (ok[u]) F::template store<1>(a[u], r[u]);
+      if (ok[u]) F::template store<TV>(a[u], r[u]);
   }
 }
 

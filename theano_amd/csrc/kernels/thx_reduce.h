@@ -2,7 +2,7 @@
 // fused per-result epilogue.
 //
 // A generated functor R supplies
-//   enum { NIN, NOUT };
+//   enum { NIN, NOUT, NEX };                             // NEX host scalars feed the epilogue
 //   struct Acc;                                          // one field per reduction
 //   template <int V> struct Regs;                        // one Vec per input
 //   static void init(Acc&);                              // identities
@@ -21,9 +21,11 @@
 
 namespace thx {
 
-template <int NOUT>
+// Where results go, plus the values of the host scalars the epilogue uses.
+template <int NOUT, int NEX>
 struct RedOut {
   char* ptr[NOUT];
+  unsigned long long ex[NEX > 0 ? NEX : 1];
 };
 
 // ---------------------------------------------------------------------------
@@ -31,11 +33,11 @@ struct RedOut {
 // the vectorised dimension. TPR threads cooperate on one output; a block holds
 // BLOCK / TPR outputs. Covers trailing-axis reductions, whole-array reductions
 // (one output, many slices) and outer x kept x inner patterns (RA > 1).
-template <int NIN, int NOUT, int NK, class IT>
+template <int NIN, int NOUT, int NEX, int NK, class IT>
 struct RowParams {
   char* in[NIN];
   unsigned long long imm[NIN];
-  RedOut<NOUT> out;
+  RedOut<NOUT, NEX> out;
   char* partial;          // Acc[S][n_out] when S > 1
   long long n_out;
   long long nvec;         // vectors in one output's reduce domain (RA * RC / VEC)
@@ -85,7 +87,7 @@ struct RedAcc {
 // Plan members: typedef IT; enum { NK, VEC, UNR, BLOCK, TPR, RA2 (1 when RA > 1) };
 // static constexpr int mode(int input).
 template <class R, class P>
-__device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, P::NK, typename P::IT>& p) {
+__device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p) {
   typedef typename P::IT IT;
   typedef typename UnsignedOf<IT>::type UT;
   typedef typename R::Acc Acc;
@@ -175,11 +177,11 @@ __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, P:
 // side along the columns (VEC columns each, so a wave reads whole row segments)
 // and TY row lanes; per-column partials live in registers and the TY lanes are
 // merged through LDS at the end. Rows are split into S slices.
-template <int NIN, int NOUT, int NK, class IT>
+template <int NIN, int NOUT, int NEX, int NK, class IT>
 struct ColParams {
   char* in[NIN];
   unsigned long long imm[NIN];
-  RedOut<NOUT> out;
+  RedOut<NOUT, NEX> out;
   char* partial;          // Acc[S][n_out] when S > 1
   long long n_out;        // A * C
   long long rows;         // R
@@ -199,7 +201,7 @@ struct ColParams {
 // Plan members: typedef IT; enum { NK, VEC, UNR, BLOCK, TX, RR2 (1 when two
 // reduced dimensions remain after collapsing) }; mode(int).
 template <class R, class P>
-__device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, P::NK, typename P::IT>& p) {
+__device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p) {
   typedef typename P::IT IT;
   typedef typename UnsignedOf<IT>::type UT;
   typedef typename R::Acc Acc;
@@ -293,9 +295,9 @@ __device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, P:
 // ---------------------------------------------------------------------------
 // Second pass: merge the S partial Acc values of every output, slice 0 first.
 // TPO threads per output (1, 64 or BLOCK).
-template <int NOUT>
+template <int NOUT, int NEX>
 struct FinalParams {
-  RedOut<NOUT> out;
+  RedOut<NOUT, NEX> out;
   char* partial;
   long long n_out;
   int S;
@@ -303,7 +305,7 @@ struct FinalParams {
 };
 
 template <class R, int BLOCK, int TPO>
-__device__ __forceinline__ void red_final_body(const FinalParams<R::NOUT>& p) {
+__device__ __forceinline__ void red_final_body(const FinalParams<R::NOUT, R::NEX>& p) {
   typedef typename R::Acc Acc;
   __shared__ Acc lds[BLOCK / THX_WAVE];
   const Acc* part = (const Acc*)p.partial;
@@ -326,11 +328,11 @@ __device__ __forceinline__ void red_final_body(const FinalParams<R::NOUT>& p) {
 // Fallback for any mask that does not collapse to the row or column form: TPR
 // threads per output walk the flattened reduce domain and decompose every
 // index. Correct for every pattern, coalesced only by luck.
-template <int NIN, int NOUT, int NK, int NR, class IT>
+template <int NIN, int NOUT, int NEX, int NK, int NR, class IT>
 struct GenParams {
   char* in[NIN];
   unsigned long long imm[NIN];
-  RedOut<NOUT> out;
+  RedOut<NOUT, NEX> out;
   long long n_out;
   long long n_red;
   FastDiv kfd[NK];
@@ -341,7 +343,7 @@ struct GenParams {
 
 // Plan members: typedef IT; enum { NK, NR, BLOCK, TPR }.
 template <class R, class P>
-__device__ __forceinline__ void red_gen_body(const GenParams<R::NIN, R::NOUT, P::NK, P::NR, typename P::IT>& p) {
+__device__ __forceinline__ void red_gen_body(const GenParams<R::NIN, R::NOUT, R::NEX, P::NK, P::NR, typename P::IT>& p) {
   typedef typename P::IT IT;
   typedef typename UnsignedOf<IT>::type UT;
   typedef typename R::Acc Acc;

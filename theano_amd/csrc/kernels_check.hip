@@ -22,7 +22,7 @@ struct CheckF {
 };
 
 struct CheckR {
-  enum { NIN = 1, NOUT = 2 };
+  enum { NIN = 1, NOUT = 2, NEX = 1 };
   struct Acc { thx_f64 a0; thx_f32 a1; };
   template <int V> struct Regs { thx::Vec<thx_f32, V> i0; };
   THX_DEV static void init(Acc& a) { a.a0 = 0.0; a.a1 = -INFINITY; }
@@ -43,7 +43,7 @@ struct CheckR {
   THX_DEV static Acc shfl_xor(const Acc& a, int m) { Acc r; r.a0 = thx::shfl_xor_t(a.a0, m); r.a1 = thx::shfl_xor_t(a.a1, m); return r; }
   template <class O> THX_DEV static void post(const O& o, long long idx, const Acc& a) {
     ((thx_f32*)o.ptr[0])[idx] = (thx_f32)a.a0;
-    ((thx_f32*)o.ptr[1])[idx] = (thx_f32)a.a1;
+    ((thx_f32*)o.ptr[1])[idx] = (thx_f32)a.a1 / *(const thx_f32*)&o.ex[0];
   }
 };
 
@@ -60,14 +60,14 @@ struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, T
 struct PlanGen { typedef int IT; enum { NK = 3, NR = 3, BLOCK = 256, TPR = 64, NT = 0 };
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; } };
 
-struct PlanTr { typedef int IT; enum { ND = 3, TILE = 64, BLOCK = 256, NTR = 1, ESZ = 2, NT = 0 };
+struct PlanTr { typedef int IT; enum { ND = 3, TILE = 64, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2, NT = 0 };
   static constexpr int mode(int i) { constexpr int m[] = {2, 0, 0}; return m[i]; }
   static constexpr int slot(int i) { constexpr int m[] = {0, -1, -1}; return m[i]; } };
 extern "C" __global__ __launch_bounds__(256) void check_tr(thx::EwTrParams<3, 3, int> p) { thx::ew_tr_body<CheckF, PlanTr>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_ew1(thx::EwParams<3, 1, int> p) { thx::ew_body<CheckF, PlanEw1>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_ew3(thx::EwParams<3, 3, long long> p) { thx::ew_body<CheckF, PlanEw3>(p); }
-extern "C" __global__ __launch_bounds__(256) void check_row(thx::RowParams<1, 2, 2, int> p) { thx::red_row_body<CheckR, PlanRow>(p); }
-extern "C" __global__ __launch_bounds__(256) void check_rows(thx::RowParams<1, 2, 1, int> p) { thx::red_row_body<CheckR, PlanRowS>(p); }
-extern "C" __global__ __launch_bounds__(256) void check_col(thx::ColParams<1, 2, 1, int> p) { thx::red_col_body<CheckR, PlanCol>(p); }
-extern "C" __global__ __launch_bounds__(256) void check_gen(thx::GenParams<1, 2, 3, 3, int> p) { thx::red_gen_body<CheckR, PlanGen>(p); }
-extern "C" __global__ __launch_bounds__(256) void check_fin(thx::FinalParams<2> p) { thx::red_final_body<CheckR, 256, 64>(p); }
+extern "C" __global__ __launch_bounds__(256) void check_row(thx::RowParams<1, 2, 1, 2, int> p) { thx::red_row_body<CheckR, PlanRow>(p); }
+extern "C" __global__ __launch_bounds__(256) void check_rows(thx::RowParams<1, 2, 1, 1, int> p) { thx::red_row_body<CheckR, PlanRowS>(p); }
+extern "C" __global__ __launch_bounds__(256) void check_col(thx::ColParams<1, 2, 1, 1, int> p) { thx::red_col_body<CheckR, PlanCol>(p); }
+extern "C" __global__ __launch_bounds__(256) void check_gen(thx::GenParams<1, 2, 1, 3, 3, int> p) { thx::red_gen_body<CheckR, PlanGen>(p); }
+extern "C" __global__ __launch_bounds__(256) void check_fin(thx::FinalParams<2, 1> p) { thx::red_final_body<CheckR, 256, 64>(p); }

@@ -216,11 +216,33 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
         }
       int tile = 64;
       if ((int64_t)ntr * tile * (tile + 1) * esz > 60000) tile = 32;
+      // elements per access: 16 bytes of the widest operand, if extents, strides and addresses allow
+      int allsz = 1;
+      for (int o = 0; o < nops; ++o)
+        if (!views[o].imm) allsz = std::max(allsz, dtype_size(views[o].dtype));
+      int tv = std::min(4, 16 / allsz);
+      auto tv_ok = [&](int v) {
+        if (v == 1) return true;
+        if (dm.shape[tdim] % v || inner % v) return false;
+        for (int o = 0; o < nops; ++o) {
+          if (views[o].imm) continue;
+          const bool staged = slot[o] >= 0;
+          if (!staged && mode[o] != M_VEC) continue;  // broadcast operands are read one element at a time
+          if (((uintptr_t)views[o].ptr) % (size_t)(dtype_size(views[o].dtype) * v)) return false;
+          for (int d = 0; d < ND; ++d) {
+            if (staged ? d == tdim : d == ND - 1) continue;
+            if (dm.stride[o][d] % v) return false;
+          }
+        }
+        return true;
+      };
+      while (!tv_ok(tv)) tv /= 2;
+      if (env_int("THX_EW_TV", 0) == 1) tv = 1;
       if ((int64_t)ntr * tile * (tile + 1) * esz <= 60000) {
         const int block = 256;
         const int nt = env_int("THX_NT", 0);
         std::ostringstream key;
-        key << "et|nd" << ND << "|t" << tile << "|n" << ntr << "|e" << esz << (nt ? "|nt" : "") << "|m";
+        key << "et|nd" << ND << "|t" << tile << "|v" << tv << "|n" << ntr << "|e" << esz << (nt ? "|nt" : "") << "|m";
         for (int o = 0; o < nops; ++o) key << (slot[o] >= 0 ? 9 : mode[o]) << (o + 1 < nops ? "," : "");
         const std::string plan = key.str();
         set_last_plan(e->name + "|" + plan);
@@ -231,7 +253,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
         } else {
           std::ostringstream s;
           s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef int IT;\n  enum { ND = " << ND
-            << ", TILE = " << tile << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz << ", NT = " << nt
+            << ", TILE = " << tile << ", TV = " << tv << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz << ", NT = " << nt
             << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
           for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
           s << "};\n    return m[i];\n  }\n  static constexpr int slot(int i) {\n    constexpr int m[] = {";

@@ -12,7 +12,7 @@
 
 struct thx_reduce {
   std::string src, name;
-  int n_in = 0, n_out = 0, acc_bytes = 0;
+  int n_in = 0, n_out = 0, n_extra = 0, acc_bytes = 0;
   std::vector<int32_t> dtypes;
   std::unordered_map<std::string, thx::Kernel> plans;
 };
@@ -63,7 +63,8 @@ static std::string plan_struct(bool wide, const std::vector<std::pair<std::strin
   return s.str();
 }
 
-static int final_pass(thx_reduce* r, const std::vector<char*>& outp, char* partial, int64_t n_out, int S, bool dry) {
+static int final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::vector<uint64_t>& ex, char* partial,
+                      int64_t n_out, int S, bool dry) {
   const int tpo = n_out >= 1024 ? 1 : (n_out >= 16 ? 64 : 256);
   const std::string plan = "rf|t" + std::to_string(tpo);
   Kernel k;
@@ -73,7 +74,7 @@ static int final_pass(thx_reduce* r, const std::vector<char*>& outp, char* parti
   } else {
     std::ostringstream s;
     s << device_prelude() << r->src << "\nextern \"C\" __global__ __launch_bounds__(256) void thx_entry(thx::FinalParams<"
-      << r->name << "::NOUT> p) {\n  thx::red_final_body<" << r->name << ", 256, " << tpo << ">(p);\n}\n";
+      << r->name << "::NOUT, " << r->name << "::NEX> p) {\n  thx::red_final_body<" << r->name << ", 256, " << tpo << ">(p);\n}\n";
     int rc = get_kernel(s.str(), "thx_entry", &k);
     if (rc) return rc;
     r->plans[plan] = k;
@@ -81,6 +82,7 @@ static int final_pass(thx_reduce* r, const std::vector<char*>& outp, char* parti
   if (dry) return THX_OK;
   ParamPack pk;
   for (char* p : outp) pk.put<char*>(p);
+  for (uint64_t v : ex) pk.put<uint64_t>(v);
   pk.put<char*>(partial);
   pk.put<int64_t>(n_out);
   pk.put<int32_t>(S);
@@ -96,19 +98,21 @@ using namespace thx;
 
 extern "C" {
 
-int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, int n_out, const int32_t* dtypes,
-                   int acc_bytes, thx_reduce** out) {
+int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, int n_out, int n_extra,
+                   const int32_t* dtypes, int acc_bytes, thx_reduce** out) {
   if (!functor_src || !functor_name || !dtypes || !out) return fail(THX_ERR_ARG, "thx_reduce_new: null argument");
-  if (n_in < 1 || n_out < 1 || acc_bytes < 1) return fail(THX_ERR_ARG, "thx_reduce_new: needs inputs, outputs and an accumulator");
-  for (int i = 0; i < n_in + n_out; ++i)
+  if (n_in < 1 || n_out < 1 || n_extra < 0 || acc_bytes < 1)
+    return fail(THX_ERR_ARG, "thx_reduce_new: needs inputs, outputs and an accumulator");
+  for (int i = 0; i < n_in + n_out + n_extra; ++i)
     if (!dtype_size(dtypes[i])) return fail(THX_ERR_TYPE, "thx_reduce_new: unknown dtype code %d", dtypes[i]);
   thx_reduce* r = new thx_reduce;
   r->src = functor_src;
   r->name = functor_name;
   r->n_in = n_in;
   r->n_out = n_out;
+  r->n_extra = n_extra;
   r->acc_bytes = acc_bytes;
-  r->dtypes.assign(dtypes, dtypes + n_in + n_out);
+  r->dtypes.assign(dtypes, dtypes + n_in + n_out + n_extra);
   *out = r;
   return THX_OK;
 }
@@ -132,6 +136,15 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   int rc = gather_inputs("reduce", ins, NIN, r->dtypes.data(), flags, &nd, shape, &views);
   if (rc) return rc;
   if (nd > 0 && !reduce_mask) return fail(THX_ERR_ARG, "thx_reduce_call: null mask");
+  // host scalars of the epilogue follow the reduced inputs
+  std::vector<uint64_t> ex(std::max(1, r->n_extra), 0);
+  for (int j = 0; j < r->n_extra; ++j) {
+    const thx_array& a = ins[NIN + j];
+    const int want = r->dtypes[NIN + NOUT + j];
+    if (!(a.dtype & THX_HOST_SCALAR) || (a.dtype & ~THX_HOST_SCALAR) != want)
+      return fail(THX_ERR_TYPE, "reduce: epilogue operand %d must be a host scalar of dtype code %d", j, want);
+    memcpy(&ex[j], (const char*)a.base + a.offset_bytes, (size_t)dtype_size(want));
+  }
 
   // outputs: C-contiguous arrays of the kept dimensions
   int64_t kshape[THX_MAX_ND];
@@ -171,7 +184,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   }
   if (n_red == 0) {  // identity through the epilogue
     set_last_plan(r->name + "|rf|identity");
-    return final_pass(r, outp, nullptr, n_out, 0, dry);
+    return final_pass(r, outp, ex, nullptr, n_out, 0, dry);
   }
 
   // primary input: the one that spans the most memory
@@ -304,7 +317,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       s << device_prelude() << r->src
         << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TPR", tpr}, {"RA2", ra2}, {"NT", nt}}, mode)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::RowParams<" << r->name
-        << "::NIN, " << r->name << "::NOUT, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
+        << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
       rc = get_kernel(s.str(), "thx_entry", &k);
       if (rc) return rc;
@@ -317,6 +330,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
     for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
+    for (uint64_t v : ex) pk.put<uint64_t>(v);
     pk.put<char*>(rt().scratch);
     pk.put<int64_t>(n_out);
     pk.put<int64_t>(nvec);
@@ -397,7 +411,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       s << device_prelude() << r->src
         << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TX", tx}, {"RR2", rr2}, {"NT", nt}}, mode)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::ColParams<" << r->name
-        << "::NIN, " << r->name << "::NOUT, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_col_body<" << r->name
+        << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_col_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
       rc = get_kernel(s.str(), "thx_entry", &k);
       if (rc) return rc;
@@ -410,6 +424,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
     for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
+    for (uint64_t v : ex) pk.put<uint64_t>(v);
     pk.put<char*>(rt().scratch);
     pk.put<int64_t>(n_out);
     pk.put<int64_t>(rows);
@@ -447,7 +462,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       s << device_prelude() << r->src
         << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}, {"NT", 0}}, gmode)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::GenParams<" << r->name
-        << "::NIN, " << r->name << "::NOUT, ThxPlan::NK, ThxPlan::NR, ThxPlan::IT> p) {\n  thx::red_gen_body<" << r->name
+        << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::NR, ThxPlan::IT> p) {\n  thx::red_gen_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
       rc = get_kernel(s.str(), "thx_entry", &k);
       if (rc) return rc;
@@ -456,6 +471,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
     for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
+    for (uint64_t v : ex) pk.put<uint64_t>(v);
     pk.put<int64_t>(n_out);
     pk.put<int64_t>(n_red);
     for (int d = 0; d < NK; ++d) pk.put<FastDivH>(make_fastdiv(d < NKD ? (uint64_t)KD[d].extent : 1));
@@ -474,7 +490,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     rc = launch(k, r->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
     if (rc) return rc;
   }
-  if (S > 1) return final_pass(r, outp, rt().scratch, n_out, S, dry);
+  if (S > 1) return final_pass(r, outp, ex, rt().scratch, n_out, S, dry);
   return THX_OK;
 }
 

@@ -96,18 +96,21 @@ def acc_struct_bytes(acc_dtypes):
     return (off + align - 1) // align * align
 
 
-def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, post_op=None):
+def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, post_op=None, extra_dtypes=(),
+                   post_in_dtypes=None):
     """(source, name, sizeof(Acc)) for K simultaneous reductions.
 
     Per element, ``pre_op`` (nin = len(in_dtypes), nout = K; default: the single
     input itself) yields K values, each cast to its accumulator dtype and
-    folded with ``scalar_ops[k]``.  ``post_op`` (nin = K) maps the K results to
-    the outputs; the default casts result k to ``out_dtypes[k]``."""
+    folded with ``scalar_ops[k]``.  ``post_op`` (nin = K + len(extra_dtypes))
+    maps the K results, each first cast to ``post_in_dtypes`` (the dtype the
+    unfused reduction would have produced), and the extra host scalars to the
+    outputs; the default casts result k to ``out_dtypes[k]``."""
     K = len(scalar_ops)
     nin, nout = len(in_dtypes), len(out_dtypes)
     ins = ["i%d" % k for k in range(nin)]
     acc_c = [compute_ctype(dt) for dt in acc_dtypes]
-    lines = ["  enum { NIN = %d, NOUT = %d };" % (nin, nout)]
+    lines = ["  enum { NIN = %d, NOUT = %d, NEX = %d };" % (nin, nout, len(extra_dtypes))]
     lines.append("  struct Acc { %s };" % " ".join("%s a%d;" % (c, k) for k, c in enumerate(acc_c)))
     lines.append(_regs(in_dtypes, ins).rstrip("\n"))
     init = []
@@ -159,13 +162,22 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
             post.append("((%s*)o.ptr[%d])[idx] = (%s)%s;" % (storage_ctype(dt), k, storage_ctype(dt), val))
         post_stmt = "\n".join(post)
     else:
-        qnode = _scalar_node(post_op, acc_dtypes)
+        post_in = list(post_in_dtypes) if post_in_dtypes is not None else list(acc_dtypes)
+        qnode = _scalar_node(post_op, post_in + list(extra_dtypes))
         if [o.type.dtype for o in qnode.outputs] != list(out_dtypes):
             raise TypeError("epilogue gives %s, node expects %s" % ([o.type.dtype for o in qnode.outputs],
                                                                       list(out_dtypes)))
         tmp = ["q%d" % k for k in range(nout)]
         post_stmt = " ".join("%s %s;" % (compute_ctype(dt), t) for dt, t in zip(out_dtypes, tmp))
-        post_stmt += "\n" + post_op.c_code(qnode, ["a.a%d" % k for k in range(K)], tmp) + "\n"
+        # each reduction result takes the storage precision of the unfused node's output first
+        args = []
+        for k, dt in enumerate(post_in):
+            post_stmt += "\n%s r%d = (%s)(%s)%s;" % (compute_ctype(dt), k, compute_ctype(dt), storage_ctype(dt),
+                                                     "(a.a%d ? 1 : 0)" % k if dt == "bool" else "a.a%d" % k)
+            args.append("r%d" % k)
+        for j, dt in enumerate(extra_dtypes):
+            args.append("(*(const %s*)&o.ex[%d])" % (storage_ctype(dt), j))
+        post_stmt += "\n" + post_op.c_code(qnode, args, tmp) + "\n"
         post_stmt += "\n".join("((%s*)o.ptr[%d])[idx] = (%s)%s;" % (storage_ctype(dt), k, storage_ctype(dt), t)
                                for k, (dt, t) in enumerate(zip(out_dtypes, tmp)))
     lines.append("  template <class O> THX_DEV static void post(const O& o, long long idx, const Acc& a) {\n%s\n  }"

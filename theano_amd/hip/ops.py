@@ -321,9 +321,11 @@ class HipCAReduce(CAReduce):
     without prologue or epilogue; the fusion pass widens it.  The generalisation
     of ``GpuCAReduceCuda``'s ``pre_scalar_op`` (``theano/gpuarray/elemwise.py:492-493``)."""
 
-    __props__ = ("scalar_ops", "axis", "acc_dtypes", "out_dtypes", "pre_scalar_op", "post_scalar_op")
+    __props__ = ("scalar_ops", "axis", "acc_dtypes", "out_dtypes", "pre_scalar_op", "post_scalar_op",
+                 "post_in_dtypes", "n_extra")
 
-    def __init__(self, scalar_ops, axis, acc_dtypes, out_dtypes, pre_scalar_op=None, post_scalar_op=None):
+    def __init__(self, scalar_ops, axis, acc_dtypes, out_dtypes, pre_scalar_op=None, post_scalar_op=None,
+                 post_in_dtypes=None, n_extra=0):
         scalar_ops = tuple(scalar_ops)
         for op in scalar_ops:
             if op.nin not in (-1, 2) or op.nout != 1:
@@ -340,11 +342,18 @@ class HipCAReduce(CAReduce):
         self.out_dtypes = tuple(out_dtypes)
         self.pre_scalar_op = pre_scalar_op
         self.post_scalar_op = post_scalar_op
+        # with an epilogue: the dtype each reduction result has before the epilogue reads it, and the
+        # number of trailing host-scalar inputs that only the epilogue uses
+        self.post_in_dtypes = None if post_in_dtypes is None else tuple(post_in_dtypes)
+        self.n_extra = int(n_extra)
         if len(self.acc_dtypes) != len(scalar_ops):
             raise ValueError("one accumulator dtype per reduction")
+        if self.n_extra and post_scalar_op is None:
+            raise ValueError("extra scalars need an epilogue")
 
     def _props(self):
-        return (self.scalar_ops, self.axis, self.acc_dtypes, self.out_dtypes, self.pre_scalar_op, self.post_scalar_op)
+        return (self.scalar_ops, self.axis, self.acc_dtypes, self.out_dtypes, self.pre_scalar_op, self.post_scalar_op,
+                self.post_in_dtypes, self.n_extra)
 
     def __str__(self):
         ops = ",".join(str(o) for o in self.scalar_ops)
@@ -357,6 +366,11 @@ class HipCAReduce(CAReduce):
         return "HipCAReduce{%s}%s{acc=%s%s}" % (ops, ax, ",".join(self.acc_dtypes), extra)
 
     def make_node(self, *inputs):
+        extras = list(inputs[len(inputs) - self.n_extra:]) if self.n_extra else []
+        inputs = inputs[:len(inputs) - self.n_extra] if self.n_extra else inputs
+        for e in extras:
+            if not _is_host_scalar(e):
+                raise TypeError("epilogue operands must be host scalars", e)
         ins = [i if (isinstance(i.type, HipArrayType) or _is_host_scalar(i)) else as_hip_variable(i) for i in inputs]
         nd = max(i.type.ndim for i in ins)
         if any(i.type.ndim != nd for i in ins if isinstance(i.type, HipArrayType)):
@@ -369,27 +383,31 @@ class HipCAReduce(CAReduce):
                 raise ValueError("Not enough dimensions on the input to reduce on axis %s" % a)
         bcast = [all(b) for b in zip(*[i.type.broadcastable for i in ins if i.type.ndim == nd])]
         ob = [b for d, b in enumerate(bcast) if d not in axis]
-        return Apply(self, ins, [HipArrayType(dt, ob)() for dt in self.out_dtypes])
+        return Apply(self, ins + extras, [HipArrayType(dt, ob)() for dt in self.out_dtypes])
 
     def infer_shape(self, node, shapes):
-        nd = max(i.type.ndim for i in node.inputs)
+        shapes = shapes[:len(shapes) - self.n_extra] if self.n_extra else shapes
+        nd = max(i.type.ndim for i in node.inputs[:len(shapes)])
         axis = self.axis if self.axis is not None else tuple(range(nd))
         full = [max(s[d] for s in shapes if len(s) == nd) for d in range(nd)]
         kept = tuple(full[d] for d in range(nd) if d not in axis)
         return [kept for _ in node.outputs]
 
     def _handle(self, node):
-        in_dt = tuple(i.type.dtype for i in node.inputs)
-        key = (self.scalar_ops, self.acc_dtypes, self.out_dtypes, self.pre_scalar_op, self.post_scalar_op, in_dt)
+        n_red = len(node.inputs) - self.n_extra
+        in_dt = tuple(i.type.dtype for i in node.inputs[:n_red])
+        ex_dt = tuple(i.type.dtype for i in node.inputs[n_red:])
+        key = (self._props(), in_dt, ex_dt)
         h = _reduce_handles.get(key)
         if h is None:
             src, name, acc_bytes = codegen.reduce_functor(self.scalar_ops, self.acc_dtypes, in_dt, self.out_dtypes,
-                                                          self.pre_scalar_op, self.post_scalar_op)
-            all_dt = in_dt + self.out_dtypes
+                                                          self.pre_scalar_op, self.post_scalar_op, ex_dt,
+                                                          self.post_in_dtypes)
+            all_dt = in_dt + self.out_dtypes + ex_dt
             codes = (ctypes.c_int32 * len(all_dt))(*[scal.dtype_code(d) for d in all_dt])
             handle = ctypes.c_void_p()
-            check(lib.thx_reduce_new(src.encode(), name.encode(), len(in_dt), len(self.out_dtypes), codes, acc_bytes,
-                                     ctypes.byref(handle)))
+            check(lib.thx_reduce_new(src.encode(), name.encode(), len(in_dt), len(self.out_dtypes), len(ex_dt), codes,
+                                     acc_bytes, ctypes.byref(handle)))
             h = (handle, len(in_dt), len(self.out_dtypes))
             _reduce_handles[key] = h
         return h
@@ -399,13 +417,13 @@ class HipCAReduce(CAReduce):
         cache = node.tag.get("thx")
         if cache is None:
             handle, nin, nout = self._handle(node)
-            nd = max(i.type.ndim for i in node.inputs)
+            nd = max(i.type.ndim for i in node.inputs[:nin])
             axis = self.axis if self.axis is not None else tuple(range(nd))
             mask = (ctypes.c_uint8 * max(nd, 1))(*[1 if d in axis else 0 for d in range(nd)])
-            cache = node.tag["thx"] = (handle, nin, nout, (thx_array * nin)(), (thx_array * nout)(), nd, axis, mask,
-                                       [np.dtype(d) for d in self.out_dtypes])
+            cache = node.tag["thx"] = (handle, nin, nout, (thx_array * len(node.inputs))(), (thx_array * nout)(), nd,
+                                       axis, mask, [np.dtype(d) for d in self.out_dtypes])
         handle, nin, nout, ins, outs, nd, axis, mask, out_dt = cache
-        shape = _check_runtime_broadcast(node.inputs, inputs, nd)
+        shape = _check_runtime_broadcast(node.inputs[:nin], inputs[:nin], nd)
         n_red = 1
         for a in axis:
             n_red *= shape[a]

@@ -170,9 +170,16 @@ def _duplicable(fgraph, var):
 
 def _fusable(fgraph, var, out_bcast):
     node = var.owner
-    return (node is not None and isinstance(node.op, HipElemwise) and len(node.outputs) == 1 and
-            not node.op.inplace_pattern and tuple(var.type.broadcastable) == tuple(out_bcast) and
-            (fgraph.n_clients(var) == 1 or _duplicable(fgraph, var)))
+    if (node is None or not isinstance(node.op, HipElemwise) or len(node.outputs) != 1 or node.op.inplace_pattern or
+            len(var.type.broadcastable) != len(out_bcast)):
+        return False
+    if tuple(var.type.broadcastable) == tuple(out_bcast):
+        return fgraph.n_clients(var) == 1 or _duplicable(fgraph, var)
+    # a producer that is broadcast against the consumer (a per-channel cast, say) is recomputed per
+    # element only when that costs next to nothing; the reference keeps such nodes apart
+    # (theano/tensor/opt.py:7171-7175) because its C loops would redo real work
+    return (fgraph.n_clients(var) == 1 and _cheap(node.op.scalar_op) and
+            all(pb or not cb for pb, cb in zip(var.type.broadcastable, out_bcast)))
 
 
 def _fuse_node(fgraph, node):
@@ -330,6 +337,108 @@ def fuse_reduce_prologue(fgraph):
     return count
 
 
+def fuse_reduce_epilogue(fgraph):
+    """``g(reduce(...), host scalars)`` - the division of a mean, ``sqrt(var + eps)``
+    - runs in the reduction's own last step instead of a launch of its own.
+    Matches an elementwise node all of whose array inputs are results of one
+    reduction (possibly through identical keepdims DimShuffles)."""
+    count = 0
+    changed = True
+    while changed:
+        changed = False
+        for red in fgraph.toposort():
+            rop = red.op
+            if not isinstance(rop, HipCAReduce) or rop.post_scalar_op is not None or red not in fgraph.apply_nodes:
+                continue
+            cand = None
+            for r in red.outputs:
+                for c, _ in fgraph.clients.get(r, []):
+                    if c == "output":
+                        continue
+                    if isinstance(c.op, HipDimShuffle):
+                        for c2, _ in fgraph.clients.get(c.outputs[0], []):
+                            if c2 != "output" and isinstance(c2.op, HipElemwise):
+                                cand = c2
+                    elif isinstance(c.op, HipElemwise):
+                        cand = c
+                    if cand is not None:
+                        break
+                if cand is not None:
+                    break
+            if cand is None or len(cand.outputs) != 1 or cand.op.inplace_pattern:
+                continue
+            # classify the consumer's inputs
+            ds_op, ok, s_args, extras, s_extras = None, True, [], [], []
+            s_acc = [scal.Scalar(dt)() for dt in rop.out_dtypes]
+            used = set()
+            for i in cand.inputs:
+                src, this_ds = i, None
+                if src.owner is not None and isinstance(src.owner.op, HipDimShuffle):
+                    this_ds = src.owner.op
+                    src = src.owner.inputs[0]
+                if src.owner is red:
+                    if ds_op is not None and this_ds != ds_op and used:
+                        ok = False
+                        break
+                    ds_op = this_ds
+                    k = red.outputs.index(src)
+                    used.add(k)
+                    s_args.append(s_acc[k])
+                    continue
+                c = _scalar_constant(i)
+                if c is not None:
+                    s_args.append(c)
+                elif _is_host_scalar(i):
+                    sv = None
+                    for e, se in zip(extras, s_extras):
+                        if e is i:
+                            sv = se
+                    if sv is None:
+                        sv = scal.Scalar(i.type.dtype)()
+                        extras.append(i)
+                        s_extras.append(sv)
+                    s_args.append(sv)
+                else:
+                    ok = False
+                    break
+            if not ok or not used or len(extras) > 8:
+                continue
+            e_out = cand.op.scalar_op(*s_args)
+            # reduction results something else still needs stay outputs of the new node
+            keep = []
+            for k, r in enumerate(red.outputs):
+                others = False
+                for c, _ in fgraph.clients.get(r, []):
+                    if c == "output":
+                        others = True
+                    elif isinstance(c.op, HipDimShuffle) and c.op == ds_op:
+                        if any(c2 is not cand for c2, _ in fgraph.clients.get(c.outputs[0], [])):
+                            others = True
+                    elif c is not cand:
+                        others = True
+                if others or k not in used:
+                    keep.append(k)
+            post_outs = [scal.identity(s_acc[k]) for k in keep] + [e_out]
+            post = scal.Composite(s_acc + s_extras, post_outs)
+            out_dtypes = tuple(rop.out_dtypes[k] for k in keep) + (cand.outputs[0].type.dtype,)
+            n_red_in = len(red.inputs)
+            new_op = HipCAReduce(rop.scalar_ops, rop.axis, rop.acc_dtypes, out_dtypes, rop.pre_scalar_op, post,
+                                 rop.out_dtypes, len(extras))
+            new_node = new_op.make_node(*(list(red.inputs[:n_red_in]) + extras))
+            new_e = new_node.outputs[-1]
+            if ds_op is not None:
+                new_e = HipDimShuffle(ds_op.input_broadcastable, ds_op.new_order)(new_e)
+            if new_e.type != cand.outputs[0].type:
+                continue
+            for j, k in enumerate(keep):
+                fgraph.replace(red.outputs[k], new_node.outputs[j])
+            fgraph.replace(cand.outputs[0], new_e)
+            count += 1
+            changed = True
+            break
+    return count
+
+
 def _depends_on(var, node, limit=10000):
     """True when ``var`` is computed (transitively) from an output of ``node``."""
     stack, seen = [var], set()
@@ -432,5 +541,7 @@ def optimize(fgraph, fuse=True, rowchain=True):
         fuse_reduce_prologue(fgraph)
         gof.merge_identical(fgraph)
         merge_sibling_reductions(fgraph)
+        gof.merge_identical(fgraph)
+        fuse_reduce_epilogue(fgraph)
         gof.merge_identical(fgraph)
     return fgraph

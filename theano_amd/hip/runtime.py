@@ -61,8 +61,8 @@ def _load():
         "thx_elemwise_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, P(i32), P(vp)], ctypes.c_int),
         "thx_elemwise_call": ([vp, P(thx_array), P(thx_array), ctypes.c_int], ctypes.c_int),
         "thx_elemwise_free": ([vp], ctypes.c_int),
-        "thx_reduce_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, P(i32), ctypes.c_int, P(vp)],
-                           ctypes.c_int),
+        "thx_reduce_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, P(i32),
+                            ctypes.c_int, P(vp)], ctypes.c_int),
         "thx_reduce_call": ([vp, P(thx_array), P(ctypes.c_uint8), P(thx_array), ctypes.c_int], ctypes.c_int),
         "thx_reduce_free": ([vp], ctypes.c_int),
         "thx_rowchain_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, P(i32), P(i32), P(vp)],
