@@ -7,7 +7,8 @@
 //   template <int V> static void compute(Regs<V>&);     // the scalar graph, V times
 //   template <int V, class A> static void store(const A&, const Regs<V>&);
 // and a generated plan P supplies
-//   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK, NT (non-temporal accesses) };
+//   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK, NT (non-temporal accesses),
+//                                     GS (grid-stride loop over chunks) };
 //   static constexpr int mode(int operand);             // M_VEC / M_BCAST / M_GATHER
 // The host collapses dimensions, so ND is the rank after merging every pair of
 // neighbouring dimensions that all operands walk with compatible strides.
@@ -80,11 +81,12 @@ __device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename 
   typedef typename UnsignedOf<IT>::type UT;
   constexpr int VEC = P::VEC, UNR = P::UNR, ND = P::ND, NOPS = F::NOPS;
 
+  const long long step = P::GS ? (long long)gridDim.x * (P::BLOCK * UNR) : p.nvec + 1;
+  for (long long q0 = (long long)blockIdx.x * (P::BLOCK * UNR) + threadIdx.x;
+       q0 - threadIdx.x < p.nvec; q0 += step) {
   typename F::template Regs<VEC> r[UNR];
   EwAcc<P, NOPS> a[UNR];
   bool full[UNR];
-  const long long q0 = (long long)blockIdx.x * (P::BLOCK * UNR) + threadIdx.x;
-
 #pragma unroll
   for (int u = 0; u < UNR; ++u) {
     const long long q = q0 + (long long)u * P::BLOCK;
@@ -117,6 +119,7 @@ __device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename 
 #pragma unroll
   for (int u = 0; u < UNR; ++u)
     if (full[u]) F::template store<VEC>(a[u], r[u]);
+  }
 
   // ND == 1 only: the elements after the last whole vector, one per thread.
   if (ND == 1 && VEC > 1) {

@@ -47,9 +47,9 @@ struct CheckR {
   }
 };
 
-struct PlanEw1 { typedef int IT; enum { ND = 1, VEC = 4, UNR = 2, BLOCK = 256, NT = 1 };
+struct PlanEw1 { typedef int IT; enum { ND = 1, VEC = 4, UNR = 2, BLOCK = 256, NT = 1, GS = 1 };
   static constexpr int mode(int i) { constexpr int m[] = {0, 3, 0}; return m[i]; } };
-struct PlanEw3 { typedef long long IT; enum { ND = 3, VEC = 2, UNR = 1, BLOCK = 256, NT = 1 };
+struct PlanEw3 { typedef long long IT; enum { ND = 3, VEC = 2, UNR = 1, BLOCK = 256, NT = 1, GS = 0 };
   static constexpr int mode(int i) { constexpr int m[] = {2, 1, 0}; return m[i]; } };
 struct PlanRow { typedef int IT; enum { NK = 2, VEC = 4, UNR = 4, BLOCK = 256, TPR = 256, RA2 = 1, NT = 0 };
   static constexpr int mode(int i) { constexpr int m[] = {0}; return m[i]; } };

@@ -240,11 +240,11 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
       if (env_int("THX_EW_TV", 0) == 1) tv = 1;
       if ((int64_t)ntr * tile * (tile + 1) * esz <= 60000) {
         const int block = 256;
-        const int nt = env_int("THX_NT", 0);
+        const int nt = nt_choice(1);
         std::ostringstream key;
         key << "et|nd" << ND << "|t" << tile << "|v" << tv << "|n" << ntr << "|e" << esz << (nt ? "|nt" : "") << "|m";
         for (int o = 0; o < nops; ++o) key << (slot[o] >= 0 ? 9 : mode[o]) << (o + 1 < nops ? "," : "");
-        const std::string plan = key.str();
+        const std::string plan = key.str() + (fast_div() ? "|fd" : "");
         set_last_plan(e->name + "|" + plan);
         Kernel k;
         auto it = e->plans.find(plan);
@@ -300,13 +300,18 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   int unr = nvec >= (int64_t(1) << 20) ? 4 : (nvec >= (int64_t(1) << 18) ? 2 : 1);
   const int force_unr = env_int("THX_EW_UNR", 0);
   if (force_unr > 0) unr = force_unr;
-  const int block = 256;
-  const int nt = env_int("THX_NT", 0) && n * 4 >= (int64_t(1) << 24);
+  int block = 256;
+  const int force_block = env_int("THX_EW_BLOCK", 0);
+  if (force_block == 128 || force_block == 512 || force_block == 1024) block = force_block;
+  const int nt = nt_choice(0) && n * 4 >= (int64_t(1) << 24);
+  // grid-stride: a bounded number of blocks walk the index space instead of one block per chunk
+  const int gs = env_int("THX_EW_GS", 0);
 
   std::ostringstream key;
-  key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nt ? "|nt" : "") << "|m";
+  key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nt ? "|nt" : "") << (block != 256 ? "|b" + std::to_string(block) : "")
+      << (gs ? "|gs" : "") << "|m";
   for (int o = 0; o < nops; ++o) key << mode[o] << (o + 1 < nops ? "," : "");
-  const std::string plan = key.str();
+  const std::string plan = key.str() + (fast_div() ? "|fd" : "");
   set_last_plan(e->name + "|" + plan);
 
   Kernel k;
@@ -317,7 +322,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
     std::ostringstream s;
     s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
       << " IT;\n  enum { ND = " << ND << ", VEC = " << vec << ", UNR = " << unr << ", BLOCK = " << block
-      << ", NT = " << nt << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+      << ", NT = " << nt << ", GS = " << (gs ? 1 : 0) << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
     for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
     s << "};\n    return m[i];\n  }\n};\n"
       << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::EwParams<" << e->name
@@ -340,6 +345,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
 
   int64_t grid = (nvec + (int64_t)block * unr - 1) / ((int64_t)block * unr);
   if (grid < 1) grid = 1;
+  if (gs) grid = std::min<int64_t>(grid, (int64_t)(rt().ready ? rt().cus : 256) * gs);
   if (grid > 0x7fffffffLL) return fail(THX_ERR_UNSUPPORTED, "elemwise: %lld blocks exceed the grid limit", (long long)grid);
   return launch(k, e->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
 }

@@ -47,6 +47,10 @@ struct Kernel {
 // Compile (or fetch from the caches) `source`, which must define an
 // extern "C" __global__ function named `entry`.
 int get_kernel(const std::string& source, const std::string& entry, Kernel* out);
+// True (default; $THX_FAST_DIV=0 turns it off) when float32 division / sqrt are compiled to the 2.5-ulp forms.
+bool fast_div();
+// Non-temporal accesses: $THX_NT when set, else the default of the kernel family (measured per family).
+int nt_choice(int family_default);
 // The embedded device headers (thx_common.h, thx_elemwise.h, thx_reduce.h).
 const std::string& device_prelude();
 

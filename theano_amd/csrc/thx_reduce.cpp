@@ -251,12 +251,13 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   };
 
   const int block = 256;
-  const int nt = env_int("THX_NT", 0);
+  const int nt = nt_choice(0);
   std::string plan;
   Kernel k;
   ParamPack pk;
   int64_t grid = 0;
   int S = 1;
+  int launch_block = block;
 
   if (form == ROW) {
     const int64_t RC = NR ? RD.back().extent : 1;
@@ -293,10 +294,17 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     int unr = per_thread >= 4 ? 4 : per_thread >= 2 ? 2 : 1;
     const int force_unr = env_int("THX_RED_UNR", 0);
     if (force_unr > 0) unr = force_unr;
-    const int rpb = block / tpr;
+    // few outputs, long reduce domains: 1024 threads per output before resorting to a split
+    int rblock = block;
+    if (tpr == 256 && env_int("THX_RED_BIGBLOCK", 1) && ceil_div(n_out, 1) * 2 <= target_row * 4 &&
+        n_out >= cus / 2 && nvec >= 1024 * 8) {
+      rblock = 1024;
+      tpr = 1024;
+    }
+    const int rpb = rblock / tpr;
     const int64_t oblocks = ceil_div(n_out, rpb);
     int64_t chunk = nvec;
-    if (oblocks * 2 <= target_row && nvec >= (int64_t)tpr * unr * 4) {
+    if (rblock == 256 && oblocks * 2 <= target_row && nvec >= (int64_t)tpr * unr * 4) {
       int64_t want = std::min(ceil_div(target_row, oblocks), nvec / ((int64_t)tpr * unr * 2));
       if (want > 1) {
         chunk = round_up(ceil_div(nvec, want), (int64_t)tpr * unr);
@@ -308,15 +316,15 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     std::ostringstream key;
     key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|t" << tpr << "|a" << ra2 << (nt ? "|nt" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
-    plan = key.str();
+    plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
     if (it != r->plans.end() && (it->second.func || dry)) {
       k = it->second;
     } else {
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TPR", tpr}, {"RA2", ra2}, {"NT", nt}}, mode)
-        << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::RowParams<" << r->name
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"NT", nt}}, mode)
+        << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void thx_entry(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
       rc = get_kernel(s.str(), "thx_entry", &k);
@@ -345,6 +353,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     for (int i = 0; i < NIN; ++i) pk.put_index(wide, rc_stride[i]);
     pk.align(8);
     grid = oblocks * S;
+    launch_block = rblock;
   } else if (form == COL) {
     const int64_t C = KD.back().extent;
     const int ko = NKD - 1;  // outer kept dimensions
@@ -387,7 +396,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     int64_t A = 1;
     for (int d = 0; d < ko; ++d) A *= KD[d].extent;
     const int64_t per_lane = ceil_div(rows, ty);
-    int unr = per_lane >= 4 ? 4 : per_lane >= 2 ? 2 : 1;
+    int unr = per_lane >= 16 ? 8 : per_lane >= 4 ? 4 : per_lane >= 2 ? 2 : 1;
     const int force_unr = env_int("THX_RED_UNR", 0);
     if (force_unr > 0) unr = force_unr;
     const int64_t blocks0 = A * cblocks;
@@ -402,7 +411,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     std::ostringstream key;
     key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << "|r" << rr2 << (nt ? "|nt" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
-    plan = key.str();
+    plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
     if (it != r->plans.end() && (it->second.func || dry)) {
       k = it->second;
@@ -453,7 +462,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       if (views[i].imm) gmode[i] = M_IMM;
       key << gmode[i] << (i + 1 < NIN ? "," : "");
     }
-    plan = key.str();
+    plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
     if (it != r->plans.end() && (it->second.func || dry)) {
       k = it->second;
@@ -487,7 +496,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   set_last_plan(r->name + "|" + plan + (S > 1 ? "|s" + std::to_string(S) : ""));
   if (grid > 0x7fffffffLL) return fail(THX_ERR_UNSUPPORTED, "reduce: %lld blocks exceed the grid limit", (long long)grid);
   if (!dry) {
-    rc = launch(k, r->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
+    rc = launch(k, r->name + "|" + plan, (unsigned)grid, launch_block, pk.buf.data(), pk.buf.size());
     if (rc) return rc;
   }
   if (S > 1) return final_pass(r, outp, ex, rt().scratch, n_out, S, dry);

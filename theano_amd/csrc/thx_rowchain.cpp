@@ -191,12 +191,12 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
     if (span >= (int64_t(1) << 31) - 65536) wide = true;
   }
   const int block = 256;
-  const int nt = getenv("THX_NT") ? atoi(getenv("THX_NT")) : 0;
+  const int nt = nt_choice(1);
 
   std::ostringstream key;
   key << "rw|v" << vec << "|n" << nch << "|t" << tpr << (wide ? "|i64" : "|i32") << (nt ? "|nt" : "") << "|i";
   for (int i = 0; i < NIN; ++i) key << is_imm[i];
-  const std::string plan = key.str();
+  const std::string plan = key.str() + (fast_div() ? "|fd" : "");
   set_last_plan(c->name + "|" + plan);
   Kernel k;
   auto it = c->plans.find(plan);

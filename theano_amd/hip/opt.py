@@ -123,17 +123,21 @@ def _scalar_constant(var):
     return None
 
 
-_CHEAP_OPS = (scal.Cast, scal.Add, scal.Sub, scal.Mul, scal.Neg, scal.Sqr, scal.Abs, scal.Sgn, scal.Identity,
+_TRIVIAL_OPS = (scal.Cast, scal.Add, scal.Sub, scal.Mul, scal.Neg, scal.Sqr, scal.Abs, scal.Sgn, scal.Identity,
               scal.Second, scal.LogicalComparison, scal.Switch, scal.BinaryBitOp, scal.Invert, scal.Maximum,
               scal.Minimum, scal.Clip, scal.IsNan, scal.IsInf)
+# float32 division compiles to a few instructions (2.5-ulp form): cheap enough to recompute once per
+# consumer of a same-shaped value, not cheap enough to redo per element for a broadcast operand
+_CHEAP_OPS = _TRIVIAL_OPS + (scal.TrueDiv, scal.Inv)
 
 
-def _cheap(scalar_op):
+def _cheap(scalar_op, ops=None):
     """True when recomputing the op per consumer costs a few ALU instructions
-    (no division, no transcendental function)."""
+    (no transcendental function)."""
+    ops = ops or _CHEAP_OPS
     if isinstance(scalar_op, scal.Composite):
-        return all(isinstance(n.op, _CHEAP_OPS) for n in gof.io_toposort(scalar_op.inputs, scalar_op.outputs))
-    return isinstance(scalar_op, _CHEAP_OPS)
+        return all(isinstance(n.op, ops) for n in gof.io_toposort(scalar_op.inputs, scalar_op.outputs))
+    return isinstance(scalar_op, ops)
 
 
 def _absorbs(client, var):
@@ -178,7 +182,7 @@ def _fusable(fgraph, var, out_bcast):
     # a producer that is broadcast against the consumer (a per-channel cast, say) is recomputed per
     # element only when that costs next to nothing; the reference keeps such nodes apart
     # (theano/tensor/opt.py:7171-7175) because its C loops would redo real work
-    return (fgraph.n_clients(var) == 1 and _cheap(node.op.scalar_op) and
+    return (fgraph.n_clients(var) == 1 and _cheap(node.op.scalar_op, _TRIVIAL_OPS) and
             all(pb or not cb for pb, cb in zip(var.type.broadcastable, out_bcast)))
 
 
@@ -350,23 +354,35 @@ def fuse_reduce_epilogue(fgraph):
             rop = red.op
             if not isinstance(rop, HipCAReduce) or rop.post_scalar_op is not None or red not in fgraph.apply_nodes:
                 continue
-            cand = None
+            cands = []
             for r in red.outputs:
                 for c, _ in fgraph.clients.get(r, []):
                     if c == "output":
                         continue
                     if isinstance(c.op, HipDimShuffle):
                         for c2, _ in fgraph.clients.get(c.outputs[0], []):
-                            if c2 != "output" and isinstance(c2.op, HipElemwise):
-                                cand = c2
-                    elif isinstance(c.op, HipElemwise):
-                        cand = c
-                    if cand is not None:
-                        break
-                if cand is not None:
+                            if c2 != "output" and isinstance(c2.op, HipElemwise) and c2 not in cands:
+                                cands.append(c2)
+                    elif isinstance(c.op, HipElemwise) and c not in cands:
+                        cands.append(c)
+            done = False
+            for cand in cands:
+                if _try_epilogue(fgraph, red, cand):
+                    done = True
                     break
-            if cand is None or len(cand.outputs) != 1 or cand.op.inplace_pattern:
-                continue
+            if done:
+                count += 1
+                changed = True
+                break
+    return count
+
+
+def _try_epilogue(fgraph, red, cand):
+    rop = red.op
+    if True:
+        if True:
+            if len(cand.outputs) != 1 or cand.op.inplace_pattern:
+                return False
             # classify the consumer's inputs
             ds_op, ok, s_args, extras, s_extras = None, True, [], [], []
             s_acc = [scal.Scalar(dt)() for dt in rop.out_dtypes]
@@ -402,7 +418,7 @@ def fuse_reduce_epilogue(fgraph):
                     ok = False
                     break
             if not ok or not used or len(extras) > 8:
-                continue
+                return False
             e_out = cand.op.scalar_op(*s_args)
             # reduction results something else still needs stay outputs of the new node
             keep = []
@@ -429,14 +445,11 @@ def fuse_reduce_epilogue(fgraph):
             if ds_op is not None:
                 new_e = HipDimShuffle(ds_op.input_broadcastable, ds_op.new_order)(new_e)
             if new_e.type != cand.outputs[0].type:
-                continue
+                return False
             for j, k in enumerate(keep):
                 fgraph.replace(red.outputs[k], new_node.outputs[j])
             fgraph.replace(cand.outputs[0], new_e)
-            count += 1
-            changed = True
-            break
-    return count
+            return True
 
 
 def _depends_on(var, node, limit=10000):
