@@ -7,11 +7,16 @@ sum and max along axis 1, sum along axis 0, sum over all axes, prod along
 axis 1.  One step runs the five reductions once on device-resident inputs;
 ``value`` is their algorithmic bytes divided by the step time (HIP events on the
 library's stream around the K timed steps).  ``roofline`` describes the dominant
-kernel (the row-form reduction) from per-launch HIP events taken in a second
-run of the same K steps; ``cpu_baseline`` times the oracle's C restatement of
-the reference's sequential CAReduce loops on this host for the same five
-reductions.  ``other_configs`` lists the remaining four configurations,
-measured the same way with fewer steps.
+kernel, the row-form reduction behind ``sum(axis=1)``: K launches back to back
+between two HIP events on the launch stream, once alternating between two
+input arrays and once over one array.  The input is 268 MB and the device's
+last-level cache 256 MB, so a launch that follows one over the same array runs
+a few percent faster than one that follows a different array; a step holds one
+launch of each kind, and the average of the two loops divides the kernel's
+algorithmic bytes.  ``cpu_baseline`` times the oracle's C restatement of the
+reference's loops on this host.  ``other_configs`` lists the remaining four
+configurations over input sets that rotate (so that no set is still cached
+when it is used again: ``us``) and over one set (``same_input_us``).
 """
 import argparse
 import json
@@ -22,6 +27,13 @@ import time
 import numpy as np
 
 HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each
+# scaled by what the same counter reads for the --copy-probe kernel of known size), by kernel symbol.
+MEASURED_TRAFFIC = {
+    # sum(axis=1) of float32 (8192, 8192): FETCH_SIZE 131093.1 x 1.99972 KiB + WRITE_SIZE 262.0 KiB
+    "thx_rr_k1_i32_v4_u4_t256_a0_m0_fd_Ra004ded952553fcd": 268709122,
+}
 
 
 def _device_function(th, W, graph, vals):
@@ -45,11 +57,10 @@ def _time_steps(hip, step, steps, warmup):
     return gpu_ms / steps, wall_ms / steps
 
 
-def _profile_steps(hip, step, steps):
-    with hip.profile() as p:
-        for _ in range(steps):
-            step()
-    return p.kernels
+def _symbol(profile_name):
+    """Kernel symbol (what rocprofv3 lists) of a 'functor|plan' profile name."""
+    functor, plan = profile_name.split("|", 1)
+    return "thx_" + "".join(c if c.isalnum() else "_" for c in plan) + "_" + functor
 
 
 def _cpu_baseline_c2(W):
@@ -72,6 +83,20 @@ def _cpu_baseline_c2(W):
                       "are single-threaded in the reference" % dt}
 
 
+def _input_sets(vals, min_total=1 << 30, max_sets=8):
+    """Device copies of one input list, enough of them that cycling through them keeps any
+    one set from surviving in the 256 MB last-level cache between two uses."""
+    from theano_amd.hip import HipArray
+    nbytes = sum(v.nbytes for v in vals if v.size > 1)
+    n = int(min(max_sets, max(2, -(-min_total // max(nbytes, 1)))))
+    return [[HipArray.from_numpy(v) if v.size > 1 else v for v in vals] for _ in range(n)]
+
+
+def _rate(nbytes, ms):
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1), "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -79,6 +104,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the other four configurations")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also launch a plain streaming kernel (out = -x on the same (8192, 8192) float32 array, "
+                         "256 MiB read + 256 MiB written) K times: the known-size kernel that hardware counters "
+                         "of the reductions are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); got --gpus %d" % args.gpus)
@@ -92,6 +121,8 @@ def main():
     info = hip.device_info()
 
     # ---- headline: config 2 -----------------------------------------------------------------
+    # The four reductions of x share one device array and prod has its own, as the configuration
+    # states; a step runs them in the configuration's order.
     fns = []
     total_bytes = 0
     x_dev = {}
@@ -110,50 +141,83 @@ def main():
         for _, f, dev in fns:
             f(*dev)
 
+    if args.copy_probe:
+        from theano_amd import tensor as T
+        xs = T.fmatrix("x")
+        fcopy = th.function([xs], [th.Out(-xs, device=True)])
+        for _ in range(args.steps):
+            fcopy(*x_dev["normal"])
+        hip.sync()
+
     gpu_ms, wall_ms = _time_steps(hip, step, args.steps, args.warmup)
-    kernels = _profile_steps(hip, step, args.steps)
     value = total_bytes / (gpu_ms * 1e-3) / 1e9
 
-    # dominant kernel: the one with the largest share of the profiled time
-    dom = max(kernels.items(), key=lambda kv: kv[1][1])
-    dom_name, (dom_n, dom_ms) = dom
-    dom_avg_us = dom_ms / dom_n * 1e3
+    # Each reduction alone, K launches back to back between two events: over two arrays in turn
+    # (2 x 268 MB, so neither survives in the 256 MB last-level cache: "us") and over one array
+    # ("same_input_us").  A profile pass names the kernels of each reduction.
+    two = [x_dev["normal"], x_dev["prod"]]
+    per_case, case_kernels = {}, {}
+    for case, f, dev in fns:
+        turn = [0]
+
+        def rotating():
+            f(*two[turn[0] & 1])
+            turn[0] += 1
+
+        cold_ms, _ = _time_steps(hip, rotating, args.steps, 2)
+        warm_ms, _ = _time_steps(hip, lambda: f(*dev), args.steps, 2)
+        per_case[case] = _rate(W.algorithmic_bytes("c2_" + case), cold_ms)
+        per_case[case]["same_input_us"] = round(warm_ms * 1e3, 2)
+        with hip.profile() as p:
+            f(*dev)
+        case_kernels[case] = dict((_symbol(k), n) for k, (n, _) in p.kernels.items())
+        per_case[case]["kernels"] = sorted(case_kernels[case])
+
+    # Dominant kernel: the row-form reduction behind sum(axis=1).  In a step it runs once on an
+    # array that is not cached (after prod's input) and once on one that partly is (the first
+    # pass of sum over all axes, after sum(axis=0) of the same array), and the two loops above
+    # launch it K times each way, so the mean of the two is its average over the whole run.
+    dom = sorted(case_kernels["sum_axis1"])[0]
+    cold_us, warm_us = per_case["sum_axis1"]["us"], per_case["sum_axis1"]["same_input_us"]
+    dom_avg_us = 0.5 * (cold_us + warm_us)
     per_launch = 8192 * 8192 * 4 + 8192 * 4   # bytes one launch of a row / column reduction moves by definition
     achieved = per_launch / (dom_avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom_name,
-                "avg_launch_us": round(dom_avg_us, 2), "launches": dom_n}
-
-    per_case = {}
-    for case, f, dev in fns:
-        ms, _ = _time_steps(hip, lambda: f(*dev), max(5, args.steps // 2), 2)
-        b = W.algorithmic_bytes("c2_" + case)
-        per_case[case] = {"us": round(ms * 1e3, 2), "GB/s": round(b / (ms * 1e-3) / 1e9, 1),
-                          "frac_of_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(dom),
+                "kernel": dom, "avg_launch_us": round(dom_avg_us, 2), "uncached_input_us": cold_us,
+                "same_input_us": warm_us, "algorithmic_bytes_per_launch": per_launch}
 
     others = {}
     if not args.no_others:
-        specs = [("c1", W.c1_graph(), W.c1_inputs("full"), "c1"),
-                 ("c3_fwd", W.c3_graph(with_grad=False), W.c3_inputs("full", with_grad=False), "c3_fwd"),
-                 ("c3_fwd_grad", W.c3_graph(), W.c3_inputs("full"), "c3_fwd_grad"),
-                 ("c4_elemwise", W.c4_graph("elemwise"), W.c4_inputs("full"), "c4_elemwise"),
-                 ("c4_sum", W.c4_graph("sum"), W.c4_inputs("full"), "c4_sum"),
-                 ("c4_anyall", W.c4_graph("anyall"), W.c4_inputs("full", "anyall"), "c4_anyall"),
-                 ("c5_fwd", W.c5_graph(with_grad=False), W.c5_inputs("full", with_grad=False), "c5_fwd"),
-                 ("c5_grad", W.c5_graph(forward=False), W.c5_inputs("full"), "c5_grad")]
-        for name, graph, vals, bname in specs:
-            f, dev = _device_function(th, W, graph, vals)
-            ms, wms = _time_steps(hip, lambda: f(*dev), max(5, args.steps // 5), 2)
-            b = W.algorithmic_bytes(bname)
+        specs = [("c1", W.c1_graph(), W.c1_inputs("full")),
+                 ("c3_fwd", W.c3_graph(with_grad=False), W.c3_inputs("full", with_grad=False)),
+                 ("c3_fwd_grad", W.c3_graph(), W.c3_inputs("full")),
+                 ("c4_elemwise", W.c4_graph("elemwise"), W.c4_inputs("full")),
+                 ("c4_sum", W.c4_graph("sum"), W.c4_inputs("full")),
+                 ("c4_anyall", W.c4_graph("anyall"), W.c4_inputs("full", "anyall")),
+                 ("c5_fwd", W.c5_graph(with_grad=False), W.c5_inputs("full", with_grad=False)),
+                 ("c5_grad", W.c5_graph(forward=False), W.c5_inputs("full"))]
+        for name, (ins, outs), vals in specs:
+            f = th.function(ins, [th.Out(o, device=True) for o in outs])
+            sets = _input_sets(vals)
+            turn = [0]
+
+            def rotating():
+                f(*sets[turn[0] % len(sets)])
+                turn[0] += 1
+
+            ms, _ = _time_steps(hip, rotating, args.steps, 3)
+            warm_ms, _ = _time_steps(hip, lambda: f(*sets[0]), args.steps, 3)
             n_k = sum(1 for n in f.toposort() if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain"))
-            others[name] = {"us": round(ms * 1e3, 2), "GB/s": round(b / (ms * 1e-3) / 1e9, 1),
-                            "frac_of_peak": round(b / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "kernels_per_step": n_k}
-            del f, dev
+            others[name] = _rate(W.algorithmic_bytes(name), ms)
+            others[name].update({"input_sets": len(sets), "same_input_us": round(warm_ms * 1e3, 2),
+                                 "nodes_per_step": n_k})
+            del f, sets
 
     cpu = None if args.no_cpu else _cpu_baseline_c2(W)
 
     line = {
-        "metric": "achieved HBM GB/s for fused Elemwise+CAReduce at 1 MI355X",
+        "metric": "achieved HBM GB/s and % of peak for fused Elemwise+CAReduce at 1 MI355X",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(gpu_ms, 5), "wall_ms_per_step": round(wall_ms, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32 data, f64 accumulators", "data": "synthetic",
@@ -163,7 +227,6 @@ def main():
                    "algorithmic_bytes_per_step": total_bytes, "device": info["arch"],
                    "compute_units": info["compute_units"]},
         "roofline": roofline, "cpu_baseline": cpu, "per_reduction": per_case, "other_configs": others,
-        "kernels": {k: {"launches": n, "avg_us": round(ms / n * 1e3, 2)} for k, (n, ms) in kernels.items()},
     }
     print(json.dumps(line))
 

@@ -251,6 +251,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
         if (it != e->plans.end() && (it->second.func || dry)) {
           k = it->second;
         } else {
+          const std::string entry = entry_name(e->name, plan);
           std::ostringstream s;
           s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef int IT;\n  enum { ND = " << ND
             << ", TILE = " << tile << ", TV = " << tv << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz << ", NT = " << nt
@@ -259,9 +260,9 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
           s << "};\n    return m[i];\n  }\n  static constexpr int slot(int i) {\n    constexpr int m[] = {";
           for (int o = 0; o < nops; ++o) s << slot[o] << (o + 1 < nops ? ", " : "");
           s << "};\n    return m[i];\n  }\n};\n"
-            << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::EwTrParams<" << e->name
+            << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::EwTrParams<" << e->name
             << "::NOPS, ThxPlan::ND, ThxPlan::IT> p) {\n  thx::ew_tr_body<" << e->name << ", ThxPlan>(p);\n}\n";
-          rc = get_kernel(s.str(), "thx_entry", &k);
+          rc = get_kernel(s.str(), entry, &k);
           if (rc) return rc;
           e->plans[plan] = k;
         }
@@ -319,15 +320,16 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   if (it != e->plans.end() && (it->second.func || dry)) {
     k = it->second;
   } else {
+    const std::string entry = entry_name(e->name, plan);
     std::ostringstream s;
     s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
       << " IT;\n  enum { ND = " << ND << ", VEC = " << vec << ", UNR = " << unr << ", BLOCK = " << block
       << ", NT = " << nt << ", GS = " << (gs ? 1 : 0) << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
     for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
     s << "};\n    return m[i];\n  }\n};\n"
-      << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::EwParams<" << e->name
+      << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::EwParams<" << e->name
       << "::NOPS, ThxPlan::ND, ThxPlan::IT> p) {\n  thx::ew_body<" << e->name << ", ThxPlan>(p);\n}\n";
-    rc = get_kernel(s.str(), "thx_entry", &k);
+    rc = get_kernel(s.str(), entry, &k);
     if (rc) return rc;
     e->plans[plan] = k;
   }

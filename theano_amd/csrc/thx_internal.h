@@ -54,6 +54,10 @@ int nt_choice(int family_default);
 // The embedded device headers (thx_common.h, thx_elemwise.h, thx_reduce.h).
 const std::string& device_prelude();
 
+// Kernel symbol for a plan: "thx_" + plan with punctuation folded to '_' + "_" + functor, so that
+// profilers show one line per (functor, plan) instead of a shared entry name.
+std::string entry_name(const std::string& functor, const std::string& plan);
+
 // Launch with one by-value parameter block.
 int launch(const Kernel& k, const std::string& plan, unsigned grid, unsigned block,
            const void* params, size_t params_bytes);

@@ -72,10 +72,11 @@ static int final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::
   if (it != r->plans.end() && (it->second.func || dry)) {
     k = it->second;
   } else {
+    const std::string entry = entry_name(r->name, plan);
     std::ostringstream s;
-    s << device_prelude() << r->src << "\nextern \"C\" __global__ __launch_bounds__(256) void thx_entry(thx::FinalParams<"
+    s << device_prelude() << r->src << "\nextern \"C\" __global__ __launch_bounds__(256) void " << entry << "(thx::FinalParams<"
       << r->name << "::NOUT, " << r->name << "::NEX> p) {\n  thx::red_final_body<" << r->name << ", 256, " << tpo << ">(p);\n}\n";
-    int rc = get_kernel(s.str(), "thx_entry", &k);
+    int rc = get_kernel(s.str(), entry, &k);
     if (rc) return rc;
     r->plans[plan] = k;
   }
@@ -321,13 +322,14 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     if (it != r->plans.end() && (it->second.func || dry)) {
       k = it->second;
     } else {
+      const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
         << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"NT", nt}}, mode)
-        << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void thx_entry(thx::RowParams<" << r->name
+        << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void " << entry << "(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
-      rc = get_kernel(s.str(), "thx_entry", &k);
+      rc = get_kernel(s.str(), entry, &k);
       if (rc) return rc;
       r->plans[plan] = k;
     }
@@ -416,13 +418,14 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     if (it != r->plans.end() && (it->second.func || dry)) {
       k = it->second;
     } else {
+      const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
         << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TX", tx}, {"RR2", rr2}, {"NT", nt}}, mode)
-        << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::ColParams<" << r->name
+        << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::ColParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_col_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
-      rc = get_kernel(s.str(), "thx_entry", &k);
+      rc = get_kernel(s.str(), entry, &k);
       if (rc) return rc;
       r->plans[plan] = k;
     }
@@ -467,13 +470,14 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     if (it != r->plans.end() && (it->second.func || dry)) {
       k = it->second;
     } else {
+      const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
         << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}, {"NT", 0}}, gmode)
-        << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::GenParams<" << r->name
+        << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::GenParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::NR, ThxPlan::IT> p) {\n  thx::red_gen_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
-      rc = get_kernel(s.str(), "thx_entry", &k);
+      rc = get_kernel(s.str(), entry, &k);
       if (rc) return rc;
       r->plans[plan] = k;
     }

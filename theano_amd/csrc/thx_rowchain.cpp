@@ -203,15 +203,16 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
   if (it != c->plans.end() && (it->second.func || dry)) {
     k = it->second;
   } else {
+    const std::string entry = entry_name(c->name, plan);
     std::ostringstream s;
     s << device_prelude() << c->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
       << " IT;\n  enum { VEC = " << vec << ", NCH = " << nch << ", TPR = " << tpr << ", BLOCK = " << block
       << ", NT = " << nt << " };\n  static constexpr int imm(int i) {\n    constexpr int m[] = {";
     for (int i = 0; i < NIN; ++i) s << is_imm[i] << (i + 1 < NIN ? ", " : "");
     s << "};\n    return m[i];\n  }\n};\n"
-      << "extern \"C\" __global__ __launch_bounds__(" << block << ") void thx_entry(thx::RowChainParams<" << c->name
+      << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::RowChainParams<" << c->name
       << "::NIN, " << c->name << "::NOUT, ThxPlan::IT> p) {\n  thx::rowchain_body<" << c->name << ", ThxPlan>(p);\n}\n";
-    int rc = get_kernel(s.str(), "thx_entry", &k);
+    int rc = get_kernel(s.str(), entry, &k);
     if (rc) return rc;
     c->plans[plan] = k;
   }

@@ -9,6 +9,7 @@ definition of each op here exactly as the C snippets are in the reference.
 float16 values are computed in float32 (what ``Compositef32``
 :4130-4208 arranges for the reference's device code).
 """
+import hashlib
 import math
 
 import numpy as np
@@ -1210,8 +1211,12 @@ class Composite(ScalarOp):
         return Apply(op, inputs, [t() for t in op.outputs_type])
 
     def c_code(self, node, inputs, outputs):
-        # unique temporary prefix per use so that nested emission cannot clash
-        return "{\n" + self.body(list(inputs), list(outputs), prefix="c%x_" % (id(node) & 0xfffff)) + "\n}"
+        # The temporaries' prefix is a digest of the operand names: the same in every process, so
+        # that the text (and the kernel cache key made from it) is reproducible, and different
+        # between an outer Composite and one emitted inside it, whose operands are the outer's
+        # temporaries.
+        tag = hashlib.sha1(",".join(list(inputs) + list(outputs)).encode()).hexdigest()[:6]
+        return "{\n" + self.body(list(inputs), list(outputs), prefix="c%s_" % tag) + "\n}"
 
     def L_op(self, inputs, outputs, gout):
         raise NotImplementedError("grad is not implemented for Composite")
