@@ -83,6 +83,26 @@ def _cpu_baseline_c2(W):
                       "are single-threaded in the reference" % dt}
 
 
+def _cpu_baseline_other(name, vals, nbytes):
+    """One pass of the reference's host loops for another configuration
+    (oracle/cpu_backend.c) over the full-size inputs; the forward graphs only."""
+    from oracle import cpu_backend as B
+    from oracle import graph_ref as G
+    out = {}
+    kinds = {"c3_fwd": ("c3_fwd", "c3_fwd_rowloop")}.get(name, (name,))
+    for kind in kinds:
+        try:
+            _, seconds = B.run(kind, vals)
+        except KeyError:
+            return None
+        label = {"c3_fwd": "Elemwise/CAReduce chain", "c3_fwd_rowloop": "Softmax op row loop"}.get(kind, "node chain")
+        serial_only = kind in ("c3_fwd_rowloop",)
+        out[label] = {"value": round(nbytes / seconds / 1e9, 3), "unit": "GB/s", "seconds": round(seconds, 4),
+                      "cores": 1 if serial_only else int(G.lib().cpu_omp_threads()),
+                      "note": "serial loop" if serial_only else "OpenMP Elemwise nodes, serial CAReduce nodes"}
+    return out
+
+
 def _input_sets(vals, min_total=1 << 30, max_sets=8):
     """Device copies of one input list, enough of them that cycling through them keeps any
     one set from surviving in the 256 MB last-level cache between two uses."""
@@ -206,13 +226,19 @@ def main():
                 f(*sets[turn[0] % len(sets)])
                 turn[0] += 1
 
-            ms, _ = _time_steps(hip, rotating, args.steps, 3)
-            warm_ms, _ = _time_steps(hip, lambda: f(*sets[0]), args.steps, 3)
+            # the best of three runs of K steps: these kernels are short enough for one slow
+            # start of the host loop to show in a single run
+            ms = min(_time_steps(hip, rotating, args.steps, 3)[0] for _ in range(3))
+            warm_ms = min(_time_steps(hip, lambda: f(*sets[0]), args.steps, 3)[0] for _ in range(3))
             n_k = sum(1 for n in f.toposort() if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain"))
             others[name] = _rate(W.algorithmic_bytes(name), ms)
             others[name].update({"input_sets": len(sets), "same_input_us": round(warm_ms * 1e3, 2),
                                  "nodes_per_step": n_k})
             del f, sets
+            if not args.no_cpu:
+                cpu_o = _cpu_baseline_other(name, vals, W.algorithmic_bytes(name))
+                if cpu_o:
+                    others[name]["cpu_baseline"] = cpu_o
 
     cpu = None if args.no_cpu else _cpu_baseline_c2(W)
 

@@ -110,6 +110,9 @@ int thx_elemwise_new(const char* functor_src, const char* functor_name, int n_in
 #define THX_BROADCAST 1 /* size-1 input dimensions broadcast against larger ones */
 #define THX_DRY_RUN 2   /* validate, plan and compile (into the disk cache) but do not launch;
                            needs no device: the target is $THX_ARCH, default gfx950 */
+#define THX_KEEP_CACHED 4 /* an operand of this call is read again by one of the next calls (or its
+                           result is): no non-temporal accesses, so that the 256 MB last-level
+                           cache can serve the second read */
 
 /* Run on `ins` (n_in arrays) writing `outs` (n_out arrays, preallocated, every
  * one of the full result shape; an output may alias an input exactly for
@@ -126,8 +129,8 @@ typedef struct thx_reduce thx_reduce;
 /* Create a (multi-)reduction from generated device source defining a functor
  * named `functor_name` (contract in kernels/thx_reduce.h): n_in inputs feed a
  * fused prologue, n_out results of identical shape leave a fused epilogue that
- * may also read n_extra host scalars (e.g. the divisor of a mean). dtypes lists
- * inputs, outputs, then those scalars. acc_bytes = sizeof of the functor's
+ * may also read n_extra further operands (e.g. the divisor of a mean, a
+ * per-channel scale). dtypes lists inputs, outputs, then those operands. acc_bytes = sizeof of the functor's
  * accumulator struct.
  * Replaces the kernel generation of GpuCAReduceCuda
  * (theano/gpuarray/elemwise.py:1756-2420). */
@@ -136,8 +139,9 @@ int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, 
 
 /* Reduce the dimensions d with reduce_mask[d] != 0. `ins` holds the n_in reduced
  * inputs, which all have rank nd and broadcast against each other like Elemwise
- * inputs, followed by the n_extra THX_HOST_SCALAR operands of the epilogue; `outs` are C-contiguous
- * arrays of the kept dimensions, in order. A zero-length reduce domain yields
+ * inputs, followed by the n_extra operands of the epilogue: each either a THX_HOST_SCALAR or a
+ * C-contiguous device array with one element per result, read at the result's index; `outs` are
+ * C-contiguous arrays of the kept dimensions, in order. A zero-length reduce domain yields
  * the identity (the caller rejects it for max/min, as
  * theano/tensor/elemwise.py:1489-1506 does). Asynchronous.
  * Replaces the c_code_reduce_* launch routines (theano/gpuarray/elemwise.py:1095-1723). */

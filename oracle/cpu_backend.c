@@ -237,3 +237,16 @@ void cpu_c5_fwd(const uint16_t* x, const uint16_t* gamma, const uint16_t* beta, 
       }
     }
 }
+
+/* the two conversions over arrays, for the test that compares them with NumPy's */
+void cpu_h2f_array(const uint16_t* h, float* f, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) f[i] = h2f(h[i]);
+}
+
+void cpu_f2h_array(const float* f, uint16_t* h, int64_t n) {
+  for (int64_t i = 0; i < n; ++i) h[i] = f2h(f[i]);
+}
+
+/* threads an OpenMP region of this library runs with (OMP_NUM_THREADS or the core count) */
+#include <omp.h>
+int cpu_omp_threads(void) { return omp_get_max_threads(); }

@@ -153,3 +153,62 @@ def test_device_outputs_and_inputs(dry_run):
     assert isinstance(out, HipArray) and out.shape == (3, 4)
     out2 = f(out)  # a device array is accepted for a host-typed input
     assert isinstance(out2, HipArray)
+
+
+def test_factors_constant_along_the_reduced_axes_leave_the_sum():
+    """sum(c * x / d, axis) with c, d broadcast along the reduced axes becomes
+    (c / d)' * sum(x, axis): one plain sum instead of a product per element, and
+    the same values as the unrewritten graph within float32 rounding."""
+    from theano_amd import gof
+    from theano_amd.tensor import opt as topt
+    from oracle import graph_ref as G
+    t4 = T.TensorType("float32", (False,) * 4)
+    pc = T.TensorType("float32", (True, False, True, True))
+    x, g = t4("x"), t4("g")
+    gamma, std = pc("gamma"), pc("std")
+    outs = [T.sum(-(g * (gamma * x)) / (std * std), axis=(0, 2, 3)),
+            T.sum((g / std) * x, axis=(0, 2, 3), keepdims=True),
+            T.sum(g * x, axis=(0, 2, 3))]                      # nothing to pull out: left alone
+    rng = np.random.default_rng(5)
+    vals = [rng.standard_normal((5, 7, 3, 4)).astype("float32"), rng.standard_normal((5, 7, 3, 4)).astype("float32"),
+            rng.uniform(0.5, 2, (1, 7, 1, 1)).astype("float32"), rng.uniform(0.5, 2, (1, 7, 1, 1)).astype("float32")]
+    ref = G.evaluate([x, g, gamma, std], outs, vals)
+    fg = gof.FunctionGraph([x, g, gamma, std], outs)
+    topt.canonicalize(fg)
+    sums = [n for n in fg.toposort() if isinstance(n.op, Sum)]
+    for n in sums:                                                # every remaining sum reads g * x only
+        (prod,) = n.inputs
+        assert isinstance(prod.owner.op, Elemwise) and isinstance(prod.owner.op.scalar_op, scal.Mul)
+        assert set(prod.owner.inputs) == {fg.inputs[0], fg.inputs[1]}
+    got = G.evaluate(fg.inputs, fg.outputs, vals)
+    for a, b in zip(got, ref):
+        assert a.shape == b.shape and a.dtype == b.dtype
+        np.testing.assert_allclose(a, b, rtol=1e-5, atol=1e-6)
+    # integer sums are left alone: the int64 sum of an int32 product wraps differently from the product of sums
+    xi = T.imatrix("xi")
+    ci = T.TensorType("int32", (False, True))("ci")
+    fg = gof.FunctionGraph([xi, ci], [T.sum(xi * ci, axis=1)])
+    topt.canonicalize(fg)
+    (n,) = [n for n in fg.toposort() if isinstance(n.op, Sum)]
+    assert isinstance(n.inputs[0].owner.op.scalar_op, scal.Mul)
+
+
+def test_batchnorm_gradient_is_two_statistics_passes_and_one_elementwise_pass(dry_run):
+    """Configuration 5's gradient graph: per-channel factors leave the sums, the
+    sums that then read the same tensors merge, and the per-channel algebra
+    between them runs in the second reduction's epilogue, which reads gamma as a
+    per-result device operand.  Three kernels remain; the first two are told to
+    leave their inputs in the last-level cache for the ones after them."""
+    import workloads
+    ins, outs = workloads.c5_graph(forward=False)
+    f = th.function(ins, [th.Out(o, device=True) for o in outs])
+    kernels = [n for n in f.toposort() if isinstance(n.op, (HipElemwise, HipCAReduce)) and
+               any(not any(i.type.broadcastable) for i in n.inputs if hasattr(i.type, "broadcastable") and i.type.ndim)]
+    assert [type(n.op) for n in kernels] == [HipCAReduce, HipCAReduce, HipElemwise]
+    second = kernels[1]
+    assert len(second.op.scalar_ops) == 4 and second.op.n_extra >= 4
+    extras = second.inputs[len(second.inputs) - second.op.n_extra:]
+    assert any(type(e.type).__name__ == "HipArrayType" for e in extras)
+    assert [bool(n.tag.get("keep_cached")) for n in kernels] == [True, True, False]
+    small = workloads.c5_inputs("small")
+    f(*small)                                      # plans and compiles every kernel (dry run)

@@ -197,3 +197,60 @@ def test_batchnorm_gradient_closed_form():
     dscale = (dyv * xmu * invstd).sum(axes, keepdims=True)
     dx = gv * invstd * (dyv - dyv.mean(axes, keepdims=True) - xmu * invstd ** 2 * (dyv * xmu).mean(axes, keepdims=True))
     assert np.allclose(ag, dscale, rtol=1e-9) and np.allclose(ax, dx, rtol=1e-8, atol=1e-10)
+
+
+@pytest.mark.parametrize("name", ["c1", "c3_fwd", "c3_fwd_rowloop", "c4_elemwise", "c4_sum", "c4_anyall", "c5_fwd"])
+def test_cpu_backend_matches_graph_oracle(name):
+    """The hand-restated host loops of the benchmark configurations (the CPU
+    baseline) give what the node-by-node evaluation of the same graph gives:
+    integers bit for bit, floats to the accumulation-order tolerance."""
+    import workloads as W
+    from oracle import cpu_backend as B
+    graph, vals = {
+        "c1": lambda: (W.c1_graph(), W.c1_inputs("small")),
+        "c3_fwd": lambda: (W.c3_graph(with_grad=False), W.c3_inputs("small", False)),
+        "c3_fwd_rowloop": lambda: (W.c3_graph(with_grad=False), W.c3_inputs("small", False)),
+        "c4_elemwise": lambda: (W.c4_graph("elemwise"), W.c4_inputs("small")),
+        "c4_sum": lambda: (W.c4_graph("sum"), W.c4_inputs("small")),
+        "c4_anyall": lambda: (W.c4_graph("anyall"), W.c4_inputs("small", "anyall")),
+        "c5_fwd": lambda: (W.c5_graph(with_grad=False), W.c5_inputs("small", False)),
+    }[name]()
+    ref = G.evaluate(graph[0], graph[1], vals)
+    got, seconds = B.run(name, vals)
+    assert seconds >= 0 and len(got) == len(ref)
+    for g, r in zip(got, ref):
+        assert g.dtype == r.dtype and g.shape == r.shape
+        if r.dtype.kind in "iub":
+            np.testing.assert_array_equal(g, r)
+        elif r.dtype == np.float16:
+            np.testing.assert_allclose(g.astype("float32"), r.astype("float32"), rtol=2e-3, atol=2e-3)
+        else:
+            np.testing.assert_allclose(g, r, rtol=1e-5, atol=1e-6)
+
+
+def test_cpu_backend_half_conversions_match_numpy():
+    """The bit-level float16 conversions of the CPU loops agree with NumPy's:
+    every half bit pattern to float32, and float32 to half on all exact halves,
+    all midpoints between neighbouring halves (ties to even), values just beside
+    the midpoints, subnormals, overflow and NaN."""
+    import ctypes
+    L = G.lib()
+    bits = np.arange(65536, dtype=np.uint16)
+    f = np.empty(65536, np.float32)
+    L.cpu_h2f_array(bits.ctypes.data_as(ctypes.c_void_p), f.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(65536))
+    ref = bits.view(np.float16).astype(np.float32)
+    assert np.array_equal(f.view(np.uint32), ref.view(np.uint32))
+    pos = bits[bits < 0x7c00].view(np.float16).astype(np.float64)
+    mid = (pos[:-1] + pos[1:]) / 2                      # exact in float32: 11 + 1 significant bits
+    samples = np.concatenate([pos, mid, np.nextafter(mid.astype(np.float32), np.float32(0)),
+                              np.nextafter(mid.astype(np.float32), np.float32(1e9)),
+                              [65504.0, 65519.9, 65520.0, 65536.0, 1e9, np.inf, 1e-9, 2.9e-8, 2.99e-8, 3.0e-8, 6e-8]])
+    x = np.concatenate([samples, -samples]).astype(np.float32)
+    h = np.empty(x.size, np.uint16)
+    L.cpu_f2h_array(x.ctypes.data_as(ctypes.c_void_p), h.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(x.size))
+    with np.errstate(over="ignore"):
+        assert np.array_equal(h, x.astype(np.float16).view(np.uint16))
+    nan = np.array([np.nan], np.float32)
+    hn = np.empty(1, np.uint16)
+    L.cpu_f2h_array(nan.ctypes.data_as(ctypes.c_void_p), hn.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(1))
+    assert np.isnan(hn.view(np.float16)[0])

@@ -80,6 +80,30 @@ class Function(object):
         self.nodes = fgraph.toposort()
         self._prepare()
 
+    def _mark_reuse(self):
+        """``node.tag['keep_cached']`` for every kernel node that reads a full-sized array which a
+        later kernel of this function reads again, or whose result a later kernel reads: those
+        calls must not use non-temporal accesses, the later read can then come from the
+        last-level cache (a batch-norm pass over 100 MB of activations after the statistics
+        pass, for instance)."""
+        from .hip.ops import HipArrayType, HipDimShuffle
+
+        def root(v):
+            while v.owner is not None and isinstance(v.owner.op, HipDimShuffle):
+                v = v.owner.inputs[0]
+            return v
+
+        def big(v):
+            return isinstance(v.type, HipArrayType) and v.type.ndim > 0 and not any(v.type.broadcastable)
+
+        kernels = [n for n in self.nodes if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain")]
+        later = set()
+        for node in reversed(kernels):
+            mine = set(id(root(i)) for i in node.inputs if big(i))
+            outs = set(id(o) for o in node.outputs if big(o))
+            node.tag["keep_cached"] = bool((mine | outs) & later)
+            later |= mine
+
     def _prepare(self):
         from .hip.opt import DeviceConstant
         from .hip.runtime import HipArray
@@ -127,6 +151,7 @@ class Function(object):
             for o in node.outputs:
                 if id(o) not in last and id(o) not in keep:
                     self.release[k].append(self.storage[o])
+        self._mark_reuse()
         self.thunks = []
         for node in self.nodes:
             node.op.prepare_node(node)

@@ -2,7 +2,7 @@
 // fused per-result epilogue.
 //
 // A generated functor R supplies
-//   enum { NIN, NOUT, NEX };                             // NEX host scalars feed the epilogue
+//   enum { NIN, NOUT, NEX };                             // NEX further operands feed the epilogue
 //   struct Acc;                                          // one field per reduction
 //   template <int V> struct Regs;                        // one Vec per input
 //   static void init(Acc&);                              // identities
@@ -21,7 +21,8 @@
 
 namespace thx {
 
-// Where results go, plus the values of the host scalars the epilogue uses.
+// Where results go, plus the epilogue's further operands: the value of a host scalar, or the
+// address of a device array that holds one element per result.
 template <int NOUT, int NEX>
 struct RedOut {
   char* ptr[NOUT];

@@ -189,6 +189,11 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   };
   while (!vec_ok(vec)) vec /= 2;
 
+  // bytes the kernel moves: every operand that is not broadcast along the innermost dimension
+  int64_t moved = 0;
+  for (int o = 0; o < nops; ++o)
+    if (mode[o] == M_VEC || mode[o] == M_GATHER) moved += n * dtype_size(views[o].dtype);
+
   // permuted-read plan: inputs that are unit-stride along another dimension T go through LDS tiles
   if (ND >= 2 && !wide && !env_int("THX_EW_NO_TRANSPOSE", 0)) {
     bool any_gather = false, outs_ok = true;
@@ -240,7 +245,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
       if (env_int("THX_EW_TV", 0) == 1) tv = 1;
       if ((int64_t)ntr * tile * (tile + 1) * esz <= 60000) {
         const int block = 256;
-        const int nt = nt_choice(1);
+        const int nt = nt_streaming(moved, flags);
         std::ostringstream key;
         key << "et|nd" << ND << "|t" << tile << "|v" << tv << "|n" << ntr << "|e" << esz << (nt ? "|nt" : "") << "|m";
         for (int o = 0; o < nops; ++o) key << (slot[o] >= 0 ? 9 : mode[o]) << (o + 1 < nops ? "," : "");
@@ -298,13 +303,15 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   }
 
   const int64_t nvec = ND == 1 ? n / vec : n / vec;
-  int unr = nvec >= (int64_t(1) << 20) ? 4 : (nvec >= (int64_t(1) << 18) ? 2 : 1);
+  // One vector per operand and thread: measured with inputs that are not cached, a larger unroll
+  // never gains and costs registers (a seven-input float16 kernel needs 164 VGPRs at 4).
+  int unr = 1;
   const int force_unr = env_int("THX_EW_UNR", 0);
   if (force_unr > 0) unr = force_unr;
   int block = 256;
   const int force_block = env_int("THX_EW_BLOCK", 0);
   if (force_block == 128 || force_block == 512 || force_block == 1024) block = force_block;
-  const int nt = nt_choice(0) && n * 4 >= (int64_t(1) << 24);
+  const int nt = nt_streaming(moved, flags);
   // grid-stride: a bounded number of blocks walk the index space instead of one block per chunk
   const int gs = env_int("THX_EW_GS", 0);
 

@@ -137,16 +137,6 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   int rc = gather_inputs("reduce", ins, NIN, r->dtypes.data(), flags, &nd, shape, &views);
   if (rc) return rc;
   if (nd > 0 && !reduce_mask) return fail(THX_ERR_ARG, "thx_reduce_call: null mask");
-  // host scalars of the epilogue follow the reduced inputs
-  std::vector<uint64_t> ex(std::max(1, r->n_extra), 0);
-  for (int j = 0; j < r->n_extra; ++j) {
-    const thx_array& a = ins[NIN + j];
-    const int want = r->dtypes[NIN + NOUT + j];
-    if (!(a.dtype & THX_HOST_SCALAR) || (a.dtype & ~THX_HOST_SCALAR) != want)
-      return fail(THX_ERR_TYPE, "reduce: epilogue operand %d must be a host scalar of dtype code %d", j, want);
-    memcpy(&ex[j], (const char*)a.base + a.offset_bytes, (size_t)dtype_size(want));
-  }
-
   // outputs: C-contiguous arrays of the kept dimensions
   int64_t kshape[THX_MAX_ND];
   int nk_full = 0;
@@ -178,6 +168,35 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     }
     outp[o] = (char*)a.base + a.offset_bytes;
     if (((uintptr_t)outp[o]) % isz) return fail(THX_ERR_TYPE, "reduce: output %d is not aligned to its element size", o);
+  }
+  // Operands of the epilogue follow the reduced inputs: a host scalar is passed by value; a device
+  // array holds one value per result (the results' element count, C-contiguous) and is passed by
+  // address, the epilogue reads it at the result's index.
+  std::vector<uint64_t> ex(std::max(1, r->n_extra), 0);
+  for (int j = 0; j < r->n_extra; ++j) {
+    const thx_array& a = ins[NIN + j];
+    const int want = r->dtypes[NIN + NOUT + j];
+    if ((a.dtype & ~THX_HOST_SCALAR) != want)
+      return fail(THX_ERR_TYPE, "reduce: epilogue operand %d has dtype code %d, the operation was built for %d", j,
+                  a.dtype & ~THX_HOST_SCALAR, want);
+    const char* p = (const char*)a.base + a.offset_bytes;
+    if (a.dtype & THX_HOST_SCALAR) {
+      memcpy(&ex[j], p, (size_t)dtype_size(want));
+      continue;
+    }
+    int64_t count = 1, expect = dtype_size(want);
+    for (int d = a.nd - 1; d >= 0; --d) {
+      if (a.shape[d] > 1 && a.strides_bytes[d] != expect)
+        return fail(THX_ERR_TYPE, "reduce: epilogue operand %d is not C-contiguous", j);
+      expect *= a.shape[d];
+      count *= a.shape[d];
+    }
+    if (count != n_out)
+      return fail(THX_ERR_SHAPE, "Input dimension mis-match. (epilogue operand %d has %lld elements, the result has %lld)",
+                  j, (long long)count, (long long)n_out);
+    if (((uintptr_t)p) % dtype_size(want))
+      return fail(THX_ERR_TYPE, "reduce: epilogue operand %d is not aligned to its element size", j);
+    ex[j] = (uint64_t)(uintptr_t)p;
   }
   if (n_out == 0) {
     set_last_plan("red|empty");
@@ -252,7 +271,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   };
 
   const int block = 256;
-  const int nt = nt_choice(0);
+  const int nt = nt_choice(1, flags);  // a reduction reads its input once
   std::string plan;
   Kernel k;
   ParamPack pk;

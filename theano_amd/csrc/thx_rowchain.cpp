@@ -191,7 +191,10 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
     if (span >= (int64_t(1) << 31) - 65536) wide = true;
   }
   const int block = 256;
-  const int nt = nt_choice(1);
+  int64_t moved = 0;
+  for (int i = 0; i < NOPS; ++i)
+    if (c->kinds[i] == K_FULL) moved += rows * C * dtype_size(c->dtypes[i]);
+  const int nt = nt_streaming(moved, flags);
 
   std::ostringstream key;
   key << "rw|v" << vec << "|n" << nch << "|t" << tpr << (wide ? "|i64" : "|i32") << (nt ? "|nt" : "") << "|i";

@@ -209,10 +209,14 @@ bool fast_div() {
   return env ? atoi(env) != 0 : true;
 }
 
-int nt_choice(int family_default) {
+int nt_choice(int family_default, int flags) {
   const char* env = getenv("THX_NT");
-  return env ? (atoi(env) != 0) : family_default;
+  if (env) return atoi(env) != 0;
+  if (flags & THX_KEEP_CACHED) return 0;
+  return family_default;
 }
+
+int nt_streaming(int64_t moved, int flags) { return nt_choice(moved >= (int64_t(288) << 20), flags); }
 
 static uint64_t fnv1a(const std::string& s, uint64_t h) {
   for (unsigned char c : s) {

@@ -97,15 +97,17 @@ def acc_struct_bytes(acc_dtypes):
 
 
 def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, post_op=None, extra_dtypes=(),
-                   post_in_dtypes=None):
+                   post_in_dtypes=None, extra_is_array=None):
     """(source, name, sizeof(Acc)) for K simultaneous reductions.
 
     Per element, ``pre_op`` (nin = len(in_dtypes), nout = K; default: the single
     input itself) yields K values, each cast to its accumulator dtype and
     folded with ``scalar_ops[k]``.  ``post_op`` (nin = K + len(extra_dtypes))
     maps the K results, each first cast to ``post_in_dtypes`` (the dtype the
-    unfused reduction would have produced), and the extra host scalars to the
-    outputs; the default casts result k to ``out_dtypes[k]``."""
+    unfused reduction would have produced), and the extra operands (a host
+    scalar's value, or where ``extra_is_array[j]`` the element of a device array
+    at the result's index) to the outputs; the default casts result k to
+    ``out_dtypes[k]``."""
     K = len(scalar_ops)
     nin, nout = len(in_dtypes), len(out_dtypes)
     ins = ["i%d" % k for k in range(nin)]
@@ -176,7 +178,10 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
                                                      "(a.a%d ? 1 : 0)" % k if dt == "bool" else "a.a%d" % k)
             args.append("r%d" % k)
         for j, dt in enumerate(extra_dtypes):
-            args.append("(*(const %s*)&o.ex[%d])" % (storage_ctype(dt), j))
+            if extra_is_array is not None and extra_is_array[j]:
+                args.append("(((const %s*)o.ex[%d])[idx])" % (storage_ctype(dt), j))
+            else:
+                args.append("(*(const %s*)&o.ex[%d])" % (storage_ctype(dt), j))
         post_stmt += "\n" + post_op.c_code(qnode, args, tmp) + "\n"
         post_stmt += "\n".join("((%s*)o.ptr[%d])[idx] = (%s)%s;" % (storage_ctype(dt), k, storage_ctype(dt), t)
                                for k, (dt, t) in enumerate(zip(out_dtypes, tmp)))

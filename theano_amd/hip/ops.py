@@ -278,7 +278,7 @@ class HipElemwise(Elemwise):
         return h
 
     def perform(self, node, inputs, output_storage):
-        flags = call_flags()
+        flags = call_flags(node)
         cache = node.tag.get("thx")
         if cache is None:
             handle, nin, nout = self._handle(node)
@@ -343,7 +343,8 @@ class HipCAReduce(CAReduce):
         self.pre_scalar_op = pre_scalar_op
         self.post_scalar_op = post_scalar_op
         # with an epilogue: the dtype each reduction result has before the epilogue reads it, and the
-        # number of trailing host-scalar inputs that only the epilogue uses
+        # number of trailing inputs that only the epilogue uses (host scalars, or device arrays with
+        # one element per result)
         self.post_in_dtypes = None if post_in_dtypes is None else tuple(post_in_dtypes)
         self.n_extra = int(n_extra)
         if len(self.acc_dtypes) != len(scalar_ops):
@@ -369,8 +370,8 @@ class HipCAReduce(CAReduce):
         extras = list(inputs[len(inputs) - self.n_extra:]) if self.n_extra else []
         inputs = inputs[:len(inputs) - self.n_extra] if self.n_extra else inputs
         for e in extras:
-            if not _is_host_scalar(e):
-                raise TypeError("epilogue operands must be host scalars", e)
+            if not (_is_host_scalar(e) or isinstance(e.type, HipArrayType)):
+                raise TypeError("epilogue operands must be host scalars or device arrays", e)
         ins = [i if (isinstance(i.type, HipArrayType) or _is_host_scalar(i)) else as_hip_variable(i) for i in inputs]
         nd = max(i.type.ndim for i in ins)
         if any(i.type.ndim != nd for i in ins if isinstance(i.type, HipArrayType)):
@@ -397,12 +398,13 @@ class HipCAReduce(CAReduce):
         n_red = len(node.inputs) - self.n_extra
         in_dt = tuple(i.type.dtype for i in node.inputs[:n_red])
         ex_dt = tuple(i.type.dtype for i in node.inputs[n_red:])
-        key = (self._props(), in_dt, ex_dt)
+        ex_arr = tuple(isinstance(i.type, HipArrayType) for i in node.inputs[n_red:])
+        key = (self._props(), in_dt, ex_dt, ex_arr)
         h = _reduce_handles.get(key)
         if h is None:
             src, name, acc_bytes = codegen.reduce_functor(self.scalar_ops, self.acc_dtypes, in_dt, self.out_dtypes,
                                                           self.pre_scalar_op, self.post_scalar_op, ex_dt,
-                                                          self.post_in_dtypes)
+                                                          self.post_in_dtypes, ex_arr)
             all_dt = in_dt + self.out_dtypes + ex_dt
             codes = (ctypes.c_int32 * len(all_dt))(*[scal.dtype_code(d) for d in all_dt])
             handle = ctypes.c_void_p()
@@ -413,7 +415,7 @@ class HipCAReduce(CAReduce):
         return h
 
     def perform(self, node, inputs, output_storage):
-        flags = call_flags()
+        flags = call_flags(node)
         cache = node.tag.get("thx")
         if cache is None:
             handle, nin, nout = self._handle(node)
@@ -434,6 +436,11 @@ class HipCAReduce(CAReduce):
         for k, v in enumerate(inputs):
             _operand(v, nd, ins[k])
         kept = tuple(shape[d] for d in range(nd) if d not in axis)
+        for k in range(nin, len(inputs)):
+            v = inputs[k]
+            if type(v) is HipArray and [d for d in v.shape if d != 1] != [d for d in kept if d != 1]:
+                raise ValueError("Input dimension mis-match. (epilogue operand %d has shape %s, the result has %s)"
+                                 % (k - nin, v.shape, kept))
         results = []
         for k in range(nout):
             arr = HipArray._new_contiguous(kept, out_dt[k])

@@ -342,17 +342,17 @@ def fuse_reduce_prologue(fgraph):
 
 
 def fuse_reduce_epilogue(fgraph):
-    """``g(reduce(...), host scalars)`` - the division of a mean, ``sqrt(var + eps)``
-    - runs in the reduction's own last step instead of a launch of its own.
-    Matches an elementwise node all of whose array inputs are results of one
-    reduction (possibly through identical keepdims DimShuffles)."""
+    """``g(reduce(...), ...)`` - the division of a mean, ``sqrt(var + eps)``, the
+    per-channel algebra between the two passes of a batch-norm gradient - runs in
+    the reduction's own last step instead of a launch of its own; repeated until
+    no consumer qualifies, so a chain of such nodes ends up in one epilogue."""
     count = 0
     changed = True
     while changed:
         changed = False
         for red in fgraph.toposort():
             rop = red.op
-            if not isinstance(rop, HipCAReduce) or rop.post_scalar_op is not None or red not in fgraph.apply_nodes:
+            if not isinstance(rop, HipCAReduce) or red not in fgraph.apply_nodes:
                 continue
             cands = []
             for r in red.outputs:
@@ -378,78 +378,97 @@ def fuse_reduce_epilogue(fgraph):
 
 
 def _try_epilogue(fgraph, red, cand):
+    """Moves the elementwise node ``cand`` into the epilogue of the reduction
+    ``red`` (composing it with an epilogue that is already there).  Every array
+    input of ``cand`` must be a result of ``red`` (directly or through one and the
+    same keepdims DimShuffle), a host scalar, or a device array of the results'
+    own shape that does not depend on ``red`` (a per-channel scale, the result
+    of an earlier reduction): the epilogue reads that one at the result's index."""
     rop = red.op
-    if True:
-        if True:
-            if len(cand.outputs) != 1 or cand.op.inplace_pattern:
+    if len(cand.outputs) != 1 or cand.op.inplace_pattern:
+        return False
+    n_red_in = len(red.inputs) - rop.n_extra
+    extras = list(red.inputs[n_red_in:])
+    post_in = rop.post_in_dtypes if rop.post_scalar_op is not None else rop.out_dtypes
+    s_acc = [scal.Scalar(dt)() for dt in post_in]
+    s_extras = [scal.Scalar(e.type.dtype)() for e in extras]
+    if rop.post_scalar_op is None:
+        cur = list(s_acc)
+    else:
+        cur = rop.post_scalar_op(*(s_acc + s_extras), return_list=True)
+    # the DimShuffle (if any) between the reduction and the consumer
+    ds_op, seen_direct = None, False
+    for i in cand.inputs:
+        if i.owner is not None and isinstance(i.owner.op, HipDimShuffle) and i.owner.inputs[0].owner is red:
+            if ds_op is not None and i.owner.op != ds_op:
                 return False
-            # classify the consumer's inputs
-            ds_op, ok, s_args, extras, s_extras = None, True, [], [], []
-            s_acc = [scal.Scalar(dt)() for dt in rop.out_dtypes]
-            used = set()
-            for i in cand.inputs:
-                src, this_ds = i, None
-                if src.owner is not None and isinstance(src.owner.op, HipDimShuffle):
-                    this_ds = src.owner.op
-                    src = src.owner.inputs[0]
-                if src.owner is red:
-                    if ds_op is not None and this_ds != ds_op and used:
-                        ok = False
-                        break
-                    ds_op = this_ds
-                    k = red.outputs.index(src)
-                    used.add(k)
-                    s_args.append(s_acc[k])
-                    continue
-                c = _scalar_constant(i)
-                if c is not None:
-                    s_args.append(c)
-                elif _is_host_scalar(i):
-                    sv = None
-                    for e, se in zip(extras, s_extras):
-                        if e is i:
-                            sv = se
-                    if sv is None:
-                        sv = scal.Scalar(i.type.dtype)()
-                        extras.append(i)
-                        s_extras.append(sv)
-                    s_args.append(sv)
-                else:
-                    ok = False
-                    break
-            if not ok or not used or len(extras) > 8:
-                return False
-            e_out = cand.op.scalar_op(*s_args)
-            # reduction results something else still needs stay outputs of the new node
-            keep = []
-            for k, r in enumerate(red.outputs):
-                others = False
-                for c, _ in fgraph.clients.get(r, []):
-                    if c == "output":
-                        others = True
-                    elif isinstance(c.op, HipDimShuffle) and c.op == ds_op:
-                        if any(c2 is not cand for c2, _ in fgraph.clients.get(c.outputs[0], [])):
-                            others = True
-                    elif c is not cand:
-                        others = True
-                if others or k not in used:
-                    keep.append(k)
-            post_outs = [scal.identity(s_acc[k]) for k in keep] + [e_out]
-            post = scal.Composite(s_acc + s_extras, post_outs)
-            out_dtypes = tuple(rop.out_dtypes[k] for k in keep) + (cand.outputs[0].type.dtype,)
-            n_red_in = len(red.inputs)
-            new_op = HipCAReduce(rop.scalar_ops, rop.axis, rop.acc_dtypes, out_dtypes, rop.pre_scalar_op, post,
-                                 rop.out_dtypes, len(extras))
-            new_node = new_op.make_node(*(list(red.inputs[:n_red_in]) + extras))
-            new_e = new_node.outputs[-1]
-            if ds_op is not None:
-                new_e = HipDimShuffle(ds_op.input_broadcastable, ds_op.new_order)(new_e)
-            if new_e.type != cand.outputs[0].type:
-                return False
-            for j, k in enumerate(keep):
-                fgraph.replace(red.outputs[k], new_node.outputs[j])
-            fgraph.replace(cand.outputs[0], new_e)
-            return True
+            ds_op = i.owner.op
+        elif i.owner is red:
+            seen_direct = True
+    if ds_op is not None and seen_direct:
+        return False
+    if ds_op is not None:
+        layout = ds_op.make_node(red.outputs[0]).outputs[0].type.broadcastable
+    else:
+        layout = red.outputs[0].type.broadcastable
+    s_args, used = [], set()
+    for i in cand.inputs:
+        src = i.owner.inputs[0] if (ds_op is not None and i.owner is not None and i.owner.op == ds_op and
+                                   i.owner.inputs[0].owner is red) else i
+        if src.owner is red:
+            k = red.outputs.index(src)
+            used.add(k)
+            s_args.append(cur[k])
+            continue
+        c = _scalar_constant(i)
+        if c is not None:
+            s_args.append(c)
+            continue
+        per_result = (isinstance(i.type, HipArrayType) and tuple(i.type.broadcastable) == tuple(layout) and
+                      not _depends_on(i, red))
+        if not (_is_host_scalar(i) or per_result):
+            return False
+        sv = None
+        for e, se in zip(extras, s_extras):
+            if e is i:
+                sv = se
+        if sv is None:
+            sv = scal.Scalar(i.type.dtype)()
+            extras.append(i)
+            s_extras.append(sv)
+        s_args.append(sv)
+    if not used or len(extras) > 12:
+        return False
+    e_out = cand.op.scalar_op(*s_args)
+    # results something else still needs stay outputs of the new node
+    keep = []
+    for k, r in enumerate(red.outputs):
+        others = False
+        for c, _ in fgraph.clients.get(r, []):
+            if c == "output":
+                others = True
+            elif isinstance(c.op, HipDimShuffle) and c.op == ds_op:
+                if any(c2 is not cand for c2, _ in fgraph.clients.get(c.outputs[0], [])):
+                    others = True
+            elif c is not cand:
+                others = True
+        if others:
+            keep.append(k)
+    post_outs = [scal.identity(cur[k]) if cur[k] in s_acc else cur[k] for k in keep] + [e_out]
+    post = scal.Composite(s_acc + s_extras, post_outs)
+    out_dtypes = tuple(rop.out_dtypes[k] for k in keep) + (cand.outputs[0].type.dtype,)
+    new_op = HipCAReduce(rop.scalar_ops, rop.axis, rop.acc_dtypes, out_dtypes, rop.pre_scalar_op, post, post_in,
+                         len(extras))
+    new_node = new_op.make_node(*(list(red.inputs[:n_red_in]) + extras))
+    new_e = new_node.outputs[-1]
+    if ds_op is not None:
+        new_e = HipDimShuffle(ds_op.input_broadcastable, ds_op.new_order)(new_e)
+    if new_e.type != cand.outputs[0].type:
+        return False
+    for j, k in enumerate(keep):
+        fgraph.replace(red.outputs[k], new_node.outputs[j])
+    fgraph.replace(cand.outputs[0], new_e)
+    return True
 
 
 def _depends_on(var, node, limit=10000):

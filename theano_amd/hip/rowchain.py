@@ -195,7 +195,7 @@ class HipRowChain(Op):
             arr = HipArray._new_contiguous(tuple(shape), out_dt[k])
             arr.as_thx(outs[k])
             results.append(arr)
-        rc = lib.thx_rowchain_call(handle, ins, outs, call_flags())
+        rc = lib.thx_rowchain_call(handle, ins, outs, call_flags(node))
         if rc == THX_ERR_UNSUPPORTED:
             results = self._run_fallback(inputs)
         elif rc:

@@ -19,6 +19,7 @@ _LIB_PATH = os.path.join(os.path.dirname(_HERE), "csrc", "libthx_hip.so")
 THX_MAX_ND = 8
 THX_BROADCAST = 1
 THX_DRY_RUN = 2
+THX_KEEP_CACHED = 4
 THX_HOST_SCALAR = 0x100
 
 
@@ -112,8 +113,13 @@ def dry_run():
     return _dry
 
 
-def call_flags():
-    return THX_BROADCAST | (THX_DRY_RUN if _dry else 0)
+def call_flags(node=None):
+    """Flags of a kernel call; ``node.tag['keep_cached']`` (set when the function is compiled) adds
+    THX_KEEP_CACHED."""
+    f = THX_BROADCAST | (THX_DRY_RUN if _dry else 0)
+    if node is not None and node.tag.get("keep_cached"):
+        f |= THX_KEEP_CACHED
+    return f
 
 
 def init(device=None):

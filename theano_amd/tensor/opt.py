@@ -15,7 +15,7 @@ from .. import gof
 from .. import scalar as scal
 from ..gof import local_optimizer
 from . import basic as T
-from .elemwise import CAReduce, DimShuffle, Elemwise
+from .elemwise import CAReduce, DimShuffle, Elemwise, Sum
 from .type import TensorConstant, TensorType, constant
 
 
@@ -28,6 +28,10 @@ def local_dimshuffle_fold(fgraph, node):
     if not isinstance(x.type, TensorType):
         return False
     if op.new_order == tuple(range(x.type.ndim)):
+        return [x]
+    # dropping a broadcastable dimension and inserting one at the same place changes nothing
+    if (len(op.new_order) == x.type.ndim and node.outputs[0].type == x.type and
+            all(o == d or (o == "x" and x.type.broadcastable[d]) for d, o in enumerate(op.new_order))):
         return [x]
     if isinstance(x, TensorConstant):
         data = np.asarray(x.data)
@@ -159,6 +163,103 @@ def local_useless_reduce(fgraph, node):
     return False
 
 
+@local_optimizer([CAReduce])
+def local_sum_invariant_factor(fgraph, node):
+    """``sum(c * x, axis) -> c' * sum(x, axis)``, ``sum(x / c) -> sum(x) / c'`` and
+    ``sum(-x) -> -sum(x)`` for every factor ``c`` that is constant along all the
+    reduced axes (broadcastable there); ``c'`` is ``c`` without those axes.
+
+    ``local_sum_prod_mul_by_scalar`` (``theano/tensor/opt.py:5062-5149``) does
+    this for factors that are broadcastable everywhere; per-channel factors of a
+    batch-norm gradient (``sum(g * gamma * (x - mean) / std**2, axis=(0, 2, 3))``)
+    are the same case along the reduced axes only.  Products are searched
+    through nested ``mul`` / ``true_div`` / ``neg`` nodes; other users of those nodes
+    keep them.
+    Floating point sums only: an integer sum in a wider dtype does not wrap where
+    the narrower product would."""
+    op = node.op
+    if type(op) is not Sum:
+        return False
+    (x,) = node.inputs
+    out = node.outputs[0]
+    dt = x.type.dtype
+    if dt not in scal.float_dtypes or out.type.dtype not in scal.float_dtypes or x.owner is None:
+        return False
+    nd = x.type.ndim
+    axis = tuple(range(nd)) if op.axis is None else op.axis
+    if not axis:
+        return False
+
+    def invariant(v):
+        return v.type.ndim == nd and all(v.type.broadcastable[a] for a in axis)
+
+    found = [False]
+
+    def split(v):
+        """(invariant factor or None, remaining factor or None, negated) with
+        v == (-1 if negated) * invariant * remaining."""
+        if invariant(v):
+            return v, None, False
+        p = v.owner
+        if p is None or not isinstance(p.op, Elemwise) or v.type.dtype != dt:
+            return None, v, False
+        sop = p.op.scalar_op
+        if isinstance(sop, scal.Mul):
+            invs, rests, sign = [], [], False
+            for t in p.inputs:
+                if t.type.ndim != nd:
+                    return None, v, False
+                ci, ri, si = split(t)
+                sign ^= si
+                if ci is not None:
+                    invs.append(ci)
+                if ri is not None:
+                    rests.append(ri)
+            if not invs and not sign:
+                return None, v, False
+            found[0] = True
+            inv = None if not invs else (invs[0] if len(invs) == 1 else T.mul(*invs))
+            rest = None if not rests else (rests[0] if len(rests) == 1 else T.mul(*rests))
+            return inv, rest, sign
+        if isinstance(sop, scal.TrueDiv):
+            a, b = p.inputs
+            if a.type.ndim != nd or b.type.ndim != nd or a.type.dtype != dt or b.type.dtype != dt:
+                return None, v, False
+            ca, ra, sa = split(a)
+            if invariant(b):
+                found[0] = True
+                inv = T.true_div(ca, b) if ca is not None else T.inv(b)
+                return inv, ra, sa
+            if ca is None and not sa:
+                return None, v, False
+            found[0] = True
+            return ca, T.true_div(ra if ra is not None else T.ones_like(b), b), sa
+        if isinstance(sop, scal.Neg):
+            ca, ra, sa = split(p.inputs[0])
+            found[0] = True
+            return ca, ra, not sa
+        return None, v, False
+
+    inv, rest, sign = split(x)
+    if not found[0] or rest is None or (inv is None and not sign):
+        return False
+    if rest.type.dtype != dt:
+        rest = T.cast(rest, dt)
+    new = Sum(op.axis, dtype=op.dtype, acc_dtype=op.acc_dtype)(rest)
+    if inv is not None:
+        if inv.type.dtype != dt:
+            return False
+        keep = [d for d in range(nd) if d not in axis]
+        new = T.mul(DimShuffle(inv.type.broadcastable, keep)(inv), new)
+    if sign:
+        new = T.neg(new)
+    if new.type.dtype != out.type.dtype:
+        new = T.cast(new, out.type.dtype)
+    if new.type != out.type:
+        return False
+    return [new]
+
+
 @local_optimizer([T.ShapeFloat])
 def local_shape_lift(fgraph, node):
     """The extent of an elementwise / DimShuffle / reduction result is the extent
@@ -188,7 +289,7 @@ def local_shape_lift(fgraph, node):
 
 
 CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_useless_elemwise, local_fill_sink, local_useless_reduce,
-                local_dimshuffle_lift]
+                local_dimshuffle_lift, local_sum_invariant_factor]
 
 
 def canonicalize(fgraph):
