@@ -166,3 +166,17 @@ def test_host_scalar_operands_travel_by_value():
     xv = np.arange(12, dtype="float32").reshape(3, 4)
     assert_parity(f(xv, np.float32([[2.5]])), xv * np.float32(2.5) + np.float32(2.5), "immediate")
     assert "m0,3,0" in hip.last_plan() or ",3" in hip.last_plan()
+
+
+def test_inplace_elementwise_matches_out_of_place():
+    rng = np.random.default_rng(15)
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    xv, yv = rng.standard_normal((257, 130)).astype("float32"), rng.standard_normal((257, 130)).astype("float32")
+    out = (T.exp(x) * y + 1.0) * T.tanh(y)
+    f_in = th.function([x, y], out, fuse=False)
+    f_out = th.function([x, y], out, fuse=False, inplace=False)
+    assert any(n.op.inplace_pattern for n in f_in.toposort() if hasattr(n.op, "inplace_pattern"))
+    a, b = f_in(xv, yv), f_out(xv, yv)
+    assert np.array_equal(a, b)
+    assert_parity(a, G.evaluate([x, y], [out], [xv, yv])[0], "unfused in-place chain")
+    assert np.array_equal(f_in(xv, yv), a)            # the inputs were not overwritten by the first call

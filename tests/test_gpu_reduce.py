@@ -140,3 +140,36 @@ def test_fused_prologue_and_multi_output():
     av = rng.integers(-5, 6, (200, 333)).astype("int32")
     g2 = th.function([a], [T.any(a > 4), T.all(a > -6), T.any(a > 5), T.all(a > 0)])(av)
     assert [bool(v) for v in g2] == [True, True, False, False]
+
+
+def test_epilogue_chain_with_per_result_device_operands():
+    """Per-channel algebra after a reduction (other per-channel arrays, results
+    of an earlier reduction, host scalars) runs in the reduction's epilogue;
+    factors that are constant along the reduced axes leave the sums."""
+    from theano_amd.hip import HipCAReduce, HipElemwise
+    rng = np.random.default_rng(26)
+    t4 = T.TensorType("float32", (False,) * 4)
+    pc = T.TensorType("float32", (True, False, True, True))
+    x, g = t4("x"), t4("g")
+    gamma, beta = pc("gamma"), pc("beta")
+    mean = T.mean(x, axis=(0, 2, 3), keepdims=True)
+    d = x - mean
+    std = T.sqrt(T.mean(T.sqr(d), axis=(0, 2, 3), keepdims=True) + np.float32(1e-3))
+    s1 = T.sum(g * gamma * d / (std * std), axis=(0, 2, 3), keepdims=True)
+    s2 = T.sum((g / std) * d, axis=(0, 2, 3), keepdims=True)
+    outs = [s1 * gamma + beta / std, (s2 - s1) * T.exp(beta), T.sum(g, axis=(0, 2, 3))]
+    vals = [rng.standard_normal((6, 37, 5, 9)).astype("float32"), rng.standard_normal((6, 37, 5, 9)).astype("float32"),
+            rng.uniform(0.5, 2, (1, 37, 1, 1)).astype("float32"), rng.standard_normal((1, 37, 1, 1)).astype("float32")]
+    f = th.function([x, g, gamma, beta], outs)
+    kernels = [n for n in f.toposort() if isinstance(n.op, (HipCAReduce, HipElemwise))]
+    assert [type(n.op) for n in kernels] == [HipCAReduce, HipCAReduce], kernels
+    assert any(type(i.type).__name__ == "HipArrayType" for i in kernels[1].inputs[len(kernels[1].inputs) - kernels[1].op.n_extra:])
+    got = f(*vals)
+    ref = G.evaluate([x, g, gamma, beta], outs, vals)
+    for k, (a, b) in enumerate(zip(got, ref)):
+        assert_parity(a, b, "epilogue output %d" % k, tol=dict(rtol=3e-5, atol=3e-6))
+    # a per-result operand of the wrong extent is refused like any broadcast mismatch
+    bad = list(vals)
+    bad[2] = np.ones((1, 36, 1, 1), "float32")
+    with pytest.raises(ValueError):
+        f(*bad)

@@ -212,3 +212,24 @@ def test_batchnorm_gradient_is_two_statistics_passes_and_one_elementwise_pass(dr
     assert [bool(n.tag.get("keep_cached")) for n in kernels] == [True, True, False]
     small = workloads.c5_inputs("small")
     f(*small)                                      # plans and compiles every kernel (dry run)
+
+
+def test_inplace_pass_reuses_single_use_intermediates_only(dry_run):
+    """The in-place pass (InplaceElemwiseOptimizer's role): an intermediate that
+    one kernel computes and one elementwise kernel consumes is overwritten;
+    function inputs, outputs, views and values with two readers never are."""
+    x = T.fmatrix("x")
+    f = th.function([x], T.exp(x) * 2.0 + 1.0, fuse=False)
+    ew = ops_of(f, HipElemwise)
+    assert [dict(n.op.inplace_pattern) for n in ew] == [{}, {0: 0}, {0: 0}]   # exp reads the input: not in place
+    assert ew[1].op.destroy_map == {0: [0]}
+    e = T.exp(x)
+    g = th.function([x], [e + 1.0, e * 2.0], fuse=False)
+    assert all(not n.op.inplace_pattern for n in ops_of(g, HipElemwise))       # e has two readers
+    h = th.function([x], [e, e + 1.0], fuse=False)
+    assert all(not n.op.inplace_pattern for n in ops_of(h, HipElemwise))       # e is an output
+    k = th.function([x], T.sum(x, axis=0).dimshuffle("x", 0) + 1.0, fuse=False)
+    assert all(not n.op.inplace_pattern for n in ops_of(k, HipElemwise))       # a view of the sum
+    f(np.ones((3, 4), "float32"))
+    assert not any(n.op.inplace_pattern for n in ops_of(th.function([x], T.exp(x) * 2.0 + 1.0, fuse=False,
+                                                                    inplace=False), HipElemwise))

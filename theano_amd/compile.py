@@ -210,7 +210,7 @@ class Function(object):
         return list(self.nodes)
 
 
-def function(inputs, outputs, fuse=True, rowchain=True, name=None, on_unused_input="raise"):
+def function(inputs, outputs, fuse=True, rowchain=True, inplace=True, name=None, on_unused_input="raise"):
     """Compile ``outputs`` as a function of ``inputs``.
 
     ``inputs``: variables or ``In`` instances.  A host-typed input may be given
@@ -218,7 +218,8 @@ def function(inputs, outputs, fuse=True, rowchain=True, name=None, on_unused_inp
     variable, ``Out`` or a list of those; ``Out(v, device=True)`` leaves the
     result on the GPU.  Every op must have a HIP implementation.  ``fuse=False``
     keeps one kernel per graph node; ``rowchain=False`` keeps elementwise /
-    row-reduction islands as separate fused kernels."""
+    row-reduction islands as separate fused kernels; ``inplace=False`` gives
+    every elementwise result a buffer of its own."""
     from .hip import opt as hip_opt
     from .hip.ops import HipArrayType, as_hip_variable
 
@@ -249,7 +250,7 @@ def function(inputs, outputs, fuse=True, rowchain=True, name=None, on_unused_inp
     c_in = [memo[v] for v in in_vars]
     c_out = [memo[v] for v in out_vars]
     fgraph = _SharedAwareGraph(c_in, c_out, shared_inputs)
-    fgraph = hip_opt.optimize(fgraph, fuse=fuse, rowchain=rowchain)
+    fgraph = hip_opt.optimize(fgraph, fuse=fuse, rowchain=rowchain, inplace=inplace)
     return Function(fgraph, in_specs, out_specs, single, shared_inputs)
 
 

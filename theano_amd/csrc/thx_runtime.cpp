@@ -216,7 +216,11 @@ int nt_choice(int family_default, int flags) {
   return family_default;
 }
 
-int nt_streaming(int64_t moved, int flags) { return nt_choice(moved >= (int64_t(288) << 20), flags); }
+int nt_streaming(int64_t moved, int flags) {
+  // the hint only helps when this call's own traffic leaves room in the cache for what is to be kept
+  if (moved > (int64_t(256) << 20)) flags &= ~THX_KEEP_CACHED;
+  return nt_choice(moved >= (int64_t(288) << 20), flags);
+}
 
 static uint64_t fnv1a(const std::string& s, uint64_t h) {
   for (unsigned char c : s) {

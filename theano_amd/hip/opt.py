@@ -558,8 +558,38 @@ def _merge_two(a, b):
 
 
 # --------------------------------------------------------------------------
-def optimize(fgraph, fuse=True, rowchain=True):
-    """Full pipeline: clean up, lift, fuse."""
+def inplace_elemwise(fgraph):
+    """The role of ``InplaceElemwiseOptimizer`` (``theano/tensor/opt.py:150-410``):
+    an elementwise kernel writes its result over an input of identical type when
+    nothing else reads that input - it is an intermediate computed by another
+    kernel of this function, used once, not a view, not an output.  Each thread
+    reads exactly the positions it writes, so the aliasing is safe in every
+    elementwise plan.  Saves the allocation and lowers the function's peak memory;
+    on this device it moves no fewer bytes."""
+    from .rowchain import HipRowChain
+    count = 0
+    for node in fgraph.toposort():
+        op = node.op
+        if not isinstance(op, HipElemwise) or len(node.outputs) != 1 or op.inplace_pattern:
+            continue
+        out = node.outputs[0]
+        for idx, i in enumerate(node.inputs):
+            if (i.type != out.type or i.owner is None or i in fgraph.outputs or
+                    not isinstance(i.owner.op, (HipElemwise, HipCAReduce, HipRowChain))):
+                continue
+            if fgraph.n_clients(i) != 1 or list(node.inputs).count(i) != 1:
+                continue
+            new = HipElemwise(op.scalar_op, {0: idx}).make_node(*node.inputs).outputs[0]
+            if new.type != out.type:
+                continue
+            fgraph.replace(out, new)
+            count += 1
+            break
+    return count
+
+
+def optimize(fgraph, fuse=True, rowchain=True, inplace=True):
+    """Full pipeline: clean up, lift, fuse, then in-place."""
     from ..tensor.opt import canonicalize
     canonicalize(fgraph)
     fgraph = lift_to_hip(fgraph)
@@ -576,4 +606,6 @@ def optimize(fgraph, fuse=True, rowchain=True):
         gof.merge_identical(fgraph)
         fuse_reduce_epilogue(fgraph)
         gof.merge_identical(fgraph)
+    if inplace:
+        inplace_elemwise(fgraph)
     return fgraph
