@@ -54,6 +54,14 @@ enum {
  * keeps 0-d operands on the host as well (theano/gpuarray/type.py:55-57). */
 #define THX_HOST_SCALAR 0x100
 
+/* OR-ed into thx_array.dtype (THX_I64, all extents 1, base ignored) of an input of
+ * thx_reduce_call: a virtual operand whose value at an element is that element's
+ * position within the reduced dimensions, counted in C order of those dimensions -
+ * the index numpy.argmax returns after the reduced axes are moved to the end and
+ * flattened, which is how MaxAndArgmax.perform defines its second output
+ * (theano/tensor/basic.py:1311-1330). It costs no memory traffic. */
+#define THX_INDEX 0x200
+
 /* A strided view of device memory (counterpart of libgpuarray's GpuArray:
  * data, offset, nd, dimensions, byte strides, typecode). Strides may be zero
  * or negative; they must be multiples of the element size. */

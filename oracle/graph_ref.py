@@ -152,12 +152,26 @@ def eval_scalar_op(op, in_values, out_dtypes):
     return [np.asarray(fn(out_dtypes[0], *[np.asarray(v) for v in in_values]))]
 
 
+def max_and_argmax(x, axes):
+    """``MaxAndArgmax.perform`` (``theano/tensor/basic.py:1311-1330``): ``np.max``
+    over the axes; for the argmax the kept axes go in front, the reduced ones
+    (original order) are flattened and ``np.argmax`` runs over that last axis,
+    result as int64.  An empty reduced extent raises, as NumPy does."""
+    x = np.asarray(x)
+    axes = tuple(int(a) for a in axes)
+    keep = [i for i in range(x.ndim) if i not in axes]
+    t = np.transpose(x, keep + list(axes))
+    kept_shape = t.shape[:len(keep)]
+    r = t.reshape(kept_shape + (int(np.prod(t.shape[len(keep):], dtype="int64")),))
+    return np.asarray(np.max(x, axes), dtype=x.dtype), np.asarray(np.argmax(r, axis=-1), dtype="int64")
+
+
 def evaluate(inputs, outputs, values):
     """Values of ``outputs`` (theano_amd variables) given ``values`` for
     ``inputs``; every Apply node is computed separately, as an unfused graph."""
     from theano_amd import gof
     from theano_amd.tensor.elemwise import CAReduce, CAReduceDtype, DimShuffle, Elemwise
-    from theano_amd.tensor.basic import ShapeFloat
+    from theano_amd.tensor.basic import MaxAndArgmax, ShapeFloat
     env = {}
     for var, val in zip(inputs, values):
         env[var] = var.type.filter(np.asarray(val), strict=False, allow_downcast=False)
@@ -187,6 +201,8 @@ def evaluate(inputs, outputs, values):
             res = [careduce(x, sname, op.axis, acc_dt, out_dt)]
         elif isinstance(op, ShapeFloat):
             res = [np.asarray(args[0].shape[op.i], dtype=op.dtype)]
+        elif isinstance(op, MaxAndArgmax):
+            res = list(max_and_argmax(args[0], op.axis))
         else:
             raise NotImplementedError("oracle cannot evaluate %s" % op)
         for o, v in zip(node.outputs, res):

@@ -233,3 +233,33 @@ def test_inplace_pass_reuses_single_use_intermediates_only(dry_run):
     f(np.ones((3, 4), "float32"))
     assert not any(n.op.inplace_pattern for n in ops_of(th.function([x], T.exp(x) * 2.0 + 1.0, fuse=False,
                                                                     inplace=False), HipElemwise))
+
+
+def test_max_and_argmax_interface(dry_run):
+    """Output types, keepdims, the 0-d case, the zero gradient of argmax, the
+    max-only rewrite and argmin's reversal (theano/tensor/basic.py:1273-1803,
+    tests theano/tensor/tests/test_basic.py:3103-3218)."""
+    from theano_amd.hip import HipMaxAndArgmax
+    x = T.ftensor3("x")
+    m, a = T.max_and_argmax(x, axis=[1, -1])
+    assert m.type.dtype == "float32" and a.type.dtype == "int64" and m.type.ndim == 1 and a.type.ndim == 1
+    assert isinstance(m.owner.op, T.MaxAndArgmax) and m.owner.op.axis == (1, 2)
+    mk, ak = T.max_and_argmax(x, axis=0, keepdims=True)
+    assert mk.type.broadcastable == (True, False, False) and ak.type.broadcastable == (True, False, False)
+    s = T.fscalar("s")
+    v0, i0 = T.max_and_argmax(s)
+    assert v0 is s and i0.type.dtype == "int64" and int(i0.data) == 0
+    with pytest.raises(ValueError):
+        T.max_and_argmax(x, axis=3)
+    # d argmax / dx is zero; d max / dx marks the positions equal to the maximum
+    g = th.grad(T.sum(T.cast(T.argmax(x, axis=0), "float32")), x, disconnected_inputs="zero")
+    f = th.function([x], g)
+    assert not ops_of(f, HipMaxAndArgmax)
+    # nothing reads the argmax: a plain max reduction runs
+    f = th.function([x], T.max_and_argmax(x, axis=2)[0])
+    assert not ops_of(f, HipMaxAndArgmax) and len(ops_of(f, HipCAReduce)) == 1
+    # argmin(x) = argmax(-x), the negation computed inside the reduction
+    f = th.function([x], T.argmin(x, axis=1))
+    (node,) = ops_of(f, HipMaxAndArgmax)
+    assert not ops_of(f, HipElemwise) and str(node.op.pre_scalar_op) == "Composite{neg(i0)}"
+    f(np.zeros((3, 5, 7), "float32"))

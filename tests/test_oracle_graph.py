@@ -254,3 +254,41 @@ def test_cpu_backend_half_conversions_match_numpy():
     hn = np.empty(1, np.uint16)
     L.cpu_f2h_array(nan.ctypes.data_as(ctypes.c_void_p), hn.ctypes.data_as(ctypes.c_void_p), ctypes.c_int64(1))
     assert np.isnan(hn.view(np.float16)[0])
+
+
+def test_max_and_argmax_against_reference_vectors_and_brute_force():
+    """Literal answers of theano/tensor/tests/test_basic.py:3114-3119 and
+    :3304-3309, then a brute-force scan (first occurrence of the greatest value,
+    a NaN counting as the greatest) over every axis subset of small arrays with
+    ties and NaNs."""
+    import itertools
+    v, i = G.max_and_argmax(np.array([1, 2, 3, 2, -6]), (0,))
+    assert v == 3 and i == 2 and i.dtype == np.int64
+    v, i = G.max_and_argmax(np.arange(24).reshape(3, 2, 4), (1, 2))
+    assert np.array_equal(v, [7, 15, 23]) and np.array_equal(i, [7, 7, 7])
+    rng = np.random.default_rng(11)
+    x = rng.integers(0, 4, (3, 4, 5)).astype("float32")      # many ties
+    x[1, 2, 3] = np.nan
+    x[1, 3, 0] = np.nan
+    for k in (1, 2, 3):
+        for axes in itertools.combinations(range(3), k):
+            v, i = G.max_and_argmax(x, axes)
+            keep = [d for d in range(3) if d not in axes]
+            for kidx in itertools.product(*[range(x.shape[d]) for d in keep]):
+                best, best_pos, pos = None, None, 0
+                for ridx in itertools.product(*[range(x.shape[d]) for d in axes]):
+                    full = [0, 0, 0]
+                    for d, j in zip(keep, kidx):
+                        full[d] = j
+                    for d, j in zip(axes, ridx):
+                        full[d] = j
+                    e = x[tuple(full)]
+                    better = best is None or (np.isnan(e) and not np.isnan(best)) or (not np.isnan(best) and e > best)
+                    if better:
+                        best, best_pos = e, pos
+                    pos += 1
+                assert i[kidx] == best_pos and (v[kidx] == best or (np.isnan(best) and np.isnan(v[kidx])))
+    x0, a0 = T.fmatrix("x"), None
+    outs = T.max_and_argmax(x0, axis=1, keepdims=True)
+    got = G.evaluate([x0], outs, [x[0]])
+    assert got[0].shape == (4, 1) and got[1].shape == (4, 1) and got[1].dtype == np.int64

@@ -96,7 +96,7 @@ class Function(object):
         def big(v):
             return isinstance(v.type, HipArrayType) and v.type.ndim > 0 and not any(v.type.broadcastable)
 
-        kernels = [n for n in self.nodes if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain")]
+        kernels = [n for n in self.nodes if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax")]
         later = set()
         for node in reversed(kernels):
             mine = set(id(root(i)) for i in node.inputs if big(i))

@@ -32,7 +32,8 @@ namespace thx {
 enum { M_VEC = 0,      // unit stride: one wide load/store per thread
        M_BCAST = 1,    // zero stride: one element shared by the whole vector
        M_GATHER = 2,   // any other stride: one access per element
-       M_IMM = 3 };    // a single host value passed in the kernel arguments
+       M_IMM = 3,      // a single host value passed in the kernel arguments
+       M_IOTA = 4 };   // no memory: the value is the element offset itself (a position index)
 
 template <int B> struct AlignFor { enum { value = B >= 16 ? 16 : B }; };
 

@@ -68,6 +68,12 @@ struct RedAcc {
       for (int k = 0; k < N; ++k) r.v[k] = s;
       return;
     }
+    if (P::mode(I) == M_IOTA) {  // the "strides" of this operand are index multipliers
+      const IT st = vstride[I];
+#pragma unroll
+      for (int k = 0; k < N; ++k) r.v[k] = (T)(off[I] + k * st);
+      return;
+    }
     const T* b = (const T*)ptr[I] + off[I];
     if (N == 1) {
       r.v[0] = *b;
@@ -135,7 +141,6 @@ __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, R:
         ok[u] = q < j1;
         RedAcc<P, NIN> a;
         a.ptr = p.in;
-      a.imm = p.imm;
         a.imm = p.imm;
         a.vstride = p.rc_stride;
         if (P::RA2) {
@@ -251,7 +256,6 @@ __device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, R:
         ok[u] = q < r1;
         RedAcc<P, NIN> a;
         a.ptr = p.in;
-      a.imm = p.imm;
         a.imm = p.imm;
         a.vstride = p.c_stride;
         if (P::RR2) {

@@ -128,6 +128,8 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
         return fail(THX_ERR_TYPE, "elemwise: output %d has a zero stride along dimension %d", o, d);
     }
   }
+  for (int o = 0; o < e->n_in; ++o)
+    if (views[o].iota) return fail(THX_ERR_UNSUPPORTED, "elemwise: index operands are for reductions only");
   int64_t n = 1;
   for (int d = 0; d < nd; ++d) n *= shape[d];
   if (n == 0) {

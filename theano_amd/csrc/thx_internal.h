@@ -102,6 +102,7 @@ struct View {
   int dtype = 0;
   bool imm = false;     // a host scalar travelling in the kernel arguments
   uint64_t immval = 0;  // its value bytes
+  bool iota = false;    // no memory: the strides are index multipliers and the value is the offset
   int64_t stride[THX_MAX_ND] = {0};
 };
 

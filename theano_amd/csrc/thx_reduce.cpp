@@ -19,7 +19,7 @@ struct thx_reduce {
 
 namespace thx {
 
-enum { M_VEC = 0, M_BCAST = 1, M_GATHER = 2, M_IMM = 3 };
+enum { M_VEC = 0, M_BCAST = 1, M_GATHER = 2, M_IMM = 3, M_IOTA = 4 };
 
 struct Dim {
   int64_t extent;
@@ -137,6 +137,18 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   int rc = gather_inputs("reduce", ins, NIN, r->dtypes.data(), flags, &nd, shape, &views);
   if (rc) return rc;
   if (nd > 0 && !reduce_mask) return fail(THX_ERR_ARG, "thx_reduce_call: null mask");
+  // THX_INDEX operands: the element's position within the reduced dimensions, in C order
+  for (int i = 0; i < NIN; ++i) {
+    if (!(ins[i].dtype & THX_INDEX)) continue;
+    View& v = views[i];
+    v.iota = true;
+    v.ptr = nullptr;
+    int64_t mult = 1;
+    for (int d = nd - 1; d >= 0; --d) {
+      v.stride[d] = reduce_mask[d] ? mult : 0;
+      if (reduce_mask[d]) mult *= shape[d];
+    }
+  }
   // outputs: C-contiguous arrays of the kept dimensions
   int64_t kshape[THX_MAX_ND];
   int nk_full = 0;
@@ -212,6 +224,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   {
     int64_t best = -1;
     for (int i = 0; i < NIN; ++i) {
+      if (views[i].iota) continue;
       int64_t foot = 1;
       for (int d = 0; d < nd; ++d)
         if (views[i].stride[d] != 0) foot *= shape[d];
@@ -290,6 +303,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       ra_stride[i] = ra2 ? RD[0].stride[i] : 0;
       mode[i] = rc_stride[i] == 1 ? M_VEC : (rc_stride[i] == 0 ? M_BCAST : M_GATHER);
       if (views[i].imm) mode[i] = M_IMM;
+      if (views[i].iota) mode[i] = M_IOTA;
     }
     int vec = vec_width(mode);
     auto vec_ok = [&](int v) {
@@ -389,6 +403,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       r0_stride[i] = rr2 ? RD[0].stride[i] : 0;
       mode[i] = c_stride[i] == 1 ? M_VEC : (c_stride[i] == 0 ? M_BCAST : M_GATHER);
       if (views[i].imm) mode[i] = M_IMM;
+      if (views[i].iota) mode[i] = M_IOTA;
     }
     int vec = vec_width(mode);
     auto vec_ok = [&](int v) {
@@ -482,6 +497,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     key << "rg|k" << NK << "|r" << NR << (wide ? "|i64" : "|i32") << "|t" << tpr << "|m";
     for (int i = 0; i < NIN; ++i) {
       if (views[i].imm) gmode[i] = M_IMM;
+      if (views[i].iota) gmode[i] = M_IOTA;
       key << gmode[i] << (i + 1 < NIN ? "," : "");
     }
     plan = key.str() + (fast_div() ? "|fd" : "");

@@ -147,9 +147,9 @@ int gather_inputs(const char* what, const thx_array* ins, int n_in, const int32_
   for (int i = 0; i < n_in; ++i) {
     if (ins[i].nd != nd)
       return fail(THX_ERR_TYPE, "%s: input %d has rank %d, expected %d", what, i, ins[i].nd, nd);
-    if ((ins[i].dtype & ~THX_HOST_SCALAR) != dtypes[i])
+    if ((ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX)) != dtypes[i])
       return fail(THX_ERR_TYPE, "%s: input %d has dtype code %d, the operation was built for %d", what, i,
-                  ins[i].dtype & ~THX_HOST_SCALAR, dtypes[i]);
+                  ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX), dtypes[i]);
     for (int d = 0; d < nd; ++d) {
       const int64_t s = ins[i].shape[d];
       if (s < 0) return fail(THX_ERR_ARG, "%s: negative extent", what);
@@ -173,9 +173,17 @@ int gather_inputs(const char* what, const thx_array* ins, int n_in, const int32_
   for (int i = 0; i < n_in; ++i) {
     View& v = (*views)[i];
     v.ptr = (char*)ins[i].base + ins[i].offset_bytes;
-    v.dtype = ins[i].dtype & ~THX_HOST_SCALAR;
+    v.dtype = ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX);
     const int isz = dtype_size(v.dtype);
     if (!isz) return fail(THX_ERR_TYPE, "%s: unknown dtype code %d", what, v.dtype);
+    if (ins[i].dtype & THX_INDEX) {  // no memory behind it; the caller that supports it fills in the multipliers
+      if (v.dtype != THX_I64) return fail(THX_ERR_TYPE, "%s: index operand %d must be int64", what, i);
+      for (int d = 0; d < nd; ++d)
+        if (ins[i].shape[d] != 1) return fail(THX_ERR_TYPE, "%s: index operand %d must have extent 1 everywhere", what, i);
+      v.ptr = nullptr;
+      v.iota = true;
+      continue;
+    }
     if (ins[i].dtype & THX_HOST_SCALAR) {
       for (int d = 0; d < nd; ++d)
         if (ins[i].shape[d] != 1) return fail(THX_ERR_TYPE, "%s: host scalar input %d must have extent 1 everywhere", what, i);

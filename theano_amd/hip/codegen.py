@@ -190,3 +190,60 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
     text = "\n".join(lines)
     name = _name("R", text)
     return "struct %s {\n%s\n};\n" % (name, text), name, acc_struct_bytes(acc_dtypes)
+
+
+def argmax_functor(in_dtypes, value_dtype, pre_op=None):
+    """(source, name, sizeof(Acc)) of the reduction behind ``MaxAndArgmax``.
+
+    The inputs are ``in_dtypes`` followed by one int64 position operand (the
+    library's index operand: the element's position within the reduced
+    dimensions).  ``pre_op`` (default: the single input itself) gives the value;
+    the accumulator is the pair (value, position).  Merging keeps the greater
+    value, a NaN before any number, and on equal values (or two NaNs) the smaller
+    position - so the result is NumPy's first occurrence whatever order partial
+    results meet in."""
+    nin = len(in_dtypes)
+    ins = ["i%d" % k for k in range(nin)]
+    vt = compute_ctype(value_dtype)
+    lines = ["  enum { NIN = %d, NOUT = 2, NEX = 0 };" % (nin + 1)]
+    lines.append("  struct Acc { %s val; long long idx; };" % vt)
+    lines.append(_regs(list(in_dtypes) + ["int64"], ins + ["ix"]).rstrip("\n"))
+    if value_dtype in scal.float_dtypes:
+        lowest = c_literal(-np.inf, value_dtype)
+    elif value_dtype == "bool":
+        lowest = c_literal(0, value_dtype)
+    else:
+        lowest = c_literal(np.iinfo(value_dtype).min, value_dtype)
+    lines.append("  THX_DEV static void init(Acc& a) { a.val = %s; a.idx = 0x7fffffffffffffffLL; }" % lowest)
+    lines.append("  template <int V, class A> THX_DEV static void load(const A& a, Regs<V>& r) { %s a.template ld<%d>(r.ix); }"
+                 % (" ".join("a.template ld<%d>(r.%s);" % (k, nm) for k, nm in enumerate(ins)), nin))
+    if pre_op is None:
+        if nin != 1:
+            raise ValueError("without prologue the reduction takes one input")
+        pre_stmt = "v.val = (%s)i0;" % vt
+    else:
+        pnode = _scalar_node(pre_op, in_dtypes)
+        if len(pnode.outputs) != 1 or pnode.outputs[0].type.dtype != value_dtype:
+            raise TypeError("prologue must yield one %s value" % value_dtype)
+        pre_stmt = "%s p0;\n%s\nv.val = (%s)p0;" % (vt, pre_op.c_code(pnode, ins, ["p0"]), vt)
+    lines.append("  THX_DEV static void pre(%s, const long long ix, Acc& v) {\n%s\n    v.idx = ix;\n  }" % (
+        ", ".join("const %s %s" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)), _indent(pre_stmt, 4)))
+    nan_a, nan_b = ("a.val != a.val", "b.val != b.val") if value_dtype in scal.float_dtypes else ("false", "false")
+    lines.append("  THX_DEV static void comb(Acc& a, const Acc& b) {\n"
+                 "    const bool an = %s, bn = %s;\n"
+                 "    const bool take = bn ? (!an || b.idx < a.idx)\n"
+                 "                         : (!an && (b.val > a.val || (b.val == a.val && b.idx < a.idx)));\n"
+                 "    if (take) a = b;\n  }" % (nan_a, nan_b))
+    call = ", ".join(["(%s)r.%s.v[k]" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)] + ["r.ix.v[k]"])
+    lines.append("  template <int V> THX_DEV static void accum(Acc& s, const Regs<V>& r) {\n#pragma unroll\n"
+                 "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s, t); }\n  }" % call)
+    lines.append("  template <int V> THX_DEV static void accum_lanes(Acc* s, const Regs<V>& r) {\n#pragma unroll\n"
+                 "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s[k], t); }\n  }" % call)
+    lines.append("  THX_DEV static Acc shfl_xor(const Acc& a, int m) { Acc r; r.val = thx::shfl_xor_t(a.val, m); "
+                 "r.idx = thx::shfl_xor_t(a.idx, m); return r; }")
+    st = storage_ctype(value_dtype)
+    lines.append("  template <class O> THX_DEV static void post(const O& o, long long idx, const Acc& a) {\n"
+                 "    ((%s*)o.ptr[0])[idx] = (%s)a.val;\n    ((long long*)o.ptr[1])[idx] = a.idx;\n  }" % (st, st))
+    text = "\n".join(lines)
+    name = _name("A", text)
+    return "struct %s {\n%s\n};\n" % (name, text), name, 16

@@ -17,7 +17,7 @@ from ..gof import Apply, Op, Type, Variable
 from ..tensor.elemwise import CAReduce, DimShuffle, Elemwise
 from ..tensor.type import TensorType, _tensor_py_operators
 from . import codegen
-from .runtime import HipArray, call_flags, check, host_scalar_thx, lib, thx_array
+from .runtime import THX_INDEX, HipArray, call_flags, check, host_scalar_thx, lib, thx_array
 
 
 class HipArrayType(Type):
@@ -451,3 +451,98 @@ class HipCAReduce(CAReduce):
             check(rc)
         for k, arr in enumerate(results):
             output_storage[k][0] = arr
+
+
+_argmax_handles = {}
+
+
+class HipMaxAndArgmax(Op):
+    """``MaxAndArgmax`` on the device (the role of ``GpuMaxAndArgmax``,
+    ``theano/gpuarray/reduction.py:14-137``): one pass of the reduction kernels
+    over (value, position) pairs; the position comes from the library's index
+    operand, so no index array exists in memory.  ``pre_scalar_op`` (one output)
+    is an elementwise producer computed on the fly, e.g. the negation ``argmin``
+    puts in front."""
+
+    __props__ = ("axis", "pre_scalar_op")
+
+    def __init__(self, axis, pre_scalar_op=None):
+        self.axis = tuple(sorted(int(a) for a in axis))
+        self.pre_scalar_op = pre_scalar_op
+
+    def _props(self):
+        return (self.axis, self.pre_scalar_op)
+
+    def __str__(self):
+        pre = "" if self.pre_scalar_op is None else ", pre=%s" % self.pre_scalar_op
+        return "HipMaxAndArgmax{%s%s}" % (", ".join(map(str, self.axis)), pre)
+
+    def make_node(self, *inputs):
+        ins = [i if (isinstance(i.type, HipArrayType) or _is_host_scalar(i)) else as_hip_variable(i) for i in inputs]
+        nd = max(i.type.ndim for i in ins)
+        if any(i.type.ndim != nd for i in ins if isinstance(i.type, HipArrayType)):
+            raise TypeError("HipMaxAndArgmax inputs must share one rank")
+        if self.pre_scalar_op is None:
+            if len(ins) != 1:
+                raise TypeError("without prologue the reduction takes exactly one input")
+            vdt = ins[0].type.dtype
+        else:
+            vdt = self.pre_scalar_op.make_node(*[scal.Scalar(i.type.dtype)() for i in ins]).outputs[0].type.dtype
+        for a in self.axis:
+            if a < 0 or a >= nd:
+                raise ValueError("MaxAndArgmax: bad axis argument")
+        bcast = [all(b) for b in zip(*[i.type.broadcastable for i in ins if i.type.ndim == nd])]
+        ob = [b for d, b in enumerate(bcast) if d not in self.axis]
+        return Apply(self, ins, [HipArrayType(vdt, ob)(), HipArrayType("int64", ob)()])
+
+    def infer_shape(self, node, shapes):
+        nd = max(len(s) for s in shapes)
+        full = [max(s[d] for s in shapes if len(s) == nd) for d in range(nd)]
+        kept = tuple(full[d] for d in range(nd) if d not in self.axis)
+        return [kept, kept]
+
+    def _handle(self, node):
+        in_dt = tuple(i.type.dtype for i in node.inputs)
+        vdt = node.outputs[0].type.dtype
+        key = (self._props(), in_dt)
+        h = _argmax_handles.get(key)
+        if h is None:
+            src, name, acc_bytes = codegen.argmax_functor(in_dt, vdt, self.pre_scalar_op)
+            all_dt = in_dt + ("int64", vdt, "int64")
+            codes = (ctypes.c_int32 * len(all_dt))(*[scal.dtype_code(d) for d in all_dt])
+            handle = ctypes.c_void_p()
+            check(lib.thx_reduce_new(src.encode(), name.encode(), len(in_dt) + 1, 2, 0, codes, acc_bytes,
+                                     ctypes.byref(handle)))
+            h = _argmax_handles[key] = handle
+        return h
+
+    def perform(self, node, inputs, output_storage):
+        cache = node.tag.get("thx")
+        if cache is None:
+            handle = self._handle(node)
+            nin = len(node.inputs)
+            nd = max(i.type.ndim for i in node.inputs)
+            ins = (thx_array * (nin + 1))()
+            ix = ins[nin]                       # the index operand: int64, extent 1 everywhere, no memory
+            ix.base, ix.offset_bytes, ix.nd, ix.dtype = None, 0, nd, scal.dtype_code("int64") | THX_INDEX
+            for d in range(nd):
+                ix.shape[d], ix.strides_bytes[d] = 1, 0
+            mask = (ctypes.c_uint8 * max(nd, 1))(*[1 if d in self.axis else 0 for d in range(nd)])
+            cache = node.tag["thx"] = (handle, nin, ins, (thx_array * 2)(), nd, mask,
+                                       np.dtype(node.outputs[0].type.dtype))
+        handle, nin, ins, outs, nd, mask, vdt = cache
+        shape = _check_runtime_broadcast(node.inputs, inputs, nd)
+        if any(shape[a] == 0 for a in self.axis):
+            raise ValueError("attempt to get argmax of an empty sequence")
+        for k, v in enumerate(inputs):
+            _operand(v, nd, ins[k])
+        kept = tuple(shape[d] for d in range(nd) if d not in self.axis)
+        mx = HipArray._new_contiguous(kept, vdt)
+        am = HipArray._new_contiguous(kept, np.dtype("int64"))
+        mx.as_thx(outs[0])
+        am.as_thx(outs[1])
+        rc = lib.thx_reduce_call(handle, ins, mask, outs, call_flags(node))
+        if rc:
+            check(rc)
+        output_storage[0][0] = mx
+        output_storage[1][0] = am

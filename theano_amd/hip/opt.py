@@ -19,7 +19,8 @@ from ..gof import Constant, FunctionGraph
 from ..tensor import basic as T
 from ..tensor.elemwise import All, Any, CAReduce, CAReduceDtype, DimShuffle, Elemwise
 from ..tensor.type import TensorConstant, TensorType
-from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipToHost, HostToHip, _is_host_scalar,
+from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipMaxAndArgmax, HipToHost, HostToHip,
+                  _is_host_scalar,
                   as_hip_variable, hip_from_host, host_from_hip)
 from .runtime import HipArray
 
@@ -78,7 +79,7 @@ def lift_to_hip(fgraph):
     for node in fgraph.toposort():
         ins = [mapped(i) for i in node.inputs]
         op = node.op
-        if isinstance(op, (HipElemwise, HipCAReduce, HipDimShuffle, HostToHip, HipToHost, T.ShapeFloat)):
+        if isinstance(op, (HipElemwise, HipCAReduce, HipMaxAndArgmax, HipDimShuffle, HostToHip, HipToHost, T.ShapeFloat)):
             if isinstance(op, HostToHip) and isinstance(ins[0].type, HipArrayType):
                 outs = [ins[0]]
             elif isinstance(op, HipToHost) and isinstance(ins[0].type, TensorType):
@@ -99,6 +100,8 @@ def lift_to_hip(fgraph):
             if not isinstance(x.type, HipArrayType):
                 x = as_hip_variable(x)
             outs = [_lift_reduce(node, x)]
+        elif isinstance(op, T.MaxAndArgmax):
+            outs = HipMaxAndArgmax(op.axis).make_node(ins[0]).outputs
         else:
             raise NotImplementedError("%s has no HIP implementation and nothing runs on the host" % op)
         for o, no in zip(node.outputs, outs):
@@ -338,6 +341,46 @@ def fuse_reduce_prologue(fgraph):
             count += 1
             changed = True
             break
+    return count
+
+
+def fuse_argmax_prologue(fgraph):
+    """``max_and_argmax(f(a, b, ...))`` computes f on the fly when nothing else
+    reads f's result (``argmin`` is ``argmax(-x)``)."""
+    count = 0
+    for node in fgraph.toposort():
+        op = node.op
+        if not isinstance(op, HipMaxAndArgmax) or op.pre_scalar_op is not None or len(node.inputs) != 1:
+            continue
+        x = node.inputs[0]
+        p = x.owner
+        if (p is None or not isinstance(p.op, HipElemwise) or len(p.outputs) != 1 or p.op.inplace_pattern or
+                fgraph.n_clients(x) != 1):
+            continue
+        if any(isinstance(i.type, HipArrayType) and i.type.ndim != x.type.ndim for i in p.inputs):
+            continue
+        inputs, s_inputs, s_args = [], [], []
+        for v in p.inputs:
+            c = _scalar_constant(v)
+            if c is not None:
+                s_args.append(c)
+                continue
+            if v in inputs:
+                s_args.append(s_inputs[inputs.index(v)])
+                continue
+            sv = scal.Scalar(v.type.dtype)()
+            inputs.append(v)
+            s_inputs.append(sv)
+            s_args.append(sv)
+        if not inputs or len(inputs) > config.max_fused_inputs:
+            continue
+        pre = scal.Composite(s_inputs, [p.op.scalar_op(*s_args)])
+        new_node = HipMaxAndArgmax(op.axis, pre).make_node(*inputs)
+        if [o.type for o in new_node.outputs] != [o.type for o in node.outputs]:
+            continue
+        for o, no in zip(node.outputs, new_node.outputs):
+            fgraph.replace(o, no)
+        count += 1
     return count
 
 
@@ -605,6 +648,7 @@ def optimize(fgraph, fuse=True, rowchain=True, inplace=True):
         merge_sibling_reductions(fgraph)
         gof.merge_identical(fgraph)
         fuse_reduce_epilogue(fgraph)
+        fuse_argmax_prologue(fgraph)
         gof.merge_identical(fgraph)
     if inplace:
         inplace_elemwise(fgraph)

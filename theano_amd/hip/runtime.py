@@ -21,6 +21,7 @@ THX_BROADCAST = 1
 THX_DRY_RUN = 2
 THX_KEEP_CACHED = 4
 THX_HOST_SCALAR = 0x100
+THX_INDEX = 0x200
 
 
 class thx_array(ctypes.Structure):

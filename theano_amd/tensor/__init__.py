@@ -10,4 +10,4 @@ for _n in dir(_type):  # bscalar ... dtensor4 and friends
         globals()[_n] = getattr(_type, _n)
 from .elemwise import DimShuffle, Elemwise, CAReduce, CAReduceDtype, Sum, Prod, All, Any
 from .basic import *  # noqa: F401,F403
-from .basic import Max, Min, ShapeFloat, makeKeepDims, cast, round  # noqa: F401
+from .basic import Max, MaxAndArgmax, Min, ShapeFloat, makeKeepDims, cast, round  # noqa: F401

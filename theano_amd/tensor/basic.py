@@ -231,6 +231,99 @@ class Min(CAReduce):
     L_op = Max.L_op
 
 
+class MaxAndArgmax(Op):
+    """Maximum and the position of its first occurrence over ``axis`` (a sorted
+    tuple of axes) - ``theano/tensor/basic.py:1273-1483``.  The second output is
+    int64: the index ``numpy.argmax`` gives once the reduced axes are moved to the
+    end, in their original order, and flattened (``perform``, :1311-1330).  A NaN
+    is the maximum and its position the argmax, as with NumPy."""
+
+    __props__ = ("axis",)
+
+    def __init__(self, axis):
+        self.axis = tuple(sorted(int(a) for a in axis))
+
+    def _props(self):
+        return (self.axis,)
+
+    def __str__(self):
+        return "MaxAndArgmax{%s}" % ", ".join(map(str, self.axis))
+
+    def make_node(self, x):
+        x = as_tensor_variable(x)
+        for a in self.axis:
+            if a < 0 or a >= x.type.ndim:
+                raise ValueError("MaxAndArgmax: bad axis argument")
+        if not self.axis:
+            raise ValueError("MaxAndArgmax needs at least one axis")
+        b = [bb for i, bb in enumerate(x.type.broadcastable) if i not in self.axis]
+        return Apply(self, [x], [TensorType(x.type.dtype, b)(), TensorType("int64", b)()])
+
+    def infer_shape(self, node, shapes):
+        kept = tuple(s for i, s in enumerate(shapes[0]) if i not in self.axis)
+        return [kept, kept]
+
+    def perform(self, node, inputs, output_storage):
+        raise NotImplementedError("MaxAndArgmax runs on the device only; compile the graph with function()")
+
+    def connection_pattern(self, node):
+        return [[True, False]]
+
+    def L_op(self, inp, out, grads):
+        # theano/tensor/basic.py:1429-1483: the gradient flows to the positions that equal the maximum
+        (x,) = inp
+        g_max = grads[0]
+        if g_max is None or isinstance(getattr(g_max, "type", None), scal.DisconnectedType):
+            return [x.zeros_like()]
+        if x.type.dtype in discrete_dtypes:
+            return [x.zeros_like(dtype=config.floatX)]
+        pattern, k = [], 0
+        for i in range(x.type.ndim):
+            if i in self.axis:
+                pattern.append("x")
+            else:
+                pattern.append(k)
+                k += 1
+        g_max_pad = DimShuffle(g_max.type.broadcastable, pattern)(g_max)
+        xmax_pad = DimShuffle(out[0].type.broadcastable, pattern)(out[0])
+        return [eq(xmax_pad, x) * g_max_pad]
+
+
+def max_and_argmax(a, axis=None, keepdims=False):
+    """``[max, argmax]`` over ``axis`` (None: all axes) -
+    ``theano/tensor/basic.py:1651-1680``."""
+    a = as_tensor_variable(a)
+    if a.type.ndim == 0:                      # nothing to reduce: the value itself, at position 0
+        return [a, constant(0, dtype="int64")]
+    ax = sorted(set(d + a.type.ndim if d < 0 else d for d in _axis_list(axis, a.type.ndim)))
+    if not ax:
+        ax = list(range(a.type.ndim))
+    out, argout = MaxAndArgmax(ax)(a)
+    if keepdims:
+        out = makeKeepDims(a, out, ax)
+        argout = makeKeepDims(a, argout, ax)
+    return [out, argout]
+
+
+def argmax(x, axis=None, keepdims=False):
+    return max_and_argmax(x, axis, keepdims)[1]
+
+
+def argmin(x, axis=None, keepdims=False):
+    """``argmax`` of the order-reversed values, as the reference does
+    (``theano/tensor/basic.py:1779-1803``): ``-x``, ``max - x`` for unsigned
+    integers, ``~x`` for bool."""
+    x = as_tensor_variable(x)
+    dt = x.type.dtype
+    if dt in scal.float_dtypes or dt in scal.int_dtypes:
+        return argmax(-x, axis=axis, keepdims=keepdims)
+    if dt in scal.uint_dtypes:
+        return argmax(np.array(np.iinfo(dt).max, dtype=dt) - x, axis=axis, keepdims=keepdims)
+    if dt == "bool":
+        return argmax(~x, axis=axis, keepdims=keepdims)
+    raise NotImplementedError(dt)
+
+
 def max(x, axis=None, keepdims=False):
     x = as_tensor_variable(x)
     out = Max(axis)(x)

@@ -260,6 +260,18 @@ def local_sum_invariant_factor(fgraph, node):
     return [new]
 
 
+@local_optimizer([T.MaxAndArgmax])
+def local_max_and_argmax(fgraph, node):
+    """When nothing reads the argmax, the node is a plain ``max`` reduction
+    (``local_max_and_argmax``, ``theano/tensor/opt_uncanonicalize.py:51-68``)."""
+    if fgraph.n_clients(node.outputs[1]) != 0 or node.outputs[1] in fgraph.outputs:
+        return False
+    new = T.Max(node.op.axis)(node.inputs[0])
+    if new.type != node.outputs[0].type:
+        return False
+    return [new, None]
+
+
 @local_optimizer([T.ShapeFloat])
 def local_shape_lift(fgraph, node):
     """The extent of an elementwise / DimShuffle / reduction result is the extent
@@ -289,7 +301,7 @@ def local_shape_lift(fgraph, node):
 
 
 CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_useless_elemwise, local_fill_sink, local_useless_reduce,
-                local_dimshuffle_lift, local_sum_invariant_factor]
+                local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax]
 
 
 def canonicalize(fgraph):
