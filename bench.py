@@ -24,8 +24,6 @@ import os
 import sys
 import time
 
-import numpy as np
-
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each

@@ -62,6 +62,13 @@ enum {
  * (theano/tensor/basic.py:1311-1330). It costs no memory traffic. */
 #define THX_INDEX 0x200
 
+/* OR-ed into thx_array.dtype of an input or an output of a kernel call: one of the next calls reads
+ * this array (again). It is then accessed with ordinary loads / stores, so that the 256 MB
+ * last-level cache can serve the next read; arrays without the flag are streamed with
+ * non-temporal accesses wherever that is the faster choice for the call. A hint only: results
+ * never depend on it. */
+#define THX_REUSED 0x400
+
 /* A strided view of device memory (counterpart of libgpuarray's GpuArray:
  * data, offset, nd, dimensions, byte strides, typecode). Strides may be zero
  * or negative; they must be multiples of the element size. */
@@ -118,9 +125,6 @@ int thx_elemwise_new(const char* functor_src, const char* functor_name, int n_in
 #define THX_BROADCAST 1 /* size-1 input dimensions broadcast against larger ones */
 #define THX_DRY_RUN 2   /* validate, plan and compile (into the disk cache) but do not launch;
                            needs no device: the target is $THX_ARCH, default gfx950 */
-#define THX_KEEP_CACHED 4 /* an operand of this call is read again by one of the next calls (or its
-                           result is): no non-temporal accesses, so that the 256 MB last-level
-                           cache can serve the second read */
 
 /* Run on `ins` (n_in arrays) writing `outs` (n_out arrays, preallocated, every
  * one of the full result shape; an output may alias an input exactly for

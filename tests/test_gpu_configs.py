@@ -88,3 +88,27 @@ def test_config5_batchnorm_float16():
     xc = x[:, ch].astype("float64")
     ref = gamma.astype("float64")[0, ch] * (xc - xc.mean()) / np.sqrt(xc.var() + 1e-5) + beta.astype("float64")[0, ch]
     assert_parity(y[:, ch], ref.astype("float16"), "c5 full channel", tol)
+
+
+def test_nnet_row_functions_run_as_row_chains():
+    """softmax_with_bias / logsoftmax / relu of tensor.nnet against the oracle's
+    node-by-node evaluation of the same formulas (the ops' perform code,
+    theano/tensor/nnet/nnet.py:440-446, 628-633, 2209-2252), forward and gradient."""
+    from theano_amd.hip import HipRowChain
+    rng = np.random.default_rng(41)
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    b = T.fvector("b")
+    xv = (3 * rng.standard_normal((130, 777))).astype("float32")
+    yv = rng.uniform(0, 1, (130, 777)).astype("float32")
+    bv = rng.standard_normal(777).astype("float32")
+    lsm = T.nnet.logsoftmax(x)
+    swb = T.nnet.softmax_with_bias(x, b)
+    outs = [lsm, swb, T.nnet.relu(x), T.nnet.relu(x, 0.1), th.grad(T.sum(lsm * y), x), th.grad(T.sum(swb * y), b)]
+    f = th.function([x, y, b], outs)
+    assert any(isinstance(n.op, HipRowChain) for n in f.toposort())
+    got = f(xv, yv, bv)
+    ref = G.evaluate([x, y, b], outs, [xv, yv, bv])
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "nnet output %d" % k, tol=dict(rtol=2e-5, atol=2e-6))
+    assert np.allclose(np.exp(got[0]).sum(axis=1), 1.0, atol=1e-5)
+    assert np.allclose(got[1].sum(axis=1), 1.0, atol=1e-5)

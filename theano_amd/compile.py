@@ -81,11 +81,12 @@ class Function(object):
         self._prepare()
 
     def _mark_reuse(self):
-        """``node.tag['keep_cached']`` for every kernel node that reads a full-sized array which a
-        later kernel of this function reads again, or whose result a later kernel reads: those
-        calls must not use non-temporal accesses, the later read can then come from the
-        last-level cache (a batch-norm pass over 100 MB of activations after the statistics
-        pass, for instance)."""
+        """For every kernel node, the positions of the full-sized inputs that a later kernel of
+        this function reads again (``node.tag['reused_in']``) and of the outputs that a later
+        kernel reads (``node.tag['reused_out']``).  The ops pass them on as THX_REUSED, which
+        keeps those arrays out of non-temporal accesses so that the last-level cache can serve
+        the next read (a batch-norm pass over 100 MB of activations after the statistics pass,
+        a reduction over an elementwise result that is also an output)."""
         from .hip.ops import HipArrayType, HipDimShuffle
 
         def root(v):
@@ -96,13 +97,13 @@ class Function(object):
         def big(v):
             return isinstance(v.type, HipArrayType) and v.type.ndim > 0 and not any(v.type.broadcastable)
 
-        kernels = [n for n in self.nodes if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax")]
+        kernels = [n for n in self.nodes
+                   if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax")]
         later = set()
         for node in reversed(kernels):
-            mine = set(id(root(i)) for i in node.inputs if big(i))
-            outs = set(id(o) for o in node.outputs if big(o))
-            node.tag["keep_cached"] = bool((mine | outs) & later)
-            later |= mine
+            node.tag["reused_in"] = tuple(k for k, i in enumerate(node.inputs) if big(i) and id(root(i)) in later)
+            node.tag["reused_out"] = tuple(k for k, o in enumerate(node.outputs) if big(o) and id(o) in later)
+            later |= set(id(root(i)) for i in node.inputs if big(i))
 
     def _prepare(self):
         from .hip.opt import DeviceConstant

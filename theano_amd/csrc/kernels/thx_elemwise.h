@@ -7,8 +7,8 @@
 //   template <int V> static void compute(Regs<V>&);     // the scalar graph, V times
 //   template <int V, class A> static void store(const A&, const Regs<V>&);
 // and a generated plan P supplies
-//   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK, NT (non-temporal accesses),
-//                                     GS (grid-stride loop over chunks) };
+//   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK, GS (grid-stride loop over chunks) };
+//   static constexpr unsigned long long NT;             // bit i: operand i is accessed non-temporally
 //   static constexpr int mode(int operand);             // M_VEC / M_BCAST / M_GATHER
 // The host collapses dimensions, so ND is the rank after merging every pair of
 // neighbouring dimensions that all operands walk with compatible strides.
@@ -46,7 +46,7 @@ struct EwAcc {
     if (N == 1) {
       r.v[0] = *b;
     } else if (P::mode(I) == M_VEC) {
-      load_vec<T, N, P::NT != 0>(r, b);
+      load_vec<T, N, ((P::NT >> I) & 1) != 0>(r, b);
     } else if (P::mode(I) == M_BCAST) {
       const T s = *b;
 #pragma unroll
@@ -64,7 +64,7 @@ struct EwAcc {
     if (N == 1) {
       *b = r.v[0];
     } else if (P::mode(I) == M_VEC) {
-      store_vec<T, N, P::NT != 0>(b, r);
+      store_vec<T, N, ((P::NT >> I) & 1) != 0>(b, r);
     } else {
       const IT st = stride[I][P::ND - 1];
 #pragma unroll
@@ -175,7 +175,7 @@ struct TrStageAcc {  // global -> LDS for the staged inputs, nothing for the oth
     if (P::slot(I) >= 0) {
       T* tile = (T*)(lds + P::slot(I) * (P::TILE * (P::TILE + 1) * P::ESZ));
       Vec<T, N> r;
-      load_vec<T, N, P::NT != 0>(r, (const T*)ptr[I] + off[I]);
+      load_vec<T, N, ((P::NT >> I) & 1) != 0>(r, (const T*)ptr[I] + off[I]);
 #pragma unroll
       for (int k = 0; k < N; ++k) tile[cell + k] = r.v[k];
     }
@@ -205,12 +205,12 @@ struct TrAcc {  // LDS (transposed) or global -> registers, registers -> global
 #pragma unroll
       for (int k = 0; k < N; ++k) r.v[k] = s;
     } else {
-      load_vec<T, N, P::NT != 0>(r, (const T*)ptr[I] + off[I]);
+      load_vec<T, N, ((P::NT >> I) & 1) != 0>(r, (const T*)ptr[I] + off[I]);
     }
   }
   template <int I, class T, int N>
   THX_DEV void st(const Vec<T, N>& r) const {
-    store_vec<T, N, P::NT != 0>((T*)ptr[I] + off[I], r);
+    store_vec<T, N, ((P::NT >> I) & 1) != 0>((T*)ptr[I] + off[I], r);
   }
 };
 

@@ -78,7 +78,7 @@ struct RedAcc {
     if (N == 1) {
       r.v[0] = *b;
     } else if (P::mode(I) == M_VEC) {
-      load_vec<T, N, P::NT != 0>(r, b);
+      load_vec<T, N, ((P::NT >> I) & 1) != 0>(r, b);
     } else if (P::mode(I) == M_BCAST) {
       const T s = *b;
 #pragma unroll

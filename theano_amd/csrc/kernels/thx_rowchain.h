@@ -26,7 +26,8 @@ struct RowChainParams {
   IT out_rstride[NOUT];
 };
 
-// Plan members: typedef IT; enum { VEC, NCH, TPR, BLOCK, NT }; static constexpr int imm(int input).
+// Plan members: typedef IT; enum { VEC, NCH, TPR, BLOCK }; static constexpr unsigned long long NT, NTO (bit i:
+// input / output i is accessed non-temporally); static constexpr int imm(int input).
 template <class C, class P>
 struct RowCtx {
   typedef typename P::IT IT;
@@ -53,7 +54,7 @@ struct RowCtx {
       Vec<T, VEC> r;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) r.v[k] = T();
-      if (valid(ch)) load_vec<T, VEC, P::NT != 0>(r, base + (IT)(ch * TPR + lane) * VEC);
+      if (valid(ch)) load_vec<T, VEC, ((P::NT >> I) & 1) != 0>(r, base + (IT)(ch * TPR + lane) * VEC);
 #pragma unroll
       for (int k = 0; k < VEC; ++k) v[ch][k] = (CT)r.v[k];
     }
@@ -82,7 +83,7 @@ struct RowCtx {
       Vec<T, VEC> r;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) r.v[k] = (T)v[ch][k];
-      if (live && valid(ch)) store_vec<T, VEC, P::NT != 0>(base + (IT)(ch * TPR + lane) * VEC, r);
+      if (live && valid(ch)) store_vec<T, VEC, ((P::NTO >> O) & 1) != 0>(base + (IT)(ch * TPR + lane) * VEC, r);
     }
   }
   template <int O, class T, class CT>

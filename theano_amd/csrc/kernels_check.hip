@@ -47,20 +47,20 @@ struct CheckR {
   }
 };
 
-struct PlanEw1 { typedef int IT; enum { ND = 1, VEC = 4, UNR = 2, BLOCK = 256, NT = 1, GS = 1 };
+struct PlanEw1 { typedef int IT; enum { ND = 1, VEC = 4, UNR = 2, BLOCK = 256, GS = 1 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {0, 3, 0}; return m[i]; } };
-struct PlanEw3 { typedef long long IT; enum { ND = 3, VEC = 2, UNR = 1, BLOCK = 256, NT = 1, GS = 0 };
+struct PlanEw3 { typedef long long IT; enum { ND = 3, VEC = 2, UNR = 1, BLOCK = 256, GS = 0 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {2, 1, 0}; return m[i]; } };
-struct PlanRow { typedef int IT; enum { NK = 2, VEC = 4, UNR = 4, BLOCK = 256, TPR = 256, RA2 = 1, NT = 0 };
+struct PlanRow { typedef int IT; enum { NK = 2, VEC = 4, UNR = 4, BLOCK = 256, TPR = 256, RA2 = 1 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {0}; return m[i]; } };
-struct PlanRowS { typedef int IT; enum { NK = 1, VEC = 1, UNR = 1, BLOCK = 256, TPR = 16, RA2 = 0, NT = 1 };
+struct PlanRowS { typedef int IT; enum { NK = 1, VEC = 1, UNR = 1, BLOCK = 256, TPR = 16, RA2 = 0 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; } };
-struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, TX = 64, RR2 = 1, NT = 1 };
+struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, TX = 64, RR2 = 1 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {0}; return m[i]; } };
-struct PlanGen { typedef int IT; enum { NK = 3, NR = 3, BLOCK = 256, TPR = 64, NT = 0 };
+struct PlanGen { typedef int IT; enum { NK = 3, NR = 3, BLOCK = 256, TPR = 64 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; } };
 
-struct PlanTr { typedef int IT; enum { ND = 3, TILE = 64, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2, NT = 0 };
+struct PlanTr { typedef int IT; enum { ND = 3, TILE = 64, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2, 0, 0}; return m[i]; }
   static constexpr int slot(int i) { constexpr int m[] = {0, -1, -1}; return m[i]; } };
 extern "C" __global__ __launch_bounds__(256) void check_tr(thx::EwTrParams<3, 3, int> p) { thx::ew_tr_body<CheckF, PlanTr>(p); }

@@ -110,12 +110,14 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
     const thx_array& a = outs[o];
     View& v = views[e->n_in + o];
     if (a.nd != nd) return fail(THX_ERR_TYPE, "elemwise: output %d has rank %d, expected %d", o, a.nd, nd);
-    if (a.dtype != e->dtypes[e->n_in + o])
-      return fail(THX_ERR_TYPE, "elemwise: output %d has dtype code %d, the operation was built for %d", o, a.dtype,
+    const int adt = a.dtype & ~THX_REUSED;
+    if (adt != e->dtypes[e->n_in + o])
+      return fail(THX_ERR_TYPE, "elemwise: output %d has dtype code %d, the operation was built for %d", o, adt,
                   e->dtypes[e->n_in + o]);
-    const int isz = dtype_size(a.dtype);
+    const int isz = dtype_size(adt);
     v.ptr = (char*)a.base + a.offset_bytes;
-    v.dtype = a.dtype;
+    v.dtype = adt;
+    v.reused = (a.dtype & THX_REUSED) != 0;
     if (((uintptr_t)v.ptr) % isz) return fail(THX_ERR_TYPE, "elemwise: output %d is not aligned to its element size", o);
     for (int d = 0; d < nd; ++d) {
       if (a.shape[d] != shape[d])
@@ -247,9 +249,11 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
       if (env_int("THX_EW_TV", 0) == 1) tv = 1;
       if ((int64_t)ntr * tile * (tile + 1) * esz <= 60000) {
         const int block = 256;
-        const int nt = nt_streaming(moved, flags);
+        const uint64_t nt = nt_mask(nt_streaming(moved), views);
         std::ostringstream key;
-        key << "et|nd" << ND << "|t" << tile << "|v" << tv << "|n" << ntr << "|e" << esz << (nt ? "|nt" : "") << "|m";
+        key << "et|nd" << ND << "|t" << tile << "|v" << tv << "|n" << ntr << "|e" << esz;
+        if (nt) key << "|nt" << std::hex << nt << std::dec;
+        key << "|m";
         for (int o = 0; o < nops; ++o) key << (slot[o] >= 0 ? 9 : mode[o]) << (o + 1 < nops ? "," : "");
         const std::string plan = key.str() + (fast_div() ? "|fd" : "");
         set_last_plan(e->name + "|" + plan);
@@ -261,8 +265,8 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
           const std::string entry = entry_name(e->name, plan);
           std::ostringstream s;
           s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef int IT;\n  enum { ND = " << ND
-            << ", TILE = " << tile << ", TV = " << tv << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz << ", NT = " << nt
-            << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+            << ", TILE = " << tile << ", TV = " << tv << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz
+            << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
           for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
           s << "};\n    return m[i];\n  }\n  static constexpr int slot(int i) {\n    constexpr int m[] = {";
           for (int o = 0; o < nops; ++o) s << slot[o] << (o + 1 < nops ? ", " : "");
@@ -313,13 +317,14 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   int block = 256;
   const int force_block = env_int("THX_EW_BLOCK", 0);
   if (force_block == 128 || force_block == 512 || force_block == 1024) block = force_block;
-  const int nt = nt_streaming(moved, flags);
+  const uint64_t nt = nt_mask(nt_streaming(moved), views);
   // grid-stride: a bounded number of blocks walk the index space instead of one block per chunk
   const int gs = env_int("THX_EW_GS", 0);
 
   std::ostringstream key;
-  key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nt ? "|nt" : "") << (block != 256 ? "|b" + std::to_string(block) : "")
-      << (gs ? "|gs" : "") << "|m";
+  key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr;
+  if (nt) key << "|nt" << std::hex << nt << std::dec;
+  key << (block != 256 ? "|b" + std::to_string(block) : "") << (gs ? "|gs" : "") << "|m";
   for (int o = 0; o < nops; ++o) key << mode[o] << (o + 1 < nops ? "," : "");
   const std::string plan = key.str() + (fast_div() ? "|fd" : "");
   set_last_plan(e->name + "|" + plan);
@@ -333,7 +338,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
     std::ostringstream s;
     s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
       << " IT;\n  enum { ND = " << ND << ", VEC = " << vec << ", UNR = " << unr << ", BLOCK = " << block
-      << ", NT = " << nt << ", GS = " << (gs ? 1 : 0) << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+      << ", GS = " << (gs ? 1 : 0) << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
     for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
     s << "};\n    return m[i];\n  }\n};\n"
       << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::EwParams<" << e->name

@@ -49,13 +49,12 @@ struct Kernel {
 int get_kernel(const std::string& source, const std::string& entry, Kernel* out);
 // True (default; $THX_FAST_DIV=0 turns it off) when float32 division / sqrt are compiled to the 2.5-ulp forms.
 bool fast_div();
-// Non-temporal accesses: $THX_NT when set; never when the call's flags say that an operand is read
-// again soon (THX_KEEP_CACHED); else the default of the kernel family (measured per family).
-int nt_choice(int family_default, int flags);
+// Non-temporal accesses: $THX_NT when set, else the default of the kernel family (measured per family).
+int nt_choice(int family_default);
 // Elementwise and row-chain kernels: non-temporal when the operands together (`moved` bytes) exceed
 // what the 256 MB last-level cache can keep for a consumer; measured on inputs that are not cached,
 // non-temporal accesses are 4-8% faster from about 300 MB up and 2-3% slower below.
-int nt_streaming(int64_t moved, int flags);
+int nt_streaming(int64_t moved);
 // The embedded device headers (thx_common.h, thx_elemwise.h, thx_reduce.h).
 const std::string& device_prelude();
 
@@ -103,8 +102,13 @@ struct View {
   bool imm = false;     // a host scalar travelling in the kernel arguments
   uint64_t immval = 0;  // its value bytes
   bool iota = false;    // no memory: the strides are index multipliers and the value is the offset
+  bool reused = false;  // THX_REUSED: a later call reads it, keep it cacheable
   int64_t stride[THX_MAX_ND] = {0};
 };
+
+// Bit mask over operands: the call-wide choice `nt`, withdrawn from operands flagged THX_REUSED
+// (unless $THX_NT forces it).
+uint64_t nt_mask(int nt, const std::vector<View>& views);
 
 // Check ranks/dtypes, compute the broadcast shape of `ins`, convert strides to
 // elements (0 on broadcast dimensions). `what` names the operation in messages.

@@ -53,11 +53,11 @@ static int env_int(const char* name, int dflt) {
 }
 
 static std::string plan_struct(bool wide, const std::vector<std::pair<std::string, int64_t>>& consts,
-                               const std::vector<int>& mode) {
+                               const std::vector<int>& mode, uint64_t nt) {
   std::ostringstream s;
   s << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int") << " IT;\n  enum { ";
   for (size_t i = 0; i < consts.size(); ++i) s << consts[i].first << " = " << consts[i].second << (i + 1 < consts.size() ? ", " : "");
-  s << " };\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+  s << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
   for (size_t i = 0; i < mode.size(); ++i) s << mode[i] << (i + 1 < mode.size() ? ", " : "");
   s << "};\n    return m[i];\n  }\n};\n";
   return s.str();
@@ -165,10 +165,11 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   for (int o = 0; o < NOUT; ++o) {
     const thx_array& a = outs[o];
     if (a.nd != nk_full) return fail(THX_ERR_TYPE, "reduce: output %d has rank %d, expected %d", o, a.nd, nk_full);
-    if (a.dtype != r->dtypes[NIN + o])
-      return fail(THX_ERR_TYPE, "reduce: output %d has dtype code %d, the operation was built for %d", o, a.dtype,
+    const int adt = a.dtype & ~THX_REUSED;   // results are small: the hint changes nothing for them
+    if (adt != r->dtypes[NIN + o])
+      return fail(THX_ERR_TYPE, "reduce: output %d has dtype code %d, the operation was built for %d", o, adt,
                   r->dtypes[NIN + o]);
-    const int isz = dtype_size(a.dtype);
+    const int isz = dtype_size(adt);
     int64_t expect = isz;
     for (int d = nk_full - 1; d >= 0; --d) {
       if (a.shape[d] != kshape[d])
@@ -188,9 +189,9 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   for (int j = 0; j < r->n_extra; ++j) {
     const thx_array& a = ins[NIN + j];
     const int want = r->dtypes[NIN + NOUT + j];
-    if ((a.dtype & ~THX_HOST_SCALAR) != want)
+    if ((a.dtype & ~(THX_HOST_SCALAR | THX_REUSED)) != want)
       return fail(THX_ERR_TYPE, "reduce: epilogue operand %d has dtype code %d, the operation was built for %d", j,
-                  a.dtype & ~THX_HOST_SCALAR, want);
+                  a.dtype & ~(THX_HOST_SCALAR | THX_REUSED), want);
     const char* p = (const char*)a.base + a.offset_bytes;
     if (a.dtype & THX_HOST_SCALAR) {
       memcpy(&ex[j], p, (size_t)dtype_size(want));
@@ -284,7 +285,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   };
 
   const int block = 256;
-  const int nt = nt_choice(1, flags);  // a reduction reads its input once
+  const uint64_t nt = nt_mask(nt_choice(1), views);  // a reduction streams whatever nothing reads again
   std::string plan;
   Kernel k;
   ParamPack pk;
@@ -348,7 +349,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     if (ra2 && nvec >= (int64_t(1) << 31) - 65536) wide = true;
     const int NK = std::max(1, NKD);
     std::ostringstream key;
-    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|t" << tpr << "|a" << ra2 << (nt ? "|nt" : "") << "|m";
+    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|t" << tpr << "|a" << ra2 << (nt ? "|nt" + std::to_string(nt) : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -358,7 +359,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"NT", nt}}, mode)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}}, mode, nt)
         << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void " << entry << "(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -445,7 +446,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       }
     }
     std::ostringstream key;
-    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << "|r" << rr2 << (nt ? "|nt" : "") << "|m";
+    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << "|r" << rr2 << (nt ? "|nt" + std::to_string(nt) : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -455,7 +456,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TX", tx}, {"RR2", rr2}, {"NT", nt}}, mode)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", block}, {"TX", tx}, {"RR2", rr2}}, mode, nt)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::ColParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_col_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -508,7 +509,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}, {"NT", 0}}, gmode)
+        << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}}, gmode, 0)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::GenParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::NR, ThxPlan::IT> p) {\n  thx::red_gen_body<" << r->name
         << ", ThxPlan>(p);\n}\n";

@@ -105,7 +105,7 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
   for (int i = 0; i < NOPS; ++i) {
     const thx_array& a = i < NIN ? ins[i] : outs[i - NIN];
     const int kind = c->kinds[i];
-    const int dt = a.dtype & ~THX_HOST_SCALAR;
+    const int dt = a.dtype & ~(THX_HOST_SCALAR | THX_REUSED);
     if (dt != c->dtypes[i]) return fail(THX_ERR_TYPE, "rowchain: operand %d has dtype code %d, expected %d", i, dt, c->dtypes[i]);
     const int isz = dtype_size(dt);
     char* p = (char*)a.base + a.offset_bytes;
@@ -194,10 +194,22 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
   int64_t moved = 0;
   for (int i = 0; i < NOPS; ++i)
     if (c->kinds[i] == K_FULL) moved += rows * C * dtype_size(c->dtypes[i]);
-  const int nt = nt_streaming(moved, flags);
+  // non-temporal per operand: the call-wide choice, withdrawn from operands a later call reads
+  uint64_t nt_in = 0, nt_out = 0;
+  if (nt_streaming(moved)) {
+    const bool forced = getenv("THX_NT") != nullptr;
+    for (int i = 0; i < NOPS && i < 64; ++i) {
+      const thx_array& a = i < NIN ? ins[i] : outs[i - NIN];
+      if (!forced && (a.dtype & THX_REUSED)) continue;
+      if (i < NIN) nt_in |= uint64_t(1) << i;
+      else nt_out |= uint64_t(1) << (i - NIN);
+    }
+  }
 
   std::ostringstream key;
-  key << "rw|v" << vec << "|n" << nch << "|t" << tpr << (wide ? "|i64" : "|i32") << (nt ? "|nt" : "") << "|i";
+  key << "rw|v" << vec << "|n" << nch << "|t" << tpr << (wide ? "|i64" : "|i32");
+  if (nt_in | nt_out) key << "|nt" << nt_in << "_" << nt_out;
+  key << "|i";
   for (int i = 0; i < NIN; ++i) key << is_imm[i];
   const std::string plan = key.str() + (fast_div() ? "|fd" : "");
   set_last_plan(c->name + "|" + plan);
@@ -210,7 +222,8 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
     std::ostringstream s;
     s << device_prelude() << c->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
       << " IT;\n  enum { VEC = " << vec << ", NCH = " << nch << ", TPR = " << tpr << ", BLOCK = " << block
-      << ", NT = " << nt << " };\n  static constexpr int imm(int i) {\n    constexpr int m[] = {";
+      << " };\n  static constexpr unsigned long long NT = " << nt_in << "ull, NTO = " << nt_out
+      << "ull;\n  static constexpr int imm(int i) {\n    constexpr int m[] = {";
     for (int i = 0; i < NIN; ++i) s << is_imm[i] << (i + 1 < NIN ? ", " : "");
     s << "};\n    return m[i];\n  }\n};\n"
       << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::RowChainParams<" << c->name

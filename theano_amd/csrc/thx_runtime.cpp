@@ -147,9 +147,9 @@ int gather_inputs(const char* what, const thx_array* ins, int n_in, const int32_
   for (int i = 0; i < n_in; ++i) {
     if (ins[i].nd != nd)
       return fail(THX_ERR_TYPE, "%s: input %d has rank %d, expected %d", what, i, ins[i].nd, nd);
-    if ((ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX)) != dtypes[i])
+    if ((ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX | THX_REUSED)) != dtypes[i])
       return fail(THX_ERR_TYPE, "%s: input %d has dtype code %d, the operation was built for %d", what, i,
-                  ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX), dtypes[i]);
+                  ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX | THX_REUSED), dtypes[i]);
     for (int d = 0; d < nd; ++d) {
       const int64_t s = ins[i].shape[d];
       if (s < 0) return fail(THX_ERR_ARG, "%s: negative extent", what);
@@ -173,7 +173,8 @@ int gather_inputs(const char* what, const thx_array* ins, int n_in, const int32_
   for (int i = 0; i < n_in; ++i) {
     View& v = (*views)[i];
     v.ptr = (char*)ins[i].base + ins[i].offset_bytes;
-    v.dtype = ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX);
+    v.reused = (ins[i].dtype & THX_REUSED) != 0;
+    v.dtype = ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX | THX_REUSED);
     const int isz = dtype_size(v.dtype);
     if (!isz) return fail(THX_ERR_TYPE, "%s: unknown dtype code %d", what, v.dtype);
     if (ins[i].dtype & THX_INDEX) {  // no memory behind it; the caller that supports it fills in the multipliers
@@ -217,18 +218,21 @@ bool fast_div() {
   return env ? atoi(env) != 0 : true;
 }
 
-int nt_choice(int family_default, int flags) {
+int nt_choice(int family_default) {
   const char* env = getenv("THX_NT");
-  if (env) return atoi(env) != 0;
-  if (flags & THX_KEEP_CACHED) return 0;
-  return family_default;
+  return env ? (atoi(env) != 0) : family_default;
 }
 
-int nt_streaming(int64_t moved, int flags) {
-  // the hint only helps when this call's own traffic leaves room in the cache for what is to be kept
-  if (moved > (int64_t(256) << 20)) flags &= ~THX_KEEP_CACHED;
-  return nt_choice(moved >= (int64_t(288) << 20), flags);
+uint64_t nt_mask(int nt, const std::vector<View>& views) {
+  if (!nt) return 0;
+  const bool forced = getenv("THX_NT") != nullptr;
+  uint64_t m = 0;
+  for (size_t i = 0; i < views.size() && i < 64; ++i)
+    if (forced || !views[i].reused) m |= uint64_t(1) << i;
+  return m;
 }
+
+int nt_streaming(int64_t moved) { return nt_choice(moved >= (int64_t(288) << 20)); }
 
 static uint64_t fnv1a(const std::string& s, uint64_t h) {
   for (unsigned char c : s) {

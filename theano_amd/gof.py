@@ -9,7 +9,6 @@ is the one documented for Theano ops (``doc/extending/op.txt``: ``make_node``
 (``Apply`` :50, ``Variable`` :270, ``Constant`` :559), ``theano/gof/op.py:793``
 and ``theano/gof/fg.py``.
 """
-from collections import OrderedDict, deque
 
 
 class MethodNotDefined(NotImplementedError):

@@ -17,7 +17,7 @@ from ..gof import Apply, Op, Type, Variable
 from ..tensor.elemwise import CAReduce, DimShuffle, Elemwise
 from ..tensor.type import TensorType, _tensor_py_operators
 from . import codegen
-from .runtime import THX_INDEX, HipArray, call_flags, check, host_scalar_thx, lib, thx_array
+from .runtime import THX_INDEX, HipArray, call_flags, check, host_scalar_thx, lib, mark_reused, thx_array
 
 
 class HipArrayType(Type):
@@ -304,6 +304,7 @@ class HipElemwise(Elemwise):
                 arr = HipArray._new_contiguous(shape, out_dt[k])
             arr.as_thx(outs[k])
             results.append(arr)
+        mark_reused(node, ins, outs)
         rc = lib.thx_elemwise_call(handle, ins, outs, flags)
         if rc:
             check(rc)
@@ -446,6 +447,7 @@ class HipCAReduce(CAReduce):
             arr = HipArray._new_contiguous(kept, out_dt[k])
             arr.as_thx(outs[k])
             results.append(arr)
+        mark_reused(node, ins, outs)
         rc = lib.thx_reduce_call(handle, ins, mask, outs, flags)
         if rc:
             check(rc)
@@ -541,6 +543,7 @@ class HipMaxAndArgmax(Op):
         am = HipArray._new_contiguous(kept, np.dtype("int64"))
         mx.as_thx(outs[0])
         am.as_thx(outs[1])
+        mark_reused(node, ins, outs)
         rc = lib.thx_reduce_call(handle, ins, mask, outs, call_flags(node))
         if rc:
             check(rc)

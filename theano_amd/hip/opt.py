@@ -15,14 +15,12 @@ import numpy as np
 from .. import gof
 from .. import scalar as scal
 from ..config import config
-from ..gof import Constant, FunctionGraph
+from ..gof import Constant
 from ..tensor import basic as T
 from ..tensor.elemwise import All, Any, CAReduce, CAReduceDtype, DimShuffle, Elemwise
 from ..tensor.type import TensorConstant, TensorType
 from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipMaxAndArgmax, HipToHost, HostToHip,
-                  _is_host_scalar,
-                  as_hip_variable, hip_from_host, host_from_hip)
-from .runtime import HipArray
+                  _is_host_scalar, as_hip_variable, hip_from_host, host_from_hip)
 
 
 class DeviceConstant(Constant):

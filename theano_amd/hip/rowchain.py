@@ -20,10 +20,9 @@ from .. import gof
 from .. import scalar as scal
 from ..gof import Apply, Op
 from ..scalar import Scalar, compute_ctype, storage_ctype
-from ..tensor.type import TensorType
 from . import codegen
 from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, _is_host_scalar)
-from .runtime import HipArray, call_flags, check, host_scalar_thx, lib, thx_array
+from .runtime import HipArray, call_flags, check, host_scalar_thx, lib, mark_reused, thx_array
 
 FULL, ROW, COL, SCALAR = 0, 1, 2, 3
 THX_ERR_UNSUPPORTED = 6
@@ -195,6 +194,7 @@ class HipRowChain(Op):
             arr = HipArray._new_contiguous(tuple(shape), out_dt[k])
             arr.as_thx(outs[k])
             results.append(arr)
+        mark_reused(node, ins, outs)
         rc = lib.thx_rowchain_call(handle, ins, outs, call_flags(node))
         if rc == THX_ERR_UNSUPPORTED:
             results = self._run_fallback(inputs)

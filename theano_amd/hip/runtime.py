@@ -19,9 +19,9 @@ _LIB_PATH = os.path.join(os.path.dirname(_HERE), "csrc", "libthx_hip.so")
 THX_MAX_ND = 8
 THX_BROADCAST = 1
 THX_DRY_RUN = 2
-THX_KEEP_CACHED = 4
 THX_HOST_SCALAR = 0x100
 THX_INDEX = 0x200
+THX_REUSED = 0x400
 
 
 class thx_array(ctypes.Structure):
@@ -115,12 +115,17 @@ def dry_run():
 
 
 def call_flags(node=None):
-    """Flags of a kernel call; ``node.tag['keep_cached']`` (set when the function is compiled) adds
-    THX_KEEP_CACHED."""
-    f = THX_BROADCAST | (THX_DRY_RUN if _dry else 0)
-    if node is not None and node.tag.get("keep_cached"):
-        f |= THX_KEEP_CACHED
-    return f
+    """Flags of a kernel call."""
+    return THX_BROADCAST | (THX_DRY_RUN if _dry else 0)
+
+
+def mark_reused(node, ins, outs):
+    """OR THX_REUSED into the descriptors of the operands that a later kernel of the same
+    function reads (positions recorded in ``node.tag`` when the function was compiled)."""
+    for k in node.tag.get("reused_in", ()):
+        ins[k].dtype |= THX_REUSED
+    for k in node.tag.get("reused_out", ()):
+        outs[k].dtype |= THX_REUSED
 
 
 def init(device=None):

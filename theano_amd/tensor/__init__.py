@@ -11,3 +11,4 @@ for _n in dir(_type):  # bscalar ... dtensor4 and friends
 from .elemwise import DimShuffle, Elemwise, CAReduce, CAReduceDtype, Sum, Prod, All, Any
 from .basic import *  # noqa: F401,F403
 from .basic import Max, MaxAndArgmax, Min, ShapeFloat, makeKeepDims, cast, round  # noqa: F401
+from . import nnet  # noqa: F401,E402
