@@ -15,8 +15,9 @@ a few percent faster than one that follows a different array; a step holds one
 launch of each kind, and the average of the two loops divides the kernel's
 algorithmic bytes.  ``cpu_baseline`` times the oracle's C restatement of the
 reference's loops on this host.  ``other_configs`` lists the remaining four
-configurations over input sets that rotate (so that no set is still cached
-when it is used again: ``us``) and over one set (``same_input_us``).
+configurations (and max_and_argmax of the configuration-2 matrix) over input
+sets that rotate (so that no set is still cached when it is used again: ``us``)
+and over one set (``same_input_us``).
 """
 import argparse
 import json
@@ -214,7 +215,9 @@ def main():
                  ("c4_sum", W.c4_graph("sum"), W.c4_inputs("full")),
                  ("c4_anyall", W.c4_graph("anyall"), W.c4_inputs("full", "anyall")),
                  ("c5_fwd", W.c5_graph(with_grad=False), W.c5_inputs("full", with_grad=False)),
-                 ("c5_grad", W.c5_graph(forward=False), W.c5_inputs("full"))]
+                 ("c5_grad", W.c5_graph(forward=False), W.c5_inputs("full")),
+                 ("c2_argmax_axis1", W.c2_argmax_graph(1), W.c2_inputs("max_axis1", "full")),
+                 ("c2_argmax_axis0", W.c2_argmax_graph(0), W.c2_inputs("max_axis1", "full"))]
         for name, (ins, outs), vals in specs:
             f = th.function(ins, [th.Out(o, device=True) for o in outs])
             sets = _input_sets(vals)
@@ -228,7 +231,8 @@ def main():
             # start of the host loop to show in a single run
             ms = min(_time_steps(hip, rotating, args.steps, 3)[0] for _ in range(3))
             warm_ms = min(_time_steps(hip, lambda: f(*sets[0]), args.steps, 3)[0] for _ in range(3))
-            n_k = sum(1 for n in f.toposort() if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain"))
+            n_k = sum(1 for n in f.toposort()
+                      if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax"))
             others[name] = _rate(W.algorithmic_bytes(name), ms)
             others[name].update({"input_sets": len(sets), "same_input_us": round(warm_ms * 1e3, 2),
                                  "nodes_per_step": n_k})

@@ -112,3 +112,32 @@ def test_nnet_row_functions_run_as_row_chains():
         assert_parity(g, r, "nnet output %d" % k, tol=dict(rtol=2e-5, atol=2e-6))
     assert np.allclose(np.exp(got[0]).sum(axis=1), 1.0, atol=1e-5)
     assert np.allclose(got[1].sum(axis=1), 1.0, atol=1e-5)
+
+
+def test_batch_normalization_helpers_forward_grad_and_inference():
+    """tensor.nnet.batch_normalization_train / _train_grad / _test (the graphs
+    the reference lowers its AbstractBatchNorm ops to, theano/tensor/nnet/bn.py:679-789)
+    against the oracle; the explicit gradient formula and grad() of the forward
+    graph must agree with each other as well."""
+    rng = np.random.default_rng(42)
+    t4 = T.TensorType("float32", (False,) * 4)
+    pc = T.TensorType("float32", (True, False, True, True))
+    x, dy = t4("x"), t4("dy")
+    g, b, rm, rv = pc("g"), pc("b"), pc("rm"), pc("rv")
+    out, mean, invstd, nrm, nrv = T.nnet.batch_normalization_train(x, g, b, "spatial", 1e-5, 0.1, rm, rv)
+    gx, gg, gb = T.nnet.batch_normalization_train_grad(x, dy, g, mean, invstd, "spatial")
+    ax, ag, ab = th.grad(T.sum(out * dy), [x, g, b])
+    inf = T.nnet.batch_normalization_test(x, g, b, rm, rv, "spatial", 1e-5)
+    outs = [out, mean, invstd, nrm, nrv, gx, gg, gb, ax, ag, ab, inf]
+    vals = [rng.normal(0.5, 2.0, (9, 33, 7, 11)).astype("float32"), rng.standard_normal((9, 33, 7, 11)).astype("float32"),
+            rng.uniform(0.5, 1.5, (1, 33, 1, 1)).astype("float32"), rng.standard_normal((1, 33, 1, 1)).astype("float32"),
+            rng.standard_normal((1, 33, 1, 1)).astype("float32"), rng.uniform(0.5, 1.5, (1, 33, 1, 1)).astype("float32")]
+    ins = [x, dy, g, b, rm, rv]
+    got = th.function(ins, outs)(*vals)
+    ref = G.evaluate(ins, outs, vals)
+    for k, (a, r) in enumerate(zip(got, ref)):
+        assert_parity(a, r, "batch norm output %d" % k, tol=dict(rtol=5e-5, atol=5e-6))
+    for a, c in zip(got[5:8], got[8:11]):
+        assert np.allclose(a, c, rtol=1e-4, atol=1e-5)
+    xhat = (got[0] - vals[3]) / vals[2]
+    assert np.allclose(xhat.mean(axis=(0, 2, 3)), 0, atol=1e-5) and np.allclose(xhat.std(axis=(0, 2, 3)), 1, atol=1e-3)

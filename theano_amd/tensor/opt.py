@@ -114,6 +114,52 @@ def local_useless_elemwise(fgraph, node):
 
 
 @local_optimizer([Elemwise])
+def local_constant_fold(fgraph, node):
+    """Arithmetic on scalar constants is done when the function is compiled
+    (``constant_folding``, ``theano/tensor/opt.py:6600-6660``, restricted to
+    all-broadcastable constants and to + - * / neg sqr inv cast, evaluated in
+    the node's output dtype as the C expression would be): ``pow(x, 2.0 - 1)``
+    from the gradient of a square becomes ``pow(x, 1.0)`` and then ``x``."""
+    if len(node.outputs) != 1 or not node.inputs:
+        return False
+    out = node.outputs[0]
+    odt = out.type.dtype
+    if odt == "bool" or not all(isinstance(i, TensorConstant) and all(i.type.broadcastable) and
+                                i.type.dtype != "bool" for i in node.inputs):
+        return False
+    sop = node.op.scalar_op
+    vals = [np.asarray(i.data).reshape(()).astype(odt) for i in node.inputs]
+    with np.errstate(all="ignore"):
+        if isinstance(sop, scal.Add):
+            res = vals[0]
+            for v in vals[1:]:
+                res = res + v
+        elif isinstance(sop, scal.Mul):
+            res = vals[0]
+            for v in vals[1:]:
+                res = res * v
+        elif isinstance(sop, scal.Sub):
+            res = vals[0] - vals[1]
+        elif isinstance(sop, scal.TrueDiv) and odt in scal.float_dtypes:
+            res = vals[0] / vals[1]
+        elif isinstance(sop, scal.Neg):
+            res = -vals[0]
+        elif isinstance(sop, scal.Sqr):
+            res = vals[0] * vals[0]
+        elif isinstance(sop, scal.Inv) and odt in scal.float_dtypes:
+            res = np.asarray(1, odt) / vals[0]
+        elif isinstance(sop, (scal.Cast, scal.Identity)):
+            src = np.asarray(node.inputs[0].data).reshape(())
+            if odt not in scal.float_dtypes and not np.isfinite(src):
+                return False
+            res = src.astype(odt)
+        else:
+            return False
+    new = TensorConstant(out.type, np.asarray(res, dtype=odt).reshape((1,) * out.type.ndim))
+    return [new]
+
+
+@local_optimizer([Elemwise])
 def local_fill_sink(fgraph, node):
     """An elementwise consumer broadcasts anyway: f(second(a, b), c) -> f(b, c)
     as long as the other inputs still give the result its full pattern."""
@@ -300,7 +346,8 @@ def local_shape_lift(fgraph, node):
     return False
 
 
-CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_useless_elemwise, local_fill_sink, local_useless_reduce,
+CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_constant_fold, local_useless_elemwise, local_fill_sink,
+                local_useless_reduce,
                 local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax]
 
 

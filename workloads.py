@@ -42,6 +42,12 @@ def c2_graph(case):
     return [x], [out]
 
 
+def c2_argmax_graph(axis):
+    """max_and_argmax of the configuration-2 matrix: the caller-side form of max."""
+    x = T.fmatrix("x")
+    return [x], T.max_and_argmax(x, axis=axis)
+
+
 def c2_inputs(case, scale="full"):
     n = 8192 if scale == "full" else 384
     if case == "prod_axis1":
@@ -132,6 +138,9 @@ def algorithmic_bytes(name, scale="full"):
     if name == "c1":
         n = 4096 if scale == "full" else 250
         return 2 * n * n * f4 + 8
+    if name.startswith("c2_argmax"):  # max (float32) and argmax (int64) per kept index
+        n = 8192 if scale == "full" else 384
+        return n * n * f4 + n * (f4 + 8)
     if name.startswith("c2"):
         n = 8192 if scale == "full" else 384
         return n * n * f4 + (4 if name == "c2_sum_all" else n * f4)
