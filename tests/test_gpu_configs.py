@@ -141,3 +141,30 @@ def test_batch_normalization_helpers_forward_grad_and_inference():
         assert np.allclose(a, c, rtol=1e-4, atol=1e-5)
     xhat = (got[0] - vals[3]) / vals[2]
     assert np.allclose(xhat.mean(axis=(0, 2, 3)), 0, atol=1e-5) and np.allclose(xhat.std(axis=(0, 2, 3)), 1, atol=1e-3)
+
+
+def test_more_than_2_to_31_elements_use_64_bit_indexing():
+    """A 2^31 + 4096 element int8 vector (and its (2, n/2) view): elementwise,
+    row and column reductions and argmax index with 64-bit offsets; results
+    against NumPy on the whole array."""
+    n = 2 ** 31 + 4096
+    rng = np.random.default_rng(43)
+    base = rng.integers(-100, 100, 1 << 20).astype("int8")
+    val = np.tile(base, n // base.size + 1)[:n]
+    val[n - 5] = 127                                   # the last maximum sits beyond 2^31
+    val[7] = -128
+    v = T.TensorType("int8", (False,))("v")
+    f = th.function([v], [T.sum(v), T.max_and_argmax(v)[1], th.Out((v + np.int8(1)) ^ np.int8(3), device=True)])
+    s, am, ew = f(val)
+    assert "i64" in hip.last_plan()
+    assert s == val.sum(dtype=np.int64)
+    assert am == int(np.argmax(val))
+    tail = ew.to_numpy()[n - 4096:]
+    assert np.array_equal(tail, (val[n - 4096:] + np.int8(1)) ^ np.int8(3))
+    del ew
+    m = T.TensorType("int8", (False, False))("m")
+    g = th.function([m], [T.sum(m, axis=1), T.sum(m, axis=0)])
+    r1, r0 = g(val.reshape(2, n // 2))
+    assert np.array_equal(r1, val.reshape(2, n // 2).sum(axis=1, dtype=np.int64))
+    assert np.array_equal(r0[:4096], val.reshape(2, n // 2)[:, :4096].sum(axis=0, dtype=np.int64))
+    assert r0.sum() == s

@@ -264,3 +264,21 @@ def test_max_and_argmax_interface(dry_run):
     (node,) = ops_of(f, HipMaxAndArgmax)
     assert not ops_of(f, HipElemwise) and str(node.op.pre_scalar_op) == "Composite{neg(i0)}"
     f(np.zeros((3, 5, 7), "float32"))
+
+
+def test_plans_for_arrays_beyond_32_bit_limits(dry_run):
+    """Planning only (no memory is touched in a dry run): more than 2^31 elements
+    switch the kernels to 64-bit offsets; more vectors than one dispatch has
+    work-items (2^32 - 1) switch the elementwise kernel to a grid-stride loop."""
+    from theano_amd import hip
+    v = T.TensorType("int8", (False,))("v")
+    f = th.function([v], th.Out(v + np.int8(1), device=True))
+    big = np.lib.stride_tricks.as_strided(np.zeros((), "int8"), shape=(2 ** 31 + 4096,), strides=(0,))
+    f(big)
+    assert "|i64|" in hip.last_plan() and "|gs" not in hip.last_plan()
+    huge = np.lib.stride_tricks.as_strided(np.zeros((), "int8"), shape=(2 ** 37,), strides=(0,))
+    f(huge)
+    assert "|i64|" in hip.last_plan() and "|gs|" in hip.last_plan()
+    g = th.function([v], T.sum(v))
+    g(huge)
+    assert "|i64|" in hip.last_plan()

@@ -20,6 +20,8 @@ namespace thx {
 
 enum { M_VEC = 0, M_BCAST = 1, M_GATHER = 2, M_IMM = 3 };
 
+static int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
 struct Dims {
   int nd = 0;
   int64_t shape[THX_MAX_ND];
@@ -288,7 +290,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
             outer *= dm.shape[d];
           }
         const int64_t grid = outer * tiles_t * tiles_i;
-        if (grid <= 0x7fffffffLL) {
+        if (grid * 256 <= 0xffffffffLL) {
           ParamPack pk;
           for (int o = 0; o < nops; ++o) pk.put<char*>(views[o].ptr);
           for (int o = 0; o < nops; ++o) pk.put<uint64_t>(views[o].immval);
@@ -318,8 +320,10 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   const int force_block = env_int("THX_EW_BLOCK", 0);
   if (force_block == 128 || force_block == 512 || force_block == 1024) block = force_block;
   const uint64_t nt = nt_mask(nt_streaming(moved), views);
-  // grid-stride: a bounded number of blocks walk the index space instead of one block per chunk
-  const int gs = env_int("THX_EW_GS", 0);
+  // grid-stride: a bounded number of blocks walk the index space instead of one block per chunk;
+  // needed once one block per chunk would exceed the 2^32 - 1 work-items a dispatch can carry
+  int gs = env_int("THX_EW_GS", 0);
+  if (!gs && ceil_div64(nvec, (int64_t)block * unr) * block > 0xffffffffLL) gs = 64;
 
   std::ostringstream key;
   key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr;
@@ -362,7 +366,8 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   int64_t grid = (nvec + (int64_t)block * unr - 1) / ((int64_t)block * unr);
   if (grid < 1) grid = 1;
   if (gs) grid = std::min<int64_t>(grid, (int64_t)(rt().ready ? rt().cus : 256) * gs);
-  if (grid > 0x7fffffffLL) return fail(THX_ERR_UNSUPPORTED, "elemwise: %lld blocks exceed the grid limit", (long long)grid);
+  if (grid * block > 0xffffffffLL)
+    return fail(THX_ERR_UNSUPPORTED, "elemwise: %lld blocks of %d exceed the work-items of one dispatch", (long long)grid, block);
   return launch(k, e->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
 }
 

@@ -270,10 +270,12 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   else if (iabs(RD.back().stride[primary]) == 1) form = ROW;
   else if (KD.back().stride[primary] == 1) form = COL;
   else form = ROW;
+  // the column form counts columns in 32 bits
+  if (form == COL && KD.back().extent >= (int64_t(1) << 31) - 65536) form = GEN;
   const char* force = getenv("THX_RED_FORM");
   if (force && NR <= 2 && NR > 0) {
     if (!strcmp(force, "row")) form = ROW;
-    if (!strcmp(force, "col") && NKD > 0) form = COL;
+    if (!strcmp(force, "col") && NKD > 0 && KD.back().extent < (int64_t(1) << 31) - 65536) form = COL;
     if (!strcmp(force, "gen")) form = GEN;
   }
 
@@ -534,7 +536,9 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   }
 
   set_last_plan(r->name + "|" + plan + (S > 1 ? "|s" + std::to_string(S) : ""));
-  if (grid > 0x7fffffffLL) return fail(THX_ERR_UNSUPPORTED, "reduce: %lld blocks exceed the grid limit", (long long)grid);
+  if (grid * launch_block > 0xffffffffLL)
+    return fail(THX_ERR_UNSUPPORTED, "reduce: %lld blocks of %d exceed the work-items of one dispatch", (long long)grid,
+                launch_block);
   if (!dry) {
     rc = launch(k, r->name + "|" + plan, (unsigned)grid, launch_block, pk.buf.data(), pk.buf.size());
     if (rc) return rc;

@@ -246,7 +246,8 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
   pk.align(8);
   const int rpb = block / tpr;
   const int64_t grid = (rows + rpb - 1) / rpb;
-  if (grid > 0x7fffffffLL) return fail(THX_ERR_UNSUPPORTED, "rowchain: %lld blocks exceed the grid limit", (long long)grid);
+  if (grid * block > 0xffffffffLL)
+    return fail(THX_ERR_UNSUPPORTED, "rowchain: %lld blocks of %d exceed the work-items of one dispatch", (long long)grid, block);
   return launch(k, c->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
 }
 

@@ -280,6 +280,8 @@ class HipArray(object):
         a = np.asarray(a)
         if a.dtype not in _CODE_OF:
             raise TypeError("dtype %s is not supported on the device" % a.dtype)
+        if _dry:                       # shapes only: nothing is copied, so nothing needs to exist
+            return cls.empty(a.shape, a.dtype)
         a = np.asarray(a, order="C")
         out = cls.empty(a.shape, a.dtype)
         if a.nbytes and not out.buffer.fake:

@@ -1,0 +1,496 @@
+"""The ops either side of an elementwise / reduction island: basic indexing,
+its scatter-back gradient, reshaping, broadcasting fills and joining.
+
+Graph-level mirrors of ``Subtensor`` / ``IncSubtensor``
+(``theano/tensor/subtensor.py:318-780, 1175-1560``), ``Reshape`` / ``flatten``
+(``theano/tensor/basic.py:4701-4920, 5160-5220``), ``Alloc`` (:2769-2960) and
+``Join`` / ``Split`` (:4120-4470, 3700-3860), restricted to what needs no
+host-side integer arithmetic in the graph: indices and slice bounds are Python
+integers, and shapes that depend on run-time extents are written as "like
+dimension d of input k".  None of them computes on the host: ``perform``
+exists only on the device subclasses (``theano_amd/hip/views.py``), where a
+view costs nothing and a copy is one elementwise kernel.
+"""
+import numpy as np
+
+from ..gof import Apply, Op
+from . import basic as T
+from .type import TensorType, as_tensor_variable
+
+
+def _no_host(op):
+    raise NotImplementedError("%s runs on the device only; compile the graph with function()" % op)
+
+
+# --------------------------------------------------------------------------
+def normalize_index(idx, ndim):
+    """A tuple of ints and slices (with int / None fields), one per indexed
+    dimension; Ellipsis expands, missing trailing dimensions are full slices."""
+    if not isinstance(idx, tuple):
+        idx = (idx,)
+    if sum(1 for i in idx if i is Ellipsis) > 1:
+        raise IndexError("an index can only have a single ellipsis")
+    if any(i is None for i in idx):
+        raise NotImplementedError("newaxis in an index: use dimshuffle")
+    n_real = sum(1 for i in idx if i is not Ellipsis)
+    if n_real > ndim:
+        raise IndexError("too many indices for a tensor of rank %d" % ndim)
+    out = []
+    for i in idx:
+        if i is Ellipsis:
+            out.extend([slice(None)] * (ndim - n_real))
+        elif isinstance(i, slice):
+            for f in (i.start, i.stop, i.step):
+                if f is not None and not isinstance(f, (int, np.integer)):
+                    raise NotImplementedError("slice bounds must be Python integers (got %r)" % (f,))
+            if i.step == 0:
+                raise ValueError("slice step cannot be zero")
+            out.append(slice(*[None if f is None else int(f) for f in (i.start, i.stop, i.step)]))
+        elif isinstance(i, (int, np.integer)):
+            out.append(int(i))
+        else:
+            raise NotImplementedError("only integers and slices index a tensor here (got %r)" % (i,))
+    out.extend([slice(None)] * (ndim - len(out)))
+    return tuple(out)
+
+
+def index_view(shape, strides, offset, idx_list):
+    """(shape, strides, offset) of ``x[idx_list]`` for an array header, with
+    NumPy's rules: negative indices count from the end, an integer out of range
+    raises IndexError, slice bounds are clipped."""
+    new_shape, new_strides = [], []
+    for d, i in enumerate(idx_list):
+        n, st = shape[d], strides[d]
+        if isinstance(i, slice):
+            start, stop, step = i.indices(n)
+            length = len(range(start, stop, step))
+            offset += start * st
+            new_shape.append(length)
+            new_strides.append(st * step)
+        else:
+            j = i + n if i < 0 else i
+            if j < 0 or j >= n:
+                raise IndexError("index %d is out of bounds for axis %d with size %d" % (i, d, n))
+            offset += j * st
+    return tuple(new_shape), tuple(new_strides), offset
+
+
+def _idx_key(idx_list):
+    return tuple(("s", i.start, i.stop, i.step) if isinstance(i, slice) else ("i", i) for i in idx_list)
+
+
+class Subtensor(Op):
+    """``x[idx_list]`` with integers and constant slices: a view
+    (``theano/tensor/subtensor.py:318-780``; ``view_map = {0: [0]}`` :513)."""
+
+    __props__ = ("idx_key",)
+    view_map = {0: [0]}
+
+    def __init__(self, idx_list):
+        self.idx_list = tuple(idx_list)
+        self.idx_key = _idx_key(self.idx_list)
+
+    def _props(self):
+        return (self.idx_key,)
+
+    def __str__(self):
+        def one(i):
+            if isinstance(i, slice):
+                return ":".join("" if f is None else str(f) for f in (i.start, i.stop, i.step))
+            return str(i)
+        return "%s{%s}" % (type(self).__name__, ", ".join(one(i) for i in self.idx_list))
+
+    def out_broadcastable(self, in_broadcastable):
+        # a full slice keeps the flag (theano/tensor/subtensor.py:470-500); any other slice may be empty
+        return tuple(b and i == slice(None) for b, i in zip(in_broadcastable, self.idx_list) if isinstance(i, slice))
+
+    def make_node(self, x):
+        x = as_tensor_variable(x)
+        if len(self.idx_list) != x.type.ndim:
+            raise IndexError("index of %d entries for a tensor of rank %d" % (len(self.idx_list), x.type.ndim))
+        return Apply(self, [x], [TensorType(x.type.dtype, self.out_broadcastable(x.type.broadcastable))()])
+
+    def infer_shape(self, node, shapes):
+        shape, _, _ = index_view(shapes[0], [1] * len(shapes[0]), 0, self.idx_list)
+        return [shape]
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def L_op(self, inputs, outputs, grads):
+        (x,) = inputs
+        (g,) = grads
+        return [IncSubtensor(self.idx_list)(x.zeros_like(), g)]
+
+
+class IncSubtensor(Op):
+    """``x`` with ``x[idx_list]`` incremented by (or set to) ``y``
+    (``theano/tensor/subtensor.py:1175-1560``).  A new array: the input is not
+    modified."""
+
+    __props__ = ("idx_key", "set_instead_of_inc")
+
+    def __init__(self, idx_list, set_instead_of_inc=False):
+        self.idx_list = tuple(idx_list)
+        self.idx_key = _idx_key(self.idx_list)
+        self.set_instead_of_inc = bool(set_instead_of_inc)
+
+    def _props(self):
+        return (self.idx_key, self.set_instead_of_inc)
+
+    def __str__(self):
+        return "%s{%s;%s}" % (type(self).__name__, "Set" if self.set_instead_of_inc else "Inc",
+                              str(Subtensor(self.idx_list))[len("Subtensor{"):-1])
+
+    def make_node(self, x, y):
+        x, y = as_tensor_variable(x), as_tensor_variable(y)
+        if y.type.dtype != x.type.dtype:
+            y = T.cast(y, x.type.dtype)
+        sub = Subtensor(self.idx_list).make_node(x).outputs[0]
+        if y.type.ndim > sub.type.ndim:
+            raise TypeError("the increment has rank %d, the indexed region rank %d" % (y.type.ndim, sub.type.ndim))
+        return Apply(self, [x, y], [x.type()])
+
+    def infer_shape(self, node, shapes):
+        return [shapes[0]]
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def L_op(self, inputs, outputs, grads):
+        x, y = inputs
+        (g,) = grads
+        gy = Subtensor(self.idx_list)(g)
+        # y may have been broadcast into the region: sum the gradient back (subtensor.py:1520-1560)
+        sub_ndim = gy.type.ndim
+        if y.type.ndim < sub_ndim:
+            gy = T.sum(gy, axis=tuple(range(sub_ndim - y.type.ndim)))
+        bdims = [d for d in range(y.type.ndim) if y.type.broadcastable[d] and not gy.type.broadcastable[d]]
+        if bdims:
+            gy = T.sum(gy, axis=tuple(bdims), keepdims=True)
+            gy = T.DimShuffle(gy.type.broadcastable, list(range(gy.type.ndim)))(gy) if gy.type != y.type else gy
+        if self.set_instead_of_inc:
+            gx = IncSubtensor(self.idx_list, True)(g, T.zeros_like(Subtensor(self.idx_list)(g)))
+        else:
+            gx = g
+        return [gx, gy]
+
+
+def subtensor(x, idx):
+    x = as_tensor_variable(x)
+    idx_list = normalize_index(idx, x.type.ndim)
+    if all(i == slice(None) for i in idx_list):
+        return x
+    return Subtensor(idx_list)(x)
+
+
+def inc_subtensor(x, y, idx=None):
+    """``inc_subtensor(x[idx], y)`` written as ``inc_subtensor(x, y, idx)``."""
+    x = as_tensor_variable(x)
+    return IncSubtensor(normalize_index(idx if idx is not None else (), x.type.ndim))(x, y)
+
+
+def set_subtensor(x, y, idx=None):
+    x = as_tensor_variable(x)
+    return IncSubtensor(normalize_index(idx if idx is not None else (), x.type.ndim), True)(x, y)
+
+
+# --------------------------------------------------------------------------
+class Reshape(Op):
+    """``x`` with a new shape (``theano/tensor/basic.py:4701-4920``).  ``pattern``
+    has one entry per output dimension: a non-negative int, ``-1`` (at most one,
+    inferred) or ``(k, d)``: the extent of dimension ``d`` of input ``k``.
+    Inputs after the first are read for their shape only.  A view when the
+    input is C-contiguous, else a copy."""
+
+    __props__ = ("pattern",)
+    view_map = {0: [0]}
+
+    def __init__(self, pattern):
+        pat = []
+        for p in pattern:
+            if isinstance(p, tuple):
+                pat.append((int(p[0]), int(p[1])))
+            else:
+                p = int(p)
+                if p < -1:
+                    raise ValueError("invalid extent %d in a shape" % p)
+                pat.append(p)
+        if sum(1 for p in pat if p == -1) > 1:
+            raise ValueError("can only specify one unknown dimension")
+        self.pattern = tuple(pat)
+
+    def _props(self):
+        return (self.pattern,)
+
+    def __str__(self):
+        return "%s{%s}" % (type(self).__name__, ", ".join(
+            "in%d.shape[%d]" % p if isinstance(p, tuple) else str(p) for p in self.pattern))
+
+    def make_node(self, x, *like):
+        ins = [as_tensor_variable(x)] + [as_tensor_variable(v) for v in like]
+        bcast = []
+        for p in self.pattern:
+            if isinstance(p, tuple):
+                k, d = p
+                if k >= len(ins) or d >= ins[k].type.ndim:
+                    raise ValueError("shape entry %s refers to a missing input dimension" % (p,))
+                bcast.append(ins[k].type.broadcastable[d])
+            else:
+                bcast.append(p == 1)
+        return Apply(self, ins, [TensorType(ins[0].type.dtype, bcast)()])
+
+    def resolve(self, shapes):
+        """The concrete output shape given the inputs' shapes."""
+        total = 1
+        for s in shapes[0]:
+            total *= s
+        out, known, unknown = [], 1, None
+        for j, p in enumerate(self.pattern):
+            v = shapes[p[0]][p[1]] if isinstance(p, tuple) else p
+            if v == -1:
+                unknown = j
+                out.append(-1)
+            else:
+                out.append(int(v))
+                known *= int(v)
+        if unknown is not None:
+            if known == 0 or total % known:
+                raise ValueError("cannot reshape array of size %d into shape %s" % (total, tuple(out)))
+            out[unknown] = total // known
+        elif known != total:
+            raise ValueError("cannot reshape array of size %d into shape %s" % (total, tuple(out)))
+        return tuple(out)
+
+    def infer_shape(self, node, shapes):
+        return [self.resolve(shapes)]
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def L_op(self, inputs, outputs, grads):
+        x = inputs[0]
+        (g,) = grads
+        gx = Reshape([(1, d) for d in range(x.type.ndim)])(g, x)
+        if gx.type != x.type:          # broadcast flags the pattern could not know
+            gx = T.DimShuffle(gx.type.broadcastable, list(range(x.type.ndim)))(gx)
+        return [gx] + [v.zeros_like() for v in inputs[1:]]
+
+    def connection_pattern(self, node):
+        return [[True]] + [[False]] * (len(node.inputs) - 1)
+
+
+def reshape(x, newshape):
+    """``newshape``: ints, at most one -1, or ``x.shape[d]``-style entries given
+    as ``(variable, d)`` pairs."""
+    x = as_tensor_variable(x)
+    if isinstance(newshape, (int, np.integer)):
+        newshape = (newshape,)
+    like, pattern = [], []
+    for p in newshape:
+        if isinstance(p, tuple):
+            v, d = p
+            v = as_tensor_variable(v)
+            if v is x:
+                pattern.append((0, int(d)))
+            else:
+                if v not in like:
+                    like.append(v)
+                pattern.append((1 + like.index(v), int(d)))
+        else:
+            pattern.append(int(p))
+    return Reshape(pattern)(x, *like)
+
+
+def flatten(x, ndim=1):
+    """Keep the first ``ndim - 1`` dimensions, merge the rest
+    (``theano/tensor/basic.py:5160-5220``)."""
+    x = as_tensor_variable(x)
+    if ndim < 1 or ndim > max(x.type.ndim, 1):
+        raise ValueError("invalid output ndimensions (%d) for flatten" % ndim)
+    if x.type.ndim == ndim:
+        return x
+    return Reshape([(0, d) for d in range(ndim - 1)] + [-1])(x)
+
+
+# --------------------------------------------------------------------------
+class Alloc(Op):
+    """``value`` broadcast to a shape (``theano/tensor/basic.py:2769-2960``).
+    ``pattern`` as for :class:`Reshape` without ``-1``; inputs after the first
+    are read for their shape only."""
+
+    __props__ = ("pattern",)
+
+    def __init__(self, pattern):
+        pat = []
+        for p in pattern:
+            if isinstance(p, tuple):
+                pat.append((int(p[0]), int(p[1])))
+            else:
+                if int(p) < 0:
+                    raise ValueError("invalid extent %d in a shape" % int(p))
+                pat.append(int(p))
+        self.pattern = tuple(pat)
+
+    def _props(self):
+        return (self.pattern,)
+
+    def __str__(self):
+        return "%s{%s}" % (type(self).__name__, ", ".join(
+            "in%d.shape[%d]" % p if isinstance(p, tuple) else str(p) for p in self.pattern))
+
+    def make_node(self, value, *like):
+        ins = [as_tensor_variable(value)] + [as_tensor_variable(v) for v in like]
+        v = ins[0]
+        if v.type.ndim > len(self.pattern):
+            raise TypeError("the value has more dimensions (%d) than the shape (%d)" % (v.type.ndim, len(self.pattern)))
+        bcast = []
+        for p in self.pattern:
+            bcast.append(ins[p[0]].type.broadcastable[p[1]] if isinstance(p, tuple) else p == 1)
+        return Apply(self, ins, [TensorType(v.type.dtype, bcast)()])
+
+    def resolve(self, shapes):
+        return tuple(int(shapes[p[0]][p[1]]) if isinstance(p, tuple) else p for p in self.pattern)
+
+    def infer_shape(self, node, shapes):
+        return [self.resolve(shapes)]
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def L_op(self, inputs, outputs, grads):
+        v = inputs[0]
+        (g,) = grads
+        nd_out, nd_v = len(self.pattern), v.type.ndim
+        gv = g
+        if nd_out > nd_v:
+            gv = T.sum(gv, axis=tuple(range(nd_out - nd_v)))
+        b = [d for d in range(nd_v) if v.type.broadcastable[d] and not gv.type.broadcastable[d]]
+        if b:
+            gv = T.sum(gv, axis=tuple(b), keepdims=True)
+        if gv.type.dtype != v.type.dtype:
+            gv = T.cast(gv, v.type.dtype)
+        return [gv] + [i.zeros_like() for i in inputs[1:]]
+
+    def connection_pattern(self, node):
+        return [[True]] + [[False]] * (len(node.inputs) - 1)
+
+
+def alloc(value, *shape):
+    """``shape`` entries: ints or ``(variable, d)`` pairs."""
+    like, pattern = [], []
+    for p in shape:
+        if isinstance(p, tuple):
+            v = as_tensor_variable(p[0])
+            if v not in like:
+                like.append(v)
+            pattern.append((1 + like.index(v), int(p[1])))
+        else:
+            pattern.append(int(p))
+    return Alloc(pattern)(value, *like)
+
+
+# --------------------------------------------------------------------------
+class Join(Op):
+    """Concatenation along ``axis`` (``theano/tensor/basic.py:4120-4470``)."""
+
+    __props__ = ("axis",)
+
+    def __init__(self, axis):
+        self.axis = int(axis)
+
+    def _props(self):
+        return (self.axis,)
+
+    def __str__(self):
+        return "%s{axis=%d}" % (type(self).__name__, self.axis)
+
+    def make_node(self, *tensors):
+        ts = [as_tensor_variable(t) for t in tensors]
+        if not ts:
+            raise ValueError("Cannot join an empty list of tensors")
+        nd = ts[0].type.ndim
+        if any(t.type.ndim != nd for t in ts):
+            raise TypeError("Join() can only join tensors with the same number of dimensions.")
+        if not 0 <= self.axis < nd:
+            raise IndexError("Join axis %d out of bounds [0, %d)" % (self.axis, nd))
+        dtype = ts[0].type.dtype
+        for t in ts[1:]:
+            dtype = T.scal.upcast(dtype, t.type.dtype)
+        ts = [t if t.type.dtype == dtype else T.cast(t, dtype) for t in ts]
+        # a dimension is broadcastable when it is in any input (then all must have extent 1); never the joined one
+        bcast = [any(t.type.broadcastable[d] for t in ts) for d in range(nd)]
+        bcast[self.axis] = len(ts) == 1 and ts[0].type.broadcastable[self.axis]
+        return Apply(self, ts, [TensorType(dtype, bcast)()])
+
+    def infer_shape(self, node, shapes):
+        out = list(shapes[0])
+        out[self.axis] = sum(s[self.axis] for s in shapes)
+        return [tuple(out)]
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def L_op(self, inputs, outputs, grads):
+        (g,) = grads
+        if outputs[0].type.dtype not in T.continuous_dtypes:
+            return [i.zeros_like(dtype=T.config.floatX) for i in inputs]
+        return [JoinPart(self.axis, k)(g, *inputs) for k in range(len(inputs))]
+
+
+class JoinPart(Op):
+    """The slice of a joined tensor that came from input ``k``: the gradient of
+    ``Join`` (the role of ``Split``, ``theano/tensor/basic.py:3700-3860``).  The
+    original tensors are read for their extents only.  A view."""
+
+    __props__ = ("axis", "k")
+    view_map = {0: [0]}
+
+    def __init__(self, axis, k):
+        self.axis, self.k = int(axis), int(k)
+
+    def _props(self):
+        return (self.axis, self.k)
+
+    def __str__(self):
+        return "%s{axis=%d, part=%d}" % (type(self).__name__, self.axis, self.k)
+
+    def make_node(self, g, *tensors):
+        g = as_tensor_variable(g)
+        ts = [as_tensor_variable(t) for t in tensors]
+        part = ts[self.k]
+        return Apply(self, [g] + ts, [TensorType(g.type.dtype, part.type.broadcastable)()])
+
+    def infer_shape(self, node, shapes):
+        return [shapes[1 + self.k]]
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def connection_pattern(self, node):
+        return [[True]] + [[False]] * (len(node.inputs) - 1)
+
+    def L_op(self, inputs, outputs, grads):
+        raise NotImplementedError("second derivatives through join are not implemented")
+
+
+def join(axis, *tensors):
+    ts = [as_tensor_variable(t) for t in tensors]
+    nd = ts[0].type.ndim
+    axis = axis + nd if axis < 0 else axis
+    if len(ts) == 1:
+        return ts[0]
+    return Join(axis)(*ts)
+
+
+concatenate = lambda tensors, axis=0: join(axis, *tensors)  # noqa: E731
+
+
+def stack(tensors, axis=0):
+    """New axis at ``axis``, then join (``theano/tensor/basic.py:4560-4640``)."""
+    ts = [as_tensor_variable(t) for t in tensors]
+    nd = ts[0].type.ndim
+    axis = axis + nd + 1 if axis < 0 else axis
+    order = list(range(nd))
+    order.insert(axis, "x")
+    return join(axis, *[t.dimshuffle(*order) for t in ts])
