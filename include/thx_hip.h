@@ -129,6 +129,9 @@ int thx_elemwise_new(const char* functor_src, const char* functor_name, int n_in
 /* Run on `ins` (n_in arrays) writing `outs` (n_out arrays, preallocated, every
  * one of the full result shape; an output may alias an input exactly for
  * in-place operation). All arrays must have the same rank (<= THX_MAX_ND).
+ * The result shape is the broadcast of the inputs; where every input has
+ * extent 1 the outputs' extent counts (a fill), and outputs may be strided
+ * views (a copy into a slice of a larger array).
  * Fails with THX_ERR_SHAPE on a dimension mis-match. Asynchronous.
  * Replaces GpuElemwise_call(ge, args, GE_BROADCAST) (theano/gpuarray/elemwise.py:376). */
 int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* outs, int flags);

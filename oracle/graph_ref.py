@@ -172,6 +172,7 @@ def evaluate(inputs, outputs, values):
     from theano_amd import gof
     from theano_amd.tensor.elemwise import CAReduce, CAReduceDtype, DimShuffle, Elemwise
     from theano_amd.tensor.basic import MaxAndArgmax, ShapeFloat
+    from theano_amd.tensor import views as V
     env = {}
     for var, val in zip(inputs, values):
         env[var] = var.type.filter(np.asarray(val), strict=False, allow_downcast=False)
@@ -203,6 +204,26 @@ def evaluate(inputs, outputs, values):
             res = [np.asarray(args[0].shape[op.i], dtype=op.dtype)]
         elif isinstance(op, MaxAndArgmax):
             res = list(max_and_argmax(args[0], op.axis))
+        elif isinstance(op, V.Subtensor):          # NumPy basic indexing is the definition (subtensor.py:318-780)
+            res = [args[0][op.idx_list]]
+        elif isinstance(op, V.IncSubtensor):       # subtensor.py:1460-1500
+            x = np.array(args[0], copy=True)
+            if op.set_instead_of_inc:
+                x[op.idx_list] = args[1]
+            else:
+                x[op.idx_list] += args[1]
+            res = [x]
+        elif isinstance(op, V.Reshape):
+            res = [np.reshape(args[0], op.resolve([a.shape for a in args]))]
+        elif isinstance(op, V.Alloc):
+            res = [np.array(np.broadcast_to(args[0], op.resolve([a.shape for a in args])))]
+        elif isinstance(op, V.Join):
+            res = [np.concatenate(args, axis=op.axis)]
+        elif isinstance(op, V.JoinPart):
+            at = sum(a.shape[op.axis] for a in args[1:1 + op.k])
+            idx = [slice(None)] * args[0].ndim
+            idx[op.axis] = slice(at, at + args[1 + op.k].shape[op.axis])
+            res = [args[0][tuple(idx)]]
         else:
             raise NotImplementedError("oracle cannot evaluate %s" % op)
         for o, v in zip(node.outputs, res):

@@ -1,0 +1,104 @@
+"""GPU parity of indexing, inc/set_subtensor, reshape, alloc and join against
+the oracle (NumPy's basic indexing / reshape / broadcast_to / concatenate), alone
+and feeding fused elementwise and reduction kernels, forward and gradient."""
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import hip, tensor as T
+from theano_amd.hip import HipCAReduce, HipElemwise
+from oracle import graph_ref as G
+from conftest import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def both(ins, outs, vals):
+    f = th.function(ins, outs)
+    return f, f(*vals), G.evaluate(ins, outs, vals)
+
+
+def test_views_feed_kernels_without_copies():
+    rng = np.random.default_rng(51)
+    x = T.ftensor3("x")
+    y = T.fmatrix("y")
+    xv = rng.standard_normal((40, 50, 64)).astype("float32")
+    yv = rng.standard_normal((50, 64)).astype("float32")
+    outs = [x[1:30:3, ::-2, 4:60] * 2 + 1, T.sum(x[-1] * y, axis=1), T.max(x[..., 1:-1], axis=(0, 2)),
+            T.exp(x.reshape((-1, 64))[100:300]), T.sum(x.reshape((x.shape[0], -1)), axis=1),
+            x[:, 100:, :] + 1, x[5, 6], T.max_and_argmax(x[:, ::2, 3], axis=0)[1]]
+    f, got, ref = both([x, y], outs, [xv, yv])
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "view case %d" % k)
+    # indexing and reshaping a contiguous array launch nothing: one kernel per output that computes
+    kernels = [n for n in f.toposort() if isinstance(n.op, (HipElemwise, HipCAReduce))]
+    assert len(kernels) == 6
+
+
+def test_reshape_of_strided_array_copies_once():
+    rng = np.random.default_rng(52)
+    x = T.imatrix("x")
+    xv = rng.integers(-100, 100, (70, 90)).astype("int32")
+    outs = [x.dimshuffle(1, 0).reshape((-1,)), T.flatten(x[::2, 1::3], 1), x[::-1].reshape((90, 70)) + 1]
+    f, got, ref = both([x], outs, [xv])
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert g.dtype == r.dtype and np.array_equal(g, r), k
+    with pytest.raises(ValueError):
+        th.function([x], x.reshape((7, -1, 13)))(xv)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "int64", "float16", "bool"])
+def test_alloc_join_stack_inc_set(dtype):
+    rng = np.random.default_rng(53)
+    m = T.TensorType(dtype, (False, False))
+    x, y = m("x"), m("y")
+    r = T.TensorType(dtype, (True, False))("r")
+    if dtype == "bool":
+        xv, yv, rv = [rng.integers(0, 2, s).astype(dtype) for s in ((33, 47), (33, 47), (1, 47))]
+    else:
+        xv, yv, rv = [rng.integers(-9, 9, s).astype(dtype) for s in ((33, 47), (33, 47), (1, 47))]
+    outs = [T.alloc(r, 5, x.shape[0], 47), T.join(0, x, r, y[:7]), T.join(1, x[:, :5], y), T.stack([x, y], axis=1),
+            T.set_subtensor(x, y[:3, 2:9], (slice(4, 7), slice(10, 17))), T.set_subtensor(x, r, (slice(None, None, 5),)),
+            T.alloc(np.asarray(1, dtype), 3, 4)]
+    if dtype != "bool":
+        outs.append(T.inc_subtensor(x, y[:, ::2], (slice(None), slice(1, 25))))
+        outs.append(T.inc_subtensor(x, r, (slice(2, 9),)))
+    f, got, ref = both([x, y, r], outs, [xv, yv, rv])
+    for k, (g, rr) in enumerate(zip(got, ref)):
+        assert g.dtype == rr.dtype and g.shape == rr.shape and np.array_equal(g, rr), (dtype, k)
+    assert np.array_equal(f(xv, yv, rv)[4], ref[4])            # inputs were not modified by the first call
+    with pytest.raises(ValueError):
+        th.function([x, y], T.join(0, x, y[:, :5]))(xv, yv)
+    with pytest.raises(IndexError):
+        th.function([x], x[40])(xv)
+
+
+def test_gradients_through_views():
+    rng = np.random.default_rng(54)
+    x = T.ftensor3("x")
+    y = T.fmatrix("y")
+    r = T.frow("r")
+    xv = rng.standard_normal((6, 9, 16)).astype("float32")
+    yv = rng.standard_normal((9, 16)).astype("float32")
+    rv = rng.standard_normal((1, 16)).astype("float32")
+    cost = (T.sum(T.sqr(x[1:3, ::-2, 4])) + T.sum(T.exp(x.reshape((-1, 16))[3:7] * 0.1)) +
+            T.sum(T.join(0, y, r, y[:2]) ** 3) + T.sum(T.alloc(r, 3, y.shape[0], 16) * x[:3]) +
+            T.sum(T.sqr(T.inc_subtensor(x, y[:2, 1:3], (slice(1, 3), 0, slice(2, 4))))) +
+            T.sum(T.set_subtensor(x, r, (2, slice(None, None, 2))) * x) +
+            T.sum(T.stack([y, y * 2], axis=1)[:, 1] * y))
+    grads = th.grad(cost, [x, y, r])
+    f, got, ref = both([x, y, r], [cost] + grads, [xv, yv, rv])
+    for k, (g, rr) in enumerate(zip(got, ref)):
+        assert_parity(g, rr, "gradient %d" % k, tol=dict(rtol=2e-5, atol=2e-5))
+
+
+def test_minibatch_slices_of_a_large_matrix():
+    """Consecutive row blocks of the configuration-2 matrix reduce to the same
+    values as the whole matrix does."""
+    import workloads as W
+    (val,) = W.c2_inputs("sum_axis1", "full")
+    x = T.fmatrix("x")
+    parts = [T.sum(x[k * 2048:(k + 1) * 2048], axis=1) for k in range(4)]
+    f = th.function([x], [T.join(0, *parts), T.sum(x, axis=1)])
+    joined, whole = f(val)
+    assert np.array_equal(joined, whole)

@@ -292,3 +292,58 @@ def test_max_and_argmax_against_reference_vectors_and_brute_force():
     outs = T.max_and_argmax(x0, axis=1, keepdims=True)
     got = G.evaluate([x0], outs, [x[0]])
     assert got[0].shape == (4, 1) and got[1].shape == (4, 1) and got[1].dtype == np.int64
+
+
+def test_view_ops_against_numpy_and_finite_differences():
+    """Indexing, inc/set_subtensor, reshape, flatten, alloc, join and stack: the
+    node-by-node evaluation equals the NumPy expression it stands for, and the
+    gradients that the ops' L_op build agree with central differences."""
+    from theano_amd.gradient import numeric_grad
+    rng = np.random.default_rng(6)
+    x = T.TensorType("float64", (False, False, False))("x")
+    y = T.TensorType("float64", (False, False))("y")
+    r = T.TensorType("float64", (True, False))("r")
+    xv, yv, rv = rng.standard_normal((4, 5, 6)), rng.standard_normal((5, 6)), rng.standard_normal((1, 6))
+    cases = [
+        (x[1:3, ::-2, 4], xv[1:3, ::-2, 4]),
+        (x[-1], xv[-1]),
+        (x[..., 1:-1], xv[..., 1:-1]),
+        (x[:, 10:, :], xv[:, 10:, :]),                                  # empty result
+        (x.reshape((-1, 6)), xv.reshape(-1, 6)),
+        (x.reshape((x.shape[0], -1)), xv.reshape(4, -1)),
+        (T.flatten(x.dimshuffle(2, 0, 1), 2), xv.transpose(2, 0, 1).reshape(6, -1)),
+        (T.alloc(r, 3, y.shape[0], 6), np.broadcast_to(rv, (3, 5, 6))),
+        (T.join(0, y, r, y[:2]), np.concatenate([yv, rv, yv[:2]], axis=0)),
+        (T.stack([y, y * 2], axis=1), np.stack([yv, yv * 2], axis=1)),
+        (T.inc_subtensor(x, y[:2, 1:3], (slice(1, 3), 0, slice(2, 4))), None),
+        (T.set_subtensor(x, r, (2, slice(None, None, 2))), None),
+    ]
+    exp10 = xv.copy()
+    exp10[1:3, 0, 2:4] += yv[:2, 1:3]
+    exp11 = xv.copy()
+    exp11[2, ::2] = rv
+    cases[10] = (cases[10][0], exp10)
+    cases[11] = (cases[11][0], exp11)
+    for k, (var, expect) in enumerate(cases):
+        got = G.evaluate([x, y, r], [var], [xv, yv, rv])[0]
+        assert got.shape == expect.shape and np.array_equal(got, expect), k
+        assert var.type.ndim == expect.ndim
+    with pytest.raises(IndexError):
+        G.evaluate([x], [x[7]], [xv])
+    with pytest.raises(TypeError):
+        list(x)
+    # gradients through every op
+    w = rng.standard_normal((4, 2)) + 2
+    cost = (T.sum(T.sqr(x[1:3, ::-2, 4]) * w[1:3, :1]) + T.sum(T.exp(x.reshape((-1, 6))[3:7] * 0.1)) +
+            T.sum(T.join(0, y, r, y[:2]) ** 3) + T.sum(T.alloc(r, 3, y.shape[0], 6) * x[:3]) +
+            T.sum(T.sqr(T.inc_subtensor(x, y[:2, 1:3], (slice(1, 3), 0, slice(2, 4))))) +
+            T.sum(T.set_subtensor(x, r, (2, slice(None, None, 2))) * x) +
+            T.sum(T.stack([y, y * 2], axis=1)[:, 1] * y))
+    grads = th.grad(cost, [x, y, r])
+
+    def f(a, b, c):
+        return float(G.evaluate([x, y, r], [cost], [a, b, c])[0])
+    num = numeric_grad(f, [xv, yv, rv])
+    ana = G.evaluate([x, y, r], grads, [xv, yv, rv])
+    for a, n in zip(ana, num):
+        assert a.shape == n.shape and np.allclose(a, n, rtol=1e-5, atol=1e-6)

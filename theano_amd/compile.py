@@ -87,11 +87,11 @@ class Function(object):
         keeps those arrays out of non-temporal accesses so that the last-level cache can serve
         the next read (a batch-norm pass over 100 MB of activations after the statistics pass,
         a reduction over an elementwise result that is also an output)."""
-        from .hip.ops import HipArrayType, HipDimShuffle
+        from .hip.ops import HipArrayType
 
-        def root(v):
-            while v.owner is not None and isinstance(v.owner.op, HipDimShuffle):
-                v = v.owner.inputs[0]
+        def root(v):   # the array a chain of views looks at
+            while v.owner is not None and getattr(v.owner.op, "view_map", None):
+                v = v.owner.inputs[v.owner.op.view_map[0][0]]
             return v
 
         def big(v):

@@ -107,6 +107,16 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   std::vector<View> views;
   int rc = gather_inputs("elemwise", ins, e->n_in, e->dtypes.data(), flags, &nd, shape, &views);
   if (rc) return rc;
+  // Inputs that all have extent 1 along a dimension broadcast to the outputs' extent there
+  // (a fill: every input is a scalar and the output alone carries the shape).
+  if ((flags & THX_BROADCAST) && e->n_out > 0 && outs[0].nd == nd) {
+    for (int d = 0; d < nd; ++d) {
+      if (shape[d] == 1 && outs[0].shape[d] != 1) {
+        shape[d] = outs[0].shape[d];
+        for (int i = 0; i < e->n_in; ++i) views[i].stride[d] = 0;
+      }
+    }
+  }
   views.resize(nops);
   for (int o = 0; o < e->n_out; ++o) {
     const thx_array& a = outs[o];

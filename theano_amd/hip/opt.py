@@ -19,6 +19,7 @@ from ..gof import Constant
 from ..tensor import basic as T
 from ..tensor.elemwise import All, Any, CAReduce, CAReduceDtype, DimShuffle, Elemwise
 from ..tensor.type import TensorConstant, TensorType
+from . import views as hip_views
 from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipMaxAndArgmax, HipToHost, HostToHip,
                   _is_host_scalar, as_hip_variable, hip_from_host, host_from_hip)
 
@@ -77,7 +78,8 @@ def lift_to_hip(fgraph):
     for node in fgraph.toposort():
         ins = [mapped(i) for i in node.inputs]
         op = node.op
-        if isinstance(op, (HipElemwise, HipCAReduce, HipMaxAndArgmax, HipDimShuffle, HostToHip, HipToHost, T.ShapeFloat)):
+        if isinstance(op, (HipElemwise, HipCAReduce, HipMaxAndArgmax, HipDimShuffle, HostToHip, HipToHost, T.ShapeFloat) +
+                      hip_views.DEVICE_OPS):
             if isinstance(op, HostToHip) and isinstance(ins[0].type, HipArrayType):
                 outs = [ins[0]]
             elif isinstance(op, HipToHost) and isinstance(ins[0].type, TensorType):
@@ -100,6 +102,9 @@ def lift_to_hip(fgraph):
             outs = [_lift_reduce(node, x)]
         elif isinstance(op, T.MaxAndArgmax):
             outs = HipMaxAndArgmax(op.axis).make_node(ins[0]).outputs
+        elif type(op) in hip_views.LIFT:
+            outs = hip_views.LIFT[type(op)](op).make_node(*ins).outputs
+
         else:
             raise NotImplementedError("%s has no HIP implementation and nothing runs on the host" % op)
         for o, no in zip(node.outputs, outs):

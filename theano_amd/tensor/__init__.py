@@ -12,3 +12,5 @@ from .elemwise import DimShuffle, Elemwise, CAReduce, CAReduceDtype, Sum, Prod, 
 from .basic import *  # noqa: F401,F403
 from .basic import Max, MaxAndArgmax, Min, ShapeFloat, makeKeepDims, cast, round  # noqa: F401
 from . import nnet  # noqa: F401,E402
+from .views import (Alloc, IncSubtensor, Join, Reshape, Subtensor, alloc, concatenate, flatten, inc_subtensor,  # noqa: F401,E402
+                    join, reshape, set_subtensor, stack, subtensor)

@@ -140,6 +140,31 @@ class _tensor_py_operators(object):
     def T(self):
         return self.dimshuffle(*reversed(range(self.ndim)))
 
+    def __getitem__(self, idx):
+        from . import views
+        return views.subtensor(self, idx)
+
+    def __iter__(self):
+        # without this Python would iterate through __getitem__ forever
+        raise TypeError("a symbolic tensor cannot be iterated over; index it explicitly")
+
+    @property
+    def shape(self):
+        """``x.shape[d]`` is the pair ``(x, d)``: the way ``reshape`` and ``alloc`` name an extent
+        that is only known when the function runs."""
+        return tuple((self, d) for d in range(self.ndim))
+
+    def reshape(self, *shape):
+        from . import views
+        if len(shape) == 1 and isinstance(shape[0], (list, tuple)) and not (
+                len(shape[0]) == 2 and hasattr(shape[0][0], "type")):
+            shape = tuple(shape[0])
+        return views.reshape(self, shape)
+
+    def flatten(self, ndim=1):
+        from . import views
+        return views.flatten(self, ndim)
+
     def astype(self, dtype):
         return self._b().cast(self, dtype)
 

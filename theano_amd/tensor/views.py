@@ -168,7 +168,6 @@ class IncSubtensor(Op):
         bdims = [d for d in range(y.type.ndim) if y.type.broadcastable[d] and not gy.type.broadcastable[d]]
         if bdims:
             gy = T.sum(gy, axis=tuple(bdims), keepdims=True)
-            gy = T.DimShuffle(gy.type.broadcastable, list(range(gy.type.ndim)))(gy) if gy.type != y.type else gy
         if self.set_instead_of_inc:
             gx = IncSubtensor(self.idx_list, True)(g, T.zeros_like(Subtensor(self.idx_list)(g)))
         else:
