@@ -52,6 +52,9 @@ def test_nan_is_the_maximum_and_first_nan_wins():
     val[10, 2999] = np.nan
     val[20, :] = -np.inf
     val[21, :] = np.inf
+    val[30, :] = -1.0
+    val[30, 1500] = 0.0                       # +0 after -0: equal values, the first one is the argmax
+    val[30, 700] = -0.0
     for ax in (0, 1, None):
         got, ref, plan = run(x, T.max_and_argmax(x, axis=ax), val)
         same(got, ref, "nan axis %s [%s]" % (ax, plan))

@@ -10,6 +10,8 @@
 //   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK, GS (grid-stride loop over chunks) };
 //   static constexpr unsigned long long NT;             // bit i: operand i is accessed non-temporally
 //   static constexpr int mode(int operand);             // M_VEC / M_BCAST / M_GATHER
+//   static constexpr int sclass(int operand, int dim);  // stride is 0 / is 1 / anything (2)
+//   static constexpr int alias(int operand);            // first operand with identical strides
 // The host collapses dimensions, so ND is the rank after merging every pair of
 // neighbouring dimensions that all operands walk with compatible strides.
 #pragma once
@@ -73,6 +75,12 @@ struct EwAcc {
   }
 };
 
+// coordinate * stride with the multiply only where the plan could not rule it out
+template <class P, class IT>
+THX_DEV IT ew_term(int operand, int dim, IT coord, IT stride) {
+  return P::sclass(operand, dim) == 0 ? (IT)0 : (P::sclass(operand, dim) == 1 ? coord : coord * stride);
+}
+
 // One thread handles UNR vectors, BLOCK apart, so a wave's accesses stay
 // contiguous; all loads are issued before any arithmetic or store.
 template <class F, class P>
@@ -94,22 +102,31 @@ __device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename 
     a[u].ptr = p.ptr;
     a[u].imm = p.imm;
     a[u].stride = p.stride;
+    // offset of the vector in every operand: sum over dimensions of coordinate * stride, where the
+    // plan says which strides are 0 or 1 (no multiply; 32-bit integer multiplies run at quarter
+    // rate) and which operands walk memory exactly like an earlier one (same offset)
     if (ND == 1) {
 #pragma unroll
-      for (int i = 0; i < NOPS; ++i) a[u].off[i] = (IT)(q * VEC) * p.stride[i][0];
+      for (int i = 0; i < NOPS; ++i) a[u].off[i] = ew_term<P>(i, 0, (IT)(q * VEC), p.stride[i][0]);
     } else {
       UT rem = (UT)(full[u] ? q : 0), c;
       divmod(rem, p.fd[ND - 1], rem, c);
 #pragma unroll
-      for (int i = 0; i < NOPS; ++i) a[u].off[i] = (IT)(c * VEC) * p.stride[i][ND - 1];
+      for (int i = 0; i < NOPS; ++i)
+        if (P::alias(i) == i) a[u].off[i] = ew_term<P>(i, ND - 1, (IT)(c * VEC), p.stride[i][ND - 1]);
 #pragma unroll
       for (int d = ND - 2; d >= 1; --d) {
         divmod(rem, p.fd[d], rem, c);
 #pragma unroll
-        for (int i = 0; i < NOPS; ++i) a[u].off[i] += (IT)c * p.stride[i][d];
+        for (int i = 0; i < NOPS; ++i)
+          if (P::alias(i) == i) a[u].off[i] += ew_term<P>(i, d, (IT)c, p.stride[i][d]);
       }
 #pragma unroll
-      for (int i = 0; i < NOPS; ++i) a[u].off[i] += (IT)rem * p.stride[i][0];
+      for (int i = 0; i < NOPS; ++i)
+        if (P::alias(i) == i) a[u].off[i] += ew_term<P>(i, 0, (IT)rem, p.stride[i][0]);
+#pragma unroll
+      for (int i = 0; i < NOPS; ++i)
+        if (P::alias(i) != i) a[u].off[i] = a[u].off[P::alias(i)];
     }
     if (full[u]) F::template load<VEC>(a[u], r[u]);
   }

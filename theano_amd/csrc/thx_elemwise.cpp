@@ -335,8 +335,27 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   int gs = env_int("THX_EW_GS", 0);
   if (!gs && ceil_div64(nvec, (int64_t)block * unr) * block > 0xffffffffLL) gs = 64;
 
+  // per operand and dimension: is the stride 0, 1 or anything; and which earlier operand has the
+  // very same strides (its offset is reused)
+  std::vector<std::vector<int>> sclass(nops, std::vector<int>(ND, 2));
+  std::vector<int> alias(nops);
+  std::string skey;
+  for (int o = 0; o < nops; ++o) {
+    alias[o] = o;
+    for (int d = 0; d < ND; ++d) {
+      const int64_t st = views[o].imm ? 0 : dm.stride[o][d];
+      sclass[o][d] = st == 0 ? 0 : (st == 1 ? 1 : 2);
+    }
+    for (int q = 0; q < o && alias[o] == o; ++q)
+      if (!views[o].imm && !views[q].imm &&
+          std::equal(dm.stride[q].begin(), dm.stride[q].begin() + ND, dm.stride[o].begin()))
+        alias[o] = q;
+    for (int d = 0; d < ND; ++d) skey += char('0' + sclass[o][d]);
+    if (alias[o] != o) skey += "a" + std::to_string(alias[o]);
+    if (o + 1 < nops) skey += ".";
+  }
   std::ostringstream key;
-  key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr;
+  key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|s" << skey;
   if (nt) key << "|nt" << std::hex << nt << std::dec;
   key << (block != 256 ? "|b" + std::to_string(block) : "") << (gs ? "|gs" : "") << "|m";
   for (int o = 0; o < nops; ++o) key << mode[o] << (o + 1 < nops ? "," : "");
@@ -354,6 +373,14 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
       << " IT;\n  enum { ND = " << ND << ", VEC = " << vec << ", UNR = " << unr << ", BLOCK = " << block
       << ", GS = " << (gs ? 1 : 0) << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
     for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
+    s << "};\n    return m[i];\n  }\n  static constexpr int sclass(int i, int d) {\n    constexpr int m[][" << ND << "] = {";
+    for (int o = 0; o < nops; ++o) {
+      s << "{";
+      for (int d = 0; d < ND; ++d) s << sclass[o][d] << (d + 1 < ND ? ", " : "");
+      s << "}" << (o + 1 < nops ? ", " : "");
+    }
+    s << "};\n    return m[i][d];\n  }\n  static constexpr int alias(int i) {\n    constexpr int m[] = {";
+    for (int o = 0; o < nops; ++o) s << alias[o] << (o + 1 < nops ? ", " : "");
     s << "};\n    return m[i];\n  }\n};\n"
       << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::EwParams<" << e->name
       << "::NOPS, ThxPlan::ND, ThxPlan::IT> p) {\n  thx::ew_body<" << e->name << ", ThxPlan>(p);\n}\n";

@@ -293,7 +293,10 @@ static int compile_source(const std::string& src, const std::string& arch, std::
                                    "-packed-fp32-ops"};
   // float32 division and sqrt within 2.5 ulp instead of correctly rounded: a tenth of the instructions,
   // and two orders of magnitude inside the float32 parity tolerance (rtol 1e-5)
-  if (fast_div()) opts.push_back("-fno-hip-fp32-correctly-rounded-divide-sqrt");
+  if (fast_div()) {
+    opts.push_back("-fno-hip-fp32-correctly-rounded-divide-sqrt");
+    opts.push_back("-DTHX_FAST_DIV");
+  }
   r = hiprtcCompileProgram(prog, (int)opts.size(), opts.data());
   if (r != HIPRTC_SUCCESS) {
     size_t n = 0;
@@ -324,6 +327,11 @@ int get_kernel(const std::string& source, const std::string& entry, Kernel* out)
       *out = it->second;
       return THX_OK;
     }
+  }
+  if (const char* dump = getenv("THX_DUMP_DIR")) {  // the generated source, named by its entry point
+    mkdirs(dump);
+    std::ofstream f(std::string(dump) + "/" + entry + ".hip");
+    f << source;
   }
   std::vector<char> code;
   const std::string& dir = cache_dir();

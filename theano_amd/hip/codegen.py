@@ -192,7 +192,7 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
     return "struct %s {\n%s\n};\n" % (name, text), name, acc_struct_bytes(acc_dtypes)
 
 
-def argmax_functor(in_dtypes, value_dtype, pre_op=None):
+def argmax_functor(in_dtypes, value_dtype, pre_op=None, packed=False):
     """(source, name, sizeof(Acc)) of the reduction behind ``MaxAndArgmax``.
 
     The inputs are ``in_dtypes`` followed by one int64 position operand (the
@@ -201,12 +201,24 @@ def argmax_functor(in_dtypes, value_dtype, pre_op=None):
     the accumulator is the pair (value, position).  Merging keeps the greater
     value, a NaN before any number, and on equal values (or two NaNs) the smaller
     position - so the result is NumPy's first occurrence whatever order partial
-    results meet in."""
+    results meet in.
+
+    ``packed`` (values of at most 32 bits, fewer than 2^31 reduced elements per
+    result): the pair travels as one unsigned 64-bit key - the value mapped to an
+    order-preserving unsigned 32-bit number (every NaN to the largest) in the high
+    half, the complemented position in the low half - so merging is a single
+    64-bit maximum instead of a cascade of comparisons and selects."""
     nin = len(in_dtypes)
     ins = ["i%d" % k for k in range(nin)]
     vt = compute_ctype(value_dtype)
+    st = storage_ctype(value_dtype)
+    if packed and np.dtype(value_dtype).itemsize > 4:
+        raise ValueError("packed keys hold values of at most 32 bits")
     lines = ["  enum { NIN = %d, NOUT = 2, NEX = 0 };" % (nin + 1)]
-    lines.append("  struct Acc { %s val; long long idx; };" % vt)
+    if packed:
+        lines.append("  struct Acc { unsigned long long key; };")
+    else:
+        lines.append("  struct Acc { %s val; long long idx; };" % vt)
     lines.append(_regs(list(in_dtypes) + ["int64"], ins + ["ix"]).rstrip("\n"))
     if value_dtype in scal.float_dtypes:
         lowest = c_literal(-np.inf, value_dtype)
@@ -214,36 +226,62 @@ def argmax_functor(in_dtypes, value_dtype, pre_op=None):
         lowest = c_literal(0, value_dtype)
     else:
         lowest = c_literal(np.iinfo(value_dtype).min, value_dtype)
-    lines.append("  THX_DEV static void init(Acc& a) { a.val = %s; a.idx = 0x7fffffffffffffffLL; }" % lowest)
+    if packed:
+        lines.append("  THX_DEV static void init(Acc& a) { a.key = 0ull; }")
+    else:
+        lines.append("  THX_DEV static void init(Acc& a) { a.val = %s; a.idx = 0x7fffffffffffffffLL; }" % lowest)
     lines.append("  template <int V, class A> THX_DEV static void load(const A& a, Regs<V>& r) { %s a.template ld<%d>(r.ix); }"
                  % (" ".join("a.template ld<%d>(r.%s);" % (k, nm) for k, nm in enumerate(ins)), nin))
     if pre_op is None:
         if nin != 1:
             raise ValueError("without prologue the reduction takes one input")
-        pre_stmt = "v.val = (%s)i0;" % vt
+        value_stmt = "const %s val = (%s)i0;" % (vt, vt)
     else:
         pnode = _scalar_node(pre_op, in_dtypes)
         if len(pnode.outputs) != 1 or pnode.outputs[0].type.dtype != value_dtype:
             raise TypeError("prologue must yield one %s value" % value_dtype)
-        pre_stmt = "%s p0;\n%s\nv.val = (%s)p0;" % (vt, pre_op.c_code(pnode, ins, ["p0"]), vt)
-    lines.append("  THX_DEV static void pre(%s, const long long ix, Acc& v) {\n%s\n    v.idx = ix;\n  }" % (
+        value_stmt = "%s p0;\n%s\nconst %s val = (%s)p0;" % (vt, pre_op.c_code(pnode, ins, ["p0"]), vt, vt)
+    if packed:
+        if value_dtype in scal.float_dtypes:        # float16 widens exactly to float32
+            # adding +0 turns -0 into +0: the two compare equal, so they must share one key
+            to_key = ("const float f = (float)val + 0.0f;\nunsigned int b = __float_as_uint(f);\n"
+                      "b = (f != f) ? 0xffffffffu : (b ^ ((b >> 31) ? 0xffffffffu : 0x80000000u));")
+            from_key = ("const unsigned int k = (unsigned int)(a.key >> 32);\n"
+                        "const %s val = (%s)(k == 0xffffffffu ? __uint_as_float(0x7fc00000u) : "
+                        "__uint_as_float((k >> 31) ? (k ^ 0x80000000u) : ~k));" % (st, st))
+        elif value_dtype in scal.int_dtypes:
+            to_key = "const unsigned int b = (unsigned int)(int)val ^ 0x80000000u;"
+            from_key = "const %s val = (%s)(int)((unsigned int)(a.key >> 32) ^ 0x80000000u);" % (st, st)
+        else:                                        # unsigned integers and bool
+            to_key = "const unsigned int b = (unsigned int)val;"
+            from_key = "const %s val = (%s)(unsigned int)(a.key >> 32);" % (st, st)
+        pre_stmt = "%s\n%s\nv.key = ((unsigned long long)b << 32) | (unsigned int)~(unsigned int)ix;" % (value_stmt, to_key)
+        comb = "    if (b.key > a.key) a.key = b.key;"
+        shfl = "Acc r; r.key = thx::shfl_xor_t(a.key, m); return r;"
+        post = ("%s\n((%s*)o.ptr[0])[idx] = val;\n"
+                "((long long*)o.ptr[1])[idx] = (long long)(unsigned int)~(unsigned int)a.key;" % (from_key, st))
+        size = 8
+    else:
+        pre_stmt = "%s\nv.val = val;\nv.idx = ix;" % value_stmt
+        nan_a, nan_b = ("a.val != a.val", "b.val != b.val") if value_dtype in scal.float_dtypes else ("false", "false")
+        comb = ("    const bool an = %s, bn = %s;\n"
+                "    const bool take = bn ? (!an || b.idx < a.idx)\n"
+                "                         : (!an && (b.val > a.val || (b.val == a.val && b.idx < a.idx)));\n"
+                "    if (take) a = b;" % (nan_a, nan_b))
+        shfl = "Acc r; r.val = thx::shfl_xor_t(a.val, m); r.idx = thx::shfl_xor_t(a.idx, m); return r;"
+        post = "((%s*)o.ptr[0])[idx] = (%s)a.val;\n((long long*)o.ptr[1])[idx] = a.idx;" % (st, st)
+        size = 16
+    lines.append("  THX_DEV static void pre(%s, const long long ix, Acc& v) {\n%s\n  }" % (
         ", ".join("const %s %s" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)), _indent(pre_stmt, 4)))
-    nan_a, nan_b = ("a.val != a.val", "b.val != b.val") if value_dtype in scal.float_dtypes else ("false", "false")
-    lines.append("  THX_DEV static void comb(Acc& a, const Acc& b) {\n"
-                 "    const bool an = %s, bn = %s;\n"
-                 "    const bool take = bn ? (!an || b.idx < a.idx)\n"
-                 "                         : (!an && (b.val > a.val || (b.val == a.val && b.idx < a.idx)));\n"
-                 "    if (take) a = b;\n  }" % (nan_a, nan_b))
+    lines.append("  THX_DEV static void comb(Acc& a, const Acc& b) {\n%s\n  }" % comb)
     call = ", ".join(["(%s)r.%s.v[k]" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)] + ["r.ix.v[k]"])
     lines.append("  template <int V> THX_DEV static void accum(Acc& s, const Regs<V>& r) {\n#pragma unroll\n"
                  "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s, t); }\n  }" % call)
     lines.append("  template <int V> THX_DEV static void accum_lanes(Acc* s, const Regs<V>& r) {\n#pragma unroll\n"
                  "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s[k], t); }\n  }" % call)
-    lines.append("  THX_DEV static Acc shfl_xor(const Acc& a, int m) { Acc r; r.val = thx::shfl_xor_t(a.val, m); "
-                 "r.idx = thx::shfl_xor_t(a.idx, m); return r; }")
-    st = storage_ctype(value_dtype)
-    lines.append("  template <class O> THX_DEV static void post(const O& o, long long idx, const Acc& a) {\n"
-                 "    ((%s*)o.ptr[0])[idx] = (%s)a.val;\n    ((long long*)o.ptr[1])[idx] = a.idx;\n  }" % (st, st))
+    lines.append("  THX_DEV static Acc shfl_xor(const Acc& a, int m) { %s }" % shfl)
+    lines.append("  template <class O> THX_DEV static void post(const O& o, long long idx, const Acc& a) {\n%s\n  }"
+                 % _indent(post, 4))
     text = "\n".join(lines)
     name = _name("A", text)
-    return "struct %s {\n%s\n};\n" % (name, text), name, 16
+    return "struct %s {\n%s\n};\n" % (name, text), name, size

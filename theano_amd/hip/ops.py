@@ -503,13 +503,13 @@ class HipMaxAndArgmax(Op):
         kept = tuple(full[d] for d in range(nd) if d not in self.axis)
         return [kept, kept]
 
-    def _handle(self, node):
+    def _handle(self, node, packed):
         in_dt = tuple(i.type.dtype for i in node.inputs)
         vdt = node.outputs[0].type.dtype
-        key = (self._props(), in_dt)
+        key = (self._props(), in_dt, packed)
         h = _argmax_handles.get(key)
         if h is None:
-            src, name, acc_bytes = codegen.argmax_functor(in_dt, vdt, self.pre_scalar_op)
+            src, name, acc_bytes = codegen.argmax_functor(in_dt, vdt, self.pre_scalar_op, packed)
             all_dt = in_dt + ("int64", vdt, "int64")
             codes = (ctypes.c_int32 * len(all_dt))(*[scal.dtype_code(d) for d in all_dt])
             handle = ctypes.c_void_p()
@@ -521,7 +521,9 @@ class HipMaxAndArgmax(Op):
     def perform(self, node, inputs, output_storage):
         cache = node.tag.get("thx")
         if cache is None:
-            handle = self._handle(node)
+            small = np.dtype(node.outputs[0].type.dtype).itemsize <= 4
+            # one 64-bit key per (value, position) pair while positions fit 31 bits, else the pair itself
+            handle = (self._handle(node, True) if small else None, self._handle(node, False))
             nin = len(node.inputs)
             nd = max(i.type.ndim for i in node.inputs)
             ins = (thx_array * (nin + 1))()
@@ -534,8 +536,12 @@ class HipMaxAndArgmax(Op):
                                        np.dtype(node.outputs[0].type.dtype))
         handle, nin, ins, outs, nd, mask, vdt = cache
         shape = _check_runtime_broadcast(node.inputs, inputs, nd)
-        if any(shape[a] == 0 for a in self.axis):
+        n_red = 1
+        for a in self.axis:
+            n_red *= shape[a]
+        if n_red == 0:
             raise ValueError("attempt to get argmax of an empty sequence")
+        handle = handle[0] if (handle[0] is not None and n_red < 2 ** 31) else handle[1]
         for k, v in enumerate(inputs):
             _operand(v, nd, ins[k])
         kept = tuple(shape[d] for d in range(nd) if d not in self.axis)

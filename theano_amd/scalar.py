@@ -663,6 +663,10 @@ class TrueDiv(BinaryScalarOp):
     def c_code(self, node, inputs, outputs):
         if all(i.type.dtype in discrete_dtypes for i in node.inputs):
             return "%s = ((double)%s) / %s;" % (outputs[0], inputs[0], inputs[1])
+        if node.outputs[0].type.dtype in ("float16", "float32"):
+            # single-precision division goes through the device helper (a plain `/` unless the
+            # library was asked for the 2.5-ulp form); the reference's text is `x / y`
+            return "%s = thx_fdiv(%s, %s);" % (outputs[0], inputs[0], inputs[1])
         return "%s = %s / %s;" % (outputs[0], inputs[0], inputs[1])
 
     def L_op(self, inputs, outputs, gout):
@@ -989,6 +993,10 @@ neg = Neg(same_out_nobool, name="neg")
 
 class Inv(UnaryScalarOp):
     def c_code(self, node, inputs, outputs):
+        if node.outputs[0].type.dtype in ("float16", "float32"):
+            # the reference's `1.0 / x` is a double division rounded to float; on the device the
+            # single-precision helper gives the same value to within its 2.5 ulp
+            return "%s = thx_fdiv(1.0f, %s);" % (outputs[0], inputs[0])
         return "%s = 1.0 / %s;" % (outputs[0], inputs[0])
 
     def L_op(self, inputs, outputs, gout):
@@ -1041,7 +1049,7 @@ class ScalarSigmoid(UnaryScalarOp):
         t = node.inputs[0].type.dtype
         (x,), (z,) = inputs, outputs
         if t in ("float32", "float16"):
-            return "%s = %s < -88.0f ? 0.0f : %s > 15.0f ? 1.0f : 1.0f / (1.0f + expf(-%s));" % (z, x, x, x)
+            return "%s = %s < -88.0f ? 0.0f : %s > 15.0f ? 1.0f : thx_fdiv(1.0f, 1.0f + expf(-%s));" % (z, x, x, x)
         if t == "float64":
             return "%s = %s < -709.0 ? 0.0 : %s > 19.0 ? 1.0 : 1.0 / (1.0 + exp(-%s));" % (z, x, x, x)
         raise NotImplementedError("only floating point is implemented")
