@@ -30,8 +30,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each
 # scaled by what the same counter reads for the --copy-probe kernel of known size), by kernel symbol.
 MEASURED_TRAFFIC = {
-    # sum(axis=1) of float32 (8192, 8192): FETCH_SIZE 131093.1 x 1.99972 KiB + WRITE_SIZE 262.0 KiB
-    "thx_rr_k1_i32_v4_u4_t256_a0_m0_fd_Ra004ded952553fcd": 268709122,
+    # sum(axis=1) of float32 (8192, 8192): FETCH_SIZE 131091.1 x 1.99979 KiB + WRITE_SIZE 256.4 x 0.99875 KiB
+    "thx_rr_k1_i32_v4_u4_t256_a0_nt1_m0_fd_Ra004ded952553fcd": 268709251,
 }
 
 

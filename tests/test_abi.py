@@ -107,3 +107,27 @@ def test_every_kernel_family_compiles_for_gfx950(dry_run):
         th.function([v], out)(np.zeros((33, 40), dt))
     stats = hip.cache_stats()
     assert stats["compiled"] + stats["disk_hits"] > 0
+
+
+def test_header_constants_match_the_binding():
+    """Flag and dtype values written in include/thx_hip.h are the ones the ctypes
+    binding uses."""
+    header = open(os.path.join(ROOT, "include", "thx_hip.h")).read()
+    defines = dict((k, int(v, 0)) for k, v in re.findall(r"#define\s+(THX_[A-Z_]+)\s+(0x[0-9a-fA-F]+|\d+)", header))
+    for name in ("THX_BROADCAST", "THX_DRY_RUN", "THX_HOST_SCALAR", "THX_INDEX", "THX_REUSED"):
+        assert defines[name] == getattr(runtime, name), name
+    enum = re.search(r"THX_BOOL = 0.*?THX_NDTYPES = 12", header, re.S).group(0)
+    codes = dict((k, int(v)) for k, v in re.findall(r"(THX_[A-Z0-9]+) = (\d+)", enum))
+    from theano_amd import scalar as scal
+    names = {"bool": "BOOL", "int8": "I8", "uint8": "U8", "int16": "I16", "uint16": "U16", "int32": "I32",
+             "uint32": "U32", "int64": "I64", "uint64": "U64", "float16": "F16", "float32": "F32", "float64": "F64"}
+    for dt, short in names.items():
+        assert scal.dtype_code(dt) == codes["THX_" + short], dt
+
+
+def test_generated_sources_can_be_dumped(dry_run, tmp_path, monkeypatch):
+    monkeypatch.setenv("THX_DUMP_DIR", str(tmp_path))
+    x = T.fmatrix("x")
+    th.function([x], T.tanh(x) * 3.5 + 0.25)(np.zeros((5, 77), "float32"))
+    files = [f for f in os.listdir(str(tmp_path)) if f.endswith(".hip")]
+    assert files and any("tanh" in open(os.path.join(str(tmp_path), f)).read() for f in files)
