@@ -131,3 +131,23 @@ def test_generated_sources_can_be_dumped(dry_run, tmp_path, monkeypatch):
     th.function([x], T.tanh(x) * 3.5 + 0.25)(np.zeros((5, 77), "float32"))
     files = [f for f in os.listdir(str(tmp_path)) if f.endswith(".hip")]
     assert files and any("tanh" in open(os.path.join(str(tmp_path), f)).read() for f in files)
+
+
+def test_product_never_touches_the_oracle_or_a_host_fallback():
+    """Nothing under theano_amd/ imports, loads or names the oracle, NumPy
+    never computes an op's result there (perform of every host op raises), and
+    the binding refuses to import without the HIP library."""
+    pkg = os.path.join(ROOT, "theano_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".cpp", ".h", ".hip")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text.replace("noracle", ""), os.path.join(dirpath, f)
+    x = T.fmatrix("x")
+    for var in (T.exp(x), T.sum(x, axis=0), T.max_and_argmax(x, axis=1)[1], x[1:3], x.reshape((-1,)),
+                T.join(0, x, x), T.alloc(x, 2, 3, 4)):
+        node = var.owner
+        with pytest.raises(NotImplementedError):
+            node.op.perform(node, [np.zeros((3, 4), "float32")] * len(node.inputs), [[None] for _ in node.outputs])
+    src = open(os.path.join(pkg, "hip", "runtime.py")).read()
+    assert "ctypes.CDLL" in src and "raise" in src[src.index("_LIB_PATH"):src.index("ctypes.CDLL")]
