@@ -92,7 +92,12 @@ struct RedAcc {
 };
 
 // Plan members: typedef IT; enum { NK, VEC, UNR, BLOCK, TPR, RA2 (1 when RA > 1) };
-// static constexpr int mode(int input).
+// static constexpr int mode(int input); static constexpr int sclass(int input, int which).
+template <class P, class IT>
+THX_DEV IT red_term(int input, int which, IT coord, IT stride) {
+  return P::sclass(input, which) == 0 ? (IT)0 : (P::sclass(input, which) == 1 ? coord : coord * stride);
+}
+
 template <class R, class P>
 __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p) {
   typedef typename P::IT IT;
@@ -143,15 +148,17 @@ __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, R:
         a.ptr = p.in;
         a.imm = p.imm;
         a.vstride = p.rc_stride;
+        // P::sclass(input, 0 | 1): the stride along RA | RC is 0, is 1, or anything - a multiply only
+        // in the last case (32-bit integer multiplies run at quarter rate)
         if (P::RA2) {
           UT ra, cv;
           divmod((UT)(ok[u] ? q : j0), p.rcv, ra, cv);
 #pragma unroll
           for (int i = 0; i < NIN; ++i)
-            a.off[i] = base[i] + (IT)ra * p.ra_stride[i] + (IT)(cv * VEC) * p.rc_stride[i];
+            a.off[i] = base[i] + red_term<P>(i, 0, (IT)ra, p.ra_stride[i]) + red_term<P>(i, 1, (IT)(cv * VEC), p.rc_stride[i]);
         } else {
 #pragma unroll
-          for (int i = 0; i < NIN; ++i) a.off[i] = base[i] + (IT)(q * VEC) * p.rc_stride[i];
+          for (int i = 0; i < NIN; ++i) a.off[i] = base[i] + red_term<P>(i, 1, (IT)(q * VEC), p.rc_stride[i]);
         }
         if (ok[u]) R::template load<VEC>(a, r[u]);
       }

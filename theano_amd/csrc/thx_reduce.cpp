@@ -3,6 +3,7 @@
 // slice split for the device, compiles on first use and launches one or two
 // passes.
 #include <algorithm>
+#include <array>
 #include <cstdlib>
 #include <cstring>
 #include <sstream>
@@ -53,13 +54,21 @@ static int env_int(const char* name, int dflt) {
 }
 
 static std::string plan_struct(bool wide, const std::vector<std::pair<std::string, int64_t>>& consts,
-                               const std::vector<int>& mode, uint64_t nt) {
+                               const std::vector<int>& mode, uint64_t nt,
+                               const std::vector<std::array<int, 2>>& sclass = {}) {
   std::ostringstream s;
   s << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int") << " IT;\n  enum { ";
   for (size_t i = 0; i < consts.size(); ++i) s << consts[i].first << " = " << consts[i].second << (i + 1 < consts.size() ? ", " : "");
   s << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
   for (size_t i = 0; i < mode.size(); ++i) s << mode[i] << (i + 1 < mode.size() ? ", " : "");
-  s << "};\n    return m[i];\n  }\n};\n";
+  s << "};\n    return m[i];\n  }\n";
+  if (!sclass.empty()) {
+    s << "  static constexpr int sclass(int i, int w) {\n    constexpr int m[][2] = {";
+    for (size_t i = 0; i < sclass.size(); ++i)
+      s << "{" << sclass[i][0] << ", " << sclass[i][1] << "}" << (i + 1 < sclass.size() ? ", " : "");
+    s << "};\n    return m[i][w];\n  }\n";
+  }
+  s << "};\n";
   return s.str();
 }
 
@@ -350,8 +359,16 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     }
     if (ra2 && nvec >= (int64_t(1) << 31) - 65536) wide = true;
     const int NK = std::max(1, NKD);
+    std::vector<std::array<int, 2>> sclass(NIN);
+    std::string skey;
+    for (int i = 0; i < NIN; ++i) {
+      auto cls = [](int64_t st) { return st == 0 ? 0 : (st == 1 ? 1 : 2); };
+      sclass[i] = {views[i].imm ? 0 : cls(ra_stride[i]), views[i].imm ? 0 : cls(rc_stride[i])};
+      skey += char('0' + sclass[i][0]);
+      skey += char('0' + sclass[i][1]);
+    }
     std::ostringstream key;
-    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|t" << tpr << "|a" << ra2 << (nt ? "|nt" + std::to_string(nt) : "") << "|m";
+    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -361,7 +378,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}}, mode, nt)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}}, mode, nt, sclass)
         << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void " << entry << "(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";

@@ -458,6 +458,32 @@ def _try_epilogue(fgraph, red, cand):
     else:
         layout = red.outputs[0].type.broadcastable
     s_args, used = [], set()
+
+    def operand(i, depth):
+        """Scalar expression for an input that does not come from ``red``: a constant, a host
+        scalar or per-result device array (an extra operand of the epilogue), or a cheap
+        elementwise node over such values (a cast of gamma, say), recomputed in the epilogue."""
+        c = _scalar_constant(i)
+        if c is not None:
+            return c
+        per_result = (isinstance(i.type, HipArrayType) and tuple(i.type.broadcastable) == tuple(layout) and
+                      not _depends_on(i, red))
+        if not (_is_host_scalar(i) or per_result):
+            return None
+        p = i.owner
+        if (per_result and p is not None and isinstance(p.op, HipElemwise) and len(p.outputs) == 1 and depth < 4 and
+                _cheap(p.op.scalar_op, _TRIVIAL_OPS)):
+            args = [operand(v, depth + 1) for v in p.inputs]
+            if all(a is not None for a in args):
+                return p.op.scalar_op(*args)
+        for e, se in zip(extras, s_extras):
+            if e is i:
+                return se
+        sv = scal.Scalar(i.type.dtype)()
+        extras.append(i)
+        s_extras.append(sv)
+        return sv
+
     for i in cand.inputs:
         src = i.owner.inputs[0] if (ds_op is not None and i.owner is not None and i.owner.op == ds_op and
                                    i.owner.inputs[0].owner is red) else i
@@ -470,19 +496,10 @@ def _try_epilogue(fgraph, red, cand):
         if c is not None:
             s_args.append(c)
             continue
-        per_result = (isinstance(i.type, HipArrayType) and tuple(i.type.broadcastable) == tuple(layout) and
-                      not _depends_on(i, red))
-        if not (_is_host_scalar(i) or per_result):
+        expr = operand(i, 0)
+        if expr is None:
             return False
-        sv = None
-        for e, se in zip(extras, s_extras):
-            if e is i:
-                sv = se
-        if sv is None:
-            sv = scal.Scalar(i.type.dtype)()
-            extras.append(i)
-            s_extras.append(sv)
-        s_args.append(sv)
+        s_args.append(expr)
     if not used or len(extras) > 12:
         return False
     e_out = cand.op.scalar_op(*s_args)
@@ -652,6 +669,8 @@ def optimize(fgraph, fuse=True, rowchain=True, inplace=True):
         gof.merge_identical(fgraph)
         fuse_reduce_epilogue(fgraph)
         fuse_argmax_prologue(fgraph)
+        gof.merge_identical(fgraph)
+        fuse_elemwise(fgraph)          # producers that lost their other clients to an epilogue
         gof.merge_identical(fgraph)
     if inplace:
         inplace_elemwise(fgraph)

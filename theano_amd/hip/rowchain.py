@@ -284,7 +284,12 @@ def _grow(fgraph, seed, nd):
             if m in island or m not in fgraph.apply_nodes or not _eligible(m, nd):
                 continue
             if isinstance(m.op, HipDimShuffle) and m.inputs[0].owner not in island:
-                continue
+                # reached from a consumer: the keepdims view joins together with its reduction
+                prod = m.inputs[0].owner
+                if prod not in fgraph.apply_nodes or not _eligible(prod, nd):
+                    continue
+                island.add(prod)
+                frontier.append(prod)
             island.add(m)
             frontier.append(m)
     # a DimShuffle only belongs with its reduction; drop strays whose producer never joined
