@@ -183,15 +183,28 @@ def subtensor(x, idx):
     return Subtensor(idx_list)(x)
 
 
-def inc_subtensor(x, y, idx=None):
-    """``inc_subtensor(x[idx], y)`` written as ``inc_subtensor(x, y, idx)``."""
+def _inc_or_set(x, y, idx, set_instead_of_inc):
     x = as_tensor_variable(x)
-    return IncSubtensor(normalize_index(idx if idx is not None else (), x.type.ndim))(x, y)
+    if idx is None:
+        # the reference's calling convention: inc_subtensor(x[idx], y) - the first argument is the
+        # indexed view, the op is applied to what it indexes (theano/tensor/subtensor.py:1040-1110)
+        if x.owner is None or not isinstance(x.owner.op, Subtensor):
+            raise TypeError("x must be the result of a subtensor operation (or pass the index as third argument)")
+        idx_list, x = x.owner.op.idx_list, x.owner.inputs[0]
+    else:
+        idx_list = normalize_index(idx, x.type.ndim)
+    return IncSubtensor(idx_list, set_instead_of_inc)(x, y)
+
+
+def inc_subtensor(x, y, idx=None):
+    """``inc_subtensor(x[idx], y)`` as in the reference, or ``inc_subtensor(x, y, idx)``: a copy of
+    the indexed tensor with the region incremented by ``y``."""
+    return _inc_or_set(x, y, idx, False)
 
 
 def set_subtensor(x, y, idx=None):
-    x = as_tensor_variable(x)
-    return IncSubtensor(normalize_index(idx if idx is not None else (), x.type.ndim), True)(x, y)
+    """``set_subtensor(x[idx], y)`` or ``set_subtensor(x, y, idx)``."""
+    return _inc_or_set(x, y, idx, True)
 
 
 # --------------------------------------------------------------------------
