@@ -235,8 +235,13 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
           slot[o] = ntr++;
           esz = std::max(esz, dtype_size(views[o].dtype));
         }
-      int tile = 64;
+      // 128-byte row segments are enough for the memory system, and the smaller tile keeps four times
+      // as many blocks in flight around the barrier between the two phases: 53.0 us against 60.0 us for
+      // the int32 (64, 128, 56, 56) permuted read with 64 x 64 tiles
+      int tile = esz >= 4 ? 32 : 64;
       if ((int64_t)ntr * tile * (tile + 1) * esz > 60000) tile = 32;
+      const int force_tile = env_int("THX_EW_TILE", 0);
+      if (force_tile == 32 || force_tile == 64) tile = force_tile;
       // elements per access: 16 bytes of the widest operand, if extents, strides and addresses allow
       int allsz = 1;
       for (int o = 0; o < nops; ++o)
