@@ -28,11 +28,17 @@ import time
 HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each
-# scaled by what the same counter reads for the --copy-probe kernel of known size), by kernel symbol.
+# scaled by what the same counter reads for the --copy-probe kernel of known size), by kernel family
+# and functor (the rest of a kernel symbol spells tuning choices that do not change its traffic).
 MEASURED_TRAFFIC = {
-    # sum(axis=1) of float32 (8192, 8192): FETCH_SIZE 131091.1 x 1.99979 KiB + WRITE_SIZE 256.4 x 0.99875 KiB
-    "thx_rr_k1_i32_v4_u4_t256_a0_nt1_m0_fd_Ra004ded952553fcd": 268709251,
+    # sum(axis=1) of float32 (8192, 8192): FETCH_SIZE 131091.1 x 1.99979 KiB + WRITE_SIZE 256.3 x 0.99864 KiB
+    "rr:Ra004ded952553fcd": 268709587,
 }
+
+
+def _traffic(symbol):
+    parts = symbol.split("_")
+    return MEASURED_TRAFFIC.get("%s:%s" % (parts[1], parts[-1]))
 
 
 def _device_function(th, W, graph, vals):
@@ -202,7 +208,7 @@ def main():
     per_launch = 8192 * 8192 * 4 + 8192 * 4   # bytes one launch of a row / column reduction moves by definition
     achieved = per_launch / (dom_avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(dom),
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": _traffic(dom),
                 "kernel": dom, "avg_launch_us": round(dom_avg_us, 2), "uncached_input_us": cold_us,
                 "same_input_us": warm_us, "algorithmic_bytes_per_launch": per_launch}
 
