@@ -168,3 +168,34 @@ def test_more_than_2_to_31_elements_use_64_bit_indexing():
     assert np.array_equal(r1, val.reshape(2, n // 2).sum(axis=1, dtype=np.int64))
     assert np.array_equal(r0[:4096], val.reshape(2, n // 2)[:, :4096].sum(axis=0, dtype=np.int64))
     assert r0.sum() == s
+
+
+def test_sgd_steps_with_shared_weights_and_updates():
+    """Ten steps of logistic regression on device-resident weights (shared
+    variables updated by the function itself) against the same steps in NumPy."""
+    rng = np.random.default_rng(44)
+    n, d = 512, 96
+    xv = rng.standard_normal((n, d)).astype("float32")
+    tv = (rng.uniform(size=(n, 1)) < 0.5).astype("float32")
+    w0 = (0.1 * rng.standard_normal((1, d))).astype("float32")
+    w = th.shared(w0, name="w", broadcastable=(True, False))
+    b = th.shared(np.zeros((1, 1), "float32"), name="b", broadcastable=(True, True))
+    x, t = T.fmatrix("x"), T.fcol("t")
+    z = T.sum(x * w, axis=1, keepdims=True) + b
+    p = T.sigmoid(z)
+    loss = T.mean(-t * T.log(p) - (1 - t) * T.log(1 - p))
+    gw, gb = th.grad(loss, [w, b])
+    lr = np.float32(0.5)
+    step = th.function([x, t], loss, updates=[(w, w - lr * gw), (b, b - lr * gb)])
+    wn, bn = w0.astype("float64"), np.zeros((1, 1))
+    for _ in range(10):
+        got = float(step(xv, tv))
+        zn = (xv * wn).sum(axis=1, keepdims=True) + bn
+        pn = 1 / (1 + np.exp(-zn))
+        ref = float(np.mean(-tv * np.log(pn) - (1 - tv) * np.log(1 - pn)))
+        assert abs(got - ref) < 1e-4 * max(1.0, abs(ref))
+        dz = (pn - tv) / n
+        wn = wn - 0.5 * (dz * xv).sum(axis=0, keepdims=True)
+        bn = bn - 0.5 * dz.sum(keepdims=True)
+    assert np.allclose(w.get_value(), wn, rtol=1e-3, atol=1e-4)
+    assert np.allclose(b.get_value(), bn, rtol=1e-3, atol=1e-4)

@@ -282,3 +282,27 @@ def test_plans_for_arrays_beyond_32_bit_limits(dry_run):
     g = th.function([v], T.sum(v))
     g(huge)
     assert "|i64|" in hip.last_plan()
+
+
+def test_updates_replace_shared_values_after_the_call(dry_run):
+    """function(..., updates=[(w, new_w)]): type checks of theano/compile/pfunc.py
+    and the new value lands in the shared variable's container."""
+    w = th.shared(np.zeros((3, 4), "float32"), name="w")
+    x = T.fmatrix("x")
+    f = th.function([x], T.sum(x * w), updates=[(w, w + x)])
+    before = w.container[0]
+    f(np.ones((3, 4), "float32"))
+    assert w.container[0] is not before and w.container[0].shape == (3, 4)
+    g = th.function([x], None, updates={w: w * 2 - x})
+    assert g(np.ones((3, 4), "float32")) == []
+    with pytest.raises(TypeError):
+        th.function([x], [], updates=[(w, T.cast(w, "float64"))])      # dtype must not change
+    with pytest.raises(TypeError):
+        th.function([x], [], updates=[(x, x + 1)])                     # only shared variables are updated
+    with pytest.raises(ValueError):
+        th.function([x], [], updates=[(w, w + 1), (w, w + 2)])
+    # a view of the shared value is copied, never stored as an alias of the old buffer
+    h = th.function([], [], updates=[(w, w[::-1])])
+    old = w.container[0]
+    h()
+    assert w.container[0].buffer is not old.buffer

@@ -70,7 +70,8 @@ def shared(value, name=None, broadcastable=None):
 class Function(object):
     """Callable produced by ``function``."""
 
-    def __init__(self, fgraph, in_specs, out_specs, single_output, shared_inputs):
+    def __init__(self, fgraph, in_specs, out_specs, single_output, shared_inputs, update_targets=()):
+        self.update_targets = list(update_targets)
         self.fgraph = fgraph
         self.maker = self  # so that f.maker.fgraph reads as with the reference
         self.in_specs = in_specs
@@ -198,6 +199,16 @@ class Function(object):
             for cell in self.release[k]:
                 cell[0] = None
         results = [self.storage[o][0] for o in self.fgraph.outputs]
+        if self.update_targets:
+            n_out = len(results) - len(self.update_targets)
+            new_values = results[n_out:]
+            results = results[:n_out]
+            held = set(id(s.container[0].buffer) for s in self.shared_inputs)
+            held |= set(id(a.buffer) for a in args if isinstance(a, HipArray))
+            for sv, val in zip(self.update_targets, new_values):
+                if id(val.buffer) in held:   # a view of a shared variable or of an argument: take a private copy
+                    val = val.copy()
+                sv.container[0] = val
         for v in self.fgraph.inputs:
             self.storage[v][0] = None
         for o in self.fgraph.outputs:
@@ -211,13 +222,17 @@ class Function(object):
         return list(self.nodes)
 
 
-def function(inputs, outputs, fuse=True, rowchain=True, inplace=True, name=None, on_unused_input="raise"):
+def function(inputs, outputs, updates=None, fuse=True, rowchain=True, inplace=True, name=None,
+             on_unused_input="raise"):
     """Compile ``outputs`` as a function of ``inputs``.
 
     ``inputs``: variables or ``In`` instances.  A host-typed input may be given
     a ``HipArray`` at call time, which skips the upload.  ``outputs``: a
     variable, ``Out`` or a list of those; ``Out(v, device=True)`` leaves the
-    result on the GPU.  Every op must have a HIP implementation.  ``fuse=False``
+    result on the GPU.  ``updates``: pairs (or a dict) of shared variable and
+    the expression whose value replaces its content after each call, as in
+    ``theano.function`` (``theano/compile/pfunc.py:60-230``).  Every op must
+    have a HIP implementation.  ``fuse=False``
     keeps one kernel per graph node; ``rowchain=False`` keeps elementwise /
     row-reduction islands as separate fused kernels; ``inplace=False`` gives
     every elementwise result a buffer of its own."""
@@ -225,6 +240,8 @@ def function(inputs, outputs, fuse=True, rowchain=True, inplace=True, name=None,
     from .hip.ops import HipArrayType, as_hip_variable
 
     in_specs = [i if isinstance(i, In) else In(i) for i in inputs]
+    if outputs is None:
+        outputs = []
     single = not isinstance(outputs, (list, tuple))
     out_list = [outputs] if single else list(outputs)
     out_specs = [o if isinstance(o, Out) else Out(o) for o in out_list]
@@ -236,6 +253,26 @@ def function(inputs, outputs, fuse=True, rowchain=True, inplace=True, name=None,
         if spec.device and isinstance(v.type, TensorType):
             v = as_hip_variable(v)
         out_vars.append(v)
+    # updates: new values of shared variables, computed with the outputs and stored after the call
+    # (theano/compile/pfunc.py:60-230); each must have the type of the variable it replaces
+    update_targets = []
+    if updates:
+        pairs = list(updates.items()) if isinstance(updates, dict) else list(updates)
+        for sv, new in pairs:
+            if not isinstance(sv, SharedVariable):
+                raise TypeError("update target must be a shared variable", sv)
+            if sv in update_targets:
+                raise ValueError("this shared variable already has an update expression", sv)
+            if not isinstance(new, Variable):
+                new = as_tensor_variable(new)
+            if isinstance(new.type, TensorType):
+                new = as_hip_variable(new)
+            if new.type != sv.type:
+                raise TypeError("an update must have the same type as the original shared variable "
+                                "(shared_var=%s, shared_var.type=%s, update_val=%s, update_val.type=%s)"
+                                % (sv, sv.type, new, new.type))
+            update_targets.append(sv)
+            out_vars.append(new)
     in_vars = [s.variable for s in in_specs]
     shared_inputs = [v for v in gof.graph_inputs(out_vars) if isinstance(v, SharedVariable)]
     used = set(id(v) for v in gof.graph_inputs(out_vars))
@@ -252,7 +289,7 @@ def function(inputs, outputs, fuse=True, rowchain=True, inplace=True, name=None,
     c_out = [memo[v] for v in out_vars]
     fgraph = _SharedAwareGraph(c_in, c_out, shared_inputs)
     fgraph = hip_opt.optimize(fgraph, fuse=fuse, rowchain=rowchain, inplace=inplace)
-    return Function(fgraph, in_specs, out_specs, single, shared_inputs)
+    return Function(fgraph, in_specs, out_specs, single, shared_inputs, update_targets)
 
 
 class _SharedAwareGraph(FunctionGraph):

@@ -329,6 +329,17 @@ class HipArray(object):
             axes = tuple(reversed(range(self.ndim)))
         return self.view([self.shape[a] for a in axes], [self.strides[a] for a in axes])
 
+    def copy(self):
+        """A C-contiguous device copy."""
+        out = HipArray.empty(self.shape, self.dtype)
+        if self.size and not out.buffer.fake:
+            if self.c_contiguous:
+                check(lib.thx_d2d(out.ptr, self.ptr, self.nbytes))
+            else:
+                from .views import copy_into
+                copy_into(self, out)
+        return out
+
     # -- transfers
     def to_numpy(self):
         """Copy to host; strided views are copied as the byte span they cover
