@@ -90,7 +90,7 @@ def _cpu_baseline_c2(W):
 
 def _cpu_baseline_other(name, vals, nbytes):
     """One pass of the reference's host loops for another configuration
-    (oracle/cpu_backend.c) over the full-size inputs; the forward graphs only."""
+    (oracle/cpu_backend.c) over the full-size inputs."""
     from oracle import cpu_backend as B
     from oracle import graph_ref as G
     out = {}

@@ -250,3 +250,121 @@ void cpu_f2h_array(const float* f, uint16_t* h, int64_t n) {
 /* threads an OpenMP region of this library runs with (OMP_NUM_THREADS or the core count) */
 #include <omp.h>
 int cpu_omp_threads(void) { return omp_get_max_threads(); }
+
+/* ---- configuration 3, forward + gradient of sum(out * y) with respect to x -------------------------
+ * The forward chain of cpu_c3_chain, then the gradient graph as reverse mode builds it and
+ * elementwise fusion partitions it (islands end at every CAReduce):
+ *   t  = y * e / (s * s)                      Elemwise (OpenMP), materialised
+ *   gs = -sum(t, 1)                           Sum, float64 accumulator, serial
+ *   u  = (y / s + gs) * e                     Elemwise, materialised
+ *   gm = -sum(u, 1)                           Sum, serial
+ *   dx = u + eq(m, x) * gm                    Elemwise (gradient through max: positions equal to it)
+ * out, dx: (R, C); e, t, u: (R, C) scratch; rowmax, rowsum, gs, gm: (R,). */
+void cpu_c3_fwd_grad(const float* x, const float* y, float* out, float* dx, float* e, float* t, float* u,
+                     float* rowmax, float* rowsum, float* gs, float* gm, int64_t R, int64_t C) {
+  cpu_c3_chain(x, out, e, rowmax, rowsum, R, C);
+#pragma omp parallel for if (R * C >= OMP_MIN)
+  for (int64_t r = 0; r < R; ++r) {
+    const float s = rowsum[r];
+    for (int64_t c = 0; c < C; ++c) t[r * C + c] = y[r * C + c] * e[r * C + c] / (s * s);
+  }
+  for (int64_t r = 0; r < R; ++r) {
+    double acc = 0.0;
+    for (int64_t c = 0; c < C; ++c) acc = acc + (double)t[r * C + c];
+    gs[r] = -(float)acc;
+  }
+#pragma omp parallel for if (R * C >= OMP_MIN)
+  for (int64_t r = 0; r < R; ++r) {
+    const float s = rowsum[r], g = gs[r];
+    for (int64_t c = 0; c < C; ++c) u[r * C + c] = (y[r * C + c] / s + g) * e[r * C + c];
+  }
+  for (int64_t r = 0; r < R; ++r) {
+    double acc = 0.0;
+    for (int64_t c = 0; c < C; ++c) acc = acc + (double)u[r * C + c];
+    gm[r] = -(float)acc;
+  }
+#pragma omp parallel for if (R * C >= OMP_MIN)
+  for (int64_t r = 0; r < R; ++r) {
+    const float m = rowmax[r], g = gm[r];
+    for (int64_t c = 0; c < C; ++c) dx[r * C + c] = u[r * C + c] + (x[r * C + c] == m ? 1.0f : 0.0f) * g;
+  }
+}
+
+/* ---- configuration 5, gradients of sum(y * g) with respect to x, gamma, beta ----------------------
+ * Forward statistics as in cpu_c5_fwd (xf, mean, d = sqr(xf - mean), var), then with
+ * std = sqrt(var + eps), D = xf - mean, G = cast(g, float32):
+ *   dbeta  = sum(G)                            Sum per channel, float64 accumulator (float32 input), serial
+ *   sgd    = sum(G * D)                        Elemwise product materialised in d, then Sum
+ *   dgamma = sgd / std
+ *   dvar   = -gamma * sgd / (std * std) / (2 * std)                                  per channel
+ *   dd     = G * gamma / std + 2 * D * dvar / M                                      Elemwise, materialised
+ *   dmean  = -sum(dd)                          Sum
+ *   dx     = cast(dd + dmean / M, float16)     Elemwise
+ * xf, gf, d: (N*Ch*HW) float32 scratch; per-channel arrays of Ch floats. */
+static void sum64_over_n_hw(const float* v, float* s, int64_t N, int64_t Ch, int64_t HW) {
+  for (int64_t c = 0; c < Ch; ++c) {
+    double acc = 0.0;
+    for (int64_t n = 0; n < N; ++n) {
+      const float* q = v + (n * Ch + c) * HW;
+      for (int64_t p = 0; p < HW; ++p) acc = acc + (double)q[p];
+    }
+    s[c] = (float)acc;
+  }
+}
+
+void cpu_c5_grad(const uint16_t* x, const uint16_t* gamma, const uint16_t* g, uint16_t* dx, uint16_t* dgamma,
+                 uint16_t* dbeta, float* xf, float* gf, float* d, float* mean, float* var, float* tmp,
+                 int64_t N, int64_t Ch, int64_t HW) {
+  const int64_t n_all = N * Ch * HW;
+  const float M = (float)(N * HW);
+#pragma omp parallel for if (n_all >= OMP_MIN)
+  for (int64_t i = 0; i < n_all; ++i) xf[i] = h2f(x[i]);
+  sum_over_n_hw(xf, mean, N, Ch, HW);
+  for (int64_t c = 0; c < Ch; ++c) mean[c] = mean[c] / M;
+#pragma omp parallel for if (n_all >= OMP_MIN)
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t c = 0; c < Ch; ++c)
+      for (int64_t p = 0; p < HW; ++p) {
+        const int64_t i = (n * Ch + c) * HW + p;
+        const float t = xf[i] - mean[c];
+        d[i] = t * t;
+      }
+  sum_over_n_hw(d, var, N, Ch, HW);
+  for (int64_t c = 0; c < Ch; ++c) var[c] = sqrtf(var[c] / M + 1e-5f);   /* var now holds std */
+#pragma omp parallel for if (n_all >= OMP_MIN)
+  for (int64_t i = 0; i < n_all; ++i) gf[i] = h2f(g[i]);
+  sum64_over_n_hw(gf, tmp, N, Ch, HW);                                     /* tmp = dbeta */
+  for (int64_t c = 0; c < Ch; ++c) dbeta[c] = f2h(tmp[c]);
+#pragma omp parallel for if (n_all >= OMP_MIN)
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t c = 0; c < Ch; ++c)
+      for (int64_t p = 0; p < HW; ++p) {
+        const int64_t i = (n * Ch + c) * HW + p;
+        d[i] = gf[i] * (xf[i] - mean[c]);
+      }
+  sum64_over_n_hw(d, tmp, N, Ch, HW);                                      /* tmp = sum(G * D) */
+  for (int64_t c = 0; c < Ch; ++c) {
+    const float sd = var[c], gm = h2f(gamma[c]);
+    dgamma[c] = f2h(tmp[c] / sd);
+    tmp[c] = -gm * tmp[c] / (sd * sd) / (2.0f * sd);                       /* tmp = dvar */
+  }
+#pragma omp parallel for if (n_all >= OMP_MIN)
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t c = 0; c < Ch; ++c) {
+      const float sd = var[c], gm = h2f(gamma[c]), dv = tmp[c], m = mean[c];
+      for (int64_t p = 0; p < HW; ++p) {
+        const int64_t i = (n * Ch + c) * HW + p;
+        d[i] = gf[i] * gm / sd + 2.0f * (xf[i] - m) * dv / M;
+      }
+    }
+  sum64_over_n_hw(d, mean, N, Ch, HW);                                     /* mean now holds sum(dd) */
+#pragma omp parallel for if (n_all >= OMP_MIN)
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t c = 0; c < Ch; ++c) {
+      const float dm = -mean[c] / M;
+      for (int64_t p = 0; p < HW; ++p) {
+        const int64_t i = (n * Ch + c) * HW + p;
+        dx[i] = f2h(d[i] + dm);
+      }
+    }
+}

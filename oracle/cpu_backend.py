@@ -2,7 +2,7 @@
 ``cpu_baseline`` leg of ``bench.py`` may import this.
 
 ctypes front end of ``oracle/cpu_backend.c``: the host loops Theano's C backend
-runs for benchmark configurations 1, 3, 4 and 5 (OpenMP Elemwise nodes above
+runs for benchmark configurations 1, 3, 4 and 5, forward and gradient (OpenMP Elemwise nodes above
 200000 elements, serial CAReduce nodes, intermediates materialised between
 nodes; ``theano/tensor/elemwise.py:1100-1102``,
 ``theano/tensor/elemwise_cgen.py:406-409, 465-527``).  ``run(name, inputs)``
@@ -50,6 +50,27 @@ def run(name, inputs):
             t0 = time.perf_counter()
             L.cpu_c3_rowloop(_p(x), _p(out), _i64(R), _i64(C))
         return [out], time.perf_counter() - t0
+    if name == "c3_fwd_grad":
+        x, y = inputs
+        R, C = x.shape
+        out, dx = np.empty_like(x), np.empty_like(x)
+        e, t, u = np.empty_like(x), np.empty_like(x), np.empty_like(x)
+        rows = [np.empty(R, "float32") for _ in range(4)]
+        t0 = time.perf_counter()
+        L.cpu_c3_fwd_grad(_p(x), _p(y), _p(out), _p(dx), _p(e), _p(t), _p(u), _p(rows[0]), _p(rows[1]), _p(rows[2]),
+                          _p(rows[3]), _i64(R), _i64(C))
+        return [out, dx], time.perf_counter() - t0
+    if name == "c5_grad":
+        x, gamma, beta, g = inputs
+        N, Ch, H, Wd = x.shape
+        dx = np.empty_like(x)
+        dgamma, dbeta = np.empty_like(gamma), np.empty_like(beta)
+        xf, gf, d = [np.empty(x.shape, "float32") for _ in range(3)]
+        mean, var, tmp = [np.empty(Ch, "float32") for _ in range(3)]
+        t0 = time.perf_counter()
+        L.cpu_c5_grad(_p(x), _p(gamma), _p(g), _p(dx), _p(dgamma), _p(dbeta), _p(xf), _p(gf), _p(d), _p(mean), _p(var),
+                      _p(tmp), _i64(N), _i64(Ch), _i64(H * Wd))
+        return [dx, dgamma, dbeta], time.perf_counter() - t0
     if name in ("c4_elemwise", "c4_sum"):
         a, b, bias = inputs
         N, Ch, H, Wd = a.shape

@@ -199,7 +199,8 @@ def test_batchnorm_gradient_closed_form():
     assert np.allclose(ag, dscale, rtol=1e-9) and np.allclose(ax, dx, rtol=1e-8, atol=1e-10)
 
 
-@pytest.mark.parametrize("name", ["c1", "c3_fwd", "c3_fwd_rowloop", "c4_elemwise", "c4_sum", "c4_anyall", "c5_fwd"])
+@pytest.mark.parametrize("name", ["c1", "c3_fwd", "c3_fwd_rowloop", "c3_fwd_grad", "c4_elemwise", "c4_sum", "c4_anyall",
+                                  "c5_fwd", "c5_grad"])
 def test_cpu_backend_matches_graph_oracle(name):
     """The hand-restated host loops of the benchmark configurations (the CPU
     baseline) give what the node-by-node evaluation of the same graph gives:
@@ -214,6 +215,8 @@ def test_cpu_backend_matches_graph_oracle(name):
         "c4_sum": lambda: (W.c4_graph("sum"), W.c4_inputs("small")),
         "c4_anyall": lambda: (W.c4_graph("anyall"), W.c4_inputs("small", "anyall")),
         "c5_fwd": lambda: (W.c5_graph(with_grad=False), W.c5_inputs("small", False)),
+        "c3_fwd_grad": lambda: (W.c3_graph(), W.c3_inputs("small")),
+        "c5_grad": lambda: (W.c5_graph(forward=False), W.c5_inputs("small")),
     }[name]()
     ref = G.evaluate(graph[0], graph[1], vals)
     got, seconds = B.run(name, vals)
