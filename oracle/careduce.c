@@ -17,13 +17,14 @@
  * (PyArray_CopyInto, elemwise.py:1549-1554) is done by the caller.
  * Per-op expressions follow theano/scalar/basic.py: Add :1707-1716,
  * Mul :1752-1761, Maximum :1632-1639, Minimum :1669-1675, OR/XOR/AND
- * :1561-1600 (bool add/mul are || and &&).
+ * :1561-1600 (bool add/mul are || and &&); mul_without_zeros
+ * theano/tensor/elemwise.py:2072-2077 (identity 0).
  */
 #include <math.h>
 #include <stdint.h>
 #include <string.h>
 
-enum { OP_ADD = 0, OP_MUL = 1, OP_MAX = 2, OP_MIN = 3, OP_AND = 4, OP_OR = 5, OP_XOR = 6 };
+enum { OP_ADD = 0, OP_MUL = 1, OP_MAX = 2, OP_MIN = 3, OP_AND = 4, OP_OR = 5, OP_XOR = 6, OP_MULNZ = 7 };
 enum { T_BOOL = 0, T_I8, T_U8, T_I16, T_U16, T_I32, T_U32, T_I64, T_U64, T_F16, T_F32, T_F64 };
 
 #define MAXND 16
@@ -92,6 +93,12 @@ SUMPROD(i32, int32_t, f64, double)
 SUMPROD(i64, int64_t, f64, double)
 SUMPROD(i8, int8_t, f32, float)
 
+/* theano/tensor/elemwise.py:2075-2077 with x = accumulator, y = element */
+#define MULNZSTMT acc = ((acc == 0) ? (x) : (((x) == 0) ? (acc) : ((x) * (acc))))
+DEFINE_REDUCE(mulnz_f32_f64, float, double, MULNZSTMT)
+DEFINE_REDUCE(mulnz_f32_f32, float, float, MULNZSTMT)
+DEFINE_REDUCE(mulnz_f64_f64, double, double, MULNZSTMT)
+
 #define MAXMIN_F(N, T)                           \
   DEFINE_REDUCE(max_##N##_##N, T, T, MAXSTMT)    \
   DEFINE_REDUCE(min_##N##_##N, T, T, MINSTMT)
@@ -146,6 +153,8 @@ static const entry_t table[] = {
     EMM(T_U16, u16),  EMM(T_I32, i32),  EMM(T_U32, u32),   EMM(T_I64, i64), EMM(T_U64, u64),
     EBIT(T_BOOL, bool), EBIT(T_I8, i8), EBIT(T_U8, u8), EBIT(T_I16, i16), EBIT(T_U16, u16), EBIT(T_I32, i32),
     EBIT(T_U32, u32),   EBIT(T_I64, i64), EBIT(T_U64, u64),
+    E(OP_MULNZ, T_F32, T_F64, mulnz_f32_f64), E(OP_MULNZ, T_F32, T_F32, mulnz_f32_f32),
+    E(OP_MULNZ, T_F64, T_F64, mulnz_f64_f64),
 };
 
 static int tsize(int t) {

@@ -34,7 +34,7 @@ _lib = None
 
 _DT_CODE = {"bool": 0, "int8": 1, "uint8": 2, "int16": 3, "uint16": 4, "int32": 5, "uint32": 6, "int64": 7,
             "uint64": 8, "float16": 9, "float32": 10, "float64": 11}
-_OP_CODE = {"Add": 0, "Mul": 1, "Maximum": 2, "Minimum": 3, "AND": 4, "OR": 5, "XOR": 6}
+_OP_CODE = {"Add": 0, "Mul": 1, "Maximum": 2, "Minimum": 3, "AND": 4, "OR": 5, "XOR": 6, "MulWithoutZeros": 7}
 
 # theano/tensor/elemwise.py:1733-1741 and :1748-1759
 SUM_OUT_DTYPE = dict(bool="int64", int8="int64", int16="int64", int32="int64", uint8="uint64", uint16="uint64",
@@ -58,7 +58,7 @@ def reduce_identity(op_name, dtype):
     """theano/tensor/elemwise.py:1470-1488 and the ops' own identities
     (theano/scalar/basic.py:1554, 1570, 1586, 1700, 1742)."""
     dt = np.dtype(dtype)
-    if op_name == "Add" or op_name in ("OR", "XOR"):
+    if op_name == "Add" or op_name in ("OR", "XOR", "MulWithoutZeros"):   # elemwise.py:2061
         return np.zeros((), dt)
     if op_name == "Mul":
         return np.ones((), dt)

@@ -16,6 +16,29 @@ VECTORS = [
     {"name": "prod_axis1_no_zeros", "cite": "theano/tensor/tests/test_elemwise.py:674-680",
      "graph": "prod_axis1", "dtype": "float32",
      "input": [[1, 2, 3], [4, 5, 6], [7, 8, 9]], "expected": [6, 120, 504]},
+    {"name": "prod_without_zeros_axis1", "cite": "theano/tensor/tests/test_elemwise.py:704-709",
+     "graph": "prod_without_zeros_axis1", "dtype": "float64",
+     "input": [[1, 2, 3], [0, 5, 6], [0, 0, 9]], "expected": [6, 30, 9]},
+    {"name": "prod_without_zeros_axis0", "cite": "theano/tensor/tests/test_elemwise.py:704-713",
+     "graph": "prod_without_zeros_axis0", "dtype": "float64",
+     "input": [[1, 2, 3], [0, 5, 6], [0, 0, 9]], "expected": [1, 10, 162]},
+    {"name": "prod_grad_axis1_zeros_a", "cite": "theano/tensor/tests/test_elemwise.py:723-736",
+     "graph": "prod_grad_axis1", "dtype": "float64",
+     "input": [[1, 2, 3], [0, 5, 6], [0, 0, 9]], "expected": [[6.0, 3.0, 2.0], [30.0, 0.0, 0.0], [0.0, 0.0, 0.0]]},
+    {"name": "prod_grad_axis1_zeros_b", "cite": "theano/tensor/tests/test_elemwise.py:723-740",
+     "graph": "prod_grad_axis1", "dtype": "float64",
+     "input": [[1, 2, 0], [0, 5, 6], [7, 8, 9], [9, 10, 0]],
+     "expected": [[0.0, 0.0, 2.0], [30.0, 0.0, 0.0], [72.0, 63.0, 56.0], [0.0, 0.0, 90.0]]},
+    {"name": "prod_grad_axis0_zeros", "cite": "theano/tensor/tests/test_elemwise.py:742-748",
+     "graph": "prod_grad_axis0", "dtype": "float64",
+     "input": [[1, 2, 0], [0, 5, 6], [7, 8, 9], [9, 10, 0]],
+     "expected": [[0.0, 400.0, 0.0], [63.0, 160.0, 0.0], [0.0, 100.0, 0.0], [0.0, 80.0, 0.0]]},
+    {"name": "prod_all_no_zeros_grad", "cite": "theano/tensor/tests/test_elemwise.py:682-689",
+     "graph": "prod_all_no_zeros_grad", "dtype": "float64", "input": [[1, 2, 3], [4, 5, 6], [7, 8, 9]],
+     "expected": [[362880.0, 181440.0, 120960.0], [90720.0, 72576.0, 60480.0], [51840.0, 45360.0, 40320.0]]},
+    {"name": "prod_all_no_zeros_second_grad", "cite": "theano/tensor/tests/test_elemwise.py:682-694",
+     "graph": "prod_all_no_zeros_second_grad", "dtype": "float64", "input": [[1, 2, 3], [4, 5, 6], [7, 8, 9]],
+     "expected": [[663696.0, 422568.0, 301872.0], [233964.0, 190800.0, 161016.0], [139248.0, 122652.0, 109584.0]]},
     {"name": "sum_needs_float64_accumulator", "cite": "theano/tensor/tests/test_elemwise.py:953-966",
      "graph": "sum_all", "dtype": "float32", "input": [1e8, 1, -1e8], "expected": 1.0},
     {"name": "max_and_argmax_vector", "cite": "theano/tensor/tests/test_basic.py:3114-3119",

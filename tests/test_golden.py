@@ -23,6 +23,17 @@ def build(entry):
     if g == "prod_axis1":
         x = T.TensorType(dt, (False, False))("x")
         return [x], [T.prod(x, axis=1)], [data.astype(dt)]
+    if g in ("prod_without_zeros_axis1", "prod_without_zeros_axis0"):
+        from theano_amd.tensor.elemwise import ProdWithoutZeros
+        x = T.TensorType(dt, (False, False))("x")
+        return [x], [ProdWithoutZeros(axis=int(g[-1]))(x)], [data.astype(dt)]
+    if g in ("prod_grad_axis1", "prod_grad_axis0"):
+        x = T.TensorType(dt, (False, False))("x")
+        return [x], [th.grad(T.sum(T.prod(x, axis=int(g[-1]))), x)], [data.astype(dt)]
+    if g in ("prod_all_no_zeros_grad", "prod_all_no_zeros_second_grad"):
+        x = T.TensorType(dt, (False, False))("x")
+        gx = th.grad(T.prod(x, no_zeros_in_input=True), x)
+        return [x], [gx if g.endswith("zeros_grad") else th.grad(T.sum(gx), x)], [data.astype(dt)]
     if g == "sum_all":
         x = T.TensorType(dt, (False,))("x")
         return [x], [T.sum(x)], [data.astype(dt)]

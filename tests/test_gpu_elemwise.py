@@ -180,3 +180,33 @@ def test_inplace_elementwise_matches_out_of_place():
     assert np.array_equal(a, b)
     assert_parity(a, G.evaluate([x, y], [out], [xv, yv])[0], "unfused in-place chain")
     assert np.array_equal(f_in(xv, yv), a)            # the inputs were not overwritten by the first call
+
+
+@pytest.mark.gpu
+def test_column_major_inputs_give_column_major_outputs():
+    """All inputs that are not broadcast along every dimension column-major (and not also
+    row-major): the output is allocated column-major too (theano/tensor/elemwise.py:928-937),
+    so the kernel streams; one row-major input, here also a (1, n) row, switches it back."""
+    from theano_amd.hip import HipArray
+    rng = np.random.default_rng(21)
+    a = np.asfortranarray(rng.standard_normal((130, 70)).astype("float32"))
+    b = np.asfortranarray(rng.standard_normal((130, 70)).astype("float32"))
+    row = rng.standard_normal((1, 70)).astype("float32")
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    r = T.TensorType("float32", (True, False))("r")
+    s = T.TensorType("float32", (True, True))("s")
+    f = th.function([x, y, s], [th.Out(T.exp(x) * y + s, device=True)])
+    one = np.full((1, 1), 0.5, "float32")
+    out = f(HipArray.from_numpy(a), HipArray.from_numpy(b), one)[0]
+    assert out.is_fortran and out.strides == (4, 130 * 4)
+    assert np.allclose(out.to_numpy(), np.exp(a) * b + one, rtol=1e-5, atol=1e-6)
+    out = f(HipArray.from_numpy(a), HipArray.from_numpy(np.ascontiguousarray(b)), one)[0]
+    assert out.c_contiguous
+    assert np.allclose(out.to_numpy(), np.exp(a) * b + one, rtol=1e-5, atol=1e-6)
+    g = th.function([x, y, r], [th.Out(T.exp(x) * y + r, device=True)])
+    out = g(HipArray.from_numpy(a), HipArray.from_numpy(b), row)[0]
+    assert out.c_contiguous
+    assert np.allclose(out.to_numpy(), np.exp(a) * b + row, rtol=1e-5, atol=1e-6)
+    # through the host boundary
+    got = th.function([x, y, s], [T.exp(x) * y + s])(a, b, one)[0]
+    assert np.allclose(got, np.exp(a) * b + one, rtol=1e-5, atol=1e-6)

@@ -173,3 +173,28 @@ def test_epilogue_chain_with_per_result_device_operands():
     bad[2] = np.ones((1, 36, 1, 1), "float32")
     with pytest.raises(ValueError):
         f(*bad)
+
+
+@pytest.mark.gpu
+def test_prod_gradient_with_zeros_and_prod_without_zeros():
+    """Zero-aware gradient of Prod on random data with planted zeros (groups with none,
+    one and several), against the oracle and against the closed form: the product of
+    the other elements of the group."""
+    from theano_amd.tensor.elemwise import ProdWithoutZeros
+    rng = np.random.default_rng(33)
+    xv = rng.uniform(0.5, 1.5, (37, 29))
+    xv[3, 4] = 0.0
+    xv[5, 1] = xv[5, 20] = 0.0
+    xv[30, :] = 0.0
+    x = T.dmatrix("x")
+    for axis in (0, 1):
+        ins, outs = [x], [th.grad(T.sum(T.prod(x, axis=axis)), x), ProdWithoutZeros(axis=axis)(x)]
+        got = th.function(ins, outs)(xv)
+        ref = G.evaluate(ins, outs, [xv])
+        for g, r in zip(got, ref):
+            assert np.allclose(g, r, rtol=1e-12, atol=0)
+        want = np.empty_like(xv)
+        for idx in np.ndindex(*xv.shape):
+            group = xv[:, idx[1]] if axis == 0 else xv[idx[0], :]
+            want[idx] = np.prod(np.delete(group, idx[axis]))
+        assert np.allclose(got[0], want, rtol=1e-10)

@@ -306,3 +306,35 @@ def test_updates_replace_shared_values_after_the_call(dry_run):
     old = w.container[0]
     h()
     assert w.container[0].buffer is not old.buffer
+
+
+def test_rop_matches_finite_differences_and_lop_matches_grad():
+    """Jacobian-times-vector of an Elemwise / DimShuffle / Sum / Subtensor graph
+    against central differences along the direction, and vector-times-Jacobian
+    against grad of the weighted sum (theano/tests/test_rop.py:62-150 checks
+    Rop the same way, against a scan-built Jacobian)."""
+    from oracle import graph_ref as G
+    rng = np.random.default_rng(5)
+    x, v = T.dmatrix("x"), T.dmatrix("v")
+    b = T.dvector("b")
+    y = T.sum(T.tanh(x * b.dimshuffle("x", 0)) * x[:, ::-1], axis=0) + T.exp(b)
+    jv = th.Rop(y, x, v)
+    xv, vv, bv = rng.standard_normal((4, 3)), rng.standard_normal((4, 3)), rng.standard_normal(3)
+    got = G.evaluate([x, v, b], [jv], [xv, vv, bv])[0]
+    eps = 1e-6
+    f = lambda xx: G.evaluate([x, b], [y], [xx, bv])[0]
+    want = (f(xv + eps * vv) - f(xv - eps * vv)) / (2 * eps)
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-8)
+
+    w = T.dvector("w")
+    vj = th.Lop(y, x, w)
+    ref = th.grad(T.sum(y * w), x)
+    wv = rng.standard_normal(3)
+    a, c = G.evaluate([x, b, w], [vj, ref], [xv, bv, wv])
+    assert np.allclose(a, c, rtol=1e-12)
+
+    # two variables at once: J_x v + J_b u
+    u = T.dvector("u")
+    both = G.evaluate([x, v, b, u], [th.Rop(y, [x, b], [v, u])], [xv, vv, bv, wv])[0]
+    fb = lambda t: G.evaluate([x, b], [y], [xv + t * vv, bv + t * wv])[0]
+    assert np.allclose(both, (fb(eps) - fb(-eps)) / (2 * eps), rtol=1e-6, atol=1e-8)

@@ -94,6 +94,74 @@ def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
     return result[0] if single else result
 
 
+def Lop(f, wrt, eval_points):
+    """L operator: eval_points times the Jacobian of ``f`` with respect to
+    ``wrt`` (``theano/gradient.py:348-411``): reverse mode seeded with
+    ``eval_points`` as the gradients of ``f``."""
+    fs = list(f) if isinstance(f, (list, tuple)) else [f]
+    eps = list(eval_points) if isinstance(eval_points, (list, tuple)) else [eval_points]
+    if len(fs) != len(eps):
+        raise ValueError("Lop needs one evaluation point per element of f")
+    return grad(None, wrt, known_grads=dict(zip(fs, eps)))
+
+
+def Rop(f, wrt, eval_points, disconnected_outputs="raise"):
+    """R operator: the Jacobian of ``f`` with respect to ``wrt`` times
+    ``eval_points`` (``theano/gradient.py:155-345``).  Forward mode: every node
+    between ``wrt`` and ``f`` is asked for ``R_op(inputs, eval_points)``;
+    graph inputs outside ``wrt`` contribute zeros."""
+    from .tensor import basic as T
+    from .tensor.type import as_tensor_variable
+
+    single = not isinstance(f, (list, tuple))
+    fs = [f] if single else list(f)
+    wrt = list(wrt) if isinstance(wrt, (list, tuple)) else [wrt]
+    eval_points = list(eval_points) if isinstance(eval_points, (list, tuple)) else [eval_points]
+    if len(wrt) != len(eval_points):
+        raise ValueError("Rop needs one evaluation point per element of wrt")
+    eval_points = [as_tensor_variable(e) for e in eval_points]
+    for k, (w, e) in enumerate(zip(wrt, eval_points)):
+        if w.type.ndim != e.type.ndim:
+            raise ValueError("Element %d of wrt/eval_point have mismatched dimensionality: %d versus %d"
+                             % (k, w.type.ndim, e.type.ndim))
+    point_of = dict((id(w), e) for w, e in zip(wrt, eval_points))
+    seen = {}
+
+    for node in gof.io_toposort([], fs):
+        if any(id(o) in point_of for o in node.outputs) and all(id(o) in point_of for o in node.outputs):
+            continue
+        local = []
+        for inp in node.inputs:
+            if id(inp) in point_of:
+                pt = point_of[id(inp)]
+            elif inp.owner is None:
+                pt = T.zeros_like(inp) if hasattr(inp.type, "broadcastable") else None
+            else:
+                pt = seen[id(inp.owner)][inp.owner.outputs.index(inp)]
+            if pt is not None and hasattr(inp.type, "dtype") and pt.type.dtype != inp.type.dtype:
+                pt = T.cast(pt, inp.type.dtype)
+            local.append(pt)
+        try:
+            seen[id(node)] = node.op.R_op(node.inputs, local)
+        except gof.MethodNotDefined:
+            raise NotImplementedError("%s does not define R_op" % node.op)
+
+    result = []
+    for out in fs:
+        if id(out) in point_of:
+            result.append(point_of[id(out)])
+            continue
+        r = seen[id(out.owner)][out.owner.outputs.index(out)] if out.owner is not None else None
+        if r is None:
+            if disconnected_outputs == "raise":
+                raise DisconnectedInputError("Rop method was asked to compute the gradient with respect to a variable "
+                                             "that is not part of the computational graph of variables in wrt, or is "
+                                             "used only by a non-differentiable operator: %s" % out)
+            r = T.zeros_like(out)
+        result.append(r)
+    return result[0] if single else result
+
+
 def _match_broadcast(g, var):
     """Make the gradient's static broadcast pattern equal to the variable's."""
     from .tensor import basic as T

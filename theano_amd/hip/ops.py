@@ -282,10 +282,14 @@ class HipElemwise(Elemwise):
         cache = node.tag.get("thx")
         if cache is None:
             handle, nin, nout = self._handle(node)
+            # inputs whose layout decides the outputs' (theano/tensor/elemwise.py:928-937): all but
+            # the ones broadcast along every dimension
+            full = [k for k, v in enumerate(node.inputs) if not all(v.type.broadcastable)]
             cache = node.tag["thx"] = (handle, nin, nout, (thx_array * nin)(), (thx_array * nout)(),
                                        node.outputs[0].type.ndim, dict(self.inplace_pattern),
-                                       [np.dtype(o.type.dtype) for o in node.outputs])
-        handle, nin, nout, ins, outs, nd, inplace, out_dt = cache
+                                       [np.dtype(o.type.dtype) for o in node.outputs],
+                                       full if node.outputs[0].type.ndim > 1 else [])
+        handle, nin, nout, ins, outs, nd, inplace, out_dt, full = cache
         shape = _check_runtime_broadcast(node.inputs, inputs, nd)
         k = 0
         for v in inputs:
@@ -294,12 +298,22 @@ class HipElemwise(Elemwise):
             else:
                 host_scalar_thx(v, nd, ins[k])
             k += 1
+        # column-major outputs when every such input is column-major, as the reference allocates them
+        fortran = False
+        for k in full:
+            v = inputs[k]
+            if type(v) is not HipArray or not v.is_fortran:
+                break
+        else:
+            fortran = bool(full)
         results = []
         for k in range(nout):
             if k in inplace:
                 arr = inputs[inplace[k]]
                 if arr.shape != shape:
                     raise ValueError("in-place output %d has shape %s, the result has %s" % (k, arr.shape, shape))
+            elif fortran:
+                arr = HipArray._new_fortran(shape, out_dt[k])
             else:
                 arr = HipArray._new_contiguous(shape, out_dt[k])
             arr.as_thx(outs[k])

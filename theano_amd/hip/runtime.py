@@ -263,6 +263,14 @@ class HipArray(object):
         self.code = _CODE_OF[dtype]
         return self
 
+    @classmethod
+    def _new_fortran(cls, shape, dtype):
+        """Column-major counterpart of ``_new_contiguous``."""
+        self = cls._new_contiguous(tuple(reversed(shape)), dtype)
+        self.shape = shape
+        self.strides = tuple(reversed(self.strides))
+        return self
+
     # -- construction
     @classmethod
     def empty(cls, shape, dtype):
@@ -282,6 +290,8 @@ class HipArray(object):
             raise TypeError("dtype %s is not supported on the device" % a.dtype)
         if _dry:                       # shapes only: nothing is copied, so nothing needs to exist
             return cls.empty(a.shape, a.dtype)
+        if a.ndim > 1 and a.flags.f_contiguous and not a.flags.c_contiguous:
+            return cls.from_numpy(a.T).transpose()      # column-major arrays keep their layout
         a = np.asarray(a, order="C")
         out = cls.empty(a.shape, a.dtype)
         if a.nbytes and not out.buffer.fake:
@@ -316,6 +326,20 @@ class HipArray(object):
                 return False
             expect *= max(s, 1)
         return True
+
+    @property
+    def is_fortran(self):
+        """Column-major contiguous and not row-major contiguous (NumPy's
+        ``PyArray_ISFORTRAN``)."""
+        shape, strides = self.shape, self.strides
+        if len(shape) < 2 or (strides[-1] == self.dtype.itemsize and shape[-1] > 1):
+            return False
+        expect = self.dtype.itemsize
+        for s, st in zip(shape, strides):
+            if s > 1 and st != expect:
+                return False
+            expect *= max(s, 1)
+        return not self.c_contiguous
 
     def __repr__(self):
         return "HipArray(shape=%s, dtype=%s, strides=%s)" % (self.shape, self.dtype, self.strides)

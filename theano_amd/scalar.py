@@ -637,6 +637,24 @@ class Sub(BinaryScalarOp):
 add, mul, sub = Add(upcast_out, name="add"), Mul(upcast_out, name="mul"), Sub(upcast_out_nobool, name="sub")
 
 
+class MulWithoutZeros(BinaryScalarOp):
+    """Product that skips zeros: the combiner of ProdWithoutZeros, which the
+    gradient of Prod uses for groups holding exactly one zero
+    (``theano/tensor/elemwise.py:2054-2083``).  Its identity is 0, not 1, so
+    that a group of zeros reduces to 0."""
+
+    identity = 0
+    commutative = True
+    associative = True
+
+    def c_code(self, node, inputs, outputs):
+        x, y = inputs
+        return "%s = ((%s == 0) ? (%s) : ((%s == 0) ? (%s) : ((%s) * (%s))));" % (outputs[0], x, y, y, x, y, x)
+
+
+mul_without_zeros = MulWithoutZeros(upcast_out, name="mul_without_zeros")
+
+
 def int_or_true_div(x_discrete, y_discrete):
     """Which division ``x / y`` means (``theano/scalar/basic.py:1826-1873``)."""
     if x_discrete and y_discrete:

@@ -94,6 +94,11 @@ class DimShuffle(Op):
             rval.insert(augm, 1)
         return [rval]
 
+    def R_op(self, inputs, eval_points):
+        if None in eval_points:
+            return [None]
+        return [self(*eval_points)]
+
     def grad(self, inp, grads):
         (x,) = inp
         (gz,) = grads
@@ -180,6 +185,26 @@ class Elemwise(Op):
             except TypeError:
                 pass
         return [[True] * len(node.outputs) for _ in node.inputs]
+
+    def R_op(self, inputs, eval_points):
+        """Sum over the inputs of d out / d input times that input's evaluation
+        point (``theano/tensor/elemwise.py:499-531``); inputs without a
+        gradient count as zero."""
+        from . import basic
+        outs = self.make_node(*inputs).outputs
+        rval = []
+        for idx, out in enumerate(outs):
+            ograds = [basic.zeros_like(o) for o in outs]
+            ograds[idx] = basic.ones_like(out)
+            bgrads = self._bgrad(inputs, outs, ograds)
+            acc = None
+            for g, pt in zip(bgrads, eval_points):
+                if g is None or isinstance(g.type, DisconnectedType) or pt is None:
+                    continue
+                term = basic.mul(g, pt)
+                acc = term if acc is None else basic.add(acc, term)
+            rval.append(acc)
+        return rval
 
     def L_op(self, inputs, outs, ograds):
         rval = self._bgrad(inputs, outs, ograds)
@@ -442,27 +467,32 @@ class Sum(CAReduceDtype):
         gx = Elemwise(scal.second)(x, DimShuffle(gz.type.broadcastable, new_dims)(gz))
         return [gx]
 
+    def R_op(self, inputs, eval_points):
+        if None in eval_points:
+            return [None]
+        return [self(*eval_points)]
+
 
 class Prod(CAReduceDtype):
-    """Product along axes.  The gradient implemented here is the one the
-    reference uses when ``no_zeros_in_input`` is set
-    (``theano/tensor/elemwise.py:1928-2048``): prod / x * gz."""
+    """Product along axes (``theano/tensor/elemwise.py:1905-2051``).  The
+    gradient divides the product by each element where a group holds no zero,
+    takes the product of the other elements (ProdWithoutZeros) where it holds
+    exactly one, and is zero where it holds more; ``no_zeros_in_input`` keeps
+    only the first case."""
 
-    __props__ = ("axis", "dtype", "acc_dtype", "no_zeros_in_input")
+    __props__ = ("axis", "dtype", "acc_dtype")
 
     def __init__(self, axis=None, dtype=None, acc_dtype=None, no_zeros_in_input=False):
         CAReduceDtype.__init__(self, scal.mul, axis=axis, dtype=dtype, acc_dtype=acc_dtype)
         self.no_zeros_in_input = no_zeros_in_input
 
     def _props(self):
-        return (self.axis, self.dtype, self.acc_dtype, self.no_zeros_in_input)
+        return (self.axis, self.dtype, self.acc_dtype)
 
     def L_op(self, inp, out, grads):
         (x,) = inp
-        if out[0].type.dtype in scal.discrete_dtypes or x.type.dtype in scal.discrete_dtypes:
+        if out[0].type.dtype in scal.discrete_dtypes or self.acc_dtype in scal.discrete_dtypes:
             return [x.zeros_like(dtype=config.floatX)]
-        if not self.no_zeros_in_input:
-            raise NotImplementedError("Prod gradient is only implemented for no_zeros_in_input=True")
         gz = as_tensor_variable(grads[0])
         axis = self.axis
         if axis is None:
@@ -476,8 +506,39 @@ class Prod(CAReduceDtype):
             else:
                 new_dims.append(i)
                 i += 1
-        ds = DimShuffle(gz.type.broadcastable, new_dims)
-        prod_out = ds(out[0])
-        gz = ds(gz)
-        from . import basic
-        return [basic.true_div(basic.mul(prod_out, gz), x)]
+
+        def over_groups(v):
+            return DimShuffle(v.type.broadcastable, new_dims)(v)
+
+        from . import basic as T
+        prod_out = over_groups(out[0])
+        gz = over_groups(gz)
+        without_zeros = T.true_div(T.mul(gz, prod_out), x)
+        if self.no_zeros_in_input:
+            return [without_zeros]
+        where_zeros = T.eq(x, 0.0)
+        n_zeros = T.sum(where_zeros, axis=self.axis)
+        single_zero = over_groups(T.eq(n_zeros, 1))
+        where_single_zero = T.mul(single_zero, where_zeros)
+        # only groups with one zero and a non-zero incoming gradient keep their values
+        taken = T.mul(T.mul(single_zero, T.neq(gz, 0.0)), x)
+        others = over_groups(ProdWithoutZeros(axis=self.axis)(taken))
+        no_zero = over_groups(T.eq(n_zeros, 0))
+        return [T.switch(no_zero, without_zeros, T.mul(T.switch(where_single_zero, others, 0.0), gz))]
+
+
+class ProdWithoutZeros(CAReduceDtype):
+    """Product of the non-zero elements along axes; 0 for a group of zeros
+    (``theano/tensor/elemwise.py:2086-2101``)."""
+
+    __props__ = ("axis", "dtype", "acc_dtype")
+
+    def __init__(self, axis=None, dtype=None, acc_dtype=None):
+        CAReduceDtype.__init__(self, scal.mul_without_zeros, axis=axis, dtype=dtype, acc_dtype=acc_dtype)
+
+    def _props(self):
+        return (self.axis, self.dtype, self.acc_dtype)
+
+    def grad(self, inp, grads):
+        raise NotImplementedError("second derivatives of prod(a) are not supported; if a holds no zeros use "
+                                  "prod(a, no_zeros_in_input=True)")

@@ -122,6 +122,11 @@ class Subtensor(Op):
         (g,) = grads
         return [IncSubtensor(self.idx_list)(x.zeros_like(), g)]
 
+    def R_op(self, inputs, eval_points):
+        if eval_points[0] is None:
+            return [None]
+        return [self(eval_points[0])]
+
 
 class IncSubtensor(Op):
     """``x`` with ``x[idx_list]`` incremented by (or set to) ``y``
@@ -156,6 +161,11 @@ class IncSubtensor(Op):
 
     def perform(self, node, inputs, output_storage):
         _no_host(self)
+
+    def R_op(self, inputs, eval_points):
+        if None in eval_points[:2]:
+            return [None]
+        return [self(eval_points[0], eval_points[1])]
 
     def L_op(self, inputs, outputs, grads):
         x, y = inputs
@@ -288,6 +298,11 @@ class Reshape(Op):
             gx = T.DimShuffle(gx.type.broadcastable, list(range(x.type.ndim)))(gx)
         return [gx] + [v.zeros_like() for v in inputs[1:]]
 
+    def R_op(self, inputs, eval_points):
+        if eval_points[0] is None:
+            return [None]
+        return [self(eval_points[0], *inputs[1:])]
+
     def connection_pattern(self, node):
         return [[True]] + [[False]] * (len(node.inputs) - 1)
 
@@ -384,6 +399,11 @@ class Alloc(Op):
             gv = T.cast(gv, v.type.dtype)
         return [gv] + [i.zeros_like() for i in inputs[1:]]
 
+    def R_op(self, inputs, eval_points):
+        if eval_points[0] is None:
+            return [None]
+        return [self(eval_points[0], *inputs[1:])]
+
     def connection_pattern(self, node):
         return [[True]] + [[False]] * (len(node.inputs) - 1)
 
@@ -448,6 +468,11 @@ class Join(Op):
         if outputs[0].type.dtype not in T.continuous_dtypes:
             return [i.zeros_like(dtype=T.config.floatX) for i in inputs]
         return [JoinPart(self.axis, k)(g, *inputs) for k in range(len(inputs))]
+
+    def R_op(self, inputs, eval_points):
+        if None in eval_points:
+            return [None]
+        return [self(*eval_points)]
 
 
 class JoinPart(Op):
