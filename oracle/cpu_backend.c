@@ -368,3 +368,51 @@ void cpu_c5_grad(const uint16_t* x, const uint16_t* gamma, const uint16_t* g, ui
       }
     }
 }
+
+/* ---- configuration 2 with OpenMP over the outputs: NOT the reference's behaviour ------------------
+ * The reference's CAReduce loops carry no OpenMP pragma (theano/tensor/elemwise_cgen.py:465-527).
+ * These variants only show what the same host could do with all its cores: rows (axis 1) or
+ * blocks of columns (axis 0) are spread over threads, each output still accumulated in order
+ * in float64; the sum over all axes adds per-row partial sums, so its rounding may differ from
+ * the serial loop's in the last place.  which: 0 sum axis 1, 1 max axis 1, 2 sum axis 0,
+ * 3 sum of everything (out[0]), 4 prod axis 1. */
+void cpu_c2_parallel(const float* x, float* out, int64_t R, int64_t C, int which) {
+  if (which == 0 || which == 1 || which == 4) {
+#pragma omp parallel for
+    for (int64_t r = 0; r < R; ++r) {
+      const float* q = x + r * C;
+      if (which == 1) {
+        float acc = -INFINITY;
+        for (int64_t c = 0; c < C; ++c) acc = q[c] > acc ? q[c] : (acc >= q[c] ? acc : NAN);
+        out[r] = acc;
+      } else {
+        double acc = which == 0 ? 0.0 : 1.0;
+        if (which == 0)
+          for (int64_t c = 0; c < C; ++c) acc = acc + (double)q[c];
+        else
+          for (int64_t c = 0; c < C; ++c) acc = acc * (double)q[c];
+        out[r] = (float)acc;
+      }
+    }
+  } else if (which == 2) {
+    enum { CB = 256 };
+#pragma omp parallel for
+    for (int64_t c0 = 0; c0 < C; c0 += CB) {
+      double acc[CB];
+      const int64_t n = C - c0 < CB ? C - c0 : CB;
+      for (int64_t c = 0; c < n; ++c) acc[c] = 0.0;
+      for (int64_t r = 0; r < R; ++r)
+        for (int64_t c = 0; c < n; ++c) acc[c] = acc[c] + (double)x[r * C + c0 + c];
+      for (int64_t c = 0; c < n; ++c) out[c0 + c] = (float)acc[c];
+    }
+  } else {
+    double total = 0.0;
+#pragma omp parallel for reduction(+ : total)
+    for (int64_t r = 0; r < R; ++r) {
+      double acc = 0.0;
+      for (int64_t c = 0; c < C; ++c) acc = acc + (double)x[r * C + c];
+      total += acc;
+    }
+    out[0] = (float)total;
+  }
+}

@@ -27,6 +27,21 @@ def _i64(v):
     return ctypes.c_int64(int(v))
 
 
+def c2_parallel(x, which):
+    """(result, seconds) of one reduction of configuration 2 with OpenMP over the outputs:
+    NOT what the reference does (its CAReduce loops are serial); reported for context only.
+    ``which``: sum_axis1, max_axis1, sum_axis0, sum_all, prod_axis1."""
+    L = graph_ref.lib()
+    x = np.ascontiguousarray(x, "float32")
+    R, C = x.shape
+    code = ["sum_axis1", "max_axis1", "sum_axis0", "sum_all", "prod_axis1"].index(which)
+    out = np.empty({2: C, 3: 1}.get(code, R), "float32")
+    t0 = time.perf_counter()
+    L.cpu_c2_parallel(_p(x), _p(out), _i64(R), _i64(C), ctypes.c_int(code))
+    dt = time.perf_counter() - t0
+    return (out.reshape(()) if code == 3 else out), dt
+
+
 def run(name, inputs):
     """(outputs, seconds) of one configuration's CPU loops.  ``inputs`` are
     the C-contiguous NumPy arrays of ``workloads.<config>_inputs``."""

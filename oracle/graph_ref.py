@@ -166,6 +166,46 @@ def max_and_argmax(x, axes):
     return np.asarray(np.max(x, axes), dtype=x.dtype), np.asarray(np.argmax(r, axis=-1), dtype="int64")
 
 
+def _softmax(x):
+    """Softmax.perform, theano/tensor/nnet/nnet.py:440-444"""
+    e_x = np.exp(x - x.max(axis=1)[:, None])
+    return e_x / e_x.sum(axis=1)[:, None]
+
+
+def _softmax_with_bias(x, b):
+    """SoftmaxWithBias.perform, theano/tensor/nnet/nnet.py:73-104"""
+    if b.shape[0] != x.shape[1]:
+        raise ValueError("b must have same number of columns as x")
+    if x.size == 0:
+        return np.zeros(x.shape, dtype=x.dtype)
+    x_dtype = x.dtype
+    if x.dtype == "float16":
+        x = x.astype("float32")
+    x_plus_b = x + b[None, :]
+    e_x = np.exp(x_plus_b - x_plus_b.max(axis=1)[:, None])
+    e_x *= 1.0 / e_x.sum(axis=1)[:, None]
+    return e_x.astype(x_dtype, copy=False)
+
+
+def _softmax_grad(dy, sm):
+    """SoftmaxGrad.perform, theano/tensor/nnet/nnet.py:316-323"""
+    dx = np.zeros_like(sm)
+    for i in range(sm.shape[0]):
+        dy_times_sm_i = dy[i] * sm[i]
+        dx[i] = dy_times_sm_i - sum(dy_times_sm_i) * sm[i]
+    return dx
+
+
+def _logsoftmax(x):
+    """LogSoftmax.perform, theano/tensor/nnet/nnet.py:628-633"""
+    xdev = x - x.max(axis=1)[:, None]
+    return xdev - np.log(np.sum(np.exp(xdev), axis=1, keepdims=True))
+
+
+_ROW_OPS = {"Softmax": _softmax, "SoftmaxWithBias": _softmax_with_bias, "SoftmaxGrad": _softmax_grad,
+            "LogSoftmax": _logsoftmax}
+
+
 def evaluate(inputs, outputs, values):
     """Values of ``outputs`` (theano_amd variables) given ``values`` for
     ``inputs``; every Apply node is computed separately, as an unfused graph."""
@@ -224,6 +264,8 @@ def evaluate(inputs, outputs, values):
             idx = [slice(None)] * args[0].ndim
             idx[op.axis] = slice(at, at + args[1 + op.k].shape[op.axis])
             res = [args[0][tuple(idx)]]
+        elif type(op).__name__ in _ROW_OPS:
+            res = [_ROW_OPS[type(op).__name__](*args).astype(node.outputs[0].type.dtype, copy=False)]
         else:
             raise NotImplementedError("oracle cannot evaluate %s" % op)
         for o, v in zip(node.outputs, res):

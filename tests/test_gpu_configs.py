@@ -199,3 +199,31 @@ def test_sgd_steps_with_shared_weights_and_updates():
         bn = bn - 0.5 * dz.sum(keepdims=True)
     assert np.allclose(w.get_value(), wn, rtol=1e-3, atol=1e-4)
     assert np.allclose(b.get_value(), bn, rtol=1e-3, atol=1e-4)
+
+
+def test_softmax_ops_and_the_rewrites_that_produce_them():
+    """Softmax / SoftmaxGrad / LogSoftmax nodes (evaluated by the oracle with the
+    reference's perform formulas, theano/tensor/nnet/nnet.py:316-323, 440-444, 628-633)
+    against the kernels their lowered graphs compile to; the unstabilised quotient
+    exp(x) / sum(exp(x)) and log(softmax(x)) are recognised, so that rows holding large
+    values stay finite (softmax_simplifier :888-925, local_logsoftmax :749-769)."""
+    from theano_amd.hip import HipRowChain
+    N = T.nnet
+    rng = np.random.default_rng(43)
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    xv = (3 * rng.standard_normal((257, 1000))).astype("float32")
+    xv[0, 5] = 300.0                                 # exp overflows in float32
+    yv = rng.uniform(0, 1, (257, 1000)).astype("float32")
+    sm = N.softmax(x)
+    cost = -T.sum(T.log(sm) * y)
+    outs = [sm, N.softmax_graph(x), T.log(sm), th.grad(cost, x), N.softmax_grad(y, sm), th.Rop(sm, x, y)]
+    f = th.function([x, y], outs)
+    kernels = [n for n in f.toposort() if type(n.op).__name__.startswith("Hip") and
+               type(n.op).__name__ not in ("HipDimShuffle", "HipToHost")]
+    assert len(kernels) == 1 and isinstance(kernels[0].op, HipRowChain), kernels
+    got = f(xv, yv)
+    ref = G.evaluate([x, y], [sm, sm, N.logsoftmax(x), th.grad(-T.sum(N.logsoftmax(x) * y), x), N.softmax_grad(y, sm),
+                              N.softmax_grad(y, sm)], [xv, yv])
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert np.isfinite(g).all(), k
+        assert_parity(g, r, "softmax output %d" % k, tol=dict(rtol=2e-5, atol=2e-6))

@@ -338,3 +338,90 @@ def test_rop_matches_finite_differences_and_lop_matches_grad():
     both = G.evaluate([x, v, b, u], [th.Rop(y, [x, b], [v, u])], [xv, vv, bv, wv])[0]
     fb = lambda t: G.evaluate([x, b], [y], [xv + t * vv, bv + t * wv])[0]
     assert np.allclose(both, (fb(eps) - fb(-eps)) / (2 * eps), rtol=1e-6, atol=1e-8)
+
+
+def _ops_of(fg):
+    return [type(n.op).__name__ for n in fg.toposort()]
+
+
+def test_softmax_ops_make_node_grad_and_rewrites():
+    """The row-softmax Op family: interface checks (theano/tensor/nnet/nnet.py:62-72,
+    303-315, 424-437), the rewrites that produce the ops (softmax_simplifier :888-925,
+    local_softmax_with_bias :822-885, local_logsoftmax :749-769, local_logsoftmax_grad
+    :772-804) and the lowering that leaves only Elemwise / CAReduce / DimShuffle nodes."""
+    import warnings
+    from theano_amd import gof
+    from theano_amd.tensor import nnet as N, opt as topt
+    from oracle import graph_ref as G
+    rng = np.random.default_rng(3)
+    x, y = T.dmatrix("x"), T.dmatrix("y")
+    b = T.dvector("b")
+    with pytest.raises(ValueError):
+        N.softmax_op(T.lmatrix())
+    with pytest.raises(ValueError):
+        N.softmax_op(T.TensorType("float32", (False,) * 3)())
+    with pytest.raises(ValueError):
+        N.softmax_with_bias(x, x)
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        assert N.softmax_op(b).type.ndim == 2          # vectors are padded to one row
+    assert N.softmax_op == N.Softmax() and hash(N.softmax_op) == hash(N.Softmax())
+
+    # the unstabilised quotient becomes the op: finite results where exp overflows
+    fg = gof.FunctionGraph([x], [N.softmax_graph(x)])
+    gof.merge_identical(fg)                        # the two exp(x) nodes become one
+    gof.apply_local(fg, topt.CANONICALIZE + N.RECOGNIZE)
+    assert _ops_of(fg) == ["Softmax"]
+    xv = rng.standard_normal((5, 7)) * 3
+    xv[0, 0] = 800.0
+    got = G.evaluate(fg.inputs, fg.outputs, [xv])[0]
+    assert np.isfinite(got).all() and np.allclose(got.sum(1), 1.0)
+
+    # softmax(x + b) -> softmax_with_bias; log(softmax) -> logsoftmax, also in the gradient
+    fg = gof.FunctionGraph([x, b], [N.softmax(x + b.dimshuffle("x", 0))])
+    gof.apply_local(fg, topt.CANONICALIZE + N.RECOGNIZE)
+    assert _ops_of(fg) == ["SoftmaxWithBias"]
+    cost = T.sum(T.log(N.softmax(x)) * y)
+    fg = gof.FunctionGraph([x, y], [cost, th.grad(cost, x)])
+    gof.merge_identical(fg)
+    gof.apply_local(fg, topt.CANONICALIZE + N.RECOGNIZE)
+    names = _ops_of(fg)
+    assert "LogSoftmax" in names and "SoftmaxGrad" not in names and names.count("Softmax") == 1
+
+    # values and gradients of the ops (evaluated by the reference's perform formulas)
+    # against the lowered Elemwise / CAReduce graphs and against closed forms
+    yv, bv = rng.uniform(0, 1, (5, 7)), rng.standard_normal(7)
+    sm, lsm, swb = N.softmax(x), N.logsoftmax(x), N.softmax_with_bias(x, b)
+    outs = [sm, lsm, swb, th.grad(T.sum(sm * y), x), th.grad(T.sum(lsm * y), x), th.grad(T.sum(swb * y), b),
+            th.grad(T.sum(th.grad(T.sum(sm * y), x) ** 2), x), th.Rop(sm, x, y)]
+    as_ops = G.evaluate([x, y, b], outs, [xv, yv, bv])
+    fg = gof.FunctionGraph([x, y, b], outs)
+    topt.canonicalize(fg)
+    assert set(_ops_of(fg)) <= {"Elemwise", "DimShuffle", "Sum", "Max", "CAReduce"}
+    lowered = G.evaluate(fg.inputs, fg.outputs, [xv, yv, bv])
+    for a, l in zip(as_ops, lowered):
+        assert np.allclose(a, l, rtol=1e-10, atol=1e-12)
+    e = np.exp(xv - xv.max(1, keepdims=True))
+    p = e / e.sum(1, keepdims=True)
+    from scipy.special import log_softmax
+    assert np.allclose(as_ops[0], p) and np.allclose(as_ops[1], log_softmax(xv, axis=1))
+    assert np.isfinite(as_ops[1]).all()                # row 0 holds 800: log(softmax) itself gives -inf there
+    assert np.allclose(as_ops[3], p * (yv - (p * yv).sum(1, keepdims=True)))
+    assert np.allclose(as_ops[4], yv - yv.sum(1, keepdims=True) * p)
+    assert np.allclose(as_ops[7], as_ops[3])           # symmetric Jacobian
+
+
+def test_softmax_op_graphs_compile_to_one_row_kernel():
+    from theano_amd import hip
+    from theano_amd.tensor import nnet as N
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    hip.set_dry_run(True)
+    try:
+        cost = T.sum(T.log(N.softmax(x)) * y)
+        f = th.function([x, y], [N.softmax(x), th.grad(cost, x)])
+        f(np.zeros((4, 64), "float32"), np.zeros((4, 64), "float32"))
+        kernels = [type(n.op).__name__ for n in f.toposort() if type(n.op).__name__.startswith("Hip")
+                   and type(n.op).__name__ not in ("HipDimShuffle", "HipToHost")]
+        assert kernels == ["HipRowChain"], kernels
+    finally:
+        hip.set_dry_run(False)

@@ -350,3 +350,22 @@ def test_view_ops_against_numpy_and_finite_differences():
     ana = G.evaluate([x, y, r], grads, [xv, yv, rv])
     for a, n in zip(ana, num):
         assert a.shape == n.shape and np.allclose(a, n, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("which", ["sum_axis1", "max_axis1", "sum_axis0", "sum_all", "prod_axis1"])
+def test_parallel_reduce_variant_agrees_with_the_serial_loops(which):
+    """The OpenMP variant reported beside the CPU baseline (not reference behaviour) gives
+    the serial loops' results: bit for bit except for the sum of everything, whose partial
+    sums are added in another order."""
+    from oracle import cpu_backend as B
+    import workloads as W
+    x = W.c2_inputs(which, "small")[0]
+    op, axis, acc = {"sum_axis1": ("Add", (1,), "float64"), "max_axis1": ("Maximum", (1,), "float32"),
+                     "sum_axis0": ("Add", (0,), "float64"), "sum_all": ("Add", None, "float64"),
+                     "prod_axis1": ("Mul", (1,), "float64")}[which]
+    want = G.careduce(x, op, axis, acc, "float32")
+    got, _ = B.c2_parallel(x, which)
+    if which == "sum_all":
+        assert np.allclose(got, want, rtol=1e-6)
+    else:
+        assert np.array_equal(got, want)

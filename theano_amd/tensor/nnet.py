@@ -1,41 +1,307 @@
-"""Row-wise activations of ``theano.tensor.nnet`` written as Elemwise / CAReduce
-graphs, so that they run as one fused row kernel each (forward and gradient).
+"""Row-wise activations of ``theano.tensor.nnet``.
 
-The reference implements ``softmax`` / ``logsoftmax`` as hand-written ops
-(``theano/tensor/nnet/nnet.py:411-600, 603-700``) and rewrites user-written
-``exp(x) / exp(x).sum(-1)`` graphs into them (``softmax_simplifier`` :888-925,
-``local_logsoftmax`` :703-722).  Here the direction is the opposite: the op's
-``perform`` formula is the graph, gradients come from ``grad`` of that graph
-and the row-chain fusion turns either into a single launch.
+``Softmax`` / ``SoftmaxWithBias`` / ``SoftmaxGrad`` / ``LogSoftmax`` exist as graph
+nodes with the reference's interface (``theano/tensor/nnet/nnet.py:43-120, 292-345,
+411-470, 602-650``): same ``make_node`` checks, gradients expressed through each other,
+``R_op``, ``infer_shape``.  The rewrites that produce them are kept too
+(``softmax_simplifier`` :888-925, ``local_softmax_with_bias`` :822-885,
+``local_logsoftmax`` :749-769, ``local_logsoftmax_grad`` :772-804).  Where the
+reference then runs hand-written C per op, these nodes are lowered, right before the
+graph is lifted, to the Elemwise / CAReduce graph of their ``perform`` formulas, and the
+row-chain fusion turns each (forward, gradient, or both at once) into one launch.
 """
+import warnings
+
+from .. import gof
+from .. import scalar as scal
+from ..gof import Apply, Op, local_optimizer
 from . import basic as T
+from .elemwise import DimShuffle, Elemwise, Sum
 from .type import as_tensor_variable
 
 sigmoid = T.sigmoid
 softplus = T.softplus
 
+_FLOATS = ("float16", "float32", "float64")
+
+
+def _no_host(op):
+    raise NotImplementedError("%s has no host implementation: it is lowered to Elemwise / CAReduce nodes before "
+                              "the graph runs" % op)
+
+
+def _row_input(x, who):
+    x = as_tensor_variable(x)
+    if x.type.ndim not in (1, 2) or x.type.dtype not in _FLOATS:
+        raise ValueError("x must be 1-d or 2-d tensor of floats. Got %s" % x.type)
+    if x.type.ndim == 1:
+        warnings.warn("DEPRECATION: If x is a vector, %s will not automatically pad x anymore in next releases. "
+                      "If you need it, please do it manually." % who, stacklevel=4)
+        x = x.dimshuffle("x", 0)
+    return x
+
+
+def _rows(v):
+    """(n,) per-row values as an (n, 1) column."""
+    return v.dimshuffle(0, "x")
+
+
+class Softmax(Op):
+    """``e = exp(x - max(x, 1)); e / sum(e, 1)`` per row
+    (``theano/tensor/nnet/nnet.py:411-456``)."""
+
+    __props__ = ()
+
+    def make_node(self, x):
+        x = _row_input(x, "Softmax")
+        return Apply(self, [x], [x.type()])
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def infer_shape(self, node, shapes):
+        return shapes
+
+    def L_op(self, inputs, outputs, grads):
+        return [softmax_grad(grads[0], outputs[0])]
+
+    def R_op(self, inputs, eval_points):
+        # the Jacobian is symmetric: same expression as the gradient
+        if None in eval_points:
+            return [None]
+        return self.L_op(inputs, [self(*inputs)], eval_points)
+
+    @staticmethod
+    def lower(x):
+        e = T.exp(x - T.max(x, axis=1, keepdims=True))
+        return e / T.sum(e, axis=1, keepdims=True)
+
+
+class SoftmaxWithBias(Op):
+    """Softmax of ``x + b`` with ``b`` a vector along the rows
+    (``theano/tensor/nnet/nnet.py:43-115``)."""
+
+    __props__ = ()
+
+    def make_node(self, x, b):
+        x, b = as_tensor_variable(x), as_tensor_variable(b)
+        if x.type.ndim != 2 or x.type.dtype not in _FLOATS:
+            raise ValueError("x must be 2-d tensor of floats")
+        if b.type.ndim != 1 or b.type.dtype not in _FLOATS:
+            raise ValueError("b must be 1-d tensor of floats")
+        return Apply(self, [x, b], [x.type()])
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def infer_shape(self, node, shapes):
+        return [shapes[0]]
+
+    def L_op(self, inputs, outputs, grads):
+        dx = softmax_grad(grads[0], outputs[0])
+        return [dx, T.sum(dx, axis=0)]
+
+    @staticmethod
+    def lower(x, b):
+        # float16 rows are computed in float32 and cast back (nnet.py:93-104)
+        dt = x.type.dtype
+        if dt == "float16":
+            x = T.cast(x, "float32")
+        r = Softmax.lower(x + b.dimshuffle("x", 0))
+        return T.cast(r, dt) if r.type.dtype != dt else r
+
+
+class SoftmaxGrad(Op):
+    """``dx = dy * sm - sum(dy * sm, 1) * sm`` per row
+    (``theano/tensor/nnet/nnet.py:292-335``)."""
+
+    __props__ = ()
+
+    def make_node(self, dy, sm):
+        dy, sm = as_tensor_variable(dy), as_tensor_variable(sm)
+        if dy.type.ndim not in (1, 2) or dy.type.dtype not in _FLOATS:
+            raise ValueError("dy must be 1-d or 2-d tensor of floats. Got %s" % dy.type)
+        if dy.type.ndim == 1:
+            dy = dy.dimshuffle("x", 0)
+        if sm.type.ndim == 1:
+            sm = sm.dimshuffle("x", 0)
+        return Apply(self, [dy, sm], [sm.type()])
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def infer_shape(self, node, shapes):
+        return [shapes[1]]
+
+    def L_op(self, inputs, outputs, grads):
+        dy, sm = inputs
+        (g,) = grads
+        tmp = g + T.neg(_rows(T.sum(g * sm, axis=1)))
+        tmp2 = _rows(T.sum(dy * sm, axis=1))
+        return [tmp * sm, tmp * dy - g * tmp2]
+
+    @staticmethod
+    def lower(dy, sm):
+        t = dy * sm
+        r = t - T.sum(t, axis=1, keepdims=True) * sm
+        return T.cast(r, sm.type.dtype) if r.type.dtype != sm.type.dtype else r
+
+
+class LogSoftmax(Op):
+    """``xdev = x - max(x, 1); xdev - log(sum(exp(xdev), 1))`` per row
+    (``theano/tensor/nnet/nnet.py:602-646``)."""
+
+    __props__ = ()
+
+    def make_node(self, x):
+        x = _row_input(x, "LogSoftmax")
+        return Apply(self, [x], [x.type()])
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def infer_shape(self, node, shapes):
+        return shapes
+
+    def L_op(self, inputs, outputs, grads):
+        sm = softmax_op(inputs[0])
+        return [grads[0] - T.sum(grads[0], axis=1, keepdims=True) * sm]
+
+    def R_op(self, inputs, eval_points):
+        if None in eval_points:
+            return [None]
+        return self.L_op(inputs, None, eval_points)
+
+    @staticmethod
+    def lower(x):
+        xdev = x - T.max(x, axis=1, keepdims=True)
+        return xdev - T.log(T.sum(T.exp(xdev), axis=1, keepdims=True))
+
+
+softmax_op, softmax_with_bias = Softmax(), SoftmaxWithBias()
+softmax_grad, logsoftmax_op = SoftmaxGrad(), LogSoftmax()
+
+
+def softmax_graph(c):
+    """The unstabilised expression ``softmax_simplifier`` recognises (nnet.py:807-808)."""
+    c = as_tensor_variable(c)
+    return T.exp(c) / T.sum(T.exp(c), axis=-1, keepdims=True)
+
 
 def softmax(c):
-    """``Softmax.perform`` (``theano/tensor/nnet/nnet.py:440-446``):
-    ``e = exp(x - max(x, -1)); e / sum(e, -1)``."""
+    """``softmax_op`` for vectors and matrices (``theano/tensor/nnet/nnet.py:811-815``);
+    tensors of higher rank, which the reference's op refuses, get the same formula along
+    their last axis as a plain graph."""
+    c = as_tensor_variable(c)
+    if c.type.broadcastable[-1]:
+        warnings.warn("The softmax is applied on a dimension of shape 1, which does not have a semantic meaning.")
+    if c.type.ndim <= 2:
+        return softmax_op(c)
     return T.softmax(c)
 
 
-def softmax_with_bias(x, b):
-    """``SoftmaxWithBias`` (``theano/tensor/nnet/nnet.py:43-90``): softmax of
-    ``x + b`` with ``b`` a vector along the last axis."""
-    x, b = as_tensor_variable(x), as_tensor_variable(b)
-    if b.type.ndim != 1:
-        raise ValueError("b must be a 1-d tensor")
-    return T.softmax(x + b.dimshuffle(*(["x"] * (x.type.ndim - 1) + [0])))
-
-
 def logsoftmax(c):
-    """``LogSoftmax.perform`` (``theano/tensor/nnet/nnet.py:628-633``):
-    ``xdev = x - max(x, -1); xdev - log(sum(exp(xdev), -1))``."""
-    x = as_tensor_variable(c)
-    xdev = x - T.max(x, axis=-1, keepdims=True)
+    c = as_tensor_variable(c)
+    if c.type.ndim <= 2:
+        return logsoftmax_op(c)
+    xdev = c - T.max(c, axis=-1, keepdims=True)
     return xdev - T.log(T.sum(T.exp(xdev), axis=-1, keepdims=True))
+
+
+# ---- rewrites --------------------------------------------------------------------------------------
+
+def _is_elemwise(var, scalar_cls):
+    return (var.owner is not None and isinstance(var.owner.op, Elemwise) and
+            isinstance(var.owner.op.scalar_op, scalar_cls))
+
+
+@local_optimizer([Elemwise])
+def local_softmax_simplifier(fgraph, node):
+    """``exp(x) / sum(exp(x), 1).dimshuffle(0, 'x')`` on a float matrix -> ``softmax(x)``
+    (``softmax_simplifier``, nnet.py:888-925; the reference runs it inside the
+    multiplication canonizer over lists of numerators and denominators, here the
+    two-operand quotient is matched)."""
+    if not isinstance(node.op.scalar_op, scal.TrueDiv) or len(node.inputs) != 2:
+        return False
+    num, den = node.inputs
+    if num.type.ndim != 2 or not num.type.dtype.startswith("float") or not _is_elemwise(num, type(scal.exp)):
+        return False
+    if den.owner is None or not isinstance(den.owner.op, DimShuffle) or den.owner.op.new_order != (0, "x"):
+        return False
+    z = den.owner.inputs[0]
+    if z.owner is None or not isinstance(z.owner.op, Sum) or z.owner.op.axis != (1,):
+        return False
+    if z.owner.inputs[0] is not num or z.type.dtype != num.type.dtype:
+        return False
+    return [softmax_op(num.owner.inputs[0])]
+
+
+@local_optimizer([Softmax])
+def local_softmax_with_bias(fgraph, node):
+    """``softmax(matrix + vector.dimshuffle('x', 0))`` -> ``softmax_with_bias(matrix, vector)``
+    (nnet.py:822-885)."""
+    (x,) = node.inputs
+    if not _is_elemwise(x, scal.Add):
+        return False
+    vectors, others = [], []
+    for t in x.owner.inputs:
+        if tuple(t.type.broadcastable) == (True, False):
+            if (t.owner is not None and isinstance(t.owner.op, DimShuffle) and
+                    tuple(t.owner.inputs[0].type.broadcastable) == (False,)):
+                vectors.append(t.owner.inputs[0])
+            else:
+                vectors.append(DimShuffle((True, False), (1,))(t))
+        else:
+            others.append(t)
+    if not others:
+        others.append(vectors.pop().dimshuffle("x", 0))
+    if not vectors:
+        return False
+    vsum = T.add(*vectors) if len(vectors) > 1 else vectors[0]
+    msum = T.add(*others) if len(others) > 1 else others[0]
+    try:
+        res = softmax_with_bias(msum, vsum)
+    except (ValueError, TypeError):
+        return False
+    return [res] if res.type == node.outputs[0].type else False
+
+
+@local_optimizer([Elemwise])
+def local_logsoftmax(fgraph, node):
+    """``log(softmax(x))`` -> ``logsoftmax(x)`` (nnet.py:749-769)."""
+    if not isinstance(node.op.scalar_op, type(scal.log)) or len(node.inputs) != 1:
+        return False
+    p = node.inputs[0].owner
+    if p is None or not isinstance(p.op, Softmax):
+        return False
+    return [logsoftmax_op(p.inputs[0])]
+
+
+@local_optimizer([SoftmaxGrad])
+def local_logsoftmax_grad(fgraph, node):
+    """``softmax_grad(g / sm, sm)`` with ``sm = softmax(x)``: the gradient of
+    ``log(softmax(x))``, rewritten to ``g - sum(g, 1, keepdims) * sm`` without the division
+    (nnet.py:772-804)."""
+    dy, sm = node.inputs
+    if not _is_elemwise(dy, scal.TrueDiv) or len(dy.owner.inputs) != 2:
+        return False
+    g, den = dy.owner.inputs
+    if den is not sm or sm.owner is None or not isinstance(sm.owner.op, Softmax):
+        return False
+    if g.type.broadcastable[1] and not sm.type.broadcastable[1]:
+        g = T.second(sm, g)
+    res = g - T.sum(g, axis=1, keepdims=True) * sm
+    return [res] if res.type == node.outputs[0].type else False
+
+
+@local_optimizer([Softmax, SoftmaxWithBias, SoftmaxGrad, LogSoftmax])
+def local_lower_row_ops(fgraph, node):
+    res = node.op.lower(*node.inputs)
+    return [res] if res.type == node.outputs[0].type else False
+
+
+RECOGNIZE = [local_softmax_simplifier, local_softmax_with_bias, local_logsoftmax, local_logsoftmax_grad]
+LOWER = [local_lower_row_ops]
 
 
 def relu(x, alpha=0):

@@ -352,7 +352,15 @@ CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_constant_fold, lo
 
 
 def canonicalize(fgraph):
+    """Clean-ups to a fixed point, together with the rewrites that recognise row softmax
+    expressions; then the row ops are lowered to Elemwise / CAReduce graphs and those are
+    cleaned up in turn."""
+    from . import nnet
     gof.merge_identical(fgraph)
-    gof.apply_local(fgraph, CANONICALIZE)
+    gof.apply_local(fgraph, CANONICALIZE + nnet.RECOGNIZE)
     gof.merge_identical(fgraph)
+    if gof.apply_local(fgraph, nnet.LOWER):
+        gof.merge_identical(fgraph)
+        gof.apply_local(fgraph, CANONICALIZE)
+        gof.merge_identical(fgraph)
     return fgraph
