@@ -338,6 +338,29 @@ round_half_to_even = _libm(np.rint)
 round_half_away_from_zero = _libm(lambda a: np.where(a > 0, np.floor(a + 0.5), np.ceil(a - 0.5)))
 
 
+def _special(name):
+    """scipy.special is what the reference's ``impl`` calls for these ops
+    (``theano/scalar/basic_scipy.py:32-36`` and alike)."""
+    def f(out_dtype, x):
+        import scipy.special
+        ct = "float32" if str(out_dtype) == "float16" else out_dtype
+        with np.errstate(all="ignore"):
+            return _conv(getattr(scipy.special, name)(_conv(x, ct)), out_dtype)
+    return f
+
+
+erf, erfc, erfcx = _special("erf"), _special("erfc"), _special("erfcx")
+erfinv, erfcinv = _special("erfinv"), _special("erfcinv")
+gamma, gammaln, psi = _special("gamma"), _special("gammaln"), _special("psi")
+
+
+def tri_gamma(out_dtype, x):
+    import scipy.special
+    ct = "float32" if str(out_dtype) == "float16" else out_dtype
+    with np.errstate(all="ignore"):
+        return _conv(scipy.special.polygamma(1, _conv(x, ct)), out_dtype)
+
+
 def arctan2(out_dtype, y, x):
     ct = "float32" if str(out_dtype) == "float16" else out_dtype
     return _conv(np.arctan2(_conv(y, ct), _conv(x, ct)), out_dtype)
@@ -384,5 +407,6 @@ BY_CLASS = {
     "RoundHalfAwayFromZero": round_half_away_from_zero, "Cos": cos, "Sin": sin, "Tan": tan, "ArcCos": arccos,
     "ArcSin": arcsin, "ArcTan": arctan, "ArcTan2": arctan2, "Cosh": cosh, "Sinh": sinh, "Tanh": tanh,
     "ArcCosh": arccosh, "ArcSinh": arcsinh, "ArcTanh": arctanh, "ScalarSigmoid": scalar_sigmoid,
-    "ScalarSoftplus": scalar_softplus,
+    "ScalarSoftplus": scalar_softplus, "Erf": erf, "Erfc": erfc, "Erfcx": erfcx, "Erfinv": erfinv, "Erfcinv": erfcinv,
+    "Gamma": gamma, "GammaLn": gammaln, "Psi": psi, "TriGamma": tri_gamma,
 }

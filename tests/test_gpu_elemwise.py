@@ -210,3 +210,28 @@ def test_column_major_inputs_give_column_major_outputs():
     # through the host boundary
     got = th.function([x, y, s], [T.exp(x) * y + s])(a, b, one)[0]
     assert np.allclose(got, np.exp(a) * b + one, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+def test_special_functions_against_scipy(dtype):
+    """erf / erfc / erfcx / erfinv / erfcinv / gamma / gammaln / psi / tri_gamma
+    (theano/scalar/basic_scipy.py:29-470) against scipy.special, which is what the
+    reference's own impl calls, and their gradients against the oracle's evaluation of
+    the same gradient graphs."""
+    rng = np.random.default_rng(17)
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == "float32" else dict(rtol=1e-11, atol=1e-12)
+    x = T.TensorType(dtype, (False,))("x")
+    wide = np.concatenate([rng.uniform(-4, 4, 3000), rng.uniform(0.05, 30, 3000)]).astype(dtype)
+    unit = rng.uniform(-0.999, 0.999, 6000).astype(dtype)
+    pos = np.concatenate([rng.uniform(0.05, 30, 5000), rng.uniform(-5.9, -0.1, 1000)]).astype(dtype)
+    pos = pos[np.abs(pos - np.round(pos)) > 0.05]      # stay away from the poles
+    cases = [("erf", wide), ("erfc", wide), ("erfcx", wide), ("erfinv", unit), ("erfcinv", (1 + unit).astype(dtype)),
+             ("gamma", pos), ("gammaln", pos), ("psi", pos), ("tri_gamma", pos)]
+    for name, vals in cases:
+        op = getattr(T, name)
+        outs = [op(x)] if name == "tri_gamma" else [op(x), th.grad(T.sum(op(x)), x)]
+        got = th.function([x], outs)(vals)
+        ref = G.evaluate([x], outs, [vals])
+        for k, (g, r) in enumerate(zip(got, ref)):
+            assert_parity(g, r, "%s output %d" % (name, k), tol=tol)

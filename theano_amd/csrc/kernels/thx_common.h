@@ -44,6 +44,47 @@ __device__ __forceinline__ float thx_fdiv(float a, float b) {
 __device__ __forceinline__ float thx_fdiv(float a, float b) { return a / b; }
 #endif
 
+// Digamma and trigamma (the reference ships its own C for both, theano/scalar/basic_scipy.py:
+// 340-391, 430-470): arguments below 10 are moved up with psi(x) = psi(x + 1) - 1/x and
+// psi'(x) = psi'(x + 1) + 1/x^2, negative ones first reflected to 1 - x, then the asymptotic
+// series in 1/x^2 is summed in double precision.  Poles (0, -1, -2, ...) give NaN.
+__device__ inline double thx_psi(double x) {
+  double r = 0.0;
+  if (x <= 0.0) {
+    if (x == floor(x)) return NAN;
+    r = -3.14159265358979323846 / tan(3.14159265358979323846 * x);
+    x = 1.0 - x;
+  }
+  while (x < 10.0) {
+    r -= 1.0 / x;
+    x += 1.0;
+  }
+  const double f = 1.0 / (x * x);
+  const double t = f * (1.0 / 12 - f * (1.0 / 120 - f * (1.0 / 252 - f * (1.0 / 240 - f * (1.0 / 132)))));
+  return r + log(x) - 0.5 / x - t;
+}
+__device__ inline float thx_psi(float x) { return (float)thx_psi((double)x); }
+
+__device__ inline double thx_trigamma(double x) {
+  double r = 0.0, sign = 1.0;
+  if (x <= 0.0) {
+    if (x == floor(x)) return NAN;
+    const double s = sin(3.14159265358979323846 * x);
+    r = 9.86960440108935861883 / (s * s);
+    sign = -1.0;
+    x = 1.0 - x;
+  }
+  double acc = 0.0;
+  while (x < 10.0) {
+    acc += 1.0 / (x * x);
+    x += 1.0;
+  }
+  const double f = 1.0 / (x * x);
+  const double t = f * (1.0 / 6 - f * (1.0 / 30 - f * (1.0 / 42 - f * (1.0 / 30 - f * (5.0 / 66)))));
+  return r + sign * (acc + 1.0 / x + 0.5 * f + t / x);
+}
+__device__ inline float thx_trigamma(float x) { return (float)thx_trigamma((double)x); }
+
 namespace thx {
 
 // How one operand is addressed along the vectorised (innermost) dimension.

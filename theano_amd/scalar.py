@@ -305,8 +305,9 @@ class specific_out(object):
 
 # --------------------------------------------------------------------------
 def _fn(name, dtype):
-    """libm-style function name for the compute type of ``dtype``."""
-    return name if compute_ctype(dtype) == "thx_f64" else name + "f"
+    """libm-style function name for the compute type of ``dtype``; helpers of
+    the kernel prelude (``thx_*``) are overloaded instead."""
+    return name if compute_ctype(dtype) == "thx_f64" or name.startswith("thx_") else name + "f"
 
 
 def c_literal(value, dtype):
@@ -958,6 +959,19 @@ tanh = _unary_math("Tanh", "tanh", lambda x, z, gz: gz * (1 - sqr(z)))
 arccosh = _unary_math("ArcCosh", "acosh", lambda x, z, gz: gz / sqrt(sqr(x) - 1))
 arcsinh = _unary_math("ArcSinh", "asinh", lambda x, z, gz: gz / sqrt(sqr(x) + 1))
 arctanh = _unary_math("ArcTanh", "atanh", lambda x, z, gz: gz / (1 - sqr(x)))
+
+# Special functions (``theano/scalar/basic_scipy.py:29-391``): the device math library has the
+# error and gamma functions; digamma and trigamma are helpers of the kernel prelude.
+_TWO_OVER_SQRT_PI = 2.0 / math.sqrt(math.pi)
+erf = _unary_math("Erf", "erf", lambda x, z, gz: gz * _TWO_OVER_SQRT_PI * exp(-x * x))
+erfc = _unary_math("Erfc", "erfc", lambda x, z, gz: -gz * _TWO_OVER_SQRT_PI * exp(-x * x))
+erfcx = _unary_math("Erfcx", "erfcx", lambda x, z, gz: gz * (-_TWO_OVER_SQRT_PI + (2.0 * x) * z))
+erfinv = _unary_math("Erfinv", "erfinv", lambda x, z, gz: gz * (1.0 / _TWO_OVER_SQRT_PI) * exp(z * z))
+erfcinv = _unary_math("Erfcinv", "erfcinv", lambda x, z, gz: -gz * (1.0 / _TWO_OVER_SQRT_PI) * exp(z * z))
+gamma = _unary_math("Gamma", "tgamma", lambda x, z, gz: gz * z * psi(x))
+gammaln = _unary_math("GammaLn", "lgamma", lambda x, z, gz: gz * psi(x))
+psi = _unary_math("Psi", "thx_psi", lambda x, z, gz: gz * tri_gamma(x))
+tri_gamma = _unary_math("TriGamma", "thx_trigamma", None)
 
 
 class Trunc(UnaryScalarOp):

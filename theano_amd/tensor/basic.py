@@ -52,6 +52,10 @@ arccos, arcsin, arctan, arctan2 = (_elemwise(scal.arccos, "arccos"), _elemwise(s
                                    _elemwise(scal.arctan, "arctan"), _elemwise(scal.arctan2, "arctan2"))
 cosh, sinh, tanh = _elemwise(scal.cosh, "cosh"), _elemwise(scal.sinh, "sinh"), _elemwise(scal.tanh, "tanh")
 arccosh, arcsinh, arctanh = _elemwise(scal.arccosh, "arccosh"), _elemwise(scal.arcsinh, "arcsinh"), _elemwise(scal.arctanh, "arctanh")
+erf, erfc, erfcx = _elemwise(scal.erf, "erf"), _elemwise(scal.erfc, "erfc"), _elemwise(scal.erfcx, "erfcx")
+erfinv, erfcinv = _elemwise(scal.erfinv, "erfinv"), _elemwise(scal.erfcinv, "erfcinv")
+gamma, gammaln = _elemwise(scal.gamma, "gamma"), _elemwise(scal.gammaln, "gammaln")
+psi, tri_gamma = _elemwise(scal.psi, "psi"), _elemwise(scal.tri_gamma, "tri_gamma")
 sigmoid = _elemwise(scal.scalar_sigmoid, "sigmoid")
 softplus = _elemwise(scal.scalar_softplus, "softplus")
 
