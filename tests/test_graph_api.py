@@ -197,7 +197,9 @@ def test_batchnorm_gradient_is_two_statistics_passes_and_one_elementwise_pass(dr
     """Configuration 5's gradient graph: per-channel factors leave the sums, the
     sums that then read the same tensors merge, and the per-channel algebra
     between them runs in the second reduction's epilogue, which reads gamma as a
-    per-result device operand.  Three kernels remain; the first two are told which
+    per-result device operand.  The first pass yields mean and standard deviation
+    together (shifted sums in float64 beside the mean's own sum).  Three kernels
+    remain; the first two are told which
     of their inputs a later kernel reads again (those stay cacheable)."""
     import workloads
     ins, outs = workloads.c5_graph(forward=False)
@@ -205,8 +207,9 @@ def test_batchnorm_gradient_is_two_statistics_passes_and_one_elementwise_pass(dr
     kernels = [n for n in f.toposort() if isinstance(n.op, (HipElemwise, HipCAReduce)) and
                any(not any(i.type.broadcastable) for i in n.inputs if hasattr(i.type, "broadcastable") and i.type.ndim)]
     assert [type(n.op) for n in kernels] == [HipCAReduce, HipCAReduce, HipElemwise]
-    second = kernels[1]
-    assert len(second.op.scalar_ops) == 4 and second.op.n_extra >= 4
+    first, second = kernels[0], kernels[1]
+    assert len(first.op.scalar_ops) == 3 and len(first.outputs) == 2
+    assert len(second.op.scalar_ops) == 3 and second.op.n_extra >= 4
     extras = second.inputs[len(second.inputs) - second.op.n_extra:]
     assert any(type(e.type).__name__ == "HipArrayType" for e in extras)
     # x is read again after the first pass, x and g after the second; the last pass streams everything
@@ -425,3 +428,51 @@ def test_softmax_op_graphs_compile_to_one_row_kernel():
         assert kernels == ["HipRowChain"], kernels
     finally:
         hip.set_dry_run(False)
+
+
+def test_single_pass_variance_rewrite_keeps_the_values():
+    """sum(sqr(x - mean(x))) rewritten to shifted sums in float64: the canonicalised graph,
+    evaluated node by node, against the two-pass graph and against NumPy's float64 variance;
+    also for a channel whose first element is an outlier, a constant channel, reduction over
+    all axes, and float64 data (left alone)."""
+    from theano_amd import gof, config
+    from theano_amd.tensor import opt as topt
+    from oracle import graph_ref as G
+    rng = np.random.default_rng(9)
+    x4 = T.TensorType("float16", (False,) * 4)("x")
+    xf = T.cast(x4, "float32")
+    outs = [T.var(xf, axis=(0, 2, 3), keepdims=True), T.mean(xf, axis=(0, 2, 3), keepdims=True), T.std(xf, axis=(0, 2, 3))]
+    xv = rng.normal(0.5, 2.0, (6, 5, 7, 8)).astype("float16")
+    xv[0, 1, 0, 0] = 3000.0          # the shift of channel 1 is an outlier
+    xv[:, 2] = 1.25                   # a constant channel: variance exactly 0
+    fg = gof.FunctionGraph([x4], outs)
+    topt.canonicalize(fg)
+    sums = [n for n in fg.toposort() if type(n.op).__name__ == "Sum"]
+    assert len(sums) == 3 and all(n.inputs[0].type.ndim == 4 for n in sums), [str(n) for n in sums]
+    assert sorted(n.outputs[0].type.dtype for n in sums) == ["float32", "float64", "float64"]
+    got = G.evaluate(fg.inputs, fg.outputs, [xv])
+    with config.change_flags(single_pass_variance=False):
+        fg2 = gof.FunctionGraph([x4], outs)
+        topt.canonicalize(fg2)
+        assert len([n for n in fg2.toposort() if type(n.op).__name__ == "Sum"]) == 2
+        two_pass = G.evaluate(fg2.inputs, fg2.outputs, [xv])
+    x64 = xv.astype("float64")
+    exact = [x64.var(axis=(0, 2, 3), keepdims=True), x64.mean(axis=(0, 2, 3), keepdims=True), x64.std(axis=(0, 2, 3))]
+    for g, t, e in zip(got, two_pass, exact):
+        assert g.dtype == t.dtype == np.float32 and g.shape == t.shape
+        assert np.allclose(g, e, rtol=2e-6, atol=1e-7)
+        assert np.allclose(t, e, rtol=2e-6, atol=1e-7)
+    assert got[0][0, 2, 0, 0] == 0.0 and got[2][2] == 0.0
+
+    m = T.fmatrix("m")
+    fg = gof.FunctionGraph([m], [T.var(m), T.var(m, axis=0), T.var(m, axis=1, keepdims=True)])
+    topt.canonicalize(fg)
+    mv = rng.normal(-3.0, 0.1, (33, 17)).astype("float32")
+    for g, e in zip(G.evaluate(fg.inputs, fg.outputs, [mv]),
+                    [mv.astype("float64").var(), mv.astype("float64").var(0), mv.astype("float64").var(1, keepdims=True)]):
+        assert np.allclose(g, e, rtol=1e-5)
+
+    d = T.dmatrix("d")
+    fg = gof.FunctionGraph([d], [T.var(d, axis=0)])
+    topt.canonicalize(fg)
+    assert len([n for n in fg.toposort() if type(n.op).__name__ == "Sum"]) == 2      # still two passes

@@ -16,6 +16,9 @@ class _Config(object):
     # Largest number of inputs a fused Elemwise may take: the kernel argument
     # block is 4096 bytes (same budget as theano/gpuarray/elemwise.py:44-83).
     max_fused_inputs = 32
+    # sum(sqr(x - mean(x))) over float16 / float32 data becomes one pass of shifted sums
+    # accumulated in float64, merged with the pass that computes the mean
+    single_pass_variance = True
 
     @contextlib.contextmanager
     def change_flags(self, **kw):

@@ -46,6 +46,22 @@ def _rows(v):
     return v.dimshuffle(0, "x")
 
 
+def _row_max_already_subtracted(x):
+    """``x`` is ``y - max(y, 1, keepdims)``: its row maxima are exactly 0, so subtracting
+    them again changes nothing (a user-written stable softmax that the simplifier turned
+    into the op)."""
+    from .elemwise import CAReduce
+    if x.owner is None or not isinstance(x.owner.op, Elemwise) or not isinstance(x.owner.op.scalar_op, scal.Sub):
+        return False
+    y, m = x.owner.inputs
+    if m.owner is None or not isinstance(m.owner.op, DimShuffle) or m.owner.op.new_order != (0, "x"):
+        return False
+    r = m.owner.inputs[0]
+    return (r.owner is not None and isinstance(r.owner.op, CAReduce) and
+            isinstance(r.owner.op.scalar_op, scal.Maximum) and not isinstance(r.owner.op.scalar_op, scal.Minimum) and
+            r.owner.op.axis == (1,) and r.owner.inputs[0] is y)
+
+
 class Softmax(Op):
     """``e = exp(x - max(x, 1)); e / sum(e, 1)`` per row
     (``theano/tensor/nnet/nnet.py:411-456``)."""
@@ -73,7 +89,9 @@ class Softmax(Op):
 
     @staticmethod
     def lower(x):
-        e = T.exp(x - T.max(x, axis=1, keepdims=True))
+        if not _row_max_already_subtracted(x):
+            x = x - T.max(x, axis=1, keepdims=True)
+        e = T.exp(x)
         return e / T.sum(e, axis=1, keepdims=True)
 
 

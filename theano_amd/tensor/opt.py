@@ -346,9 +346,117 @@ def local_shape_lift(fgraph, node):
     return False
 
 
+def _strip_broadcast_shuffle(v):
+    """``v`` without DimShuffles that only insert or drop broadcastable dimensions."""
+    while v.owner is not None and isinstance(v.owner.op, DimShuffle):
+        order = [o for o in v.owner.op.new_order if o != "x"]
+        if order != sorted(order):
+            break
+        v = v.owner.inputs[0]
+    return v
+
+
+def _extent_source(x, v, axes):
+    """True when ``v`` is ``x`` or feeds ``x`` through Elemwise nodes without being
+    broadcast along ``axes``: its extents along them are ``x``'s."""
+    if x is v:
+        return True
+    if x.owner is None or not isinstance(x.owner.op, Elemwise):
+        return False
+    return any(i.type.ndim == x.type.ndim and not any(i.type.broadcastable[a] for a in axes) and
+               _extent_source(i, v, axes) for i in x.owner.inputs)
+
+
+@local_optimizer([Sum])
+def local_single_pass_variance(fgraph, node):
+    """``sum(sqr(x - mean(x, A)), A)`` on float16 / float32 data -> shifted sums in one pass:
+
+        d = x - c,  c = the first element along A (per kept index)
+        sum(sqr(x - mean)) = sum(d^2) - sum(d)^2 / N,      N = number of reduced elements
+
+    with both sums accumulated in float64, so that the subtraction costs nothing the data's
+    own precision could show (the shift keeps d within the spread of the data unless the first
+    element is an outlier by many orders of magnitude).  The two sums read the same operand as
+    the mean's own sum, so the three merge into one pass over x where the two-pass form of
+    ``var`` (``theano/tensor/basic.py:3430-3459``) needs two.  float64 data keeps two passes:
+    there is no wider accumulator to absorb the cancellation."""
+    from ..config import config
+    from .views import Subtensor
+    if not config.single_pass_variance:
+        return False
+    (sq,) = node.inputs
+    out = node.outputs[0]
+    if out.type.dtype not in ("float32", "float64") or sq.type.dtype not in ("float16", "float32"):
+        return False
+    if sq.owner is None or not isinstance(sq.owner.op, Elemwise) or not isinstance(sq.owner.op.scalar_op, scal.Sqr):
+        return False
+    diff = sq.owner.inputs[0]
+    if (diff.owner is None or not isinstance(diff.owner.op, Elemwise) or
+            not isinstance(diff.owner.op.scalar_op, scal.Sub)):
+        return False
+    x, mb = diff.owner.inputs
+    nd = x.type.ndim
+    axes = tuple(range(nd)) if node.op.axis is None else tuple(node.op.axis)
+    if not axes or x.type.dtype not in ("float16", "float32") or any(x.type.broadcastable[a] for a in axes):
+        return False
+    if mb.type.ndim != nd or not all(mb.type.broadcastable[a] for a in axes):
+        return False
+    # mean = sum(x, A) / extent / extent ... with one ShapeFloat divisor per reduced axis
+    divisors, cur = [], _strip_broadcast_shuffle(mb)
+    while (cur.owner is not None and isinstance(cur.owner.op, Elemwise) and
+           isinstance(cur.owner.op.scalar_op, scal.TrueDiv)):
+        divisors.append(_strip_broadcast_shuffle(cur.owner.inputs[1]))
+        cur = _strip_broadcast_shuffle(cur.owner.inputs[0])
+    if cur.owner is None or not isinstance(cur.owner.op, Sum) or cur.owner.inputs[0] is not x:
+        return False
+    m_axes = tuple(range(nd)) if cur.owner.op.axis is None else tuple(cur.owner.op.axis)
+    if m_axes != axes:
+        return False
+    seen = []
+    for dv in divisors:
+        if dv.owner is None or not isinstance(dv.owner.op, T.ShapeFloat):
+            return False
+        if not _extent_source(x, dv.owner.inputs[0], axes):
+            return False
+        seen.append(dv.owner.op.i)
+    if sorted(seen) != list(axes):
+        return False
+    # the shift: first element along the reduced axes, taken from the array the casts start from
+    src = x
+    while (src.owner is not None and isinstance(src.owner.op, Elemwise) and
+           isinstance(src.owner.op.scalar_op, scal.Cast) and len(src.owner.inputs) == 1):
+        src = src.owner.inputs[0]
+    if src.owner is not None and isinstance(src.owner.op, Elemwise):
+        return False            # x would have to be kept in memory only for the shift
+    first = Subtensor([0 if d in axes else slice(None) for d in range(nd)])(src)
+    order, k = [], 0
+    for d in range(nd):
+        if d in axes:
+            order.append("x")
+        else:
+            order.append(k)
+            k += 1
+    cb = DimShuffle(first.type.broadcastable, order)(first)
+    if src is x:
+        d = T.sub(x, cb)
+    else:
+        a, c0 = scal.Scalar(x.type.dtype)(), scal.Scalar(src.type.dtype)()
+        d = Elemwise(scal.Composite([a, c0], [scal.sub(a, scal.cast(c0, x.type.dtype))]))(x, cb)
+    d = T.cast(d, "float64")          # squares exact, and one fused multiply-add per element
+    s1 = Sum(node.op.axis, dtype="float64", acc_dtype="float64")(d)
+    s2 = Sum(node.op.axis, dtype="float64", acc_dtype="float64")(T.sqr(d))
+    n = None
+    for dv in divisors:
+        e = T.ShapeFloat(dv.owner.op.i, "float64")(dv.owner.inputs[0])
+        n = e if n is None else T.mul(n, e)
+    res = T.maximum(T.sub(s2, T.true_div(T.mul(s1, s1), n)), np.float64(0.0))
+    res = T.cast(res, out.type.dtype)
+    return [res] if res.type == out.type else False
+
+
 CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_constant_fold, local_useless_elemwise, local_fill_sink,
                 local_useless_reduce,
-                local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax]
+                local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_single_pass_variance]
 
 
 def canonicalize(fgraph):
