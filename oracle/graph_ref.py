@@ -202,6 +202,38 @@ def _logsoftmax(x):
     return xdev - np.log(np.sum(np.exp(xdev), axis=1, keepdims=True))
 
 
+def _bn_train(op, x, scale, bias, epsilon, running_average_factor, running_mean=None, running_var=None):
+    """AbstractBatchNormTrain.perform, theano/tensor/nnet/bn.py:475-499"""
+    axes = op.axes
+    mean = x.mean(axes, keepdims=True)
+    var = x.var(axes, keepdims=True)
+    invstd = 1.0 / np.sqrt(var + epsilon)
+    res = [(x - mean) * (scale * invstd) + bias, mean, invstd]
+    if running_mean is not None:
+        res.append(running_mean * (1.0 - running_average_factor) + mean * running_average_factor)
+        m = float(np.prod(x.shape) / np.prod(scale.shape))
+        res.append(running_var * (1.0 - running_average_factor) + (m / (m - 1)) * var * running_average_factor)
+    return res
+
+
+def _bn_inference(op, x, scale, bias, estimated_mean, estimated_variance, epsilon):
+    """AbstractBatchNormInference.perform, theano/tensor/nnet/bn.py:568-571"""
+    return [(x - estimated_mean) * (scale / np.sqrt(estimated_variance + epsilon)) + bias]
+
+
+def _bn_train_grad(op, x, dy, scale, x_mean, x_invstd, epsilon):
+    """AbstractBatchNormTrainGrad.perform, theano/tensor/nnet/bn.py:659-676"""
+    axes = op.axes
+    x_diff = x - x_mean
+    mean_dy_x_diff = np.mean(dy * x_diff, axis=axes, keepdims=True)
+    c = (dy * x_invstd) - (x_diff * mean_dy_x_diff * (x_invstd ** 3))
+    return [scale * (c - np.mean(c, axis=axes, keepdims=True)), np.sum(dy * x_invstd * x_diff, axis=axes, keepdims=True),
+            np.sum(dy, axis=axes, keepdims=True)]
+
+
+_BN_OPS = {"AbstractBatchNormTrain": _bn_train, "AbstractBatchNormInference": _bn_inference,
+           "AbstractBatchNormTrainGrad": _bn_train_grad}
+
 _ROW_OPS = {"Softmax": _softmax, "SoftmaxWithBias": _softmax_with_bias, "SoftmaxGrad": _softmax_grad,
             "LogSoftmax": _logsoftmax}
 
@@ -264,6 +296,9 @@ def evaluate(inputs, outputs, values):
             idx = [slice(None)] * args[0].ndim
             idx[op.axis] = slice(at, at + args[1 + op.k].shape[op.axis])
             res = [args[0][tuple(idx)]]
+        elif type(op).__name__ in _BN_OPS:
+            res = [np.asarray(r).astype(o.type.dtype, copy=False)
+                   for r, o in zip(_BN_OPS[type(op).__name__](op, *args), node.outputs)]
         elif type(op).__name__ in _ROW_OPS:
             res = [_ROW_OPS[type(op).__name__](*args).astype(node.outputs[0].type.dtype, copy=False)]
         else:

@@ -312,10 +312,17 @@ def local_logsoftmax_grad(fgraph, node):
     return [res] if res.type == node.outputs[0].type else False
 
 
-@local_optimizer([Softmax, SoftmaxWithBias, SoftmaxGrad, LogSoftmax])
 def local_lower_row_ops(fgraph, node):
+    if not hasattr(node.op, "lower"):
+        return False
     res = node.op.lower(*node.inputs)
-    return [res] if res.type == node.outputs[0].type else False
+    res = list(res) if isinstance(res, (list, tuple)) else [res]
+    if len(res) != len(node.outputs) or any(r.type != o.type for r, o in zip(res, node.outputs)):
+        return False
+    return res
+
+
+local_lower_row_ops = local_optimizer(None)(local_lower_row_ops)
 
 
 RECOGNIZE = [local_softmax_simplifier, local_softmax_with_bias, local_logsoftmax, local_logsoftmax_grad]
@@ -347,59 +354,301 @@ def _bn_axes(axes, ndim):
     return axes
 
 
+def _as_common_dtype(*vs):
+    dt = scal.upcast(*[v.type.dtype for v in vs])
+    return [v if v.type.dtype == dt else T.cast(v, dt) for v in vs]
+
+
+def _check_axes(axes, ndim):
+    if min(axes) < 0 or max(axes) >= ndim:
+        raise ValueError("axes should be less than ndim (<%d), but %s given" % (ndim, str(axes)))
+
+
+class AbstractBatchNormTrain(Op):
+    """Training-mode batch normalization over ``axes``
+    (``theano/tensor/nnet/bn.py:364-499``): inputs ``x, scale, bias, epsilon,
+    running_average_factor[, running_mean, running_var]``, outputs ``out, mean, invstd[,
+    new_running_mean, new_running_var]``.  The gradient through ``out`` is
+    ``AbstractBatchNormTrainGrad`` of the saved mean and inverse standard deviation."""
+
+    __props__ = ("axes",)
+
+    def __init__(self, axes=(0,)):
+        assert isinstance(axes, (tuple, list)) and len(axes) > 0
+        self.axes = tuple(int(a) for a in axes)
+
+    def _props(self):
+        return (self.axes,)
+
+    def make_node(self, x, scale, bias, epsilon=1e-4, running_average_factor=0.1, running_mean=None, running_var=None):
+        x, scale, bias = as_tensor_variable(x), as_tensor_variable(scale), as_tensor_variable(bias)
+        epsilon, raf = as_tensor_variable(epsilon), as_tensor_variable(running_average_factor)
+        assert x.type.ndim == scale.type.ndim == bias.type.ndim
+        assert (running_mean is None) == (running_var is None)
+        if running_mean is not None:
+            running_mean, running_var = as_tensor_variable(running_mean), as_tensor_variable(running_var)
+            assert running_mean.type.ndim == x.type.ndim and running_var.type.ndim == x.type.ndim
+            x, scale, bias, running_mean, running_var = _as_common_dtype(x, scale, bias, running_mean, running_var)
+        else:
+            x, scale, bias = _as_common_dtype(x, scale, bias)
+        inputs = [x, scale, bias, epsilon, raf]
+        outs = [x.type(), scale.type(), scale.type()]
+        if running_mean is not None:
+            inputs += [running_mean, running_var]
+            outs += [scale.type(), scale.type()]
+        return Apply(self, inputs, outs)
+
+    def infer_shape(self, node, shapes):
+        return [shapes[0]] + [shapes[1]] * (len(node.outputs) - 1)
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def L_op(self, inputs, outputs, grads):
+        x, scale, bias, epsilon = inputs[:4]
+        dy = grads[0]
+        if isinstance(dy.type, scal.DisconnectedType):
+            dy = T.zeros_like(outputs[0])
+        _, x_mean, x_invstd = outputs[:3]
+        res = AbstractBatchNormTrainGrad(self.axes)(x, dy, scale, x_mean, x_invstd, epsilon, return_list=True)
+        # The reference stops here (bn.py:447-459): gradients that arrive through the saved mean
+        # and inverse standard deviation are dropped, which loses terms of second derivatives.
+        # They are added when present: d mean / dx = 1 / m, d invstd / dx = -invstd^3 (x - mean) / m.
+        extra = None
+        m = None
+        for a in self.axes:
+            e = T.ShapeFloat(a, x.type.dtype)(x)
+            m = e if m is None else m * e
+        if len(grads) > 1 and not isinstance(grads[1].type, scal.DisconnectedType):
+            extra = T.second(x, grads[1]) / m
+        if len(grads) > 2 and not isinstance(grads[2].type, scal.DisconnectedType):
+            term = grads[2] * (-(x_invstd ** 3)) * (x - x_mean) / m
+            extra = term if extra is None else extra + term
+        if extra is not None:
+            res[0] = res[0] + extra
+        return res + [scal.DisconnectedType()() for _ in inputs[3:]]
+
+    def connection_pattern(self, node):
+        n_out = len(node.outputs)
+        pat = [[True, True, True] + [True] * (n_out - 3)]                   # x
+        pat += [[True, True, True] + [False] * (n_out - 3) for _ in range(2)]  # scale, bias
+        pat += [[False] * n_out for _ in range(2)]                          # epsilon, running_average_factor
+        for k in range(5, len(node.inputs)):                                # running statistics: their new value only
+            pat.append([j == 3 + (k - 5) for j in range(n_out)])
+        return pat
+
+    def lower(self, x, scale, bias, epsilon, raf, running_mean=None, running_var=None):
+        # local_abstract_batch_norm_train, bn.py:679-726
+        axes = self.axes
+        _check_axes(axes, x.type.ndim)
+        mean = T.mean(x, axis=axes, keepdims=True)
+        var = T.var(x, axis=axes, keepdims=True)
+        if epsilon.type.dtype != var.type.dtype:
+            epsilon = T.cast(epsilon, var.type.dtype)      # the epsilon should not upcast the dtype
+        invstd = T.inv(T.sqrt(var + epsilon))
+        results = [(x - mean) * (scale * invstd) + bias, mean, invstd]
+        if running_mean is not None:
+            if raf.type.dtype != var.type.dtype:
+                raf = T.cast(raf, var.type.dtype)
+            results.append(running_mean * (1.0 - raf) + mean * raf)
+            m = None
+            for a in axes:                                 # elements per statistic
+                e = T.ShapeFloat(a, var.type.dtype)(x)
+                m = e if m is None else m * e
+            results.append(running_var * (1.0 - raf) + (m / (m - 1)) * var * raf)
+        return results
+
+
+class AbstractBatchNormInference(Op):
+    """``(x - mean) * (scale / sqrt(var + eps)) + bias`` with given statistics
+    (``theano/tensor/nnet/bn.py:502-572``)."""
+
+    __props__ = ("axes",)
+
+    def __init__(self, axes=(0,)):
+        assert isinstance(axes, (tuple, list)) and len(axes) > 0
+        self.axes = tuple(int(a) for a in axes)
+
+    def _props(self):
+        return (self.axes,)
+
+    def make_node(self, x, scale, bias, estimated_mean, estimated_variance, epsilon=1e-4):
+        vs = [as_tensor_variable(v) for v in (x, scale, bias, estimated_mean, estimated_variance)]
+        epsilon = as_tensor_variable(epsilon)
+        vs = _as_common_dtype(*vs)
+        assert len(set(v.type.ndim for v in vs)) == 1
+        return Apply(self, vs + [epsilon], [vs[0].type()])
+
+    def infer_shape(self, node, shapes):
+        return [shapes[0]]
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def connection_pattern(self, node):
+        return [[True], [True], [True], [True], [True], [False]]
+
+    def L_op(self, inputs, outputs, grads):
+        x, scale, bias, est_mean, est_var, epsilon = inputs
+        dy = grads[0]
+        axes = self.axes
+        _check_axes(axes, x.type.ndim)
+        if epsilon.type.dtype != est_var.type.dtype:
+            epsilon = T.cast(epsilon, est_var.type.dtype)
+        est_var_eps = est_var + epsilon
+        est_std = T.sqrt(est_var_eps)
+        dx = dy * (scale / est_std)
+        dscale = T.sum(dy * (x - est_mean), axis=axes, keepdims=True) / est_std
+        dbias = T.sum(dy, axis=axes, keepdims=True)
+        dmean = -T.sum(dy, axis=axes, keepdims=True) * (scale / est_std)
+        dvar = -T.sum(dy * (x - est_mean), axis=axes, keepdims=True) * (scale / (2.0 * est_var_eps * est_std))
+        return [dx, dscale, dbias, dmean, dvar, scal.DisconnectedType()()]
+
+    def lower(self, x, scale, bias, estimated_mean, estimated_variance, epsilon):
+        # local_abstract_batch_norm_inference, bn.py:765-789
+        if epsilon.type.dtype != estimated_variance.type.dtype:
+            epsilon = T.cast(epsilon, estimated_variance.type.dtype)
+        return [(x - estimated_mean) * (scale / T.sqrt(estimated_variance + epsilon)) + bias]
+
+
+class AbstractBatchNormTrainGrad(Op):
+    """Gradients of training-mode batch normalization with respect to the inputs, the
+    scale and the bias, from the saved mean and inverse standard deviation
+    (``theano/tensor/nnet/bn.py:575-676``)."""
+
+    __props__ = ("axes",)
+
+    def __init__(self, axes=(0,)):
+        assert isinstance(axes, (tuple, list)) and len(axes) > 0
+        self.axes = tuple(int(a) for a in axes)
+
+    def _props(self):
+        return (self.axes,)
+
+    def make_node(self, x, dy, scale, x_mean, x_invstd, epsilon=1e-4):
+        vs = [as_tensor_variable(v) for v in (x, dy, scale, x_mean, x_invstd)]
+        epsilon = as_tensor_variable(epsilon)
+        vs = _as_common_dtype(*vs)
+        assert len(set(v.type.ndim for v in vs)) == 1
+        return Apply(self, vs + [epsilon], [vs[0].type(), vs[2].type(), vs[2].type()])
+
+    def infer_shape(self, node, shapes):
+        return [shapes[0], shapes[2], shapes[2]]
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def connection_pattern(self, node):
+        return [[True, True, False], [True, True, True], [True, False, False], [True, True, False],
+                [True, True, False], [False, False, False]]
+
+    def L_op(self, inputs, outputs, grads):
+        # second derivatives, bn.py:601-650
+        x, dy, scale, x_mean, x_invstd, epsilon = inputs
+        ddinputs, ddscale, ddbias = grads
+        axes = self.axes
+        disc = lambda g: isinstance(g.type, scal.DisconnectedType)   # noqa: E731
+        mean = lambda v: T.mean(v, axis=axes, keepdims=True)         # noqa: E731
+        total = lambda v: T.sum(v, axis=axes, keepdims=True)         # noqa: E731
+        x_diff = x - x_mean
+        mean_dy_x_diff = mean(dy * x_diff)
+        acc = {"x": None, "dy": None, "scale": None, "mean": None, "invstd": None}
+
+        def add(key, term, sign=1):
+            term = term if sign > 0 else -term
+            acc[key] = term if acc[key] is None else acc[key] + term
+
+        if not disc(ddinputs):
+            ccc = scale * (ddinputs - mean(ddinputs))
+            ddd = (x_invstd ** 3) * (ccc * mean(dy * x_diff) + dy * mean(ccc * x_diff))
+            add("x", ddd, -1)
+            add("dy", (ccc * x_invstd) - ((x_invstd ** 3) * x_diff * mean(ccc * x_diff)))
+            eee = (dy * x_invstd) - ((x_invstd ** 3) * x_diff * mean_dy_x_diff)
+            add("scale", total(ddinputs * (eee - mean(eee))))
+            add("mean", total(ddd))
+            add("invstd", total(ccc * (dy - 3 * (x_invstd ** 2) * x_diff * mean_dy_x_diff)))
+        if not disc(ddscale):
+            add("x", x_invstd * ddscale * dy)
+            add("dy", x_invstd * ddscale * x_diff)
+            add("mean", x_invstd * ddscale * total(dy), -1)
+            add("invstd", ddscale * total(dy * x_diff))
+        if not disc(ddbias):
+            add("dy", T.second(dy, ddbias))
+        res = [acc[k] for k in ("x", "dy", "scale", "mean", "invstd")]
+        return [scal.DisconnectedType()() if r is None else r for r in res] + [scal.DisconnectedType()()]
+
+    def lower(self, x, dy, scale, x_mean, x_invstd, epsilon):
+        # local_abstract_batch_norm_train_grad, bn.py:730-761
+        axes = self.axes
+        _check_axes(axes, x.type.ndim)
+        x_diff = x - x_mean
+        mean_dy_x_diff = T.mean(dy * x_diff, axis=axes, keepdims=True)
+        c = (dy * x_invstd) - x_diff * (mean_dy_x_diff * (x_invstd ** 3))
+        return [scale * (c - T.mean(c, axis=axes, keepdims=True)),
+                T.sum(dy * x_invstd * x_diff, axis=axes, keepdims=True), T.sum(dy, axis=axes, keepdims=True)]
+
+
+def _bn_params(ndim, axes, params, names):
+    """Parameters given with the input's rank must be broadcastable along ``axes``; given
+    with one dimension per non-normalized axis they are padded (bn.py:186-232)."""
+    non_bc = tuple(d for d in range(ndim) if d not in axes)
+    params = [as_tensor_variable(p) for p in params]
+    nd0 = params[0].type.ndim
+    if nd0 not in (ndim, len(non_bc)) or any(p.type.ndim != nd0 for p in params):
+        raise ValueError("%s dimensionality must match the number of non-normalized axes, or have the same "
+                         "number of dimensions as the inputs; got %s instead of %d"
+                         % (" and ".join(names), [p.type.ndim for p in params], len(non_bc)))
+    if nd0 == ndim:
+        for p, n in zip(params, names):
+            if not all(p.type.broadcastable[a] for a in axes):
+                raise TypeError("%s must be broadcastable along the normalized axes %s" % (n, axes))
+        return params, None
+    pattern = ["x"] * ndim
+    for i, a in enumerate(non_bc):
+        pattern[a] = i
+    return [p.dimshuffle(*pattern) for p in params], non_bc
+
+
 def batch_normalization_train(inputs, gamma, beta, axes="per-activation", epsilon=1e-4,
                               running_average_factor=0.1, running_mean=None, running_var=None):
-    """Training-mode batch normalization as the graph the reference lowers
-    ``AbstractBatchNormTrain`` to (``local_abstract_batch_norm_train``,
-    ``theano/tensor/nnet/bn.py:679-726``): ``mean`` and two-pass ``var`` over
-    ``axes`` (keepdims), ``invstd = inv(sqrt(var + eps))``,
-    ``out = (x - mean) * (gamma * invstd) + beta``.  ``gamma`` / ``beta`` (and
-    the running statistics) have the input's rank with extent 1 along ``axes``.
-    Returns ``(out, mean, invstd)`` plus the updated running mean and variance
-    when those are given."""
+    """Training-mode batch normalization (``theano/tensor/nnet/bn.py:79-263``): an
+    ``AbstractBatchNormTrain`` node.  Returns ``(out, mean, invstd)`` plus the updated
+    running mean and variance when those are given.  ``gamma`` / ``beta`` (and the running
+    statistics) have the input's rank with broadcastable extent 1 along ``axes``, or one
+    dimension per remaining axis."""
     x = as_tensor_variable(inputs)
-    gamma, beta = as_tensor_variable(gamma), as_tensor_variable(beta)
     axes = _bn_axes(axes, x.type.ndim)
-    mean = T.mean(x, axis=axes, keepdims=True)
-    var = T.var(x, axis=axes, keepdims=True)
-    eps = T.cast(as_tensor_variable(epsilon), var.type.dtype)
-    invstd = T.inv(T.sqrt(var + eps))
-    out = (x - mean) * (gamma * invstd) + beta
-    results = [out, mean, invstd]
-    if running_mean is not None:
-        running_mean = as_tensor_variable(running_mean)
-        results.append(running_mean * (1.0 - running_average_factor) + mean * running_average_factor)
-    if running_var is not None:
-        running_var = as_tensor_variable(running_var)
-        m = None
-        for a in axes:                                   # elements per statistic
-            e = T.ShapeFloat(a, var.type.dtype)(x)
-            m = e if m is None else m * e
-        results.append(running_var * (1.0 - running_average_factor) + (m / (m - 1)) * var * running_average_factor)
+    if (running_mean is None) != (running_var is None):
+        raise ValueError("running_mean and running_var must either both be given or both be None")
+    import numpy as np
+    if np.asarray(epsilon, dtype=T.config.floatX) < 1e-5:
+        raise ValueError("epsilon must be at least 1e-5, got %s" % str(epsilon))
+    names = ["gamma", "beta"] + (["running_mean", "running_var"] if running_mean is not None else [])
+    given = [gamma, beta] + ([running_mean, running_var] if running_mean is not None else [])
+    params, non_bc = _bn_params(x.type.ndim, axes, given, names)
+    op = AbstractBatchNormTrain(axes)
+    eps = np.asarray(epsilon, dtype=T.config.floatX)
+    results = op(x, params[0], params[1], eps, running_average_factor, *params[2:], return_list=True)
+    if non_bc is not None:
+        results = [results[0]] + [r.dimshuffle(*non_bc) for r in results[1:]]
     return tuple(results)
 
 
-def batch_normalization_train_grad(x, dy, scale, x_mean, x_invstd, axes="per-activation"):
-    """The graph ``AbstractBatchNormTrainGrad`` lowers to
-    (``theano/tensor/nnet/bn.py:730-761``): gradients with respect to the inputs,
-    the scale and the bias, given the saved mean and inverse standard deviation."""
-    x, dy = as_tensor_variable(x), as_tensor_variable(dy)
+def batch_normalization_train_grad(x, dy, scale, x_mean, x_invstd, axes="per-activation", epsilon=1e-4):
+    """An ``AbstractBatchNormTrainGrad`` node: gradients with respect to the inputs, the
+    scale and the bias, given the saved mean and inverse standard deviation."""
+    x = as_tensor_variable(x)
     axes = _bn_axes(axes, x.type.ndim)
-    x_diff = x - x_mean
-    mean_dy_x_diff = T.mean(dy * x_diff, axis=axes, keepdims=True)
-    c = (dy * x_invstd) - x_diff * (mean_dy_x_diff * (x_invstd ** 3))
-    g_wrt_inputs = scale * (c - T.mean(c, axis=axes, keepdims=True))
-    g_wrt_scale = T.sum(dy * x_invstd * x_diff, axis=axes, keepdims=True)
-    g_wrt_bias = T.sum(dy, axis=axes, keepdims=True)
-    return g_wrt_inputs, g_wrt_scale, g_wrt_bias
+    return tuple(AbstractBatchNormTrainGrad(axes)(x, dy, scale, x_mean, x_invstd, epsilon, return_list=True))
 
 
 def batch_normalization_test(inputs, gamma, beta, mean, var, axes="per-activation", epsilon=1e-4):
-    """Inference-mode batch normalization (``local_abstract_batch_norm_inference``,
-    ``theano/tensor/nnet/bn.py:765-789``):
-    ``(x - mean) * (gamma / sqrt(var + eps)) + beta``, one elementwise kernel."""
+    """Inference-mode batch normalization (``theano/tensor/nnet/bn.py:266-361``): an
+    ``AbstractBatchNormInference`` node, one elementwise kernel once lowered."""
     x = as_tensor_variable(inputs)
-    var = as_tensor_variable(var)
-    _bn_axes(axes, x.type.ndim)
-    eps = T.cast(as_tensor_variable(epsilon), var.type.dtype)
-    return (x - mean) * (gamma / T.sqrt(var + eps)) + beta
+    axes = _bn_axes(axes, x.type.ndim)
+    import numpy as np
+    if np.asarray(epsilon, dtype=T.config.floatX) < 1e-5:
+        raise ValueError("epsilon must be at least 1e-5, got %s" % str(epsilon))
+    params, _ = _bn_params(x.type.ndim, axes, [gamma, beta, mean, var], ["gamma", "beta", "mean", "var"])
+    return AbstractBatchNormInference(axes)(x, *params, np.asarray(epsilon, dtype=T.config.floatX))
