@@ -535,3 +535,25 @@ def test_abstract_batch_norm_ops_lower_to_the_reference_formulas():
     xv = vals[0]
     assert np.allclose(as_ops[3], vals[4] * 0.75 + xv.mean((0, 2, 3)) * 0.25)
     assert np.allclose(as_ops[4], vals[5] * 0.75 + xv.var((0, 2, 3)) * n_per / (n_per - 1) * 0.25)
+
+
+def test_ops_and_graphs_pickle(dry_run):
+    """Ops pickle by value of their props and compare equal afterwards, graphs keep their
+    structure (the role of theano/misc/pkl_utils.py for this path): every op of the
+    compiled benchmark graphs, and an uncompiled graph with gradients evaluated before
+    and after a round trip."""
+    import pickle
+    import workloads as W
+    from oracle import graph_ref as G
+    for g in (W.c1_graph(), W.c3_graph(), W.c4_graph("all"), W.c5_graph(), W.c2_argmax_graph(1)):
+        for n in th.function(*g).toposort():
+            again = pickle.loads(pickle.dumps(n.op))
+            assert again == n.op and hash(again) == hash(n.op), n.op
+    x = T.fmatrix("x")
+    y = T.sum(T.exp(x) * T.nnet.sigmoid(x) + T.erf(x) % 3, axis=1)
+    z = T.nnet.softmax(x)[:, ::2].reshape((-1,))
+    gx = th.grad(T.sum(y) + T.sum(z * z), x)
+    x2, outs2 = pickle.loads(pickle.dumps((x, [y, z, gx])))
+    v = np.random.default_rng(0).standard_normal((4, 6)).astype("float32")
+    for a, b in zip(G.evaluate([x], [y, z, gx], [v]), G.evaluate([x2], outs2, [v])):
+        assert np.array_equal(a, b)

@@ -425,7 +425,7 @@ def _cmp(name, sym):
     class _C(LogicalComparison):
         def c_code(self, node, inputs, outputs):
             return "%s = (%s %s %s);" % (outputs[0], inputs[0], sym, inputs[1])
-    _C.__name__ = name
+    _C.__name__ = _C.__qualname__ = name      # instances pickle by reference to the module-level name
     _C.commutative = sym in ("==", "!=")
     return _C
 
@@ -933,7 +933,8 @@ def _unary_math(cname, fname, grad_fn, policy=upgrade_to_float):
             if grad_fn is None:
                 return _zero_grads(inputs)
             return [grad_fn(x, outputs[0], gout[0])]
-    _U.__name__ = cname
+    _U.__name__ = _U.__qualname__ = cname
+    globals()[cname] = _U            # importable by name: instances pickle by reference to their class
     return _U(policy, name=fname if fname != "fabs" else "abs")
 
 
