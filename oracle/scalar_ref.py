@@ -213,10 +213,21 @@ def mod_fast(out_dtype, x, y):
 
 
 def int_div_fast(out_dtype, x, y):
+    """Integers: NumPy's ``//`` (floor, zero divisors give 0 as on the device).  Floats follow
+    the C text (``theano/scalar/basic.py:1985-2025``): ``floor(x / y)`` over the magnitudes
+    with the quotient rounded in C's common type first - so a quotient that rounds up to an
+    integer floors to that integer - and the sign cases corrected through ``fmod``."""
     ct = c_common_type(x.dtype, y.dtype)
     a, b = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
     with np.errstate(all="ignore"):
-        r = np.where(b == 0, 0, np.floor_divide(a, np.where(b == 0, 1, b)))
+        if np.dtype(ct).kind == "f":
+            pp = np.floor(a / b)
+            mm = np.floor((-a) / (-b))
+            pm = -np.floor(a / (-b)) - np.where(np.fmod(a, -b) == 0, 0, 1)
+            mp = -np.floor((-a) / b) - np.where(np.fmod(-a, b) == 0, 0, 1)
+            r = np.where(b == 0, pp, np.where(b < 0, np.where(a < 0, mm, pm), np.where(a < 0, mp, pp)))
+        else:
+            r = np.where(b == 0, 0, np.floor_divide(a, np.where(b == 0, 1, b)))
     return _conv(r, out_dtype)
 
 

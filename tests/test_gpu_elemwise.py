@@ -235,3 +235,28 @@ def test_special_functions_against_scipy(dtype):
         ref = G.evaluate([x], outs, [vals])
         for k, (g, r) in enumerate(zip(got, ref)):
             assert_parity(g, r, "%s output %d" % (name, k), tol=tol)
+
+
+@pytest.mark.gpu
+def test_float_floor_division_is_exact_at_integer_quotients():
+    """x // y and x % y on float32 where x is an exact multiple of y: the quotient handed
+    to floor must be the correctly rounded one (an ulp low would lose a whole unit),
+    whatever division the kernels are built with; also int64 // float32, which C evaluates
+    in float32 (theano/scalar/basic.py:1985-2025)."""
+    rng = np.random.default_rng(77)
+    k = rng.integers(-200, 200, 20000).astype("float32")
+    y = (rng.integers(1, 64, 20000) / 8.0).astype("float32") * rng.choice([-1, 1], 20000).astype("float32")
+    x = (k * y).astype("float32")                       # exact: small integers times eighths
+    a, b = T.fvector("a"), T.fvector("b")
+    q, r = th.function([a, b], [a // b, a % b])(x, y)
+    assert np.array_equal(q, k) and np.array_equal(r, np.zeros_like(r))
+    ref = G.evaluate([a, b], [a // b, a % b], [x + 0.25, y])
+    got = th.function([a, b], [a // b, a % b])(x + np.float32(0.25), y)
+    assert np.array_equal(got[0], ref[0]) and np.allclose(got[1], ref[1], rtol=1e-6, atol=1e-6)
+    i, f = T.lvector("i"), T.fvector("f")
+    iv = rng.integers(-1000, 1000, 5000)
+    fv = rng.uniform(0.5, 3.0, 5000).astype("float32")
+    fv[:3], iv[:3] = np.float32(1.96), 49              # 49 / 1.96f rounds to 25.0f
+    got = th.function([i, f], i // f)(iv, fv)
+    assert got.dtype == np.float64 and got[0] == 25.0
+    assert np.array_equal(got, G.evaluate([i, f], [i // f], [iv, fv])[0])

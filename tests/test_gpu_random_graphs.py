@@ -1,0 +1,253 @@
+"""Seeded random graphs through the whole pipeline (rewrites, fusion, planners, kernels)
+against the oracle's node-by-node evaluation: random ranks and extents, operands that
+are broadcast, of lower rank, transposed or strided views, chains of elementwise ops,
+then reductions over random axes with siblings and epilogues.  The generator is
+deterministic; a failure names its seed.
+
+``test_generator_builds_valid_graphs`` runs the same graphs on the CPU in dry-run mode
+(rewrites, planning and kernel compilation, no execution)."""
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import tensor as T
+from oracle import graph_ref as G
+from conftest import assert_parity
+
+EXTENTS = [1, 2, 3, 5, 7, 8, 16, 33, 64]
+
+FLOAT_UNARY = [T.tanh, T.sigmoid, T.sin, T.cos, abs, T.sqr, T.neg, lambda v: T.exp(T.minimum(v, 3.0)),
+               lambda v: T.sqrt(abs(v) + 0.5), lambda v: T.log(abs(v) + 1.0)]
+FLOAT_BINARY = [T.add, T.sub, T.mul, T.maximum, T.minimum, lambda a, b: a / (abs(b) + 1.0),
+                lambda a, b: T.switch(T.gt(a, b), a, b * 0.5), lambda a, b: T.switch(T.le(a, 0.1), b, a)]
+INT_UNARY = [abs, T.neg, lambda v: v % 7, lambda v: v // 3, lambda v: ~v, lambda v: T.right_shift(v, 2)]
+INT_BINARY = [T.add, T.sub, T.mul, T.maximum, T.minimum, lambda a, b: a & b, lambda a, b: a | b, lambda a, b: a ^ b,
+              lambda a, b: T.switch(T.gt(a, b), a, b)]
+
+
+def make_input(rng, k, shape, dtype):
+    """A term of the full rank (or lower) built from a fresh input variable through views:
+    (variable, value, term)."""
+    nd = len(shape)
+    bc = [bool(rng.random() < 0.25) for _ in range(nd)]
+    if all(bc) and nd:
+        bc[int(rng.integers(nd))] = False
+    ishape = [1 if b else s for b, s in zip(bc, shape)]
+    lead = 0
+    while lead < nd - 1 and ishape[lead] == 1 and rng.random() < 0.5:      # lower rank: padded on the left
+        lead += 1
+    ishape, bc = ishape[lead:], bc[lead:]
+    r = len(ishape)
+    perm = list(rng.permutation(r)) if r > 1 and rng.random() < 0.4 else list(range(r))
+    src_shape = [ishape[p] for p in perm]
+    src_bc = [bc[p] for p in perm]
+    step_dim = int(rng.integers(r)) if r and rng.random() < 0.3 else None
+    if step_dim is not None and src_bc[step_dim]:
+        step_dim = None
+    alloc = list(src_shape)
+    if step_dim is not None:
+        alloc[step_dim] = 2 * alloc[step_dim] + 1
+    var = T.TensorType(dtype, tuple(src_bc))("in%d" % k)
+    if dtype.startswith("float"):
+        val = rng.uniform(-2, 2, alloc).astype(dtype)
+    elif dtype == "bool":
+        val = rng.random(alloc) < 0.5
+    else:
+        val = rng.integers(-50, 50, alloc).astype(dtype)
+    term = var
+    if step_dim is not None:
+        term = term[tuple(slice(1, None, 2) if d == step_dim else slice(None) for d in range(r))]
+    if perm != list(range(r)):
+        inv = [perm.index(d) for d in range(r)]
+        term = term.dimshuffle(*inv)
+    return var, val, term
+
+
+def random_graph(seed):
+    rng = np.random.default_rng(seed)
+    dtype = str(rng.choice(["float32", "float32", "float64", "int32", "int16", "int64"]))
+    nd = int(rng.integers(1, 5))
+    shape = [int(rng.choice(EXTENTS)) for _ in range(nd)]
+    while np.prod(shape) > 150000:
+        shape[int(np.argmax(shape))] //= 2
+    floating = dtype.startswith("float")
+    unary, binary = (FLOAT_UNARY, FLOAT_BINARY) if floating else (INT_UNARY, INT_BINARY)
+    ins, vals, terms = [], [], []
+    for k in range(int(rng.integers(1, 5))):
+        v, val, t = make_input(rng, k, shape, dtype)
+        ins.append(v)
+        vals.append(val)
+        terms.append(t)
+    # one term of the full shape, so that the result has it whatever the others broadcast
+    full = T.TensorType(dtype, (False,) * nd)("full")
+    ins.append(full)
+    vals.append((np.random.default_rng(seed + 1).uniform(-2, 2, shape).astype(dtype) if floating else
+                 np.random.default_rng(seed + 1).integers(-50, 50, shape).astype(dtype)))
+    terms.append(full)
+    for _ in range(int(rng.integers(2, 8))):
+        if rng.random() < 0.4:
+            a = terms[int(rng.integers(len(terms)))]
+            terms.append(unary[int(rng.integers(len(unary)))](a))
+        else:
+            a = terms[int(rng.integers(len(terms)))]
+            b = terms[int(rng.integers(len(terms)))]
+            terms.append(binary[int(rng.integers(len(binary)))](a, b))
+    e = terms[-1] + full if terms[-1].type.ndim < nd or any(terms[-1].type.broadcastable) else terms[-1]
+    outs = []
+    mode = int(rng.integers(4))
+    axes = sorted(set(int(a) for a in rng.integers(0, nd, int(rng.integers(1, nd + 1)))))
+    axis = None if rng.random() < 0.2 else tuple(axes)
+    if mode == 0:
+        outs.append(e)
+    elif mode == 1:
+        red = [T.sum, T.max, T.min][int(rng.integers(3))]
+        outs.append(red(e, axis=axis))
+    elif mode == 2:                                  # siblings over the same axes, one with an epilogue
+        keep = bool(rng.random() < 0.5)
+        s = T.sum(e, axis=axis, keepdims=keep)
+        m = T.max(e, axis=axis, keepdims=keep)
+        outs += [s, m, (T.cast(s, "float32") * 0.5 + 1.0) if not floating else s * 0.5 + m]
+    else:                                            # a reduction fed back into the elementwise result
+        if floating:
+            outs.append(e - T.mean(e, axis=axis, keepdims=True))
+            outs.append(T.prod(T.tanh(e) * 0.5 + 1.0, axis=axis))
+        else:
+            outs.append(e - T.max(e, axis=axis, keepdims=True))
+            outs.append(T.any(T.gt(e, 40), axis=axis))
+            outs.append(T.all(T.lt(e, 1000), axis=axis))
+    return ins, outs, vals
+
+
+def random_mixed_graph(seed):
+    """Mixed input dtypes within one family (C promotion rules decide the rest), casts,
+    integer division and modulo with both signs, comparisons feeding arithmetic, and the
+    callers around the path: max_and_argmax, mean / var / std, softmax, reshape, join,
+    set / inc_subtensor."""
+    rng = np.random.default_rng(seed)
+    floating = bool(rng.random() < 0.5)
+    family = ["float16", "float32", "float32", "float64"] if floating else ["bool", "int8", "uint8", "int16", "int32", "int64"]
+    nd = int(rng.integers(1, 4))
+    shape = [int(rng.choice(EXTENTS[1:])) for _ in range(nd)]
+    ins, vals, terms = [], [], []
+    for k in range(int(rng.integers(2, 5))):
+        dt = str(rng.choice(family))
+        v, val, t = make_input(rng, k, shape, dt)
+        ins.append(v)
+        vals.append(val)
+        terms.append(t)
+    dt = str(rng.choice(family[1:]))
+    full = T.TensorType(dt, (False,) * nd)("full")
+    ins.append(full)
+    vals.append(np.random.default_rng(seed + 1).uniform(-2, 2, shape).astype(dt) if floating else
+                np.random.default_rng(seed + 1).integers(-50, 50, shape).astype(dt))
+    terms.append(full)
+    if floating:
+        unary = FLOAT_UNARY + [lambda v: T.cast(v, "float32"), lambda v: T.cast(T.gt(v, 0.0), "float32") * v,
+                               T.floor, T.round_half_to_even, lambda v: T.clip(v, -1.0, 1.5)]
+        binary = FLOAT_BINARY + [lambda a, b: T.pow(abs(a) + 0.5, T.clip(b, -2.0, 2.0)), lambda a, b: T.mod(a, abs(b) + 0.5)]
+    else:
+        unary = INT_UNARY + [lambda v: T.cast(v, "int32"), lambda v: T.cast(v, "int8"), lambda v: T.cast(T.gt(v, 3), "int16") + v,
+                             lambda v: T.sgn(v)]
+        binary = INT_BINARY[:5] + [lambda a, b: T.int_div(a, abs(b) + 1), lambda a, b: T.int_div(a, -(abs(b) + 1)),
+                                   lambda a, b: T.mod(a, abs(b) + 1), lambda a, b: T.mod(a, -(abs(b) + 1)),
+                                   lambda a, b: T.true_div(a, abs(b) + 1), lambda a, b: T.eq(a, b) + T.cast(a, "int32")]
+    for _ in range(int(rng.integers(2, 7))):
+        a = terms[int(rng.integers(len(terms)))]
+        if rng.random() < 0.4:
+            try:
+                terms.append(unary[int(rng.integers(len(unary)))](a))
+            except TypeError:          # e.g. ~ of a float produced by true_div, - of a bool
+                continue
+        else:
+            b = terms[int(rng.integers(len(terms)))]
+            try:
+                terms.append(binary[int(rng.integers(len(binary)))](a, b))
+            except TypeError:
+                continue
+    e = terms[-1]
+    if e.type.ndim < nd or any(e.type.broadcastable) or e.type.dtype == "bool":
+        e = e + full
+    fl = e.type.dtype.startswith("float")
+    axis = int(rng.integers(nd))
+    mode = int(rng.integers(6))
+    if mode == 0:
+        outs = list(T.max_and_argmax(e, axis=axis)) + [T.argmin(e, axis=None if nd > 1 and rng.random() < 0.3 else axis)]
+        if e.type.dtype in ("int8", "bool", "uint8"):     # argmin negates: wraps for the smallest int8 as in the reference
+            outs = outs[:2]
+    elif mode == 1:
+        ef = e if fl else T.cast(e, "float32")
+        outs = [T.mean(ef, axis=axis), T.var(ef, axis=axis, keepdims=True), T.std(ef)]
+    elif mode == 2:
+        ef = e if fl else T.cast(e, "float64")
+        m = ef.reshape((-1, shape[-1])) if nd > 1 else ef.reshape((1, -1))
+        sm = T.nnet.softmax(m)
+        outs = [sm, T.nnet.logsoftmax(m), th.grad(T.sum(sm * sm), m)] if ef.type.dtype != "float16" else [sm]
+    elif mode == 3:
+        outs = [T.join(axis, e, e * 2), T.stack([e, -e] if e.type.dtype != "uint8" else [e, e]), e.flatten()]
+    elif mode == 4:
+        idx = tuple(slice(0, None, 2) if d == axis else slice(None) for d in range(nd))
+        outs = [T.inc_subtensor(e[idx], e[idx]), T.set_subtensor(e[idx], T.zeros_like(e[idx])), T.sum(e[idx], axis=axis)]
+    else:
+        outs = [T.sum(e, axis=axis), T.prod(T.cast(T.gt(e, 0), "int8") + 1, axis=axis), T.any(e, axis=axis), T.all(e)]
+    return ins, outs, vals
+
+
+SEEDS = list(range(100, 180))
+MIXED_SEEDS = list(range(500, 580))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", SEEDS)
+def test_random_graph_matches_the_oracle(seed):
+    ins, outs, vals = random_graph(seed)
+    with np.errstate(all="ignore"):
+        ref = G.evaluate(ins, outs, vals)
+    got = th.function(ins, outs, on_unused_input="ignore")(*vals)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "seed %d output %d" % (seed, k))
+
+
+def check_mixed(seed, **flags):
+    from conftest import TOL
+    ins, outs, vals = random_mixed_graph(seed)
+    with np.errstate(all="ignore"):
+        ref = G.evaluate(ins, outs, vals)
+    got = th.function(ins, outs, on_unused_input="ignore", **flags)(*vals)
+    # the narrowest floating type anywhere upstream leaves its rounding in wider results
+    from theano_amd import gof
+    seen = set(v.type.dtype for v in ins)
+    for n in gof.io_toposort(ins, outs):
+        seen.update(o.type.dtype for o in n.outputs)
+    narrowest = [d for d in ("float16", "float32", "float64") if d in seen]
+    for k, (g, r) in enumerate(zip(got, ref)):
+        tol = TOL[narrowest[0]] if narrowest and r.dtype.kind == "f" else None
+        assert_parity(g, r, "seed %d output %d" % (seed, k), tol=tol)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", MIXED_SEEDS)
+def test_random_mixed_graph_matches_the_oracle(seed):
+    check_mixed(seed)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", MIXED_SEEDS[:30])
+def test_random_mixed_graph_without_fusion_and_in_place(seed):
+    check_mixed(seed, fuse=False)
+
+
+def test_generator_builds_valid_graphs(dry_run):
+    for seed in MIXED_SEEDS[:12]:
+        ins, outs, vals = random_mixed_graph(seed)
+        with np.errstate(all="ignore"):
+            ref = G.evaluate(ins, outs, vals)
+        got = th.function(ins, outs, on_unused_input="ignore")(*vals)
+        assert [g.shape for g in got] == [r.shape for r in ref], seed
+        assert [g.dtype for g in got] == [r.dtype for r in ref], seed
+    for seed in SEEDS[:12]:
+        ins, outs, vals = random_graph(seed)
+        with np.errstate(all="ignore"):
+            ref = G.evaluate(ins, outs, vals)
+        got = th.function(ins, outs, on_unused_input="ignore")(*vals)
+        assert [g.shape for g in got] == [r.shape for r in ref], seed
+        assert [g.dtype for g in got] == [r.dtype for r in ref], seed

@@ -198,3 +198,19 @@ def test_prod_gradient_with_zeros_and_prod_without_zeros():
             group = xv[:, idx[1]] if axis == 0 else xv[idx[0], :]
             want[idx] = np.prod(np.delete(group, idx[axis]))
         assert np.allclose(got[0], want, rtol=1e-10)
+
+
+@pytest.mark.gpu
+def test_epilogue_operand_that_is_a_strided_view():
+    """A per-result operand of a fused epilogue may be any view (every other element of a
+    vector, a column of a matrix): the epilogue reads it at the result's index."""
+    rng = np.random.default_rng(8)
+    x, m = T.fmatrix("x"), T.fmatrix("m")
+    v = T.fvector("v")
+    outs = [T.sum(x, axis=1) * v[1::2] + m[:, 2], T.max(x, axis=0) / (abs(m.T[1]) + 1.0)]
+    xv = rng.standard_normal((37, 37)).astype("float32")
+    vals = [xv, rng.standard_normal((37, 5)).astype("float32"), rng.standard_normal(75).astype("float32")]
+    f = th.function([x, m, v], outs)
+    assert not any(type(n.op).__name__ == "HipElemwise" for n in f.toposort())     # both are epilogues
+    for g, r in zip(f(*vals), G.evaluate([x, m, v], outs, vals)):
+        assert_parity(g, r, "strided epilogue operand")

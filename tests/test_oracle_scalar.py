@@ -112,3 +112,34 @@ def test_product_dtype_tables_against_reference_literals():
     # upcast follows NumPy array promotion
     for a, b in itertools.product(scal.all_dtypes, repeat=2):
         assert scal.upcast(a, b) == str((np.zeros((), a) + np.zeros((), b)).dtype)
+
+
+def test_float_int_div_follows_the_c_text():
+    """IntDiv on floats is ``floor(x / y)`` over magnitudes with sign corrections
+    (theano/scalar/basic.py:1985-2025), the quotient rounded in C's common type before
+    the floor: equal to Python's ``//`` except where that rounding reaches an integer
+    (49 / float32(1.96) rounds to 25.0f, the exact quotient is 24.9999995)."""
+    rng = np.random.default_rng(2)
+    for dt in ("float32", "float64"):
+        a = rng.uniform(-50, 50, 20000).astype(dt)
+        b = rng.uniform(-7, 7, 20000).astype(dt)
+        got = S.int_div_fast(dt, a, b)
+        exact = np.floor(a.astype("float64") / b.astype("float64"))
+        frac = np.abs(a.astype("float64") / b.astype("float64") - np.round(a.astype("float64") / b.astype("float64")))
+        away = frac > 1e-4                       # away from integers rounding cannot matter
+        assert away.sum() > 19000 and np.array_equal(got[away], exact[away].astype(dt))
+        # scalar transcription of the four sign cases on every element
+        for x, y, z in zip(a[:500], b[:500], got[:500]):
+            T_ = np.dtype(dt).type
+            q = lambda p, r: np.floor(T_(p) / T_(r))           # noqa: E731
+            if y < 0:
+                want = q(-x, -y) if x < 0 else -q(x, -y) - (0 if np.fmod(T_(x), T_(-y)) == 0 else 1)
+            else:
+                want = -q(-x, y) - (0 if np.fmod(T_(-x), T_(y)) == 0 else 1) if x < 0 else q(x, y)
+            assert z == want
+    knife = S.int_div_fast("float64", np.asarray([49], "int64"), np.asarray([1.96], "float32"))
+    assert knife.dtype == np.float64 and knife[0] == 25.0     # int64 / float32 is a float32 division in C
+    assert S.int_div_fast("float64", np.asarray([49.0]), np.asarray([1.96]))[0] == 25.0   # 49 / 1.96 == 25.0 in double too
+    assert S.int_div_fast("float64", np.asarray([49.0]), np.asarray([np.float32(1.96)], "float64"))[0] == 24.0
+    assert np.array_equal(S.int_div_fast("float32", np.asarray([7.5, -7.5, 7.5, -7.5], "float32"),
+                                         np.asarray([2, 2, -2, -2], "float32")), [3, -4, -4, 3])

@@ -44,6 +44,15 @@ __device__ __forceinline__ float thx_fdiv(float a, float b) {
 __device__ __forceinline__ float thx_fdiv(float a, float b) { return a / b; }
 #endif
 
+// x / y in the type C gives the quotient, correctly rounded even when single-precision division
+// is built in its 2.5-ulp form: a double quotient rounded to float is the correctly rounded float
+// quotient (53 >= 2 * 24 + 2 bits).
+template <class A, class B>
+__device__ __forceinline__ auto thx_exact_div(A a, B b) -> decltype(a / b) {
+  typedef decltype(a / b) R;
+  return (R)((double)a / (double)b);
+}
+
 // Digamma and trigamma (the reference ships its own C for both, theano/scalar/basic_scipy.py:
 // 340-391, 430-470): arguments below 10 are moved up with psi(x) = psi(x + 1) - 1/x and
 // psi'(x) = psi'(x + 1) + 1/x^2, negative ones first reflected to 1 - x, then the asymptotic

@@ -448,14 +448,18 @@ class HipCAReduce(CAReduce):
             for op in self.scalar_ops:
                 if codegen.reduce_identity(op, "float32") is None or isinstance(op, (scal.Maximum, scal.Minimum)):
                     raise ValueError("Input of CAReduce{%s} has zero-size on axis %s" % (op, axis))
-        for k, v in enumerate(inputs):
-            _operand(v, nd, ins[k])
         kept = tuple(shape[d] for d in range(nd) if d not in axis)
         for k in range(nin, len(inputs)):
             v = inputs[k]
-            if type(v) is HipArray and [d for d in v.shape if d != 1] != [d for d in kept if d != 1]:
-                raise ValueError("Input dimension mis-match. (epilogue operand %d has shape %s, the result has %s)"
-                                 % (k - nin, v.shape, kept))
+            if type(v) is HipArray:
+                if [d for d in v.shape if d != 1] != [d for d in kept if d != 1]:
+                    raise ValueError("Input dimension mis-match. (epilogue operand %d has shape %s, the result has %s)"
+                                     % (k - nin, v.shape, kept))
+                if not v.c_contiguous:          # the epilogue reads one value per result at the result's index
+                    inputs = list(inputs)
+                    inputs[k] = v.copy()
+        for k, v in enumerate(inputs):
+            _operand(v, nd, ins[k])
         results = []
         for k in range(nout):
             arr = HipArray._new_contiguous(kept, out_dt[k])

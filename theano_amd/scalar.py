@@ -714,8 +714,10 @@ class IntDiv(BinaryScalarOp):
             m = lambda a, b: "(%s %% %s)" % (a, b)
             zero = "%s = 0;" % z
         else:
+            # the quotient must be the correctly rounded one whatever division the kernels are
+            # built with: floor() of a quotient that is an ulp low loses a whole unit
             fl, fm = _fn("floor", t), _fn("fmod", t)
-            d = lambda a, b: "%s(%s / %s)" % (fl, a, b)
+            d = lambda a, b: "%s(thx_exact_div(%s, %s))" % (fl, a, b)
             m = lambda a, b: "%s(%s, %s)" % (fm, a, b)
             zero = "%s = %s;" % (z, d(x, y))
         nx, ny = "(-%s)" % x, "(-%s)" % y
