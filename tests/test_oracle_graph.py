@@ -369,3 +369,52 @@ def test_parallel_reduce_variant_agrees_with_the_serial_loops(which):
         assert np.allclose(got, want, rtol=1e-6)
     else:
         assert np.array_equal(got, want)
+
+
+UNARY_GRAD_CASES = [
+    ("exp", -2, 2), ("exp2", -2, 2), ("expm1", -1, 1), ("log", 0.5, 3), ("log2", 0.5, 3), ("log10", 0.5, 3),
+    ("log1p", -0.5, 2), ("sqrt", 0.5, 3), ("sqr", -2, 2), ("neg", -2, 2), ("inv", 0.5, 2), ("abs_", 0.2, 2),
+    ("sin", -2, 2), ("cos", -2, 2), ("tan", -1, 1), ("arcsin", -0.9, 0.9), ("arccos", -0.9, 0.9), ("arctan", -2, 2),
+    ("sinh", -2, 2), ("cosh", -2, 2), ("tanh", -2, 2), ("arcsinh", -2, 2), ("arccosh", 1.5, 3), ("arctanh", -0.9, 0.9),
+    ("sigmoid", -3, 3), ("softplus", -3, 3), ("erf", -2, 2), ("erfc", -2, 2), ("erfcx", -1, 2), ("erfinv", -0.9, 0.9),
+    ("erfcinv", 0.1, 1.9), ("gamma", 0.5, 3), ("gammaln", 0.5, 3), ("psi", 0.5, 3),
+]
+BINARY_GRAD_CASES = [
+    ("add", -2, 2, -2, 2), ("sub", -2, 2, -2, 2), ("mul", -2, 2, -2, 2), ("true_div", -2, 2, 0.5, 2),
+    ("pow", 0.5, 2, -2, 2), ("maximum", -2, 2, -2, 2), ("minimum", -2, 2, -2, 2), ("arctan2", -2, 2, 0.5, 2),
+    ("mod", 0.1, 5, 0.7, 2),
+]
+
+
+@pytest.mark.parametrize("case", UNARY_GRAD_CASES + BINARY_GRAD_CASES, ids=lambda c: c[0])
+def test_scalar_op_gradients_against_finite_differences(case):
+    """Every differentiable ScalarOp's L_op (theano/scalar/basic.py, basic_scipy.py), lifted to
+    tensors by Elemwise._bgrad, against central differences of the oracle's forward values."""
+    from theano_amd.gradient import numeric_grad
+    rng = np.random.default_rng(sum(ord(ch) for ch in case[0]))
+    op = getattr(T, case[0])
+    n_in = (len(case) - 1) // 2
+    xs = [T.dvector("x%d" % k) for k in range(n_in)]
+    w = rng.uniform(0.5, 1.5, 7)
+    cost = T.sum(op(*xs) * w)
+    grads = th.grad(cost, xs)
+    vals = [rng.uniform(case[1 + 2 * k], case[2 + 2 * k], 7) for k in range(n_in)]
+    if case[0] == "mod":                 # keep away from the jumps
+        vals[0] = vals[1] * (np.floor(vals[0] / vals[1]) + rng.uniform(0.2, 0.8, 7))
+    num = numeric_grad(lambda *a: float(G.evaluate(xs, [cost], list(a))[0]), vals)
+    ana = G.evaluate(xs, grads, vals)
+    for a, n in zip(ana, num):
+        assert np.allclose(a, n, rtol=2e-5, atol=1e-7), (case[0], a, n)
+
+
+def test_clip_and_switch_gradients():
+    from theano_amd.gradient import numeric_grad
+    rng = np.random.default_rng(4)
+    x, lo, hi = T.dvector("x"), T.dvector("lo"), T.dvector("hi")
+    cost = T.sum(T.clip(x, lo, hi) * 1.5 + T.switch(T.gt(x, 0.3), T.sqr(x), -hi))
+    grads = th.grad(cost, [x, lo, hi])
+    vals = [rng.uniform(-2, 2, 40), rng.uniform(-1.5, -0.5, 40), rng.uniform(0.5, 1.5, 40)]
+    vals[0][np.abs(vals[0] - 0.3) < 0.01] += 0.05
+    num = numeric_grad(lambda *a: float(G.evaluate([x, lo, hi], [cost], list(a))[0]), vals)
+    for a, n in zip(G.evaluate([x, lo, hi], grads, vals), num):
+        assert np.allclose(a, n, rtol=2e-5, atol=1e-7)
