@@ -94,7 +94,7 @@ def random_graph(seed):
             terms.append(binary[int(rng.integers(len(binary)))](a, b))
     e = terms[-1] + full if terms[-1].type.ndim < nd or any(terms[-1].type.broadcastable) else terms[-1]
     outs = []
-    mode = int(rng.integers(4))
+    mode = int(rng.integers(5 if floating else 4))
     axes = sorted(set(int(a) for a in rng.integers(0, nd, int(rng.integers(1, nd + 1)))))
     axis = None if rng.random() < 0.2 else tuple(axes)
     if mode == 0:
@@ -107,6 +107,11 @@ def random_graph(seed):
         s = T.sum(e, axis=axis, keepdims=keep)
         m = T.max(e, axis=axis, keepdims=keep)
         outs += [s, m, (T.cast(s, "float32") * 0.5 + 1.0) if not floating else s * 0.5 + m]
+    elif mode == 4:                                  # reverse mode through the chain, broadcast inputs included
+        cost = T.sum(e * e) + T.sum(T.max(e, axis=axis))
+        used = set(id(v) for v in th.gof.graph_inputs([cost]))
+        wrt = [v for v in ins if id(v) in used]
+        outs += [cost] + th.grad(cost, wrt)
     else:                                            # a reduction fed back into the elementwise result
         if floating:
             outs.append(e - T.mean(e, axis=axis, keepdims=True))
@@ -192,7 +197,7 @@ def random_mixed_graph(seed):
     return ins, outs, vals
 
 
-SEEDS = list(range(100, 180))
+SEEDS = list(range(100, 200))
 MIXED_SEEDS = list(range(500, 580))
 
 

@@ -214,3 +214,21 @@ def test_epilogue_operand_that_is_a_strided_view():
     assert not any(type(n.op).__name__ == "HipElemwise" for n in f.toposort())     # both are epilogues
     for g, r in zip(f(*vals), G.evaluate([x, m, v], outs, vals)):
         assert_parity(g, r, "strided epilogue operand")
+
+
+@pytest.mark.gpu
+def test_transposed_reduction_result_is_not_fused_as_an_epilogue():
+    """sum(x, 1).dimshuffle(2, 'x', 1, 0) * y: the consumer works in a transposed layout, so
+    y is not a per-result operand of the reduction (with equal extents a shape check could
+    not tell); only DimShuffles that insert or drop broadcast dimensions sit between a
+    reduction and its epilogue."""
+    rng = np.random.default_rng(10)
+    x = T.TensorType("float32", (False,) * 4)("x")
+    y = T.TensorType("float32", (False, True, False, False))("y")
+    r = T.sum(x, axis=1)
+    outs = [r.dimshuffle(2, "x", 1, 0) * y, r.dimshuffle(0, "x", 1, 2) * y]
+    vals = [rng.standard_normal((5, 3, 5, 5)).astype("float32"), rng.standard_normal((5, 1, 5, 5)).astype("float32")]
+    for g, w in zip(th.function([x, y], outs)(*vals), G.evaluate([x, y], outs, vals)):
+        assert_parity(g, w, "transposed consumer of a reduction")
+    f = th.function([x, y], outs[1:])
+    assert not any(type(n.op).__name__ == "HipElemwise" for n in f.toposort())      # this one is an epilogue

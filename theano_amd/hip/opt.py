@@ -454,6 +454,11 @@ def _try_epilogue(fgraph, red, cand):
     if ds_op is not None and seen_direct:
         return False
     if ds_op is not None:
+        # only DimShuffles that insert or drop broadcast dimensions: with a transposition in
+        # between, "the result's index" is no longer the consumer's index
+        kept_order = [o for o in ds_op.new_order if o != "x"]
+        if kept_order != sorted(kept_order):
+            return False
         layout = ds_op.make_node(red.outputs[0]).outputs[0].type.broadcastable
     else:
         layout = red.outputs[0].type.broadcastable
