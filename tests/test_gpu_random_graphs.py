@@ -15,6 +15,7 @@ from oracle import graph_ref as G
 from conftest import assert_parity
 
 EXTENTS = [1, 2, 3, 5, 7, 8, 16, 33, 64]
+MAX_ELEMENTS = 150000
 
 FLOAT_UNARY = [T.tanh, T.sigmoid, T.sin, T.cos, abs, T.sqr, T.neg, lambda v: T.exp(T.minimum(v, 3.0)),
                lambda v: T.sqrt(abs(v) + 0.5), lambda v: T.log(abs(v) + 1.0)]
@@ -68,7 +69,7 @@ def random_graph(seed):
     dtype = str(rng.choice(["float32", "float32", "float64", "int32", "int16", "int64"]))
     nd = int(rng.integers(1, 5))
     shape = [int(rng.choice(EXTENTS)) for _ in range(nd)]
-    while np.prod(shape) > 150000:
+    while np.prod(shape) > MAX_ELEMENTS:
         shape[int(np.argmax(shape))] //= 2
     floating = dtype.startswith("float")
     unary, binary = (FLOAT_UNARY, FLOAT_BINARY) if floating else (INT_UNARY, INT_BINARY)
