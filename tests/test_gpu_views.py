@@ -102,3 +102,25 @@ def test_minibatch_slices_of_a_large_matrix():
     f = th.function([x], [T.join(0, *parts), T.sum(x, axis=1)])
     joined, whole = f(val)
     assert np.array_equal(joined, whole)
+
+
+@pytest.mark.gpu
+def test_shape_entries_are_symbolic_scalars():
+    """x.shape[d] is a 0-d int64 variable (Shape_i, theano/compile/ops.py:377-470): it divides
+    a sum, scales a tensor (travelling to the kernel by value), names extents for reshape and
+    alloc, and follows the array it is called with."""
+    rng = np.random.default_rng(3)
+    x = T.fmatrix("x")
+    n, m = x.shape
+    assert n.type.ndim == 0 and n.type.dtype == "int64"
+    outs = [T.sum(x, axis=0) / n, x * m + n, T.alloc(np.float32(2.0), m, n) + x.T, x.reshape((m, n)), T.sum(x) / (n * m)]
+    f = th.function([x], outs)
+    for shape in ((5, 7), (33, 2)):
+        xv = rng.standard_normal(shape).astype("float32")
+        got = f(xv)
+        ref = G.evaluate([x], outs, [xv])
+        for g, r in zip(got, ref):
+            assert_parity(g, r, "shape arithmetic")
+        assert np.allclose(got[0], xv.astype("float64").sum(0) / shape[0]) and got[3].shape == shape[::-1]
+    with pytest.raises(TypeError):
+        x.reshape((n * m,))               # arithmetic on extents is not a shape entry

@@ -109,12 +109,13 @@ def tensor_from_scalar(s):
 
 # --------------------------------------------------------------------------
 class ShapeFloat(Op):
-    """Extent of dimension ``i`` of the input as a 0-d floating tensor.
+    """Extent of dimension ``i`` of the input as a 0-d tensor of ``dtype``.
 
-    Stands for ``cast(shape(x)[i], dtype)`` in ``mean`` / ``var``
-    (``theano/tensor/basic.py:3352-3373``).  It runs on the host and reads only
-    array metadata, whichever memory the array lives in; fused consumers take
-    its value as a kernel argument."""
+    With a floating dtype it stands for ``cast(shape(x)[i], dtype)`` in ``mean`` /
+    ``var`` (``theano/tensor/basic.py:3352-3373``), with int64 for ``Shape_i``
+    (``theano/compile/ops.py:377-470``), what ``x.shape[i]`` is.  It runs on the host
+    and reads only array metadata, whichever memory the array lives in; fused
+    consumers take its value as a kernel argument."""
 
     __props__ = ("i", "dtype")
 
@@ -342,6 +343,18 @@ def min(x, axis=None, keepdims=False):
     if keepdims:
         out = makeKeepDims(x, out, axis)
     return out
+
+
+def shape_i(x, i):
+    """``x.shape[i]`` as a 0-d int64 variable."""
+    x = as_tensor_variable(x)
+    if x.type.broadcastable[i]:
+        return constant(np.int64(1))
+    return ShapeFloat(i, "int64")(x)
+
+
+def Shape_i(i):
+    return ShapeFloat(i, "int64")
 
 
 def mean(input, axis=None, dtype=None, keepdims=False, acc_dtype=None):

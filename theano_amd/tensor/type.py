@@ -150,14 +150,15 @@ class _tensor_py_operators(object):
 
     @property
     def shape(self):
-        """``x.shape[d]`` is the pair ``(x, d)``: the way ``reshape`` and ``alloc`` name an extent
-        that is only known when the function runs."""
-        return tuple((self, d) for d in range(self.ndim))
+        """The extents as a tuple of 0-d int64 variables (``Shape_i``,
+        ``theano/compile/ops.py:377-470``): metadata read on the host when the function runs.
+        They take part in arithmetic as host scalars, and ``reshape`` / ``alloc`` accept them
+        as "the extent of dimension d of that tensor"."""
+        return tuple(self._b().shape_i(self, d) for d in range(self.ndim))
 
     def reshape(self, *shape):
         from . import views
-        if len(shape) == 1 and isinstance(shape[0], (list, tuple)) and not (
-                len(shape[0]) == 2 and hasattr(shape[0][0], "type")):
+        if len(shape) == 1 and isinstance(shape[0], (list, tuple)) and views._extent_entry(shape[0]) is None:
             shape = tuple(shape[0])
         return views.reshape(self, shape)
 

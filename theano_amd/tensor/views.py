@@ -307,14 +307,38 @@ class Reshape(Op):
         return [[True]] + [[False]] * (len(node.inputs) - 1)
 
 
+def _extent_entry(p):
+    """A shape entry that names a run-time extent: ``v.shape[d]`` (a Shape_i variable) or the
+    pair ``(v, d)``; returns that pair, or None for anything else."""
+    if isinstance(p, (tuple, list)):
+        if (len(p) == 2 and hasattr(p[0], "type") and isinstance(p[1], (int, np.integer)) and
+                0 <= p[1] < getattr(p[0].type, "ndim", 0)):
+            return tuple(p)
+        return None
+    if hasattr(p, "owner"):
+        if p.owner is not None and isinstance(p.owner.op, T.ShapeFloat):
+            return (p.owner.inputs[0], p.owner.op.i)
+        if hasattr(p, "data") and p.type.ndim == 0:
+            return None
+        raise TypeError("a symbolic shape entry must be a constant or some tensor's shape[d]; arithmetic on "
+                        "extents is not supported here: %s" % p)
+    return None
+
+
+def _int_entry(p):
+    return int(np.asarray(p.data)) if hasattr(p, "data") else int(p)
+
+
 def reshape(x, newshape):
-    """``newshape``: ints, at most one -1, or ``x.shape[d]``-style entries given
-    as ``(variable, d)`` pairs."""
+    """``newshape``: ints, at most one -1, or ``v.shape[d]`` entries."""
     x = as_tensor_variable(x)
-    if isinstance(newshape, (int, np.integer)):
+    if isinstance(newshape, (int, np.integer)) or hasattr(newshape, "owner"):
         newshape = (newshape,)
     like, pattern = [], []
     for p in newshape:
+        e = _extent_entry(p)
+        if e is not None:
+            p = e
         if isinstance(p, tuple):
             v, d = p
             v = as_tensor_variable(v)
@@ -325,7 +349,7 @@ def reshape(x, newshape):
                     like.append(v)
                 pattern.append((1 + like.index(v), int(d)))
         else:
-            pattern.append(int(p))
+            pattern.append(_int_entry(p))
     return Reshape(pattern)(x, *like)
 
 
@@ -409,16 +433,19 @@ class Alloc(Op):
 
 
 def alloc(value, *shape):
-    """``shape`` entries: ints or ``(variable, d)`` pairs."""
+    """``shape`` entries: ints or ``v.shape[d]``."""
     like, pattern = [], []
     for p in shape:
+        e = _extent_entry(p)
+        if e is not None:
+            p = e
         if isinstance(p, tuple):
             v = as_tensor_variable(p[0])
             if v not in like:
                 like.append(v)
             pattern.append((1 + like.index(v), int(p[1])))
         else:
-            pattern.append(int(p))
+            pattern.append(_int_entry(p))
     return Alloc(pattern)(value, *like)
 
 
