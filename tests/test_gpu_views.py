@@ -119,8 +119,10 @@ def test_shape_entries_are_symbolic_scalars():
         xv = rng.standard_normal(shape).astype("float32")
         got = f(xv)
         ref = G.evaluate([x], outs, [xv])
+        from conftest import TOL
         for g, r in zip(got, ref):
-            assert_parity(g, r, "shape arithmetic")
+            # float32 / int64 is a float32 division in C, whatever the result is stored in
+            assert_parity(g, r, "shape arithmetic", tol=TOL["float32"])
         assert np.allclose(got[0], xv.astype("float64").sum(0) / shape[0]) and got[3].shape == shape[::-1]
     with pytest.raises(TypeError):
         x.reshape((n * m,))               # arithmetic on extents is not a shape entry
