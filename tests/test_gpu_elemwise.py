@@ -260,3 +260,27 @@ def test_float_floor_division_is_exact_at_integer_quotients():
     got = th.function([i, f], i // f)(iv, fv)
     assert got.dtype == np.float64 and got[0] == 25.0
     assert np.array_equal(got, G.evaluate([i, f], [i // f], [iv, fv])[0])
+
+
+@pytest.mark.gpu
+def test_multi_output_kernels_from_merged_siblings():
+    """Adam-style updates in one kernel with three results (float32 and float16 storage,
+    a transposed operand), against the oracle; plus an integer pair with different dtypes."""
+    rng = np.random.default_rng(31)
+    p, g, m, v = [T.fmatrix(n) for n in "pgmv"]
+    m2 = 0.9 * m + 0.1 * g
+    v2 = 0.999 * v + 0.001 * T.sqr(g)
+    p2 = p - 0.01 * m2 / (T.sqrt(v2) + 1e-8)
+    outs = [m2, v2, p2, T.cast(p2, "float16"), p2.T * g.T]
+    f = th.function([p, g, m, v], outs)
+    assert sum(1 for n in f.toposort() if type(n.op).__name__ == "HipElemwise") <= 2
+    vals = [rng.standard_normal((257, 129)).astype("float32") for _ in range(3)] + [rng.uniform(0.1, 1, (257, 129)).astype("float32")]
+    for k, (a, b) in enumerate(zip(f(*vals), G.evaluate([p, g, m, v], outs, vals))):
+        assert_parity(a, b, "adam output %d" % k, tol=dict(rtol=2e-3, atol=2e-3) if b.dtype == np.float16 else None)
+    i, j = T.imatrix("i"), T.imatrix("j")
+    outs = [(i & j) + 1, T.cast(i, "int8") ^ T.cast(j, "int8"), T.gt(i, j), i.astype("int64") * j]
+    vals = [rng.integers(-2 ** 20, 2 ** 20, (65, 33)).astype("int32") for _ in range(2)]
+    f = th.function([i, j], outs)
+    assert sum(1 for n in f.toposort() if type(n.op).__name__ == "HipElemwise") == 1
+    for a, b in zip(f(*vals), G.evaluate([i, j], outs, vals)):
+        assert_parity(a, b, "integer siblings")

@@ -88,10 +88,14 @@ def test_fusion_respects_broadcast_pattern_and_client_count():
     # (case 71 of theano/tensor/tests/test_opt.py:1107-1111)
     f = th.function([x, s], x + T.sin(s))
     assert len(ops_of(f, HipElemwise)) == 2
-    # an expensive producer with two clients is computed once, not duplicated
+    # an expensive producer with two clients is computed once, not duplicated: without the sibling
+    # merge it keeps a kernel of its own, with it both consumers and the producer are one kernel
     e = T.exp(x)
     g = th.function([x], [e + 1, e * 2])
-    assert len(ops_of(g, HipElemwise)) == 3
+    (only,) = ops_of(g, HipElemwise)
+    from theano_amd import gof
+    inner = gof.io_toposort(only.op.scalar_op.inputs, only.op.scalar_op.outputs)
+    assert len(only.outputs) == 2 and sum(1 for n in inner if n.op == scal.exp) == 1
 
 
 def test_config1_is_one_kernel_with_scalars_passed_by_value():
@@ -557,3 +561,25 @@ def test_ops_and_graphs_pickle(dry_run):
     v = np.random.default_rng(0).standard_normal((4, 6)).astype("float32")
     for a, b in zip(G.evaluate([x], [y, z, gx], [v]), G.evaluate([x2], outs2, [v])):
         assert np.array_equal(a, b)
+
+
+def test_sibling_elementwise_kernels_merge_into_one_with_several_results(dry_run):
+    """An Adam step: both moment updates and the parameter update read g, m, v, p once and
+    write three arrays in one kernel; kernels of different shapes, or one feeding the other
+    through a reduction, stay apart."""
+    p, g, m, v = [T.fmatrix(n) for n in "pgmv"]
+    m2 = 0.9 * m + 0.1 * g
+    v2 = 0.999 * v + 0.001 * T.sqr(g)
+    p2 = p - 0.01 * m2 / (T.sqrt(v2) + 1e-8)
+    f = th.function([p, g, m, v], [m2, v2, p2])
+    (k,) = ops_of(f, HipElemwise)
+    assert len(k.outputs) == 3 and len(k.inputs) == 4
+    f(*[np.zeros((3, 4), "float32")] * 4)
+    # different shapes: a row result and a matrix result do not merge
+    r = T.frow("r")
+    h = th.function([p, r], [p * 2.0, r * 3.0])
+    assert len(ops_of(h, HipElemwise)) == 2
+    # a dependency through a reduction keeps two kernels
+    s = T.sum(p * 2.0, axis=0, keepdims=True)
+    d = th.function([p], [T.exp(p), p / s])
+    assert len(ops_of(d, HipElemwise)) == 2 or len(ops_of(d, HipCAReduce)) == 1

@@ -152,7 +152,7 @@ def _absorbs(client, var):
         return False
     op = client.op
     if isinstance(op, HipElemwise):
-        return (len(client.outputs) == 1 and not op.inplace_pattern and
+        return (not op.inplace_pattern and
                 tuple(client.outputs[0].type.broadcastable) == tuple(var.type.broadcastable))
     if isinstance(op, HipCAReduce):
         return op.post_scalar_op is None and all(
@@ -195,9 +195,9 @@ def _fusable(fgraph, var, out_bcast):
 def _fuse_node(fgraph, node):
     """Splice single-client elementwise producers of ``node`` into it
     (acceptance rule of ``theano/tensor/opt.py:7168-7218``)."""
-    if not isinstance(node.op, HipElemwise) or len(node.outputs) != 1 or node.op.inplace_pattern:
+    if not isinstance(node.op, HipElemwise) or node.op.inplace_pattern:
         return None
-    out = node.outputs[0]
+    out = node.outputs[0]               # the results of one node share a broadcast pattern
     inputs, s_inputs = [], []
 
     def scalar_for(v):
@@ -234,14 +234,14 @@ def _fuse_node(fgraph, node):
                 s_args.append(scalar_for(i))
     if not fused or not inputs:
         return None
-    s_out = node.op.scalar_op(*s_args)
-    if s_out.type.dtype != out.type.dtype:
+    s_outs = node.op.scalar_op(*s_args, return_list=True)
+    if [s.type.dtype for s in s_outs] != [o.type.dtype for o in node.outputs]:
         return None
-    comp = scal.Composite(s_inputs, [s_out])
-    new_out = HipElemwise(comp)(*inputs)
-    if new_out.type != out.type:
+    comp = scal.Composite(s_inputs, s_outs)
+    new_outs = HipElemwise(comp).make_node(*inputs).outputs
+    if [n.type for n in new_outs] != [o.type for o in node.outputs]:
         return None
-    return new_out
+    return new_outs
 
 
 def fuse_elemwise(fgraph):
@@ -254,9 +254,10 @@ def fuse_elemwise(fgraph):
         for node in reversed(fgraph.toposort()):
             if node not in fgraph.apply_nodes:
                 continue
-            new_out = _fuse_node(fgraph, node)
-            if new_out is not None:
-                fgraph.replace(node.outputs[0], new_out)
+            new_outs = _fuse_node(fgraph, node)
+            if new_outs is not None:
+                for o, no in zip(node.outputs, new_outs):
+                    fgraph.replace(o, no)
                 changed = True
                 total += 1
     return total
@@ -625,6 +626,73 @@ def _merge_two(a, b):
     return op.make_node(*inputs)
 
 
+def merge_sibling_elemwise(fgraph):
+    """Two elementwise kernels of one and the same shape become one kernel with several results
+    when that saves reading an array again: siblings that read a common array (the two moment
+    updates of an Adam step), or a kernel and a consumer of its results that something else
+    needs as well (the parameter update that reads both new moments, which are outputs too).
+    Equal shapes are certain because both hold an array of exactly the results' broadcast
+    pattern in common; apart from the direct use of one's results by the other, neither may
+    depend on the other.  The reference's GPU op stops at one output
+    (``theano/gpuarray/elemwise.py:114-115``); the kernels here take several."""
+    count = 0
+    changed = True
+    while changed:
+        changed = False
+        nodes = [n for n in fgraph.toposort() if isinstance(n.op, HipElemwise) and not n.op.inplace_pattern]
+        for ai, a in enumerate(nodes):
+            pa = tuple(a.outputs[0].type.broadcastable)
+            if all(pa):
+                continue
+            full_a = set(id(i) for i in a.inputs if isinstance(i.type, HipArrayType) and
+                         tuple(i.type.broadcastable) == pa)
+            full_a.update(id(o) for o in a.outputs)
+            for b in nodes[ai + 1:]:
+                if tuple(b.outputs[0].type.broadcastable) != pa:
+                    continue
+                if not any(id(i) in full_a for i in b.inputs):
+                    continue
+                if any(i.owner is not a and _depends_on(i, a) for i in b.inputs):
+                    continue
+                if any(_depends_on(i, b) for i in a.inputs):
+                    continue
+                inputs, s_inputs = [], []
+
+                def scalar_for(v):
+                    for t, sv in zip(inputs, s_inputs):
+                        if t is v:
+                            return sv
+                    sv = scal.Scalar(v.type.dtype)()
+                    inputs.append(v)
+                    s_inputs.append(sv)
+                    return sv
+
+                a_souts = a.op.scalar_op(*[scalar_for(v) for v in a.inputs], return_list=True)
+                b_args = [a_souts[a.outputs.index(v)] if v.owner is a else scalar_for(v) for v in b.inputs]
+                b_souts = b.op.scalar_op(*b_args, return_list=True)
+                # results of the first kernel that only the second one read stay inside
+                keep = [k for k, o in enumerate(a.outputs)
+                        if any(c is not b for c, _ in fgraph.clients.get(o, []))]
+                olds = [a.outputs[k] for k in keep] + list(b.outputs)
+                if len(inputs) > config.max_fused_inputs or len(olds) > 8:
+                    continue
+                # an array that is both read and produced here would be an output equal to an input
+                s_outs = [a_souts[k] for k in keep] + b_souts
+                if any(so in s_inputs for so in s_outs):
+                    continue
+                merged = HipElemwise(scal.Composite(s_inputs, s_outs)).make_node(*inputs)
+                if [o.type for o in merged.outputs] != [o.type for o in olds]:
+                    continue
+                for o, no in zip(olds, merged.outputs):
+                    fgraph.replace(o, no)
+                count += 1
+                changed = True
+                break
+            if changed:
+                break
+    return count
+
+
 # --------------------------------------------------------------------------
 def inplace_elemwise(fgraph):
     """The role of ``InplaceElemwiseOptimizer`` (``theano/tensor/opt.py:150-410``):
@@ -677,6 +745,9 @@ def optimize(fgraph, fuse=True, rowchain=True, inplace=True):
         gof.merge_identical(fgraph)
         fuse_elemwise(fgraph)          # producers that lost their other clients to an epilogue
         gof.merge_identical(fgraph)
+        if merge_sibling_elemwise(fgraph):
+            fuse_elemwise(fgraph)      # a producer whose clients all ended up in one kernel joins it
+            gof.merge_identical(fgraph)
     if inplace:
         inplace_elemwise(fgraph)
     return fgraph
