@@ -1,7 +1,6 @@
 """GPU parity of MaxAndArgmax / argmax / argmin against the oracle (NumPy's
 first-occurrence rule, as MaxAndArgmax.perform): every kernel form, ties, NaNs,
 integer and float16 values, split reductions, strided inputs."""
-import itertools
 
 import numpy as np
 import pytest

@@ -1,5 +1,4 @@
 """GPU parity of CAReduce against the oracle over shapes, masks, ops and dtypes."""
-import itertools
 
 import numpy as np
 import pytest

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import theano_amd as th
-from theano_amd import hip, tensor as T
+from theano_amd import tensor as T
 from theano_amd.hip import HipCAReduce, HipElemwise
 from oracle import graph_ref as G
 from conftest import assert_parity

@@ -7,7 +7,6 @@ file the Python side has to find.
 """
 import os
 import subprocess
-import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 KERNEL_HEADERS = ["thx_common.h", "thx_elemwise.h", "thx_reduce.h", "thx_rowchain.h"]

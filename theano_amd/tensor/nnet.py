@@ -12,7 +12,6 @@ row-chain fusion turns each (forward, gradient, or both at once) into one launch
 """
 import warnings
 
-from .. import gof
 from .. import scalar as scal
 from ..gof import Apply, Op, local_optimizer
 from . import basic as T
