@@ -379,7 +379,8 @@ def local_single_pass_variance(fgraph, node):
     element is an outlier by many orders of magnitude).  The two sums read the same operand as
     the mean's own sum, so the three merge into one pass over x where the two-pass form of
     ``var`` (``theano/tensor/basic.py:3430-3459``) needs two.  float64 data keeps two passes:
-    there is no wider accumulator to absorb the cancellation."""
+    there is no wider accumulator to absorb the cancellation.  With nothing to reduce (an
+    empty extent) taking the first element raises IndexError where the two-pass form yields NaN."""
     from ..config import config
     from .views import Subtensor
     if not config.single_pass_variance:
