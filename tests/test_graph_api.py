@@ -583,3 +583,34 @@ def test_sibling_elementwise_kernels_merge_into_one_with_several_results(dry_run
     s = T.sum(p * 2.0, axis=0, keepdims=True)
     d = th.function([p], [T.exp(p), p / s])
     assert len(ops_of(d, HipElemwise)) == 2 or len(ops_of(d, HipCAReduce)) == 1
+
+
+def test_nested_sums_and_products_become_one_reduction():
+    """Sum(Sum(x, a), b) -> Sum(x, a + b') with the outer axes renumbered, Prod likewise, every
+    axis -> None (theano/tensor/opt.py:5479-5563); an inner result that something else reads
+    stays.  Values against NumPy."""
+    from theano_amd import gof
+    from theano_amd.tensor import opt as topt
+    from oracle import graph_ref as G
+    x = T.TensorType("float64", (False,) * 4)("x")
+    xv = np.random.default_rng(1).uniform(0.5, 1.5, (3, 4, 5, 6))
+    cases = [(T.sum(T.sum(x, axis=1), axis=1), xv.sum(axis=(1, 2)), (1, 2)),
+             (T.sum(T.sum(x, axis=(0, 3)), axis=0), xv.sum(axis=(0, 1, 3)), (0, 1, 3)),
+             (T.sum(T.sum(x, axis=2), axis=(0, 2)), xv.sum(axis=(0, 2, 3)), (0, 2, 3)),
+             (T.prod(T.prod(x, axis=3), axis=0), xv.prod(axis=(0, 3)), (0, 3)),
+             (T.sum(T.sum(x, axis=(1, 2))), xv.sum(), None),
+             (T.sum(x, axis=(0, 1, 2, 3)), xv.sum(), None)]
+    for out, want, axis in cases:
+        fg = gof.FunctionGraph([x], [out])
+        topt.canonicalize(fg)
+        reds = [n for n in fg.toposort() if isinstance(n.op, CAReduce)]
+        assert len(reds) == 1 and reds[0].op.axis == axis, (str(out), [str(n) for n in reds])
+        assert np.allclose(G.evaluate(fg.inputs, fg.outputs, [xv])[0], want, rtol=1e-13)
+    inner = T.sum(x, axis=1)
+    fg = gof.FunctionGraph([x], [T.sum(inner, axis=1), inner * 2])
+    topt.canonicalize(fg)
+    assert len([n for n in fg.toposort() if isinstance(n.op, CAReduce)]) == 2
+    # sum of a product of sums is not touched
+    fg = gof.FunctionGraph([x], [T.sum(T.prod(x, axis=1), axis=1)])
+    topt.canonicalize(fg)
+    assert len([n for n in fg.toposort() if isinstance(n.op, CAReduce)]) == 2

@@ -210,6 +210,37 @@ def local_useless_reduce(fgraph, node):
 
 
 @local_optimizer([CAReduce])
+def local_op_of_op(fgraph, node):
+    """``Sum(Sum(x, a), b) -> Sum(x, a + b')`` and the same for ``Prod`` when nothing else reads
+    the inner result (``theano/tensor/opt.py:5497-5563``): one pass, one rounding to the output
+    dtype; ``Sum{every axis} -> Sum{None}`` so that equal reductions merge (:5479-5494)."""
+    from .elemwise import Prod
+    op = node.op
+    if type(op) not in (Sum, Prod):
+        return False
+    (x,) = node.inputs
+    cls = type(op)
+    if op.axis is not None and set(op.axis) == set(range(x.type.ndim)) and x.type.ndim > 0:
+        new = cls(None, dtype=op.dtype, acc_dtype=op.acc_dtype)(x)
+        return [new] if new.type == node.outputs[0].type else False
+    p = x.owner
+    if p is None or type(p.op) is not cls or fgraph.n_clients(x) != 1:
+        return False
+    if p.op.axis is None or op.axis is None:
+        new_axis = None
+    else:
+        new_axis = list(p.op.axis)
+        for i in op.axis:                      # positions of the outer axes in the inner input
+            j = i
+            for ii in sorted(p.op.axis):
+                if j >= ii:
+                    j += 1
+            new_axis.append(j)
+    new = cls(new_axis, dtype=op.dtype)(p.inputs[0])
+    return [new] if new.type == node.outputs[0].type else False
+
+
+@local_optimizer([CAReduce])
 def local_sum_invariant_factor(fgraph, node):
     """``sum(c * x, axis) -> c' * sum(x, axis)``, ``sum(x / c) -> sum(x) / c'`` and
     ``sum(-x) -> -sum(x)`` for every factor ``c`` that is constant along all the
@@ -456,7 +487,7 @@ def local_single_pass_variance(fgraph, node):
 
 
 CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_constant_fold, local_useless_elemwise, local_fill_sink,
-                local_useless_reduce,
+                local_useless_reduce, local_op_of_op,
                 local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_single_pass_variance]
 
 
