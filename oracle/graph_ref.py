@@ -16,10 +16,17 @@ own backend would node by node:
   dtype (``elemwise.py:1549-1554``).  Zero-length max / min raise ValueError
   (``elemwise.py:1489-1506``).
 * ``DimShuffle``: the strided view of ``theano/tensor/c_code/dimshuffle.c:55-98``.
+* ``MaxAndArgmax``, the view ops (NumPy basic indexing, reshape, broadcast_to, concatenate),
+  the row-softmax ops and the batch-normalization ops: the reference's ``perform`` formulas
+  (``theano/tensor/basic.py:1311-1330``, ``theano/tensor/nnet/nnet.py:73-104, 316-323,
+  440-444, 628-633``, ``theano/tensor/nnet/bn.py:475-499, 568-571, 659-676``).
 
-Pinned by tests/test_oracle_graph.py against the reference's literal test
-answers (``theano/tensor/tests/test_elemwise.py:654-748, 953-966``; fusion table
-``theano/tensor/tests/test_opt.py:964-1112``) and NumPy closed forms.
+Pinned by tests/test_oracle_graph.py and tests/test_golden.py against the reference's
+literal test answers (``theano/tensor/tests/test_elemwise.py:654-748, 953-966``; fusion
+table ``theano/tensor/tests/test_opt.py:964-1112``; ``test_basic.py:3114-3119, 3304-3309``)
+and NumPy closed forms; the softmax and batch-normalization formulas by
+tests/test_graph_api.py against ``scipy.special.log_softmax``, closed-form gradients,
+NumPy's mean / var and reverse mode through plain graphs.  No function here is unpinned.
 """
 import ctypes
 import os

@@ -18,7 +18,12 @@ comparisons and bit ops against the truth tables of
 (``theano/tensor/tests/test_elemwise.py:525-538``); dtype rules against the
 literal tables of ``theano/scalar/basic.py:855-870`` and
 ``theano/scalar/tests/test_basic.py:264-380``; ``right_shift(a, 3) ==
-int_div(a, 8)`` (no shift op exists in the reference).
+int_div(a, 8)`` (no shift op exists in the reference); float IntDiv against a
+scalar transcription of the four sign cases and against exact floor division away
+from integer quotients.  The special functions are ``scipy.special`` itself, which
+is what the reference's ``impl`` calls (``theano/scalar/basic_scipy.py:32-36``); every
+differentiable op's value is tied to its neighbours' by the finite-difference
+gradient checks of tests/test_oracle_graph.py.  No function here is unpinned.
 """
 import numpy as np
 
