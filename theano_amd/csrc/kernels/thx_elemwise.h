@@ -160,12 +160,12 @@ __device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename 
 // ---------------------------------------------------------------------------
 // Permuted-read variant. Some inputs are unit-stride along a dimension T that
 // is not the innermost one of the result (a dimshuffled view). A block owns a
-// TILE x TILE patch of (T, innermost): those inputs are read in rows along T
-// - full cache lines - into LDS and read back transposed, while every other
-// operand is accessed along the innermost dimension. Rows of a tile are padded
-// by one element so that the transposed reads hit distinct banks.
+// TT x TI patch of (T, innermost): those inputs are read in rows of TT elements
+// along T - whole cache lines - into LDS and read back transposed, while every
+// other operand is accessed along the innermost dimension. Rows of a tile are
+// padded by one element so that the transposed reads hit distinct banks.
 //
-// Extra plan members: enum { TILE, TV (elements per access), NTR (staged
+// Extra plan members: enum { TT, TI, TV (elements per access), NTR (staged
 // inputs), ESZ (largest staged element) }; static constexpr int slot(int
 // operand): LDS slot or -1.
 template <int NOPS, int ND, class IT>
@@ -186,11 +186,11 @@ struct TrStageAcc {  // global -> LDS for the staged inputs, nothing for the oth
   char* const* ptr;
   unsigned char* lds;
   IT off[NOPS];
-  int cell;  // LDS index of the first element: row * (TILE + 1) + position along T
+  int cell;  // LDS index of the first element: row * (TT + 1) + position along T
   template <int I, class T, int N>
   THX_DEV void ld(Vec<T, N>&) const {
     if (P::slot(I) >= 0) {
-      T* tile = (T*)(lds + P::slot(I) * (P::TILE * (P::TILE + 1) * P::ESZ));
+      T* tile = (T*)(lds + P::slot(I) * (P::TI * (P::TT + 1) * P::ESZ));
       Vec<T, N> r;
       load_vec<T, N, ((P::NT >> I) & 1) != 0>(r, (const T*)ptr[I] + off[I]);
 #pragma unroll
@@ -206,13 +206,13 @@ struct TrAcc {  // LDS (transposed) or global -> registers, registers -> global
   const unsigned long long* imm;
   const unsigned char* lds;
   IT off[NOPS];
-  int cell;  // LDS index of the first element: position along the inner dimension * (TILE + 1) + row along T
+  int cell;  // LDS index of the first element: position along the inner dimension * (TT + 1) + row along T
   template <int I, class T, int N>
   THX_DEV void ld(Vec<T, N>& r) const {
     if (P::slot(I) >= 0) {
-      const T* tile = (const T*)(lds + P::slot(I) * (P::TILE * (P::TILE + 1) * P::ESZ));
+      const T* tile = (const T*)(lds + P::slot(I) * (P::TI * (P::TT + 1) * P::ESZ));
 #pragma unroll
-      for (int k = 0; k < N; ++k) r.v[k] = tile[cell + k * (P::TILE + 1)];
+      for (int k = 0; k < N; ++k) r.v[k] = tile[cell + k * (P::TT + 1)];
     } else if (P::mode(I) == M_IMM) {
       const T s = *(const T*)&imm[I];
 #pragma unroll
@@ -237,12 +237,17 @@ struct TrAcc {  // LDS (transposed) or global -> registers, registers -> global
 template <class F, class P>
 __device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, typename P::IT>& p) {
   typedef typename P::IT IT;
-  constexpr int TILE = P::TILE, TV = P::TV, NOPS = F::NOPS, ND = P::ND;
-  constexpr int LPR = TILE / TV;            // lanes per tile row
-  constexpr int RPP = P::BLOCK / LPR;       // tile rows per pass
-  constexpr int PASSES = TILE / RPP;
-  constexpr int UNR = PASSES < 4 ? PASSES : 4;
-  __shared__ __attribute__((aligned(16))) unsigned char lds[P::NTR * TILE * (TILE + 1) * P::ESZ];
+  constexpr int TT = P::TT, TI = P::TI, TV = P::TV, NOPS = F::NOPS, ND = P::ND;
+  constexpr int LPR_S = TT / TV;              // staging: lanes per row along T
+  constexpr int RPP_S = P::BLOCK / LPR_S;     //          rows (positions along the inner dimension) per pass
+  constexpr int PASSES_S = TI / RPP_S;
+  constexpr int LPR_C = TI / TV;              // computing: lanes per row along the inner dimension
+  constexpr int RPP_C = P::BLOCK / LPR_C;     //            rows (positions along T) per pass
+  constexpr int PASSES_C = TT / RPP_C;
+  constexpr int UNR = PASSES_C < 4 ? PASSES_C : 4;
+  static_assert(PASSES_S >= 1 && PASSES_C >= 1 && PASSES_S * RPP_S == TI && PASSES_C * RPP_C == TT,
+                "tile and block do not divide");
+  __shared__ __attribute__((aligned(16))) unsigned char lds[P::NTR * TI * (TT + 1) * P::ESZ];
 
   unsigned rem = blockIdx.x, ti, tt, c;
   divmod(rem, p.tiles_i, rem, ti);
@@ -260,21 +265,21 @@ __device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, type
 #pragma unroll
     for (int i = 0; i < NOPS; ++i) base[i] += (IT)rem * p.ostride[i][0];
   }
-  const int t0 = tt * TILE, i0 = ti * TILE;
-  const int lane = threadIdx.x % LPR, row = threadIdx.x / LPR;
+  const int t0 = tt * TT, i0 = ti * TI;
 
   // stage: lanes run along T
   {
     typename F::template Regs<TV> dummy;
+    const int lane = threadIdx.x % LPR_S, row = threadIdx.x / LPR_S;
     const int t = t0 + lane * TV;
 #pragma unroll
-    for (int k = 0; k < PASSES; ++k) {
-      const int ii = row + k * RPP, i = i0 + ii;
+    for (int k = 0; k < PASSES_S; ++k) {
+      const int ii = row + k * RPP_S, i = i0 + ii;
       if (t < p.ext_t && i < p.ext_i) {
         TrStageAcc<P, NOPS> a;
         a.ptr = p.ptr;
         a.lds = lds;
-        a.cell = ii * (TILE + 1) + lane * TV;
+        a.cell = ii * (TT + 1) + lane * TV;
 #pragma unroll
         for (int o = 0; o < NOPS; ++o) a.off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
         F::template load<TV>(a, dummy);
@@ -284,20 +289,21 @@ __device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, type
   __syncthreads();
 
   // compute: lanes run along the innermost dimension
+  const int lane = threadIdx.x % LPR_C, row = threadIdx.x / LPR_C;
   const int i = i0 + lane * TV;
 #pragma unroll
-  for (int k0 = 0; k0 < PASSES; k0 += UNR) {
+  for (int k0 = 0; k0 < PASSES_C; k0 += UNR) {
     typename F::template Regs<TV> r[UNR];
     TrAcc<P, NOPS> a[UNR];
     bool ok[UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      const int tl = row + (k0 + u) * RPP, t = t0 + tl;
+      const int tl = row + (k0 + u) * RPP_C, t = t0 + tl;
       ok[u] = t < p.ext_t && i < p.ext_i;
       a[u].ptr = p.ptr;
       a[u].imm = p.imm;
       a[u].lds = lds;
-      a[u].cell = lane * TV * (TILE + 1) + tl;
+      a[u].cell = lane * TV * (TT + 1) + tl;
 #pragma unroll
       for (int o = 0; o < NOPS; ++o) a[u].off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
       if (ok[u]) F::template load<TV>(a[u], r[u]);

@@ -66,7 +66,7 @@ struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, T
 struct PlanGen { typedef int IT; enum { NK = 3, NR = 3, BLOCK = 256, TPR = 64 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; } };
 
-struct PlanTr { typedef int IT; enum { ND = 3, TILE = 64, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2 }; static constexpr unsigned long long NT = 0ull;
+struct PlanTr { typedef int IT; enum { ND = 3, TT = 64, TI = 32, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2, 0, 0}; return m[i]; }
   static constexpr int slot(int i) { constexpr int m[] = {0, -1, -1}; return m[i]; } };
 extern "C" __global__ __launch_bounds__(256) void check_tr(thx::EwTrParams<3, 3, int> p) { thx::ew_tr_body<CheckF, PlanTr>(p); }

@@ -242,6 +242,16 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
       if ((int64_t)ntr * tile * (tile + 1) * esz > 60000) tile = 32;
       const int force_tile = env_int("THX_EW_TILE", 0);
       if (force_tile == 32 || force_tile == 64) tile = force_tile;
+      // extents of the tile along T (rows read from the permuted inputs) and along the inner dimension
+      int tile_t = tile, tile_i = tile;
+      {
+        const int ft = env_int("THX_EW_TILE_T", 0), fi = env_int("THX_EW_TILE_I", 0);
+        auto pow2 = [](int v) { return v >= 8 && v <= 256 && (v & (v - 1)) == 0; };
+        if (pow2(ft) && pow2(fi) && ft * fi >= 1024) {
+          tile_t = ft;
+          tile_i = fi;
+        }
+      }
       // elements per access: 16 bytes of the widest operand, if extents, strides and addresses allow
       int allsz = 1;
       for (int o = 0; o < nops; ++o)
@@ -264,11 +274,11 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
       };
       while (!tv_ok(tv)) tv /= 2;
       if (env_int("THX_EW_TV", 0) == 1) tv = 1;
-      if ((int64_t)ntr * tile * (tile + 1) * esz <= 60000) {
+      if ((int64_t)ntr * tile_i * (tile_t + 1) * esz <= 60000) {
         const int block = 256;
         const uint64_t nt = nt_mask(nt_streaming(moved), views);
         std::ostringstream key;
-        key << "et|nd" << ND << "|t" << tile << "|v" << tv << "|n" << ntr << "|e" << esz;
+        key << "et|nd" << ND << "|t" << tile_t << "x" << tile_i << "|v" << tv << "|n" << ntr << "|e" << esz;
         if (nt) key << "|nt" << std::hex << nt << std::dec;
         key << "|m";
         for (int o = 0; o < nops; ++o) key << (slot[o] >= 0 ? 9 : mode[o]) << (o + 1 < nops ? "," : "");
@@ -282,7 +292,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
           const std::string entry = entry_name(e->name, plan);
           std::ostringstream s;
           s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef int IT;\n  enum { ND = " << ND
-            << ", TILE = " << tile << ", TV = " << tv << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz
+            << ", TT = " << tile_t << ", TI = " << tile_i << ", TV = " << tv << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz
             << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
           for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
           s << "};\n    return m[i];\n  }\n  static constexpr int slot(int i) {\n    constexpr int m[] = {";
@@ -296,7 +306,7 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
         }
         if (dry) return THX_OK;
         const int64_t ext_t = dm.shape[tdim], ext_i = inner;
-        const int64_t tiles_t = (ext_t + tile - 1) / tile, tiles_i = (ext_i + tile - 1) / tile;
+        const int64_t tiles_t = (ext_t + tile_t - 1) / tile_t, tiles_i = (ext_i + tile_i - 1) / tile_i;
         int64_t outer = 1;
         std::vector<int> odims;
         for (int d = 0; d < ND - 1; ++d)
