@@ -44,6 +44,20 @@ __device__ __forceinline__ float thx_fdiv(float a, float b) {
 __device__ __forceinline__ float thx_fdiv(float a, float b) { return a / b; }
 #endif
 
+// 1 / (1 + exp(-x)) for -88 <= x <= 15 (the caller applies the reference's saturation outside).
+// In the 2.5-ulp build the exponential is one hardware exp2 of the rounded product x * log2(e),
+// whose rounding is a relative error of up to |x| * 4e-8 in exp(-x); it reaches the result only
+// where exp(-x) dominates it: below 8.5e-7 relative wherever the result exceeds 1e-6, 3.8e-6 at
+// x = -88 (where the result is 1e-38).  The reciprocal is one hardware rcp: its argument lies in
+// [1, 2e38], where rcp needs no rescaling.  8 instructions instead of 22.
+#ifdef THX_FAST_DIV
+__device__ __forceinline__ float thx_sigmoid_core(float x) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * -1.44269504088896340736f));
+}
+#else
+__device__ __forceinline__ float thx_sigmoid_core(float x) { return 1.0f / (1.0f + expf(-x)); }
+#endif
+
 // x / y in the type C gives the quotient, correctly rounded even when single-precision division
 // is built in its 2.5-ulp form: a double quotient rounded to float is the correctly rounded float
 // quotient (53 >= 2 * 24 + 2 bits).

@@ -1084,7 +1084,7 @@ class ScalarSigmoid(UnaryScalarOp):
         t = node.inputs[0].type.dtype
         (x,), (z,) = inputs, outputs
         if t in ("float32", "float16"):
-            return "%s = %s < -88.0f ? 0.0f : %s > 15.0f ? 1.0f : thx_fdiv(1.0f, 1.0f + expf(-%s));" % (z, x, x, x)
+            return "%s = %s < -88.0f ? 0.0f : %s > 15.0f ? 1.0f : thx_sigmoid_core(%s);" % (z, x, x, x)
         if t == "float64":
             return "%s = %s < -709.0 ? 0.0 : %s > 19.0 ? 1.0 : 1.0 / (1.0 + exp(-%s));" % (z, x, x, x)
         raise NotImplementedError("only floating point is implemented")
