@@ -926,7 +926,10 @@ def _unary_math(cname, fname, grad_fn, policy=upgrade_to_float):
     class _U(UnaryScalarOp):
         def c_code(self, node, inputs, outputs):
             ot = node.outputs[0].type.dtype
-            return "%s = %s((%s)%s);" % (outputs[0], _fn(fname, ot), compute_ctype(ot), inputs[0])
+            fn = _fn(fname, ot)
+            if fn == "expf":
+                fn = "thx_fexp"        # expf, or exp2 of x * log2(e) in the 2.5-ulp build
+            return "%s = %s((%s)%s);" % (outputs[0], fn, compute_ctype(ot), inputs[0])
 
         def L_op(self, inputs, outputs, gout):
             (x,) = inputs
