@@ -284,3 +284,27 @@ def test_multi_output_kernels_from_merged_siblings():
     assert sum(1 for n in f.toposort() if type(n.op).__name__ == "HipElemwise") == 1
     for a, b in zip(f(*vals), G.evaluate([i, j], outs, vals)):
         assert_parity(a, b, "integer siblings")
+
+
+@pytest.mark.gpu
+def test_exact_float32_math_when_the_fast_forms_are_switched_off(monkeypatch):
+    """THX_FAST_DIV=0: float32 division and square root correctly rounded (bit-equal to
+    NumPy's), exp / sigmoid from the math library (within 2 ulp of the double result); the
+    default build stays inside rtol 1e-5 on the same inputs."""
+    rng = np.random.default_rng(5)
+    a, b = T.fvector("a"), T.fvector("b")
+    av = np.concatenate([rng.uniform(-87, 87, 50000), rng.uniform(-2, 2, 50000)]).astype("float32")
+    bv = rng.uniform(0.01, 50, av.size).astype("float32")
+    outs = [a / b, T.sqrt(b), T.exp(a), T.sigmoid(a)]
+    fast = th.function([a, b], outs)(av, bv)
+    monkeypatch.setenv("THX_FAST_DIV", "0")
+    exact = th.function([a, b], outs)(av, bv)
+    assert "|fd" not in hip.last_plan()
+    assert np.array_equal(exact[0], av / bv) and np.array_equal(exact[1], np.sqrt(bv))
+    e64 = np.exp(av.astype("float64"))
+    assert np.max(np.abs(exact[2] - e64) / e64) < 2.5e-7
+    s64 = 1.0 / (1.0 + np.exp(-av.astype("float64")))
+    ok = av > -80                                      # below, results are denormal
+    assert np.max(np.abs(exact[3][ok] - s64[ok]) / s64[ok]) < 4e-7
+    for f, e in zip(fast, exact):
+        assert np.allclose(f, e, rtol=1e-5, atol=1e-37)
