@@ -95,6 +95,11 @@ def ones_like(model, dtype=None):
     return fill(model, constant(1, dtype=dtype))
 
 
+def iround(a, mode="half_away_from_zero"):
+    """``cast(round(a, mode), 'int64')`` (``theano/tensor/basic.py:2168-2171``)."""
+    return cast(round(a, mode), "int64")
+
+
 def round(a, mode="half_away_from_zero"):
     if mode == "half_away_from_zero":
         return round_half_away_from_zero(a)
