@@ -284,13 +284,14 @@ def evaluate(inputs, outputs, values):
         elif isinstance(op, MaxAndArgmax):
             res = list(max_and_argmax(args[0], op.axis))
         elif isinstance(op, V.Subtensor):          # NumPy basic indexing is the definition (subtensor.py:318-780)
-            res = [args[0][op.idx_list]]
+            res = [args[0][V.resolve_index(op.idx_list, args[1:])]]
         elif isinstance(op, V.IncSubtensor):       # subtensor.py:1460-1500
             x = np.array(args[0], copy=True)
+            idx = V.resolve_index(op.idx_list, args[2:])
             if op.set_instead_of_inc:
-                x[op.idx_list] = args[1]
+                x[idx] = args[1]
             else:
-                x[op.idx_list] += args[1]
+                x[idx] += args[1]
             res = [x]
         elif isinstance(op, V.Reshape):
             res = [np.reshape(args[0], op.resolve([a.shape for a in args]))]

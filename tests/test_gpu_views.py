@@ -126,3 +126,41 @@ def test_shape_entries_are_symbolic_scalars():
         assert np.allclose(got[0], xv.astype("float64").sum(0) / shape[0]) and got[3].shape == shape[::-1]
     with pytest.raises(TypeError):
         x.reshape((n * m,))               # arithmetic on extents is not a shape entry
+
+
+@pytest.mark.gpu
+def test_symbolic_slices_and_givens_minibatches():
+    """x[a:b], x[i], x[::s] with integer scalar variables (theano/tensor/subtensor.py:318-420)
+    and the minibatch idiom: a shared data set, an index input and
+    givens={x: data[i * n:(i + 1) * n]} (theano/compile/pfunc.py:365-420)."""
+    rng = np.random.default_rng(12)
+    x = T.fmatrix("x")
+    a, b, s, i = T.lscalar("a"), T.lscalar("b"), T.lscalar("s"), T.iscalar("i")
+    outs = [x[a:b] * 2.0, x[i], x[::s, 1:], T.sum(x[a:], axis=0), th.grad(T.sum(x[a:b, i] ** 2), x),
+            T.set_subtensor(x[a:b, ::2], 1.5), T.inc_subtensor(x[i], x[-1])]
+    f = th.function([x, a, b, s, i], outs)
+    xv = rng.standard_normal((23, 9)).astype("float32")
+    for av, bv, sv, iv in ((3, 11, 2, 4), (0, 23, 5, -2), (-7, -1, 3, 0), (5, 5, 1, 8)):
+        got = f(xv, av, bv, sv, iv)
+        ref = G.evaluate([x, a, b, s, i], outs, [xv, np.int64(av), np.int64(bv), np.int64(sv), np.int32(iv)])
+        for g, r in zip(got, ref):
+            assert_parity(g, r, "symbolic index %s" % ((av, bv, sv, iv),))
+        assert np.array_equal(got[1], xv[iv]) and np.array_equal(got[2], xv[::sv, 1:])
+    with pytest.raises(IndexError):
+        f(xv, 0, 1, 1, 9)
+
+    data = th.shared(rng.standard_normal((100, 16)).astype("float32"), name="data")
+    w = th.shared(np.zeros(16, "float32"), name="w")
+    n = 20
+    cost = T.mean(T.sqr(T.sum(x * w, axis=1) - 1.0))
+    step = th.function([i], cost, givens={x: data[i * n:(i + 1) * n]}, updates=[(w, w - 0.05 * th.grad(cost, w))])
+    dv, wv = data.get_value(), np.zeros(16, "float32")
+    for k in (0, 3, 4, 1):
+        batch = dv[k * n:(k + 1) * n]
+        r = batch @ wv - 1.0
+        want = np.mean(r * r)
+        wv = wv - 0.05 * (2.0 / n) * (batch.T @ r)
+        assert np.allclose(step(k), want, rtol=1e-4)
+    assert np.allclose(w.get_value(), wv, rtol=1e-4, atol=1e-6)
+    with pytest.raises(TypeError):
+        th.function([i], cost, givens={x: T.cast(data[i:i + 2], "float64")})

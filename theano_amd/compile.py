@@ -222,7 +222,7 @@ class Function(object):
         return list(self.nodes)
 
 
-def function(inputs, outputs, updates=None, fuse=True, rowchain=True, inplace=True, name=None,
+def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=True, inplace=True, name=None,
              on_unused_input="raise"):
     """Compile ``outputs`` as a function of ``inputs``.
 
@@ -231,7 +231,10 @@ def function(inputs, outputs, updates=None, fuse=True, rowchain=True, inplace=Tr
     variable, ``Out`` or a list of those; ``Out(v, device=True)`` leaves the
     result on the GPU.  ``updates``: pairs (or a dict) of shared variable and
     the expression whose value replaces its content after each call, as in
-    ``theano.function`` (``theano/compile/pfunc.py:60-230``).  Every op must
+    ``theano.function`` (``theano/compile/pfunc.py:60-230``).  ``givens``: pairs (or a
+    dict) of a variable and the expression of the same type that stands for it in this
+    function, e.g. ``{x: data[i * n:(i + 1) * n]}`` with ``data`` shared and ``i`` an
+    input (``theano/compile/pfunc.py:365-420``).  Every op must
     have a HIP implementation.  ``fuse=False``
     keeps one kernel per graph node; ``rowchain=False`` keeps elementwise /
     row-reduction islands as separate fused kernels; ``inplace=False`` gives
@@ -273,6 +276,20 @@ def function(inputs, outputs, updates=None, fuse=True, rowchain=True, inplace=Tr
                                 % (sv, sv.type, new, new.type))
             update_targets.append(sv)
             out_vars.append(new)
+    if givens:
+        pairs = list(givens.items()) if isinstance(givens, dict) else list(givens)
+        swap = {}
+        for var, rep in pairs:
+            if not isinstance(rep, Variable):
+                rep = as_tensor_variable(rep)
+            vt, rt = var.type, rep.type
+            if (getattr(vt, "dtype", None) != getattr(rt, "dtype", None) or
+                    tuple(getattr(vt, "broadcastable", ())) != tuple(getattr(rt, "broadcastable", ()))):
+                raise TypeError("Cannot use a shared variable or expression of type %s as a replacement for a "
+                                "variable of type %s in givens" % (rt, vt))
+            swap[var] = rep
+        memo = gof.clone_get_equiv([], out_vars, copy_inputs=False, memo=dict(swap))
+        out_vars = [memo[v] for v in out_vars]
     in_vars = [s.variable for s in in_specs]
     shared_inputs = [v for v in gof.graph_inputs(out_vars) if isinstance(v, SharedVariable)]
     used = set(id(v) for v in gof.graph_inputs(out_vars))

@@ -278,7 +278,8 @@ def clone_get_equiv(inputs, outputs, copy_inputs=True, memo=None):
         new_node = node.clone_with_new_inputs([memo[i] for i in node.inputs])
         memo[node] = new_node
         for o, no in zip(node.outputs, new_node.outputs):
-            memo[o] = no
+            if o not in memo:       # a variable the caller mapped to something else keeps that mapping
+                memo[o] = no
     for o in outputs:
         if o not in memo:
             memo[o] = o.clone() if (copy_inputs and o.owner is None and not isinstance(o, Constant)) else o

@@ -82,7 +82,9 @@ def lift_to_hip(fgraph):
                       hip_views.DEVICE_OPS):
             if isinstance(op, HostToHip) and isinstance(ins[0].type, HipArrayType):
                 outs = [ins[0]]
-            elif isinstance(op, HipToHost) and isinstance(ins[0].type, TensorType):
+            elif isinstance(op, HipToHost):
+                # transfers inside the graph are cut (theano/gpuarray/opt.py:566-737): every lifted
+                # consumer takes the device value, and results go back to the host at the outputs
                 outs = [ins[0]]
             else:
                 outs = op.make_node(*ins).outputs

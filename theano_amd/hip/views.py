@@ -69,32 +69,41 @@ def _as_device_value(v, dtype):
     return np.asarray(v, dtype=dtype).reshape((1,) * np.ndim(v))
 
 
+def _index_values(vals):
+    """Run-time values of an index's scalar inputs; one computed on the device (``i * n``) is
+    fetched, which waits for the kernels before it."""
+    return [v.to_numpy() if isinstance(v, HipArray) else v for v in vals]
+
+
 class HipSubtensor(V.Subtensor):
-    def make_node(self, x):
+    def make_node(self, x, *scalars):
         x = as_hip_variable(x)
-        if len(self.idx_list) != x.type.ndim:
-            raise IndexError("index of %d entries for a tensor of rank %d" % (len(self.idx_list), x.type.ndim))
-        return Apply(self, [x], [HipArrayType(x.type.dtype, self.out_broadcastable(x.type.broadcastable))()])
+        self.check_inputs(x, scalars)
+        return Apply(self, [x] + list(scalars),
+                     [HipArrayType(x.type.dtype, self.out_broadcastable(x.type.broadcastable))()])
 
     def perform(self, node, inputs, output_storage):
-        (x,) = inputs
-        shape, strides, offset = V.index_view(x.shape, x.strides, x.offset, self.idx_list)
+        x = inputs[0]
+        idx = V.resolve_index(self.idx_list, _index_values(inputs[1:])) if len(inputs) > 1 else self.idx_list
+        shape, strides, offset = V.index_view(x.shape, x.strides, x.offset, idx)
         output_storage[0][0] = x.view(shape, strides, offset)
 
 
 class HipIncSubtensor(V.IncSubtensor):
-    def make_node(self, x, y):
+    def make_node(self, x, y, *scalars):
         x = as_hip_variable(x)
         y = _device(y)
         if y.type.dtype != x.type.dtype:
             raise TypeError("the increment must have the dtype of the tensor (%s), got %s" % (x.type.dtype, y.type.dtype))
-        return Apply(self, [x, y], [x.type()])
+        V.Subtensor(self.idx_list).check_inputs(x, scalars)
+        return Apply(self, [x, y] + list(scalars), [x.type()])
 
     def perform(self, node, inputs, output_storage):
-        x, y = inputs
+        x, y = inputs[:2]
+        idx = V.resolve_index(self.idx_list, _index_values(inputs[2:])) if len(inputs) > 2 else self.idx_list
         out = HipArray.empty(x.shape, x.dtype)
         copy_into(x, out)
-        shape, strides, offset = V.index_view(out.shape, out.strides, out.offset, self.idx_list)
+        shape, strides, offset = V.index_view(out.shape, out.strides, out.offset, idx)
         region = out.view(shape, strides, offset)
         yv = _as_device_value(y, x.dtype)
         if region.size:

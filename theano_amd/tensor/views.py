@@ -23,9 +23,73 @@ def _no_host(op):
 
 
 # --------------------------------------------------------------------------
+class Sym(object):
+    """Place of the k-th scalar input of the node in an index: ``x[i]`` or ``x[a:b]`` with
+    integer scalar variables, read on the host when the function runs
+    (``theano/tensor/subtensor.py:318-420`` keeps scalar types in ``idx_list`` the same way)."""
+
+    __slots__ = ("k",)
+
+    def __init__(self, k):
+        self.k = int(k)
+
+    def __eq__(self, other):
+        return type(other) is Sym and other.k == self.k
+
+    def __hash__(self):
+        return hash(("Sym", self.k))
+
+    def __repr__(self):
+        return "i%d" % self.k
+
+
+def _is_index_variable(v):
+    if not hasattr(v, "type") or not hasattr(v, "owner"):
+        return False
+    dt = getattr(v.type, "dtype", "")
+    if getattr(v.type, "ndim", 0) != 0 or not (dt.startswith("int") or dt.startswith("uint")):
+        raise TypeError("a symbolic index must be an integer scalar, got %s" % (v.type,))
+    return True
+
+
+def split_symbolic(idx_list):
+    """(template, variables): every scalar variable in ``idx_list`` replaced by a ``Sym``."""
+    syms = []
+
+    def place(f):
+        if _is_index_variable(f):
+            for k, v in enumerate(syms):
+                if v is f:
+                    return Sym(k)
+            syms.append(f)
+            return Sym(len(syms) - 1)
+        return f
+
+    out = []
+    for i in idx_list:
+        if isinstance(i, slice):
+            out.append(slice(place(i.start), place(i.stop), place(i.step)))
+        else:
+            out.append(place(i))
+    return tuple(out), syms
+
+
+def resolve_index(template, values):
+    """The concrete index for the run-time ``values`` of the node's scalar inputs."""
+    def val(f):
+        return int(np.asarray(values[f.k])) if type(f) is Sym else f
+    return tuple(slice(val(i.start), val(i.stop), val(i.step)) if isinstance(i, slice) else val(i) for i in template)
+
+
+def n_symbolic(template):
+    ks = [f.k for i in template for f in ((i.start, i.stop, i.step) if isinstance(i, slice) else (i,)) if type(f) is Sym]
+    return max(ks) + 1 if ks else 0
+
+
 def normalize_index(idx, ndim):
     """A tuple of ints and slices (with int / None fields), one per indexed
-    dimension; Ellipsis expands, missing trailing dimensions are full slices."""
+    dimension; Ellipsis expands, missing trailing dimensions are full slices.
+    Integer scalar variables may stand where integers do."""
     if not isinstance(idx, tuple):
         idx = (idx,)
     if sum(1 for i in idx if i is Ellipsis) > 1:
@@ -41,15 +105,18 @@ def normalize_index(idx, ndim):
             out.extend([slice(None)] * (ndim - n_real))
         elif isinstance(i, slice):
             for f in (i.start, i.stop, i.step):
-                if f is not None and not isinstance(f, (int, np.integer)):
-                    raise NotImplementedError("slice bounds must be Python integers (got %r)" % (f,))
-            if i.step == 0:
+                if f is not None and not isinstance(f, (int, np.integer)) and not _is_index_variable(f):
+                    raise NotImplementedError("slice bounds must be integers or integer scalar variables (got %r)" % (f,))
+            if isinstance(i.step, (int, np.integer)) and i.step == 0:
                 raise ValueError("slice step cannot be zero")
-            out.append(slice(*[None if f is None else int(f) for f in (i.start, i.stop, i.step)]))
+            out.append(slice(*[f if (f is None or hasattr(f, "type")) else int(f) for f in (i.start, i.stop, i.step)]))
         elif isinstance(i, (int, np.integer)):
             out.append(int(i))
+        elif _is_index_variable(i):
+            out.append(i)
         else:
-            raise NotImplementedError("only integers and slices index a tensor here (got %r)" % (i,))
+            raise NotImplementedError("only integers, integer scalar variables and slices index a tensor here "
+                                      "(got %r)" % (i,))
     out.extend([slice(None)] * (ndim - len(out)))
     return tuple(out)
 
@@ -79,8 +146,13 @@ def _idx_key(idx_list):
     return tuple(("s", i.start, i.stop, i.step) if isinstance(i, slice) else ("i", i) for i in idx_list)
 
 
+def _full_slice(i):
+    return isinstance(i, slice) and i.start is None and i.stop is None and i.step is None
+
+
 class Subtensor(Op):
-    """``x[idx_list]`` with integers and constant slices: a view
+    """``x[idx_list]`` with integers and slices, constant or given by integer scalar
+    variables (the node's further inputs): a view
     (``theano/tensor/subtensor.py:318-780``; ``view_map = {0: [0]}`` :513)."""
 
     __props__ = ("idx_key",)
@@ -102,30 +174,43 @@ class Subtensor(Op):
 
     def out_broadcastable(self, in_broadcastable):
         # a full slice keeps the flag (theano/tensor/subtensor.py:470-500); any other slice may be empty
-        return tuple(b and i == slice(None) for b, i in zip(in_broadcastable, self.idx_list) if isinstance(i, slice))
+        return tuple(b and _full_slice(i) for b, i in zip(in_broadcastable, self.idx_list) if isinstance(i, slice))
 
-    def make_node(self, x):
-        x = as_tensor_variable(x)
+    def check_inputs(self, x, scalars):
         if len(self.idx_list) != x.type.ndim:
             raise IndexError("index of %d entries for a tensor of rank %d" % (len(self.idx_list), x.type.ndim))
-        return Apply(self, [x], [TensorType(x.type.dtype, self.out_broadcastable(x.type.broadcastable))()])
+        if len(scalars) != n_symbolic(self.idx_list):
+            raise ValueError("the index names %d scalar inputs, %d were given" % (n_symbolic(self.idx_list), len(scalars)))
+        for v in scalars:
+            _is_index_variable(v)
+
+    def make_node(self, x, *scalars):
+        x = as_tensor_variable(x)
+        scalars = [as_tensor_variable(v) for v in scalars]
+        self.check_inputs(x, scalars)
+        return Apply(self, [x] + scalars, [TensorType(x.type.dtype, self.out_broadcastable(x.type.broadcastable))()])
 
     def infer_shape(self, node, shapes):
+        if n_symbolic(self.idx_list):
+            raise NotImplementedError("the shape of a symbolic slice is known only when the function runs")
         shape, _, _ = index_view(shapes[0], [1] * len(shapes[0]), 0, self.idx_list)
         return [shape]
 
     def perform(self, node, inputs, output_storage):
         _no_host(self)
 
+    def connection_pattern(self, node):
+        return [[True]] + [[False]] * (len(node.inputs) - 1)
+
     def L_op(self, inputs, outputs, grads):
-        (x,) = inputs
+        x = inputs[0]
         (g,) = grads
-        return [IncSubtensor(self.idx_list)(x.zeros_like(), g)]
+        return [IncSubtensor(self.idx_list)(x.zeros_like(), g, *inputs[1:])] + [T.scal.DisconnectedType()() for _ in inputs[1:]]
 
     def R_op(self, inputs, eval_points):
         if eval_points[0] is None:
             return [None]
-        return [self(eval_points[0])]
+        return [self(eval_points[0], *inputs[1:])]
 
 
 class IncSubtensor(Op):
@@ -147,14 +232,18 @@ class IncSubtensor(Op):
         return "%s{%s;%s}" % (type(self).__name__, "Set" if self.set_instead_of_inc else "Inc",
                               str(Subtensor(self.idx_list))[len("Subtensor{"):-1])
 
-    def make_node(self, x, y):
+    def make_node(self, x, y, *scalars):
         x, y = as_tensor_variable(x), as_tensor_variable(y)
+        scalars = [as_tensor_variable(v) for v in scalars]
         if y.type.dtype != x.type.dtype:
             y = T.cast(y, x.type.dtype)
-        sub = Subtensor(self.idx_list).make_node(x).outputs[0]
+        sub = Subtensor(self.idx_list).make_node(x, *scalars).outputs[0]
         if y.type.ndim > sub.type.ndim:
             raise TypeError("the increment has rank %d, the indexed region rank %d" % (y.type.ndim, sub.type.ndim))
-        return Apply(self, [x, y], [x.type()])
+        return Apply(self, [x, y] + scalars, [x.type()])
+
+    def connection_pattern(self, node):
+        return [[True], [True]] + [[False]] * (len(node.inputs) - 2)
 
     def infer_shape(self, node, shapes):
         return [shapes[0]]
@@ -165,12 +254,13 @@ class IncSubtensor(Op):
     def R_op(self, inputs, eval_points):
         if None in eval_points[:2]:
             return [None]
-        return [self(eval_points[0], eval_points[1])]
+        return [self(eval_points[0], eval_points[1], *inputs[2:])]
 
     def L_op(self, inputs, outputs, grads):
-        x, y = inputs
+        x, y = inputs[:2]
+        scalars = list(inputs[2:])
         (g,) = grads
-        gy = Subtensor(self.idx_list)(g)
+        gy = Subtensor(self.idx_list)(g, *scalars)
         # y may have been broadcast into the region: sum the gradient back (subtensor.py:1520-1560)
         sub_ndim = gy.type.ndim
         if y.type.ndim < sub_ndim:
@@ -179,18 +269,19 @@ class IncSubtensor(Op):
         if bdims:
             gy = T.sum(gy, axis=tuple(bdims), keepdims=True)
         if self.set_instead_of_inc:
-            gx = IncSubtensor(self.idx_list, True)(g, T.zeros_like(Subtensor(self.idx_list)(g)))
+            gx = IncSubtensor(self.idx_list, True)(g, T.zeros_like(Subtensor(self.idx_list)(g, *scalars)), *scalars)
         else:
             gx = g
-        return [gx, gy]
+        return [gx, gy] + [T.scal.DisconnectedType()() for _ in scalars]
 
 
 def subtensor(x, idx):
     x = as_tensor_variable(x)
     idx_list = normalize_index(idx, x.type.ndim)
-    if all(i == slice(None) for i in idx_list):
+    if all(_full_slice(i) for i in idx_list):
         return x
-    return Subtensor(idx_list)(x)
+    template, syms = split_symbolic(idx_list)
+    return Subtensor(template)(x, *syms)
 
 
 def _inc_or_set(x, y, idx, set_instead_of_inc):
@@ -200,10 +291,10 @@ def _inc_or_set(x, y, idx, set_instead_of_inc):
         # indexed view, the op is applied to what it indexes (theano/tensor/subtensor.py:1040-1110)
         if x.owner is None or not isinstance(x.owner.op, Subtensor):
             raise TypeError("x must be the result of a subtensor operation (or pass the index as third argument)")
-        idx_list, x = x.owner.op.idx_list, x.owner.inputs[0]
+        template, syms, x = x.owner.op.idx_list, list(x.owner.inputs[1:]), x.owner.inputs[0]
     else:
-        idx_list = normalize_index(idx, x.type.ndim)
-    return IncSubtensor(idx_list, set_instead_of_inc)(x, y)
+        template, syms = split_symbolic(normalize_index(idx, x.type.ndim))
+    return IncSubtensor(template, set_instead_of_inc)(x, y, *syms)
 
 
 def inc_subtensor(x, y, idx=None):
