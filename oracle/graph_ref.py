@@ -299,6 +299,9 @@ def evaluate(inputs, outputs, values):
             res = [np.array(np.broadcast_to(args[0], op.resolve([a.shape for a in args])))]
         elif isinstance(op, V.Join):
             res = [np.concatenate(args, axis=op.axis)]
+        elif isinstance(op, V.Rebroadcast):        # theano/compile/ops.py:711-722
+            op.check(args[0].shape)
+            res = [args[0]]
         elif isinstance(op, V.JoinPart):
             at = sum(a.shape[op.axis] for a in args[1:1 + op.k])
             idx = [slice(None)] * args[0].ndim

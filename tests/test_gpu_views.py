@@ -164,3 +164,25 @@ def test_symbolic_slices_and_givens_minibatches():
     assert np.allclose(w.get_value(), wv, rtol=1e-4, atol=1e-6)
     with pytest.raises(TypeError):
         th.function([i], cost, givens={x: T.cast(data[i:i + 2], "float64")})
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("k", range(5))
+def test_composed_front_ends_on_the_device(k):
+    """power / square / sign / rint / deg2rad / ptp, largest / smallest, isclose / allclose,
+    floor_div / ceil_intdiv, the shape helpers, stacks, split, zeros / ones and Rebroadcast
+    through the HIP path against NumPy (the cases of tests/test_oracle_graph.py)."""
+    from test_oracle_graph import _front_end_cases
+    name, ins, outs, vals, want = _front_end_cases()[k]
+    got = th.function(ins, outs)(*vals)
+    for g, w in zip(got, want):
+        w = np.asarray(w)
+        assert g.shape == w.shape, (name, g.shape, w.shape)
+        if w.dtype.kind in "biu":
+            assert np.array_equal(g, w), name
+        else:
+            assert np.allclose(g, w, rtol=1e-12, equal_nan=True), name
+    if k == 4:
+        x = T.dmatrix("x")
+        with pytest.raises(ValueError):
+            th.function([x], T.addbroadcast(x, 0) * 2.0)(np.zeros((2, 3)))

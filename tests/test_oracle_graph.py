@@ -418,3 +418,66 @@ def test_clip_and_switch_gradients():
     num = numeric_grad(lambda *a: float(G.evaluate([x, lo, hi], [cost], list(a))[0]), vals)
     for a, n in zip(G.evaluate([x, lo, hi], grads, vals), num):
         assert np.allclose(a, n, rtol=2e-5, atol=1e-7)
+
+
+def _front_end_cases():
+    """(name, inputs, outputs builder, values, NumPy answers) for the composed front ends."""
+    rng = np.random.default_rng(21)
+    x, y = T.dmatrix("x"), T.dmatrix("y")
+    i, j = T.lmatrix("i"), T.lmatrix("j")
+    xv, yv = rng.standard_normal((4, 6)), rng.standard_normal((4, 6))
+    yv[0, :3] = xv[0, :3] * (1 + 1e-7)
+    xn, yn = xv.copy(), yv.copy()
+    xn[1, 0] = yn[1, 0] = np.nan
+    xn[1, 1] = yn[1, 1] = np.inf
+    xn[1, 2], yn[1, 2] = np.inf, -np.inf
+    iv, jv = rng.integers(-20, 20, (4, 6)), rng.integers(1, 7, (4, 6)) * rng.choice([-1, 1], (4, 6))
+    r = T.TensorType("float64", (False, False, False))("r")
+    rv = rng.standard_normal((2, 1, 5))
+    return [
+        ("named ops", [x, y], [T.power(abs(x), y), T.square(x), T.absolute(x), T.sign(x), T.rint(x * 3), T.deg2rad(x),
+                               T.rad2deg(x), T.ptp(x, axis=1), T.ptp(x)], [xv, yv],
+         [np.abs(xv) ** yv, xv * xv, np.abs(xv), np.sign(xv), np.rint(xv * 3), np.deg2rad(xv), np.rad2deg(xv),
+          np.ptp(xv, axis=1), np.ptp(xv)]),
+        ("largest / smallest", [x, y], [T.largest(x, y), T.smallest(x, y), T.largest(x, y, x * y), T.smallest(x, y, x - y)],
+         [xv, yv], [np.maximum(xv, yv), np.minimum(xv, yv), np.maximum(np.maximum(xv, yv), xv * yv),
+                    np.minimum(np.minimum(xv, yv), xv - yv)]),
+        ("isclose / allclose", [x, y], [T.isclose(x, y), T.isclose(x, y, equal_nan=True), T.allclose(x, y),
+                                        T.allclose(x, x + 1e-12)], [xn, yn],
+         [np.isclose(xn, yn), np.isclose(xn, yn, equal_nan=True), np.allclose(xn, yn), False]),
+        ("integer division", [i, j], [T.floor_div(i, j), T.ceil_intdiv(i, j)], [iv, jv],
+         [iv // jv, -((-iv) // jv)]),
+        ("shape helpers", [x, r], [T.shape_padleft(x, 2), T.shape_padright(x), T.shape_padaxis(x, 1), T.transpose(x),
+                                   T.transpose(r, (2, 0, 1)), T.swapaxes(r, 0, 2), T.zeros((3, x.shape[1])) + x[:3],
+                                   T.ones((2, 2), "int8"), T.vertical_stack(x, x * 2), T.horizontal_stack(x, x[:, :1])] +
+         T.split(x, [1, 3, 2], 3, axis=1) + [T.addbroadcast(r[:, :1], 1) + r, T.unbroadcast(T.shape_padleft(x), 0)],
+         [xv, rv],
+         [xv[None, None], xv[:, :, None], xv[:, None, :], xv.T, rv.transpose(2, 0, 1), rv.swapaxes(0, 2),
+          xv[:3].astype("float64"), np.ones((2, 2), "int8"), np.vstack([xv, xv * 2]), np.hstack([xv, xv[:, :1]]),
+          xv[:, :1], xv[:, 1:4], xv[:, 4:], rv + rv, xv[None]]),
+    ]
+
+
+@pytest.mark.parametrize("k", range(5))
+def test_composed_front_ends_against_numpy(k):
+    name, ins, outs, vals, want = _front_end_cases()[k]
+    with np.errstate(all="ignore"):
+        got = G.evaluate(ins, outs, vals)
+    for g, w in zip(got, want):
+        w = np.asarray(w)
+        assert g.shape == w.shape, (name, g.shape, w.shape)
+        assert np.allclose(g, w, rtol=1e-12, equal_nan=True), name
+
+
+def test_rebroadcast_checks_extents_and_keeps_gradients():
+    x = T.dmatrix("x")
+    b = T.addbroadcast(x, 0)
+    assert b.type.broadcastable == (True, False) and str(b.owner.op) == "Rebroadcast{1}"
+    assert T.addbroadcast(b, 0) is b and T.patternbroadcast(x, (False, False)) is x
+    with pytest.raises(ValueError):
+        G.evaluate([x], [b], [np.zeros((2, 3))])
+    y = T.drow("y")
+    g = th.grad(T.sum(T.unbroadcast(y, 0) * 3.0), y)
+    assert g.type == y.type and np.allclose(G.evaluate([y], [g], [np.ones((1, 4))])[0], 3.0)
+    with pytest.raises(ValueError):
+        T.addbroadcast(x, 2)

@@ -89,6 +89,20 @@ class HipSubtensor(V.Subtensor):
         output_storage[0][0] = x.view(shape, strides, offset)
 
 
+class HipRebroadcast(V.Rebroadcast):
+    def __init__(self, axis):
+        V.Rebroadcast.__init__(self, *axis)
+
+    def make_node(self, x):
+        x = as_hip_variable(x)
+        return Apply(self, [x], [HipArrayType(x.type.dtype, self.out_type(x))()])
+
+    def perform(self, node, inputs, output_storage):
+        (x,) = inputs
+        self.check(x.shape)
+        output_storage[0][0] = x
+
+
 class HipIncSubtensor(V.IncSubtensor):
     def make_node(self, x, y, *scalars):
         x = as_hip_variable(x)
@@ -206,5 +220,6 @@ LIFT = {V.Subtensor: lambda op: HipSubtensor(op.idx_list),
         V.Reshape: lambda op: HipReshape(op.pattern),
         V.Alloc: lambda op: HipAlloc(op.pattern),
         V.Join: lambda op: HipJoin(op.axis),
-        V.JoinPart: lambda op: HipJoinPart(op.axis, op.k)}
-DEVICE_OPS = (HipSubtensor, HipIncSubtensor, HipReshape, HipAlloc, HipJoin, HipJoinPart)
+        V.JoinPart: lambda op: HipJoinPart(op.axis, op.k),
+        V.Rebroadcast: lambda op: HipRebroadcast(op.axis)}
+DEVICE_OPS = (HipSubtensor, HipIncSubtensor, HipReshape, HipAlloc, HipJoin, HipJoinPart, HipRebroadcast)

@@ -12,5 +12,6 @@ from .elemwise import DimShuffle, Elemwise, CAReduce, CAReduceDtype, Sum, Prod, 
 from .basic import *  # noqa: F401,F403
 from .basic import Max, MaxAndArgmax, Min, ShapeFloat, makeKeepDims, cast, round  # noqa: F401
 from . import nnet  # noqa: F401,E402
-from .views import (Alloc, IncSubtensor, Join, Reshape, Subtensor, alloc, concatenate, flatten, inc_subtensor,  # noqa: F401,E402
-                    join, reshape, set_subtensor, stack, subtensor)
+from .views import (Alloc, IncSubtensor, Join, Rebroadcast, Reshape, Subtensor, addbroadcast, alloc,  # noqa: F401,E402
+                    concatenate, flatten, horizontal_stack, inc_subtensor, join, patternbroadcast, reshape,
+                    set_subtensor, split, stack, subtensor, unbroadcast, vertical_stack)

@@ -437,3 +437,126 @@ def softmax(x):
     x = as_tensor_variable(x)
     e = exp(x - max(x, axis=-1, keepdims=True))
     return e / sum(e, axis=-1, keepdims=True)
+
+
+# ---- further front ends of theano/tensor/basic.py, all compositions of the ops above ---------------
+floor_div, power, square, absolute, sign = int_div, pow, sqr, abs_, sgn
+rint = round_half_to_even
+
+
+def deg2rad(a):
+    """``a * (pi / 180)`` (``theano/scalar/basic.py:2845-2862``)."""
+    a = as_tensor_variable(a)
+    dt = a.type.dtype if a.type.dtype in scal.float_dtypes else scal.upgrade_to_float(scal.Scalar(a.type.dtype))[0].dtype
+    return cast(a, dt) * np.asarray(np.pi / 180.0, dt)
+
+
+def rad2deg(a):
+    """``a * (180 / pi)`` (``theano/scalar/basic.py:2874-2891``)."""
+    a = as_tensor_variable(a)
+    dt = a.type.dtype if a.type.dtype in scal.float_dtypes else scal.upgrade_to_float(scal.Scalar(a.type.dtype))[0].dtype
+    return cast(a, dt) * np.asarray(180.0 / np.pi, dt)
+
+
+def smallest(*args):
+    """Elementwise smallest of the arguments (``theano/tensor/basic.py:1809-1820``)."""
+    if len(args) == 2:
+        a, b = args
+        return switch(lt(a, b), a, b)
+    from .views import stack
+    return min(stack(list(args)), axis=0)
+
+
+def largest(*args):
+    """Elementwise largest of the arguments (``theano/tensor/basic.py:1824-1835``)."""
+    if len(args) == 2:
+        a, b = args
+        return switch(gt(a, b), a, b)
+    from .views import stack
+    return max(stack(list(args)), axis=0)
+
+
+def ceil_intdiv(a, b):
+    """``ceil(a / b)`` without leaving the integers (``theano/tensor/basic.py:3601-3620``)."""
+    div = int_div(a, b)
+    return cast(neq(mod(a, b), 0), div.type.dtype) + div
+
+
+def isclose(a, b, rtol=1.e-5, atol=1.e-8, equal_nan=False):
+    """``numpy.isclose`` as a graph (``theano/tensor/basic.py:1942-2030``): within tolerance and
+    neither NaN nor infinite, or infinities of the same sign, or (``equal_nan``) both NaN."""
+    a, b = as_tensor_variable(a), as_tensor_variable(b)
+    close_prelim = le(abs_(a - b), atol + rtol * abs_(b))
+    a_nan, b_nan = isnan(a), isnan(b)
+    a_inf, b_inf = isinf(a), isinf(b)
+    nans_or_infs = or_(or_(a_nan, b_nan), or_(a_inf, b_inf))
+    close = and_(close_prelim, invert(nans_or_infs))
+    inf_eq = and_(and_(a_inf, b_inf), eq(a_inf * sgn(a), b_inf * sgn(b)))
+    close_with_infs = or_(close, inf_eq)
+    if equal_nan:
+        return or_(close_with_infs, and_(a_nan, b_nan))
+    return close_with_infs
+
+
+def allclose(a, b, rtol=1.e-5, atol=1.e-8, equal_nan=False):
+    """``all(isclose(a, b))`` (``theano/tensor/basic.py:1908-1939``)."""
+    return all(isclose(a, b, rtol, atol, equal_nan))
+
+
+def ptp(a, axis=None):
+    """Range of values, ``max - min`` along an axis (``theano/tensor/basic.py:6722-6746``)."""
+    a = as_tensor_variable(a)
+    return max(a, axis) - min(a, axis)
+
+
+def shape_padleft(t, n_ones=1):
+    """``theano/tensor/basic.py:4559-4573``"""
+    t = as_tensor_variable(t)
+    return t.dimshuffle(*(["x"] * n_ones + list(range(t.type.ndim))))
+
+
+def shape_padright(t, n_ones=1):
+    """``theano/tensor/basic.py:4576-4590``"""
+    t = as_tensor_variable(t)
+    return t.dimshuffle(*(list(range(t.type.ndim)) + ["x"] * n_ones))
+
+
+def shape_padaxis(t, axis):
+    """A broadcastable dimension inserted at ``axis`` (``theano/tensor/basic.py:4593-4630``)."""
+    t = as_tensor_variable(t)
+    nd = t.type.ndim + 1
+    if not -nd <= axis < nd:
+        raise IndexError("axis {0} is out of bounds [-{1}, {1})".format(axis, nd))
+    axis = axis + nd if axis < 0 else axis
+    pattern = list(range(t.type.ndim))
+    pattern.insert(axis, "x")
+    return t.dimshuffle(*pattern)
+
+
+def transpose(x, axes=None):
+    """``theano/tensor/basic.py:3701-3716``"""
+    x = as_tensor_variable(x)
+    axes = list(range(x.type.ndim - 1, -1, -1)) if axes is None else list(axes)
+    return x.dimshuffle(*axes)
+
+
+def swapaxes(y, axis1, axis2):
+    """``theano/tensor/basic.py:6753-6760``"""
+    y = as_tensor_variable(y)
+    order = list(range(y.type.ndim))
+    order[axis1], order[axis2] = order[axis2], order[axis1]
+    return y.dimshuffle(*order)
+
+
+def zeros(shape, dtype=None):
+    """``alloc(0, *shape)`` (``theano/tensor/basic.py:2550-2558``); entries: ints or ``v.shape[d]``."""
+    from .views import alloc
+    shape = list(shape) if isinstance(shape, (list, tuple)) else [shape]
+    return alloc(np.array(0, dtype=dtype or config.floatX), *shape)
+
+
+def ones(shape, dtype=None):
+    """``alloc(1, *shape)`` (``theano/tensor/basic.py:2561-2569``)."""
+    from .views import alloc
+    shape = list(shape) if isinstance(shape, (list, tuple)) else [shape]
+    return alloc(np.array(1, dtype=dtype or config.floatX), *shape)

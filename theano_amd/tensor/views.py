@@ -649,3 +649,125 @@ def stack(tensors, axis=0):
     order = list(range(nd))
     order.insert(axis, "x")
     return join(axis, *[t.dimshuffle(*order) for t in ts])
+
+
+def horizontal_stack(*args):
+    """``concatenate(args, axis=1)`` of matrices (``theano/tensor/basic.py:4832-4851``)."""
+    for a in args:
+        if as_tensor_variable(a).type.ndim != 2:
+            raise ValueError("Too many dimensions for horizontal_stack: use join")
+    return concatenate(list(args), axis=1)
+
+
+def vertical_stack(*args):
+    """``concatenate(args, axis=0)`` of matrices (``theano/tensor/basic.py:4854-4865``)."""
+    for a in args:
+        if as_tensor_variable(a).type.ndim != 2:
+            raise ValueError("Too many dimensions for vertical_stack: use join")
+    return concatenate(list(args), axis=0)
+
+
+def split(x, splits_size, n_splits, axis=0):
+    """The ``n_splits`` consecutive parts of ``x`` along ``axis`` with the given (constant)
+    lengths, as views (``theano/tensor/basic.py:3794-3797``; the reference's ``Split`` also takes
+    symbolic lengths and checks that they add up to the extent when it runs)."""
+    x = as_tensor_variable(x)
+    sizes = [int(v) for v in splits_size]
+    if len(sizes) != n_splits:
+        raise ValueError("In Split.perform(), len(splits) != len_splits.", (len(sizes), n_splits))
+    axis = axis + x.type.ndim if axis < 0 else axis
+    parts, at = [], 0
+    for n in sizes:
+        idx = [slice(None)] * x.type.ndim
+        idx[axis] = slice(at, at + n)
+        parts.append(x[tuple(idx)])
+        at += n
+    return parts
+
+
+class Rebroadcast(Op):
+    """The same array with another static broadcast pattern: ``(axis, flag)`` pairs; making a
+    dimension broadcastable is checked against its extent when the function runs
+    (``theano/compile/ops.py:647-760``).  A view."""
+
+    __props__ = ("axis",)
+    view_map = {0: [0]}
+
+    def __init__(self, *axis):
+        items = sorted((int(a), bool(b)) for a, b in axis)
+        self.axis = tuple(items)
+
+    def _props(self):
+        return (self.axis,)
+
+    def __str__(self):
+        flags = dict(self.axis)
+        pattern = ["?"] * (1 + builtins_max(flags)) if flags else []
+        for k, v in flags.items():
+            pattern[k] = str(int(v))
+        return "%s{%s}" % (type(self).__name__, ",".join(pattern))
+
+    def out_type(self, x):
+        flags = dict(self.axis)
+        if flags and x.type.ndim <= builtins_max(flags):
+            raise ValueError("Trying to rebroadcast non-existent dimension")
+        return [flags.get(i, b) for i, b in enumerate(x.type.broadcastable)]
+
+    def make_node(self, x):
+        x = as_tensor_variable(x)
+        return Apply(self, [x], [TensorType(x.type.dtype, self.out_type(x))()])
+
+    def check(self, shape):
+        for a, flag in self.axis:
+            if flag and shape[a] != 1:
+                raise ValueError("Dimension %s in Rebroadcast's input was supposed to be 1 (got %s instead)" % (a, shape[a]))
+
+    def perform(self, node, inputs, output_storage):
+        _no_host(self)
+
+    def infer_shape(self, node, shapes):
+        return [tuple(1 if dict(self.axis).get(d) else s for d, s in enumerate(shapes[0]))]
+
+    def L_op(self, inputs, outputs, grads):
+        # restore the input's pattern (theano/compile/ops.py:724-732)
+        (x,) = inputs
+        (g,) = grads
+        return [Rebroadcast(*[(a, x.type.broadcastable[a]) for a, _ in self.axis])(g)]
+
+    def R_op(self, inputs, eval_points):
+        if eval_points[0] is None:
+            return [None]
+        return [self(eval_points[0])]
+
+
+def builtins_max(d):
+    import builtins
+    return builtins.max(d)
+
+
+def addbroadcast(x, *axes):
+    """``theano/tensor/basic.py:4066-4093``"""
+    x = as_tensor_variable(x)
+    if any(a >= x.type.ndim for a in axes):
+        raise ValueError("Trying to rebroadcast non-existent dimension")
+    if all(x.type.broadcastable[a] for a in axes):
+        return x
+    return Rebroadcast(*[(a, True) for a in axes])(x)
+
+
+def unbroadcast(x, *axes):
+    """``theano/tensor/basic.py:4096-4123``"""
+    x = as_tensor_variable(x)
+    if any(a >= x.type.ndim for a in axes):
+        raise ValueError("Trying to rebroadcast non-existent dimension")
+    if not any(x.type.broadcastable[a] for a in axes):
+        return x
+    return Rebroadcast(*[(a, False) for a in axes])(x)
+
+
+def patternbroadcast(x, broadcastable):
+    """``theano/tensor/basic.py:4126-4153``"""
+    x = as_tensor_variable(x)
+    if tuple(x.type.broadcastable) == tuple(bool(b) for b in broadcastable):
+        return x
+    return Rebroadcast(*[(i, bool(b)) for i, b in enumerate(broadcastable)])(x)
