@@ -145,7 +145,11 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); got --gpus %d" % args.gpus)
 
-    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    root = os.path.dirname(os.path.abspath(__file__))
+    sys.path.insert(0, root)
+    if not os.path.exists(os.path.join(root, "theano_amd", "csrc", "libthx_hip.so")):   # a fresh checkout
+        from theano_amd.csrc import build as lib_build
+        lib_build.build()
     import theano_amd as th
     from theano_amd import hip
     import workloads as W

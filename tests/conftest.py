@@ -11,6 +11,10 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    # the tests load the library that is built; only where none is (a fresh checkout) do they build it
+    if not os.path.exists(os.path.join(ROOT, "theano_amd", "csrc", "libthx_hip.so")):
+        from theano_amd.csrc import build as lib_build
+        lib_build.build()
 
 
 # tolerances of the parity bar, by storage dtype
