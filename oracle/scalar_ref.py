@@ -377,6 +377,35 @@ def tri_gamma(out_dtype, x):
         return _conv(scipy.special.polygamma(1, _conv(x, ct)), out_dtype)
 
 
+j0, j1, i0, i1 = _special("j0"), _special("j1"), _special("i0"), _special("i1")
+
+
+def _special2(fn):
+    """Binary scipy functions: both arguments in the output's compute type."""
+    def f(out_dtype, a, b):
+        ct = "float32" if str(out_dtype) == "float16" else out_dtype
+        with np.errstate(all="ignore"):
+            return _conv(fn(_conv(a, ct).astype("float64"), _conv(b, ct).astype("float64")), out_dtype)
+    return f
+
+
+def _sp():
+    import scipy.special
+    return scipy.special
+
+
+gammainc = _special2(lambda k, x: _sp().gammainc(k, x))
+gammaincc = _special2(lambda k, x: _sp().gammaincc(k, x))
+gammau = _special2(lambda k, x: _sp().gammaincc(k, x) * _sp().gamma(k))       # basic_scipy.py:631-632
+gammal = _special2(lambda k, x: _sp().gammainc(k, x) * _sp().gamma(k))        # basic_scipy.py:674-675
+
+
+def chi2sf(out_dtype, x, k):
+    import scipy.stats
+    with np.errstate(all="ignore"):
+        return _conv(scipy.stats.chi2.sf(np.asarray(x, "float64"), np.asarray(k, "float64")), out_dtype)
+
+
 def arctan2(out_dtype, y, x):
     ct = "float32" if str(out_dtype) == "float16" else out_dtype
     return _conv(np.arctan2(_conv(y, ct), _conv(x, ct)), out_dtype)
@@ -424,5 +453,6 @@ BY_CLASS = {
     "ArcSin": arcsin, "ArcTan": arctan, "ArcTan2": arctan2, "Cosh": cosh, "Sinh": sinh, "Tanh": tanh,
     "ArcCosh": arccosh, "ArcSinh": arcsinh, "ArcTanh": arctanh, "ScalarSigmoid": scalar_sigmoid,
     "ScalarSoftplus": scalar_softplus, "Erf": erf, "Erfc": erfc, "Erfcx": erfcx, "Erfinv": erfinv, "Erfcinv": erfcinv,
-    "Gamma": gamma, "GammaLn": gammaln, "Psi": psi, "TriGamma": tri_gamma,
+    "Gamma": gamma, "GammaLn": gammaln, "Psi": psi, "TriGamma": tri_gamma, "J0": j0, "J1": j1, "I0": i0, "I1": i1,
+    "GammaInc": gammainc, "GammaIncC": gammaincc, "GammaU": gammau, "GammaL": gammal, "Chi2SF": chi2sf,
 }

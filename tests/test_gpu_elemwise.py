@@ -308,3 +308,37 @@ def test_exact_float32_math_when_the_fast_forms_are_switched_off(monkeypatch):
     assert np.max(np.abs(exact[3][ok] - s64[ok]) / s64[ok]) < 4e-7
     for f, e in zip(fast, exact):
         assert np.allclose(f, e, rtol=1e-5, atol=1e-37)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+def test_bessel_and_incomplete_gamma_functions_against_scipy(dtype):
+    """j0 / j1 / i0 / i1 and gammainc / gammaincc / gammau / gammal / chi2sf
+    (theano/scalar/basic_scipy.py:482-857) against scipy, which the reference's impl calls."""
+    import scipy.special
+    import scipy.stats
+    rng = np.random.default_rng(23)
+    tol = dict(rtol=2e-5, atol=2e-6) if dtype == "float32" else dict(rtol=1e-10, atol=1e-13)
+    x = T.TensorType(dtype, (False,))("x")
+    k = T.TensorType(dtype, (False,))("k")
+    xv = np.concatenate([rng.uniform(-12, 12, 4000), [0.0]]).astype(dtype)
+    got = th.function([x], [T.j0(x), T.j1(x), T.i0(x), T.i1(x), th.grad(T.sum(T.j1(x)), x), th.grad(T.sum(T.i1(x)), x)])(xv)
+    x64 = xv.astype("float64")
+    want = [scipy.special.j0(x64), scipy.special.j1(x64), scipy.special.i0(x64), scipy.special.i1(x64),
+            scipy.special.jvp(1, x64), scipy.special.ivp(1, x64)]
+    for g, w in zip(got, want):
+        assert g.dtype == np.dtype(dtype) and np.allclose(g, w, **tol)
+    kv = rng.uniform(0.1, 40, 6000).astype(dtype)
+    pv = np.concatenate([rng.uniform(0.01, 80, 5998), [0.0, 1e-3]]).astype(dtype)
+    outs = [T.gammainc(k, x), T.gammaincc(k, x), T.gammal(k, x), T.gammau(k, x), T.chi2sf(x, k)]
+    got = th.function([k, x], outs)(kv, pv)
+    k64, p64 = kv.astype("float64"), pv.astype("float64")
+    want = [scipy.special.gammainc(k64, p64), scipy.special.gammaincc(k64, p64),
+            scipy.special.gammainc(k64, p64) * scipy.special.gamma(k64),
+            scipy.special.gammaincc(k64, p64) * scipy.special.gamma(k64), scipy.stats.chi2.sf(p64, k64)]
+    for j, (g, w) in enumerate(zip(got, want)):
+        assert g.dtype == np.dtype("float64" if j == 4 else dtype), j
+        assert np.allclose(g, w.astype(g.dtype), rtol=tol["rtol"] * 5, atol=tol["atol"]), j
+    ref = G.evaluate([k, x], outs, [kv, pv])
+    for g, r in zip(got, ref):
+        assert np.allclose(g, r, rtol=tol["rtol"] * 5, atol=tol["atol"])

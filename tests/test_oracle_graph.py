@@ -378,6 +378,7 @@ UNARY_GRAD_CASES = [
     ("sinh", -2, 2), ("cosh", -2, 2), ("tanh", -2, 2), ("arcsinh", -2, 2), ("arccosh", 1.5, 3), ("arctanh", -0.9, 0.9),
     ("sigmoid", -3, 3), ("softplus", -3, 3), ("erf", -2, 2), ("erfc", -2, 2), ("erfcx", -1, 2), ("erfinv", -0.9, 0.9),
     ("erfcinv", 0.1, 1.9), ("gamma", 0.5, 3), ("gammaln", 0.5, 3), ("psi", 0.5, 3),
+    ("j0", -6, 6), ("j1", -6, 6), ("i0", -3, 3), ("i1", -3, 3),
 ]
 BINARY_GRAD_CASES = [
     ("add", -2, 2, -2, 2), ("sub", -2, 2, -2, 2), ("mul", -2, 2, -2, 2), ("true_div", -2, 2, 0.5, 2),

@@ -118,6 +118,56 @@ __device__ inline double thx_trigamma(double x) {
 }
 __device__ inline float thx_trigamma(float x) { return (float)thx_trigamma((double)x); }
 
+// Modified Bessel functions of the first kind for any sign of the argument: the device library's
+// cyl_bessel_i1 gives NaN below zero; I0 is even and I1 odd.
+__device__ inline double thx_i0(double x) { return cyl_bessel_i0(fabs(x)); }
+__device__ inline float thx_i0(float x) { return cyl_bessel_i0f(fabsf(x)); }
+__device__ inline double thx_i1(double x) { return copysign(cyl_bessel_i1(fabs(x)), x); }
+__device__ inline float thx_i1(float x) { return copysignf(cyl_bessel_i1f(fabsf(x)), x); }
+
+// Regularized incomplete gamma functions P(k, x) and Q(k, x) = 1 - P (the reference ships C for
+// them too, theano/scalar/c_code/gamma.c): the power series of P for x < k + 1, the continued
+// fraction of Q (modified Lentz evaluation) beyond, each scaled by exp(-x + k ln x - lgamma(k));
+// computed in double precision.  k <= 0 or x < 0 give NaN.
+__device__ inline double thx_gamma_p_series(double k, double x) {
+  double term = 1.0 / k, sum = term;
+  for (int n = 1; n < 1000; ++n) {
+    term *= x / (k + n);
+    sum += term;
+    if (fabs(term) < fabs(sum) * 1e-17) break;
+  }
+  return sum * exp(-x + k * log(x) - lgamma(k));
+}
+__device__ inline double thx_gamma_q_fraction(double k, double x) {
+  const double tiny = 1e-300;
+  double b = x + 1.0 - k, c = 1.0 / tiny, d = 1.0 / b, h = d;
+  for (int i = 1; i < 1000; ++i) {
+    const double an = -i * (i - k);
+    b += 2.0;
+    d = an * d + b;
+    if (fabs(d) < tiny) d = tiny;
+    c = b + an / c;
+    if (fabs(c) < tiny) c = tiny;
+    d = 1.0 / d;
+    const double del = d * c;
+    h *= del;
+    if (fabs(del - 1.0) < 1e-16) break;
+  }
+  return h * exp(-x + k * log(x) - lgamma(k));
+}
+__device__ inline double thx_gammainc(double k, double x) {
+  if (!(k > 0.0) || !(x >= 0.0)) return NAN;
+  if (x == 0.0) return 0.0;
+  if (isinf(x)) return 1.0;
+  return x < k + 1.0 ? thx_gamma_p_series(k, x) : 1.0 - thx_gamma_q_fraction(k, x);
+}
+__device__ inline double thx_gammaincc(double k, double x) {
+  if (!(k > 0.0) || !(x >= 0.0)) return NAN;
+  if (x == 0.0) return 1.0;
+  if (isinf(x)) return 0.0;
+  return x < k + 1.0 ? 1.0 - thx_gamma_p_series(k, x) : thx_gamma_q_fraction(k, x);
+}
+
 namespace thx {
 
 // How one operand is addressed along the vectorised (innermost) dimension.

@@ -978,6 +978,54 @@ gamma = _unary_math("Gamma", "tgamma", lambda x, z, gz: gz * z * psi(x))
 gammaln = _unary_math("GammaLn", "lgamma", lambda x, z, gz: gz * psi(x))
 psi = _unary_math("Psi", "thx_psi", lambda x, z, gz: gz * tri_gamma(x))
 tri_gamma = _unary_math("TriGamma", "thx_trigamma", None)
+# Bessel functions (``theano/scalar/basic_scipy.py:714-857``); J1' and I1' are written through the
+# recurrences J1' = J0 - J1 / x and I1' = I0 - I1 / x (the reference's (J0 - J2) / 2 and (I0 + I2) / 2)
+j0 = _unary_math("J0", "j0", lambda x, z, gz: -gz * j1(x))
+j1 = _unary_math("J1", "j1", lambda x, z, gz: gz * switch(eq(x, 0), 0.5, j0(x) - z / x))
+i0 = _unary_math("I0", "thx_i0", lambda x, z, gz: gz * i1(x))
+i1 = _unary_math("I1", "thx_i1", lambda x, z, gz: gz * switch(eq(x, 0), 0.5, i0(x) - z / x))
+
+
+def upgrade_to_float64(*types):
+    """Always float64 (``theano/scalar/basic.py:914-920``)."""
+    return (float64,)
+
+
+class _IncompleteGamma(BinaryScalarOp):
+    """Regularized incomplete gamma functions and their relatives
+    (``theano/scalar/basic_scipy.py:482-711``), evaluated by the kernel prelude's helpers in
+    double precision.  Not differentiable, as in the reference."""
+
+    expr = None
+
+    def c_code(self, node, inputs, outputs):
+        a, b = ["((double)%s)" % i for i in inputs]
+        return "%s = %s;" % (outputs[0], self.expr % dict(a=a, b=b))
+
+
+class GammaInc(_IncompleteGamma):           # P(k, x)
+    expr = "thx_gammainc(%(a)s, %(b)s)"
+
+
+class GammaIncC(_IncompleteGamma):          # Q(k, x)
+    expr = "thx_gammaincc(%(a)s, %(b)s)"
+
+
+class GammaU(_IncompleteGamma):             # upper incomplete gamma: Q(k, x) * gamma(k)
+    expr = "thx_gammaincc(%(a)s, %(b)s) * tgamma(%(a)s)"
+
+
+class GammaL(_IncompleteGamma):             # lower incomplete gamma: P(k, x) * gamma(k)
+    expr = "thx_gammainc(%(a)s, %(b)s) * tgamma(%(a)s)"
+
+
+class Chi2SF(_IncompleteGamma):             # chi-square survival function of x with k degrees of freedom
+    expr = "thx_gammaincc(0.5 * %(b)s, 0.5 * %(a)s)"
+
+
+gammainc, gammaincc = GammaInc(upgrade_to_float, name="gammainc"), GammaIncC(upgrade_to_float, name="gammaincc")
+gammau, gammal = GammaU(upgrade_to_float, name="gammau"), GammaL(upgrade_to_float, name="gammal")
+chi2sf = Chi2SF(upgrade_to_float64, name="chi2sf")
 
 
 class Trunc(UnaryScalarOp):

@@ -56,6 +56,9 @@ erf, erfc, erfcx = _elemwise(scal.erf, "erf"), _elemwise(scal.erfc, "erfc"), _el
 erfinv, erfcinv = _elemwise(scal.erfinv, "erfinv"), _elemwise(scal.erfcinv, "erfcinv")
 gamma, gammaln = _elemwise(scal.gamma, "gamma"), _elemwise(scal.gammaln, "gammaln")
 psi, tri_gamma = _elemwise(scal.psi, "psi"), _elemwise(scal.tri_gamma, "tri_gamma")
+j0, j1, i0, i1 = _elemwise(scal.j0, "j0"), _elemwise(scal.j1, "j1"), _elemwise(scal.i0, "i0"), _elemwise(scal.i1, "i1")
+gammainc, gammaincc = _elemwise(scal.gammainc, "gammainc"), _elemwise(scal.gammaincc, "gammaincc")
+gammau, gammal, chi2sf = _elemwise(scal.gammau, "gammau"), _elemwise(scal.gammal, "gammal"), _elemwise(scal.chi2sf, "chi2sf")
 sigmoid = _elemwise(scal.scalar_sigmoid, "sigmoid")
 softplus = _elemwise(scal.scalar_softplus, "softplus")
 
