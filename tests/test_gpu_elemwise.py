@@ -338,7 +338,8 @@ def test_bessel_and_incomplete_gamma_functions_against_scipy(dtype):
             scipy.special.gammaincc(k64, p64) * scipy.special.gamma(k64), scipy.stats.chi2.sf(p64, k64)]
     for j, (g, w) in enumerate(zip(got, want)):
         assert g.dtype == np.dtype("float64" if j == 4 else dtype), j
-        assert np.allclose(g, w.astype(g.dtype), rtol=tol["rtol"] * 5, atol=tol["atol"]), j
+        with np.errstate(over="ignore"):             # gamma(k) leaves float32's range for k > 35: inf on both sides
+            assert np.allclose(g, w.astype(g.dtype), rtol=tol["rtol"] * 5, atol=tol["atol"]), j
     ref = G.evaluate([k, x], outs, [kv, pv])
     for g, r in zip(got, ref):
         assert np.allclose(g, r, rtol=tol["rtol"] * 5, atol=tol["atol"])
