@@ -151,3 +151,32 @@ def test_product_never_touches_the_oracle_or_a_host_fallback():
             node.op.perform(node, [np.zeros((3, 4), "float32")] * len(node.inputs), [[None] for _ in node.outputs])
     src = open(os.path.join(pkg, "hip", "runtime.py")).read()
     assert "ctypes.CDLL" in src and "raise" in src[src.index("_LIB_PATH"):src.index("ctypes.CDLL")]
+
+
+def _build_c_client(tmp_path):
+    import subprocess
+    exe = str(tmp_path / "abi_client")
+    libdir = os.path.join(ROOT, "theano_amd", "csrc")
+    cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", os.path.join(ROOT, "tests", "abi_client.c"),
+           "-I", os.path.join(ROOT, "include"), "-L", libdir, "-lthx_hip", "-Wl,-rpath," + libdir, "-o", exe]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
+    return exe
+
+
+def test_a_plain_c_host_binds_the_library(tmp_path):
+    """include/thx_hip.h is valid C99 and a host written in C (tests/abi_client.c) can create an
+    operation from functor text and have it planned and compiled; no Python, no C++ types."""
+    import subprocess
+    exe = _build_c_client(tmp_path)
+    res = subprocess.run([exe, "dry"], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0 and res.stdout.strip().endswith("ok"), res.stdout + res.stderr
+    assert "AxPlusB|e" in res.stdout
+
+
+@pytest.mark.gpu
+def test_the_c_host_runs_on_the_device(tmp_path):
+    import subprocess
+    exe = _build_c_client(tmp_path)
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0 and res.stdout.strip().endswith("ok"), res.stdout + res.stderr
