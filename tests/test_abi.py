@@ -158,7 +158,7 @@ def _build_c_client(tmp_path):
     exe = str(tmp_path / "abi_client")
     libdir = os.path.join(ROOT, "theano_amd", "csrc")
     cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", os.path.join(ROOT, "tests", "abi_client.c"),
-           "-I", os.path.join(ROOT, "include"), "-L", libdir, "-lthx_hip", "-Wl,-rpath," + libdir, "-o", exe]
+           "-I", os.path.join(ROOT, "include"), "-L", libdir, "-lthx_hip", "-lm", "-Wl,-rpath," + libdir, "-o", exe]
     res = subprocess.run(cmd, capture_output=True, text=True)
     assert res.returncode == 0, res.stderr
     return exe
