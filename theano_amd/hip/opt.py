@@ -638,60 +638,58 @@ def merge_sibling_elemwise(fgraph):
     depend on the other.  The reference's GPU op stops at one output
     (``theano/gpuarray/elemwise.py:114-115``); the kernels here take several."""
     count = 0
-    changed = True
-    while changed:
-        changed = False
-        nodes = [n for n in fgraph.toposort() if isinstance(n.op, HipElemwise) and not n.op.inplace_pattern]
-        for ai, a in enumerate(nodes):
-            pa = tuple(a.outputs[0].type.broadcastable)
-            if all(pa):
+    nodes = [n for n in fgraph.toposort() if isinstance(n.op, HipElemwise) and not n.op.inplace_pattern]
+    for ai in range(len(nodes)):
+        a = nodes[ai]
+        if a not in fgraph.apply_nodes:
+            continue
+        pa = tuple(a.outputs[0].type.broadcastable)
+        if all(pa):
+            continue
+        for bi in range(ai + 1, len(nodes)):
+            b = nodes[bi]
+            if b not in fgraph.apply_nodes or tuple(b.outputs[0].type.broadcastable) != pa:
                 continue
             full_a = set(id(i) for i in a.inputs if isinstance(i.type, HipArrayType) and
                          tuple(i.type.broadcastable) == pa)
             full_a.update(id(o) for o in a.outputs)
-            for b in nodes[ai + 1:]:
-                if tuple(b.outputs[0].type.broadcastable) != pa:
-                    continue
-                if not any(id(i) in full_a for i in b.inputs):
-                    continue
-                if any(i.owner is not a and _depends_on(i, a) for i in b.inputs):
-                    continue
-                if any(_depends_on(i, b) for i in a.inputs):
-                    continue
-                inputs, s_inputs = [], []
+            if not any(id(i) in full_a for i in b.inputs):
+                continue
+            if any(i.owner is not a and _depends_on(i, a) for i in b.inputs):
+                continue
+            if any(_depends_on(i, b) for i in a.inputs):
+                continue
+            inputs, s_inputs = [], []
 
-                def scalar_for(v):
-                    for t, sv in zip(inputs, s_inputs):
-                        if t is v:
-                            return sv
-                    sv = scal.Scalar(v.type.dtype)()
-                    inputs.append(v)
-                    s_inputs.append(sv)
-                    return sv
+            def scalar_for(v):
+                for t, sv in zip(inputs, s_inputs):
+                    if t is v:
+                        return sv
+                sv = scal.Scalar(v.type.dtype)()
+                inputs.append(v)
+                s_inputs.append(sv)
+                return sv
 
-                a_souts = a.op.scalar_op(*[scalar_for(v) for v in a.inputs], return_list=True)
-                b_args = [a_souts[a.outputs.index(v)] if v.owner is a else scalar_for(v) for v in b.inputs]
-                b_souts = b.op.scalar_op(*b_args, return_list=True)
-                # results of the first kernel that only the second one read stay inside
-                keep = [k for k, o in enumerate(a.outputs)
-                        if any(c is not b for c, _ in fgraph.clients.get(o, []))]
-                olds = [a.outputs[k] for k in keep] + list(b.outputs)
-                if len(inputs) > config.max_fused_inputs or len(olds) > 8:
-                    continue
-                # an array that is both read and produced here would be an output equal to an input
-                s_outs = [a_souts[k] for k in keep] + b_souts
-                if any(so in s_inputs for so in s_outs):
-                    continue
-                merged = HipElemwise(scal.Composite(s_inputs, s_outs)).make_node(*inputs)
-                if [o.type for o in merged.outputs] != [o.type for o in olds]:
-                    continue
-                for o, no in zip(olds, merged.outputs):
-                    fgraph.replace(o, no)
-                count += 1
-                changed = True
-                break
-            if changed:
-                break
+            a_souts = a.op.scalar_op(*[scalar_for(v) for v in a.inputs], return_list=True)
+            b_args = [a_souts[a.outputs.index(v)] if v.owner is a else scalar_for(v) for v in b.inputs]
+            b_souts = b.op.scalar_op(*b_args, return_list=True)
+            # results of the first kernel that only the second one read stay inside
+            keep = [k for k, o in enumerate(a.outputs)
+                    if any(c is not b for c, _ in fgraph.clients.get(o, []))]
+            olds = [a.outputs[k] for k in keep] + list(b.outputs)
+            if len(inputs) > config.max_fused_inputs or len(olds) > 8:
+                continue
+            # an array that is both read and produced here would be an output equal to an input
+            s_outs = [a_souts[k] for k in keep] + b_souts
+            if any(so in s_inputs for so in s_outs):
+                continue
+            merged = HipElemwise(scal.Composite(s_inputs, s_outs)).make_node(*inputs)
+            if [o.type for o in merged.outputs] != [o.type for o in olds]:
+                continue
+            for o, no in zip(olds, merged.outputs):
+                fgraph.replace(o, no)
+            count += 1
+            a = merged              # keeps collecting partners among the nodes that follow
     return count
 
 
