@@ -91,6 +91,19 @@ def test_hip_path_reproduces_reference_vectors(entry):
     check(entry, th.function(ins, outs)(*vals))
 
 
+@pytest.mark.parametrize("entry", VECTORS, ids=[v["name"] for v in VECTORS])
+def test_vector_graphs_compile_without_a_rewrite_cycle(entry, dry_run):
+    """The graph rewriter warns when rewrites keep undoing each other; none of the
+    reference's test graphs may trigger that."""
+    import warnings
+    ins, outs, vals = build(entry)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        got = th.function(ins, outs)(*vals)
+    want = expected(entry, len(got))
+    assert [np.asarray(g).shape for g in got] == [w.shape if w.ndim else np.asarray(g).shape for g, w in zip(got, want)]
+
+
 def test_fixture_file_matches_its_generator():
     import importlib.util
     spec = importlib.util.spec_from_file_location("make_vectors", os.path.join(HERE, "golden", "make_vectors.py"))

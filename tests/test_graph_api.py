@@ -614,3 +614,34 @@ def test_nested_sums_and_products_become_one_reduction():
     fg = gof.FunctionGraph([x], [T.sum(T.prod(x, axis=1), axis=1)])
     topt.canonicalize(fg)
     assert len([n for n in fg.toposort() if isinstance(n.op, CAReduce)]) == 2
+
+
+def test_deep_chain_is_canonicalized_to_a_fixed_point_quickly(dry_run):
+    """A rewrite whose result enables the next one (here: one per layer) is followed along the
+    chain inside one sweep: a 40-layer network with its gradient compiles in seconds and ends
+    up as one row-wise kernel plus the final sum."""
+    import time, warnings
+    from theano_amd.hip.rowchain import HipRowChain
+    x = T.fmatrix("x")
+    h = x
+    for _ in range(40):
+        h = T.tanh(h * 1.01 + T.mean(h, axis=1, keepdims=True)) * T.nnet.sigmoid(h)
+    cost = T.sum(h * h)
+    g = th.grad(cost, x)
+    t0 = time.time()
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        f = th.function([x], [cost, g])
+    assert time.time() - t0 < 30
+    kinds = [type(n.op).__name__ for n in f.toposort()]
+    assert kinds.count("HipRowChain") == 1 and kinds.count("HipElemwise") == 0, kinds
+
+
+def test_sum_of_reciprocal_with_constant_numerator_terminates(dry_run):
+    """sum(c / x): the constant leaves the sum once (c * sum(1 / x)) and the rewriter stops."""
+    import warnings
+    x = T.dmatrix("x")
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        f = th.function([x], T.sum(2.0 / x) + T.sum(T.ones_like(x) / x))
+    assert f is not None

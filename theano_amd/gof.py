@@ -304,6 +304,8 @@ class FunctionGraph(object):
     (``theano/gof/fg.py``).  The string 'output' stands for the graph's own
     use of an output variable."""
 
+    import_log = None   # a list while a rewriter wants to know which nodes a replacement brings in
+
     def __init__(self, inputs, outputs, clone_graph=True):
         if clone_graph:
             inputs, outputs = clone(inputs, outputs)
@@ -329,16 +331,34 @@ class FunctionGraph(object):
             self.variables.add(var)
             self.clients.setdefault(var, [])
             return
-        for node in io_toposort(list(self.variables), [var]):
-            self._import_node(node)
+        # post-order walk over the producers that are not part of the graph yet
+        stack = [(var.owner, False)]
+        while stack:
+            node, expanded = stack.pop()
+            if node in self.apply_nodes:
+                continue
+            if expanded:
+                self._import_node(node)
+                continue
+            stack.append((node, True))
+            for i in node.inputs:
+                if i in self.variables:
+                    continue
+                if i.owner is None:
+                    self._import_var(i)
+                else:
+                    stack.append((i.owner, False))
 
     def _import_node(self, node):
+        """Adds a node whose inputs are all part of the graph (or become so here)."""
         if node in self.apply_nodes:
             return
         for i in node.inputs:
             if i not in self.variables:
                 self._import_var(i)
         self.apply_nodes.add(node)
+        if self.import_log is not None:
+            self.import_log.append(node)
         for o in node.outputs:
             self.variables.add(o)
             self.clients.setdefault(o, [])
@@ -415,11 +435,11 @@ class LocalOptimizer(object):
 class FromFunctionLocalOptimizer(LocalOptimizer):
     def __init__(self, fn, tracks=None):
         self.fn = fn
-        self.tracks = tracks
+        self.tracks = tuple(tracks) if tracks is not None else None
         self.__name__ = fn.__name__
 
     def transform(self, fgraph, node):
-        if self.tracks is not None and not isinstance(node.op, tuple(self.tracks)):
+        if self.tracks is not None and not isinstance(node.op, self.tracks):
             return False
         return self.fn(fgraph, node)
 
@@ -434,19 +454,25 @@ def local_optimizer(tracks=None):
 
 
 def apply_local(fgraph, opts, order="in_to_out", max_passes=64):
-    """Apply local rewrites over the whole graph until nothing changes."""
+    """Apply local rewrites over the whole graph until nothing changes.  Within a
+    pass, the nodes a replacement brings in and the consumers of the replaced value
+    are visited right away (a chain of rewrites that feed one another does not cost
+    one pass per link); a pass that changes nothing ends the loop."""
     changed_any = False
+    budget = None
     for _ in range(max_passes):
         changed = False
         nodes = fgraph.toposort()
         if order == "out_to_in":
             nodes.reverse()
-        for node in nodes:
+        if budget is None:
+            budget = 32 * len(nodes) + 512      # rewrites that undo each other must not spin
+        nodes.reverse()                          # a stack: the next node is at the end
+        while nodes and budget > 0:
+            node = nodes.pop()
             if node not in fgraph.apply_nodes:
                 continue
             for opt in opts:
-                if node not in fgraph.apply_nodes:
-                    break
                 repl = opt.transform(fgraph, node)
                 if not repl:
                     continue
@@ -454,13 +480,26 @@ def apply_local(fgraph, opts, order="in_to_out", max_passes=64):
                     pairs = list(repl.items())
                 else:
                     pairs = list(zip(node.outputs, repl))
+                fgraph.import_log = fresh = []
+                touched = []
                 for old, new in pairs:
                     if new is not None:
                         fgraph.replace(old, new)
+                        touched.extend(c for c, _ in fgraph.clients.get(new, []) if c != "output")
+                fgraph.import_log = None
+                again = [n for n in fresh + touched + [node] if n in fgraph.apply_nodes]
+                if order == "out_to_in":
+                    again.reverse()
+                nodes.extend(reversed(again))
                 changed = True
+                budget -= 1
                 break
         changed_any = changed_any or changed
         if not changed:
+            break
+        if budget <= 0:
+            import warnings
+            warnings.warn("graph rewriting stopped early: the rewrites keep replacing each other's results")
             break
     return changed_any
 

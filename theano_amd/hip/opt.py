@@ -294,7 +294,10 @@ def fuse_reduce_prologue(fgraph):
     changed = True
     while changed:
         changed = False
-        for node in fgraph.toposort():
+        work = [n for n in fgraph.toposort() if isinstance(n.op, HipCAReduce)]
+        work.reverse()
+        while work:
+            node = work.pop()
             op = node.op
             if not isinstance(op, HipCAReduce) or op.post_scalar_op is not None or node not in fgraph.apply_nodes:
                 continue
@@ -346,7 +349,7 @@ def fuse_reduce_prologue(fgraph):
                 fgraph.replace(o, no)
             count += 1
             changed = True
-            break
+            work.append(new_node)       # its new operands may have absorbable producers too
     return count
 
 
@@ -399,7 +402,10 @@ def fuse_reduce_epilogue(fgraph):
     changed = True
     while changed:
         changed = False
-        for red in fgraph.toposort():
+        work = [n for n in fgraph.toposort() if isinstance(n.op, HipCAReduce)]
+        work.reverse()
+        while work:
+            red = work.pop()
             rop = red.op
             if not isinstance(rop, HipCAReduce) or red not in fgraph.apply_nodes:
                 continue
@@ -414,28 +420,27 @@ def fuse_reduce_epilogue(fgraph):
                                 cands.append(c2)
                     elif isinstance(c.op, HipElemwise) and c not in cands:
                         cands.append(c)
-            done = False
             for cand in cands:
-                if _try_epilogue(fgraph, red, cand):
-                    done = True
+                new_red = _try_epilogue(fgraph, red, cand)
+                if new_red is not None:
+                    count += 1
+                    changed = True
+                    work.append(new_red)    # the next consumer in the chain
                     break
-            if done:
-                count += 1
-                changed = True
-                break
     return count
 
 
 def _try_epilogue(fgraph, red, cand):
     """Moves the elementwise node ``cand`` into the epilogue of the reduction
-    ``red`` (composing it with an epilogue that is already there).  Every array
+    ``red`` (composing it with an epilogue that is already there); returns the new
+    reduction node, or None.  Every array
     input of ``cand`` must be a result of ``red`` (directly or through one and the
     same keepdims DimShuffle), a host scalar, or a device array of the results'
     own shape that does not depend on ``red`` (a per-channel scale, the result
     of an earlier reduction): the epilogue reads that one at the result's index."""
     rop = red.op
     if len(cand.outputs) != 1 or cand.op.inplace_pattern:
-        return False
+        return None
     n_red_in = len(red.inputs) - rop.n_extra
     extras = list(red.inputs[n_red_in:])
     post_in = rop.post_in_dtypes if rop.post_scalar_op is not None else rop.out_dtypes
@@ -450,18 +455,18 @@ def _try_epilogue(fgraph, red, cand):
     for i in cand.inputs:
         if i.owner is not None and isinstance(i.owner.op, HipDimShuffle) and i.owner.inputs[0].owner is red:
             if ds_op is not None and i.owner.op != ds_op:
-                return False
+                return None
             ds_op = i.owner.op
         elif i.owner is red:
             seen_direct = True
     if ds_op is not None and seen_direct:
-        return False
+        return None
     if ds_op is not None:
         # only DimShuffles that insert or drop broadcast dimensions: with a transposition in
         # between, "the result's index" is no longer the consumer's index
         kept_order = [o for o in ds_op.new_order if o != "x"]
         if kept_order != sorted(kept_order):
-            return False
+            return None
         layout = ds_op.make_node(red.outputs[0]).outputs[0].type.broadcastable
     else:
         layout = red.outputs[0].type.broadcastable
@@ -506,10 +511,10 @@ def _try_epilogue(fgraph, red, cand):
             continue
         expr = operand(i, 0)
         if expr is None:
-            return False
+            return None
         s_args.append(expr)
     if not used or len(extras) > 12:
-        return False
+        return None
     e_out = cand.op.scalar_op(*s_args)
     # results something else still needs stay outputs of the new node
     keep = []
@@ -535,15 +540,20 @@ def _try_epilogue(fgraph, red, cand):
     if ds_op is not None:
         new_e = HipDimShuffle(ds_op.input_broadcastable, ds_op.new_order)(new_e)
     if new_e.type != cand.outputs[0].type:
-        return False
+        return None
     for j, k in enumerate(keep):
         fgraph.replace(red.outputs[k], new_node.outputs[j])
     fgraph.replace(cand.outputs[0], new_e)
-    return True
+    return new_node
 
 
-def _depends_on(var, node, limit=10000):
-    """True when ``var`` is computed (transitively) from an output of ``node``."""
+def _depends_on(var, node, limit=10000, pos=None):
+    """True when ``var`` is computed (transitively) from an output of ``node``.  ``pos``: positions
+    in a topological order; a producer placed before ``node`` cannot depend on it."""
+    if pos is not None and var.owner is not None:
+        pv, pn = pos.get(var.owner), pos.get(node)
+        if pv is not None and pn is not None and pv < pn:
+            return False
     stack, seen = [var], set()
     while stack and len(seen) < limit:
         v = stack.pop()
@@ -638,7 +648,9 @@ def merge_sibling_elemwise(fgraph):
     depend on the other.  The reference's GPU op stops at one output
     (``theano/gpuarray/elemwise.py:114-115``); the kernels here take several."""
     count = 0
-    nodes = [n for n in fgraph.toposort() if isinstance(n.op, HipElemwise) and not n.op.inplace_pattern]
+    order = fgraph.toposort()
+    pos = dict((n, k) for k, n in enumerate(order))
+    nodes = [n for n in order if isinstance(n.op, HipElemwise) and not n.op.inplace_pattern]
     for ai in range(len(nodes)):
         a = nodes[ai]
         if a not in fgraph.apply_nodes:
@@ -655,9 +667,9 @@ def merge_sibling_elemwise(fgraph):
             full_a.update(id(o) for o in a.outputs)
             if not any(id(i) in full_a for i in b.inputs):
                 continue
-            if any(i.owner is not a and _depends_on(i, a) for i in b.inputs):
+            if any(i.owner is not a and _depends_on(i, a, pos=pos) for i in b.inputs):
                 continue
-            if any(_depends_on(i, b) for i in a.inputs):
+            if any(_depends_on(i, b, pos=pos) for i in a.inputs):
                 continue
             inputs, s_inputs = [], []
 
@@ -689,6 +701,7 @@ def merge_sibling_elemwise(fgraph):
             for o, no in zip(olds, merged.outputs):
                 fgraph.replace(o, no)
             count += 1
+            pos[merged] = min(pos[a], pos[b])   # nothing placed before both can depend on the merged node
             a = merged              # keeps collecting partners among the nodes that follow
     return count
 

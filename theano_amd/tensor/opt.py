@@ -310,7 +310,9 @@ def local_sum_invariant_factor(fgraph, node):
             if ca is None and not sa:
                 return None, v, False
             found[0] = True
-            return ca, T.true_div(ra if ra is not None else T.ones_like(b), b), sa
+            # an invariant numerator over a varying denominator leaves the reciprocal (not
+            # ones / b: that quotient would be split again, forever)
+            return ca, (T.true_div(ra, b) if ra is not None else T.inv(b)), sa
         if isinstance(sop, scal.Neg):
             ca, ra, sa = split(p.inputs[0])
             found[0] = True
