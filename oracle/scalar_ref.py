@@ -23,7 +23,11 @@ scalar transcription of the four sign cases and against exact floor division awa
 from integer quotients.  The special functions are ``scipy.special`` itself, which
 is what the reference's ``impl`` calls (``theano/scalar/basic_scipy.py:32-36``); every
 differentiable op's value is tied to its neighbours' by the finite-difference
-gradient checks of tests/test_oracle_graph.py.  No function here is unpinned.
+gradient checks of tests/test_oracle_graph.py.  The approximate sigmoid is pinned by
+hand-evaluated points on each of its pieces, its symmetry and its known distance to
+the sigmoid; softsign by exact quotients; the fused sigmoid cross-entropy by
+``log(1 + e^x) - x t`` and, where that is well conditioned, the two-logarithm
+definition.  No function here is unpinned.
 """
 import numpy as np
 
@@ -440,6 +444,36 @@ def scalar_softplus(out_dtype, x):
     return _conv(r, out_dtype)
 
 
+def ultra_fast_scalar_sigmoid(out_dtype, x):
+    """theano/tensor/nnet/sigm.py:210-229 (the C text): pieces in double, rounded to the output type at
+    each assignment to a variable of that type."""
+    ot = np.dtype(out_dtype)
+    h = (0.5 * x.astype("float64")).astype(ot)
+
+    def piece(v):
+        v = v.astype("float64")
+        return np.where(v < 1.7, 1.5 * v / (1 + v), np.where(v < 3, 0.935409070603099 + 0.0458812946797165 * (v - 1.7),
+                                                             0.99505475368673))
+    with np.errstate(all="ignore"):
+        t = np.where(h >= 0, piece(h), -piece(-h)).astype(ot)
+    return _conv((0.5 * (t.astype("float64") + 1.0)).astype(ot), out_dtype)
+
+
+def sigmoid_binary_crossentropy(out_dtype, x, t):
+    """theano/tensor/nnet/nnet.py:2048: softplus(-abs(x)) + x * ((x > 0) - t), every step in the output's
+    compute type."""
+    ct = "float32" if str(out_dtype) == "float16" else out_dtype
+    xc, tc = _conv(x, ct), _conv(t, ct)
+    sp = scalar_softplus(ct, -np.abs(xc))
+    return _conv(sp + xc * ((xc > 0).astype(ct) - tc), out_dtype)
+
+
+def scalar_softsign(out_dtype, x):
+    """theano/tensor/nnet/nnet.py:2511: x / (1.0 + fabs(x)), in double, rounded on assignment."""
+    xd = x.astype("float64")
+    return _conv((xd / (1.0 + np.abs(xd))).astype(np.dtype(out_dtype)), out_dtype)
+
+
 # scalar op class name -> restatement
 BY_CLASS = {
     "Add": add, "Mul": mul, "Sub": sub, "TrueDiv": true_div, "IntDiv": int_div_fast, "Mod": mod_fast, "Pow": pow_,
@@ -455,4 +489,6 @@ BY_CLASS = {
     "ScalarSoftplus": scalar_softplus, "Erf": erf, "Erfc": erfc, "Erfcx": erfcx, "Erfinv": erfinv, "Erfcinv": erfcinv,
     "Gamma": gamma, "GammaLn": gammaln, "Psi": psi, "TriGamma": tri_gamma, "J0": j0, "J1": j1, "I0": i0, "I1": i1,
     "GammaInc": gammainc, "GammaIncC": gammaincc, "GammaU": gammau, "GammaL": gammal, "Chi2SF": chi2sf,
+    "UltraFastScalarSigmoid": ultra_fast_scalar_sigmoid, "ScalarSoftsign": scalar_softsign,
+    "SigmoidBinaryCrossentropy": sigmoid_binary_crossentropy,
 }

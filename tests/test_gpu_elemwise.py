@@ -343,3 +343,45 @@ def test_bessel_and_incomplete_gamma_functions_against_scipy(dtype):
     ref = G.evaluate([k, x], outs, [kv, pv])
     for g, r in zip(got, ref):
         assert np.allclose(g, r, rtol=tol["rtol"] * 5, atol=tol["atol"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+def test_sigmoid_family_and_stabilised_forms(dtype):
+    """Activations of theano/tensor/nnet (sigm.py, nnet.py:2008-2050, 2437-2516) against closed forms in float64,
+    with arguments far enough out that the unstabilised formulas overflow; approximate sigmoids against the
+    oracle's restatement of their C text."""
+    from theano_amd.tensor import nnet
+    rng = np.random.default_rng(31)
+    x = T.TensorType(dtype, (False, False))("x")
+    t = T.TensorType(dtype, (False, False))("t")
+    big = 80.0 if dtype == "float32" else 700.0
+    xv = np.concatenate([rng.uniform(-big, big, (37, 50)), rng.uniform(-3, 3, (37, 50)), [[0.0] * 50]]).astype(dtype)
+    tv = rng.uniform(0, 1, xv.shape).astype(dtype)
+    x64, t64 = xv.astype("float64"), tv.astype("float64")
+    sp = np.logaddexp(0, x64)                                    # softplus
+    sg = np.exp(-np.logaddexp(0, -x64))                          # sigmoid
+    outs = [T.log(nnet.sigmoid(x)), T.log(1 - nnet.sigmoid(x)), T.log1p(T.exp(x)), T.exp(x) / (1 + T.exp(x)),
+            1.0 / (1.0 + T.exp(-x)), nnet.sigmoid(x) * T.exp(-x), nnet.binary_crossentropy(nnet.sigmoid(x), t),
+            nnet.sigmoid_binary_crossentropy(x, t), nnet.elu(x), nnet.selu(x), nnet.hard_sigmoid(x),
+            th.grad(T.sum(nnet.sigmoid_binary_crossentropy(x, t)), x), th.grad(T.sum(nnet.softsign(x)), x),
+            th.grad(T.sum(nnet.elu(x, 0.5)), x)]
+    bce = t64 * (sp - x64) + (1 - t64) * sp
+    elu = np.where(x64 > 0, x64, np.expm1(np.minimum(x64, 0)))
+    # Python floats become constants of dtype floatX (theano/scalar/basic.py:309-312): rounded to float32 by default
+    scale, alpha = (float(np.dtype(th.config.floatX).type(c)) for c in (1.0507009873554804934193349852946,
+                                                                       1.6732632423543772848170429916717))
+    want = [x64 - sp, -sp, sp, sg, sg, np.exp(-sp), bce, bce, elu,
+            scale * np.where(x64 > 0, x64, alpha * np.expm1(np.minimum(x64, 0))),
+            np.clip(0.2 * x64 + 0.5, 0, 1), sg - t64, 1 / (1 + np.abs(x64)) ** 2,
+            np.where(x64 > 0, 1.0, 0.5 * np.exp(np.minimum(x64, 0)))]
+    got = th.function([x, t], outs)(xv, tv)
+    # the reference's softplus returns x itself beyond 16 (float64), dropping log1p(exp(-16)) = 1.1e-7 of 16: 7e-9
+    tol = dict(rtol=2e-5, atol=1e-6) if dtype == "float32" else dict(rtol=1e-8, atol=1e-13)
+    for j, (g, w) in enumerate(zip(got, want)):
+        assert g.dtype == np.dtype(dtype) and np.all(np.isfinite(g)), j
+        assert np.allclose(g, w, **tol), (j, np.abs(g - w).max())
+    approx = [nnet.ultra_fast_sigmoid(x), nnet.softsign(x)]
+    got, ref = run_both([x], approx, [xv])
+    for g, r in zip(got, ref):
+        assert_parity(g, r, "approximate sigmoid / softsign")
+    assert np.abs(got[0] - sg).max() < 0.028

@@ -645,3 +645,44 @@ def test_sum_of_reciprocal_with_constant_numerator_terminates(dry_run):
         warnings.simplefilter("error")
         f = th.function([x], T.sum(2.0 / x) + T.sum(T.ones_like(x) / x))
     assert f is not None
+
+
+def test_sigmoid_and_softplus_stabilisation_rewrites(dry_run):
+    """The patterns of theano/tensor/nnet/sigm.py:378-425, 588-640, 845-905 become sigmoid / softplus nodes."""
+    from theano_amd.tensor import nnet
+    x, t = T.dmatrix("x"), T.dmatrix("t")
+
+    def kernels(v):
+        return [str(n.op) for n in th.function([x, t], v, on_unused_input="ignore").toposort() if "Host" not in str(n.op)]
+
+    assert kernels(T.log(nnet.sigmoid(x))) == ["HipElemwise{Composite{neg(scalar_softplus(neg(i0)))}}"]
+    assert kernels(T.log(1 - nnet.sigmoid(x))) == ["HipElemwise{Composite{neg(scalar_softplus(i0))}}"]
+    assert kernels(T.log1p(T.exp(x))) == ["HipElemwise{scalar_softplus}"]
+    assert kernels(T.log1p(-nnet.sigmoid(x))) == ["HipElemwise{Composite{neg(scalar_softplus(i0))}}"]
+    assert kernels(T.exp(x) / (1 + T.exp(x))) == ["HipElemwise{scalar_sigmoid}"]
+    assert kernels(1.0 / (1.0 + T.exp(-x))) == ["HipElemwise{scalar_sigmoid}"]
+    assert kernels(nnet.sigmoid(x) * T.exp(-x)) == ["HipElemwise{Composite{scalar_sigmoid(neg(i0))}}"]
+    (k,) = kernels(3.0 * t / ((1 + T.exp(x)) * t))
+    assert "exp" not in k and "scalar_sigmoid(neg(i1))" in k
+    (k,) = kernels(nnet.binary_crossentropy(nnet.sigmoid(x), t))
+    assert "log" not in k and k.count("scalar_softplus") == 2
+    # the fused cross-entropy differentiates to sigmoid(x) - t, also at x = 0
+    (k,) = kernels(th.grad(T.sum(nnet.sigmoid_binary_crossentropy(x, t)), x))
+    assert k == "HipElemwise{Composite{sub(scalar_sigmoid(i0), i1)}}", k
+    # 2 + exp(x) is not 1 + exp(x)
+    (k,) = kernels(1.0 / (2.0 + T.exp(x)))
+    assert "sigmoid" not in k
+
+
+def test_activation_front_ends(dry_run):
+    from theano_amd.tensor import nnet
+    x = T.fmatrix("x")
+    i = T.imatrix("i")
+    assert nnet.hard_sigmoid(x).type.dtype == "float32" and nnet.hard_sigmoid(i).type.dtype == "float64"
+    assert nnet.ultra_fast_sigmoid(x).type.dtype == "float32" and nnet.softsign(x).type.dtype == "float32"
+    assert nnet.elu(x).type == x.type and nnet.selu(x).type.dtype == "float32"
+    assert nnet.categorical_crossentropy(nnet.softmax(x), x).type.ndim == 1
+    with pytest.raises(NotImplementedError):
+        nnet.categorical_crossentropy(nnet.softmax(x), T.ivector("y"))
+    with pytest.raises(Exception):
+        th.grad(T.sum(nnet.ultra_fast_sigmoid(x)), x)      # no gradient, as in the reference

@@ -143,3 +143,45 @@ def test_float_int_div_follows_the_c_text():
     assert S.int_div_fast("float64", np.asarray([49.0]), np.asarray([np.float32(1.96)], "float64"))[0] == 24.0
     assert np.array_equal(S.int_div_fast("float32", np.asarray([7.5, -7.5, 7.5, -7.5], "float32"),
                                          np.asarray([2, 2, -2, -2], "float32")), [3, -4, -4, 3])
+
+
+def test_ultra_fast_sigmoid_and_softsign_known_answers():
+    """theano/tensor/nnet/sigm.py:179-230 and nnet.py:2484-2516.  Pinned by values worked out by hand
+    from the three pieces (x = 2 -> h = 1 -> 1.5 / 2 -> 0.875; x = 4 -> h = 2 on the linear piece; the two
+    plateaus), by the symmetry f(-x) = 1 - f(x), and by the distance to the sigmoid: the rational piece
+    1.5 h / (1 + h) is furthest from tanh(h) near h = 0.3 (0.346 against 0.291), half of that for the sigmoid."""
+    x = np.array([0.0, 2.0, -2.0, 4.0, 100.0, -100.0])
+    got = S.ultra_fast_scalar_sigmoid("float64", x)
+    lin = 0.935409070603099 + 0.0458812946797165 * 0.3
+    want = [0.5, 0.875, 0.125, 0.5 * (lin + 1), 0.5 * (0.99505475368673 + 1), 0.5 * (1 - 0.99505475368673)]
+    assert np.allclose(got, want, rtol=0, atol=1e-15)
+    grid = np.linspace(-15, 15, 3001)
+    uf = S.ultra_fast_scalar_sigmoid("float64", grid)
+    assert 0.027 < np.max(np.abs(uf - 1 / (1 + np.exp(-grid)))) < 0.028
+    assert np.allclose(uf + uf[::-1], 1.0, atol=1e-15)
+    # the pieces do not meet at h = 1.7: the rational piece ends at 2.55 / 2.7, the linear one starts lower
+    step = S.ultra_fast_scalar_sigmoid("float64", np.array([np.nextafter(3.4, 0), 3.4]))
+    assert np.allclose(step, [0.5 * (2.55 / 2.7 + 1), 0.5 * (0.935409070603099 + 1)], rtol=0, atol=1e-15)
+    assert S.ultra_fast_scalar_sigmoid("float32", grid.astype("float32")).dtype == np.float32
+    ss = S.scalar_softsign("float64", np.array([1.0, -3.0, 0.0, 1e300]))
+    assert np.array_equal(ss, [0.5, -0.75, 0.0, 1.0])
+    assert S.scalar_softsign("float32", np.array([1.0], "float32")).dtype == np.float32
+
+
+def test_sigmoid_binary_crossentropy_closed_form():
+    """nnet.py:2048 is -(t log s + (1 - t) log(1 - s)) with s = sigmoid(x), i.e. log(1 + e^x) - x t, and stays
+    finite where s rounds to 0 or 1."""
+    rng = np.random.default_rng(3)
+    x = np.concatenate([rng.uniform(-700, 700, 500), rng.uniform(-4, 4, 500), [0.0]])
+    t = rng.uniform(0, 1, x.shape)
+    got = S.sigmoid_binary_crossentropy("float64", x, t)
+    assert np.allclose(got, np.logaddexp(0, x) - x * t, rtol=1e-13, atol=1e-300)
+    small = np.abs(x) < 10                      # beyond, 1 - s has few digits left
+    s = 1 / (1 + np.exp(-x[small]))
+    assert np.allclose(got[small], -(t[small] * np.log(s) + (1 - t[small]) * np.log1p(-s)), rtol=1e-9, atol=1e-11)
+    x32 = x.astype("float32").clip(-80, 80)
+    got32 = S.sigmoid_binary_crossentropy("float32", x32, t.astype("float32"))
+    assert got32.dtype == np.float32
+    want = np.logaddexp(0, x32.astype("float64")) - x32 * t
+    # x * ((x > 0) - t) rounds (x > 0) - t to float32 first: an absolute error of |x| * 6e-8
+    assert np.all(np.abs(got32 - want) <= 2e-6 * np.abs(want) + 2e-7 * np.abs(x32) + 1e-7)

@@ -1165,6 +1165,78 @@ class ScalarSoftplus(UnaryScalarOp):
 scalar_softplus = ScalarSoftplus(upgrade_to_float, name="scalar_softplus")
 
 
+class SigmoidBinaryCrossentropy(BinaryScalarOp):
+    """``softplus(-|x|) + x * ((x > 0) - t)``: the cross-entropy of ``sigmoid(x)`` against the probability
+    ``t`` in its overflow-free form, with the gradients the reference attaches to that formula,
+    ``sigmoid(x) - t`` and ``-x`` (theano/tensor/nnet/nnet.py:2028-2050; the formula's own derivative
+    is off by one half at x = 0, where |x| has none)."""
+
+    def c_code(self, node, inputs, outputs):
+        ot = node.outputs[0].type.dtype
+        ct = compute_ctype(ot)
+        (x, t), (z,) = inputs, outputs
+        lo = "-745.0" if ot == "float64" else "-103.0f"
+        ex = _fn("exp", ot)
+        ex = "thx_fexp" if ex == "expf" else ex
+        return ("{ const %(ct)s thx_x = (%(ct)s)%(x)s; const %(ct)s thx_a = -%(fabs)s(thx_x); "
+                "const %(ct)s thx_sp = thx_a < %(lo)s ? (%(ct)s)0 : %(log1p)s(%(exp)s(thx_a)); "
+                "%(z)s = thx_sp + thx_x * ((%(ct)s)(thx_x > 0) - (%(ct)s)%(t)s); }") % dict(
+                    ct=ct, x=x, t=t, z=z, lo=lo, fabs=_fn("fabs", ot), log1p=_fn("log1p", ot), exp=ex)
+
+    def L_op(self, inputs, outputs, gout):
+        x, t = inputs
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            return [i.zeros_like(dtype=config.floatX) for i in inputs]
+        return [gz * (scalar_sigmoid(x) - t), gz * (-x)]
+
+
+sigmoid_binary_crossentropy = SigmoidBinaryCrossentropy(upgrade_to_float, name="sigmoid_binary_crossentropy")
+
+
+class UltraFastScalarSigmoid(UnaryScalarOp):
+    """0.5 * (t(0.5 * x) + 1) with a three-piece rational / linear / constant stand-in t for tanh
+    (theano/tensor/nnet/sigm.py:179-230): a speed option, within 0.028 of the sigmoid.  As in the
+    reference's C text the pieces are evaluated in double and rounded to the output type where the C
+    code assigns to a variable of that type."""
+
+    def c_code(self, node, inputs, outputs):
+        (x,), (z,) = inputs, outputs
+        ct = compute_ctype(node.outputs[0].type.dtype)
+        piece = ("(%(v)s < 1.7 ? (1.5 * %(v)s / (1 + %(v)s)) : (%(v)s < 3 ? (0.935409070603099 + "
+                 "0.0458812946797165 * (%(v)s - 1.7)) : 0.99505475368673))")
+        return ("{ const %(ct)s thx_h = (%(ct)s)(0.5 * (double)%(x)s); const %(ct)s thx_m = -thx_h; %(ct)s thx_t; "
+                "if (thx_h >= 0) thx_t = (%(ct)s)" + piece % {"v": "(double)thx_h"} + "; else thx_t = (%(ct)s)(-" +
+                piece % {"v": "(double)thx_m"} + "); %(z)s = (%(ct)s)(0.5 * ((double)thx_t + 1.)); }") % dict(ct=ct, x=x, z=z)
+
+    def L_op(self, inputs, outputs, gout):
+        raise MethodNotDefined("grad", type(self))       # as in the reference: the op is put in after the gradient
+
+
+ultra_fast_scalar_sigmoid = UltraFastScalarSigmoid(upgrade_to_float, name="ultra_fast_scalar_sigmoid")
+
+
+class ScalarSoftsign(UnaryScalarOp):
+    """x / (1 + |x|) (theano/tensor/nnet/nnet.py:2484-2516; the constant is a double in the C text)."""
+
+    def c_code(self, node, inputs, outputs):
+        (x,), (z,) = inputs, outputs
+        if node.inputs[0].type.dtype not in ("float32", "float64"):
+            raise NotImplementedError("only floating point x is implemented")
+        ct = compute_ctype(node.outputs[0].type.dtype)
+        return "%s = (%s)((double)%s / (1.0 + fabs((double)%s)));" % (z, ct, x, x)
+
+    def L_op(self, inputs, outputs, gout):
+        (x,) = inputs
+        if x.type.dtype not in float_dtypes:
+            raise NotImplementedError("softsign gradient: floating point only")
+        d = 1.0 + abs_(x)
+        return [gout[0] / (d * d)]
+
+
+scalar_softsign = ScalarSoftsign(upgrade_to_float, name="scalar_softsign")
+
+
 # --------------------------------------------------------------------------
 class DisconnectedType(Type):
     """Type of the placeholder gradient for an input the cost does not depend

@@ -324,8 +324,196 @@ def local_lower_row_ops(fgraph, node):
 local_lower_row_ops = local_optimizer(None)(local_lower_row_ops)
 
 
-RECOGNIZE = [local_softmax_simplifier, local_softmax_with_bias, local_logsoftmax, local_logsoftmax_grad]
+# ---- sigmoid / softplus stabilisation (theano/tensor/nnet/sigm.py:378-425, 588-640, 845-905) ----
+def _const_value(v):
+    """Python float of an all-broadcastable constant (also under a DimShuffle), else None."""
+    from .type import TensorConstant
+    if v.owner is not None and isinstance(v.owner.op, DimShuffle):
+        v = v.owner.inputs[0]
+    if isinstance(v, TensorConstant) and all(v.type.broadcastable):
+        return float(v.data.reshape(()))
+    return None
+
+
+def _is_const(v, value):
+    c = _const_value(v)
+    return c is not None and abs(c - value) <= 1e-8 + 1e-5 * abs(value)
+
+
+def _arg_of(var, scalar_cls):
+    return var.owner.inputs[0] if _is_elemwise(var, scalar_cls) else None
+
+
+def _negated(t):
+    """-t, without stacking a negation on a negation."""
+    inner = _arg_of(t, scal.Neg)
+    return inner if inner is not None else T.neg(t)
+
+
+def _one_plus_exp(v):
+    """x if v is ``1 + exp(x)`` (either order), else None (``is_1pexp``, sigm.py:428-462)."""
+    if not _is_elemwise(v, scal.Add) or len(v.owner.inputs) != 2:
+        return None
+    a, b = v.owner.inputs
+    for one, e in ((a, b), (b, a)):
+        x = _arg_of(e, type(scal.exp))
+        if x is not None and _is_const(one, 1.0):
+            return x
+    return None
+
+
+def _same_type(new, node):
+    return [new] if new.type == node.outputs[0].type else False
+
+
+@local_optimizer([Elemwise])
+def local_log_of_sigmoid(fgraph, node):
+    """``log(sigmoid(x)) -> -softplus(-x)``, ``log(1 - sigmoid(x)) -> -softplus(x)``,
+    ``log1p(exp(x)) -> softplus(x)``, ``log1p(-sigmoid(x)) -> -softplus(x)``: finite where the
+    plain formulas give -inf (``logsigm_to_softplus``, ``log1msigm_to_softplus``,
+    ``log1pexp_to_softplus``, ``log1p_neg_sigmoid``, sigm.py:378-425)."""
+    sop = node.op.scalar_op
+    if len(node.inputs) != 1 or node.outputs[0].type.dtype not in _FLOATS:
+        return False
+    (v,) = node.inputs
+    if isinstance(sop, type(scal.log)):
+        x = _arg_of(v, scal.ScalarSigmoid)
+        if x is not None:
+            return _same_type(T.neg(softplus(_negated(x))), node)
+        if _is_elemwise(v, scal.Sub) and _is_const(v.owner.inputs[0], 1.0):
+            x = _arg_of(v.owner.inputs[1], scal.ScalarSigmoid)
+            if x is not None and x.type.broadcastable == v.type.broadcastable:
+                return _same_type(T.neg(softplus(x)), node)
+        return False
+    if isinstance(sop, type(scal.log1p)):
+        x = _arg_of(v, type(scal.exp))
+        if x is not None:
+            return _same_type(softplus(x), node)
+        inner = _arg_of(v, scal.Neg)
+        x = _arg_of(inner, scal.ScalarSigmoid) if inner is not None else None
+        if x is not None:
+            return _same_type(T.neg(softplus(x)), node)
+    return False
+
+
+def _factors(v):
+    return list(v.owner.inputs) if _is_elemwise(v, scal.Mul) else [v]
+
+
+@local_optimizer([Elemwise])
+def local_exp_over_1_plus_exp(fgraph, node):
+    """``exp(x) / (1 + exp(x)) -> sigmoid(x)`` and ``c / (1 + exp(x)) -> c * sigmoid(-x)``, also with
+    further factors on either side of the division (sigm.py:588-640): no overflow of exp."""
+    if not isinstance(node.op.scalar_op, scal.TrueDiv) or node.outputs[0].type.dtype not in _FLOATS:
+        return False
+    num, den = node.inputs
+    num_f, den_rest, sigmoids = _factors(num), [], []
+    for d in _factors(den):
+        x = _one_plus_exp(d)
+        if x is None or d.type.dtype != node.outputs[0].type.dtype:
+            den_rest.append(d)
+            continue
+        for k, f in enumerate(num_f):
+            if _arg_of(f, type(scal.exp)) is x:
+                del num_f[k]
+                sigmoids.append(sigmoid(x))
+                break
+        else:
+            sigmoids.append(sigmoid(_negated(x)))
+    if not sigmoids:
+        return False
+    num_f = [f for f in num_f if not _is_const(f, 1.0)] + sigmoids
+    new = num_f[0] if len(num_f) == 1 else T.mul(*num_f)
+    if den_rest:
+        new = new / (den_rest[0] if len(den_rest) == 1 else T.mul(*den_rest))
+    return _same_type(new, node)
+
+
+@local_optimizer([Elemwise])
+def local_sigm_times_exp(fgraph, node):
+    """``sigmoid(x) * exp(-x) -> sigmoid(-x)`` and ``sigmoid(-x) * exp(x) -> sigmoid(x)`` among the
+    factors of one product (the flat case of sigm.py:845-905)."""
+    if not isinstance(node.op.scalar_op, scal.Mul):
+        return False
+    fs = list(node.inputs)
+    for i, f in enumerate(fs):
+        x = _arg_of(f, scal.ScalarSigmoid)
+        if x is None:
+            continue
+        for j, g in enumerate(fs):
+            e = _arg_of(g, type(scal.exp))
+            if e is None or j == i:
+                continue
+            if _arg_of(e, scal.Neg) is x or _arg_of(x, scal.Neg) is e:
+                rest = [h for k, h in enumerate(fs) if k not in (i, j)]
+                new = sigmoid(_negated(x))
+                if rest:
+                    new = T.mul(*(rest + [new]))
+                if new.type.broadcastable != node.outputs[0].type.broadcastable:
+                    return False
+                return _same_type(new, node)
+    return False
+
+
+RECOGNIZE = [local_softmax_simplifier, local_softmax_with_bias, local_logsoftmax, local_logsoftmax_grad,
+             local_log_of_sigmoid, local_exp_over_1_plus_exp, local_sigm_times_exp]
 LOWER = [local_lower_row_ops]
+
+
+ultra_fast_sigmoid = T._elemwise(scal.ultra_fast_scalar_sigmoid, "ultra_fast_sigmoid")
+softsign = T._elemwise(scal.scalar_softsign, "softsign")
+
+
+def hard_sigmoid(x):
+    """``clip(0.2 * x + 0.5, 0, 1)`` in the dtype ``upgrade_to_float`` gives (sigm.py:278-297)."""
+    x = as_tensor_variable(x)
+    out_dtype = scal.upgrade_to_float(scal.Scalar(x.type.dtype))[0].dtype
+    slope = T.constant(0.2, dtype=out_dtype)
+    shift = T.constant(0.5, dtype=out_dtype)
+    return T.clip(x * slope + shift, 0, 1)
+
+
+def elu(x, alpha=1):
+    """``x if x > 0 else alpha * (exp(x) - 1)`` (nnet.py:2437-2456)."""
+    x = as_tensor_variable(x)
+    return T.switch(x > 0, x, alpha * T.expm1(x))
+
+
+def selu(x):
+    """``scale * elu(x, alpha)`` with the self-normalising constants (nnet.py:2459-2481)."""
+    alpha = 1.6732632423543772848170429916717
+    scale = 1.0507009873554804934193349852946
+    return scale * elu(x, alpha)
+
+
+def binary_crossentropy(output, target):
+    """``-(target * log(output) + (1 - target) * log(1 - output))``, per component (nnet.py:2008-2025)."""
+    output, target = as_tensor_variable(output), as_tensor_variable(target)
+    return -(target * T.log(output) + (1.0 - target) * T.log(1.0 - output))
+
+
+_sigmoid_binary_crossentropy = T._elemwise(scal.sigmoid_binary_crossentropy, "sigmoid_binary_crossentropy")
+
+
+def sigmoid_binary_crossentropy(output, target):
+    """Cross-entropy of ``sigmoid(output)`` against ``target`` in its stable form
+    ``softplus(-|output|) + output * ((output > 0) - target)``, with the gradients
+    ``sigmoid(output) - target`` and ``-output`` (nnet.py:2028-2050).  Where the reference wraps the
+    formula in an inlined sub-graph with overridden gradients, this is one scalar op of the same
+    formula and gradients: it fuses like any other."""
+    return _sigmoid_binary_crossentropy(as_tensor_variable(output), as_tensor_variable(target))
+
+
+def categorical_crossentropy(coding_dist, true_dist):
+    """``-sum(true_dist * log(coding_dist), axis=-1)`` for a distribution per row
+    (nnet.py:2053-2102).  The form that takes one class index per row goes through advanced
+    indexing, which this package does not have."""
+    coding_dist, true_dist = as_tensor_variable(coding_dist), as_tensor_variable(true_dist)
+    if true_dist.type.ndim == coding_dist.type.ndim:
+        return -T.sum(true_dist * T.log(coding_dist), axis=coding_dist.type.ndim - 1)
+    if true_dist.type.ndim == coding_dist.type.ndim - 1:
+        raise NotImplementedError("categorical_crossentropy with class indices needs advanced indexing")
+    raise TypeError("rank mismatch between coding and true distributions")
 
 
 def relu(x, alpha=0):
