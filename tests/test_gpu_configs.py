@@ -227,3 +227,45 @@ def test_softmax_ops_and_the_rewrites_that_produce_them():
     for k, (g, r) in enumerate(zip(got, ref)):
         assert np.isfinite(g).all(), k
         assert_parity(g, r, "softmax output %d" % k, tol=dict(rtol=2e-5, atol=2e-6))
+
+
+def test_rows_too_long_for_one_block_and_strided_rows_take_the_fused_multi_kernel_path():
+    """Softmax, log-softmax and their gradients on rows of 50 000 elements (beyond what one block keeps in
+    registers) and on a transposed operand: the row-chain node then runs its island as reductions with fused
+    prologues / epilogues - 3 launches for a softmax - with the same results."""
+    from theano_amd.hip import HipRowChain
+    rng = np.random.default_rng(43)
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    sm = T.nnet.softmax(x)
+    outs = [sm, T.nnet.logsoftmax(x), th.grad(T.sum(sm * y), x)]
+    f = th.function([x, y], outs)
+    chains = [n for n in f.toposort() if isinstance(n.op, HipRowChain)]
+    assert chains
+    xv = (3 * rng.standard_normal((6, 50000))).astype("float32")
+    yv = rng.uniform(0, 1, (6, 50000)).astype("float32")
+    got = f(xv, yv)
+    ref = G.evaluate([x, y], outs, [xv, yv])
+    for k, (g, r) in enumerate(zip(got[:2], ref[:2])):
+        assert_parity(g, r, "long rows, output %d" % k, tol=dict(rtol=2e-5, atol=2e-6))
+    assert np.allclose(got[0].sum(axis=1), 1.0, atol=1e-5)
+    # SoftmaxGrad.perform adds a row's 50 000 float32 products one by one in float32 (nnet.py:321, off by
+    # 6e-5 here); the device accumulates in double like the op's C code (nnet.py:396): compare with float64
+    x64, y64 = xv.astype("float64"), yv.astype("float64")
+    e = np.exp(x64 - x64.max(axis=1, keepdims=True))
+    s64 = e / e.sum(axis=1, keepdims=True)
+    assert_parity(got[2], (s64 * (y64 - (s64 * y64).sum(axis=1, keepdims=True))).astype("float32"),
+                  "long rows, gradient", tol=dict(rtol=2e-5, atol=2e-6))
+    plans = [n.op._fallback_plan for n in chains if getattr(n.op, "_fallback_plan", None) is not None]
+    assert plans, "the one-kernel form was not expected to take these rows"
+    # the softmax alone: row max, sum of exp (prologue-fused), normalise
+    g = th.function([x], sm)
+    g(xv)
+    (chain,) = [n for n in g.toposort() if isinstance(n.op, HipRowChain)]
+    kinds = [type(n.op).__name__ for n in chain.op._fallback_plan[2] if type(n.op).__name__ != "HipDimShuffle"]
+    assert sorted(kinds) == ["HipCAReduce", "HipCAReduce", "HipElemwise"], kinds
+    # rows that are not contiguous: the same function on a transposed view
+    z = T.fmatrix("z")
+    h = th.function([z], T.nnet.softmax(z.T))
+    zv = (2 * rng.standard_normal((700, 90))).astype("float32")
+    e = np.exp(zv.T.astype("float64") - zv.T.max(axis=1, keepdims=True))
+    assert np.allclose(h(zv), e / e.sum(axis=1, keepdims=True), rtol=2e-5, atol=1e-7)

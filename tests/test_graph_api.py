@@ -686,3 +686,23 @@ def test_activation_front_ends(dry_run):
         nnet.categorical_crossentropy(nnet.softmax(x), T.ivector("y"))
     with pytest.raises(Exception):
         th.grad(T.sum(nnet.ultra_fast_sigmoid(x)), x)      # no gradient, as in the reference
+
+
+def test_exp_feeding_a_sum_and_a_division_is_recomputed_not_stored(dry_run):
+    """Without the row-chain kernel a softmax is three launches - row max, sum of exp(x - max) computed on the
+    fly, exp(x - max) / sum - because one exp per consumer is cheaper than writing the exponentials and
+    reading them back; the flag that allows no transcendental in a duplicated producer gives four."""
+    from theano_amd.hip import HipCAReduce
+    x = T.fmatrix("x")
+    e = T.exp(x - T.max(x, axis=1, keepdims=True))
+    sm = e / T.sum(e, axis=1, keepdims=True)
+    f = th.function([x], sm, rowchain=False)
+    assert (len(ops_of(f, HipCAReduce)), len(ops_of(f, HipElemwise))) == (2, 1)
+    with th.config.change_flags(duplicate_transcendentals=0):
+        g = th.function([x], sm, rowchain=False)
+    assert (len(ops_of(g, HipCAReduce)), len(ops_of(g, HipElemwise))) == (2, 2)
+    # a per-row value broadcast against the reduction's operand is never recomputed per element
+    r = T.exp(T.max(x, axis=1, keepdims=True))
+    h = th.function([x], [T.sum(x * r, axis=0), x + r], rowchain=False)
+    pro = [n for n in ops_of(h, HipCAReduce) if n.op.pre_scalar_op is not None]
+    assert all("exp" not in str(n.op.pre_scalar_op) for n in pro)

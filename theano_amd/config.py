@@ -19,6 +19,10 @@ class _Config(object):
     # sum(sqr(x - mean(x))) over float16 / float32 data becomes one pass of shifted sums
     # accumulated in float64, merged with the pass that computes the mean
     single_pass_variance = True
+    # An elementwise result that several kernels read is recomputed inside each of them, instead of
+    # written once and read back, when it costs a few ALU instructions and at most this many calls of
+    # exp / log / sqrt / tanh / sigmoid
+    duplicate_transcendentals = int(os.environ.get("THEANO_AMD_DUP_TRANSCENDENTALS", "1"))
 
     @contextlib.contextmanager
     def change_flags(self, **kw):

@@ -139,13 +139,20 @@ _TRIVIAL_OPS = (scal.Cast, scal.Add, scal.Sub, scal.Mul, scal.Neg, scal.Sqr, sca
 _CHEAP_OPS = _TRIVIAL_OPS + (scal.TrueDiv, scal.Inv)
 
 
-def _cheap(scalar_op, ops=None):
-    """True when recomputing the op per consumer costs a few ALU instructions
-    (no transcendental function)."""
+# one hardware transcendental plus a few multiplies: worth redoing once per consumer kernel when that saves
+# writing a full-size array and reading it back, never per element of a broadcast
+_TRANSCENDENTAL_OPS = tuple(type(o) for o in (scal.exp, scal.exp2, scal.expm1, scal.log, scal.log2, scal.log10,
+                                              scal.log1p, scal.sqrt, scal.tanh)) + (scal.ScalarSigmoid,)
+
+
+def _cheap(scalar_op, ops=None, transcendentals=0):
+    """True when recomputing the op per consumer costs a few ALU instructions (at most
+    ``transcendentals`` calls of exp / log / sqrt / tanh / sigmoid among them)."""
     ops = ops or _CHEAP_OPS
-    if isinstance(scalar_op, scal.Composite):
-        return all(isinstance(n.op, ops) for n in gof.io_toposort(scalar_op.inputs, scalar_op.outputs))
-    return isinstance(scalar_op, ops)
+    sops = ([n.op for n in gof.io_toposort(scalar_op.inputs, scalar_op.outputs)]
+            if isinstance(scalar_op, scal.Composite) else [scalar_op])
+    heavy = [o for o in sops if not isinstance(o, ops)]
+    return len(heavy) <= transcendentals and all(isinstance(o, _TRANSCENDENTAL_OPS) for o in heavy)
 
 
 def _absorbs(client, var):
@@ -168,7 +175,18 @@ def _duplicable(fgraph, var):
     it back: inputs x consumers <= inputs + output x (1 + consumers)."""
     node = var.owner
     clients = fgraph.clients.get(var, [])
-    if len(clients) < 2 or len(clients) > 8 or not _cheap(node.op.scalar_op):
+    if len(clients) < 2 or len(clients) > 8:
+        return False
+    # exp(x - m) read by a sum and by a division is worth two evaluations (the sum's kernel never writes
+    # it); among elementwise consumers only, the sibling merge computes it once in one kernel anyway
+    def full_size_operand_of(c):
+        if c == "output" or not isinstance(c.op, HipCAReduce):
+            return False
+        arrays = [i.type.broadcastable for i in c.inputs[:len(c.inputs) - c.op.n_extra] if isinstance(i.type, HipArrayType)]
+        return tuple(var.type.broadcastable) == tuple(all(bs) for bs in zip(*arrays))
+
+    feeds_reduction = any(full_size_operand_of(c) for c, _ in clients)   # per element of a broadcast: never
+    if not _cheap(node.op.scalar_op, transcendentals=config.duplicate_transcendentals if feeds_reduction else 0):
         return False
     if not all(_absorbs(c, var) for c, _ in clients):
         return False
@@ -748,19 +766,25 @@ def optimize(fgraph, fuse=True, rowchain=True, inplace=True):
         if rowchain:
             from .rowchain import fuse_row_chains
             fuse_row_chains(fgraph)
-        merge_sibling_reductions(fgraph)
-        fuse_reduce_prologue(fgraph)
-        gof.merge_identical(fgraph)
-        merge_sibling_reductions(fgraph)
-        gof.merge_identical(fgraph)
-        fuse_reduce_epilogue(fgraph)
-        fuse_argmax_prologue(fgraph)
-        gof.merge_identical(fgraph)
-        fuse_elemwise(fgraph)          # producers that lost their other clients to an epilogue
-        gof.merge_identical(fgraph)
-        if merge_sibling_elemwise(fgraph):
-            fuse_elemwise(fgraph)      # a producer whose clients all ended up in one kernel joins it
-            gof.merge_identical(fgraph)
+        fuse_around_reductions(fgraph)
     if inplace:
         inplace_elemwise(fgraph)
     return fgraph
+
+
+def fuse_around_reductions(fgraph):
+    """The passes that follow elementwise fusion on a lifted graph: reductions take in their
+    elementwise producers and consumers, siblings share a launch."""
+    merge_sibling_reductions(fgraph)
+    fuse_reduce_prologue(fgraph)
+    gof.merge_identical(fgraph)
+    merge_sibling_reductions(fgraph)
+    gof.merge_identical(fgraph)
+    fuse_reduce_epilogue(fgraph)
+    fuse_argmax_prologue(fgraph)
+    gof.merge_identical(fgraph)
+    fuse_elemwise(fgraph)          # producers that lost their other clients to an epilogue
+    gof.merge_identical(fgraph)
+    if merge_sibling_elemwise(fgraph):
+        fuse_elemwise(fgraph)      # a producer whose clients all ended up in one kernel joins it
+        gof.merge_identical(fgraph)

@@ -204,11 +204,26 @@ class HipRowChain(Op):
             output_storage[k][0] = arr
 
     def _run_fallback(self, inputs):
-        """Shapes or strides the one-kernel form does not take (very long rows,
-        non-contiguous rows): run the island node by node on the device."""
-        inner_in, inner_out = self.fallback
+        """Shapes or strides the one-kernel form does not take (rows too long for the registers of
+        one block, non-contiguous rows): the island runs as reductions that compute their
+        elementwise producers and consumers on the fly plus the elementwise kernels in between,
+        fused the first time this is needed; intermediate results are dropped after their last use."""
+        plan = getattr(self, "_fallback_plan", None)
+        if plan is None:
+            from . import opt
+            fg = gof.FunctionGraph(*self.fallback)
+            opt.fuse_around_reductions(fg)
+            opt.inplace_elemwise(fg)
+            order = fg.toposort()
+            last_use = {}
+            for k, n in enumerate(order):
+                for i in n.inputs:
+                    last_use[id(i)] = k
+            keep = set(id(o) for o in fg.outputs) | set(id(i) for i in fg.inputs)
+            plan = self._fallback_plan = (list(fg.inputs), list(fg.outputs), order, last_use, keep)
+        inner_in, inner_out, order, last_use, keep = plan
         storage = dict((id(v), [val]) for v, val in zip(inner_in, inputs))
-        for n in gof.io_toposort(inner_in, inner_out):
+        for k, n in enumerate(order):
             args = []
             for i in n.inputs:
                 cell = storage.get(id(i))
@@ -219,6 +234,9 @@ class HipRowChain(Op):
             n.op.perform(n, args, cells)
             for o, c in zip(n.outputs, cells):
                 storage[id(o)] = c
+            for i in n.inputs:
+                if last_use.get(id(i)) == k and id(i) not in keep:
+                    storage.pop(id(i), None)
         return [storage[id(o)][0] for o in inner_out]
 
 

@@ -1283,6 +1283,16 @@ class Composite(ScalarOp):
                         n2.inputs = [repl.get(i, i) for i in n2.inputs]
                     changed = True
                     break
+        # equal ops on the same values are computed once (the merge of theano/scalar/basic.py:3915-3925)
+        first, repl = {}, {}
+        for node in gof.io_toposort(inputs, outputs):
+            node.inputs = [repl.get(i, i) for i in node.inputs]
+            key = (node.op, tuple(("c", str(i.type), repr(i.data)) if isinstance(i, Constant) else id(i)
+                                  for i in node.inputs))
+            prev = first.setdefault(key, node)
+            if prev is not node:
+                repl.update(zip(node.outputs, prev.outputs))
+        outputs = [repl.get(o, o) for o in outputs]
         self.inputs = inputs
         self.outputs = outputs
         self.inputs_type = tuple(i.type for i in inputs)
