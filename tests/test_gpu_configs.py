@@ -230,9 +230,10 @@ def test_softmax_ops_and_the_rewrites_that_produce_them():
 
 
 def test_rows_too_long_for_one_block_and_strided_rows_take_the_fused_multi_kernel_path():
-    """Softmax, log-softmax and their gradients on rows of 50 000 elements (beyond what one block keeps in
+    """Softmax, log-softmax and their gradients on rows of 100 000 elements (beyond what one block keeps in
     registers) and on a transposed operand: the row-chain node then runs its island as reductions with fused
-    prologues / epilogues - 3 launches for a softmax - with the same results."""
+    prologues / epilogues - 3 launches for a softmax - with the same results.  Rows of 50 000 elements still
+    fit one block of 1024 threads."""
     from theano_amd.hip import HipRowChain
     rng = np.random.default_rng(43)
     x, y = T.fmatrix("x"), T.fmatrix("y")
@@ -241,14 +242,20 @@ def test_rows_too_long_for_one_block_and_strided_rows_take_the_fused_multi_kerne
     f = th.function([x, y], outs)
     chains = [n for n in f.toposort() if isinstance(n.op, HipRowChain)]
     assert chains
-    xv = (3 * rng.standard_normal((6, 50000))).astype("float32")
-    yv = rng.uniform(0, 1, (6, 50000)).astype("float32")
+    for cols in (50000, 100000):
+        xv = (3 * rng.standard_normal((6, cols))).astype("float32")
+        ev = np.exp(xv.astype("float64") - xv.max(axis=1, keepdims=True))
+        one = th.function([x], sm)
+        assert np.allclose(one(xv), ev / ev.sum(axis=1, keepdims=True), rtol=2e-5, atol=1e-9), cols
+        (chain,) = [n for n in one.toposort() if isinstance(n.op, HipRowChain)]
+        assert (getattr(chain.op, "_fallback_plan", None) is None) == (cols == 50000)
+    yv = rng.uniform(0, 1, xv.shape).astype("float32")
     got = f(xv, yv)
     ref = G.evaluate([x, y], outs, [xv, yv])
     for k, (g, r) in enumerate(zip(got[:2], ref[:2])):
         assert_parity(g, r, "long rows, output %d" % k, tol=dict(rtol=2e-5, atol=2e-6))
     assert np.allclose(got[0].sum(axis=1), 1.0, atol=1e-5)
-    # SoftmaxGrad.perform adds a row's 50 000 float32 products one by one in float32 (nnet.py:321, off by
+    # SoftmaxGrad.perform adds a row's 100 000 float32 products one by one in float32 (nnet.py:321, off by
     # 6e-5 here); the device accumulates in double like the op's C code (nnet.py:396): compare with float64
     x64, y64 = xv.astype("float64"), yv.astype("float64")
     e = np.exp(x64 - x64.max(axis=1, keepdims=True))

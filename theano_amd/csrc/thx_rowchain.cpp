@@ -14,6 +14,7 @@ struct thx_rowchain {
   int n_in = 0, n_out = 0;
   std::vector<int32_t> dtypes, kinds;
   std::unordered_map<std::string, thx::Kernel> plans;
+  std::unordered_map<std::string, int> spill_bytes;  // per plan: private memory per thread of the compiled kernel
 };
 
 namespace thx {
@@ -176,6 +177,11 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
   } else if (cv <= 16 * 256) {
     tpr = 256;
     nch = (int)((cv + 255) / 256);
+  } else if (cv <= 16 * 1024 && !(getenv("THX_ROW_BIG") && atoi(getenv("THX_ROW_BIG")) == 0)) {
+    // one block of 1024 threads per row (128 registers per thread: chains that keep several row-sized
+    // values alive spill, and are turned away below)
+    tpr = 1024;
+    nch = (int)((cv + 1023) / 1024);
   } else {
     return fail(THX_ERR_UNSUPPORTED, "rowchain: rows of %lld elements do not fit in registers", (long long)C);
   }
@@ -190,7 +196,7 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
     int64_t span = (rows - 1) * (rstride[i] < 0 ? -rstride[i] : rstride[i]) + C;
     if (span >= (int64_t(1) << 31) - 65536) wide = true;
   }
-  const int block = 256;
+  const int block = tpr == 1024 ? 1024 : 256;
   int64_t moved = 0;
   for (int i = 0; i < NOPS; ++i)
     if (c->kinds[i] == K_FULL) moved += rows * C * dtype_size(c->dtypes[i]);
@@ -233,6 +239,19 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
     c->plans[plan] = k;
   }
   if (dry) return THX_OK;
+  if (tpr == 1024) {
+    // a row per 1024-thread block leaves 128 registers a thread; a chain that needs more keeps its rows
+    // in private memory, which costs more traffic than the separate kernels the caller falls back to
+    auto sp = c->spill_bytes.find(plan);
+    if (sp == c->spill_bytes.end()) {
+      int bytes = 0;
+      THX_HIP_CHECK(hipFuncGetAttribute(&bytes, HIP_FUNC_ATTRIBUTE_LOCAL_SIZE_BYTES, k.func));
+      sp = c->spill_bytes.emplace(plan, bytes).first;
+    }
+    if (sp->second > 0 && !(getenv("THX_ROW_BIG") && atoi(getenv("THX_ROW_BIG")) == 2))
+      return fail(THX_ERR_UNSUPPORTED, "rowchain: rows of %lld elements need %d bytes of private memory per thread",
+                  (long long)C, sp->second);
+  }
 
   ParamPack pk;
   for (int i = 0; i < NIN; ++i) pk.put<char*>(ptr[i]);
