@@ -385,3 +385,11 @@ def test_sigmoid_family_and_stabilised_forms(dtype):
     for g, r in zip(got, ref):
         assert_parity(g, r, "approximate sigmoid / softsign")
     assert np.abs(got[0] - sg).max() < 0.028
+
+
+def test_gradient_of_log_one_minus_sigmoid_reference_values():
+    """The literal answers of test_grad_useless_sum (theano/tensor/tests/test_elemwise.py:1281-1297)."""
+    x = T.TensorType("float32", (True,))("x")
+    f = th.function([x], th.grad(T.log(1.0 - T.nnet.sigmoid(x))[0], x))
+    got = [f(np.array([v], "float32")) for v in (-100, -1, 0, 1, 100)]
+    assert np.allclose(got, [[-3.72007598e-44], [-0.26894142], [-0.5], [-0.73105858], [-1.]])

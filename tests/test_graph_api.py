@@ -706,3 +706,66 @@ def test_exp_feeding_a_sum_and_a_division_is_recomputed_not_stored(dry_run):
     h = th.function([x], [T.sum(x * r, axis=0), x + r], rowchain=False)
     pro = [n for n in ops_of(h, HipCAReduce) if n.op.pre_scalar_op is not None]
     assert all("exp" not in str(n.op.pre_scalar_op) for n in pro)
+
+
+def test_gradient_corner_cases_of_the_reference_elemwise_tests(dry_run):
+    """theano/tensor/tests/test_elemwise.py:1154-1350: gradients through all / any and through integer-valued
+    costs are zeros, comparisons pass no gradient, a gradient an op declares not implemented raises only when
+    it is asked for, and gradients with respect to broadcast inputs build."""
+    from oracle import graph_ref as G
+    from theano_amd import gradient
+    x = T.bmatrix("x")
+    xv = np.random.RandomState(0).binomial(1, 0.5, (5, 7)).astype("int8")
+    for red in (x.all(), x.any()):
+        gx = th.grad(red, x)
+        for v in (xv, np.zeros_like(xv), np.ones_like(xv)):
+            g = G.evaluate([x], [gx], [v])[0]
+            assert g.shape == v.shape and np.all(g == 0)
+        th.function([x], gx)
+    b, i8 = T.TensorType("bool", ())("b"), T.TensorType("int8", ())("i")
+    assert [g.type.dtype for g in th.grad(b * i8, [b, i8])] == ["float32", "float32"]
+    ints = [T.TensorType("int32", ())(n) for n in "xyz"]
+    assert len(th.grad(T.clip(*ints), ints)) == 3
+    s = T.fvector("s")
+    scores = T.ones_like(s) - s + s * 2
+    g = th.grad((scores * (scores > 0)).sum(), s)
+    assert np.array_equal(G.evaluate([s], [g], [np.array([0.5, -3, 2], "float32")])[0], [1, 0, 1])
+    t4 = T.TensorType("float32", (True, False, False, False))("x4")
+    y4 = T.TensorType("float32", (True, True, False, False))("y4")
+    gx4, gy4 = th.grad(T.tanh(t4 + y4).sum(), [t4, y4])
+    assert gx4.type == t4.type and gy4.type == y4.type
+
+    class Scale(scal.ScalarOp):
+        nin = 2
+
+        def __init__(self):
+            self.output_types_preference = scal.upgrade_to_float
+            self.name = "scale"
+
+        def L_op(self, inputs, outputs, gout):
+            n, v = inputs
+            return [gradient.grad_not_implemented(self, 0, n), gout[0] * n]
+
+    op = Elemwise(Scale())
+    v = T.TensorType("float32", ())("v")
+    th.grad(op(2, v), v)
+    with pytest.raises(gradient.NullTypeGradError):
+        th.grad(op(v, 2), v)
+    with pytest.raises(gradient.NullTypeGradError):
+        th.grad(T.exp(op(v, 2)) * 3, v)          # also through further nodes
+
+
+def test_gradient_of_log_one_minus_sigmoid_cancels_to_minus_sigmoid(dry_run):
+    """test_grad_useless_sum, theano/tensor/tests/test_elemwise.py:1262-1297: no Sum node for a broadcastable
+    input, and the factor 1 - sigmoid(x) leaves the quotient, so the compiled kernel is -(g * sigmoid(x))."""
+    from theano_amd import gof
+    x = T.TensorType("float32", (True,))("x")
+    g = th.grad(T.log(1.0 - T.nnet.sigmoid(x))[0], x)
+    assert not any(isinstance(n.op, Sum) for n in gof.io_toposort([x], [g]))
+    f = th.function([x], g)
+    (k,) = ops_of(f, HipElemwise)
+    assert str(k.op.scalar_op) == "Composite{neg(mul(i0, scalar_sigmoid(i1)))}"
+    # a factor that gives the result its shape stays
+    m, r = T.fmatrix("m"), T.frow("r")
+    h = th.function([m, r], (r / m) * m)
+    assert any("true_div" in str(n.op) or "mul" in str(n.op) for n in h.toposort())

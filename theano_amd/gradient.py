@@ -17,6 +17,43 @@ class DisconnectedInputError(ValueError):
     pass
 
 
+class NullTypeGradError(TypeError):
+    """The gradient asked for runs through a term an op declared not implemented or undefined."""
+
+
+class NullType(gof.Type):
+    """Type of the placeholder an ``L_op`` returns for a gradient it cannot give
+    (``theano/gof/null_type.py``): no value, only a reason."""
+
+    def __init__(self, why_null="(no default value given)"):
+        self.why_null = why_null
+
+    def filter(self, data, strict=False, allow_downcast=None):
+        raise ValueError("No values may be assigned to a NullType")
+
+    def __eq__(self, other):
+        return type(self) == type(other)
+
+    def __hash__(self):
+        return hash(type(self))
+
+    def __str__(self):
+        return "NullType"
+
+
+def grad_not_implemented(op, x_pos, x, comment=""):
+    """What an ``L_op`` returns for input ``x_pos`` when that gradient is not implemented
+    (``theano/gradient.py:1995-2034``); asking for it raises NullTypeGradError."""
+    return NullType("This variable is Null because the grad method for input %s (%s) of the %s op is not "
+                    "implemented. %s" % (x_pos, x, op, comment))()
+
+
+def grad_undefined(op, x_pos, x, comment=""):
+    """Same, for a gradient that is mathematically undefined (``theano/gradient.py:2037-2074``)."""
+    return NullType("This variable is Null because the grad method for input %s (%s) of the %s op is "
+                    "mathematically undefined. %s" % (x_pos, x, op, comment))()
+
+
 def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
     """Symbolic gradient of the 0-d ``cost`` with respect to ``wrt`` (a variable
     or a list of variables)."""
@@ -29,9 +66,9 @@ def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
     if cost is not None:
         if cost.type.ndim != 0:
             raise TypeError("cost must be a scalar.")
-        if cost.type.dtype not in scal.continuous_dtypes:
-            raise TypeError("cost must be floating point, not %s" % cost.type.dtype)
-        grads[cost] = T.ones_like(cost)
+        # an integer-valued cost has zero gradients everywhere (theano/gradient.py:_float_ones_like)
+        grads[cost] = (T.ones_like(cost) if cost.type.dtype in scal.continuous_dtypes
+                       else T.ones_like(cost, dtype=config.floatX))
     for var, g in (known_grads or {}).items():
         grads[var] = as_tensor_variable(g)
     outputs = list(grads.keys())
@@ -49,6 +86,7 @@ def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
             continue
         ograds = []
         connected = False
+        null = None
         for o in node.outputs:
             g = grads.get(o)
             if g is None:
@@ -56,7 +94,15 @@ def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
             else:
                 connected = True
                 ograds.append(g)
+                if isinstance(g.type, NullType):
+                    null = g
         if not connected:
+            continue
+        if null is not None:
+            # nothing can be said about what lies behind an unknown gradient
+            for i in node.inputs:
+                if id(i) in depends:
+                    grads[i] = null
             continue
         if len(node.outputs) == 1 and getattr(node.outputs[0].type, "dtype", "float32") not in scal.continuous_dtypes:
             # integer-valued results carry no gradient to their inputs
@@ -75,6 +121,11 @@ def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
                 continue
             if id(i) not in depends:
                 continue
+            if isinstance(g.type, NullType):
+                grads[i] = g
+                continue
+            if i in grads and isinstance(grads[i].type, NullType):
+                continue
             if g.type.dtype not in scal.continuous_dtypes:
                 continue
             if hasattr(i.type, "broadcastable") and g.type.broadcastable != i.type.broadcastable:
@@ -84,6 +135,8 @@ def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
     result = []
     for w in wrt_list:
         g = grads.get(w)
+        if g is not None and isinstance(g.type, NullType):
+            raise NullTypeGradError("grad encountered a NaN. " + g.type.why_null)
         if g is None:
             if disconnected_inputs == "raise":
                 raise DisconnectedInputError("grad method was asked to compute the gradient with respect to a "

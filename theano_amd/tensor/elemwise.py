@@ -211,7 +211,7 @@ class Elemwise(Op):
         if any(o.type.dtype not in scal.continuous_dtypes for o in outs):
             new = []
             for elem, ipt in zip(rval, inputs):
-                if isinstance(elem.type, DisconnectedType):
+                if isinstance(elem.type, DisconnectedType) or not hasattr(elem.type, "dtype"):
                     new.append(elem)
                 else:
                     z = ipt.zeros_like()
@@ -221,7 +221,7 @@ class Elemwise(Op):
             return new
         from . import basic
         for i, ipt in enumerate(inputs):
-            if rval[i] is None or isinstance(rval[i].type, DisconnectedType):
+            if rval[i] is None or isinstance(rval[i].type, DisconnectedType) or not hasattr(rval[i].type, "dtype"):
                 continue
             to_sum = [j for j, b in enumerate(ipt.type.broadcastable) if b and not outs[0].type.broadcastable[j]]
             if to_sum:
@@ -231,8 +231,11 @@ class Elemwise(Op):
     def _bgrad(self, inputs, outputs, ograds):
         """Gradient w.r.t. the broadcast inputs: take the scalar op's symbolic
         gradient and rebuild it as a graph of Elemwise nodes."""
+        def passes_through(t):
+            return isinstance(t.type, DisconnectedType) or not hasattr(t.type, "dtype")    # no value behind it
+
         def as_scalar(t):
-            if isinstance(t.type, DisconnectedType):
+            if passes_through(t):
                 return t
             return Scalar(t.type.dtype)()
 
@@ -246,7 +249,7 @@ class Elemwise(Op):
         memo = {}
 
         def transform(r):
-            if isinstance(r.type, DisconnectedType):
+            if passes_through(r):
                 return r
             for group, tgroup in ((scalar_inputs, inputs), (scalar_outputs, outputs), (scalar_ograds, ograds)):
                 for s, t in zip(group, tgroup):

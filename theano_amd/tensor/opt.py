@@ -488,9 +488,66 @@ def local_single_pass_variance(fgraph, node):
     return [res] if res.type == out.type else False
 
 
+@local_optimizer([Elemwise])
+def local_cancel_common_factors(fgraph, node):
+    """``(a / b) * b -> a``: a factor that appears above and below the line of one product -
+    written with any nesting of ``mul``, ``true_div``, ``neg`` and ``inv`` of one float dtype -
+    is dropped from both (the part of ``local_mul_canonizer``, ``theano/tensor/opt.py:4700-5060``,
+    that turns the gradient of ``log(1 - sigmoid(x))``, ``-(g / (1 - s)) * s * (1 - s)``, into
+    ``-(g * s)``, finite where ``1 - s`` rounds to zero).  Left alone when nothing cancels or
+    when the dropped factor was what gave the result its shape."""
+    out = node.outputs[0]
+    if not isinstance(node.op.scalar_op, (scal.Mul, scal.TrueDiv)) or out.type.dtype not in scal.float_dtypes:
+        return False
+    dt = out.type.dtype
+    num, den = [], []
+
+    def collect(v, above, depth):
+        """Appends the factors of v to num / den; returns whether v is negated."""
+        p = v.owner
+        if (p is not None and isinstance(p.op, Elemwise) and v.type.dtype == dt and depth < 16 and
+                all(i.type.dtype == dt for i in p.inputs)):
+            sop = p.op.scalar_op
+            if isinstance(sop, scal.Mul):
+                sign = False
+                for i in p.inputs:
+                    sign ^= collect(i, above, depth + 1)
+                return sign
+            if isinstance(sop, scal.TrueDiv):
+                a, b = p.inputs
+                return collect(a, above, depth + 1) ^ collect(b, not above, depth + 1)
+            if isinstance(sop, scal.Neg):
+                return not collect(p.inputs[0], above, depth + 1)
+            if isinstance(sop, scal.Inv):
+                return collect(p.inputs[0], not above, depth + 1)
+        (num if above else den).append(v)
+        return False
+
+    sign = collect(out, True, 0)
+    dropped = False
+    for v in list(num):
+        for k, w in enumerate(den):
+            if w is v:
+                num.remove(v)
+                del den[k]
+                dropped = True
+                break
+    if not dropped:
+        return False
+    new = constant(1.0, dtype=dt) if not num else (num[0] if len(num) == 1 else T.mul(*num))
+    if den:
+        new = T.true_div(new, den[0] if len(den) == 1 else T.mul(*den))
+    if sign:
+        new = T.neg(new)
+    if new.type.ndim < out.type.ndim:
+        new = T.shape_padleft(new, out.type.ndim - new.type.ndim)
+    return [new] if new.type == out.type else False
+
+
 CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_constant_fold, local_useless_elemwise, local_fill_sink,
                 local_useless_reduce, local_op_of_op,
-                local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_single_pass_variance]
+                local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_single_pass_variance,
+                local_cancel_common_factors]
 
 
 def canonicalize(fgraph):
