@@ -393,3 +393,44 @@ def test_gradient_of_log_one_minus_sigmoid_reference_values():
     f = th.function([x], th.grad(T.log(1.0 - T.nnet.sigmoid(x))[0], x))
     got = [f(np.array([v], "float32")) for v in (-100, -1, 0, 1, 100)]
     assert np.allclose(got, [[-3.72007598e-44], [-0.26894142], [-0.5], [-0.73105858], [-1.]])
+
+
+def test_pow_over_every_pair_of_integer_and_float_dtypes():
+    """test_elemwise_pow, theano/gpuarray/tests/test_elemwise.py:43-70: base ** exponent for every pair of
+    (u)int8-64 and float16/32/64 dtypes gives NumPy's dtype and values (small exact integers)."""
+    dtypes = ["uint8", "uint16", "uint32", "uint64", "int8", "int16", "int32", "int64", "float16", "float32", "float64"]
+    rng = np.random.RandomState(0)
+    for db in dtypes:
+        base = T.TensorType(db, (False,))("b")
+        exps = [T.TensorType(de, (False,))("e_" + de) for de in dtypes]
+        bv = rng.randint(0, 5, size=10).astype(db)
+        evs = [rng.randint(0, 3, size=10).astype(de) for de in dtypes]
+        got = th.function([base] + exps, [base ** e for e in exps])(bv, *evs)
+        for de, ev, g in zip(dtypes, evs, got):
+            want = bv ** ev
+            assert g.dtype == want.dtype, (db, de, g.dtype, want.dtype)
+            if g.dtype.kind in "iu":
+                assert np.array_equal(g, want), (db, de, g, want)
+            else:                                # the device's pow is within a place of the host's, not identical
+                tol = {"float16": 2e-3, "float32": 1e-6, "float64": 1e-12}[str(g.dtype)]
+                assert np.allclose(g, want, rtol=tol, atol=0), (db, de, g, want)
+
+
+@pytest.mark.parametrize("nd", [2, 8])
+def test_add_and_mul_of_64_operands(nd):
+    """test_many_arg_elemwise, theano/gpuarray/tests/test_opt.py:531-572: more operands than one kernel
+    takes are split over several kernels, in 2 and in 8 dimensions."""
+    from theano_amd.hip import HipElemwise
+    rng = np.random.RandomState([1, 2, 3])
+    shape = [rng.randint(1, 5) for _ in range(nd)]
+    args = [rng.randn(*shape).astype("float32") for _ in range(64)]
+    sym = [T.TensorType("float32", (False,) * nd)() for _ in range(64)]
+    for op, npop in ((T.add, np.add), (T.mul, np.multiply)):
+        f = th.function(sym, op(*sym))
+        kernels = [n for n in f.toposort() if isinstance(n.op, HipElemwise)]
+        assert len(kernels) > 1 and all(len(n.inputs) <= th.config.max_fused_inputs for n in kernels)
+        want = args[0].astype("float64")
+        for a in args[1:]:
+            want = npop(want, a)
+        # 63 float32 additions of N(0, 1) terms: rounding of partial sums near 8 in magnitude, against float64
+        assert np.allclose(f(*args), want, rtol=1e-5, atol=3e-5 if op is T.add else 1e-30)

@@ -769,3 +769,14 @@ def test_gradient_of_log_one_minus_sigmoid_cancels_to_minus_sigmoid(dry_run):
     m, r = T.fmatrix("m"), T.frow("r")
     h = th.function([m, r], (r / m) * m)
     assert any("true_div" in str(n.op) or "mul" in str(n.op) for n in h.toposort())
+
+
+def test_more_operands_than_a_kernel_takes_are_split(dry_run):
+    """add / mul of 64 tensors (theano/gpuarray/tests/test_opt.py:531-572) compile to kernels of at most
+    ``max_fused_inputs`` operands, and fusion does not grow a node past that limit afterwards."""
+    sym = [T.fmatrix() for _ in range(64)]
+    for op in (T.add, T.mul):
+        f = th.function(sym, op(*sym) * 2.0)
+        kernels = ops_of(f, HipElemwise)
+        assert len(kernels) > 1 and all(len(n.inputs) <= th.config.max_fused_inputs for n in kernels)
+        f(*[np.zeros((3, 4), "float32")] * 64)           # plans and compiles

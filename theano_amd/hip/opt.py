@@ -252,7 +252,7 @@ def _fuse_node(fgraph, node):
                 fused = True
             else:
                 s_args.append(scalar_for(i))
-    if not fused or not inputs:
+    if not fused or not inputs or len(inputs) > max(config.max_fused_inputs, len(node.inputs)):
         return None
     s_outs = node.op.scalar_op(*s_args, return_list=True)
     if [s.type.dtype for s in s_outs] != [o.type.dtype for o in node.outputs]:

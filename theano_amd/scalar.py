@@ -772,7 +772,16 @@ mod = Mod(upcast_out, name="mod")
 class Pow(BinaryScalarOp):
     def c_code(self, node, inputs, outputs):
         # C's pow(): arguments promote to double
-        return "%s = pow((double)%s, (double)%s);" % (outputs[0], inputs[0], inputs[1])
+        (x, y), (z,) = inputs, outputs
+        if node.outputs[0].type.dtype in discrete_dtypes:
+            # The host libm the reference runs on returns whole powers of whole numbers exactly, and the
+            # conversion to the integer result truncates.  The device's pow may come out one place short
+            # (pow(3, 1) = 2.9999999999999996 would truncate to 2): round powers with exponents >= 0, which
+            # are whole; negative exponents give at most 1/2 in magnitude beyond |base| = 1 and still truncate.
+            ct = storage_ctype(node.outputs[0].type.dtype)
+            return ("{ const double thx_p = pow((double)%s, (double)%s); %s = ((double)%s < 0) ? (%s)thx_p : (%s)rint(thx_p); }"
+                    % (x, y, z, y, ct, ct))
+        return "%s = pow((double)%s, (double)%s);" % (z, x, y)
 
     def L_op(self, inputs, outputs, gout):
         x, y = inputs

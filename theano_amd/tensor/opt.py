@@ -13,6 +13,7 @@ import numpy as np
 
 from .. import gof
 from .. import scalar as scal
+from ..config import config
 from ..gof import local_optimizer
 from . import basic as T
 from .elemwise import CAReduce, DimShuffle, Elemwise, Sum
@@ -544,10 +545,26 @@ def local_cancel_common_factors(fgraph, node):
     return [new] if new.type == out.type else False
 
 
+@local_optimizer([Elemwise])
+def local_split_huge_add_or_mul(fgraph, node):
+    """``add`` / ``mul`` of more operands than one kernel takes becomes a tree of nodes of at most
+    ``config.max_fused_inputs`` operands each (``split_inputs``, ``theano/gpuarray/opt.py:800-839``); fusion
+    respects the same limit, so no other node can outgrow it."""
+    limit = config.max_fused_inputs
+    if not isinstance(node.op.scalar_op, (scal.Add, scal.Mul)) or len(node.inputs) <= limit:
+        return False
+    terms = list(node.inputs)
+    while len(terms) > limit:
+        terms = [node.op(*terms[k:k + limit]) if len(terms[k:k + limit]) > 1 else terms[k]
+                 for k in range(0, len(terms), limit)]
+    new = node.op(*terms)
+    return [new] if new.type == node.outputs[0].type else False
+
+
 CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_constant_fold, local_useless_elemwise, local_fill_sink,
                 local_useless_reduce, local_op_of_op,
                 local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_single_pass_variance,
-                local_cancel_common_factors]
+                local_cancel_common_factors, local_split_huge_add_or_mul]
 
 
 def canonicalize(fgraph):

@@ -162,6 +162,11 @@ class _tensor_py_operators(object):
             shape = tuple(shape[0])
         return views.reshape(self, shape)
 
+    def fill(self, value):
+        """A tensor of this one's shape filled with ``value`` (``theano/tensor/var.py:_tensor_py_operators.fill``)."""
+        from . import basic
+        return basic.fill(self, value)
+
     def flatten(self, ndim=1):
         from . import views
         return views.flatten(self, ndim)
