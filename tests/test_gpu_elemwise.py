@@ -434,3 +434,36 @@ def test_add_and_mul_of_64_operands(nd):
             want = npop(want, a)
         # 63 float32 additions of N(0, 1) terms: rounding of partial sums near 8 in magnitude, against float64
         assert np.allclose(f(*args), want, rtol=1e-5, atol=3e-5 if op is T.add else 1e-30)
+
+
+def test_float16_composites_and_casts():
+    """test_composite_elemwise_float16 and test_cast_float16, theano/gpuarray/tests/test_elemwise.py:152-207:
+    mixed float16 / integer / float32 expressions fuse and run, and every cast to and from float16 gives
+    NumPy's ``astype`` (the reference only compiles the first two graphs; here they are also checked
+    against the oracle)."""
+    rng = np.random.default_rng(51)
+    w, x, y = T.bvector("w"), T.TensorType("float16", (False,))("x"), T.fvector("y")
+    cz = T.tanh(x + T.cast(y, "float16"))
+    o = cz - cz ** 2 + T.cast(x, "int16") + T.cast(x, "float32") + T.cast(w, "float16") - T.constant(np.float16(1.0))
+    vals = [rng.integers(-5, 5, 300).astype("int8"), rng.uniform(-4, 4, 300).astype("float16"),
+            rng.uniform(-2, 2, 300).astype("float32")]
+    got, ref = run_both([w, x, y], [o], vals)
+    assert got[0].dtype == ref[0].dtype == np.float32
+    assert_parity(got[0], ref[0], "float16 composite", tol=dict(rtol=2e-3, atol=2e-3))
+    v = T.TensorType("uint8", (False,))("v")
+    hs = [T.TensorType("float16", (False,))(n) for n in "abcd"]
+    o2 = T.switch(v, T.mul(hs[0], hs[1], hs[2]), hs[3])
+    vals2 = [rng.integers(0, 2, 300).astype("uint8")] + [rng.uniform(-2, 2, 300).astype("float16") for _ in hs]
+    got, ref = run_both([v] + hs, [o2], vals2)
+    assert got[0].dtype == np.float16
+    assert_parity(got[0], ref[0], "float16 switch", tol=dict(rtol=2e-3, atol=2e-3))
+    f16, f32, i8 = T.TensorType("float16", (False,))("h"), T.fvector("f"), T.bvector("i")
+    outs = [f16.astype("float32"), f32.astype("float16"), f32.astype("float64"), f16.astype("int8"),
+            f32.astype("int8"), i8.astype("float16"), i8.astype("float32")]
+    d1 = (rng.random(4) * 10).astype("float16")
+    d2 = (rng.random(5) * 10).astype("float32")
+    d3 = (rng.random(6) * 10).astype("int8")
+    res = th.function([f16, f32, i8], outs)(d1, d2, d3)
+    srcs = [d1, d2, d2, d1, d2, d3, d3]
+    for r, o, d in zip(res, outs, srcs):
+        assert r.dtype == np.dtype(o.type.dtype) and np.array_equal(r, d.astype(o.type.dtype))
