@@ -118,6 +118,21 @@ def test_reduce_prologue_fusion_and_sibling_merge():
     assert len(red.outputs) == 2 and red.op.scalar_ops == (scal.or_, scal.and_)
 
 
+def test_reductions_sharing_only_a_broadcast_operand_stay_apart(dry_run):
+    """Two reductions over arrays of different run-time shape that share a (1, C) weight must not
+    merge into one kernel: a common operand that is broadcast in both proves nothing about the
+    other operands' extents."""
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    w = T.frow("w")
+    f = th.function([x, y, w], [T.sum(T.exp(x) * w), T.sum(T.tanh(y) * w)])
+    assert len(ops_of(f, HipCAReduce)) == 2
+    f(np.zeros((4, 8), "float32"), np.zeros((6, 8), "float32"), np.zeros((1, 8), "float32"))
+    # a shared full-shaped operand still merges the two
+    g = th.function([x, w], [T.sum(T.exp(x) * w), T.sum(T.tanh(x) * w)])
+    (red,) = ops_of(g, HipCAReduce)
+    assert len(red.outputs) == 2
+
+
 def test_gradient_graph_contains_only_path_ops():
     x, y = T.fmatrix("x"), T.frow("y")
     cost = T.sum(T.tanh(x * y))

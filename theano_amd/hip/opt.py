@@ -586,9 +586,9 @@ def _depends_on(var, node, limit=10000, pos=None):
 
 def merge_sibling_reductions(fgraph):
     """Two reductions over the same axes whose inputs have the same full shape
-    pattern and share at least one input become one multi-output reduction, so
-    shared operands are read once (e.g. ``sum(g)`` and ``sum(g * xhat)``, or
-    ``any`` and ``all`` of one tensor)."""
+    pattern and share at least one input of that full shape become one
+    multi-output reduction, so shared operands are read once (e.g. ``sum(g)`` and
+    ``sum(g * xhat)``, or ``any`` and ``all`` of one tensor)."""
     count = 0
     changed = True
     while changed:
@@ -599,15 +599,19 @@ def merge_sibling_reductions(fgraph):
             for b in reds[ai + 1:]:
                 if a.op.axis != b.op.axis:
                     continue
-                if not set(id(i) for i in a.inputs if isinstance(i.type, HipArrayType)) & set(
-                        id(i) for i in b.inputs if isinstance(i.type, HipArrayType)):
-                    continue
                 if a.outputs[0].type.broadcastable != b.outputs[0].type.broadcastable:
                     continue
                 nd = max(i.type.ndim for i in a.inputs)
                 pa = [all(bb) for bb in zip(*[i.type.broadcastable for i in a.inputs if i.type.ndim == nd])]
                 pb = [all(bb) for bb in zip(*[i.type.broadcastable for i in b.inputs if i.type.ndim == nd])]
                 if pa != pb:
+                    continue
+                # Equal run-time shapes are certain only when the two share an array that spans the whole
+                # reduce domain: a common operand that is broadcast in both (a per-channel weight) says
+                # nothing about the extents of the others.
+                full_a = set(id(i) for i in a.inputs if isinstance(i.type, HipArrayType) and
+                             list(i.type.broadcastable) == pa)
+                if not any(id(i) in full_a for i in b.inputs):
                     continue
                 if any(_depends_on(i, a) for i in b.inputs) or any(_depends_on(i, b) for i in a.inputs):
                     continue
