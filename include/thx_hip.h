@@ -162,6 +162,29 @@ int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, 
  * Replaces the c_code_reduce_* launch routines (theano/gpuarray/elemwise.py:1095-1723). */
 int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_mask,
                     const thx_array* outs, int flags);
+
+/* Size of the library's fixed scratch array, which every GPU the library runs on holds from the
+ * moment the library is loaded until the process ends. */
+#define THX_STATIC_SCRATCH_BYTES 4194304
+
+/* thx_reduce_call for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in
+ * the reference.  Same arguments and results as thx_reduce_call, but the call never
+ * allocates or frees device memory:
+ *  - the partial results of a split reduction (S slices x results x accumulator bytes) go to the
+ *    fixed scratch array instead of an allocated buffer; a reduction that needs more than
+ *    THX_STATIC_SCRATCH_BYTES fails with THX_ERR_UNSUPPORTED and launches nothing;
+ *  - compiling or loading a kernel allocates, so every kernel the call needs must already be
+ *    loaded: run thx_reduce_call once on operands of the same layout beforehand (a warm-up);
+ *    otherwise the call fails with THX_ERR_UNSUPPORTED and launches nothing;
+ *  - thx_init must have been called (it resolves the array's device address); THX_DRY_RUN is
+ *    refused; launches are never bracketed by profiling events.
+ * Every call on a GPU shares that GPU's one array, which keeps the last call's contents: each
+ * call overwrites every partial result before it reads it, so nothing needs clearing, but two
+ * calls that overlap in time on one GPU (from different streams or threads) race.  Calls on the
+ * library's one in-order stream never overlap. */
+int thx_reduce_call_static(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_mask,
+                           const thx_array* outs, int flags);
 int thx_reduce_free(thx_reduce* r);
 
 /* ---- Row chains ------------------------------------------------------------ */

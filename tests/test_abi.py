@@ -24,6 +24,29 @@ def test_library_exports_every_declared_symbol():
     assert not missing, missing
 
 
+def test_fixed_scratch_array_is_visible_to_the_runtime(tmp_path):
+    """hipGetSymbolAddress finds a device variable by name in the library's gfx950 code object, so the
+    fixed scratch array of thx_reduce_call_static must be a global symbol there, of the size the
+    header states (a local one makes thx_init abort on a GPU)."""
+    import subprocess
+    readelf, objcopy = "/opt/rocm/llvm/bin/llvm-readelf", "/opt/rocm/llvm/bin/llvm-objcopy"
+    if not (os.path.exists(readelf) and os.path.exists(objcopy)):
+        pytest.skip("no llvm binutils")
+    fat = str(tmp_path / "fat.bin")
+    subprocess.run([objcopy, "-O", "binary", "--only-section=.hip_fatbin", runtime._LIB_PATH, fat], check=True)
+    data = open(fat, "rb").read()
+    starts = [m.start() for m in re.finditer(b"\x7fELF", data)]
+    header = open(os.path.join(ROOT, "include", "thx_hip.h")).read()
+    size = int(re.search(r"#define\s+THX_STATIC_SCRATCH_BYTES\s+(\d+)", header).group(1))
+    found = []
+    for k, s in enumerate(starts):
+        co = str(tmp_path / ("co%d.elf" % k))
+        open(co, "wb").write(data[s:starts[k + 1] if k + 1 < len(starts) else len(data)])
+        out = subprocess.run([readelf, "-s", co], capture_output=True, text=True).stdout
+        found += [l.split() for l in out.splitlines() if l.strip().endswith("scratch") and "OBJECT" in l]
+    assert found and all(f[2] == str(size) and f[4] == "GLOBAL" for f in found), found
+
+
 def test_error_codes_map_to_exceptions():
     e = ctypes.c_void_p()
     dt = (ctypes.c_int32 * 2)(99, 10)

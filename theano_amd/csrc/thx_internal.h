@@ -34,6 +34,9 @@ struct Runtime {
   hipStream_t stream = nullptr;
   char* scratch = nullptr;  // partial results of split reductions
   size_t scratch_bytes = 0;
+  // Device address of the library's fixed scratch array on `device` (thx_reduce_call_static),
+  // resolved once in thx_init; null until then.
+  char* static_scratch = nullptr;
 };
 Runtime& rt();
 int ensure_init();
@@ -62,9 +65,10 @@ const std::string& device_prelude();
 // profilers show one line per (functor, plan) instead of a shared entry name.
 std::string entry_name(const std::string& functor, const std::string& plan);
 
-// Launch with one by-value parameter block.
+// Launch with one by-value parameter block.  `bare`: never bracket the launch with profiling
+// events (creating an event allocates; callers that must not allocate pass true).
 int launch(const Kernel& k, const std::string& plan, unsigned grid, unsigned block,
-           const void* params, size_t params_bytes);
+           const void* params, size_t params_bytes, bool bare = false);
 
 // ---- array helpers ----------------------------------------------------------
 int dtype_size(int dtype);

@@ -72,14 +72,26 @@ static std::string plan_struct(bool wide, const std::vector<std::pair<std::strin
   return s.str();
 }
 
+static int final_tpo(int64_t n_out) { return n_out >= 1024 ? 1 : (n_out >= 16 ? 64 : 256); }
+
+// The message of a call that may neither compile nor load a kernel and finds the one it needs missing.
+static int not_loaded(const thx_reduce* r, const std::string& plan) {
+  return fail(THX_ERR_UNSUPPORTED,
+              "thx_reduce_call_static: kernel '%s|%s' is not loaded; loading one allocates device memory, so run "
+              "thx_reduce_call once on operands of this layout first", r->name.c_str(), plan.c_str());
+}
+
+// `fixed`: the call comes from thx_reduce_call_static - only kernels that are already loaded, no events.
 static int final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::vector<uint64_t>& ex, char* partial,
-                      int64_t n_out, int S, bool dry) {
-  const int tpo = n_out >= 1024 ? 1 : (n_out >= 16 ? 64 : 256);
+                      int64_t n_out, int S, bool dry, bool fixed = false) {
+  const int tpo = final_tpo(n_out);
   const std::string plan = "rf|t" + std::to_string(tpo);
   Kernel k;
   auto it = r->plans.find(plan);
   if (it != r->plans.end() && (it->second.func || dry)) {
     k = it->second;
+  } else if (fixed) {
+    return not_loaded(r, plan);
   } else {
     const std::string entry = entry_name(r->name, plan);
     std::ostringstream s;
@@ -99,7 +111,29 @@ static int final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::
   pk.put<int32_t>(0);
   pk.align(8);
   const int64_t grid = ceil_div(n_out, 256 / tpo);
-  return launch(k, r->name + "|" + plan, (unsigned)grid, 256, pk.buf.data(), pk.buf.size());
+  return launch(k, r->name + "|" + plan, (unsigned)grid, 256, pk.buf.data(), pk.buf.size(), fixed);
+}
+
+// Where the partial results of a split reduction go: the buffer the library allocates and grows
+// (thx_reduce_call), or the fixed array (thx_reduce_call_static), which cannot grow.  In the fixed
+// case the second pass's kernel is looked up here too, so that a miss is reported before the
+// first pass is launched.
+static int partial_buffer(thx_reduce* r, size_t bytes, int64_t n_out, bool fixed, char** out) {
+  if (!fixed) {
+    int rc = ensure_scratch(bytes);
+    if (rc) return rc;
+    *out = rt().scratch;
+    return THX_OK;
+  }
+  if (bytes > (size_t)THX_STATIC_SCRATCH_BYTES)
+    return fail(THX_ERR_UNSUPPORTED,
+                "thx_reduce_call_static: this reduction needs %zu bytes of partial results, the fixed scratch array "
+                "holds %zu; use thx_reduce_call", bytes, (size_t)THX_STATIC_SCRATCH_BYTES);
+  const std::string fplan = "rf|t" + std::to_string(final_tpo(n_out));
+  auto it = r->plans.find(fplan);
+  if (it == r->plans.end() || !it->second.func) return not_loaded(r, fplan);
+  *out = rt().static_scratch;
+  return THX_OK;
 }
 
 }  // namespace thx
@@ -132,10 +166,20 @@ int thx_reduce_free(thx_reduce* r) {
   return THX_OK;
 }
 
-int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_mask, const thx_array* outs, int flags) {
+}  // extern "C"
+
+// Both entry points.  `fixed` (thx_reduce_call_static): partial results go to the library's fixed
+// scratch array, and nothing on the way may allocate device memory - no hipMalloc / hipFree, no
+// compilation or module load (a kernel that is not loaded yet is an error), no event creation.
+static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_mask, const thx_array* outs, int flags,
+                       bool fixed) {
   if (!r || !ins || !outs) return fail(THX_ERR_ARG, "thx_reduce_call: null argument");
   const bool dry = (flags & THX_DRY_RUN) != 0;
-  if (!dry) {
+  if (fixed) {
+    if (dry) return fail(THX_ERR_ARG, "thx_reduce_call_static: THX_DRY_RUN is for thx_reduce_call");
+    if (!rt().ready || !rt().static_scratch)
+      return fail(THX_ERR_ARG, "thx_reduce_call_static: call thx_init first (it resolves the scratch array's address)");
+  } else if (!dry) {
     int rc = ensure_init();
     if (rc) return rc;
   }
@@ -226,7 +270,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   }
   if (n_red == 0) {  // identity through the epilogue
     set_last_plan(r->name + "|rf|identity");
-    return final_pass(r, outp, ex, nullptr, n_out, 0, dry);
+    return final_pass(r, outp, ex, nullptr, n_out, 0, dry, fixed);
   }
 
   // primary input: the one that spans the most memory
@@ -303,6 +347,7 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
   int64_t grid = 0;
   int S = 1;
   int launch_block = block;
+  char* partial = nullptr;  // Acc[S][n_out] of a split reduction
 
   if (form == ROW) {
     const int64_t RC = NR ? RD.back().extent : 1;
@@ -374,6 +419,8 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     auto it = r->plans.find(plan);
     if (it != r->plans.end() && (it->second.func || dry)) {
       k = it->second;
+    } else if (fixed) {
+      return not_loaded(r, plan);
     } else {
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
@@ -387,14 +434,14 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       r->plans[plan] = k;
     }
     if (!dry && S > 1) {
-      rc = ensure_scratch((size_t)S * n_out * r->acc_bytes);
+      rc = partial_buffer(r, (size_t)S * n_out * r->acc_bytes, n_out, fixed, &partial);
       if (rc) return rc;
     }
     for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
     for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
     for (uint64_t v : ex) pk.put<uint64_t>(v);
-    pk.put<char*>(rt().scratch);
+    pk.put<char*>(partial);
     pk.put<int64_t>(n_out);
     pk.put<int64_t>(nvec);
     pk.put<int64_t>(chunk);
@@ -489,6 +536,8 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     auto it = r->plans.find(plan);
     if (it != r->plans.end() && (it->second.func || dry)) {
       k = it->second;
+    } else if (fixed) {
+      return not_loaded(r, plan);
     } else {
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
@@ -502,14 +551,14 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
       r->plans[plan] = k;
     }
     if (!dry && S > 1) {
-      rc = ensure_scratch((size_t)S * n_out * r->acc_bytes);
+      rc = partial_buffer(r, (size_t)S * n_out * r->acc_bytes, n_out, fixed, &partial);
       if (rc) return rc;
     }
     for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
     for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
     for (uint64_t v : ex) pk.put<uint64_t>(v);
-    pk.put<char*>(rt().scratch);
+    pk.put<char*>(partial);
     pk.put<int64_t>(n_out);
     pk.put<int64_t>(rows);
     pk.put<int64_t>(rps);
@@ -543,6 +592,8 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     auto it = r->plans.find(plan);
     if (it != r->plans.end() && (it->second.func || dry)) {
       k = it->second;
+    } else if (fixed) {
+      return not_loaded(r, plan);
     } else {
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
@@ -576,11 +627,22 @@ int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_m
     return fail(THX_ERR_UNSUPPORTED, "reduce: %lld blocks of %d exceed the work-items of one dispatch", (long long)grid,
                 launch_block);
   if (!dry) {
-    rc = launch(k, r->name + "|" + plan, (unsigned)grid, launch_block, pk.buf.data(), pk.buf.size());
+    rc = launch(k, r->name + "|" + plan, (unsigned)grid, launch_block, pk.buf.data(), pk.buf.size(), fixed);
     if (rc) return rc;
   }
-  if (S > 1) return final_pass(r, outp, ex, rt().scratch, n_out, S, dry);
+  if (S > 1) return final_pass(r, outp, ex, partial, n_out, S, dry, fixed);
   return THX_OK;
+}
+
+extern "C" {
+
+int thx_reduce_call(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_mask, const thx_array* outs, int flags) {
+  return reduce_impl(r, ins, reduce_mask, outs, flags, false);
+}
+
+int thx_reduce_call_static(thx_reduce* r, const thx_array* ins, const uint8_t* reduce_mask, const thx_array* outs,
+                           int flags) {
+  return reduce_impl(r, ins, reduce_mask, outs, flags, true);
 }
 
 }  // extern "C"

@@ -17,6 +17,16 @@
 
 #include "thx_internal.h"
 
+// Fixed scratch memory for thx_reduce_call_static: partial results of a split reduction, laid out
+// [slice][output] like the allocated scratch buffer.  It is part of the library's code object, so
+// every GPU the library runs on holds its own copy from load time until the process ends, and no
+// call ever has to allocate it.  In host code the name `scratch` is only a handle for
+// hipGetSymbolAddress: the device address is resolved once per device in thx_init and that
+// address is what kernels and copies receive.  (No `used` attribute here: it makes the compiler emit
+// the variable before it has seen the host code that refers to it, the device symbol then stays
+// local, and the runtime, which finds the array by name, aborts in hipGetSymbolAddress.)
+static __device__ __align__(256) unsigned char scratch[THX_STATIC_SCRATCH_BYTES];
+
 namespace thx {
 
 // ---------------------------------------------------------------------------
@@ -52,6 +62,9 @@ static std::unordered_map<std::string, Kernel> g_kernels;  // by hash of source
 static std::unordered_map<size_t, std::vector<void*>> g_free;
 static std::unordered_map<void*, size_t> g_live;
 
+enum { kMaxDevices = 64 };
+static char* g_static_scratch[kMaxDevices] = {nullptr};  // device address of `scratch`, per device
+
 // profiling
 struct ProfRec {
   std::string plan;
@@ -73,8 +86,17 @@ static int init_locked(int device) {
   hipError_t e = hipGetDeviceCount(&count);
   if (e != hipSuccess || count == 0)
     return fail(THX_ERR_HIP, "thx_init: no HIP device is visible (%s)", hipGetErrorString(e));
-  if (device >= count) return fail(THX_ERR_ARG, "thx_init: device %d of %d", device, count);
+  if (device >= count || device >= kMaxDevices) return fail(THX_ERR_ARG, "thx_init: device %d of %d", device, count);
   THX_HIP_CHECK(hipSetDevice(device));
+  if (!g_static_scratch[device]) {  // with `device` current: each GPU has the array at its own address
+    void* p = nullptr;
+    hipError_t se = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (se != hipSuccess || !p)
+      return fail(THX_ERR_HIP, "thx_init: hipGetSymbolAddress(scratch) failed on device %d: %s", device,
+                  hipGetErrorString(se));
+    g_static_scratch[device] = (char*)p;
+  }
+  r.static_scratch = g_static_scratch[device];
   hipDeviceProp_t prop;
   THX_HIP_CHECK(hipGetDeviceProperties(&prop, device));
   r.device = device;
@@ -378,7 +400,7 @@ std::string entry_name(const std::string& functor, const std::string& plan) {
 }
 
 int launch(const Kernel& k, const std::string& plan_in, unsigned grid, unsigned block, const void* params,
-           size_t params_bytes) {
+           size_t params_bytes, bool bare) {
   const std::string& plan = plan_in;
   if (!k.func) return fail(THX_ERR_HIP, "launch of '%s' without a loaded kernel", plan.c_str());
   if (params_bytes > 4096)
@@ -387,7 +409,7 @@ int launch(const Kernel& k, const std::string& plan_in, unsigned grid, unsigned 
   void* extra[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(params), HIP_LAUNCH_PARAM_BUFFER_SIZE,
                    &params_bytes, HIP_LAUNCH_PARAM_END};
   Runtime& r = rt();
-  if (!g_profiling) {
+  if (!g_profiling || bare) {
     THX_HIP_CHECK(hipModuleLaunchKernel(k.func, grid, 1, 1, block, 1, 1, 0, r.stream, nullptr, extra));
     return THX_OK;
   }
