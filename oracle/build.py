@@ -9,7 +9,7 @@ import os
 import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["careduce.c", "cpu_backend.c"]
+SOURCES = ["careduce.c", "cpu_backend.c", "libm_ref.c"]
 LIB = os.path.join(HERE, "_build", "liboracle.so")
 
 

@@ -141,15 +141,23 @@ def _check_broadcast(node, values):
                                  % (owner[d], d, shape[d], k, d, val.shape[d]))
 
 
-def eval_scalar_op(op, in_values, out_dtypes):
+def _wide(dtype):
+    """float16 / float32 -> float64; every other dtype stays."""
+    return "float64" if str(dtype) in ("float16", "float32") else str(dtype)
+
+
+def eval_scalar_op(op, in_values, out_dtypes, wide=False):
     """Evaluate a theano_amd ScalarOp (or Composite) over whole arrays."""
     name = type(op).__name__
+    if wide:
+        out_dtypes = [_wide(d) for d in out_dtypes]
+        in_values = [np.asarray(v).astype(_wide(np.asarray(v).dtype), copy=False) for v in in_values]
     if name == "Composite":
         from theano_amd import gof
         env = dict(zip(op.inputs, in_values))
         for node in gof.io_toposort(op.inputs, op.outputs):
             args = [env[i] if i in env else np.asarray(i.data) for i in node.inputs]
-            outs = eval_scalar_op(node.op, args, [o.type.dtype for o in node.outputs])
+            outs = eval_scalar_op(node.op, args, [o.type.dtype for o in node.outputs], wide)
             for o, v in zip(node.outputs, outs):
                 env[o] = v
         return [env[o] if o in env else np.asarray(o.data) for o in op.outputs]
@@ -245,9 +253,15 @@ _ROW_OPS = {"Softmax": _softmax, "SoftmaxWithBias": _softmax_with_bias, "Softmax
             "LogSoftmax": _logsoftmax}
 
 
-def evaluate(inputs, outputs, values):
+def evaluate(inputs, outputs, values, wide=False):
     """Values of ``outputs`` (theano_amd variables) given ``values`` for
-    ``inputs``; every Apply node is computed separately, as an unfused graph."""
+    ``inputs``; every Apply node is computed separately, as an unfused graph.
+
+    ``wide=True`` gives the graph's mathematical value instead of the reference's arithmetic: every
+    float16 / float32 value, intermediate, accumulator and result is float64 (casts between float
+    types then change nothing), integer and boolean nodes are evaluated as they are.  Tests use it as
+    the truth that both this oracle and the device are measured against where float32 rounding noise
+    of the reference's own evaluation order exceeds the parity tolerance."""
     from theano_amd import gof
     from theano_amd.tensor.elemwise import CAReduce, CAReduceDtype, DimShuffle, Elemwise
     from theano_amd.tensor.basic import MaxAndArgmax, ShapeFloat
@@ -255,14 +269,19 @@ def evaluate(inputs, outputs, values):
     env = {}
     for var, val in zip(inputs, values):
         env[var] = var.type.filter(np.asarray(val), strict=False, allow_downcast=False)
+        if wide:
+            env[var] = env[var].astype(_wide(env[var].dtype), copy=False)
+    odt = (lambda o: _wide(o.type.dtype)) if wide else (lambda o: o.type.dtype)
     for node in gof.io_toposort(inputs, outputs):
         args = [env[i] if i in env else np.asarray(i.data) for i in node.inputs]
+        if wide:
+            args = [a.astype(_wide(a.dtype), copy=False) for a in args]
         op = node.op
         if isinstance(op, Elemwise):
             _check_broadcast(node, args)
-            res = eval_scalar_op(op.scalar_op, args, [o.type.dtype for o in node.outputs])
+            res = eval_scalar_op(op.scalar_op, args, [o.type.dtype for o in node.outputs], wide)
             shape = np.broadcast_shapes(*[a.shape for a in args])
-            res = [np.broadcast_to(r, shape).astype(o.type.dtype, copy=False) if o.type.dtype != "bool"
+            res = [np.broadcast_to(r, shape).astype(odt(o), copy=False) if o.type.dtype != "bool"
                    else np.broadcast_to(r, shape) != 0 for r, o in zip(res, node.outputs)]
         elif isinstance(op, DimShuffle):
             res = [dimshuffle(args[0], op.new_order)]
@@ -278,9 +297,11 @@ def evaluate(inputs, outputs, values):
                 acc_dt = "bool" if out_dt == "bool" else idt
             if acc_dt == "float32" and idt == "float16":
                 x = x.astype("float32")
+            if wide:
+                acc_dt, out_dt = _wide(acc_dt), _wide(out_dt)
             res = [careduce(x, sname, op.axis, acc_dt, out_dt)]
         elif isinstance(op, ShapeFloat):
-            res = [np.asarray(args[0].shape[op.i], dtype=op.dtype)]
+            res = [np.asarray(args[0].shape[op.i], dtype=_wide(op.dtype) if wide else op.dtype)]
         elif isinstance(op, MaxAndArgmax):
             res = list(max_and_argmax(args[0], op.axis))
         elif isinstance(op, V.Subtensor):          # NumPy basic indexing is the definition (subtensor.py:318-780)
@@ -308,10 +329,10 @@ def evaluate(inputs, outputs, values):
             idx[op.axis] = slice(at, at + args[1 + op.k].shape[op.axis])
             res = [args[0][tuple(idx)]]
         elif type(op).__name__ in _BN_OPS:
-            res = [np.asarray(r).astype(o.type.dtype, copy=False)
+            res = [np.asarray(r).astype(odt(o), copy=False)
                    for r, o in zip(_BN_OPS[type(op).__name__](op, *args), node.outputs)]
         elif type(op).__name__ in _ROW_OPS:
-            res = [_ROW_OPS[type(op).__name__](*args).astype(node.outputs[0].type.dtype, copy=False)]
+            res = [_ROW_OPS[type(op).__name__](*args).astype(odt(node.outputs[0]), copy=False)]
         else:
             raise NotImplementedError("oracle cannot evaluate %s" % op)
         for o, v in zip(node.outputs, res):

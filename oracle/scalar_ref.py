@@ -355,7 +355,18 @@ cosh, sinh, tanh = _libm(np.cosh), _libm(np.sinh), _libm(np.tanh)
 arccosh, arcsinh, arctanh = _libm(np.arccosh), _libm(np.arcsinh), _libm(np.arctanh)
 trunc = _libm(np.trunc)
 round_half_to_even = _libm(np.rint)
-round_half_away_from_zero = _libm(lambda a: np.where(a > 0, np.floor(a + 0.5), np.ceil(a - 0.5)))
+
+
+def _c_round(a):
+    """C ``round()`` (the reference's C text, ``theano/scalar/basic.py:2686``): the nearest integer, halves
+    away from zero.  ``floor(a + 0.5)`` - what the reference's Python ``impl`` does (:2640-2643) - is not the
+    same function: ``a + 0.5`` is itself rounded, so 0.49999997f becomes 1 and odd integers from 2**23
+    up move by one.  Exact here: ``a - trunc(a)`` has no rounding error."""
+    t = np.trunc(a)
+    return t + np.copysign((np.abs(a - t) >= 0.5).astype(a.dtype), a)
+
+
+round_half_away_from_zero = _libm(_c_round)
 
 
 def _special(name):

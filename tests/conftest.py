@@ -38,6 +38,33 @@ def assert_parity(got, ref, what="", tol=None):
             what, (~ok).sum(), ok.size, t, tuple(bad), got[tuple(bad)], ref[tuple(bad)]))
 
 
+def assert_within_reference_error(got, ref, truth, what="", tol=None):
+    """The parity bar for results where the reference's own float32 evaluation order is farther
+    from the exact value than the tolerance allows (a difference of nearly equal numbers, a float32
+    accumulator over many terms): `truth` is the graph's value in float64 (the oracle's wide mode)
+    and errors are counted in units of the bar, |v - truth| / (atol + rtol |truth|).  The device result
+    must be within the bar of the truth, or at least no farther from it than the reference's
+    arithmetic (`ref`, the oracle) is at its worst element.  Integer results must be equal."""
+    got, ref, truth = np.asarray(got), np.asarray(ref), np.asarray(truth)
+    assert got.shape == ref.shape == truth.shape, "%s: shapes %s %s %s" % (what, got.shape, ref.shape, truth.shape)
+    assert got.dtype == ref.dtype, "%s: dtype %s != %s" % (what, got.dtype, ref.dtype)
+    if ref.dtype.kind in "biu":
+        assert np.array_equal(got, ref), "%s: integer results differ" % what
+        return
+    t = tol or TOL[str(ref.dtype)]
+    w = truth.astype("float64")
+    fin = np.isfinite(w)
+    assert np.array_equal(got.astype("float64")[~fin], w[~fin], equal_nan=True), "%s: non-finite values differ" % what
+    unit = t["atol"] + t["rtol"] * np.abs(w[fin])
+    e_got = np.abs(got.astype("float64")[fin] - w[fin]) / unit
+    e_ref = np.abs(ref.astype("float64")[fin] - w[fin]) / unit
+    worst_ref = float(e_ref.max()) if e_ref.size else 0.0
+    worst_got = float(e_got.max()) if e_got.size else 0.0
+    assert worst_got <= max(1.0, worst_ref), (
+        "%s: device result is %.2f bars (%s) from the float64 value, the reference's own arithmetic %.2f"
+        % (what, worst_got, t, worst_ref))
+
+
 @pytest.fixture
 def dry_run():
     """Run the HIP path in dry-run mode: kernels are planned and compiled for

@@ -104,6 +104,25 @@ def test_strided_views_zero_extents_and_errors():
     assert np.array_equal(mv, [7, 15, 23]) and np.array_equal(iv, [7, 7, 7])
 
 
+def test_argmax_through_the_generic_reduction_form():
+    """Three reduced dimensions that do not collapse (axes 0, 2, 4 of a 6-d array) take the generic
+    kernel, where the position operand is computed from a full index decomposition; ties and NaNs included."""
+    rng = np.random.default_rng(36)
+    t6 = T.TensorType("float32", (False,) * 6)("t6")
+    val = rng.integers(-3, 4, (3, 4, 5, 6, 7, 2)).astype("float32")      # many ties: the first occurrence must win
+    val[1, 2, 3, 4, 5, 1] = np.nan
+    f = th.function([t6], T.max_and_argmax(t6, axis=(0, 2, 4)))
+    mv, iv = f(val)
+    assert "|rg|" in hip.last_plan(), hip.last_plan()
+    ref_m, ref_i = G.max_and_argmax(val, (0, 2, 4))
+    assert np.array_equal(mv, ref_m, equal_nan=True) and np.array_equal(iv, ref_i) and iv.dtype == np.int64
+    i6 = T.TensorType("int16", (False,) * 6)("i6")
+    vi = rng.integers(-300, 300, (3, 4, 5, 6, 7, 2)).astype("int16")
+    mv, iv = th.function([i6], T.max_and_argmax(i6, axis=(0, 2, 4)))(vi)
+    ref_m, ref_i = G.max_and_argmax(vi, (0, 2, 4))
+    assert np.array_equal(mv, ref_m) and np.array_equal(iv, ref_i)
+
+
 def test_gradient_of_max_through_max_and_argmax():
     rng = np.random.default_rng(35)
     x = T.fmatrix("x")

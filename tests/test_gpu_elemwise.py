@@ -109,6 +109,49 @@ def test_sigmoid_thresholds_and_nan_handling():
         assert_parity(g, r, "special values")
 
 
+def test_round_half_away_from_zero_is_c_round_on_the_device():
+    """theano/scalar/basic.py:2686 emits C round(): halves away from zero, and nothing like
+    floor(x + 0.5) at 0.49999997 or at odd integers from 2**23 up.  Bit-exact against the oracle
+    (itself pinned against the host's libm) over the finite range, float32 and float64."""
+    from test_oracle_scalar import ROUND_PINS, finite_float32_sweep
+    x, d = T.fvector("x"), T.dvector("d")
+    f = th.function([x, d], [T.round_half_away_from_zero(x), T.round_half_away_from_zero(d),
+                             T.round(x, mode="half_away_from_zero")])
+    pins = np.array([p for p, _ in ROUND_PINS], "float64")
+    got32, got64, got_front = f(pins.astype("float32"), pins)
+    for (p, want), g in zip(ROUND_PINS, got32):
+        if want is not None:
+            assert float(g) == want and np.signbit(g) == np.signbit(np.float32(want)), (p, g)
+    assert got64[-1] == 4503599627370497.0 and np.array_equal(got_front, got32)
+    xv = np.concatenate([finite_float32_sweep(), np.array([np.inf, -np.inf, np.nan], "float32")])
+    dv = xv.astype("float64") * 1.0000001
+    got, ref = run_both([x, d], [T.round_half_away_from_zero(x), T.round_half_away_from_zero(d)], [xv, dv])
+    for g, r in zip(got, ref):
+        assert g.dtype == r.dtype and np.array_equal(g, r, equal_nan=True)
+        assert np.array_equal(np.signbit(g), np.signbit(r))
+
+
+def test_exp_sigmoid_softplus_over_the_whole_finite_float32_range():
+    """The default float32 exp is one hardware exp2 of x * log2(e) (relative error up to |x| * 4e-8) and
+    the sigmoid core one exp2 and one rcp: checked against the oracle at the float32 bar (rtol 1e-5,
+    atol 1e-6) over every exponent of the finite range and around each saturation threshold."""
+    from test_oracle_scalar import finite_float32_sweep
+    x = T.fvector("x")
+    xv = finite_float32_sweep()
+    outs = [T.exp(x), T.sigmoid(x), T.softplus(x), T.expm1(x), T.tanh(x), T.exp(-x) * 2]
+    with np.errstate(all="ignore"):
+        got, ref = run_both([x], outs, [xv])
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "output %d" % k)            # float32: rtol 1e-5, atol 1e-6; inf / nan must coincide
+    # the same through a float64 graph at the float64 bar
+    d = T.dvector("d")
+    dv = xv.astype("float64") * 7.0
+    with np.errstate(all="ignore"):
+        got, ref = run_both([d], [T.exp(d), T.sigmoid(d), T.softplus(d)], [dv])
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "float64 output %d" % k, tol=dict(rtol=1e-12, atol=1e-300))
+
+
 def test_weird_strides_five_dims():
     # theano/tensor/tests/test_elemwise.py:305-318
     rng = np.random.default_rng(11)

@@ -6,7 +6,7 @@ import pytest
 import theano_amd as th
 from theano_amd import hip, tensor as T
 from oracle import graph_ref as G
-from conftest import assert_parity
+from conftest import assert_parity, assert_within_reference_error
 from test_oracle_graph import CAREDUCE_CASES
 
 pytestmark = pytest.mark.gpu
@@ -87,6 +87,93 @@ def test_dtype_coverage(dtype):
             check(x, T.sum(x, axis=axis, dtype="float64"), v, "sum to f64")
 
 
+BIT_REDUCERS = {"and_": np.bitwise_and, "or_": np.bitwise_or, "xor": np.bitwise_xor}
+
+
+def _np_bit_reduce(ufunc, v, axis):
+    """NumPy's answer the way theano/tensor/tests/test_elemwise.py:334-347, 443-456 builds it: one axis at
+    a time, highest first, with the op's identity (-1 for and, 0 for or / xor) where an axis is empty."""
+    axes = range(v.ndim) if axis is None else [a + v.ndim if a < 0 else a for a in axis]
+    for a in sorted(axes, reverse=True):
+        v = ufunc.reduce(v, axis=a)
+    return np.asarray(v)
+
+
+@pytest.mark.parametrize("dtype", ["int8", "uint8", "int32"])
+@pytest.mark.parametrize("opname", sorted(BIT_REDUCERS))
+def test_bitwise_careduce_reference_case_table(opname, dtype):
+    """CAReduce{and_, or_, xor} on integers (theano/tensor/tests/test_elemwise.py:352-366, 443-460, run there for
+    int8 / uint8): the reference's shape x axis table with its 0 / 1 inputs and with random bit patterns, then
+    shapes long enough for every kernel form and for split reductions.  Bit-exact against NumPy and the oracle."""
+    from theano_amd import scalar as scal
+    from theano_amd.tensor.elemwise import CAReduce
+    rng = np.random.default_rng(31)
+    info = np.iinfo(dtype)
+    big = [((4100, 3), (0,)), ((3, 4100), (1,)), ((300000,), None), ((1025, 1025), (0,)), ((1025, 1025), (1,)),
+           ((1025, 1025), None), ((33, 65, 17), (0, 2)), ((2100, 2100), None)]
+    for shape, axis in list(CAREDUCE_CASES) + big:
+        x = T.TensorType(dtype, [s == 1 for s in shape])("x")
+        out = CAReduce(getattr(scal, opname), axis=axis)(x)
+        assert out.type.dtype == dtype
+        f = th.function([x], out)
+        samples = [(rng.random(shape) < 0.5).astype(dtype),
+                   rng.integers(info.min, int(info.max) + 1, shape, dtype="int64").astype(dtype)]
+        if opname == "and_":      # mostly-ones patterns, so that an and over many elements is not simply 0
+            samples.append((rng.integers(info.min, int(info.max) + 1, shape, dtype="int64") |
+                            rng.integers(info.min, int(info.max) + 1, shape, dtype="int64") | 0x55).astype(dtype))
+        for v in samples:
+            got = f(v)
+            want = _np_bit_reduce(BIT_REDUCERS[opname], v, axis)
+            ref = G.evaluate([x], [out], [v])[0]
+            what = "%s %s %s %s [%s]" % (opname, dtype, shape, axis, hip.last_plan())
+            assert got.dtype == want.dtype == ref.dtype and got.shape == want.shape, what
+            assert np.array_equal(got, want) and np.array_equal(got, ref), what
+
+
+def test_1024_thread_row_plan():
+    """Few results with long reduce domains (128 to 1024 results of at least 8192 vectors each) take the
+    1024-threads-per-result form of the row kernel instead of a split: the plan behind batch-norm's
+    per-channel statistics.  Single reductions, the two-reduced-dimension variant, a fused prologue with two
+    inputs, several accumulators with an epilogue, float16 storage - all against the oracle."""
+    rng = np.random.default_rng(41)
+    x = T.fmatrix("x")
+    for shape in ((128, 32768), (200, 40004)):
+        v = rng.standard_normal(shape).astype("float32")
+        for name in ("sum", "max", "min"):
+            check(x, REDUCERS[name](x, 1), v, "%s %s" % (name, shape))
+            assert "|t1024|" in hip.last_plan(), hip.last_plan()
+        vp = rng.uniform(0.999, 1.001, shape).astype("float32")
+        check(x, x.prod(axis=1), vp, "prod %s" % (shape,))
+        assert "|t1024|" in hip.last_plan()
+    t, u = T.ftensor3("t"), T.ftensor3("u")
+    tv, uv = (rng.standard_normal((6, 160, 7000)).astype("float32") for _ in range(2))
+    check(t, t.sum(axis=(0, 2)), tv, "outer x kept x inner")
+    assert "|t1024|a1|" in hip.last_plan(), hip.last_plan()
+    outs = [T.sum(t * u, axis=(0, 2)), T.sum(T.sqr(t - u), axis=(0, 2)) / np.float32(42000.0), T.max(t + u, axis=(0, 2))]
+    got = th.function([t, u], outs)(tv, uv)
+    plan = hip.last_plan()
+    ref = G.evaluate([t, u], outs, [tv, uv])
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "two-input prologue, output %d [%s]" % (k, plan))
+    f = th.function([t, u], outs)
+    assert len([n for n in f.toposort() if type(n.op).__name__ == "HipCAReduce"]) == 1 and "|t1024|" in plan, plan
+    # float16 storage, float32 statistics with float32 accumulators, per-channel epilogue (mean and mean of squares)
+    h = T.TensorType("float16", (False,) * 4)("h")
+    hv = rng.normal(0.5, 2.0, (16, 128, 70, 64)).astype("float16")
+    hf = T.cast(h, "float32")
+    m = np.float32(16 * 70 * 64)
+    outs = [T.sum(hf, axis=(0, 2, 3), acc_dtype="float32") / m, T.sum(T.sqr(hf), axis=(0, 2, 3), acc_dtype="float32") / m]
+    got = th.function([h], outs)(hv)
+    plan = hip.last_plan()
+    assert "|t1024|" in plan, plan
+    truth = [hv.astype("float64").mean(axis=(0, 2, 3)), (hv.astype("float64") ** 2).mean(axis=(0, 2, 3))]
+    ref = G.evaluate([h], outs, [hv])
+    for g, r, w in zip(got, ref, truth):
+        # float32 accumulators over 71680 terms: the sequential oracle itself is ~1e-4 from the float64 value, the
+        # tree-ordered kernel closer
+        assert_within_reference_error(g, r, w, "float16 statistics [%s]" % plan)
+
+
 def test_precision_of_default_accumulator():
     # theano/tensor/tests/test_elemwise.py:953-966
     x = T.fvector("x")
@@ -133,12 +220,30 @@ def test_fused_prologue_and_multi_output():
     f = th.function([x, y, r], outs)
     got = f(xv, yv, rv)
     ref = G.evaluate([x, y, r], outs, [xv, yv, rv])
-    for k, (g, rr) in enumerate(zip(got, ref)):
-        assert_parity(g, rr, "fused reduce %d" % k, tol=dict(rtol=2e-5, atol=2e-6))
+    truth = G.evaluate([x, y, r], outs, [xv, yv, rv], wide=True)
+    for k, (g, rr, w) in enumerate(zip(got, ref, truth)):
+        if k < 4:
+            assert_parity(g, rr, "fused reduce %d" % k)
+        else:   # var / std: x - mean(x) is a float32 difference that the squares inherit, in the reference as here
+            assert_within_reference_error(g, rr, w, "fused reduce %d" % k)
     a = T.imatrix("a")
     av = rng.integers(-5, 6, (200, 333)).astype("int32")
     g2 = th.function([a], [T.any(a > 4), T.all(a > -6), T.any(a > 5), T.all(a > 0)])(av)
     assert [bool(v) for v in g2] == [True, True, False, False]
+
+
+def test_reductions_over_different_shapes_that_share_a_broadcast_weight():
+    """Two losses over different batch sizes that share a (1, C) parameter: separate kernels, both right."""
+    rng = np.random.default_rng(27)
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    w = T.frow("w")
+    outs = [T.sum(T.exp(x) * w), T.sum(T.tanh(y) * w), T.sum(x * w, axis=0), T.sum(y * w, axis=0)]
+    vals = [rng.standard_normal((4, 8)).astype("float32"), rng.standard_normal((6, 8)).astype("float32"),
+            rng.standard_normal((1, 8)).astype("float32")]
+    got = th.function([x, y, w], outs)(*vals)
+    ref = G.evaluate([x, y, w], outs, vals)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "shared weight, output %d" % k)
 
 
 def test_epilogue_chain_with_per_result_device_operands():
@@ -165,8 +270,10 @@ def test_epilogue_chain_with_per_result_device_operands():
     assert any(type(i.type).__name__ == "HipArrayType" for i in kernels[1].inputs[len(kernels[1].inputs) - kernels[1].op.n_extra:])
     got = f(*vals)
     ref = G.evaluate([x, g, gamma, beta], outs, vals)
-    for k, (a, b) in enumerate(zip(got, ref)):
-        assert_parity(a, b, "epilogue output %d" % k, tol=dict(rtol=3e-5, atol=3e-6))
+    truth = G.evaluate([x, g, gamma, beta], outs, vals, wide=True)
+    for k, (a, b, w) in enumerate(zip(got, ref, truth)):
+        # sums of g * (x - mean) are sums of signed terms near zero, and (s2 - s1) a difference of two of them
+        assert_within_reference_error(a, b, w, "epilogue output %d" % k)
     # a per-result operand of the wrong extent is refused like any broadcast mismatch
     bad = list(vals)
     bad[2] = np.ones((1, 36, 1, 1), "float32")

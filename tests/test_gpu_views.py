@@ -8,7 +8,7 @@ import theano_amd as th
 from theano_amd import tensor as T
 from theano_amd.hip import HipCAReduce, HipElemwise
 from oracle import graph_ref as G
-from conftest import assert_parity
+from conftest import assert_parity, assert_within_reference_error
 
 pytestmark = pytest.mark.gpu
 
@@ -88,8 +88,11 @@ def test_gradients_through_views():
             T.sum(T.stack([y, y * 2], axis=1)[:, 1] * y))
     grads = th.grad(cost, [x, y, r])
     f, got, ref = both([x, y, r], [cost] + grads, [xv, yv, rv])
-    for k, (g, rr) in enumerate(zip(got, ref)):
-        assert_parity(g, rr, "gradient %d" % k, tol=dict(rtol=2e-5, atol=2e-5))
+    truth = G.evaluate([x, y, r], [cost] + grads, [xv, yv, rv], wide=True)
+    for k, (g, rr, w) in enumerate(zip(got, ref, truth)):
+        # the cost adds seven float32 sums of either sign (the oracle's own total is a few bars from the
+        # float64 value): held to that value, no farther from it than the oracle is
+        assert_within_reference_error(g, rr, w, "gradient %d" % k)
 
 
 def test_minibatch_slices_of_a_large_matrix():

@@ -185,3 +185,86 @@ def test_sigmoid_binary_crossentropy_closed_form():
     want = np.logaddexp(0, x32.astype("float64")) - x32 * t
     # x * ((x > 0) - t) rounds (x > 0) - t to float32 first: an absolute error of |x| * 6e-8
     assert np.all(np.abs(got32 - want) <= 2e-6 * np.abs(want) + 2e-7 * np.abs(x32) + 1e-7)
+
+
+# ---- the host's libm, called through the C text the reference emits (oracle/libm_ref.c) ----------
+LIBM_OPS = {"round": 0, "exp": 1, "sigmoid": 2, "softplus": 3, "log1p": 4, "expm1": 5, "tanh": 6, "sqrt": 7, "log": 8}
+
+
+def libm(op, x):
+    """The reference's C expression for `op`, evaluated by the host's libm."""
+    import ctypes
+    from oracle import graph_ref
+    L = graph_ref.lib()
+    x = np.ascontiguousarray(x)
+    z = np.empty_like(x)
+    fn = L.libm_unary_f32 if x.dtype == np.float32 else L.libm_unary_f64
+    rc = fn(ctypes.c_int(LIBM_OPS[op]), x.ctypes.data_as(ctypes.c_void_p), z.ctypes.data_as(ctypes.c_void_p),
+            ctypes.c_int64(x.size))
+    assert rc == 0
+    return z
+
+
+def finite_float32_sweep(n=200001):
+    """Every exponent of the finite float32 range, both signs, plus the values around the saturation
+    thresholds of sigmoid / softplus / exp."""
+    rng = np.random.default_rng(99)
+    bits = rng.integers(0, 0x7f800000, n, dtype=np.uint32) | (rng.integers(0, 2, n, dtype=np.uint32) << 31)
+    wide = bits.view("float32")
+    mid = rng.uniform(-110, 110, n).astype("float32")
+    edges = np.array([-103.5, -103, -102.5, -88.5, -88, -87.5, 13.5, 14, 14.5, 15, 15.5, 88, 88.7, 88.8, 0.0, -0.0],
+                     "float32")
+    return np.concatenate([wide, mid, edges])
+
+
+ROUND_PINS = [(0.49999997, 0.0), (-0.49999997, -0.0), (0.5, 1.0), (-0.5, -1.0), (2.5, 3.0), (-2.5, -3.0),
+              (8388609.0, 8388609.0), (-8388609.0, -8388609.0), (1.5, 2.0), (0.0, 0.0), (4503599627370497.0, None)]
+
+
+def test_round_half_away_from_zero_is_c_round():
+    """C round() (theano/scalar/basic.py:2686), not floor(x + 0.5): known answers where the two differ,
+    then the host libm's roundf / round over the finite range and every half below 2**24."""
+    for x, want in ROUND_PINS:
+        if want is None:
+            continue
+        got = S.round_half_away_from_zero("float32", np.asarray(x, "float32"))
+        assert float(got) == want and np.signbit(got) == np.signbit(np.float32(want)), (x, got)
+    # float64: 2**52 + 1 is odd and exact; x + 0.5 would round to even
+    assert float(S.round_half_away_from_zero("float64", np.asarray(4503599627370497.0))) == 4503599627370497.0
+    assert float(S.round_half_away_from_zero("float64", np.asarray(0.49999999999999994))) == 0.0
+    halves = (np.arange(-(1 << 22), 1 << 22, 64513, dtype="float64") + 0.5).astype("float32")
+    for x in (finite_float32_sweep(), halves, np.array([np.inf, -np.inf], "float32")):
+        got, want = S.round_half_away_from_zero("float32", x), libm("round", x)
+        assert np.array_equal(got, want) and np.array_equal(np.signbit(got), np.signbit(want))
+        x64 = x.astype("float64") * 1.0000001
+        assert np.array_equal(S.round_half_away_from_zero("float64", x64), libm("round", x64))
+    assert np.isnan(S.round_half_away_from_zero("float32", np.asarray(np.nan, "float32")))
+
+
+@pytest.mark.parametrize("op", ["exp", "sigmoid", "softplus", "log1p", "expm1", "tanh", "sqrt", "log"])
+def test_numpy_restatements_agree_with_the_host_libm(op):
+    """The oracle evaluates unary math with NumPy; the reference's C backend calls the host's libm.
+    Over the whole finite float32 range the two agree to a few units in the last place - two orders of
+    magnitude inside the float32 parity bar - with identical saturation (0, 1, x, inf) and NaNs."""
+    x = finite_float32_sweep()
+    if op in ("log", "sqrt"):
+        x = np.abs(x)
+    if op == "log1p":
+        x = np.where(x < -1, -x, x)
+    fn = {"sigmoid": S.scalar_sigmoid, "softplus": S.scalar_softplus}.get(op) or getattr(S, op)
+    with np.errstate(all="ignore"):
+        got, want = fn("float32", x), libm(op, x)
+    assert got.dtype == want.dtype == np.float32
+    fin = np.isfinite(want) & (np.abs(want) >= np.float32(1.2e-38))      # normal results: relative agreement
+    np.testing.assert_allclose(got[fin], want[fin], rtol=5e-7, atol=0)
+    assert np.array_equal(got[~np.isfinite(want)], want[~np.isfinite(want)], equal_nan=True)
+    small = np.isfinite(want) & ~fin                                      # denormal results: absolute
+    np.testing.assert_allclose(got[small], want[small], rtol=0, atol=1e-44)
+    x64 = x.astype("float64") * 3.0
+    if op == "log1p":
+        x64 = np.where(x64 < -1, -x64, x64)
+    with np.errstate(all="ignore"):
+        got64, want64 = fn("float64", x64), libm(op, x64)
+    fin = np.isfinite(want64) & (np.abs(want64) >= 2.3e-308)
+    np.testing.assert_allclose(got64[fin], want64[fin], rtol=1e-15, atol=0)
+    assert np.array_equal(got64[~np.isfinite(want64)], want64[~np.isfinite(want64)], equal_nan=True)

@@ -69,7 +69,7 @@ struct RedAcc {
       return;
     }
     if (P::mode(I) == M_IOTA) {  // the "strides" of this operand are index multipliers
-      const IT st = vstride[I];
+      const IT st = N > 1 ? vstride[I] : (IT)0;  // the generic form loads single elements and has no vector stride
 #pragma unroll
       for (int k = 0; k < N; ++k) r.v[k] = (T)(off[I] + k * st);
       return;
