@@ -246,6 +246,40 @@ def test_reductions_over_different_shapes_that_share_a_broadcast_weight():
         assert_parity(g, r, "shared weight, output %d" % k)
 
 
+def test_sums_over_results_of_a_reduction_over_the_same_elements_share_its_pass():
+    """sum(g * (x - mean(x))) and its relatives: the mean leaves the prologue (sum(g * x) - mean * sum(g)), the
+    reductions merge into the pass that computes the mean, their epilogues chained.  float32 and float64 data,
+    row, column and per-channel layouts; values held to the float64 value like every difference of sums."""
+    from theano_amd.hip import HipCAReduce
+    rng = np.random.default_rng(28)
+    for dtype, shape, axes in (("float32", (6, 37, 5, 9), (0, 2, 3)), ("float32", (300, 515), (1,)),
+                               ("float32", (301, 64), (0,)), ("float64", (40, 33, 7), (0, 2))):
+        nd = len(shape)
+        tt = T.TensorType(dtype, (False,) * nd)
+        x, g = tt("x"), tt("g")
+        mean = T.mean(x, axis=axes, keepdims=True)
+        istd = 1 / T.sqrt(T.mean(T.sqr(x - mean), axis=axes, keepdims=True) + np.asarray(1e-3, dtype))
+        outs = [T.sum(g * (x - mean), axis=axes), T.sum((x - mean) * istd * g, axis=axes, keepdims=True) * istd,
+                T.sum(g - mean, axis=axes), T.sum(x * g, axis=axes) / T.sum(x, axis=axes)]
+        vals = [rng.normal(0.7, 1.5, shape).astype(dtype), rng.standard_normal(shape).astype(dtype)]
+        f = th.function([x, g], outs)
+        reds = [n for n in f.toposort() if isinstance(n.op, HipCAReduce)]
+        if dtype == "float32" and axes != (1,):      # (last-axis islands are row chains; float64 variances keep two passes)
+            assert len(reds) == 1 and len(reds[0].op.scalar_ops) == 5, [str(n.op)[:60] for n in reds]
+        got = f(*vals)
+        ref = G.evaluate([x, g], outs, vals)
+        truth = G.evaluate([x, g], outs, vals, wide=True) if dtype == "float32" else ref
+        for k, (a, b, w) in enumerate(zip(got, ref, truth)):
+            assert_within_reference_error(a, b, w, "%s %s output %d" % (dtype, shape, k),
+                                          tol=None if dtype == "float32" else dict(rtol=1e-11, atol=1e-11))
+        with th.config.change_flags(merge_dependent_reductions=False):
+            plain = th.function([x, g], outs)
+        if axes != (1,):
+            assert len([n for n in plain.toposort() if isinstance(n.op, HipCAReduce)]) > 1
+        for a, b in zip(got, plain(*vals)):
+            np.testing.assert_allclose(a, b, rtol=2e-5 if dtype == "float32" else 1e-11, atol=2e-5 if dtype == "float32" else 1e-11)
+
+
 def test_epilogue_chain_with_per_result_device_operands():
     """Per-channel algebra after a reduction (other per-channel arrays, results
     of an earlier reduction, host scalars) runs in the reduction's epilogue;
@@ -264,10 +298,18 @@ def test_epilogue_chain_with_per_result_device_operands():
     outs = [s1 * gamma + beta / std, (s2 - s1) * T.exp(beta), T.sum(g, axis=(0, 2, 3))]
     vals = [rng.standard_normal((6, 37, 5, 9)).astype("float32"), rng.standard_normal((6, 37, 5, 9)).astype("float32"),
             rng.uniform(0.5, 2, (1, 37, 1, 1)).astype("float32"), rng.standard_normal((1, 37, 1, 1)).astype("float32")]
-    f = th.function([x, g, gamma, beta], outs)
-    kernels = [n for n in f.toposort() if isinstance(n.op, (HipCAReduce, HipElemwise))]
+    with th.config.change_flags(merge_dependent_reductions=False):
+        f2 = th.function([x, g, gamma, beta], outs)
+    kernels = [n for n in f2.toposort() if isinstance(n.op, (HipCAReduce, HipElemwise))]
     assert [type(n.op) for n in kernels] == [HipCAReduce, HipCAReduce], kernels
     assert any(type(i.type).__name__ == "HipArrayType" for i in kernels[1].inputs[len(kernels[1].inputs) - kernels[1].op.n_extra:])
+    # by default the second reduction gives up the mean in its prologue and joins the first one's pass
+    f = th.function([x, g, gamma, beta], outs)
+    kernels = [n for n in f.toposort() if isinstance(n.op, (HipCAReduce, HipElemwise))]
+    assert [type(n.op) for n in kernels] == [HipCAReduce], kernels
+    assert any(type(i.type).__name__ == "HipArrayType" for i in kernels[0].inputs[len(kernels[0].inputs) - kernels[0].op.n_extra:])
+    for a, b in zip(f(*vals), f2(*vals)):
+        np.testing.assert_allclose(a, b, rtol=3e-5, atol=3e-6)
     got = f(*vals)
     ref = G.evaluate([x, g, gamma, beta], outs, vals)
     truth = G.evaluate([x, g, gamma, beta], outs, vals, wide=True)

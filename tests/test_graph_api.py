@@ -212,29 +212,36 @@ def test_factors_constant_along_the_reduced_axes_leave_the_sum():
     assert isinstance(n.inputs[0].owner.op.scalar_op, scal.Mul)
 
 
-def test_batchnorm_gradient_is_two_statistics_passes_and_one_elementwise_pass(dry_run):
-    """Configuration 5's gradient graph: per-channel factors leave the sums, the
-    sums that then read the same tensors merge, and the per-channel algebra
-    between them runs in the second reduction's epilogue, which reads gamma as a
-    per-result device operand.  The first pass yields mean and standard deviation
-    together (shifted sums in float64 beside the mean's own sum).  Three kernels
-    remain; the first two are told which
-    of their inputs a later kernel reads again (those stay cacheable)."""
+def test_batchnorm_gradient_is_one_statistics_pass_and_one_elementwise_pass(dry_run):
+    """Configuration 5's gradient graph: per-channel factors leave the sums; the mean leaves the
+    prologue of sum(g * (x - mean)), which becomes sum(g * x) - mean * sum(g); that reduction then
+    depends on the statistics of x through its epilogue only and joins their pass.  One kernel reads
+    x and g once and yields mean, standard deviation and the three per-channel sums (six accumulators,
+    the per-channel algebra chained in its epilogue, gamma a per-result device operand); one elementwise
+    kernel follows.  The first is told that x and g are read again (they stay cacheable).  With the
+    rewrite switched off the graph keeps its two statistics passes."""
     import workloads
     ins, outs = workloads.c5_graph(forward=False)
+
+    def kernels_of(f):
+        return [n for n in f.toposort() if isinstance(n.op, (HipElemwise, HipCAReduce)) and
+                any(not any(i.type.broadcastable) for i in n.inputs if hasattr(i.type, "broadcastable") and i.type.ndim)]
+
     f = th.function(ins, [th.Out(o, device=True) for o in outs])
-    kernels = [n for n in f.toposort() if isinstance(n.op, (HipElemwise, HipCAReduce)) and
-               any(not any(i.type.broadcastable) for i in n.inputs if hasattr(i.type, "broadcastable") and i.type.ndim)]
-    assert [type(n.op) for n in kernels] == [HipCAReduce, HipCAReduce, HipElemwise]
-    first, second = kernels[0], kernels[1]
-    assert len(first.op.scalar_ops) == 3 and len(first.outputs) == 2
-    assert len(second.op.scalar_ops) == 3 and second.op.n_extra >= 4
-    extras = second.inputs[len(second.inputs) - second.op.n_extra:]
+    kernels = kernels_of(f)
+    assert [type(n.op) for n in kernels] == [HipCAReduce, HipElemwise]
+    stats = kernels[0]
+    assert len(stats.op.scalar_ops) == 6 and stats.op.acc_dtypes.count("float64") == 5
+    n_red = len(stats.inputs) - stats.op.n_extra
+    assert [str(i.type.dtype) for i in stats.inputs[:n_red] if not any(i.type.broadcastable)] == ["float16", "float16"]
+    extras = stats.inputs[n_red:]
     assert any(type(e.type).__name__ == "HipArrayType" for e in extras)
-    # x is read again after the first pass, x and g after the second; the last pass streams everything
-    assert [len(n.tag["reused_in"]) for n in kernels] == [1, 2, 0]
+    assert [len(n.tag["reused_in"]) for n in kernels] == [2, 0]
     small = workloads.c5_inputs("small")
     f(*small)                                      # plans and compiles every kernel (dry run)
+    with th.config.change_flags(merge_dependent_reductions=False):
+        g = th.function(ins, [th.Out(o, device=True) for o in outs])
+    assert [type(n.op) for n in kernels_of(g)] == [HipCAReduce, HipCAReduce, HipElemwise]
 
 
 def test_inplace_pass_reuses_single_use_intermediates_only(dry_run):

@@ -24,6 +24,10 @@ class _Config(object):
     # exp / log / sqrt / tanh / sigmoid
     duplicate_transcendentals = int(os.environ.get("THEANO_AMD_DUP_TRANSCENDENTALS", "1"))
 
+    # sum(g * (x - m)) with m a result of a reduction over the same elements becomes sum(g * x) - m * sum(g)
+    # (float64 accumulators only), and the two reductions then share one pass over memory
+    merge_dependent_reductions = True
+
     @contextlib.contextmanager
     def change_flags(self, **kw):
         old = {k: getattr(self, k) for k in kw}

@@ -91,7 +91,7 @@ struct RedAcc {
   }
 };
 
-// Plan members: typedef IT; enum { NK, VEC, UNR, BLOCK, TPR, RA2 (1 when RA > 1) };
+// Plan members: typedef IT; enum { NK, VEC, UNR, NACC, BLOCK, TPR, RA2 (1 when RA > 1) };
 // static constexpr int mode(int input); static constexpr int sclass(int input, int which).
 template <class P, class IT>
 THX_DEV IT red_term(int input, int which, IT coord, IT stride) {
@@ -129,9 +129,12 @@ __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, R:
     for (int i = 0; i < NIN; ++i) base[i] += (IT)rem * p.kstride[i][0];
   }
 
-  Acc acc[UNR];
+  // UNR vectors are in flight per thread; they are folded into NACC accumulator sets (a set per
+  // vector costs registers that long accumulator structs do not leave at 1024 threads per block)
+  constexpr int NACC = P::NACC < UNR ? P::NACC : UNR;
+  Acc acc[NACC];
 #pragma unroll
-  for (int u = 0; u < UNR; ++u) R::init(acc[u]);
+  for (int u = 0; u < NACC; ++u) R::init(acc[u]);
 
   if (live) {
     const long long j0 = (long long)s * p.chunk;
@@ -164,11 +167,11 @@ __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, R:
       }
 #pragma unroll
       for (int u = 0; u < UNR; ++u)
-        if (ok[u]) R::template accum<VEC>(acc[u], r[u]);
+        if (ok[u]) R::template accum<VEC>(acc[u % NACC], r[u]);
     }
   }
 #pragma unroll
-  for (int u = 1; u < UNR; ++u) R::comb(acc[0], acc[u]);
+  for (int u = 1; u < NACC; ++u) R::comb(acc[0], acc[u]);
 
   Acc tot;
   if (TPR > THX_WAVE) {

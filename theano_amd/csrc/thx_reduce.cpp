@@ -385,6 +385,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     int unr = per_thread >= 4 ? 4 : per_thread >= 2 ? 2 : 1;
     const int force_unr = env_int("THX_RED_UNR", 0);
     if (force_unr > 0) unr = force_unr;
+    int nacc = unr;  // accumulator sets per thread
     // few outputs, long reduce domains: 1024 threads per output before resorting to a split
     int rblock = block;
     if (tpr == 256 && env_int("THX_RED_BIGBLOCK", 1) && ceil_div(n_out, 1) * 2 <= target_row * 4 &&
@@ -392,6 +393,9 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       rblock = 1024;
       tpr = 1024;
     }
+    const int force_nacc = env_int("THX_RED_NACC", 0);
+    if (force_nacc > 0) nacc = force_nacc;
+    if (nacc > unr) nacc = unr;
     const int rpb = rblock / tpr;
     const int64_t oblocks = ceil_div(n_out, rpb);
     int64_t chunk = nvec;
@@ -413,7 +417,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       skey += char('0' + sclass[i][1]);
     }
     std::ostringstream key;
-    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << "|m";
+    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nacc != unr ? "|c" + std::to_string(nacc) : "") << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -425,7 +429,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}}, mode, nt, sclass)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"NACC", nacc}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}}, mode, nt, sclass)
         << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void " << entry << "(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";

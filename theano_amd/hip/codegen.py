@@ -96,8 +96,26 @@ def acc_struct_bytes(acc_dtypes):
     return (off + align - 1) // align * align
 
 
+def _narrow_stores(pre_stmt, narrow):
+    """The prologue's closing stores ``v.aK = (acc type)pK;`` written so that they convert to whatever
+    type field K has in the struct at hand (``Acc``, or ``Part`` with its float32 fields)."""
+    import re
+    return re.sub(r"v\.a(\d+) = \([a-z0-9_]+\)(p\d+|i0);", r"v.a\1 = (decltype(v.a\1))\2;", pre_stmt)
+
+
+def comb_part_src(scalar_ops, acc_dtypes, narrow):
+    """Statements merging two ``Part`` values: float32 addition in the narrowed fields, the
+    reduction's own op in its accumulator type in the others."""
+    out = []
+    for k, (op, dt, nw) in enumerate(zip(scalar_ops, acc_dtypes, narrow)):
+        dt = "float32" if nw else dt
+        cnode = Apply(op, [Scalar(dt)(), Scalar(dt)()], [Scalar(dt)()])
+        out.append(op.c_code(cnode, ["a.a%d" % k, "b.a%d" % k], ["a.a%d" % k]))
+    return out
+
+
 def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, post_op=None, extra_dtypes=(),
-                   post_in_dtypes=None, extra_is_array=None):
+                   post_in_dtypes=None, extra_is_array=None, half_data=False):
     """(source, name, sizeof(Acc)) for K simultaneous reductions.
 
     Per element, ``pre_op`` (nin = len(in_dtypes), nout = K; default: the single
@@ -129,16 +147,25 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
         if nin != 1 or K != 1:
             raise ValueError("a reduction without prologue takes one input and one accumulator")
         pre_stmt = "v.a0 = (%s)i0;" % acc_c[0]
+        value_dtypes = ["float32" if in_dtypes[0] == "float16" else in_dtypes[0]]
     else:
         pnode = _scalar_node(pre_op, in_dtypes)
         if len(pnode.outputs) != K:
             raise ValueError("prologue yields %d values for %d reductions" % (len(pnode.outputs), K))
         tmp = ["p%d" % k for k in range(K)]
+        value_dtypes = ["float32" if o.type.dtype == "float16" else o.type.dtype for o in pnode.outputs]
         pre_stmt = " ".join("%s %s;" % (compute_ctype(o.type.dtype), t) for o, t in zip(pnode.outputs, tmp))
         pre_stmt += "\n" + pre_op.c_code(pnode, ins, tmp) + "\n"
         pre_stmt += " ".join("v.a%d = (%s)%s;" % (k, acc_c[k], t) for k, t in enumerate(tmp))
-    lines.append("  THX_DEV static void pre(%s, Acc& v) {\n%s\n  }" % (
-        ", ".join("const %s %s" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)), _indent(pre_stmt, 4)))
+    # float32 partial sums per vector for float64 sums over float16 data (see ``half_data``)
+    narrow = [half_data and isinstance(op, scal.Add) and acc == "float64" and val == "float32"
+              for op, acc, val in zip(scalar_ops, acc_dtypes, value_dtypes)]
+    if any(narrow):
+        lines[1] += "\n  struct Part { %s };" % " ".join(
+            "%s a%d;" % ("thx_f32" if nw else c, k) for k, (c, nw) in enumerate(zip(acc_c, narrow)))
+    lines.append("  template <class AccT> THX_DEV static void pre(%s, AccT& v) {\n%s\n  }" % (
+        ", ".join("const %s %s" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)),
+        _indent(pre_stmt if not any(narrow) else _narrow_stores(pre_stmt, narrow), 4)))
     # combine: the reduction op applied to two accumulator-typed values
     comb = []
     for k, (op, dt) in enumerate(zip(scalar_ops, acc_dtypes)):
@@ -146,8 +173,19 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
         comb.append(op.c_code(cnode, ["a.a%d" % k, "b.a%d" % k], ["a.a%d" % k]))
     lines.append("  THX_DEV static void comb(Acc& a, const Acc& b) {\n%s\n  }" % _indent("\n".join(comb), 4))
     call = ", ".join("(%s)r.%s.v[k]" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins))
-    lines.append("  template <int V> THX_DEV static void accum(Acc& s, const Regs<V>& r) {\n#pragma unroll\n"
-                 "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s, t); }\n  }" % call)
+    if any(narrow):
+        # the elements of one vector meet in a Part (float32 where narrowed) before the accumulator sees them
+        comb_part = comb_part_src(scalar_ops, acc_dtypes, narrow)
+        lines.append("  THX_DEV static void comb_part(Part& a, const Part& b) {\n%s\n  }" % _indent("\n".join(comb_part), 4))
+        call0 = call.replace(".v[k]", ".v[0]")
+        widen = " ".join("w.a%d = (%s)t.a%d;" % (k, acc_c[k], k) for k in range(K))
+        lines.append("  template <int V> THX_DEV static void accum(Acc& s, const Regs<V>& r) {\n"
+                     "    Part t; pre(%s, t);\n#pragma unroll\n"
+                     "    for (int k = 1; k < V; ++k) { Part u; pre(%s, u); comb_part(t, u); }\n"
+                     "    Acc w; %s comb(s, w);\n  }" % (call0, call, widen))
+    else:
+        lines.append("  template <int V> THX_DEV static void accum(Acc& s, const Regs<V>& r) {\n#pragma unroll\n"
+                     "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s, t); }\n  }" % call)
     lines.append("  template <int V> THX_DEV static void accum_lanes(Acc* s, const Regs<V>& r) {\n#pragma unroll\n"
                  "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s[k], t); }\n  }" % call)
     lines.append("  THX_DEV static Acc shfl_xor(const Acc& a, int m) { Acc r; %s return r; }" % " ".join(

@@ -414,12 +414,18 @@ class HipCAReduce(CAReduce):
         in_dt = tuple(i.type.dtype for i in node.inputs[:n_red])
         ex_dt = tuple(i.type.dtype for i in node.inputs[n_red:])
         ex_arr = tuple(isinstance(i.type, HipArrayType) for i in node.inputs[n_red:])
-        key = (self._props(), in_dt, ex_dt, ex_arr)
+        # float16 storage behind every operand that varies along a reduced dimension
+        nd = max(i.type.ndim for i in node.inputs[:n_red])
+        axis = self.axis if self.axis is not None else tuple(range(nd))
+        data = [i for i in node.inputs[:n_red] if isinstance(i.type, HipArrayType) and
+                not all(i.type.broadcastable[a] for a in axis)]
+        half_data = bool(data) and all(i.type.dtype == "float16" for i in data)
+        key = (self._props(), in_dt, ex_dt, ex_arr, half_data)
         h = _reduce_handles.get(key)
         if h is None:
             src, name, acc_bytes = codegen.reduce_functor(self.scalar_ops, self.acc_dtypes, in_dt, self.out_dtypes,
                                                           self.pre_scalar_op, self.post_scalar_op, ex_dt,
-                                                          self.post_in_dtypes, ex_arr)
+                                                          self.post_in_dtypes, ex_arr, half_data)
             all_dt = in_dt + self.out_dtypes + ex_dt
             codes = (ctypes.c_int32 * len(all_dt))(*[scal.dtype_code(d) for d in all_dt])
             handle = ctypes.c_void_p()

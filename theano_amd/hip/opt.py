@@ -785,6 +785,14 @@ def fuse_around_reductions(fgraph):
     merge_sibling_reductions(fgraph)
     gof.merge_identical(fgraph)
     fuse_reduce_epilogue(fgraph)
+    # a sum that reads results of a reduction over the same elements joins that reduction's pass
+    from .hoist import hoist_result_operands, merge_chained_reductions
+    if config.merge_dependent_reductions:
+        if hoist_result_operands(fgraph):
+            gof.merge_identical(fgraph)
+        if merge_chained_reductions(fgraph):
+            gof.merge_identical(fgraph)
+            fuse_reduce_epilogue(fgraph)
     fuse_argmax_prologue(fgraph)
     gof.merge_identical(fgraph)
     fuse_elemwise(fgraph)          # producers that lost their other clients to an epilogue

@@ -1296,8 +1296,10 @@ class Composite(ScalarOp):
         first, repl = {}, {}
         for node in gof.io_toposort(inputs, outputs):
             node.inputs = [repl.get(i, i) for i in node.inputs]
-            key = (node.op, tuple(("c", str(i.type), repr(i.data)) if isinstance(i, Constant) else id(i)
-                                  for i in node.inputs))
+            operands = [("c", str(i.type), repr(i.data)) if isinstance(i, Constant) else ("v", id(i)) for i in node.inputs]
+            if isinstance(node.op, (Add, Mul)):      # a * b and b * a are one value
+                operands.sort()
+            key = (node.op, tuple(operands))
             prev = first.setdefault(key, node)
             if prev is not node:
                 repl.update(zip(node.outputs, prev.outputs))

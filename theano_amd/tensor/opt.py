@@ -477,7 +477,11 @@ def local_single_pass_variance(fgraph, node):
     else:
         a, c0 = scal.Scalar(x.type.dtype)(), scal.Scalar(src.type.dtype)()
         d = Elemwise(scal.Composite([a, c0], [scal.sub(a, scal.cast(c0, x.type.dtype))]))(x, cb)
-    d = T.cast(d, "float64")          # squares exact, and one fused multiply-add per element
+    if src.type.dtype != "float16":
+        d = T.cast(d, "float64")      # squares exact, and one fused multiply-add per element
+    # float16 storage: d stays float32 (exact: both operands hold 11 bits), its square is rounded to
+    # float32 (2**-24, nothing next to the data's own 2**-11) and the kernels add float32 partial
+    # sums per vector into the float64 accumulators, which keeps them off the vector ALU's limit
     s1 = Sum(node.op.axis, dtype="float64", acc_dtype="float64")(d)
     s2 = Sum(node.op.axis, dtype="float64", acc_dtype="float64")(T.sqr(d))
     n = None
