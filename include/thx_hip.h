@@ -155,7 +155,9 @@ int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, 
 /* Reduce the dimensions d with reduce_mask[d] != 0. `ins` holds the n_in reduced
  * inputs, which all have rank nd and broadcast against each other like Elemwise
  * inputs, followed by the n_extra operands of the epilogue: each either a THX_HOST_SCALAR or a
- * C-contiguous device array with one element per result, read at the result's index; `outs` are
+ * device array with one element per result, laid out like a C-contiguous array with every stride
+ * scaled by one factor (contiguous, or a view such as x[0, :, 0, 0]) and read at the result's
+ * index; `outs` are
  * C-contiguous arrays of the kept dimensions, in order. A zero-length reduce domain yields
  * the identity (the caller rejects it for max/min, as
  * theano/tensor/elemwise.py:1489-1506 does). Asynchronous.

@@ -265,7 +265,7 @@ def test_sums_over_results_of_a_reduction_over_the_same_elements_share_its_pass(
         f = th.function([x, g], outs)
         reds = [n for n in f.toposort() if isinstance(n.op, HipCAReduce)]
         if dtype == "float32" and axes != (1,):      # (last-axis islands are row chains; float64 variances keep two passes)
-            assert len(reds) == 1 and len(reds[0].op.scalar_ops) == 5, [str(n.op)[:60] for n in reds]
+            assert len(reds) == 1 and len(reds[0].op.scalar_ops) <= 5, [str(n.op)[:60] for n in reds]
         got = f(*vals)
         ref = G.evaluate([x, g], outs, vals)
         truth = G.evaluate([x, g], outs, vals, wide=True) if dtype == "float32" else ref

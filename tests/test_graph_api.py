@@ -216,7 +216,8 @@ def test_batchnorm_gradient_is_one_statistics_pass_and_one_elementwise_pass(dry_
     """Configuration 5's gradient graph: per-channel factors leave the sums; the mean leaves the
     prologue of sum(g * (x - mean)), which becomes sum(g * x) - mean * sum(g); that reduction then
     depends on the statistics of x through its epilogue only and joins their pass.  One kernel reads
-    x and g once and yields mean, standard deviation and the three per-channel sums (six accumulators,
+    x and g once and yields mean, standard deviation and the three per-channel sums (four float64
+    accumulators - sum(x), sum((x - c)^2), sum(g), sum(g x): every sum the two epilogues need is one of them -
     the per-channel algebra chained in its epilogue, gamma a per-result device operand); one elementwise
     kernel follows.  The first is told that x and g are read again (they stay cacheable).  With the
     rewrite switched off the graph keeps its two statistics passes."""
@@ -231,12 +232,12 @@ def test_batchnorm_gradient_is_one_statistics_pass_and_one_elementwise_pass(dry_
     kernels = kernels_of(f)
     assert [type(n.op) for n in kernels] == [HipCAReduce, HipElemwise]
     stats = kernels[0]
-    assert len(stats.op.scalar_ops) == 6 and stats.op.acc_dtypes.count("float64") == 5
+    assert len(stats.op.scalar_ops) == 4 and stats.op.acc_dtypes.count("float64") == 4
     n_red = len(stats.inputs) - stats.op.n_extra
     assert [str(i.type.dtype) for i in stats.inputs[:n_red] if not any(i.type.broadcastable)] == ["float16", "float16"]
     extras = stats.inputs[n_red:]
     assert any(type(e.type).__name__ == "HipArrayType" for e in extras)
-    assert [len(n.tag["reused_in"]) for n in kernels] == [2, 0]
+    assert len(kernels[0].tag["reused_in"]) >= 2 and len(kernels[1].tag["reused_in"]) == 0
     small = workloads.c5_inputs("small")
     f(*small)                                      # plans and compiles every kernel (dry run)
     with th.config.change_flags(merge_dependent_reductions=False):

@@ -154,14 +154,63 @@ class Function(object):
                 if id(o) not in last and id(o) not in keep:
                     self.release[k].append(self.storage[o])
         self._mark_reuse()
+        static = self._shape_only_nodes()
+        for k, node in enumerate(self.nodes):      # what such nodes computed is kept between calls
+            held = [self.storage[o] for s in static for o in s.outputs]
+            self.release[k] = [c for c in self.release[k] if not any(c is h for h in held)]
         self.thunks = []
         for node in self.nodes:
             node.op.prepare_node(node)
             self.thunks.append((node.op.perform, node, [self.storage[i] for i in node.inputs],
-                                [self.storage[o] for o in node.outputs]))
+                                [self.storage[o] for o in node.outputs], node in static,
+                                self.release[len(self.thunks)]))
+        self._static_key = None
         self._constants_ready = False
         self._HipArray = HipArray
         self._last_shape = {}
+
+    def _shape_only_nodes(self):
+        """Host nodes whose results depend on nothing but the shapes of the function's arguments: the
+        extents ``mean`` divides by (``ShapeFloat``) and host DimShuffles of them.  They run when the
+        argument shapes differ from the previous call's and keep their results otherwise: a
+        batch-normalisation function holds a dozen of them, each a few microseconds of host time
+        that a 20 us kernel does not hide."""
+        from .tensor.basic import ShapeFloat
+        from .tensor.elemwise import DimShuffle
+        from .tensor import views as V
+        from .hip.ops import HipDimShuffle, HipElemwise, HipCAReduce, HipMaxAndArgmax, HostToHip, HipToHost
+        inputs = set(id(v) for v in self.fgraph.inputs)
+        pure = {}
+
+        def shape_pure(v):
+            """Is the shape of ``v`` a function of the arguments' shapes alone?"""
+            if id(v) in pure:
+                return pure[id(v)]
+            if v.owner is None:
+                res = id(v) in inputs
+            else:
+                op = v.owner.op
+                if isinstance(op, (V.Subtensor, V.IncSubtensor, V.Reshape, V.Alloc)) and len(v.owner.inputs) > (
+                        2 if isinstance(op, V.IncSubtensor) else 1):
+                    res = False             # extents or indices that are run-time values
+                elif isinstance(op, (HostToHip, HipToHost, DimShuffle, HipElemwise, HipCAReduce, HipMaxAndArgmax,
+                                     V.Subtensor, V.IncSubtensor, V.Reshape, V.Alloc, V.Rebroadcast)) or (
+                                         type(op).__name__ == "HipRowChain"):
+                    res = all(shape_pure(i) for i in v.owner.inputs if hasattr(i.type, "ndim"))
+                else:
+                    res = False
+            pure[id(v)] = res
+            return res
+
+        static = set()
+        for node in self.nodes:
+            if isinstance(node.op, ShapeFloat) and shape_pure(node.inputs[0]):
+                static.add(node)
+            elif (type(node.op) is DimShuffle and node.inputs[0].owner is not None and
+                  node.inputs[0].owner in static):
+                static.add(node)
+        outs = set(id(o) for o in self.fgraph.outputs)
+        return set(n for n in static if not any(id(o) in outs for o in n.outputs))
 
     def _upload_constants(self):
         for c in self.constants:
@@ -194,10 +243,16 @@ class Function(object):
                         self._last_shape[var] = v.shape
                 except TypeError as e:
                     raise TypeError("Bad input argument to theano function with name \"%s\": %s" % (spec.name, e))
-        for k, (perform, node, ins, outs) in enumerate(self.thunks):
+        key = tuple([a.shape for a in args if hasattr(a, "shape")])
+        same = key == self._static_key
+        self._static_key = None                 # stays unset if a node raises half-way
+        for perform, node, ins, outs, static, release in self.thunks:
+            if static and same:
+                continue
             perform(node, [c[0] for c in ins], outs)
-            for cell in self.release[k]:
+            for cell in release:
                 cell[0] = None
+        self._static_key = key
         results = [self.storage[o][0] for o in self.fgraph.outputs]
         if self.update_targets:
             n_out = len(results) - len(self.update_targets)

@@ -22,11 +22,13 @@
 namespace thx {
 
 // Where results go, plus the epilogue's further operands: the value of a host scalar, or the
-// address of a device array that holds one element per result.
+// address of a device array that holds one element per result, `exs` elements apart (1 for a
+// contiguous array; a view such as x[0, :, 0, 0] has the stride of the axis it keeps).
 template <int NOUT, int NEX>
 struct RedOut {
   char* ptr[NOUT];
   unsigned long long ex[NEX > 0 ? NEX : 1];
+  long long exs[NEX > 0 ? NEX : 1];
 };
 
 // ---------------------------------------------------------------------------

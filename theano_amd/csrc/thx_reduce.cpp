@@ -82,8 +82,8 @@ static int not_loaded(const thx_reduce* r, const std::string& plan) {
 }
 
 // `fixed`: the call comes from thx_reduce_call_static - only kernels that are already loaded, no events.
-static int final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::vector<uint64_t>& ex, char* partial,
-                      int64_t n_out, int S, bool dry, bool fixed = false) {
+static int final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::vector<uint64_t>& ex,
+                      const std::vector<int64_t>& exs, char* partial, int64_t n_out, int S, bool dry, bool fixed = false) {
   const int tpo = final_tpo(n_out);
   const std::string plan = "rf|t" + std::to_string(tpo);
   Kernel k;
@@ -105,6 +105,7 @@ static int final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::
   ParamPack pk;
   for (char* p : outp) pk.put<char*>(p);
   for (uint64_t v : ex) pk.put<uint64_t>(v);
+  for (int64_t v : exs) pk.put<int64_t>(v);
   pk.put<char*>(partial);
   pk.put<int64_t>(n_out);
   pk.put<int32_t>(S);
@@ -236,9 +237,12 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     if (((uintptr_t)outp[o]) % isz) return fail(THX_ERR_TYPE, "reduce: output %d is not aligned to its element size", o);
   }
   // Operands of the epilogue follow the reduced inputs: a host scalar is passed by value; a device
-  // array holds one value per result (the results' element count, C-contiguous) and is passed by
-  // address, the epilogue reads it at the result's index.
+  // array holds one value per result (the results' element count) and is passed by address and element
+  // stride, the epilogue reads it at the result's index times that stride.  Its layout must be that of a
+  // C-contiguous array with every stride scaled by one factor (a contiguous array, or a view that keeps
+  // the results' dimensions in order, such as x[0, :, 0, 0]).
   std::vector<uint64_t> ex(std::max(1, r->n_extra), 0);
+  std::vector<int64_t> exs(std::max(1, r->n_extra), 1);
   for (int j = 0; j < r->n_extra; ++j) {
     const thx_array& a = ins[NIN + j];
     const int want = r->dtypes[NIN + NOUT + j];
@@ -250,17 +254,26 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       memcpy(&ex[j], p, (size_t)dtype_size(want));
       continue;
     }
-    int64_t count = 1, expect = dtype_size(want);
+    const int64_t isz = dtype_size(want);
+    int64_t count = 1, expect = 0;
     for (int d = a.nd - 1; d >= 0; --d) {
-      if (a.shape[d] > 1 && a.strides_bytes[d] != expect)
-        return fail(THX_ERR_TYPE, "reduce: epilogue operand %d is not C-contiguous", j);
-      expect *= a.shape[d];
+      if (a.shape[d] > 1) {
+        if (!expect) {
+          if (a.strides_bytes[d] % isz || !a.strides_bytes[d])
+            return fail(THX_ERR_TYPE, "reduce: epilogue operand %d has a stride that is not a multiple of its element size", j);
+          expect = a.strides_bytes[d];
+          exs[j] = a.strides_bytes[d] / isz;
+        }
+        if (a.strides_bytes[d] != expect)
+          return fail(THX_ERR_TYPE, "reduce: epilogue operand %d is not laid out like a C-contiguous array", j);
+        expect *= a.shape[d];
+      }
       count *= a.shape[d];
     }
     if (count != n_out)
       return fail(THX_ERR_SHAPE, "Input dimension mis-match. (epilogue operand %d has %lld elements, the result has %lld)",
                   j, (long long)count, (long long)n_out);
-    if (((uintptr_t)p) % dtype_size(want))
+    if (((uintptr_t)p) % isz)
       return fail(THX_ERR_TYPE, "reduce: epilogue operand %d is not aligned to its element size", j);
     ex[j] = (uint64_t)(uintptr_t)p;
   }
@@ -270,7 +283,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
   }
   if (n_red == 0) {  // identity through the epilogue
     set_last_plan(r->name + "|rf|identity");
-    return final_pass(r, outp, ex, nullptr, n_out, 0, dry, fixed);
+    return final_pass(r, outp, ex, exs, nullptr, n_out, 0, dry, fixed);
   }
 
   // primary input: the one that spans the most memory
@@ -445,6 +458,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
     for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
     for (uint64_t v : ex) pk.put<uint64_t>(v);
+    for (int64_t v : exs) pk.put<int64_t>(v);
     pk.put<char*>(partial);
     pk.put<int64_t>(n_out);
     pk.put<int64_t>(nvec);
@@ -562,6 +576,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
     for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
     for (uint64_t v : ex) pk.put<uint64_t>(v);
+    for (int64_t v : exs) pk.put<int64_t>(v);
     pk.put<char*>(partial);
     pk.put<int64_t>(n_out);
     pk.put<int64_t>(rows);
@@ -614,6 +629,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
     for (int o = 0; o < NOUT; ++o) pk.put<char*>(outp[o]);
     for (uint64_t v : ex) pk.put<uint64_t>(v);
+    for (int64_t v : exs) pk.put<int64_t>(v);
     pk.put<int64_t>(n_out);
     pk.put<int64_t>(n_red);
     for (int d = 0; d < NK; ++d) pk.put<FastDivH>(make_fastdiv(d < NKD ? (uint64_t)KD[d].extent : 1));
@@ -634,7 +650,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     rc = launch(k, r->name + "|" + plan, (unsigned)grid, launch_block, pk.buf.data(), pk.buf.size(), fixed);
     if (rc) return rc;
   }
-  if (S > 1) return final_pass(r, outp, ex, partial, n_out, S, dry, fixed);
+  if (S > 1) return final_pass(r, outp, ex, exs, partial, n_out, S, dry, fixed);
   return THX_OK;
 }
 

@@ -217,7 +217,7 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
             args.append("r%d" % k)
         for j, dt in enumerate(extra_dtypes):
             if extra_is_array is not None and extra_is_array[j]:
-                args.append("(((const %s*)o.ex[%d])[idx])" % (storage_ctype(dt), j))
+                args.append("(((const %s*)o.ex[%d])[idx * o.exs[%d]])" % (storage_ctype(dt), j, j))
             else:
                 args.append("(*(const %s*)&o.ex[%d])" % (storage_ctype(dt), j))
         post_stmt += "\n" + post_op.c_code(qnode, args, tmp) + "\n"

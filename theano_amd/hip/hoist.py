@@ -118,19 +118,31 @@ def _canon(v):
     return v
 
 
+_RANK = {"float16": 0, "float32": 1, "float64": 2}
+
+
 def _unique_accumulators(s_inputs, exprs, ops, acc_dts):
-    """One Composite over ``s_inputs`` yielding ``exprs`` with equal (expression, op, accumulator type)
-    triples computed once; returns (composite, ops, acc dtypes, position of each original in it)."""
+    """One Composite over ``s_inputs`` yielding ``exprs`` with equal (expression, op) pairs computed and
+    accumulated once; returns (composite, ops, acc dtypes, position of each original in it).  Two sums
+    of one expression that differ in their float accumulator type share the wider one: an accumulator
+    wider than asked for is never farther from the exact sum."""
     comp = scal.Composite(s_inputs, exprs)
+    ops, acc_dts = list(ops), list(acc_dts)
     uniq, where = [], []
     for s, o in enumerate(comp.outputs):
         for q, u in enumerate(uniq):
             same = _canon(comp.outputs[u]) is _canon(o) or (
                 isinstance(o, Constant) and isinstance(comp.outputs[u], Constant) and
                 o.type == comp.outputs[u].type and o.data == comp.outputs[u].data)
-            if same and ops[u] == ops[s] and acc_dts[u] == acc_dts[s]:
-                where.append(q)
-                break
+            if not same or ops[u] != ops[s]:
+                continue
+            if acc_dts[u] != acc_dts[s]:
+                if not (isinstance(ops[s], scal.Add) and acc_dts[u] in _RANK and acc_dts[s] in _RANK):
+                    continue
+                if _RANK[acc_dts[s]] > _RANK[acc_dts[u]]:
+                    acc_dts[u] = acc_dts[s]
+            where.append(q)
+            break
         else:
             where.append(len(uniq))
             uniq.append(s)

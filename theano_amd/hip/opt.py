@@ -660,6 +660,36 @@ def _merge_two(a, b):
     return op.make_node(*inputs)
 
 
+def share_equal_accumulators(fgraph):
+    """A multi-reduction that accumulates one expression twice with the same op - ``sum(x)`` asked for by a
+    mean and again by a variance - keeps one accumulator (the wider of two float types) and an epilogue
+    that hands it to both results."""
+    from .hoist import _unique_accumulators
+    count = 0
+    for node in fgraph.toposort():
+        op = node.op
+        if not isinstance(op, HipCAReduce) or op.pre_scalar_op is None or op.post_scalar_op is not None:
+            continue
+        pre = op.pre_scalar_op
+        new_pre, u_ops, u_accs, where = _unique_accumulators(pre.inputs, pre.outputs, op.scalar_ops, op.acc_dtypes)
+        if len(u_ops) == len(op.scalar_ops):
+            continue
+        s_acc = [scal.Scalar(dt)() for dt in u_accs]
+        post_outs = []
+        for k, dt in enumerate(op.out_dtypes):
+            r = scal.cast(s_acc[where[k]], dt)
+            post_outs.append(scal.identity(r) if r in s_acc else r)
+        new_op = HipCAReduce(tuple(u_ops), op.axis, tuple(u_accs), op.out_dtypes, new_pre, scal.Composite(s_acc, post_outs),
+                             tuple(u_accs), 0)
+        new_node = new_op.make_node(*node.inputs)
+        if [o.type for o in new_node.outputs] != [o.type for o in node.outputs]:
+            continue
+        for o, no in zip(node.outputs, new_node.outputs):
+            fgraph.replace(o, no)
+        count += 1
+    return count
+
+
 def merge_sibling_elemwise(fgraph):
     """Two elementwise kernels of one and the same shape become one kernel with several results
     when that saves reading an array again: siblings that read a common array (the two moment
@@ -784,6 +814,7 @@ def fuse_around_reductions(fgraph):
     gof.merge_identical(fgraph)
     merge_sibling_reductions(fgraph)
     gof.merge_identical(fgraph)
+    share_equal_accumulators(fgraph)
     fuse_reduce_epilogue(fgraph)
     # a sum that reads results of a reduction over the same elements joins that reduction's pass
     from .hoist import hoist_result_operands, merge_chained_reductions

@@ -243,6 +243,18 @@ class HipArray(object):
         self.code = _CODE_OF[self.dtype]
 
     @classmethod
+    def _raw(cls, buffer, offset, shape, strides, dtype, code):
+        """A view from fields that are already of the right kind (tuples of ints, a np.dtype)."""
+        self = cls.__new__(cls)
+        self.buffer = buffer
+        self.offset = offset
+        self.shape = shape
+        self.strides = strides
+        self.dtype = dtype
+        self.code = code
+        return self
+
+    @classmethod
     def _new_contiguous(cls, shape, dtype):
         """``empty`` for callers that already hold a tuple of ints and a np.dtype."""
         self = cls.__new__(cls)
@@ -328,6 +340,22 @@ class HipArray(object):
         return True
 
     @property
+    def scaled_contiguous(self):
+        """The layout of a C-contiguous array with every stride multiplied by one non-zero factor: a
+        contiguous array, or a view that keeps its dimensions in order (``x[0, :, 0, 0]``, ``x[::2]``)."""
+        expect = 0
+        for s, st in zip(reversed(self.shape), reversed(self.strides)):
+            if s > 1:
+                if not expect:
+                    if st == 0 or st % self.dtype.itemsize:
+                        return False
+                    expect = st
+                if st != expect:
+                    return False
+                expect *= s
+        return True
+
+    @property
     def is_fortran(self):
         """Column-major contiguous and not row-major contiguous (NumPy's
         ``PyArray_ISFORTRAN``)."""
@@ -398,17 +426,11 @@ class HipArray(object):
         a = out if out is not None else thx_array()
         a.base = self.buffer.ptr
         a.offset_bytes = self.offset
-        a.nd = len(self.shape)
+        n = len(self.shape)
+        a.nd = n
         a.dtype = self.code
-        shp, st = a.shape, a.strides_bytes
-        i = 0
-        for s in self.shape:
-            shp[i] = s
-            i += 1
-        i = 0
-        for s in self.strides:
-            st[i] = s
-            i += 1
+        a.shape[:n] = self.shape
+        a.strides_bytes[:n] = self.strides
         return a
 
 

@@ -482,13 +482,20 @@ def local_single_pass_variance(fgraph, node):
     # float16 storage: d stays float32 (exact: both operands hold 11 bits), its square is rounded to
     # float32 (2**-24, nothing next to the data's own 2**-11) and the kernels add float32 partial
     # sums per vector into the float64 accumulators, which keeps them off the vector ALU's limit
-    s1 = Sum(node.op.axis, dtype="float64", acc_dtype="float64")(d)
     s2 = Sum(node.op.axis, dtype="float64", acc_dtype="float64")(T.sqr(d))
-    n = None
-    for dv in divisors:
-        e = T.ShapeFloat(dv.owner.op.i, "float64")(dv.owner.inputs[0])
-        n = e if n is None else T.mul(n, e)
-    res = T.maximum(T.sub(s2, T.true_div(T.mul(s1, s1), n)), np.float64(0.0))
+    # sum(d) = sum(x) - N c with sum(x) in float64: the same accumulator serves the mean (its own sum asks for
+    # the same values), so the pass keeps two running sums per element instead of three.  With
+    # dm = sum(x) / N - c the correction sum(d)^2 / N is N dm^2; the extents enter one by one, as host
+    # scalars of the nodes that use them (a product node of their own would be a kernel of its own).
+    exts = [T.ShapeFloat(dv.owner.op.i, "float64")(dv.owner.inputs[0]) for dv in divisors]
+    dm = Sum(node.op.axis, dtype="float64", acc_dtype="float64")(x)
+    for e in exts:
+        dm = T.true_div(dm, e)
+    dm = T.sub(dm, T.cast(first, "float64"))
+    corr = T.mul(dm, dm)
+    for e in exts:
+        corr = T.mul(corr, e)
+    res = T.maximum(T.sub(s2, corr), np.float64(0.0))
     res = T.cast(res, out.type.dtype)
     return [res] if res.type == out.type else False
 
