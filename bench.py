@@ -250,7 +250,7 @@ def main():
             ms = min(_time_steps(hip, rotating, args.steps, 3)[0] for _ in range(3))
             warm_ms = min(_time_steps(hip, lambda: f(*sets[0]), args.steps, 3)[0] for _ in range(3))
             n_k = sum(1 for n in f.toposort()
-                      if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax"))
+                      if type(n.op).__name__ in ("HipElemwise", "HipElemwiseReduce", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax"))
             others[name] = _rate(W.algorithmic_bytes(name), ms)
             others[name].update({"input_sets": len(sets), "same_input_us": round(warm_ms * 1e3, 2),
                                  "nodes_per_step": n_k})

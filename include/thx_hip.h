@@ -112,6 +112,7 @@ int thx_cache_stats(int64_t* compiled, int64_t* disk_hits, int64_t* mem_hits);
 /* ---- Elemwise ------------------------------------------------------------ */
 
 typedef struct thx_elemwise thx_elemwise;
+typedef struct thx_reduce thx_reduce;
 
 /* Create an n-ary elementwise operation from generated device source defining
  * a functor type named `functor_name` (see kernels/thx_elemwise.h for the
@@ -137,9 +138,23 @@ int thx_elemwise_new(const char* functor_src, const char* functor_name, int n_in
 int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* outs, int flags);
 int thx_elemwise_free(thx_elemwise* e);
 
+/* An elementwise result that is stored and also reduced over every dimension but the last (the
+ * per-channel sum of an NHWC tensor that is an output as well): the reference runs GpuElemwise_call
+ * and then a GpuCAReduceCuda kernel that reads the result back (theano/gpuarray/elemwise.py:376,
+ * 1095-1723).  thx_elemwise_attach_reduce names the reduction `r` (created with thx_reduce_new,
+ * no further epilogue operands) whose n_in inputs are the outputs which_outputs[0 .. n_in) of `e`;
+ * the functor source given to thx_elemwise_new must then hold r's functor too and name it
+ * (`typedef <r's functor> Red;` plus `red_lanes`, see kernels/thx_elemwise.h).
+ * thx_elemwise_reduce_call = thx_elemwise_call plus that reduction into `red_outs` (C-contiguous,
+ * one element per index of the last dimension): inside the same kernel where the access plan allows
+ * it (permuted reads through LDS tiles), else by a reduction launched on the stored results.
+ * Asynchronous; same error behaviour as thx_elemwise_call. */
+int thx_elemwise_attach_reduce(thx_elemwise* e, thx_reduce* r, const int32_t* which_outputs);
+int thx_elemwise_reduce_call(thx_elemwise* e, const thx_array* ins, const thx_array* outs,
+                             const thx_array* red_outs, int flags);
+
 /* ---- CAReduce ------------------------------------------------------------ */
 
-typedef struct thx_reduce thx_reduce;
 
 /* Create a (multi-)reduction from generated device source defining a functor
  * named `functor_name` (contract in kernels/thx_reduce.h): n_in inputs feed a

@@ -280,6 +280,61 @@ def test_sums_over_results_of_a_reduction_over_the_same_elements_share_its_pass(
             np.testing.assert_allclose(a, b, rtol=2e-5 if dtype == "float32" else 1e-11, atol=2e-5 if dtype == "float32" else 1e-11)
 
 
+def test_stored_elementwise_result_and_its_reduction_over_all_but_the_last_axis():
+    """r = f(...) is an output and so is reduce(r, all axes but the last): one node (HipElemwiseReduce).  Through
+    permuted views (NCHW read as NHWC) the kernel that stores r accumulates the per-channel results as well
+    ('er' plan, partials merged by the reduction's final pass); with any other layout the library reduces the
+    stored result.  Integer results bit-exact, float32 at the float32 bar; ragged extents, one group and many."""
+    from theano_amd.hip import HipElemwiseReduce
+    rng = np.random.default_rng(29)
+    cases = [("int32", (3, 128, 7, 9)), ("int32", (5, 130, 33, 37)), ("int32", (2, 16, 4, 4)), ("float32", (9, 64, 20, 24)),
+             ("float32", (4, 36, 50, 70)), ("int16", (6, 64, 18, 32))]
+    for dtype, shape in cases:
+        t4 = T.TensorType(dtype, (False,) * 4)
+        a, b = t4("a"), t4("b")
+        av, bv = a.dimshuffle(0, 2, 3, 1), b.dimshuffle(0, 2, 3, 1)
+        if dtype == "float32":
+            r = T.tanh(av) * bv + av
+            vals = [rng.standard_normal(shape).astype(dtype) for _ in range(2)]
+            outs = [r, T.sum(r, axis=(0, 1, 2))]
+        else:
+            r = ((av & bv) ^ (av >> 2)) % 51 + bv
+            info = np.iinfo(dtype)
+            vals = [rng.integers(info.min // 4, info.max // 4, shape).astype(dtype) for _ in range(2)]
+            outs = [r, T.sum(r, axis=(0, 1, 2), dtype="int64")]
+        f = th.function([a, b], outs)
+        kinds = [type(n.op).__name__ for n in f.toposort() if type(n.op).__name__.startswith("Hip") and
+                 type(n.op).__name__ not in ("HipDimShuffle", "HipToHost")]
+        assert kinds == ["HipElemwiseReduce"], kinds
+        got = f(*vals)
+        plan = hip.last_plan()
+        assert "|er|" in plan or "rf|" in plan, plan
+        ref = G.evaluate([a, b], outs, vals)
+        assert_parity(got[0], ref[0], "%s %s elementwise result [%s]" % (dtype, shape, plan))
+        if dtype == "float32":
+            # the sum of the values this kernel stored (a last-place difference of tanh per element is inside the
+            # bar for r, but 14 000 of them do not cancel in a sum that itself nearly cancels)
+            want = got[0].astype("float64").sum(axis=(0, 1, 2)).astype("float32")
+            assert_parity(got[1], want, "%s %s sum of the stored result [%s]" % (dtype, shape, plan))
+            np.testing.assert_allclose(got[1], ref[1], rtol=1e-4, atol=1e-4)
+        else:
+            assert_parity(got[1], ref[1], "%s %s sum [%s]" % (dtype, shape, plan))
+    # no permuted read: the same node, reduced by a second launch of the library's own choosing
+    x = T.fmatrix("x")
+    r = T.exp(x) * T.tanh(x) + T.log1p(x * x)       # too much arithmetic to be recomputed inside the reduction
+    outs = [r, T.sum(r, axis=0)]
+    xv = rng.standard_normal((700, 96)).astype("float32")
+    f = th.function([x], outs)
+    assert any(isinstance(n.op, HipElemwiseReduce) for n in f.toposort())
+    got = f(xv)
+    assert " + " in hip.last_plan(), hip.last_plan()
+    for g, rr in zip(got, G.evaluate([x], outs, [xv])):
+        assert_parity(g, rr, "unpermuted")
+    # an empty leading extent: the results are the reductions' identities
+    e = th.function([x], [x + 1, T.sum(x + 1, axis=0)])(np.zeros((0, 5), "float32"))
+    assert e[0].shape == (0, 5) and np.array_equal(e[1], np.zeros(5, "float32"))
+
+
 def test_epilogue_chain_with_per_result_device_operands():
     """Per-channel algebra after a reduction (other per-channel arrays, results
     of an earlier reduction, host scalars) runs in the reduction's epilogue;

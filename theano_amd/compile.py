@@ -99,7 +99,7 @@ class Function(object):
             return isinstance(v.type, HipArrayType) and v.type.ndim > 0 and not any(v.type.broadcastable)
 
         kernels = [n for n in self.nodes
-                   if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax")]
+                   if type(n.op).__name__ in ("HipElemwise", "HipElemwiseReduce", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax")]
         later = set()
         for node in reversed(kernels):
             node.tag["reused_in"] = tuple(k for k, i in enumerate(node.inputs) if big(i) and id(root(i)) in later)

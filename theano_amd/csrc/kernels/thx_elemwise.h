@@ -168,6 +168,14 @@ __device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename 
 // Extra plan members: enum { TT, TI, TV (elements per access), NTR (staged
 // inputs), ESZ (largest staged element) }; static constexpr int slot(int
 // operand): LDS slot or -1.
+//
+// With plan member RED = 1 the kernel also reduces results over every dimension but the innermost
+// (the per-channel sum of an NHWC result that is written anyway): the functor names a reduction
+// functor `Red` (contract in thx_reduce.h) and feeds it element k of a thread's results through
+// `red_lane`.  A block then walks `rowtiles / groups` tiles of one and the same innermost range,
+// keeps TV accumulators per thread across them, merges the rows of its tile shape through LDS
+// and leaves one partial per innermost index, laid out [group][index] for the reductions' final
+// pass (or the result itself when there is one group).
 template <int NOPS, int ND, class IT>
 struct EwTrParams {
   char* ptr[NOPS];
@@ -178,6 +186,15 @@ struct EwTrParams {
   IT ostride[NOPS][ND];     // strides along the outer dimensions
   IT tstride[NOPS];
   IT istride[NOPS];
+};
+
+// What the reducing variant needs beyond EwTrParams.
+template <int NOUT, int NEX>
+struct EwRedParams {
+  RedOut<NOUT, NEX> out;    // results of the reduction (one element per innermost index)
+  char* partial;            // Acc[groups][ext_i] when groups > 1
+  int rowtiles;             // tiles over all dimensions but the innermost one
+  int groups;               // blocks that share one innermost range
 };
 
 template <class P, int NOPS>
@@ -235,85 +252,145 @@ struct TrAcc {  // LDS (transposed) or global -> registers, registers -> global
 // dimension while computing. The host guarantees that both extents are
 // multiples of TV and that every vector access is aligned.
 template <class F, class P>
-__device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, typename P::IT>& p) {
+struct EwTrTile {
   typedef typename P::IT IT;
-  constexpr int TT = P::TT, TI = P::TI, TV = P::TV, NOPS = F::NOPS, ND = P::ND;
-  constexpr int LPR_S = TT / TV;              // staging: lanes per row along T
-  constexpr int RPP_S = P::BLOCK / LPR_S;     //          rows (positions along the inner dimension) per pass
-  constexpr int PASSES_S = TI / RPP_S;
-  constexpr int LPR_C = TI / TV;              // computing: lanes per row along the inner dimension
-  constexpr int RPP_C = P::BLOCK / LPR_C;     //            rows (positions along T) per pass
-  constexpr int PASSES_C = TT / RPP_C;
-  constexpr int UNR = PASSES_C < 4 ? PASSES_C : 4;
+  static constexpr int TT = P::TT, TI = P::TI, TV = P::TV, NOPS = F::NOPS, ND = P::ND;
+  static constexpr int LPR_S = TT / TV;              // staging: lanes per row along T
+  static constexpr int RPP_S = P::BLOCK / LPR_S;     //          rows (positions along the inner dimension) per pass
+  static constexpr int PASSES_S = TI / RPP_S;
+  static constexpr int LPR_C = TI / TV;              // computing: lanes per row along the inner dimension
+  static constexpr int RPP_C = P::BLOCK / LPR_C;     //            rows (positions along T) per pass
+  static constexpr int PASSES_C = TT / RPP_C;
+  static constexpr int UNR = PASSES_C < 4 ? PASSES_C : 4;
+  static constexpr int LDS_BYTES = P::NTR * TI * (TT + 1) * P::ESZ;
   static_assert(PASSES_S >= 1 && PASSES_C >= 1 && PASSES_S * RPP_S == TI && PASSES_C * RPP_C == TT,
                 "tile and block do not divide");
-  __shared__ __attribute__((aligned(16))) unsigned char lds[P::NTR * TI * (TT + 1) * P::ESZ];
 
-  unsigned rem = blockIdx.x, ti, tt, c;
-  divmod(rem, p.tiles_i, rem, ti);
-  divmod(rem, p.tiles_t, rem, tt);
-  IT base[NOPS];
+  // One tile: `rem` counts tiles over the dimensions other than the innermost, `ti` tiles along it.
+  // ACC: per-thread accumulators of the reducing variant (one per element of a vector), or a dummy.
+  template <class ACC>
+  static __device__ __forceinline__ void run(const EwTrParams<NOPS, ND, IT>& p, unsigned char* lds, unsigned rem,
+                                             unsigned ti, ACC* acc) {
+    unsigned tt, c;
+    divmod(rem, p.tiles_t, rem, tt);
+    IT base[NOPS];
 #pragma unroll
-  for (int i = 0; i < NOPS; ++i) base[i] = 0;
+    for (int i = 0; i < NOPS; ++i) base[i] = 0;
 #pragma unroll
-  for (int d = ND - 3; d >= 1; --d) {
-    divmod(rem, p.ofd[d], rem, c);
+    for (int d = ND - 3; d >= 1; --d) {
+      divmod(rem, p.ofd[d], rem, c);
 #pragma unroll
-    for (int i = 0; i < NOPS; ++i) base[i] += (IT)c * p.ostride[i][d];
-  }
-  if (ND >= 3) {
+      for (int i = 0; i < NOPS; ++i) base[i] += (IT)c * p.ostride[i][d];
+    }
+    if (ND >= 3) {
 #pragma unroll
-    for (int i = 0; i < NOPS; ++i) base[i] += (IT)rem * p.ostride[i][0];
-  }
-  const int t0 = tt * TT, i0 = ti * TI;
+      for (int i = 0; i < NOPS; ++i) base[i] += (IT)rem * p.ostride[i][0];
+    }
+    const int t0 = tt * TT, i0 = ti * TI;
 
-  // stage: lanes run along T
-  {
-    typename F::template Regs<TV> dummy;
-    const int lane = threadIdx.x % LPR_S, row = threadIdx.x / LPR_S;
-    const int t = t0 + lane * TV;
+    // stage: lanes run along T
+    {
+      typename F::template Regs<TV> dummy;
+      const int lane = threadIdx.x % LPR_S, row = threadIdx.x / LPR_S;
+      const int t = t0 + lane * TV;
 #pragma unroll
-    for (int k = 0; k < PASSES_S; ++k) {
-      const int ii = row + k * RPP_S, i = i0 + ii;
-      if (t < p.ext_t && i < p.ext_i) {
-        TrStageAcc<P, NOPS> a;
-        a.ptr = p.ptr;
-        a.lds = lds;
-        a.cell = ii * (TT + 1) + lane * TV;
+      for (int k = 0; k < PASSES_S; ++k) {
+        const int ii = row + k * RPP_S, i = i0 + ii;
+        if (t < p.ext_t && i < p.ext_i) {
+          TrStageAcc<P, NOPS> a;
+          a.ptr = p.ptr;
+          a.lds = lds;
+          a.cell = ii * (TT + 1) + lane * TV;
 #pragma unroll
-        for (int o = 0; o < NOPS; ++o) a.off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
-        F::template load<TV>(a, dummy);
+          for (int o = 0; o < NOPS; ++o) a.off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
+          F::template load<TV>(a, dummy);
+        }
+      }
+    }
+    __syncthreads();
+
+    // compute: lanes run along the innermost dimension
+    const int lane = threadIdx.x % LPR_C, row = threadIdx.x / LPR_C;
+    const int i = i0 + lane * TV;
+#pragma unroll
+    for (int k0 = 0; k0 < PASSES_C; k0 += UNR) {
+      typename F::template Regs<TV> r[UNR];
+      TrAcc<P, NOPS> a[UNR];
+      bool ok[UNR];
+#pragma unroll
+      for (int u = 0; u < UNR; ++u) {
+        const int tl = row + (k0 + u) * RPP_C, t = t0 + tl;
+        ok[u] = t < p.ext_t && i < p.ext_i;
+        a[u].ptr = p.ptr;
+        a[u].imm = p.imm;
+        a[u].lds = lds;
+        a[u].cell = lane * TV * (TT + 1) + tl;
+#pragma unroll
+        for (int o = 0; o < NOPS; ++o) a[u].off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
+        if (ok[u]) F::template load<TV>(a[u], r[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < UNR; ++u)
+        if (ok[u]) F::template compute<TV>(r[u]);
+#pragma unroll
+      for (int u = 0; u < UNR; ++u)
+        if (ok[u]) F::template store<TV>(a[u], r[u]);
+      if constexpr (P::RED != 0) {
+#pragma unroll
+        for (int u = 0; u < UNR; ++u)
+          if (ok[u]) F::template red_lanes<TV>(acc, r[u]);
       }
     }
   }
-  __syncthreads();
+};
 
-  // compute: lanes run along the innermost dimension
-  const int lane = threadIdx.x % LPR_C, row = threadIdx.x / LPR_C;
-  const int i = i0 + lane * TV;
+template <class F, class P>
+__device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, typename P::IT>& p) {
+  typedef EwTrTile<F, P> Tile;
+  __shared__ __attribute__((aligned(16))) unsigned char lds[Tile::LDS_BYTES];
+  unsigned rem = blockIdx.x, ti;
+  divmod(rem, p.tiles_i, rem, ti);
+  Tile::run(p, lds, rem, ti, (int*)nullptr);
+}
+
+// The reducing variant: block b owns the innermost range b % tiles_i and the tiles g, g + groups, ...
+// (g = b / tiles_i) over the other dimensions.
+template <class F, class P>
+__device__ __forceinline__ void ew_tr_red_body(const EwTrParams<F::NOPS, P::ND, typename P::IT>& p,
+                                               const EwRedParams<F::Red::NOUT, F::Red::NEX>& q) {
+  typedef EwTrTile<F, P> Tile;
+  typedef typename F::Red R;
+  typedef typename R::Acc Acc;
+  constexpr int TI = P::TI, TV = P::TV, RPP = Tile::RPP_C;
+  constexpr int RED_BYTES = RPP * TI * (int)sizeof(Acc);
+  __shared__ __attribute__((aligned(16))) unsigned char lds[Tile::LDS_BYTES > RED_BYTES ? Tile::LDS_BYTES : RED_BYTES];
+  unsigned g = blockIdx.x, ti;
+  divmod(g, p.tiles_i, g, ti);
+  Acc acc[TV];
 #pragma unroll
-  for (int k0 = 0; k0 < PASSES_C; k0 += UNR) {
-    typename F::template Regs<TV> r[UNR];
-    TrAcc<P, NOPS> a[UNR];
-    bool ok[UNR];
+  for (int k = 0; k < TV; ++k) R::init(acc[k]);
+  for (unsigned j = g; j < (unsigned)q.rowtiles; j += (unsigned)q.groups) {
+    Tile::run(p, lds, j, ti, acc);
+    __syncthreads();              // the next tile's staging overwrites what this tile's compute phase read
+  }
+  // merge the RPP row lanes of the block: [row][position along the innermost dimension]
+  Acc* red = (Acc*)lds;
+  const int lane = threadIdx.x % Tile::LPR_C, row = threadIdx.x / Tile::LPR_C;
 #pragma unroll
-    for (int u = 0; u < UNR; ++u) {
-      const int tl = row + (k0 + u) * RPP_C, t = t0 + tl;
-      ok[u] = t < p.ext_t && i < p.ext_i;
-      a[u].ptr = p.ptr;
-      a[u].imm = p.imm;
-      a[u].lds = lds;
-      a[u].cell = lane * TV * (TT + 1) + tl;
-#pragma unroll
-      for (int o = 0; o < NOPS; ++o) a[u].off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
-      if (ok[u]) F::template load<TV>(a[u], r[u]);
+  for (int k = 0; k < TV; ++k) red[row * TI + lane * TV + k] = acc[k];
+  __syncthreads();
+  if (threadIdx.x < TI) {
+    const int i = (int)ti * TI + threadIdx.x;
+    if (i < p.ext_i) {
+      Acc tot = red[threadIdx.x];
+#pragma unroll 4
+      for (int y = 1; y < RPP; ++y) R::comb(tot, red[y * TI + threadIdx.x]);
+      if (q.groups == 1) {
+        R::post(q.out, (long long)i, tot);
+      } else {
+        ((Acc*)q.partial)[(long long)g * p.ext_i + i] = tot;
+      }
     }
-#pragma unroll
-    for (int u = 0; u < UNR; ++u)
-      if (ok[u]) F::template compute<TV>(r[u]);
-#pragma unroll
-    for (int u = 0; u < UNR; ++u)
-      if (ok[u]) F::template store<TV>(a[u], r[u]);
   }
 }
 

@@ -5,8 +5,8 @@
 #include <hip/hip_runtime.h>
 
 #include "kernels/thx_common.h"
-#include "kernels/thx_elemwise.h"
 #include "kernels/thx_reduce.h"
+#include "kernels/thx_elemwise.h"
 #include "kernels/thx_rowchain.h"
 
 struct CheckF {
@@ -47,6 +47,15 @@ struct CheckR {
   }
 };
 
+// an elementwise functor with an attached reduction of its result (permuted-read kernel, reducing variant)
+struct CheckFR : CheckF {
+  typedef CheckR Red;
+  template <int V, class AccT> THX_DEV static void red_lanes(AccT* acc, const Regs<V>& r) {
+#pragma unroll
+    for (int k = 0; k < V; ++k) { Red::Acc t; Red::pre((thx_f32)r.o0.v[k], t); Red::comb(acc[k], t); }
+  }
+};
+
 struct PlanEw1 { typedef int IT; enum { ND = 1, VEC = 4, UNR = 2, BLOCK = 256, GS = 1 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {0, 3, 0}; return m[i]; }
   static constexpr int sclass(int i, int d) { constexpr int m[][1] = {{1}, {0}, {1}}; return m[i][d]; }
@@ -66,9 +75,13 @@ struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, T
 struct PlanGen { typedef int IT; enum { NK = 3, NR = 3, BLOCK = 256, TPR = 64 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; } };
 
-struct PlanTr { typedef int IT; enum { ND = 3, TT = 64, TI = 32, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2 }; static constexpr unsigned long long NT = 0ull;
+struct PlanTr { typedef int IT; enum { ND = 3, TT = 64, TI = 32, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2, RED = 0 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2, 0, 0}; return m[i]; }
   static constexpr int slot(int i) { constexpr int m[] = {0, -1, -1}; return m[i]; } };
+struct PlanTrRed { typedef int IT; enum { ND = 3, TT = 32, TI = 32, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2, RED = 1 }; static constexpr unsigned long long NT = 0ull;
+  static constexpr int mode(int i) { constexpr int m[] = {2, 0, 0}; return m[i]; }
+  static constexpr int slot(int i) { constexpr int m[] = {0, -1, -1}; return m[i]; } };
+extern "C" __global__ __launch_bounds__(256) void check_tr_red(thx::EwTrParams<3, 3, int> p, thx::EwRedParams<2, 1> q) { thx::ew_tr_red_body<CheckFR, PlanTrRed>(p, q); }
 extern "C" __global__ __launch_bounds__(256) void check_tr(thx::EwTrParams<3, 3, int> p) { thx::ew_tr_body<CheckF, PlanTr>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_ew1(thx::EwParams<3, 1, int> p) { thx::ew_body<CheckF, PlanEw1>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_ew3(thx::EwParams<3, 3, long long> p) { thx::ew_body<CheckF, PlanEw3>(p); }

@@ -9,13 +9,6 @@
 
 #include "thx_internal.h"
 
-struct thx_elemwise {
-  std::string src, name;
-  int n_in = 0, n_out = 0;
-  std::vector<int32_t> dtypes;
-  std::unordered_map<std::string, thx::Kernel> plans;
-};
-
 namespace thx {
 
 enum { M_VEC = 0, M_BCAST = 1, M_GATHER = 2, M_IMM = 3 };
@@ -94,7 +87,13 @@ int thx_elemwise_free(thx_elemwise* e) {
   return THX_OK;
 }
 
-int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* outs, int flags) {
+}  // extern "C"
+
+// thx_elemwise_call and thx_elemwise_reduce_call.  With `red_outs` the operation's attached reduction is
+// computed as well: inside the permuted-read kernel when that plan is taken and the results' innermost
+// dimension is the one the reduction keeps (*fused = true), otherwise the caller reduces the stored results.
+static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array* outs, const thx_array* red_outs,
+                         int flags, bool* fused) {
   if (!e || !ins || !outs) return fail(THX_ERR_ARG, "thx_elemwise_call: null argument");
   const bool dry = (flags & THX_DRY_RUN) != 0;
   if (!dry) {
@@ -276,9 +275,17 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
       if (env_int("THX_EW_TV", 0) == 1) tv = 1;
       if ((int64_t)ntr * tile_i * (tile_t + 1) * esz <= 60000) {
         const int block = 256;
+        // the attached reduction rides along when it keeps exactly the innermost dimension of the results
+        // (which the collapse must have left alone) and the row lanes of a block fit the LDS
+        thx_reduce* R = red_outs ? e->red : nullptr;
+        const int rpp_c = block / (tile_i / tv);
+        const bool red = R && !env_int("THX_EW_NO_FUSED_REDUCE", 0) && nd >= 2 && inner == shape[nd - 1] &&
+                         tile_t % rpp_c == 0 && (int64_t)rpp_c * tile_i * R->acc_bytes <= 60000;
+        if (R && !red)   // the caller reduces the stored results next: they stay cacheable
+          for (int w : e->red_of) views[e->n_in + w].reused = true;
         const uint64_t nt = nt_mask(nt_streaming(moved), views);
         std::ostringstream key;
-        key << "et|nd" << ND << "|t" << tile_t << "x" << tile_i << "|v" << tv << "|n" << ntr << "|e" << esz;
+        key << (red ? "er|nd" : "et|nd") << ND << "|t" << tile_t << "x" << tile_i << "|v" << tv << "|n" << ntr << "|e" << esz;
         if (nt) key << "|nt" << std::hex << nt << std::dec;
         key << "|m";
         for (int o = 0; o < nops; ++o) key << (slot[o] >= 0 ? 9 : mode[o]) << (o + 1 < nops ? "," : "");
@@ -293,18 +300,23 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
           std::ostringstream s;
           s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef int IT;\n  enum { ND = " << ND
             << ", TT = " << tile_t << ", TI = " << tile_i << ", TV = " << tv << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz
+            << ", RED = " << (red ? 1 : 0)
             << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
           for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
           s << "};\n    return m[i];\n  }\n  static constexpr int slot(int i) {\n    constexpr int m[] = {";
           for (int o = 0; o < nops; ++o) s << slot[o] << (o + 1 < nops ? ", " : "");
-          s << "};\n    return m[i];\n  }\n};\n"
-            << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::EwTrParams<" << e->name
-            << "::NOPS, ThxPlan::ND, ThxPlan::IT> p) {\n  thx::ew_tr_body<" << e->name << ", ThxPlan>(p);\n}\n";
+          s << "};\n    return m[i];\n  }\n};\n";
+          if (red)
+            s << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::EwTrParams<" << e->name
+              << "::NOPS, ThxPlan::ND, ThxPlan::IT> p, thx::EwRedParams<" << R->name << "::NOUT, " << R->name
+              << "::NEX> q) {\n  thx::ew_tr_red_body<" << e->name << ", ThxPlan>(p, q);\n}\n";
+          else
+            s << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::EwTrParams<" << e->name
+              << "::NOPS, ThxPlan::ND, ThxPlan::IT> p) {\n  thx::ew_tr_body<" << e->name << ", ThxPlan>(p);\n}\n";
           rc = get_kernel(s.str(), entry, &k);
           if (rc) return rc;
           e->plans[plan] = k;
         }
-        if (dry) return THX_OK;
         const int64_t ext_t = dm.shape[tdim], ext_i = inner;
         const int64_t tiles_t = (ext_t + tile_t - 1) / tile_t, tiles_i = (ext_i + tile_i - 1) / tile_i;
         int64_t outer = 1;
@@ -314,8 +326,51 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
             odims.push_back(d);
             outer *= dm.shape[d];
           }
-        const int64_t grid = outer * tiles_t * tiles_i;
+        // reducing variant: `groups` blocks share one innermost range and split the other tiles evenly
+        const int64_t rowtiles = outer * tiles_t;
+        int64_t groups = 1;
+        if (red) {
+          const int64_t cus = rt().ready ? rt().cus : 256;
+          const int bpc = std::max(1, env_int("THX_EW_RED_BLOCKS_PER_CU", 6));  // 4 to 6 measured best (partials stay few)
+          const int64_t g0 = std::max<int64_t>(1, std::min(rowtiles, cus * bpc / tiles_i));
+          groups = ceil_div64(rowtiles, ceil_div64(rowtiles, g0));
+        }
+        std::vector<char*> routp;
+        std::vector<uint64_t> rex(1, 0);
+        std::vector<int64_t> rexs(1, 1);
+        if (red) {
+          for (int o = 0; o < R->n_out; ++o) {
+            const thx_array& a = red_outs[o];
+            const int adt = a.dtype & ~THX_REUSED;
+            int64_t count = 1;
+            for (int d = 0; d < a.nd; ++d) count *= a.shape[d];
+            int64_t expect = dtype_size(adt);
+            bool contiguous = true;
+            for (int d = a.nd - 1; d >= 0; --d) {
+              if (a.shape[d] > 1 && a.strides_bytes[d] != expect) contiguous = false;
+              expect *= a.shape[d];
+            }
+            if (adt != R->dtypes[R->n_in + o] || count != ext_i || !contiguous)
+              return fail(THX_ERR_TYPE, "elemwise: reduction result %d must be a C-contiguous array of %lld elements of "
+                          "dtype code %d", o, (long long)ext_i, R->dtypes[R->n_in + o]);
+            routp.push_back((char*)a.base + a.offset_bytes);
+          }
+          if (rowtiles >= (int64_t(1) << 31)) return fail(THX_ERR_UNSUPPORTED, "elemwise: %lld tiles", (long long)rowtiles);
+        }
+        if (dry) {
+          if (red && groups > 1) {
+            rc = reduce_final_pass(R, routp, rex, rexs, nullptr, ext_i, (int)groups, true, false);
+            if (rc) return rc;
+          }
+          if (fused) *fused = red;
+          return THX_OK;
+        }
+        const int64_t grid = red ? groups * tiles_i : outer * tiles_t * tiles_i;
         if (grid * 256 <= 0xffffffffLL) {
+          if (red && groups > 1) {
+            rc = ensure_scratch((size_t)groups * ext_i * R->acc_bytes);
+            if (rc) return rc;
+          }
           ParamPack pk;
           for (int o = 0; o < nops; ++o) pk.put<char*>(views[o].ptr);
           for (int o = 0; o < nops; ++o) pk.put<uint64_t>(views[o].immval);
@@ -329,12 +384,30 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
           for (int o = 0; o < nops; ++o) pk.put<int32_t>((int32_t)dm.stride[o][tdim]);
           for (int o = 0; o < nops; ++o) pk.put<int32_t>((int32_t)dm.stride[o][ND - 1]);
           pk.align(8);
-          return launch(k, e->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
+          if (red) {
+            for (char* q : routp) pk.put<char*>(q);
+            pk.put<uint64_t>(0);   // no further operands of the epilogue
+            pk.put<int64_t>(1);
+            pk.put<char*>(groups > 1 ? rt().scratch : nullptr);
+            pk.put<int32_t>((int32_t)rowtiles);
+            pk.put<int32_t>((int32_t)groups);
+            pk.align(8);
+          }
+          rc = launch(k, e->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
+          if (rc) return rc;
+          if (red && groups > 1) {
+            rc = reduce_final_pass(R, routp, rex, rexs, rt().scratch, ext_i, (int)groups, false, false);
+            if (rc) return rc;
+          }
+          if (fused) *fused = red;
+          return THX_OK;
         }
       }
     }
   }
 
+  if (red_outs && e->red)   // the caller reduces the stored results next: they stay cacheable
+    for (int w : e->red_of) views[e->n_in + w].reused = true;
   const int64_t nvec = ND == 1 ? n / vec : n / vec;
   // One vector per operand and thread: measured with inputs that are not cached, a larger unroll
   // never gains and costs registers (a seven-input float16 kernel needs 164 VGPRs at 4).
@@ -421,6 +494,50 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
   if (grid * block > 0xffffffffLL)
     return fail(THX_ERR_UNSUPPORTED, "elemwise: %lld blocks of %d exceed the work-items of one dispatch", (long long)grid, block);
   return launch(k, e->name + "|" + plan, (unsigned)grid, block, pk.buf.data(), pk.buf.size());
+}
+
+extern "C" {
+
+int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* outs, int flags) {
+  return elemwise_impl(e, ins, outs, nullptr, flags, nullptr);
+}
+
+int thx_elemwise_attach_reduce(thx_elemwise* e, thx_reduce* r, const int32_t* which_outputs) {
+  if (!e || !r || !which_outputs) return fail(THX_ERR_ARG, "thx_elemwise_attach_reduce: null argument");
+  if (r->n_extra) return fail(THX_ERR_UNSUPPORTED, "thx_elemwise_attach_reduce: the reduction's epilogue may take no further operands");
+  for (int i = 0; i < r->n_in; ++i) {
+    const int w = which_outputs[i];
+    if (w < 0 || w >= e->n_out) return fail(THX_ERR_ARG, "thx_elemwise_attach_reduce: output %d of %d", w, e->n_out);
+    if (r->dtypes[i] != e->dtypes[e->n_in + w])
+      return fail(THX_ERR_TYPE, "thx_elemwise_attach_reduce: the reduction reads dtype code %d, output %d has %d",
+                  r->dtypes[i], w, e->dtypes[e->n_in + w]);
+  }
+  e->red = r;
+  e->red_of.assign(which_outputs, which_outputs + r->n_in);
+  return THX_OK;
+}
+
+int thx_elemwise_reduce_call(thx_elemwise* e, const thx_array* ins, const thx_array* outs, const thx_array* red_outs,
+                             int flags) {
+  if (!e || !red_outs) return fail(THX_ERR_ARG, "thx_elemwise_reduce_call: null argument");
+  if (!e->red) return fail(THX_ERR_ARG, "thx_elemwise_reduce_call: no reduction is attached to this operation");
+  bool fused = false;
+  int rc = elemwise_impl(e, ins, outs, red_outs, flags, &fused);
+  if (rc || fused) return rc;
+  // any other plan: the stored results are reduced over every dimension but the last
+  thx_reduce* r = e->red;
+  const int nd = outs[0].nd;
+  if (nd < 1) return fail(THX_ERR_TYPE, "thx_elemwise_reduce_call: results of rank 0 have nothing to reduce");
+  std::vector<thx_array> rin(r->n_in);
+  for (int i = 0; i < r->n_in; ++i) {
+    rin[i] = outs[e->red_of[i]];
+  }
+  uint8_t mask[THX_MAX_ND];
+  for (int d = 0; d < nd; ++d) mask[d] = d < nd - 1;
+  const std::string plan = thx_last_plan();
+  rc = thx_reduce_call(r, rin.data(), mask, red_outs, flags);
+  if (!rc) set_last_plan(plan + " + " + thx_last_plan());
+  return rc;
 }
 
 }  // extern "C"

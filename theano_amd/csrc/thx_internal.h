@@ -6,6 +6,7 @@
 
 #include <cstdint>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "../../include/thx_hip.h"
@@ -119,4 +120,29 @@ uint64_t nt_mask(int nt, const std::vector<View>& views);
 int gather_inputs(const char* what, const thx_array* ins, int n_in, const int32_t* dtypes, int flags,
                   int* nd_out, int64_t* shape, std::vector<View>* views);
 
+}  // namespace thx
+
+// ---- operation handles --------------------------------------------------------
+struct thx_reduce {
+  std::string src, name;
+  int n_in = 0, n_out = 0, n_extra = 0, acc_bytes = 0;
+  std::vector<int32_t> dtypes;
+  std::unordered_map<std::string, thx::Kernel> plans;
+};
+
+struct thx_elemwise {
+  std::string src, name;
+  int n_in = 0, n_out = 0;
+  std::vector<int32_t> dtypes;
+  std::unordered_map<std::string, thx::Kernel> plans;
+  // the reduction attached by thx_elemwise_attach_reduce: its inputs are the outputs red_of[0..] of this operation
+  thx_reduce* red = nullptr;
+  std::vector<int32_t> red_of;
+};
+
+namespace thx {
+// Second pass of a split reduction (merges S partial accumulators per result in slice order and runs the
+// epilogue); S = 0 writes the identity through the epilogue.  `fixed`: nothing that allocates.
+int reduce_final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::vector<uint64_t>& ex,
+                      const std::vector<int64_t>& exs, char* partial, int64_t n_out, int S, bool dry, bool fixed);
 }  // namespace thx

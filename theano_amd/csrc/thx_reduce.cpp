@@ -11,13 +11,6 @@
 
 #include "thx_internal.h"
 
-struct thx_reduce {
-  std::string src, name;
-  int n_in = 0, n_out = 0, n_extra = 0, acc_bytes = 0;
-  std::vector<int32_t> dtypes;
-  std::unordered_map<std::string, thx::Kernel> plans;
-};
-
 namespace thx {
 
 enum { M_VEC = 0, M_BCAST = 1, M_GATHER = 2, M_IMM = 3, M_IOTA = 4 };
@@ -82,8 +75,8 @@ static int not_loaded(const thx_reduce* r, const std::string& plan) {
 }
 
 // `fixed`: the call comes from thx_reduce_call_static - only kernels that are already loaded, no events.
-static int final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::vector<uint64_t>& ex,
-                      const std::vector<int64_t>& exs, char* partial, int64_t n_out, int S, bool dry, bool fixed = false) {
+int reduce_final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::vector<uint64_t>& ex,
+                      const std::vector<int64_t>& exs, char* partial, int64_t n_out, int S, bool dry, bool fixed) {
   const int tpo = final_tpo(n_out);
   const std::string plan = "rf|t" + std::to_string(tpo);
   Kernel k;
@@ -283,7 +276,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
   }
   if (n_red == 0) {  // identity through the epilogue
     set_last_plan(r->name + "|rf|identity");
-    return final_pass(r, outp, ex, exs, nullptr, n_out, 0, dry, fixed);
+    return reduce_final_pass(r, outp, ex, exs, nullptr, n_out, 0, dry, fixed);
   }
 
   // primary input: the one that spans the most memory
@@ -650,7 +643,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     rc = launch(k, r->name + "|" + plan, (unsigned)grid, launch_block, pk.buf.data(), pk.buf.size(), fixed);
     if (rc) return rc;
   }
-  if (S > 1) return final_pass(r, outp, ex, exs, partial, n_out, S, dry, fixed);
+  if (S > 1) return reduce_final_pass(r, outp, ex, exs, partial, n_out, S, dry, fixed);
   return THX_OK;
 }
 

@@ -1,7 +1,7 @@
 """HIP backend: runtime binding, device ops and the rewrites that lift a graph onto them."""
 from .runtime import (HipArray, HipRuntimeError, cache_stats, device_info, dry_run, init, last_plan, profile,  # noqa: F401
                       set_dry_run, sync, timer_start, timer_stop)
-from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipMaxAndArgmax, HipToHost, HostToHip,  # noqa: F401
+from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipElemwiseReduce, HipMaxAndArgmax, HipToHost, HostToHip,  # noqa: F401
                   as_hip_variable,
                   hip_from_host, host_from_hip)
 from . import opt  # noqa: F401

@@ -34,8 +34,12 @@ def _regs(dtypes, names):
         "thx::Vec<%s, V> %s;" % (storage_ctype(dt), nm) for dt, nm in zip(dtypes, names))
 
 
-def elemwise_functor(scalar_op, in_dtypes, out_dtypes=None):
-    """(source, functor name, output dtypes) for an n-ary elementwise op."""
+def elemwise_functor(scalar_op, in_dtypes, out_dtypes=None, red=None):
+    """(source, functor name, output dtypes) for an n-ary elementwise op.
+
+    ``red = (name of a reduction functor, indices of the outputs it reads)``: the functor names
+    that reduction (``Red``) and feeds it, element by element, the results a thread holds
+    (``red_lanes``); the source of the reduction functor must precede this one's."""
     node = _scalar_node(scalar_op, in_dtypes)
     odt = [o.type.dtype for o in node.outputs]
     if out_dtypes is not None and list(out_dtypes) != odt:
@@ -60,6 +64,13 @@ def elemwise_functor(scalar_op, in_dtypes, out_dtypes=None):
                 "    for (int k = 0; k < V; ++k) { %s apply(%s); %s }\n  }" % (decl, call, back))
     body.append("  template <int V, class A> THX_DEV static void store(const A& a, const Regs<V>& r) { %s }" % " ".join(
         "a.template st<%d>(r.%s);" % (nin + k, nm) for k, nm in enumerate(outs)))
+    if red is not None:
+        rname, which = red
+        feed = ", ".join("(%s)r.%s.v[k]" % (compute_ctype(odt[w]), outs[w]) for w in which)
+        body.append("  typedef %s Red;" % rname)
+        body.append("  template <int V, class AccT> THX_DEV static void red_lanes(AccT* acc, const Regs<V>& r) {\n"
+                    "#pragma unroll\n    for (int k = 0; k < V; ++k) { typename Red::Acc t; Red::pre(%s, t); "
+                    "Red::comb(acc[k], t); }\n  }" % feed)
     text = "\n".join(body)
     name = _name("F", text)
     return "struct %s {\n%s\n};\n" % (name, text), name, odt

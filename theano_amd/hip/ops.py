@@ -496,6 +496,111 @@ class HipCAReduce(CAReduce):
             output_storage[k][0] = arr
 
 
+_elemwise_reduce_handles = {}
+
+
+class HipElemwiseReduce(HipElemwise):
+    """An elementwise kernel that also reduces some of its results over every dimension but the last:
+    ``r = f(a, b, ...)`` stored, and ``reduce(r, axis=all but the last)`` alongside, e.g. the per-channel
+    sum of an NHWC result that is an output too.  Outputs: the elementwise results, then one reduction
+    result per entry of ``red_of`` (the index of the elementwise output it reduces).  Where the kernel
+    reads its inputs through LDS tiles (permuted views) the reduction rides along in the same launch
+    and the result is never read back; otherwise the library reduces the stored result.  The
+    reference runs GpuElemwise and GpuCAReduceCuda one after the other
+    (``theano/gpuarray/elemwise.py:376, 1095-1723``)."""
+
+    __props__ = ("scalar_op", "red_of", "red_scalar_ops", "red_acc_dtypes", "red_out_dtypes")
+
+    def __init__(self, scalar_op, red_of, red_scalar_ops, red_acc_dtypes, red_out_dtypes):
+        HipElemwise.__init__(self, scalar_op, None)
+        self.red_of = tuple(int(k) for k in red_of)
+        self.red_scalar_ops = tuple(red_scalar_ops)
+        self.red_acc_dtypes = tuple(red_acc_dtypes)
+        self.red_out_dtypes = tuple(red_out_dtypes)
+
+    def _props(self):
+        return (self.scalar_op, self.red_of, self.red_scalar_ops, self.red_acc_dtypes, self.red_out_dtypes)
+
+    def __str__(self):
+        return "HipElemwiseReduce{%s; %s}" % (self.scalar_op, ", ".join(
+            "%s(out %d)" % (o, k) for o, k in zip(self.red_scalar_ops, self.red_of)))
+
+    def make_node(self, *inputs):
+        base = HipElemwise.make_node(self, *inputs)
+        nd = base.outputs[0].type.ndim
+        if nd < 2:
+            raise TypeError("HipElemwiseReduce needs results of rank 2 or more")
+        last = base.outputs[0].type.broadcastable[-1]
+        outs = [o.type() for o in base.outputs] + [HipArrayType(dt, (last,))() for dt in self.red_out_dtypes]
+        return Apply(self, base.inputs, outs)
+
+    def infer_shape(self, node, shapes):
+        n_ew = len(node.outputs) - len(self.red_of)
+        nd = node.outputs[0].type.ndim
+        full = [max(s[d] for s in shapes if len(s) == nd) for d in range(nd)]
+        return [tuple(full)] * n_ew + [(full[-1],)] * len(self.red_of)
+
+    def _handle(self, node):
+        in_dt = tuple(i.type.dtype for i in node.inputs)
+        key = (self._props(), in_dt)
+        h = _elemwise_reduce_handles.get(key)
+        if h is None:
+            n_ew = len(node.outputs) - len(self.red_of)
+            ew_dt = [o.type.dtype for o in node.outputs[:n_ew]]
+            red_in = tuple(ew_dt[k] for k in self.red_of)
+            K = len(self.red_of)
+            if K == 1:
+                pre = None
+            else:       # several reductions in one functor: input j feeds accumulator j
+                s_in = [scal.Scalar(dt)() for dt in red_in]
+                pre = scal.Composite(s_in, [scal.identity(v) for v in s_in])
+            rsrc, rname, acc_bytes = codegen.reduce_functor(self.red_scalar_ops, self.red_acc_dtypes, red_in,
+                                                            self.red_out_dtypes, pre)
+            fsrc, fname, out_dt = codegen.elemwise_functor(self.scalar_op, in_dt, ew_dt, red=(rname, self.red_of))
+            rcodes = (ctypes.c_int32 * (2 * K))(*[scal.dtype_code(d) for d in red_in + self.red_out_dtypes])
+            rh = ctypes.c_void_p()
+            check(lib.thx_reduce_new(rsrc.encode(), rname.encode(), K, K, 0, rcodes, acc_bytes, ctypes.byref(rh)))
+            codes = (ctypes.c_int32 * (len(in_dt) + n_ew))(*[scal.dtype_code(d) for d in in_dt + tuple(out_dt)])
+            eh = ctypes.c_void_p()
+            check(lib.thx_elemwise_new((rsrc + fsrc).encode(), fname.encode(), len(in_dt), n_ew, codes, ctypes.byref(eh)))
+            check(lib.thx_elemwise_attach_reduce(eh, rh, (ctypes.c_int32 * K)(*self.red_of)))
+            h = _elemwise_reduce_handles[key] = (eh, rh, len(in_dt), n_ew)
+        return h
+
+    def perform(self, node, inputs, output_storage):
+        cache = node.tag.get("thx")
+        if cache is None:
+            eh, rh, nin, n_ew = self._handle(node)
+            K = len(self.red_of)
+            cache = node.tag["thx"] = (eh, nin, n_ew, K, (thx_array * nin)(), (thx_array * n_ew)(), (thx_array * K)(),
+                                       node.outputs[0].type.ndim, [np.dtype(o.type.dtype) for o in node.outputs])
+        eh, nin, n_ew, K, ins, outs, routs, nd, out_dt = cache
+        shape = _check_runtime_broadcast(node.inputs, inputs, nd)
+        for op in self.red_scalar_ops:
+            if 0 in shape[:-1] and isinstance(op, (scal.Maximum, scal.Minimum)):
+                raise ValueError("Input of CAReduce{%s} has zero-size on axis %s" % (op, tuple(range(nd - 1))))
+        for k, v in enumerate(inputs):
+            if type(v) is HipArray:
+                v.as_thx(ins[k])
+            else:
+                host_scalar_thx(v, nd, ins[k])
+        results = []
+        for k in range(n_ew):
+            arr = HipArray._new_contiguous(shape, out_dt[k])
+            arr.as_thx(outs[k])
+            results.append(arr)
+        for k in range(K):
+            arr = HipArray._new_contiguous((shape[-1],), out_dt[n_ew + k])
+            arr.as_thx(routs[k])
+            results.append(arr)
+        mark_reused(node, ins, outs)
+        rc = lib.thx_elemwise_reduce_call(eh, ins, outs, routs, call_flags(node))
+        if rc:
+            check(rc)
+        for k, arr in enumerate(results):
+            output_storage[k][0] = arr
+
+
 _argmax_handles = {}
 
 

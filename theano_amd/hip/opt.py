@@ -20,7 +20,8 @@ from ..tensor import basic as T
 from ..tensor.elemwise import All, Any, CAReduce, CAReduceDtype, DimShuffle, Elemwise
 from ..tensor.type import TensorConstant, TensorType
 from . import views as hip_views
-from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipMaxAndArgmax, HipToHost, HostToHip,
+from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipElemwiseReduce, HipMaxAndArgmax, HipToHost,
+                  HostToHip,
                   _is_host_scalar, as_hip_variable, hip_from_host, host_from_hip)
 
 
@@ -789,6 +790,47 @@ def inplace_elemwise(fgraph):
     return count
 
 
+def fuse_reduction_of_stored_result(fgraph):
+    """An elementwise result that something else needs as well (it is an output, say) and a plain reduction
+    of it over every dimension but the last - the per-channel sum of an NHWC result - become one node,
+    whose kernel accumulates while it stores wherever its access plan allows (``HipElemwiseReduce``).  Runs
+    after every other fusion pass: those would have folded the elementwise node into the reduction had
+    nothing else read it."""
+    count = 0
+    for red in fgraph.toposort():
+        op = red.op
+        if (type(op) is not HipCAReduce or red not in fgraph.apply_nodes or op.pre_scalar_op is not None or
+                op.post_scalar_op is not None or len(op.scalar_ops) != 1 or len(red.inputs) != 1):
+            continue
+        x = red.inputs[0]
+        ew = x.owner
+        if ew is None or type(ew.op) is not HipElemwise or ew.op.inplace_pattern:
+            continue
+        nd = x.type.ndim
+        if nd < 2 or op.axis != tuple(range(nd - 1)) or any(x.type.broadcastable[:-1]):
+            continue
+        if isinstance(op.scalar_ops[0], (scal.Maximum, scal.Minimum)) or codegen_identity(op.scalar_ops[0]) is None:
+            continue            # the zero-length error of max / min stays with the plain reduction
+        new_op = HipElemwiseReduce(ew.op.scalar_op, (ew.outputs.index(x),), op.scalar_ops, op.acc_dtypes, op.out_dtypes)
+        new = new_op.make_node(*ew.inputs)
+        n_ew = len(ew.outputs)
+        if [o.type for o in new.outputs] != [o.type for o in ew.outputs] + [red.outputs[0].type]:
+            continue
+        for o, no in zip(ew.outputs, new.outputs[:n_ew]):
+            fgraph.replace(o, no)
+        fgraph.replace(red.outputs[0], new.outputs[n_ew])
+        count += 1
+    return count
+
+
+def codegen_identity(scalar_op):
+    from .codegen import reduce_identity
+    try:
+        return reduce_identity(scalar_op, "int64")
+    except Exception:
+        return None
+
+
 def optimize(fgraph, fuse=True, rowchain=True, inplace=True):
     """Full pipeline: clean up, lift, fuse, then in-place."""
     from ..tensor.opt import canonicalize
@@ -801,6 +843,7 @@ def optimize(fgraph, fuse=True, rowchain=True, inplace=True):
             from .rowchain import fuse_row_chains
             fuse_row_chains(fgraph)
         fuse_around_reductions(fgraph)
+        fuse_reduction_of_stored_result(fgraph)
     if inplace:
         inplace_elemwise(fgraph)
     return fgraph

@@ -63,6 +63,9 @@ def _load():
         "thx_elemwise_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, P(i32), P(vp)], ctypes.c_int),
         "thx_elemwise_call": ([vp, P(thx_array), P(thx_array), ctypes.c_int], ctypes.c_int),
         "thx_elemwise_free": ([vp], ctypes.c_int),
+        "thx_elemwise_attach_reduce": ([vp, vp, P(i32)], ctypes.c_int),
+        "thx_elemwise_reduce_call": ([vp, P(thx_array), P(thx_array), P(thx_array), ctypes.c_int], ctypes.c_int),
+        "thx_reduce_call_static": ([vp, P(thx_array), P(ctypes.c_uint8), P(thx_array), ctypes.c_int], ctypes.c_int),
         "thx_reduce_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, P(i32),
                             ctypes.c_int, P(vp)], ctypes.c_int),
         "thx_reduce_call": ([vp, P(thx_array), P(ctypes.c_uint8), P(thx_array), ctypes.c_int], ctypes.c_int),
