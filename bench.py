@@ -27,18 +27,26 @@ import time
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch from hardware counters (rocprofv3 --pmc FETCH_SIZE, then WRITE_SIZE, each
-# scaled by what the same counter reads for the --copy-probe kernel of known size), by kernel family
-# and functor (the rest of a kernel symbol spells tuning choices that do not change its traffic).
-MEASURED_TRAFFIC = {
-    # sum(axis=1) of float32 (8192, 8192): FETCH_SIZE 131091.1 x 1.99980 KiB + WRITE_SIZE 256.4 x 0.99888 KiB
-    "rr:Ra004ded952553fcd": 268709742,
-}
+TRAFFIC_SUMMARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "all_configs_hbm_traffic.txt")
 
 
-def _traffic(symbol):
-    parts = symbol.split("_")
-    return MEASURED_TRAFFIC.get("%s:%s" % (parts[1], parts[-1]))
+def _traffic(symbol, grid=None):
+    """HBM bytes per launch of the kernel `symbol` as the hardware counters measured them (rocprofv3 --pmc
+    FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads for the --copy-probe kernel of
+    known size): read from the tracked summary of those runs, whose table lines are
+    `<kernel symbol> <grid> <launches> <FETCH_SIZE> <WRITE_SIZE> <HBM bytes> ...`.  None, with a warning,
+    when the summary has no line for this kernel (its text changed since the counters were taken)."""
+    try:
+        with open(TRAFFIC_SUMMARY) as f:
+            rows = [l.split() for l in f if l.startswith("thx_")]
+    except OSError:
+        rows = []
+    hits = [r for r in rows if r[0] == symbol and len(r) >= 6 and (grid is None or r[1] == str(grid))]
+    if not hits:
+        sys.stderr.write("bench.py: no measured HBM traffic for %s in %s; roofline.traffic is null\n"
+                         % (symbol, os.path.relpath(TRAFFIC_SUMMARY)))
+        return None
+    return int(float(hits[0][5]))
 
 
 def _device_function(th, W, graph, vals):
@@ -220,7 +228,7 @@ def main():
     per_launch = 8192 * 8192 * 4 + 8192 * 4   # bytes one launch of a row / column reduction moves by definition
     achieved = per_launch / (dom_avg_us * 1e-6) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": _traffic(dom),
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": _traffic(dom, 8192 * 256),
                 "kernel": dom, "avg_launch_us": round(dom_avg_us, 2), "uncached_input_us": cold_us,
                 "same_input_us": warm_us, "algorithmic_bytes_per_launch": per_launch}
 
@@ -262,6 +270,11 @@ def main():
 
     cpu = None if args.no_cpu else _cpu_baseline_c2(W)
 
+    # the weakest timed workload, next to the headline
+    fracs = dict(("c2_" + k, v["frac_of_peak"]) for k, v in per_case.items())
+    fracs.update((k, v["frac_of_peak"]) for k, v in others.items())
+    worst = min(fracs, key=fracs.get)
+
     line = {
         "metric": "achieved HBM GB/s and % of peak for fused Elemwise+CAReduce at 1 MI355X",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -273,7 +286,9 @@ def main():
                                "sum all axes, prod axis=1; one step = the five reductions",
                    "algorithmic_bytes_per_step": total_bytes, "device": info["arch"],
                    "compute_units": info["compute_units"]},
-        "roofline": roofline, "cpu_baseline": cpu, "per_reduction": per_case, "other_configs": others,
+        "roofline": roofline, "cpu_baseline": cpu,
+        "worst_config": {"name": worst, "frac": fracs[worst], "us": (per_case.get(worst[3:]) or others.get(worst))["us"]},
+        "per_reduction": per_case, "other_configs": others,
     }
     print(json.dumps(line))
 

@@ -104,6 +104,27 @@ def test_strided_views_zero_extents_and_errors():
     assert np.array_equal(mv, [7, 15, 23]) and np.array_equal(iv, [7, 7, 7])
 
 
+def test_lowest_values_everywhere_and_walks_that_do_not_follow_positions():
+    """A thread keeps the first of equal values without comparing positions where positions only grow along its walk;
+    where they do not (reduced dimensions of a transposed view, walked by stride) the full rule applies.  An
+    accumulator that nothing ever beat - every element is the lowest value of its type - answers position 0."""
+    rng = np.random.default_rng(37)
+    for dtype, low in (("int8", -128), ("uint8", 0), ("int32", -2 ** 31), ("float32", -np.inf), ("float16", -np.inf)):
+        m = T.TensorType(dtype, (False, False))("m")
+        val = np.full((70, 5000), low, dtype)
+        val[5, 4000:] = 1                                   # one row with something above the lowest value
+        for ax in (0, 1, None):
+            got, ref, plan = run(m, T.max_and_argmax(m, axis=ax), val)
+            same(got, ref, "all lowest %s axis %s [%s]" % (dtype, ax, plan))
+    t = T.ftensor3("t")
+    val = rng.integers(-2, 3, (37, 41, 43)).astype("float32")
+    for order in ((2, 1, 0), (1, 0, 2), (0, 2, 1), (2, 0, 1)):
+        for axes in ((0, 1), (1, 2), (0, 2), (0, 1, 2), (1,)):
+            out = T.max_and_argmax(t.dimshuffle(*order), axis=list(axes))
+            got, ref, plan = run(t, out, val)
+            same(got, ref, "transposed %s axes %s [%s]" % (order, axes, plan))
+
+
 def test_argmax_through_the_generic_reduction_form():
     """Three reduced dimensions that do not collapse (axes 0, 2, 4 of a 6-d array) take the generic
     kernel, where the position operand is computed from a full index decomposition; ties and NaNs included."""

@@ -335,6 +335,56 @@ def test_stored_elementwise_result_and_its_reduction_over_all_but_the_last_axis(
     assert e[0].shape == (0, 5) and np.array_equal(e[1], np.zeros(5, "float32"))
 
 
+def test_split_any_all_finish_in_one_launch():
+    """any / all over long reduce domains: the slices of a split reduction settle the result through one
+    atomic add each on a single word per result (plan suffix 'tk'), which the last slice puts back to zero.
+    Row and column forms, one and several results, every combination of answers, and the same function
+    called again and again with inputs whose answers differ (a word left dirty would show at once)."""
+    rng = np.random.default_rng(30)
+    x = T.imatrix("x")
+    both = th.function([x], [T.any(x > 0), T.all(x > 0), T.any(x > 5)])
+    rows = th.function([x], [T.any(x > 0, axis=1), T.all(x > 0, axis=1)])
+    cols = th.function([x], [T.any(x > 0, axis=0), T.all(x > 0, axis=0)])
+    base = rng.integers(1, 5, (3000, 2048)).astype("int32")          # all positive, none above 5
+    variants = []
+    for kind in range(4):
+        v = base.copy()
+        if kind in (1, 3):
+            v[rng.integers(0, 3000), rng.integers(0, 2048)] = -7      # all(x > 0) turns false
+        if kind in (2, 3):
+            v[2999, 2047] = 9                                         # any(x > 5) turns true, in the last slice
+        variants.append(v)
+    variants.append(-base)                                            # nothing positive at all
+    for rep in range(2):
+        for v in variants:
+            got = both(v)
+            assert "|tk|" in hip.last_plan() and "|s" in hip.last_plan().split("|m")[-1], hip.last_plan()
+            assert [bool(g) for g in got] == [bool((v > 0).any()), bool((v > 0).all()), bool((v > 5).any())]
+    wide = rng.integers(-3, 4, (4, 1 << 20)).astype("int32")
+    wide[1] = np.abs(wide[1]) + 1
+    wide[2] = -np.abs(wide[2])
+    for _ in range(2):
+        a, b = rows(wide)
+        assert "|tk|" in hip.last_plan(), hip.last_plan()
+        assert np.array_equal(a, (wide > 0).any(axis=1)) and np.array_equal(b, (wide > 0).all(axis=1))
+    tall = rng.integers(-3, 4, (200000, 8)).astype("int32")
+    tall[:, 1] = np.abs(tall[:, 1]) + 1
+    tall[:, 2] = -np.abs(tall[:, 2])
+    for _ in range(2):
+        a, b = cols(tall)
+        assert "|tk|" in hip.last_plan() and "|rc|" in hip.last_plan(), hip.last_plan()
+        assert np.array_equal(a, (tall > 0).any(axis=0)) and np.array_equal(b, (tall > 0).all(axis=0))
+    # the two-launch form gives the same answers
+    import os
+    os.environ["THX_RED_TICKET"] = "0"
+    try:
+        got = both(variants[3])
+        assert "|tk|" not in hip.last_plan()
+        assert [bool(g) for g in got] == [True, False, True]
+    finally:
+        del os.environ["THX_RED_TICKET"]
+
+
 def test_epilogue_chain_with_per_result_device_operands():
     """Per-channel algebra after a reduction (other per-channel arrays, results
     of an earlier reduction, host scalars) runs in the reduction's epilogue;

@@ -17,6 +17,17 @@
 // merges them in slice order, so results are reproducible run to run. (Merging
 // inside the first launch by the last block to arrive was measured slower on
 // gfx950: the device-scope release each block needs costs more than a launch.)
+//
+// Functors whose accumulators are all boolean (any / all) may instead supply
+//   static unsigned long long ticket_pack(const Acc&);   // one count per accumulator, 16 bits each
+//   static Acc ticket_unpack(unsigned long long);
+// and plans with TICKET = 1 then finish in the first launch: every slice adds its packed flags plus
+// 1 << 48 to ONE 64-bit word per output with a single atomic add.  That word is the only object
+// shared between the slices, so the atomic operation's own total order decides everything: the
+// slice that reads S - 1 in the count field has, in the value the add returned, the contributions of
+// all the others, writes the result and puts the word back to zero for the next launch.  No fence,
+// no partials, no second launch; counts of true / false flags are order-free, so the result is
+// reproducible.
 #pragma once
 
 namespace thx {
@@ -36,6 +47,18 @@ struct RedOut {
 // the vectorised dimension. TPR threads cooperate on one output; a block holds
 // BLOCK / TPR outputs. Covers trailing-axis reductions, whole-array reductions
 // (one output, many slices) and outer x kept x inner patterns (RA > 1).
+// The slice holding `tot` for output `o` checks in; the last one to do so writes the result.
+// `words`: one zero word per output, zero again when the kernel ends.
+template <class R, class O>
+THX_DEV void ticket_finish(const O& out, unsigned long long* words, long long o, int S, const typename R::Acc& tot) {
+  const unsigned long long mine = R::ticket_pack(tot) + (1ull << 48);
+  const unsigned long long before = __hip_atomic_fetch_add(words + o, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if ((int)(before >> 48) == S - 1) {
+    R::post(out, o, R::ticket_unpack(before + mine));
+    __hip_atomic_store(words + o, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
 template <int NIN, int NOUT, int NEX, int NK, class IT>
 struct RowParams {
   char* in[NIN];
@@ -93,7 +116,7 @@ struct RedAcc {
   }
 };
 
-// Plan members: typedef IT; enum { NK, VEC, UNR, NACC, BLOCK, TPR, RA2 (1 when RA > 1) };
+// Plan members: typedef IT; enum { NK, VEC, UNR, NACC, BLOCK, TPR, RA2 (1 when RA > 1), TICKET };
 // static constexpr int mode(int input); static constexpr int sclass(int input, int which).
 template <class P, class IT>
 THX_DEV IT red_term(int input, int which, IT coord, IT stride) {
@@ -185,8 +208,12 @@ __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, R:
     if (live && t == 0) R::post(p.out, o, tot);
     return;
   }
-  Acc* part = (Acc*)p.partial;
-  if (live && t == 0) part[(long long)s * p.n_out + o] = tot;
+  if constexpr (P::TICKET != 0) {
+    if (live && t == 0) ticket_finish<R>(p.out, (unsigned long long*)p.partial, o, p.S, tot);
+  } else {
+    Acc* part = (Acc*)p.partial;
+    if (live && t == 0) part[(long long)s * p.n_out + o] = tot;
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -217,7 +244,7 @@ struct ColParams {
 };
 
 // Plan members: typedef IT; enum { NK, VEC, UNR, BLOCK, TX, RR2 (1 when two
-// reduced dimensions remain after collapsing) }; mode(int).
+// reduced dimensions remain after collapsing), TICKET }; mode(int).
 template <class R, class P>
 __device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p) {
   typedef typename P::IT IT;
@@ -302,6 +329,8 @@ __device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, R:
       const long long o = a_idx * p.cols + col;
       if (p.S == 1) {
         R::post(p.out, o, tot);
+      } else if constexpr (P::TICKET != 0) {
+        ticket_finish<R>(p.out, (unsigned long long*)p.partial, o, p.S, tot);
       } else {
         part[(long long)s * p.n_out + o] = tot;
       }

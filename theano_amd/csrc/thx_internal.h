@@ -11,6 +11,8 @@
 
 #include "../../include/thx_hip.h"
 
+#define THX_TICKET_WORDS 4096
+
 namespace thx {
 
 // ---- errors ---------------------------------------------------------------
@@ -38,6 +40,8 @@ struct Runtime {
   // Device address of the library's fixed scratch array on `device` (thx_reduce_call_static),
   // resolved once in thx_init; null until then.
   char* static_scratch = nullptr;
+  // Device address of THX_TICKET_WORDS zero words for reductions that finish with one atomic add per slice.
+  char* ticket_words = nullptr;
 };
 Runtime& rt();
 int ensure_init();
@@ -128,6 +132,7 @@ struct thx_reduce {
   int n_in = 0, n_out = 0, n_extra = 0, acc_bytes = 0;
   std::vector<int32_t> dtypes;
   std::unordered_map<std::string, thx::Kernel> plans;
+  bool has_ticket = false;  // the functor packs its accumulators into counts (ticket_pack / ticket_unpack)
 };
 
 struct thx_elemwise {

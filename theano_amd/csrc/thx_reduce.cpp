@@ -151,6 +151,7 @@ int thx_reduce_new(const char* functor_src, const char* functor_name, int n_in, 
   r->n_extra = n_extra;
   r->acc_bytes = acc_bytes;
   r->dtypes.assign(dtypes, dtypes + n_in + n_out + n_extra);
+  r->has_ticket = r->src.find("ticket_pack") != std::string::npos;
   *out = r;
   return THX_OK;
 }
@@ -354,6 +355,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
   int S = 1;
   int launch_block = block;
   char* partial = nullptr;  // Acc[S][n_out] of a split reduction
+  bool one_launch = false;  // the slices settle the result among themselves (ticket_finish)
 
   if (form == ROW) {
     const int64_t RC = NR ? RD.back().extent : 1;
@@ -386,7 +388,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     const int64_t nvec = RA * RC / vec;
     int tpr = nvec >= 512 ? 256 : nvec >= 64 ? 64 : nvec >= 16 ? 16 : nvec >= 4 ? 4 : 1;
     const int force_tpr = env_int("THX_RED_TPR", 0);
-    if (force_tpr > 0) tpr = force_tpr;
+    if (force_tpr > 0 && force_tpr <= 256 && (force_tpr & (force_tpr - 1)) == 0) tpr = force_tpr;
     const int64_t per_thread = ceil_div(nvec, tpr);
     int unr = per_thread >= 4 ? 4 : per_thread >= 2 ? 2 : 1;
     const int force_unr = env_int("THX_RED_UNR", 0);
@@ -399,20 +401,36 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       rblock = 1024;
       tpr = 1024;
     }
+    const bool bigblock = rblock == 1024;
+    // a split reduction of one (or very few) results with larger blocks: fewer slices for the same number of waves
+    const int split_threads = env_int("THX_RED_SPLIT_THREADS", 0);
+    if (!bigblock && tpr == 256 && (split_threads == 512 || split_threads == 1024) && n_out * 2 <= target_row)
+      rblock = tpr = split_threads;
+    // Slices that settle the result with one atomic add each (any / all) queue up on one word: few, large
+    // slices - one block of 1024 threads per compute unit - keep that queue short (19.2 us against 21.8 us
+    // with two blocks of 256 per unit for the (64, 128, 56, 56) int32 any + all; 20.5 us with a second launch).
+    int64_t want_blocks = target_row;
+    if (!bigblock && tpr == 256 && !split_threads && r->has_ticket && n_out <= THX_TICKET_WORDS && n_out * 2 <= cus &&
+        env_int("THX_RED_TICKET", 1) && !bpc) {
+      rblock = tpr = 1024;
+      want_blocks = cus;
+    }
     const int force_nacc = env_int("THX_RED_NACC", 0);
     if (force_nacc > 0) nacc = force_nacc;
     if (nacc > unr) nacc = unr;
     const int rpb = rblock / tpr;
     const int64_t oblocks = ceil_div(n_out, rpb);
     int64_t chunk = nvec;
-    if (rblock == 256 && oblocks * 2 <= target_row && nvec >= (int64_t)tpr * unr * 4) {
-      int64_t want = std::min(ceil_div(target_row, oblocks), nvec / ((int64_t)tpr * unr * 2));
+    if (!bigblock && oblocks * 2 <= want_blocks && nvec >= (int64_t)tpr * unr * 4) {
+      int64_t want = std::min(ceil_div(want_blocks, oblocks), nvec / ((int64_t)tpr * unr * 2));
       if (want > 1) {
         chunk = round_up(ceil_div(nvec, want), (int64_t)tpr * unr);
         S = (int)ceil_div(nvec, chunk);
       }
     }
     if (ra2 && nvec >= (int64_t(1) << 31) - 65536) wide = true;
+    const bool ticket = S > 1 && r->has_ticket && n_out <= THX_TICKET_WORDS && S < 65536 && env_int("THX_RED_TICKET", 1);
+    one_launch = ticket;
     const int NK = std::max(1, NKD);
     std::vector<std::array<int, 2>> sclass(NIN);
     std::string skey;
@@ -423,7 +441,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       skey += char('0' + sclass[i][1]);
     }
     std::ostringstream key;
-    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nacc != unr ? "|c" + std::to_string(nacc) : "") << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << "|m";
+    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nacc != unr ? "|c" + std::to_string(nacc) : "") << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -435,7 +453,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"NACC", nacc}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}}, mode, nt, sclass)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"NACC", nacc}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"TICKET", ticket ? 1 : 0}}, mode, nt, sclass)
         << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void " << entry << "(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -444,8 +462,12 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       r->plans[plan] = k;
     }
     if (!dry && S > 1) {
-      rc = partial_buffer(r, (size_t)S * n_out * r->acc_bytes, n_out, fixed, &partial);
-      if (rc) return rc;
+      if (ticket) {
+        partial = rt().ticket_words;
+      } else {
+        rc = partial_buffer(r, (size_t)S * n_out * r->acc_bytes, n_out, fixed, &partial);
+        if (rc) return rc;
+      }
     }
     for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
@@ -540,8 +562,10 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
         S = (int)ceil_div(rows, rps);
       }
     }
+    const bool ticket = S > 1 && r->has_ticket && n_out <= THX_TICKET_WORDS && S < 65536 && env_int("THX_RED_TICKET", 1);
+    one_launch = ticket;
     std::ostringstream key;
-    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << (cblock != 256 ? "|b" + std::to_string(cblock) : "") << "|r" << rr2 << (nt ? "|nt" + std::to_string(nt) : "") << "|m";
+    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << (cblock != 256 ? "|b" + std::to_string(cblock) : "") << "|r" << rr2 << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -553,7 +577,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", cblock}, {"TX", tx}, {"RR2", rr2}}, mode, nt)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", cblock}, {"TX", tx}, {"RR2", rr2}, {"TICKET", ticket ? 1 : 0}}, mode, nt)
         << "extern \"C\" __global__ __launch_bounds__(" << cblock << ") void " << entry << "(thx::ColParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_col_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -562,8 +586,12 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       r->plans[plan] = k;
     }
     if (!dry && S > 1) {
-      rc = partial_buffer(r, (size_t)S * n_out * r->acc_bytes, n_out, fixed, &partial);
-      if (rc) return rc;
+      if (ticket) {
+        partial = rt().ticket_words;
+      } else {
+        rc = partial_buffer(r, (size_t)S * n_out * r->acc_bytes, n_out, fixed, &partial);
+        if (rc) return rc;
+      }
     }
     for (int i = 0; i < NIN; ++i) pk.put<char*>(views[i].ptr);
     for (int i = 0; i < NIN; ++i) pk.put<uint64_t>(views[i].immval);
@@ -643,7 +671,8 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     rc = launch(k, r->name + "|" + plan, (unsigned)grid, launch_block, pk.buf.data(), pk.buf.size(), fixed);
     if (rc) return rc;
   }
-  if (S > 1) return reduce_final_pass(r, outp, ex, exs, partial, n_out, S, dry, fixed);
+  if (S > 1 && !one_launch)
+    return reduce_final_pass(r, outp, ex, exs, partial, n_out, S, dry, fixed);
   return THX_OK;
 }
 

@@ -27,6 +27,11 @@
 // local, and the runtime, which finds the array by name, aborts in hipGetSymbolAddress.)
 static __device__ __align__(256) unsigned char scratch[THX_STATIC_SCRATCH_BYTES];
 
+// One 64-bit word per result for reductions that finish through a single atomic add per slice
+// (kernels/thx_reduce.h, ticket_finish).  Zero when the library is loaded; every kernel that uses
+// the words leaves them zero.  Resolved like `scratch`.
+static __device__ __align__(256) unsigned long long ticket_words[THX_TICKET_WORDS];
+
 namespace thx {
 
 // ---------------------------------------------------------------------------
@@ -64,6 +69,7 @@ static std::unordered_map<void*, size_t> g_live;
 
 enum { kMaxDevices = 64 };
 static char* g_static_scratch[kMaxDevices] = {nullptr};  // device address of `scratch`, per device
+static char* g_ticket_words[kMaxDevices] = {nullptr};    // device address of `ticket_words`, per device
 
 // profiling
 struct ProfRec {
@@ -97,6 +103,15 @@ static int init_locked(int device) {
     g_static_scratch[device] = (char*)p;
   }
   r.static_scratch = g_static_scratch[device];
+  if (!g_ticket_words[device]) {
+    void* p = nullptr;
+    hipError_t se = hipGetSymbolAddress(&p, HIP_SYMBOL(ticket_words));
+    if (se != hipSuccess || !p)
+      return fail(THX_ERR_HIP, "thx_init: hipGetSymbolAddress(ticket_words) failed on device %d: %s", device,
+                  hipGetErrorString(se));
+    g_ticket_words[device] = (char*)p;
+  }
+  r.ticket_words = g_ticket_words[device];
   hipDeviceProp_t prop;
   THX_HIP_CHECK(hipGetDeviceProperties(&prop, device));
   r.device = device;

@@ -236,6 +236,14 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
                                for k, (dt, t) in enumerate(zip(out_dtypes, tmp)))
     lines.append("  template <class O> THX_DEV static void post(const O& o, long long idx, const Acc& a) {\n%s\n  }"
                  % _indent(post_stmt, 4))
+    # any / all: the slices of a split reduction settle the result with one atomic add each (thx_reduce.h)
+    if K <= 3 and all(dt == "bool" and isinstance(op, (scal.OR, scal.AND)) for op, dt in zip(scalar_ops, acc_dtypes)):
+        pack = " | ".join("((unsigned long long)(%sa.a%d ? 1 : 0) << %d)" % ("" if isinstance(op, scal.OR) else "!", k, 16 * k)
+                          for k, op in enumerate(scalar_ops))
+        unpack = " ".join("a.a%d = ((w >> %d) & 0xffffull) %s 0;" % (k, 16 * k, "!=" if isinstance(op, scal.OR) else "==")
+                          for k, op in enumerate(scalar_ops))
+        lines.append("  THX_DEV static unsigned long long ticket_pack(const Acc& a) { return %s; }" % pack)
+        lines.append("  THX_DEV static Acc ticket_unpack(unsigned long long w) { Acc a; %s return a; }" % unpack)
     text = "\n".join(lines)
     name = _name("R", text)
     return "struct %s {\n%s\n};\n" % (name, text), name, acc_struct_bytes(acc_dtypes)
