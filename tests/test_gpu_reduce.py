@@ -65,6 +65,39 @@ def test_shapes_and_masks(shape, mask):
     check(xi, xi.sum(axis=axis), vi, "int16 sum %s %s" % (shape, mask))
 
 
+def _reference_gpu_table():
+    import json
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "gpu_reduce_cases.json")) as f:
+        d = json.load(f)
+    return [(tuple(s), None if a is None else tuple(a), False) for s, a in d["cases"]] + [
+        (tuple(s), None if a is None else tuple(a), True) for s, a in d["reference_skips"]]
+
+
+@pytest.mark.parametrize("which", ["float32", "int64"])
+def test_reference_gpu_shape_and_mask_table(which):
+    """Every entry of the reference's GPU reduction table (theano/gpuarray/tests/test_elemwise.py:266-346: shapes
+    with an extent above 4096 in each position x every reduce mask, degenerate and empty extents), and the
+    entries it leaves out because GpuCAReduceCuda has no kernel for the mask - sum and max (min, prod for the
+    small ones) against the oracle; float32 and int64 as there."""
+    rng = np.random.default_rng(33)
+    for shape, axis, skipped in _reference_gpu_table():
+        x = T.TensorType(which, [s == 1 for s in shape])("x")
+        n = int(np.prod(shape, dtype="int64"))
+        v = (rng.standard_normal(shape).astype("float32") if which == "float32"
+             else rng.integers(-2 ** 40, 2 ** 40, shape).astype("int64"))
+        red = [shape[a] for a in (range(len(shape)) if axis is None else axis)]
+        names = ["sum", "max"] + (["min", "prod"] if n <= 4096 else [])
+        for name in names:
+            out = REDUCERS[name](x, axis)
+            if 0 in red and name in ("max", "min"):
+                with pytest.raises(ValueError):
+                    th.function([x], out)(v)
+                continue
+            vv = (v % 7 - 3) if (name == "prod" and which == "int64") else v
+            check(x, out, vv, "%s %s %s %s%s" % (name, which, shape, axis, " (not in the reference's run)" if skipped else ""))
+
+
 @pytest.mark.parametrize("dtype", ["bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64",
                                    "float16", "float32", "float64"])
 def test_dtype_coverage(dtype):
@@ -383,6 +416,40 @@ def test_split_any_all_finish_in_one_launch():
         assert [bool(g) for g in got] == [True, False, True]
     finally:
         del os.environ["THX_RED_TICKET"]
+
+
+def test_more_work_than_one_dispatch_holds_is_strided_over_the_blocks(monkeypatch):
+    """A dispatch carries at most 2^32 - 1 work-items.  Reductions with more (block of results) x (slice) pieces
+    than that take the striding kernels (plan suffix 'gs'), in which a block handles pieces blockIdx.x,
+    blockIdx.x + gridDim.x, ...  The limit is lowered here so that arrays of ordinary size reach them: row, column
+    and generic forms, a second result, an argmax and a NaN in the last piece."""
+    monkeypatch.setenv("THX_RED_MAX_DISPATCH", "4096")
+    rng = np.random.default_rng(41)
+    x = T.fmatrix("x")
+    val = rng.standard_normal((5000, 96)).astype("float32")
+    val[4999, 95] = np.nan
+    for axis, form in ((1, "|rr|"), (0, "|rc|")):
+        outs = [T.sum(x, axis=axis), T.max(x, axis=axis)]
+        got = th.function([x], outs)(val)
+        assert form in hip.last_plan() and "|gs|" in hip.last_plan(), hip.last_plan()
+        ref = G.evaluate([x], outs, [val])
+        assert np.allclose(got[0], ref[0], rtol=1e-6, atol=1e-6, equal_nan=True)
+        assert np.array_equal(got[1], ref[1], equal_nan=True)
+        mv, iv = th.function([x], T.max_and_argmax(x, axis=axis))(val)
+        assert "|gs|" in hip.last_plan(), hip.last_plan()
+        ref_m, ref_i = G.max_and_argmax(val, (axis,))
+        assert np.array_equal(mv, ref_m, equal_nan=True) and np.array_equal(iv, ref_i)
+    wide = rng.standard_normal((3, 70000)).astype("float32")          # few results: still split into slices
+    got = th.function([x], T.sum(x, axis=1))(wide)
+    assert np.allclose(got, wide.astype("float64").sum(axis=1), rtol=1e-6)
+    tall = rng.integers(-9, 9, (70000, 40)).astype("float32")
+    got = th.function([x], [T.sum(x, axis=0), T.min(x, axis=0)])(tall)
+    assert np.array_equal(got[0], tall.sum(axis=0)) and np.array_equal(got[1], tall.min(axis=0))
+    t6 = T.TensorType("int32", (False,) * 6)("t6")
+    v6 = rng.integers(-100, 100, (3, 14, 5, 16, 7, 12)).astype("int32")
+    got = th.function([t6], T.sum(t6, axis=(0, 2, 4)))(v6)
+    assert "|rg|" in hip.last_plan() and "|gs|" in hip.last_plan(), hip.last_plan()
+    assert got.dtype == np.int64 and np.array_equal(got, v6.sum(axis=(0, 2, 4)))
 
 
 def test_epilogue_chain_with_per_result_device_operands():

@@ -66,6 +66,7 @@ struct RowParams {
   RedOut<NOUT, NEX> out;
   char* partial;          // Acc[S][n_out] when S > 1
   long long n_out;
+  long long nblocks;      // blocks of work; more than the grid holds when the plan strides (GS)
   long long nvec;         // vectors in one output's reduce domain (RA * RC / VEC)
   long long chunk;        // vectors per slice
   int S;                  // slices per output
@@ -116,15 +117,32 @@ struct RedAcc {
   }
 };
 
-// Plan members: typedef IT; enum { NK, VEC, UNR, NACC, BLOCK, TPR, RA2 (1 when RA > 1), TICKET };
+// Plan members: typedef IT; enum { NK, VEC, UNR, NACC, BLOCK, TPR, RA2 (1 when RA > 1), TICKET, GS };
 // static constexpr int mode(int input); static constexpr int sclass(int input, int which).
 template <class P, class IT>
 THX_DEV IT red_term(int input, int which, IT coord, IT stride) {
   return P::sclass(input, which) == 0 ? (IT)0 : (P::sclass(input, which) == 1 ? coord : coord * stride);
 }
 
+// A dispatch carries at most 2^32 - 1 work-items: plans with GS = 1 launch fewer blocks than there is
+// work and every block takes the pieces blockIdx.x, blockIdx.x + gridDim.x, ...
+template <class R, class P>
+__device__ __forceinline__ void red_row_block(const RowParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p, long long bid);
+
 template <class R, class P>
 __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p) {
+  if constexpr (P::GS != 0) {
+    for (long long b = blockIdx.x; b < p.nblocks; b += gridDim.x) {
+      red_row_block<R, P>(p, b);
+      __syncthreads();
+    }
+  } else {
+    red_row_block<R, P>(p, blockIdx.x);
+  }
+}
+
+template <class R, class P>
+__device__ __forceinline__ void red_row_block(const RowParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p, long long bid) {
   typedef typename P::IT IT;
   typedef typename UnsignedOf<IT>::type UT;
   typedef typename R::Acc Acc;
@@ -132,7 +150,6 @@ __device__ __forceinline__ void red_row_body(const RowParams<R::NIN, R::NOUT, R:
   constexpr int RPB = P::BLOCK / TPR;
   __shared__ Acc lds[P::BLOCK / THX_WAVE];
 
-  const long long bid = blockIdx.x;
   const long long ob = bid / p.S;
   const int s = (int)(bid - ob * p.S);
   const long long o = ob * RPB + threadIdx.x / TPR;
@@ -229,6 +246,7 @@ struct ColParams {
   RedOut<NOUT, NEX> out;
   char* partial;          // Acc[S][n_out] when S > 1
   long long n_out;        // A * C
+  long long nblocks;      // blocks of work; more than the grid holds when the plan strides (GS)
   long long rows;         // R
   long long rows_per_slice;
   int cols;               // C
@@ -244,9 +262,24 @@ struct ColParams {
 };
 
 // Plan members: typedef IT; enum { NK, VEC, UNR, BLOCK, TX, RR2 (1 when two
-// reduced dimensions remain after collapsing), TICKET }; mode(int).
+// reduced dimensions remain after collapsing), TICKET, GS }; mode(int).
+template <class R, class P>
+__device__ __forceinline__ void red_col_block(const ColParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p, long long bid);
+
 template <class R, class P>
 __device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p) {
+  if constexpr (P::GS != 0) {
+    for (long long b = blockIdx.x; b < p.nblocks; b += gridDim.x) {
+      red_col_block<R, P>(p, b);
+      __syncthreads();
+    }
+  } else {
+    red_col_block<R, P>(p, blockIdx.x);
+  }
+}
+
+template <class R, class P>
+__device__ __forceinline__ void red_col_block(const ColParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p, long long bid) {
   typedef typename P::IT IT;
   typedef typename UnsignedOf<IT>::type UT;
   typedef typename R::Acc Acc;
@@ -254,7 +287,6 @@ __device__ __forceinline__ void red_col_body(const ColParams<R::NIN, R::NOUT, R:
   constexpr int TY = P::BLOCK / TX;
   __shared__ Acc lds[TY][VEC][TX];
 
-  long long bid = blockIdx.x;
   const int cb = (int)(bid % p.cblocks);
   bid /= p.cblocks;
   const int s = (int)(bid % p.S);
@@ -380,6 +412,7 @@ struct GenParams {
   unsigned long long imm[NIN];
   RedOut<NOUT, NEX> out;
   long long n_out;
+  long long nblocks;      // blocks of work; more than the grid holds when the plan strides (GS)
   long long n_red;
   FastDiv kfd[NK];
   FastDiv rfd[NR];
@@ -387,15 +420,30 @@ struct GenParams {
   IT rstride[NIN][NR];
 };
 
-// Plan members: typedef IT; enum { NK, NR, BLOCK, TPR }.
+// Plan members: typedef IT; enum { NK, NR, BLOCK, TPR, GS }.
+template <class R, class P>
+__device__ __forceinline__ void red_gen_block(const GenParams<R::NIN, R::NOUT, R::NEX, P::NK, P::NR, typename P::IT>& p, long long bid);
+
 template <class R, class P>
 __device__ __forceinline__ void red_gen_body(const GenParams<R::NIN, R::NOUT, R::NEX, P::NK, P::NR, typename P::IT>& p) {
+  if constexpr (P::GS != 0) {
+    for (long long b = blockIdx.x; b < p.nblocks; b += gridDim.x) {
+      red_gen_block<R, P>(p, b);
+      __syncthreads();
+    }
+  } else {
+    red_gen_block<R, P>(p, blockIdx.x);
+  }
+}
+
+template <class R, class P>
+__device__ __forceinline__ void red_gen_block(const GenParams<R::NIN, R::NOUT, R::NEX, P::NK, P::NR, typename P::IT>& p, long long bid) {
   typedef typename P::IT IT;
   typedef typename UnsignedOf<IT>::type UT;
   typedef typename R::Acc Acc;
   constexpr int NIN = R::NIN, NK = P::NK, NR = P::NR, TPR = P::TPR;
   __shared__ Acc lds[P::BLOCK / THX_WAVE];
-  const long long o = (long long)blockIdx.x * (P::BLOCK / TPR) + threadIdx.x / TPR;
+  const long long o = bid * (P::BLOCK / TPR) + threadIdx.x / TPR;
   const int t = threadIdx.x % TPR;
   const bool live = o < p.n_out;
   IT base[NIN];

@@ -105,6 +105,8 @@ int reduce_final_pass(thx_reduce* r, const std::vector<char*>& outp, const std::
   pk.put<int32_t>(0);
   pk.align(8);
   const int64_t grid = ceil_div(n_out, 256 / tpo);
+  if (grid * 256 > 0xffffffffLL)   // a reduction is only split when it has few outputs
+    return fail(THX_ERR_UNSUPPORTED, "reduce: second pass over %lld outputs", (long long)n_out);
   return launch(k, r->name + "|" + plan, (unsigned)grid, 256, pk.buf.data(), pk.buf.size(), fixed);
 }
 
@@ -351,7 +353,10 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
   std::string plan;
   Kernel k;
   ParamPack pk;
-  int64_t grid = 0;
+  int64_t nblocks = 0;     // pieces of work: (block of outputs) x (slice of the reduce domain)
+  bool gs = false;         // more pieces than one dispatch holds blocks
+  const int forced_limit = env_int("THX_RED_MAX_DISPATCH", 0);   // a smaller limit, to exercise the striding kernels
+  const int64_t max_dispatch = forced_limit >= 1024 ? forced_limit : 0xffffffffLL;
   int S = 1;
   int launch_block = block;
   char* partial = nullptr;  // Acc[S][n_out] of a split reduction
@@ -440,8 +445,10 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       skey += char('0' + sclass[i][0]);
       skey += char('0' + sclass[i][1]);
     }
+    nblocks = oblocks * S;
+    gs = nblocks * rblock > max_dispatch;
     std::ostringstream key;
-    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nacc != unr ? "|c" + std::to_string(nacc) : "") << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << "|m";
+    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nacc != unr ? "|c" + std::to_string(nacc) : "") << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << (gs ? "|gs" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -453,7 +460,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"NACC", nacc}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"TICKET", ticket ? 1 : 0}}, mode, nt, sclass)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"NACC", nacc}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"TICKET", ticket ? 1 : 0}, {"GS", gs ? 1 : 0}}, mode, nt, sclass)
         << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void " << entry << "(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -476,6 +483,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     for (int64_t v : exs) pk.put<int64_t>(v);
     pk.put<char*>(partial);
     pk.put<int64_t>(n_out);
+    pk.put<int64_t>(nblocks);
     pk.put<int64_t>(nvec);
     pk.put<int64_t>(chunk);
     pk.put<int32_t>(S);
@@ -487,7 +495,6 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     for (int i = 0; i < NIN; ++i) pk.put_index(wide, ra_stride[i]);
     for (int i = 0; i < NIN; ++i) pk.put_index(wide, rc_stride[i]);
     pk.align(8);
-    grid = oblocks * S;
     launch_block = rblock;
   } else if (form == COL) {
     int cblock = block;   // threads per block of the column kernel
@@ -564,8 +571,10 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     }
     const bool ticket = S > 1 && r->has_ticket && n_out <= THX_TICKET_WORDS && S < 65536 && env_int("THX_RED_TICKET", 1);
     one_launch = ticket;
+    nblocks = blocks0 * S;
+    gs = nblocks * cblock > max_dispatch;
     std::ostringstream key;
-    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << (cblock != 256 ? "|b" + std::to_string(cblock) : "") << "|r" << rr2 << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << "|m";
+    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << (cblock != 256 ? "|b" + std::to_string(cblock) : "") << "|r" << rr2 << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << (gs ? "|gs" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -577,7 +586,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", cblock}, {"TX", tx}, {"RR2", rr2}, {"TICKET", ticket ? 1 : 0}}, mode, nt)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", cblock}, {"TX", tx}, {"RR2", rr2}, {"TICKET", ticket ? 1 : 0}, {"GS", gs ? 1 : 0}}, mode, nt)
         << "extern \"C\" __global__ __launch_bounds__(" << cblock << ") void " << entry << "(thx::ColParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_col_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -600,6 +609,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     for (int64_t v : exs) pk.put<int64_t>(v);
     pk.put<char*>(partial);
     pk.put<int64_t>(n_out);
+    pk.put<int64_t>(nblocks);
     pk.put<int64_t>(rows);
     pk.put<int64_t>(rps);
     pk.put<int32_t>((int32_t)C);
@@ -615,14 +625,15 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     for (int i = 0; i < NIN; ++i) pk.put_index(wide, c_stride[i]);
     pk.align(8);
     if (C >= (int64_t(1) << 31)) return fail(THX_ERR_UNSUPPORTED, "reduce: %lld kept columns", (long long)C);
-    grid = blocks0 * S;
     launch_block = cblock;
   } else {
     const int NK = std::max(1, NKD);
     const int tpr = n_red >= 512 ? 256 : n_red >= 64 ? 64 : 1;
     std::vector<int> gmode(NIN, M_GATHER);
+    nblocks = ceil_div(n_out, block / tpr);
+    gs = nblocks * block > max_dispatch;
     std::ostringstream key;
-    key << "rg|k" << NK << "|r" << NR << (wide ? "|i64" : "|i32") << "|t" << tpr << "|m";
+    key << "rg|k" << NK << "|r" << NR << (wide ? "|i64" : "|i32") << "|t" << tpr << (gs ? "|gs" : "") << "|m";
     for (int i = 0; i < NIN; ++i) {
       if (views[i].imm) gmode[i] = M_IMM;
       if (views[i].iota) gmode[i] = M_IOTA;
@@ -638,7 +649,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}}, gmode, 0)
+        << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}, {"GS", gs ? 1 : 0}}, gmode, 0)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::GenParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::NR, ThxPlan::IT> p) {\n  thx::red_gen_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -652,6 +663,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     for (uint64_t v : ex) pk.put<uint64_t>(v);
     for (int64_t v : exs) pk.put<int64_t>(v);
     pk.put<int64_t>(n_out);
+    pk.put<int64_t>(nblocks);
     pk.put<int64_t>(n_red);
     for (int d = 0; d < NK; ++d) pk.put<FastDivH>(make_fastdiv(d < NKD ? (uint64_t)KD[d].extent : 1));
     for (int d = 0; d < NR; ++d) pk.put<FastDivH>(make_fastdiv((uint64_t)RD[d].extent));
@@ -660,13 +672,12 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     for (int i = 0; i < NIN; ++i)
       for (int d = 0; d < NR; ++d) pk.put_index(wide, RD[d].stride[i]);
     pk.align(8);
-    grid = ceil_div(n_out, block / tpr);
   }
 
   set_last_plan(r->name + "|" + plan + (S > 1 ? "|s" + std::to_string(S) : ""));
-  if (grid * launch_block > 0xffffffffLL)
-    return fail(THX_ERR_UNSUPPORTED, "reduce: %lld blocks of %d exceed the work-items of one dispatch", (long long)grid,
-                launch_block);
+  // One dispatch carries at most 2^32 - 1 work-items: beyond that the kernel is the striding variant (GS) and each
+  // block takes several pieces of work.
+  const int64_t grid = gs ? std::max<int64_t>(1, max_dispatch / launch_block) : nblocks;
   if (!dry) {
     rc = launch(k, r->name + "|" + plan, (unsigned)grid, launch_block, pk.buf.data(), pk.buf.size(), fixed);
     if (rc) return rc;
