@@ -45,13 +45,15 @@ enum {
 enum {
   THX_BOOL = 0, THX_I8 = 1, THX_U8 = 2, THX_I16 = 3, THX_U16 = 4, THX_I32 = 5,
   THX_U32 = 6, THX_I64 = 7, THX_U64 = 8, THX_F16 = 9, THX_F32 = 10, THX_F64 = 11,
-  THX_NDTYPES = 12
+  THX_C64 = 12, THX_C128 = 13,   /* (real, imaginary) pairs of float32 / float64, NumPy's layout */
+  THX_NDTYPES = 14
 };
 
 /* OR-ed into thx_array.dtype of an INPUT: `base + offset_bytes` is HOST memory
  * holding one element (all extents 1). Its value is copied into the kernel
  * arguments at call time, so it costs no device memory traffic. The reference
- * keeps 0-d operands on the host as well (theano/gpuarray/type.py:55-57). */
+ * keeps 0-d operands on the host as well (theano/gpuarray/type.py:55-57).
+ * Elements of up to 8 bytes only: a THX_C128 value goes through device memory. */
 #define THX_HOST_SCALAR 0x100
 
 /* OR-ed into thx_array.dtype (THX_I64, all extents 1, base ignored) of an input of

@@ -47,7 +47,7 @@ _OP_CODE = {"Add": 0, "Mul": 1, "Maximum": 2, "Minimum": 3, "AND": 4, "OR": 5, "
 SUM_OUT_DTYPE = dict(bool="int64", int8="int64", int16="int64", int32="int64", uint8="uint64", uint16="uint64",
                      uint32="uint64")
 SUM_ACC_DTYPE = dict(bool="int64", int8="int64", int16="int64", int32="int64", uint8="uint64", uint16="uint64",
-                     uint32="uint64", float16="float32", float32="float64")
+                     uint32="uint64", float16="float32", float32="float64", complex64="complex128")
 
 
 def lib():
@@ -90,6 +90,15 @@ def careduce(x, op_name, axis, acc_dtype, out_dtype):
     if op_name in ("Maximum", "Minimum") and any(x.shape[a] == 0 for a in axis):
         raise ValueError("Input of CAReduce{%s} has zero-size on axis %s" % (op_name.lower(), axis))
     acc_dtype, out_dtype = str(acc_dtype), str(out_dtype)
+    if x.dtype.kind == "c":
+        # complex sums and products: the accumulator type's own + and * over the reduced elements (the reference's
+        # struct operators, theano/scalar/basic.py:518-548, which are NumPy's up to the last place); NumPy adds
+        # pairwise, which in a complex128 accumulator is far inside any tolerance a complex64 result is held to
+        if op_name not in ("Add", "Mul"):
+            raise NotImplementedError("no restatement for %s over complex numbers" % op_name)
+        ufunc = np.add if op_name == "Add" else np.multiply
+        with np.errstate(all="ignore"):
+            return np.asarray(ufunc.reduce(x.astype(acc_dtype), axis=axis)).astype(out_dtype)
     if x.dtype == np.float16:
         x = x.astype("float32")  # no float16 C code exists in the reference (elemwise.py:1395-1398)
         if acc_dtype == "float16":  # max / min: exact in any precision
@@ -142,7 +151,9 @@ def _check_broadcast(node, values):
 
 
 def _wide(dtype):
-    """float16 / float32 -> float64; every other dtype stays."""
+    """float16 / float32 -> float64, complex64 -> complex128; every other dtype stays."""
+    if str(dtype) == "complex64":
+        return "complex128"
     return "float64" if str(dtype) in ("float16", "float32") else str(dtype)
 
 
@@ -161,7 +172,7 @@ def eval_scalar_op(op, in_values, out_dtypes, wide=False):
             for o, v in zip(node.outputs, outs):
                 env[o] = v
         return [env[o] if o in env else np.asarray(o.data) for o in op.outputs]
-    fn = scalar_ref.BY_CLASS.get(name)
+    fn = scalar_ref.restatement(name, out_dtypes[0], [np.asarray(v).dtype for v in in_values])
     if fn is None:
         raise NotImplementedError("no restatement of scalar op %s" % name)
     return [np.asarray(fn(out_dtypes[0], *[np.asarray(v) for v in in_values]))]

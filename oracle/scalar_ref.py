@@ -485,6 +485,112 @@ def scalar_softsign(out_dtype, x):
     return _conv((xd / (1.0 + np.abs(xd))).astype(np.dtype(out_dtype)), out_dtype)
 
 
+# ---- Bessel functions of real order ------------------------------------------------------------
+# theano/scalar/basic_scipy.py:698-726, 786-811: scipy.special.jv / iv themselves.
+jv = _special2(lambda v, x: _sp().jv(v, x))
+iv = _special2(lambda v, x: _sp().iv(v, x))
+
+
+# ---- complex numbers ---------------------------------------------------------------------------
+# The reference evaluates every op on complex values through NumPy on the host (``impl``; only +, -, *, /,
+# unary -, abs, == and casts also have C text, theano/scalar/basic.py:498-641, 2459-2460): operands are
+# converted to the result type and NumPy's complex loops do the rest.  These restatements are those NumPy
+# calls.  Pinning (tests/test_oracle_scalar.py): the four arithmetic operations against the reference's C
+# struct formulas written out in real arithmetic; exp / log / sqrt / sin / cos / sinh / cosh / tanh against
+# their definitions through real functions (Euler's formula, log|z| + i arg z, the principal root squared
+# back, the addition theorems); pow against repeated multiplication; abs against hypot; real, imag, conj,
+# angle, complex and complex_from_polar against hand-written values.
+def _is_complex(dt):
+    return str(dt).startswith("complex")
+
+
+def _cwide(out_dtype, *xs):
+    with np.errstate(all="ignore"):
+        return [_conv(x, out_dtype) for x in xs]
+
+
+def _cplx_unary(npfn):
+    def f(out_dtype, x):
+        with np.errstate(all="ignore"):
+            return _conv(npfn(_conv(x, out_dtype)), out_dtype)
+    return f
+
+
+def _cplx_nary(npfn):
+    def f(out_dtype, *xs):
+        with np.errstate(all="ignore"):
+            r = _conv(xs[0], out_dtype)
+            for x in xs[1:]:
+                r = npfn(r, _conv(x, out_dtype))
+            return _conv(r, out_dtype)
+    return f
+
+
+def _cplx_compare(npfn):
+    def f(out_dtype, a, b):
+        up = np.result_type(np.asarray(a).dtype, np.asarray(b).dtype)
+        return npfn(_conv(a, up), _conv(b, up))
+    return f
+
+
+def real(out_dtype, x):
+    return _conv(np.real(x), out_dtype)
+
+
+def imag(out_dtype, x):
+    return _conv(np.imag(x), out_dtype)
+
+
+def angle(out_dtype, x):
+    return _conv(np.angle(x), out_dtype)
+
+
+def conj(out_dtype, x):
+    return _conv(np.conj(x), out_dtype)
+
+
+def complex_(out_dtype, x, y):
+    part = "float32" if str(out_dtype) == "complex64" else "float64"
+    r = np.empty(np.broadcast(x, y).shape, out_dtype)
+    r.real, r.imag = _conv(x, part), _conv(y, part)
+    return r
+
+
+def complex_from_polar(out_dtype, r, theta):
+    """theano/scalar/basic.py:3746-3753: (r cos theta, r sin theta) in the precision of the result's parts."""
+    part = "float32" if str(out_dtype) == "complex64" else "float64"
+    rr, tt = _conv(r, part), _conv(theta, part)
+    return complex_(out_dtype, rr * np.cos(tt), rr * np.sin(tt))
+
+
+COMPLEX_BY_CLASS = {
+    "Add": _cplx_nary(np.add), "Mul": _cplx_nary(np.multiply), "Sub": _cplx_nary(np.subtract),
+    "TrueDiv": _cplx_nary(np.divide), "Pow": _cplx_nary(np.power), "Neg": _cplx_unary(np.negative),
+    "Sqr": _cplx_unary(np.square), "Inv": _cplx_unary(np.reciprocal), "Exp": _cplx_unary(np.exp),
+    "Expm1": _cplx_unary(np.expm1), "Log": _cplx_unary(np.log), "Log2": _cplx_unary(np.log2),
+    "Log10": _cplx_unary(np.log10), "Log1p": _cplx_unary(np.log1p), "Sqrt": _cplx_unary(np.sqrt),
+    "Sin": _cplx_unary(np.sin), "Cos": _cplx_unary(np.cos), "Tan": _cplx_unary(np.tan), "Sinh": _cplx_unary(np.sinh),
+    "Cosh": _cplx_unary(np.cosh), "Tanh": _cplx_unary(np.tanh), "Identity": _cplx_unary(lambda x: x),
+    "Cast": _cplx_unary(lambda x: x), "Conj": conj,
+    "Abs": lambda out_dtype, x: _conv(np.abs(x), out_dtype),
+    "EQ": _cplx_compare(np.equal), "NEQ": _cplx_compare(np.not_equal),
+    "IsNan": lambda out_dtype, x: np.isnan(x), "IsInf": lambda out_dtype, x: np.isinf(x),
+    "Switch": lambda out_dtype, c, a, b: np.where(np.asarray(c) != 0, _conv(a, out_dtype), _conv(b, out_dtype)),
+    "Second": lambda out_dtype, x, y: _conv(np.broadcast_to(y, np.broadcast(x, y).shape), out_dtype),
+    "Real": real, "Imag": imag, "Angle": angle, "Complex": complex_, "ComplexFromPolar": complex_from_polar,
+}
+
+
+def restatement(class_name, out_dtype, in_dtypes):
+    """The function restating scalar op ``class_name`` for these operand types."""
+    if _is_complex(out_dtype) or any(_is_complex(d) for d in in_dtypes):
+        fn = COMPLEX_BY_CLASS.get(class_name)
+        if fn is None:
+            raise NotImplementedError("no restatement of scalar op %s over complex numbers" % class_name)
+        return fn
+    return BY_CLASS.get(class_name)
+
+
 # scalar op class name -> restatement
 BY_CLASS = {
     "Add": add, "Mul": mul, "Sub": sub, "TrueDiv": true_div, "IntDiv": int_div_fast, "Mod": mod_fast, "Pow": pow_,
@@ -501,5 +607,7 @@ BY_CLASS = {
     "Gamma": gamma, "GammaLn": gammaln, "Psi": psi, "TriGamma": tri_gamma, "J0": j0, "J1": j1, "I0": i0, "I1": i1,
     "GammaInc": gammainc, "GammaIncC": gammaincc, "GammaU": gammau, "GammaL": gammal, "Chi2SF": chi2sf,
     "UltraFastScalarSigmoid": ultra_fast_scalar_sigmoid, "ScalarSoftsign": scalar_softsign,
-    "SigmoidBinaryCrossentropy": sigmoid_binary_crossentropy,
+    "SigmoidBinaryCrossentropy": sigmoid_binary_crossentropy, "Jv": jv, "Iv": iv,
+    "Real": real, "Imag": imag, "Angle": angle, "Conj": conj, "Complex": complex_,
+    "ComplexFromPolar": complex_from_polar,
 }

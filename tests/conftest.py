@@ -19,7 +19,9 @@ def pytest_configure(config):
 
 # tolerances of the parity bar, by storage dtype
 TOL = {"float32": dict(rtol=1e-5, atol=1e-6), "float64": dict(rtol=1e-12, atol=1e-12),
-       "float16": dict(rtol=2e-3, atol=2e-3)}
+       "float16": dict(rtol=2e-3, atol=2e-3),
+       # complex values: the float bars of their parts, applied to the modulus of the difference
+       "complex64": dict(rtol=1e-5, atol=1e-6), "complex128": dict(rtol=1e-12, atol=1e-12)}
 
 
 def assert_parity(got, ref, what="", tol=None):
@@ -31,7 +33,8 @@ def assert_parity(got, ref, what="", tol=None):
         assert np.array_equal(got, ref), "%s: integer results differ" % what
         return
     t = tol or TOL[str(ref.dtype)]
-    ok = np.isclose(got.astype("float64"), ref.astype("float64"), equal_nan=True, **t)
+    wide = "complex128" if ref.dtype.kind == "c" else "float64"
+    ok = np.isclose(got.astype(wide), ref.astype(wide), equal_nan=True, **t)
     if not ok.all():
         bad = np.argwhere(~ok)[0]
         raise AssertionError("%s: %d of %d values outside %s, first at %s: got %r, expected %r" % (

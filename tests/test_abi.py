@@ -119,9 +119,11 @@ def test_every_kernel_family_compiles_for_gfx950(dry_run):
     assert "|rg|" in _plans(th.function([t6], t6.sum(axis=(0, 2, 4))), f32(3, 4, 5, 6, 7, 8))
     # every storage dtype goes through the elementwise and the reduction templates
     for dt in ("bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64", "float16",
-               "float32", "float64"):
+               "float32", "float64", "complex64", "complex128"):
         v = T.TensorType(dt, (False, False))("v")
-        if dt == "bool":
+        if dt.startswith("complex"):
+            out = [v * v + 1, v.sum(axis=0), abs(v).max(axis=1)]
+        elif dt == "bool":
             out = [v & v, T.any(v, axis=0), T.all(v, axis=1)]
         elif dt.startswith("float"):
             out = [v * v + 1, v.sum(axis=0), v.max(axis=1)]
@@ -139,11 +141,13 @@ def test_header_constants_match_the_binding():
     defines = dict((k, int(v, 0)) for k, v in re.findall(r"#define\s+(THX_[A-Z_]+)\s+(0x[0-9a-fA-F]+|\d+)", header))
     for name in ("THX_BROADCAST", "THX_DRY_RUN", "THX_HOST_SCALAR", "THX_INDEX", "THX_REUSED"):
         assert defines[name] == getattr(runtime, name), name
-    enum = re.search(r"THX_BOOL = 0.*?THX_NDTYPES = 12", header, re.S).group(0)
+    enum = re.search(r"THX_BOOL = 0.*?THX_NDTYPES = 14", header, re.S).group(0)
     codes = dict((k, int(v)) for k, v in re.findall(r"(THX_[A-Z0-9]+) = (\d+)", enum))
     from theano_amd import scalar as scal
     names = {"bool": "BOOL", "int8": "I8", "uint8": "U8", "int16": "I16", "uint16": "U16", "int32": "I32",
-             "uint32": "U32", "int64": "I64", "uint64": "U64", "float16": "F16", "float32": "F32", "float64": "F64"}
+             "uint32": "U32", "int64": "I64", "uint64": "U64", "float16": "F16", "float32": "F32", "float64": "F64",
+             "complex64": "C64", "complex128": "C128"}
+    assert set(names) == set(scal.all_dtypes)
     for dt, short in names.items():
         assert scal.dtype_code(dt) == codes["THX_" + short], dt
 

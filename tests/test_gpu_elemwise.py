@@ -330,6 +330,46 @@ def test_multi_output_kernels_from_merged_siblings():
 
 
 @pytest.mark.gpu
+def test_user_written_composite_with_several_results():
+    """An Elemwise over a Composite with more than one result, as a user writes it: every result on its own (the
+    results nothing reads leave the Composite first: theano/tensor/tests/test_opt.py:1364-1382), all results
+    together, and results that feed further elementwise work and a reduction."""
+    from theano_amd import scalar as scal
+    from theano_amd.tensor.elemwise import Elemwise
+    sx = scal.float32()
+    pair = Elemwise(scalar_op=scal.Composite([sx], [sx + 1, sx - 1]))
+    X = T.fmatrix("X")
+    o = pair(X)
+    for k, want in ((0, [[2.0]]), (1, [[0.0]])):
+        f = th.function([X], o[k])
+        kernels = [n for n in f.toposort() if isinstance(n.op, hip.HipElemwise)]
+        assert len(kernels) == 1 and len(kernels[0].outputs) == 1
+        assert np.array_equal(f(np.array([[1.0]], "float32")), np.array(want, "float32"))
+    rng = np.random.default_rng(17)
+    sy = scal.float32()
+    three = Elemwise(scalar_op=scal.Composite([sx, sy], [sx + sy, sx * sy, scal.exp(sx) - sy]))
+    Y = T.frow("Y")
+    r = three(X, Y)
+    xv = rng.standard_normal((301, 77)).astype("float32")
+    yv = rng.standard_normal((1, 77)).astype("float32")
+    got = th.function([X, Y], r)(xv, yv)
+    assert np.array_equal(got[0], xv + yv) and np.array_equal(got[1], xv * yv)
+    assert_parity(got[2], G.evaluate([X, Y], [r[2]], [xv, yv])[0])
+    outs = [r[0] * 2 + r[2], T.sum(r[1], axis=0), T.tanh(r[0]), T.max(r[2])]
+    got = th.function([X, Y], outs)(xv, yv)
+    ref = G.evaluate([X, Y], outs, [xv, yv])
+    for g, w in zip(got, ref):
+        assert_parity(g, w)
+    # the same Composite over integers, exact
+    ix, iy = scal.int32(), scal.int32()
+    both = Elemwise(scalar_op=scal.Composite([ix, iy], [ix // iy, ix % iy]))
+    A, B = T.imatrix("A"), T.imatrix("B")
+    av = rng.integers(-1000, 1000, (50, 60)).astype("int32")
+    bv = rng.integers(1, 30, (50, 60)).astype("int32") * rng.choice([-1, 1], (50, 60)).astype("int32")
+    q, m = th.function([A, B], both(A, B))(av, bv)
+    assert np.array_equal(q, av // bv) and np.array_equal(m, av % bv)
+
+
 def test_exact_float32_math_when_the_fast_forms_are_switched_off(monkeypatch):
     """THX_FAST_DIV=0: float32 division and square root correctly rounded (bit-equal to
     NumPy's), exp / sigmoid from the math library (within 2 ulp of the double result); the
@@ -386,6 +426,53 @@ def test_bessel_and_incomplete_gamma_functions_against_scipy(dtype):
     ref = G.evaluate([k, x], outs, [kv, pv])
     for g, r in zip(got, ref):
         assert np.allclose(g, r, rtol=tol["rtol"] * 5, atol=tol["atol"])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float64"])
+def test_bessel_functions_of_real_order_against_scipy(dtype):
+    """jv / iv (theano/scalar/basic_scipy.py:698-726, 786-811; scipy.special.jv / iv in the reference): orders of
+    either sign, whole and fractional, arguments from the series' range through the transition to the oscillating /
+    growing one, whole orders at negative arguments, the special points, and the gradient with respect to the
+    argument, (f(v - 1, x) -+ f(v + 1, x)) / 2."""
+    import scipy.special
+    rng = np.random.default_rng(29)
+    v, x = T.TensorType(dtype, (False,))("v"), T.TensorType(dtype, (False,))("x")
+    n = 6000
+    vv = np.concatenate([rng.uniform(0, 5, n), rng.uniform(-6, 0, n), rng.uniform(0, 60, n),
+                         rng.integers(-8, 9, n).astype("float64")]).astype(dtype)
+    xv = np.concatenate([rng.uniform(0, 2, n), rng.uniform(0.05, 40, n), rng.uniform(0, 120, n),
+                         rng.uniform(-30, 30, n)]).astype(dtype)
+    outs = [T.jv(v, x), T.iv(v, x)]
+    got = th.function([v, x], outs)(vv, xv)
+    v64, x64 = vv.astype("float64"), xv.astype("float64")
+    with np.errstate(all="ignore"):
+        want = [scipy.special.jv(v64, x64), scipy.special.iv(v64, x64)]
+    tol = dict(rtol=2e-5, atol=2e-6) if dtype == "float32" else dict(rtol=2e-10, atol=1e-12)
+    for name, g, w in zip(("jv", "iv"), got, want):
+        assert g.dtype == np.dtype(dtype)
+        with np.errstate(all="ignore"):
+            w = w.astype(dtype)                     # values beyond float32's range are infinite on both sides
+        ok = np.isclose(g, w, equal_nan=True, **tol)
+        assert ok.all(), "%s: %d values differ, first at v=%r x=%r: got %r, scipy %r" % (
+            name, (~ok).sum(), vv[~ok][0], xv[~ok][0], g[~ok][0], w[~ok][0])
+    ref = G.evaluate([v, x], outs, [vv, xv])
+    for g, r in zip(got, ref):
+        assert np.isclose(g, r, equal_nan=True, **tol).all()
+    # special points: x = 0 for every kind of order, NaN operands, fractional orders left of zero
+    pv = np.array([0, 1, 2.5, -1, -0.5, -1.5, -2.5, 0.5, np.nan, 1, 2], dtype)
+    px = np.array([0, 0, 0, 0, 0, 0, 0, -1.0, 1, np.nan, 1e-30], dtype)
+    got = th.function([v, x], outs)(pv, px)
+    with np.errstate(all="ignore"):
+        assert np.isclose(got[0], scipy.special.jv(pv, px).astype(dtype), rtol=tol["rtol"], atol=0, equal_nan=True).all()
+        assert np.isclose(got[1], scipy.special.iv(pv, px).astype(dtype), rtol=tol["rtol"], atol=0, equal_nan=True).all()
+    # gradient with respect to the argument; none with respect to the order
+    gv = rng.uniform(0.2, 6, 2000).astype(dtype)
+    gx = rng.uniform(0.2, 15, 2000).astype(dtype)
+    dj, di = th.function([v, x], [th.grad(T.sum(T.jv(v, x)), x), th.grad(T.sum(T.iv(v, x)), x)])(gv, gx)
+    assert np.allclose(dj, scipy.special.jvp(gv.astype("float64"), gx.astype("float64")), **tol)
+    assert np.allclose(di, scipy.special.ivp(gv.astype("float64"), gx.astype("float64")), rtol=tol["rtol"] * 5, atol=tol["atol"])
+    with pytest.raises(th.gradient.NullTypeGradError):
+        th.grad(T.sum(T.jv(v, x)), v)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float64"])

@@ -803,3 +803,22 @@ def test_more_operands_than_a_kernel_takes_are_split(dry_run):
         kernels = ops_of(f, HipElemwise)
         assert len(kernels) > 1 and all(len(n.inputs) <= th.config.max_fused_inputs for n in kernels)
         f(*[np.zeros((3, 4), "float32")] * 64)           # plans and compiles
+
+
+def test_results_of_a_composite_that_nothing_reads_are_dropped():
+    """theano/tensor/tests/test_opt.py:1364-1382 (local_useless_composite): one node, one output; the gradient of
+    a Composite stays unimplemented (theano/scalar/basic.py:4096-4097)."""
+    sx = scal.float32()
+    comp = scal.Composite([sx], [sx + 1, sx - 1])
+    X = T.fmatrix()
+    o = Elemwise(scalar_op=comp)(X)
+    assert len(o) == 2
+    for k, name in ((0, "add"), (1, "sub")):
+        f = th.function([X], o[k])
+        (node,) = ops_of(f, HipElemwise)
+        assert len(node.outputs) == 1 and name in str(node.op)
+    f = th.function([X], o)
+    (node,) = ops_of(f, HipElemwise)
+    assert len(node.outputs) == 2
+    with pytest.raises(NotImplementedError):
+        th.grad(T.sum(o[0]), X)

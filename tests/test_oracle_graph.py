@@ -90,9 +90,9 @@ def test_dtype_tables_of_the_product_match_reference_literals():
     # theano/tensor/tests/test_elemwise.py:828-836 and :854-865
     out_tbl = dict(bool="int64", int8="int64", int16="int64", int32="int64", uint8="uint64", uint16="uint64",
                    uint32="uint64")
-    acc_tbl = dict(out_tbl, float16="float32", float32="float64")
+    acc_tbl = dict(out_tbl, float16="float32", float32="float64", complex64="complex128")
     for dt in ("bool", "int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64", "float16",
-               "float32", "float64"):
+               "float32", "float64", "complex64", "complex128"):
         x = T.TensorType(dt, (False, False))()
         for method in ("sum", "prod"):
             s = getattr(x, method)(axis=0)

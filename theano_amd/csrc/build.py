@@ -9,7 +9,7 @@ import os
 import subprocess
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-KERNEL_HEADERS = ["thx_common.h", "thx_reduce.h", "thx_elemwise.h", "thx_rowchain.h"]
+KERNEL_HEADERS = ["thx_common.h", "thx_special.h", "thx_reduce.h", "thx_elemwise.h", "thx_rowchain.h"]
 SOURCES = ["thx_runtime.cpp", "thx_elemwise.cpp", "thx_reduce.cpp", "thx_rowchain.cpp", "thx_prelude.cpp"]
 LIB = os.path.join(HERE, "libthx_hip.so")
 # Packed FP32 instructions stay off in every translation unit of the library.

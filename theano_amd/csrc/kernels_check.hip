@@ -5,6 +5,7 @@
 #include <hip/hip_runtime.h>
 
 #include "kernels/thx_common.h"
+#include "kernels/thx_special.h"
 #include "kernels/thx_reduce.h"
 #include "kernels/thx_elemwise.h"
 #include "kernels/thx_rowchain.h"

@@ -247,6 +247,8 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
                   a.dtype & ~(THX_HOST_SCALAR | THX_REUSED), want);
     const char* p = (const char*)a.base + a.offset_bytes;
     if (a.dtype & THX_HOST_SCALAR) {
+      if (dtype_size(want) > 8)
+        return fail(THX_ERR_TYPE, "reduce: epilogue operand %d: values of %d bytes do not travel by value", j, dtype_size(want));
       memcpy(&ex[j], p, (size_t)dtype_size(want));
       continue;
     }

@@ -111,7 +111,7 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
     const int isz = dtype_size(dt);
     char* p = (char*)a.base + a.offset_bytes;
     if (a.dtype & THX_HOST_SCALAR) {
-      if (kind != K_SCALAR || i >= NIN) return fail(THX_ERR_TYPE, "rowchain: operand %d cannot be a host scalar", i);
+      if (kind != K_SCALAR || i >= NIN || isz > 8) return fail(THX_ERR_TYPE, "rowchain: operand %d cannot be a host scalar", i);
       memcpy(&imm[i], p, (size_t)isz);
       is_imm[i] = 1;
       continue;

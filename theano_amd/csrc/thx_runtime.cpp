@@ -152,12 +152,13 @@ int ensure_scratch(size_t bytes) {
 // ---------------------------------------------------------------------------
 // helpers
 int dtype_size(int dtype) {
-  static const int sz[THX_NDTYPES] = {1, 1, 1, 2, 2, 4, 4, 8, 8, 2, 4, 8};
+  static const int sz[THX_NDTYPES] = {1, 1, 1, 2, 2, 4, 4, 8, 8, 2, 4, 8, 8, 16};
   return (dtype >= 0 && dtype < THX_NDTYPES) ? sz[dtype] : 0;
 }
 const char* dtype_ctype(int dtype) {
   static const char* nm[THX_NDTYPES] = {"thx_bool", "thx_i8",  "thx_u8",  "thx_i16", "thx_u16", "thx_i32",
-                                        "thx_u32",  "thx_i64", "thx_u64", "thx_f16", "thx_f32", "thx_f64"};
+                                        "thx_u32",  "thx_i64", "thx_u64", "thx_f16", "thx_f32", "thx_f64",
+                                        "thx_c64",  "thx_c128"};
   return (dtype >= 0 && dtype < THX_NDTYPES) ? nm[dtype] : "void";
 }
 
@@ -226,6 +227,7 @@ int gather_inputs(const char* what, const thx_array* ins, int n_in, const int32_
       for (int d = 0; d < nd; ++d)
         if (ins[i].shape[d] != 1) return fail(THX_ERR_TYPE, "%s: host scalar input %d must have extent 1 everywhere", what, i);
       if (!v.ptr) return fail(THX_ERR_ARG, "%s: host scalar input %d is null", what, i);
+      if (isz > 8) return fail(THX_ERR_TYPE, "%s: host scalar input %d: values of %d bytes do not travel by value", what, i, isz);
       v.imm = true;
       memcpy(&v.immval, v.ptr, (size_t)isz);
       v.ptr = nullptr;

@@ -89,6 +89,8 @@ def reduce_identity(scalar_op, dtype):
         if scalar_op.identity is None:
             return None
         return c_literal(scalar_op.identity, dtype)
+    if dtype in scal.complex_dtypes:
+        raise NotImplementedError("maximum / minimum of complex numbers (theano/scalar/basic.py:1635, 1674)")
     if dtype in scal.float_dtypes:
         return c_literal(np.inf if big else -np.inf, dtype)
     if dtype == "bool":

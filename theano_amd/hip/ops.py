@@ -77,8 +77,9 @@ HipArrayType.Variable = HipArrayVariable
 
 def _is_host_scalar(var):
     """A host tensor whose every dimension is broadcastable travels as a
-    kernel argument instead of being copied to the device."""
-    return isinstance(var.type, TensorType) and all(var.type.broadcastable)
+    kernel argument instead of being copied to the device (values of up to 8
+    bytes: a complex128 goes through device memory like any array)."""
+    return isinstance(var.type, TensorType) and all(var.type.broadcastable) and var.type.dtype != "complex128"
 
 
 def as_hip_variable(x):

@@ -57,7 +57,7 @@ def lift_to_hip(fgraph):
     no host execution to fall back to."""
     mapping = {}
     for i in fgraph.inputs:
-        if isinstance(i.type, TensorType) and not all(i.type.broadcastable):
+        if isinstance(i.type, TensorType) and not _is_host_scalar(i):
             mapping[i] = hip_from_host(i)
         else:
             mapping[i] = i
@@ -66,7 +66,7 @@ def lift_to_hip(fgraph):
         if v in mapping:
             return mapping[v]
         if isinstance(v, Constant):
-            if isinstance(v.type, TensorType) and not all(v.type.broadcastable):
+            if isinstance(v.type, TensorType) and not _is_host_scalar(v):
                 mapping[v] = DeviceConstant(HipArrayType(v.type.dtype, v.type.broadcastable), v.data, name=v.name)
             else:
                 mapping[v] = v
@@ -90,8 +90,6 @@ def lift_to_hip(fgraph):
             else:
                 outs = op.make_node(*ins).outputs
         elif isinstance(op, Elemwise):
-            if len(node.outputs) != 1:
-                raise NotImplementedError("multi-output Elemwise cannot be lifted: %s" % op)
             outs = HipElemwise(op.scalar_op, op.inplace_pattern).make_node(*ins).outputs
         elif isinstance(op, DimShuffle):
             if isinstance(ins[0].type, HipArrayType):

@@ -9,6 +9,7 @@ definition of each op here exactly as the C snippets are in the reference.
 float16 values are computed in float32 (what ``Compositef32``
 :4130-4208 arranges for the reference's device code).
 """
+import builtins
 import hashlib
 import math
 
@@ -23,8 +24,9 @@ int_dtypes = ("int8", "int16", "int32", "int64")
 uint_dtypes = ("uint8", "uint16", "uint32", "uint64")
 integer_dtypes = int_dtypes + uint_dtypes
 discrete_dtypes = ("bool",) + integer_dtypes
-continuous_dtypes = float_dtypes
-all_dtypes = discrete_dtypes + float_dtypes
+complex_dtypes = ("complex64", "complex128")
+continuous_dtypes = float_dtypes + complex_dtypes
+all_dtypes = discrete_dtypes + float_dtypes + complex_dtypes
 
 # dtype -> (ABI code, storage C type, compute C type)
 _DTYPE_INFO = {
@@ -32,6 +34,7 @@ _DTYPE_INFO = {
     "int16": (3, "thx_i16", "thx_i16"), "uint16": (4, "thx_u16", "thx_u16"), "int32": (5, "thx_i32", "thx_i32"),
     "uint32": (6, "thx_u32", "thx_u32"), "int64": (7, "thx_i64", "thx_i64"), "uint64": (8, "thx_u64", "thx_u64"),
     "float16": (9, "thx_f16", "thx_f32"), "float32": (10, "thx_f32", "thx_f32"), "float64": (11, "thx_f64", "thx_f64"),
+    "complex64": (12, "thx_c64", "thx_c64"), "complex128": (13, "thx_c128", "thx_c128"),
 }
 
 
@@ -99,6 +102,7 @@ bool_ = Scalar("bool")
 int8, int16, int32, int64 = Scalar("int8"), Scalar("int16"), Scalar("int32"), Scalar("int64")
 uint8, uint16, uint32, uint64 = Scalar("uint8"), Scalar("uint16"), Scalar("uint32"), Scalar("uint64")
 float16, float32, float64 = Scalar("float16"), Scalar("float32"), Scalar("float64")
+complex64, complex128 = Scalar("complex64"), Scalar("complex128")
 
 
 class _scalar_py_operators(object):
@@ -256,6 +260,27 @@ def same_out(t):
     return (t,)
 
 
+def _no_complex(types, what="complex argument not supported"):
+    if any(t.dtype in complex_dtypes for t in types):
+        raise TypeError(what)
+
+
+def upcast_out_no_complex(*types):
+    _no_complex(types, "complex type are not supported")
+    return upcast_out(*types)
+
+
+def upgrade_to_float_no_complex(*types):
+    _no_complex(types)
+    return upgrade_to_float(*types)
+
+
+def real_out(t):
+    """The type of one component: float32 for complex64, float64 for complex128, the type itself
+    otherwise (``theano/scalar/basic.py:1008-1019``)."""
+    return ({"complex64": float32, "complex128": float64}.get(t.dtype, t),)
+
+
 def same_out_nobool(t):
     if t == bool_:
         raise TypeError("bool input not supported")
@@ -315,6 +340,10 @@ def c_literal(value, dtype):
     dtype = str(dtype)
     if dtype == "bool":
         return "((thx_bool)%d)" % (1 if value else 0)
+    if dtype in complex_dtypes:
+        v = builtins.complex(np.asarray(value, dtype=dtype))
+        part = "float32" if dtype == "complex64" else "float64"
+        return "%s(%s, %s)" % (compute_ctype(dtype), c_literal(v.real, part), c_literal(v.imag, part))
     if dtype in float_dtypes:
         v = float(np.asarray(value, dtype=dtype))
         ct = compute_ctype(dtype)
@@ -424,6 +453,11 @@ class LogicalComparison(BinaryScalarOp):
 def _cmp(name, sym):
     class _C(LogicalComparison):
         def c_code(self, node, inputs, outputs):
+            if any(i.type.dtype in complex_dtypes for i in node.inputs):
+                if sym not in ("==", "!="):
+                    raise NotImplementedError("complex numbers have no order (theano/scalar/basic.py:1280-1350)")
+                ct = compute_ctype(upcast(*[i.type.dtype for i in node.inputs]))
+                return "%s = ((%s)%s %s (%s)%s);" % (outputs[0], ct, inputs[0], sym, ct, inputs[1])
             return "%s = (%s %s %s);" % (outputs[0], inputs[0], sym, inputs[1])
     _C.__name__ = _C.__qualname__ = name      # instances pickle by reference to the module-level name
     _C.commutative = sym in ("==", "!=")
@@ -447,6 +481,8 @@ class IsNan(FixedLogicalComparison):
     def c_code(self, node, inputs, outputs):
         if node.inputs[0].type.dtype in discrete_dtypes:
             return "%s = 0;" % outputs[0]
+        if node.inputs[0].type.dtype in complex_dtypes:
+            return "%s = (isnan(%s.re) || isnan(%s.im)) ? 1 : 0;" % (outputs[0], inputs[0], inputs[0])
         return "%s = isnan(%s) ? 1 : 0;" % (outputs[0], inputs[0])
 
 
@@ -454,6 +490,8 @@ class IsInf(FixedLogicalComparison):
     def c_code(self, node, inputs, outputs):
         if node.inputs[0].type.dtype in discrete_dtypes:
             return "%s = 0;" % outputs[0]
+        if node.inputs[0].type.dtype in complex_dtypes:
+            return "%s = (isinf(%s.re) || isinf(%s.im)) ? 1 : 0;" % (outputs[0], inputs[0], inputs[0])
         return "%s = isinf(%s) ? 1 : 0;" % (outputs[0], inputs[0])
 
 
@@ -467,6 +505,12 @@ class Switch(ScalarOp):
         return list(upcast_out(types[1], types[2]))
 
     def c_code(self, node, inputs, outputs):
+        ot = node.outputs[0].type.dtype
+        if node.inputs[0].type.dtype in complex_dtypes:
+            raise NotImplementedError("switch on a complex condition")
+        if ot in complex_dtypes:
+            ct = compute_ctype(ot)
+            return "%s = %s ? (%s)%s : (%s)%s;" % (outputs[0], inputs[0], ct, inputs[1], ct, inputs[2])
         return "%s = %s ? %s : %s;" % (outputs[0], inputs[0], inputs[1], inputs[2])
 
     def L_op(self, inputs, outputs, gout):
@@ -568,6 +612,8 @@ class Maximum(BinaryScalarOp):
 
     def c_code(self, node, inputs, outputs):
         x, y = inputs
+        if node.outputs[0].type.dtype in complex_dtypes:
+            raise NotImplementedError("maximum / minimum of complex numbers (theano/scalar/basic.py:1635, 1674)")
         nan = "NAN" if node.outputs[0].type.dtype in float_dtypes else "0"
         # both comparisons, so that a NaN on either side gives NaN
         return "%s = ((%s) > (%s) ? (%s) : ((%s) >= (%s) ? (%s) : %s));" % (outputs[0], y, x, y, x, y, x, nan)
@@ -584,6 +630,8 @@ class Maximum(BinaryScalarOp):
 class Minimum(Maximum):
     def c_code(self, node, inputs, outputs):
         x, y = inputs
+        if node.outputs[0].type.dtype in complex_dtypes:
+            raise NotImplementedError("maximum / minimum of complex numbers (theano/scalar/basic.py:1635, 1674)")
         nan = "NAN" if node.outputs[0].type.dtype in float_dtypes else "0"
         return "%s = ((%s) < (%s) ? (%s) : ((%s) <= (%s) ? (%s) : %s));" % (outputs[0], y, x, y, x, y, x, nan)
 
@@ -592,6 +640,17 @@ maximum, minimum = Maximum(upcast_out, name="maximum"), Minimum(upcast_out, name
 
 
 # ---- arithmetic (theano/scalar/basic.py:1699-2261) ------------------------------
+def _to_complex_result(node, inputs):
+    """Operand expressions converted to the result type when that is complex: every operand is
+    widened first and the operation runs in the result type, as NumPy's loops do (the reference's
+    C mixes types through overloads, ``theano/scalar/basic.py:584-631``)."""
+    ot = node.outputs[0].type.dtype
+    if ot not in complex_dtypes:
+        return list(inputs)
+    ct = compute_ctype(ot)
+    return ["(%s)%s" % (ct, i) for i in inputs]
+
+
 class Add(ScalarOp):
     identity = 0
     commutative = True
@@ -599,6 +658,7 @@ class Add(ScalarOp):
 
     def c_code(self, node, inputs, outputs):
         sym = " || " if node.outputs[0].type == bool_ else " + "
+        inputs = _to_complex_result(node, inputs)
         return "%s = %s;" % (outputs[0], sym.join(inputs) if inputs else "0")
 
     def L_op(self, inputs, outputs, gout):
@@ -615,6 +675,7 @@ class Mul(ScalarOp):
 
     def c_code(self, node, inputs, outputs):
         sym = " && " if node.outputs[0].type == bool_ else " * "
+        inputs = _to_complex_result(node, inputs)
         return "%s = %s;" % (outputs[0], sym.join(inputs) if inputs else "1")
 
     def L_op(self, inputs, outputs, gout):
@@ -626,6 +687,7 @@ class Mul(ScalarOp):
 
 class Sub(BinaryScalarOp):
     def c_code(self, node, inputs, outputs):
+        inputs = _to_complex_result(node, inputs)
         return "%s = %s - %s;" % (outputs[0], inputs[0], inputs[1])
 
     def L_op(self, inputs, outputs, gout):
@@ -682,6 +744,9 @@ class TrueDiv(BinaryScalarOp):
     def c_code(self, node, inputs, outputs):
         if all(i.type.dtype in discrete_dtypes for i in node.inputs):
             return "%s = ((double)%s) / %s;" % (outputs[0], inputs[0], inputs[1])
+        if node.outputs[0].type.dtype in complex_dtypes:
+            x, y = _to_complex_result(node, inputs)
+            return "%s = %s / %s;" % (outputs[0], x, y)
         if node.outputs[0].type.dtype in ("float16", "float32"):
             # single-precision division goes through the device helper (a plain `/` unless the
             # library was asked for the 2.5-ulp form); the reference's text is `x / y`
@@ -709,6 +774,8 @@ class IntDiv(BinaryScalarOp):
         x, y = inputs
         (z,) = outputs
         t = upcast(*[i.type.dtype for i in node.inputs])
+        if t in complex_dtypes:
+            raise TypeError("floor division is not defined for complex numbers (theano/scalar/basic.py:1947-1949)")
         if t in discrete_dtypes:
             d = lambda a, b: "(%s / %s)" % (a, b)
             m = lambda a, b: "(%s %% %s)" % (a, b)
@@ -743,6 +810,8 @@ class Mod(BinaryScalarOp):
         x, y = inputs
         (z,) = outputs
         t = upcast(*[i.type.dtype for i in node.inputs])
+        if t in complex_dtypes:
+            raise TypeError("modulo is not defined for complex numbers (theano/scalar/basic.py:2050-2052)")
         if t in discrete_dtypes:
             m = lambda a, b: "(%s %% %s)" % (a, b)
             zero = "%s = 0;" % z
@@ -773,6 +842,9 @@ class Pow(BinaryScalarOp):
     def c_code(self, node, inputs, outputs):
         # C's pow(): arguments promote to double
         (x, y), (z,) = inputs, outputs
+        if node.outputs[0].type.dtype in complex_dtypes:
+            x, y = _to_complex_result(node, inputs)
+            return "%s = thx_cpow(%s, %s);" % (z, x, y)
         if node.outputs[0].type.dtype in discrete_dtypes:
             # The host libm the reference runs on returns whole powers of whole numbers exactly, and the
             # conversion to the integer result truncates.  The device's pow may come out one place short
@@ -800,7 +872,7 @@ class Clip(ScalarOp):
     nin = 3
 
     def output_types(self, types):
-        return list(upcast_out(*types))
+        return list(upcast_out_no_complex(*types))
 
     def c_code(self, node, inputs, outputs):
         x, lo, hi = inputs
@@ -884,13 +956,21 @@ def cast(x, dtype):
     dtype = str(dtype)
     if x.type.dtype == dtype:
         return x
+    if x.type.dtype in complex_dtypes and dtype not in complex_dtypes:
+        raise TypeError("Casting from complex to real is ambiguous: consider real(), imag(), angle() or abs()")
     return _cast_mapping[dtype](x)
 
 
 class Abs(UnaryScalarOp):
+    def output_types(self, types):
+        # the modulus of a complex number is real (theano/scalar/basic.py:2421-2430)
+        return list(real_out(types[0]))
+
     def c_code(self, node, inputs, outputs):
         t = node.inputs[0].type.dtype
         (x,), (z,) = inputs, outputs
+        if t in complex_dtypes:
+            return "%s = thx_cabs(%s);" % (z, x)
         if t in int_dtypes:
             return "%s = (%s < 0) ? -%s : %s;" % (z, x, x, x)
         if t in float_dtypes:
@@ -901,6 +981,8 @@ class Abs(UnaryScalarOp):
         (x,) = inputs
         if outputs[0].type.dtype in discrete_dtypes:
             return [x.zeros_like(dtype=config.floatX)]
+        if x.type.dtype in complex_dtypes:
+            return [gout[0] * x / abs_(x)]       # theano/scalar/basic.py:2447
         return [gout[0] * sgn(x)]
 
 
@@ -911,6 +993,7 @@ class Sgn(UnaryScalarOp):
     def output_types(self, types):
         if types[0] == bool_:
             raise TypeError(types[0])
+        _no_complex(types, "complex has no sgn")
         return [types[0]]
 
     def c_code(self, node, inputs, outputs):
@@ -935,6 +1018,10 @@ def _unary_math(cname, fname, grad_fn, policy=upgrade_to_float):
     class _U(UnaryScalarOp):
         def c_code(self, node, inputs, outputs):
             ot = node.outputs[0].type.dtype
+            if ot in complex_dtypes:
+                if fname not in _COMPLEX_MATH:
+                    raise NotImplementedError("%s has no device code for complex numbers" % fname)
+                return "%s = thx_c%s((%s)%s);" % (outputs[0], fname, compute_ctype(ot), inputs[0])
             fn = _fn(fname, ot)
             if fn == "expf":
                 fn = "thx_fexp"        # expf, or exp2 of x * log2(e) in the 2.5-ulp build
@@ -944,6 +1031,8 @@ def _unary_math(cname, fname, grad_fn, policy=upgrade_to_float):
             (x,) = inputs
             if outputs[0].type.dtype in discrete_dtypes:
                 return [x.zeros_like(dtype=config.floatX)]
+            if outputs[0].type.dtype in complex_dtypes:
+                raise NotImplementedError("gradient of %s for complex numbers (the reference has none either)" % fname)
             if grad_fn is None:
                 return _zero_grads(inputs)
             return [grad_fn(x, outputs[0], gout[0])]
@@ -952,8 +1041,11 @@ def _unary_math(cname, fname, grad_fn, policy=upgrade_to_float):
     return _U(policy, name=fname if fname != "fabs" else "abs")
 
 
-ceil = _unary_math("Ceil", "ceil", None)
-floor = _unary_math("Floor", "floor", None)
+# the functions with a complex form among the device helpers
+_COMPLEX_MATH = ("exp", "expm1", "log", "log2", "log10", "log1p", "sqrt", "sin", "cos", "tan", "sinh", "cosh", "tanh")
+
+ceil = _unary_math("Ceil", "ceil", None, upgrade_to_float_no_complex)
+floor = _unary_math("Floor", "floor", None, upgrade_to_float_no_complex)
 log = _unary_math("Log", "log", lambda x, z, gz: gz / x)
 log2 = _unary_math("Log2", "log2", lambda x, z, gz: gz / (x * math.log(2.0)))
 log10 = _unary_math("Log10", "log10", lambda x, z, gz: gz / (x * math.log(10.0)))
@@ -1262,6 +1354,139 @@ class DisconnectedType(Type):
 
     def __str__(self):
         return "DisconnectedType"
+
+
+# ---- complex numbers (theano/scalar/basic.py:3623-3761) -----------------------------------
+# The reference runs these five through NumPy on the host (none has C code there); here they are
+# device code like every other op.
+class Real(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        if node.inputs[0].type.dtype in complex_dtypes:
+            return "%s = %s.re;" % (outputs[0], inputs[0])
+        return "%s = %s;" % (outputs[0], inputs[0])
+
+    def L_op(self, inputs, outputs, gout):
+        if inputs[0].type.dtype in complex_dtypes:
+            return [complex(gout[0], 0)]
+        return [gout[0]] if inputs[0].type.dtype in float_dtypes else _zero_grads(inputs)
+
+
+class Imag(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        if node.inputs[0].type.dtype in complex_dtypes:
+            return "%s = %s.im;" % (outputs[0], inputs[0])
+        return "%s = 0;" % outputs[0]
+
+    def L_op(self, inputs, outputs, gout):
+        (x,) = inputs
+        if x.type.dtype in complex_dtypes:
+            return [complex(0, gout[0])]
+        return [second(x, 0)] if x.type.dtype in float_dtypes else _zero_grads(inputs)
+
+
+class Angle(UnaryScalarOp):
+    """Argument of a complex number, always float64 as in the reference
+    (``theano/scalar/basic.py:3660-3693``; NumPy computes it in the precision of the input)."""
+
+    def c_code(self, node, inputs, outputs):
+        t = node.inputs[0].type.dtype
+        if t in complex_dtypes:
+            return "%s = thx_cangle(%s);" % (outputs[0], inputs[0])
+        # np.angle of a real: 0 or pi (NaN stays), in the precision of the input
+        if t in ("float16", "float32"):
+            return "%s = atan2f(0.0f, (float)%s);" % (outputs[0], inputs[0])
+        return "%s = atan2(0.0, (double)%s);" % (outputs[0], inputs[0])
+
+    def L_op(self, inputs, outputs, gout):
+        (c,) = inputs
+        if c.type.dtype not in complex_dtypes:
+            return [second(c, 0)] if c.type.dtype in float_dtypes else _zero_grads(inputs)
+        # d theta = (x dy - y dx) / r^2
+        x, y = real(c), imag(c)
+        r2 = x * x + y * y
+        return [cast(complex(-gout[0] * y / r2, gout[0] * x / r2), c.type.dtype)]
+
+
+class Complex(BinaryScalarOp):
+    def output_types(self, types):
+        for t in types:
+            if t.dtype in complex_dtypes:
+                raise TypeError(t)
+        up = upcast(*[t.dtype for t in types])
+        return [complex128 if up in ("float64", "int64", "uint64", "int32", "uint32") else complex64]
+
+    def c_code(self, node, inputs, outputs):
+        ot = node.outputs[0].type.dtype
+        part = "thx_f32" if ot == "complex64" else "thx_f64"
+        return "%s = %s((%s)%s, (%s)%s);" % (outputs[0], compute_ctype(ot), part, inputs[0], part, inputs[1])
+
+    def L_op(self, inputs, outputs, gout):
+        x, y = inputs
+        (gz,) = gout
+        return [g if i.type.dtype in float_dtypes else i.zeros_like(dtype=config.floatX)
+                for i, g in ((x, cast(real(gz), x.type.dtype)), (y, cast(imag(gz), y.type.dtype)))]
+
+
+class Conj(UnaryScalarOp):
+    def c_code(self, node, inputs, outputs):
+        if node.inputs[0].type.dtype in complex_dtypes:
+            return "%s = thx_cconj(%s);" % (outputs[0], inputs[0])
+        return "%s = %s;" % (outputs[0], inputs[0])
+
+
+class ComplexFromPolar(BinaryScalarOp):
+    """``r (cos theta + i sin theta)``.  The reference's host implementation raises ValueError for a negative
+    radius (``theano/scalar/basic.py:3746-3748``); device code cannot raise and stores the value the formula
+    gives."""
+
+    def output_types(self, types):
+        return Complex.output_types(self, types)
+
+    def c_code(self, node, inputs, outputs):
+        ot = node.outputs[0].type.dtype
+        part = "thx_f32" if ot == "complex64" else "thx_f64"
+        return "%s = thx_cpolar((%s)%s, (%s)%s);" % (outputs[0], part, inputs[0], part, inputs[1])
+
+
+real, imag = Real(real_out, name="real"), Imag(real_out, name="imag")
+angle = Angle(specific_out(float64), name="angle")
+complex = Complex(name="complex")
+conj = Conj(same_out_min8, name="conj")
+complex_from_polar = ComplexFromPolar(name="complex_from_polar")
+
+
+# ---- Bessel functions of real order (theano/scalar/basic_scipy.py:698-726, 786-811) ------------
+class _BesselOfOrder(BinaryScalarOp):
+    """``scipy.special.jv`` / ``iv`` in the reference (host only); device helpers here, evaluated in
+    double precision whatever the result type.  No gradient with respect to the order."""
+
+    fn = None
+    sign = None
+
+    def c_code(self, node, inputs, outputs):
+        _no_complex([i.type for i in node.inputs])
+        return "%s = %s((double)%s, (double)%s);" % (outputs[0], self.fn, inputs[0], inputs[1])
+
+    def L_op(self, inputs, outputs, gout):
+        from .gradient import grad_not_implemented
+        v, x = inputs
+        (gz,) = gout
+        if outputs[0].type.dtype in discrete_dtypes:
+            return _zero_grads(inputs)
+        me = type(self)(upgrade_to_float, name=self.name)
+        lower, upper = me(v - 1, x), me(v + 1, x)
+        return [grad_not_implemented(self, 0, v), gz * (lower + upper if self.sign > 0 else lower - upper) / 2.]
+
+
+class Jv(_BesselOfOrder):
+    fn, sign = "thx_jv", -1
+
+
+class Iv(_BesselOfOrder):
+    fn, sign = "thx_iv", 1
+
+
+jv, iv = Jv(upgrade_to_float, name="jv"), Iv(upgrade_to_float, name="iv")
 
 
 # --------------------------------------------------------------------------

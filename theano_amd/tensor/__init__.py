@@ -6,7 +6,7 @@ from .type import (TensorType, TensorVariable, TensorConstant, as_tensor_variabl
                    dscalar, dvector, dmatrix, drow, dcol, dtensor3, dtensor4)
 from . import type as _type
 for _n in dir(_type):  # bscalar ... dtensor4 and friends
-    if _n[0] in "bwilhfd" and _n[1:] in ("scalar", "vector", "matrix", "row", "col", "tensor3", "tensor4"):
+    if _n[0] in "bwilhfdcz" and _n[1:] in ("scalar", "vector", "matrix", "row", "col", "tensor3", "tensor4"):
         globals()[_n] = getattr(_type, _n)
 from .elemwise import DimShuffle, Elemwise, CAReduce, CAReduceDtype, Sum, Prod, All, Any
 from .basic import *  # noqa: F401,F403

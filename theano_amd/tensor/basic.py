@@ -57,7 +57,11 @@ erfinv, erfcinv = _elemwise(scal.erfinv, "erfinv"), _elemwise(scal.erfcinv, "erf
 gamma, gammaln = _elemwise(scal.gamma, "gamma"), _elemwise(scal.gammaln, "gammaln")
 psi, tri_gamma = _elemwise(scal.psi, "psi"), _elemwise(scal.tri_gamma, "tri_gamma")
 j0, j1, i0, i1 = _elemwise(scal.j0, "j0"), _elemwise(scal.j1, "j1"), _elemwise(scal.i0, "i0"), _elemwise(scal.i1, "i1")
+jv, iv = _elemwise(scal.jv, "jv"), _elemwise(scal.iv, "iv")
 gammainc, gammaincc = _elemwise(scal.gammainc, "gammainc"), _elemwise(scal.gammaincc, "gammaincc")
+real, imag, angle, conj = (_elemwise(scal.real, "real"), _elemwise(scal.imag, "imag"), _elemwise(scal.angle, "angle"),
+                           _elemwise(scal.conj, "conj"))
+complex, complex_from_polar = _elemwise(scal.complex, "complex"), _elemwise(scal.complex_from_polar, "complex_from_polar")
 gammau, gammal, chi2sf = _elemwise(scal.gammau, "gammau"), _elemwise(scal.gammal, "gammal"), _elemwise(scal.chi2sf, "chi2sf")
 sigmoid = _elemwise(scal.scalar_sigmoid, "sigmoid")
 softplus = _elemwise(scal.scalar_softplus, "softplus")
@@ -81,6 +85,9 @@ def cast(x, dtype):
     x = as_tensor_variable(x)
     if x.type.dtype == dtype:
         return x
+    if x.type.dtype in scal.complex_dtypes and dtype not in scal.complex_dtypes:
+        # theano/tensor/basic.py:1263-1266
+        raise TypeError("Casting from complex to real is ambiguous: consider real(), imag(), angle() or abs()")
     return _cast_ops[dtype](x)
 
 

@@ -406,7 +406,7 @@ class CAReduceDtype(CAReduce):
         acc = self.acc_dtype
         if acc is None:
             return dict(bool="int64", int8="int64", int16="int64", int32="int64", uint8="uint64", uint16="uint64",
-                        uint32="uint64", float16="float32", float32="float64").get(idtype, idtype)
+                        uint32="uint64", float16="float32", float32="float64", complex64="complex128").get(idtype, idtype)
         if acc in scal.continuous_dtypes and idtype in scal.discrete_dtypes:
             return acc
         up = scal.upcast(idtype, acc)

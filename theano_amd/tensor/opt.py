@@ -115,6 +115,21 @@ def local_useless_elemwise(fgraph, node):
 
 
 @local_optimizer([Elemwise])
+def local_useless_composite(fgraph, node):
+    """An Elemwise of a Composite with several results, some of which nothing reads: the Composite is rebuilt
+    with the results in use only (``theano/tensor/opt.py:7473-7491``)."""
+    comp = node.op.scalar_op
+    if not isinstance(comp, scal.Composite) or len(node.outputs) < 2:
+        return False
+    used = [i for i, o in enumerate(node.outputs) if fgraph.clients.get(o)]
+    if not used or len(used) == len(node.outputs):
+        return False
+    smaller = scal.Composite(comp.inputs, [comp.outputs[i] for i in used])
+    new = Elemwise(smaller).make_node(*node.inputs).outputs
+    return {node.outputs[i]: n for i, n in zip(used, new)}
+
+
+@local_optimizer([Elemwise])
 def local_constant_fold(fgraph, node):
     """Arithmetic on scalar constants is done when the function is compiled
     (``constant_folding``, ``theano/tensor/opt.py:6600-6660``, restricted to
@@ -572,7 +587,8 @@ def local_split_huge_add_or_mul(fgraph, node):
     return [new] if new.type == node.outputs[0].type else False
 
 
-CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_constant_fold, local_useless_elemwise, local_fill_sink,
+CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_useless_composite, local_constant_fold,
+                local_useless_elemwise, local_fill_sink,
                 local_useless_reduce, local_op_of_op,
                 local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_single_pass_variance,
                 local_cancel_common_factors, local_split_huge_add_or_mul]

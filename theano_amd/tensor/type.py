@@ -174,6 +174,15 @@ class _tensor_py_operators(object):
     def astype(self, dtype):
         return self._b().cast(self, dtype)
 
+    # -- complex numbers (theano/tensor/var.py: real, imag, conj)
+    real = property(lambda self: self._b().real(self))
+    imag = property(lambda self: self._b().imag(self))
+
+    def conj(self):
+        return self._b().conj(self)
+
+    conjugate = conj
+
     def zeros_like(self, dtype=None):
         return self._b().zeros_like(self, dtype=dtype)
 
@@ -277,7 +286,7 @@ def _mk(dtype, bcast):
 
 
 for _p, _dt in (("b", "int8"), ("w", "int16"), ("i", "int32"), ("l", "int64"), ("h", "float16"),
-                ("f", "float32"), ("d", "float64")):
+                ("f", "float32"), ("d", "float64"), ("c", "complex64"), ("z", "complex128")):
     globals()[_p + "scalar"] = _mk(_dt, ())
     globals()[_p + "vector"] = _mk(_dt, (False,))
     globals()[_p + "matrix"] = _mk(_dt, (False, False))
