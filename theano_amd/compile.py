@@ -9,6 +9,7 @@ results after their last use (the loop of ``theano/gof/vm.py:237-305``).
 import numpy as np
 
 from . import gof
+from .config import config
 from .gof import Constant, FunctionGraph, Variable
 from .tensor.type import TensorType, as_tensor_variable
 
@@ -67,10 +68,90 @@ def shared(value, name=None, broadcastable=None):
     return _Shared(t, t.filter(value), name=name)
 
 
+class NanGuardError(FloatingPointError):
+    """A node produced NaN or infinity under ``mode='nan_guard'``."""
+
+
+class CheckModeError(RuntimeError):
+    """``mode='check'`` found an overwritten argument or a result that depends on the rewrites."""
+
+
+def _guarded(perform):
+    """``perform`` followed by a scan of every floating-point result for NaN and infinity: the check of
+    ``NanGuardMode`` (``theano/compile/nanguardmode.py:230-300``), after each node as there."""
+    def run(node, inputs, outs):
+        perform(node, inputs, outs)
+        for k, cell in enumerate(outs):
+            v = cell[0]
+            if v is None or not hasattr(v, "dtype") or np.dtype(v.dtype).kind not in "fc":
+                continue
+            host = v.to_numpy() if hasattr(v, "to_numpy") else np.asarray(v)
+            if host.size and not np.isfinite(host).all():
+                what = "NaN" if np.isnan(host).any() else "Inf"
+                raise NanGuardError("%s in output %d of %s (inputs: %s)" % (
+                    what, k, node, ", ".join("%s%s" % (getattr(i, "dtype", type(i).__name__),
+                                                     tuple(getattr(i, "shape", ()))) for i in inputs)))
+    return run
+
+
+class CheckedFunction(object):
+    """What ``function(..., mode='check')`` returns: the host-side counterpart of the in-place and
+    aliasing checks of ``DebugMode`` (``BadDestroyMap`` / ``BadOptimization``,
+    ``theano/compile/debugmode.py:130-330``).  Every call
+    (1) runs the same graph compiled without fusion, row chains and in-place operation, one kernel per
+        node, on the arguments;
+    (2) runs the optimised function;
+    (3) raises ``CheckModeError`` if an argument's contents changed (an in-place kernel wrote into an
+        array it does not own), or a result or the new value of a shared variable differs between the
+        two beyond ``config.check_mode_tolerance`` (integers and booleans: at all).
+    Meant for debugging: it costs two runs and copies of every argument and result."""
+
+    def __init__(self, primary, reference, n_updates):
+        self.primary, self.reference, self.n_updates = primary, reference, n_updates
+        self.maker = primary
+        self.fgraph = primary.fgraph
+
+    def toposort(self):
+        return self.primary.toposort()
+
+    @staticmethod
+    def _host(v):
+        return v.to_numpy() if hasattr(v, "to_numpy") else np.array(v)
+
+    def __call__(self, *args):
+        before = [self._host(a) for a in args]
+        ref = self.reference(*args)
+        ref = list(ref) if isinstance(ref, (list, tuple)) else [ref]
+        got = self.primary(*args)
+        for k, (a, b) in enumerate(zip(args, before)):
+            now = self._host(a)
+            if now.shape != b.shape or not np.array_equal(now, b, equal_nan=now.dtype.kind in "fc"):
+                raise CheckModeError("argument %d (%s) was overwritten by the call" % (k, self.primary.in_specs[k].name))
+        outs = list(got) if isinstance(got, (list, tuple)) else [got]
+        news = [sv.container[0] for sv in self.primary.update_targets]
+        names = ["output %d" % k for k in range(len(outs))] + ["update of %s" % sv for sv in self.primary.update_targets]
+        for name, g, r in zip(names, outs + news, ref):
+            g, r = self._host(g), self._host(r)
+            if g.shape != r.shape or g.dtype != r.dtype:
+                raise CheckModeError("%s: %s%s with the rewrites, %s%s without" % (name, g.dtype, g.shape, r.dtype, r.shape))
+            if g.dtype.kind in "fc":
+                rtol, atol = config.check_mode_tolerance.get(str(g.dtype), (0.0, 0.0))
+                ok = np.isclose(g, r, rtol=rtol, atol=atol, equal_nan=True)
+            else:
+                ok = g == r
+            if not np.all(ok):
+                bad = tuple(np.argwhere(~np.asarray(ok))[0])
+                raise CheckModeError("%s differs between the optimised function and one kernel per node: %d of %d "
+                                     "values, first at %s: %r against %r" % (name, int((~ok).sum()), ok.size, bad,
+                                                                            g[bad], r[bad]))
+        return got
+
+
 class Function(object):
     """Callable produced by ``function``."""
 
-    def __init__(self, fgraph, in_specs, out_specs, single_output, shared_inputs, update_targets=()):
+    def __init__(self, fgraph, in_specs, out_specs, single_output, shared_inputs, update_targets=(), nan_guard=False):
+        self.nan_guard = nan_guard
         self.update_targets = list(update_targets)
         self.fgraph = fgraph
         self.maker = self  # so that f.maker.fgraph reads as with the reference
@@ -161,7 +242,8 @@ class Function(object):
         self.thunks = []
         for node in self.nodes:
             node.op.prepare_node(node)
-            self.thunks.append((node.op.perform, node, [self.storage[i] for i in node.inputs],
+            self.thunks.append((_guarded(node.op.perform) if self.nan_guard else node.op.perform, node,
+                                [self.storage[i] for i in node.inputs],
                                 [self.storage[o] for o in node.outputs], node in static,
                                 self.release[len(self.thunks)]))
         self._static_key = None
@@ -278,7 +360,7 @@ class Function(object):
 
 
 def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=True, inplace=True, name=None,
-             on_unused_input="raise"):
+             on_unused_input="raise", mode=None):
     """Compile ``outputs`` as a function of ``inputs``.
 
     ``inputs``: variables or ``In`` instances.  A host-typed input may be given
@@ -293,7 +375,10 @@ def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=Tru
     have a HIP implementation.  ``fuse=False``
     keeps one kernel per graph node; ``rowchain=False`` keeps elementwise /
     row-reduction islands as separate fused kernels; ``inplace=False`` gives
-    every elementwise result a buffer of its own."""
+    every elementwise result a buffer of its own.  ``mode``: None, ``'nan_guard'`` (every node's
+    floating-point results are scanned for NaN / infinity, ``NanGuardError``) or ``'check'`` (see
+    ``CheckedFunction``: arguments must come back unchanged and results must not depend on fusion or
+    in-place operation)."""
     from .hip import opt as hip_opt
     from .hip.ops import HipArrayType, as_hip_variable
 
@@ -360,8 +445,18 @@ def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=Tru
     c_in = [memo[v] for v in in_vars]
     c_out = [memo[v] for v in out_vars]
     fgraph = _SharedAwareGraph(c_in, c_out, shared_inputs)
+    if mode not in (None, "nan_guard", "check"):
+        raise ValueError("mode must be None, 'nan_guard' or 'check'", mode)
     fgraph = hip_opt.optimize(fgraph, fuse=fuse, rowchain=rowchain, inplace=inplace)
-    return Function(fgraph, in_specs, out_specs, single, shared_inputs, update_targets)
+    primary = Function(fgraph, in_specs, out_specs, single, shared_inputs, update_targets, nan_guard=mode == "nan_guard")
+    if mode != "check":
+        return primary
+    # the same outputs and new shared values, as plain results of a function without the rewrites
+    ref_outs = [Out(v, device=spec.device) for v, spec in zip(out_vars, out_specs)]
+    ref_outs += [Out(v, device=True) for v in out_vars[len(out_specs):]]
+    reference = function(in_specs, ref_outs, givens=None, fuse=False, rowchain=False, inplace=False,
+                         on_unused_input="ignore")
+    return CheckedFunction(primary, reference, len(update_targets))
 
 
 class _SharedAwareGraph(FunctionGraph):

@@ -28,6 +28,12 @@ class _Config(object):
     # (float64 accumulators only), and the two reductions then share one pass over memory
     merge_dependent_reductions = True
 
+    # function(..., mode="check"): how far a result of the optimised function may be from the same graph run
+    # one kernel per node, (rtol, atol) by result dtype.  A fused kernel keeps in float32 registers what the
+    # separate kernels round to the storage type in between, hence the width of the float16 entry.
+    check_mode_tolerance = {"float16": (1e-2, 1e-2), "float32": (1e-4, 1e-5), "float64": (1e-9, 1e-10),
+                            "complex64": (1e-4, 1e-5), "complex128": (1e-9, 1e-10)}
+
     @contextlib.contextmanager
     def change_flags(self, **kw):
         old = {k: getattr(self, k) for k in kw}
