@@ -326,9 +326,9 @@ def evaluate(inputs, outputs, values, wide=False):
                 x[idx] += args[1]
             res = [x]
         elif isinstance(op, V.Reshape):
-            res = [np.reshape(args[0], op.resolve([a.shape for a in args]))]
+            res = [np.reshape(args[0], op.resolve([a.shape for a in args], args))]
         elif isinstance(op, V.Alloc):
-            res = [np.array(np.broadcast_to(args[0], op.resolve([a.shape for a in args])))]
+            res = [np.array(np.broadcast_to(args[0], op.resolve([a.shape for a in args], args)))]
         elif isinstance(op, V.Join):
             res = [np.concatenate(args, axis=op.axis)]
         elif isinstance(op, V.Rebroadcast):        # theano/compile/ops.py:711-722

@@ -128,7 +128,41 @@ def test_shape_entries_are_symbolic_scalars():
             assert_parity(g, r, "shape arithmetic", tol=TOL["float32"])
         assert np.allclose(got[0], xv.astype("float64").sum(0) / shape[0]) and got[3].shape == shape[::-1]
     with pytest.raises(TypeError):
-        x.reshape((n * m,))               # arithmetic on extents is not a shape entry
+        x.reshape((T.sum(x),))            # a float is not a shape entry
+
+
+@pytest.mark.gpu
+def test_shapes_computed_from_extents_and_scalar_arguments():
+    """reshape / alloc take arithmetic over extents (evaluated on the host from array metadata) and integer scalar
+    variables (read on the host when the function runs): the idioms x.reshape((x.shape[0], -1)),
+    x.reshape((x.shape[0], x.shape[1] * x.shape[2])), alloc(0., n, m + 1) of theano/tensor/basic.py:2769-2960,
+    4701-4920, with the gradient flowing back through the reshape."""
+    rng = np.random.default_rng(4)
+    x = T.ftensor3("x")
+    n, m = T.iscalar("n"), T.lscalar("m")
+    outs = [x.reshape((x.shape[0], x.shape[1] * x.shape[2])), x.reshape((x.shape[0] * x.shape[1] // 2, 2, -1)),
+            T.alloc(np.float32(1.5), x.shape[0] + 1, n, T.maximum(m, 2)), x.reshape((n, -1)) * 2,
+            T.alloc(x[0, 0], n * 2 - 1, x.shape[2]), x.flatten(2).reshape((x.shape[0], x.shape[1], x.shape[2])) + 1,
+            T.alloc(np.float32(0), T.minimum(x.shape[0], x.shape[1]) % 3, 4)]
+    f = th.function([x, n, m], outs)
+    for shape, nv, mv in (((4, 6, 5), 8, 3), ((2, 8, 3), 4, 1), ((6, 2, 7), 12, 9)):
+        xv = rng.standard_normal(shape).astype("float32")
+        got = f(xv, np.int32(nv), np.int64(mv))
+        ref = G.evaluate([x, n, m], outs, [xv, np.int32(nv), np.int64(mv)])
+        for g, r in zip(got, ref):
+            assert_parity(g, r, "computed shapes %s" % (shape,))
+        assert got[0].shape == (shape[0], shape[1] * shape[2]) and got[2].shape == (shape[0] + 1, nv, max(mv, 2))
+        assert np.array_equal(got[3], xv.reshape(nv, -1) * 2)
+    with pytest.raises(ValueError):
+        f(np.zeros((4, 6, 5), "float32"), np.int32(7), np.int64(3))        # 120 elements do not split into 7 rows
+    with pytest.raises(ValueError):
+        th.function([x, n], T.alloc(np.float32(0), n - 5, 2))(np.zeros((1, 1, 1), "float32"), np.int32(3))
+    # the gradient goes back through a computed shape
+    w = T.fmatrix("w")
+    cost = T.sum(T.sqr(x.reshape((x.shape[0], x.shape[1] * x.shape[2])) * w))
+    gx = th.function([x, w], th.grad(cost, x))
+    xv, wv = rng.standard_normal((3, 4, 5)).astype("float32"), rng.standard_normal((3, 20)).astype("float32")
+    assert np.allclose(gx(xv, wv), (2 * xv.reshape(3, 20) * wv * wv).reshape(3, 4, 5), rtol=1e-5)
 
 
 @pytest.mark.gpu

@@ -137,7 +137,7 @@ class HipReshape(V.Reshape):
 
     def perform(self, node, inputs, output_storage):
         x = inputs[0]
-        shape = self.resolve([np.shape(v) if not isinstance(v, HipArray) else v.shape for v in inputs])
+        shape = self.resolve([np.shape(v) if not isinstance(v, HipArray) else v.shape for v in inputs], inputs)
         if not x.c_contiguous:
             flat = HipArray.empty(x.shape, x.dtype)
             copy_into(x, flat)
@@ -159,7 +159,7 @@ class HipAlloc(V.Alloc):
 
     def perform(self, node, inputs, output_storage):
         v = inputs[0]
-        shape = self.resolve([np.shape(i) if not isinstance(i, HipArray) else i.shape for i in inputs])
+        shape = self.resolve([np.shape(i) if not isinstance(i, HipArray) else i.shape for i in inputs], inputs)
         dtype = np.dtype(node.outputs[0].type.dtype)
         vs = v.shape if isinstance(v, HipArray) else np.shape(v)
         for a, b in zip(reversed(vs), reversed(shape)):

@@ -158,8 +158,12 @@ class _tensor_py_operators(object):
 
     def reshape(self, *shape):
         from . import views
-        if len(shape) == 1 and isinstance(shape[0], (list, tuple)) and views._extent_entry(shape[0]) is None:
-            shape = tuple(shape[0])
+        one = shape[0] if len(shape) == 1 else None
+        is_pair = (isinstance(one, (list, tuple)) and len(one) == 2 and hasattr(one[0], "type") and
+                   isinstance(one[1], (int, np.integer)) and
+                   0 <= one[1] < getattr(one[0].type, "ndim", 0))   # x.reshape((v, d)): the extent of v along d
+        if isinstance(one, (list, tuple)) and not is_pair:
+            shape = tuple(one)
         return views.reshape(self, shape)
 
     def fill(self, value):

@@ -13,6 +13,7 @@ view costs nothing and a copy is one elementwise kernel.
 """
 import numpy as np
 
+from .. import scalar as scal
 from ..gof import Apply, Op
 from . import basic as T
 from .type import TensorType, as_tensor_variable
@@ -309,26 +310,95 @@ def set_subtensor(x, y, idx=None):
 
 
 # --------------------------------------------------------------------------
+# --------------------------------------------------------------------------
+# Entries of the shape patterns of Reshape and Alloc:
+#   n               a plain extent (Reshape: -1 = inferred)
+#   (k, d)          the extent of dimension d of input k
+#   ("in", k)       the value of input k, an integer scalar read on the host when the function runs
+#   (op, a, b)      op in _SHAPE_OPS over two entries: arithmetic on extents, evaluated on the host from array
+#                   metadata (x.reshape((x.shape[0], x.shape[1] * x.shape[2])), alloc(0., n // 2, m + 1), ...)
+_SHAPE_OPS = {"add": lambda a, b: a + b, "sub": lambda a, b: a - b, "mul": lambda a, b: a * b,
+              "floordiv": lambda a, b: a // b, "mod": lambda a, b: a % b, "max": max, "min": min}
+
+
+def _norm_entry(p, allow_unknown):
+    if isinstance(p, tuple):
+        if len(p) == 2 and p[0] == "in":
+            return ("in", int(p[1]))
+        if len(p) == 3 and p[0] in _SHAPE_OPS:
+            return (p[0], _norm_entry(p[1], False), _norm_entry(p[2], False))
+        if len(p) == 2 and not isinstance(p[0], str):
+            return (int(p[0]), int(p[1]))
+        raise ValueError("invalid shape entry %r" % (p,))
+    p = int(p)
+    if p < (-1 if allow_unknown else 0):
+        raise ValueError("invalid extent %d in a shape" % p)
+    return p
+
+
+def _entry_inputs(p):
+    """Indices of the node inputs an entry reads."""
+    if not isinstance(p, tuple):
+        return []
+    if p[0] == "in":
+        return [p[1]]
+    if p[0] in _SHAPE_OPS:
+        return _entry_inputs(p[1]) + _entry_inputs(p[2])
+    return [p[0]]
+
+
+def _eval_entry(p, shapes, values):
+    if not isinstance(p, tuple):
+        return p
+    if p[0] == "in":
+        if values is None:
+            raise ValueError("this shape depends on the value of an input, not only on shapes")
+        v = values[p[1]]
+        return int(np.asarray(v.to_numpy() if hasattr(v, "to_numpy") else v).reshape(()))
+    if p[0] in _SHAPE_OPS:
+        return int(_SHAPE_OPS[p[0]](_eval_entry(p[1], shapes, values), _eval_entry(p[2], shapes, values)))
+    return int(shapes[p[0]][p[1]])
+
+
+def _entry_str(p):
+    if not isinstance(p, tuple):
+        return str(p)
+    if p[0] == "in":
+        return "in%d" % p[1]
+    if p[0] in _SHAPE_OPS:
+        return "%s(%s, %s)" % (p[0], _entry_str(p[1]), _entry_str(p[2]))
+    return "in%d.shape[%d]" % p
+
+
+def _entry_broadcastable(p, ins):
+    if isinstance(p, tuple):
+        return ins[p[0]].type.broadcastable[p[1]] if not isinstance(p[0], str) else False
+    return p == 1
+
+
+def _check_entries(pattern, ins):
+    for p in pattern:
+        for k in _entry_inputs(p):
+            if k >= len(ins):
+                raise ValueError("shape entry %s refers to a missing input" % _entry_str(p))
+    for p in pattern:
+        if isinstance(p, tuple) and not isinstance(p[0], str) and p[1] >= ins[p[0]].type.ndim:
+            raise ValueError("shape entry %s refers to a missing input dimension" % (p,))
+
+
 class Reshape(Op):
     """``x`` with a new shape (``theano/tensor/basic.py:4701-4920``).  ``pattern``
     has one entry per output dimension: a non-negative int, ``-1`` (at most one,
-    inferred) or ``(k, d)``: the extent of dimension ``d`` of input ``k``.
-    Inputs after the first are read for their shape only.  A view when the
+    inferred), ``(k, d)``: the extent of dimension ``d`` of input ``k``, ``("in", k)``: the
+    run-time value of the integer scalar input ``k``, or arithmetic over such entries.
+    Inputs after the first are read for their shape (or scalar value) only.  A view when the
     input is C-contiguous, else a copy."""
 
     __props__ = ("pattern",)
     view_map = {0: [0]}
 
     def __init__(self, pattern):
-        pat = []
-        for p in pattern:
-            if isinstance(p, tuple):
-                pat.append((int(p[0]), int(p[1])))
-            else:
-                p = int(p)
-                if p < -1:
-                    raise ValueError("invalid extent %d in a shape" % p)
-                pat.append(p)
+        pat = [_norm_entry(p, True) for p in pattern]
         if sum(1 for p in pat if p == -1) > 1:
             raise ValueError("can only specify one unknown dimension")
         self.pattern = tuple(pat)
@@ -337,30 +407,25 @@ class Reshape(Op):
         return (self.pattern,)
 
     def __str__(self):
-        return "%s{%s}" % (type(self).__name__, ", ".join(
-            "in%d.shape[%d]" % p if isinstance(p, tuple) else str(p) for p in self.pattern))
+        return "%s{%s}" % (type(self).__name__, ", ".join(_entry_str(p) for p in self.pattern))
 
     def make_node(self, x, *like):
         ins = [as_tensor_variable(x)] + [as_tensor_variable(v) for v in like]
-        bcast = []
-        for p in self.pattern:
-            if isinstance(p, tuple):
-                k, d = p
-                if k >= len(ins) or d >= ins[k].type.ndim:
-                    raise ValueError("shape entry %s refers to a missing input dimension" % (p,))
-                bcast.append(ins[k].type.broadcastable[d])
-            else:
-                bcast.append(p == 1)
+        _check_entries(self.pattern, ins)
+        bcast = [_entry_broadcastable(p, ins) for p in self.pattern]
         return Apply(self, ins, [TensorType(ins[0].type.dtype, bcast)()])
 
-    def resolve(self, shapes):
-        """The concrete output shape given the inputs' shapes."""
+    def resolve(self, shapes, values=None):
+        """The concrete output shape given the inputs' shapes (and, for entries that read an input's value,
+        the inputs themselves)."""
         total = 1
         for s in shapes[0]:
             total *= s
         out, known, unknown = [], 1, None
         for j, p in enumerate(self.pattern):
-            v = shapes[p[0]][p[1]] if isinstance(p, tuple) else p
+            v = _eval_entry(p, shapes, values)
+            if v < -1 or (v == -1 and isinstance(p, tuple)):
+                raise ValueError("negative extent %d from shape entry %s" % (v, _entry_str(p)))
             if v == -1:
                 unknown = j
                 out.append(-1)
@@ -398,50 +463,72 @@ class Reshape(Op):
         return [[True]] + [[False]] * (len(node.inputs) - 1)
 
 
-def _extent_entry(p):
-    """A shape entry that names a run-time extent: ``v.shape[d]`` (a Shape_i variable) or the
-    pair ``(v, d)``; returns that pair, or None for anything else."""
-    if isinstance(p, (tuple, list)):
-        if (len(p) == 2 and hasattr(p[0], "type") and isinstance(p[1], (int, np.integer)) and
-                0 <= p[1] < getattr(p[0].type, "ndim", 0)):
-            return tuple(p)
-        return None
-    if hasattr(p, "owner"):
-        if p.owner is not None and isinstance(p.owner.op, T.ShapeFloat):
-            return (p.owner.inputs[0], p.owner.op.i)
-        if hasattr(p, "data") and p.type.ndim == 0:
-            return None
-        raise TypeError("a symbolic shape entry must be a constant or some tensor's shape[d]; arithmetic on "
-                        "extents is not supported here: %s" % p)
-    return None
+class _ShapeArgs(object):
+    """Collects the inputs a shape pattern refers to while the entries given by the caller are
+    translated: tensors whose extents are read, and integer scalars read for their value."""
 
+    def __init__(self, first=None):
+        self.ins = [] if first is None else [first]
+        self.base = 1 if first is None else 0      # Alloc's input 0 is the value, never a shape source
 
-def _int_entry(p):
-    return int(np.asarray(p.data)) if hasattr(p, "data") else int(p)
+    def index(self, v):
+        for k, u in enumerate(self.ins):
+            if u is v:
+                return k + self.base
+        self.ins.append(v)
+        return len(self.ins) - 1 + self.base
+
+    def extra(self):
+        return self.ins[1:] if self.base == 0 else self.ins
+
+    def entry(self, p):
+        """The pattern entry for one element of a shape argument: an int, ``v.shape[d]``, a pair ``(v, d)``,
+        an integer scalar variable, or arithmetic (+ - * // % maximum minimum) over those."""
+        from .elemwise import DimShuffle, Elemwise
+        if isinstance(p, (tuple, list)):
+            if (len(p) == 2 and hasattr(p[0], "type") and isinstance(p[1], (int, np.integer)) and
+                    0 <= p[1] < getattr(p[0].type, "ndim", 0)):
+                return (self.index(as_tensor_variable(p[0])), int(p[1]))
+            raise TypeError("invalid shape entry %r" % (p,))
+        if not hasattr(p, "owner"):
+            return int(p)
+        if hasattr(p, "data"):
+            if np.asarray(p.data).size != 1:
+                raise TypeError("a shape entry must be a scalar: %s" % p)
+            return int(np.asarray(p.data).reshape(()))
+        dt = getattr(p.type, "dtype", "")
+        if not all(p.type.broadcastable) or not (dt.startswith("int") or dt.startswith("uint")):
+            raise TypeError("a symbolic shape entry must be an integer scalar, got %s" % (p.type,))
+        node = p.owner
+        if node is not None:
+            if isinstance(node.op, T.ShapeFloat):
+                return (self.index(node.inputs[0]), node.op.i)
+            if isinstance(node.op, DimShuffle):
+                return self.entry(node.inputs[0])
+            if isinstance(node.op, Elemwise):
+                sop = node.op.scalar_op
+                name = {scal.Add: "add", scal.Mul: "mul", scal.Sub: "sub", scal.IntDiv: "floordiv", scal.Mod: "mod",
+                        scal.Maximum: "max", scal.Minimum: "min"}.get(type(sop))
+                if isinstance(sop, (scal.Cast, scal.Identity)):
+                    return self.entry(node.inputs[0])
+                if name is not None and len(node.inputs) >= 2:
+                    e = self.entry(node.inputs[0])
+                    for other in node.inputs[1:]:
+                        e = (name, e, self.entry(other))
+                    return e
+        return ("in", self.index(p))
 
 
 def reshape(x, newshape):
-    """``newshape``: ints, at most one -1, or ``v.shape[d]`` entries."""
+    """``newshape``: ints, at most one -1, ``v.shape[d]`` entries, integer scalar variables (read on the host
+    when the function runs) and arithmetic over those (``theano/tensor/basic.py:4701-4920`` takes any integer
+    vector; here the entries are given one by one)."""
     x = as_tensor_variable(x)
     if isinstance(newshape, (int, np.integer)) or hasattr(newshape, "owner"):
         newshape = (newshape,)
-    like, pattern = [], []
-    for p in newshape:
-        e = _extent_entry(p)
-        if e is not None:
-            p = e
-        if isinstance(p, tuple):
-            v, d = p
-            v = as_tensor_variable(v)
-            if v is x:
-                pattern.append((0, int(d)))
-            else:
-                if v not in like:
-                    like.append(v)
-                pattern.append((1 + like.index(v), int(d)))
-        else:
-            pattern.append(_int_entry(p))
-    return Reshape(pattern)(x, *like)
+    args = _ShapeArgs(x)
+    pattern = [args.entry(p) for p in newshape]
+    return Reshape(pattern)(x, *args.extra())
 
 
 def flatten(x, ndim=1):
@@ -464,35 +551,28 @@ class Alloc(Op):
     __props__ = ("pattern",)
 
     def __init__(self, pattern):
-        pat = []
-        for p in pattern:
-            if isinstance(p, tuple):
-                pat.append((int(p[0]), int(p[1])))
-            else:
-                if int(p) < 0:
-                    raise ValueError("invalid extent %d in a shape" % int(p))
-                pat.append(int(p))
-        self.pattern = tuple(pat)
+        self.pattern = tuple(_norm_entry(p, False) for p in pattern)
 
     def _props(self):
         return (self.pattern,)
 
     def __str__(self):
-        return "%s{%s}" % (type(self).__name__, ", ".join(
-            "in%d.shape[%d]" % p if isinstance(p, tuple) else str(p) for p in self.pattern))
+        return "%s{%s}" % (type(self).__name__, ", ".join(_entry_str(p) for p in self.pattern))
 
     def make_node(self, value, *like):
         ins = [as_tensor_variable(value)] + [as_tensor_variable(v) for v in like]
         v = ins[0]
         if v.type.ndim > len(self.pattern):
             raise TypeError("the value has more dimensions (%d) than the shape (%d)" % (v.type.ndim, len(self.pattern)))
-        bcast = []
-        for p in self.pattern:
-            bcast.append(ins[p[0]].type.broadcastable[p[1]] if isinstance(p, tuple) else p == 1)
+        _check_entries(self.pattern, ins)
+        bcast = [_entry_broadcastable(p, ins) for p in self.pattern]
         return Apply(self, ins, [TensorType(v.type.dtype, bcast)()])
 
-    def resolve(self, shapes):
-        return tuple(int(shapes[p[0]][p[1]]) if isinstance(p, tuple) else p for p in self.pattern)
+    def resolve(self, shapes, values=None):
+        out = tuple(_eval_entry(p, shapes, values) for p in self.pattern)
+        if any(v < 0 for v in out):
+            raise ValueError("negative extent in shape %s" % (out,))
+        return out
 
     def infer_shape(self, node, shapes):
         return [self.resolve(shapes)]
@@ -524,20 +604,10 @@ class Alloc(Op):
 
 
 def alloc(value, *shape):
-    """``shape`` entries: ints or ``v.shape[d]``."""
-    like, pattern = [], []
-    for p in shape:
-        e = _extent_entry(p)
-        if e is not None:
-            p = e
-        if isinstance(p, tuple):
-            v = as_tensor_variable(p[0])
-            if v not in like:
-                like.append(v)
-            pattern.append((1 + like.index(v), int(p[1])))
-        else:
-            pattern.append(_int_entry(p))
-    return Alloc(pattern)(value, *like)
+    """``shape`` entries: ints, ``v.shape[d]``, integer scalar variables, arithmetic over those."""
+    args = _ShapeArgs()
+    pattern = [args.entry(p) for p in shape]
+    return Alloc(pattern)(value, *args.extra())
 
 
 # --------------------------------------------------------------------------
