@@ -465,6 +465,15 @@ def test_bessel_functions_of_real_order_against_scipy(dtype):
     with np.errstate(all="ignore"):
         assert np.isclose(got[0], scipy.special.jv(pv, px).astype(dtype), rtol=tol["rtol"], atol=0, equal_nan=True).all()
         assert np.isclose(got[1], scipy.special.iv(pv, px).astype(dtype), rtol=tol["rtol"], atol=0, equal_nan=True).all()
+    if dtype == "float64":
+        # large arguments (Hankel's expansion): against a 40-digit evaluation, SciPy itself drifts there
+        mpmath = pytest.importorskip("mpmath")
+        mpmath.mp.dps = 40
+        bx = rng.uniform(1e3, 1e7, 60)
+        bv = rng.uniform(-1, 1, 60) * np.sqrt(bx)
+        truth = np.array([float(mpmath.besselj(mpmath.mpf(float(a)), mpmath.mpf(float(b)))) for a, b in zip(bv, bx)])
+        big = th.function([v, x], T.jv(v, x))(bv, bx)
+        assert (np.abs(big - truth) / np.sqrt(2 / (np.pi * bx))).max() < 1e-12
     # gradient with respect to the argument; none with respect to the order
     gv = rng.uniform(0.2, 6, 2000).astype(dtype)
     gx = rng.uniform(0.2, 15, 2000).astype(dtype)

@@ -49,6 +49,17 @@ def test_bessel_of_real_order(host, name):
     v, x = rng.integers(-6, 7, n).astype("float64"), rng.uniform(-20, 20, n)       # whole orders take any argument
     got, want = _bessel(host, "host_" + name, v, x), ref(v, x)
     assert (np.abs(got - want) / (1 + np.abs(want))).max() < 1e-13
+    if name == "jv":
+        # large arguments take Hankel's expansion; SciPy itself drifts there (1e-9 of the envelope at x = 1e6 and
+        # nothing right beyond 1e8), so the truth is mpmath's
+        mpmath = pytest.importorskip("mpmath")
+        mpmath.mp.dps = 40
+        for lo, hi in ((30, 100), (1e3, 1e5), (1e5, 1e7), (1e7, 1e9)):
+            x = rng.uniform(lo, hi, 40)
+            v = rng.uniform(-1, 1, 40) * np.sqrt(x)
+            truth = np.array([float(mpmath.besselj(mpmath.mpf(float(a)), mpmath.mpf(float(b)))) for a, b in zip(v, x)])
+            got = _bessel(host, "host_jv", v, x)
+            assert (np.abs(got - truth) / np.sqrt(2 / (np.pi * x))).max() < 5e-14, (lo, hi)
     pv = np.array([0, 1, 2.5, -1, -0.5, -1.5, -2.5, 0.5, np.nan, 1])
     px = np.array([0, 0, 0, 0, 0, 0, 0, -1.0, 1, np.nan])
     assert np.array_equal(_bessel(host, "host_" + name, pv, px), ref(pv, px), equal_nan=True)

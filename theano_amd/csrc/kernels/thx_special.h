@@ -427,6 +427,35 @@ __device__ inline thx_bessel_pair thx_bessel_ik(double v, double x) {   // v >= 
   return out;
 }
 
+// Hankel's asymptotic expansion, for x >= 30 and x >= v^2 (any real v): sqrt(2 / (pi x)) (P cos chi - Q sin chi),
+// chi = x - (v / 2 + 1 / 4) pi, P and Q the even and odd terms of sum_k a_k(v) / x^k with
+// a_k = (4 v^2 - 1)(4 v^2 - 9)...(4 v^2 - (2k - 1)^2) / (k! 8^k).  In that range the terms fall below 1e-17 of the
+// sum long before they start to grow (at k ~ 2x).  cos and sin of chi come from those of x and of the order's part
+// separately: forming chi first would lose the digits of the order's part in a large x.  The continued fraction
+// of the general route takes about x iterations and loses accuracy with each, so it stops here.
+__device__ inline double thx_jv_large_x(double v, double x) {
+  const double pi = 3.14159265358979323846, mu = 4.0 * v * v;
+  double term = 1.0, P = 1.0, Q = 0.0;
+  for (int k = 1; k < 200; ++k) {
+    const double odd = 2.0 * k - 1.0;
+    const double next = term * (mu - odd * odd) / (8.0 * k * x);
+    if (fabs(next) > fabs(term) && k > 1) break;
+    term = next;
+    // k = 1, 2, 3, 4, ...: Q +, P -, Q -, P +
+    if (k & 1) Q += (k & 2) ? -term : term;
+    else P += (k & 2) ? -term : term;
+    if (fabs(term) < 1e-17 * (fabs(P) + fabs(Q))) break;
+  }
+  double sx, cx, sa, ca;
+  sincos(x, &sx, &cx);
+  // (v / 2 + 1 / 4) pi reduced by whole turns first: v / 2 + 1 / 4 = n + f with |f| <= 1 (two turns are 4 in these units)
+  const double h = 0.5 * v + 0.25;
+  const double f = h - 2.0 * floor(h * 0.5);       // in [0, 2): whole multiples of 2 pi dropped exactly
+  sincos(f * pi, &sa, &ca);
+  const double cchi = cx * ca + sx * sa, schi = sx * ca - cx * sa;
+  return sqrt(2.0 / (pi * x)) * (P * cchi - Q * schi);
+}
+
 // J_v(x) for any real order and argument.
 __device__ inline double thx_jv(double v, double x) {
   if (isnan(v) || isnan(x)) return NAN;
@@ -442,6 +471,7 @@ __device__ inline double thx_jv(double v, double x) {
     return copysign(INFINITY, tgamma(v + 1.0));   // (x / 2)^v / Gamma(v + 1) diverges for non-whole v < 0
   }
   if (isinf(x)) return 0.0;
+  if (x >= 30.0 && x >= v * v) return thx_jv_large_x(v, x);
   if (v >= 0.0) return thx_bessel_jy(v, x).first;
   const double a = -v;
   const thx_bessel_pair p = thx_bessel_jy(a, x);
