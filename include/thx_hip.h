@@ -228,6 +228,15 @@ int thx_rowchain_new(const char* functor_src, const char* functor_name, int n_in
  * unfused nodes - when rows are not unit-stride, leading dimensions do not
  * collapse to one row stride, or a row exceeds 16384 vector slots. */
 int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* outs, int flags);
+/* Reductions of the chain run over `axes` of the full shape instead of its last axis: reduced axes
+ * may lie before and after one run of adjacent kept axes (axes (0, 2, 3) of [N, C, H, W] keep C, the
+ * batch-normalisation statistics of theano/tensor/nnet/bn.py:364-760), and at least one must trail
+ * them. ROW operands then hold one value per kept index (extent 1 on every reduced axis, or the
+ * kept axes alone); COL operands are not taken. Such chains run in the held form only (one block per
+ * kept index keeps that index's whole reduce domain on chip, kernels/thx_rowchain.h), which
+ * thx_rowchain_call refuses with THX_ERR_UNSUPPORTED when a reduce domain exceeds what one compute
+ * unit's registers and LDS hold or when there are too few kept indices to occupy the device. */
+int thx_rowchain_set_axes(thx_rowchain* c, int n_axes, const int32_t* axes);
 int thx_rowchain_free(thx_rowchain* c);
 
 /* ---- inspection and timing ------------------------------------------------ */

@@ -279,10 +279,12 @@ def test_softmax_ops_and_the_rewrites_that_produce_them():
 
 
 def test_rows_too_long_for_one_block_and_strided_rows_take_the_fused_multi_kernel_path():
-    """Softmax, log-softmax and their gradients on rows of 100 000 elements (beyond what one block keeps in
-    registers) and on a transposed operand: the row-chain node then runs its island as reductions with fused
-    prologues / epilogues - 3 launches for a softmax - with the same results.  Rows of 50 000 elements still
-    fit one block of 1024 threads."""
+    """Softmax, log-softmax and their gradients on long rows and on a transposed operand.  Rows of 50 000
+    float32 elements fit the registers of one block of 1024 threads; rows of 100 000 stay on chip in the
+    held form (registers plus LDS, per-element values recomputed in every pass over them); rows of 250 000
+    are beyond one compute unit, and the row-chain node then runs its island as reductions with fused
+    prologues / epilogues - 3 launches for a softmax - with the same results."""
+    from theano_amd import hip
     from theano_amd.hip import HipRowChain
     rng = np.random.default_rng(43)
     x, y = T.fmatrix("x"), T.fmatrix("y")
@@ -291,31 +293,43 @@ def test_rows_too_long_for_one_block_and_strided_rows_take_the_fused_multi_kerne
     f = th.function([x, y], outs)
     chains = [n for n in f.toposort() if isinstance(n.op, HipRowChain)]
     assert chains
-    for cols in (50000, 100000):
+    for cols, form in ((50000, "|rw|"), (100000, "|rh|"), (250000, None)):
         xv = (3 * rng.standard_normal((6, cols))).astype("float32")
         ev = np.exp(xv.astype("float64") - xv.max(axis=1, keepdims=True))
         one = th.function([x], sm)
         assert np.allclose(one(xv), ev / ev.sum(axis=1, keepdims=True), rtol=2e-5, atol=1e-9), cols
         (chain,) = [n for n in one.toposort() if isinstance(n.op, HipRowChain)]
-        assert (getattr(chain.op, "_fallback_plan", None) is None) == (cols == 50000)
+        assert (getattr(chain.op, "_fallback_function", None) is None) == (form is not None)
+        if form:
+            assert form in hip.last_plan(), (cols, hip.last_plan())
     yv = rng.uniform(0, 1, xv.shape).astype("float32")
     got = f(xv, yv)
     ref = G.evaluate([x, y], outs, [xv, yv])
     truth = G.evaluate([x, y], outs, [xv, yv], wide=True)
-    # Softmax.perform and SoftmaxGrad.perform add a row's 100 000 float32 terms one by one in float32
-    # (nnet.py:321, 443; the gradient is off by 6e-5 here); the device accumulates in double like the ops'
+    # Softmax.perform and SoftmaxGrad.perform add a row's 250 000 float32 terms one by one in float32
+    # (nnet.py:321, 443); the device accumulates in double like the ops'
     # C code (nnet.py:396): held to the float64 value, no farther from it than the oracle is
     for k, (g, r, w) in enumerate(zip(got, ref, truth)):
         assert_within_reference_error(g, r, w, "long rows, output %d" % k)
     assert np.allclose(got[0].sum(axis=1), 1.0, atol=1e-5)
-    plans = [n.op._fallback_plan for n in chains if getattr(n.op, "_fallback_plan", None) is not None]
+    plans = [n.op._fallback_function for n in chains if getattr(n.op, "_fallback_function", None) is not None]
     assert plans, "the one-kernel form was not expected to take these rows"
     # the softmax alone: row max, sum of exp (prologue-fused), normalise
     g = th.function([x], sm)
     g(xv)
     (chain,) = [n for n in g.toposort() if isinstance(n.op, HipRowChain)]
-    kinds = [type(n.op).__name__ for n in chain.op._fallback_plan[2] if type(n.op).__name__ != "HipDimShuffle"]
+    kinds = [type(n.op).__name__ for n in chain.op._fallback_function.toposort() if type(n.op).__name__ != "HipDimShuffle"]
     assert sorted(kinds) == ["HipCAReduce", "HipCAReduce", "HipElemwise"], kinds
+    # softmax and log-softmax of rows of 100 000 in one held chain
+    xh = (3 * rng.standard_normal((6, 100000))).astype("float32")
+    outs2 = [sm, T.nnet.logsoftmax(x)]
+    f2 = th.function([x], outs2)
+    got = f2(xh)
+    assert "|rh|" in hip.last_plan()
+    ref = G.evaluate([x], outs2, [xh])
+    truth = G.evaluate([x], outs2, [xh], wide=True)
+    for k, (g_, r, w) in enumerate(zip(got, ref, truth)):
+        assert_within_reference_error(g_, r, w, "held rows, output %d" % k)
     # rows that are not contiguous: the same function on a transposed view
     z = T.fmatrix("z")
     h = th.function([z], T.nnet.softmax(z.T))

@@ -1,6 +1,8 @@
 """Host-side mirror of the reference's Op interface: node construction, type
 inference, error behaviour, gradients' graph structure and what the rewrite
 pipeline (lift + fuse) produces."""
+import os
+
 import numpy as np
 import pytest
 
@@ -228,7 +230,9 @@ def test_batchnorm_gradient_is_one_statistics_pass_and_one_elementwise_pass(dry_
         return [n for n in f.toposort() if isinstance(n.op, (HipElemwise, HipCAReduce)) and
                 any(not any(i.type.broadcastable) for i in n.inputs if hasattr(i.type, "broadcastable") and i.type.ndim)]
 
-    f = th.function(ins, [th.Out(o, device=True) for o in outs])
+    # (the form that runs when a channel's elements do not fit on chip; otherwise the whole graph is one held chain)
+    with th.config.change_flags(held_chains=False):
+        f = th.function(ins, [th.Out(o, device=True) for o in outs])
     kernels = kernels_of(f)
     assert [type(n.op) for n in kernels] == [HipCAReduce, HipElemwise]
     stats = kernels[0]
@@ -240,9 +244,52 @@ def test_batchnorm_gradient_is_one_statistics_pass_and_one_elementwise_pass(dry_
     assert len(kernels[0].tag["reused_in"]) >= 2 and len(kernels[1].tag["reused_in"]) == 0
     small = workloads.c5_inputs("small")
     f(*small)                                      # plans and compiles every kernel (dry run)
-    with th.config.change_flags(merge_dependent_reductions=False):
+    with th.config.change_flags(merge_dependent_reductions=False, held_chains=False):
         g = th.function(ins, [th.Out(o, device=True) for o in outs])
     assert [type(n.op) for n in kernels_of(g)] == [HipCAReduce, HipCAReduce, HipElemwise]
+
+
+def test_batchnorm_graphs_become_one_held_chain(dry_run):
+    """Per-channel statistics followed by the normalisation (reductions over axes (0, 2, 3) whose results
+    feed elementwise work on the same array) form one HipRowChain over those axes: the kernel keeps each
+    channel's elements on chip between the statistics and the store.  The three sums of the forward graph
+    share one loop, the store is the second; a graph that only takes the statistics reads its operand once
+    either way and stays with the reduction kernels.  When a call's shapes are turned away the chain runs
+    its island as the separate kernels of the test above."""
+    import workloads
+    from theano_amd import hip
+    from theano_amd.hip.rowchain import HipRowChain
+    ins, outs = workloads.c5_graph(with_grad=False)
+    f = th.function(ins, [th.Out(o, device=True) for o in outs])
+    (chain,) = ops_of(f, HipRowChain)
+    assert chain.op.program.axes == (0, 2, 3) and chain.op.program.held_passes == 2
+    assert " void held(" in chain.op.src and " void row(" not in chain.op.src
+    assert not ops_of(f, HipCAReduce) and not ops_of(f, HipElemwise)
+    f(*workloads.c5_inputs("small", with_grad=False))
+    assert "|rh|" in hip.last_plan()
+    # statistics alone: nothing to keep the values for
+    x = ins[0]
+    xf = T.cast(x, "float32")
+    mean = T.mean(xf, axis=(0, 2, 3), keepdims=True)
+    var = T.mean(T.sqr(xf - mean), axis=(0, 2, 3), keepdims=True)
+    g = th.function([x], [th.Out(mean, device=True), th.Out(var, device=True)])
+    assert not ops_of(g, HipRowChain)
+    # gradient: x and g both held at this size; turned away (THX_HELD=0) the same node runs its island unfused
+    ins, outs = workloads.c5_graph(forward=False)
+    h = th.function(ins, [th.Out(o, device=True) for o in outs])
+    (chain,) = ops_of(h, HipRowChain)
+    small = workloads.c5_inputs("small")
+    h(*small)
+    assert "|rh|" in hip.last_plan()
+    os.environ["THX_HELD"] = "0"
+    try:
+        h2 = th.function(ins, [th.Out(o, device=True) for o in outs])
+        h2(*small)
+        assert "|rh|" not in hip.last_plan()
+        inner = ops_of(h2, HipRowChain)[0].op._fallback_function
+        assert [type(n.op) for n in inner.toposort() if isinstance(n.op, (HipCAReduce, HipElemwise))][-2:] == [HipCAReduce, HipElemwise]
+    finally:
+        del os.environ["THX_HELD"]
 
 
 def test_inplace_pass_reuses_single_use_intermediates_only(dry_run):

@@ -28,6 +28,10 @@ class _Config(object):
     # (float64 accumulators only), and the two reductions then share one pass over memory
     merge_dependent_reductions = True
 
+    # Islands of elementwise nodes and reductions over axes other than the last (the per-channel statistics
+    # of batch normalisation) run as one kernel that keeps each kept index's reduce domain on chip
+    held_chains = os.environ.get("THEANO_AMD_HELD_CHAINS", "1") != "0"
+
     # function(..., mode="check"): how far a result of the optimised function may be from the same graph run
     # one kernel per node, (rtol, atol) by result dtype.  A fused kernel keeps in float32 registers what the
     # separate kernels round to the storage type in between, hence the width of the float16 entry.

@@ -17,6 +17,7 @@ import hashlib
 import numpy as np
 
 from .. import gof
+from ..config import config
 from .. import scalar as scal
 from ..gof import Apply, Op
 from ..scalar import Scalar, compute_ctype, storage_ctype
@@ -28,20 +29,48 @@ FULL, ROW, COL, SCALAR = 0, 1, 2, 3
 THX_ERR_UNSUPPORTED = 6
 
 
-def _klass(var, nd):
-    """Operand class of a rank-``nd`` variable by its broadcast pattern."""
+def _klass(var, nd, red=None):
+    """Operand class of a rank-``nd`` variable by its broadcast pattern, for reductions over the
+    axes ``red`` (default: the last one): ROW is one value per kept index, COL (last-axis chains
+    only) one value per position along the reduced axis."""
     b = var.type.broadcastable
+    n_red = 1 if red is None else len(red)
+    if len(b) == nd - n_red:
+        # the kept axes alone (a reduction's result before keepdims): one value per kept index
+        return SCALAR if all(b) else (None if any(b) else ROW)
     if len(b) != nd:
         return None
     if not any(b):
         return FULL
     if all(b):
         return SCALAR
-    if b[-1] and not any(b[:-1]):
+    if red is None or tuple(red) == (nd - 1,):
+        if b[-1] and not any(b[:-1]):
+            return ROW
+        if not b[-1] and all(b[:-1]):
+            return COL
+        return None
+    if all(b[d] == (d in red) for d in range(nd)):
         return ROW
-    if not b[-1] and all(b[:-1]):
-        return COL
     return None
+
+
+def _chain_axes(nd, axis):
+    """The reduced axes as a sorted tuple if a chain can run over them: the kept axes are adjacent
+    and at least one reduced axis trails them (it is walked with unit stride)."""
+    red = tuple(range(nd)) if axis is None else tuple(sorted(axis))
+    if not red or len(set(red)) != len(red) or red[-1] != nd - 1:
+        return None
+    kept = [d for d in range(nd) if d not in red]
+    if kept and kept != list(range(kept[0], kept[-1] + 1)):
+        return None
+    return red
+
+
+def _row_shape(full, red, keepdims):
+    if keepdims:
+        return tuple(1 if d in red else n for d, n in enumerate(full))
+    return tuple(n for d, n in enumerate(full) if d not in red)
 
 
 class RowProgram(object):
@@ -52,6 +81,8 @@ class RowProgram(object):
         self.steps = []        # ("ew", scalar_op, arg ids, out ids) | ("red", scalar_op, acc, out dtype, arg, out)
         self.var = {}          # id -> (per_element, dtype)
         self.outputs = []      # (var id, kind, dtype)
+        self.axes = None       # reduced axes of the full shape; None: the last one
+        self.held_passes = 0
         self._next = 0
 
     def new_var(self, per_element, dtype):
@@ -113,10 +144,158 @@ class RowProgram(object):
             st = "store_full" if kind == FULL else "store_row"
             lines.append("x.template %s<%d, %s, %s>(%s);" % (st, k, storage_ctype(dt), ct, nm(vid)))
         body = "\n".join("    " + l for l in "\n".join(lines).splitlines())
-        text = "  enum { NIN = %d, NOUT = %d };\n%s\n  template <class X> THX_DEV static void row(X& x) {\n%s\n  }" % (
-            len(self.in_kinds), len(self.outputs), "\n".join(ops), body)
-        name = "C" + hashlib.sha1((text + repr(self.in_kinds)).encode()).hexdigest()[:16]
+        text = "  enum { NIN = %d, NOUT = %d };\n%s\n" % (len(self.in_kinds), len(self.outputs), "\n".join(ops))
+        if self.axes is None:
+            text += "  template <class X> THX_DEV static void row(X& x) {\n%s\n  }" % body
+        held = self._held_lines()
+        if held is not None and self.held_passes >= 2:   # one pass gains nothing from keeping the values
+            text += "\n  template <class X> THX_DEV static void held(X& x) {\n%s\n  }" % "\n".join(
+                "    " + l for l in "\n".join(held).splitlines())
+        name = "C" + hashlib.sha1((text + repr(self.in_kinds) + repr(self.axes)).encode()).hexdigest()[:16]
         return "struct %s {\n%s\n};\n" % (name, text), name
+
+    def _held_lines(self):
+        """The island for the held form (kernels/thx_rowchain.h): full-shaped inputs stay on chip in
+        their storage type and nothing per element is kept between two loops over them; every loop
+        (one per group of independent reductions, one for the stores) recomputes the elementwise
+        steps it needs.  None when an operand has no place in that form."""
+        self.held_passes = 0       # loops over the held values
+        if COL in self.in_kinds or FULL not in self.in_kinds:
+            return None
+        n_in = len(self.in_kinds)
+        lines = []
+        nm = lambda i: ("e%d" if self.var[i][0] else "s%d") % i
+        full_in = [k for k, kind in enumerate(self.in_kinds) if kind == FULL]
+        for k, (kind, dt) in enumerate(zip(self.in_kinds, self.in_dtypes)):
+            ct, st = compute_ctype(dt), storage_ctype(dt)
+            if kind == FULL:
+                lines.append("typename X::template Held<%d, %s> h%d; x.template hold<%d, %s>(h%d);" % (k, st, k, k, st, k))
+            else:
+                lines.append("%s s%d; x.template %s<%d, %s, %s>(s%d);" % (
+                    ct, k, "load_row" if kind == ROW else "load_scalar", k, st, ct, k))
+        producer = {}          # per-element variable -> its elementwise step
+        for step in self.steps:
+            if step[0] == "ew" and any(self.var[o][0] for o in step[3]):
+                for o in step[3]:
+                    producer[o] = step
+
+        def closure(vid, steps, inputs, scalars):
+            """Elementwise steps (in program order), held inputs and per-index scalars behind a
+            per-element variable."""
+            if not self.var[vid][0]:
+                scalars.add(vid)
+                return
+            if vid < n_in:
+                inputs.add(vid)
+                return
+            step = producer[vid]
+            if any(step is t for t in steps):
+                return
+            for a in step[2]:
+                closure(a, steps, inputs, scalars)
+            steps.append(step)
+
+        def loop(reds, stores):
+            steps, inputs, scalars = [], set(), set()
+            for r in reds:
+                closure(r[4], steps, inputs, scalars)
+            for n, (vid, kind, dt) in stores:
+                closure(vid, steps, inputs, scalars)
+            out = []
+            if stores:
+                out.append("typename X::Pos q = x.begin();")
+            out.append("_Pragma(\"unroll\") for (int ch = 0; ch < X::NCH; ++ch) {")
+            out.append("  if (x.valid(ch)) {")
+            for k in sorted(inputs):
+                st = storage_ctype(self.in_dtypes[k])
+                out.append("    const thx::Vec<%s, X::VEC> r%d = x.template get<%d, %s>(h%d, ch);" % (st, k, k, st, k))
+            for n, (vid, kind, dt) in stores:
+                out.append("    thx::Vec<%s, X::VEC> o%d;" % (storage_ctype(dt), n))
+            out.append("    _Pragma(\"unroll\") for (int j = 0; j < X::VEC; ++j) {")
+            for k in sorted(inputs):
+                ct = compute_ctype(self.in_dtypes[k])
+                out.append("      %s e%d = (%s)r%d.v[j];" % (ct, k, ct, k))
+            for _, op, args, outs in steps:
+                node = op.make_node(*[Scalar(self.var[a][1])() for a in args])
+                for o in outs:
+                    out.append("      %s %s;" % (compute_ctype(self.var[o][1]), nm(o)))
+                out.append("      {\n%s\n      }" % op.c_code(node, [nm(a) for a in args], [nm(o) for o in outs]))
+            for r in reds:
+                act = compute_ctype(r[2])
+                out.append("      { %s t = (%s)%s; Op%d::comb(a%d, t); }" % (act, act, nm(r[4]), r[5], r[5]))
+            for n, (vid, kind, dt) in stores:
+                out.append("      o%d.v[j] = (%s)%s;" % (n, storage_ctype(dt), nm(vid)))
+            out.append("    }")
+            for n, (vid, kind, dt) in stores:
+                out.append("    x.template put<%d, %s>(q, o%d);" % (n, storage_ctype(dt), n))
+            out.append("  }")
+            if stores:
+                out.append("  x.next(q);")
+            out.append("  X::pace(ch);")
+            out.append("}")
+            return ["{"] + ["  " + l for l in out] + ["}"], scalars
+
+        pending, deferred, blocked = [], [], set()
+
+        def scalar_step(step):
+            _, op, args, outs = step
+            node = op.make_node(*[Scalar(self.var[a][1])() for a in args])
+            for o in outs:
+                lines.append("%s s%d;" % (compute_ctype(self.var[o][1]), o))
+            lines.append("{\n%s\n}" % op.c_code(node, [nm(a) for a in args], [nm(o) for o in outs]))
+
+        def flush():
+            """One loop for the reductions collected so far, then the per-index steps that waited for
+            their results."""
+            if pending:
+                self.held_passes += 1
+                for r in pending:
+                    lines.append("%s a%d = %s;" % (compute_ctype(r[2]), r[5], codegen.reduce_identity(r[1], r[2])))
+                text, _ = loop(pending, [])
+                lines.extend(text)
+                for k in full_in:
+                    lines.append("x.template fence<%d, %s>(h%d);" % (k, storage_ctype(self.in_dtypes[k]), k))
+                for _, op, acc_dt, out_dt, arg, out in pending:
+                    act, oct_ = compute_ctype(acc_dt), compute_ctype(out_dt)
+                    lines.append("a%d = x.template allreduce<Op%d, %s>(a%d);" % (out, out, act, out))
+                    val = "a%d" % out
+                    if out_dt == "bool":
+                        val = "(%s ? 1 : 0)" % val
+                    lines.append("%s s%d = (%s)(%s)%s;" % (oct_, out, oct_, storage_ctype(out_dt), val))
+            for step in deferred:
+                scalar_step(step)
+            del pending[:], deferred[:]
+            blocked.clear()
+
+        for step in self.steps:
+            if step[0] == "ew":
+                _, op, args, outs = step
+                if any(self.var[o][0] for o in outs):
+                    continue           # per element: recomputed inside the loops that need it
+                if blocked.intersection(args):
+                    deferred.append(step)       # reads a reduction that later ones may still join
+                    blocked.update(outs)
+                else:
+                    scalar_step(step)
+            else:
+                if codegen.reduce_identity(step[1], step[2]) is None:
+                    return None
+                steps, inputs, scalars = [], set(), set()
+                closure(step[4], steps, inputs, scalars)
+                if blocked.intersection(scalars):
+                    flush()
+                pending.append(step)
+                blocked.add(step[5])
+        flush()
+        stores = [(n, o) for n, o in enumerate(self.outputs) if o[1] == FULL]
+        if stores:
+            self.held_passes += 1
+            text, _ = loop([], stores)
+            lines.extend(text)
+        for n, (vid, kind, dt) in enumerate(self.outputs):
+            if kind != FULL:
+                lines.append("x.template store_row<%d, %s, %s>(%s);" % (n, storage_ctype(dt), compute_ctype(self.var[vid][1]), nm(vid)))
+        return lines
 
 
 _handles = {}
@@ -130,13 +309,14 @@ class HipRowChain(Op):
     def __init__(self, program, out_types, fallback):
         self.program = program
         self.src, self.name = program.source()
-        self.signature = (self.name, tuple(program.in_kinds), tuple(str(t) for t in out_types))
+        self.signature = (self.name, tuple(program.in_kinds), tuple(str(t) for t in out_types), program.axes)
         self.out_types = list(out_types)
         self.fallback = fallback   # (inner input variables, inner output variables) of the original island
 
     def __str__(self):
         n_red = sum(1 for s in self.program.steps if s[0] == "red")
-        return "HipRowChain{%d steps, %d reductions}" % (len(self.program.steps), n_red)
+        over = "" if self.program.axes is None else ", axes %s" % (self.program.axes,)
+        return "HipRowChain{%d steps, %d reductions%s}" % (len(self.program.steps), n_red, over)
 
     def make_node(self, *inputs):
         return Apply(self, list(inputs), [t() for t in self.out_types])
@@ -147,14 +327,13 @@ class HipRowChain(Op):
             if k == FULL:
                 full = tuple(s)
         out = []
+        red = self._red(len(full))
         for (vid, kind, dt), t in zip(self.program.outputs, self.out_types):
-            if kind == FULL:
-                out.append(full)
-            elif t.ndim == len(full):
-                out.append(full[:-1] + (1,))
-            else:
-                out.append(full[:-1])
+            out.append(full if kind == FULL else _row_shape(full, red, t.ndim == len(full)))
         return out
+
+    def _red(self, nd):
+        return (nd - 1,) if self.program.axes is None else self.program.axes
 
     def _handle(self):
         h = _handles.get(self.signature)
@@ -167,6 +346,8 @@ class HipRowChain(Op):
             handle = ctypes.c_void_p()
             check(lib.thx_rowchain_new(self.src.encode(), self.name.encode(), len(p.in_kinds), len(p.outputs), codes, kk,
                                        ctypes.byref(handle)))
+            if p.axes is not None:
+                check(lib.thx_rowchain_set_axes(handle, len(p.axes), (ctypes.c_int32 * len(p.axes))(*p.axes)))
             h = _handles[self.signature] = handle
         return h
 
@@ -183,87 +364,83 @@ class HipRowChain(Op):
                 full = v.shape
                 break
         nd = len(full)
-        for k, v in enumerate(inputs):
-            if type(v) is HipArray:
-                v.as_thx(ins[k])
-            else:
-                host_scalar_thx(v, nd, ins[k])
-        results = []
-        for k, ((vid, kind, dt), t) in enumerate(zip(p.outputs, self.out_types)):
-            shape = full if kind == FULL else (full[:-1] + (1,) if t.ndim == nd else full[:-1])
-            arr = HipArray._new_contiguous(tuple(shape), out_dt[k])
-            arr.as_thx(outs[k])
-            results.append(arr)
-        mark_reused(node, ins, outs)
-        rc = lib.thx_rowchain_call(handle, ins, outs, call_flags(node))
-        if rc == THX_ERR_UNSUPPORTED:
+        red = self._red(nd)
+        layout = tuple((v.shape, v.strides) for v in inputs if type(v) is HipArray)
+        refused = node.tag.setdefault("thx_refused", set())
+        if layout in refused:           # turned away before with these shapes and strides
             results = self._run_fallback(inputs)
-        elif rc:
-            check(rc)
+        else:
+            for k, v in enumerate(inputs):
+                if type(v) is HipArray:
+                    v.as_thx(ins[k])
+                else:
+                    host_scalar_thx(v, nd, ins[k])
+            results = []
+            for k, ((vid, kind, dt), t) in enumerate(zip(p.outputs, self.out_types)):
+                shape = full if kind == FULL else _row_shape(full, red, t.ndim == nd)
+                arr = HipArray._new_contiguous(tuple(shape), out_dt[k])
+                arr.as_thx(outs[k])
+                results.append(arr)
+            mark_reused(node, ins, outs)
+            rc = lib.thx_rowchain_call(handle, ins, outs, call_flags(node))
+            if rc == THX_ERR_UNSUPPORTED:
+                refused.add(layout)
+                del results
+                results = self._run_fallback(inputs)
+            elif rc:
+                check(rc)
         for k, arr in enumerate(results):
             output_storage[k][0] = arr
 
     def _run_fallback(self, inputs):
-        """Shapes or strides the one-kernel form does not take (rows too long for the registers of
-        one block, non-contiguous rows): the island runs as reductions that compute their
-        elementwise producers and consumers on the fly plus the elementwise kernels in between,
-        fused the first time this is needed; intermediate results are dropped after their last use."""
-        plan = getattr(self, "_fallback_plan", None)
-        if plan is None:
+        """Shapes or strides the one-kernel form does not take (reduce domains too long for the
+        registers and LDS of one block, rows that are not contiguous, too few kept indices): the island
+        runs as reductions that compute their elementwise producers and consumers on the fly plus the
+        elementwise kernels in between, compiled the first time this is needed like any function
+        (same rewrites after row chains, same reuse marks, intermediate results dropped after their
+        last use)."""
+        f = getattr(self, "_fallback_function", None)
+        if f is None:
             from . import opt
+            from ..compile import Function, In, Out
             fg = gof.FunctionGraph(*self.fallback)
             opt.fuse_around_reductions(fg)
+            opt.fuse_reduction_of_stored_result(fg)
             opt.inplace_elemwise(fg)
-            order = fg.toposort()
-            last_use = {}
-            for k, n in enumerate(order):
-                for i in n.inputs:
-                    last_use[id(i)] = k
-            keep = set(id(o) for o in fg.outputs) | set(id(i) for i in fg.inputs)
-            plan = self._fallback_plan = (list(fg.inputs), list(fg.outputs), order, last_use, keep)
-        inner_in, inner_out, order, last_use, keep = plan
-        storage = dict((id(v), [val]) for v, val in zip(inner_in, inputs))
-        for k, n in enumerate(order):
-            args = []
-            for i in n.inputs:
-                cell = storage.get(id(i))
-                if cell is None:
-                    cell = storage[id(i)] = [np.asarray(i.data)]
-                args.append(cell[0])
-            cells = [[None] for _ in n.outputs]
-            n.op.perform(n, args, cells)
-            for o, c in zip(n.outputs, cells):
-                storage[id(o)] = c
-            for i in n.inputs:
-                if last_use.get(id(i)) == k and id(i) not in keep:
-                    storage.pop(id(i), None)
-        return [storage[id(o)][0] for o in inner_out]
+            f = self._fallback_function = Function(fg, [In(v) for v in fg.inputs],
+                                                   [Out(o, device=True) for o in fg.outputs], False, [])
+        return f(*inputs)
 
 
 # --------------------------------------------------------------------------
-def _eligible(node, nd):
+def _eligible(node, nd, red):
     op = node.op
+    last = red == (nd - 1,)
     if isinstance(op, HipElemwise):
         if len(node.outputs) != 1 or op.inplace_pattern:
             return False
-        if _klass(node.outputs[0], nd) not in (FULL, ROW):
+        if _klass(node.outputs[0], nd, red) not in (FULL, ROW):
             return False
         for i in node.inputs:
             if isinstance(i.type, HipArrayType):
-                if _klass(i, nd) is None:
+                k = _klass(i, nd, red)
+                if k is None or (k == COL and not last):
                     return False
             elif not _is_host_scalar(i):
                 return False
         return True
     if isinstance(op, HipCAReduce):
         return (len(op.scalar_ops) == 1 and op.pre_scalar_op is None and op.post_scalar_op is None and
-                len(node.inputs) == 1 and node.inputs[0].type.ndim == nd and op.axis == (nd - 1,) and
-                _klass(node.inputs[0], nd) == FULL and op.acc_dtypes[0] != "float16")
+                len(node.inputs) == 1 and node.inputs[0].type.ndim == nd and
+                _chain_axes(nd, op.axis) == red and
+                _klass(node.inputs[0], nd, red) == FULL and op.acc_dtypes[0] != "float16")
     if isinstance(op, HipDimShuffle):
         x = node.inputs[0]
-        return (x.type.ndim == nd - 1 and not any(x.type.broadcastable) and
-                op.new_order == tuple(range(nd - 1)) + ("x",) and x.owner is not None and
-                isinstance(x.owner.op, HipCAReduce))
+        kept = iter(range(nd - len(red)))
+        keepdims = tuple("x" if d in red else next(kept) for d in range(nd))
+        return (x.type.ndim == nd - len(red) and not any(x.type.broadcastable) and
+                tuple(op.new_order) == keepdims and x.owner is not None and
+                isinstance(x.owner.op, (HipCAReduce, HipElemwise)))
     return False
 
 
@@ -278,19 +455,20 @@ def fuse_row_chains(fgraph):
             if not isinstance(seed.op, HipCAReduce) or seed not in fgraph.apply_nodes:
                 continue
             nd = seed.inputs[0].type.ndim
-            if nd < 1 or not _eligible(seed, nd):
+            red = _chain_axes(nd, seed.op.axis) if nd >= 1 else None
+            if red is None or (red != (nd - 1,) and not config.held_chains) or not _eligible(seed, nd, red):
                 continue
-            island = _grow(fgraph, seed, nd)
+            island = _grow(fgraph, seed, nd, red)
             if island is None:
                 continue
-            if _replace(fgraph, island, nd):
+            if _replace(fgraph, island, nd, red):
                 count += 1
                 changed = True
                 break
     return count
 
 
-def _grow(fgraph, seed, nd):
+def _grow(fgraph, seed, nd, red):
     island = {seed}
     frontier = [seed]
     while frontier:
@@ -299,12 +477,12 @@ def _grow(fgraph, seed, nd):
         for o in n.outputs:
             neigh.extend(c for c, _ in fgraph.clients.get(o, []) if c != "output")
         for m in neigh:
-            if m in island or m not in fgraph.apply_nodes or not _eligible(m, nd):
+            if m in island or m not in fgraph.apply_nodes or not _eligible(m, nd, red):
                 continue
             if isinstance(m.op, HipDimShuffle) and m.inputs[0].owner not in island:
                 # reached from a consumer: the keepdims view joins together with its reduction
                 prod = m.inputs[0].owner
-                if prod not in fgraph.apply_nodes or not _eligible(prod, nd):
+                if prod not in fgraph.apply_nodes or not _eligible(prod, nd, red):
                     continue
                 island.add(prod)
                 frontier.append(prod)
@@ -339,10 +517,12 @@ def _grow(fgraph, seed, nd):
     return island
 
 
-def _replace(fgraph, island, nd):
+def _replace(fgraph, island, nd, red):
     order = [n for n in fgraph.toposort() if n in island]
     produced = set(id(o) for m in island for o in m.outputs)
     prog = RowProgram()
+    if red != (nd - 1,):
+        prog.axes = red
     ext_inputs, ids = [], {}
 
     def var_id(v):
@@ -350,7 +530,7 @@ def _replace(fgraph, island, nd):
             return ids[id(v)]
         # an external operand
         if isinstance(v.type, HipArrayType):
-            k = _klass(v, nd)
+            k = _klass(v, nd, red)
         else:
             k = SCALAR
         if k is None:
@@ -388,7 +568,7 @@ def _replace(fgraph, island, nd):
                 args.append(var_id(i))
             sop = scal.Composite(s_in, [op.scalar_op(*s_args)]) if len(s_in) != len(n.inputs) else op.scalar_op
             per_elem = any(prog.var[a][0] for a in args)
-            if per_elem != (_klass(n.outputs[0], nd) == FULL):
+            if per_elem != (_klass(n.outputs[0], nd, red) == FULL):
                 return False
             out = prog.new_var(per_elem, n.outputs[0].type.dtype)
             ids[id(n.outputs[0])] = out
@@ -411,11 +591,17 @@ def _replace(fgraph, island, nd):
         return False
     out_types = []
     for o in outs:
-        kind = FULL if (o.type.ndim == nd and _klass(o, nd) == FULL) else ROW
+        kind = FULL if (o.type.ndim == nd and _klass(o, nd, red) == FULL) else ROW
         prog.outputs.append((ids[id(o)], kind, o.type.dtype))
         out_types.append(o.type)
     if len(ext_inputs) + len(outs) > 48:
         return False
+    if prog.axes is not None:
+        # worth holding the values only for a full-sized result that is computed from reductions of them
+        # (statistics alone are one streaming pass of the merged reduction kernels, which is faster)
+        prog.source()
+        if prog.held_passes < 2 or not any(kind == FULL for _, kind, _ in prog.outputs):
+            return False
     # fallback: a private copy of the island
     memo = dict((v, v.type()) for v in ext_inputs)
     inner_in = [memo[v] for v in ext_inputs]

@@ -73,6 +73,7 @@ def _load():
         "thx_rowchain_new": ([ctypes.c_char_p, ctypes.c_char_p, ctypes.c_int, ctypes.c_int, P(i32), P(i32), P(vp)],
                              ctypes.c_int),
         "thx_rowchain_call": ([vp, P(thx_array), P(thx_array), ctypes.c_int], ctypes.c_int),
+        "thx_rowchain_set_axes": ([vp, ctypes.c_int, P(i32)], ctypes.c_int),
         "thx_rowchain_free": ([vp], ctypes.c_int),
         "thx_profile_begin": ([], ctypes.c_int),
         "thx_profile_end": ([ctypes.c_char_p, sz], ctypes.c_int),
