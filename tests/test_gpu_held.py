@@ -1,0 +1,160 @@
+"""Held chains on the device: reductions over the axes around a kept axis (or over long rows) with the
+elementwise work on their results, one kernel that keeps each kept index's elements on chip.  Every case is
+compared with the oracle's node-by-node evaluation of the same graph; ``hip.last_plan()`` shows which form ran
+('rh' = held, anything else = the island's separate kernels)."""
+import os
+
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import hip, tensor as T
+from theano_amd.hip import HipRowChain
+from oracle import graph_ref as G
+from conftest import assert_parity, assert_within_reference_error
+
+pytestmark = pytest.mark.gpu
+
+
+def tensor(dtype, nd, name):
+    return T.TensorType(dtype, (False,) * nd)(name)
+
+
+def per_index(dtype, nd, kept, name):
+    return T.TensorType(dtype, tuple(d not in kept for d in range(nd)))(name)
+
+
+def batch_norm(x, gamma, beta, axes, eps=1e-5):
+    xf = T.cast(x, "float32") if x.type.dtype == "float16" else x
+    mean = T.mean(xf, axis=axes, keepdims=True)
+    var = T.mean(T.sqr(xf - mean), axis=axes, keepdims=True)
+    y = T.cast(gamma, xf.type.dtype) * (xf - mean) / T.sqrt(var + np.asarray(eps, xf.type.dtype)) + T.cast(beta, xf.type.dtype)
+    return T.cast(y, x.type.dtype), mean, var
+
+
+def check(ins, outs, vals, what, tol=None, held=True):
+    f = th.function(ins, outs)
+    got = f(*vals)
+    chains = [n for n in f.toposort() if isinstance(n.op, HipRowChain)]
+    assert chains, what
+    ran_held = "|rh|" in hip.last_plan()
+    assert ran_held == held, (what, hip.last_plan())
+    ref = G.evaluate(ins, outs, vals)
+    truth = G.evaluate(ins, outs, vals, wide=True)
+    for k, (g, r, w) in enumerate(zip(got, ref, truth)):
+        if tol is not None:
+            assert_parity(g, r, "%s output %d" % (what, k), tol=tol)
+        else:
+            assert_within_reference_error(g, r, w, "%s output %d" % (what, k))
+    return f
+
+
+@pytest.mark.parametrize("dtype,shape", [
+    ("float32", (5, 7, 3, 8)),          # one chunk of 256 threads, most lanes idle
+    ("float32", (33, 19, 6, 10)),       # vectors of 4, ragged last chunk
+    ("float32", (16, 9, 5, 7)),         # 35 elements per slab: no vector width divides them
+    ("float16", (40, 12, 14, 16)),      # vectors of 8 float16 values
+    ("float16", (130, 6, 28, 28)),      # 1024-thread blocks, 13 chunks, some of them in LDS
+    ("float64", (12, 10, 4, 6)),
+])
+def test_batch_norm_forward_with_statistics_as_outputs(dtype, shape):
+    """y, the channel means and the channel variances from one kernel; float32 / float64 against the
+    oracle at their bars (no farther from the float64 value than the oracle), float16 storage at 2e-3."""
+    rng = np.random.default_rng(sum(shape))
+    nd, kept = 4, (1,)
+    x = tensor(dtype, nd, "x")
+    gamma, beta = per_index(dtype, nd, kept, "gamma"), per_index(dtype, nd, kept, "beta")
+    y, mean, var = batch_norm(x, gamma, beta, (0, 2, 3))
+    pshape = (1, shape[1], 1, 1)
+    vals = [rng.normal(0.4, 1.7, shape).astype(dtype), rng.normal(1.0, 0.2, pshape).astype(dtype),
+            rng.normal(0.0, 0.3, pshape).astype(dtype)]
+    tol = dict(rtol=2e-3, atol=2e-3) if dtype == "float16" else dict(rtol=1e-11, atol=1e-11) if dtype == "float64" else None
+    check([x, gamma, beta], [y, mean, var], vals, "batch norm %s %s" % (dtype, shape), tol)
+
+
+def test_two_full_operands_residual_and_scale():
+    """Two full-sized inputs held together (a residual branch added before the statistics), a full-sized
+    float32 result and a per-channel result; statistics over (0, 2) of a rank-3 array."""
+    rng = np.random.default_rng(5)
+    x, r = tensor("float32", 3, "x"), tensor("float32", 3, "r")
+    w = per_index("float32", 3, (1,), "w")
+    s = x + r
+    m = T.mean(s, axis=(0, 2), keepdims=True)
+    c = s - m
+    norm = T.sqrt(T.sum(T.sqr(c), axis=(0, 2), keepdims=True))
+    outs = [w * c / (norm + np.float32(1e-3)), T.max(abs(c), axis=(0, 2))]
+    vals = [rng.standard_normal((21, 11, 36)).astype("float32"), rng.standard_normal((21, 11, 36)).astype("float32"),
+            rng.uniform(0.5, 2, (1, 11, 1)).astype("float32")]
+    check([x, r, w], outs, vals, "residual")
+
+
+def test_kept_axes_are_a_block_of_two_and_nothing_kept():
+    """Instance-norm style statistics: axes (2, 3) reduced, (0, 1) kept (one block per (n, c) pair, a single
+    slab each); and a normalisation by the statistics of the whole array (one kept index)."""
+    rng = np.random.default_rng(6)
+    x = tensor("float32", 4, "x")
+    mean = T.mean(x, axis=(2, 3), keepdims=True)
+    var = T.mean(T.sqr(x - mean), axis=(2, 3), keepdims=True)
+    outs = [(x - mean) / T.sqrt(var + np.float32(1e-5))]
+    check([x], outs, [rng.normal(1.0, 2.0, (6, 5, 12, 20)).astype("float32")], "instance norm")
+    z = tensor("float32", 2, "z")
+    zc = z - T.mean(z)
+    outs = [zc / T.sqrt(T.mean(T.sqr(zc)))]
+    check([z], outs, [rng.normal(-2.0, 3.0, (70, 36)).astype("float32")], "whole-array standardisation")
+
+
+def test_strided_operands_and_shapes_the_held_form_turns_away():
+    """Views: every other sample of a larger array (slab stride doubles) is taken; a view whose trailing
+    axis is not contiguous is turned away and the island runs as separate kernels, same results.  A second
+    call with other shapes on the same function plans again."""
+    rng = np.random.default_rng(7)
+    x = tensor("float32", 4, "x")
+    g, b = per_index("float32", 4, (1,), "g"), per_index("float32", 4, (1,), "b")
+    y, mean, var = batch_norm(x[::2], g, b, (0, 2, 3))
+    vals = [rng.normal(0.0, 1.0, (24, 8, 6, 12)).astype("float32"), rng.normal(1, 0.1, (1, 8, 1, 1)).astype("float32"),
+            rng.normal(0, 0.1, (1, 8, 1, 1)).astype("float32")]
+    f = check([x, g, b], [y, mean], vals, "every other sample")
+    vals2 = [rng.normal(0.0, 1.0, (10, 8, 3, 20)).astype("float32")] + vals[1:]
+    got = f(*vals2)
+    assert "|rh|" in hip.last_plan()
+    ref = G.evaluate([x, g, b], [y, mean], vals2)
+    for k, (a, r) in enumerate(zip(got, ref)):
+        assert_parity(a, r, "second shape, output %d" % k, tol=dict(rtol=2e-5, atol=2e-6))
+    y2, _, _ = batch_norm(x[:, :, :, ::2], g, b, (0, 2, 3))
+    check([x, g, b], [y2], vals, "strided trailing axis", held=False)
+
+
+def test_domains_beyond_one_compute_unit_and_the_switch():
+    """160 000 float32 elements per channel exceed the registers and LDS of one block: turned away, separate
+    kernels, same result.  THX_HELD=0 turns every shape away."""
+    rng = np.random.default_rng(8)
+    x = tensor("float32", 4, "x")
+    g, b = per_index("float32", 4, (1,), "g"), per_index("float32", 4, (1,), "b")
+    y, mean, var = batch_norm(x, g, b, (0, 2, 3))
+    vals = [rng.normal(0.2, 1.0, (100, 3, 40, 40)).astype("float32"), rng.normal(1, 0.1, (1, 3, 1, 1)).astype("float32"),
+            rng.normal(0, 0.1, (1, 3, 1, 1)).astype("float32")]
+    check([x, g, b], [y, var], vals, "large channels", held=False)
+    small = [vals[0][:4, :, :5, :8].copy()] + vals[1:]
+    os.environ["THX_HELD"] = "0"
+    try:
+        check([x, g, b], [y, var], small, "switched off", held=False)
+    finally:
+        del os.environ["THX_HELD"]
+    check([x, g, b], [y, var], small, "switched on")
+
+
+def test_integer_chain_is_bit_exact():
+    """Integer statistics and integer results: per-channel sum and maximum of an int32 array and the
+    array recentred by an integer mean; equal to NumPy bit for bit."""
+    rng = np.random.default_rng(9)
+    x = tensor("int32", 4, "x")
+    s = T.sum(x, axis=(0, 2, 3), keepdims=True, dtype="int64")
+    m = T.max(x, axis=(0, 2, 3), keepdims=True)
+    out = T.cast(x, "int64") * np.int64(1200) - s + T.cast(m, "int64")
+    xv = rng.integers(-1000, 1000, (10, 7, 8, 12)).astype("int32")
+    f = th.function([x], [out, s])
+    got, gs = f(xv)
+    assert [n for n in f.toposort() if isinstance(n.op, HipRowChain)] and "|rh|" in hip.last_plan()
+    sv = xv.astype("int64").sum((0, 2, 3), keepdims=True)
+    assert np.array_equal(gs, sv)
+    assert np.array_equal(got, xv.astype("int64") * 1200 - sv + xv.max((0, 2, 3), keepdims=True).astype("int64"))

@@ -37,22 +37,22 @@ def _klass(var, nd, red=None):
     n_red = 1 if red is None else len(red)
     if len(b) == nd - n_red:
         # the kept axes alone (a reduction's result before keepdims): one value per kept index
-        return SCALAR if all(b) else (None if any(b) else ROW)
+        return ROW if not any(b) else (SCALAR if all(b) else None)
     if len(b) != nd:
         return None
     if not any(b):
         return FULL
-    if all(b):
-        return SCALAR
     if red is None or tuple(red) == (nd - 1,):
+        if all(b):
+            return SCALAR
         if b[-1] and not any(b[:-1]):
             return ROW
         if not b[-1] and all(b[:-1]):
             return COL
         return None
     if all(b[d] == (d in red) for d in range(nd)):
-        return ROW
-    return None
+        return ROW          # also the keepdims form of a reduction over every axis
+    return SCALAR if all(b) else None
 
 
 def _chain_axes(nd, axis):
@@ -409,7 +409,7 @@ class HipRowChain(Op):
             opt.inplace_elemwise(fg)
             f = self._fallback_function = Function(fg, [In(v) for v in fg.inputs],
                                                    [Out(o, device=True) for o in fg.outputs], False, [])
-        return f(*inputs)
+        return f.call_trusted(inputs)
 
 
 # --------------------------------------------------------------------------
