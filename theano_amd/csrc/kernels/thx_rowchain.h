@@ -178,6 +178,14 @@ struct HeldCtx {
   // scheduler interleaves many chunks (and hoists the LDS reads of all of them) for parallelism the
   // four waves of a SIMD already provide, and the registers that takes push held values out to memory.
   THX_DEV static void pace(int) { __builtin_amdgcn_sched_barrier(0); }
+  // An accumulator at the end of a chunk: its value exists here, so the arithmetic that feeds it cannot
+  // drift below the loads of the chunks that follow (which would keep all their data alive).
+  template <class A>
+  THX_DEV static void pin(A& a) {
+    if constexpr (sizeof(A) == 4 || sizeof(A) == 8) {
+      if constexpr (__is_trivially_copyable(A) && !__is_class(A)) asm volatile("" : "+v"(a));
+    }
+  }
 
   // (slab, vector inside the slab) of this thread's chunk; recomputed by every loop that needs
   // addresses, through an opaque copy so that the compiler does not keep NCH offsets alive instead
@@ -202,7 +210,6 @@ struct HeldCtx {
     enum { BYTES = VEC * (int)sizeof(T), WORDS = (BYTES + 3) / 4, NL = P::nlds(I), NR = NCH - NL };
     unsigned w[NR > 0 ? NR : 1][WORDS];
   };
-
   template <int I, class T>
   THX_DEV void hold(Held<I, T>& h) const {
     typedef Held<I, T> H;
@@ -258,6 +265,23 @@ struct HeldCtx {
   THX_DEV void put(const Pos& q, const Vec<T, VEC>& v) const {
     char* base = p.out[O] + (IT)k * p.out_sk[O];
     store_vec<T, VEC, ((P::NTO >> O) & 1) != 0>((T*)(base + (IT)q.ra * p.out_sa[O] + (IT)q.cv * (VEC * (int)sizeof(T))), v);
+  }
+  // A value that is the same in every lane moves to scalar registers: a chain carries a dozen or more
+  // per-index values through its loops, and the vector registers are for the held elements.
+  template <class CT>
+  THX_DEV static CT uni(CT v) {
+    if constexpr (sizeof(CT) == 4) {
+      return __builtin_bit_cast(CT, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+    } else if constexpr (sizeof(CT) == 8) {
+      const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+      const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
+      const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
+      return __builtin_bit_cast(CT, ((unsigned long long)hi << 32) | lo);
+    } else if constexpr (sizeof(CT) < 4) {
+      return (CT)__builtin_amdgcn_readfirstlane((int)v);
+    } else {
+      return v;
+    }
   }
   template <int I, class T, class CT>
   THX_DEV void load_row(CT& s) const {

@@ -171,8 +171,8 @@ class RowProgram(object):
             if kind == FULL:
                 lines.append("typename X::template Held<%d, %s> h%d; x.template hold<%d, %s>(h%d);" % (k, st, k, k, st, k))
             else:
-                lines.append("%s s%d; x.template %s<%d, %s, %s>(s%d);" % (
-                    ct, k, "load_row" if kind == ROW else "load_scalar", k, st, ct, k))
+                lines.append("%s s%d; x.template %s<%d, %s, %s>(s%d); s%d = X::uni(s%d);" % (
+                    ct, k, "load_row" if kind == ROW else "load_scalar", k, st, ct, k, k, k))
         producer = {}          # per-element variable -> its elementwise step
         for step in self.steps:
             if step[0] == "ew" and any(self.var[o][0] for o in step[3]):
@@ -231,6 +231,8 @@ class RowProgram(object):
             out.append("  }")
             if stores:
                 out.append("  x.next(q);")
+            for r in reds:
+                out.append("  X::pin(a%d);" % r[5])
             out.append("  X::pace(ch);")
             out.append("}")
             return ["{"] + ["  " + l for l in out] + ["}"], scalars
@@ -243,6 +245,8 @@ class RowProgram(object):
             for o in outs:
                 lines.append("%s s%d;" % (compute_ctype(self.var[o][1]), o))
             lines.append("{\n%s\n}" % op.c_code(node, [nm(a) for a in args], [nm(o) for o in outs]))
+            for o in outs:
+                lines.append("s%d = X::uni(s%d);" % (o, o))
 
         def flush():
             """One loop for the reductions collected so far, then the per-index steps that waited for
@@ -261,7 +265,7 @@ class RowProgram(object):
                     val = "a%d" % out
                     if out_dt == "bool":
                         val = "(%s ? 1 : 0)" % val
-                    lines.append("%s s%d = (%s)(%s)%s;" % (oct_, out, oct_, storage_ctype(out_dt), val))
+                    lines.append("%s s%d = X::uni((%s)(%s)%s);" % (oct_, out, oct_, storage_ctype(out_dt), val))
             for step in deferred:
                 scalar_step(step)
             del pending[:], deferred[:]
