@@ -217,6 +217,31 @@ struct TrStageAcc {  // global -> LDS for the staged inputs, nothing for the oth
 };
 
 template <class P, int NOPS>
+struct TrFetchAcc {  // global -> registers for the staged inputs, nothing for the others
+  typedef typename P::IT IT;
+  char* const* ptr;
+  IT off[NOPS];
+  template <int I, class T, int N>
+  THX_DEV void ld(Vec<T, N>& r) const {
+    if (P::slot(I) >= 0) load_vec<T, N, ((P::NT >> I) & 1) != 0>(r, (const T*)ptr[I] + off[I]);
+  }
+};
+
+template <class P, int NOPS>
+struct TrPutAcc {  // registers -> LDS for the staged inputs (visits the operands like a load)
+  unsigned char* lds;
+  int cell;  // LDS index of the first element: row * (TT + 1) + position along T
+  template <int I, class T, int N>
+  THX_DEV void ld(Vec<T, N>& r) const {
+    if (P::slot(I) >= 0) {
+      T* tile = (T*)(lds + P::slot(I) * (P::TI * (P::TT + 1) * P::ESZ));
+#pragma unroll
+      for (int k = 0; k < N; ++k) tile[cell + k] = r.v[k];
+    }
+  }
+};
+
+template <class P, int NOPS>
 struct TrAcc {  // LDS (transposed) or global -> registers, registers -> global
   typedef typename P::IT IT;
   char* const* ptr;
@@ -266,14 +291,11 @@ struct EwTrTile {
   static_assert(PASSES_S >= 1 && PASSES_C >= 1 && PASSES_S * RPP_S == TI && PASSES_C * RPP_C == TT,
                 "tile and block do not divide");
 
-  // One tile: `rem` counts tiles over the dimensions other than the innermost, `ti` tiles along it.
-  // ACC: per-thread accumulators of the reducing variant (one per element of a vector), or a dummy.
-  template <class ACC>
-  static __device__ __forceinline__ void run(const EwTrParams<NOPS, ND, IT>& p, unsigned char* lds, unsigned rem,
-                                             unsigned ti, ACC* acc) {
+  // Where tile `rem` (counted over the dimensions other than the innermost) starts: element offsets of
+  // every operand without the tile's own two dimensions, and its first position along T.
+  static __device__ __forceinline__ void locate(const EwTrParams<NOPS, ND, IT>& p, unsigned rem, IT (&base)[NOPS], int& t0) {
     unsigned tt, c;
     divmod(rem, p.tiles_t, rem, tt);
-    IT base[NOPS];
 #pragma unroll
     for (int i = 0; i < NOPS; ++i) base[i] = 0;
 #pragma unroll
@@ -286,35 +308,55 @@ struct EwTrTile {
 #pragma unroll
       for (int i = 0; i < NOPS; ++i) base[i] += (IT)rem * p.ostride[i][0];
     }
-    const int t0 = tt * TT, i0 = ti * TI;
+    t0 = tt * TT;
+  }
 
-    // stage: lanes run along T
-    {
-      typename F::template Regs<TV> dummy;
-      const int lane = threadIdx.x % LPR_S, row = threadIdx.x / LPR_S;
-      const int t = t0 + lane * TV;
+  typedef typename F::template Regs<TV> Regs;
+
+  // stage, first half: the staged inputs of one tile from memory into registers (lanes run along T)
+  static __device__ __forceinline__ void fetch(const EwTrParams<NOPS, ND, IT>& p, const IT (&base)[NOPS], int t0, int i0,
+                                               Regs (&s)[PASSES_S]) {
+    const int lane = threadIdx.x % LPR_S, row = threadIdx.x / LPR_S;
+    const int t = t0 + lane * TV;
 #pragma unroll
-      for (int k = 0; k < PASSES_S; ++k) {
-        const int ii = row + k * RPP_S, i = i0 + ii;
-        if (t < p.ext_t && i < p.ext_i) {
-          TrStageAcc<P, NOPS> a;
-          a.ptr = p.ptr;
-          a.lds = lds;
-          a.cell = ii * (TT + 1) + lane * TV;
+    for (int k = 0; k < PASSES_S; ++k) {
+      const int i = i0 + row + k * RPP_S;
+      if (t < p.ext_t && i < p.ext_i) {
+        TrFetchAcc<P, NOPS> a;
+        a.ptr = p.ptr;
 #pragma unroll
-          for (int o = 0; o < NOPS; ++o) a.off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
-          F::template load<TV>(a, dummy);
-        }
+        for (int o = 0; o < NOPS; ++o) a.off[o] = base[o] + (IT)t * p.tstride[o] + (IT)i * p.istride[o];
+        F::template load<TV>(a, s[k]);
       }
     }
-    __syncthreads();
+  }
+  // stage, second half: registers into the LDS tile
+  static __device__ __forceinline__ void put(const EwTrParams<NOPS, ND, IT>& p, unsigned char* lds, int t0, int i0,
+                                             Regs (&s)[PASSES_S]) {
+    const int lane = threadIdx.x % LPR_S, row = threadIdx.x / LPR_S;
+    const int t = t0 + lane * TV;
+#pragma unroll
+    for (int k = 0; k < PASSES_S; ++k) {
+      const int ii = row + k * RPP_S;
+      if (t < p.ext_t && i0 + ii < p.ext_i) {
+        TrPutAcc<P, NOPS> a;
+        a.lds = lds;
+        a.cell = ii * (TT + 1) + lane * TV;
+        F::template load<TV>(a, s[k]);
+      }
+    }
+  }
 
-    // compute: lanes run along the innermost dimension
+  // compute: lanes run along the innermost dimension.  ACC: per-thread accumulators of the reducing
+  // variant (one per element of a vector), or a dummy.
+  template <class ACC>
+  static __device__ __forceinline__ void compute(const EwTrParams<NOPS, ND, IT>& p, const unsigned char* lds,
+                                                 const IT (&base)[NOPS], int t0, int i0, ACC* acc) {
     const int lane = threadIdx.x % LPR_C, row = threadIdx.x / LPR_C;
     const int i = i0 + lane * TV;
 #pragma unroll
     for (int k0 = 0; k0 < PASSES_C; k0 += UNR) {
-      typename F::template Regs<TV> r[UNR];
+      Regs r[UNR];
       TrAcc<P, NOPS> a[UNR];
       bool ok[UNR];
 #pragma unroll
@@ -341,6 +383,21 @@ struct EwTrTile {
           if (ok[u]) F::template red_lanes<TV>(acc, r[u]);
       }
     }
+  }
+
+  // One tile start to end: `rem` counts tiles over the dimensions other than the innermost, `ti` tiles along it.
+  template <class ACC>
+  static __device__ __forceinline__ void run(const EwTrParams<NOPS, ND, IT>& p, unsigned char* lds, unsigned rem,
+                                             unsigned ti, ACC* acc) {
+    IT base[NOPS];
+    int t0;
+    locate(p, rem, base, t0);
+    const int i0 = ti * TI;
+    Regs s[PASSES_S];
+    fetch(p, base, t0, i0, s);
+    put(p, lds, t0, i0, s);
+    __syncthreads();
+    compute(p, lds, base, t0, i0, acc);
   }
 };
 
@@ -369,9 +426,34 @@ __device__ __forceinline__ void ew_tr_red_body(const EwTrParams<F::NOPS, P::ND, 
   Acc acc[TV];
 #pragma unroll
   for (int k = 0; k < TV; ++k) R::init(acc[k]);
-  for (unsigned j = g; j < (unsigned)q.rowtiles; j += (unsigned)q.groups) {
-    Tile::run(p, lds, j, ti, acc);
-    __syncthreads();              // the next tile's staging overwrites what this tile's compute phase read
+  // The block walks its tiles with the next tile's inputs already on their way: memory -> registers for
+  // tile j + groups is issued before tile j is computed from LDS and stored.
+  {
+    typedef typename P::IT IT;
+    const int i0 = ti * TI;
+    typename Tile::Regs s[Tile::PASSES_S];
+    IT base[F::NOPS], nbase[F::NOPS];
+    int t0 = 0, nt0 = 0;
+    unsigned j = g;
+    if (j < (unsigned)q.rowtiles) {
+      Tile::locate(p, j, base, t0);
+      Tile::fetch(p, base, t0, i0, s);
+    }
+    while (j < (unsigned)q.rowtiles) {
+      Tile::put(p, lds, t0, i0, s);
+      __syncthreads();
+      const unsigned jn = j + (unsigned)q.groups;
+      if (jn < (unsigned)q.rowtiles) {
+        Tile::locate(p, jn, nbase, nt0);
+        Tile::fetch(p, nbase, nt0, i0, s);
+      }
+      Tile::compute(p, lds, base, t0, i0, acc);
+      __syncthreads();            // the next tile's staging overwrites what this tile's compute phase read
+#pragma unroll
+      for (int o = 0; o < F::NOPS; ++o) base[o] = nbase[o];
+      t0 = nt0;
+      j = jn;
+    }
   }
   // merge the RPP row lanes of the block: [row][position along the innermost dimension]
   Acc* red = (Acc*)lds;
