@@ -385,29 +385,55 @@ struct EwTrTile {
     }
   }
 
-  // One tile start to end: `rem` counts tiles over the dimensions other than the innermost, `ti` tiles along it.
+  // Tiles first, first + step, ... below `total`, counted with the innermost dimension fastest.  The next
+  // tile's inputs are on their way (memory -> registers) while this one is computed from LDS and stored;
+  // with two LDS buffers (P::NBUF) one barrier per tile is enough: a buffer is staged again only after the
+  // barrier of the tile in between, which every thread reaches after it has finished reading that buffer.
   template <class ACC>
-  static __device__ __forceinline__ void run(const EwTrParams<NOPS, ND, IT>& p, unsigned char* lds, unsigned rem,
-                                             unsigned ti, ACC* acc) {
-    IT base[NOPS];
-    int t0;
-    locate(p, rem, base, t0);
-    const int i0 = ti * TI;
+  static __device__ __forceinline__ void walk(const EwTrParams<NOPS, ND, IT>& p, unsigned char* lds, unsigned first,
+                                              unsigned step, unsigned total, ACC* acc) {
     Regs s[PASSES_S];
-    fetch(p, base, t0, i0, s);
-    put(p, lds, t0, i0, s);
-    __syncthreads();
-    compute(p, lds, base, t0, i0, acc);
+    IT base[NOPS], nbase[NOPS];
+    int t0 = 0, nt0 = 0, i0 = 0, ni0 = 0;
+    unsigned id = first;
+    if (id < total) {
+      unsigned rem, ti;
+      divmod(id, p.tiles_i, rem, ti);
+      locate(p, rem, base, t0);
+      i0 = ti * TI;
+      fetch(p, base, t0, i0, s);
+    }
+    int b = 0;
+    while (id < total) {
+      unsigned char* buf = lds + b * LDS_BYTES;
+      put(p, buf, t0, i0, s);
+      __syncthreads();
+      const unsigned next = id + step;
+      if (next < total) {
+        unsigned rem, ti;
+        divmod(next, p.tiles_i, rem, ti);
+        locate(p, rem, nbase, nt0);
+        ni0 = ti * TI;
+        fetch(p, nbase, nt0, ni0, s);
+      }
+      compute(p, buf, base, t0, i0, acc);
+      if (P::NBUF == 1) __syncthreads();   // the next tile's staging overwrites what this tile's compute phase read
+      else b ^= 1;
+#pragma unroll
+      for (int o = 0; o < NOPS; ++o) base[o] = nbase[o];
+      t0 = nt0;
+      i0 = ni0;
+      id = next;
+    }
   }
 };
 
+// One block per tile, or (P::PERSIST) a grid of resident blocks that stride over the tiles.
 template <class F, class P>
-__device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, typename P::IT>& p) {
+__device__ __forceinline__ void ew_tr_body(const EwTrParams<F::NOPS, P::ND, typename P::IT>& p, unsigned total) {
   typedef EwTrTile<F, P> Tile;
-  __shared__ __attribute__((aligned(16))) unsigned char lds[Tile::LDS_BYTES];
-  unsigned rem = blockIdx.x, ti;
-  divmod(rem, p.tiles_i, rem, ti);
-  Tile::run(p, lds, rem, ti, (int*)nullptr);
+  __shared__ __attribute__((aligned(16))) unsigned char lds[Tile::LDS_BYTES * P::NBUF];
+  Tile::walk(p, lds, blockIdx.x, P::PERSIST ? gridDim.x : total, total, (int*)nullptr);
 }
 
 // The reducing variant: block b owns the innermost range b % tiles_i and the tiles g, g + groups, ...
@@ -420,41 +446,14 @@ __device__ __forceinline__ void ew_tr_red_body(const EwTrParams<F::NOPS, P::ND, 
   typedef typename R::Acc Acc;
   constexpr int TI = P::TI, TV = P::TV, RPP = Tile::RPP_C;
   constexpr int RED_BYTES = RPP * TI * (int)sizeof(Acc);
-  __shared__ __attribute__((aligned(16))) unsigned char lds[Tile::LDS_BYTES > RED_BYTES ? Tile::LDS_BYTES : RED_BYTES];
+  __shared__ __attribute__((aligned(16))) unsigned char lds[Tile::LDS_BYTES * P::NBUF > RED_BYTES ? Tile::LDS_BYTES * P::NBUF : RED_BYTES];
   unsigned g = blockIdx.x, ti;
   divmod(g, p.tiles_i, g, ti);
   Acc acc[TV];
 #pragma unroll
   for (int k = 0; k < TV; ++k) R::init(acc[k]);
-  // The block walks its tiles with the next tile's inputs already on their way: memory -> registers for
-  // tile j + groups is issued before tile j is computed from LDS and stored.
-  {
-    typedef typename P::IT IT;
-    const int i0 = ti * TI;
-    typename Tile::Regs s[Tile::PASSES_S];
-    IT base[F::NOPS], nbase[F::NOPS];
-    int t0 = 0, nt0 = 0;
-    unsigned j = g;
-    if (j < (unsigned)q.rowtiles) {
-      Tile::locate(p, j, base, t0);
-      Tile::fetch(p, base, t0, i0, s);
-    }
-    while (j < (unsigned)q.rowtiles) {
-      Tile::put(p, lds, t0, i0, s);
-      __syncthreads();
-      const unsigned jn = j + (unsigned)q.groups;
-      if (jn < (unsigned)q.rowtiles) {
-        Tile::locate(p, jn, nbase, nt0);
-        Tile::fetch(p, nbase, nt0, i0, s);
-      }
-      Tile::compute(p, lds, base, t0, i0, acc);
-      __syncthreads();            // the next tile's staging overwrites what this tile's compute phase read
-#pragma unroll
-      for (int o = 0; o < F::NOPS; ++o) base[o] = nbase[o];
-      t0 = nt0;
-      j = jn;
-    }
-  }
+  Tile::walk(p, lds, g * p.tiles_i.d + ti, (unsigned)q.groups * p.tiles_i.d, (unsigned)q.rowtiles * p.tiles_i.d, acc);
+  __syncthreads();                // the merge below reuses the tile buffers
   // merge the RPP row lanes of the block: [row][position along the innermost dimension]
   Acc* red = (Acc*)lds;
   const int lane = threadIdx.x % Tile::LPR_C, row = threadIdx.x / Tile::LPR_C;

@@ -76,14 +76,14 @@ struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, T
 struct PlanGen { typedef int IT; enum { NK = 3, NR = 3, BLOCK = 256, TPR = 64, GS = 1 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; } };
 
-struct PlanTr { typedef int IT; enum { ND = 3, TT = 64, TI = 32, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2, RED = 0 }; static constexpr unsigned long long NT = 0ull;
+struct PlanTr { typedef int IT; enum { ND = 3, TT = 64, TI = 32, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2, RED = 0, NBUF = 2, PERSIST = 1 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2, 0, 0}; return m[i]; }
   static constexpr int slot(int i) { constexpr int m[] = {0, -1, -1}; return m[i]; } };
-struct PlanTrRed { typedef int IT; enum { ND = 3, TT = 32, TI = 32, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2, RED = 1 }; static constexpr unsigned long long NT = 0ull;
+struct PlanTrRed { typedef int IT; enum { ND = 3, TT = 32, TI = 32, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2, RED = 1, NBUF = 1, PERSIST = 0 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2, 0, 0}; return m[i]; }
   static constexpr int slot(int i) { constexpr int m[] = {0, -1, -1}; return m[i]; } };
 extern "C" __global__ __launch_bounds__(256) void check_tr_red(thx::EwTrParams<3, 3, int> p, thx::EwRedParams<2, 1> q) { thx::ew_tr_red_body<CheckFR, PlanTrRed>(p, q); }
-extern "C" __global__ __launch_bounds__(256) void check_tr(thx::EwTrParams<3, 3, int> p) { thx::ew_tr_body<CheckF, PlanTr>(p); }
+extern "C" __global__ __launch_bounds__(256) void check_tr(thx::EwTrParams<3, 3, int> p, unsigned total) { thx::ew_tr_body<CheckF, PlanTr>(p, total); }
 extern "C" __global__ __launch_bounds__(256) void check_ew1(thx::EwParams<3, 1, int> p) { thx::ew_body<CheckF, PlanEw1>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_ew3(thx::EwParams<3, 3, long long> p) { thx::ew_body<CheckF, PlanEw3>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_row(thx::RowParams<1, 2, 1, 2, int> p) { thx::red_row_body<CheckR, PlanRow>(p); }

@@ -284,8 +284,16 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
         if (R && !red)   // the caller reduces the stored results next: they stay cacheable
           for (int w : e->red_of) views[e->n_in + w].reused = true;
         const uint64_t nt = nt_mask(nt_streaming(moved), views);
+        // Measured on the int32 (64, 128, 56, 56) permuted read and left off: two tile buffers (one barrier per
+        // tile instead of two) change nothing, 58.9 us against 58.8 us with the channel sum attached; resident
+        // blocks that stride over the tiles with the next tile's loads in flight match one block per tile at 4-6
+        // blocks per compute unit (53.2-53.5 us against 53.5 us) and lose at 8 (56.1 us).
+        const int64_t lds_one = (int64_t)ntr * tile_i * (tile_t + 1) * esz;
+        const int nbuf = (2 * lds_one <= 60000 && env_int("THX_EW_TR_NBUF", 1) == 2) ? 2 : 1;
+        const bool persist = !red && env_int("THX_EW_TR_PERSIST", 0) != 0;
         std::ostringstream key;
-        key << (red ? "er|nd" : "et|nd") << ND << "|t" << tile_t << "x" << tile_i << "|v" << tv << "|n" << ntr << "|e" << esz;
+        key << (red ? "er|nd" : "et|nd") << ND << "|t" << tile_t << "x" << tile_i << "|v" << tv << "|n" << ntr << "|e" << esz
+            << (nbuf == 2 ? "|b2" : "") << (persist ? "|p" : "");
         if (nt) key << "|nt" << std::hex << nt << std::dec;
         key << "|m";
         for (int o = 0; o < nops; ++o) key << (slot[o] >= 0 ? 9 : mode[o]) << (o + 1 < nops ? "," : "");
@@ -300,7 +308,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
           std::ostringstream s;
           s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef int IT;\n  enum { ND = " << ND
             << ", TT = " << tile_t << ", TI = " << tile_i << ", TV = " << tv << ", BLOCK = " << block << ", NTR = " << ntr << ", ESZ = " << esz
-            << ", RED = " << (red ? 1 : 0)
+            << ", RED = " << (red ? 1 : 0) << ", NBUF = " << nbuf << ", PERSIST = " << (persist ? 1 : 0)
             << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
           for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
           s << "};\n    return m[i];\n  }\n  static constexpr int slot(int i) {\n    constexpr int m[] = {";
@@ -312,7 +320,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
               << "::NEX> q) {\n  thx::ew_tr_red_body<" << e->name << ", ThxPlan>(p, q);\n}\n";
           else
             s << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::EwTrParams<" << e->name
-              << "::NOPS, ThxPlan::ND, ThxPlan::IT> p) {\n  thx::ew_tr_body<" << e->name << ", ThxPlan>(p);\n}\n";
+              << "::NOPS, ThxPlan::ND, ThxPlan::IT> p, unsigned total) {\n  thx::ew_tr_body<" << e->name << ", ThxPlan>(p, total);\n}\n";
           rc = get_kernel(s.str(), entry, &k);
           if (rc) return rc;
           e->plans[plan] = k;
@@ -365,8 +373,14 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
           if (fused) *fused = red;
           return THX_OK;
         }
-        const int64_t grid = red ? groups * tiles_i : outer * tiles_t * tiles_i;
-        if (grid * 256 <= 0xffffffffLL) {
+        const int64_t all_tiles = outer * tiles_t * tiles_i;
+        int64_t grid = red ? groups * tiles_i : all_tiles;
+        if (persist) {
+          const int64_t cus = rt().ready ? rt().cus : 256;
+          const int64_t per_cu = std::max<int64_t>(1, std::min<int64_t>(env_int("THX_EW_TR_BLOCKS_PER_CU", 8), (150 * 1024) / std::max<int64_t>(1, nbuf * lds_one)));
+          grid = std::min(grid, cus * per_cu);
+        }
+        if (all_tiles * 256 <= 0xffffffffLL) {
           if (red && groups > 1) {
             rc = ensure_scratch((size_t)groups * ext_i * R->acc_bytes);
             if (rc) return rc;
@@ -384,6 +398,10 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
           for (int o = 0; o < nops; ++o) pk.put<int32_t>((int32_t)dm.stride[o][tdim]);
           for (int o = 0; o < nops; ++o) pk.put<int32_t>((int32_t)dm.stride[o][ND - 1]);
           pk.align(8);
+          if (!red) {
+            pk.put<uint32_t>((uint32_t)all_tiles);
+            pk.align(8);
+          }
           if (red) {
             for (char* q : routp) pk.put<char*>(q);
             pk.put<uint64_t>(0);   // no further operands of the epilogue
