@@ -117,7 +117,7 @@ struct RedAcc {
   }
 };
 
-// Plan members: typedef IT; enum { NK, VEC, UNR, NACC, BLOCK, TPR, RA2 (1 when RA > 1), TICKET, GS };
+// Plan members: typedef IT; enum { NK, VEC, UNR, NACC, BLOCK, TPR, RA2 (1 when RA > 1), TICKET, GS, XCD };
 // static constexpr int mode(int input); static constexpr int sclass(int input, int which).
 template <class P, class IT>
 THX_DEV IT red_term(int input, int which, IT coord, IT stride) {
@@ -150,6 +150,7 @@ __device__ __forceinline__ void red_row_block(const RowParams<R::NIN, R::NOUT, R
   constexpr int RPB = P::BLOCK / TPR;
   __shared__ Acc lds[P::BLOCK / THX_WAVE];
 
+  if constexpr (P::XCD != 0) bid = (bid & 7) * (p.nblocks >> 3) + (bid >> 3);   // a contiguous eighth of the results per die
   const long long ob = bid / p.S;
   const int s = (int)(bid - ob * p.S);
   const long long o = ob * RPB + threadIdx.x / TPR;

@@ -169,7 +169,11 @@ struct HeldCtx {
   unsigned k, t;
 
   THX_DEV HeldCtx(const HeldParams<C::NIN, C::NOUT, IT>& p_, unsigned char* s) : p(p_), stash(s) {
-    k = blockIdx.x;
+    // Consecutive blocks go to the eight dies in turn, each with its own L2.  Neighbouring kept indices
+    // share cache lines where their slabs meet (a 1568-byte slab ends inside a 128-byte line), so each die
+    // takes one contiguous eighth of the indices and those lines are fetched once.
+    const unsigned b = blockIdx.x, nb = gridDim.x;
+    k = (nb & 7) == 0 ? (b & 7) * (nb >> 3) + (b >> 3) : b;
     t = threadIdx.x;
   }
   // chunks below NFULL are inside the reduce domain for every thread

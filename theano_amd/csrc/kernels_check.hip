@@ -65,10 +65,10 @@ struct PlanEw3 { typedef long long IT; enum { ND = 3, VEC = 2, UNR = 1, BLOCK = 
   static constexpr int mode(int i) { constexpr int m[] = {2, 1, 0}; return m[i]; }
   static constexpr int sclass(int i, int d) { constexpr int m[][3] = {{2, 2, 2}, {0, 1, 0}, {2, 2, 1}}; return m[i][d]; }
   static constexpr int alias(int i) { constexpr int m[] = {0, 1, 2}; return m[i]; } };
-struct PlanRow { typedef int IT; enum { NK = 2, VEC = 4, UNR = 4, NACC = 2, BLOCK = 256, TPR = 256, RA2 = 1, TICKET = 0, GS = 1 }; static constexpr unsigned long long NT = 0ull;
+struct PlanRow { typedef int IT; enum { NK = 2, VEC = 4, UNR = 4, NACC = 2, BLOCK = 256, TPR = 256, RA2 = 1, TICKET = 0, GS = 1, XCD = 0 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {0}; return m[i]; }
   static constexpr int sclass(int i, int w) { constexpr int m[][2] = {{2, 1}}; return m[i][w]; } };
-struct PlanRowS { typedef int IT; enum { NK = 1, VEC = 1, UNR = 1, NACC = 1, BLOCK = 256, TPR = 16, RA2 = 0, TICKET = 0, GS = 0 }; static constexpr unsigned long long NT = 1ull;
+struct PlanRowS { typedef int IT; enum { NK = 1, VEC = 1, UNR = 1, NACC = 1, BLOCK = 256, TPR = 16, RA2 = 0, TICKET = 0, GS = 0, XCD = 1 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; }
   static constexpr int sclass(int i, int w) { constexpr int m[][2] = {{0, 2}}; return m[i][w]; } };
 struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, TX = 64, RR2 = 1, TICKET = 0, GS = 1 }; static constexpr unsigned long long NT = 1ull;

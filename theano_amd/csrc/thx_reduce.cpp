@@ -456,8 +456,12 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     }
     nblocks = oblocks * S;
     gs = nblocks * rblock > max_dispatch;
+    // One 1024-thread block per result whose reduce domain is slabs around the kept axis: the slabs of
+    // neighbouring results meet inside cache lines, so each die (blocks go to the eight dies in turn, one L2
+    // each) takes a contiguous eighth of the results and fetches those lines once.
+    const bool xcd = bigblock && ra2 && S == 1 && !gs && nblocks % 8 == 0 && env_int("THX_RED_XCD", 1);
     std::ostringstream key;
-    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nacc != unr ? "|c" + std::to_string(nacc) : "") << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << (gs ? "|gs" : "") << "|m";
+    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nacc != unr ? "|c" + std::to_string(nacc) : "") << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << (gs ? "|gs" : "") << (xcd ? "|x8" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -469,7 +473,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"NACC", nacc}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"TICKET", ticket ? 1 : 0}, {"GS", gs ? 1 : 0}}, mode, nt, sclass)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"NACC", nacc}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"TICKET", ticket ? 1 : 0}, {"GS", gs ? 1 : 0}, {"XCD", xcd ? 1 : 0}}, mode, nt, sclass)
         << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void " << entry << "(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
