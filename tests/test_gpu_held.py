@@ -158,3 +158,81 @@ def test_integer_chain_is_bit_exact():
     sv = xv.astype("int64").sum((0, 2, 3), keepdims=True)
     assert np.array_equal(gs, sv)
     assert np.array_equal(got, xv.astype("int64") * 1200 - sv + xv.max((0, 2, 3), keepdims=True).astype("int64"))
+
+
+# ---- seeded random normalisation graphs -------------------------------------------------------------------
+EXTENTS = [1, 2, 3, 5, 7, 8, 16, 33, 64]
+
+
+def random_normalisation_graph(seed):
+    """A full-sized float operand (sometimes every other slice of a larger array, sometimes the sum of two
+    operands), statistics over a random set of axes that a chain can take (the kept axes adjacent, a reduced axis
+    last) with or without keepdims in between, a per-index scale, and one to three results: the normalised array,
+    a second full-sized result, per-index statistics."""
+    rng = np.random.default_rng(seed)
+    nd = int(rng.integers(2, 5))
+    shape = [int(rng.choice(EXTENTS[1:])) for _ in range(nd)]
+    dtype = str(rng.choice(["float16", "float32", "float32", "float64"]))
+    k0 = int(rng.integers(0, nd))                   # kept axes [k0, k1); reduced before and after
+    k1 = int(rng.integers(k0, nd))
+    axes = tuple(d for d in range(nd) if not (k0 <= d < k1))
+    kept = tuple(range(k0, k1))
+    ins, vals = [], []
+
+    def operand(name):
+        step = int(rng.integers(nd)) if rng.random() < 0.3 else None
+        alloc = [2 * s + 1 if d == step and d != nd - 1 else s for d, s in enumerate(shape)]
+        v = tensor(dtype, nd, name)
+        ins.append(v)
+        vals.append(rng.normal(0.3, 1.5, alloc).astype(dtype))
+        if step is not None and step != nd - 1:
+            return v[tuple(slice(1, None, 2) if d == step else slice(None) for d in range(nd))]
+        return v
+
+    x = operand("x")
+    if rng.random() < 0.35:
+        x = x + operand("r")
+    xf = T.cast(x, "float32") if dtype == "float16" else x
+    cdt = xf.type.dtype
+    if rng.random() < 0.5:
+        mean = T.mean(xf, axis=axes, keepdims=True)
+    else:                                           # the reduction's plain result, broadcast back by hand
+        m = T.mean(xf, axis=axes)
+        it = iter(range(len(kept)))
+        mean = m.dimshuffle(*["x" if d in axes else next(it) for d in range(nd)])
+    c = xf - mean
+    var = T.mean(T.sqr(c), axis=axes, keepdims=True)
+    y = c / T.sqrt(var + np.asarray(0.1, cdt))
+    if rng.random() < 0.6:
+        w = per_index(dtype, nd, kept, "w")
+        ins.append(w)
+        vals.append(rng.uniform(0.5, 2.0, [s if d in kept else 1 for d, s in enumerate(shape)]).astype(dtype))
+        y = y * T.cast(w, cdt)
+    outs = [T.cast(y, dtype)]
+    extra = int(rng.integers(3))
+    if extra == 1:
+        outs.append(T.max(abs(c), axis=axes))
+    elif extra == 2:
+        outs += [T.tanh(c) * np.asarray(0.5, cdt), var]
+    return ins, outs, vals, dtype
+
+
+NORM_SEEDS = list(range(900, 960))
+
+
+@pytest.mark.parametrize("seed", NORM_SEEDS)
+def test_random_normalisation_graph_matches_the_oracle(seed):
+    ins, outs, vals, dtype = random_normalisation_graph(seed)
+    f = th.function(ins, outs)
+    got = f(*vals)
+    ref = G.evaluate(ins, outs, vals)
+    truth = G.evaluate(ins, outs, vals, wide=True)
+    # float16 operands: the separate nodes round x + r and every other intermediate to float16, the chain
+    # keeps them in float32 until the store; near a zero of x - mean that is more than the float16 bar apart,
+    # so the device is held to the float64 value (within the bar, or no farther from it than the oracle)
+    for k, (g, r, w) in enumerate(zip(got, ref, truth)):
+        if dtype == "float64":
+            assert_parity(g, r, "seed %d output %d" % (seed, k), tol=dict(rtol=1e-11, atol=1e-11))
+        else:
+            assert_within_reference_error(g, r, w, "seed %d output %d" % (seed, k),
+                                          tol=dict(rtol=2e-3, atol=2e-3) if dtype == "float16" else None)
