@@ -1,0 +1,154 @@
+"""Cases of the reference's own elemwise tests (``theano/tensor/tests/test_elemwise.py``) that the other test
+files do not already restate: graph-level ones run on the CPU, value-level ones on the device."""
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import scalar as scal
+from theano_amd import tensor as T
+
+AXES = [None, 0, 1, [0, 1], np.array(1), [np.array(0), np.array(1)]]
+
+
+def test_reduce_axes_of_every_kind():
+    """``test_reduce_axes`` (:110-153): ints, lists, 0-d arrays and lists of 0-d arrays as ``axis`` of sum, mean,
+    max, min, argmax and var, as functions and as methods."""
+    for a in AXES:
+        x = T.matrix()
+        for res in (x.sum(a), x.mean(a), x.max(a), x.min(a), x.argmax(a), x.var(a), T.argmin(x, a)):
+            want = 0 if (a is None or isinstance(a, list)) else 1
+            assert res.type.ndim == want, (a, res)
+
+
+def test_fill_methods_and_gradients_build():
+    """``test_fill_var`` (:293), ``test_fill_grad`` (:297), ``test_elemwise_grad_broadcast`` (:1300),
+    ``test_clip_grad_int`` (:1313), ``test_elemwise_grad_bool`` (:1186): graphs that once crashed while built."""
+    T.matrix().fill(3)
+    x = T.TensorType(th.config.floatX, [0, 1, 0])("x")
+    y = T.TensorType(th.config.floatX, [0, 1, 0])("y")
+    th.grad(T.second(x, y).sum(), y)
+    x = T.TensorType("float32", (True, False, False, False))("x")
+    y = T.TensorType("float32", (True, True, False, False))("y")
+    th.grad(T.tanh(x).sum(), x)
+    th.grad(T.tanh(x + y).sum(), y)
+    gx, gy = th.grad(T.tanh(x + y).sum(), [x, y])
+    assert gx.type.broadcastable == x.type.broadcastable and gy.type.broadcastable == y.type.broadcastable
+    a, b, c = T.iscalar(), T.iscalar(), T.iscalar()
+    th.grad(T.clip(a, b, c), [a, b, c])
+    p, q = T.scalar(dtype="bool"), T.bscalar()
+    th.grad(p * q, [p, q])
+
+
+def test_mean_dtypes():
+    """``T_mean_dtype`` (:969-1035): a mean is float64 for discrete inputs and keeps floating and complex dtypes; a
+    custom dtype decides the result the same way, unsuitable ones raise TypeError from the inner sum, and the
+    gradient can be taken wherever the result is real."""
+    axes = [None, 0, 1, [], [0], [1], [0, 1]]
+    for idx, dtype in enumerate(scal.all_dtypes):
+        m = T.matrix(dtype=dtype).mean(axis=axes[idx % len(axes)])
+        assert m.dtype == ("float64" if dtype in scal.discrete_dtypes else dtype), (dtype, m.dtype)
+    idx = compiled = 0
+    for input_dtype in scal.all_dtypes:
+        x = T.matrix(dtype=input_dtype)
+        for sum_dtype in scal.all_dtypes:
+            axis = axes[idx % len(axes)]
+            try:
+                mean_var = x.mean(dtype=sum_dtype, axis=axis)
+            except TypeError:
+                pass
+            else:
+                assert mean_var.dtype == ("float64" if sum_dtype in scal.discrete_dtypes else sum_dtype)
+                if ("complex" in input_dtype or "complex" in sum_dtype) and input_dtype != sum_dtype:
+                    continue
+                compiled += 1
+                if "complex" not in mean_var.dtype:
+                    th.grad(mean_var.sum(), x, disconnected_inputs="ignore")
+            idx += 1
+    assert compiled > 100
+
+
+def test_comparisons_refuse_truth_tests_and_python_protocols():
+    """``a < b < c`` must not silently drop ``a < b`` (``theano/tensor/var.py:52-95``); divmod, ceil / floor /
+    trunc, the math methods, norm, squeeze, transpose, copy (``var.py:196-256, 300-330, 629-636, 686-698, 817``)."""
+    import math
+    a, b, c = T.vector("a"), T.vector("b"), T.vector("c")
+    with pytest.raises(TypeError, match="boolean operations"):
+        a < b < c
+    with pytest.raises(TypeError):
+        bool(a >= b)
+    assert bool(a) and bool(a + b)
+    q, r = divmod(a, b)
+    assert str(q.owner.op.scalar_op) == "int_div" and str(r.owner.op.scalar_op) == "mod"
+    q, r = divmod(3.0, b)
+    assert q.owner.inputs[1] is b or q.owner.inputs[1].owner is not None
+    for fn, name in ((math.ceil, "ceil"), (math.floor, "floor"), (math.trunc, "trunc")):
+        assert str(fn(a).owner.op.scalar_op) == name
+    for name in ("arccos", "arccosh", "arcsin", "arcsinh", "arctan", "arctanh", "ceil", "cos", "cosh", "exp", "floor",
+                 "log", "sin", "sinh", "sqrt", "tan", "tanh", "trunc"):
+        assert getattr(a, name)().owner.op is getattr(T, name)(a).owner.op or \
+            getattr(a, name)().owner.op == getattr(T, name)(a).owner.op, name
+    m = T.TensorType("float32", (False, True, False))("m")
+    assert m.squeeze().type.broadcastable == (False, False)
+    assert m.transpose(2, 0, 1).type.broadcastable == (False, False, True)
+    assert m.transpose().type.broadcastable == (False, True, False) and m.swapaxes(0, 1).type.broadcastable == (True, False, False)
+    assert m.norm(2, axis=0).type.ndim == 2 and m.norm(1, axis=0, keepdims=True).type.ndim == 3
+    with pytest.raises(NotImplementedError):
+        m.norm(0)
+    assert m.copy(name="again").name == "again" and m.ravel().type.ndim == 1
+    assert m.clip(0, 1).type == m.type and m.round().type == m.type and m.ptp(0).type.ndim == 2
+
+
+@pytest.mark.gpu
+def test_same_input_twice_six_operands_and_rank_limit():
+    """``test_same_inputs`` (:320): ``x + x``; ``test_input_dimensions_overflow`` (:1215): six vectors of 2048
+    elements added; ``test_too_big_rank`` (:104): a DimShuffle past the array rank limit raises ValueError when run."""
+    rng = np.random.default_rng(0)
+    x = T.matrix("x")
+    xv = rng.standard_normal((2, 2)).astype("float32")
+    assert np.array_equal(th.function([x], x + x)(xv), xv + xv)
+    vs = [T.vector(n) for n in "abcdef"]
+    s = vs[0]
+    for v in vs[1:]:
+        s = s + v
+    vals = [rng.standard_normal(2 ** 11).astype("float32") for _ in vs]
+    want = vals[0]
+    for v in vals[1:]:
+        want = want + v
+    assert np.array_equal(th.function(vs, s)(*vals), want)
+    v = T.vector("v")
+    f = th.function([v], v.dimshuffle(*(("x",) * 8 + (0,))) * 2)
+    with pytest.raises(ValueError, match="dimensions"):
+        f(np.zeros(3, "float32"))
+
+
+@pytest.mark.gpu
+def test_gradients_of_all_any_clip_and_a_hinge_loss():
+    """``TestBitOpReduceGrad`` (:1154-1182): gradients of all / any are zeros of the input's shape;
+    ``test_clip_grad`` (:1251) at a value below, between and above the bounds; ``test_gt_grad`` (:1226): the
+    hinge loss whose gradient once failed to be recognised as valid (the dot written as a broadcast product);
+    ``test_mean_precision`` (:1037): the mean of [1e8, 1, -1e8] in float32 is 1/3."""
+    rng = np.random.default_rng(1)
+    x = T.bmatrix("x")
+    x_random = rng.binomial(n=1, p=0.5, size=(5, 7)).astype("int8")
+    for red in (x.all(), x.any()):
+        f = th.function([x], th.grad(red, x))
+        for xv in (x_random, np.zeros_like(x_random), np.ones_like(x_random)):
+            g = f(xv)
+            assert g.shape == xv.shape and np.all(g == 0)
+    v, lo, hi = T.dvector("v"), T.dscalar("lo"), T.dscalar("hi")
+    gv, glo, ghi = th.function([v, lo, hi], th.grad(T.clip(v, lo, hi).sum(), [v, lo, hi]))(
+        np.asarray([-1.0, 0.5, 2.0]), 0.0, 1.0)
+    assert np.array_equal(gv, [0.0, 1.0, 0.0]) and glo == 1.0 and ghi == 1.0
+    inp, wrong_in = T.vector("inp"), T.vector("wrong")
+    W = th.shared(np.random.RandomState(1234).uniform(-1, 1, (2, 2)).astype("float32"), name="weights")
+    correct = T.sum(inp.dimshuffle(0, "x") * W, axis=0)
+    wrong = T.sum(wrong_in.dimshuffle(0, "x") * W, axis=0)
+    scores = T.ones_like(correct) - correct + wrong
+    cost = (scores * (scores > 0)).sum()
+    g = th.function([inp, wrong_in], th.grad(cost, inp))
+    iv, wv = np.asarray([0.3, -0.2], "float32"), np.asarray([0.1, 0.4], "float32")
+    Wv = W.get_value()
+    sc = 1 - iv @ Wv + wv @ Wv
+    assert np.allclose(g(iv, wv), -(Wv * (sc > 0)).sum(axis=1), rtol=1e-5, atol=1e-6)
+    m = th.shared(np.asarray([1e8, 1, -1e8], dtype="float32"))
+    assert np.allclose(th.function([], m.mean())(), 1.0 / 3)

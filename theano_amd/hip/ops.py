@@ -17,7 +17,7 @@ from ..gof import Apply, Op, Type, Variable
 from ..tensor.elemwise import CAReduce, DimShuffle, Elemwise
 from ..tensor.type import TensorType, _tensor_py_operators
 from . import codegen
-from .runtime import THX_INDEX, HipArray, call_flags, check, host_scalar_thx, lib, mark_reused, thx_array
+from .runtime import THX_INDEX, THX_MAX_ND, HipArray, call_flags, check, host_scalar_thx, lib, mark_reused, thx_array
 
 
 class HipArrayType(Type):
@@ -165,6 +165,9 @@ class HipDimShuffle(DimShuffle):
         if x.ndim != len(self.input_broadcastable):
             raise TypeError("input has %d dimensions, DimShuffle was built for %d" %
                             (x.ndim, len(self.input_broadcastable)))
+        if len(self.new_order) > THX_MAX_ND:    # the reference raises ValueError past NumPy's limit (test_too_big_rank)
+            raise ValueError("DimShuffle to rank %d: device arrays have at most %d dimensions" %
+                             (len(self.new_order), THX_MAX_ND))
         for d in self.drop:
             if x.shape[d] != 1:
                 raise ValueError("cannot drop dimension %d of extent %d" % (d, x.shape[d]))

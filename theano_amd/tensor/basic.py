@@ -372,6 +372,17 @@ def Shape_i(i):
     return ShapeFloat(i, "int64")
 
 
+def divmod(x, y):
+    """Elementwise ``(x // y, x % y)`` (``theano/tensor/basic.py:3562-3564``)."""
+    return int_div(x, y), mod(x, y)
+
+
+def squeeze(x):
+    """``x`` without its broadcastable dimensions: a view (``theano/tensor/extra_ops.py:556-579``)."""
+    x = as_tensor_variable(x)
+    return x.dimshuffle([i for i in range(x.type.ndim) if not x.type.broadcastable[i]])
+
+
 def mean(input, axis=None, dtype=None, keepdims=False, acc_dtype=None):
     """Sum divided by the extent of every reduced axis in turn; float16 inputs
     are summed in float32 and the result is cast back."""
@@ -381,7 +392,7 @@ def mean(input, axis=None, dtype=None, keepdims=False, acc_dtype=None):
     else:
         sum_dtype = "float32" if input.type.dtype == "float16" else None
     s = sum(input, axis=axis, dtype=sum_dtype, keepdims=keepdims, acc_dtype=acc_dtype)
-    shp_dtype = "float32" if s.type.dtype in ("float16", "float32") else "float64"
+    shp_dtype = "float32" if s.type.dtype in ("float16", "float32", "complex64") else "float64"
     for i in _axis_list(axis, input.type.ndim):
         s = true_div(s, ShapeFloat(i if i >= 0 else i + input.type.ndim, shp_dtype)(input))
     if s.type.dtype in discrete_dtypes:

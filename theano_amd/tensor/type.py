@@ -100,10 +100,24 @@ class _tensor_py_operators(object):
     def __abs__(self): return self._b().abs_(self)
     def __neg__(self): return self._b().neg(self)
     def __invert__(self): return self._b().invert(self)
-    def __lt__(self, o): return self._b().lt(self, o)
-    def __le__(self, o): return self._b().le(self, o)
-    def __gt__(self, o): return self._b().gt(self, o)
-    def __ge__(self, o): return self._b().ge(self, o)
+    # Results of the ordering operators refuse to be truth-tested, so that `a < b < c` (Python's
+    # `(a < b) and (b < c)`) fails loudly instead of silently dropping `a < b`
+    # (theano/tensor/var.py:52-95); every other variable is truthy.
+    _is_nonzero = True
+
+    def _comparison(self, rval):
+        rval._is_nonzero = False
+        return rval
+
+    def __lt__(self, o): return self._comparison(self._b().lt(self, o))
+    def __le__(self, o): return self._comparison(self._b().le(self, o))
+    def __gt__(self, o): return self._comparison(self._b().gt(self, o))
+    def __ge__(self, o): return self._comparison(self._b().ge(self, o))
+
+    def __bool__(self):
+        if self._is_nonzero:
+            return True
+        raise TypeError("Variables do not support boolean operations.")
     def __and__(self, o): return self._b().and_(self, o)
     def __or__(self, o): return self._b().or_(self, o)
     def __xor__(self, o): return self._b().xor(self, o)
@@ -220,6 +234,74 @@ class _tensor_py_operators(object):
 
     def all(self, axis=None, keepdims=False):
         return self._b().all(self, axis=axis, keepdims=keepdims)
+
+    def argmax(self, axis=None, keepdims=False):
+        return self._b().argmax(self, axis=axis, keepdims=keepdims)
+
+    def argmin(self, axis=None, keepdims=False):
+        return self._b().argmin(self, axis=axis, keepdims=keepdims)
+
+    def norm(self, L, axis=None, keepdims=False):
+        """``(sum |x|^L)^(1/L)`` (``theano/tensor/var.py:686-698``); L = 0 and infinity are not implemented
+        there either."""
+        if L == 0 or np.isinf(L):
+            raise NotImplementedError()
+        b = self._b()
+        y = b.pow(b.pow(abs(self), L).sum(axis=axis), 1.0 / L)
+        return b.makeKeepDims(self, y, axis) if keepdims else y
+
+    def ptp(self, axis=None):
+        return self._b().ptp(self, axis)
+
+    # -- further elementwise methods of theano/tensor/var.py
+    def clip(self, a_min, a_max):
+        return self._b().clip(self, a_min, a_max)
+
+    def round(self, mode=None):
+        return self._b().round(self, mode) if mode is not None else self._b().round(self)
+
+    def copy(self, name=None):
+        out = self._b().tensor_copy(self)
+        out.name = name
+        return out
+
+    def transpose(self, *axes):
+        if len(axes) == 1 and isinstance(axes[0], (list, tuple)):
+            axes = tuple(axes[0])
+        return self._b().transpose(self, axes if axes and axes != (None,) else None)
+
+    def swapaxes(self, axis1, axis2):
+        return self._b().swapaxes(self, axis1, axis2)
+
+    def ravel(self):
+        return self.flatten()
+
+    def squeeze(self):
+        return self._b().squeeze(self)
+
+    def __divmod__(self, o): return self._b().divmod(self, o)
+    def __rdivmod__(self, o): return self._b().divmod(o, self)
+    def __ceil__(self): return self._b().ceil(self)
+    def __floor__(self): return self._b().floor(self)
+    def __trunc__(self): return self._b().trunc(self)
+    def arccos(self): return self._b().arccos(self)
+    def arccosh(self): return self._b().arccosh(self)
+    def arcsin(self): return self._b().arcsin(self)
+    def arcsinh(self): return self._b().arcsinh(self)
+    def arctan(self): return self._b().arctan(self)
+    def arctanh(self): return self._b().arctanh(self)
+    def ceil(self): return self._b().ceil(self)
+    def cos(self): return self._b().cos(self)
+    def cosh(self): return self._b().cosh(self)
+    def exp(self): return self._b().exp(self)
+    def floor(self): return self._b().floor(self)
+    def log(self): return self._b().log(self)
+    def sin(self): return self._b().sin(self)
+    def sinh(self): return self._b().sinh(self)
+    def sqrt(self): return self._b().sqrt(self)
+    def tan(self): return self._b().tan(self)
+    def tanh(self): return self._b().tanh(self)
+    def trunc(self): return self._b().trunc(self)
 
 
 class TensorVariable(_tensor_py_operators, Variable):
