@@ -152,3 +152,58 @@ def test_gradients_of_all_any_clip_and_a_hinge_loss():
     assert np.allclose(g(iv, wv), -(Wv * (sc > 0)).sum(axis=1), rtol=1e-5, atol=1e-6)
     m = th.shared(np.asarray([1e8, 1, -1e8], dtype="float32"))
     assert np.allclose(th.function([], m.mean())(), 1.0 / 3)
+
+
+@pytest.mark.gpu
+def test_gpu_optimizer_cases_of_the_reference():
+    """``theano/gpuarray/tests/test_opt.py``: ``test_reduce`` (:143) - sum / prod with a float32 accumulator, max
+    and min over axis 0 run as one reduction node; ``test_local_gpu_elemwise_careduce`` (:362) - sqr / abs producers
+    end up as the reduction's ``pre_scalar_op`` for axis None, 0 and 1; ``test_local_gpu_elemwise`` (:457) - int8 +
+    float32 + float32 is one kernel whether the Composite is built by fusion or by the user, with several results,
+    and on every other row of its operands."""
+    from theano_amd.hip import HipCAReduce, HipElemwise
+    rng = np.random.default_rng(3)
+
+    def kernels(f, cls):
+        return [n for n in f.toposort() if isinstance(n.op, cls)]
+
+    val = rng.random((10, 11)).astype("float32")
+    for method, param in (("sum", dict(acc_dtype="float32")), ("prod", dict(acc_dtype="float32")), ("max", {}), ("min", {})):
+        m = T.fmatrix()
+        f = th.function([m], getattr(m, method)(axis=0, **param))
+        res = f(val)
+        assert res.shape == (11,) and np.allclose(res, getattr(val, method)(axis=0), rtol=1e-5)
+        assert len(kernels(f, HipCAReduce)) == 1 and not kernels(f, HipElemwise)
+
+    x = T.matrix()
+    data = rng.random((3, 4)).astype(th.config.floatX)
+    for fn, pre in ((lambda v, axis: (v * v).sum(axis=axis), "sqr"), (lambda v, axis: abs(v).sum(axis=axis), "abs"),
+                    (lambda v, axis: abs(v).max(axis=axis), "abs")):
+        for axis in (None, 0, 1):
+            f = th.function([x], fn(x, axis))
+            (red,) = kernels(f, HipCAReduce)
+            assert not kernels(f, HipElemwise) and pre in str(red.op.pre_scalar_op), (pre, axis, red.op)
+            assert np.allclose(fn(data, axis), f(data), rtol=1e-5)
+
+    a, b, c = T.bmatrix(), T.fmatrix(), T.fmatrix()
+    a_v = (rng.random((4, 5)) * 10).astype("int8")
+    b_v = (rng.random((4, 5)) * 10).astype("float32")
+    c_v = (rng.random((4, 5)) * 10).astype("float32")
+    f = th.function([a, b, c], a + b + c)
+    assert len(kernels(f, HipElemwise)) == 1 and np.allclose(f(a_v, b_v, c_v), a_v + b_v + c_v)
+    a_s, b_s, c_s = scal.int8(), scal.float32(), scal.float32()
+    out_op = T.Elemwise(scal.Composite([a_s, b_s, c_s], [a_s + b_s + c_s]))
+    f = th.function([a, b, c], out_op(a, b, c))
+    assert len(kernels(f, HipElemwise)) == 1 and np.allclose(f(a_v, b_v, c_v), a_v + b_v + c_v)
+    # several results (the part the reference's test never reaches: GpuElemwise took one output only)
+    a_s = scal.float32()
+    af = T.fmatrix()
+    outs_op = T.Elemwise(scal.Composite([a_s, b_s, c_s], [a_s + b_s, a_s * c_s]))
+    f = th.function([af, b, c], outs_op(af, b, c))
+    assert len(kernels(f, HipElemwise)) == 1
+    av = a_v.astype("float32")
+    o0, o1 = f(av, b_v, c_v)
+    assert np.allclose(o0, av + b_v) and np.allclose(o1, av * c_v)
+    cs = th.shared(c_v)
+    o0, o1 = th.function([af, b], outs_op(af[::2], b[::2], cs[::2]))(av, b_v)
+    assert np.allclose(o0, av[::2] + b_v[::2]) and np.allclose(o1, av[::2] * c_v[::2])

@@ -587,11 +587,21 @@ def local_split_huge_add_or_mul(fgraph, node):
     return [new] if new.type == node.outputs[0].type else False
 
 
+@local_optimizer([Elemwise])
+def local_mul_to_sqr(fgraph, node):
+    """``x * x -> sqr(x)`` (``theano/tensor/opt.py:5865-5876``): one operand to fetch instead of two, and the
+    form the reductions' prologues and the variance rewrite look for."""
+    if not isinstance(node.op.scalar_op, scal.Mul) or len(node.inputs) != 2 or node.inputs[0] is not node.inputs[1]:
+        return False
+    new = T.sqr(node.inputs[0])
+    return [new] if new.type == node.outputs[0].type else False
+
+
 CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_useless_composite, local_constant_fold,
                 local_useless_elemwise, local_fill_sink,
                 local_useless_reduce, local_op_of_op,
                 local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_single_pass_variance,
-                local_cancel_common_factors, local_split_huge_add_or_mul]
+                local_cancel_common_factors, local_split_huge_add_or_mul, local_mul_to_sqr]
 
 
 def canonicalize(fgraph):
