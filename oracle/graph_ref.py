@@ -146,8 +146,14 @@ def _check_broadcast(node, values):
             if owner[d] is None:
                 owner[d], shape[d] = k, val.shape[d]
             elif val.shape[d] != shape[d]:
-                raise ValueError("Input dimension mis-match. (input[%d].shape[%d] = %d, input[%d].shape[%d] = %d)"
-                                 % (owner[d], d, shape[d], k, d, val.shape[d]))
+                # Elemwise.perform (theano/tensor/elemwise.py:720-751) objects only when the largest extent of
+                # the dimension is not 1: an extent of 1 beside an empty operand passes and the result is empty
+                # (out_shape 0 when any extent is 0) - the `empty` case of theano/tensor/tests/test_basic.py:680
+                if (val.shape[d], shape[d]) == (0, 1):
+                    owner[d], shape[d] = k, 0
+                elif (val.shape[d], shape[d]) != (1, 0):
+                    raise ValueError("Input dimension mis-match. (input[%d].shape[%d] = %d, input[%d].shape[%d] = %d)"
+                                     % (owner[d], d, shape[d], k, d, val.shape[d]))
 
 
 def _wide(dtype):

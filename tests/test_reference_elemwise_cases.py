@@ -207,3 +207,54 @@ def test_gpu_optimizer_cases_of_the_reference():
     cs = th.shared(c_v)
     o0, o1 = th.function([af, b], outs_op(af[::2], b[::2], cs[::2]))(av, b_v)
     assert np.allclose(o0, av[::2] + b_v[::2]) and np.allclose(o1, av[::2] * c_v[::2])
+
+
+def test_oracle_lets_an_extent_of_one_pass_beside_an_empty_operand():
+    """``Elemwise.perform`` (``theano/tensor/elemwise.py:720-751``) raises only when the largest extent of a
+    dimension is not 1; ``[] + [1]`` is the `empty` good case of every binary tester
+    (``theano/tensor/tests/test_basic.py:680``).  (2, 3) + (1, 3) typed without broadcasting still raises."""
+    from oracle import graph_ref as G
+    a, b = T.vector("a"), T.vector("b")
+    (out,) = G.evaluate([a, b], [a + b], [np.asarray([], "float32"), np.asarray([1], "float32")])
+    assert out.shape == (0,) and out.dtype == np.float32
+    x, y = T.matrix("x"), T.matrix("y")
+    with pytest.raises(ValueError, match="mis-match"):
+        G.evaluate([x, y], [x + y], [np.zeros((2, 3), "float32"), np.zeros((1, 3), "float32")])
+
+
+@pytest.mark.gpu
+def test_named_input_patterns_of_the_binary_testers():
+    """``_good_broadcast_binary_normal`` (``theano/tensor/tests/test_basic.py:664-682``) by name - same_shapes,
+    not_same_dimensions, scalar, row, column, integers, uint32, uint16, dtype_mixup_1 / 2, complex1 / 2, empty -
+    for add, sub, mul, true_div, maximum and minimum against the oracle; and the two must-raise cases (:686-688)."""
+    from oracle import graph_ref as G
+    from conftest import assert_parity
+    rng = np.random.default_rng(11)
+    rand = lambda *s: rng.uniform(-1, 1, s).astype("float32")
+    randint = lambda *s: rng.integers(-5, 6, s).astype("int32")
+    randc = lambda *s: (rng.uniform(-1, 1, s) + 1j * rng.uniform(-1, 1, s)).astype("complex64")
+    cases = dict(
+        same_shapes=(rand(2, 3), rand(2, 3)), not_same_dimensions=(rand(2, 2), rand(2)), scalar=(rand(2, 3), rand(1, 1)),
+        row=(rand(2, 3), rand(1, 3)), column=(rand(2, 3), rand(2, 1)), integers=(randint(2, 3), randint(2, 3)),
+        uint32=(rng.integers(0, 9, (2, 3)).astype("uint32"), rng.integers(1, 9, (2, 3)).astype("uint32")),
+        uint16=(rng.integers(0, 9, (2, 3)).astype("uint16"), rng.integers(1, 9, (2, 3)).astype("uint16")),
+        dtype_mixup_1=(rand(2, 3), randint(2, 3)), dtype_mixup_2=(randint(2, 3), rand(2, 3)),
+        complex1=(randc(2, 3), randc(2, 3)), complex2=(randc(2, 3), rand(2, 3)),
+        empty=(np.asarray([], dtype="float32"), np.asarray([1], dtype="float32")))
+    for name, (av, bv) in cases.items():
+        # as the testers do: a dimension is typed broadcastable exactly when its extent is 1, except in `empty`
+        bc = lambda v: [s == 1 for s in v.shape] if name != "empty" else [False] * v.ndim
+        a, b = T.TensorType(str(av.dtype), bc(av))("a"), T.TensorType(str(bv.dtype), bc(bv))("b")
+        bsafe = T.switch(T.eq(b, 0), T.ones_like(b), b) if bv.dtype.kind in "iu" else b
+        outs = [a + b, a - b, a * b, a / bsafe]
+        if av.dtype.kind != "c":
+            outs += [T.maximum(a, b), T.minimum(a, b)]
+        got = th.function([a, b], outs)(av, bv)
+        ref = G.evaluate([a, b], outs, [av, bv])
+        for k, (g, r) in enumerate(zip(got, ref)):
+            assert_parity(g, r, "%s op %d" % (name, k))
+    x, y = T.matrix("x"), T.matrix("y")
+    f = th.function([x, y], x + y)
+    for bad in ((rand(2, 3), rand(3, 2)), (rand(2, 3), rand(1, 2))):
+        with pytest.raises(ValueError):
+            f(*bad)

@@ -235,8 +235,14 @@ def _check_runtime_broadcast(node_inputs, values, nd):
             if owner[d] is None:
                 owner[d], shape[d] = k, vshape[d]
             elif vshape[d] != shape[d]:
-                raise ValueError("Input dimension mis-match. (input[%d].shape[%d] = %d, input[%d].shape[%d] = %d)" %
-                                 (owner[d], d, shape[d], k, d, vshape[d]))
+                # an extent of 1 beside an empty operand is let through and the result is empty, as in
+                # Elemwise.perform (theano/tensor/elemwise.py:720-751: the check fires only when the largest
+                # extent is not 1; `[] + [1]` is a good case of the reference's broadcast testers)
+                if (vshape[d], shape[d]) == (0, 1):
+                    owner[d], shape[d] = k, 0
+                elif (vshape[d], shape[d]) != (1, 0):
+                    raise ValueError("Input dimension mis-match. (input[%d].shape[%d] = %d, input[%d].shape[%d] = %d)" %
+                                     (owner[d], d, shape[d], k, d, vshape[d]))
     return tuple(shape)
 
 
