@@ -258,3 +258,53 @@ def test_named_input_patterns_of_the_binary_testers():
     for bad in ((rand(2, 3), rand(3, 2)), (rand(2, 3), rand(1, 2))):
         with pytest.raises(ValueError):
             f(*bad)
+
+
+def test_composite_cases_of_the_scalar_tests():
+    """``theano/scalar/tests/test_basic.py`` ``test_composite`` (:72-184): ``clone_float32`` leaves no float16
+    variable, nested Composites are inlined, constants stay literals of the code, ``make_node`` accepts variables
+    of other types and rebuilds, and the values of `test_straightforward`, `test_with_constants` and
+    `test_many_outputs` come out of the oracle's evaluation of the Composite."""
+    from theano_amd import gof
+    from theano_amd.scalar import Composite
+    from oracle import graph_ref as G
+
+    def has_f16(comp):
+        vs = set(comp.inputs) | set(comp.outputs)
+        for n in gof.io_toposort(comp.inputs, comp.outputs):
+            vs |= set(n.inputs) | set(n.outputs)
+        return any(v.type.dtype == "float16" for v in vs)
+
+    w, x, y = scal.int8(), scal.float16(), scal.float32()
+    cz = Composite([x, y], [scal.tanh(x + scal.cast(y, "float16"))])
+    c = Composite([w, x, y], [cz(x, y) - cz(x, y) ** 2 + scal.cast(x, "int16") + scal.cast(x, "float32") +
+                              scal.cast(w, "float16") - scal.constant(np.float16(1.0))])
+    assert has_f16(c) and not has_f16(c.clone_float32())
+    v, w, x, y, z = scal.uint8(), scal.float16(), scal.float16(), scal.float16(), scal.float16()
+    c = Composite([v, w, x, y, z], [scal.switch(v, scal.mul(w, x, y), z)])
+    assert has_f16(c) and not has_f16(c.clone_float32())
+    assert [i.type.dtype for i in c.clone_float32().inputs] == ["uint8"] + ["float32"] * 4
+
+    x, y, z = scal.float64("x"), scal.float64("y"), scal.float64("z")
+    C = Composite([x, y], [x + y])
+    CC = Composite([x, y], [C(x * y, y)])
+    assert not isinstance(CC.outputs[0].owner.op, Composite)
+    e = scal.mul(scal.add(70.0, y), scal.div_proxy(x, y))
+    node = Composite([x, y], [e]).make_node(x, y)
+    assert "70.0" in node.op.c_code(node, ["x", "y"], ["z"])
+
+    def run(comp, *vals):
+        ins = [T.TensorType(i.type.dtype, ())() for i in comp.inputs]
+        outs = T.Elemwise(comp)(*ins)
+        outs = outs if isinstance(outs, (list, tuple)) else [outs]
+        return [float(o) for o in G.evaluate(ins, list(outs), [np.asarray(v, i.type.dtype) for v, i in zip(vals, ins)])]
+
+    assert run(Composite([x, y], [scal.mul(scal.add(x, y), scal.div_proxy(x, y))]), 1.0, 2.0) == [1.5]
+    assert run(Composite([x, y], [e]), 1.0, 2.0) == [36.0]
+    assert run(Composite([x, y, z], [x + y + z, x + y * z, x / y]), 1.0, 2.0, 3.0) == [6.0, 7.0, 0.5]
+    # test_make_node_continue_graph (:165-184): operands that are results of other scalar computation
+    si0, si1, si2 = scal.int8(), scal.int8(), scal.float32()
+    sop = Composite([si0, si1, si2], [(si0 * si1) / si2])
+    a, b, cc, d = scal.int8(), scal.int8(), scal.float32(), scal.float32()
+    rebuilt = sop.make_node(a * d, b, cc)
+    assert rebuilt.op.inputs_type[0].dtype == "float32"

@@ -1622,6 +1622,43 @@ class Composite(ScalarOp):
         op = Composite(new_ins, [memo.get(o, o) for o in self.outputs])
         return Apply(op, inputs, [t() for t in op.outputs_type])
 
+    def clone_float32(self):
+        """The same Composite with every float16 value computed in float32 (``Compositef32`` and
+        ``Composite.clone_float32``, ``theano/scalar/basic.py:4130-4208``, what ``GpuElemwise`` hands to its
+        kernel generator): float16 inputs and constants become float32, a cast from float32 to float16 and a
+        cast of a float16 value to the type it now has disappear, any other cast to float16 becomes a cast to
+        float32.  (The kernels here widen float16 on load and round on store, so the generated code of a
+        float16 Composite already computes this way; the method is the reference's interface to that form.)"""
+        mapping = {}
+        for i in self.inputs:
+            mapping[i] = float32() if i.type.dtype == "float16" else i.type()
+        for node in gof.io_toposort(self.inputs, self.outputs):
+            for i in node.inputs:
+                if i not in mapping:
+                    if not isinstance(i, Constant):
+                        raise ValueError("Composite graph uses a variable that is not an input: %s" % i)
+                    mapping[i] = constant(np.float32(i.data)) if i.type.dtype == "float16" else i
+            out = node.outputs[0]
+            if isinstance(node.op, Cast):
+                inp = mapping[node.inputs[0]]
+                to_half = node.op.o_type.dtype == "float16"
+                if to_half and node.inputs[0].type.dtype == "float32":
+                    mapping[out] = inp                      # float32 -> float16: gone
+                    continue
+                o_type = float32 if to_half else node.op.o_type
+                src_is_half = inp.type.dtype == "float16" if to_half else node.inputs[0].type.dtype == "float16"
+                if (to_half or src_is_half) and o_type == inp.type:
+                    mapping[out] = inp                      # a cast to the type the value already has
+                    continue
+                mapping[out] = cast(inp, o_type.dtype)
+                continue
+            new_node = node.op.make_node(*[mapping[i] for i in node.inputs])
+            if any(o.type.dtype == "float16" for o in new_node.outputs):
+                raise TypeError("%s still yields float16 from float32 operands" % node.op)
+            for o, no in zip(node.outputs, new_node.outputs):
+                mapping[o] = no
+        return Composite([mapping[i] for i in self.inputs], [mapping[o] for o in self.outputs])
+
     def c_code(self, node, inputs, outputs):
         # The temporaries' prefix is a digest of the operand names: the same in every process, so
         # that the text (and the kernel cache key made from it) is reproducible, and different
