@@ -312,6 +312,7 @@ struct HeldCtx {
       A b = shfl_xor_t(a, m);
       Op::comb(a, b);
     }
+    if (NW == 1) return a;          // a block of one wave: the butterfly was all of it
     __syncthreads();
     if ((t & (THX_WAVE - 1)) == 0) lds[t / THX_WAVE] = a;
     __syncthreads();

@@ -198,10 +198,12 @@ static int held_call(thx_rowchain* c, const thx_array* ins, const thx_array* out
   const int64_t bv = B / vec;
   if (A * bv >= (int64_t(1) << 30)) return fail(THX_ERR_UNSUPPORTED, "rowchain: reduce domains of %lld elements", (long long)(A * B));
   const int64_t nvec = A * bv;
-  int block = nvec > 256 * 8 ? 1024 : 256;
+  // one wave for short domains (many kept indices of a few hundred elements: no barrier, no idle waves),
+  // 256 threads up to 8 vectors each, 1024 beyond
+  int block = nvec > 256 * 8 ? 1024 : nvec > 64 * 8 ? 256 : 64;
   {
     const int fb = env_int("THX_HELD_BLOCK", 0);
-    if (fb == 256 || fb == 512 || fb == 1024) block = fb;
+    if (fb == 64 || fb == 256 || fb == 512 || fb == 1024) block = fb;
   }
   const int nch = (int)((nvec + block - 1) / block);
   // what one thread holds: dwords per chunk and input; registers first, then LDS
@@ -212,7 +214,7 @@ static int held_call(thx_rowchain* c, const thx_array* ins, const thx_array* out
       words[i] = (vec * dtype_size(c->dtypes[i]) + 3) / 4;
       total += nch * words[i];
     }
-  const int reg_budget = env_int("THX_HELD_REGS", block == 1024 ? 64 : block == 512 ? 160 : 320);
+  const int reg_budget = env_int("THX_HELD_REGS", block == 1024 ? 64 : block == 512 ? 160 : 320);  // (64 / 256 threads: 512 registers a lane)
   const int lds_budget = 144 * 1024;
   int need = total - reg_budget, lds_bytes = 0;
   for (int i = 0; i < NIN && need > 0; ++i) {
