@@ -374,11 +374,15 @@ class HipRowChain(Op):
         if layout in refused:           # turned away before with these shapes and strides
             results = self._run_fallback(inputs)
         else:
+            last = node.tag.get("thx_last")
+            if last is None:
+                last = node.tag["thx_last"] = [None] * len(inputs)
             for k, v in enumerate(inputs):
                 if type(v) is HipArray:
                     v.as_thx(ins[k])
-                else:
+                elif last[k] is not v:          # the same host array as last time: its descriptor stands
                     host_scalar_thx(v, nd, ins[k])
+                    last[k] = v
             results = []
             for k, ((vid, kind, dt), t) in enumerate(zip(p.outputs, self.out_types)):
                 shape = full if kind == FULL else _row_shape(full, red, t.ndim == nd)
