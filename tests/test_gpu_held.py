@@ -236,3 +236,26 @@ def test_random_normalisation_graph_matches_the_oracle(seed):
         else:
             assert_within_reference_error(g, r, w, "seed %d output %d" % (seed, k),
                                           tol=dict(rtol=2e-3, atol=2e-3) if dtype == "float16" else None)
+
+
+@pytest.mark.parametrize("dtype", ["complex64", "complex128", "int8", "uint16", "int64", "bool"])
+def test_chains_over_every_dtype_family(dtype):
+    """A sum over the last axis (row chain) and over axes (0, 2) (held chain) multiplied back into the operand,
+    in complex, small-integer, wide-integer and bool arithmetic; integers and bools bit for bit."""
+    rng = np.random.default_rng(21)
+    for axes, shape in (((1,), (6, 40)), ((0, 2), (5, 7, 12))):
+        z = tensor(dtype, len(shape), "z")
+        s = T.sum(z, axis=axes, keepdims=True)
+        out = (z & T.cast(s, "bool")) if dtype == "bool" else z * s
+        if dtype.startswith("complex"):
+            zv = (rng.uniform(-1, 1, shape) + 1j * rng.uniform(-1, 1, shape)).astype(dtype)
+        elif dtype == "bool":
+            zv = rng.random(shape) < 0.4
+        else:
+            zv = rng.integers(0 if dtype.startswith("u") else -9, 10, shape).astype(dtype)
+        f = th.function([z], [out, s])
+        got = f(zv)
+        assert [n for n in f.toposort() if isinstance(n.op, HipRowChain)], (dtype, axes)
+        ref = G.evaluate([z], [out, s], [zv])
+        for k, (g, r) in enumerate(zip(got, ref)):
+            assert_parity(g, r, "%s %s output %d" % (dtype, axes, k))
