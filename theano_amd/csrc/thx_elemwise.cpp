@@ -339,7 +339,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
         int64_t groups = 1;
         if (red) {
           const int64_t cus = rt().ready ? rt().cus : 256;
-          const int bpc = std::max(1, env_int("THX_EW_RED_BLOCKS_PER_CU", 6));  // 4 to 6 measured best (partials stay few)
+          const int bpc = std::max(1, env_int("THX_EW_RED_BLOCKS_PER_CU", 4));  // 3 to 6 measured within 1 %, 8 and 2 worse (partials stay few)
           const int64_t g0 = std::max<int64_t>(1, std::min(rowtiles, cus * bpc / tiles_i));
           groups = ceil_div64(rowtiles, ceil_div64(rowtiles, g0));
         }
