@@ -623,6 +623,18 @@ def test_ops_and_graphs_pickle(dry_run):
         for n in th.function(*g).toposort():
             again = pickle.loads(pickle.dumps(n.op))
             assert again == n.op and hash(again) == hash(n.op), n.op
+    # a chain node that has compiled its island as separate kernels (device handles inside) still pickles
+    from theano_amd.hip.rowchain import HipRowChain
+    os.environ["THX_HELD"] = "0"
+    try:
+        f = th.function(*W.c5_graph(with_grad=False))
+        f(*W.c5_inputs("small", with_grad=False))
+    finally:
+        del os.environ["THX_HELD"]
+    (chain,) = ops_of(f, HipRowChain)
+    assert chain.op._fallback_function is not None
+    again = pickle.loads(pickle.dumps(chain.op))
+    assert again == chain.op and not hasattr(again, "_fallback_function")
     x = T.fmatrix("x")
     y = T.sum(T.exp(x) * T.nnet.sigmoid(x) + T.erf(x) % 3, axis=1)
     z = T.nnet.softmax(x)[:, ::2].reshape((-1,))

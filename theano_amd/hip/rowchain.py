@@ -325,6 +325,12 @@ class HipRowChain(Op):
     def make_node(self, *inputs):
         return Apply(self, list(inputs), [t() for t in self.out_types])
 
+    def __getstate__(self):
+        # the compiled form of the island (device handles inside) is rebuilt on first use
+        d = dict(self.__dict__)
+        d.pop("_fallback_function", None)
+        return d
+
     def infer_shape(self, node, shapes):
         full = None
         for s, k in zip(shapes, self.program.in_kinds):
@@ -371,6 +377,8 @@ class HipRowChain(Op):
         red = self._red(nd)
         layout = tuple((v.shape, v.strides) for v in inputs if type(v) is HipArray)
         refused = node.tag.setdefault("thx_refused", set())
+        if len(refused) > 256:          # a function called with ever new shapes: start over
+            refused.clear()
         if layout in refused:           # turned away before with these shapes and strides
             results = self._run_fallback(inputs)
         else:
