@@ -259,3 +259,35 @@ def test_chains_over_every_dtype_family(dtype):
         ref = G.evaluate([z], [out, s], [zv])
         for k, (g, r) in enumerate(zip(got, ref)):
             assert_parity(g, r, "%s %s output %d" % (dtype, axes, k))
+
+
+def random_normalisation_gradient(seed):
+    """The graph of ``random_normalisation_graph`` followed by the gradient of sum(y * gy) with respect to its
+    full-sized operands (gy one more full-sized input): chains that hold two or three operands and loop over
+    them three or four times."""
+    ins, outs, vals, dtype = random_normalisation_graph(seed)
+    rng = np.random.default_rng(seed + 7)
+    y = outs[0]
+    gy = tensor(dtype, y.type.ndim, "gy")
+    wide = "float32" if dtype == "float16" else dtype
+    cost = T.sum(T.cast(y, wide) * T.cast(gy, wide))
+    wrt = [v for v in ins if v.type.ndim == y.type.ndim and not any(v.type.broadcastable)]
+    grads = [T.cast(g, dtype) for g in th.grad(cost, wrt)]
+    shape = G.evaluate(ins, [y], vals)[0].shape
+    return ins + [gy], grads + ([y] if seed % 2 else []), vals + [rng.standard_normal(shape).astype(dtype)], dtype
+
+
+@pytest.mark.parametrize("seed", list(range(100, 124)))
+def test_random_normalisation_gradient_matches_the_oracle(seed):
+    ins, outs, vals, dtype = random_normalisation_gradient(seed)
+    f = th.function(ins, outs)
+    got = f(*vals)
+    assert [n for n in f.toposort() if isinstance(n.op, HipRowChain)], seed
+    ref = G.evaluate(ins, outs, vals)
+    truth = G.evaluate(ins, outs, vals, wide=True)
+    for k, (g, r, w) in enumerate(zip(got, ref, truth)):
+        if dtype == "float64":
+            assert_parity(g, r, "seed %d output %d" % (seed, k), tol=dict(rtol=1e-10, atol=1e-10))
+        else:
+            assert_within_reference_error(g, r, w, "seed %d output %d" % (seed, k),
+                                          tol=dict(rtol=2e-3, atol=2e-3) if dtype == "float16" else None)
