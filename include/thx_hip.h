@@ -127,7 +127,10 @@ int thx_elemwise_new(const char* functor_src, const char* functor_name, int n_in
 
 #define THX_BROADCAST 1 /* size-1 input dimensions broadcast against larger ones */
 #define THX_DRY_RUN 2   /* validate, plan and compile (into the disk cache) but do not launch;
-                           needs no device: the target is $THX_ARCH, default gfx950 */
+                           needs no device: the target is $THX_ARCH, default gfx950, and device
+                           arrays may carry a null base (their addresses then count as aligned).
+                           Without this flag an array that has elements and a null base is
+                           refused with THX_ERR_ARG before anything is launched. */
 
 /* Run on `ins` (n_in arrays) writing `outs` (n_out arrays, preallocated, every
  * one of the full result shape; an output may alias an input exactly for

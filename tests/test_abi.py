@@ -88,6 +88,32 @@ def test_c_level_shape_check(dry_run):
     assert rc == 2 and b"mis-match" in runtime.lib.thx_last_error()
 
 
+def test_a_host_scalar_without_an_address_is_refused(dry_run):
+    # the planner itself reads a scalar passed from the host: a null base is refused even in a dry run,
+    # where device arrays need no address
+    from theano_amd.hip.ops import HipElemwise
+    from theano_amd import scalar as scal
+    x, y = T.fmatrix(), T.fscalar()
+    node = HipElemwise(scal.add).make_node(x, y.dimshuffle("x", "x"))
+    handle, _, _ = node.op._handle(node)
+    a = runtime.HipArray.empty((4, 5), "float32")
+    o = runtime.HipArray.empty((4, 5), "float32")
+    ins = (runtime.thx_array * 2)()
+    a.as_thx(ins[0])
+    two = np.full((1, 1), 2.0, "float32")
+    runtime.host_scalar_thx(two, 2, ins[1])
+    outs = (runtime.thx_array * 1)()
+    o.as_thx(outs[0])
+    flags = runtime.THX_BROADCAST | runtime.THX_DRY_RUN
+    assert runtime.lib.thx_elemwise_call(handle, ins, outs, flags) == 0
+    ins[0].base = None
+    outs[0].base = None
+    assert runtime.lib.thx_elemwise_call(handle, ins, outs, flags) == 0
+    ins[1].base = None
+    assert runtime.lib.thx_elemwise_call(handle, ins, outs, flags) == 7
+    assert b"no base address" in runtime.lib.thx_last_error()
+
+
 def test_zero_length_max_raises(dry_run):
     x = T.fmatrix()
     f = th.function([x], x.max(axis=1))
@@ -207,3 +233,55 @@ def test_the_c_host_runs_on_the_device(tmp_path):
     exe = _build_c_client(tmp_path)
     res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
     assert res.returncode == 0 and res.stdout.strip().endswith("ok"), res.stdout + res.stderr
+
+
+@pytest.mark.gpu
+def test_device_operands_without_an_address_are_refused_before_any_launch():
+    # every family of entry points: a null base behind a non-empty array comes back as THX_ERR_ARG, nothing runs
+    from theano_amd.hip.ops import HipElemwise
+    from theano_amd import scalar as scal
+    runtime.init()
+    a = runtime.HipArray.from_numpy(np.ones((4, 5), "float32"))
+    b = runtime.HipArray.from_numpy(np.ones((4, 5), "float32"))
+    o = runtime.HipArray.empty((4, 5), "float32")
+    x, y = T.fmatrix(), T.fmatrix()
+    node = HipElemwise(scal.add).make_node(x, y)
+    handle, _, _ = node.op._handle(node)
+    for which in ("in", "out"):
+        ins = (runtime.thx_array * 2)()
+        a.as_thx(ins[0]); b.as_thx(ins[1])
+        outs = (runtime.thx_array * 1)()
+        o.as_thx(outs[0])
+        if which == "in":
+            ins[1].base = None
+        else:
+            outs[0].base = None
+        assert runtime.lib.thx_elemwise_call(handle, ins, outs, runtime.THX_BROADCAST) == 7
+        assert b"no base address" in runtime.lib.thx_last_error()
+    # the same operands with their addresses run
+    ins = (runtime.thx_array * 2)()
+    a.as_thx(ins[0]); b.as_thx(ins[1])
+    outs = (runtime.thx_array * 1)()
+    o.as_thx(outs[0])
+    assert runtime.lib.thx_elemwise_call(handle, ins, outs, runtime.THX_BROADCAST) == 0
+    np.testing.assert_array_equal(o.to_numpy(), np.full((4, 5), 2, "float32"))
+
+    from theano_amd.hip import codegen
+    src, name, acc_bytes = codegen.reduce_functor((scal.add,), ("float64",), ("float32",), ("float32",), None)
+    codes = (ctypes.c_int32 * 2)(scal.dtype_code("float32"), scal.dtype_code("float32"))
+    rhandle = ctypes.c_void_p()
+    runtime.check(runtime.lib.thx_reduce_new(src.encode(), name.encode(), 1, 1, 0, codes, acc_bytes, ctypes.byref(rhandle)))
+    mask = (ctypes.c_uint8 * 2)(0, 1)
+    r = runtime.HipArray.empty((4,), "float32")
+    for which in ("in", "out"):
+        ins = (runtime.thx_array * 1)()
+        a.as_thx(ins[0])
+        outs = (runtime.thx_array * 1)()
+        r.as_thx(outs[0])
+        if which == "in":
+            ins[0].base = None
+        else:
+            outs[0].base = None
+        assert runtime.lib.thx_reduce_call(rhandle, ins, mask, outs, 0) == 7
+        assert b"no base address" in runtime.lib.thx_last_error()
+    runtime.lib.thx_reduce_free(rhandle)

@@ -126,6 +126,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
       return fail(THX_ERR_TYPE, "elemwise: output %d has dtype code %d, the operation was built for %d", o, adt,
                   e->dtypes[e->n_in + o]);
     const int isz = dtype_size(adt);
+    if (null_base(a, dry)) return fail(THX_ERR_ARG, "elemwise: output %d has no base address", o);
     v.ptr = (char*)a.base + a.offset_bytes;
     v.dtype = adt;
     v.reused = (a.dtype & THX_REUSED) != 0;
@@ -361,6 +362,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
             if (adt != R->dtypes[R->n_in + o] || count != ext_i || !contiguous)
               return fail(THX_ERR_TYPE, "elemwise: reduction result %d must be a C-contiguous array of %lld elements of "
                           "dtype code %d", o, (long long)ext_i, R->dtypes[R->n_in + o]);
+            if (null_base(a, dry)) return fail(THX_ERR_ARG, "elemwise: reduction result %d has no base address", o);
             routp.push_back((char*)a.base + a.offset_bytes);
           }
           if (rowtiles >= (int64_t(1) << 31)) return fail(THX_ERR_UNSUPPORTED, "elemwise: %lld tiles", (long long)rowtiles);

@@ -18,6 +18,16 @@ namespace thx {
 // ---- errors ---------------------------------------------------------------
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 void set_last_plan(const std::string& plan);
+// True when `a` has elements and no address to read them at: such an operand must be refused before a
+// kernel or a host copy dereferences it.  A dry run launches nothing and needs no device addresses; a scalar
+// passed from the host is read by the planner itself and always needs one.
+inline bool null_base(const thx_array& a, bool dry) {
+  if (a.base || (a.dtype & THX_INDEX)) return false;
+  if (dry && !(a.dtype & THX_HOST_SCALAR)) return false;
+  for (int d = 0; d < a.nd && d < THX_MAX_ND; ++d)
+    if (a.shape[d] == 0) return false;
+  return true;
+}
 
 #define THX_HIP_CHECK(expr)                                                        \
   do {                                                                             \

@@ -229,6 +229,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
         return fail(THX_ERR_TYPE, "reduce: output %d is not C-contiguous", o);
       expect *= a.shape[d];
     }
+    if (null_base(a, dry)) return fail(THX_ERR_ARG, "reduce: output %d has no base address", o);
     outp[o] = (char*)a.base + a.offset_bytes;
     if (((uintptr_t)outp[o]) % isz) return fail(THX_ERR_TYPE, "reduce: output %d is not aligned to its element size", o);
   }
@@ -245,6 +246,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     if ((a.dtype & ~(THX_HOST_SCALAR | THX_REUSED)) != want)
       return fail(THX_ERR_TYPE, "reduce: epilogue operand %d has dtype code %d, the operation was built for %d", j,
                   a.dtype & ~(THX_HOST_SCALAR | THX_REUSED), want);
+    if (null_base(a, dry)) return fail(THX_ERR_ARG, "reduce: epilogue operand %d has no base address", j);
     const char* p = (const char*)a.base + a.offset_bytes;
     if (a.dtype & THX_HOST_SCALAR) {
       if (dtype_size(want) > 8)

@@ -127,6 +127,7 @@ static int held_call(thx_rowchain* c, const thx_array* ins, const thx_array* out
     const int dt = a.dtype & ~(THX_HOST_SCALAR | THX_REUSED);
     if (dt != c->dtypes[i]) return fail(THX_ERR_TYPE, "rowchain: operand %d has dtype code %d, expected %d", i, dt, c->dtypes[i]);
     const int isz = dtype_size(dt);
+    if (null_base(a, dry)) return fail(THX_ERR_ARG, "rowchain: operand %d has no base address", i);
     char* p = (char*)a.base + a.offset_bytes;
     if (a.dtype & THX_HOST_SCALAR) {
       if (kind != K_SCALAR || i >= NIN || isz > 8) return fail(THX_ERR_TYPE, "rowchain: operand %d cannot be a host scalar", i);
@@ -411,6 +412,7 @@ int thx_rowchain_call(thx_rowchain* c, const thx_array* ins, const thx_array* ou
     const int dt = a.dtype & ~(THX_HOST_SCALAR | THX_REUSED);
     if (dt != c->dtypes[i]) return fail(THX_ERR_TYPE, "rowchain: operand %d has dtype code %d, expected %d", i, dt, c->dtypes[i]);
     const int isz = dtype_size(dt);
+    if (null_base(a, dry)) return fail(THX_ERR_ARG, "rowchain: operand %d has no base address", i);
     char* p = (char*)a.base + a.offset_bytes;
     if (a.dtype & THX_HOST_SCALAR) {
       if (kind != K_SCALAR || i >= NIN || isz > 8) return fail(THX_ERR_TYPE, "rowchain: operand %d cannot be a host scalar", i);

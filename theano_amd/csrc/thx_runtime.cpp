@@ -210,6 +210,7 @@ int gather_inputs(const char* what, const thx_array* ins, int n_in, const int32_
   views->assign(n_in, View());
   for (int i = 0; i < n_in; ++i) {
     View& v = (*views)[i];
+    if (null_base(ins[i], (flags & THX_DRY_RUN) != 0)) return fail(THX_ERR_ARG, "%s: input %d has no base address", what, i);
     v.ptr = (char*)ins[i].base + ins[i].offset_bytes;
     v.reused = (ins[i].dtype & THX_REUSED) != 0;
     v.dtype = ins[i].dtype & ~(THX_HOST_SCALAR | THX_INDEX | THX_REUSED);
