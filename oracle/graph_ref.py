@@ -178,7 +178,10 @@ def eval_scalar_op(op, in_values, out_dtypes, wide=False):
             for o, v in zip(node.outputs, outs):
                 env[o] = v
         return [env[o] if o in env else np.asarray(o.data) for o in op.outputs]
-    fn = scalar_ref.restatement(name, out_dtypes[0], [np.asarray(v).dtype for v in in_values])
+    if name == "InRange":
+        fn = scalar_ref.in_range(op.openlow, op.openhi)
+    else:
+        fn = scalar_ref.restatement(name, out_dtypes[0], [np.asarray(v).dtype for v in in_values])
     if fn is None:
         raise NotImplementedError("no restatement of scalar op %s" % name)
     return [np.asarray(fn(out_dtypes[0], *[np.asarray(v) for v in in_values]))]

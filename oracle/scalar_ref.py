@@ -265,6 +265,31 @@ lt, gt, le, ge, eq, neq = (_cmp(np.less), _cmp(np.greater), _cmp(np.less_equal),
                            _cmp(np.equal), _cmp(np.not_equal))
 
 
+def in_range(openlow, openhi):
+    """``InRange.c_code`` (``theano/scalar/basic.py:1452-1460``): ``x > low && x < hi`` with ``>=`` / ``<=``
+    at a closed end; each comparison converts its two operands as C does."""
+    lo, hi = (gt if openlow else ge), (lt if openhi else le)
+
+    def f(out_dtype, x, low, high):
+        return np.logical_and(lo(out_dtype, x, low), hi(out_dtype, x, high))
+    return f
+
+
+def _angle_unit(factor):
+    """``Deg2Rad`` / ``Rad2Deg.c_code`` (``theano/scalar/basic.py:3110-3149``): ``z = x * (M_PI / 180.0)`` resp.
+    ``x * (180.0 / M_PI)`` - the product is taken in double precision whatever x is (an integer, a float32 and a
+    float16 operand all promote to double against the double constant), then converted to the result type."""
+    def f(out_dtype, x):
+        prod = x.astype("float64") * np.float64(factor)
+        if str(out_dtype) == "float16":       # float16 values are computed as float and stored as half
+            prod = _conv(prod, "float32")
+        return _conv(prod, out_dtype)
+    return f
+
+
+deg2rad, rad2deg = _angle_unit(np.pi / 180.0), _angle_unit(180.0 / np.pi)
+
+
 def _bit(fn):
     def f(out_dtype, x, y):
         if str(out_dtype) == "bool":
@@ -609,5 +634,5 @@ BY_CLASS = {
     "UltraFastScalarSigmoid": ultra_fast_scalar_sigmoid, "ScalarSoftsign": scalar_softsign,
     "SigmoidBinaryCrossentropy": sigmoid_binary_crossentropy, "Jv": jv, "Iv": iv,
     "Real": real, "Imag": imag, "Angle": angle, "Conj": conj, "Complex": complex_,
-    "ComplexFromPolar": complex_from_polar,
+    "ComplexFromPolar": complex_from_polar, "Deg2Rad": deg2rad, "Rad2Deg": rad2deg,
 }

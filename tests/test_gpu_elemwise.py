@@ -101,6 +101,36 @@ def test_unary_math(dtype):
         assert_parity(g, r, "%s unary %d" % (dtype, k), tol=tol)
 
 
+def test_angle_units_and_range_tests_follow_the_c_text():
+    """deg2rad / rad2deg multiply by a double constant and round once; InRange is two comparisons under C's
+    conversions (theano/scalar/basic.py:3086-3150, 1434-1481): bit for bit against the oracle."""
+    from theano_amd import scalar as scal
+    from theano_amd.tensor.elemwise import Elemwise
+    rng = np.random.default_rng(12)
+    for dtype in ("float32", "float64", "float16", "int8", "int32", "uint16"):
+        x = T.TensorType(dtype, (False, False))("x")
+        xv = rand(rng, (37, 129), dtype) if np.dtype(dtype).kind in "iu" else rng.uniform(-720, 720, (37, 129)).astype(dtype)
+        got, ref = run_both([x], [T.deg2rad(x), T.rad2deg(x)], [xv])
+        for g, r in zip(got, ref):
+            assert g.dtype == r.dtype and np.array_equal(g, r), dtype
+    x, lo, hi = T.fmatrix("x"), T.TensorType("int8", (False, False))("lo"), T.TensorType("float64", (True, False))("hi")
+    xv = rng.integers(-4, 5, (50, 70)).astype("float32")
+    lov = rng.integers(-4, 5, (50, 70)).astype("int8")
+    hiv = rng.integers(-4, 5, (1, 70)).astype("float64")
+    outs = [Elemwise(scal.InRange(a, b))(x, lo, hi) for a in (False, True) for b in (False, True)]
+    got, ref = run_both([x, lo, hi], outs, [xv, lov, hiv])
+    for g, r in zip(got, ref):
+        assert g.dtype == np.bool_ and np.array_equal(g, r)
+    assert got[0].sum() > got[3].sum() > 0        # the closed range holds more points than the open one
+    # gradients: a constant factor; none through a range test
+    x = T.fmatrix("x")
+    gx = th.grad(T.sum(T.deg2rad(x) * T.rad2deg(x)), x)
+    xv = rng.standard_normal((9, 11)).astype("float32")
+    got, ref = run_both([x], [gx], [xv])
+    assert_parity(got[0], ref[0], "angle unit gradient")
+    np.testing.assert_allclose(got[0], 2 * xv, rtol=1e-6)
+
+
 def test_sigmoid_thresholds_and_nan_handling():
     x = T.fvector("x")
     xv = np.array([-100, -88.5, -88, -30, 0, 14.9, 15, 15.1, 100, np.nan, np.inf, -np.inf], "float32")

@@ -398,3 +398,74 @@ def test_bessel_functions_of_real_order_known_answers():
     assert np.allclose(S.jv("float64", v - 1, x) + S.jv("float64", v + 1, x), 2 * v / x * S.jv("float64", v, x), rtol=1e-10, atol=1e-13)
     assert np.allclose(S.iv("float64", v - 1, x) - S.iv("float64", v + 1, x), 2 * v / x * S.iv("float64", v, x), rtol=1e-10)
     assert S.jv("float32", v.astype("float32"), x.astype("float32")).dtype == np.float32
+
+
+def test_angle_units_multiply_in_double_and_round_once():
+    """Deg2Rad / Rad2Deg (theano/scalar/basic.py:3110-3149) against Python float arithmetic element by element
+    (a float32 operand times the double constant, rounded to float32 once - not NumPy's float32 deg2rad, which
+    multiplies by the rounded constant), known angles, and the integer operands the reference upgrades."""
+    import math
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-720, 720, 4000).astype("float32")
+    want = np.array([np.float32(float(v) * (math.pi / 180.0)) for v in x])
+    got = S.deg2rad("float32", x)
+    assert got.dtype == np.float32 and np.array_equal(got, want)
+    assert np.any(got != np.deg2rad(x))          # the float32 product differs in the last place somewhere
+    want = np.array([np.float32(float(v) * (180.0 / math.pi)) for v in x])
+    assert np.array_equal(S.rad2deg("float32", x), want)
+    assert S.deg2rad("float64", np.array([180.0, 90.0, -360.0]))[0] == math.pi
+    assert np.array_equal(S.deg2rad("float64", np.array([180.0, 90.0, -360.0])), [math.pi, math.pi / 2, -2 * math.pi])
+    assert np.array_equal(S.rad2deg("float64", np.array([math.pi, -math.pi / 2])), [180.0, -90.0])
+    i8 = np.array([-128, -90, 0, 45, 127], "int8")
+    assert np.array_equal(S.deg2rad("float32", i8), np.array([np.float32(int(v) * (math.pi / 180.0)) for v in i8]))
+    i32 = np.array([-(2 ** 31), 7, 2 ** 31 - 1], "int32")
+    assert np.array_equal(S.rad2deg("float64", i32), np.array([int(v) * (180.0 / math.pi) for v in i32]))
+    # float16: computed as float, stored as half
+    h = np.array([1.0, 33.5, -270.0], "float16")
+    want = np.array([np.float16(np.float32(float(v) * (math.pi / 180.0))) for v in h])
+    assert np.array_equal(S.deg2rad("float16", h), want)
+    # the scalar ops route to these restatements with the reference's result types
+    from theano_amd import scalar as scal
+    from oracle import graph_ref as G
+    for dt, out in (("int8", "float32"), ("int16", "float32"), ("int32", "float64"), ("float16", "float16"),
+                    ("float32", "float32"), ("float64", "float64")):
+        node = scal.deg2rad.make_node(scal.Scalar(dt)())
+        assert node.outputs[0].type.dtype == out
+    (r,) = G.eval_scalar_op(scal.rad2deg, [x], ["float32"])
+    assert np.array_equal(r, S.rad2deg("float32", x))
+
+
+def test_in_range_is_the_two_comparisons_of_the_c_text():
+    """InRange (theano/scalar/basic.py:1434-1481) against Python's comparisons on every triple of a small grid,
+    open and closed ends, integers against floats, and unsigned operands."""
+    from theano_amd import scalar as scal
+    from oracle import graph_ref as G
+    grid = [-2, -1, 0, 1, 2, 3]
+    xs, lows, his = np.meshgrid(grid, grid, grid, indexing="ij")
+    for openlow in (False, True):
+        for openhi in (False, True):
+            op = scal.InRange(openlow, openhi)
+            want = np.array([[(x > l if openlow else x >= l) and (x < h if openhi else x <= h)
+                              for l, h in zip(ls, hs)] for x, ls, hs in
+                             zip(xs.ravel()[:, None], lows.ravel()[:, None], his.ravel()[:, None])]).reshape(xs.shape)
+            for dts in (("int32",) * 3, ("float32", "int8", "float64"), ("int16", "float32", "float32")):
+                args = [a.astype(d) for a, d in zip((xs, lows, his), dts)]
+                (got,) = G.eval_scalar_op(op, args, ["bool"])
+                assert got.dtype == np.bool_ and np.array_equal(got, want), (openlow, openhi, dts)
+    assert scal.inopenrange == scal.InRange(True, True) and scal.inclosedrange == scal.InRange(False, False)
+    assert scal.inopenrange != scal.inclosedrange and hash(scal.inopenrange) == hash(scal.InRange(True, True))
+    node = scal.inclosedrange.make_node(scal.float32(), scal.int8(), scal.float64())
+    assert node.outputs[0].type.dtype == "bool"
+    assert "x >= lo && x <= hi" in scal.inclosedrange.c_code(node, ["x", "lo", "hi"], ["z"])
+    assert "x > lo && x < hi" in scal.inopenrange.c_code(node, ["x", "lo", "hi"], ["z"])
+    # unsigned against signed converts as C does: -1 < 1u is false there
+    u = np.array([1], "uint32")
+    (got,) = G.eval_scalar_op(scal.inopenrange, [u, np.array([-1], "int32"), np.array([5], "uint32")], ["bool"])
+    assert not got[0]
+
+
+def test_cast_ops_carry_the_module_level_names_of_the_reference():
+    from theano_amd import scalar as scal
+    for dt in scal.all_dtypes:
+        op = getattr(scal, "convert_to_" + dt)
+        assert isinstance(op, scal.Cast) and op.o_type.dtype == dt and op.name == "convert_to_" + dt

@@ -498,6 +498,41 @@ class IsInf(FixedLogicalComparison):
 isnan, isinf = IsNan(name="isnan"), IsInf(name="isinf")
 
 
+class InRange(ScalarOp):
+    """``low < x < hi`` with either end open or closed (``theano/scalar/basic.py:1434-1481``)."""
+    nin = 3
+    __props__ = ("openlow", "openhi")
+
+    def __init__(self, openlow, openhi, name=None):
+        ScalarOp.__init__(self, None, name)
+        self.openlow, self.openhi = bool(openlow), bool(openhi)
+
+    def _props(self):
+        return (self.openlow, self.openhi)
+
+    def output_types(self, types):
+        return [bool_]
+
+    def c_code(self, node, inputs, outputs):
+        if any(i.type.dtype in complex_dtypes for i in node.inputs):
+            raise NotImplementedError("complex numbers have no order (theano/scalar/basic.py:1280-1350)")
+        x, low, hi = inputs
+        return "%s = (%s %s %s && %s %s %s);" % (outputs[0], x, ">" if self.openlow else ">=", low,
+                                                 x, "<" if self.openhi else "<=", hi)
+
+    def L_op(self, inputs, outputs, gout):
+        if any(i.type.dtype in complex_dtypes for i in inputs):
+            raise NotImplementedError("no gradient of InRange for complex numbers")
+        return _zero_grads(inputs)
+
+    def make_new_inplace(self, output_types_preference=None, name=None):
+        return type(self)(self.openlow, self.openhi, name)
+
+
+inopenrange = InRange(True, True, name="inopenrange")
+inclosedrange = InRange(False, False, name="inclosedrange")
+
+
 class Switch(ScalarOp):
     nin = 3
 
@@ -947,6 +982,8 @@ class Cast(UnaryScalarOp):
 
 
 _cast_mapping = dict((dt, Cast(Scalar(dt), name="convert_to_" + dt)) for dt in all_dtypes)
+# convert_to_bool ... convert_to_complex128, the module-level names of theano/scalar/basic.py:2403-2417
+globals().update(("convert_to_" + dt, op) for dt, op in _cast_mapping.items())
 
 
 def cast(x, dtype):
@@ -1141,6 +1178,39 @@ class Trunc(UnaryScalarOp):
 
 
 trunc = Trunc(upgrade_to_float, name="trunc")
+
+
+class _AngleUnit(UnaryScalarOp):
+    """``x * factor`` with the factor a double constant, as the reference's C text has it: an
+    integer or float32 operand is multiplied in double precision and rounded to the result type
+    once (``theano/scalar/basic.py:3086-3150``)."""
+    factor = 1.0
+
+    def c_code(self, node, inputs, outputs):
+        if node.inputs[0].type.dtype in complex_dtypes:
+            raise NotImplementedError("%s of a complex number" % self)
+        return "%s = %s * (%r);" % (outputs[0], inputs[0], self.factor)
+
+    def L_op(self, inputs, outputs, gout):
+        (x,) = inputs
+        (gz,) = gout
+        if gz.type.dtype in complex_dtypes:
+            raise NotImplementedError("gradient of %s for complex numbers" % self)
+        if outputs[0].type.dtype in discrete_dtypes:
+            return _zero_grads(inputs)
+        return [gz * self.factor]
+
+
+class Deg2Rad(_AngleUnit):
+    factor = math.pi / 180.0
+
+
+class Rad2Deg(_AngleUnit):
+    factor = 180.0 / math.pi
+
+
+deg2rad = Deg2Rad(upgrade_to_float, name="deg2rad")
+rad2deg = Rad2Deg(upgrade_to_float, name="rad2deg")
 
 
 class RoundHalfToEven(UnaryScalarOp):

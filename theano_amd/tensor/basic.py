@@ -465,18 +465,9 @@ floor_div, power, square, absolute, sign = int_div, pow, sqr, abs_, sgn
 rint = round_half_to_even
 
 
-def deg2rad(a):
-    """``a * (pi / 180)`` (``theano/scalar/basic.py:2845-2862``)."""
-    a = as_tensor_variable(a)
-    dt = a.type.dtype if a.type.dtype in scal.float_dtypes else scal.upgrade_to_float(scal.Scalar(a.type.dtype))[0].dtype
-    return cast(a, dt) * np.asarray(np.pi / 180.0, dt)
-
-
-def rad2deg(a):
-    """``a * (180 / pi)`` (``theano/scalar/basic.py:2874-2891``)."""
-    a = as_tensor_variable(a)
-    dt = a.type.dtype if a.type.dtype in scal.float_dtypes else scal.upgrade_to_float(scal.Scalar(a.type.dtype))[0].dtype
-    return cast(a, dt) * np.asarray(180.0 / np.pi, dt)
+# ``x * (pi / 180)`` and ``x * (180 / pi)`` as the reference's scalar ops compute them: the product in
+# double precision, rounded to the result type once (``theano/tensor/basic.py:2280-2288``)
+deg2rad, rad2deg = _elemwise(scal.deg2rad, "deg2rad"), _elemwise(scal.rad2deg, "rad2deg")
 
 
 def smallest(*args):
