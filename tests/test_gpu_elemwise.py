@@ -636,3 +636,70 @@ def test_float16_composites_and_casts():
     srcs = [d1, d2, d2, d1, d2, d3, d3]
     for r, o, d in zip(res, outs, srcs):
         assert r.dtype == np.dtype(o.type.dtype) and np.array_equal(r, d.astype(o.type.dtype))
+
+
+def test_inplace_operations_overwrite_their_first_argument():
+    """theano/tensor/inplace.py through function(accept_inplace=True): results equal the out-of-place
+    operation's converted to the first operand's type, and the first argument holds the result after
+    the call (theano/tensor/tests/test_basic.py:653-657) - a host array, a device array, a strided
+    device view; an argument that had to be converted is left alone."""
+    from theano_amd.hip.runtime import HipArray
+    from theano_amd.tensor import inplace as I
+    rng = np.random.default_rng(21)
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    cases = [(I.add_inplace, np.add), (I.sub_inplace, np.subtract), (I.mul_inplace, np.multiply),
+             (I.true_div_inplace, np.true_divide), (I.maximum_inplace, np.maximum), (I.minimum_inplace, np.minimum),
+             (I.pow_inplace, lambda a, b: np.abs(a) ** b)]
+    for op, npf in cases:
+        xv = rng.uniform(0.5, 2.0, (33, 65)).astype("float32")
+        yv = rng.uniform(0.5, 2.0, (33, 65)).astype("float32")
+        want = npf(xv, yv).astype("float32")
+        f = th.function([x, y], op(x, y), accept_inplace=True)
+        got = f(xv, yv)
+        np.testing.assert_allclose(got, want, rtol=1e-6)
+        assert np.array_equal(xv, got), op
+    for op, npf in [(I.exp_inplace, np.exp), (I.neg_inplace, np.negative), (I.sqr_inplace, np.square),
+                    (I.abs__inplace, np.abs), (I.floor_inplace, np.floor), (I.tanh_inplace, np.tanh),
+                    (I.deg2rad_inplace, np.deg2rad)]:
+        xv = rng.uniform(-2.0, 2.0, (17, 129)).astype("float32")
+        want = npf(xv)
+        got = th.function([x], op(x), accept_inplace=True)(xv)
+        np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-7)
+        assert np.array_equal(xv, got), op
+    # mixed types: the result is converted to the first operand's type (transfer_type(0))
+    i, d = T.imatrix("i"), T.dmatrix("d")
+    iv = rng.integers(-50, 50, (9, 40)).astype("int32")
+    dv = rng.uniform(-3, 3, (9, 40))
+    want = (iv.astype("float64") * dv).astype("int32")          # C conversion: truncation toward zero
+    got = th.function([i, d], I.mul_inplace(i, d), accept_inplace=True)(iv, dv)
+    assert got.dtype == np.int32 and np.array_equal(got, want) and np.array_equal(iv, want)
+    # a chain over one buffer, and another reader of the old value
+    f = th.function([x, y], [I.mul_inplace(I.exp_inplace(x), y), x * 2], accept_inplace=True)
+    xv = rng.standard_normal((20, 30)).astype("float32")
+    yv = rng.standard_normal((20, 30)).astype("float32")
+    old = xv.copy()
+    r0, r1 = f(xv, yv)
+    np.testing.assert_allclose(r0, np.exp(old) * yv, rtol=2e-6)
+    assert np.array_equal(r1, old * 2) and np.array_equal(xv, r0)
+    # device arguments: overwritten on the device, also through a strided view
+    f = th.function([x, y], I.add_inplace(x, y), accept_inplace=True)
+    xv = rng.standard_normal((40, 50)).astype("float32")
+    yv = rng.standard_normal((40, 50)).astype("float32")
+    xd = HipArray.from_numpy(xv)
+    got = f(xd, yv)
+    assert np.array_equal(got, xv + yv) and np.array_equal(xd.to_numpy(), xv + yv)
+    big = HipArray.from_numpy(np.zeros((50, 80), "float32"))
+    view = big.view((40, 50), (4, 320))        # big.T[0:40, 0:50]
+    from theano_amd.hip.views import copy_into
+    copy_into(HipArray.from_numpy(xv), view)
+    got = f(view, yv)
+    back = big.to_numpy()
+    assert np.array_equal(got, xv + yv) and np.array_equal(back.T[0:40, 0:50], xv + yv)
+    assert not back.T[40:].any() and not back.T[:, 50:].any()
+    # an argument that is converted on the way in was copied: nothing to overwrite
+    lst = [[1.0, 2.0], [3.0, 4.0]]
+    got = f(lst, np.ones((2, 2), "float32"))
+    assert np.array_equal(got, [[2, 3], [4, 5]]) and lst == [[1.0, 2.0], [3.0, 4.0]]
+    ro = np.ones((2, 2), "float32")
+    ro.flags.writeable = False
+    assert np.array_equal(f(ro, ro), np.full((2, 2), 2, "float32")) and np.array_equal(ro, np.ones((2, 2)))

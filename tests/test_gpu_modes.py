@@ -37,15 +37,26 @@ def test_check_mode_passes_correct_functions_and_returns_their_results():
     th.function([h], [T.tanh(h * 3 + 1) * h, T.sum(h * h, axis=1)], mode="check")(xv.astype("float16"))
 
 
-def test_check_mode_reports_an_overwritten_argument():
-    """An elementwise node built with an in-place pattern on a function argument (the rewrite pass never does
-    that; a hand-built node can): harmless for a host argument, which is uploaded into a private buffer, but a
-    device array handed in by the caller comes back changed."""
+def test_check_mode_reports_an_overwritten_argument(monkeypatch):
+    """A deliberately wrong in-place pass (it lets a kernel write over a function argument, which the real
+    pass never does): harmless for a host argument, which is uploaded into a private buffer, but a device
+    array handed in by the caller comes back changed."""
+    from theano_amd.hip import opt as hip_opt
     rng = np.random.default_rng(62)
     x, y = T.fmatrix("x"), T.fmatrix("y")
-    destructive = Elemwise(scal.add, inplace_pattern={0: 0})(x, y)
+    real = hip_opt.inplace_elemwise
+
+    def broken(fgraph, *a, **k):
+        out = real(fgraph, *a, **k)
+        for node in fgraph.toposort():
+            if isinstance(node.op, hip.HipElemwise) and not node.op.inplace_pattern and len(node.outputs) == 1:
+                new = hip.HipElemwise(node.op.scalar_op, {0: 0}).make_node(*node.inputs).outputs[0]
+                fgraph.replace(node.outputs[0], new)
+        return out
+
+    monkeypatch.setattr(hip_opt, "inplace_elemwise", broken)
     xv, yv = rng.standard_normal((33, 50)).astype("float32"), rng.standard_normal((33, 50)).astype("float32")
-    f = th.function([x, y], destructive * 2, mode="check")
+    f = th.function([x, y], (x + y) * 2, mode="check")
     assert np.allclose(f(xv, yv), (xv + yv) * 2)
     with pytest.raises(th.CheckModeError, match="argument 0"):
         f(HipArray.from_numpy(xv), HipArray.from_numpy(yv))

@@ -908,3 +908,57 @@ def test_shape_patterns_of_reshape_and_alloc():
                 lambda: V.Alloc([-1]), lambda: V.Reshape([-1, -1])):
         with pytest.raises((TypeError, ValueError)):
             bad()
+
+
+def test_inplace_module_names_and_types():
+    """theano/tensor/inplace.py: 68 ``*_inplace`` Elemwise instances (the scalar op with transfer_type(0),
+    inplace_pattern {0: 0}) and transpose_inplace."""
+    from theano_amd.tensor import inplace as I
+    assert len(I.__all__) == 69
+    for name in I.__all__:
+        if name == "transpose_inplace":
+            continue
+        op = getattr(I, name)
+        assert isinstance(op, Elemwise) and op.inplace_pattern == ((0, 0),) and op.destroy_map == {0: [0]}
+        assert type(op.scalar_op) is type(getattr(scal, name[:-len("_inplace")]))
+        assert op.scalar_op.output_types_preference == scal.transfer_type(0)
+    x, i = T.fmatrix(), T.imatrix()
+    assert I.add_inplace(x, i).type == x.type           # the result takes the first operand's type
+    assert I.add_inplace(i, x).type == i.type
+    with pytest.raises(TypeError, match="incompatible data types"):
+        I.lt_inplace(x, x)                              # a bool result cannot overwrite a float32 operand
+    b = T.TensorType("bool", (False, False))()
+    assert I.lt_inplace(b, b).type == b.type
+    with pytest.raises(ValueError, match="broadcasted dimensions"):
+        I.add_inplace(T.frow(), x)                      # the result is larger than the operand it would overwrite
+    t = I.transpose_inplace(T.ftensor3())
+    assert isinstance(t.owner.op, DimShuffle) and t.owner.op.new_order == (2, 1, 0)
+    assert I.add_inplace == Elemwise(scal.Add(scal.transfer_type(0)), {0: 0})
+    assert I.add_inplace != T.add
+
+
+def test_graphs_with_inplace_operations_need_accept_inplace(dry_run):
+    """theano/compile/function_module.py:183-190; protected variables and double destruction as the
+    DestroyHandler and Supervisor of the reference report them."""
+    from theano_amd import gof
+    from theano_amd.tensor import inplace as I
+    x, y = T.fmatrix("x"), T.fmatrix("y")
+    with pytest.raises(TypeError, match="Graph must not contain inplace operations"):
+        th.function([x, y], I.add_inplace(x, y))
+    f = th.function([x, y], I.add_inplace(x, y), accept_inplace=True)
+    assert f.writeback == [0] and [type(n.op).__name__ for n in f.nodes].count("HipElemwise") == 1
+    # a chain over one buffer: the argument takes the last value; the other reader of x sees the old one,
+    # in one fused kernel with it
+    f = th.function([x, y], [I.mul_inplace(I.exp_inplace(x), y), x * 2], accept_inplace=True)
+    assert f.writeback == [0] and [type(n.op).__name__ for n in f.nodes].count("HipElemwise") == 1
+    # an intermediate that is overwritten: nothing to store back
+    f = th.function([x, y], I.sub_inplace(x * y, y), accept_inplace=True)
+    assert f.writeback == []
+    with pytest.raises(gof.InconsistencyError, match="Multiple destroyers"):
+        th.function([x], [I.exp_inplace(x), I.neg_inplace(x)], accept_inplace=True)
+    with pytest.raises(gof.InconsistencyError, match="protected"):
+        th.function([x], I.add_inplace(T.constant(np.ones((2, 2), "float32")), x), accept_inplace=True)
+    with pytest.raises(NotImplementedError, match="view of a function argument"):
+        th.function([x], I.exp_inplace(x.T), accept_inplace=True)
+    with pytest.raises(ValueError, match="leaves its arguments alone"):
+        th.function([x, y], I.add_inplace(x, y), accept_inplace=True, mode="check")

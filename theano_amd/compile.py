@@ -150,9 +150,13 @@ class CheckedFunction(object):
 class Function(object):
     """Callable produced by ``function``."""
 
-    def __init__(self, fgraph, in_specs, out_specs, single_output, shared_inputs, update_targets=(), nan_guard=False):
+    def __init__(self, fgraph, in_specs, out_specs, single_output, shared_inputs, update_targets=(), nan_guard=False,
+                 writeback=()):
         self.nan_guard = nan_guard
         self.update_targets = list(update_targets)
+        # positions of the arguments that take the trailing (hidden) results after each call: what the
+        # caller's in-place operations overwrote
+        self.writeback = list(writeback)
         self.fgraph = fgraph
         self.maker = self  # so that f.maker.fgraph reads as with the reference
         self.in_specs = in_specs
@@ -350,6 +354,10 @@ class Function(object):
                 cell[0] = None
         self._static_key = key
         results = [self.storage[o][0] for o in self.fgraph.outputs]
+        if self.writeback:
+            n_keep = len(results) - len(self.writeback)
+            self._write_back(args, results[n_keep:])
+            results = results[:n_keep]
         if self.update_targets:
             n_out = len(results) - len(self.update_targets)
             new_values = results[n_out:]
@@ -369,12 +377,28 @@ class Function(object):
             return results[0]
         return results
 
+    def _write_back(self, args, values):
+        """Store each hidden result into the argument its operation overwrites: a device argument takes a
+        device copy (whatever its strides), a writable host array of the input's dtype takes the values;
+        an argument that had to be converted on the way in was copied then, and stays as it is - as with
+        the reference, whose ``filter`` makes that copy."""
+        from .hip.views import copy_into
+        for k, val in zip(self.writeback, values):
+            a = args[k]
+            if isinstance(a, self._HipArray):
+                if a.shape != val.shape:
+                    raise ValueError("in-place result has shape %s, argument %d has %s" % (val.shape, k, a.shape))
+                if val.size and not val.buffer.fake:
+                    copy_into(val, a)
+            elif type(a) is np.ndarray and a.dtype == val.dtype and a.shape == val.shape and a.flags.writeable:
+                a[...] = val.to_numpy()
+
     def toposort(self):
         return list(self.nodes)
 
 
 def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=True, inplace=True, name=None,
-             on_unused_input="raise", mode=None):
+             on_unused_input="raise", mode=None, accept_inplace=False):
     """Compile ``outputs`` as a function of ``inputs``.
 
     ``inputs``: variables or ``In`` instances.  A host-typed input may be given
@@ -392,7 +416,9 @@ def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=Tru
     every elementwise result a buffer of its own.  ``mode``: None, ``'nan_guard'`` (every node's
     floating-point results are scanned for NaN / infinity, ``NanGuardError``) or ``'check'`` (see
     ``CheckedFunction``: arguments must come back unchanged and results must not depend on fusion or
-    in-place operation)."""
+    in-place operation).  ``accept_inplace``: the graph may hold operations that overwrite an operand
+    (``theano.tensor.inplace``); without it such a graph is refused, as in the reference
+    (``theano/compile/function_module.py:183-190``) - see ``_functional_form`` for how they run."""
     from .hip import opt as hip_opt
     from .hip.ops import HipArrayType, as_hip_variable
 
@@ -461,8 +487,18 @@ def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=Tru
     fgraph = _SharedAwareGraph(c_in, c_out, shared_inputs)
     if mode not in (None, "nan_guard", "check"):
         raise ValueError("mode must be None, 'nan_guard' or 'check'", mode)
+    destroyers = [n for n in fgraph.toposort() if getattr(n.op, "destroy_map", None)]
+    writeback = []
+    if destroyers:
+        if not accept_inplace:
+            raise TypeError("Graph must not contain inplace operations", destroyers[0], destroyers[0].op)
+        fgraph, writeback = _functional_form(fgraph, destroyers, shared_inputs)
+        if writeback and mode == "check":
+            raise ValueError("mode='check' verifies that a call leaves its arguments alone; this graph overwrites "
+                             "argument %d in place" % writeback[0])
     fgraph = hip_opt.optimize(fgraph, fuse=fuse, rowchain=rowchain, inplace=inplace)
-    primary = Function(fgraph, in_specs, out_specs, single, shared_inputs, update_targets, nan_guard=mode == "nan_guard")
+    primary = Function(fgraph, in_specs, out_specs, single, shared_inputs, update_targets, nan_guard=mode == "nan_guard",
+                       writeback=writeback)
     if mode != "check":
         return primary
     # the same outputs and new shared values, as plain results of a function without the rewrites
@@ -471,6 +507,55 @@ def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=Tru
     reference = function(in_specs, ref_outs, givens=None, fuse=False, rowchain=False, inplace=False,
                          on_unused_input="ignore")
     return CheckedFunction(primary, reference, len(update_targets))
+
+
+def _functional_form(fgraph, destroyers, shared_inputs):
+    """Graphs with the user's in-place elementwise operations (``theano.tensor.inplace``), made safe to
+    reorder and fuse: every such node is replaced by the same scalar operation writing a buffer of its
+    own, so that whatever else reads the overwritten variable reads its old value - the order the
+    reference's DestroyHandler forces (``theano/gof/destroyhandler.py``).  Where the overwritten variable
+    is an argument of the function the new result becomes one more (hidden, device) output that
+    ``Function`` stores into the argument after the call; an intermediate result that is overwritten
+    cannot be observed and needs nothing.  As in the reference, constants and shared variables are
+    protected and one variable takes one destroyer.  Returns the rebuilt graph and, per hidden output in
+    order, the position of the argument that receives it."""
+    from .hip.ops import as_hip_variable
+    from .tensor.elemwise import Elemwise
+
+    def root(v):
+        seen_view = False
+        while v.owner is not None and getattr(v.owner.op, "view_map", None):
+            v = v.owner.inputs[v.owner.op.view_map[0][0]]
+            seen_view = True
+        return v, seen_view
+
+    shared = set(id(v) for v in shared_inputs)
+    taken = set()
+    origin = {}       # id(result written over an argument's buffer) -> position of that argument
+    final = {}        # position of an argument -> the last result written over it (chains of in-place nodes)
+    for node in destroyers:
+        if not isinstance(node.op, Elemwise):
+            raise NotImplementedError("in-place operation %s" % node.op)
+        new = Elemwise(node.op.scalar_op, name=node.op.name).make_node(*node.inputs)
+        for o, idxs in node.op.destroy_map.items():
+            victim, through_view = root(node.inputs[idxs[0]])
+            if isinstance(victim, Constant) or id(victim) in shared:
+                raise gof.InconsistencyError("Trying to destroy a protected Variable.", victim)
+            if id(victim) in taken:
+                raise gof.InconsistencyError("Multiple destroyers of %s" % victim)
+            taken.add(id(victim))
+            pos = fgraph.inputs.index(victim) if victim in fgraph.inputs else origin.get(id(victim))
+            if pos is not None:
+                if through_view:
+                    raise NotImplementedError("in-place operation on a view of a function argument (%s)" % node.op)
+                origin[id(new.outputs[o])] = pos
+                final[pos] = new.outputs[o]
+        for o, no in zip(node.outputs, new.outputs):
+            fgraph.replace(o, no)
+    writeback = sorted(final)
+    if writeback:
+        fgraph = fgraph.rebuild(list(fgraph.outputs) + [as_hip_variable(final[pos]) for pos in writeback])
+    return fgraph, writeback
 
 
 class _SharedAwareGraph(FunctionGraph):
