@@ -552,3 +552,32 @@ def test_transposed_reduction_result_is_not_fused_as_an_epilogue():
         assert_parity(g, w, "transposed consumer of a reduction")
     f = th.function([x, y], outs[1:])
     assert not any(type(n.op).__name__ == "HipElemwise" for n in f.toposort())      # this one is an epilogue
+
+
+def test_negated_max_of_a_negation_runs_as_min_with_the_same_values():
+    """-max(-x) (the reference's spelling of tensor.min, rewritten to one min reduction for floats) against the
+    oracle's evaluation of the written graph: NaN rows, signed zeros, infinities; integers keep the written form
+    and agree at the most negative value, where the two forms differ."""
+    rng = np.random.default_rng(5)
+    for dtype in ("float32", "float64", "float16"):
+        x = T.TensorType(dtype, (False, False))("x")
+        v = rng.standard_normal((37, 300)).astype(dtype)
+        v[3, 5] = np.nan
+        v[4, :] = np.inf
+        v[5, 7] = -np.inf
+        v[6, :] = 0.0
+        v[6, 11] = -0.0
+        for axis in (0, 1, None):
+            out = -T.max(-x, axis=axis)
+            got = th.function([x], out)(v)
+            ref = G.evaluate([x], [out], [v])[0]
+            assert got.dtype == ref.dtype and np.array_equal(got, ref, equal_nan=True), (dtype, axis)
+            assert np.array_equal(got, np.min(v, axis=axis), equal_nan=True)
+    i = T.imatrix("i")
+    iv = rng.integers(-100, 100, (20, 50)).astype("int32")
+    iv[2, 3] = -2 ** 31
+    out = -T.max(-i, axis=1)
+    got = th.function([i], out)(iv)
+    assert np.array_equal(got, G.evaluate([i], [out], [iv])[0])
+    # -(-2**31) wraps to -2**31, the smallest value: the written form skips that element, a min would return it
+    assert got[2] == np.delete(iv[2], 3).min() and np.array_equal(np.delete(got, 2), np.delete(iv.min(axis=1), 2))

@@ -962,3 +962,21 @@ def test_graphs_with_inplace_operations_need_accept_inplace(dry_run):
         th.function([x], I.exp_inplace(x.T), accept_inplace=True)
     with pytest.raises(ValueError, match="leaves its arguments alone"):
         th.function([x, y], I.add_inplace(x, y), accept_inplace=True, mode="check")
+
+
+def test_negated_max_of_a_negation_is_a_min(dry_run):
+    """local_max_to_min (theano/tensor/opt_uncanonicalize.py:71-94): -max(-x) compiles to one min reduction
+    for floating-point operands; integers keep the written form (the two differ at the most negative value
+    and over unsigned types)."""
+    x = T.fmatrix("x")
+    f = th.function([x], -T.max(-x, axis=1))
+    red = [n.op for n in f.toposort() if isinstance(n.op, HipCAReduce)]
+    assert len(red) == 1 and isinstance(red[0].scalar_ops[0], scal.Minimum)
+    assert red[0].pre_scalar_op is None and red[0].post_scalar_op is None
+    assert not any(isinstance(n.op, HipElemwise) for n in f.toposort())
+    i = T.imatrix("i")
+    f = th.function([i], -T.max(-i, axis=1), rowchain=False)
+    red = [n.op for n in f.toposort() if isinstance(n.op, HipCAReduce)]
+    assert len(red) == 1 and isinstance(red[0].scalar_ops[0], scal.Maximum)
+    from theano_amd.tensor import elemwise as E
+    assert E.MulWithoutZeros is scal.MulWithoutZeros and E.mul_without_zeros is scal.mul_without_zeros

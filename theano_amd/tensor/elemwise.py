@@ -530,6 +530,10 @@ class Prod(CAReduceDtype):
         return [T.switch(no_zero, without_zeros, T.mul(T.switch(where_single_zero, others, 0.0), gz))]
 
 
+# the scalar op behind ProdWithoutZeros lives here in the reference (theano/tensor/elemwise.py:2054-2083)
+MulWithoutZeros, mul_without_zeros = scal.MulWithoutZeros, scal.mul_without_zeros
+
+
 class ProdWithoutZeros(CAReduceDtype):
     """Product of the non-zero elements along axes; 0 for a group of zeros
     (``theano/tensor/elemwise.py:2086-2101``)."""

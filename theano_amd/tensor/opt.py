@@ -367,6 +367,27 @@ def local_max_and_argmax(fgraph, node):
     return [new, None]
 
 
+@local_optimizer([Elemwise])
+def local_max_to_min(fgraph, node):
+    """``-max(-x) -> min(x)`` (``local_max_to_min``, ``theano/tensor/opt_uncanonicalize.py:71-94``), the form
+    the reference's ``tensor.min`` writes.  Kept to floating-point operands, where negation is exact: over
+    unsigned integers and at the most negative signed value the two sides differ."""
+    if not isinstance(node.op.scalar_op, scal.Neg) or len(node.inputs) != 1:
+        return False
+    red = node.inputs[0].owner
+    if red is None or not isinstance(red.op, CAReduce) or not isinstance(red.op.scalar_op, scal.Maximum):
+        return False
+    inner = red.inputs[0].owner
+    if (inner is None or not isinstance(inner.op, Elemwise) or not isinstance(inner.op.scalar_op, scal.Neg) or
+            len(inner.inputs) != 1):
+        return False
+    x = inner.inputs[0]
+    if x.type.dtype not in scal.float_dtypes:
+        return False
+    new = T.Min(red.op.axis)(x)
+    return [new] if new.type == node.outputs[0].type else False
+
+
 @local_optimizer([T.ShapeFloat])
 def local_shape_lift(fgraph, node):
     """The extent of an elementwise / DimShuffle / reduction result is the extent
@@ -600,7 +621,8 @@ def local_mul_to_sqr(fgraph, node):
 CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_useless_composite, local_constant_fold,
                 local_useless_elemwise, local_fill_sink,
                 local_useless_reduce, local_op_of_op,
-                local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_single_pass_variance,
+                local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_max_to_min,
+                local_single_pass_variance,
                 local_cancel_common_factors, local_split_huge_add_or_mul, local_mul_to_sqr]
 
 
