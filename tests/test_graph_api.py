@@ -980,3 +980,29 @@ def test_negated_max_of_a_negation_is_a_min(dry_run):
     assert len(red) == 1 and isinstance(red[0].scalar_ops[0], scal.Maximum)
     from theano_amd.tensor import elemwise as E
     assert E.MulWithoutZeros is scal.MulWithoutZeros and E.mul_without_zeros is scal.mul_without_zeros
+
+
+def test_tensor_type_value_helpers():
+    """values_eq, may_share_memory, value_zeros, value_validity_msg, to_scalar_type, get_shape_info / get_size,
+    convert_variable and filter_variable (theano/tensor/type.py:202-310, 552-610)."""
+    t = T.TensorType("float32", (False, True))
+    nan = np.array([[np.nan], [1.0]], "float32")
+    assert t.values_eq(nan, nan.copy()) and not t.values_eq(nan, nan.astype("float64"))
+    assert t.values_eq(nan, nan.astype("float64"), force_same_dtype=False) and not t.values_eq(nan, nan[:1])
+    a = np.zeros(4)
+    assert t.may_share_memory(a, a[1:]) and not t.may_share_memory(a, a.copy()) and not t.may_share_memory(a, 3)
+    z = t.value_zeros((5, 1))
+    assert z.dtype == np.float32 and z.shape == (5, 1) and not z.any()
+    assert t.value_validity_msg(z) == "value is valid" and "broadcastable" in t.value_validity_msg(np.zeros((2, 2), "float32"))
+    assert t.to_scalar_type() == scal.float32 and t.get_size(t.get_shape_info(z)) == 20
+    both = T.TensorType("float32", (True, True))()
+    assert t.filter_variable(both).type == t and T.fmatrix().type.filter_variable(both).type == T.fmatrix().type
+    assert t.convert_variable(T.fmatrix()) is None and t.convert_variable(T.dmatrix()) is None
+    v = t()
+    assert t.filter_variable(v) is v
+    with pytest.raises(TypeError, match="Cannot convert Type"):
+        t.filter_variable(T.fmatrix())                   # a broadcastable dimension cannot be promised
+    with pytest.raises(TypeError):
+        t.filter_variable(both, allow_convert=False)
+    c = t.filter_variable(np.ones((3, 1), "float32"))
+    assert c.type == t and c.data.shape == (3, 1)

@@ -83,8 +83,9 @@ def test_comparisons_refuse_truth_tests_and_python_protocols():
     assert q.owner.inputs[1] is b or q.owner.inputs[1].owner is not None
     for fn, name in ((math.ceil, "ceil"), (math.floor, "floor"), (math.trunc, "trunc")):
         assert str(fn(a).owner.op.scalar_op) == name
-    for name in ("arccos", "arccosh", "arcsin", "arcsinh", "arctan", "arctanh", "ceil", "cos", "cosh", "exp", "floor",
-                 "log", "sin", "sinh", "sqrt", "tan", "tanh", "trunc"):
+    for name in ("arccos", "arccosh", "arcsin", "arcsinh", "arctan", "arctanh", "ceil", "cos", "cosh", "deg2rad", "exp",
+                 "exp2", "expm1", "floor", "log", "log10", "log1p", "log2", "rad2deg", "sin", "sinh", "sqrt", "tan",
+                 "tanh", "trunc"):
         assert getattr(a, name)().owner.op is getattr(T, name)(a).owner.op or \
             getattr(a, name)().owner.op == getattr(T, name)(a).owner.op, name
     m = T.TensorType("float32", (False, True, False))("m")
@@ -96,6 +97,8 @@ def test_comparisons_refuse_truth_tests_and_python_protocols():
         m.norm(0)
     assert m.copy(name="again").name == "again" and m.ravel().type.ndim == 1
     assert m.clip(0, 1).type == m.type and m.round().type == m.type and m.ptp(0).type.ndim == 2
+    # size: the product of the extents, a 0-d int64 (var.py:289-290)
+    assert m.size.type.dtype == "int64" and m.size.type.ndim == 0 and T.scalar().size.data == 1
 
 
 @pytest.mark.gpu

@@ -86,6 +86,65 @@ class TensorType(Type):
         return bool(np.allclose(a, b, rtol=rtol or 1e-5, atol=atol or tol, equal_nan=True))
 
 
+    # -- the value-level helpers of theano/tensor/type.py:202-310, 552-610
+    @staticmethod
+    def values_eq(a, b, force_same_dtype=True):
+        """Exact equality of two values, NaNs and infinities in the same places counting as equal."""
+        a, b = np.asarray(a), np.asarray(b)
+        if a.shape != b.shape or (force_same_dtype and a.dtype != b.dtype):
+            return False
+        return bool(np.array_equal(a, b, equal_nan=a.dtype.kind in "fc" and b.dtype.kind in "fc"))
+
+    @staticmethod
+    def may_share_memory(a, b):
+        return bool(isinstance(a, np.ndarray) and isinstance(b, np.ndarray) and np.may_share_memory(a, b))
+
+    def value_zeros(self, shape):
+        return np.zeros(shape, dtype=self.dtype)
+
+    def value_validity_msg(self, a):
+        try:
+            self.filter(a, strict=True)
+        except Exception as e:
+            return str(e)
+        return "value is valid"
+
+    def to_scalar_type(self):
+        return scal.Scalar(self.dtype)
+
+    def get_shape_info(self, obj):
+        return obj.shape
+
+    def get_size(self, shape_info):
+        n = self.numpy_dtype.itemsize
+        for s in shape_info:
+            n *= int(s)
+        return n
+
+    def convert_variable(self, var):
+        """``var`` under this type's broadcast pattern when it has the same dtype and rank and is at least as
+        broadcastable wherever this type is; None otherwise."""
+        vt = var.type
+        if (type(self) is type(vt) and self.dtype == vt.dtype and self.ndim == vt.ndim and
+                all(sb == ob or ob for sb, ob in zip(self.broadcastable, vt.broadcastable))):
+            from .views import patternbroadcast
+            return patternbroadcast(var, self.broadcastable)
+        return None
+
+    def filter_variable(self, other, allow_convert=True):
+        """A symbolic variable (or a value, made a constant) as a variable of this type, or TypeError."""
+        if not isinstance(other, Variable):
+            other = constant(self.filter(other))
+        if other.type == self:
+            return other
+        if allow_convert:
+            conv = self.convert_variable(other)
+            if conv is not None and conv.type == self:
+                return conv
+        raise TypeError("Cannot convert Type %s (of Variable %s) into Type %s. You can try to manually convert %s "
+                        "into a %s." % (other.type, other, self, other, self))
+
+
 class _tensor_py_operators(object):
     """Arithmetic, comparison and reduction sugar on tensor variables."""
 
@@ -169,6 +228,15 @@ class _tensor_py_operators(object):
         They take part in arithmetic as host scalars, and ``reshape`` / ``alloc`` accept them
         as "the extent of dimension d of that tensor"."""
         return tuple(self._b().shape_i(self, d) for d in range(self.ndim))
+
+    @property
+    def size(self):
+        """The number of elements, the product of the extents (``theano/tensor/var.py:289-290``): a 0-d
+        int64 host value like the extents themselves."""
+        n = None
+        for d in self.shape:
+            n = d if n is None else n * d
+        return n if n is not None else self._b().constant(np.int64(1))
 
     def reshape(self, *shape):
         from . import views
@@ -293,9 +361,16 @@ class _tensor_py_operators(object):
     def ceil(self): return self._b().ceil(self)
     def cos(self): return self._b().cos(self)
     def cosh(self): return self._b().cosh(self)
+    def deg2rad(self): return self._b().deg2rad(self)
     def exp(self): return self._b().exp(self)
+    def exp2(self): return self._b().exp2(self)
+    def expm1(self): return self._b().expm1(self)
     def floor(self): return self._b().floor(self)
     def log(self): return self._b().log(self)
+    def log10(self): return self._b().log10(self)
+    def log1p(self): return self._b().log1p(self)
+    def log2(self): return self._b().log2(self)
+    def rad2deg(self): return self._b().rad2deg(self)
     def sin(self): return self._b().sin(self)
     def sinh(self): return self._b().sinh(self)
     def sqrt(self): return self._b().sqrt(self)
