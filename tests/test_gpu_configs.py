@@ -336,3 +336,13 @@ def test_rows_too_long_for_one_block_and_strided_rows_take_the_fused_multi_kerne
     zv = (2 * rng.standard_normal((700, 90))).astype("float32")
     e = np.exp(zv.T.astype("float64") - zv.T.max(axis=1, keepdims=True))
     assert np.allclose(h(zv), e / e.sum(axis=1, keepdims=True), rtol=2e-5, atol=1e-7)
+
+
+def test_elemwise_time_test_script_runs():
+    """The timing script for the reference's own on-path benchmark (theano/misc/elemwise_time_test.py:
+    2*x + x*x and tanh(x) over 200 000 floats) runs and reports sane call times."""
+    from theano_amd.misc.elemwise_time_test import elemwise_op_time
+    host, device = elemwise_op_time(N=200000, loops=30)
+    for t in host + device:
+        assert 1e-6 < t < 5e-2
+    assert device[0] < host[0] and device[1] < host[1]      # no upload / download on the device-resident call
