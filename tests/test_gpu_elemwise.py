@@ -703,3 +703,45 @@ def test_inplace_operations_overwrite_their_first_argument():
     ro = np.ones((2, 2), "float32")
     ro.flags.writeable = False
     assert np.array_equal(f(ro, ro), np.full((2, 2), 2, "float32")) and np.array_equal(ro, np.ones((2, 2)))
+
+
+def test_verify_grad_and_gradient_only_operations():
+    """verify_grad (theano/gradient.py:1625-1800) accepts right gradients and names a wrong one; grad_clip's
+    documented example (:2208-2215): d/dx grad_clip(x, -1, 1)**2 at 2.0 is 1.0 where d/dx x**2 is 4.0."""
+    from theano_amd import gradient as G, scalar as scal
+    from theano_amd.tensor.elemwise import Elemwise
+    rng = np.random.RandomState(7)
+    pts = [rng.uniform(0.5, 1.5, (3, 4)), rng.uniform(0.5, 1.5, (1, 4))]
+    G.verify_grad(lambda a, b: T.tanh(a * b) + T.log(a) / b, pts, rng=rng)
+    G.verify_grad(lambda a: T.sum(T.exp(a), axis=0), [pts[0].astype("float32")], rng=rng)
+    G.verify_grad(lambda a: T.max(a, axis=1), [pts[0]], rng=rng)
+    G.verify_grad(lambda a: T.prod(a, axis=1) * T.sum(T.sqr(a)), [pts[0]], rng=rng)
+    e = T.exp
+    G.verify_grad(lambda a: e(a - T.max(a, axis=1, keepdims=True)) / T.sum(e(a - T.max(a, axis=1, keepdims=True)), axis=1,
+                                                                           keepdims=True), [pts[0]], rng=rng)
+    with pytest.raises(TypeError, match="rng"):
+        G.verify_grad(T.exp, [pts[0]])
+    with pytest.raises(TypeError, match="floating point"):
+        G.verify_grad(T.exp, [np.arange(4)], rng=rng)
+
+    class WrongSqr(scal.Sqr):                       # the gradient of x**2 claimed to be x
+        def L_op(self, inputs, outputs, gout):
+            return [gout[0] * inputs[0]]
+    wrong = Elemwise(WrongSqr(scal.same_out, name="wrong_sqr"))
+    with pytest.raises(G.GradientError) as info:
+        G.verify_grad(wrong, [pts[0]], rng=rng)
+    assert info.value.abs_err > info.value.abs_tol and "exceed tolerance" in str(info.value)
+    # gradient-only operations on the device
+    x = T.fscalar("x")
+    z, z2 = th.grad(G.grad_clip(x, -1, 1) ** 2, x), th.grad(x ** 2, x)
+    got = th.function([x], [z, z2])(np.float32(2.0))
+    assert got[0] == 1.0 and got[1] == 4.0
+    v = T.fvector("v")
+    vv = np.array([-2.0, 0.25, 3.0], "float32")
+    f = th.function([v], [th.grad(T.sum(G.zero_grad(T.exp(v)) * v), v), th.grad(T.sum(G.grad_scale(T.sqr(v), 0.5)), v),
+                          th.grad(T.sum(G.grad_clip(T.sqr(v), -1, 1) * 3 * v), v), G.grad_clip(v, 0, 0) + G.zero_grad(v)])
+    g0, g1, g2, fwd = f(vv)
+    np.testing.assert_allclose(g0, np.exp(vv), rtol=1e-6)
+    np.testing.assert_allclose(g1, vv, rtol=1e-6)                       # 0.5 * 2v
+    np.testing.assert_allclose(g2, 3 * vv ** 2 + np.clip(3 * vv, -1, 1) * 2 * vv, rtol=1e-6)
+    assert np.array_equal(fwd, 2 * vv)

@@ -1006,3 +1006,29 @@ def test_tensor_type_value_helpers():
         t.filter_variable(both, allow_convert=False)
     c = t.filter_variable(np.ones((3, 1), "float32"))
     assert c.type == t and c.data.shape == (3, 1)
+
+
+def test_gradient_only_operations(dry_run):
+    """zero_grad / disconnected_grad / undefined_grad / grad_clip / grad_scale (theano/gradient.py:2022-2300):
+    identity in the forward pass - compiled graphs do not contain them - and the documented effect on gradients."""
+    from theano_amd import gradient as G
+    x = T.fvector("x")
+    f = th.function([x], [G.grad_clip(x * x, -1, 1).sum(), G.zero_grad(x) + G.disconnected_grad(x) + G.grad_scale(x, 2)])
+    assert not any(isinstance(n.op, G._GradView) for n in f.toposort())
+    g = th.grad(T.sum(G.zero_grad(T.exp(x)) * x), x)          # exp(x) counts as a constant: d/dx = exp(x)
+    ops = [str(n.op) for n in th.function([x], g).toposort()]
+    assert len(ops) == 3 and "exp" in ops[1] and "0.0" in ops[1], ops      # exp(x) + 0 * exp(x): zeros flow back
+    g = th.grad(T.sum(G.disconnected_grad(T.exp(x)) * x), x)
+    assert [str(n.op) for n in th.function([x], g).toposort()] == ["HostToHip", "HipElemwise{exp}", "HipToHost"]
+    with pytest.raises(G.DisconnectedInputError):
+        th.grad(T.sum(G.disconnected_grad(x)), x, disconnected_inputs="raise")
+    assert th.grad(T.sum(G.zero_grad(x)), x, disconnected_inputs="raise") is not None    # connected, with zeros
+    with pytest.raises(G.NullTypeGradError, match="mathematically undefined"):
+        th.grad(T.sum(G.undefined_grad(x) * 2), x)
+    with pytest.warns(UserWarning, match="deprecated"):
+        G.consider_constant(x)
+    with pytest.raises(ValueError):
+        G.GradClip(1, -1)
+    assert G.GradClip(0, 1) == G.GradClip(-5, 5) and G.zero_grad_ == G.ZeroGrad() and G.zero_grad_ != G.disconnected_grad_
+    g = th.grad(T.sum(G.grad_scale(T.exp(x), 0.5)), x)
+    assert "0.5" in " ".join(str(n.op) for n in th.function([x], g).toposort())

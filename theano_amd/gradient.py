@@ -250,3 +250,278 @@ def numeric_grad(f, pts, eps=None):
             gflat[j] = (fp - fm) / (2 * h)
         out.append(g)
     return out
+
+
+# ---- verify_grad (theano/gradient.py:1420-1830) ---------------------------------------------------
+TYPE_EPS = {"float64": 1e-7, "float32": 3e-4, "float16": 1e-1}       # finite-difference steps, per dtype
+
+
+class GradientError(Exception):
+    """A gradient was computed, but it is not the finite-difference one."""
+
+    def __init__(self, arg, err_pos, shape, val1, val2, abs_err, rel_err, abs_tol, rel_tol):
+        Exception.__init__(self)
+        self.arg, self.err_pos, self.shape, self.val1, self.val2 = arg, err_pos, shape, val1, val2
+        self.abs_err, self.rel_err, self.abs_tol, self.rel_tol = abs_err, rel_err, abs_tol, rel_tol
+
+    def __str__(self):
+        return ("GradientError: numeric gradient and analytic gradient exceed tolerance:\n"
+                "        At position %i of argument %i with shape %s,\n"
+                "            val1 = %f      ,  val2 = %f\n"
+                "            abs. error = %f,  abs. tolerance = %f\n"
+                "            rel. error = %f,  rel. tolerance = %f\n%s" % (
+                    self.err_pos, self.arg, self.shape, self.val1, self.val2, self.abs_err, self.abs_tol,
+                    self.rel_err, self.rel_tol, ", ".join(str(a) for a in self.args)))
+
+
+def _one_sided_grad(f, pts, eps):
+    """Forward differences of the scalar function ``f`` with one step size for every element, computed in
+    the widest dtype among ``pts`` (``numeric_grad.__init__``, ``theano/gradient.py:1437-1530``)."""
+    wide = max((p.dtype for p in pts), key=lambda d: d.itemsize)
+    pts = [np.array(p, dtype=wide) for p in pts]
+    f0 = float(f(*pts))
+    out = []
+    for p in pts:
+        g = np.zeros(p.shape, wide)
+        flat, gflat = p.reshape(-1), g.reshape(-1)
+        for j in range(flat.size):
+            old = flat[j]
+            flat[j] = old + eps
+            gflat[j] = (float(f(*pts)) - f0) / eps
+            flat[j] = old
+        out.append(g)
+    return out
+
+
+def _abs_rel_err(a, b):
+    """|a - b| and |a - b| / max(|a| + |b|, 1e-8) (``numeric_grad.abs_rel_err``, :1532-1557)."""
+    a, b = np.asarray(a, "float64"), np.asarray(b, "float64")
+    abs_err = abs(a - b)
+    return abs_err, abs_err / np.maximum(abs(a) + abs(b), 1e-8)
+
+
+def _max_err(analytic, numeric, abs_tol, rel_tol):
+    """The element where min(abs_err / abs_tol, rel_err / rel_tol) is largest over all arguments: (argument,
+    flat position, abs_err, rel_err) there (``numeric_grad.max_err``, :1579-1611)."""
+    best = None
+    for k, (a, b) in enumerate(zip(analytic, numeric)):
+        if np.shape(a) != np.shape(b):
+            raise ValueError("argument element %i has wrong shape %s" % (k, (np.shape(a), np.shape(b))))
+        abs_err, rel_err = _abs_rel_err(a, b)
+        if not np.all(np.isfinite(abs_err)):
+            raise ValueError("abs_err not finite", repr(abs_err))
+        if not np.all(np.isfinite(rel_err)):
+            raise ValueError("rel_err not finite", repr(rel_err))
+        if abs_err.size == 0:
+            continue
+        scaled = np.minimum(abs_err / abs_tol, rel_err / rel_tol).reshape(-1)
+        j = int(scaled.argmax())
+        if best is None or scaled[j] > best[0]:
+            best = (scaled[j], k, j, abs_err.reshape(-1)[j], rel_err.reshape(-1)[j])
+    if best is None:
+        return 0, 0, 0.0, 0.0
+    return best[1:]
+
+
+def verify_grad(fun, pt, n_tests=2, rng=None, eps=None, out_type=None, abs_tol=None, rel_tol=None, mode=None,
+                cast_to_output_type=False, no_debug_ref=True):
+    """Check the symbolic gradient of ``fun`` (a function of symbolic tensors returning one tensor, or an
+    op) at the list of floating-point arrays ``pt`` against forward differences, as the reference's
+    ``verify_grad`` does (``theano/gradient.py:1625-1800``): the result is projected on a random direction
+    with entries in [0.5, 1.5) to make a scalar cost, ``n_tests`` times; an element whose absolute *and*
+    relative error both exceed the tolerances (defaults 5e-2 / 1e-2 / 1e-4 for float16 / 32 / 64, the
+    loosest among ``pt``) raises ``GradientError``.  The functions run on the device."""
+    from . import compile as C
+    from .tensor import basic as T
+    from .tensor.type import TensorType
+    if not isinstance(pt, (list, tuple)):
+        raise TypeError("pt must be a list of arrays")
+    pt = [np.array(p) for p in pt]
+    for i, p in enumerate(pt):
+        if str(p.dtype) not in TYPE_EPS:
+            raise TypeError('verify_grad can work only with floating point inputs, but input %i has dtype "%s".'
+                            % (i, p.dtype))
+    type_tol = dict(float16=5e-2, float32=1e-2, float64=1e-4)
+    if abs_tol is None:
+        abs_tol = max(type_tol[str(p.dtype)] for p in pt)
+    if rel_tol is None:
+        rel_tol = max(type_tol[str(p.dtype)] for p in pt)
+    if rng is None:
+        raise TypeError("rng should be a valid instance of numpy.random.RandomState.")
+    if eps is None:
+        eps = max(TYPE_EPS[str(p.dtype)] for p in pt)
+    tensor_pt = [TensorType(str(p.dtype), tuple(s == 1 for s in p.shape))(name="input %i" % i) for i, p in enumerate(pt)]
+    o_output = fun(*tensor_pt)
+    if isinstance(o_output, (list, tuple)):
+        raise NotImplementedError("cant (yet) autotest gradient of fun with multiple outputs")
+    specs = [C.In(v, allow_downcast=True) for v in tensor_pt]
+
+    def function(outputs):
+        return C.function(specs, outputs, on_unused_input="ignore", accept_inplace=True, mode=mode)
+
+    o_fn_out = function(o_output)(*[p.copy() for p in pt])
+    if isinstance(o_fn_out, (tuple, list)):
+        raise TypeError("It seems like you are trying to use verify_grad on an op or a function which outputs a "
+                        "list: there should be a single (array-like) output instead")
+
+    def random_projection():
+        plain = (rng.random_sample(o_fn_out.shape) if hasattr(rng, "random_sample") else rng.random(o_fn_out.shape)) + 0.5
+        dt = o_output.type.dtype if (cast_to_output_type and o_output.type.dtype == "float32") else out_type or "float64"
+        return np.asarray(plain, dtype=dt)
+
+    t_r = C.shared(random_projection(), name="random_projection",
+                   broadcastable=tuple(o_output.type.broadcastable))
+    cost = T.sum(t_r * o_output)
+    cost_fn = function(cost)
+    grad_fn = function(grad(cost, tensor_pt, disconnected_inputs="ignore"))
+    for test_num in range(n_tests):
+        try:
+            num_grad = _one_sided_grad(cost_fn, [p.copy() for p in pt], eps)
+            analytic = grad_fn(*[p.copy() for p in pt])
+            max_arg, max_pos, max_abs, max_rel = _max_err(analytic, num_grad, abs_tol, rel_tol)
+            if max_abs > abs_tol and max_rel > rel_tol:
+                raise GradientError(max_arg, max_pos, np.shape(analytic[max_arg]),
+                                    np.asarray(analytic[max_arg]).reshape(-1)[max_pos],
+                                    num_grad[max_arg].reshape(-1)[max_pos], max_abs, max_rel, abs_tol, rel_tol)
+            if test_num < n_tests - 1:
+                t_r.set_value(random_projection())
+        except Exception as e:
+            e.args += ("\nThe error happened with the following inputs:", pt, "\nThe value of eps is:", eps,
+                       "\nThe out_type is:", out_type)
+            raise
+
+
+verify_grad.E_grad = GradientError
+
+
+# ---- identity operations that change the gradient only (theano/gradient.py:2022-2300) -----------------
+class _GradView(gof.Op):
+    """The value of the operand, unchanged; the subclasses say what flows back through it.  Compiled
+    functions never run these nodes: ``local_remove_grad_views`` takes them out before the graph is
+    lifted (the reference does the same, ``theano/tensor/opt.py:local_grad_clip`` and
+    ``theano/compile/ops.py`` ``local_useless_*`` for ViewOp), so they cost nothing in the forward pass."""
+    view_map = {0: [0]}
+    __props__ = ()
+
+    def make_node(self, x):
+        from .tensor.type import as_tensor_variable
+        if not isinstance(x, gof.Variable):
+            x = as_tensor_variable(x)
+        return gof.Apply(self, [x], [x.type()])
+
+    def perform(self, node, inputs, output_storage):
+        output_storage[0][0] = inputs[0]
+
+    def infer_shape(self, node, shapes):
+        return shapes
+
+    def __eq__(self, other):
+        return type(self) is type(other)
+
+    def __hash__(self):
+        return hash(type(self))
+
+    def __str__(self):
+        return type(self).__name__
+
+
+class ZeroGrad(_GradView):
+    """Gradients flow back through as zeros (:2057-2092)."""
+
+    def L_op(self, inputs, outputs, gout):
+        return [g.zeros_like() for g in gout]
+
+    def R_op(self, inputs, eval_points):
+        if eval_points[0] is None:
+            return [None]
+        return [eval_points[0].zeros_like()]
+
+
+class ConsiderConstant(ZeroGrad):
+    """The deprecated spelling of ZeroGrad (:2022-2054)."""
+
+
+class DisconnectedGrad(_GradView):
+    """Nothing flows back: the operand is disconnected from the cost through this path (:2133-2173)."""
+
+    def L_op(self, inputs, outputs, gout):
+        return [DisconnectedType()() for _ in gout]
+
+    def R_op(self, inputs, eval_points):
+        return [None]
+
+    def connection_pattern(self, node):
+        return [[False]]
+
+
+class UndefinedGrad(_GradView):
+    """Asking for a gradient through this raises (:2095-2130)."""
+
+    def L_op(self, inputs, outputs, gout):
+        return [grad_undefined(self, i, x) for i, x in enumerate(inputs)]
+
+    def R_op(self, inputs, eval_points):
+        return [None]
+
+    def connection_pattern(self, node):
+        return [[True]]
+
+
+class GradClip(_GradView):
+    """The gradient is clipped to [clip_lower_bound, clip_upper_bound] on the way back (:2176-2232).  The
+    bounds take no part in equality, as in the reference: they do not change what the node computes."""
+
+    def __init__(self, clip_lower_bound, clip_upper_bound):
+        self.clip_lower_bound, self.clip_upper_bound = clip_lower_bound, clip_upper_bound
+        if not self.clip_upper_bound >= self.clip_lower_bound:
+            raise ValueError("clip_upper_bound must be at least clip_lower_bound")
+
+    def L_op(self, inputs, outputs, gout):
+        from .tensor import basic as T
+        return [T.clip(g, self.clip_lower_bound, self.clip_upper_bound) for g in gout]
+
+
+class GradScale(_GradView):
+    """The gradient is multiplied by ``multiplier`` on the way back (:2235-2275)."""
+
+    def __init__(self, multiplier):
+        self.multiplier = multiplier
+
+    def L_op(self, inputs, outputs, gout):
+        return [self.multiplier * g for g in gout]
+
+
+consider_constant_, zero_grad_, undefined_grad_, disconnected_grad_ = (ConsiderConstant(), ZeroGrad(), UndefinedGrad(),
+                                                                     DisconnectedGrad())
+
+
+def consider_constant(x):
+    """Deprecated: ``zero_grad`` or ``disconnected_grad``."""
+    import warnings
+    warnings.warn("consider_constant() is deprecated, use zero_grad() or disconnected_grad() instead.", stacklevel=2)
+    return consider_constant_(x)
+
+
+def zero_grad(x):
+    """``x``, with zeros for the gradient of everything behind it."""
+    return zero_grad_(x)
+
+
+def undefined_grad(x):
+    """``x``; taking a gradient through it raises NullTypeGradError."""
+    return undefined_grad_(x)
+
+
+def disconnected_grad(x):
+    """``x``, with nothing behind it reachable from the cost through this path."""
+    return disconnected_grad_(x)
+
+
+def grad_clip(x, lower_bound, upper_bound):
+    """``x`` in the forward pass; its gradient clipped elementwise to [lower_bound, upper_bound]."""
+    return GradClip(lower_bound, upper_bound)(x)
+
+
+def grad_scale(x, multiplier):
+    """``x`` in the forward pass; its gradient multiplied by ``multiplier``."""
+    return GradScale(multiplier)(x)

@@ -388,6 +388,21 @@ def local_max_to_min(fgraph, node):
     return [new] if new.type == node.outputs[0].type else False
 
 
+def _grad_view_op():
+    from ..gradient import _GradView
+    return _GradView
+
+
+@local_optimizer(None)
+def local_remove_grad_views(fgraph, node):
+    """``zero_grad`` / ``disconnected_grad`` / ``grad_clip`` / ``grad_scale`` nodes only matter while gradients
+    are derived: in a graph that is compiled they stand for their operand (``local_grad_clip``,
+    ``theano/tensor/opt.py:7500-7520``; the ViewOp removals of ``theano/compile/ops.py``)."""
+    if not isinstance(node.op, _grad_view_op()):
+        return False
+    return [node.inputs[0]]
+
+
 @local_optimizer([T.ShapeFloat])
 def local_shape_lift(fgraph, node):
     """The extent of an elementwise / DimShuffle / reduction result is the extent
@@ -618,7 +633,7 @@ def local_mul_to_sqr(fgraph, node):
     return [new] if new.type == node.outputs[0].type else False
 
 
-CANONICALIZE = [local_shape_lift, local_dimshuffle_fold, local_useless_composite, local_constant_fold,
+CANONICALIZE = [local_remove_grad_views, local_shape_lift, local_dimshuffle_fold, local_useless_composite, local_constant_fold,
                 local_useless_elemwise, local_fill_sink,
                 local_useless_reduce, local_op_of_op,
                 local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_max_to_min,
