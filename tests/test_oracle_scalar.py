@@ -469,3 +469,26 @@ def test_cast_ops_carry_the_module_level_names_of_the_reference():
     for dt in scal.all_dtypes:
         op = getattr(scal, "convert_to_" + dt)
         assert isinstance(op, scal.Cast) and op.o_type.dtype == dt and op.name == "convert_to_" + dt
+
+
+def test_scalar_type_tuples_constructors_and_output_policies():
+    """theano/scalar/basic.py:679-687 (type tuples), :818-833 (ints / floats / complexs), :90-95 (as_common_dtype),
+    :943-979 (int_out / float_out and the no-complex policies), :2036 (floor_div)."""
+    from theano_amd import scalar as scal, tensor as T
+    assert [t.dtype for t in scal.all_types] == list(scal.all_dtypes)
+    assert scal.discrete_types == (scal.bool_,) + scal.int_types + scal.uint_types
+    assert scal.continuous_types == scal.float_types + scal.complex_types
+    a, b = scal.ints("a", "b")
+    assert a.type == scal.int64 and b.name == "b" and scal.floats("x").type == scal.float64
+    assert [v.type for v in scal.complexs64("u v")] == [scal.complex64] * 2 and scal.complexs("z").type == scal.complex128
+    x, y = scal.as_common_dtype(scal.int8("i"), scal.float32("f"))
+    assert x.type == y.type == scal.float32
+    x, y = scal.as_common_dtype(T.imatrix(), T.fmatrix())
+    assert x.type.dtype == y.type.dtype == "float64"
+    assert scal.int_out(scal.int8, scal.float32) == (scal.int64,) and scal.float_out(scal.int8) == (scal.float64,)
+    assert scal.int_out_nocomplex(scal.int8) == (scal.int64,) and scal.float_out_nocomplex(scal.int8) == (scal.float64,)
+    assert scal.same_out_nocomplex(scal.float16) == (scal.float16,)
+    for policy in (scal.same_out_nocomplex, scal.int_out_nocomplex, scal.float_out_nocomplex):
+        with pytest.raises(TypeError, match="complex"):
+            policy(scal.complex64)
+    assert scal.floor_div is scal.int_div

@@ -105,6 +105,36 @@ float16, float32, float64 = Scalar("float16"), Scalar("float32"), Scalar("float6
 complex64, complex128 = Scalar("complex64"), Scalar("complex128")
 
 
+# the type tuples and constructors of theano/scalar/basic.py:679-687, 818-833
+int_types, uint_types = (int8, int16, int32, int64), (uint8, uint16, uint32, uint64)
+float_types, complex_types = (float16, float32, float64), (complex64, complex128)
+integer_types = int_types + uint_types
+discrete_types = (bool_,) + integer_types
+continuous_types = float_types + complex_types
+all_types = discrete_types + continuous_types
+
+
+def _multi(scalar_type):
+    """``ints("a b")``-style constructors: one variable for one name, a list for several."""
+    def make(*names):
+        if len(names) == 1 and isinstance(names[0], str) and " " in names[0]:
+            names = tuple(names[0].split())
+        made = [scalar_type(n) for n in names]
+        return made[0] if len(made) == 1 else made
+    return make
+
+
+ints, floats = _multi(int64), _multi(float64)
+complexs = complexs128 = _multi(complex128)
+complexs64 = _multi(complex64)
+
+
+def as_common_dtype(*vars):
+    """The variables (scalar or tensor) cast to the upcast of their dtypes (``theano/scalar/basic.py:90-95``)."""
+    dtype = upcast(*[v.type.dtype for v in vars])
+    return tuple(v.astype(dtype) for v in vars)
+
+
 class _scalar_py_operators(object):
     """Operator overloads so that gradient formulas read like arithmetic."""
 
@@ -279,6 +309,29 @@ def real_out(t):
     """The type of one component: float32 for complex64, float64 for complex128, the type itself
     otherwise (``theano/scalar/basic.py:1008-1019``)."""
     return ({"complex64": float32, "complex128": float64}.get(t.dtype, t),)
+
+
+def int_out(*types):
+    return (int64,)
+
+
+def float_out(*types):
+    return (float64,)
+
+
+def same_out_nocomplex(t):
+    _no_complex([t])
+    return (t,)
+
+
+def int_out_nocomplex(*types):
+    _no_complex(types)
+    return (int64,)
+
+
+def float_out_nocomplex(*types):
+    _no_complex(types)
+    return (float64,)
 
 
 def same_out_nobool(t):
@@ -836,6 +889,7 @@ class IntDiv(BinaryScalarOp):
 
 
 int_div = IntDiv(upcast_out, name="int_div")
+floor_div = int_div
 
 
 class Mod(BinaryScalarOp):
