@@ -581,3 +581,34 @@ def test_negated_max_of_a_negation_runs_as_min_with_the_same_values():
     assert np.array_equal(got, G.evaluate([i], [out], [iv])[0])
     # -(-2**31) wraps to -2**31, the smallest value: the written form skips that element, a min would return it
     assert got[2] == np.delete(iv[2], 3).min() and np.array_equal(np.delete(got, 2), np.delete(iv.min(axis=1), 2))
+
+
+def test_max_of_a_computed_value_and_its_gradient_see_the_same_bits():
+    """The gradient of max compares the reduction's result with its operand for equality.  When the operand is
+    a computed value, the kernel that reduces it and the kernel that compares it must agree to the last bit:
+    the operand is stored once and read by both (never recomputed per kernel), and sqrt / division / exp have
+    one spelled-out lowering.  Every reduced slice must find its maximum again."""
+    rng = np.random.default_rng(11)
+    x = T.TensorType("float32", (False,) * 4)("x")
+    y = T.TensorType("float32", (False,) * 4)("y")
+    xv = rng.standard_normal((16, 6, 64, 5)).astype("float32")
+    yv = rng.uniform(0.5, 1.5, xv.shape).astype("float32")
+    families = [lambda a, b: T.exp(T.minimum(T.sqrt(abs(a) + 0.5), 3.0)),
+                lambda a, b: a * b + a / (b + 2.0),
+                lambda a, b: T.tanh(a * 1.7 + b) / T.sqrt(b),
+                lambda a, b: T.sqr(a) * b + b * 0.3 + a]
+    for axis in ((0, 1), (1, 3), (0, 2, 3), (3,), None):
+        for fam in families:
+            e = fam(x, y)
+            m = T.max(e, axis=axis, keepdims=True)
+            hits = T.eq(m, e)
+            # the comparison runs in an elementwise kernel (its result is an output), the max in a reduction
+            got_hits, got_m, got_e = th.function([x, y], [hits, m, e], on_unused_input="ignore")(xv, yv)
+            assert np.array_equal(got_e.max(axis=axis, keepdims=True), got_m), (axis, hip.last_plan())
+            assert got_hits.any(axis=axis).all(), (axis, hip.last_plan())
+            # and through the gradient: each slice passes its incoming gradient to (at least) one element
+            g = th.grad(T.sum(T.max(e, axis=axis) * 1.0), x)
+            gv, ev = th.function([x, y], [g, e], on_unused_input="ignore")(xv, yv)
+            assert np.isfinite(gv).all()
+            at_max = ev == ev.max(axis=axis, keepdims=True)
+            assert np.array_equal(gv != 0, at_max & (gv != 0)) and (np.abs(gv) > 0).any(axis=axis).all(), axis

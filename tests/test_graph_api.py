@@ -1032,3 +1032,35 @@ def test_gradient_only_operations(dry_run):
     assert G.GradClip(0, 1) == G.GradClip(-5, 5) and G.zero_grad_ == G.ZeroGrad() and G.zero_grad_ != G.disconnected_grad_
     g = th.grad(T.sum(G.grad_scale(T.exp(x), 0.5)), x)
     assert "0.5" in " ".join(str(n.op) for n in th.function([x], g).toposort())
+
+
+def test_operand_of_a_max_that_something_else_reads_is_stored_not_recomputed(dry_run):
+    """A cheap elementwise result read by a sum and by another kernel is recomputed in each; read by a max or
+    min (whose gradient compares the result with the operand for equality) it is computed and stored once."""
+    x = T.fmatrix("x")
+    e = T.exp(x * 2.0)
+    f = th.function([x], [T.sum(e, axis=0), e * 3.0], rowchain=False)
+    red = [n.op for n in f.toposort() if isinstance(n.op, HipCAReduce)]
+    assert len(red) == 1 and red[0].pre_scalar_op is not None              # recomputed inside the sum
+    for reducer in (T.max, T.min):
+        f = th.function([x], [reducer(e, axis=0), e * 3.0], rowchain=False)
+        red = [n.op for n in f.toposort() if isinstance(n.op, HipCAReduce)]
+        assert len(red) == 1 and red[0].pre_scalar_op is None, red              # reads the stored values
+    i = T.imatrix("i")
+    f = th.function([i], [T.max(i * 2 + 1, axis=0), (i * 2 + 1) * 3], rowchain=False)   # integers are exact: recomputed
+    red = [n.op for n in f.toposort() if isinstance(n.op, HipCAReduce)]
+    assert len(red) == 1 and red[0].pre_scalar_op is not None
+    # a batch-norm-shaped chain evaluates its closures once per loop: fine for a max whose result is only used
+    # arithmetically, not when a later step tests it against the value for equality (the gradient of max)
+    x4 = T.ftensor4("x4")
+    e4 = T.exp(x4 * 0.5)
+    m4 = T.max(e4, axis=(0, 2, 3), keepdims=True)
+
+    def held_chains(f):
+        return [n for n in f.toposort() if type(n.op).__name__ == "HipRowChain" and n.op.program.axes == (0, 2, 3)]
+    assert len(held_chains(th.function([x4], e4 / m4 + T.sum(e4, axis=(0, 2, 3), keepdims=True)))) == 1
+    g = th.grad(T.sum(T.max(e4, axis=(0, 2, 3)) * T.sum(e4, axis=(0, 2, 3))), x4)
+    f = th.function([x4], g)
+    assert not held_chains(f)
+    red = [n.op for n in f.toposort() if isinstance(n.op, HipCAReduce)]
+    assert red and all(r.pre_scalar_op is None or "exp" not in str(r.pre_scalar_op) for r in red)

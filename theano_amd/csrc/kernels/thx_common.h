@@ -44,6 +44,23 @@ __device__ __forceinline__ float thx_fdiv(float a, float b) {
 __device__ __forceinline__ float thx_fdiv(float a, float b) { return a / b; }
 #endif
 
+// Square root in single precision as the generated per-element code spells it.  With THX_FAST_DIV: one
+// v_sqrt_f32 (1 ulp); operands below 2^-96 are scaled by 2^32 first so that denormals keep their precision.
+// The compiler's own lowering of sqrtf under the 2.5-ulp flag depends on the surrounding code (the
+// permission is dropped where the optimiser vectorises the call, and the correctly rounded sequence comes
+// out instead), so one expression compiled into two kernels, or into two loops of one kernel, could differ
+// in the last bit - and a gradient of max, which compares the reduction's result with its recomputed
+// operand for equality, would then miss the maximum.  Spelled out, every copy agrees.
+#ifdef THX_FAST_DIV
+__device__ __forceinline__ float thx_fsqrt(float x) {
+  const bool small = x < 0x1.0p-96f;
+  const float r = __builtin_amdgcn_sqrtf(small ? x * 0x1.0p+32f : x);
+  return small ? r * 0x1.0p-16f : r;
+}
+#else
+__device__ __forceinline__ float thx_fsqrt(float x) { return sqrtf(x); }
+#endif
+
 // exp(x) in single precision.  In the 2.5-ulp build: one hardware exp2 of the rounded product
 // x * log2(e); the rounding of the product is a relative error of up to |x| * 4e-8 in the result
 // (3.8e-6 at the ends of the finite range, |x| = 88), overflow gives infinity and underflow zero as

@@ -176,6 +176,14 @@ def _duplicable(fgraph, var):
     clients = fgraph.clients.get(var, [])
     if len(clients) < 2 or len(clients) > 8:
         return False
+    # The gradient of max / min (and what users write with argmax) compares the reduction's result with
+    # its operand for equality: both kernels must see the very same floating-point values, which two
+    # compilations of one expression do not promise (contraction into fused multiply-adds depends on the
+    # surrounding code).  Such an operand is stored once and read back.
+    if var.type.dtype in scal.continuous_dtypes and any(
+            c != "output" and (isinstance(c.op, HipMaxAndArgmax) or (isinstance(c.op, HipCAReduce) and any(
+                isinstance(o, (scal.Maximum, scal.Minimum)) for o in c.op.scalar_ops))) for c, _ in clients):
+        return False
     # exp(x - m) read by a sum and by a division is worth two evaluations (the sum's kernel never writes
     # it); among elementwise consumers only, the sibling merge computes it once in one kernel anyway
     def full_size_operand_of(c):

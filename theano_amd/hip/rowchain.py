@@ -73,6 +73,15 @@ def _row_shape(full, red, keepdims):
     return tuple(n for d, n in enumerate(full) if d not in red)
 
 
+def _tests_equality(scalar_op):
+    """Does the scalar operation (or a Composite's inner graph) compare values with == or != ?"""
+    if isinstance(scalar_op, (scal.EQ, scal.NEQ)):
+        return True
+    if isinstance(scalar_op, scal.Composite):
+        return any(_tests_equality(n.op) for n in gof.io_toposort(scalar_op.inputs, scalar_op.outputs))
+    return False
+
+
 class RowProgram(object):
     """Straight-line program over per-element values and per-row scalars."""
 
@@ -283,6 +292,13 @@ class RowProgram(object):
                     scalar_step(step)
             else:
                 if codegen.reduce_identity(step[1], step[2]) is None:
+                    return None
+                # max / min of a computed floating-point value that a later step tests for equality (the gradient
+                # of max does: eq(max, value)) needs the very same bits in both places, which a second evaluation
+                # in another loop does not promise; values held as they were read always qualify
+                if (isinstance(step[1], (scal.Maximum, scal.Minimum)) and step[4] >= n_in and
+                        self.var[step[4]][1] in scal.continuous_dtypes and
+                        any(t[0] == "ew" and _tests_equality(t[1]) for t in self.steps[self.steps.index(step) + 1:])):
                     return None
                 steps, inputs, scalars = [], set(), set()
                 closure(step[4], steps, inputs, scalars)

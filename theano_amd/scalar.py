@@ -1116,6 +1116,8 @@ def _unary_math(cname, fname, grad_fn, policy=upgrade_to_float):
             fn = _fn(fname, ot)
             if fn == "expf":
                 fn = "thx_fexp"        # expf, or exp2 of x * log2(e) in the 2.5-ulp build
+            elif fn == "sqrtf":
+                fn = "thx_fsqrt"       # sqrtf, or one hardware sqrt in the 2.5-ulp build: the same bits in every kernel
             return "%s = %s((%s)%s);" % (outputs[0], fn, compute_ctype(ot), inputs[0])
 
         def L_op(self, inputs, outputs, gout):
