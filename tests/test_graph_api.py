@@ -962,6 +962,9 @@ def test_graphs_with_inplace_operations_need_accept_inplace(dry_run):
         th.function([x], I.exp_inplace(x.T), accept_inplace=True)
     with pytest.raises(ValueError, match="leaves its arguments alone"):
         th.function([x, y], I.add_inplace(x, y), accept_inplace=True, mode="check")
+    # overwriting an intermediate is invisible to the caller: check mode takes it
+    f = th.function([x, y], I.sub_inplace(x * y, y), accept_inplace=True, mode="check")
+    assert isinstance(f, th.compile.CheckedFunction) and f.primary.writeback == []
 
 
 def test_negated_max_of_a_negation_is_a_min(dry_run):

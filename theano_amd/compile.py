@@ -505,7 +505,7 @@ def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=Tru
     ref_outs = [Out(v, device=spec.device) for v, spec in zip(out_vars, out_specs)]
     ref_outs += [Out(v, device=True) for v in out_vars[len(out_specs):]]
     reference = function(in_specs, ref_outs, givens=None, fuse=False, rowchain=False, inplace=False,
-                         on_unused_input="ignore")
+                         on_unused_input="ignore", accept_inplace=accept_inplace)
     return CheckedFunction(primary, reference, len(update_targets))
 
 
