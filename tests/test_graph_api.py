@@ -1067,3 +1067,30 @@ def test_operand_of_a_max_that_something_else_reads_is_stored_not_recomputed(dry
     assert not held_chains(f)
     red = [n.op for n in f.toposort() if isinstance(n.op, HipCAReduce)]
     assert red and all(r.pre_scalar_op is None or "exp" not in str(r.pre_scalar_op) for r in red)
+
+
+def test_input_options(dry_run):
+    """In(strict=, allow_downcast=, mutable=, borrow=) and function(allow_input_downcast=)
+    (theano/compile/io.py:40-216, theano/compile/function.py:70-300)."""
+    from theano_amd.compile import In
+    x = T.fvector("x")
+    v64, v32 = np.ones(4, "float64"), np.ones(4, "float32")
+    f = th.function([x], x + 1)
+    f(v32)
+    with pytest.raises(TypeError, match="precision"):
+        f(v64)                                                    # float64 values do not go into a float32 input
+    th.function([x], x + 1, allow_input_downcast=True)(v64)
+    th.function([In(x, allow_downcast=True)], x + 1)(v64)
+    g = th.function([In(x, strict=True)], x + 1)
+    g(v32)
+    for bad in ([1.0, 2.0, 3.0, 4.0], np.ones(4, "float16"), v64):
+        with pytest.raises(TypeError):
+            g(bad)                                                # strict: no conversion at all
+    f([1.0, 2.0])                                                  # without it Python numbers convert
+    spec = In(x, mutable=True)
+    assert spec.mutable and spec.borrow and In(x, borrow=True).mutable and not In(x).mutable
+    assert In(x, name="data").name == "data" and In(x).name == "x"
+    with pytest.raises(ValueError):
+        In(x, strict=True, allow_downcast=True)
+    with pytest.raises(NotImplementedError):
+        In(x, value=v32)

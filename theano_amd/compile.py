@@ -15,10 +15,25 @@ from .tensor.type import TensorType, as_tensor_variable
 
 
 class In(object):
-    def __init__(self, variable, name=None, borrow=False, allow_downcast=None):
+    """An input with options (``theano/compile/io.py:40-216``).  ``strict``: the argument must already have
+    the input's dtype and rank (no conversion); ``allow_downcast``: conversions that lose precision are
+    accepted; ``mutable`` / ``borrow``: permission for the function to overwrite the argument - what
+    ``accept_inplace`` graphs do to the arguments their operations destroy, with or without it, as in the
+    reference.  Default values and per-input updates (``value=``, ``update=``) belong to shared variables
+    here: ``shared(...)`` with ``function(updates=...)``."""
+
+    def __init__(self, variable, name=None, value=None, update=None, mutable=None, strict=False, allow_downcast=None,
+                 autoname=True, implicit=None, borrow=None, shared=False):
+        if value is not None or update is not None or implicit or shared:
+            raise NotImplementedError("In(value=, update=, implicit=, shared=): use a shared variable and "
+                                      "function(updates=...)")
+        if strict and allow_downcast:
+            raise ValueError("In(strict=True) excludes allow_downcast")
         self.variable = variable
-        self.name = name or variable.name
-        self.borrow = borrow
+        self.name = name or (variable.name if autoname else None)
+        self.borrow = bool(borrow) if borrow is not None else bool(mutable)
+        self.mutable = bool(mutable) if mutable is not None else self.borrow
+        self.strict = bool(strict)
         self.allow_downcast = allow_downcast
 
 
@@ -324,7 +339,7 @@ class Function(object):
                 self.storage[var][0] = a
             else:
                 try:
-                    v = self.storage[var][0] = var.type.filter(a, strict=False, allow_downcast=spec.allow_downcast)
+                    v = self.storage[var][0] = var.type.filter(a, strict=spec.strict, allow_downcast=spec.allow_downcast)
                     if type(v) is np.ndarray:
                         self._last_shape[var] = v.shape
                 except TypeError as e:
@@ -398,7 +413,7 @@ class Function(object):
 
 
 def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=True, inplace=True, name=None,
-             on_unused_input="raise", mode=None, accept_inplace=False):
+             on_unused_input="raise", mode=None, accept_inplace=False, allow_input_downcast=None):
     """Compile ``outputs`` as a function of ``inputs``.
 
     ``inputs``: variables or ``In`` instances.  A host-typed input may be given
@@ -416,13 +431,14 @@ def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=Tru
     every elementwise result a buffer of its own.  ``mode``: None, ``'nan_guard'`` (every node's
     floating-point results are scanned for NaN / infinity, ``NanGuardError``) or ``'check'`` (see
     ``CheckedFunction``: arguments must come back unchanged and results must not depend on fusion or
-    in-place operation).  ``accept_inplace``: the graph may hold operations that overwrite an operand
+    in-place operation).  ``allow_input_downcast``: arguments of plain (non-``In``) inputs may be converted
+    with loss of precision, e.g. float64 values for a float32 input.  ``accept_inplace``: the graph may hold operations that overwrite an operand
     (``theano.tensor.inplace``); without it such a graph is refused, as in the reference
     (``theano/compile/function_module.py:183-190``) - see ``_functional_form`` for how they run."""
     from .hip import opt as hip_opt
     from .hip.ops import HipArrayType, as_hip_variable
 
-    in_specs = [i if isinstance(i, In) else In(i) for i in inputs]
+    in_specs = [i if isinstance(i, In) else In(i, allow_downcast=allow_input_downcast) for i in inputs]
     if outputs is None:
         outputs = []
     single = not isinstance(outputs, (list, tuple))
