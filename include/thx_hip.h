@@ -255,6 +255,24 @@ const char* thx_last_plan(void);
 int thx_profile_begin(void);
 int thx_profile_end(char* buf, size_t cap);
 
+/* ---- recorded launch sequences -------------------------------------------
+ * No counterpart in the reference (every GpuElemwise / GpuCAReduceCuda call is
+ * launched on its own, theano/gpuarray/elemwise.py:376, :1095-1723).  For hosts
+ * whose per-launch cost exceeds the kernels' run time: everything the library
+ * launches between thx_capture_begin and thx_capture_end is recorded into a HIP
+ * graph instead of run; thx_graph_launch replays it on the library's stream with
+ * the very same addresses, so the caller keeps every array that took part alive
+ * and unmoved until thx_graph_free.  Calls that wait for the device (thx_d2h,
+ * thx_h2d, thx_sync, thx_timer_stop, thx_profile_*) must not be made while a
+ * capture is open; run the sequence once before capturing it, so that kernels
+ * are loaded and the allocation pool is warm.  thx_capture_end(NULL) abandons
+ * the recording. */
+typedef struct thx_graph thx_graph;
+int thx_capture_begin(void);
+int thx_capture_end(thx_graph** out);
+int thx_graph_launch(thx_graph* g);
+int thx_graph_free(thx_graph* g);
+
 /* Whole-region timing: events recorded on the library's stream. */
 int thx_timer_start(void);
 int thx_timer_stop(float* elapsed_ms); /* synchronises */

@@ -392,6 +392,29 @@ class Function(object):
             return results[0]
         return results
 
+    def capture(self, *args):
+        """Record one call of this function on device-resident arguments as a HIP graph: returns
+        ``(results, graph)``; every ``graph.launch()`` runs the function's kernels again on the same argument
+        arrays and writes the same result arrays, at the cost of one launch for the whole sequence.  For
+        functions of several small kernels, where the host's work per launch exceeds the kernels' run time.
+        The arguments and results must be device arrays (``Out(v, device=True)``): a transfer would wait for
+        the device in the middle of the recording.  The function is run once first, so that its kernels are
+        loaded and the shapes it depends on are known; calls that the function makes differently from one
+        run to the next (a row chain turned away at run time, say) are recorded as this call made them."""
+        from .hip.ops import HipToHost
+        from .hip.runtime import capture
+        if self.update_targets or self.writeback:
+            raise ValueError("capture: a function with updates or in-place arguments changes state on the host")
+        if not all(isinstance(a, self._HipArray) for a in args):
+            raise TypeError("capture: every argument must be a device array")
+        if any(isinstance(n.op, HipToHost) for n in self.nodes):
+            raise TypeError("capture: the function copies results to the host; ask for device results, "
+                            "Out(v, device=True)")
+        self(*args)                         # loads the kernels, warms the pool, runs the shape-only nodes
+        with capture() as c:
+            results = self(*args)
+        return results, c.graph
+
     def _write_back(self, args, values):
         """Store each hidden result into the argument its operation overwrites: a device argument takes a
         device copy (whatever its strides), a writable host array of the input's dtype takes the values;

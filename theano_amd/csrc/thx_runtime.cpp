@@ -652,4 +652,63 @@ int thx_timer_stop(float* elapsed_ms) {
   return THX_OK;
 }
 
+// ---- launch sequences recorded once and replayed (HIP graphs) ---------------------------------------------
+struct thx_graph {
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+};
+
+static bool g_capturing = false;
+
+int thx_capture_begin(void) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  if (g_capturing) return fail(THX_ERR_ARG, "thx_capture_begin: a capture is already open");
+  if (g_profiling) return fail(THX_ERR_ARG, "thx_capture_begin: not while profiling (its events are not part of the work)");
+  THX_HIP_CHECK(hipStreamBeginCapture(rt().stream, hipStreamCaptureModeRelaxed));
+  g_capturing = true;
+  return THX_OK;
+}
+
+int thx_capture_end(thx_graph** out) {
+  if (!g_capturing) return fail(THX_ERR_ARG, "thx_capture_end: no capture is open");
+  g_capturing = false;
+  hipGraph_t graph = nullptr;
+  hipError_t e = hipStreamEndCapture(rt().stream, &graph);
+  if (e != hipSuccess || !graph)
+    return fail(THX_ERR_HIP, "hipStreamEndCapture failed: %s (a call that waits for the device ends a capture)",
+                hipGetErrorString(e));
+  if (!out) {                      // the caller only wanted to leave capture mode
+    (void)hipGraphDestroy(graph);
+    return THX_OK;
+  }
+  hipGraphExec_t exec = nullptr;
+  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  if (e != hipSuccess) {
+    (void)hipGraphDestroy(graph);
+    return fail(THX_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  }
+  thx_graph* g = new thx_graph;
+  g->graph = graph;
+  g->exec = exec;
+  *out = g;
+  return THX_OK;
+}
+
+int thx_graph_launch(thx_graph* g) {
+  if (!g || !g->exec) return fail(THX_ERR_ARG, "thx_graph_launch: null graph");
+  if (g_capturing) return fail(THX_ERR_ARG, "thx_graph_launch: a capture is open");
+  THX_HIP_CHECK(hipGraphLaunch(g->exec, rt().stream));
+  return THX_OK;
+}
+
+int thx_graph_free(thx_graph* g) {
+  if (!g) return THX_OK;
+  if (rt().ready) (void)hipStreamSynchronize(rt().stream);
+  if (g->exec) (void)hipGraphExecDestroy(g->exec);
+  if (g->graph) (void)hipGraphDestroy(g->graph);
+  delete g;
+  return THX_OK;
+}
+
 }  // extern "C"

@@ -1,5 +1,5 @@
 """HIP backend: runtime binding, device ops and the rewrites that lift a graph onto them."""
-from .runtime import (HipArray, HipRuntimeError, cache_stats, device_info, dry_run, init, last_plan, profile,  # noqa: F401
+from .runtime import (Graph, HipArray, HipRuntimeError, cache_stats, capture, device_info, dry_run, init, last_plan, profile,  # noqa: F401
                       set_dry_run, sync, timer_start, timer_stop)
 from .ops import (HipArrayType, HipCAReduce, HipDimShuffle, HipElemwise, HipElemwiseReduce, HipMaxAndArgmax, HipToHost, HostToHip,  # noqa: F401
                   as_hip_variable,

@@ -79,6 +79,10 @@ def _load():
         "thx_profile_end": ([ctypes.c_char_p, sz], ctypes.c_int),
         "thx_timer_start": ([], ctypes.c_int),
         "thx_timer_stop": ([P(ctypes.c_float)], ctypes.c_int),
+        "thx_capture_begin": ([], ctypes.c_int),
+        "thx_capture_end": ([P(vp)], ctypes.c_int),
+        "thx_graph_launch": ([vp], ctypes.c_int),
+        "thx_graph_free": ([vp], ctypes.c_int),
     }
     for name, (argtypes, restype) in sigs.items():
         fn = getattr(lib, name, None)
@@ -196,6 +200,57 @@ def timer_stop():
 
 
 # --------------------------------------------------------------------------
+_capture_keep = None      # while a capture is open: the buffers allocated inside it, which its graph owns
+
+
+class Graph(object):
+    """A recorded sequence of launches (``capture``): ``launch()`` replays it on the library's stream.  The
+    graph owns every buffer that was allocated while it was recorded - replays write to those addresses."""
+
+    def __init__(self, handle, buffers):
+        self._handle, self._buffers = handle, buffers
+
+    def launch(self):
+        check(lib.thx_graph_launch(self._handle))
+
+    def __del__(self):
+        try:
+            if self._handle is not None:
+                lib.thx_graph_free(self._handle)
+                self._handle = None
+        except Exception:
+            pass
+
+
+class capture(object):
+    """``with capture() as c: ...`` records what the library launches inside the block instead of running it;
+    ``c.graph`` is the replayable result.  Nothing inside may wait for the device (no ``to_numpy``, no host
+    arguments or results), and the same calls should have run once before, so that their kernels are loaded."""
+
+    def __enter__(self):
+        global _capture_keep
+        if _dry:
+            raise HipRuntimeError("nothing is launched in dry-run mode: there is nothing to capture")
+        if _capture_keep is not None:
+            raise HipRuntimeError("a capture is already open")
+        init()
+        check(lib.thx_capture_begin())
+        _capture_keep = []
+        self.graph = None
+        return self
+
+    def __exit__(self, et, ev, tb):
+        global _capture_keep
+        kept, _capture_keep = _capture_keep, None
+        if et is not None:
+            lib.thx_capture_end(None)
+            return False
+        h = ctypes.c_void_p()
+        check(lib.thx_capture_end(ctypes.byref(h)))
+        self.graph = Graph(h, kept)
+        return False
+
+
 class _Buffer(object):
     """One pooled device allocation, released when the last view dies."""
 
@@ -212,6 +267,8 @@ class _Buffer(object):
         p = ctypes.c_void_p()
         check(lib.thx_alloc(max(int(nbytes), 1), ctypes.byref(p)))
         self.ptr = p.value
+        if _capture_keep is not None:
+            _capture_keep.append(self)
 
     def __del__(self):
         try:
