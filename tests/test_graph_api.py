@@ -1094,3 +1094,16 @@ def test_input_options(dry_run):
         In(x, strict=True, allow_downcast=True)
     with pytest.raises(NotImplementedError):
         In(x, value=v32)
+
+
+def test_type_constructors_of_every_rank_and_their_plurals():
+    """tensor5 ... tensor7 with their dtype prefixes, and matrices('a', 'b') / fvectors(3) ...
+    (theano/tensor/basic.py:644-790)."""
+    assert T.tensor5().type.ndim == 5 and T.ftensor6("u").type == T.TensorType("float32", (False,) * 6)
+    assert T.ztensor7().type.dtype == "complex128" and T.btensor5().type.dtype == "int8" and T.ltensor7("q").name == "q"
+    a, b = T.fmatrices("a", "b")
+    assert a.type == b.type == T.fmatrix().type and (a.name, b.name) == ("a", "b")
+    assert [v.type.ndim for v in T.tensor3s(2)] == [3, 3] and T.ivectors("k").type == T.ivector().type
+    assert [v.name for v in T.dscalars(["p", "q", "r"])] == ["p", "q", "r"]
+    assert T.lrows("r").type.broadcastable == (True, False) and T.dcols("c").type.broadcastable == (False, True)
+    assert len(T.tensor7s("a", "b", "c")) == 3 and T.dtensor5s("u", "v")[1].type.ndim == 5

@@ -6,7 +6,10 @@ from .type import (TensorType, TensorVariable, TensorConstant, as_tensor_variabl
                    dscalar, dvector, dmatrix, drow, dcol, dtensor3, dtensor4)
 from . import type as _type
 for _n in dir(_type):  # bscalar ... dtensor4 and friends
-    if _n[0] in "bwilhfdcz" and _n[1:] in ("scalar", "vector", "matrix", "row", "col", "tensor3", "tensor4"):
+    if _n[0] in "bwilhfdcz" and _n[1:] in ("scalar", "vector", "matrix", "row", "col", "tensor3", "tensor4", "tensor5",
+                                           "tensor6", "tensor7"):
+        globals()[_n] = getattr(_type, _n)
+    if _n.lstrip("fdil") in _type._PLURAL.values() or _n in ("tensor5", "tensor6", "tensor7"):
         globals()[_n] = getattr(_type, _n)
 from .elemwise import DimShuffle, Elemwise, CAReduce, CAReduceDtype, Sum, Prod, All, Any
 from .basic import *  # noqa: F401,F403

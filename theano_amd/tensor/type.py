@@ -455,6 +455,8 @@ for _p, _dt in (("b", "int8"), ("w", "int16"), ("i", "int32"), ("l", "int64"), (
     globals()[_p + "col"] = _mk(_dt, (False, True))
     globals()[_p + "tensor3"] = _mk(_dt, (False,) * 3)
     globals()[_p + "tensor4"] = _mk(_dt, (False,) * 4)
+    for _nd in (5, 6, 7):
+        globals()[_p + "tensor%d" % _nd] = _mk(_dt, (False,) * _nd)
 
 
 def scalar(name=None, dtype=None):
@@ -485,5 +487,39 @@ def tensor4(name=None, dtype=None):
     return TensorType(dtype or config.floatX, (False,) * 4)(name)
 
 
+def tensor5(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, (False,) * 5)(name)
+
+
+def tensor6(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, (False,) * 6)(name)
+
+
+def tensor7(name=None, dtype=None):
+    return TensorType(dtype or config.floatX, (False,) * 7)(name)
+
+
 def tensor(dtype, broadcastable, name=None):
     return TensorType(dtype, broadcastable)(name)
+
+
+def _plural(make):
+    """``matrices('a', 'b')`` / ``matrices(3)``: several variables of one constructor at once, a single one for a
+    single name (``_multi``, ``theano/tensor/basic.py:644-661``)."""
+    def many(*names):
+        if len(names) == 1 and isinstance(names[0], (int, np.integer)) and not isinstance(names[0], bool):
+            return [make() for _ in range(int(names[0]))]
+        if len(names) == 1 and isinstance(names[0], (list, tuple)):
+            names = tuple(names[0])
+        if len(names) == 1:
+            return make(names[0])
+        return [make(n) for n in names]
+    return many
+
+
+_PLURAL = {"scalar": "scalars", "vector": "vectors", "matrix": "matrices", "row": "rows", "col": "cols",
+           "tensor3": "tensor3s", "tensor4": "tensor4s", "tensor5": "tensor5s", "tensor6": "tensor6s",
+           "tensor7": "tensor7s"}
+for _one, _many in _PLURAL.items():
+    for _p in ("", "f", "d", "i", "l"):
+        globals()[_p + _many] = _plural(globals()[_p + _one])
