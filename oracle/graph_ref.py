@@ -169,7 +169,7 @@ def eval_scalar_op(op, in_values, out_dtypes, wide=False):
     if wide:
         out_dtypes = [_wide(d) for d in out_dtypes]
         in_values = [np.asarray(v).astype(_wide(np.asarray(v).dtype), copy=False) for v in in_values]
-    if name == "Composite":
+    if any(c.__name__ == "Composite" for c in type(op).__mro__):      # Composite and its subclasses: node by node
         from theano_amd import gof
         env = dict(zip(op.inputs, in_values))
         for node in gof.io_toposort(op.inputs, op.outputs):

@@ -291,3 +291,24 @@ def test_random_normalisation_gradient_matches_the_oracle(seed):
         else:
             assert_within_reference_error(g, r, w, "seed %d output %d" % (seed, k),
                                           tol=dict(rtol=2e-3, atol=2e-3) if dtype == "float16" else None)
+
+
+def test_batch_normalization_with_given_statistics_runs_as_one_kernel_per_direction():
+    """nnet.batch_normalization (statistics supplied by the caller) in both modes, with gradients, against the
+    oracle; float32 and float16 activations with per-channel parameters."""
+    from theano_amd.tensor import nnet as N
+    rng = np.random.default_rng(17)
+    for dtype, tol in (("float32", None), ("float16", dict(rtol=2e-3, atol=2e-3))):
+        x = tensor(dtype, 4, "x")
+        g, b, m, s = [per_index(dtype, 4, (1,), n) for n in "gbms"]
+        ins = [x, g, b, m, s]
+        vals = [rng.standard_normal((6, 9, 5, 7)).astype(dtype)] + [rng.uniform(0.5, 1.5, (1, 9, 1, 1)).astype(dtype)
+                                                                     for _ in range(4)]
+        for mode in ("low_mem", "high_mem"):
+            out = N.batch_normalization(x, g, b, m, s, mode)
+            outs = [out] + th.grad(T.sum(T.cast(out, "float32") * T.cast(x, "float32")), ins)
+            got = th.function(ins, outs)(*vals)
+            ref = G.evaluate(ins, outs, vals)
+            truth = G.evaluate(ins, outs, vals, wide=True)
+            for k, (a, r, w) in enumerate(zip(got, ref, truth)):
+                assert_within_reference_error(a, r, w, "%s %s output %d" % (dtype, mode, k), tol=tol)

@@ -1107,3 +1107,35 @@ def test_type_constructors_of_every_rank_and_their_plurals():
     assert [v.name for v in T.dscalars(["p", "q", "r"])] == ["p", "q", "r"]
     assert T.lrows("r").type.broadcastable == (True, False) and T.dcols("c").type.broadcastable == (False, True)
     assert len(T.tensor7s("a", "b", "c")) == 3 and T.dtensor5s("u", "v")[1].type.ndim == 5
+
+
+def test_batch_normalization_with_given_statistics_and_nnet_aliases(dry_run):
+    """nnet.batch_normalization (theano/tensor/nnet/bn.py:14-97): 'low_mem' is one Elemwise over BNComposite whose
+    written-out gradients equal those of the 'high_mem' expression; the scalar ops and in-place variants that
+    sigm.py exports (:29-300)."""
+    import pickle
+    from oracle import graph_ref as G
+    from theano_amd.tensor import nnet as N
+    x = T.fmatrix("x")
+    g, b, m, s = [T.frow(n) for n in "gbms"]
+    ins = [x, g, b, m, s]
+    lo, hi = N.batch_normalization(x, g, b, m, s), N.batch_normalization(x, g, b, m, s, "high_mem")
+    assert isinstance(lo.owner.op.scalar_op, N.BNComposite) and len(lo.owner.inputs) == 5
+    rng = np.random.default_rng(0)
+    vals = [rng.standard_normal((5, 7)).astype("float32")] + [rng.uniform(0.5, 1.5, (1, 7)).astype("float32") for _ in range(4)]
+    r = G.evaluate(ins, [lo, hi] + th.grad(T.sum(lo * x), ins) + th.grad(T.sum(hi * x), ins), vals)
+    xv, gv, bv, mv, sv = [v.astype("float64") for v in vals]
+    np.testing.assert_allclose(r[0], (xv - mv) / sv * gv + bv, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(r[1], r[0], rtol=1e-5, atol=1e-6)
+    for a, c in zip(r[2:7], r[7:12]):
+        np.testing.assert_allclose(a, c, rtol=3e-5, atol=2e-6)
+    assert pickle.loads(pickle.dumps(lo.owner.op)) == lo.owner.op
+    with pytest.raises(ValueError, match="low_mem"):
+        N.batch_normalization(x, g, b, m, s, "medium_mem")
+    f = th.function(ins, [lo] + th.grad(T.sum(lo * x), ins))
+    assert sum(isinstance(n.op, HipElemwise) for n in f.toposort()) == 1        # forward and dx in one kernel
+    assert N.ScalarSigmoid is scal.ScalarSigmoid and N.scalar_softplus is scal.scalar_softplus
+    assert N.ultra_fast_scalar_sigmoid is scal.ultra_fast_scalar_sigmoid
+    for op, base in ((N.sigmoid_inplace, scal.ScalarSigmoid), (N.softplus_inplace, scal.ScalarSoftplus),
+                     (N.ultra_fast_sigmoid_inplace, scal.UltraFastScalarSigmoid)):
+        assert isinstance(op.scalar_op, base) and op.destroy_map == {0: [0]} and op(x).type == x.type

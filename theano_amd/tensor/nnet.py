@@ -20,6 +20,16 @@ from .type import as_tensor_variable
 
 sigmoid = T.sigmoid
 softplus = T.softplus
+# the scalar ops behind them live in this module in the reference (theano/tensor/nnet/sigm.py:29-300)
+ScalarSigmoid, ScalarSoftplus, UltraFastScalarSigmoid = scal.ScalarSigmoid, scal.ScalarSoftplus, scal.UltraFastScalarSigmoid
+scalar_sigmoid, scalar_softplus, ultra_fast_scalar_sigmoid = (scal.scalar_sigmoid, scal.scalar_softplus,
+                                                              scal.ultra_fast_scalar_sigmoid)
+sigmoid_inplace = Elemwise(scal.scalar_sigmoid.make_new_inplace(scal.transfer_type(0), name="sigmoid_inplace"), {0: 0},
+                           name="sigmoid_inplace")
+softplus_inplace = Elemwise(scal.scalar_softplus.make_new_inplace(scal.transfer_type(0), name="softplus_inplace"), {0: 0},
+                            name="softplus_inplace")
+ultra_fast_sigmoid_inplace = Elemwise(scal.ultra_fast_scalar_sigmoid.make_new_inplace(
+    scal.transfer_type(0), name="ultra_fast_sigmoid_inplace"), {0: 0}, name="ultra_fast_sigmoid_inplace")
 
 _FLOATS = ("float16", "float32", "float64")
 
@@ -827,6 +837,43 @@ def batch_normalization_train_grad(x, dy, scale, x_mean, x_invstd, axes="per-act
     x = as_tensor_variable(x)
     axes = _bn_axes(axes, x.type.ndim)
     return tuple(AbstractBatchNormTrainGrad(axes)(x, dy, scale, x_mean, x_invstd, epsilon, return_list=True))
+
+
+class BNComposite(scal.Composite):
+    """``(x - mean) / std * gamma + beta`` as one scalar operation with the gradients written out
+    (``theano/tensor/nnet/bn.py:14-39``): nothing is kept for the backward pass."""
+
+    def __init__(self, dtype):
+        self.dtype = dtype
+        x, mean, std, gamma, beta = [scal.Scalar(dtype)() for _ in range(5)]
+        out = scal.add(scal.mul(scal.true_div(scal.sub(x, mean), std), gamma), beta)
+        scal.Composite.__init__(self, [x, mean, std, gamma, beta], [out])
+
+    def make_new_inplace(self, output_types_preference=None, name=None):
+        return self
+
+    def __reduce__(self):
+        return (BNComposite, (self.dtype,))
+
+    def L_op(self, inputs, outputs, gout):
+        x, mean, std, gamma, beta = inputs
+        (top,) = gout
+        top_gamma = top * gamma
+        x_mean = x - mean
+        dx = top_gamma / std
+        return [dx, -dx, -(top_gamma * x_mean) / (std * std), top * x_mean / std, top]
+
+
+def batch_normalization(inputs, gamma, beta, mean, std, mode="low_mem"):
+    """``(inputs - mean) * (gamma / std) + beta`` with statistics the caller supplies
+    (``theano/tensor/nnet/bn.py:42-97``).  'low_mem': one elementwise node over ``BNComposite``, whose gradient
+    recomputes what it needs; 'high_mem': the expression written with separate nodes."""
+    if mode == "low_mem":
+        inputs = as_tensor_variable(inputs)
+        return Elemwise(BNComposite(inputs.type.dtype))(inputs, mean, std, gamma, beta)
+    if mode == "high_mem":
+        return (inputs - mean) * (gamma / std) + beta
+    raise ValueError('mode must be either "low_mem", "high_mem"')
 
 
 def batch_normalization_test(inputs, gamma, beta, mean, var, axes="per-activation", epsilon=1e-4):
