@@ -27,7 +27,10 @@ gradient checks of tests/test_oracle_graph.py.  The approximate sigmoid is pinne
 hand-evaluated points on each of its pieces, its symmetry and its known distance to
 the sigmoid; softsign by exact quotients; the fused sigmoid cross-entropy by
 ``log(1 + e^x) - x t`` and, where that is well conditioned, the two-logarithm
-definition.  No function here is unpinned.
+definition.  The angle-unit conversions are pinned element by element against Python float
+arithmetic (the double product rounded once - which NumPy's float32 ``deg2rad`` is not) and by
+known angles; the range test against Python's comparisons on every triple of a small grid, for
+the four open / closed combinations and mixed operand types.  No function here is unpinned.
 """
 import numpy as np
 
