@@ -64,3 +64,29 @@ def test_what_cannot_be_captured_is_refused():
     assert np.array_equal(f(xd).to_numpy(), np.full((4, 5), 2, "float32"))
     with pytest.raises(ValueError, match="no capture is open"):
         hip.runtime.check(hip.runtime.lib.thx_capture_end(None))          # none open
+
+
+def test_chain_nodes_replay_too_held_and_turned_away():
+    """Batch-normalisation graphs: a held chain (one kernel), and a chain that is turned away at run time and runs
+    its island through the inner function - both record and replay to the eager results."""
+    rng = np.random.default_rng(9)
+    x4 = T.TensorType("float32", (False,) * 4)("x")
+    g4 = T.TensorType("float32", (False,) * 4)("g")
+    mean = T.mean(x4, axis=(0, 2, 3), keepdims=True)
+    var = T.mean(T.sqr(x4 - mean), axis=(0, 2, 3), keepdims=True)
+    y = (x4 - mean) / T.sqrt(var + np.float32(1e-5))
+    dx = th.grad(T.sum(y * g4), x4)
+    for shape in ((8, 12, 10, 14), (64, 4, 300, 300)):      # the second: too much per channel to hold, turned away
+        f = th.function([x4, g4], _device_outs([y, dx]))
+        eager = th.function([x4, g4], _device_outs([y, dx]))
+        xd = HipArray.from_numpy(rng.standard_normal(shape).astype("float32"))
+        gd = HipArray.from_numpy(rng.standard_normal(shape).astype("float32"))
+        results, graph = f.capture(xd, gd)
+        for replay in range(3):
+            copy_into(HipArray.from_numpy(rng.normal(replay, 2.0, shape).astype("float32")), xd)
+            hip.sync()
+            graph.launch()
+            got = [r.to_numpy() for r in results]
+            want = [r.to_numpy() for r in eager(xd, gd)]
+            for k, (a, b) in enumerate(zip(got, want)):
+                assert np.array_equal(a, b), (shape, replay, k)
