@@ -745,3 +745,20 @@ def test_verify_grad_and_gradient_only_operations():
     np.testing.assert_allclose(g1, vv, rtol=1e-6)                       # 0.5 * 2v
     np.testing.assert_allclose(g2, 3 * vv ** 2 + np.clip(3 * vv, -1, 1) * 2 * vv, rtol=1e-6)
     assert np.array_equal(fwd, 2 * vv)
+
+
+def test_fp_contract_off_gives_the_unfused_float32_arithmetic(monkeypatch):
+    """$THX_FP_CONTRACT=off (read when a kernel is first compiled): a multiply followed by an add is two roundings,
+    as NumPy's float32 arithmetic does them - bit for bit; the default lets the compiler fuse them into one
+    (closer to the exact value, but one expression compiled into two kernels need not fuse alike).  The
+    expressions carry constants no other test uses, so that their kernels are compiled here."""
+    rng = np.random.default_rng(31)
+    x, y, z = T.fmatrix("x"), T.fmatrix("y"), T.fmatrix("z")
+    xv, yv, zv = [rng.standard_normal((97, 130)).astype("float32") for _ in range(3)]
+    f32 = np.float32
+    want = xv * yv + zv * f32(1.2578125) - f32(0.3720703125)
+    want2 = (xv * yv + zv) * yv - xv * zv * f32(3.0791015625)
+    monkeypatch.setenv("THX_FP_CONTRACT", "off")
+    got, got2 = th.function([x, y, z], [x * y + z * f32(1.2578125) - f32(0.3720703125),
+                                        (x * y + z) * y - x * z * f32(3.0791015625)])(xv, yv, zv)
+    assert np.array_equal(got, want) and np.array_equal(got2, want2)

@@ -282,11 +282,19 @@ static uint64_t fnv1a(const std::string& s, uint64_t h) {
   return h;
 }
 
+// $THX_FP_CONTRACT = on | off | fast: how the compiler may fuse a multiply with a following add.  Unset, the
+// compiler's default for device code (fast: across statements) stays.
+static const char* fp_contract() {
+  const char* v = getenv("THX_FP_CONTRACT");
+  if (!v) return "";
+  return !strcmp(v, "on") ? "on" : !strcmp(v, "off") ? "off" : !strcmp(v, "fast") ? "fast" : "";
+}
+
 static std::string source_hash(const std::string& src, const std::string& arch) {
   int maj = 0, min = 0;
   hiprtcVersion(&maj, &min);
   std::string salted = src + "\n//" + arch + "/" + std::to_string(maj) + "." + std::to_string(min) +
-                       (fast_div() ? "/fd" : "");
+                       (fast_div() ? "/fd" : "") + (fp_contract()[0] ? std::string("/c") + fp_contract() : std::string());
   char buf[40];
   snprintf(buf, sizeof buf, "%016llx%016llx", (unsigned long long)fnv1a(salted, 1469598103934665603ULL),
            (unsigned long long)fnv1a(salted, 0x9e3779b97f4a7c15ULL));
@@ -337,6 +345,8 @@ static int compile_source(const std::string& src, const std::string& arch, std::
     opts.push_back("-fno-hip-fp32-correctly-rounded-divide-sqrt");
     opts.push_back("-DTHX_FAST_DIV");
   }
+  const std::string contract = std::string("-ffp-contract=") + fp_contract();
+  if (fp_contract()[0]) opts.push_back(contract.c_str());
   r = hiprtcCompileProgram(prog, (int)opts.size(), opts.data());
   if (r != HIPRTC_SUCCESS) {
     size_t n = 0;
