@@ -1139,3 +1139,28 @@ def test_batch_normalization_with_given_statistics_and_nnet_aliases(dry_run):
     for op, base in ((N.sigmoid_inplace, scal.ScalarSigmoid), (N.softplus_inplace, scal.ScalarSoftplus),
                      (N.ultra_fast_sigmoid_inplace, scal.UltraFastScalarSigmoid)):
         assert isinstance(op.scalar_op, base) and op.destroy_map == {0: [0]} and op(x).type == x.type
+
+
+def test_device_type_value_helpers(dry_run):
+    """HipArrayType: filter_variable / convert_variable (a host variable is moved, a broader broadcast pattern is
+    narrowed), may_share_memory for views of one allocation, value_zeros, get_size, values_eq(_approx)
+    (theano/gpuarray/type.py:204-420)."""
+    from theano_amd.hip.ops import HipArrayType
+    from theano_amd.hip.runtime import HipArray
+    t = HipArrayType("float32", (False, True))
+    for v in (T.fcol(), T.TensorType("float32", (True, True))(), HipArrayType("float32", (True, True))(), t()):
+        assert t.filter_variable(v).type == t
+    own = t()
+    assert t.filter_variable(own) is own and t.convert_variable(T.dmatrix()) is None and t.convert_variable(T.fmatrix()) is None
+    with pytest.raises(TypeError, match="Cannot convert Type"):
+        t.filter_variable(T.fmatrix())
+    assert t.filter_variable(np.ones((2, 1), "float32")).type == t
+    a = HipArray.empty((4, 1), "float32")
+    assert t.may_share_memory(a, a.view((2, 1), (4, 4))) and not t.may_share_memory(a, HipArray.empty((4, 1), "float32"))
+    assert not t.may_share_memory(a, np.zeros(3)) and t.get_size(t.get_shape_info(a)) == 16
+    z = t.value_zeros((3, 1))
+    assert isinstance(z, HipArray) and z.shape == (3, 1) and str(z.dtype) == "float32"
+    assert t.values_eq(a, a) and t.values_eq_approx(a, a) and not t.values_eq(a, z)
+    c = T.TensorType("float32", (True, True))("c")
+    f = th.function([c], t.filter_variable(c) + 1)
+    assert [type(n.op).__name__ for n in f.toposort()][0] == "HostToHip"

@@ -67,6 +67,65 @@ class HipArrayType(Type):
     def as_tensor_variable(self, var):
         return host_from_hip(var)
 
+    # -- the value-level helpers of theano/gpuarray/type.py:260-420; comparisons bring the values to the host
+    @staticmethod
+    def _host(v):
+        return v.to_numpy() if isinstance(v, HipArray) else np.asarray(v)
+
+    @classmethod
+    def values_eq(cls, a, b, force_same_dtype=True):
+        return TensorType.values_eq(cls._host(a), cls._host(b), force_same_dtype)
+
+    @classmethod
+    def values_eq_approx(cls, a, b, rtol=None, atol=None):
+        return TensorType.values_eq_approx(cls._host(a), cls._host(b), rtol, atol)
+
+    @staticmethod
+    def may_share_memory(a, b):
+        """Two device arrays may overlap when they are views of one allocation (``:300-306``)."""
+        return isinstance(a, HipArray) and isinstance(b, HipArray) and a.buffer is b.buffer
+
+    def value_zeros(self, shape):
+        return HipArray.from_numpy(np.zeros(shape, dtype=self.dtype))
+
+    def get_shape_info(self, obj):
+        return obj.shape
+
+    def get_size(self, shape_info):
+        n = np.dtype(self.dtype).itemsize
+        for s in shape_info:
+            n *= int(s)
+        return n
+
+    def convert_variable(self, var):
+        """``var`` under this type's broadcast pattern (a host variable is moved to the device first) when dtype
+        and rank agree and it is at least as broadcastable wherever this type is; None otherwise (``:243-258``)."""
+        vt = var.type
+        if vt == self:
+            return var
+        if (isinstance(vt, (TensorType, HipArrayType)) and vt.dtype == self.dtype and vt.ndim == self.ndim and
+                all(sb == ob or ob for sb, ob in zip(self.broadcastable, vt.broadcastable))):
+            # the pattern is changed on the host-typed variable; the transfers either side of it are cut when
+            # the graph is compiled
+            host = var if isinstance(vt, TensorType) else host_from_hip(var)
+            return as_hip_variable(TensorType(self.dtype, self.broadcastable).convert_variable(host))
+        return None
+
+    def filter_variable(self, other, allow_convert=True):
+        """A symbolic variable (or a value, made a device constant's source) as a variable of this type, or
+        TypeError (``:204-241``)."""
+        if not isinstance(other, Variable):
+            from ..tensor.type import constant
+            other = constant(TensorType(self.dtype, self.broadcastable).filter(other))
+        if other.type == self:
+            return other
+        if allow_convert:
+            conv = self.convert_variable(other)
+            if conv is not None and conv.type == self:
+                return conv
+        raise TypeError("Cannot convert Type %s (of Variable %s) into Type %s. You can try to manually convert %s "
+                        "into a %s." % (other.type, other, self, other, self))
+
 
 class HipArrayVariable(_tensor_py_operators, Variable):
     pass
