@@ -721,6 +721,8 @@ def test_verify_grad_and_gradient_only_operations():
                                                                            keepdims=True), [pts[0]], rng=rng)
     with pytest.raises(TypeError, match="rng"):
         G.verify_grad(T.exp, [pts[0]])
+    from theano_amd.tests import unittest_tools as utt
+    utt.verify_grad(T.tanh, [pts[0]])                 # seeds NumPy's generator itself
     with pytest.raises(TypeError, match="floating point"):
         G.verify_grad(T.exp, [np.arange(4)], rng=rng)
 
