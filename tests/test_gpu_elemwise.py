@@ -139,6 +139,38 @@ def test_sigmoid_thresholds_and_nan_handling():
         assert_parity(g, r, "special values")
 
 
+def test_division_operator_on_integer_tensors_is_numpy_true_division():
+    """`x / y` on integer tensors is true division with a floatX result (``theano/tensor/var.py:199-206``,
+    ``theano/scalar/basic.py:1891-1915``: ``(double)x / y`` rounded to floatX), never the truncating one.
+    The expectation is NumPy's own `/`, not the oracle's walk over this package's graph."""
+    rng = np.random.default_rng(77)
+    i, j, b = T.imatrix("i"), T.imatrix("j"), T.bmatrix("b")
+    iv = rng.integers(-2 ** 20, 2 ** 20, (61, 130)).astype("int32")
+    jv = rng.integers(1, 1000, (61, 130)).astype("int32") * rng.choice([-1, 1], (61, 130)).astype("int32")
+    bv = rng.integers(-128, 128, (61, 130)).astype("int8")
+    bv[bv == 0] = 5
+    f = th.function([i, j, b], [i / j, b / 2, 2 / i, b / b, i / b, 7 / b, (i / j) * 2])
+    iv_nz = np.where(iv == 0, 3, iv).astype("int32")
+    got = f(iv_nz, jv, bv)
+    want = [iv_nz / jv, bv / 2, 2 / iv_nz, bv / bv, iv_nz / bv, 7 / bv, (iv_nz / jv) * 2]
+    for k, (g, w) in enumerate(zip(got, want)):
+        assert g.dtype == np.dtype(th.config.floatX), (k, g.dtype)
+        assert_parity(g, w.astype(th.config.floatX), "true division %d" % k)
+    assert not np.array_equal(got[0], (iv_nz // jv).astype(got[0].dtype))      # it is not the truncating division
+    q, r = th.function([i, j], list(divmod(i, j)))(iv, jv)
+    wq, wr = np.divmod(iv, jv)
+    assert q.dtype == r.dtype == np.int32 and np.array_equal(q, wq) and np.array_equal(r, wr)
+
+
+def test_round_defaults_to_half_to_even_like_numpy():
+    """``theano/tensor/basic.py:2175-2192``: `round(a)` and `a.round()` round halves to even."""
+    x = T.fvector("x")
+    xv = np.array([-2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 3.5, 0.49999997, 8388609.0, 1.25, -7.75], "float32")
+    got = th.function([x], [T.round(x), x.round(), T.iround(x)])(xv)
+    assert np.array_equal(got[0], np.round(xv)) and np.array_equal(got[1], np.round(xv))
+    assert got[2].dtype == np.int64 and np.array_equal(got[2], np.round(xv).astype("int64"))
+
+
 def test_round_half_away_from_zero_is_c_round_on_the_device():
     """theano/scalar/basic.py:2686 emits C round(): halves away from zero, and nothing like
     floor(x + 0.5) at 0.49999997 or at odd integers from 2**23 up.  Bit-exact against the oracle

@@ -42,7 +42,8 @@ def test_python_literals_pick_the_smallest_dtype():
     f = T.fmatrix()
     assert (f + 1e-5).type.dtype == "float32"  # floatX = float32 keeps float literals narrow
     assert (f * 2).type.dtype == "float32"
-    assert (x / 2).type.dtype == "int32"       # int / int is integer division under int_division='int'
+    assert (x / 2).type.dtype == "float32"     # `/` is true division: floatX for two integer operands (var.py:199-200)
+    assert x.__div__(2).type.dtype == "int32"  # Python 2's `/`: integer division under int_division='int'
     assert T.true_div(x, 2).type.dtype == "float32"
 
 

@@ -1,0 +1,269 @@
+"""What Python's operators and the tensor methods build: the operation and the result dtype of each,
+as the reference's ``_tensor_py_operators`` (``theano/tensor/var.py:38-830``) and its
+``test_arithmetic_cast`` (``theano/tensor/tests/test_basic.py:6919-7060``) fix them.
+
+The expectations are written from the cited lines, not taken from this package: the operator table
+names the operation each ``__op__`` calls there, the dtype rule is the reference test's own comparison
+with NumPy's result types."""
+import operator
+
+import numpy as np
+import pytest
+
+import theano_amd as th
+from theano_amd import config
+from theano_amd import scalar as scal
+from theano_amd import tensor as T
+from theano_amd.tensor.elemwise import CAReduce, DimShuffle, Elemwise
+
+REAL = ["bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64", "float16", "float32", "float64"]
+INTS = REAL[:9]
+NUMERIC = REAL[1:] + ["complex64", "complex128"]          # get_numeric_types(with_complex=True), test_basic.py:140-190
+
+
+def op_name(v):
+    """Name of the scalar operation of the Elemwise that computes ``v``."""
+    assert isinstance(v.owner.op, Elemwise), v.owner.op
+    return v.owner.op.scalar_op.name
+
+
+# operator -> the tensor function var.py calls for it (line cited), for a tensor on the left and on the right
+BINARY = [
+    (operator.add, "add", "var.py:129-145, 234-235"),
+    (operator.sub, "sub", "var.py:147-153, 237-238"),
+    (operator.mul, "mul", "var.py:155-161, 240-241"),
+    (operator.truediv, "true_div", "var.py:199-200, 205-206 (the later definitions replace `__truediv__ = __div__`)"),
+    (operator.floordiv, "int_div", "var.py:202-203, 208-209"),
+    (operator.mod, "mod", "var.py:184-194, 246-247"),
+    (operator.pow, "pow", "var.py:176-182, 252-253"),
+]
+BITWISE = [(operator.and_, "and_", "var.py:101-102, 110-111"), (operator.or_, "or_", "var.py:104-105, 113-114"),
+           (operator.xor, "xor", "var.py:107-108, 116-117")]
+COMPARE = [(operator.lt, "lt"), (operator.le, "le"), (operator.gt, "gt"), (operator.ge, "ge")]   # var.py:55-73
+
+
+@pytest.mark.parametrize("left,right", [("int32", "int32"), ("int8", "float32"), ("float32", "float32"),
+                                        ("float64", "int16"), ("uint8", "uint8")])
+def test_binary_operators_build_the_reference_operations(left, right):
+    a, b = T.matrix(dtype=left), T.matrix(dtype=right)
+    for fn, name, _where in BINARY:
+        assert op_name(fn(a, b)) == name, (fn, name)
+        # a Python number on either side: the reflected method of the variable runs
+        assert op_name(fn(a, 3)) == name and op_name(fn(3, a)) == name, (fn, name)
+        assert fn(3, a).owner.inputs[1].owner.inputs[0] is a if fn(3, a).owner.inputs[1].owner else True
+
+
+def test_division_operator_is_true_division_on_integers():
+    """``theano/tensor/var.py:199-206``: `/` and its reflection are true_div whatever the operand types; the
+    result of two discrete operands is floatX (``TrueDiv.output_types``, ``theano/scalar/basic.py:1891-1897``).
+    Only Python 2's ``__div__`` goes through ``div_proxy`` (``var.py:162-174, 243-244``)."""
+    for floatX in ("float32", "float64"):
+        with config.change_flags(floatX=floatX):
+            for dt in INTS:
+                x = T.matrix(dtype=dt)
+                for v in (x / x, x / 2, 2 / x, x / np.int8(2), x.__truediv__(x), x.__rtruediv__(2)):
+                    assert op_name(v) == "true_div" and v.dtype == floatX, (dt, v.dtype)
+                # the literal 2 is an int8 constant (the smallest dtype that holds it)
+                assert op_name(x // 2) == "int_div" and (x // 2).dtype == str(np.result_type(dt, "int8"))
+            x = T.imatrix()
+            assert (x / T.fmatrix()).dtype == "float64" and (x / T.dmatrix()).dtype == "float64"
+            assert (T.bmatrix() / T.fmatrix()).dtype == "float32"
+    x = T.imatrix()
+    with config.change_flags(int_division="int"):
+        assert op_name(x.__div__(x)) == "int_div" and x.__div__(x).dtype == "int32"
+        assert op_name(x.__rdiv__(2)) == "int_div" and op_name(x.__div__(T.fmatrix())) == "true_div"
+    with config.change_flags(int_division="floatX"):
+        assert op_name(x.__div__(x)) == "true_div" and x.__div__(x).dtype == config.floatX
+    with config.change_flags(int_division="raise"):
+        with pytest.raises(scal.IntegerDivisionError):
+            x.__div__(x)
+        assert op_name(x / x) == "true_div"          # `/` itself never consults the flag
+
+
+def test_scalar_variables_divide_by_operand_type():
+    """``theano/scalar/basic.py:755-759, 780-781``: on Scalar variables both ``__truediv__`` and ``__div__`` are
+    ``div_proxy``: integer division for two discrete operands under int_division='int'."""
+    i, j, f = scal.int32("i"), scal.int8("j"), scal.float32("f")
+    with config.change_flags(int_division="int"):
+        assert (i / j).owner.op is scal.int_div and (i / j).type.dtype == "int32"
+        assert (i / f).owner.op is scal.true_div and (i / f).type.dtype == "float64"
+    with config.change_flags(int_division="floatX"):
+        assert (i / j).owner.op is scal.true_div and (i / j).type.dtype == config.floatX
+    with config.change_flags(int_division="raise"), pytest.raises(scal.IntegerDivisionError):
+        i / j
+    assert (i // j).owner.op is scal.int_div and (i % j).owner.op is scal.mod
+
+
+def test_bitwise_comparison_and_unary_operators():
+    a, b = T.imatrix(), T.bmatrix()
+    for fn, name, _where in BITWISE:
+        assert op_name(fn(a, b)) == name and fn(a, b).dtype == "int32"
+        assert op_name(fn(a, 5)) == name and op_name(fn(5, a)) == name
+    for fn, name in COMPARE:
+        v = fn(a, b)
+        assert op_name(v) == name and v.dtype == "bool"
+        with pytest.raises(TypeError, match="boolean operations"):       # var.py:79-95: `a < b < c` must fail
+            bool(v)
+    assert bool(a + b)                                                     # any other variable is truthy
+    assert op_name(-a) == "neg" and op_name(abs(a)) == "abs_" and op_name(~a) == "invert"     # var.py:40-44, 98-99
+    f = T.fmatrix()
+    assert op_name(a.astype("float32")).startswith("convert_to_") or "Cast" in str(a.astype("float32").owner.op)
+    with pytest.raises(Exception):
+        ~f                                                                 # bit operations need integers
+    q, r = divmod(a, b)                                                    # var.py:196-197 -> floor_div, mod_check
+    assert op_name(q) == "int_div" and op_name(r) == "mod"
+    q, r = divmod(7, a)                                                    # var.py:249-250
+    assert op_name(q) == "int_div" and op_name(r) == "mod"
+    assert op_name(a.__ceil__() if False else f.__ceil__()) == "ceil" and op_name(f.__floor__()) == "floor"
+    assert op_name(f.__trunc__()) == "trunc"                               # var.py:255-262
+
+
+def test_mod_refuses_complex_operands_when_the_graph_is_built():
+    """``mod_check``, ``theano/tensor/basic.py:3622-3629``: ComplexError (a NotImplementedError) from `%` and divmod."""
+    z, x = T.cmatrix(), T.fmatrix()
+    assert issubclass(scal.ComplexError, NotImplementedError)
+    for bad in (lambda: z % x, lambda: x % z, lambda: z % 2, lambda: divmod(z, x)):
+        with pytest.raises(scal.ComplexError):
+            bad()
+    zs = scal.complex64("z")
+    with pytest.raises(scal.ComplexError):
+        zs % scal.float32("x")
+
+
+def test_numpy_values_on_the_left_reach_the_reflected_operators():
+    """``__array_priority__ = 1000`` (``theano/tensor/var.py:733``): NumPy defers to the variable instead of
+    broadcasting over it."""
+    x = T.fmatrix()
+    for left in (np.float32(2), np.arange(3, dtype="float32"), np.int64(3)):
+        for fn, name, _where in BINARY[:5]:
+            v = fn(left, x)
+            assert isinstance(v, T.TensorVariable) and op_name(v) == name
+
+
+METHODS = [  # method, module-level function it must equal (var.py:390-470, 637-780)
+    "arccos", "arccosh", "arcsin", "arcsinh", "arctan", "arctanh", "ceil", "cos", "cosh", "deg2rad", "exp", "exp2",
+    "expm1", "floor", "log", "log10", "log1p", "log2", "rad2deg", "sin", "sinh", "sqrt", "tan", "tanh", "trunc"]
+
+
+def test_elementwise_methods_build_the_module_level_operations():
+    x = T.fmatrix()
+    for m in METHODS:
+        v, w = getattr(x, m)(), getattr(T, m)(x)
+        assert v.owner.op == w.owner.op and v.dtype == w.dtype, m
+    assert x.clip(0, 1).owner.op == T.clip(x, 0, 1).owner.op
+    assert op_name(x.round()) == "round_half_to_even" and op_name(x.round("half_away_from_zero")) == "round_half_away_from_zero"
+    z = T.cmatrix()
+    assert op_name(z.real) == "real" and op_name(z.imag) == "imag" and op_name(z.conj()) == "conj"
+    assert x.conj() is x or op_name(x.conj()) == "conj"
+
+
+def test_reduction_methods_and_their_result_dtypes():
+    """var.py:637-692; the dtype tables of ``theano/tensor/elemwise.py:1721-1780``."""
+    i8, f32, f16 = T.bmatrix(), T.fmatrix(), T.hmatrix() if hasattr(T, "hmatrix") else T.matrix(dtype="float16")
+    for meth in ("sum", "prod"):
+        assert getattr(i8, meth)().dtype == "int64" and getattr(i8, meth)(axis=0).dtype == "int64"
+        assert getattr(T.matrix(dtype="uint16"), meth)().dtype == "uint64"
+        assert getattr(f32, meth)(axis=1).dtype == "float32" and getattr(f32, meth)(axis=1).owner.op.acc_dtype == "float64"
+        assert getattr(f16, meth)().dtype == "float16" and getattr(f16, meth)().owner.op.acc_dtype == "float32"
+        assert getattr(f32, meth)(dtype="float64").dtype == "float64"
+    assert f32.mean(axis=0).dtype == "float32" and i8.mean().dtype == "float64" and f16.mean().dtype == "float16"
+    assert f32.max(axis=1).dtype == "float32" and i8.min().dtype == "int8"
+    assert i8.any().dtype == "bool" and f32.all(axis=0).dtype == "bool"
+    assert f32.argmax(axis=1).dtype == "int64" and f32.argmin().dtype == "int64"
+    assert f32.var(axis=0).dtype == "float32" and f32.std().dtype == "float32"
+    for meth in ("sum", "prod", "max", "min", "mean", "any", "all", "argmax"):
+        kept = getattr(f32, meth)(axis=1, keepdims=True)
+        assert kept.type.broadcastable == (False, True), meth
+        assert getattr(f32, meth)(axis=1).type.broadcastable == (False,), meth
+    assert f32.norm(2).ndim == 0 and f32.norm(1, axis=0).ndim == 1 and f32.ptp(axis=1).ndim == 1
+    with pytest.raises(NotImplementedError):
+        f32.norm(0)
+
+
+def test_view_methods():
+    """var.py:264-420: T / transpose / dimshuffle / flatten / ravel / reshape / swapaxes / squeeze build views."""
+    x = T.ftensor3()
+    assert isinstance(x.T.owner.op, DimShuffle) and x.T.owner.op.new_order == (2, 1, 0)
+    assert x.transpose().owner.op.new_order == (2, 1, 0)
+    assert x.transpose(1, 0, 2).owner.op.new_order == (1, 0, 2) and x.transpose((1, 2, 0)).owner.op.new_order == (1, 2, 0)
+    assert x.dimshuffle(0, "x", 2, 1).type.broadcastable == (False, True, False, False)
+    assert x.dimshuffle((2, 0, 1)).owner.op.new_order == (2, 0, 1)
+    assert x.swapaxes(0, 2).owner.op.new_order == (2, 1, 0)
+    assert x.flatten().ndim == 1 and x.flatten(2).ndim == 2 and x.ravel().ndim == 1
+    assert x.reshape((2, -1)).ndim == 2
+    r = T.frow()
+    assert r.squeeze().ndim == 1
+    assert x.ndim == 3 and x.dtype == "float32" and x.broadcastable == (False, False, False)
+    assert x.zeros_like().dtype == "float32" and x.ones_like(dtype="int8").dtype == "int8"
+    # Second takes its result dtype from the value (transfer_type(1), theano/scalar/basic.py:2264-2270)
+    assert x.fill(3).dtype == "int8" and x.fill(3).broadcastable == x.broadcastable and x.fill(1.5).dtype == "float32"
+    c = x.copy(name="again")
+    assert c.name == "again" and c.type == x.type
+    with pytest.raises(TypeError):
+        iter(x)                                                            # var.py:605-613
+
+
+# --------------------------------------------------------------------------
+# test_arithmetic_cast (test_basic.py:6919-7060): result dtypes of + - * / // over every pair of numeric
+# dtypes and every mix of 0-d and 1-d operands, compared with NumPy's, under cast_policy 'numpy+floatX'.
+def _make(kind, dtype):
+    if kind == "scalar":
+        return T.scalar(dtype=dtype), np.array(1, dtype=dtype)
+    if kind == "array":
+        return T.vector(dtype=dtype), np.array([1], dtype=dtype)
+    return scal.Scalar(dtype)(), np.array(1, dtype=dtype)
+
+
+COMBOS = [("scalar", "scalar"), ("array", "array"), ("scalar", "array"), ("array", "scalar"), ("i_scalar", "i_scalar")]
+
+
+@pytest.mark.parametrize("floatX", ["float32", "float64"])
+@pytest.mark.parametrize("fn", [operator.add, operator.sub, operator.mul, operator.truediv, operator.floordiv],
+                         ids=["add", "sub", "mul", "div", "floordiv"])
+def test_arithmetic_cast(fn, floatX):
+    checked = 0
+    with config.change_flags(cast_policy="numpy+floatX", floatX=floatX, int_division="int"):
+        for a_type in NUMERIC:
+            for b_type in NUMERIC:
+                if fn is operator.floordiv and ("complex" in a_type or "complex" in b_type):
+                    continue       # NumPy no longer defines floor division of complex numbers: nothing to compare with
+                both_discrete = a_type in INTS and b_type in INTS
+                for combo in COMBOS:
+                    (ta, na), (tb, nb) = _make(combo[0], a_type), _make(combo[1], b_type)
+                    if fn is operator.sub and na.dtype == nb.dtype == np.bool_:
+                        continue
+                    got = fn(ta, tb).type.dtype
+                    checked += 1
+                    if fn is operator.truediv and both_discrete:
+                        if combo[0] == "i_scalar":
+                            # Scalar variables: div_proxy -> int_div under int_division='int' (scalar/basic.py:755-759)
+                            assert got == scal.upcast(a_type, b_type), (a_type, b_type, combo, got)
+                        else:
+                            # tensors: true_div of two discrete operands is floatX (scalar/basic.py:1891-1897)
+                            assert got == floatX, (a_type, b_type, combo, got)
+                        continue
+                    wanted = scal.upcast(str(fn(na, nb).dtype), str(fn(nb, na).dtype))
+                    if got == wanted:
+                        continue
+                    if floatX == "float32" and "float64" not in (a_type, b_type) and wanted == "float64":
+                        assert got == "float32", (a_type, b_type, combo, got)       # floatX is kept
+                        continue
+                    raise AssertionError("%s of %s and %s as %s: %s, NumPy gives %s" % (
+                        fn.__name__, a_type, b_type, combo, got, wanted))
+    assert checked >= 600
+
+
+def test_numpy_floatx_policy_for_python_literals():
+    """``NumpyAutocaster`` (``theano/scalar/basic.py:170-180``): under 'numpy+floatX' a Python float becomes floatX,
+    a NumPy float64 stays; under 'numpy' NumPy decides; `upcast` narrows only what promotion widened
+    (``:59-87``)."""
+    with config.change_flags(cast_policy="numpy+floatX", floatX="float32"):
+        assert scal.convert(1.1).dtype == np.float32 and scal.convert(np.float64(1.1)).dtype == np.float64
+        assert scal.convert(3).dtype == np.int64
+        assert scal.upcast("int32", "float32") == "float32" and scal.upcast("int32", "float64") == "float64"
+        assert scal.upcast("int64", "int32") == "int64" and scal.upcast("complex64", "int32") == "complex128"
+    with config.change_flags(cast_policy="numpy", floatX="float32"):
+        assert scal.convert(1.1).dtype == np.float64 and scal.upcast("int32", "float32") == "float64"
+    with config.change_flags(cast_policy="custom", floatX="float32"):
+        assert scal.convert(1.1).dtype == np.float32 and scal.convert(3).dtype == np.int8
+        assert scal.upcast("int32", "float32") == "float64"

@@ -51,16 +51,29 @@ def compute_ctype(dtype):
 
 
 def upcast(dtype, *dtypes):
-    """Result dtype of mixing the given dtypes: NumPy array promotion
-    (``theano/scalar/basic.py:59-87`` with cast_policy 'custom')."""
-    z = np.zeros((), dtype=dtype)
-    for dt in dtypes:
+    """Result dtype of mixing the given dtypes: NumPy array promotion.  Under cast_policy
+    'numpy+floatX' a float64 (float32) that NumPy's promotion alone produced - no operand was that
+    wide - is narrowed to a float32 (float16) floatX (``theano/scalar/basic.py:59-87``)."""
+    names = [str(np.dtype(dt)) for dt in (dtype,) + dtypes]
+    z = np.zeros((), dtype=names[0])
+    for dt in names[1:]:
         z = z + np.zeros((), dtype=dt)
-    return str(z.dtype)
+    rval = str(z.dtype)
+    if config.cast_policy == "numpy+floatX":
+        if config.floatX == "float32" and rval == "float64" and "float64" not in names:
+            return "float32"
+        if (config.floatX == "float16" and rval in ("float64", "float32") and "float64" not in names and
+                "float32" not in names):
+            return "float16"
+    return rval
 
 
 class IntegerDivisionError(Exception):
     pass
+
+
+class ComplexError(NotImplementedError):
+    """An operation that complex numbers do not have (``theano/scalar/basic.py:43-48``)."""
 
 
 # --------------------------------------------------------------------------
@@ -159,7 +172,7 @@ class _scalar_py_operators(object):
     def __truediv__(self, o): return div_proxy(self, o)
     __div__ = __truediv__
     def __floordiv__(self, o): return int_div(self, o)
-    def __mod__(self, o): return mod(self, o)
+    def __mod__(self, o): return mod_check(self, o)
     def __pow__(self, o): return pow(self, o)
     def __radd__(self, o): return add(o, self)
     def __rsub__(self, o): return sub(o, self)
@@ -200,9 +213,14 @@ Scalar.Constant = ScalarConstant
 
 def _autocast(x):
     """dtype chosen for a Python literal (``NumpyAutocaster``,
-    ``theano/scalar/basic.py:132-214``, cast_policy 'custom')."""
+    ``theano/scalar/basic.py:132-214``).  cast_policy 'numpy' takes NumPy's choice, 'numpy+floatX' too except
+    that a Python float becomes floatX; the rest of the function is the 'custom' policy."""
     if isinstance(x, (bool, np.bool_)):
         return np.asarray(x, dtype="bool")
+    if config.cast_policy in ("numpy", "numpy+floatX"):
+        if config.cast_policy == "numpy+floatX" and isinstance(x, float) and not hasattr(x, "dtype"):
+            return np.asarray(x, dtype=config.floatX)
+        return np.asarray(x)
     if isinstance(x, (int, np.integer)) and not hasattr(x, "dtype"):
         for dt in int_dtypes:
             try:
@@ -863,7 +881,7 @@ class IntDiv(BinaryScalarOp):
         (z,) = outputs
         t = upcast(*[i.type.dtype for i in node.inputs])
         if t in complex_dtypes:
-            raise TypeError("floor division is not defined for complex numbers (theano/scalar/basic.py:1947-1949)")
+            raise ComplexError("floor division (//) is not defined for complex numbers (theano/scalar/basic.py:1947-1949)")
         if t in discrete_dtypes:
             d = lambda a, b: "(%s / %s)" % (a, b)
             m = lambda a, b: "(%s %% %s)" % (a, b)
@@ -900,7 +918,7 @@ class Mod(BinaryScalarOp):
         (z,) = outputs
         t = upcast(*[i.type.dtype for i in node.inputs])
         if t in complex_dtypes:
-            raise TypeError("modulo is not defined for complex numbers (theano/scalar/basic.py:2050-2052)")
+            raise ComplexError("the mod operator (%) is not defined for complex numbers (theano/scalar/basic.py:2050-2052)")
         if t in discrete_dtypes:
             m = lambda a, b: "(%s %% %s)" % (a, b)
             zero = "%s = 0;" % z
@@ -925,6 +943,15 @@ class Mod(BinaryScalarOp):
 
 
 mod = Mod(upcast_out, name="mod")
+
+
+def mod_check(x, y):
+    """``x % y`` of the operators: refuses complex operands when the graph is built
+    (``theano/scalar/basic.py:2038-2045``)."""
+    x, y = as_scalar(x), as_scalar(y)
+    if x.type.dtype in complex_dtypes or y.type.dtype in complex_dtypes:
+        raise ComplexError("the mod operator (%) is not defined for complex numbers (theano/scalar/basic.py:2050-2052)")
+    return mod(x, y)
 
 
 class Pow(BinaryScalarOp):

@@ -105,12 +105,15 @@ def ones_like(model, dtype=None):
     return fill(model, constant(1, dtype=dtype))
 
 
-def iround(a, mode="half_away_from_zero"):
+def iround(a, mode=None):
     """``cast(round(a, mode), 'int64')`` (``theano/tensor/basic.py:2168-2171``)."""
     return cast(round(a, mode), "int64")
 
 
-def round(a, mode="half_away_from_zero"):
+def round(a, mode=None):
+    """Rounding of halves to even (the default, NumPy's) or away from zero (``theano/tensor/basic.py:2175-2192``)."""
+    if mode is None:
+        mode = "half_to_even"
     if mode == "half_away_from_zero":
         return round_half_away_from_zero(a)
     if mode == "half_to_even":
@@ -372,9 +375,18 @@ def Shape_i(i):
     return ShapeFloat(i, "int64")
 
 
+def mod_check(x, y):
+    """``x % y`` of the operators: complex operands are refused when the graph is built
+    (``theano/tensor/basic.py:3622-3629``)."""
+    if as_tensor_variable(x).type.dtype in scal.complex_dtypes or as_tensor_variable(y).type.dtype in scal.complex_dtypes:
+        raise scal.ComplexError("the mod operator (%) is not defined for complex numbers "
+                                "(theano/scalar/basic.py:2050-2052)")
+    return mod(x, y)
+
+
 def divmod(x, y):
     """Elementwise ``(x // y, x % y)`` (``theano/tensor/basic.py:3562-3564``)."""
-    return int_div(x, y), mod(x, y)
+    return int_div(x, y), mod_check(x, y)
 
 
 def squeeze(x):

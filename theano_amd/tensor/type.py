@@ -151,6 +151,9 @@ class _tensor_py_operators(object):
     dtype = property(lambda self: self.type.dtype)
     ndim = property(lambda self: self.type.ndim)
     broadcastable = property(lambda self: self.type.broadcastable)
+    # `numpy_value * variable` reaches __rmul__ instead of NumPy trying to broadcast over the variable
+    # (theano/tensor/var.py:733)
+    __array_priority__ = 1000
 
     def _b(self):
         from . import basic
@@ -188,16 +191,18 @@ class _tensor_py_operators(object):
     def __add__(self, o): return self._b().add(self, o)
     def __sub__(self, o): return self._b().sub(self, o)
     def __mul__(self, o): return self._b().mul(self, o)
-    def __truediv__(self, o): return self._b().div_proxy(self, o)
-    __div__ = __truediv__
+    # `/` is true division whatever the operand types; only Python 2's `__div__` chose between the
+    # two divisions by type (theano/tensor/var.py:162-174, 199-209)
+    def __truediv__(self, o): return self._b().true_div(self, o)
+    def __div__(self, o): return self._b().div_proxy(self, o)
     def __floordiv__(self, o): return self._b().int_div(self, o)
-    def __mod__(self, o): return self._b().mod(self, o)
+    def __mod__(self, o): return self._b().mod_check(self, o)
     def __pow__(self, o): return self._b().pow(self, o)
     def __radd__(self, o): return self._b().add(o, self)
     def __rsub__(self, o): return self._b().sub(o, self)
     def __rmul__(self, o): return self._b().mul(o, self)
-    def __rtruediv__(self, o): return self._b().div_proxy(o, self)
-    __rdiv__ = __rtruediv__
+    def __rtruediv__(self, o): return self._b().true_div(o, self)
+    def __rdiv__(self, o): return self._b().div_proxy(o, self)
     def __rfloordiv__(self, o): return self._b().int_div(o, self)
     def __rmod__(self, o): return self._b().mod(o, self)
     def __rpow__(self, o): return self._b().pow(o, self)
@@ -326,7 +331,7 @@ class _tensor_py_operators(object):
         return self._b().clip(self, a_min, a_max)
 
     def round(self, mode=None):
-        return self._b().round(self, mode) if mode is not None else self._b().round(self)
+        return self._b().round(self, mode)
 
     def copy(self, name=None):
         out = self._b().tensor_copy(self)
