@@ -1187,3 +1187,32 @@ def test_unittest_tools_seed_and_compare(monkeypatch):
         utt.assert_allclose(a, a + np.float32(1e-2))
     with pytest.raises(utt.WrongValue):
         utt.assert_allclose(a, a[:3])
+
+
+def test_shape_only_nodes_rerun_when_list_arguments_change_length(dry_run):
+    """The extent `mean` divides by is kept between calls with equal argument shapes; the shapes are those of
+    the filtered values, so two Python lists of different lengths (which have no `.shape` themselves) count as
+    different and the extent is read again."""
+    from theano_amd.tensor.basic import ShapeFloat
+    x = T.fvector("x")
+    f = th.function([x], T.mean(x))
+    runs = []
+    nodes = [n for n in f.nodes if isinstance(n.op, ShapeFloat)]
+    assert nodes
+    for k, th_ in enumerate(f.thunks):
+        if th_[1] in nodes:
+            perform = th_[0]
+
+            def counted(node, ins, outs, _p=perform):
+                runs.append(tuple(np.shape(i) for i in ins))
+                return _p(node, ins, outs)
+            f.thunks[k] = (counted,) + tuple(th_[1:])
+    f([1, 2, 3])
+    f([1, 2, 3])
+    assert runs == [((3,),)]
+    f([1, 2, 3, 4])
+    assert runs == [((3,),), ((4,),)]
+    f(np.zeros(4, "float32"))
+    assert len(runs) == 2
+    f(np.zeros(5, "float32"))
+    assert len(runs) == 3

@@ -266,6 +266,7 @@ class Function(object):
                                 [self.storage[o] for o in node.outputs], node in static,
                                 self.release[len(self.thunks)]))
         self._static_key = None
+        self._input_cells = [self.storage[v] for v in self.fgraph.inputs]
         self._constants_ready = False
         self._HipArray = HipArray
         self._last_shape = {}
@@ -358,8 +359,10 @@ class Function(object):
 
     def _run(self, args):
         HipArray = self._HipArray
-        key = tuple([a.shape for a in args if hasattr(a, "shape")])
-        same = key == self._static_key
+        # the shapes of the values the nodes will read (the filtered arguments: a list has become an array),
+        # never those of the raw arguments; a value without a shape never matches
+        key = tuple([getattr(c[0], "shape", None) for c in self._input_cells])
+        same = key == self._static_key and None not in key
         self._static_key = None                 # stays unset if a node raises half-way
         for perform, node, ins, outs, static, release in self.thunks:
             if static and same:
