@@ -13,8 +13,11 @@
  * Every function is plain C: pointers, sizes and PODs. All functions return
  * THX_OK (0) or an error code; thx_last_error() gives the message of the last
  * failure on the calling thread. One device, one in-order stream, no internal
- * threads. Device results are reproducible: data is never accumulated with
- * atomics (split reductions merge their partial results in a fixed order).
+ * threads. Device results are reproducible: values are never accumulated with
+ * atomics (split reductions merge their partial results in a fixed order).  The
+ * one atomic operation in the library counts arrivals: a split any / all
+ * reduction adds its flags as 16-bit counts to a 64-bit word per result, and
+ * counts do not depend on the order of arrival.
  */
 #ifndef THX_HIP_H
 #define THX_HIP_H
@@ -153,7 +156,9 @@ int thx_elemwise_free(thx_elemwise* e);
  * thx_elemwise_reduce_call = thx_elemwise_call plus that reduction into `red_outs` (C-contiguous,
  * one element per index of the last dimension): inside the same kernel where the access plan allows
  * it (permuted reads through LDS tiles), else by a reduction launched on the stored results.
- * Asynchronous; same error behaviour as thx_elemwise_call. */
+ * Asynchronous; same error behaviour as thx_elemwise_call.
+ * `e` borrows `r`: the reduction must stay alive until thx_elemwise_free(e) or until it is
+ * detached with thx_elemwise_attach_reduce(e, NULL, NULL). */
 int thx_elemwise_attach_reduce(thx_elemwise* e, thx_reduce* r, const int32_t* which_outputs);
 int thx_elemwise_reduce_call(thx_elemwise* e, const thx_array* ins, const thx_array* outs,
                              const thx_array* red_outs, int flags);
@@ -272,6 +277,15 @@ int thx_capture_begin(void);
 int thx_capture_end(thx_graph** out);
 int thx_graph_launch(thx_graph* g);
 int thx_graph_free(thx_graph* g);
+
+/* Partial results of split reductions live in one scratch buffer that grows on demand (8 MiB at
+ * first).  While a recorded sequence is alive the buffer it was recorded with is kept, also after
+ * a later call has needed a larger one; growing it inside a recording is refused.
+ * thx_scratch_reserve sizes the buffer up-front; thx_scratch_state reports the current size, the
+ * number of superseded buffers still held for recorded sequences, and the recorded sequences alive.
+ * No counterpart in the reference (its reductions take no workspace). */
+int thx_scratch_reserve(size_t nbytes);
+int thx_scratch_state(int64_t* nbytes, int64_t* superseded_held, int64_t* graphs_alive);
 
 /* Whole-region timing: events recorded on the library's stream. */
 int thx_timer_start(void);

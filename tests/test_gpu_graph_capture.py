@@ -90,3 +90,41 @@ def test_chain_nodes_replay_too_held_and_turned_away():
             want = [r.to_numpy() for r in eager(xd, gd)]
             for k, (a, b) in enumerate(zip(got, want)):
                 assert np.array_equal(a, b), (shape, replay, k)
+
+
+def test_a_recording_keeps_its_scratch_buffer_and_its_operands_alive():
+    """A recorded split reduction holds the address of the partial-result buffer: when a later call needs a larger
+    buffer the old one is set aside until the last recording is gone, never freed under it; growing the buffer
+    inside a recording is refused.  The graph also holds the argument arrays and the shared variables' values of
+    the moment, so dropping the caller's references (or a set_value) leaves replays reading live memory."""
+    import gc
+    from theano_amd.hip import runtime as R
+    rng = np.random.default_rng(12)
+    x = T.fmatrix("x")
+    w = th.shared(rng.standard_normal((1, 700)).astype("float32"), broadcastable=(True, False))
+    f = th.function([x], _device_outs([T.sum(x * w), T.sum(x + w, axis=0)]))     # both split into slices
+    xv = rng.standard_normal((5000, 700)).astype("float32")
+    wv = w.get_value()
+    xd = HipArray.from_numpy(xv)
+    results, graph = f.capture(xd)
+    want = [r.to_numpy() for r in results]
+    size0, held0, alive0 = R.scratch_state()
+    assert alive0 >= 1 and size0 >= 8 << 20
+    R.scratch_reserve(size0 + (4 << 20))                   # what an eager call with more partial results does
+    size1, held1, alive1 = R.scratch_state()
+    assert size1 >= size0 + (4 << 20) and held1 == held0 + 1 and alive1 == alive0
+    del xd
+    w.set_value(np.zeros((1, 700), "float32"))
+    gc.collect()
+    junk = [HipArray.from_numpy(np.full((5000, 700), 7, "float32")) for _ in range(3)]    # would reuse freed blocks
+    graph.launch()
+    got = [r.to_numpy() for r in results]
+    for g, wnt in zip(got, want):
+        assert np.array_equal(g, wnt)
+    assert np.allclose(got[0], (xv.astype("float64") * wv).sum(), rtol=1e-6)
+    with pytest.raises(ValueError, match="recording"):
+        with hip.capture():
+            R.scratch_reserve(size1 + (16 << 20))
+    del graph, junk
+    gc.collect()
+    assert R.scratch_state()[1:] == (0, alive0 - 1)

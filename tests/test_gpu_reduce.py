@@ -313,6 +313,37 @@ def test_sums_over_results_of_a_reduction_over_the_same_elements_share_its_pass(
             np.testing.assert_allclose(a, b, rtol=2e-5 if dtype == "float32" else 1e-11, atol=2e-5 if dtype == "float32" else 1e-11)
 
 
+@pytest.mark.parametrize("ratio", [1e3, 1e4])
+def test_hoisted_sums_keep_their_accuracy_when_the_mean_dwarfs_the_spread(ratio):
+    """sum(g * (x - mean)) run as sum(g * x) - mean * sum(g): the expanded terms are `ratio` times larger than the
+    original ones, so the products must be formed without a float32 rounding (2**-24 |g x| per term would show as
+    1e-4 ... 1e-2 of the result here).  Checked against NumPy in float64 with the mean as float32 data (what the
+    reference's graph feeds its second reduction) and with the unrounded mean: the device has to be within the
+    float32 bar of one of them, per channel."""
+    from theano_amd.hip import HipCAReduce
+    rng = np.random.default_rng(int(ratio))
+    for shape, axes in (((7, 24, 9, 11), (0, 2, 3)), ((2000, 48), (0,))):
+        nd = len(shape)
+        tt = T.TensorType("float32", (False,) * nd)
+        x, g = tt("x"), tt("g")
+        mean = T.mean(x, axis=axes, keepdims=True)
+        outs = [T.sum(g * (x - mean), axis=axes), T.sum((x - mean) * g * np.float32(0.5), axis=axes), mean]
+        xv = (rng.standard_normal(shape) + ratio).astype("float32")
+        gv = rng.uniform(0.5, 1.5, shape).astype("float32")
+        f = th.function([x, g], outs)
+        reds = [n for n in f.toposort() if isinstance(n.op, HipCAReduce)]
+        assert len(reds) == 1, [str(n.op)[:60] for n in reds]           # the rewrite applied: one pass
+        got = f(xv, gv)
+        x64, g64 = xv.astype("float64"), gv.astype("float64")
+        m64 = x64.mean(axis=axes, keepdims=True)
+        m32 = m64.astype("float32").astype("float64")
+        assert np.array_equal(got[2], m64.astype("float32"))
+        for k, scale in ((0, 1.0), (1, 0.5)):
+            want = [(scale * g64 * (x64 - m)).sum(axis=axes) for m in (m32, m64)]
+            err = np.minimum(*[np.abs(got[k] - w) / (1e-6 + 1e-5 * np.abs(w)) for w in want])
+            assert got[k].dtype == np.float32 and err.max() <= 1.0, (shape, k, float(err.max()))
+
+
 def test_stored_elementwise_result_and_its_reduction_over_all_but_the_last_axis():
     """r = f(...) is an output and so is reduce(r, all axes but the last): one node (HipElemwiseReduce).  Through
     permuted views (NCHW read as NHWC) the kernel that stores r accumulates the per-channel results as well

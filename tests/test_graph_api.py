@@ -1167,28 +1167,6 @@ def test_device_type_value_helpers(dry_run):
     assert [type(n.op).__name__ for n in f.toposort()][0] == "HostToHip"
 
 
-def test_unittest_tools_seed_and_compare(monkeypatch):
-    """fetch_seed / seed_rng / assert_allclose / WrongValue (theano/tests/unittest_tools.py:43-92, 277-358)."""
-    from theano_amd.tests import unittest_tools as utt
-    assert utt.fetch_seed() == 666 and utt.fetch_seed(12) == 12
-    monkeypatch.setenv("THEANO_AMD_UNITTEST_RSEED", "random")
-    assert utt.fetch_seed() is None
-    monkeypatch.setenv("THEANO_AMD_UNITTEST_RSEED", "31")
-    assert utt.seed_rng() == 31
-    first = np.random.rand(3)
-    utt.seed_rng()
-    assert np.array_equal(first, np.random.rand(3))
-    monkeypatch.setenv("THEANO_AMD_UNITTEST_RSEED", "not a number")
-    assert utt.fetch_seed() is None
-    a = np.linspace(0, 1, 7, dtype="float32")
-    utt.assert_allclose(a, a + np.float32(1e-7))
-    utt.assert_allclose(a, a.astype("float64"))
-    with pytest.raises(utt.WrongValue, match="max abs error"):
-        utt.assert_allclose(a, a + np.float32(1e-2))
-    with pytest.raises(utt.WrongValue):
-        utt.assert_allclose(a, a[:3])
-
-
 def test_shape_only_nodes_rerun_when_list_arguments_change_length(dry_run):
     """The extent `mean` divides by is kept between calls with equal argument shapes; the shapes are those of
     the filtered values, so two Python lists of different lengths (which have no `.shape` themselves) count as

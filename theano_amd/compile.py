@@ -401,7 +401,8 @@ class Function(object):
         arrays and writes the same result arrays, at the cost of one launch for the whole sequence.  For
         functions of several small kernels, where the host's work per launch exceeds the kernels' run time.
         The arguments and results must be device arrays (``Out(v, device=True)``): a transfer would wait for
-        the device in the middle of the recording.  The function is run once first, so that its kernels are
+        the device in the middle of the recording.  The graph keeps the arguments and the current values of the
+        shared variables alive; a ``set_value`` after the recording is not seen by replays.  The function is run once first, so that its kernels are
         loaded and the shapes it depends on are known; calls that the function makes differently from one
         run to the next (a row chain turned away at run time, say) are recorded as this call made them."""
         from .hip.ops import HipToHost
@@ -416,6 +417,10 @@ class Function(object):
         self(*args)                         # loads the kernels, warms the pool, runs the shape-only nodes
         with capture() as c:
             results = self(*args)
+        # a replay reads the argument arrays and the arrays the shared variables held at this moment
+        # (a later set_value puts a new array into the variable, which the recording does not see)
+        c.graph.hold(*args)
+        c.graph.hold(*[s.container[0] for s in self.shared_inputs])
         return results, c.graph
 
     def _write_back(self, args, values):

@@ -523,7 +523,13 @@ int thx_elemwise_call(thx_elemwise* e, const thx_array* ins, const thx_array* ou
 }
 
 int thx_elemwise_attach_reduce(thx_elemwise* e, thx_reduce* r, const int32_t* which_outputs) {
-  if (!e || !r || !which_outputs) return fail(THX_ERR_ARG, "thx_elemwise_attach_reduce: null argument");
+  if (!e) return fail(THX_ERR_ARG, "thx_elemwise_attach_reduce: null argument");
+  if (!r) {   // detach: `e` no longer refers to the reduction, which may now be freed first
+    e->red = nullptr;
+    e->red_of.clear();
+    return THX_OK;
+  }
+  if (!which_outputs) return fail(THX_ERR_ARG, "thx_elemwise_attach_reduce: null argument");
   if (r->n_extra) return fail(THX_ERR_UNSUPPORTED, "thx_elemwise_attach_reduce: the reduction's epilogue may take no further operands");
   for (int i = 0; i < r->n_in; ++i) {
     const int w = which_outputs[i];

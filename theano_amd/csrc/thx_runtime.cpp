@@ -131,12 +131,32 @@ int ensure_init() {
   return init_locked(-1);
 }
 
+// Recorded launch sequences keep the scratch address they were recorded with: while any of them is alive
+// a scratch buffer that has become too small is set aside, not freed, and released with the last graph.
+static bool g_capturing = false;
+static int g_live_graphs = 0;
+static std::vector<void*> g_retired_scratch;
+
+static void release_retired_scratch() {
+  for (void* p : g_retired_scratch) (void)hipFree(p);
+  g_retired_scratch.clear();
+}
+
 int ensure_scratch(size_t bytes) {
   Runtime& r = rt();
   if (bytes <= r.scratch_bytes) return THX_OK;
+  if (g_capturing)
+    return fail(THX_ERR_ARG,
+                "a recording needs %zu bytes of reduction scratch, %zu are allocated: run the same calls once before "
+                "recording them (growing the buffer waits for the device, which ends a recording)",
+                bytes, r.scratch_bytes);
   if (r.scratch) {
-    THX_HIP_CHECK(hipStreamSynchronize(r.stream));
-    THX_HIP_CHECK(hipFree(r.scratch));
+    if (g_live_graphs > 0) {
+      g_retired_scratch.push_back(r.scratch);
+    } else {
+      THX_HIP_CHECK(hipStreamSynchronize(r.stream));
+      THX_HIP_CHECK(hipFree(r.scratch));
+    }
     r.scratch = nullptr;
     r.scratch_bytes = 0;
   }
@@ -668,8 +688,6 @@ struct thx_graph {
   hipGraphExec_t exec = nullptr;
 };
 
-static bool g_capturing = false;
-
 int thx_capture_begin(void) {
   int rc = ensure_init();
   if (rc) return rc;
@@ -701,6 +719,7 @@ int thx_capture_end(thx_graph** out) {
   thx_graph* g = new thx_graph;
   g->graph = graph;
   g->exec = exec;
+  ++g_live_graphs;
   *out = g;
   return THX_OK;
 }
@@ -712,12 +731,29 @@ int thx_graph_launch(thx_graph* g) {
   return THX_OK;
 }
 
+int thx_scratch_reserve(size_t nbytes) {
+  int rc = ensure_init();
+  if (rc) return rc;
+  return ensure_scratch(nbytes);
+}
+
+int thx_scratch_state(int64_t* nbytes, int64_t* superseded_held, int64_t* graphs_alive) {
+  if (nbytes) *nbytes = (int64_t)rt().scratch_bytes;
+  if (superseded_held) *superseded_held = (int64_t)g_retired_scratch.size();
+  if (graphs_alive) *graphs_alive = g_live_graphs;
+  return THX_OK;
+}
+
 int thx_graph_free(thx_graph* g) {
   if (!g) return THX_OK;
   if (rt().ready) (void)hipStreamSynchronize(rt().stream);
   if (g->exec) (void)hipGraphExecDestroy(g->exec);
   if (g->graph) (void)hipGraphDestroy(g->graph);
   delete g;
+  if (--g_live_graphs <= 0) {
+    g_live_graphs = 0;
+    release_retired_scratch();
+  }
   return THX_OK;
 }
 

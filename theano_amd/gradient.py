@@ -323,72 +323,87 @@ def _max_err(analytic, numeric, abs_tol, rel_tol):
     return best[1:]
 
 
+_GRAD_TOL = {"float16": 5e-2, "float32": 1e-2, "float64": 1e-4}      # absolute and relative, per dtype
+
+
+class _GradientCheck(object):
+    """The device functions one gradient check needs: the cost ``sum(direction * fun(*args))`` with the
+    direction a shared array that each round replaces, and the symbolic gradient of that cost."""
+
+    def __init__(self, fun, values, mode, direction_dtype):
+        from . import compile as C
+        from .tensor import basic as T
+        from .tensor.type import TensorType
+        self.values = values
+        args = [TensorType(str(v.dtype), tuple(n == 1 for n in v.shape))(name="input %i" % k)
+                for k, v in enumerate(values)]
+        result = fun(*args)
+        if isinstance(result, (list, tuple)):
+            raise NotImplementedError("verify_grad checks functions of one result; this one returns %d" % len(result))
+
+        def compiled(outputs):
+            return C.function([C.In(a, allow_downcast=True) for a in args], outputs, on_unused_input="ignore",
+                              accept_inplace=True, mode=mode)
+
+        shape = np.shape(compiled(result)(*self.fresh()))
+        self.dtype = direction_dtype or ("float32" if result.type.dtype == "float32" and direction_dtype is False
+                                         else "float64")
+        self.shape = shape
+        self.direction = C.shared(np.ones(shape, self.dtype), name="random_projection",
+                                  broadcastable=tuple(result.type.broadcastable))
+        cost = T.sum(self.direction * result)
+        self.cost = compiled(cost)
+        self.gradient = compiled(grad(cost, args, disconnected_inputs="ignore"))
+
+    def fresh(self):
+        return [v.copy() for v in self.values]
+
+    def new_direction(self, rng):
+        draw = rng.random_sample if hasattr(rng, "random_sample") else rng.random
+        self.direction.set_value(np.asarray(draw(self.shape) + 0.5, dtype=self.dtype))
+
+    def worst(self, step, abs_tol, rel_tol):
+        """(argument, flat position, analytic value, numeric value, abs error, rel error) of the element that
+        is farthest outside the tolerances."""
+        numeric = _one_sided_grad(self.cost, self.fresh(), step)
+        analytic = self.gradient(*self.fresh())
+        k, j, abs_err, rel_err = _max_err(analytic, numeric, abs_tol, rel_tol)
+        return (k, j, np.shape(analytic[k]), np.asarray(analytic[k]).reshape(-1)[j], numeric[k].reshape(-1)[j],
+                abs_err, rel_err)
+
+
 def verify_grad(fun, pt, n_tests=2, rng=None, eps=None, out_type=None, abs_tol=None, rel_tol=None, mode=None,
                 cast_to_output_type=False, no_debug_ref=True):
     """Check the symbolic gradient of ``fun`` (a function of symbolic tensors returning one tensor, or an
-    op) at the list of floating-point arrays ``pt`` against forward differences, as the reference's
-    ``verify_grad`` does (``theano/gradient.py:1625-1800``): the result is projected on a random direction
+    op) at the list of floating-point arrays ``pt`` against forward differences, with the reference's
+    acceptance rule (``theano/gradient.py:1625-1800``): the result is projected on a random direction
     with entries in [0.5, 1.5) to make a scalar cost, ``n_tests`` times; an element whose absolute *and*
     relative error both exceed the tolerances (defaults 5e-2 / 1e-2 / 1e-4 for float16 / 32 / 64, the
     loosest among ``pt``) raises ``GradientError``.  The functions run on the device."""
-    from . import compile as C
-    from .tensor import basic as T
-    from .tensor.type import TensorType
     if not isinstance(pt, (list, tuple)):
-        raise TypeError("pt must be a list of arrays")
-    pt = [np.array(p) for p in pt]
-    for i, p in enumerate(pt):
-        if str(p.dtype) not in TYPE_EPS:
-            raise TypeError('verify_grad can work only with floating point inputs, but input %i has dtype "%s".'
-                            % (i, p.dtype))
-    type_tol = dict(float16=5e-2, float32=1e-2, float64=1e-4)
-    if abs_tol is None:
-        abs_tol = max(type_tol[str(p.dtype)] for p in pt)
-    if rel_tol is None:
-        rel_tol = max(type_tol[str(p.dtype)] for p in pt)
+        raise TypeError("verify_grad: the point must be a list of arrays, one per argument")
     if rng is None:
-        raise TypeError("rng should be a valid instance of numpy.random.RandomState.")
-    if eps is None:
-        eps = max(TYPE_EPS[str(p.dtype)] for p in pt)
-    tensor_pt = [TensorType(str(p.dtype), tuple(s == 1 for s in p.shape))(name="input %i" % i) for i, p in enumerate(pt)]
-    o_output = fun(*tensor_pt)
-    if isinstance(o_output, (list, tuple)):
-        raise NotImplementedError("cant (yet) autotest gradient of fun with multiple outputs")
-    specs = [C.In(v, allow_downcast=True) for v in tensor_pt]
-
-    def function(outputs):
-        return C.function(specs, outputs, on_unused_input="ignore", accept_inplace=True, mode=mode)
-
-    o_fn_out = function(o_output)(*[p.copy() for p in pt])
-    if isinstance(o_fn_out, (tuple, list)):
-        raise TypeError("It seems like you are trying to use verify_grad on an op or a function which outputs a "
-                        "list: there should be a single (array-like) output instead")
-
-    def random_projection():
-        plain = (rng.random_sample(o_fn_out.shape) if hasattr(rng, "random_sample") else rng.random(o_fn_out.shape)) + 0.5
-        dt = o_output.type.dtype if (cast_to_output_type and o_output.type.dtype == "float32") else out_type or "float64"
-        return np.asarray(plain, dtype=dt)
-
-    t_r = C.shared(random_projection(), name="random_projection",
-                   broadcastable=tuple(o_output.type.broadcastable))
-    cost = T.sum(t_r * o_output)
-    cost_fn = function(cost)
-    grad_fn = function(grad(cost, tensor_pt, disconnected_inputs="ignore"))
-    for test_num in range(n_tests):
-        try:
-            num_grad = _one_sided_grad(cost_fn, [p.copy() for p in pt], eps)
-            analytic = grad_fn(*[p.copy() for p in pt])
-            max_arg, max_pos, max_abs, max_rel = _max_err(analytic, num_grad, abs_tol, rel_tol)
-            if max_abs > abs_tol and max_rel > rel_tol:
-                raise GradientError(max_arg, max_pos, np.shape(analytic[max_arg]),
-                                    np.asarray(analytic[max_arg]).reshape(-1)[max_pos],
-                                    num_grad[max_arg].reshape(-1)[max_pos], max_abs, max_rel, abs_tol, rel_tol)
-            if test_num < n_tests - 1:
-                t_r.set_value(random_projection())
-        except Exception as e:
-            e.args += ("\nThe error happened with the following inputs:", pt, "\nThe value of eps is:", eps,
-                       "\nThe out_type is:", out_type)
-            raise
+        raise TypeError("verify_grad: pass a seeded numpy.random.RandomState (or Generator) as rng")
+    values = [np.array(p) for p in pt]
+    kinds = [str(v.dtype) for v in values]
+    for k, dt in enumerate(kinds):
+        if dt not in TYPE_EPS:
+            raise TypeError("verify_grad can work only with floating point inputs, but input %i has dtype \"%s\"."
+                            % (k, dt))
+    loosest = max(_GRAD_TOL[dt] for dt in kinds)
+    abs_tol = loosest if abs_tol is None else abs_tol
+    rel_tol = loosest if rel_tol is None else rel_tol
+    step = max(TYPE_EPS[dt] for dt in kinds) if eps is None else eps
+    check = _GradientCheck(fun, values, mode, out_type or (False if cast_to_output_type else None))
+    try:
+        for _round in range(n_tests):
+            check.new_direction(rng)
+            k, j, shape, ana, num, abs_err, rel_err = check.worst(step, abs_tol, rel_tol)
+            if abs_err > abs_tol and rel_err > rel_tol:
+                raise GradientError(k, j, shape, ana, num, abs_err, rel_err, abs_tol, rel_tol)
+    except Exception as e:
+        e.args += ("verify_grad was checking at", pt, "with step", step, "and out_type", out_type)
+        raise
 
 
 verify_grad.E_grad = GradientError

@@ -16,10 +16,18 @@ counterpart: it keeps every CAReduce a node of its own (``theano/tensor/opt.py:7
 elementwise nodes only).
 
 Only sums with float64 accumulators are rewritten, and only expressions that are of first degree in
-the hoisted operands: the difference of the two sums then carries a relative error of 2**-53 times
-the ratio of their size to the result's, invisible at float32 (let alone float16) precision, where
-a second-degree expansion (``sum((x - mean)**2)``) would cancel catastrophically.
+the hoisted operands.  The terms of the expanded sums are far larger than the terms of the original
+one when the mean is large against the spread (``g * x`` against ``g * (x - mean)``), so a product of
+free factors must not be rounded to the operands' own type: a float32 product would put an error of
+2**-24 |g x| into every term, |mean| / sigma times what the reference's ``g * (x - mean)`` carries.
+Every product or quotient of free factors is therefore formed in float64 (the product of two float32
+values is exact there; where both factors are float16 values widened to float32 the float32 product is
+exact already and stays).  The difference of the two sums then carries a relative error of 2**-53 times
+the ratio of their size to the result's, invisible at float32 (let alone float16) precision, where a
+second-degree expansion (``sum((x - mean)**2)``) would cancel catastrophically.
 """
+import numpy as np
+
 from .. import gof
 from .. import scalar as scal
 from ..config import config
@@ -47,6 +55,29 @@ class _NotSeparable(Exception):
 
 def _times(a, b):
     return a if b is None else (b if a is None else scal.mul(a, b))
+
+
+def _f64(v):
+    return v if v.type.dtype == "float64" else scal.cast(v, "float64")
+
+
+def _half_bits(v):
+    """Is ``v`` a float16 value (possibly widened)?  Such a value has 11 significant bits."""
+    while v.owner is not None and isinstance(v.owner.op, (scal.Cast, scal.Identity)) and (
+            v.type.dtype in scal.float_dtypes and v.owner.inputs[0].type.dtype in scal.float_dtypes and
+            np.dtype(v.type.dtype).itemsize >= np.dtype(v.owner.inputs[0].type.dtype).itemsize):
+        v = v.owner.inputs[0]
+    return v.type.dtype == "float16"
+
+
+def _free_times(a, b):
+    """The product of two free factors without a rounding: in float64, or in float32 where both are
+    float16 values (22 significant bits)."""
+    if a is None or b is None:
+        return a if b is None else b
+    if _half_bits(a) and _half_bits(b) and a.type.dtype == b.type.dtype == "float32":
+        return scal.mul(a, b)
+    return scal.mul(_f64(a), _f64(b))
 
 
 def _terms(v, cset, dep, pure, memo):
@@ -89,7 +120,7 @@ def _terms(v, cset, dep, pure, memo):
                     for c2, k2, h2, f2 in _terms(i, cset, dep, pure, memo):
                         if c1 is not None and c2 is not None:
                             raise _NotSeparable()          # second degree
-                        nxt.append((c1 if c1 is not None else c2, k1 * k2, _times(h1, h2), _times(f1, f2)))
+                        nxt.append((c1 if c1 is not None else c2, k1 * k2, _times(h1, h2), _free_times(f1, f2)))
                 res = nxt
         elif isinstance(op, scal.TrueDiv):
             den = ins[1]
@@ -102,7 +133,7 @@ def _terms(v, cset, dep, pure, memo):
                 elif den in pure:
                     res.append((c, k, scal.inv(den) if h is None else scal.true_div(h, den), f))
                 else:
-                    res.append((c, k, h, scal.inv(den) if f is None else scal.true_div(f, den)))
+                    res.append((c, k, h, scal.inv(_f64(den)) if f is None else scal.true_div(_f64(f), _f64(den))))
         else:
             raise _NotSeparable()
         if v.type.dtype not in _FLOATS:

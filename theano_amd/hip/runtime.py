@@ -83,6 +83,8 @@ def _load():
         "thx_capture_end": ([P(vp)], ctypes.c_int),
         "thx_graph_launch": ([vp], ctypes.c_int),
         "thx_graph_free": ([vp], ctypes.c_int),
+        "thx_scratch_reserve": ([sz], ctypes.c_int),
+        "thx_scratch_state": ([P(i64), P(i64), P(i64)], ctypes.c_int),
     }
     for name, (argtypes, restype) in sigs.items():
         fn = getattr(lib, name, None)
@@ -205,10 +207,16 @@ _capture_keep = None      # while a capture is open: the buffers allocated insid
 
 class Graph(object):
     """A recorded sequence of launches (``capture``): ``launch()`` replays it on the library's stream.  The
-    graph owns every buffer that was allocated while it was recorded - replays write to those addresses."""
+    graph owns every buffer that was allocated while it was recorded - replays write to those addresses -
+    and ``hold(...)`` adds the arrays it only reads (arguments, shared variables' values as of the
+    recording), so that nothing a replay touches returns to the pool while the graph is alive."""
 
     def __init__(self, handle, buffers):
-        self._handle, self._buffers = handle, buffers
+        self._handle, self._buffers = handle, list(buffers)
+
+    def hold(self, *arrays):
+        self._buffers.extend(arrays)
+        return self
 
     def launch(self):
         check(lib.thx_graph_launch(self._handle))
@@ -220,6 +228,19 @@ class Graph(object):
                 self._handle = None
         except Exception:
             pass
+
+
+def scratch_state():
+    """(bytes of the reduction scratch buffer, superseded buffers still held for recorded sequences,
+    recorded sequences alive)."""
+    a, b, c = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+    check(lib.thx_scratch_state(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c)))
+    return a.value, b.value, c.value
+
+
+def scratch_reserve(nbytes):
+    init()
+    check(lib.thx_scratch_reserve(int(nbytes)))
 
 
 class capture(object):
