@@ -64,6 +64,30 @@ def test_config3_softmax_and_gradient():
     assert_within_reference_error(dx[rows], ref[1], sm * (y[rows] - (sm * y[rows]).sum(1, keepdims=True)), "c3 grad rows")
 
 
+def test_config3_gradient_alone_full_size():
+    """The gradient of config 3 given only x and y (no softmax among the results): one launch that reads x and y and
+    writes dx; rows of dx sum to zero, the first rows equal the closed form and what the forward + gradient
+    function returns."""
+    from theano_amd.hip import HipRowChain
+    parity(W.c3_graph(forward=False), W.c3_inputs("small"), "c3 grad alone small")
+    ins, outs = W.c3_graph(forward=False)
+    x, y = W.c3_inputs("full")
+    f = th.function(ins, outs)
+    kernels = [n for n in f.toposort() if type(n.op).__name__ in ("HipElemwise", "HipCAReduce", "HipRowChain")]
+    assert len(kernels) == 1 and isinstance(kernels[0].op, HipRowChain), kernels
+    (dx,) = f(x, y)
+    assert dx.shape == x.shape and dx.dtype == np.float32
+    assert np.abs(dx.astype("float64").sum(1)).max() < 1e-5
+    rows = slice(0, 64)
+    e = np.exp(x[rows].astype("float64") - x[rows].max(1, keepdims=True))
+    sm = e / e.sum(1, keepdims=True)
+    ref = G.evaluate(ins, outs, [x[rows], y[rows]])
+    assert_within_reference_error(dx[rows], ref[0], sm * (y[rows] - (sm * y[rows]).sum(1, keepdims=True)), "c3 grad alone rows")
+    ins2, outs2 = W.c3_graph()
+    both = th.function(ins2, outs2)(x[:4096], y[:4096])
+    assert_parity(dx[:4096], both[1], "gradient alone against forward + gradient")
+
+
 def test_config4_integer_path():
     parity(W.c4_graph("all"), W.c4_inputs("small"), "c4 small")
     ins, outs = W.c4_graph("all")

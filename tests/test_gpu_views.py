@@ -223,3 +223,43 @@ def test_composed_front_ends_on_the_device(k):
         x = T.dmatrix("x")
         with pytest.raises(ValueError):
             th.function([x], T.addbroadcast(x, 0) * 2.0)(np.zeros((2, 3)))
+
+
+def test_reshape_takes_its_shape_as_one_integer_vector():
+    """``reshape(x, shape_vector, ndim=n)`` (``theano/tensor/basic.py:4858-4960, 5049-5068``): the vector is an
+    argument of the function, read on the host when it runs and never copied to the device; one element may be -1;
+    a vector of the wrong length or a shape of the wrong size is a ValueError; the gradient flows back to x.
+    ``alloc`` takes elements of such a vector.  Expected values are NumPy's own reshape / broadcast."""
+    rng = np.random.default_rng(61)
+    x, s = T.fmatrix("x"), T.lvector("s")
+    y = x.reshape(s, ndim=3)
+    assert y.type.ndim == 3 and y.type.broadcastable == (False, False, False)
+    f = th.function([x, s], [y * 2 + 1, T.sum(T.reshape(x, s, ndim=3), axis=(0, 2)), th.grad(T.sum(T.sqr(y)), x)])
+    assert not any(type(n.op).__name__ == "HostToHip" and n.inputs[0] is not None and n.inputs[0].type.ndim == 1
+                   for n in f.toposort()), "the shape vector went to the device"
+    xv = rng.standard_normal((12, 10)).astype("float32")
+    for shp in ([2, 6, 10], [5, 4, 6], np.array([3, -1, 8]), np.array([-1, 1, 120], "int32")):
+        got = f(xv, shp)
+        want = xv.reshape(tuple(int(v) for v in shp))
+        assert got[0].shape == want.shape and np.array_equal(got[0], want * 2 + 1)
+        assert_parity(got[1], want.astype("float64").sum(axis=(0, 2)).astype("float32"), "sum of the reshaped array")
+        assert np.array_equal(got[2], 2 * xv)
+    for bad in ([12, 10], [7, 2, 9], [-1, -1, 10]):
+        with pytest.raises(ValueError):
+            f(xv, bad)
+    with pytest.raises(ValueError, match="ndim"):
+        T.reshape(x, s)                                    # the rank must be known when the graph is built
+    with pytest.raises(TypeError):
+        T.reshape(x, T.fvector(), ndim=2)                  # theano/tensor/basic.py:4888-4892
+    assert T.reshape(x, T.constant(np.array([3, 40]))).type.ndim == 2      # a constant vector tells its length
+    # elements of a shape vector as alloc's extents, and arithmetic over them
+    v = T.fvector("v")
+    g = th.function([v, s], T.alloc(v, s[0], s[1] * 2, v.shape[0]) + np.float32(1))
+    vv = rng.standard_normal(7).astype("float32")
+    got = g(vv, [3, 2, 99])
+    assert got.shape == (3, 4, 7) and np.array_equal(got, np.broadcast_to(vv, (3, 4, 7)) + np.float32(1))
+    with pytest.raises(ValueError):
+        g(vv, [3])
+    # the vector may also be computed on the device: then its values are fetched
+    h = th.function([x, s], x.reshape(s * 2, ndim=2))
+    assert np.array_equal(h(xv, [2, 15]), xv.reshape(4, 30))

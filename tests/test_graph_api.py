@@ -1194,3 +1194,29 @@ def test_shape_only_nodes_rerun_when_list_arguments_change_length(dry_run):
     assert len(runs) == 2
     f(np.zeros(5, "float32"))
     assert len(runs) == 3
+
+
+def test_reshape_with_a_shape_vector_argument(dry_run):
+    """reshape(x, v, ndim=n) with v an integer vector argument (theano/tensor/basic.py:4858-4960, 5049-5068): the rank
+    comes from ndim, the vector stays on the host, its elements are checked when the function runs."""
+    from theano_amd.tensor.views import Reshape
+    x, s = T.fmatrix("x"), T.lvector("s")
+    y = x.reshape(s, ndim=3)
+    assert isinstance(y.owner.op, Reshape) and y.type.ndim == 3 and str(y.owner.op) == "Reshape{in1[0], in1[1], in1[2]}"
+    assert T.reshape(x, s, ndim=3).owner.op == y.owner.op
+    f = th.function([x, s], y + 1)
+    names = [type(n.op).__name__ for n in f.toposort()]
+    assert names.count("HostToHip") == 1 and "HipReshape" in names
+    xv = np.zeros((4, 6), "float32")
+    assert f(xv, [2, 3, 4]).shape == (2, 3, 4) and f(xv, np.array([4, -1, 2])).shape == (4, 3, 2)
+    for bad in ([2, 3], [5, 5, 1], [-1, -1, 6]):
+        with pytest.raises(ValueError):
+            f(xv, bad)
+    with pytest.raises(ValueError, match="ndim"):
+        T.reshape(x, s)
+    with pytest.raises(ValueError):
+        x.reshape((2, 12), ndim=3)
+    z = T.alloc(np.float32(1.5), s[0], s[1] * 2)
+    assert str(z.owner.op) == "Alloc{in1[0], mul(in1[1], 2)}"
+    g = th.function([s], z)
+    assert [type(n.op).__name__ for n in g.toposort()] == ["HipAlloc", "HipToHost"] and g([3, 4]).shape == (3, 8)

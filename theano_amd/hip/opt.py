@@ -51,13 +51,31 @@ def _lift_reduce(node, x):
                        (acc,), (out,))(x)
 
 
+def _shape_vector_inputs(fgraph):
+    """Function inputs that every client reads as a whole shape vector on the host (``reshape(x, v, ndim=n)``):
+    they are never copied to the device."""
+    from ..tensor import views as V
+    keep = set()
+    for i in fgraph.inputs:
+        if not isinstance(i.type, TensorType) or i.type.ndim != 1 or i.type.dtype not in scal.discrete_dtypes:
+            continue
+        clients = fgraph.clients.get(i, []) if hasattr(fgraph, "clients") else []
+        uses = [(node, k) for node, k in clients if node != "output"]
+        if uses and len(uses) == len(clients) and all(
+                isinstance(node.op, (V.Reshape, V.Alloc)) and k in V.vector_inputs(node.op.pattern) and k > 0
+                for node, k in uses):
+            keep.add(i)
+    return keep
+
+
 def lift_to_hip(fgraph):
     """Return a new FunctionGraph computing the same outputs with device ops.
     Raises NotImplementedError for an op with no device counterpart: there is
     no host execution to fall back to."""
     mapping = {}
+    shape_vectors = _shape_vector_inputs(fgraph)
     for i in fgraph.inputs:
-        if isinstance(i.type, TensorType) and not _is_host_scalar(i):
+        if isinstance(i.type, TensorType) and not _is_host_scalar(i) and i not in shape_vectors:
             mapping[i] = hip_from_host(i)
         else:
             mapping[i] = i

@@ -128,9 +128,17 @@ class HipIncSubtensor(V.IncSubtensor):
         output_storage[0][0] = out
 
 
+def _shape_operands(pattern, like, first):
+    """The inputs after the first `first` ones as a device op takes them: arrays whose extents are read go to the
+    device like any array, host scalars stay, and an integer vector that is read for its values (a shape given as
+    one vector) stays on the host when it is there - its elements are needed before anything can be launched."""
+    vec = V.vector_inputs(pattern)
+    return [v if (k + first in vec and not isinstance(v.type, HipArrayType)) else _device(v) for k, v in enumerate(like)]
+
+
 class HipReshape(V.Reshape):
     def make_node(self, x, *like):
-        ins = [as_hip_variable(x)] + [_device(v) for v in like]
+        ins = [as_hip_variable(x)] + _shape_operands(self.pattern, like, 1)
         host = V.Reshape.make_node(self, *[V.TensorType(i.type.dtype, i.type.broadcastable)() for i in ins])
         ot = host.outputs[0].type
         return Apply(self, ins, [HipArrayType(ot.dtype, ot.broadcastable)()])
@@ -152,7 +160,7 @@ class HipReshape(V.Reshape):
 
 class HipAlloc(V.Alloc):
     def make_node(self, value, *like):
-        ins = [_device(value)] + [_device(v) for v in like]
+        ins = [_device(value)] + _shape_operands(self.pattern, like, 1)
         host = V.Alloc.make_node(self, *[V.TensorType(i.type.dtype, i.type.broadcastable)() for i in ins])
         ot = host.outputs[0].type
         return Apply(self, ins, [HipArrayType(ot.dtype, ot.broadcastable)()])

@@ -243,15 +243,24 @@ class _tensor_py_operators(object):
             n = d if n is None else n * d
         return n if n is not None else self._b().constant(np.int64(1))
 
-    def reshape(self, *shape):
+    def reshape(self, *shape, **kw):
+        """``x.reshape((a, b))``, ``x.reshape(a, b)`` or ``x.reshape(shape_vector, ndim=n)``
+        (``theano/tensor/var.py:297-330``)."""
         from . import views
+        ndim = kw.pop("ndim", None)
+        if kw:
+            raise TypeError("reshape() got unexpected keyword arguments %s" % sorted(kw))
+        if ndim is not None and not isinstance(ndim, (int, np.integer)):
+            raise ValueError("Expected ndim to be an integer, is " + str(type(ndim)))
+        if len(shape) == 1 and hasattr(shape[0], "owner") and getattr(shape[0].type, "ndim", 0) == 1:
+            return views.reshape(self, shape[0], ndim=ndim)
         one = shape[0] if len(shape) == 1 else None
         is_pair = (isinstance(one, (list, tuple)) and len(one) == 2 and hasattr(one[0], "type") and
                    isinstance(one[1], (int, np.integer)) and
                    0 <= one[1] < getattr(one[0].type, "ndim", 0))   # x.reshape((v, d)): the extent of v along d
         if isinstance(one, (list, tuple)) and not is_pair:
             shape = tuple(one)
-        return views.reshape(self, shape)
+        return views.reshape(self, shape, ndim=ndim)
 
     def fill(self, value):
         """A tensor of this one's shape filled with ``value`` (``theano/tensor/var.py:_tensor_py_operators.fill``)."""

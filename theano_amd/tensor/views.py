@@ -315,6 +315,9 @@ def set_subtensor(x, y, idx=None):
 #   n               a plain extent (Reshape: -1 = inferred)
 #   (k, d)          the extent of dimension d of input k
 #   ("in", k)       the value of input k, an integer scalar read on the host when the function runs
+#   ("vec", k, j, n) element j of input k, an integer vector of n elements (n = -1: of any length) read on the host
+#                   when the function runs (reshape(x, shape_vector, ndim=n), alloc(v, shape_vector[0], ...)); in a
+#                   Reshape such an element may be -1
 #   (op, a, b)      op in _SHAPE_OPS over two entries: arithmetic on extents, evaluated on the host from array
 #                   metadata (x.reshape((x.shape[0], x.shape[1] * x.shape[2])), alloc(0., n // 2, m + 1), ...)
 _SHAPE_OPS = {"add": lambda a, b: a + b, "sub": lambda a, b: a - b, "mul": lambda a, b: a * b,
@@ -325,6 +328,8 @@ def _norm_entry(p, allow_unknown):
     if isinstance(p, tuple):
         if len(p) == 2 and p[0] == "in":
             return ("in", int(p[1]))
+        if len(p) == 4 and p[0] == "vec":
+            return ("vec", int(p[1]), int(p[2]), int(p[3]))
         if len(p) == 3 and p[0] in _SHAPE_OPS:
             return (p[0], _norm_entry(p[1], False), _norm_entry(p[2], False))
         if len(p) == 2 and not isinstance(p[0], str):
@@ -340,7 +345,7 @@ def _entry_inputs(p):
     """Indices of the node inputs an entry reads."""
     if not isinstance(p, tuple):
         return []
-    if p[0] == "in":
+    if p[0] in ("in", "vec"):
         return [p[1]]
     if p[0] in _SHAPE_OPS:
         return _entry_inputs(p[1]) + _entry_inputs(p[2])
@@ -355,9 +360,35 @@ def _eval_entry(p, shapes, values):
             raise ValueError("this shape depends on the value of an input, not only on shapes")
         v = values[p[1]]
         return int(np.asarray(v.to_numpy() if hasattr(v, "to_numpy") else v).reshape(()))
+    if p[0] == "vec":
+        if values is None:
+            raise ValueError("this shape depends on the value of an input, not only on shapes")
+        v = values[p[1]]
+        v = np.asarray(v.to_numpy() if hasattr(v, "to_numpy") else v)
+        if v.ndim != 1 or (v.shape[0] != p[3] if p[3] >= 0 else v.shape[0] <= p[2]):
+            # theano/tensor/basic.py:4918-4921
+            raise ValueError("shape argument has incorrect length %s, should be %s" % (
+                v.shape, p[3] if p[3] >= 0 else "more than %d" % p[2]))
+        return int(v[p[2]])
     if p[0] in _SHAPE_OPS:
         return int(_SHAPE_OPS[p[0]](_eval_entry(p[1], shapes, values), _eval_entry(p[2], shapes, values)))
     return int(shapes[p[0]][p[1]])
+
+
+def vector_inputs(pattern):
+    """Indices of the inputs a pattern reads as whole integer vectors (on the host)."""
+    out = set()
+
+    def walk(p):
+        if isinstance(p, tuple):
+            if p[0] == "vec":
+                out.add(p[1])
+            elif p[0] in _SHAPE_OPS:
+                walk(p[1])
+                walk(p[2])
+    for p in pattern:
+        walk(p)
+    return out
 
 
 def _entry_str(p):
@@ -365,6 +396,8 @@ def _entry_str(p):
         return str(p)
     if p[0] == "in":
         return "in%d" % p[1]
+    if p[0] == "vec":
+        return "in%d[%d]" % (p[1], p[2])
     if p[0] in _SHAPE_OPS:
         return "%s(%s, %s)" % (p[0], _entry_str(p[1]), _entry_str(p[2]))
     return "in%d.shape[%d]" % p
@@ -424,9 +457,11 @@ class Reshape(Op):
         out, known, unknown = [], 1, None
         for j, p in enumerate(self.pattern):
             v = _eval_entry(p, shapes, values)
-            if v < -1 or (v == -1 and isinstance(p, tuple)):
+            if v < -1 or (v == -1 and isinstance(p, tuple) and p[0] != "vec"):
                 raise ValueError("negative extent %d from shape entry %s" % (v, _entry_str(p)))
             if v == -1:
+                if unknown is not None:
+                    raise ValueError("can only specify one unknown dimension")
                 unknown = j
                 out.append(-1)
             else:
@@ -501,6 +536,14 @@ class _ShapeArgs(object):
             raise TypeError("a symbolic shape entry must be an integer scalar, got %s" % (p.type,))
         node = p.owner
         if node is not None:
+            if (isinstance(node.op, Subtensor) and len(node.inputs) == 1 and node.inputs[0].type.ndim == 1 and
+                    isinstance(node.op.idx_list[0], (int, np.integer)) and node.op.idx_list[0] >= 0 and
+                    node.inputs[0].type.dtype in scal.discrete_dtypes):
+                # shape_vector[j]: read from the vector on the host, no device round trip (length -1: any length
+                # that has an element j)
+                v = node.inputs[0]
+                n = _vector_length(v)
+                return ("vec", self.index(v), int(node.op.idx_list[0]), -1 if n is None else n)
             if isinstance(node.op, T.ShapeFloat):
                 return (self.index(node.inputs[0]), node.op.i)
             if isinstance(node.op, DimShuffle):
@@ -519,13 +562,54 @@ class _ShapeArgs(object):
         return ("in", self.index(p))
 
 
-def reshape(x, newshape):
-    """``newshape``: ints, at most one -1, ``v.shape[d]`` entries, integer scalar variables (read on the host
-    when the function runs) and arithmetic over those (``theano/tensor/basic.py:4701-4920`` takes any integer
-    vector; here the entries are given one by one)."""
+def _vector_length(v):
+    """The number of elements of the integer vector variable ``v`` when the graph tells it (a constant, a join
+    or stack of scalars; ``get_vector_length``, ``theano/tensor/basic.py:4470-4550``), else None."""
+    if hasattr(v, "data"):
+        return int(np.asarray(v.data).shape[0])
+    node = v.owner
+    if node is not None and isinstance(node.op, Join) and node.op.axis == 0:
+        parts = [_vector_length(i) for i in node.inputs]
+        return None if any(n is None for n in parts) else sum(parts)
+    if node is not None and type(node.op).__name__ == "DimShuffle" and node.inputs[0].type.ndim == 0 and v.type.ndim == 1:
+        return 1
+    return None
+
+
+def reshape(x, newshape, ndim=None):
+    """``newshape``: a list of ints (at most one -1), ``v.shape[d]`` entries, integer scalar variables and arithmetic
+    over those - or ONE integer vector (a constant, or a variable read on the host when the function runs, whose
+    length ``ndim`` gives when the graph does not tell it; ``theano/tensor/basic.py:4858-4960, 5049-5068``).  An
+    element of a run-time vector may be -1, as in NumPy."""
     x = as_tensor_variable(x)
+    if hasattr(newshape, "owner") and getattr(newshape.type, "ndim", 0) == 1:
+        vec = newshape
+        dt = vec.type.dtype
+        if not (dt.startswith("int") or dt.startswith("uint")):
+            raise TypeError("Shape must be integers", vec, dt)
+        if hasattr(vec, "data"):
+            newshape = [int(n) for n in np.asarray(vec.data)]
+            if ndim is not None and ndim != len(newshape):
+                raise ValueError("the shape has %d entries, ndim says %d" % (len(newshape), ndim))
+        else:
+            n = _vector_length(vec)
+            if n is None:
+                n = ndim
+            elif ndim is not None and ndim != n:
+                raise ValueError("the shape vector has %d entries, ndim says %d" % (n, ndim))
+            if n is None:
+                raise ValueError("The length of the provided shape (%s) cannot be automatically determined, so the "
+                                 "number of dimensions of the reshaped variable is unknown. You can provide the "
+                                 "'ndim' keyword argument to 'reshape' to avoid this problem." % vec)
+            args = _ShapeArgs(x)
+            k = args.index(vec)
+            return Reshape([("vec", k, j, n) for j in range(n)])(x, *args.extra())
+    elif hasattr(newshape, "owner") and getattr(newshape.type, "ndim", 0) > 1:
+        raise TypeError("New shape in reshape must be a vector or a list/tuple of scalar. Got %s" % newshape)
     if isinstance(newshape, (int, np.integer)) or hasattr(newshape, "owner"):
         newshape = (newshape,)
+    if ndim is not None and ndim != len(newshape):
+        raise ValueError("the shape has %d entries, ndim says %d" % (len(newshape), ndim))
     args = _ShapeArgs(x)
     pattern = [args.entry(p) for p in newshape]
     return Reshape(pattern)(x, *args.extra())
