@@ -16,8 +16,10 @@ launch of each kind, and the average of the two loops divides the kernel's
 algorithmic bytes.  ``cpu_baseline`` times the oracle's C restatement of the
 reference's loops on this host.  ``other_configs`` lists the remaining four
 configurations (and max_and_argmax of the configuration-2 matrix) over input
-sets that rotate (so that no set is still cached when it is used again: ``us``)
-and over one set (``same_input_us``).
+sets that rotate (so that no set is still cached when it is used again: ``us``,
+the median of nine runs of K steps, ``min_us`` the fastest of them) and over one
+set (``same_input_us``), each with the symbols of the kernels it launches.  Every
+timed leg starts on a device that has been kept busy for 40 ms (``_settle``).
 """
 import argparse
 import json
@@ -73,6 +75,19 @@ def _time_steps(hip, step, steps, warmup):
     gpu_ms = hip.timer_stop()
     wall_ms = (time.perf_counter() - t0) * 1e3
     return gpu_ms / steps, wall_ms / steps
+
+
+def _settle(hip, step, ms=40.0, chunk=10):
+    """Run `step` until the device has been busy for about `ms` milliseconds.  After an idle period the
+    device needs some 20 ms of continuous work to reach its steady clocks: the arithmetic-heavy kernels (the
+    held chain of config 5, the tile kernels of config 4, argmax) run 5 - 20 % slower in between, the plain
+    streaming reductions do not change.  Untimed."""
+    busy = 0.0
+    while busy < ms:
+        hip.timer_start()
+        for _ in range(chunk):
+            step()
+        busy += hip.timer_stop()
 
 
 def _symbol(profile_name):
@@ -199,6 +214,7 @@ def main():
             fcopy(*x_dev["normal"])
         hip.sync()
 
+    _settle(hip, step)
     gpu_ms, wall_ms = _time_steps(hip, step, args.steps, args.warmup)
     value = total_bytes / (gpu_ms * 1e-3) / 1e9
 
@@ -259,10 +275,12 @@ def main():
                 f(*sets[turn[0] % len(sets)])
                 turn[0] += 1
 
-            # three runs of K steps each: the median is the figure (`us`), the fastest run is listed beside it
-            runs = sorted(_time_steps(hip, rotating, args.steps, 3)[0] for _ in range(3))
-            ms = runs[1]
-            warm_ms = sorted(_time_steps(hip, lambda: f(*sets[0]), args.steps, 3)[0] for _ in range(3))[1]
+            # nine runs of K steps each on a device at its steady clocks: the median is the figure (`us`), the
+            # fastest run is listed beside it
+            _settle(hip, rotating)
+            runs = sorted(_time_steps(hip, rotating, args.steps, 3)[0] for _ in range(9))
+            ms = runs[len(runs) // 2]
+            warm_ms = sorted(_time_steps(hip, lambda: f(*sets[0]), args.steps, 3)[0] for _ in range(5))[2]
             n_k = sum(1 for n in f.toposort()
                       if type(n.op).__name__ in ("HipElemwise", "HipElemwiseReduce", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax"))
             with hip.profile() as p:

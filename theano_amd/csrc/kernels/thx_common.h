@@ -239,6 +239,33 @@ THX_DEV void store_vec(T* b, const Vec<T, N>& r) {
   }
 }
 
+// Sums over the V float16 elements of a vector, two elements per instruction (v_dot2_f32_f16: both products
+// and both additions in float32, the products exact; float16 denormals count, measured): the sum of the
+// elements, and the sum of the pairwise products of two vectors.
+typedef _Float16 thx_f16x2 __attribute__((ext_vector_type(2)));
+
+template <int V>
+THX_DEV float half_dot(const Vec<thx_f16, V>& a, const Vec<thx_f16, V>& b) {
+  static_assert(V % 2 == 0, "pairs of elements");
+  const thx_f16x2* pa = (const thx_f16x2*)&a;
+  const thx_f16x2* pb = (const thx_f16x2*)&b;
+  float acc = 0.0f;
+#pragma unroll
+  for (int k = 0; k < V / 2; ++k) acc = __builtin_amdgcn_fdot2(pa[k], pb[k], acc, false);
+  return acc;
+}
+
+template <int V>
+THX_DEV float half_sum(const Vec<thx_f16, V>& a) {
+  static_assert(V % 2 == 0, "pairs of elements");
+  const thx_f16x2* pa = (const thx_f16x2*)&a;
+  const thx_f16x2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+  float acc = 0.0f;
+#pragma unroll
+  for (int k = 0; k < V / 2; ++k) acc = __builtin_amdgcn_fdot2(pa[k], ones, acc, false);
+  return acc;
+}
+
 // Division by a run-time constant d >= 2 for dividends below 2^31:
 // q = mulhi(n, m) >> s with m = ceil(2^(31+L)/d), s = L-1, L = ceil(log2 d).
 struct FastDiv {

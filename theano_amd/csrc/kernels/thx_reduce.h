@@ -183,6 +183,23 @@ __device__ __forceinline__ void red_row_block(const RowParams<R::NIN, R::NOUT, R
     const long long j0 = (long long)s * p.chunk;
     long long j1 = j0 + p.chunk;
     if (j1 > p.nvec) j1 = p.nvec;
+    // RA > 1: a thread's vectors are TPR apart, so their (slab, position in the slab) coordinates and every
+    // operand's offset advance by the same amounts from one vector to the next - additions and one compare
+    // instead of a division and two or three quarter-rate multiplies per vector
+    IT cur[NIN], step[NIN], wrap[NIN];
+    UT cv = 0, dcv = 0;
+    if (P::RA2) {
+      UT ra, dra;
+      divmod((UT)(j0 + t), p.rcv, ra, cv);
+      divmod((UT)TPR, p.rcv, dra, dcv);
+#pragma unroll
+      for (int i = 0; i < NIN; ++i) {
+        const IT along = red_term<P>(i, 1, (IT)VEC, p.rc_stride[i]);      // offset of one vector along RC
+        cur[i] = base[i] + red_term<P>(i, 0, (IT)ra, p.ra_stride[i]) + (IT)cv * along;
+        step[i] = red_term<P>(i, 0, (IT)dra, p.ra_stride[i]) + (IT)dcv * along;
+        wrap[i] = red_term<P>(i, 0, (IT)1, p.ra_stride[i]) - (IT)p.rcv.d * along;
+      }
+    }
     for (long long j = j0 + t; j < j1; j += (long long)TPR * UNR) {
       typename R::template Regs<VEC> r[UNR];
       bool ok[UNR];
@@ -197,16 +214,20 @@ __device__ __forceinline__ void red_row_block(const RowParams<R::NIN, R::NOUT, R
         // P::sclass(input, 0 | 1): the stride along RA | RC is 0, is 1, or anything - a multiply only
         // in the last case (32-bit integer multiplies run at quarter rate)
         if (P::RA2) {
-          UT ra, cv;
-          divmod((UT)(ok[u] ? q : j0), p.rcv, ra, cv);
 #pragma unroll
-          for (int i = 0; i < NIN; ++i)
-            a.off[i] = base[i] + red_term<P>(i, 0, (IT)ra, p.ra_stride[i]) + red_term<P>(i, 1, (IT)(cv * VEC), p.rc_stride[i]);
+          for (int i = 0; i < NIN; ++i) a.off[i] = cur[i];
+          if (ok[u]) R::template load<VEC>(a, r[u]);
+          // on to the vector TPR further (never dereferenced once it lies beyond the slice)
+          cv += dcv;
+          const bool over = cv >= p.rcv.d;
+          cv -= over ? p.rcv.d : 0;
+#pragma unroll
+          for (int i = 0; i < NIN; ++i) cur[i] += step[i] + (over ? wrap[i] : (IT)0);
         } else {
 #pragma unroll
           for (int i = 0; i < NIN; ++i) a.off[i] = base[i] + red_term<P>(i, 1, (IT)(q * VEC), p.rc_stride[i]);
+          if (ok[u]) R::template load<VEC>(a, r[u]);
         }
-        if (ok[u]) R::template load<VEC>(a, r[u]);
       }
 #pragma unroll
       for (int u = 0; u < UNR; ++u)

@@ -116,6 +116,48 @@ def _narrow_stores(pre_stmt, narrow):
     return re.sub(r"v\.a(\d+) = \([a-z0-9_]+\)(p\d+|i0);", r"v.a\1 = (decltype(v.a\1))\2;", pre_stmt)
 
 
+def _half_products(pre_op, in_dtypes, narrow):
+    """For each narrowed sum k whose per-element value is a float16 input widened to float32, its square, or
+    the product of two such inputs: ``{k: (a, b)}`` with the input positions (``b`` None for a plain sum).
+    Those sums are formed two elements at a time straight from the packed halves (``thx::half_dot``); a
+    product of two float16 values is exact in float32, so nothing is lost against widening first."""
+    if not isinstance(pre_op, scal.Composite):
+        return {}
+
+    def source(v):
+        """Position of the float16 input that ``v`` is a widened copy of, or None."""
+        while v.owner is not None and isinstance(v.owner.op, (scal.Cast, scal.Identity)) and (
+                v.type.dtype == "float32" and v.owner.inputs[0].type.dtype in ("float16", "float32")):
+            v = v.owner.inputs[0]
+        if v in pre_op.inputs:
+            k = pre_op.inputs.index(v)
+            return k if in_dtypes[k] == "float16" else None
+        return None
+
+    found = {}
+    for k, (out, nw) in enumerate(zip(pre_op.outputs, narrow)):
+        if not nw or out.type.dtype != "float32":
+            continue
+        a = source(out)
+        if a is not None:
+            found[k] = (a, None)
+            continue
+        v = out
+        while v.owner is not None and isinstance(v.owner.op, scal.Identity):
+            v = v.owner.inputs[0]
+        if v.owner is None:
+            continue
+        if isinstance(v.owner.op, scal.Mul) and len(v.owner.inputs) == 2:
+            a, b = source(v.owner.inputs[0]), source(v.owner.inputs[1])
+            if a is not None and b is not None:
+                found[k] = (a, b)
+        elif isinstance(v.owner.op, scal.Sqr):
+            a = source(v.owner.inputs[0])
+            if a is not None:
+                found[k] = (a, a)
+    return found
+
+
 def comb_part_src(scalar_ops, acc_dtypes, narrow):
     """Statements merging two ``Part`` values: float32 addition in the narrowed fields, the
     reduction's own op in its accumulator type in the others."""
@@ -192,10 +234,17 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
         lines.append("  THX_DEV static void comb_part(Part& a, const Part& b) {\n%s\n  }" % _indent("\n".join(comb_part), 4))
         call0 = call.replace(".v[k]", ".v[0]")
         widen = " ".join("w.a%d = (%s)t.a%d;" % (k, acc_c[k], k) for k in range(K))
+        # sums of float16 inputs and of their pairwise products come from the packed halves, two elements per
+        # instruction; the per-element form of those fields above is then dead code the compiler drops
+        dots = _half_products(pre_op, in_dtypes, narrow) if pre_op is not None else {}
+        packed = " ".join("t.a%d = thx::half_%s;" % (k, "sum<V>(r.%s)" % ins[a] if b is None else
+                                                     "dot<V>(r.%s, r.%s)" % (ins[a], ins[b]))
+                          for k, (a, b) in sorted(dots.items()))
+        packed = "    if constexpr (V %% 2 == 0) { %s }\n" % packed if packed else ""
         lines.append("  template <int V> THX_DEV static void accum(Acc& s, const Regs<V>& r) {\n"
                      "    Part t; pre(%s, t);\n#pragma unroll\n"
-                     "    for (int k = 1; k < V; ++k) { Part u; pre(%s, u); comb_part(t, u); }\n"
-                     "    Acc w; %s comb(s, w);\n  }" % (call0, call, widen))
+                     "    for (int k = 1; k < V; ++k) { Part u; pre(%s, u); comb_part(t, u); }\n%s"
+                     "    Acc w; %s comb(s, w);\n  }" % (call0, call, packed, widen))
     else:
         lines.append("  template <int V> THX_DEV static void accum(Acc& s, const Regs<V>& r) {\n#pragma unroll\n"
                      "    for (int k = 0; k < V; ++k) { Acc t; pre(%s, t); comb(s, t); }\n  }" % call)
