@@ -77,12 +77,16 @@ def _time_steps(hip, step, steps, warmup):
     return gpu_ms / steps, wall_ms / steps
 
 
-def _settle(hip, step, ms=40.0, chunk=10):
+SETTLE_MS = [40.0]
+
+
+def _settle(hip, step, ms=None, chunk=10):
     """Run `step` until the device has been busy for about `ms` milliseconds.  After an idle period the
     device needs some 20 ms of continuous work to reach its steady clocks: the arithmetic-heavy kernels (the
     held chain of config 5, the tile kernels of config 4, argmax) run 5 - 20 % slower in between, the plain
     streaming reductions do not change.  Untimed."""
     busy = 0.0
+    ms = SETTLE_MS[0] if ms is None else ms
     while busy < ms:
         hip.timer_start()
         for _ in range(chunk):
@@ -165,6 +169,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the other four configurations")
+    ap.add_argument("--settle-ms", type=float, default=40.0,
+                    help="milliseconds of untimed work before each timed leg (0 under a counter-collecting profiler, "
+                         "which serialises every launch)")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also launch a plain streaming kernel (out = -x on the same (8192, 8192) float32 array, "
                          "256 MiB read + 256 MiB written) K times: the known-size kernel that hardware counters "
@@ -184,6 +191,7 @@ def main():
 
     hip.init()
     info = hip.device_info()
+    SETTLE_MS[0] = max(0.0, args.settle_ms)
 
     # ---- headline: config 2 -----------------------------------------------------------------
     # The four reductions of x share one device array and prod has its own, as the configuration
