@@ -795,3 +795,63 @@ def test_fp_contract_off_gives_the_unfused_float32_arithmetic(monkeypatch):
     got, got2 = th.function([x, y, z], [x * y + z * f32(1.2578125) - f32(0.3720703125),
                                         (x * y + z) * y - x * z * f32(3.0791015625)])(xv, yv, zv)
     assert np.array_equal(got, want) and np.array_equal(got2, want2)
+
+
+ARITH_DTYPES = ["int8", "uint8", "int16", "int32", "int64", "float16", "float32", "float64"]
+
+
+@pytest.mark.parametrize("left", ARITH_DTYPES)
+def test_arithmetic_over_every_pair_of_dtypes_against_numpy(left):
+    """+ * / // between a `left` vector and a vector of every other dtype, values and result dtypes against NumPy's own
+    arithmetic (not the oracle's walk over this package's graph): the value side of test_arithmetic_cast
+    (theano/tensor/tests/test_basic.py:6919-7060).  `/` of two integer operands is floatX (float32 here) holding the
+    float64 quotient rounded once (``TrueDiv.c_code``, theano/scalar/basic.py:1899-1915)."""
+    from conftest import TOL
+    rng = np.random.default_rng(abs(hash(left)) % 1000)
+
+    def values(dt, n=517):
+        if np.dtype(dt).kind == "u":
+            return rng.integers(1, 12, n).astype(dt)
+        if np.dtype(dt).kind == "i":
+            v = rng.integers(-11, 12, n)
+            v[v == 0] = 7
+            return v.astype(dt)
+        return (rng.uniform(0.5, 4.0, n) * rng.choice([-1.0, 1.0], n)).astype(dt)
+
+    x = T.TensorType(left, (False,))("x")
+    ys = [T.TensorType(dt, (False,))("y_" + dt) for dt in ARITH_DTYPES]
+    outs = []
+    for y in ys:
+        outs += [x + y, x * y, x / y, x // y]
+    f = th.function([x] + ys, outs)
+    xv, yvs = values(left), [values(dt) for dt in ARITH_DTYPES]
+    got = f(xv, *yvs)
+    k = 0
+    for dt, yv in zip(ARITH_DTYPES, yvs):
+        up = np.result_type(left, dt)
+        both_int = np.dtype(left).kind in "iu" and np.dtype(dt).kind in "iu"
+        # The type the arithmetic happens in is C's, as in the reference's generated code: double if an operand is
+        # double, else float if an operand is floating (float16 storage computes in float32), whatever type the
+        # result is then stored in - float32 + int32 is a float32 sum stored as float64.
+        if "float64" in (left, dt):
+            ct = "float64"
+        elif both_int:
+            ct = None
+        else:
+            ct = "float32"
+        if both_int:
+            want = [xv.astype(up) + yv.astype(up), xv.astype(up) * yv.astype(up),
+                    (xv.astype("float64") / yv.astype("float64")).astype("float32"),
+                    np.floor_divide(xv.astype(up), yv.astype(up))]
+        else:
+            xc, yc = xv.astype(ct), yv.astype(ct)
+            want = [(xc + yc).astype(up), (xc * yc).astype(up), (xc / yc).astype(up), np.floor(xc / yc).astype(up)]
+        for name, g, w in zip(("add", "mul", "true_div", "int_div"), got[k:k + 4], want):
+            what = "%s %s %s" % (left, name, dt)
+            assert g.dtype == w.dtype, (what, g.dtype, w.dtype)
+            if w.dtype.kind in "iu" or name == "int_div":
+                assert np.array_equal(g, w), what                 # integers, and floors (whole numbers): exact
+            else:
+                bar = TOL["float16" if w.dtype == np.float16 else (ct or "float32")]
+                assert_parity(g, w, what, tol=bar)
+        k += 4
