@@ -432,6 +432,60 @@ def test_user_written_composite_with_several_results():
     assert np.array_equal(q, av // bv) and np.array_equal(m, av % bv)
 
 
+def test_fast_division_over_the_whole_float32_range():
+    """The default float32 division (one hardware reciprocal of the divisor's mantissa, the exponent applied in two
+    halves) over random bit patterns of the whole finite range on both sides - denormal operands, quotients that
+    overflow, underflow or land among the denormals - and the special values: within 2.5 ulp of the exact quotient
+    (1.5 units of the smallest denormal where the quotient is denormal), infinities, zeros with their signs and NaN
+    exactly where IEEE division has them.  Once with a divisor per element and once with one divisor per row (the
+    form whose divisor half the compiler computes once)."""
+    rng = np.random.default_rng(2024)
+    n = 400000
+
+    def patterns(k):
+        bits = rng.integers(0, 0x7f800000, k, dtype=np.uint32) | (rng.integers(0, 2, k, dtype=np.uint32) << 31)
+        return bits.view("float32")
+
+    special = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1.0, -1.0, 1e-45, -1e-45, 1.1754944e-38, 3.4028235e38,
+                        -3.4028235e38, 2.0 ** -126, 2.0 ** 127, 2.0 ** -149, 3.0, 1.0 / 3.0], "float32")
+    av = np.concatenate([patterns(n), np.repeat(special, len(special)), rng.uniform(-4, 4, n).astype("float32")])
+    bv = np.concatenate([patterns(n), np.tile(special, len(special)), rng.uniform(-4, 4, n).astype("float32")])
+    a, b = T.fvector("a"), T.fvector("b")
+    got = th.function([a, b], a / b)(av, bv)
+    assert "|fd" in hip.last_plan()
+
+    def check(g, x, y, what):
+        with np.errstate(all="ignore"):
+            exact = x.astype("float64") / y.astype("float64")
+            want = exact.astype("float32")
+        special_case = ~np.isfinite(want) | (want == 0) | ~np.isfinite(exact)
+        # where IEEE gives infinity, zero or NaN: the same, sign included - except at the two edges of the range,
+        # where a quotient within 2.5 ulp of the largest finite value / of the smallest denormal may round either way
+        near_top = np.isfinite(exact) & (np.abs(exact) > 3.4028e38)
+        near_zero = np.isfinite(exact) & (np.abs(exact) < 3e-45)
+        strict = special_case & ~near_top & ~near_zero
+        assert np.array_equal(g[strict], want[strict], equal_nan=True), what
+        assert np.array_equal(np.signbit(g[strict & ~np.isnan(want)]), np.signbit(want[strict & ~np.isnan(want)])), what
+        rest = ~special_case
+        ulp = np.maximum(np.spacing(np.abs(want[rest]).astype("float32")).astype("float64"), 2.0 ** -149)
+        err = np.abs(g[rest].astype("float64") - exact[rest]) / ulp
+        assert err.max() <= 2.5, (what, float(err.max()), x[rest][err.argmax()], y[rest][err.argmax()])
+        edge = near_top | near_zero
+        assert np.all(np.isinf(g[near_top]) | (np.abs(g[near_top]) >= 3.4028e38)) and np.all(np.abs(g[near_zero]) <= 4.5e-45), what
+        return float(err.max())
+
+    worst = check(got, av, bv, "divisor per element")
+    # one divisor per row
+    m = T.fmatrix("m")
+    c = T.fcol("c")
+    rows = np.concatenate([patterns(3000), special])
+    mv = np.concatenate([patterns(len(rows) * 64), ]).reshape(len(rows), 64)
+    mv[:, :len(special)] = special
+    got2 = th.function([m, c], m / c)(mv, rows.reshape(-1, 1))
+    check(got2.reshape(-1), mv.reshape(-1), np.repeat(rows, 64), "divisor per row")
+    assert worst > 0.5          # it is the approximate form that ran
+
+
 def test_exact_float32_math_when_the_fast_forms_are_switched_off(monkeypatch):
     """THX_FAST_DIV=0: float32 division and square root correctly rounded (bit-equal to
     NumPy's), exp / sigmoid from the math library (within 2 ulp of the double result); the

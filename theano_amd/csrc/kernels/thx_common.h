@@ -26,19 +26,27 @@ typedef double thx_f64;
 #define THX_DEV __device__ __forceinline__
 #define THX_WAVE 64
 
-// Single-precision division as the generated per-element code spells it.  With THX_FAST_DIV:
-// both operands scaled to [0.5, 1) by their exponents, one v_rcp_f32 (1 ulp), one multiply and the
-// exponent difference put back - within 2.5 ulp of the quotient for every finite input including
-// denormals, and 0, infinity and NaN come out as IEEE division gives them.  (The compiler flag
-// that asks for the same lowering of `/` is lost on the way through the optimiser for these
-// kernels; spelling it out is what makes it stick.)  When the divisor is shared by the elements
-// of a vector - a per-channel scale - its half of the work is done once.
+// Single-precision division as the generated per-element code spells it.  With THX_FAST_DIV: the
+// divisor b = mb * 2^eb (mb in [0.5, 1)) becomes the factor r1 = rcp(mb) * 2^-eb (one v_rcp_f32, 1 ulp) and
+// the quotient is a * r1, one rounding.  So that r1 stays a normal number for every b, the exponent it
+// carries is eb clamped to [-120, 120] and what remains of it (nothing unless |b| is beyond 2^+-120) is a
+// second, exact factor f2 = 2^(h - eb): the result is (a * r1) * f2, within 2.5 ulp of the quotient for
+// every finite input including denormals, and 0, infinity and NaN come out as IEEE division gives them.
+// The intermediate product equals the quotient in the common case; for |b| > 2^119 it is larger by at most
+// 2^8 while the quotient cannot exceed 2^9, for |b| < 2^-121 it is smaller by at most 2^-28 while a * r1
+// is at least 2^-29 for any non-zero a: it overflows or goes denormal only where the quotient does.
+// Everything but the two multiplications depends on b alone, so a divisor shared by many elements - a
+// row's sum, a per-channel scale, any loop invariant - costs two multiplications per element, where
+// scaling both operands by their exponents cost five.  (The compiler flag that asks for a 2.5-ulp lowering
+// of `/` is lost on the way through the optimiser for these kernels; spelling it out is what makes it stick.)
 #ifdef THX_FAST_DIV
 __device__ __forceinline__ float thx_fdiv(float a, float b) {
   const float mb = __builtin_amdgcn_frexp_mantf(b);
-  const float ma = __builtin_amdgcn_frexp_mantf(a);
-  const int e = __builtin_amdgcn_frexp_expf(a) - __builtin_amdgcn_frexp_expf(b);
-  return __builtin_ldexpf(ma * __builtin_amdgcn_rcpf(mb), e);
+  const int eb = __builtin_amdgcn_frexp_expf(b);
+  const int h = eb < -120 ? -120 : (eb > 120 ? 120 : eb);
+  const float r1 = __builtin_ldexpf(__builtin_amdgcn_rcpf(mb), -h);
+  const float f2 = __builtin_ldexpf(1.0f, h - eb);
+  return (a * r1) * f2;
 }
 #else
 __device__ __forceinline__ float thx_fdiv(float a, float b) { return a / b; }
