@@ -17,7 +17,7 @@ algorithmic bytes.  ``cpu_baseline`` times the oracle's C restatement of the
 reference's loops on this host.  ``other_configs`` lists the remaining four
 configurations (and max_and_argmax of the configuration-2 matrix) over input
 sets that rotate (so that no set is still cached when it is used again: ``us``,
-the median of nine runs of K steps, ``min_us`` the fastest of them) and over one
+the median of nine runs of max(K, 50) steps, ``min_us`` the fastest of them) and over one
 set (``same_input_us``), each with the symbols of the kernels it launches.  Every
 timed leg starts on a device that has been kept busy for 40 ms (``_settle``).
 """
@@ -283,18 +283,20 @@ def main():
                 f(*sets[turn[0] % len(sets)])
                 turn[0] += 1
 
-            # nine runs of K steps each on a device at its steady clocks: the median is the figure (`us`), the
-            # fastest run is listed beside it
+            # nine runs of max(K, 50) steps each on a device at its steady clocks: the median is the figure (`us`),
+            # the fastest run is listed beside it (a run of 20 steps lasts under a millisecond, and the start of each
+            # run - the first launch after the event - then weighs 0.5 - 1 us per step)
+            k_other = max(args.steps, 50)
             _settle(hip, rotating)
-            runs = sorted(_time_steps(hip, rotating, args.steps, 3)[0] for _ in range(9))
+            runs = sorted(_time_steps(hip, rotating, k_other, 3)[0] for _ in range(9))
             ms = runs[len(runs) // 2]
-            warm_ms = sorted(_time_steps(hip, lambda: f(*sets[0]), args.steps, 3)[0] for _ in range(5))[2]
+            warm_ms = sorted(_time_steps(hip, lambda: f(*sets[0]), k_other, 3)[0] for _ in range(5))[2]
             n_k = sum(1 for n in f.toposort()
                       if type(n.op).__name__ in ("HipElemwise", "HipElemwiseReduce", "HipCAReduce", "HipRowChain", "HipMaxAndArgmax"))
             with hip.profile() as p:
                 f(*sets[0])
             others[name] = _rate(W.algorithmic_bytes(name), ms)
-            others[name].update({"min_us": round(runs[0] * 1e3, 2), "input_sets": len(sets),
+            others[name].update({"min_us": round(runs[0] * 1e3, 2), "steps_per_run": k_other, "input_sets": len(sets),
                                  "same_input_us": round(warm_ms * 1e3, 2), "nodes_per_step": n_k,
                                  "kernels": sorted(_symbol(k) for k in p.kernels)})
             if name in REAL_BYTES:
