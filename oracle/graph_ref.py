@@ -6,7 +6,8 @@ Evaluates an *unlifted, unfused* theano_amd graph on the CPU the way Theano's
 own backend would node by node:
 
 * ``Elemwise``: broadcast check of ``Elemwise.perform``
-  (``theano/tensor/elemwise.py:720-740``), then the scalar op's C semantics
+  (``theano/tensor/elemwise.py:720-740``), the node's output dtype checked against the oracle's own
+  table (``oracle/dtype_rules.py``), then the scalar op's C semantics
   from ``oracle.scalar_ref`` applied to whole arrays; Composite nodes are
   evaluated op by op.
 * ``CAReduce`` family: dtype tables re-stated here from
@@ -33,7 +34,7 @@ import os
 
 import numpy as np
 
-from . import scalar_ref
+from . import dtype_rules, scalar_ref
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = os.path.join(_HERE, "_build", "liboracle.so")
@@ -163,6 +164,14 @@ def _wide(dtype):
     return "float64" if str(dtype) in ("float16", "float32") else str(dtype)
 
 
+def _check_dtypes(scalar_op, node):
+    """The node's output dtype against the oracle's own table: the dtype the product's make_node
+    inferred is not taken on trust."""
+    from theano_amd import config
+    dtype_rules.check_node(scalar_op, [i.type.dtype for i in node.inputs], [o.type.dtype for o in node.outputs],
+                           floatX=config.floatX, cast_policy=config.cast_policy)
+
+
 def eval_scalar_op(op, in_values, out_dtypes, wide=False):
     """Evaluate a theano_amd ScalarOp (or Composite) over whole arrays."""
     name = type(op).__name__
@@ -173,6 +182,7 @@ def eval_scalar_op(op, in_values, out_dtypes, wide=False):
         from theano_amd import gof
         env = dict(zip(op.inputs, in_values))
         for node in gof.io_toposort(op.inputs, op.outputs):
+            _check_dtypes(node.op, node)
             args = [env[i] if i in env else np.asarray(i.data) for i in node.inputs]
             outs = eval_scalar_op(node.op, args, [o.type.dtype for o in node.outputs], wide)
             for o, v in zip(node.outputs, outs):
@@ -299,6 +309,7 @@ def evaluate(inputs, outputs, values, wide=False):
         op = node.op
         if isinstance(op, Elemwise):
             _check_broadcast(node, args)
+            _check_dtypes(op.scalar_op, node)
             res = eval_scalar_op(op.scalar_op, args, [o.type.dtype for o in node.outputs], wide)
             shape = np.broadcast_shapes(*[a.shape for a in args])
             res = [np.broadcast_to(r, shape).astype(odt(o), copy=False) if o.type.dtype != "bool"
