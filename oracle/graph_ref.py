@@ -323,9 +323,11 @@ def evaluate(inputs, outputs, values, wide=False):
             if isinstance(op, CAReduceDtype):
                 out_dt = op.dtype if op.dtype is not None else SUM_OUT_DTYPE.get(idt, idt)
                 acc_dt = op.acc_dtype if op.acc_dtype is not None else SUM_ACC_DTYPE.get(idt, idt)
-            else:
-                out_dt = node.outputs[0].type.dtype
+            else:                                   # elemwise.py:1273-1274; All / Any: 1597-1598, 1628-1629
+                out_dt = "bool" if type(op).__name__ in ("All", "Any") else idt
                 acc_dt = "bool" if out_dt == "bool" else idt
+            assert node.outputs[0].type.dtype == out_dt, "%s of %s is %s, the reference gives %s" % (
+                op, idt, node.outputs[0].type.dtype, out_dt)
             if acc_dt == "float32" and idt == "float16":
                 x = x.astype("float32")
             if wide:
