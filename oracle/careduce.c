@@ -73,25 +73,30 @@ typedef struct {
   DEFINE_REDUCE(add_##IN_N##_##ACC_N, IN_T, ACC_T, acc = acc + x)          \
   DEFINE_REDUCE(mul_##IN_N##_##ACC_N, IN_T, ACC_T, acc = acc * x)
 
-SUMPROD(bool, uint8_t, i64, int64_t)
-SUMPROD(i8, int8_t, i64, int64_t)
-SUMPROD(i16, int16_t, i64, int64_t)
-SUMPROD(i32, int32_t, i64, int64_t)
-SUMPROD(i64, int64_t, i64, int64_t)
-SUMPROD(u8, uint8_t, u64, uint64_t)
-SUMPROD(u16, uint16_t, u64, uint64_t)
-SUMPROD(u32, uint32_t, u64, uint64_t)
-SUMPROD(u64, uint64_t, u64, uint64_t)
-SUMPROD(f32, float, f64, double)
-SUMPROD(f32, float, f32, float)
-SUMPROD(f64, double, f64, double)
-SUMPROD(i8, int8_t, i8, int8_t)
-SUMPROD(i16, int16_t, i16, int16_t)
-SUMPROD(i32, int32_t, i32, int32_t)
-SUMPROD(u8, uint8_t, u8, uint8_t)
-SUMPROD(i32, int32_t, f64, double)
-SUMPROD(i64, int64_t, f64, double)
-SUMPROD(i8, int8_t, f32, float)
+/* every input type with every accumulator type a caller may ask for (acc_dtype=..., elemwise.py:1760-1780);
+ * float16 inputs arrive converted to float32, bool and float16 accumulators have no C code */
+#define SUMPROD_INTO(ACC_N, ACC_T)       \
+  SUMPROD(bool, uint8_t, ACC_N, ACC_T)   \
+  SUMPROD(i8, int8_t, ACC_N, ACC_T)      \
+  SUMPROD(u8, uint8_t, ACC_N, ACC_T)     \
+  SUMPROD(i16, int16_t, ACC_N, ACC_T)    \
+  SUMPROD(u16, uint16_t, ACC_N, ACC_T)   \
+  SUMPROD(i32, int32_t, ACC_N, ACC_T)    \
+  SUMPROD(u32, uint32_t, ACC_N, ACC_T)   \
+  SUMPROD(i64, int64_t, ACC_N, ACC_T)    \
+  SUMPROD(u64, uint64_t, ACC_N, ACC_T)   \
+  SUMPROD(f32, float, ACC_N, ACC_T)      \
+  SUMPROD(f64, double, ACC_N, ACC_T)
+SUMPROD_INTO(i8, int8_t)
+SUMPROD_INTO(u8, uint8_t)
+SUMPROD_INTO(i16, int16_t)
+SUMPROD_INTO(u16, uint16_t)
+SUMPROD_INTO(i32, int32_t)
+SUMPROD_INTO(u32, uint32_t)
+SUMPROD_INTO(i64, int64_t)
+SUMPROD_INTO(u64, uint64_t)
+SUMPROD_INTO(f32, float)
+SUMPROD_INTO(f64, double)
 
 /* theano/tensor/elemwise.py:2075-2077 with x = accumulator, y = element */
 #define MULNZSTMT acc = ((acc == 0) ? (x) : (((x) == 0) ? (acc) : ((x) * (acc))))
@@ -140,15 +145,17 @@ typedef struct {
 
 #define E(OP, IN, ACC, NAME) {OP, IN, ACC, (reduce_fn)NAME}
 #define ESP(INC, INN, ACCC, ACCN) E(OP_ADD, INC, ACCC, add_##INN##_##ACCN), E(OP_MUL, INC, ACCC, mul_##INN##_##ACCN)
+#define ESP_INTO(ACCC, ACCN)                                                                                   \
+  ESP(T_BOOL, bool, ACCC, ACCN), ESP(T_I8, i8, ACCC, ACCN), ESP(T_U8, u8, ACCC, ACCN), ESP(T_I16, i16, ACCC, ACCN),  \
+      ESP(T_U16, u16, ACCC, ACCN), ESP(T_I32, i32, ACCC, ACCN), ESP(T_U32, u32, ACCC, ACCN),                     \
+      ESP(T_I64, i64, ACCC, ACCN), ESP(T_U64, u64, ACCC, ACCN), ESP(T_F32, f32, ACCC, ACCN),                     \
+      ESP(T_F64, f64, ACCC, ACCN)
 #define EMM(C, N) E(OP_MAX, C, C, max_##N##_##N), E(OP_MIN, C, C, min_##N##_##N)
 #define EBIT(C, N) E(OP_AND, C, C, and_##N##_##N), E(OP_OR, C, C, or_##N##_##N), E(OP_XOR, C, C, xor_##N##_##N)
 
 static const entry_t table[] = {
-    ESP(T_BOOL, bool, T_I64, i64), ESP(T_I8, i8, T_I64, i64),   ESP(T_I16, i16, T_I64, i64), ESP(T_I32, i32, T_I64, i64),
-    ESP(T_I64, i64, T_I64, i64),   ESP(T_U8, u8, T_U64, u64),   ESP(T_U16, u16, T_U64, u64), ESP(T_U32, u32, T_U64, u64),
-    ESP(T_U64, u64, T_U64, u64),   ESP(T_F32, f32, T_F64, f64), ESP(T_F32, f32, T_F32, f32), ESP(T_F64, f64, T_F64, f64),
-    ESP(T_I8, i8, T_I8, i8),       ESP(T_I16, i16, T_I16, i16), ESP(T_I32, i32, T_I32, i32), ESP(T_U8, u8, T_U8, u8),
-    ESP(T_I32, i32, T_F64, f64),   ESP(T_I64, i64, T_F64, f64), ESP(T_I8, i8, T_F32, f32),
+    ESP_INTO(T_I8, i8),   ESP_INTO(T_U8, u8),   ESP_INTO(T_I16, i16), ESP_INTO(T_U16, u16), ESP_INTO(T_I32, i32),
+    ESP_INTO(T_U32, u32), ESP_INTO(T_I64, i64), ESP_INTO(T_U64, u64), ESP_INTO(T_F32, f32), ESP_INTO(T_F64, f64),
     EMM(T_F32, f32),  EMM(T_F64, f64),  EMM(T_BOOL, bool), EMM(T_I8, i8),   EMM(T_U8, u8),   EMM(T_I16, i16),
     EMM(T_U16, u16),  EMM(T_I32, i32),  EMM(T_U32, u32),   EMM(T_I64, i64), EMM(T_U64, u64),
     EBIT(T_BOOL, bool), EBIT(T_I8, i8), EBIT(T_U8, u8), EBIT(T_I16, i16), EBIT(T_U16, u16), EBIT(T_I32, i32),

@@ -91,6 +91,8 @@ def careduce(x, op_name, axis, acc_dtype, out_dtype):
     if op_name in ("Maximum", "Minimum") and any(x.shape[a] == 0 for a in axis):
         raise ValueError("Input of CAReduce{%s} has zero-size on axis %s" % (op_name.lower(), axis))
     acc_dtype, out_dtype = str(acc_dtype), str(out_dtype)
+    if not axis:        # no axis: the reference emits an identity Elemwise, no accumulator (elemwise.py:1410-1417)
+        return np.array(x).astype(out_dtype) if out_dtype != "bool" else np.array(x) != 0
     if x.dtype.kind == "c":
         # complex sums and products: the accumulator type's own + and * over the reduced elements (the reference's
         # struct operators, theano/scalar/basic.py:518-548, which are NumPy's up to the last place); NumPy adds
@@ -326,8 +328,13 @@ def evaluate(inputs, outputs, values, wide=False):
             else:                                   # elemwise.py:1273-1274; All / Any: 1597-1598, 1628-1629
                 out_dt = "bool" if type(op).__name__ in ("All", "Any") else idt
                 acc_dt = "bool" if out_dt == "bool" else idt
-            assert node.outputs[0].type.dtype == out_dt, "%s of %s is %s, the reference gives %s" % (
-                op, idt, node.outputs[0].type.dtype, out_dt)
+            decl = node.inputs[0].type.dtype            # as declared: ``idt`` is already float64 in wide mode
+            if isinstance(op, CAReduceDtype):
+                want = op.dtype if op.dtype is not None else SUM_OUT_DTYPE.get(decl, decl)
+            else:
+                want = "bool" if out_dt == "bool" else decl
+            assert node.outputs[0].type.dtype == want, "%s of %s is %s, the reference gives %s" % (
+                op, node.inputs[0].type.dtype, node.outputs[0].type.dtype, want)
             if acc_dt == "float32" and idt == "float16":
                 x = x.astype("float32")
             if wide:

@@ -285,3 +285,46 @@ def test_device_operands_without_an_address_are_refused_before_any_launch():
         assert runtime.lib.thx_reduce_call(rhandle, ins, mask, outs, 0) == 7
         assert b"no base address" in runtime.lib.thx_last_error()
     runtime.lib.thx_reduce_free(rhandle)
+
+
+def _damaged_cache_round_trip(tmp_path, dry):
+    import subprocess
+    import sys
+    prog = ("import numpy as np, theano_amd as th, theano_amd.tensor as T\n"
+            "from theano_amd import hip\n"
+            "from theano_amd.hip import runtime\n"
+            "hip.set_dry_run(%r)\n"
+            "x = T.fvector()\n"
+            "print(th.function([x], x * 3 + 1)(np.arange(5, dtype='float32')).tolist(), runtime.cache_stats())\n" % dry)
+    env = dict(os.environ, THX_CACHE_DIR=str(tmp_path), PYTHONPATH=os.path.dirname(os.path.dirname(__file__)))
+
+    def run():
+        res = subprocess.run([sys.executable, "-c", prog], capture_output=True, text=True, timeout=300, env=env)
+        assert res.returncode == 0, res.stdout + res.stderr
+        assert dry or res.stdout.startswith("[1.0, 4.0, 7.0, 10.0, 13.0]"), res.stdout
+        stats = eval(res.stdout[res.stdout.index("]") + 1:])
+        return stats["compiled"], stats["disk_hits"]
+
+    compiled, disk = run()
+    files = sorted(tmp_path.glob("*.hsaco"))
+    assert compiled >= 1 and disk == 0 and len(files) == compiled
+    assert run() == (0, compiled)                           # served from the disk
+    for k, f in enumerate(files):
+        blob = f.read_bytes()
+        f.write_bytes(blob[:len(blob) // 2] if k % 2 == 0 else b"not a code object")
+    assert run() == (compiled, 0)                           # every one built again
+    assert run() == (0, compiled)                           # and the files on the disk are good again
+    blob = files[0].read_bytes()
+    files[0].write_bytes(blob[:-1])                         # one byte short: the section table ends outside the file
+    assert run()[0] == 1
+
+
+def test_a_damaged_cached_code_object_is_rebuilt(tmp_path):
+    """A file in the kernel cache that is not a whole code object (cut in half, one byte short, something else
+    altogether) is never handed to the module loader: it is dropped and the kernel is compiled again."""
+    _damaged_cache_round_trip(tmp_path, True)
+
+
+@pytest.mark.gpu
+def test_a_damaged_cached_code_object_is_rebuilt_and_runs(tmp_path):
+    _damaged_cache_round_trip(tmp_path, False)

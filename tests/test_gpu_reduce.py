@@ -648,3 +648,88 @@ def test_max_of_a_computed_value_and_its_gradient_see_the_same_bits():
             assert np.isfinite(gv).all()
             at_max = ev == ev.max(axis=axis, keepdims=True)
             assert np.array_equal(gv != 0, at_max & (gv != 0)) and (np.abs(gv) > 0).any(axis=axis).all(), axis
+
+
+REAL_DTYPES = ("bool", "int8", "int16", "int32", "int64", "uint8", "uint16", "uint32", "uint64", "float16", "float32",
+               "float64")
+T_REDUCE_AXES = [None, 0, 1, [], [0], [1], [0, 1]]        # theano/tensor/tests/test_elemwise.py:816
+
+
+def _reduce_dtype_data(rng, dtype, method, narrow):
+    data = (rng.random((3, 4)) * 10).astype(dtype)         # test_elemwise.py:891-892
+    return data[0:1] if method == "prod" and narrow else data
+
+
+def _check_integer_of_a_float_accumulation(x, var, data, what):
+    """A floating-point accumulation cast to an integer at the end: the accumulator's rounding depends on the
+    order of the operations, so the integer agrees to a float32 accumulator's accuracy and to one unit, not bit
+    for bit."""
+    got = th.function([x], var)(data)
+    ref = G.evaluate([x], [var], [data])[0]
+    assert got.dtype == ref.dtype and got.shape == ref.shape, what
+    g, r = got.astype("float64"), ref.astype("float64")
+    assert np.all(abs(g - r) <= 1 + 1e-6 * abs(r)), (what, got, ref)
+
+
+@pytest.mark.parametrize("method", ["sum", "prod"])
+def test_custom_output_dtype_of_every_real_pair(method):
+    """``T_reduce_dtype.test_reduce_custom_dtype`` (``theano/tensor/tests/test_elemwise.py:874-912``, run on the
+    device by ``T_gpureduce_dtype``, ``theano/gpuarray/tests/test_elemwise.py:367-381``): every input dtype with every
+    requested output dtype, the axis cycling through the reference's list; the reference only runs the function,
+    here the value is held against the oracle (exact for integer results)."""
+    rng = np.random.default_rng(41)
+    idx = 0
+    for input_dtype in REAL_DTYPES:
+        x = T.matrix(dtype=input_dtype)
+        for output_dtype in REAL_DTYPES:
+            axis = T_REDUCE_AXES[idx % len(T_REDUCE_AXES)]
+            var = getattr(x, method)(dtype=output_dtype, axis=axis)
+            assert var.dtype == output_dtype
+            narrow = output_dtype in ("float16", "int8", "uint8", "int16", "uint16")
+            data = _reduce_dtype_data(rng, input_dtype, method, narrow)
+            # float16 is accumulated in float32: a wider result carries that accumulator's rounding
+            tol = (dict(rtol=1e-5, atol=1e-6) if input_dtype == "float16" and output_dtype == "float64" else
+                   dict(rtol=1e-12, atol=1e-12) if output_dtype == "float64" else None)
+            what = "%s %s -> %s axis %s" % (method, input_dtype, output_dtype, axis)
+            if input_dtype.startswith("float") and not output_dtype.startswith("float"):
+                _check_integer_of_a_float_accumulation(x, var, data, what)
+            else:
+                check(x, var, data, what, tol)
+            idx += 1
+
+
+@pytest.mark.parametrize("method", ["sum", "prod"])
+def test_custom_accumulator_dtype_of_every_real_pair(method):
+    """``T_reduce_dtype.test_reduce_custom_acc_dtype`` (``theano/tensor/tests/test_elemwise.py:914-950``): an
+    accumulator that would lose precision is a TypeError, a float16 one is turned away when the kernel is
+    built, every other one runs and matches the oracle's accumulation in that dtype."""
+    from theano_amd import scalar as scal
+    rng = np.random.default_rng(42)
+    idx = 0
+    for input_dtype in REAL_DTYPES:
+        x = T.matrix(dtype=input_dtype)
+        for acc_dtype in REAL_DTYPES:
+            axis = T_REDUCE_AXES[idx % len(T_REDUCE_AXES)]
+            idx += 1
+            up = scal.upcast(input_dtype, acc_dtype)
+            if acc_dtype == up or (input_dtype in T.discrete_dtypes and acc_dtype in T.continuous_dtypes):
+                var = getattr(x, method)(acc_dtype=acc_dtype, axis=axis)
+                assert var.owner.op.acc_dtype == acc_dtype
+                if acc_dtype == "bool":             # 1 + 1 stored in an npy_bool: the reference's C code leaves a 2 in
+                    continue                        # a boolean and its Python path an or - nothing to hold a value to
+                if acc_dtype == "float16" and axis != []:   # no C code for it in the reference either (elemwise.py:1395-1398);
+                    # over no axis at all nothing is accumulated (elemwise.py:1410-1417)
+                    with pytest.raises(NotImplementedError, match="float16 accumulators"):
+                        th.function([x], var)(np.ones((3, 4), input_dtype))
+                    continue
+                narrow = acc_dtype in ("float16", "int8", "uint8", "int16", "uint16") or var.dtype == "float16"
+                data = _reduce_dtype_data(rng, input_dtype, method, narrow)
+                tol = dict(rtol=1e-12, atol=1e-12) if var.dtype == "float64" and acc_dtype == "float64" else None
+                what = "%s %s acc %s axis %s" % (method, input_dtype, acc_dtype, axis)
+                if acc_dtype.startswith("float") and not var.dtype.startswith("float"):
+                    _check_integer_of_a_float_accumulation(x, var, data, what)
+                else:
+                    check(x, var, data, what, tol)
+            else:
+                with pytest.raises(TypeError):
+                    getattr(x, method)(acc_dtype=acc_dtype, axis=axis)

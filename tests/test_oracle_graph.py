@@ -86,6 +86,36 @@ def test_strided_and_transposed_inputs():
     assert np.allclose(G.careduce(v, "Add", (0, 2), "float64", "float32"), v.astype("float64").sum((0, 2)), rtol=1e-6)
 
 
+def test_every_accumulator_a_caller_may_ask_for():
+    """Sums and products of every real input type in every accumulator type that ``acc_dtype=`` accepts
+    (theano/tensor/elemwise.py:1760-1780): integer accumulators against NumPy's modular ``ufunc.reduce(dtype=acc)``,
+    floating-point ones against a loop over the elements in that type's own NumPy scalars."""
+    rng = np.random.default_rng(7)
+    reals = ("bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64", "float32", "float64")
+    for idt in reals:
+        x = (rng.random((5, 7)) * 10).astype(idt) if idt != "bool" else rng.random((5, 7)) < 0.6
+        for acc in reals[1:]:
+            up = str(np.promote_types(idt, acc))
+            if not (acc == up or (np.dtype(idt).kind in "biu" and np.dtype(acc).kind == "f")):
+                continue                                        # refused as a loss of precision
+            for name, ufunc in (("Add", np.add), ("Mul", np.multiply)):
+                got = G.careduce(x, name, (1,), acc, acc)
+                assert got.dtype == np.dtype(acc)
+                if np.dtype(acc).kind in "iu":
+                    with np.errstate(over="ignore"):
+                        want = ufunc.reduce(x, axis=1, dtype=acc)
+                    assert np.array_equal(got, want), (idt, acc, name)
+                else:
+                    t = np.dtype(acc).type
+                    want = []
+                    for row in x:
+                        a = t(0) if name == "Add" else t(1)
+                        for v in row:       # C: a floating accumulator at least as wide as x makes the common type its own
+                            a = t(ufunc(a, t(v)))
+                        want.append(a)
+                    assert np.array_equal(got, np.asarray(want, acc)), (idt, acc, name)
+
+
 def test_dtype_tables_of_the_product_match_reference_literals():
     # theano/tensor/tests/test_elemwise.py:828-836 and :854-865
     out_tbl = dict(bool="int64", int8="int64", int16="int64", int32="int64", uint8="uint64", uint16="uint64",

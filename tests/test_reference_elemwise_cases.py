@@ -311,3 +311,38 @@ def test_composite_cases_of_the_scalar_tests():
     a, b, cc, d = scal.int8(), scal.int8(), scal.float32(), scal.float32()
     rebuilt = sop.make_node(a * d, b, cc)
     assert rebuilt.op.inputs_type[0].dtype == "float32"
+
+
+def test_softmax_quotient_in_both_spellings_compiles_to_one_row_node(dry_run):
+    """``Test_softmax_opt.test_basic`` and ``test_basic_keepdims``
+    (``theano/tensor/nnet/tests/test_nnet.py:1472-1505``): ``exp(c) / exp(c).sum(axis=1)`` with the sum brought back
+    by ``dimshuffle(0, 'x')`` or by ``keepdims=True`` is recognised as the softmax op - here: one row-chain node
+    and no division node beside it."""
+    for spell in (lambda c: T.exp(c) / T.exp(c).sum(axis=1).dimshuffle(0, "x"),
+                  lambda c: T.exp(c) / T.exp(c).sum(axis=1, keepdims=True)):
+        c = T.matrix()
+        f = th.function([c], spell(c))
+        work = [type(n.op).__name__ for n in f.toposort() if type(n.op).__name__.startswith("Hip")
+                and type(n.op).__name__ not in ("HostToHip", "HipToHost")]
+        assert work == ["HipRowChain"], work
+
+
+@pytest.mark.gpu
+def test_bitwise_operators_on_signed_integers():
+    """``test_bitwise`` (``theano/tensor/tests/test_basic.py:4772-4819``): ``|``, ``^``, ``&`` and ``~`` on int8 ..
+    int64 vectors against Python's operators on the same arrays, and ``xor_inplace`` leaves its result in the
+    caller's array as well."""
+    from theano_amd.tensor import inplace
+    for dtype in ("int8", "int16", "int32", "int64"):
+        x, y = T.vector(dtype=dtype), T.vector(dtype=dtype)
+        l, r = np.asarray([0, 0, 1, 1], dtype=dtype), np.asarray([0, 1, 0, 1], dtype=dtype)
+        for expr, want in ((x | y, l | r), (x ^ y, l ^ r), (x & y, l & r)):
+            v = th.function([x, y], expr)(l, r)
+            assert v.dtype == np.dtype(dtype) and np.array_equal(v, want), (dtype, v, want)
+        v = th.function([x, y], inplace.xor_inplace(x, y), accept_inplace=True)(l, r)
+        assert np.array_equal(v, [0, 1, 1, 0]) and np.array_equal(l, [0, 1, 1, 0])     # "test the in-place stuff"
+        fn = th.function([x], ~x)
+        top = np.iinfo(dtype).max
+        for vals in ([0, 0, 1, 1], [0, 1, 0, 1], [-1, top, top - 1, np.iinfo(dtype).min]):
+            a = np.asarray(vals, dtype=dtype)
+            assert np.array_equal(fn(a), ~a), (dtype, a)

@@ -385,6 +385,33 @@ static int compile_source(const std::string& src, const std::string& arch, std::
   return THX_OK;
 }
 
+// Is `b` a whole 64-bit ELF file?  The module loader does not check what it is given - half a code object or
+// a file of something else ends the process inside it - so a cached file is loaded only if its header, its
+// program and section header tables and every section's bytes lie inside the file (the section header table is
+// the last thing in a code object: a file that was cut short fails here).
+static bool elf_complete(const std::vector<char>& b) {
+  const size_t n = b.size();
+  if (n < 64 || memcmp(b.data(), "\177ELF", 4) != 0 || b[4] != 2 /* ELFCLASS64 */ || b[5] != 1 /* little-endian */) return false;
+  auto u16 = [&](size_t off) { uint16_t v; memcpy(&v, b.data() + off, 2); return (uint64_t)v; };
+  auto u32 = [&](size_t off) { uint32_t v; memcpy(&v, b.data() + off, 4); return (uint64_t)v; };
+  auto u64 = [&](size_t off) { uint64_t v; memcpy(&v, b.data() + off, 8); return v; };
+  auto inside = [&](uint64_t off, uint64_t len) { return off <= n && len <= n - off; };
+  const uint64_t phoff = u64(0x20), shoff = u64(0x28);
+  const uint64_t phentsize = u16(0x36), phnum = u16(0x38), shentsize = u16(0x3a), shnum = u16(0x3c);
+  if (!shnum || shentsize < 64 || !inside(shoff, shentsize * shnum)) return false;
+  if (phnum && (phentsize < 56 || !inside(phoff, phentsize * phnum))) return false;
+  for (uint64_t i = 0; i < shnum; ++i) {
+    const size_t h = (size_t)(shoff + i * shentsize);
+    if (u32(h + 4) == 8 /* SHT_NOBITS: no bytes in the file */) continue;
+    if (!inside(u64(h + 0x18), u64(h + 0x20))) return false;
+  }
+  for (uint64_t i = 0; i < phnum; ++i) {
+    const size_t h = (size_t)(phoff + i * phentsize);
+    if (!inside(u64(h + 0x08), u64(h + 0x20))) return false;   // p_offset, p_filesz
+  }
+  return true;
+}
+
 int get_kernel(const std::string& source, const std::string& entry, Kernel* out) {
   std::lock_guard<std::mutex> lk(g_mu);
   const std::string arch = target_arch();
@@ -406,10 +433,26 @@ int get_kernel(const std::string& source, const std::string& entry, Kernel* out)
   std::vector<char> code;
   const std::string& dir = cache_dir();
   const std::string path = dir.empty() ? "" : dir + "/" + h + ".hsaco";
+  Kernel k;
   if (!path.empty()) {
     std::ifstream f(path, std::ios::binary);
     if (f) {
       code.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+      // A cached file that is not a whole code object (cut short, overwritten), or one the device will
+      // not load, is dropped and built again.
+      bool good = !code.empty() && elf_complete(code);
+      if (good && have_device &&
+          (hipModuleLoadData(&k.module, code.data()) != hipSuccess ||
+           hipModuleGetFunction(&k.func, k.module, entry.c_str()) != hipSuccess)) {
+        (void)hipGetLastError();
+        if (k.module) (void)hipModuleUnload(k.module);
+        k = Kernel();
+        good = false;
+      }
+      if (!good) {
+        code.clear();
+        unlink(path.c_str());
+      }
       if (!code.empty()) ++g_n_disk;
     }
   }
@@ -424,7 +467,7 @@ int get_kernel(const std::string& source, const std::string& entry, Kernel* out)
       if (f) {
         f.write(code.data(), (std::streamsize)code.size());
         f.close();
-        if (rename(tmp.c_str(), path.c_str()) != 0) unlink(tmp.c_str());
+        if (!f || rename(tmp.c_str(), path.c_str()) != 0) unlink(tmp.c_str());   // a short write (disk full) is not kept
       }
     }
   }
@@ -432,9 +475,14 @@ int get_kernel(const std::string& source, const std::string& entry, Kernel* out)
     *out = Kernel();
     return THX_OK;
   }
-  Kernel k;
-  THX_HIP_CHECK(hipModuleLoadData(&k.module, code.data()));
-  THX_HIP_CHECK(hipModuleGetFunction(&k.func, k.module, entry.c_str()));
+  if (!k.func) {
+    THX_HIP_CHECK(hipModuleLoadData(&k.module, code.data()));
+    hipError_t fe = hipModuleGetFunction(&k.func, k.module, entry.c_str());
+    if (fe != hipSuccess) {
+      (void)hipModuleUnload(k.module);
+      return fail(THX_ERR_HIP, "hipModuleGetFunction(%s): %s", entry.c_str(), hipGetErrorString(fe));
+    }
+  }
   g_kernels[h] = k;
   *out = k;
   return THX_OK;
@@ -558,8 +606,11 @@ int thx_pool_trim(void) {
   if (!rt().ready) return THX_OK;
   THX_HIP_CHECK(hipStreamSynchronize(rt().stream));
   for (auto& kv : g_free) {
-    for (void* q : kv.second) THX_HIP_CHECK(hipFree(q));
-    kv.second.clear();
+    while (!kv.second.empty()) {
+      void* q = kv.second.back();
+      kv.second.pop_back();  // off the list before the call: a failed hipFree must not leave it to be handed out
+      THX_HIP_CHECK(hipFree(q));
+    }
   }
   return THX_OK;
 }
