@@ -331,7 +331,7 @@ def test_max_and_argmax_interface(dry_run):
     with pytest.raises(ValueError):
         T.max_and_argmax(x, axis=3)
     # d argmax / dx is zero; d max / dx marks the positions equal to the maximum
-    g = th.grad(T.sum(T.cast(T.argmax(x, axis=0), "float32")), x, disconnected_inputs="zero")
+    g = th.grad(T.sum(T.cast(T.argmax(x, axis=0), "float32")), x, disconnected_inputs="ignore")
     f = th.function([x], g)
     assert not ops_of(f, HipMaxAndArgmax)
     # nothing reads the argmax: a plain max reduction runs
@@ -1220,3 +1220,77 @@ def test_reshape_with_a_shape_vector_argument(dry_run):
     assert str(z.owner.op) == "Alloc{in1[0], mul(in1[1], 2)}"
     g = th.function([s], z)
     assert [type(n.op).__name__ for n in g.toposort()] == ["HipAlloc", "HipToHost"] and g([3, 4]).shape == (3, 8)
+
+
+def test_grad_arguments_of_the_reference(dry_run):
+    """``theano.grad``'s arguments and corner cases as the reference's tests state them
+    (``theano/tests/test_gradient.py``: test_grad_name :205, test_downcast_dtype :394, test_grad_constant :414,
+    test_dxdx :487, test_known_grads_integers :504, test_undefined_cost_grad :522, test_disconnected_cost_grad :540,
+    TestConsiderConstant :603-640, TestDisconnectedGrad :698-770)."""
+    import inspect
+    import warnings
+    from theano_amd import gradient as GR
+    from oracle import graph_ref as G
+    fx = lambda v: np.asarray(v, th.config.floatX)                          # noqa: E731
+    assert list(inspect.signature(th.grad).parameters) == [
+        "cost", "wrt", "consider_constant", "disconnected_inputs", "add_names", "known_grads", "return_disconnected",
+        "null_gradients"]
+    assert inspect.signature(th.grad).parameters["disconnected_inputs"].default == "raise"
+    # names
+    x, A = T.vector("x"), T.matrix("A")
+    f = T.sum(x * T.sum(A * x.dimshuffle("x", 0), axis=1))
+    f.name = "f"
+    assert th.grad(f, x).name == "(df/dx)" and th.grad(f, x, add_names=False).name is None
+    # what flows back to a float32 variable is float32, whatever the cost was promoted to
+    xs = T.fscalar("x")
+    y = xs * 2
+    z = T.lscalar("z")
+    c = y + z
+    dc_dx, dc_dy, dc_dz, dc_dc = th.grad(c, [xs, y, z, c])
+    assert dc_dx.dtype == "float32" and all(g.dtype in ("float32", "float64") for g in (dc_dy, dc_dz, dc_dc))
+    # a tuple in, a tuple out
+    assert isinstance(th.grad(c, (xs, y)), tuple) and isinstance(th.grad(c, [xs, y]), list)
+    # consider_constant stops what goes through an expression, not what arrives at it
+    a, b = T.scalar("a"), T.scalar("b")
+    g_a = th.grad(a + b, a, consider_constant=[a])
+    assert float(G.evaluate([a, b], [g_a], [fx(1.0), fx(0.5)])[0]) == 1.0
+    w = a * 3
+    with pytest.raises(GR.DisconnectedInputError):
+        th.grad(w + b, a, consider_constant=[w])
+    g = th.grad(w * w + a, a, consider_constant=[w])                        # only the direct term survives
+    assert float(G.evaluate([a], [g], [fx(2.0)])[0]) == 1.0
+    # d x / d x of an integer is 1
+    i = T.iscalar("i")
+    assert float(G.evaluate([i], [th.grad(i, i)], [np.int32(12)])[0]) == 1.0
+    ge = T.scalar("ge")
+    g = th.grad(cost=None, known_grads={i: ge}, wrt=i)
+    assert float(G.evaluate([ge], [g], [fx(0.6)])[0]) == np.asarray(0.6, th.config.floatX)
+    # a cost declared undefined / disconnected through known_grads
+    j = T.iscalar("j")
+    cost = i + j
+    with pytest.raises(GR.NullTypeGradError):
+        th.grad(cost, [i, j], known_grads={cost: GR.NullType()()})
+    assert isinstance(th.grad(cost, i, known_grads={cost: GR.NullType()()}, null_gradients="return").type, GR.NullType)
+    with pytest.raises(GR.DisconnectedInputError):
+        th.grad(cost, [i, j], known_grads={cost: GR.DisconnectedType()()}, disconnected_inputs="raise")
+    # what comes back for a variable outside the graph
+    u = T.vector("u")
+    with pytest.raises(GR.DisconnectedInputError):
+        th.grad(T.sum(x), u)
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        zero = th.grad(T.sum(x), u, disconnected_inputs="warn")
+    assert len(seen) == 1 and "not part of the computational graph" in str(seen[0].message)
+    assert np.array_equal(G.evaluate([u], [zero], [fx(np.ones(3))])[0], np.zeros(3))
+    assert th.grad(T.sum(x), u, disconnected_inputs="ignore", return_disconnected="None") is None
+    d = th.grad(T.sum(x), u, disconnected_inputs="ignore", return_disconnected="Disconnected")
+    assert isinstance(d.type, GR.DisconnectedType)
+    for bad in (dict(disconnected_inputs="zero"), dict(return_disconnected="none"), dict(null_gradients="ignore")):
+        with pytest.raises(ValueError):
+            th.grad(T.sum(x), x, **bad)
+    # reaching the cost through an integer-valued result only: connected, zeros
+    gz = th.grad(T.sum(T.cast(T.gt(x, 0), "float32")), x)
+    assert np.array_equal(G.evaluate([x], [gz], [fx(np.arange(3.0))])[0], np.zeros(3))
+    # the first operand of fill is not connected (theano/scalar/basic.py:2283-2287)
+    with pytest.raises(GR.DisconnectedInputError):
+        th.grad(T.sum(T.fill(x, a)), x)

@@ -267,3 +267,29 @@ def test_numpy_floatx_policy_for_python_literals():
     with config.change_flags(cast_policy="custom", floatX="float32"):
         assert scal.convert(1.1).dtype == np.float32 and scal.convert(3).dtype == np.int8
         assert scal.upcast("int32", "float32") == "float64"
+
+
+def test_older_spellings_of_flatten_stack_and_the_like_constructors():
+    """``flatten(x, outdim=)`` (``theano/tensor/basic.py:5252-5262``), ``stack(a, b, c)`` and the keyword forms
+    (``:4678-4705``), ``zeros_like(..., opt=True)`` (``:2542-2547``), ``mean(op=True)`` (``:3328-3344``)."""
+    import warnings
+    x = T.tensor3("x")
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        assert T.flatten(x, outdim=2).type.ndim == 2 and T.flatten(x).type.ndim == 1
+        a, b = T.matrix("a"), T.matrix("b")
+        old = T.stack(a, b)
+    with pytest.raises(ValueError):
+        T.flatten(x, ndim=2, outdim=2)
+    new = T.stack([a, b])
+    assert old.type == new.type and old.type.ndim == 3
+    assert T.stack([a, b], 2).type == T.stack([a, b], axis=2).type == T.stack(tensors=[a, b], axis=2).type
+    with pytest.raises(Exception):
+        T.stack([])
+    s = T.scalar("s", dtype="float32")
+    z = T.zeros_like(s, opt=True)
+    assert z.owner is None and z.type == s.type and float(z.data) == 0.0
+    assert T.zeros_like(a, opt=True).owner is not None          # a matrix still needs the fill
+    assert T.ones_like(s, dtype="int8", opt=True).owner is not None    # another dtype is another type
+    with pytest.raises(NotImplementedError):
+        T.mean(a, op=True)

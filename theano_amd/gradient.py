@@ -3,7 +3,7 @@
 A reduced form of ``theano/gradient.py`` (``grad`` :414, ``_populate_grad_dict``
 :977-1430): walk the nodes between ``wrt`` and ``cost`` from the cost down,
 ask every op for ``L_op(inputs, outputs, output_grads)`` and accumulate the
-terms per variable.  Disconnected inputs yield zeros.
+terms per variable.
 """
 import numpy as np
 
@@ -54,14 +54,43 @@ def grad_undefined(op, x_pos, x, comment=""):
                     "mathematically undefined. %s" % (x_pos, x, op, comment))()
 
 
-def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
-    """Symbolic gradient of the 0-d ``cost`` with respect to ``wrt`` (a variable
-    or a list of variables)."""
+def grad(cost, wrt, consider_constant=None, disconnected_inputs="raise", add_names=True, known_grads=None,
+         return_disconnected="zero", null_gradients="raise"):
+    """Symbolic gradient of the 0-d ``cost`` with respect to ``wrt`` (a variable, a list or a tuple of
+    variables), with the arguments of ``theano.grad`` (``theano/gradient.py:414-628``):
+
+    ``consider_constant``: expressions nothing is propagated through.  ``disconnected_inputs``: what happens
+    when an element of ``wrt`` is not part of the graph of the cost, or only reaches it through operands an op
+    declares unconnected (``connection_pattern``) - ``'raise'`` DisconnectedInputError, ``'warn'`` or
+    ``'ignore'``; in the last two cases ``return_disconnected`` says what comes back: ``'zero'``, ``'None'`` or
+    ``'Disconnected'`` (a variable of DisconnectedType).  A variable that reaches the cost only through
+    integer-valued results is connected, with a gradient of zeros.  ``known_grads``: gradients given for
+    variables of the graph (``cost`` may then be None).  ``null_gradients``: ``'raise'`` NullTypeGradError for a
+    gradient an op declared undefined or not implemented, or ``'return'`` the NullType variable.
+    ``add_names``: a named cost and a named variable name their gradient ``(dcost/dvar)``."""
+    import warnings
     from .tensor import basic as T
     from .tensor.type import as_tensor_variable
 
+    if disconnected_inputs not in ("ignore", "warn", "raise"):
+        raise ValueError("Invalid value for keyword 'disconnected_inputs', valid values are 'ignore', 'warn' and "
+                         "'raise'.")
+    if return_disconnected not in ("zero", "None", "Disconnected"):
+        raise ValueError("Invalid value for keyword 'return_disconnected', valid values are 'zero', 'None' and "
+                         "'Disconnected'.")
+    if null_gradients not in ("raise", "return"):
+        raise ValueError("Invalid value for keyword 'null_gradients', valid values are 'raise' and 'return'.")
+    if cost is None and known_grads is None:
+        raise AssertionError("cost and known_grads can't both be None.")
+    if cost is not None and isinstance(cost.type, NullType):
+        raise ValueError("Can't differentiate a NaN cost. cost is NaN because " + cost.type.why_null)
+    as_tuple = isinstance(wrt, tuple)
     single = not isinstance(wrt, (list, tuple))
     wrt_list = [wrt] if single else list(wrt)
+    for w in wrt_list:
+        if not isinstance(w, gof.Variable):
+            raise TypeError("Expected Variable, got %s of type %s" % (w, type(w)))
+    constant = set(id(v) for v in (consider_constant or ()))
     grads = {}
     if cost is not None:
         if cost.type.ndim != 0:
@@ -70,33 +99,49 @@ def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
         grads[cost] = (T.ones_like(cost) if cost.type.dtype in scal.continuous_dtypes
                        else T.ones_like(cost, dtype=config.floatX))
     for var, g in (known_grads or {}).items():
-        grads[var] = as_tensor_variable(g)
+        g = as_tensor_variable(g) if not isinstance(g, gof.Variable) else g
+        if not isinstance(g.type, (NullType, DisconnectedType)) and g.type.dtype not in scal.continuous_dtypes:
+            raise TypeError("Gradients must always be NullType, DisconnectedType, or continuous, but grad was given "
+                            "a known_grad of type " + str(g.type))
+        grads[var] = g
     outputs = list(grads.keys())
 
-    # nodes on a path from wrt to the outputs
+    # nodes on a path from wrt to the outputs; nothing is computed "from" an expression held constant
     order = gof.io_toposort([], outputs)
     depends = set(id(w) for w in wrt_list)
     for node in order:
         if any(id(i) in depends for i in node.inputs):
             for o in node.outputs:
-                depends.add(id(o))
+                if id(o) not in constant:       # a gradient may arrive at such an expression, none goes through it
+                    depends.add(id(o))
+    # variables with a path to an output (one whose gradient is not given as disconnected) along which every op
+    # declares its operand connected
+    connected = set(id(o) for o in outputs if not isinstance(grads[o].type, DisconnectedType))
+    for node in reversed(order):
+        hit = [k for k, o in enumerate(node.outputs) if id(o) in connected and id(o) not in constant]
+        if not hit:
+            continue
+        pattern = node.op.connection_pattern(node)
+        for k, i in enumerate(node.inputs):
+            if any(pattern[k][o] for o in hit):
+                connected.add(id(i))
 
     for node in reversed(order):
         if not any(id(o) in depends for o in node.outputs):
             continue
         ograds = []
-        connected = False
+        live = False
         null = None
         for o in node.outputs:
-            g = grads.get(o)
-            if g is None:
+            g = grads.get(o) if id(o) not in constant else None
+            if g is None or isinstance(g.type, DisconnectedType):
                 ograds.append(DisconnectedType()())
             else:
-                connected = True
+                live = True
                 ograds.append(g)
                 if isinstance(g.type, NullType):
                     null = g
-        if not connected:
+        if not live:
             continue
         if null is not None:
             # nothing can be said about what lies behind an unknown gradient
@@ -110,6 +155,11 @@ def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
         # replace missing output grads by zeros for ops that cannot take placeholders
         ograds = [T.zeros_like(o) if isinstance(g.type, DisconnectedType) and len(node.outputs) > 1 else g
                   for o, g in zip(node.outputs, ograds)]
+        # the gradient of a floating-point result enters the op in that result's own dtype
+        # (theano/gradient.py:1107-1115): what flows back to a float32 variable stays float32
+        ograds = [g.astype(o.type.dtype) if (hasattr(g.type, "dtype") and getattr(o.type, "dtype", None) is not None and
+                                             o.type.dtype not in scal.discrete_dtypes and g.type.dtype != o.type.dtype)
+                  else g for o, g in zip(node.outputs, ograds)]
         try:
             igrads = node.op.L_op(node.inputs, node.outputs, ograds)
         except gof.MethodNotDefined:
@@ -130,24 +180,40 @@ def grad(cost, wrt, known_grads=None, disconnected_inputs="zero"):
                 continue
             if hasattr(i.type, "broadcastable") and g.type.broadcastable != i.type.broadcastable:
                 g = _match_broadcast(g, i)
-            grads[i] = g if i not in grads else T.add(grads[i], g)
+            grads[i] = g if i not in grads or isinstance(grads[i].type, DisconnectedType) else T.add(grads[i], g)
 
     result = []
     for w in wrt_list:
         g = grads.get(w)
         if g is not None and isinstance(g.type, NullType):
-            raise NullTypeGradError("grad encountered a NaN. " + g.type.why_null)
-        if g is None:
-            if disconnected_inputs == "raise":
-                raise DisconnectedInputError("grad method was asked to compute the gradient with respect to a "
-                                             "variable that is not part of the computational graph of the cost: %s" % w)
-            dt = w.type.dtype if w.type.dtype in scal.continuous_dtypes else config.floatX
-            g = T.zeros_like(w, dtype=dt)
+            if null_gradients == "raise":
+                raise NullTypeGradError("tensor.grad encountered a NaN. " + g.type.why_null)
+            result.append(g)
+            continue
+        if g is None or isinstance(g.type, DisconnectedType):
+            float_zeros = lambda: T.zeros_like(                                             # noqa: E731
+                w, dtype=w.type.dtype if w.type.dtype in scal.continuous_dtypes else config.floatX)
+            if id(w) in connected and g is None:
+                g = float_zeros()               # reaches the cost, through integer-valued results only
+            else:
+                message = ("grad method was asked to compute the gradient with respect to a variable that is not "
+                           "part of the computational graph of the cost, or is used only by a non-differentiable "
+                           "operator: %s" % w)
+                if disconnected_inputs == "raise":
+                    raise DisconnectedInputError(message)
+                if disconnected_inputs == "warn":
+                    warnings.warn(message, stacklevel=2)
+                g = (float_zeros() if return_disconnected == "zero" else None if return_disconnected == "None"
+                     else DisconnectedType()())
+        elif add_names and cost is not None and cost.name is not None and w.name is not None:
+            g.name = "(d%s/d%s)" % (cost.name, w.name)
         result.append(g)
-    return result[0] if single else result
+    if single:
+        return result[0]
+    return tuple(result) if as_tuple else result
 
 
-def Lop(f, wrt, eval_points):
+def Lop(f, wrt, eval_points, consider_constant=None, disconnected_inputs="raise"):
     """L operator: eval_points times the Jacobian of ``f`` with respect to
     ``wrt`` (``theano/gradient.py:348-411``): reverse mode seeded with
     ``eval_points`` as the gradients of ``f``."""
@@ -155,7 +221,7 @@ def Lop(f, wrt, eval_points):
     eps = list(eval_points) if isinstance(eval_points, (list, tuple)) else [eval_points]
     if len(fs) != len(eps):
         raise ValueError("Lop needs one evaluation point per element of f")
-    return grad(None, wrt, known_grads=dict(zip(fs, eps)))
+    return grad(None, wrt, known_grads=dict(zip(fs, eps)), disconnected_inputs=disconnected_inputs)
 
 
 def Rop(f, wrt, eval_points, disconnected_outputs="raise"):

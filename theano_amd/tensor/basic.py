@@ -91,18 +91,27 @@ def cast(x, dtype):
     return _cast_ops[dtype](x)
 
 
-def zeros_like(model, dtype=None):
+def zeros_like(model, dtype=None, opt=False):
+    """``fill(model, 0)``; with ``opt`` the bare constant when it already has ``model``'s type
+    (``theano/tensor/basic.py:2521-2547``)."""
     model = as_tensor_variable(model)
     if dtype is None:
         dtype = model.type.dtype
-    return fill(model, constant(0, dtype=dtype))
+    ret = constant(0, dtype=dtype)
+    if opt and ret.type == model.type:
+        return ret
+    return fill(model, ret)
 
 
-def ones_like(model, dtype=None):
+def ones_like(model, dtype=None, opt=False):
+    """``fill(model, 1)`` (``theano/tensor/basic.py:2493-2518``)."""
     model = as_tensor_variable(model)
     if dtype is None:
         dtype = model.type.dtype
-    return fill(model, constant(1, dtype=dtype))
+    ret = constant(1, dtype=dtype)
+    if opt and ret.type == model.type:
+        return ret
+    return fill(model, ret)
 
 
 def iround(a, mode=None):
@@ -395,10 +404,14 @@ def squeeze(x):
     return x.dimshuffle([i for i in range(x.type.ndim) if not x.type.broadcastable[i]])
 
 
-def mean(input, axis=None, dtype=None, keepdims=False, acc_dtype=None):
+def mean(input, axis=None, dtype=None, op=False, keepdims=False, acc_dtype=None):
     """Sum divided by the extent of every reduced axis in turn; float16 inputs
-    are summed in float32 and the result is cast back."""
+    are summed in float32 and the result is cast back.  ``op=True`` asks the reference for its
+    host-only ``Mean`` op (``theano/tensor/basic.py:3246-3288, 3328-3344``), which has no device form."""
     input = as_tensor_variable(input)
+    if op:
+        raise NotImplementedError("mean(op=True): the Mean op computes on the host in float64; call "
+                                  "mean(..., op=False), which sums and divides on the device")
     if dtype is not None:
         sum_dtype = dtype
     else:

@@ -615,9 +615,17 @@ def reshape(x, newshape, ndim=None):
     return Reshape(pattern)(x, *args.extra())
 
 
-def flatten(x, ndim=1):
+def flatten(x, ndim=None, outdim=None):
     """Keep the first ``ndim - 1`` dimensions, merge the rest
-    (``theano/tensor/basic.py:5160-5220``)."""
+    (``theano/tensor/basic.py:5252-5310``; ``outdim`` is the older name of ``ndim``)."""
+    if outdim is not None and ndim is not None:
+        raise ValueError("You should only specify ndim")
+    if outdim is not None:
+        import warnings
+        warnings.warn("flatten outdim parameter is deprecated, use ndim instead.")
+        ndim = outdim
+    if ndim is None:
+        ndim = 1
     x = as_tensor_variable(x)
     if ndim < 1 or ndim > max(x.type.ndim, 1):
         raise ValueError("invalid output ndimensions (%d) for flatten" % ndim)
@@ -795,8 +803,24 @@ def join(axis, *tensors):
 concatenate = lambda tensors, axis=0: join(axis, *tensors)  # noqa: E731
 
 
-def stack(tensors, axis=0):
-    """New axis at ``axis``, then join (``theano/tensor/basic.py:4560-4640``)."""
+def stack(*tensors, **kwargs):
+    """``stack(tensors, axis=0)``: new axis at ``axis``, then join; ``stack(a, b, ...)`` is the older spelling of
+    ``stack([a, b, ...], axis=0)`` (``theano/tensor/basic.py:4630-4745``)."""
+    if not tensors and not kwargs:
+        raise Exception("theano.tensor.stack(tensors, axis) must have at least one parameter")
+    if not kwargs and not isinstance(tensors[0], (list, tuple)):
+        import warnings
+        warnings.warn("stack(*tensors) interface is deprecated, use stack(tensors, axis=0) instead.",
+                      DeprecationWarning, stacklevel=2)
+        axis = 0
+    elif "tensors" in kwargs:
+        tensors, axis = kwargs["tensors"], kwargs.get("axis", 0)
+    else:
+        axis = tensors[1] if len(tensors) == 2 else kwargs.get("axis", 0)
+        tensors = tensors[0]
+    if len(tensors) == 0:
+        raise Exception("tensors is empty. You should at least provide one tensor to "
+                        "theano.tensor.stack(tensors, axis).")
     ts = [as_tensor_variable(t) for t in tensors]
     nd = ts[0].type.ndim
     axis = axis + nd + 1 if axis < 0 else axis
