@@ -1294,3 +1294,30 @@ def test_grad_arguments_of_the_reference(dry_run):
     # the first operand of fill is not connected (theano/scalar/basic.py:2283-2287)
     with pytest.raises(GR.DisconnectedInputError):
         th.grad(T.sum(T.fill(x, a)), x)
+
+
+def test_function_takes_the_references_arguments_in_its_order(dry_run):
+    """``theano.function(inputs, outputs=None, mode=None, updates=None, givens=None, no_default_updates=False,
+    accept_inplace=False, name=None, rebuild_strict=True, allow_input_downcast=None, profile=None,
+    on_unused_input=None)`` (``theano/compile/function.py:74-77``); unused inputs
+    (``theano/compile/function_module.py:1594-1625``)."""
+    import inspect
+    import warnings
+    params = inspect.signature(th.function).parameters
+    assert list(params)[:12] == ["inputs", "outputs", "mode", "updates", "givens", "no_default_updates", "accept_inplace",
+                                 "name", "rebuild_strict", "allow_input_downcast", "profile", "on_unused_input"]
+    assert all(params[p].kind is inspect.Parameter.KEYWORD_ONLY for p in list(params)[12:])
+    x, y = T.fvector("x"), T.fvector("y")
+    s = th.shared(np.zeros(3, "float32"))
+    f = th.function([x], x * 2, None, [(s, s + x)])                  # mode, then updates, by position
+    assert f.update_targets == [s]
+    assert th.function([x], None, updates=[(s, s + x)])(np.ones(3, "float32")) == []
+    with pytest.raises(th.UnusedInputError, match="index 1 is not part"):
+        th.function([x, y], x * 2)
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        th.function([x, y], x * 2, on_unused_input="warn")
+    assert len(seen) == 1 and "on_unused_input='raise'" in str(seen[0].message)
+    th.function([x, y], x * 2, on_unused_input="ignore")
+    with pytest.raises(ValueError):
+        th.function([x], x * 2, on_unused_input="never")

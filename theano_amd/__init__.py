@@ -7,4 +7,4 @@ CAReduce / DimShuffle nodes onto HIP ops backed by ``libthx_hip.so``.
 from .config import config  # noqa: F401
 from . import gof, scalar, tensor  # noqa: F401
 from .gradient import grad, Lop, Rop  # noqa: F401
-from .compile import CheckModeError, NanGuardError, function, In, Out, shared  # noqa: F401
+from .compile import CheckModeError, NanGuardError, UnusedInputError, function, In, Out, shared  # noqa: F401

@@ -83,6 +83,10 @@ def shared(value, name=None, broadcastable=None):
     return _Shared(t, t.filter(value), name=name)
 
 
+class UnusedInputError(Exception):
+    """A symbolic input passed to ``function`` is not needed (``theano/compile/function_module.py:34-40``)."""
+
+
 class NanGuardError(FloatingPointError):
     """A node produced NaN or infinity under ``mode='nan_guard'``."""
 
@@ -443,9 +447,15 @@ class Function(object):
         return list(self.nodes)
 
 
-def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=True, inplace=True, name=None,
-             on_unused_input="raise", mode=None, accept_inplace=False, allow_input_downcast=None):
-    """Compile ``outputs`` as a function of ``inputs``.
+def function(inputs, outputs=None, mode=None, updates=None, givens=None, no_default_updates=False, accept_inplace=False,
+             name=None, rebuild_strict=True, allow_input_downcast=None, profile=None, on_unused_input=None, *,
+             fuse=True, rowchain=True, inplace=True):
+    """Compile ``outputs`` as a function of ``inputs``: the arguments of ``theano.function`` in its order
+    (``theano/compile/function.py:74-77``), then this package's own switches, by keyword only.
+    ``no_default_updates`` and ``rebuild_strict`` are accepted for that order's sake (shared variables here have
+    no default updates, and replacements in ``givens`` must keep the type); ``profile`` must stay unset -
+    ``theano_amd.hip.runtime.profile`` times the kernels of any call.  ``on_unused_input``: 'raise' (the
+    default, None), 'warn' or 'ignore'.
 
     ``inputs``: variables or ``In`` instances.  A host-typed input may be given
     a ``HipArray`` at call time, which skips the upload.  ``outputs``: a
@@ -520,12 +530,28 @@ def function(inputs, outputs, updates=None, givens=None, fuse=True, rowchain=Tru
     in_vars = [s.variable for s in in_specs]
     shared_inputs = [v for v in gof.graph_inputs(out_vars) if isinstance(v, SharedVariable)]
     used = set(id(v) for v in gof.graph_inputs(out_vars))
-    if on_unused_input == "raise":
-        for v in in_vars:
+    if on_unused_input is None:
+        on_unused_input = "raise"
+    if on_unused_input not in ("raise", "warn", "ignore"):
+        raise ValueError("Invalid value for keyword on_unused_input of theano.function: '%s'.\nValid values are "
+                         "'raise', 'warn', and 'ignore'." % on_unused_input)
+    if profile:
+        raise NotImplementedError("function(profile=...): use theano_amd.hip.runtime.profile() around the calls")
+    if on_unused_input != "ignore":
+        for k, v in enumerate(in_vars):
             if id(v) not in used:
-                raise ValueError("theano function was asked to create a function computing outputs given certain "
-                                 "inputs, but the provided input variable %s is not part of the computational graph "
-                                 "needed to compute the outputs." % v)
+                msg = ("theano.function was asked to create a function computing outputs given certain inputs, but "
+                       "the provided input variable at index %i is not part of the computational graph needed to "
+                       "compute the outputs: %s.\n" % (k, v))
+                if on_unused_input == "warn":
+                    import warnings
+                    warnings.warn(msg + "To make this warning into an error, you can pass the parameter "
+                                  "on_unused_input='raise' to theano.function. To disable it completely, use "
+                                  "on_unused_input='ignore'.", stacklevel=2)
+                else:
+                    raise UnusedInputError(msg + "To make this error into a warning, you can pass the parameter "
+                                           "on_unused_input='warn' to theano.function. To disable it completely, "
+                                           "use on_unused_input='ignore'.")
     # clone everything except shared variables
     memo = dict((s, s) for s in shared_inputs)
     memo = gof.clone_get_equiv(in_vars, out_vars, copy_inputs=True, memo=memo)
