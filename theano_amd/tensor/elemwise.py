@@ -117,8 +117,11 @@ class Elemwise(Op):
 
     __props__ = ("scalar_op", "inplace_pattern")
 
-    def __init__(self, scalar_op, inplace_pattern=None, name=None):
+    def __init__(self, scalar_op, inplace_pattern=None, name=None, nfunc_spec=None, openmp=None):
+        # nfunc_spec names the NumPy function the reference's host ``perform`` may call and ``openmp`` switches its C
+        # loop's pragma (theano/tensor/elemwise.py:389-414): neither changes what is computed; the first is kept
         self.name = name
+        self.nfunc_spec = nfunc_spec if nfunc_spec is not None else getattr(scalar_op, "nfunc_spec", None)
         self.scalar_op = scalar_op
         self.inplace_pattern = tuple(sorted((inplace_pattern or {}).items())) if not isinstance(
             inplace_pattern, tuple) else inplace_pattern

@@ -13,7 +13,8 @@ from ..gof import Apply, Constant, Type, Variable
 class TensorType(Type):
     """dtype plus, per dimension, whether its extent is known to be 1."""
 
-    def __init__(self, dtype, broadcastable, name=None):
+    def __init__(self, dtype, broadcastable, name=None, sparse_grad=False):
+        self.sparse_grad = sparse_grad        # a hint for gradients of indexing ops; nothing here reads it
         if dtype == "floatX":
             dtype = config.floatX
         self.dtype = str(dtype)
@@ -180,6 +181,9 @@ class _tensor_py_operators(object):
         if self._is_nonzero:
             return True
         raise TypeError("Variables do not support boolean operations.")
+
+    __nonzero__ = __bool__          # its Python 2 name, theano/tensor/var.py:98-105
+
     def __and__(self, o): return self._b().and_(self, o)
     def __or__(self, o): return self._b().or_(self, o)
     def __xor__(self, o): return self._b().xor(self, o)
