@@ -12,7 +12,7 @@ import pytest
 import theano_amd as th
 from theano_amd import tensor as T
 from oracle import graph_ref as G
-from conftest import assert_parity
+from conftest import assert_parity, assert_within_reference_error
 
 EXTENTS = [1, 2, 3, 5, 7, 8, 16, 33, 64]
 MAX_ELEMENTS = 150000
@@ -129,6 +129,48 @@ def random_mixed_graph(seed):
     integer division and modulo with both signs, comparisons feeding arithmetic, and the
     callers around the path: max_and_argmax, mean / var / std, softmax, reshape, join,
     set / inc_subtensor."""
+    rng, ins, vals, e, nd, shape = _mixed_expression(seed)
+    fl = e.type.dtype.startswith("float")
+    axis = int(rng.integers(nd))
+    mode = int(rng.integers(6))
+    if mode == 0:
+        outs = list(T.max_and_argmax(e, axis=axis)) + [T.argmin(e, axis=None if nd > 1 and rng.random() < 0.3 else axis)]
+        if e.type.dtype in ("int8", "bool", "uint8"):     # argmin negates: wraps for the smallest int8 as in the reference
+            outs = outs[:2]
+    elif mode == 1:
+        ef = e if fl else T.cast(e, "float32")
+        outs = [T.mean(ef, axis=axis), T.var(ef, axis=axis, keepdims=True), T.std(ef)]
+    elif mode == 2:
+        ef = e if fl else T.cast(e, "float64")
+        m = ef.reshape((-1, shape[-1])) if nd > 1 else ef.reshape((1, -1))
+        sm = T.nnet.softmax(m)
+        outs = [sm, T.nnet.logsoftmax(m), th.grad(T.sum(sm * sm), m)] if ef.type.dtype != "float16" else [sm]
+    elif mode == 3:
+        outs = [T.join(axis, e, e * 2), T.stack([e, -e] if e.type.dtype != "uint8" else [e, e]), e.flatten()]
+    elif mode == 4:
+        idx = tuple(slice(0, None, 2) if d == axis else slice(None) for d in range(nd))
+        outs = [T.inc_subtensor(e[idx], e[idx]), T.set_subtensor(e[idx], T.zeros_like(e[idx])), T.sum(e[idx], axis=axis)]
+    else:
+        outs = [T.sum(e, axis=axis), T.prod(T.cast(T.gt(e, 0), "int8") + 1, axis=axis), T.any(e, axis=axis), T.all(e)]
+    return ins, outs, vals
+
+
+def random_mixed_gradient_graph(seed):
+    """Reverse mode through a chain over float16 / float32 / float64 operands: every result's gradient enters
+    its op in the result's own dtype, so the casts between the widths are part of what is compared."""
+    while True:                                        # the next seed that draws the floating-point family
+        rng, ins, vals, e, nd, shape = _mixed_expression(seed)
+        if e.type.dtype.startswith("float") and any(v.type.dtype.startswith("float") for v in ins):
+            break
+        seed += 7919
+    axis = int(rng.integers(nd))
+    cost = T.sum(e * e, dtype="float64" if e.type.dtype == "float64" else "float32") + T.sum(T.mean(e, axis=axis))
+    used = set(id(v) for v in th.gof.graph_inputs([cost]))
+    wrt = [v for v in ins if id(v) in used and v.type.dtype.startswith("float")]
+    return ins, [cost] + th.grad(cost, wrt, disconnected_inputs="ignore"), vals
+
+
+def _mixed_expression(seed):
     rng = np.random.default_rng(seed)
     floating = bool(rng.random() < 0.5)
     family = ["float16", "float32", "float32", "float64"] if floating else ["bool", "int8", "uint8", "int16", "int32", "int64"]
@@ -173,29 +215,7 @@ def random_mixed_graph(seed):
     e = terms[-1]
     if e.type.ndim < nd or any(e.type.broadcastable) or e.type.dtype == "bool":
         e = e + full
-    fl = e.type.dtype.startswith("float")
-    axis = int(rng.integers(nd))
-    mode = int(rng.integers(6))
-    if mode == 0:
-        outs = list(T.max_and_argmax(e, axis=axis)) + [T.argmin(e, axis=None if nd > 1 and rng.random() < 0.3 else axis)]
-        if e.type.dtype in ("int8", "bool", "uint8"):     # argmin negates: wraps for the smallest int8 as in the reference
-            outs = outs[:2]
-    elif mode == 1:
-        ef = e if fl else T.cast(e, "float32")
-        outs = [T.mean(ef, axis=axis), T.var(ef, axis=axis, keepdims=True), T.std(ef)]
-    elif mode == 2:
-        ef = e if fl else T.cast(e, "float64")
-        m = ef.reshape((-1, shape[-1])) if nd > 1 else ef.reshape((1, -1))
-        sm = T.nnet.softmax(m)
-        outs = [sm, T.nnet.logsoftmax(m), th.grad(T.sum(sm * sm), m)] if ef.type.dtype != "float16" else [sm]
-    elif mode == 3:
-        outs = [T.join(axis, e, e * 2), T.stack([e, -e] if e.type.dtype != "uint8" else [e, e]), e.flatten()]
-    elif mode == 4:
-        idx = tuple(slice(0, None, 2) if d == axis else slice(None) for d in range(nd))
-        outs = [T.inc_subtensor(e[idx], e[idx]), T.set_subtensor(e[idx], T.zeros_like(e[idx])), T.sum(e[idx], axis=axis)]
-    else:
-        outs = [T.sum(e, axis=axis), T.prod(T.cast(T.gt(e, 0), "int8") + 1, axis=axis), T.any(e, axis=axis), T.all(e)]
-    return ins, outs, vals
+    return rng, ins, vals, e, nd, shape
 
 
 SEEDS = list(range(100, 200))
@@ -213,9 +233,9 @@ def test_random_graph_matches_the_oracle(seed):
         assert_parity(g, r, "seed %d output %d" % (seed, k))
 
 
-def check_mixed(seed, **flags):
+def check_mixed(seed, generator=None, **flags):
     from conftest import TOL
-    ins, outs, vals = random_mixed_graph(seed)
+    ins, outs, vals = (generator or random_mixed_graph)(seed)
     with np.errstate(all="ignore"):
         ref = G.evaluate(ins, outs, vals)
     got = th.function(ins, outs, on_unused_input="ignore", **flags)(*vals)
@@ -225,15 +245,34 @@ def check_mixed(seed, **flags):
     for n in gof.io_toposort(ins, outs):
         seen.update(o.type.dtype for o in n.outputs)
     narrowest = [d for d in ("float16", "float32", "float64") if d in seen]
+    truth = None
     for k, (g, r) in enumerate(zip(got, ref)):
         tol = TOL[narrowest[0]] if narrowest and r.dtype.kind == "f" else None
-        assert_parity(g, r, "seed %d output %d" % (seed, k), tol=tol)
+        try:
+            assert_parity(g, r, "seed %d output %d" % (seed, k), tol=tol)
+        except AssertionError:
+            if generator is not random_mixed_gradient_graph:
+                raise
+            # A gradient through float16 nodes: the oracle rounds every node's result to float16 (1 - tanh(x)**2
+            # loses most of its digits there), a fused kernel keeps float32 between them (as the reference's
+            # GPU composites do, theano/gpuarray/elemwise.py:156-164).  Held to the float64 evaluation instead,
+            # no farther from it than the oracle is.
+            if truth is None:
+                with np.errstate(all="ignore"):
+                    truth = G.evaluate(ins, outs, vals, wide=True)
+            assert_within_reference_error(g, r, truth[k], "seed %d output %d" % (seed, k), tol=tol)
 
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("seed", MIXED_SEEDS)
 def test_random_mixed_graph_matches_the_oracle(seed):
     check_mixed(seed)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", list(range(900, 930)))
+def test_random_mixed_gradient_graph_matches_the_oracle(seed):
+    check_mixed(seed, generator=random_mixed_gradient_graph)
 
 
 @pytest.mark.gpu
@@ -257,3 +296,28 @@ def test_generator_builds_valid_graphs(dry_run):
         got = th.function(ins, outs, on_unused_input="ignore")(*vals)
         assert [g.shape for g in got] == [r.shape for r in ref], seed
         assert [g.dtype for g in got] == [r.dtype for r in ref], seed
+
+
+MIXED_GRADIENT_REGRESSIONS = [946, 1316, 1484]
+
+
+@pytest.mark.parametrize("seed", MIXED_GRADIENT_REGRESSIONS)
+def test_mixed_gradient_graphs_that_once_failed_to_build(seed, dry_run):
+    """Three graphs of the mixed-dtype gradient generator that did not get as far as a launch: 946 - the sign
+    of a float16 per-result operand inside a reduction's epilogue (the operand was used in its storage type,
+    for which ``isnan`` has no overload); 1316 - a stored elementwise result with an attached channel sum whose
+    reduced result a later kernel reads (the reuse mark indexed past the stored results); 1484 - two merges of
+    sibling elementwise kernels in a row that closed a cycle (the second merge did not see that the first
+    merged node depends on what lies between its two parts).  Planned and compiled for gfx950 here; their
+    values are checked on the device with the other seeds."""
+    ins, outs, vals = random_mixed_gradient_graph(seed)
+    with np.errstate(all="ignore"):
+        ref = G.evaluate(ins, outs, vals)
+    got = th.function(ins, outs, on_unused_input="ignore")(*vals)
+    assert [g.shape for g in got] == [r.shape for r in ref] and [g.dtype for g in got] == [r.dtype for r in ref]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", MIXED_GRADIENT_REGRESSIONS)
+def test_mixed_gradient_graphs_that_once_failed_to_build_have_the_oracles_values(seed):
+    check_mixed(seed, generator=random_mixed_gradient_graph)

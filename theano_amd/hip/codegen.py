@@ -278,10 +278,12 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
                                                      "(a.a%d ? 1 : 0)" % k if dt == "bool" else "a.a%d" % k)
             args.append("r%d" % k)
         for j, dt in enumerate(extra_dtypes):
+            # read in the storage type, used in the arithmetic type (float16 computes as float, as every kernel
+            # operand does: the scalar ops' code is written for that)
             if extra_is_array is not None and extra_is_array[j]:
-                args.append("(((const %s*)o.ex[%d])[idx * o.exs[%d]])" % (storage_ctype(dt), j, j))
+                args.append("((%s)(((const %s*)o.ex[%d])[idx * o.exs[%d]]))" % (compute_ctype(dt), storage_ctype(dt), j, j))
             else:
-                args.append("(*(const %s*)&o.ex[%d])" % (storage_ctype(dt), j))
+                args.append("((%s)(*(const %s*)&o.ex[%d]))" % (compute_ctype(dt), storage_ctype(dt), j))
         post_stmt += "\n" + post_op.c_code(qnode, args, tmp) + "\n"
         post_stmt += "\n".join("((%s*)o.ptr[%d])[idx] = (%s)%s;" % (storage_ctype(dt), k, storage_ctype(dt), t)
                                for k, (dt, t) in enumerate(zip(out_dtypes, tmp)))

@@ -662,7 +662,8 @@ class HipElemwiseReduce(HipElemwise):
             arr = HipArray._new_contiguous((shape[-1],), out_dt[n_ew + k])
             arr.as_thx(routs[k])
             results.append(arr)
-        mark_reused(node, ins, outs)
+        # the positions recorded for the node's results run over the stored results first, then the reduced ones
+        mark_reused(node, ins, [outs[k] if k < n_ew else routs[k - n_ew] for k in range(n_ew + K)])
         rc = lib.thx_elemwise_reduce_call(eh, ins, outs, routs, call_flags(node))
         if rc:
             check(rc)

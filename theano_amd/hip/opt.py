@@ -591,11 +591,13 @@ def _try_epilogue(fgraph, red, cand):
 
 
 def _depends_on(var, node, limit=10000, pos=None):
-    """True when ``var`` is computed (transitively) from an output of ``node``.  ``pos``: positions
-    in a topological order; a producer placed before ``node`` cannot depend on it."""
+    """True when ``var`` is computed (transitively) from an output of ``node``.  ``pos``: for each node the
+    span (first, last) of positions in a topological order that it stands for - one position for an original
+    node, the span of its parts for a node merged from several; a producer whose parts all lie before every
+    part of ``node`` cannot depend on it."""
     if pos is not None and var.owner is not None:
         pv, pn = pos.get(var.owner), pos.get(node)
-        if pv is not None and pn is not None and pv < pn:
+        if pv is not None and pn is not None and pv[1] < pn[0]:
             return False
     stack, seen = [var], set()
     while stack and len(seen) < limit:
@@ -726,7 +728,7 @@ def merge_sibling_elemwise(fgraph):
     (``theano/gpuarray/elemwise.py:114-115``); the kernels here take several."""
     count = 0
     order = fgraph.toposort()
-    pos = dict((n, k) for k, n in enumerate(order))
+    pos = dict((n, (k, k)) for k, n in enumerate(order))
     nodes = [n for n in order if isinstance(n.op, HipElemwise) and not n.op.inplace_pattern]
     for ai in range(len(nodes)):
         a = nodes[ai]
@@ -778,7 +780,9 @@ def merge_sibling_elemwise(fgraph):
             for o, no in zip(olds, merged.outputs):
                 fgraph.replace(o, no)
             count += 1
-            pos[merged] = min(pos[a], pos[b])   # nothing placed before both can depend on the merged node
+            # the merged node stands for both spans: what lies between its parts may depend on the first of them
+            # and be depended on by the second
+            pos[merged] = (min(pos[a][0], pos[b][0]), max(pos[a][1], pos[b][1]))
             a = merged              # keeps collecting partners among the nodes that follow
     return count
 
