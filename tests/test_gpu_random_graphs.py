@@ -64,11 +64,14 @@ def make_input(rng, k, shape, dtype):
     return var, val, term
 
 
-def random_graph(seed):
+def random_graph(seed, rank=None):
+    """``rank``: the number of dimensions instead of the 1 to 4 the seed draws (up to the library's 8)."""
     rng = np.random.default_rng(seed)
     dtype = str(rng.choice(["float32", "float32", "float64", "int32", "int16", "int64"]))
     nd = int(rng.integers(1, 5))
-    shape = [int(rng.choice(EXTENTS)) for _ in range(nd)]
+    if rank is not None:
+        nd = rank
+    shape = [int(rng.choice(EXTENTS if rank is None else EXTENTS[:7])) for _ in range(nd)]
     while np.prod(shape) > MAX_ELEMENTS:
         shape[int(np.argmax(shape))] //= 2
     floating = dtype.startswith("float")
@@ -264,6 +267,20 @@ def check_mixed(seed, generator=None, **flags):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("seed", list(range(1200, 1230)))
+def test_random_graph_of_rank_five_to_eight_matches_the_oracle(seed):
+    """The same generator at the ranks the reference's many-argument test reaches (8 dimensions,
+    ``theano/gpuarray/tests/test_opt.py:531-572``): dimension collapsing, the generic reduction form for three and
+    more reduced groups, transposed and stepped views of 5 to 8 dimensions."""
+    ins, outs, vals = random_graph(seed, rank=5 + seed % 4)
+    with np.errstate(all="ignore"):
+        ref = G.evaluate(ins, outs, vals)
+    got = th.function(ins, outs, on_unused_input="ignore")(*vals)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "seed %d output %d" % (seed, k))
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("seed", MIXED_SEEDS)
 def test_random_mixed_graph_matches_the_oracle(seed):
     check_mixed(seed)
@@ -321,3 +338,73 @@ def test_mixed_gradient_graphs_that_once_failed_to_build(seed, dry_run):
 @pytest.mark.parametrize("seed", MIXED_GRADIENT_REGRESSIONS)
 def test_mixed_gradient_graphs_that_once_failed_to_build_have_the_oracles_values(seed):
     check_mixed(seed, generator=random_mixed_gradient_graph)
+
+
+def random_update_step(seed):
+    """A momentum step on a parameter array: cost = sum(chain(p, x)), m <- 0.9 m + d cost / d p, p <- p - 0.1 m,
+    written over plain variables (for the oracle) and compiled with the state in shared variables through
+    ``givens`` and ``updates``.  Returns (function, shared p, shared m, oracle inputs, oracle outputs, x values
+    for three calls - the batch extent changes between them)."""
+    rng = np.random.default_rng(seed)
+    dtype = str(rng.choice(["float32", "float32", "float64"]))
+    nd = int(rng.integers(1, 4))
+    shape = [int(rng.choice(EXTENTS[1:])) for _ in range(nd)]
+    P = T.TensorType(dtype, (False,) * nd)("P")
+    M = T.TensorType(dtype, (False,) * nd)("M")
+    X = T.TensorType(dtype, (False,) * (nd + 1))("X")
+    terms = [P.dimshuffle("x", *range(nd)) * X, X, P.dimshuffle("x", *range(nd)) + 0 * X]
+    for _ in range(int(rng.integers(2, 6))):
+        a = terms[int(rng.integers(len(terms)))]
+        if rng.random() < 0.5:
+            terms.append(FLOAT_UNARY[int(rng.integers(len(FLOAT_UNARY)))](a))
+        else:
+            b = terms[int(rng.integers(len(terms)))]
+            terms.append(FLOAT_BINARY[int(rng.integers(len(FLOAT_BINARY)))](a, b))
+    cost = T.mean(T.sqr(terms[-1])) + T.sum(T.sqr(P)) * 0.01
+    g = th.grad(cost, P)
+    new_m = 0.9 * M + g
+    new_p = P - 0.1 * new_m
+    if dtype == "float32":
+        new_m, new_p = T.cast(new_m, dtype), T.cast(new_p, dtype)
+    p = th.shared(rng.uniform(-1, 1, shape).astype(dtype), name="p")
+    m = th.shared(np.zeros(shape, dtype), name="m")
+    with pytest.raises(TypeError):                  # a device-typed variable does not stand in for a host one
+        th.function([X], cost, givens={P: p, M: m})
+    f = th.function([X], cost, updates=[(m, new_m), (p, new_p)],
+                    givens={P: T.as_tensor_variable(p), M: T.as_tensor_variable(m)})
+    xs = [rng.uniform(-2, 2, [b] + shape).astype(dtype) for b in (3, 3, 5)]
+    return f, p, m, [X, P, M], [cost, new_m, new_p], xs
+
+
+def check_update_step(seed):
+    from conftest import TOL
+    f, p, m, o_ins, o_outs, xs = random_update_step(seed)
+    for step, xv in enumerate(xs):
+        pv, mv = p.get_value(), m.get_value()
+        with np.errstate(all="ignore"):
+            ref = G.evaluate(o_ins, o_outs, [xv, pv, mv])
+            truth = G.evaluate(o_ins, o_outs, [xv, pv, mv], wide=True)
+        cost = f(xv)
+        assert np.array_equal(pv, p.get_value()) is False or np.array_equal(ref[2], pv)     # the state moved on
+        for name, g, r, w in (("cost", cost, ref[0], truth[0]), ("m", m.get_value(), ref[1], truth[1]),
+                              ("p", p.get_value(), ref[2], truth[2])):
+            what = "seed %d call %d %s" % (seed, step, name)
+            try:
+                assert_parity(g, r, what)
+            except AssertionError:
+                assert_within_reference_error(g, r, w, what)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", list(range(1500, 1520)))
+def test_random_update_steps_with_shared_state(seed):
+    check_update_step(seed)
+
+
+def test_update_step_generator_builds(dry_run):
+    for seed in range(1500, 1506):
+        f, p, m, o_ins, o_outs, xs = random_update_step(seed)
+        before = p.get_value().shape
+        f(xs[0])
+        f(xs[2])
+        assert p.get_value().shape == before == m.get_value().shape

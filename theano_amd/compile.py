@@ -520,8 +520,7 @@ def function(inputs, outputs=None, mode=None, updates=None, givens=None, no_defa
             if not isinstance(rep, Variable):
                 rep = as_tensor_variable(rep)
             vt, rt = var.type, rep.type
-            if (getattr(vt, "dtype", None) != getattr(rt, "dtype", None) or
-                    tuple(getattr(vt, "broadcastable", ())) != tuple(getattr(rt, "broadcastable", ()))):
+            if vt != rt:        # also a device-typed variable for a host-typed one: as_tensor_variable(shared) converts
                 raise TypeError("Cannot use a shared variable or expression of type %s as a replacement for a "
                                 "variable of type %s in givens" % (rt, vt))
             swap[var] = rep
