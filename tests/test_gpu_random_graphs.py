@@ -408,3 +408,102 @@ def test_update_step_generator_builds(dry_run):
         f(xs[0])
         f(xs[2])
         assert p.get_value().shape == before == m.get_value().shape
+
+
+def random_view_graph(seed):
+    """A chain of views over one array - slices with either sign of step, integer indices, transpositions,
+    new axes, reshapes - read by an elementwise kernel, a reduction, set / inc_subtensor, and (floating point)
+    differentiated back to the array."""
+    rng = np.random.default_rng(seed)
+    dtype = str(rng.choice(["float32", "float32", "float64", "int32", "int64", "float16"]))
+    nd = int(rng.integers(2, 5))
+    shape = [int(rng.choice([2, 3, 5, 7, 8, 16, 33])) for _ in range(nd)]
+    x = T.TensorType(dtype, (False,) * nd)("x")
+    if dtype.startswith("float"):
+        xv = rng.uniform(-2, 2, shape).astype(dtype)
+    else:
+        xv = rng.integers(-50, 50, shape).astype(dtype)
+    v, cur = x, list(shape)
+
+    def a_slice(n):
+        kind = rng.integers(4)
+        if kind == 0 or n < 2:
+            return slice(None), n
+        if kind == 1:
+            a = int(rng.integers(0, n - 1))
+            b = int(rng.integers(a + 1, n + 1))
+            return slice(a, b), b - a
+        if kind == 2:
+            st = int(rng.integers(2, 4))
+            return slice(None, None, st), len(range(0, n, st))
+        st = -int(rng.integers(1, 3))
+        return slice(None, None, st), len(range(n - 1, -1, st))
+
+    for _ in range(int(rng.integers(2, 6))):
+        r = len(cur)
+        kind = int(rng.integers(5))
+        if kind == 0 and r:                                   # slices on every axis
+            idx, new = [], []
+            for n in cur:
+                s, m = a_slice(n)
+                idx.append(s)
+                new.append(m)
+            v, cur = v[tuple(idx)], new
+        elif kind == 1 and r > 1:                             # an integer index drops an axis
+            d = int(rng.integers(r))
+            k = int(rng.integers(-cur[d], cur[d]))
+            v = v[tuple([slice(None)] * d + [k])]
+            cur = cur[:d] + cur[d + 1:]
+        elif kind == 2 and r > 1:                             # transposition
+            perm = [int(p) for p in rng.permutation(r)]
+            v, cur = v.dimshuffle(*perm), [cur[p] for p in perm]
+        elif kind == 3 and r < 5:                             # a new axis
+            d = int(rng.integers(r + 1))
+            order = list(range(r))
+            order.insert(d, "x")
+            v = T.unbroadcast(v.dimshuffle(*order), d)
+            cur = cur[:d] + [1] + cur[d:]
+        elif kind == 4 and r > 1:                             # merge two neighbouring axes
+            d = int(rng.integers(r - 1))
+            new = cur[:d] + [cur[d] * cur[d + 1]] + cur[d + 2:]
+            v, cur = v.reshape(tuple(new)), new
+    r = len(cur)
+    outs = [v * 2 + 1]
+    if r:
+        axes = sorted(set(int(a) for a in rng.integers(0, r, int(rng.integers(1, r + 1)))))
+        outs.append(T.sum(v, axis=tuple(axes)))
+        idx, new = [], []
+        for n in cur:
+            s, m = a_slice(n)
+            idx.append(s)
+            new.append(m)
+        outs.append(T.set_subtensor(v[tuple(idx)], T.zeros_like(v[tuple(idx)]) + 3))
+        outs.append(T.inc_subtensor(v[tuple(idx)], v[tuple(idx)]))
+    if dtype in ("float32", "float64"):
+        outs.append(th.grad(T.sum(T.sqr(v)) + T.sum(v[tuple(idx)] if r else v), x))
+    return [x], outs, [xv]
+
+
+def check_view_graph(seed, **flags):
+    ins, outs, vals = random_view_graph(seed)
+    with np.errstate(all="ignore"):
+        ref = G.evaluate(ins, outs, vals)
+    got = th.function(ins, outs, **flags)(*vals)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert_parity(g, r, "seed %d output %d" % (seed, k))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", list(range(2500, 2540)))
+def test_random_view_graph_matches_the_oracle(seed):
+    check_view_graph(seed)
+
+
+def test_view_graph_generator_builds(dry_run):
+    for seed in range(2500, 2530):
+        ins, outs, vals = random_view_graph(seed)
+        with np.errstate(all="ignore"):
+            ref = G.evaluate(ins, outs, vals)
+        got = th.function(ins, outs)(*vals)
+        assert [g.shape for g in got] == [r.shape for r in ref], seed
+        assert [g.dtype for g in got] == [r.dtype for r in ref], seed

@@ -633,7 +633,20 @@ def local_mul_to_sqr(fgraph, node):
     return [new] if new.type == node.outputs[0].type else False
 
 
-CANONICALIZE = [local_remove_grad_views, local_shape_lift, local_dimshuffle_fold, local_useless_composite, local_constant_fold,
+@local_optimizer(None)
+def local_useless_subtensor(fgraph, node):
+    """``x[:]``, ``x[:, :]`` ...: an index of full slices only stands for its operand
+    (``local_useless_subtensor``, ``theano/tensor/opt.py:2685-2780``, its case of slices that are all None)."""
+    from . import views as V
+    if type(node.op) is not V.Subtensor or len(node.inputs) != 1:
+        return False
+    if not all(isinstance(i, slice) and i == slice(None) for i in node.op.idx_list):
+        return False
+    x = node.inputs[0]
+    return [x] if x.type == node.outputs[0].type else False
+
+
+CANONICALIZE = [local_remove_grad_views, local_useless_subtensor, local_shape_lift, local_dimshuffle_fold, local_useless_composite, local_constant_fold,
                 local_useless_elemwise, local_fill_sink,
                 local_useless_reduce, local_op_of_op,
                 local_dimshuffle_lift, local_sum_invariant_factor, local_max_and_argmax, local_max_to_min,

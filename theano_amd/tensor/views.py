@@ -279,8 +279,8 @@ class IncSubtensor(Op):
 def subtensor(x, idx):
     x = as_tensor_variable(x)
     idx_list = normalize_index(idx, x.type.ndim)
-    if all(_full_slice(i) for i in idx_list):
-        return x
+    # x[:] is a node of its own, as in the reference (set_subtensor(x[:], y) needs it); canonicalisation
+    # takes it out of a compiled graph (local_useless_subtensor)
     template, syms = split_symbolic(idx_list)
     return Subtensor(template)(x, *syms)
 
