@@ -507,3 +507,80 @@ def test_view_graph_generator_builds(dry_run):
         got = th.function(ins, outs)(*vals)
         assert [g.shape for g in got] == [r.shape for r in ref], seed
         assert [g.dtype for g in got] == [r.dtype for r in ref], seed
+
+
+CPLX_UNARY = [T.neg, T.sqr, T.conj, T.exp, lambda v: T.tanh(v * 0.5), lambda v: T.sin(v), lambda v: T.cos(v),
+              lambda v: T.sqrt(v), lambda v: T.log(v + 3.0), lambda v: T.inv(v + 3.0), lambda v: T.cast(v, "complex128")]
+CPLX_BINARY = [T.add, T.sub, T.mul, lambda a, b: a / (b + 4.0), lambda a, b: T.switch(T.eq(a, b), a, b),
+               lambda a, b: T.complex(T.real(a), T.imag(b)), lambda a, b: a * abs(b), lambda a, b: a + T.angle(b),
+               lambda a, b: T.complex_from_polar(abs(a), T.angle(b))]
+
+
+def random_complex_graph(seed):
+    """Chains over complex64 / complex128 operands mixed with real ones: arithmetic in the reference's
+    formulas (``theano/scalar/basic.py:498-641``), the parts and the polar form, sums and products."""
+    rng = np.random.default_rng(seed)
+    nd = int(rng.integers(1, 4))
+    shape = [int(rng.choice(EXTENTS[1:7])) for _ in range(nd)]
+    ins, vals, terms = [], [], []
+    for k in range(int(rng.integers(2, 4))):
+        dt = str(rng.choice(["complex64", "complex64", "complex128", "float32", "float64"]))
+        bc = [bool(rng.random() < 0.2) for _ in range(nd)]
+        if all(bc):
+            bc[0] = False
+        v = T.TensorType(dt, tuple(bc))("in%d" % k)
+        shp = [1 if b else s for b, s in zip(bc, shape)]
+        val = rng.uniform(-1.5, 1.5, shp)
+        if dt.startswith("complex"):
+            val = val + 1j * rng.uniform(-1.5, 1.5, shp)
+        ins.append(v)
+        vals.append(val.astype(dt))
+        terms.append(v)
+    full = T.TensorType("complex64", (False,) * nd)("full")
+    ins.append(full)
+    vals.append((rng.uniform(-1.5, 1.5, shape) + 1j * rng.uniform(-1.5, 1.5, shape)).astype("complex64"))
+    terms.append(full)
+    for _ in range(int(rng.integers(2, 6))):
+        a = terms[int(rng.integers(len(terms)))]
+        try:
+            if rng.random() < 0.45:
+                terms.append(CPLX_UNARY[int(rng.integers(len(CPLX_UNARY)))](a))
+            else:
+                b = terms[int(rng.integers(len(terms)))]
+                terms.append(CPLX_BINARY[int(rng.integers(len(CPLX_BINARY)))](a, b))
+        except TypeError:           # conj / the parts of a real operand, complex(...) of complex parts
+            continue
+    e = terms[-1] + full
+    axis = int(rng.integers(nd))
+    outs = [e, T.sum(e, axis=axis), T.real(e) * T.imag(e), abs(e), T.sum(abs(e) * 0.1)]
+    if shape[axis] <= 8:
+        outs.append(T.prod(e * 0.5, axis=axis))
+    return ins, outs, vals
+
+
+def check_complex_graph(seed):
+    ins, outs, vals = random_complex_graph(seed)
+    with np.errstate(all="ignore"):
+        ref = G.evaluate(ins, outs, vals)
+    got = th.function(ins, outs, on_unused_input="ignore")(*vals)
+    from conftest import TOL
+    narrow64 = any(v.type.dtype in ("complex64", "float32") for v in ins)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        tol = TOL["complex64"] if narrow64 else None
+        assert_parity(g, r, "seed %d output %d" % (seed, k), tol=tol)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", list(range(3000, 3030)))
+def test_random_complex_graph_matches_the_oracle(seed):
+    check_complex_graph(seed)
+
+
+def test_complex_graph_generator_builds(dry_run):
+    for seed in range(3000, 3020):
+        ins, outs, vals = random_complex_graph(seed)
+        with np.errstate(all="ignore"):
+            ref = G.evaluate(ins, outs, vals)
+        got = th.function(ins, outs, on_unused_input="ignore")(*vals)
+        assert [g.shape for g in got] == [r.shape for r in ref], seed
+        assert [g.dtype for g in got] == [r.dtype for r in ref], seed
