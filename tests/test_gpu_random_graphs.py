@@ -584,3 +584,108 @@ def test_complex_graph_generator_builds(dry_run):
         got = th.function(ins, outs, on_unused_input="ignore")(*vals)
         assert [g.shape for g in got] == [r.shape for r in ref], seed
         assert [g.dtype for g in got] == [r.dtype for r in ref], seed
+
+
+def random_shape_family(seed):
+    """One compiled function, many shapes: a chain over inputs whose broadcast patterns, transpositions and
+    stepped views are fixed by the seed while the extents are not.  Returns (inputs, outputs, make_values) where
+    ``make_values(rng)`` draws extents (0 and 1 included) and the matching argument arrays."""
+    rng = np.random.default_rng(seed)
+    dtype = str(rng.choice(["float32", "float32", "float64", "int32"]))
+    floating = dtype.startswith("float")
+    nd = int(rng.integers(1, 5))
+    unary, binary = (FLOAT_UNARY, FLOAT_BINARY) if floating else (INT_UNARY, INT_BINARY)
+    specs, ins, terms = [], [], []
+    for k in range(int(rng.integers(1, 4))):
+        bc = [bool(rng.random() < 0.25) for _ in range(nd)]
+        if all(bc):
+            bc[int(rng.integers(nd))] = False
+        perm = [int(p) for p in rng.permutation(nd)] if nd > 1 and rng.random() < 0.4 else list(range(nd))
+        step_dim = int(rng.integers(nd)) if rng.random() < 0.3 else None
+        if step_dim is not None and bc[perm[step_dim]]:
+            step_dim = None
+        var = T.TensorType(dtype, tuple(bc[p] for p in perm))("in%d" % k)
+        term = var
+        if step_dim is not None:
+            term = term[tuple(slice(1, None, 2) if d == step_dim else slice(None) for d in range(nd))]
+        if perm != list(range(nd)):
+            term = term.dimshuffle(*[perm.index(d) for d in range(nd)])
+        specs.append((bc, perm, step_dim))
+        ins.append(var)
+        terms.append(term)
+    full = T.TensorType(dtype, (False,) * nd)("full")
+    ins.append(full)
+    terms.append(full)
+    for _ in range(int(rng.integers(2, 7))):
+        a = terms[int(rng.integers(len(terms)))]
+        if rng.random() < 0.4:
+            terms.append(unary[int(rng.integers(len(unary)))](a))
+        else:
+            b = terms[int(rng.integers(len(terms)))]
+            terms.append(binary[int(rng.integers(len(binary)))](a, b))
+    e = terms[-1] + full
+    axes = tuple(sorted(set(int(a) for a in rng.integers(0, nd, int(rng.integers(1, nd + 1))))))
+    outs = [e, T.sum(e, axis=axes), T.sum(e), T.prod(T.cast(T.gt(e, 0), "int8") + 1, axis=axes[0])]
+    if floating:        # the reduction's result broadcast back against its operand; a maximum, because a product or a
+        outs.append(T.maximum(e, T.sum(e, axis=axes, keepdims=True)))     # sum of the two magnifies last-bit differences
+
+    def make_values(vrng):
+        shape = [int(vrng.choice([0, 1, 2, 3, 5, 8, 16, 33, 64, 130])) for _ in range(nd)]
+        while np.prod([max(s, 1) for s in shape]) > MAX_ELEMENTS:
+            shape[int(np.argmax(shape))] //= 2
+        vals = []
+        for bc, perm, step_dim in specs:
+            ishape = [1 if b else s for b, s in zip(bc, shape)]
+            alloc = [ishape[p] for p in perm]
+            if step_dim is not None:
+                alloc[step_dim] = 2 * alloc[step_dim] + 1
+            vals.append(vrng.uniform(-2, 2, alloc).astype(dtype) if floating else
+                        vrng.integers(-50, 50, alloc).astype(dtype))
+        vals.append(vrng.uniform(-2, 2, shape).astype(dtype) if floating else
+                    vrng.integers(-50, 50, shape).astype(dtype))
+        return vals
+    return ins, outs, make_values
+
+
+def check_shape_family(seed, calls=6):
+    ins, outs, make_values = random_shape_family(seed)
+    f = th.function(ins, outs, on_unused_input="ignore")
+    vrng = np.random.default_rng(seed + 77)
+    for call in range(calls):
+        vals = make_values(vrng)
+        with np.errstate(all="ignore"):
+            ref = G.evaluate(ins, outs, vals)
+        got = f(*vals)
+        truth = None
+        for k, (g, r) in enumerate(zip(got, ref)):
+            what = "seed %d call %d (full %s) output %d" % (seed, call, vals[-1].shape, k)
+            try:
+                assert_parity(g, r, what)
+            except AssertionError:
+                # sums of signed terms, and a value added to the sum it mostly cancels: the last bits of the
+                # terms decide; held to the float64 evaluation instead, no farther from it than the oracle is
+                if r.dtype.kind != "f":
+                    raise
+                if truth is None:
+                    with np.errstate(all="ignore"):
+                        truth = G.evaluate(ins, outs, vals, wide=True)
+                assert_within_reference_error(g, r, truth[k], what)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", list(range(4000, 4030)))
+def test_one_function_called_with_many_shapes(seed):
+    check_shape_family(seed)
+
+
+def test_shape_family_generator_builds(dry_run):
+    for seed in range(4000, 4012):
+        ins, outs, make_values = random_shape_family(seed)
+        f = th.function(ins, outs, on_unused_input="ignore")
+        vrng = np.random.default_rng(seed + 77)
+        for _ in range(3):
+            vals = make_values(vrng)
+            with np.errstate(all="ignore"):
+                ref = G.evaluate(ins, outs, vals)
+            got = f(*vals)
+            assert [g.shape for g in got] == [r.shape for r in ref], seed

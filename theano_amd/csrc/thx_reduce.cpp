@@ -225,7 +225,8 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       if (a.shape[d] != kshape[d])
         return fail(THX_ERR_SHAPE, "reduce: output %d has extent %lld along dimension %d, the result has %lld", o,
                     (long long)a.shape[d], d, (long long)kshape[d]);
-      if (a.shape[d] > 1 && a.strides_bytes[d] != expect)
+      // an array without elements has no layout to speak of (its strides depend on who computed them)
+      if (n_out > 0 && a.shape[d] > 1 && a.strides_bytes[d] != expect)
         return fail(THX_ERR_TYPE, "reduce: output %d is not C-contiguous", o);
       expect *= a.shape[d];
     }
@@ -256,8 +257,11 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     }
     const int64_t isz = dtype_size(want);
     int64_t count = 1, expect = 0;
+    for (int d = a.nd - 1; d >= 0; --d) count *= a.shape[d];
+    const bool has_elements = count > 0;
+    count = 1;
     for (int d = a.nd - 1; d >= 0; --d) {
-      if (a.shape[d] > 1) {
+      if (a.shape[d] > 1 && has_elements) {
         if (!expect) {
           if (a.strides_bytes[d] % isz || !a.strides_bytes[d])
             return fail(THX_ERR_TYPE, "reduce: epilogue operand %d has a stride that is not a multiple of its element size", j);
