@@ -221,10 +221,11 @@ def Lop(f, wrt, eval_points, consider_constant=None, disconnected_inputs="raise"
     eps = list(eval_points) if isinstance(eval_points, (list, tuple)) else [eval_points]
     if len(fs) != len(eps):
         raise ValueError("Lop needs one evaluation point per element of f")
-    return grad(None, wrt, known_grads=dict(zip(fs, eps)), disconnected_inputs=disconnected_inputs)
+    return grad(None, wrt, known_grads=dict(zip(fs, eps)), consider_constant=consider_constant,
+                disconnected_inputs=disconnected_inputs)
 
 
-def Rop(f, wrt, eval_points, disconnected_outputs="raise"):
+def Rop(f, wrt, eval_points, disconnected_outputs="raise", return_disconnected="zero"):
     """R operator: the Jacobian of ``f`` with respect to ``wrt`` times
     ``eval_points`` (``theano/gradient.py:155-345``).  Forward mode: every node
     between ``wrt`` and ``f`` is asked for ``R_op(inputs, eval_points)``;
@@ -272,11 +273,22 @@ def Rop(f, wrt, eval_points, disconnected_outputs="raise"):
             continue
         r = seen[id(out.owner)][out.owner.outputs.index(out)] if out.owner is not None else None
         if r is None:
+            message = ("Rop method was asked to compute the gradient with respect to a variable that is not part of "
+                       "the computational graph of variables in wrt, or is used only by a non-differentiable "
+                       "operator: %s" % out)
             if disconnected_outputs == "raise":
-                raise DisconnectedInputError("Rop method was asked to compute the gradient with respect to a variable "
-                                             "that is not part of the computational graph of variables in wrt, or is "
-                                             "used only by a non-differentiable operator: %s" % out)
-            r = T.zeros_like(out)
+                raise DisconnectedInputError(message)
+            if disconnected_outputs == "warn":
+                import warnings
+                warnings.warn(message, stacklevel=2)
+            elif disconnected_outputs != "ignore":
+                raise ValueError("Invalid value for keyword 'disconnected_inputs', valid values are 'ignore', 'warn' "
+                                 "and 'raise'.")
+            how = return_disconnected.lower()
+            if how not in ("zero", "none", "disconnected"):
+                raise ValueError("Invalid value for keyword 'return_disconnected', valid values are 'zero', 'None' "
+                                 "and 'Disconnected'.")
+            r = T.zeros_like(out) if how == "zero" else None if how == "none" else DisconnectedType()()
         result.append(r)
     return result[0] if single else result
 
