@@ -1321,3 +1321,20 @@ def test_function_takes_the_references_arguments_in_its_order(dry_run):
     th.function([x, y], x * 2, on_unused_input="ignore")
     with pytest.raises(ValueError):
         th.function([x], x * 2, on_unused_input="never")
+
+
+def test_shared_takes_the_references_arguments(dry_run):
+    """``theano.shared(value, name=None, strict=False, allow_downcast=None, **kwargs)``
+    (``theano/compile/sharedvalue.py:238-300``) with the device constructor's keywords."""
+    import inspect
+    assert list(inspect.signature(th.shared).parameters) == ["value", "name", "strict", "allow_downcast", "kwargs"]
+    s = th.shared(np.zeros((1, 3), "float32"), "s", broadcastable=(True, False), borrow=True)
+    assert s.name == "s" and s.type.broadcastable == (True, False)
+    s.set_value(np.ones((1, 3), "float32"))
+    with pytest.raises(TypeError):
+        s.set_value(np.ones((1, 3), "float64"))             # would lose precision
+    d = th.shared(np.zeros(3, "float32"), allow_downcast=True)
+    d.set_value(np.ones(3, "float64"))
+    assert d.get_value().dtype == np.float32
+    with pytest.raises(TypeError):
+        th.shared(np.zeros(3), colour="red")

@@ -58,15 +58,25 @@ class SharedVariable(Variable):
         v = self.container[0]
         return v if return_internal_type else v.to_numpy()
 
+    strict, allow_downcast = False, None
+
     def set_value(self, value, borrow=False):
-        self.container[0] = self.type.filter(value)
+        self.container[0] = self.type.filter(value, strict=self.strict, allow_downcast=self.allow_downcast)
 
     def clone(self):
         return self  # shared variables are never copied into a function graph
 
 
-def shared(value, name=None, broadcastable=None):
-    """Device-resident shared variable holding ``value``."""
+def shared(value, name=None, strict=False, allow_downcast=None, **kwargs):
+    """Device-resident shared variable holding ``value`` (``theano.shared``, ``theano/compile/sharedvalue.py:238-300``;
+    the device constructor's keywords ``broadcastable=``, ``borrow=`` and ``target=`` of
+    ``theano/gpuarray/type.py:650-700``: the value is always copied to this library's GPU).  ``strict`` and
+    ``allow_downcast`` govern later ``set_value`` calls as they govern ``filter``."""
+    broadcastable = kwargs.pop("broadcastable", None)
+    kwargs.pop("borrow", None)
+    kwargs.pop("target", None)
+    if kwargs:
+        raise TypeError("shared() got unexpected keyword arguments %s" % sorted(kwargs))
     from .hip.ops import HipArrayType, HipArrayVariable
     from .hip.runtime import HipArray
     if isinstance(value, HipArray):
@@ -80,7 +90,9 @@ def shared(value, name=None, broadcastable=None):
 
     class _Shared(SharedVariable, HipArrayVariable):
         pass
-    return _Shared(t, t.filter(value), name=name)
+    sv = _Shared(t, t.filter(value), name=name)
+    sv.strict, sv.allow_downcast = bool(strict), allow_downcast
+    return sv
 
 
 class UnusedInputError(Exception):
