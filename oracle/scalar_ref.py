@@ -11,7 +11,11 @@ expression (``c_common_type``), the operation is done in that type, and the
 result is converted to the output dtype as the C assignment does.
 
 Pinning (tests/test_oracle_scalar.py): Mod / IntDiv against Python ``%`` and
-``//`` on the exhaustive int8 grid of ``theano/tensor/tests/test_basic.py:878-896``;
+``//`` on the exhaustive int8 grid of ``theano/tensor/tests/test_basic.py:878-896``, and - for every pair
+of integer operand types, where the sign tests see each operand in its own type and the divisions C's
+common type - against the reference's C text compiled by gcc, over the ends of every type's range
+(operands whose negation overflows, which C leaves undefined and compilers treat differently, wrap here;
+that choice is pinned by literal values);
 comparisons and bit ops against the truth tables of
 ``theano/scalar/tests/test_basic.py:187-256``; sigmoid against ``1/(1+exp(-x))``
 (``theano/tensor/nnet/tests/test_sigm.py:29-41``); max/min NaN propagation
@@ -117,53 +121,88 @@ def true_div(out_dtype, x, y):
     return _arith(lambda a, b: a / b, out_dtype, x, y)
 
 
-def _c_div(a, b):
-    """C integer division: truncation toward zero (b != 0)."""
-    q = np.abs(a.astype(object)) // np.abs(b.astype(object))
-    return np.where((a < 0) != (b < 0), -q, q)
+def _promoted(dtype):
+    """C's integer promotion: every type narrower than int computes as int."""
+    d = str(dtype)
+    return "int32" if _RANK[d] <= 2 else d
 
 
-def _c_mod(a, b):
-    return a.astype(object) - _c_div(a, b) * b.astype(object)
+def _wrap_int(v, dtype):
+    """A Python int as the two's-complement value of a C integer type.  Signed overflow is undefined in C;
+    the hosts and devices the reference runs on wrap, and so does this restatement."""
+    bits = np.dtype(dtype).itemsize * 8
+    v &= (1 << bits) - 1
+    if np.dtype(dtype).kind == "i" and v >= (1 << (bits - 1)):
+        v -= 1 << bits
+    return v
+
+
+class _C(object):
+    """One C integer value with its type, for the element-by-element restatements: arithmetic follows the
+    usual arithmetic conversions, / and % truncate."""
+
+    def __init__(self, v, dtype):
+        self.t = _promoted(dtype)
+        self.v = _wrap_int(int(v), self.t)
+
+    def _pair(self, o):
+        t = c_common_type(self.t, o.t)
+        return _wrap_int(self.v, t), _wrap_int(o.v, t), t
+
+    def neg(self):
+        return _C(-self.v, self.t)
+
+    def add(self, o):
+        a, b, t = self._pair(o)
+        return _C(a + b, t)
+
+    def sub(self, o):
+        a, b, t = self._pair(o)
+        return _C(a - b, t)
+
+    def div(self, o):
+        a, b, t = self._pair(o)
+        q = abs(a) // abs(b)
+        return _C(-q if (a < 0) != (b < 0) else q, t)
+
+    def mod(self, o):
+        a, b, t = self._pair(o)
+        q = abs(a) // abs(b)
+        q = -q if (a < 0) != (b < 0) else q
+        return _C(a - q * b, t)
 
 
 def int_div(out_dtype, x, y):
-    """theano/scalar/basic.py:2009-2025: four sign cases over C division."""
+    """theano/scalar/basic.py:2009-2025, element by element: the four sign cases over C's truncating
+    division, every operand in its own C type (the sign tests see the operands as they are, the
+    divisions the usual common type)."""
     ct = c_common_type(x.dtype, y.dtype)
     if np.dtype(ct).kind == "f":
         with np.errstate(all="ignore"):
             return _conv(np.floor(_conv(x, ct) / _conv(y, ct)), out_dtype)
-    x, y = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
-    xo, yo = x.astype(object), y.astype(object)
+    x, y = np.broadcast_arrays(np.asarray(x), np.asarray(y))
     res = np.zeros(x.shape, dtype=object)
-    nz = y != 0
+    one, zero = _C(1, "int32"), _C(0, "int32")
     for idx in np.ndindex(x.shape):
-        if not nz[idx]:
+        a, b = _C(x[idx], x.dtype), _C(y[idx], y.dtype)
+        if b.v == 0:
             continue
-        a, b = int(xo[idx]), int(yo[idx])
-
-        def cdiv(p, q):
-            s = -1 if (p < 0) != (q < 0) else 1
-            return s * (abs(p) // abs(q))
-
-        def cmod(p, q):
-            return p - cdiv(p, q) * q
-        if b < 0:
-            if a < 0:
-                r = cdiv(-a, -b)
+        if b.v < 0:
+            if a.v < 0:
+                r = a.neg().div(b.neg())
             else:
-                r = -cdiv(a, -b) - (0 if cmod(a, -b) == 0 else 1)
+                r = a.div(b.neg()).neg().sub(zero if a.mod(b.neg()).v == 0 else one)
         else:
-            if a < 0:
-                r = -cdiv(-a, b) - (0 if cmod(-a, b) == 0 else 1)
+            if a.v < 0:
+                r = a.neg().div(b).neg().sub(zero if a.neg().mod(b).v == 0 else one)
             else:
-                r = cdiv(a, b)
-        res[idx] = r
+                r = a.div(b)
+        res[idx] = r.v
     return _wrap(res, out_dtype)
 
 
 def mod(out_dtype, x, y):
-    """theano/scalar/basic.py:2119-2135: remainder with the divisor's sign."""
+    """theano/scalar/basic.py:2119-2135, element by element: remainder with the divisor's sign."""
     ct = c_common_type(x.dtype, y.dtype)
     if np.dtype(ct).kind == "f":
         a, b = np.broadcast_arrays(_conv(x, "float64"), _conv(y, "float64"))
@@ -175,30 +214,26 @@ def mod(out_dtype, x, y):
                                   np.where(a < 0, -np.fmod(-a, b) + np.where(np.fmod(-a, b) != 0, b, 0),
                                            np.fmod(a, b))))
         return _conv(r, out_dtype)
-    x, y = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
-    xo, yo = x.astype(object), y.astype(object)
+    x, y = np.broadcast_arrays(np.asarray(x), np.asarray(y))
     res = np.zeros(x.shape, dtype=object)
+    zero = _C(0, "int32")
     for idx in np.ndindex(x.shape):
-        a, b = int(xo[idx]), int(yo[idx])
-        if b == 0:
+        a, b = _C(x[idx], x.dtype), _C(y[idx], y.dtype)
+        if b.v == 0:
             continue
-
-        def cmod(p, q):
-            s = -1 if (p < 0) != (q < 0) else 1
-            return p - s * (abs(p) // abs(q)) * q
-        if b < 0:
-            if a < 0:
-                r = -cmod(-a, -b)
+        if b.v < 0:
+            if a.v < 0:
+                r = a.neg().mod(b.neg()).neg()
             else:
-                m = cmod(a, -b)
-                r = m + (b if m != 0 else 0)
+                m = a.mod(b.neg())
+                r = m.add(b if m.v != 0 else zero)
         else:
-            if a < 0:
-                m = cmod(-a, b)
-                r = -m + (b if m != 0 else 0)
+            if a.v < 0:
+                m = a.neg().mod(b)
+                r = m.neg().add(b if m.v != 0 else zero)
             else:
-                r = cmod(a, b)
-        res[idx] = r
+                r = a.mod(b)
+        res[idx] = r.v
     return _wrap(res, out_dtype)
 
 
@@ -214,33 +249,77 @@ def _wrap(obj_arr, dtype):
     return flat.astype(dt).reshape(obj_arr.shape)
 
 
-def mod_fast(out_dtype, x, y):
-    """Vectorised equivalent of ``mod`` for integers: NumPy's ``%`` already has
-    the divisor's sign; zero divisors give 0 as on the device."""
-    ct = c_common_type(x.dtype, y.dtype)
-    a, b = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
+def _cneg(a):
+    """-a in C: in the promoted type, wrapping."""
     with np.errstate(all="ignore"):
-        r = np.where(b == 0, 0, np.mod(a, np.where(b == 0, 1, b)))
-    return _conv(r, out_dtype)
+        return -_conv(a, _promoted(a.dtype))
+
+
+def _cbin(fn, a, b):
+    ct = c_common_type(a.dtype, b.dtype)
+    with np.errstate(all="ignore"):
+        return fn(_conv(a, ct), _conv(b, ct))
+
+
+def _ctrunc_mod(a, b):
+    return _cbin(np.fmod, a, b)                     # on integers: C's %, the sign of the dividend
+
+
+def _ctrunc_div(a, b):
+    return _cbin(lambda p, q: (p - np.fmod(p, q)) // q, a, b)       # exact after the remainder is taken off
+
+
+def mod_fast(out_dtype, x, y):
+    """Vectorised ``mod``: the same C expressions over whole arrays (NumPy's fixed-width integers wrap as the
+    restatement's do); zero divisors give 0 as on the device."""
+    ct = c_common_type(x.dtype, y.dtype)
+    if np.dtype(ct).kind == "f":
+        return mod(out_dtype, x, y)
+    x, y = np.broadcast_arrays(np.asarray(x), np.asarray(y))
+    y1 = np.where(y == 0, np.ones((), y.dtype), y)
+    ny, nx = _cneg(y1), _cneg(x)
+    izero = np.zeros((), "int32")
+    yt = c_common_type(y.dtype, "int32")            # the type of (m != 0 ? y : 0)
+    y_or_0 = lambda m: np.where(m != 0, _conv(y1, yt), np.zeros((), yt))                   # noqa: E731
+    with np.errstate(all="ignore"):
+        mm = _cneg(_ctrunc_mod(nx, ny))
+        m = _ctrunc_mod(x, ny)
+        pm = _cbin(np.add, m, y_or_0(m))
+        m = _ctrunc_mod(nx, y1)
+        mp = _cbin(np.add, _cneg(m), y_or_0(m))
+        pp = _ctrunc_mod(x, y1)
+    pick = lambda v: _conv(v, out_dtype)                                                   # noqa: E731
+    r = np.where(y < 0, np.where(x < 0, pick(mm), pick(pm)), np.where(x < 0, pick(mp), pick(pp)))
+    return np.where(y == 0, pick(izero), r).astype(out_dtype)
 
 
 def int_div_fast(out_dtype, x, y):
-    """Integers: NumPy's ``//`` (floor, zero divisors give 0 as on the device).  Floats follow
-    the C text (``theano/scalar/basic.py:1985-2025``): ``floor(x / y)`` over the magnitudes
-    with the quotient rounded in C's common type first - so a quotient that rounds up to an
+    """Vectorised ``int_div``.  Integers: the same C expressions over whole arrays (zero divisors give 0 as on
+    the device).  Floats follow the C text (``theano/scalar/basic.py:1985-2025``): ``floor(x / y)`` over the
+    magnitudes with the quotient rounded in C's common type first - so a quotient that rounds up to an
     integer floors to that integer - and the sign cases corrected through ``fmod``."""
     ct = c_common_type(x.dtype, y.dtype)
-    a, b = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
-    with np.errstate(all="ignore"):
-        if np.dtype(ct).kind == "f":
+    if np.dtype(ct).kind == "f":
+        a, b = np.broadcast_arrays(_conv(x, ct), _conv(y, ct))
+        with np.errstate(all="ignore"):
             pp = np.floor(a / b)
             mm = np.floor((-a) / (-b))
             pm = -np.floor(a / (-b)) - np.where(np.fmod(a, -b) == 0, 0, 1)
             mp = -np.floor((-a) / b) - np.where(np.fmod(-a, b) == 0, 0, 1)
             r = np.where(b == 0, pp, np.where(b < 0, np.where(a < 0, mm, pm), np.where(a < 0, mp, pp)))
-        else:
-            r = np.where(b == 0, 0, np.floor_divide(a, np.where(b == 0, 1, b)))
-    return _conv(r, out_dtype)
+        return _conv(r, out_dtype)
+    x, y = np.broadcast_arrays(np.asarray(x), np.asarray(y))
+    y1 = np.where(y == 0, np.ones((), y.dtype), y)
+    ny, nx = _cneg(y1), _cneg(x)
+    step = lambda m: np.where(m == 0, np.zeros((), "int32"), np.ones((), "int32"))        # noqa: E731
+    with np.errstate(all="ignore"):
+        mm = _ctrunc_div(nx, ny)
+        pm = _cbin(np.subtract, _cneg(_ctrunc_div(x, ny)), step(_ctrunc_mod(x, ny)))
+        mp = _cbin(np.subtract, _cneg(_ctrunc_div(nx, y1)), step(_ctrunc_mod(nx, y1)))
+        pp = _ctrunc_div(x, y1)
+    pick = lambda v: _conv(v, out_dtype)                                                   # noqa: E731
+    r = np.where(y < 0, np.where(x < 0, pick(mm), pick(pm)), np.where(x < 0, pick(mp), pick(pp)))
+    return np.where(y == 0, pick(np.zeros((), "int32")), r).astype(out_dtype)
 
 
 def pow_(out_dtype, x, y):

@@ -689,3 +689,167 @@ def test_shape_family_generator_builds(dry_run):
                 ref = G.evaluate(ins, outs, vals)
             got = f(*vals)
             assert [g.shape for g in got] == [r.shape for r in ref], seed
+
+
+def random_argmax_graph(seed):
+    """max_and_argmax / argmax / argmin over random axis sets of a view, on values with many ties and (floating
+    point) NaN and infinities sprinkled in: the position must be NumPy's first occurrence."""
+    rng = np.random.default_rng(seed)
+    dtype = str(rng.choice(["float32", "float32", "float64", "float16", "int32", "int8", "uint8", "int64", "bool"]))
+    nd = int(rng.integers(1, 5))
+    shape = [int(rng.choice([1, 2, 3, 5, 8, 17, 64, 130])) for _ in range(nd)]
+    while np.prod(shape) > MAX_ELEMENTS:
+        shape[int(np.argmax(shape))] //= 2
+    x = T.TensorType(dtype, (False,) * nd)("x")
+    if dtype == "bool":
+        xv = rng.random(shape) < 0.3
+    elif dtype.startswith("float"):
+        xv = rng.integers(-3, 4, shape).astype(dtype)            # few distinct values: ties everywhere
+        xv += (rng.random(shape) < 0.3) * rng.standard_normal(shape).astype(dtype)
+        flat = xv.reshape(-1)
+        for special in (np.nan, np.inf, -np.inf):
+            if rng.random() < 0.4 and flat.size:
+                flat[rng.integers(0, flat.size, max(1, flat.size // 50))] = special
+    else:
+        lo = 0 if dtype.startswith("u") else -4
+        xv = rng.integers(lo, 5, shape).astype(dtype)
+    v = x
+    if nd > 1 and rng.random() < 0.4:
+        perm = [int(p) for p in rng.permutation(nd)]
+        v = v.dimshuffle(*perm)
+    if rng.random() < 0.3:
+        d = int(rng.integers(nd))
+        v = v[tuple(slice(None, None, -1) if k == d else slice(None) for k in range(nd))]
+    axes = sorted(set(int(a) for a in rng.integers(0, nd, int(rng.integers(1, nd + 1)))))
+    axis = None if rng.random() < 0.2 else (axes[0] if len(axes) == 1 and rng.random() < 0.5 else axes)
+    keep = bool(rng.random() < 0.3)
+    outs = list(T.max_and_argmax(v, axis=axis, keepdims=keep))
+    one = axes[0]
+    outs.append(T.argmax(v, axis=one))
+    if dtype not in ("int8", "uint8", "bool"):       # argmin negates its operand: wraps for the extreme integers
+        outs.append(T.argmin(v, axis=one, keepdims=keep))
+        outs.append(T.min(v, axis=axis))
+    return [x], outs, [xv]
+
+
+def check_argmax_graph(seed):
+    ins, outs, vals = random_argmax_graph(seed)
+    if 0 in vals[0].shape:
+        return
+    with np.errstate(all="ignore"):
+        ref = G.evaluate(ins, outs, vals)
+    got = th.function(ins, outs)(*vals)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert g.dtype == r.dtype and g.shape == r.shape, (seed, k)
+        assert np.array_equal(g, r, equal_nan=r.dtype.kind == "f"), "seed %d output %d: %s against %s" % (
+            seed, k, g.reshape(-1)[:8], r.reshape(-1)[:8])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", list(range(5000, 5040)))
+def test_random_argmax_graph_matches_the_oracle(seed):
+    check_argmax_graph(seed)
+
+
+def test_argmax_graph_generator_builds(dry_run):
+    for seed in range(5000, 5030):
+        ins, outs, vals = random_argmax_graph(seed)
+        with np.errstate(all="ignore"):
+            ref = G.evaluate(ins, outs, vals)
+        got = th.function(ins, outs)(*vals)
+        assert [g.shape for g in got] == [r.shape for r in ref], seed
+        assert [g.dtype for g in got] == [r.dtype for r in ref], seed
+
+
+def random_integer_graph(seed):
+    """Chains over every integer type, signed and unsigned, with values over the whole range of each (wrap-around
+    included): +, -, *, the bit operations, floor division and modulo with divisors of both signs, comparisons,
+    casts between the widths, switch; sums (wrapping in their int64 / uint64 accumulators), maxima, minima, and
+    the bitwise reductions.  int64 beside uint64 is float64 arithmetic, as NumPy's promotion says."""
+    rng = np.random.default_rng(seed)
+    family = ["bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64"]
+    nd = int(rng.integers(1, 4))
+    shape = [int(rng.choice(EXTENTS[1:])) for _ in range(nd)]
+    ins, vals, terms = [], [], []
+
+    def values(dt, shp):
+        if dt == "bool":
+            return rng.random(shp) < 0.5
+        info = np.iinfo(dt)
+        kind = rng.integers(3)
+        if kind == 0:                                   # small values
+            return rng.integers(max(info.min, -50), 50, shp).astype(dt)
+        if kind == 1:                                   # the whole range
+            return rng.integers(info.min, info.max, shp, dtype=dt, endpoint=True)
+        near = rng.integers(0, 4, shp).astype(dt)       # next to the ends
+        return np.where(rng.random(shp) < 0.5, info.max - near, info.min + near).astype(dt)
+
+    for k in range(int(rng.integers(2, 5))):
+        dt = str(rng.choice(family))
+        bc = [bool(rng.random() < 0.2) for _ in range(nd)]
+        if all(bc):
+            bc[0] = False
+        v = T.TensorType(dt, tuple(bc))("in%d" % k)
+        ins.append(v)
+        vals.append(values(dt, [1 if b else s for b, s in zip(bc, shape)]))
+        terms.append(v)
+    dt = str(rng.choice(family[1:]))
+    full = T.TensorType(dt, (False,) * nd)("full")
+    ins.append(full)
+    vals.append(values(dt, shape))
+    terms.append(full)
+    unary = [abs, lambda v: ~v, lambda v: T.cast(v, "int8"), lambda v: T.cast(v, "uint16"), lambda v: T.cast(v, "uint32"),
+             lambda v: T.cast(v, "int64"), lambda v: T.cast(v, "uint64"), lambda v: T.sqr(v), lambda v: v * 3,
+             lambda v: T.cast(T.neq(v, 0), "uint8") + v, lambda v: v // 7, lambda v: v % 5, lambda v: T.sgn(v)]
+    binary = [T.add, T.sub, T.mul, T.maximum, T.minimum, lambda a, b: a & b, lambda a, b: a | b, lambda a, b: a ^ b,
+              lambda a, b: T.int_div(a, abs(b) | 1), lambda a, b: T.mod(a, abs(b) | 1), lambda a, b: T.mod(a, -(abs(b) | 1)),
+              lambda a, b: T.switch(T.lt(a, b), a, b), lambda a, b: T.eq(a, b) + a, lambda a, b: T.ge(a, b) ^ T.le(b, a)]
+    for _ in range(int(rng.integers(2, 7))):
+        a = terms[int(rng.integers(len(terms)))]
+        try:
+            if rng.random() < 0.4:
+                t = unary[int(rng.integers(len(unary)))](a)
+            else:
+                b = terms[int(rng.integers(len(terms)))]
+                t = binary[int(rng.integers(len(binary)))](a, b)
+        except TypeError:               # bit operations on a float64 born of int64 beside uint64, - of a bool
+            continue
+        if t.type.dtype.startswith("float"):
+            continue                    # the integer family only: float64 results stay out of the chain
+        terms.append(t)
+    e = terms[-1]
+    if e.type.ndim < nd or any(e.type.broadcastable) or e.type.dtype == "bool":
+        ee = e + full
+        e = ee if not ee.type.dtype.startswith("float") else T.cast(e, "int64") + T.cast(full, "int64")
+    axis = int(rng.integers(nd))
+    outs = [e, T.sum(e, axis=axis), T.max(e, axis=axis), T.min(e), T.any(e, axis=axis), T.all(e)]
+    if shape[axis] <= 8:
+        outs.append(T.prod(e, axis=axis))
+    return ins, outs, vals
+
+
+def check_integer_graph(seed, **flags):
+    ins, outs, vals = random_integer_graph(seed)
+    with np.errstate(all="ignore"):
+        ref = G.evaluate(ins, outs, vals)
+    got = th.function(ins, outs, on_unused_input="ignore", **flags)(*vals)
+    for k, (g, r) in enumerate(zip(got, ref)):
+        assert g.dtype == r.dtype and g.shape == r.shape, (seed, k, g.dtype, r.dtype)
+        assert np.array_equal(g, r), "seed %d output %d (%s): %s against %s" % (
+            seed, k, g.dtype, g.reshape(-1)[:6], r.reshape(-1)[:6])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", list(range(6000, 6040)))
+def test_random_integer_graph_matches_the_oracle_bit_for_bit(seed):
+    check_integer_graph(seed)
+
+
+def test_integer_graph_generator_builds(dry_run):
+    for seed in range(6000, 6030):
+        ins, outs, vals = random_integer_graph(seed)
+        with np.errstate(all="ignore"):
+            ref = G.evaluate(ins, outs, vals)
+        got = th.function(ins, outs, on_unused_input="ignore")(*vals)
+        assert [g.shape for g in got] == [r.shape for r in ref], seed
+        assert [g.dtype for g in got] == [r.dtype for r in ref], seed

@@ -492,3 +492,90 @@ def test_scalar_type_tuples_constructors_and_output_policies():
         with pytest.raises(TypeError, match="complex"):
             policy(scal.complex64)
     assert scal.floor_div is scal.int_div
+
+
+_C_NAMES = {"bool": "unsigned char", "int8": "signed char", "uint8": "unsigned char", "int16": "short",
+            "uint16": "unsigned short", "int32": "int", "uint32": "unsigned int", "int64": "long long",
+            "uint64": "unsigned long long"}
+
+
+def _integer_grid(dtype):
+    if dtype == "bool":
+        return np.array([False, True])
+    info = np.iinfo(dtype)
+    vals = {info.min, info.min + 1, info.min + 2, info.max, info.max - 1, info.max - 2, 0, 1, 2, 3, 5, 7, 100}
+    if info.min < 0:
+        vals |= {-1, -2, -3, -5, -7, -100}
+    return np.array(sorted(vals), dtype=dtype)
+
+
+def test_integer_division_and_modulo_follow_c_typing_with_gcc_as_the_judge(tmp_path):
+    """The reference's C text for ``//`` and ``%`` (``theano/scalar/basic.py:2009-2025, 2119-2135``) compiled by
+    gcc for every pair of integer operand types - the sign tests see each operand in its own type, the
+    divisions C's common type, negations wrap (``-fwrapv``: what the reference's hosts do with its undefined
+    signed overflow) - against both of the oracle's restatements, over the ends of every type's range and small
+    values of either sign.  So -5 (int32) % 3 (uint32) is 1, not the 2 that converting both operands first
+    gives."""
+    import ctypes
+    import subprocess
+    types = list(_C_NAMES)
+    src = ["#define MOD(a, b) ((a) % (b))", "#define DIV(a, b) ((a) / (b))"]
+    pairs = []
+    for tx in types:
+        for ty in types:
+            out = str(np.promote_types(tx, ty))
+            if out.startswith("float"):
+                continue                                    # int64 beside uint64: the float branch of the ops
+            pairs.append((tx, ty, out))
+            cx, cy, co = _C_NAMES[tx], _C_NAMES[ty], _C_NAMES[out]
+            src.append("""
+void mod_%(tx)s_%(ty)s(const %(cx)s* xs, const %(cy)s* ys, long long* zs, int n) {
+  for (int i = 0; i < n; ++i) { %(cx)s x = xs[i]; %(cy)s y = ys[i]; %(co)s z;
+    if (y == 0) { z = 0; } else if (y < 0) { if (x < 0) { z = -(MOD(-x, -y)); } else { z = (MOD(x, -y)) + (MOD(x, -y) != 0 ? y : 0); } }
+    else { if (x < 0) { z = - MOD(-x, y) + (MOD(-x, y) != 0 ? y : 0); } else { z = MOD(x, y); } }
+    zs[i] = (long long)z; } }
+void div_%(tx)s_%(ty)s(const %(cx)s* xs, const %(cy)s* ys, long long* zs, int n) {
+  for (int i = 0; i < n; ++i) { %(cx)s x = xs[i]; %(cy)s y = ys[i]; %(co)s z;
+    if (y == 0) { z = 0; } else if (y < 0) { if (x < 0) { z = DIV(-x, -y); } else { z = -DIV(x, -y) - ((MOD(x, -y) == 0) ? 0 : 1); } }
+    else { if (x < 0) { z = -DIV(-x, y) - ((MOD(-x, y) == 0) ? 0 : 1); } else { z = DIV(x, y); } }
+    zs[i] = (long long)z; } }
+""" % dict(tx=tx, ty=ty, cx=cx, cy=cy, co=co))
+    c_file, so_file = tmp_path / "judge.c", tmp_path / "judge.so"
+    c_file.write_text("\n".join(src))
+    subprocess.run(["gcc", "-O2", "-fwrapv", "-shared", "-fPIC", "-w", str(c_file), "-o", str(so_file)], check=True)
+    lib = ctypes.CDLL(str(so_file))
+    checked = 0
+    for tx, ty, out in pairs:
+        gx, gy = _integer_grid(tx), _integer_grid(ty)
+        x = np.repeat(gx, len(gy))
+        y = np.tile(gy, len(gx))
+        keep = y != 0
+        # -x of the most negative int / long long is undefined in C and the reference's text negates both
+        # operands: what comes out depends on the compiler (gcc folds (-x) / (-y) back into x / y, which traps
+        # for y == -1 and is the exact quotient otherwise; without the fold the negation wraps).  Those operands
+        # are outside what the reference defines; the restatements' choice for them is checked below.
+        for t, v in ((tx, x), (ty, y)):
+            if t in ("int32", "int64"):
+                keep &= v != np.iinfo(t).min
+        x, y = np.ascontiguousarray(x[keep]), np.ascontiguousarray(y[keep])
+        z = np.zeros(len(x), "int64")
+        for name, slow, fast in (("mod", S.mod, S.mod_fast), ("div", S.int_div, S.int_div_fast)):
+            getattr(lib, "%s_%s_%s" % (name, tx, ty))(x.ctypes.data_as(ctypes.c_void_p), y.ctypes.data_as(ctypes.c_void_p),
+                                                    z.ctypes.data_as(ctypes.c_void_p), ctypes.c_int(len(x)))
+            want = z.astype(out) if out != "bool" else z != 0
+            for which, fn in (("element by element", slow), ("vectorised", fast)):
+                got = fn(out, x, y)
+                assert got.dtype == np.dtype(out)
+                bad = np.flatnonzero(got != want)
+                assert bad.size == 0, "%s %s(%s, %s): x=%s y=%s gives %s, gcc %s" % (
+                    which, name, tx, ty, x[bad[0]], y[bad[0]], got[bad[0]], want[bad[0]])
+            checked += len(x)
+    assert checked > 20000
+    assert int(S.mod("int64", np.asarray([-5], "int32"), np.asarray([3], "uint32"))[0]) == 1
+    # the undefined operands: negation wraps (the most negative value is its own negative), in both restatements
+    lo64, lo32 = np.asarray([np.iinfo("int64").min]), np.asarray([np.iinfo("int32").min], "int32")
+    for fn_mod, fn_div in ((S.mod, S.int_div), (S.mod_fast, S.int_div_fast)):
+        assert int(fn_mod("int64", lo64, np.asarray([5], "int8"))[0]) == 8          # -(lo % 5) + 5 with lo % 5 == -3
+        assert int(fn_div("int32", lo32, np.asarray([-128], "int8"))[0]) == -16777216
+        assert int(fn_div("int64", lo64, np.asarray([-1], "int64"))[0]) == np.iinfo("int64").min
+        assert int(fn_mod("int32", np.asarray([1], "int32"), lo32)[0]) == np.iinfo("int32").min + 1

@@ -69,6 +69,45 @@ __device__ __forceinline__ float thx_fsqrt(float x) {
 __device__ __forceinline__ float thx_fsqrt(float x) { return sqrtf(x); }
 #endif
 
+// Signed integer arithmetic in two's complement: a sum, difference, product or negation that leaves the
+// range wraps, as NumPy's does and as the reference's compiled C does on its hosts.  Written through the
+// unsigned type, because signed overflow is undefined in C++ and the compiler builds on that: abs(x) | 1
+// "cannot" be negative, so a branch on its sign disappears and x % -(abs(y) | 1) comes out with the wrong
+// sign for y = INT_MIN.  The operands take C's usual common type first, as in the reference's expressions;
+// every type but int and long long computes as written.
+template <class C> __device__ __forceinline__ C thx_wadd_(C a, C b) { return a + b; }
+template <class C> __device__ __forceinline__ C thx_wsub_(C a, C b) { return a - b; }
+template <class C> __device__ __forceinline__ C thx_wmul_(C a, C b) { return a * b; }
+__device__ __forceinline__ int thx_wadd_(int a, int b) { return (int)((unsigned)a + (unsigned)b); }
+__device__ __forceinline__ int thx_wsub_(int a, int b) { return (int)((unsigned)a - (unsigned)b); }
+__device__ __forceinline__ int thx_wmul_(int a, int b) { return (int)((unsigned)a * (unsigned)b); }
+__device__ __forceinline__ long long thx_wadd_(long long a, long long b) {
+  return (long long)((unsigned long long)a + (unsigned long long)b);
+}
+__device__ __forceinline__ long long thx_wsub_(long long a, long long b) {
+  return (long long)((unsigned long long)a - (unsigned long long)b);
+}
+__device__ __forceinline__ long long thx_wmul_(long long a, long long b) {
+  return (long long)((unsigned long long)a * (unsigned long long)b);
+}
+template <class A, class B> __device__ __forceinline__ auto thx_wadd(A a, B b) -> decltype(a + b) {
+  typedef decltype(a + b) C;
+  return thx_wadd_((C)a, (C)b);
+}
+template <class A, class B> __device__ __forceinline__ auto thx_wsub(A a, B b) -> decltype(a - b) {
+  typedef decltype(a - b) C;
+  return thx_wsub_((C)a, (C)b);
+}
+template <class A, class B> __device__ __forceinline__ auto thx_wmul(A a, B b) -> decltype(a * b) {
+  typedef decltype(a * b) C;
+  return thx_wmul_((C)a, (C)b);
+}
+template <class A> __device__ __forceinline__ auto thx_wneg(A a) -> decltype(-a) {
+  typedef decltype(-a) C;
+  return thx_wsub_((C)0, (C)a);
+}
+template <class A> __device__ __forceinline__ auto thx_wabs(A a) -> decltype(-a) { return a < 0 ? thx_wneg(a) : a; }
+
 // exp(x) in single precision.  In the 2.5-ulp build: one hardware exp2 of the rounded product
 // x * log2(e); the rounding of the product is a relative error of up to |x| * 4e-8 in the result
 // (3.8e-6 at the ends of the finite range, |x| = 88), overflow gives infinity and underflow zero as

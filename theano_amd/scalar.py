@@ -757,12 +757,23 @@ def _to_complex_result(node, inputs):
     return ["(%s)%s" % (ct, i) for i in inputs]
 
 
+def _wrapping(fn, operands):
+    """``a op b op c`` from left to right through the library's wrapping helper: signed integer results that
+    leave their range wrap as NumPy's do instead of being undefined (kernels/thx_common.h)."""
+    expr = operands[0]
+    for o in operands[1:]:
+        expr = "%s(%s, %s)" % (fn, expr, o)
+    return expr if len(operands) > 1 else "(%s)" % expr
+
+
 class Add(ScalarOp):
     identity = 0
     commutative = True
     associative = True
 
     def c_code(self, node, inputs, outputs):
+        if node.outputs[0].type.dtype in int_dtypes and inputs:
+            return "%s = %s;" % (outputs[0], _wrapping("thx_wadd", inputs))
         sym = " || " if node.outputs[0].type == bool_ else " + "
         inputs = _to_complex_result(node, inputs)
         return "%s = %s;" % (outputs[0], sym.join(inputs) if inputs else "0")
@@ -780,6 +791,8 @@ class Mul(ScalarOp):
     associative = True
 
     def c_code(self, node, inputs, outputs):
+        if node.outputs[0].type.dtype in int_dtypes and inputs:
+            return "%s = %s;" % (outputs[0], _wrapping("thx_wmul", inputs))
         sym = " && " if node.outputs[0].type == bool_ else " * "
         inputs = _to_complex_result(node, inputs)
         return "%s = %s;" % (outputs[0], sym.join(inputs) if inputs else "1")
@@ -793,6 +806,8 @@ class Mul(ScalarOp):
 
 class Sub(BinaryScalarOp):
     def c_code(self, node, inputs, outputs):
+        if node.outputs[0].type.dtype in int_dtypes:
+            return "%s = thx_wsub(%s, %s);" % (outputs[0], inputs[0], inputs[1])
         inputs = _to_complex_result(node, inputs)
         return "%s = %s - %s;" % (outputs[0], inputs[0], inputs[1])
 
@@ -893,14 +908,18 @@ class IntDiv(BinaryScalarOp):
             d = lambda a, b: "%s(thx_exact_div(%s, %s))" % (fl, a, b)
             m = lambda a, b: "%s(%s, %s)" % (fm, a, b)
             zero = "%s = %s;" % (z, d(x, y))
-        nx, ny = "(-%s)" % x, "(-%s)" % y
+        # integer negations and the final subtraction wrap (the most negative value is its own negative)
+        neg = (lambda a: "thx_wneg(%s)" % a) if t in discrete_dtypes else (lambda a: "(-%s)" % a)
+        less = (lambda a, b: "thx_wsub(%s, %s)" % (a, b)) if t in discrete_dtypes else (lambda a, b: "%s - %s" % (a, b))
+        nx, ny = neg(x), neg(y)
         return ("if (%(y)s == 0) { %(zero)s } "
                 "else if (%(y)s < 0) { if (%(x)s < 0) { %(z)s = %(mm)s; } "
-                "else { %(z)s = -%(pm)s - ((%(mpm)s == 0) ? 0 : 1); } } "
-                "else { if (%(x)s < 0) { %(z)s = -%(mp)s - ((%(mmp)s == 0) ? 0 : 1); } "
+                "else { %(z)s = %(a)s; } } "
+                "else { if (%(x)s < 0) { %(z)s = %(b)s; } "
                 "else { %(z)s = %(pp)s; } }") % dict(
-                    x=x, y=y, z=z, zero=zero, mm=d(nx, ny), pm=d(x, ny), mpm=m(x, ny), mp=d(nx, y), mmp=m(nx, y),
-                    pp=d(x, y))
+                    x=x, y=y, z=z, zero=zero, mm=d(nx, ny), pp=d(x, y),
+                    a=less(neg(d(x, ny)), "((%s == 0) ? 0 : 1)" % m(x, ny)),
+                    b=less(neg(d(nx, y)), "((%s == 0) ? 0 : 1)" % m(nx, y)))
 
     def L_op(self, inputs, outputs, gout):
         return [i.zeros_like(dtype=config.floatX) for i in inputs]
@@ -926,13 +945,19 @@ class Mod(BinaryScalarOp):
             # the reference calls the double overload whatever the input type
             m = lambda a, b: "fmod((double)%s, (double)%s)" % (a, b)
             zero = "%s = %s;" % (z, m(x, y))
-        nx, ny = "(-%s)" % x, "(-%s)" % y
+        integer = t in discrete_dtypes
+        neg = (lambda a: "thx_wneg(%s)" % a) if integer else (lambda a: "(-%s)" % a)
+        plus = (lambda a, b: "thx_wadd(%s, %s)" % (a, b)) if integer else (lambda a, b: "%s + %s" % (a, b))
+        nx, ny = neg(x), neg(y)
+        mm, pm, mp, pp = m(nx, ny), m(x, ny), m(nx, y), m(x, y)
         return ("if (%(y)s == 0) { %(zero)s } "
-                "else if (%(y)s < 0) { if (%(x)s < 0) { %(z)s = -(%(mm)s); } "
-                "else { %(z)s = (%(pm)s) + (%(pm)s != 0 ? %(y)s : 0); } } "
-                "else { if (%(x)s < 0) { %(z)s = -%(mp)s + (%(mp)s != 0 ? %(y)s : 0); } "
+                "else if (%(y)s < 0) { if (%(x)s < 0) { %(z)s = %(a)s; } "
+                "else { %(z)s = %(b)s; } } "
+                "else { if (%(x)s < 0) { %(z)s = %(c)s; } "
                 "else { %(z)s = %(pp)s; } }") % dict(
-                    x=x, y=y, z=z, zero=zero, mm=m(nx, ny), pm=m(x, ny), mp=m(nx, y), pp=m(x, y))
+                    x=x, y=y, z=z, zero=zero, pp=pp, a=neg(mm),
+                    b=plus("(%s)" % pm, "(%s != 0 ? %s : 0)" % (pm, y)),
+                    c=plus(neg(mp), "(%s != 0 ? %s : 0)" % (mp, y)))
 
     def L_op(self, inputs, outputs, gout):
         x, y = inputs
@@ -1090,7 +1115,7 @@ class Abs(UnaryScalarOp):
         if t in complex_dtypes:
             return "%s = thx_cabs(%s);" % (z, x)
         if t in int_dtypes:
-            return "%s = (%s < 0) ? -%s : %s;" % (z, x, x, x)
+            return "%s = thx_wabs(%s);" % (z, x)        # abs of the most negative value wraps to itself
         if t in float_dtypes:
             return "%s = %s(%s);" % (z, _fn("fabs", t), x)
         return "%s = %s;" % (z, x)  # bool and unsigned
@@ -1320,6 +1345,8 @@ round_half_away_from_zero = RoundHalfAwayFromZero(same_out_float_only, name="rou
 
 class Neg(UnaryScalarOp):
     def c_code(self, node, inputs, outputs):
+        if node.outputs[0].type.dtype in int_dtypes:
+            return "%s = thx_wneg(%s);" % (outputs[0], inputs[0])
         return "%s = -%s;" % (outputs[0], inputs[0])
 
     def L_op(self, inputs, outputs, gout):
@@ -1351,6 +1378,8 @@ inv = Inv(upgrade_to_float, name="inv")
 
 class Sqr(UnaryScalarOp):
     def c_code(self, node, inputs, outputs):
+        if node.outputs[0].type.dtype in int_dtypes:
+            return "%s = thx_wmul(%s, %s);" % (outputs[0], inputs[0], inputs[0])
         return "%s = %s * %s;" % (outputs[0], inputs[0], inputs[0])
 
     def L_op(self, inputs, outputs, gout):
