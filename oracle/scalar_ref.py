@@ -202,9 +202,10 @@ def int_div(out_dtype, x, y):
 
 
 def mod(out_dtype, x, y):
-    """theano/scalar/basic.py:2119-2135, element by element: remainder with the divisor's sign."""
+    """theano/scalar/basic.py:2119-2135, element by element: remainder with the divisor's sign.  The floating-point
+    text (fmod over doubles) also serves integer operands whose node type is float64: int64 beside uint64."""
     ct = c_common_type(x.dtype, y.dtype)
-    if np.dtype(ct).kind == "f":
+    if np.dtype(ct).kind == "f" or np.promote_types(np.asarray(x).dtype, np.asarray(y).dtype).kind == "f":
         a, b = np.broadcast_arrays(_conv(x, "float64"), _conv(y, "float64"))
         with np.errstate(all="ignore"):
             r = np.where(b == 0, np.fmod(a, b),
@@ -273,7 +274,7 @@ def mod_fast(out_dtype, x, y):
     """Vectorised ``mod``: the same C expressions over whole arrays (NumPy's fixed-width integers wrap as the
     restatement's do); zero divisors give 0 as on the device."""
     ct = c_common_type(x.dtype, y.dtype)
-    if np.dtype(ct).kind == "f":
+    if np.dtype(ct).kind == "f" or np.promote_types(np.asarray(x).dtype, np.asarray(y).dtype).kind == "f":
         return mod(out_dtype, x, y)
     x, y = np.broadcast_arrays(np.asarray(x), np.asarray(y))
     y1 = np.where(y == 0, np.ones((), y.dtype), y)
@@ -311,6 +312,18 @@ def int_div_fast(out_dtype, x, y):
     x, y = np.broadcast_arrays(np.asarray(x), np.asarray(y))
     y1 = np.where(y == 0, np.ones((), y.dtype), y)
     ny, nx = _cneg(y1), _cneg(x)
+    if np.promote_types(x.dtype, y.dtype).kind == "f":
+        # int64 beside uint64: the node's type is float64, so the reference takes its floating-point text
+        # (theano/scalar/basic.py:1985-2003) over integer operands - x / y is still C's integer division (in
+        # unsigned long long), floor() and fmod() see doubles, and the sign corrections negate the doubles
+        f = lambda v: np.asarray(v).astype("float64")                                      # noqa: E731
+        with np.errstate(all="ignore"):
+            mm = f(_ctrunc_div(nx, ny))
+            pm = -f(_ctrunc_div(x, ny)) - np.where(np.fmod(f(x), f(ny)) == 0, 0.0, 1.0)
+            mp = -f(_ctrunc_div(nx, y1)) - np.where(np.fmod(f(nx), f(y1)) == 0, 0.0, 1.0)
+            pp = f(_ctrunc_div(x, y1))
+        r = np.where(y < 0, np.where(x < 0, mm, pm), np.where(x < 0, mp, pp))
+        return _conv(np.where(y == 0, 0.0, r), out_dtype)
     step = lambda m: np.where(m == 0, np.zeros((), "int32"), np.ones((), "int32"))        # noqa: E731
     with np.errstate(all="ignore"):
         mm = _ctrunc_div(nx, ny)
@@ -327,13 +340,29 @@ def pow_(out_dtype, x, y):
         return _conv(np.power(x.astype("float64"), y.astype("float64")), out_dtype)
 
 
+def _pick(out_dtype, x, y, first):
+    """``y OP x ? y : (x OP= y ? x : nan)`` (theano/scalar/basic.py:1632-1639, 1669-1675): the comparisons are
+    made in C's common type, the operand that wins is stored as itself - so beside a uint64 a negative int8
+    compares as a huge number and is then stored as the negative number it is."""
+    ct = c_common_type(x.dtype, y.dtype)
+    xs, ys = np.broadcast_arrays(np.asarray(x), np.asarray(y))
+    a, b = _conv(xs, ct), _conv(ys, ct)
+    with np.errstate(all="ignore"):
+        take_y = (b > a) if first == "max" else (b < a)
+        take_x = (a >= b) if first == "max" else (a <= b)
+        if np.dtype(out_dtype).kind in "fc":
+            rest = np.where(take_x, _conv(xs, out_dtype), np.asarray(np.nan, out_dtype))
+        else:
+            rest = _conv(xs, out_dtype)       # integers always compare one way or the other
+        return np.where(take_y, _conv(ys, out_dtype), rest).astype(out_dtype)
+
+
 def maximum(out_dtype, x, y):
-    # (y > x ? y : (x >= y ? x : nan)): NaN on either side gives NaN
-    return _arith(np.maximum, out_dtype, x, y)
+    return _pick(out_dtype, x, y, "max")
 
 
 def minimum(out_dtype, x, y):
-    return _arith(np.minimum, out_dtype, x, y)
+    return _pick(out_dtype, x, y, "min")
 
 
 def _cmp(fn):
@@ -534,7 +563,12 @@ def arctan2(out_dtype, y, x):
 
 
 def scalar_sigmoid(out_dtype, x):
-    """theano/tensor/nnet/sigm.py:78-85."""
+    """theano/tensor/nnet/sigm.py:78-85; integer operands have no C code there and go through the Python
+    ``impl`` (:36-46): 0 below -30, 1 above 30, the plain formula in between."""
+    if np.asarray(x).dtype.kind in "biu":
+        xd = np.asarray(x).astype("float64")
+        with np.errstate(all="ignore"):
+            return _conv(np.where(xd < -30.0, 0.0, np.where(xd > 30.0, 1.0, 1.0 / (1.0 + np.exp(-xd)))), out_dtype)
     if str(x.dtype) in ("float32", "float16"):
         xf = x.astype("float32")
         with np.errstate(all="ignore"):
@@ -549,7 +583,12 @@ def scalar_sigmoid(out_dtype, x):
 
 
 def scalar_softplus(out_dtype, x):
-    """theano/tensor/nnet/sigm.py:356-360."""
+    """theano/tensor/nnet/sigm.py:356-360; integer operands through the Python ``impl`` (:336-346): 0 below -30,
+    x above 30, log1p(exp(x)) in between."""
+    if np.asarray(x).dtype.kind in "biu":
+        xd = np.asarray(x).astype("float64")
+        with np.errstate(all="ignore"):
+            return _conv(np.where(xd < -30.0, 0.0, np.where(xd > 30.0, xd, np.log1p(np.exp(xd)))), out_dtype)
     if str(x.dtype) in ("float32", "float16"):
         xf = x.astype("float32")
         with np.errstate(all="ignore"):

@@ -911,3 +911,52 @@ def test_arithmetic_over_every_pair_of_dtypes_against_numpy(left):
                 bar = TOL["float16" if w.dtype == np.float16 else (ct or "float32")]
                 assert_parity(g, w, what, tol=bar)
         k += 4
+
+
+_INT_TYPES = ("bool", "int8", "uint8", "int16", "uint16", "int32", "uint32", "int64", "uint64")
+
+
+def _int_grid(dtype, avoid_min):
+    if dtype == "bool":
+        return np.array([False, True])
+    info = np.iinfo(dtype)
+    vals = {info.min + 1, info.min + 2, info.max, info.max - 1, 0, 1, 2, 3, 5, 7, 100}
+    if info.min < 0:
+        vals |= {-1, -2, -3, -5, -7, -100}
+    if not avoid_min:
+        vals.add(info.min)
+    return np.array(sorted(vals), dtype=dtype)
+
+
+@pytest.mark.parametrize("opname", ["add", "sub", "mul", "maximum", "minimum", "int_div", "mod"])
+def test_binary_integer_ops_over_every_pair_of_integer_types(opname):
+    """Every pair of integer operand types, values at the ends of each range and small ones of either sign:
+    + - * wrap, maximum / minimum compare in C's common type and keep the winner's own value, // and % test each
+    operand's sign in its own type and divide in the common one (the oracle's restatements of these are pinned
+    against gcc).  The most negative int32 / int64 stay out of // and %: their negation is undefined in C."""
+    op = getattr(T, opname)
+    divides = opname in ("int_div", "mod")
+    for tx in _INT_TYPES:
+        for ty in _INT_TYPES:
+            x, y = T.vector("x", dtype=tx), T.vector("y", dtype=ty)
+            try:
+                out = op(x, y)
+            except TypeError:
+                assert opname == "sub" and tx == ty == "bool"
+                continue
+            gx, gy = _int_grid(tx, divides), _int_grid(ty, divides)
+            xv, yv = np.repeat(gx, len(gy)), np.tile(gy, len(gx))
+            if divides:
+                keep = yv != 0
+                xv, yv = xv[keep], yv[keep]
+            with np.errstate(all="ignore"):
+                ref = G.evaluate([x, y], [out], [xv, yv])[0]
+            got = th.function([x, y], out)(xv, yv)
+            assert got.dtype == ref.dtype, (opname, tx, ty)
+            if ref.dtype.kind == "f":
+                ok = (got == ref) | (np.isnan(got) & np.isnan(ref))
+            else:
+                ok = got == ref
+            bad = np.flatnonzero(~ok)
+            assert bad.size == 0, "%s(%s, %s): x=%s y=%s gives %s, the oracle %s" % (
+                opname, tx, ty, xv[bad[0]], yv[bad[0]], got[bad[0]], ref[bad[0]])

@@ -579,3 +579,95 @@ void div_%(tx)s_%(ty)s(const %(cx)s* xs, const %(cy)s* ys, long long* zs, int n)
         assert int(fn_div("int32", lo32, np.asarray([-128], "int8"))[0]) == -16777216
         assert int(fn_div("int64", lo64, np.asarray([-1], "int64"))[0]) == np.iinfo("int64").min
         assert int(fn_mod("int32", np.asarray([1], "int32"), lo32)[0]) == np.iinfo("int32").min + 1
+
+
+def test_maximum_and_minimum_follow_c_typing_with_gcc_as_the_judge(tmp_path):
+    """``z = y > x ? y : (x >= y ? x : nan(""))`` (``theano/scalar/basic.py:1632-1639, 1669-1675``) compiled by gcc
+    for every pair of integer operand types, the result in the type NumPy's promotion gives the node (a double for
+    int64 beside uint64): the comparison happens in C's common type, the winner is stored as the value it is."""
+    import ctypes
+    import subprocess
+    types = list(_C_NAMES)
+    src = ["#include <math.h>"]
+    pairs = []
+    for tx in types:
+        for ty in types:
+            out = str(np.promote_types(tx, ty))
+            co = "double" if out == "float64" else _C_NAMES[out]
+            pairs.append((tx, ty, out))
+            for name, gt, ge in (("max", ">", ">="), ("min", "<", "<=")):
+                tail = 'nan("")'
+                src.append("void %s_%s_%s(const %s* xs, const %s* ys, double* zs, int n) { for (int i = 0; i < n; ++i) { "
+                           "%s x = xs[i]; %s y = ys[i]; %s z = ((y) %s (x) ? (y) : ((x) %s (y) ? (x) : %s)); zs[i] = (double)z; } }"
+                           % (name, tx, ty, _C_NAMES[tx], _C_NAMES[ty], _C_NAMES[tx], _C_NAMES[ty], co, gt, ge, tail))
+    c_file, so_file = tmp_path / "judge.c", tmp_path / "judge.so"
+    c_file.write_text("\n".join(src))
+    subprocess.run(["gcc", "-O2", "-shared", "-fPIC", "-w", str(c_file), "-o", str(so_file), "-lm"], check=True)
+    lib = ctypes.CDLL(str(so_file))
+    checked = 0
+    for tx, ty, out in pairs:
+        gx, gy = _integer_grid(tx), _integer_grid(ty)
+        # the detour through double rounds 64-bit integers beyond 2**53 (and overflows on the way back at the top of
+        # the range): the restatement keeps the operand's own value there, like the reference's Python ``impl``
+        gx, gy = gx[abs(gx.astype("float64")) < 2.0 ** 53], gy[abs(gy.astype("float64")) < 2.0 ** 53]
+        x = np.ascontiguousarray(np.repeat(gx, len(gy)))
+        y = np.ascontiguousarray(np.tile(gy, len(gx)))
+        z = np.zeros(len(x), "float64")
+        for name, fn in (("max", S.maximum), ("min", S.minimum)):
+            getattr(lib, "%s_%s_%s" % (name, tx, ty))(x.ctypes.data_as(ctypes.c_void_p), y.ctypes.data_as(ctypes.c_void_p),
+                                                    z.ctypes.data_as(ctypes.c_void_p), ctypes.c_int(len(x)))
+            got = fn(out, x, y)
+            assert got.dtype == np.dtype(out)
+            # compared as doubles: exact for every integer type but the 64-bit ones, where both sides round alike
+            bad = np.flatnonzero(got.astype("float64") != z)
+            assert bad.size == 0, "%s(%s, %s): x=%s y=%s gives %s, gcc %s" % (
+                name, tx, ty, x[bad[0]], y[bad[0]], got[bad[0]], z[bad[0]])
+            checked += len(x)
+    assert checked > 20000
+    assert float(S.maximum("float64", np.asarray([3], "uint64"), np.asarray([-2], "int8"))[0]) == -2.0
+
+
+def test_floor_division_of_a_signed_by_an_unsigned_64_bit_integer_follows_the_float_text(tmp_path):
+    """A signed integer beside a uint64 makes a float64 node, and the reference then takes its floating-point text
+    (``theano/scalar/basic.py:1985-2003, 2009-2025``) over the integer operands: ``x / y`` stays C's integer
+    division, ``floor`` and ``fmod`` see doubles.  gcc is the judge."""
+    import ctypes
+    import subprocess
+    src = ["#include <math.h>"]
+    pairs = [(a, "uint64") for a in ("int8", "int16", "int32", "int64")] + [("uint64", b) for b in ("int8", "int16", "int32", "int64")]
+    for tx, ty in pairs:
+        src.append("""
+void div_%(tx)s_%(ty)s(const %(cx)s* xs, const %(cy)s* ys, double* zs, int n) {
+  for (int i = 0; i < n; ++i) { %(cx)s x = xs[i]; %(cy)s y = ys[i]; double z;
+    if (y < 0) { if (x < 0) { z = floor((-x) / (-y)); } else { z = -floor(x / (-y)) - ((fmod(x, (-y)) == 0) ? 0 : 1); } }
+    else { if (x < 0) { z = -floor((-x) / y) - ((fmod((-x), y) == 0) ? 0 : 1); } else { z = floor(x / y); } }
+    zs[i] = z; } }
+void mod_%(tx)s_%(ty)s(const %(cx)s* xs, const %(cy)s* ys, double* zs, int n) {
+  for (int i = 0; i < n; ++i) { %(cx)s x = xs[i]; %(cy)s y = ys[i]; double z;
+    if (y < 0) { if (x < 0) { z = -(fmod(-x, -y)); } else { z = (fmod(x, -y)) + (fmod(x, -y) != 0 ? y : 0); } }
+    else { if (x < 0) { z = - fmod(-x, y) + (fmod(-x, y) != 0 ? y : 0); } else { z = fmod(x, y); } }
+    zs[i] = z; } }""" % dict(tx=tx, ty=ty, cx=_C_NAMES[tx], cy=_C_NAMES[ty]))
+    c_file, so_file = tmp_path / "judge.c", tmp_path / "judge.so"
+    c_file.write_text("\n".join(src))
+    subprocess.run(["gcc", "-O2", "-fwrapv", "-shared", "-fPIC", "-w", str(c_file), "-o", str(so_file), "-lm"], check=True)
+    lib = ctypes.CDLL(str(so_file))
+    for tx, ty in pairs:
+        gx, gy = _integer_grid(tx), _integer_grid(ty)
+        x, y = np.repeat(gx, len(gy)), np.tile(gy, len(gx))
+        keep = y != 0
+        for t, v in ((tx, x), (ty, y)):
+            if t in ("int32", "int64"):
+                keep &= v != np.iinfo(t).min               # -x undefined
+        x, y = np.ascontiguousarray(x[keep]), np.ascontiguousarray(y[keep])
+        z = np.zeros(len(x), "float64")
+        getattr(lib, "div_%s_%s" % (tx, ty))(x.ctypes.data_as(ctypes.c_void_p), y.ctypes.data_as(ctypes.c_void_p),
+                                           z.ctypes.data_as(ctypes.c_void_p), ctypes.c_int(len(x)))
+        got = S.int_div_fast("float64", x, y)
+        bad = np.flatnonzero(got != z)
+        assert bad.size == 0, "int_div(%s, %s): x=%s y=%s gives %s, gcc %s" % (tx, ty, x[bad[0]], y[bad[0]], got[bad[0]], z[bad[0]])
+        getattr(lib, "mod_%s_%s" % (tx, ty))(x.ctypes.data_as(ctypes.c_void_p), y.ctypes.data_as(ctypes.c_void_p),
+                                           z.ctypes.data_as(ctypes.c_void_p), ctypes.c_int(len(x)))
+        for fn in (S.mod_fast, S.mod):
+            got = fn("float64", x, y)
+            bad = np.flatnonzero(got != z)
+            assert bad.size == 0, "mod(%s, %s): x=%s y=%s gives %s, gcc %s" % (tx, ty, x[bad[0]], y[bad[0]], got[bad[0]], z[bad[0]])

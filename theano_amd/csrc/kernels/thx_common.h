@@ -135,10 +135,16 @@ __device__ __forceinline__ float thx_sigmoid_core(float x) { return 1.0f / (1.0f
 // x / y in the type C gives the quotient, correctly rounded even when single-precision division
 // is built in its 2.5-ulp form: a double quotient rounded to float is the correctly rounded float
 // quotient (53 >= 2 * 24 + 2 bits).
+// Two integers divide as integers (a signed integer beside a uint64 makes a float64 node whose text still
+// divides its integer operands first).
 template <class A, class B>
 __device__ __forceinline__ auto thx_exact_div(A a, B b) -> decltype(a / b) {
   typedef decltype(a / b) R;
-  return (R)((double)a / (double)b);
+  if constexpr (R(1) / R(2) == R(0)) {
+    return a / b;
+  } else {
+    return (R)((double)a / (double)b);
+  }
 }
 
 // Digamma and trigamma (the reference ships its own C for both, theano/scalar/basic_scipy.py:

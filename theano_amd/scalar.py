@@ -720,9 +720,23 @@ class Maximum(BinaryScalarOp):
         x, y = inputs
         if node.outputs[0].type.dtype in complex_dtypes:
             raise NotImplementedError("maximum / minimum of complex numbers (theano/scalar/basic.py:1635, 1674)")
-        nan = "NAN" if node.outputs[0].type.dtype in float_dtypes else "0"
-        # both comparisons, so that a NaN on either side gives NaN
-        return "%s = ((%s) > (%s) ? (%s) : ((%s) >= (%s) ? (%s) : %s));" % (outputs[0], y, x, y, x, y, x, nan)
+        return self._pick(node, x, y, outputs[0], ">", ">=")
+
+    @staticmethod
+    def _pick(node, x, y, z, first, then):
+        """``z = y OP x ? y : (x OP= y ? x : nan(""))`` (theano/scalar/basic.py:1637-1639): both comparisons, so
+        that a NaN on either side gives NaN, made in C's common type of the operands.  The reference's ``nan("")``
+        makes the whole expression a double, so the operand that wins arrives in ``z`` as the value it is (an int8
+        of -128 beside a uint32 stays -128): each branch is converted to the result type here, which says the
+        same without the detour - and without the rounding to 53 bits that the detour gives 64-bit integers."""
+        out = node.outputs[0].type.dtype
+        if out in float_dtypes:
+            # the NaN in the result's own arithmetic type: a float NAN beside integer operands (int32 beside
+            # uint64 gives a float64 node) would make the expression a float and round the operands to 24 bits
+            nan = "NAN" if all(i.type.dtype in float_dtypes for i in node.inputs) else "((%s)NAN)" % compute_ctype(out)
+            return "%s = ((%s) %s (%s) ? (%s) : ((%s) %s (%s) ? (%s) : %s));" % (z, y, first, x, y, x, then, y, x, nan)
+        ct = storage_ctype(out) if out != "bool" else "bool"
+        return "%s = ((%s) %s (%s) ? (%s)(%s) : (%s)(%s));" % (z, y, first, x, ct, y, ct, x)
 
     def L_op(self, inputs, outputs, gout):
         x, y = inputs
@@ -738,8 +752,7 @@ class Minimum(Maximum):
         x, y = inputs
         if node.outputs[0].type.dtype in complex_dtypes:
             raise NotImplementedError("maximum / minimum of complex numbers (theano/scalar/basic.py:1635, 1674)")
-        nan = "NAN" if node.outputs[0].type.dtype in float_dtypes else "0"
-        return "%s = ((%s) < (%s) ? (%s) : ((%s) <= (%s) ? (%s) : %s));" % (outputs[0], y, x, y, x, y, x, nan)
+        return self._pick(node, x, y, outputs[0], "<", "<=")
 
 
 maximum, minimum = Maximum(upcast_out, name="maximum"), Minimum(upcast_out, name="minimum")
@@ -1417,6 +1430,12 @@ class ScalarSigmoid(UnaryScalarOp):
     def c_code(self, node, inputs, outputs):
         t = node.inputs[0].type.dtype
         (x,), (z,) = inputs, outputs
+        if t in discrete_dtypes:
+            # The reference has C code for floating-point operands only and evaluates integers through its Python
+            # ``impl`` (theano/tensor/nnet/sigm.py:36-46); here they are converted to the result's float type
+            # (int8 -> float32, int32 -> float64: upgrade_to_float) and take that type's formula.
+            t = node.outputs[0].type.dtype
+            x = "((%s)%s)" % (compute_ctype(t), x)
         if t in ("float32", "float16"):
             return "%s = %s < -88.0f ? 0.0f : %s > 15.0f ? 1.0f : thx_sigmoid_core(%s);" % (z, x, x, x)
         if t == "float64":
@@ -1435,6 +1454,9 @@ class ScalarSoftplus(UnaryScalarOp):
     def c_code(self, node, inputs, outputs):
         t = node.inputs[0].type.dtype
         (x,), (z,) = inputs, outputs
+        if t in discrete_dtypes:           # as for the sigmoid: integers take the result type's formula
+            t = node.outputs[0].type.dtype
+            x = "((%s)%s)" % (compute_ctype(t), x)
         if t in ("float32", "float16"):
             return "%s = %s < -103.0f ? 0.0f : %s > 14.0f ? %s : log1pf(expf(%s));" % (z, x, x, x, x)
         if t == "float64":
