@@ -434,9 +434,16 @@ def switch(out_dtype, c, a, b):
 
 
 def clip(out_dtype, x, lo, hi):
-    ct = c_common_type(x.dtype, lo.dtype, hi.dtype)
-    x_, lo_, hi_ = _conv(x, ct), _conv(lo, ct), _conv(hi, ct)
-    return _conv(np.where(x_ < lo_, lo_, np.where(x_ > hi_, hi_, x_)), out_dtype)
+    """``z = x < min ? min : (x > max ? max : x)`` (theano/scalar/basic.py:2240-2243): each comparison in the common
+    type of its own two operands; the inner conditional has the common type of max and x, the outer one that of
+    min and the inner - an int8 -128 beside a uint32 max becomes 4294967168 before an int64 min widens it."""
+    x, lo, hi = np.broadcast_arrays(np.asarray(x), np.asarray(lo), np.asarray(hi))
+    inner_t = c_common_type(hi.dtype, x.dtype)
+    outer_t = c_common_type(lo.dtype, inner_t)
+    with np.errstate(all="ignore"):
+        below, above = _cbin(np.less, x, lo), _cbin(np.greater, x, hi)
+        inner = np.where(above, _conv(hi, inner_t), _conv(x, inner_t))
+    return _conv(np.where(below, _conv(lo, outer_t), _conv(inner, outer_t)), out_dtype)
 
 
 def second(out_dtype, x, y):

@@ -960,3 +960,32 @@ def test_binary_integer_ops_over_every_pair_of_integer_types(opname):
             bad = np.flatnonzero(~ok)
             assert bad.size == 0, "%s(%s, %s): x=%s y=%s gives %s, the oracle %s" % (
                 opname, tx, ty, xv[bad[0]], yv[bad[0]], got[bad[0]], ref[bad[0]])
+
+
+def test_clip_and_switch_over_integer_type_combinations():
+    """``clip`` over a fixed sample of 60 triples of integer types and ``switch`` over every pair, on values at the
+    ends of each range: the conditionals convert as C's do (the oracle's restatements of both are pinned against
+    gcc) - an int8 -128 clipped against a uint32 maximum comes out as 4294967168."""
+    import itertools
+    types = [t for t in _INT_TYPES if t != "bool"]
+    small = lambda t: np.array(sorted({np.iinfo(t).min, np.iinfo(t).min + 1, 0, 1, 3, np.iinfo(t).max} |        # noqa: E731
+                                      ({-1, -3} if np.iinfo(t).min < 0 else set())), dtype=t)
+    rng = np.random.default_rng(8)
+    triples = [tuple(types[i] for i in rng.integers(0, len(types), 3)) for _ in range(60)] + [("int8", "int64", "uint32")]
+    for tx, tl, th_ in triples:
+        x, lo, hi = T.vector("x", dtype=tx), T.vector("lo", dtype=tl), T.vector("hi", dtype=th_)
+        out = T.clip(x, lo, hi)
+        vals = [np.ascontiguousarray(a.reshape(-1)) for a in np.meshgrid(small(tx), small(tl), small(th_), indexing="ij")]
+        with np.errstate(all="ignore"):
+            ref = G.evaluate([x, lo, hi], [out], vals)[0]
+        got = th.function([x, lo, hi], out)(*vals)
+        assert got.dtype == ref.dtype and np.array_equal(got, ref, equal_nan=True), (tx, tl, th_)
+    for ta, tb in itertools.product(types, repeat=2):
+        c, a, b = T.vector("c", dtype="int8"), T.vector("a", dtype=ta), T.vector("b", dtype=tb)
+        out = T.switch(c, a, b)
+        vals = [np.ascontiguousarray(v.reshape(-1)) for v in
+                np.meshgrid(np.array([0, 1, -1], "int8"), small(ta), small(tb), indexing="ij")]
+        with np.errstate(all="ignore"):
+            ref = G.evaluate([c, a, b], [out], vals)[0]
+        got = th.function([c, a, b], out)(*vals)
+        assert got.dtype == ref.dtype and np.array_equal(got, ref, equal_nan=True), (ta, tb)

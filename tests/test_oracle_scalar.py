@@ -671,3 +671,60 @@ void mod_%(tx)s_%(ty)s(const %(cx)s* xs, const %(cy)s* ys, double* zs, int n) {
             got = fn("float64", x, y)
             bad = np.flatnonzero(got != z)
             assert bad.size == 0, "mod(%s, %s): x=%s y=%s gives %s, gcc %s" % (tx, ty, x[bad[0]], y[bad[0]], got[bad[0]], z[bad[0]])
+
+
+def test_clip_and_switch_follow_c_typing_with_gcc_as_the_judge(tmp_path):
+    """``x < min ? min : x > max ? max : x`` (``theano/scalar/basic.py:2240-2243``) and ``cond ? ift : iff``
+    (``:1500-1512``) compiled by gcc for every triple / pair of integer operand types."""
+    import ctypes
+    import itertools
+    import subprocess
+    types = [t for t in _C_NAMES if t != "bool"]
+    small = lambda t: np.array(sorted({np.iinfo(t).min, np.iinfo(t).min + 1, 0, 1, 3, np.iinfo(t).max} |       # noqa: E731
+                                      ({-1, -3} if np.iinfo(t).min < 0 else set())), dtype=t)
+    src = []
+    for tx, tl, th_ in itertools.product(types, repeat=3):
+        out = str(np.result_type(tx, tl, th_))
+        if out.startswith("float"):
+            continue
+        src.append("void clip_%s_%s_%s(const %s* xs, const %s* ls, const %s* hs, long long* zs, int n) { for (int i = 0; i < n; ++i) "
+                   "{ %s x = xs[i]; %s lo = ls[i]; %s hi = hs[i]; %s z = x < lo ? lo : x > hi ? hi : x; zs[i] = (long long)z; } }"
+                   % (tx, tl, th_, _C_NAMES[tx], _C_NAMES[tl], _C_NAMES[th_], _C_NAMES[tx], _C_NAMES[tl], _C_NAMES[th_], _C_NAMES[out]))
+    for ta, tb in itertools.product(types, repeat=2):
+        out = str(np.promote_types(ta, tb))
+        if out.startswith("float"):
+            continue
+        src.append("void switch_%s_%s(const signed char* cs, const %s* as, const %s* bs, long long* zs, int n) { for (int i = 0; i < n; ++i) "
+                   "{ %s a = as[i]; %s b = bs[i]; %s z = cs[i] ? a : b; zs[i] = (long long)z; } }"
+                   % (ta, tb, _C_NAMES[ta], _C_NAMES[tb], _C_NAMES[ta], _C_NAMES[tb], _C_NAMES[out]))
+    c_file, so_file = tmp_path / "judge.c", tmp_path / "judge.so"
+    c_file.write_text("\n".join(src))
+    subprocess.run(["gcc", "-O2", "-shared", "-fPIC", "-w", str(c_file), "-o", str(so_file)], check=True)
+    lib = ctypes.CDLL(str(so_file))
+    ptr = lambda a: a.ctypes.data_as(ctypes.c_void_p)                                                           # noqa: E731
+    checked = 0
+    for tx, tl, th_ in itertools.product(types, repeat=3):
+        out = str(np.result_type(tx, tl, th_))
+        if out.startswith("float"):
+            continue
+        g = np.meshgrid(small(tx), small(tl), small(th_), indexing="ij")
+        x, lo, hi = [np.ascontiguousarray(a.reshape(-1)) for a in g]
+        z = np.zeros(len(x), "int64")
+        getattr(lib, "clip_%s_%s_%s" % (tx, tl, th_))(ptr(x), ptr(lo), ptr(hi), ptr(z), ctypes.c_int(len(x)))
+        got = S.clip(out, x, lo, hi)
+        bad = np.flatnonzero(got != z.astype(out))
+        assert bad.size == 0, "clip(%s, %s, %s): %s %s %s gives %s, gcc %s" % (
+            tx, tl, th_, x[bad[0]], lo[bad[0]], hi[bad[0]], got[bad[0]], z.astype(out)[bad[0]])
+        checked += len(x)
+    for ta, tb in itertools.product(types, repeat=2):
+        out = str(np.promote_types(ta, tb))
+        if out.startswith("float"):
+            continue
+        g = np.meshgrid(np.array([0, 1, -1], "int8"), small(ta), small(tb), indexing="ij")
+        c, a, b = [np.ascontiguousarray(v.reshape(-1)) for v in g]
+        z = np.zeros(len(c), "int64")
+        getattr(lib, "switch_%s_%s" % (ta, tb))(ptr(c), ptr(a), ptr(b), ptr(z), ctypes.c_int(len(c)))
+        got = S.switch(out, c, a, b)
+        assert np.array_equal(got, z.astype(out)), (ta, tb)
+        checked += len(c)
+    assert checked > 90000
