@@ -936,6 +936,7 @@ def test_binary_integer_ops_over_every_pair_of_integer_types(opname):
     against gcc).  The most negative int32 / int64 stay out of // and %: their negation is undefined in C."""
     op = getattr(T, opname)
     divides = opname in ("int_div", "mod")
+    problems = []                       # collected, so that one pair's failure does not hide the others
     for tx in _INT_TYPES:
         for ty in _INT_TYPES:
             x, y = T.vector("x", dtype=tx), T.vector("y", dtype=ty)
@@ -958,8 +959,10 @@ def test_binary_integer_ops_over_every_pair_of_integer_types(opname):
             else:
                 ok = got == ref
             bad = np.flatnonzero(~ok)
-            assert bad.size == 0, "%s(%s, %s): x=%s y=%s gives %s, the oracle %s" % (
-                opname, tx, ty, xv[bad[0]], yv[bad[0]], got[bad[0]], ref[bad[0]])
+            if bad.size:
+                problems.append("%s(%s, %s): x=%s y=%s gives %s, the oracle %s" % (
+                    opname, tx, ty, xv[bad[0]], yv[bad[0]], got[bad[0]], ref[bad[0]]))
+    assert not problems, "\n".join(problems[:10])
 
 
 def test_clip_and_switch_over_integer_type_combinations():
@@ -972,6 +975,7 @@ def test_clip_and_switch_over_integer_type_combinations():
                                       ({-1, -3} if np.iinfo(t).min < 0 else set())), dtype=t)
     rng = np.random.default_rng(8)
     triples = [tuple(types[i] for i in rng.integers(0, len(types), 3)) for _ in range(60)] + [("int8", "int64", "uint32")]
+    problems = []
     for tx, tl, th_ in triples:
         x, lo, hi = T.vector("x", dtype=tx), T.vector("lo", dtype=tl), T.vector("hi", dtype=th_)
         out = T.clip(x, lo, hi)
@@ -979,7 +983,8 @@ def test_clip_and_switch_over_integer_type_combinations():
         with np.errstate(all="ignore"):
             ref = G.evaluate([x, lo, hi], [out], vals)[0]
         got = th.function([x, lo, hi], out)(*vals)
-        assert got.dtype == ref.dtype and np.array_equal(got, ref, equal_nan=True), (tx, tl, th_)
+        if not (got.dtype == ref.dtype and np.array_equal(got, ref, equal_nan=True)):
+            problems.append(("clip", tx, tl, th_))
     for ta, tb in itertools.product(types, repeat=2):
         c, a, b = T.vector("c", dtype="int8"), T.vector("a", dtype=ta), T.vector("b", dtype=tb)
         out = T.switch(c, a, b)
@@ -988,4 +993,6 @@ def test_clip_and_switch_over_integer_type_combinations():
         with np.errstate(all="ignore"):
             ref = G.evaluate([c, a, b], [out], vals)[0]
         got = th.function([c, a, b], out)(*vals)
-        assert got.dtype == ref.dtype and np.array_equal(got, ref, equal_nan=True), (ta, tb)
+        if not (got.dtype == ref.dtype and np.array_equal(got, ref, equal_nan=True)):
+            problems.append(("switch", ta, tb))
+    assert not problems, problems[:10]
