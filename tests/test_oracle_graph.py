@@ -513,3 +513,40 @@ def test_rebroadcast_checks_extents_and_keeps_gradients():
     assert g.type == y.type and np.allclose(G.evaluate([y], [g], [np.ones((1, 4))])[0], 3.0)
     with pytest.raises(ValueError):
         T.addbroadcast(x, 2)
+
+
+def test_forward_and_reverse_mode_agree_on_random_graphs():
+    """<Rop(f, x, v), u> == <Lop(f, x, u), v> for the elementwise / view / sum chains of the random-graph
+    generator, both sides evaluated by the oracle in float64: every op's ``R_op`` against its ``L_op``.  Ops
+    without a forward mode (the maximum / minimum reductions, as in the reference) say so."""
+    import theano_amd as th
+    from theano_amd import gradient as GR
+    import test_gpu_random_graphs as R
+    checked = refused = 0
+    for seed in range(100, 260):
+        ins, outs, vals = R.random_graph(seed)
+        e = outs[0]
+        if not e.type.dtype.startswith("float"):
+            continue
+        fins = [i for i in ins if i.type.dtype.startswith("float")]
+        rng = np.random.default_rng(seed)
+        vs = [T.TensorType(i.type.dtype, i.type.broadcastable)("v%d" % k) for k, i in enumerate(fins)]
+        u = T.TensorType(e.type.dtype, e.type.broadcastable)("u")
+        try:
+            r = GR.Rop(e, fins, vs)
+        except NotImplementedError as err:
+            assert "R_op" in str(err)
+            refused += 1
+            continue
+        ls = GR.Lop(e, fins, u, disconnected_inputs="ignore")
+        lhs = T.sum(r * u, dtype="float64")
+        rhs = sum(T.sum(l * v, dtype="float64") for l, v in zip(ls, vs))
+        vvals = [rng.standard_normal(np.shape(vals[ins.index(i)])).astype(i.type.dtype) for i in fins]
+        with np.errstate(all="ignore"):
+            e_val = G.evaluate(ins, [e], vals)[0]
+            uval = rng.standard_normal(e_val.shape).astype(e.type.dtype)
+            a, b = G.evaluate(ins + vs + [u], [lhs, rhs], vals + vvals + [uval], wide=True)
+        if np.isfinite(a) and np.isfinite(b):
+            assert abs(a - b) <= 1e-8 * (abs(a) + abs(b)) + 1e-9, (seed, float(a), float(b))
+            checked += 1
+    assert checked >= 40 and refused >= 1, (checked, refused)

@@ -214,6 +214,11 @@ class Op(object):
     def grad(self, inputs, output_grads):
         raise MethodNotDefined("grad", type(self))
 
+    def R_op(self, inputs, eval_points):
+        """Forward-mode derivative: the op's Jacobian times ``eval_points``, one variable (or None) per output
+        (``theano/gof/op.py:PureOp.R_op``); an op that has none says so."""
+        raise MethodNotDefined("R_op", type(self))
+
     def connection_pattern(self, node):
         return [[True] * len(node.outputs) for _ in node.inputs]
 

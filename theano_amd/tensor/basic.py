@@ -168,6 +168,9 @@ class ShapeFloat(Op):
     def grad(self, inp, grads):
         return [scal.DisconnectedType()()]
 
+    def R_op(self, inputs, eval_points):
+        return [None]           # an extent does not move with the values (``Shape.R_op``, theano/compile/ops.py:279-280)
+
 
 # --------------------------------------------------------------------------
 def _axis_list(axis, ndim):
