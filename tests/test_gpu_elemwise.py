@@ -996,3 +996,32 @@ def test_clip_and_switch_over_integer_type_combinations():
         if not (got.dtype == ref.dtype and np.array_equal(got, ref, equal_nan=True)):
             problems.append(("switch", ta, tb))
     assert not problems, problems[:10]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape,perm", [((257, 129), (1, 0)), ((33, 65, 17), (2, 1, 0)), ((33, 65, 17), (1, 2, 0)),
+                                        ((9, 1, 31, 7), (3, 2, 1, 0)), ((5, 6, 7, 8, 3), (4, 2, 0, 3, 1))])
+def test_transposed_operands_and_results_walk_memory_in_order(shape, perm):
+    """Operands that are all transposed the same way give a result laid out like them only in the column-major
+    case (theano/tensor/elemwise.py:928-937); whatever the layout, the kernel walks the dimensions in the order
+    of the result's strides and the values are those of the reference."""
+    from theano_amd.hip import HipArray
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal(shape).astype("float32")
+    b = rng.standard_normal(shape).astype("float32")
+    tt = T.TensorType("float32", (False,) * len(shape))
+    x, y = tt("x"), tt("y")
+    out = T.exp(x) * y + x
+    ref = G.evaluate([x, y], [out], [a.transpose(perm), b.transpose(perm)])[0]
+    xt, yt = tt("xt"), tt("yt")
+    g = th.function([xt, yt], T.exp(xt.dimshuffle(*perm)) * yt.dimshuffle(*perm) + xt.dimshuffle(*perm))
+    assert_parity(g(a, b), ref, "transposed inside the graph %s %s [%s]" % (shape, perm, hip.last_plan()))
+    h = th.function([x, y], [th.Out(out, device=True)])
+    da, db = HipArray.from_numpy(a), HipArray.from_numpy(b)
+    got = h(da.transpose(*perm), db.transpose(*perm))[0]
+    assert_parity(got.to_numpy(), ref, "transposed device views %s %s [%s]" % (shape, perm, hip.last_plan()))
+    # one operand transposed, the other not: the result is row-major and still right
+    c = rng.standard_normal(tuple(shape[p] for p in perm)).astype("float32")
+    k = th.function([xt, y], T.exp(xt.dimshuffle(*perm)) * y + y)
+    assert_parity(k(a, c), G.evaluate([x, y], [T.exp(x) * y + y], [a.transpose(perm), c])[0],
+                  "mixed layouts %s %s [%s]" % (shape, perm, hip.last_plan()))

@@ -733,3 +733,26 @@ def test_custom_accumulator_dtype_of_every_real_pair(method):
             else:
                 with pytest.raises(TypeError):
                     getattr(x, method)(acc_dtype=acc_dtype, axis=axis)
+
+
+@pytest.mark.parametrize("shape,axis,form", [
+    ((4096, 4, 4, 4), 1, "rg"), ((4096, 4, 4, 4), 2, "rg"), ((4096, 2, 8), 1, "rg"),   # few columns and few rows
+    ((3, 40001), 0, "rg"), ((2, 40001), 0, "rg"), ((4, 40001), 0, "rg"),               # rows of an odd length
+    ((64, 3, 4097), 1, "rg"),
+    ((4, 40000), 0, "rc"), ((3, 40000), 0, "rc"), ((16, 40001), 0, "rc"),              # vectors, or enough rows
+    ((4096, 4, 64), 1, "rc")])
+def test_column_reductions_with_few_rows_choose_between_two_forms(shape, axis, form):
+    """A sum over an axis that is not the last one runs column-wise (`rc`) unless nearly all of that kernel's
+    lanes would idle or its reads could not be vectors: then one thread computes one result (`rg`).  Both give
+    the reference's values (theano/tensor/elemwise.py:1307 CAReduce.perform)."""
+    rng = np.random.default_rng(77)
+    x = T.TensorType("float32", (False,) * len(shape))("x")
+    v = rng.standard_normal(shape).astype("float32")
+    for name in ("sum", "max"):
+        out = REDUCERS[name](x, axis)
+        got = th.function([x], out)(v)
+        assert "|%s|" % form in hip.last_plan(), (shape, axis, hip.last_plan())
+        assert_parity(got, G.evaluate([x], [out], [v])[0], "%s %s axis %d [%s]" % (name, shape, axis, hip.last_plan()))
+    xi = T.TensorType("int64", (False,) * len(shape))("xi")
+    vi = rng.integers(-2 ** 62, 2 ** 62, shape)
+    check(xi, xi.sum(axis=axis), vi, "int64 sum %s axis %d" % (shape, axis))

@@ -2,6 +2,7 @@
 // access plan (rank, index width, vector width, per-operand access mode),
 // compiles the matching kernel on first use and launches it.
 #include <algorithm>
+#include <cstdint>
 #include <cstdlib>
 #include <cstring>
 #include <sstream>
@@ -160,6 +161,29 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
     dm.nd = 1;
     dm.shape[0] = 1;
     for (int o = 0; o < nops; ++o) dm.stride[o][0] = 0;
+  }
+  // Dimensions in the order of the first result's strides, largest first: operands that share a permuted layout
+  // (every one of them a transposed view, the result allocated to match) then collapse and vectorise like
+  // C-contiguous ones instead of walking memory with the longest stride innermost.  A C-ordered result keeps its
+  // order; the variant that reduces while it stores relies on that order and is left alone.
+  if (dm.nd > 1 && !(red_outs && e->red)) {
+    const std::vector<int64_t>& os = dm.stride[e->n_in];
+    std::vector<int> order(dm.nd);
+    for (int d = 0; d < dm.nd; ++d) order[d] = d;
+    // (extent-1 dimensions, whose strides mean nothing, go first: the collapse drops them)
+    auto mag = [&](int d) { return dm.shape[d] == 1 ? INT64_MAX : (os[d] < 0 ? -os[d] : os[d]); };
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return mag(a) > mag(b); });
+    bool moved = false;
+    for (int d = 0; d < dm.nd; ++d) moved = moved || order[d] != d;
+    if (moved) {
+      int64_t shp[THX_MAX_ND];
+      for (int d = 0; d < dm.nd; ++d) shp[d] = dm.shape[order[d]];
+      for (int d = 0; d < dm.nd; ++d) dm.shape[d] = shp[d];
+      for (int o = 0; o < nops; ++o) {
+        std::vector<int64_t> st(dm.stride[o]);
+        for (int d = 0; d < dm.nd; ++d) dm.stride[o][d] = st[order[d]];
+      }
+    }
   }
   collapse(&dm);
   const int ND = dm.nd;
