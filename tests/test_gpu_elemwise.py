@@ -1025,3 +1025,44 @@ def test_transposed_operands_and_results_walk_memory_in_order(shape, perm):
     k = th.function([xt, y], T.exp(xt.dimshuffle(*perm)) * y + y)
     assert_parity(k(a, c), G.evaluate([x, y], [T.exp(x) * y + y], [a.transpose(perm), c])[0],
                   "mixed layouts %s %s [%s]" % (shape, perm, hip.last_plan()))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["int8", "float16", "float32", "float64"])
+def test_operands_that_start_off_a_vector_boundary(dtype):
+    """Views that drop leading elements or columns keep full-width accesses through element-aligned pointers
+    (plans marked `|ua`): every alignment of two inputs and of the result written in place, odd lengths, rows of a
+    matrix whose pitch is odd.  Values are those of Elemwise.perform (theano/tensor/elemwise.py:790)."""
+    from theano_amd.hip import HipArray
+    rng = np.random.default_rng(44)
+    kind = np.dtype(dtype).kind
+    draw = (lambda shape: rng.integers(-50, 50, shape).astype(dtype)) if kind == "i" else \
+           (lambda shape: (rng.integers(-64, 65, shape) / 16.0).astype(dtype))
+    tol = {"float16": {"rtol": 2e-3, "atol": 2e-3}}.get(dtype)
+    vec, mat = T.TensorType(dtype, (False,)), T.TensorType(dtype, (False, False))
+    x, y, m, w = vec("x"), vec("y"), mat("m"), mat("w")
+    out = x * 2 + y
+    f = th.function([x, y], [th.Out(out, device=True)])
+    a, b = draw(50100), draw(50100)
+    da, db = HipArray.from_numpy(a), HipArray.from_numpy(b)
+    size = a.itemsize
+    marked = 0
+    for lo_a in (0, 1, 2, 3, 5, 8, 15):
+        for lo_b in (0, 1, 7):
+            for n in (50000, 49999, 40003):
+                va = da.view([n], [size], da.offset + lo_a * size)
+                vb = db.view([n], [size], db.offset + lo_b * size)
+                got = f(va, vb)[0].to_numpy()
+                marked += "|ua|" in hip.last_plan()
+                ref = G.evaluate([x, y], [out], [a[lo_a:lo_a + n], b[lo_b:lo_b + n]])[0]
+                assert_parity(got, ref, "[%d:], [%d:] of %d %s [%s]" % (lo_a, lo_b, n, dtype, hip.last_plan()), tol=tol)
+    assert marked >= 40, marked
+    # through the graph: shifted views of one array, and the same with the result written over an operand
+    g = th.function([x], x[1:] - x[:-1])
+    assert_parity(g(a), G.evaluate([x], [x[1:] - x[:-1]], [a])[0], "difference of neighbours %s [%s]" % (dtype, hip.last_plan()), tol=tol)
+    # matrices: columns dropped on the left, a pitch that is odd
+    big, other = draw((300, 1031)), draw((300, 1024))
+    out2 = m[:, 7:] + w
+    got = th.function([m, w], out2)(big, other)
+    assert "|ua|" in hip.last_plan(), hip.last_plan()
+    assert_parity(got, G.evaluate([m, w], [out2], [big, other])[0], "columns dropped %s [%s]" % (dtype, hip.last_plan()), tol=tol)

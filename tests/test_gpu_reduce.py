@@ -736,15 +736,16 @@ def test_custom_accumulator_dtype_of_every_real_pair(method):
 
 
 @pytest.mark.parametrize("shape,axis,form", [
-    ((4096, 4, 4, 4), 1, "rg"), ((4096, 4, 4, 4), 2, "rg"), ((4096, 2, 8), 1, "rg"),   # few columns and few rows
-    ((3, 40001), 0, "rg"), ((2, 40001), 0, "rg"), ((4, 40001), 0, "rg"),               # rows of an odd length
-    ((64, 3, 4097), 1, "rg"),
-    ((4, 40000), 0, "rc"), ((3, 40000), 0, "rc"), ((16, 40001), 0, "rc"),              # vectors, or enough rows
+    ((4096, 4, 4, 4), 1, "rg"), ((4096, 2, 8), 1, "rg"), ((4096, 4, 4, 4), 2, "rg"),   # few columns and few rows
+    ((3, 40001), 0, "rc"), ((2, 40001), 0, "rc"), ((64, 3, 4097), 1, "rc"),            # odd rows: element-aligned vectors
+    ((3, 13), 0, "rg"), ((64, 3, 7), 1, "rg"),                                         # too few columns for those
+    ((4, 40000), 0, "rc"), ((3, 40000), 0, "rc"), ((16, 40001), 0, "rc"),
     ((4096, 4, 64), 1, "rc")])
 def test_column_reductions_with_few_rows_choose_between_two_forms(shape, axis, form):
     """A sum over an axis that is not the last one runs column-wise (`rc`) unless nearly all of that kernel's
-    lanes would idle or its reads could not be vectors: then one thread computes one result (`rg`).  Both give
-    the reference's values (theano/tensor/elemwise.py:1307 CAReduce.perform)."""
+    lanes would idle, or there are two to four rows of too few columns to read as vectors: then one thread
+    computes one result (`rg`).  Both give the reference's values (theano/tensor/elemwise.py:1307
+    CAReduce.perform)."""
     rng = np.random.default_rng(77)
     x = T.TensorType("float32", (False,) * len(shape))("x")
     v = rng.standard_normal(shape).astype("float32")
@@ -756,3 +757,73 @@ def test_column_reductions_with_few_rows_choose_between_two_forms(shape, axis, f
     xi = T.TensorType("int64", (False,) * len(shape))("xi")
     vi = rng.integers(-2 ** 62, 2 ** 62, shape)
     check(xi, xi.sum(axis=axis), vi, "int64 sum %s axis %d" % (shape, axis))
+
+
+@pytest.mark.parametrize("dtype", ["int8", "float16", "float32", "float64", "int16"])
+def test_rows_and_columns_that_are_no_whole_number_of_vectors(dtype):
+    """Long rows whose length is odd or that start off a 16-byte boundary, and columns whose number is odd, are
+    read as full-width vectors through element-aligned pointers (plans marked `|ua`), the incomplete vector at the
+    end element by element: every element is counted once whatever the alignment, for one operand and for several
+    that are out of line by different amounts.  Values are those of CAReduce.perform
+    (theano/tensor/elemwise.py:1307)."""
+    from theano_amd.hip import HipArray
+    rng = np.random.default_rng(31)
+    kind = np.dtype(dtype).kind
+
+    def draw(shape):
+        # floats on a grid of eighths: sums and products of two are exact, so the order of the additions and the
+        # precision a product is kept in between (float32 inside a fused float16 kernel) do not show
+        return (rng.integers(-100, 100, shape).astype(dtype) if kind == "i" else
+                (rng.integers(-8, 9, shape) / 8.0).astype(dtype))
+    tol = {"float16": {"rtol": 2e-3, "atol": 2e-3}}.get(dtype)
+    vec, mat, cube = (T.TensorType(dtype, (False,) * k) for k in (1, 2, 3))
+    x, y, m, w, c = vec("x"), vec("y"), mat("m"), mat("w"), cube("c")
+    marked = 0
+    for n in (1000003, 4099, 257, 31):                  # the last two: too short to bother / to vectorise
+        v = draw(n)
+        for name in ("sum", "max"):
+            out = REDUCERS[name](x, None)
+            got = th.function([x], out)(v)
+            marked += "|ua|" in hip.last_plan()
+            assert_parity(got, G.evaluate([x], [out], [v])[0], "%s of %d %s [%s]" % (name, n, dtype, hip.last_plan()), tol=tol)
+    # every alignment of the first element and of the last
+    base = draw(70000)
+    dev = HipArray.from_numpy(base)
+    f = th.function([x], [th.Out(T.sum(x), device=True), th.Out(T.min(x), device=True)])
+    for lo in range(0, 17):
+        for hi in (70000, 69999, 69993):
+            got = f(dev.view([hi - lo], [base.itemsize], dev.offset + lo * base.itemsize))
+            ref = G.evaluate([x], [T.sum(x), T.min(x)], [base[lo:hi]])
+            for g, r in zip(got, ref):
+                assert_parity(g.to_numpy(), r, "view [%d:%d] %s [%s]" % (lo, hi, dtype, hip.last_plan()), tol=tol)
+    # rows of a matrix: each row starts somewhere else
+    for shape in ((37, 4099), (5, 100001), (300, 515)):
+        a, b = draw(shape), draw(shape)
+        out = T.sum(m * w, axis=1)
+        got = th.function([m, w], out)(a, b)
+        marked += "|ua|" in hip.last_plan()
+        assert_parity(got, G.evaluate([m, w], [out], [a, b])[0], "rows %s %s [%s]" % (shape, dtype, hip.last_plan()), tol=tol)
+        # a stepped operand beside a contiguous one, and the rows in reverse order
+        wide = draw((shape[0], 2 * shape[1]))
+        out2 = T.max(m[::-1] + w[:, ::2], axis=1)
+        got = th.function([m, w], out2)(a, wide)
+        assert_parity(got, G.evaluate([m, w], [out2], [a, wide])[0], "stepped %s %s [%s]" % (shape, dtype, hip.last_plan()), tol=tol)
+    # two operands out of line by different amounts
+    a, b = draw(50001), draw(50002)
+    out = T.sum(x * y[1:])
+    got = th.function([x, y], out)(a, b)
+    assert_parity(got, G.evaluate([x, y], [out], [a, b])[0], "different alignment %s [%s]" % (dtype, hip.last_plan()), tol=tol)
+    # columns: an odd number of them, one and two reduced axes, a view that drops the first column
+    for shape, axis in (((301, 4099), 0), ((7, 13, 1001), (0, 1)), ((5, 33, 515), 1), ((64, 3, 67), 1), ((2, 100003), 0)):
+        a = draw(shape)
+        var = mat("a") if len(shape) == 2 else cube("a")
+        for name in ("sum", "min"):
+            out = REDUCERS[name](var, axis)
+            got = th.function([var], out)(a)
+            marked += "|ua|" in hip.last_plan()
+            assert_parity(got, G.evaluate([var], [out], [a])[0], "columns %s %s %s %s [%s]" % (name, shape, axis, dtype, hip.last_plan()), tol=tol)
+        if len(shape) == 2:
+            out = T.sum(var[:, 1:] * var[:, :-1], axis=0)
+            got = th.function([var], out)(a)
+            assert_parity(got, G.evaluate([var], [out], [a])[0], "shifted columns %s %s [%s]" % (shape, dtype, hip.last_plan()), tol=tol)
+    assert marked >= (6 if np.dtype(dtype).itemsize < 8 else 4), marked

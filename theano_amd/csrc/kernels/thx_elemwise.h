@@ -48,7 +48,7 @@ struct EwAcc {
     if (N == 1) {
       r.v[0] = *b;
     } else if (P::mode(I) == M_VEC) {
-      load_vec<T, N, ((P::NT >> I) & 1) != 0>(r, b);
+      load_vec<T, N, ((P::NT >> I) & 1) != 0, P::UA != 0>(r, b);
     } else if (P::mode(I) == M_BCAST) {
       const T s = *b;
 #pragma unroll
@@ -66,7 +66,7 @@ struct EwAcc {
     if (N == 1) {
       *b = r.v[0];
     } else if (P::mode(I) == M_VEC) {
-      store_vec<T, N, ((P::NT >> I) & 1) != 0>(b, r);
+      store_vec<T, N, ((P::NT >> I) & 1) != 0, P::UA != 0>(b, r);
     } else {
       const IT st = stride[I][P::ND - 1];
 #pragma unroll

@@ -69,6 +69,7 @@ struct RowParams {
   long long nblocks;      // blocks of work; more than the grid holds when the plan strides (GS)
   long long nvec;         // vectors in one output's reduce domain (RA * RC / VEC)
   long long chunk;        // vectors per slice
+  long long rc_elems;     // elements of one row (UA)
   int S;                  // slices per output
   int pad;
   FastDiv kfd[NK];        // extents of the kept dimensions (slot 0 unused)
@@ -104,7 +105,7 @@ struct RedAcc {
     if (N == 1) {
       r.v[0] = *b;
     } else if (P::mode(I) == M_VEC) {
-      load_vec<T, N, ((P::NT >> I) & 1) != 0>(r, b);
+      load_vec<T, N, ((P::NT >> I) & 1) != 0, P::UA != 0>(r, b);
     } else if (P::mode(I) == M_BCAST) {
       const T s = *b;
 #pragma unroll
@@ -117,7 +118,9 @@ struct RedAcc {
   }
 };
 
-// Plan members: typedef IT; enum { NK, VEC, UNR, NACC, BLOCK, TPR, RA2 (1 when RA > 1), TICKET, GS, XCD };
+// Plan members: typedef IT; enum { NK, VEC, UNR, NACC, BLOCK, TPR, RA2 (1 when RA > 1), TICKET, GS, XCD, UA };
+// UA: rows whose length is no multiple of VEC, or that do not start on a vector boundary: vectors are read through
+// pointers that are only element-aligned, and the RC mod VEC elements at the end of a row one by one.
 // static constexpr int mode(int input); static constexpr int sclass(int input, int which).
 template <class P, class IT>
 THX_DEV IT red_term(int input, int which, IT coord, IT stride) {
@@ -182,7 +185,24 @@ __device__ __forceinline__ void red_row_block(const RowParams<R::NIN, R::NOUT, R
   if (live) {
     const long long j0 = (long long)s * p.chunk;
     long long j1 = j0 + p.chunk;
-    if (j1 > p.nvec) j1 = p.nvec;
+    long long nvec = p.nvec;
+    if constexpr (P::UA != 0 && P::RA2 == 0) {
+      const long long tail0 = nvec * VEC;          // first element of the tail
+      if (s == 0) {
+        for (long long idx = tail0 + t; idx < p.rc_elems; idx += TPR) {
+          typename R::template Regs<1> r1;
+          RedAcc<P, NIN> a;
+          a.ptr = p.in;
+          a.imm = p.imm;
+          a.vstride = p.rc_stride;
+#pragma unroll
+          for (int i = 0; i < NIN; ++i) a.off[i] = base[i] + red_term<P>(i, 1, (IT)idx, p.rc_stride[i]);
+          R::template load<1>(a, r1);
+          R::template accum<1>(acc[0], r1);
+        }
+      }
+    }
+    if (j1 > nvec) j1 = nvec;
     // RA > 1: a thread's vectors are TPR apart, so their (slab, position in the slab) coordinates and every
     // operand's offset advance by the same amounts from one vector to the next - additions and one compare
     // instead of a division and two or three quarter-rate multiplies per vector
@@ -284,7 +304,9 @@ struct ColParams {
 };
 
 // Plan members: typedef IT; enum { NK, VEC, UNR, BLOCK, TX, RR2 (1 when two
-// reduced dimensions remain after collapsing), TICKET, GS }; mode(int).
+// reduced dimensions remain after collapsing), TICKET, GS, UA }; mode(int).
+// UA: C is no multiple of VEC, or rows do not start on vector boundaries: element-aligned vector reads, and the
+// thread that owns the last, incomplete vector of the columns reads its columns one by one.
 template <class R, class P>
 __device__ __forceinline__ void red_col_block(const ColParams<R::NIN, R::NOUT, R::NEX, P::NK, typename P::IT>& p, long long bid);
 
@@ -316,12 +338,15 @@ __device__ __forceinline__ void red_col_block(const ColParams<R::NIN, R::NOUT, R
   const int tx = threadIdx.x % TX, ty = threadIdx.x / TX;
   const int cv = cb * TX + tx;                 // column vector owned by this thread
   const bool live = (long long)cv * VEC < p.cols;
+  // UA: the last vector of a row that is no whole number of vectors ends with the row and overlaps its
+  // neighbour; the columns it repeats are dropped when the results are written
+  const int c0 = P::UA != 0 && live && cv * VEC + VEC > p.cols && p.cols >= VEC ? p.cols - VEC : cv * VEC;
 
   IT base[NIN];
   {
     UT rem = (UT)a_idx, c;
 #pragma unroll
-    for (int i = 0; i < NIN; ++i) base[i] = (IT)(live ? cv * VEC : 0) * p.c_stride[i];
+    for (int i = 0; i < NIN; ++i) base[i] = (IT)(live ? c0 : 0) * p.c_stride[i];
 #pragma unroll
     for (int d = NK - 1; d >= 1; --d) {
       divmod(rem, p.kfd[d], rem, c);
@@ -374,9 +399,14 @@ __device__ __forceinline__ void red_col_block(const ColParams<R::NIN, R::NOUT, R
   __syncthreads();
   Acc* part = (Acc*)p.partial;
   for (int c = threadIdx.x; c < TX * VEC; c += P::BLOCK) {
-    const int x = c / VEC, k = c % VEC;
+    const int x = c / VEC;
+    int k = c % VEC;
     const long long col = (long long)cb * (TX * VEC) + c;
     if (col < p.cols) {
+      if constexpr (P::UA != 0) {
+        const long long first = col - k;                   // first column of this vector, had it not been moved
+        if (first + VEC > p.cols) k = (int)(col - (p.cols - VEC));
+      }
       Acc tot = lds[0][k][x];
 #pragma unroll
       for (int y = 1; y < TY; ++y) R::comb(tot, lds[y][k][x]);

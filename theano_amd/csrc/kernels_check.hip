@@ -57,23 +57,23 @@ struct CheckFR : CheckF {
   }
 };
 
-struct PlanEw1 { typedef int IT; enum { ND = 1, VEC = 4, UNR = 2, BLOCK = 256, GS = 1 }; static constexpr unsigned long long NT = 1ull;
+struct PlanEw1 { typedef int IT; enum { ND = 1, VEC = 4, UNR = 2, BLOCK = 256, GS = 1, UA = 1 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {0, 3, 0}; return m[i]; }
   static constexpr int sclass(int i, int d) { constexpr int m[][1] = {{1}, {0}, {1}}; return m[i][d]; }
   static constexpr int alias(int i) { constexpr int m[] = {0, 1, 0}; return m[i]; } };
-struct PlanEw3 { typedef long long IT; enum { ND = 3, VEC = 2, UNR = 1, BLOCK = 256, GS = 0 }; static constexpr unsigned long long NT = 1ull;
+struct PlanEw3 { typedef long long IT; enum { ND = 3, VEC = 2, UNR = 1, BLOCK = 256, GS = 0, UA = 0 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {2, 1, 0}; return m[i]; }
   static constexpr int sclass(int i, int d) { constexpr int m[][3] = {{2, 2, 2}, {0, 1, 0}, {2, 2, 1}}; return m[i][d]; }
   static constexpr int alias(int i) { constexpr int m[] = {0, 1, 2}; return m[i]; } };
-struct PlanRow { typedef int IT; enum { NK = 2, VEC = 4, UNR = 4, NACC = 2, BLOCK = 256, TPR = 256, RA2 = 1, TICKET = 0, GS = 1, XCD = 0 }; static constexpr unsigned long long NT = 0ull;
+struct PlanRow { typedef int IT; enum { NK = 2, VEC = 4, UNR = 4, NACC = 2, BLOCK = 256, TPR = 256, RA2 = 1, TICKET = 0, GS = 1, XCD = 0, UA = 0 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {0}; return m[i]; }
   static constexpr int sclass(int i, int w) { constexpr int m[][2] = {{2, 1}}; return m[i][w]; } };
-struct PlanRowS { typedef int IT; enum { NK = 1, VEC = 1, UNR = 1, NACC = 1, BLOCK = 256, TPR = 16, RA2 = 0, TICKET = 0, GS = 0, XCD = 1 }; static constexpr unsigned long long NT = 1ull;
+struct PlanRowS { typedef int IT; enum { NK = 1, VEC = 1, UNR = 1, NACC = 1, BLOCK = 256, TPR = 16, RA2 = 0, TICKET = 0, GS = 0, XCD = 1, UA = 1 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; }
   static constexpr int sclass(int i, int w) { constexpr int m[][2] = {{0, 2}}; return m[i][w]; } };
-struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, TX = 64, RR2 = 1, TICKET = 0, GS = 1 }; static constexpr unsigned long long NT = 1ull;
+struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, TX = 64, RR2 = 1, TICKET = 0, GS = 1, UA = 1 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {0}; return m[i]; } };
-struct PlanGen { typedef int IT; enum { NK = 3, NR = 3, BLOCK = 256, TPR = 64, GS = 1 }; static constexpr unsigned long long NT = 0ull;
+struct PlanGen { typedef int IT; enum { NK = 3, NR = 3, BLOCK = 256, TPR = 64, GS = 1, UA = 0 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; } };
 
 struct PlanTr { typedef int IT; enum { ND = 3, TT = 64, TI = 32, TV = 4, BLOCK = 256, NTR = 1, ESZ = 2, RED = 0, NBUF = 2, PERSIST = 1 }; static constexpr unsigned long long NT = 0ull;

@@ -227,7 +227,25 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
     }
     return true;
   };
+  const int vec_full = vec;
   while (!vec_ok(vec)) vec /= 2;
+  // Operands that start off a vector boundary, or whose rows do (views that drop a first element or column; float16
+  // and int8 suffer most from narrow accesses): full-width vectors through element-aligned pointers.
+  int ua = 0;
+  if (vec < vec_full && env_int("THX_EW_UA", 1)) {
+    auto ua_ok = [&](int v) {
+      if (ND > 1 && (inner % v != 0 || inner / v < 2)) return false;
+      for (int o = 0; o < nops; ++o)
+        if (mode[o] == M_VEC && ((uintptr_t)views[o].ptr) % (size_t)dtype_size(views[o].dtype)) return false;
+      return true;
+    };
+    int v = vec_full;
+    while (v > vec && !ua_ok(v)) v /= 2;
+    if (v > vec) {
+      vec = v;
+      ua = 1;
+    }
+  }
 
   // bytes the kernel moves: every operand that is not broadcast along the innermost dimension
   int64_t moved = 0;
@@ -489,7 +507,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
   std::ostringstream key;
   key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|s" << skey;
   if (nt) key << "|nt" << std::hex << nt << std::dec;
-  key << (block != 256 ? "|b" + std::to_string(block) : "") << (gs ? "|gs" : "") << "|m";
+  key << (block != 256 ? "|b" + std::to_string(block) : "") << (gs ? "|gs" : "") << (ua ? "|ua" : "") << "|m";
   for (int o = 0; o < nops; ++o) key << mode[o] << (o + 1 < nops ? "," : "");
   const std::string plan = key.str() + (fast_div() ? "|fd" : "");
   set_last_plan(e->name + "|" + plan);
@@ -503,7 +521,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
     std::ostringstream s;
     s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
       << " IT;\n  enum { ND = " << ND << ", VEC = " << vec << ", UNR = " << unr << ", BLOCK = " << block
-      << ", GS = " << (gs ? 1 : 0) << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+      << ", GS = " << (gs ? 1 : 0) << ", UA = " << ua << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
     for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
     s << "};\n    return m[i];\n  }\n  static constexpr int sclass(int i, int d) {\n    constexpr int m[][" << ND << "] = {";
     for (int o = 0; o < nops; ++o) {

@@ -369,7 +369,12 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       for (size_t d = 0; d + 1 < KD.size(); ++d)
         if (KD[d].stride[i] % 2) vectors = false;
     }
-    if (!vectors) form = GEN;
+    // ... unless the column form can read them as element-aligned vectors
+    int maxsz = 0;
+    for (int i = 0; i < NIN; ++i)
+      if (!views[i].iota && !views[i].imm && KD.back().stride[i] == 1) maxsz = std::max(maxsz, dtype_size(views[i].dtype));
+    const bool unaligned_vectors = env_int("THX_RED_UA", 1) && maxsz && KD.back().extent >= (int64_t)(16 / maxsz) * env_int("THX_RED_UA_MINVEC", 4);
+    if (!vectors && !unaligned_vectors) form = GEN;
   }
   const char* force = getenv("THX_RED_FORM");
   if (force && NR <= 2 && NR > 0) {
@@ -426,7 +431,21 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       }
       return true;
     };
+    const int vec_full = vec;
     while (!vec_ok(vec)) vec /= 2;
+    // Rows that are long but of a length that is no multiple of the vector width, or that do not start on a vector
+    // boundary (a sum of all 134 217 727 float16 elements of an array read 2 bytes per lane: 1.8 TB/s; int8: 0.75):
+    // full-width vectors through element-aligned pointers, and the last RC mod vec elements of a row one by one.
+    int ua = 0;
+    if (vec < vec_full && !ra2 && NR == 1 && RC >= (int64_t)vec_full * 16 && env_int("THX_RED_UA", 1)) {
+      bool ok = true;
+      for (int i = 0; i < NIN; ++i)
+        if (mode[i] == M_VEC && ((uintptr_t)views[i].ptr) % (size_t)dtype_size(views[i].dtype)) ok = false;
+      if (ok) {
+        vec = vec_full;
+        ua = 1;
+      }
+    }
     const int64_t nvec = RA * RC / vec;
     int tpr = nvec >= 512 ? 256 : nvec >= 64 ? 64 : nvec >= 16 ? 16 : nvec >= 4 ? 4 : 1;
     const int force_tpr = env_int("THX_RED_TPR", 0);
@@ -498,7 +517,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     // each) takes a contiguous eighth of the results and fetches those lines once.
     const bool xcd = bigblock && ra2 && S == 1 && !gs && nblocks % 8 == 0 && env_int("THX_RED_XCD", 1);
     std::ostringstream key;
-    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nacc != unr ? "|c" + std::to_string(nacc) : "") << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << (gs ? "|gs" : "") << (xcd ? "|x8" : "") << "|m";
+    key << "rr|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << (nacc != unr ? "|c" + std::to_string(nacc) : "") << "|t" << tpr << "|a" << ra2 << "|s" << skey << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << (gs ? "|gs" : "") << (xcd ? "|x8" : "") << (ua ? "|ua" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -510,7 +529,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"NACC", nacc}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"TICKET", ticket ? 1 : 0}, {"GS", gs ? 1 : 0}, {"XCD", xcd ? 1 : 0}}, mode, nt, sclass)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"NACC", nacc}, {"BLOCK", rblock}, {"TPR", tpr}, {"RA2", ra2}, {"TICKET", ticket ? 1 : 0}, {"GS", gs ? 1 : 0}, {"XCD", xcd ? 1 : 0}, {"UA", ua}}, mode, nt, sclass)
         << "extern \"C\" __global__ __launch_bounds__(" << rblock << ") void " << entry << "(thx::RowParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_row_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -536,10 +555,11 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     pk.put<int64_t>(nblocks);
     pk.put<int64_t>(nvec);
     pk.put<int64_t>(chunk);
+    pk.put<int64_t>(RC);
     pk.put<int32_t>(S);
     pk.put<int32_t>(0);
     for (int d = 0; d < NK; ++d) pk.put<FastDivH>(make_fastdiv(d < NKD ? (uint64_t)KD[d].extent : 1));
-    pk.put<FastDivH>(make_fastdiv((uint64_t)(RC / vec)));
+    pk.put<FastDivH>(make_fastdiv((uint64_t)std::max<int64_t>(1, RC / vec)));
     for (int i = 0; i < NIN; ++i)
       for (int d = 0; d < NK; ++d) pk.put_index(wide, d < NKD ? KD[d].stride[i] : 0);
     for (int i = 0; i < NIN; ++i) pk.put_index(wide, ra_stride[i]);
@@ -566,6 +586,11 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       if (views[i].iota) mode[i] = M_IOTA;
     }
     int vec = vec_width(mode);
+    // Every thread keeps one accumulator per column of its vector: at most 64 bytes of them (int8 sums with their
+    // int64 accumulators, 16384 x 16384: 2.2 TB/s with 8 columns per thread against 1.9 with 16; two long rows:
+    // 0.51 against 0.28; int16 and float16 are indifferent, 4 columns per thread lose a quarter for int16)
+    const int acc_cap = env_int("THX_RED_COL_ACCCAP", 64);
+    while (vec > 1 && vec * r->acc_bytes > acc_cap) vec /= 2;
     auto vec_ok = [&](int v) {
       if (v == 1) return true;
       if (C % v) return false;
@@ -579,10 +604,26 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       }
       return true;
     };
+    const int vec_full = vec;
     while (!vec_ok(vec)) vec /= 2;
+    // Columns that are no whole number of vectors, or rows that start off a vector boundary ((100, 100, 13421)
+    // float16 over the first two axes: 1.0 TB/s with 2-byte accesses): full-width vectors through element-aligned
+    // pointers; the thread that owns the last, incomplete vector reads its columns one by one.
+    int ua = 0;
+    if (vec < vec_full && env_int("THX_RED_UA", 1)) {
+      int v = vec_full;
+      while (v > vec && ((int64_t)cblock * v * r->acc_bytes > 32768 || C < (int64_t)v * std::max(1, env_int("THX_RED_UA_MINVEC", 4)))) v /= 2;
+      bool ok = v > vec;
+      for (int i = 0; i < NIN; ++i)
+        if (mode[i] == M_VEC && ((uintptr_t)views[i].ptr) % (size_t)dtype_size(views[i].dtype)) ok = false;
+      if (ok) {
+        vec = v;
+        ua = 1;
+      }
+    }
     if ((int64_t)cblock * vec * r->acc_bytes > 65536)
       return fail(THX_ERR_UNSUPPORTED, "reduce: accumulator of %d bytes is too large for the column kernel", r->acc_bytes);
-    const int64_t cvecs = C / vec;
+    const int64_t cvecs = ceil_div(C, (int64_t)vec);
     int tx = 1;
     while (tx < 64 && tx < cvecs) tx *= 2;
     // Few column blocks for the device (a split into 4 or more row slices ahead): narrower and taller
@@ -625,7 +666,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
     nblocks = blocks0 * S;
     gs = nblocks * cblock > max_dispatch;
     std::ostringstream key;
-    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << (cblock != 256 ? "|b" + std::to_string(cblock) : "") << "|r" << rr2 << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << (gs ? "|gs" : "") << "|m";
+    key << "rc|k" << NK << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|x" << tx << (cblock != 256 ? "|b" + std::to_string(cblock) : "") << "|r" << rr2 << (nt ? "|nt" + std::to_string(nt) : "") << (ticket ? "|tk" : "") << (gs ? "|gs" : "") << (ua ? "|ua" : "") << "|m";
     for (int i = 0; i < NIN; ++i) key << mode[i] << (i + 1 < NIN ? "," : "");
     plan = key.str() + (fast_div() ? "|fd" : "");
     auto it = r->plans.find(plan);
@@ -637,7 +678,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", cblock}, {"TX", tx}, {"RR2", rr2}, {"TICKET", ticket ? 1 : 0}, {"GS", gs ? 1 : 0}}, mode, nt)
+        << plan_struct(wide, {{"NK", NK}, {"VEC", vec}, {"UNR", unr}, {"BLOCK", cblock}, {"TX", tx}, {"RR2", rr2}, {"TICKET", ticket ? 1 : 0}, {"GS", gs ? 1 : 0}, {"UA", ua}}, mode, nt)
         << "extern \"C\" __global__ __launch_bounds__(" << cblock << ") void " << entry << "(thx::ColParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::IT> p) {\n  thx::red_col_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
@@ -700,7 +741,7 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       const std::string entry = entry_name(r->name, plan);
       std::ostringstream s;
       s << device_prelude() << r->src
-        << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}, {"GS", gs ? 1 : 0}}, gmode, 0)
+        << plan_struct(wide, {{"NK", NK}, {"NR", NR}, {"BLOCK", block}, {"TPR", tpr}, {"GS", gs ? 1 : 0}, {"UA", 0}}, gmode, 0)
         << "extern \"C\" __global__ __launch_bounds__(" << block << ") void " << entry << "(thx::GenParams<" << r->name
         << "::NIN, " << r->name << "::NOUT, " << r->name << "::NEX, ThxPlan::NK, ThxPlan::NR, ThxPlan::IT> p) {\n  thx::red_gen_body<" << r->name
         << ", ThxPlan>(p);\n}\n";
