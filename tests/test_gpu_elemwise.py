@@ -1066,3 +1066,21 @@ def test_operands_that_start_off_a_vector_boundary(dtype):
     got = th.function([m, w], out2)(big, other)
     assert "|ua|" in hip.last_plan(), hip.last_plan()
     assert_parity(got, G.evaluate([m, w], [out2], [big, other])[0], "columns dropped %s [%s]" % (dtype, hip.last_plan()), tol=tol)
+    # rows that are no whole number of vectors, next to a row and a column that broadcast
+    row = T.TensorType(dtype, (True, False))("row")
+    col = T.TensorType(dtype, (False, True))("col")
+    for shape in ((300, 1031), (7, 100003), (513, 129), (64, 33)):       # the last one: rows too short to bother
+        a2, r2, c2 = draw(shape), draw((1, shape[1])), draw((shape[0], 1))
+        out3 = [m * 2 + row, m - col]
+        got = th.function([m, row, col], out3)(a2, r2, c2)
+        if shape[1] >= 16 * (16 // a2.itemsize):
+            assert "|rg|" in hip.last_plan(), hip.last_plan()
+        ref = G.evaluate([m, row, col], out3, [a2, r2, c2])
+        for g_, r_ in zip(got, ref):
+            assert_parity(g_, r_, "ragged rows %s %s [%s]" % (shape, dtype, hip.last_plan()), tol=tol)
+    cube = T.TensorType(dtype, (False, False, False))("cube")
+    plane = T.TensorType(dtype, (False, True, False))("plane")
+    a3, p3 = draw((9, 11, 1001)), draw((9, 1, 1001))
+    out4 = cube + plane
+    got = th.function([cube, plane], out4)(a3, p3)
+    assert_parity(got, G.evaluate([cube, plane], [out4], [a3, p3])[0], "ragged rows of a cube %s [%s]" % (dtype, hip.last_plan()), tol=tol)

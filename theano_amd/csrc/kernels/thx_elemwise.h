@@ -7,7 +7,9 @@
 //   template <int V> static void compute(Regs<V>&);     // the scalar graph, V times
 //   template <int V, class A> static void store(const A&, const Regs<V>&);
 // and a generated plan P supplies
-//   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK, GS (grid-stride loop over chunks) };
+//   typedef int|long long IT;  enum { ND, VEC, UNR, BLOCK, GS (grid-stride loop over chunks),
+//     UA (vectors through element-aligned pointers), RAG (ND > 1: the rows are no whole number of vectors; the
+//     last vector of a row holds fd[ND - 1].pad elements and is handled element by element) };
 //   static constexpr unsigned long long NT;             // bit i: operand i is accessed non-temporally
 //   static constexpr int mode(int operand);             // M_VEC / M_BCAST / M_GATHER
 //   static constexpr int sclass(int operand, int dim);  // stride is 0 / is 1 / anything (2)
@@ -35,6 +37,7 @@ struct EwAcc {
   const unsigned long long* imm;
   const IT (*stride)[P::ND];
   IT off[NOPS];
+  bool last;             // RAG: this is the last vector of its row
 
   template <int I, class T, int N>
   THX_DEV void ld(Vec<T, N>& r) const {
@@ -111,6 +114,7 @@ __device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename 
     } else {
       UT rem = (UT)(full[u] ? q : 0), c;
       divmod(rem, p.fd[ND - 1], rem, c);
+      a[u].last = c + 1 == p.fd[ND - 1].d;
 #pragma unroll
       for (int i = 0; i < NOPS; ++i)
         if (P::alias(i) == i) a[u].off[i] = ew_term<P>(i, ND - 1, (IT)(c * VEC), p.stride[i][ND - 1]);
@@ -127,6 +131,21 @@ __device__ __forceinline__ void ew_body(const EwParams<F::NOPS, P::ND, typename 
 #pragma unroll
       for (int i = 0; i < NOPS; ++i)
         if (P::alias(i) != i) a[u].off[i] = a[u].off[P::alias(i)];
+    }
+    if constexpr (P::RAG != 0 && ND > 1) {
+      const int mine = (int)p.fd[ND - 1].pad;
+      if (full[u] && mine < VEC && a[u].last) {
+        for (int k = 0; k < mine; ++k) {
+          typename F::template Regs<1> r1;
+          EwAcc<P, NOPS> a1 = a[u];
+#pragma unroll
+          for (int i = 0; i < NOPS; ++i) a1.off[i] = a[u].off[i] + ew_term<P>(i, ND - 1, (IT)k, p.stride[i][ND - 1]);
+          F::template load<1>(a1, r1);
+          F::template compute<1>(r1);
+          F::template store<1>(a1, r1);
+        }
+        full[u] = false;
+      }
     }
     if (full[u]) F::template load<VEC>(a[u], r[u]);
   }

@@ -57,11 +57,11 @@ struct CheckFR : CheckF {
   }
 };
 
-struct PlanEw1 { typedef int IT; enum { ND = 1, VEC = 4, UNR = 2, BLOCK = 256, GS = 1, UA = 1 }; static constexpr unsigned long long NT = 1ull;
+struct PlanEw1 { typedef int IT; enum { ND = 1, VEC = 4, UNR = 2, BLOCK = 256, GS = 1, UA = 1, RAG = 0 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {0, 3, 0}; return m[i]; }
   static constexpr int sclass(int i, int d) { constexpr int m[][1] = {{1}, {0}, {1}}; return m[i][d]; }
   static constexpr int alias(int i) { constexpr int m[] = {0, 1, 0}; return m[i]; } };
-struct PlanEw3 { typedef long long IT; enum { ND = 3, VEC = 2, UNR = 1, BLOCK = 256, GS = 0, UA = 0 }; static constexpr unsigned long long NT = 1ull;
+struct PlanEw3 { typedef long long IT; enum { ND = 3, VEC = 2, UNR = 1, BLOCK = 256, GS = 0, UA = 1, RAG = 1 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {2, 1, 0}; return m[i]; }
   static constexpr int sclass(int i, int d) { constexpr int m[][3] = {{2, 2, 2}, {0, 1, 0}, {2, 2, 1}}; return m[i][d]; }
   static constexpr int alias(int i) { constexpr int m[] = {0, 1, 2}; return m[i]; } };

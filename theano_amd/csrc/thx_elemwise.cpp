@@ -246,6 +246,22 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
       ua = 1;
     }
   }
+  // Rows that are no whole number of vectors ((n, 1001) plus a row that broadcasts): the thread that owns the last,
+  // incomplete vector of a row handles its elements one by one; rows of 16 vectors and more.
+  int rag = 0;
+  if (vec < vec_full && ND > 1 && env_int("THX_EW_UA", 1) && env_int("THX_EW_RAGGED", 1)) {
+    bool ok = true;
+    for (int o = 0; o < nops; ++o)
+      if (mode[o] == M_VEC && ((uintptr_t)views[o].ptr) % (size_t)dtype_size(views[o].dtype)) ok = false;
+    int v = vec_full;
+    while (v > vec && inner < (int64_t)v * 16) v /= 2;
+    if (ok && v > vec && inner % v != 0) {
+      vec = v;
+      ua = 1;
+      rag = 1;
+    }
+  }
+  const int64_t row_vecs = ND > 1 ? (inner + vec - 1) / vec : 0;   // vectors in a row, the incomplete one included
 
   // bytes the kernel moves: every operand that is not broadcast along the innermost dimension
   int64_t moved = 0;
@@ -470,7 +486,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
 
   if (red_outs && e->red)   // the caller reduces the stored results next: they stay cacheable
     for (int w : e->red_of) views[e->n_in + w].reused = true;
-  const int64_t nvec = ND == 1 ? n / vec : n / vec;
+  const int64_t nvec = ND == 1 ? n / vec : (n / inner) * row_vecs;
   // One vector per operand and thread: measured with inputs that are not cached, a larger unroll
   // never gains and costs registers (a seven-input float16 kernel needs 164 VGPRs at 4).
   int unr = 1;
@@ -507,7 +523,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
   std::ostringstream key;
   key << "ew|nd" << ND << (wide ? "|i64" : "|i32") << "|v" << vec << "|u" << unr << "|s" << skey;
   if (nt) key << "|nt" << std::hex << nt << std::dec;
-  key << (block != 256 ? "|b" + std::to_string(block) : "") << (gs ? "|gs" : "") << (ua ? "|ua" : "") << "|m";
+  key << (block != 256 ? "|b" + std::to_string(block) : "") << (gs ? "|gs" : "") << (ua ? "|ua" : "") << (rag ? "|rg" : "") << "|m";
   for (int o = 0; o < nops; ++o) key << mode[o] << (o + 1 < nops ? "," : "");
   const std::string plan = key.str() + (fast_div() ? "|fd" : "");
   set_last_plan(e->name + "|" + plan);
@@ -521,7 +537,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
     std::ostringstream s;
     s << device_prelude() << e->src << "\nstruct ThxPlan {\n  typedef " << (wide ? "long long" : "int")
       << " IT;\n  enum { ND = " << ND << ", VEC = " << vec << ", UNR = " << unr << ", BLOCK = " << block
-      << ", GS = " << (gs ? 1 : 0) << ", UA = " << ua << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
+      << ", GS = " << (gs ? 1 : 0) << ", UA = " << ua << ", RAG = " << rag << " };\n  static constexpr unsigned long long NT = " << nt << "ull;\n  static constexpr int mode(int i) {\n    constexpr int m[] = {";
     for (int o = 0; o < nops; ++o) s << mode[o] << (o + 1 < nops ? ", " : "");
     s << "};\n    return m[i];\n  }\n  static constexpr int sclass(int i, int d) {\n    constexpr int m[][" << ND << "] = {";
     for (int o = 0; o < nops; ++o) {
@@ -545,7 +561,11 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
   for (int o = 0; o < nops; ++o) pk.put<uint64_t>(views[o].immval);
   pk.put<int64_t>(nvec);
   pk.put<int64_t>(n);
-  for (int d = 0; d < ND; ++d) pk.put<FastDivH>(make_fastdiv(d == ND - 1 && ND > 1 ? (uint64_t)(inner / vec) : (uint64_t)dm.shape[d]));
+  for (int d = 0; d < ND; ++d) {
+    FastDivH f = make_fastdiv(d == ND - 1 && ND > 1 ? (uint64_t)row_vecs : (uint64_t)dm.shape[d]);
+    if (d == ND - 1 && ND > 1) f.pad = (uint32_t)(inner - (row_vecs - 1) * vec);   // elements in a row's last vector
+    pk.put<FastDivH>(f);
+  }
   for (int o = 0; o < nops; ++o)
     for (int d = 0; d < ND; ++d) pk.put_index(wide, dm.stride[o][d]);
   pk.align(8);
