@@ -368,3 +368,43 @@ def test_elemwise_time_test_script_runs():
     for t in host + device:
         assert 1e-6 < t < 5e-2
     assert device[0] < host[0] and device[1] < host[1]      # no upload / download on the device-resident call
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "float64"])
+def test_row_chains_over_rows_that_are_no_whole_number_of_vectors(dtype):
+    """Softmax over 1001 or 50257 classes: the row chain keeps full-width vectors (plans marked `|ua`), the last one
+    of a row moved back so that it ends with the row; the elements it repeats are left out of the row's sums and
+    maxima.  Rows of small integers make every sum exact, so a repeated or a missed element would show in the last
+    digit; the softmax values are those of the reference's formula (theano/tensor/nnet/nnet.py:440-446)."""
+    rng = np.random.default_rng(17)
+    tol = {"float16": {"rtol": 2e-3, "atol": 2e-3}}.get(dtype)
+    mat = T.TensorType(dtype, (False, False))
+    x, g = mat("x"), mat("g")
+    marked = 0
+    for cols in (1001, 1023, 777, 4097, 50257, 9, 13, 33, 1000, 131):
+        rows = 37 if cols < 5000 else 5
+        xv = rng.integers(-3, 4, (rows, cols)).astype(dtype)
+        gv = rng.integers(-2, 3, (rows, cols)).astype(dtype)
+        sm = T.nnet.softmax(x)
+        outs = [x - T.sum(x, axis=1, keepdims=True), T.max(x * g, axis=1, keepdims=True) + x, sm, th.grad(T.sum(sm * g), x)]
+        f = th.function([x, g], outs)
+        got = f(xv, gv)
+        marked += "|ua" in hip.last_plan()
+        ref = G.evaluate([x, g], outs, [xv, gv])
+        truth = None
+        for k, (a, r) in enumerate(zip(got, ref)):
+            what = "%d columns %s output %d [%s]" % (cols, dtype, k, hip.last_plan())
+            if k < 2 and dtype != "float16":
+                assert np.array_equal(a, r), what
+            elif k < 3:
+                assert_parity(a, r, what, tol=tol)
+            else:
+                if truth is None:
+                    truth = G.evaluate([x, g], outs, [xv, gv], wide=True)
+                assert_within_reference_error(a, r, truth[k], what, tol=tol)
+    assert marked >= 6, marked
+    # rows of a view whose pitch is odd and that starts one element in
+    base = rng.integers(-3, 4, (64, 1031)).astype(dtype)
+    out = T.nnet.softmax(x[:, 1:1025])
+    got = th.function([x], out)(base)
+    assert_parity(got, G.evaluate([x], [out], [base])[0], "softmax of a shifted view %s [%s]" % (dtype, hip.last_plan()), tol=tol)

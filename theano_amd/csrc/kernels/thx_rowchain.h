@@ -21,13 +21,16 @@ struct RowChainParams {
   char* out[NOUT];
   long long rows;
   int cols;                      // row length C
-  int cv;                        // C / VEC
+  int cv;                        // vectors in a row: C / VEC, rounded up when the plan has UA
   IT in_rstride[NIN];            // elements between consecutive rows (0 for per-column operands)
   IT out_rstride[NOUT];
 };
 
-// Plan members: typedef IT; enum { VEC, NCH, TPR, BLOCK }; static constexpr unsigned long long NT, NTO (bit i:
+// Plan members: typedef IT; enum { VEC, NCH, TPR, BLOCK, UA }; static constexpr unsigned long long NT, NTO (bit i:
 // input / output i is accessed non-temporally); static constexpr int imm(int input).
+// UA: rows that do not start on vector boundaries or are no whole number of vectors long (1001 classes): vectors go
+// through element-aligned pointers, and the last vector of a row ends with the row and overlaps the one before it -
+// the elements it repeats are computed and stored twice (same values) and left out of reductions (`counts`).
 template <class C, class P>
 struct RowCtx {
   typedef typename P::IT IT;
@@ -44,6 +47,17 @@ struct RowCtx {
     if (!live) row = 0;
   }
   THX_DEV bool valid(int ch) const { return ch * TPR + lane < p.cv; }
+  // first element of the vector (ch, lane) in its row
+  THX_DEV IT first(int ch) const {
+    const int q = ch * TPR + lane;
+    if (P::UA != 0 && q == p.cv - 1) return (IT)(p.cols - VEC);
+    return (IT)q * VEC;
+  }
+  // does element k of vector ch take part in reductions (it does not when the row's last vector repeats it)
+  THX_DEV bool counts(int ch, int k) const {
+    if (P::UA == 0) return true;
+    return !(ch * TPR + lane == p.cv - 1 && k < p.cv * VEC - p.cols);
+  }
 
   // a full operand: one element per (row, column)
   template <int I, class T, class CT>
@@ -54,7 +68,7 @@ struct RowCtx {
       Vec<T, VEC> r;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) r.v[k] = T();
-      if (valid(ch)) load_vec<T, VEC, ((P::NT >> I) & 1) != 0>(r, base + (IT)(ch * TPR + lane) * VEC);
+      if (valid(ch)) load_vec<T, VEC, ((P::NT >> I) & 1) != 0, P::UA != 0>(r, base + first(ch));
 #pragma unroll
       for (int k = 0; k < VEC; ++k) v[ch][k] = (CT)r.v[k];
     }
@@ -83,7 +97,7 @@ struct RowCtx {
       Vec<T, VEC> r;
 #pragma unroll
       for (int k = 0; k < VEC; ++k) r.v[k] = (T)v[ch][k];
-      if (live && valid(ch)) store_vec<T, VEC, ((P::NTO >> O) & 1) != 0>(base + (IT)(ch * TPR + lane) * VEC, r);
+      if (live && valid(ch)) store_vec<T, VEC, ((P::NTO >> O) & 1) != 0, P::UA != 0>(base + first(ch), r);
     }
   }
   template <int O, class T, class CT>

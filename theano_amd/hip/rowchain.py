@@ -140,8 +140,8 @@ class RowProgram(object):
                     out, act, act, op.c_code(cnode, ["a", "b"], ["a"])))
                 lines.append("%s a%d = %s;" % (act, out, ident))
                 lines.append("_Pragma(\"unroll\") for (int ch = 0; ch < X::NCH; ++ch) { if (x.valid(ch)) {\n"
-                             "_Pragma(\"unroll\") for (int k = 0; k < X::VEC; ++k) { %s t = (%s)v%d[ch][k]; "
-                             "Op%d::comb(a%d, t); } } }" % (act, act, arg, out, out))
+                             "_Pragma(\"unroll\") for (int k = 0; k < X::VEC; ++k) { if (x.counts(ch, k)) { %s t = (%s)v%d[ch][k]; "
+                             "Op%d::comb(a%d, t); } } } }" % (act, act, arg, out, out))
                 lines.append("a%d = x.template allreduce<Op%d, %s>(a%d);" % (out, out, act, out))
                 val = "a%d" % out
                 if out_dt == "bool":
