@@ -625,7 +625,9 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
       return fail(THX_ERR_UNSUPPORTED, "reduce: accumulator of %d bytes is too large for the column kernel", r->acc_bytes);
     const int64_t cvecs = ceil_div(C, (int64_t)vec);
     int tx = 1;
-    while (tx < 64 && tx < cvecs) tx *= 2;
+    // two rows: two row lanes and 128 threads across instead of four lanes of which two idle
+    const int tx_max = rows <= 2 && env_int("THX_RED_WIDE_TX", 1) ? 128 : 64;
+    while (tx < tx_max && tx < cvecs) tx *= 2;
     // Few column blocks for the device (a split into 4 or more row slices ahead): narrower and taller
     // blocks instead - 16 threads across (256-byte row segments for 4-byte elements), 512 threads,
     // 4 rows in flight per thread - leave 2 slices; measured 42.0 us against 47.1 us for the
