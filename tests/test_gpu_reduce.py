@@ -827,3 +827,26 @@ def test_rows_and_columns_that_are_no_whole_number_of_vectors(dtype):
             got = th.function([var], out)(a)
             assert_parity(got, G.evaluate([var], [out], [a])[0], "shifted columns %s %s [%s]" % (shape, dtype, hip.last_plan()), tol=tol)
     assert marked >= (6 if np.dtype(dtype).itemsize < 8 else 4), marked
+
+
+@pytest.mark.parametrize("dtype", ["bool", "int8", "uint8", "int16", "uint16"])
+def test_sums_of_narrow_integers_at_their_extremes(dtype):
+    """Sums of 8- and 16-bit integers have 64-bit accumulators (theano/tensor/elemwise.py:1741-1758); the row form
+    adds the elements of one vector in 32 bits first.  Rows of nothing but the type's largest and smallest values,
+    long enough to overflow 32 bits as a whole: bit for bit."""
+    rng = np.random.default_rng(9)
+    info = None if dtype == "bool" else np.iinfo(dtype)
+    lo, hi = (0, 1) if info is None else (info.min, info.max)
+    x = T.TensorType(dtype, (False, False))("x")
+    for shape in ((3, 70001), (2, 300007), (65, 4096)):
+        for fill in ("hi", "lo", "mixed"):
+            v = (np.full(shape, hi) if fill == "hi" else np.full(shape, lo) if fill == "lo" else
+                 rng.choice([lo, hi], shape)).astype(dtype)
+            outs = [T.sum(x, axis=1), T.sum(x), T.sum(x, axis=0)] + ([T.sum(x * x, axis=1)] if dtype != "bool" else [])
+            got = th.function([x], outs)(v)
+            ref = G.evaluate([x], outs, [v])
+            for k, (a, r) in enumerate(zip(got, ref)):
+                assert a.dtype == r.dtype and np.array_equal(a, r), "%s %s %s output %d [%s]" % (dtype, shape, fill, k, hip.last_plan())
+    big = np.full((1, 40000000), hi).astype(dtype)       # 40 000 000 x 65 535 = 2.6e12
+    got = th.function([x], T.sum(x))(big)
+    assert int(got) == 40000000 * int(hi), (dtype, int(got))

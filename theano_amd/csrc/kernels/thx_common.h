@@ -341,6 +341,44 @@ THX_DEV float half_sum(const Vec<thx_f16, V>& a) {
   return acc;
 }
 
+// The sum of the V 8- or 16-bit integers of a vector, in 32 bits (16 elements cannot overflow them), four or two
+// elements per instruction (v_dot4 / v_dot2 against ones).  Left to itself the compiler widens every element to the
+// 64 bits of the accumulator first: 56 instructions per 16 bytes instead of 6.
+typedef short thx_i16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short thx_u16x2 __attribute__((ext_vector_type(2)));
+
+template <int V, class T>
+THX_DEV int packed_isum(const Vec<T, V>& a) {
+  static_assert((V * sizeof(T)) % 4 == 0 && (sizeof(T) == 1 || sizeof(T) == 2), "whole 32-bit words of narrow integers");
+  constexpr int W = V * (int)sizeof(T) / 4;
+  const unsigned* w = (const unsigned*)&a;
+  if constexpr (T(-1) < T(0)) {
+    int acc = 0;
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      if constexpr (sizeof(T) == 1) {
+        acc = __builtin_amdgcn_sdot4((int)w[k], 0x01010101, acc, false);
+      } else {
+        const thx_i16x2 ones = {1, 1};
+        acc = __builtin_amdgcn_sdot2(*(const thx_i16x2*)&w[k], ones, acc, false);
+      }
+    }
+    return acc;
+  } else {
+    unsigned acc = 0;
+#pragma unroll
+    for (int k = 0; k < W; ++k) {
+      if constexpr (sizeof(T) == 1) {
+        acc = __builtin_amdgcn_udot4(w[k], 0x01010101u, acc, false);
+      } else {
+        const thx_u16x2 ones = {1, 1};
+        acc = __builtin_amdgcn_udot2(*(const thx_u16x2*)&w[k], ones, acc, false);
+      }
+    }
+    return (int)acc;
+  }
+}
+
 // Division by a run-time constant d >= 2 for dividends below 2^31:
 // q = mulhi(n, m) >> s with m = ceil(2^(31+L)/d), s = L-1, L = ceil(log2 d).
 struct FastDiv {

@@ -136,7 +136,7 @@ def _half_products(pre_op, in_dtypes, narrow):
 
     found = {}
     for k, (out, nw) in enumerate(zip(pre_op.outputs, narrow)):
-        if not nw or out.type.dtype != "float32":
+        if nw != "float32" or out.type.dtype != "float32":
             continue
         a = source(out)
         if a is not None:
@@ -159,11 +159,11 @@ def _half_products(pre_op, in_dtypes, narrow):
 
 
 def comb_part_src(scalar_ops, acc_dtypes, narrow):
-    """Statements merging two ``Part`` values: float32 addition in the narrowed fields, the
-    reduction's own op in its accumulator type in the others."""
+    """Statements merging two ``Part`` values: addition in the partial type (``narrow[k]``, a dtype name) in
+    the narrowed fields, the reduction's own op in its accumulator type in the others."""
     out = []
     for k, (op, dt, nw) in enumerate(zip(scalar_ops, acc_dtypes, narrow)):
-        dt = "float32" if nw else dt
+        dt = nw if nw else dt
         cnode = Apply(op, [Scalar(dt)(), Scalar(dt)()], [Scalar(dt)()])
         out.append(op.c_code(cnode, ["a.a%d" % k, "b.a%d" % k], ["a.a%d" % k]))
     return out
@@ -213,11 +213,23 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
         pre_stmt += "\n" + pre_op.c_code(pnode, ins, tmp) + "\n"
         pre_stmt += " ".join("v.a%d = (%s)%s;" % (k, acc_c[k], t) for k, t in enumerate(tmp))
     # float32 partial sums per vector for float64 sums over float16 data (see ``half_data``)
-    narrow = [half_data and isinstance(op, scal.Add) and acc == "float64" and val == "float32"
-              for op, acc, val in zip(scalar_ops, acc_dtypes, value_dtypes)]
+    # ... and 32-bit partial sums per vector for 64-bit sums over 8- and 16-bit integers: the at most 16 elements
+    # of a vector cannot overflow them, and a 64-bit addition per vector replaces one per element
+    def partial_dtype(op, acc, val):
+        if not isinstance(op, scal.Add):
+            return None
+        if half_data and acc == "float64" and val == "float32":
+            return "float32"
+        if acc == "int64" and val in ("bool", "int8", "int16", "uint8", "uint16"):
+            return "int32"
+        if acc == "uint64" and val in ("bool", "uint8", "uint16"):
+            return "uint32"
+        return None
+    narrow = [partial_dtype(op, acc, val) for op, acc, val in zip(scalar_ops, acc_dtypes, value_dtypes)]
     if any(narrow):
+        part_c = {"float32": "thx_f32", "int32": "int", "uint32": "unsigned int"}
         lines[1] += "\n  struct Part { %s };" % " ".join(
-            "%s a%d;" % ("thx_f32" if nw else c, k) for k, (c, nw) in enumerate(zip(acc_c, narrow)))
+            "%s a%d;" % (part_c[nw] if nw else c, k) for k, (c, nw) in enumerate(zip(acc_c, narrow)))
     lines.append("  template <class AccT> THX_DEV static void pre(%s, AccT& v) {\n%s\n  }" % (
         ", ".join("const %s %s" % (compute_ctype(dt), nm) for dt, nm in zip(in_dtypes, ins)),
         _indent(pre_stmt if not any(narrow) else _narrow_stores(pre_stmt, narrow), 4)))
@@ -241,6 +253,10 @@ def reduce_functor(scalar_ops, acc_dtypes, in_dtypes, out_dtypes, pre_op=None, p
                                                      "dot<V>(r.%s, r.%s)" % (ins[a], ins[b]))
                           for k, (a, b) in sorted(dots.items()))
         packed = "    if constexpr (V %% 2 == 0) { %s }\n" % packed if packed else ""
+        if pre_op is None and narrow[0] in ("int32", "uint32"):
+            # the narrow integers themselves are summed: four or two of them per instruction
+            packed = ("    if constexpr ((V * sizeof(%s)) %% 4 == 0) { t.a0 = (decltype(t.a0))thx::packed_isum<V>(r.%s); }\n"
+                      % (storage_ctype(in_dtypes[0]), ins[0]))
         lines.append("  template <int V> THX_DEV static void accum(Acc& s, const Regs<V>& r) {\n"
                      "    Part t; pre(%s, t);\n#pragma unroll\n"
                      "    for (int k = 1; k < V; ++k) { Part u; pre(%s, u); comb_part(t, u); }\n%s"
