@@ -850,3 +850,59 @@ def test_sums_of_narrow_integers_at_their_extremes(dtype):
     big = np.full((1, 40000000), hi).astype(dtype)       # 40 000 000 x 65 535 = 2.6e12
     got = th.function([x], T.sum(x))(big)
     assert int(got) == 40000000 * int(hi), (dtype, int(got))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "int8", "float64", "int32"])
+def test_many_rows_of_a_few_columns(dtype):
+    """(n, C) arrays with C of 2 to 16 reduced over their rows run as one flat walk over the elements (plans `rs`):
+    every element lands in its own column whatever C, the vector width and the length's remainder are; views that
+    start off a vector boundary, two operands, and the cases the form does not take (positions, a strided
+    operand).  Values are those of CAReduce.perform (theano/tensor/elemwise.py:1307), integers and the floats'
+    grid of eighths bit for bit."""
+    from theano_amd.hip import HipArray
+    rng = np.random.default_rng(3)
+    kind = np.dtype(dtype).kind
+    draw = (lambda shape: rng.integers(-100, 100, shape).astype(dtype)) if kind == "i" else \
+           (lambda shape: (rng.integers(-8, 9, shape) / 8.0).astype(dtype))
+    tol = {"float16": {"rtol": 2e-3, "atol": 2e-3}}.get(dtype)
+    mat, cube = T.TensorType(dtype, (False, False)), T.TensorType(dtype, (False, False, False))
+    m, w, c3 = mat("m"), mat("w"), cube("c")
+    strips = 0
+    for cols in (2, 3, 5, 7, 11, 13, 16):
+        for rows in (70001, 300000):
+            a, b = draw((rows, cols)), draw((rows, cols))
+            outs = [T.sum(m, axis=0), T.max(m, axis=0), T.sum(m * w, axis=0), T.min(m + w, axis=0)]
+            ref = G.evaluate([m, w], outs, [a, b])
+            for k, out in enumerate(outs):          # one reduction per kernel ...
+                g = th.function([m, w], out, on_unused_input="ignore")(a, b)
+                strips += "|rs|" in hip.last_plan()
+                assert_parity(g, ref[k], "(%d, %d) %s output %d [%s]" % (rows, cols, dtype, k, hip.last_plan()), tol=tol)
+            if cols <= 5:                           # ... and all four in one, with four accumulators per column
+                got = th.function([m, w], outs)(a, b)
+                for k, (g, r) in enumerate(zip(got, ref)):
+                    assert_parity(g, r, "(%d, %d) %s fused output %d [%s]" % (rows, cols, dtype, k, hip.last_plan()), tol=tol)
+    assert strips >= (40 if np.dtype(dtype).itemsize <= 4 else 24), strips
+    # a view that starts one row and one element in; rows collapsed from two axes
+    base = draw(3 * 100000 + 7)
+    dev = HipArray.from_numpy(base)
+    f = th.function([m], [th.Out(T.sum(m, axis=0), device=True)])
+    for lo in (0, 1, 3, 4):
+        view = dev.view([99990, 3], [3 * base.itemsize, base.itemsize], dev.offset + lo * base.itemsize)
+        got = f(view)[0].to_numpy()
+        ref = G.evaluate([m], [T.sum(m, axis=0)], [base[lo:lo + 3 * 99990].reshape(99990, 3)])[0]
+        assert_parity(got, ref, "view from element %d %s [%s]" % (lo, dtype, hip.last_plan()), tol=tol)
+    vol = draw((300, 301, 3))
+    out = T.sum(c3, axis=(0, 1))
+    got = th.function([c3], out)(vol)
+    assert "|rs|" in hip.last_plan(), hip.last_plan()
+    assert_parity(got, G.evaluate([c3], [out], [vol])[0], "two row axes %s [%s]" % (dtype, hip.last_plan()), tol=tol)
+    # not for these: positions of the maxima, an operand that is a stepped view
+    a = draw((70001, 3))
+    val, pos = th.function([m], T.max_and_argmax(m, axis=0))(a)
+    assert "|rs|" not in hip.last_plan()
+    assert np.array_equal(pos, np.argmax(a, axis=0)) and np.array_equal(val, a.max(axis=0))
+    wide_a = draw((70001, 6))
+    out = T.sum(m[:, ::2], axis=0)
+    got = th.function([m], out)(wide_a)
+    assert "|rs|" not in hip.last_plan()
+    assert_parity(got, G.evaluate([m], [out], [wide_a])[0], "stepped columns %s" % dtype, tol=tol)

@@ -423,6 +423,104 @@ __device__ __forceinline__ void red_col_block(const ColParams<R::NIN, R::NOUT, R
 }
 
 // ---------------------------------------------------------------------------
+// "Strip" form: a C-contiguous (rows, C) array with fewer columns than a few vectors hold, reduced over the rows
+// (per-coordinate sums of n points in 3 dimensions).  The array is walked as the flat run of rows * C elements it
+// is, in whole vectors, consecutive threads on consecutive vectors.  A block takes C * BLOCK vectors at a time: a
+// thread's vector in step u is u * BLOCK vectors after its first, so its element j lies in column
+// (first + u * (BLOCK * VEC mod C) + j) mod C, where `first` - the column of the thread's very first element -
+// is the same in every round of C steps.  With the steps unrolled every accumulator index is a constant (relative
+// to `first`); the rotation by `first` happens once, when the accumulators go to LDS.
+template <int NIN, int NOUT, int NEX>
+struct StripParams {
+  char* in[NIN];
+  unsigned long long imm[NIN];
+  RedOut<NOUT, NEX> out;
+  char* partial;          // Acc[blocks][C] when there is more than one block
+  long long nvec;         // whole vectors in the array
+  long long n;            // elements in the array (rows * C)
+  int blocks;
+  int pad;
+};
+
+// Plan members: typedef IT; enum { VEC, COLS, BLOCK, UA }; mode(int) (M_VEC or M_IMM only).
+template <class R, class P>
+__device__ __forceinline__ void red_strip_body(const StripParams<R::NIN, R::NOUT, R::NEX>& p) {
+  typedef typename P::IT IT;
+  typedef typename R::Acc Acc;
+  constexpr int VEC = P::VEC, C = P::COLS, NIN = R::NIN, BLOCK = P::BLOCK;
+  constexpr int DELTA = (BLOCK * VEC) % C;
+  __shared__ Acc lds[C][BLOCK];
+
+  const int t = threadIdx.x;
+  const int first = (int)(((long long)t * VEC) % C);
+  Acc acc[C];
+#pragma unroll
+  for (int i = 0; i < C; ++i) R::init(acc[i]);
+
+  const IT no_stride[NIN] = {};
+  for (long long q0 = (long long)blockIdx.x * (C * BLOCK); q0 < p.nvec; q0 += (long long)gridDim.x * (C * BLOCK)) {
+    typename R::template Regs<VEC> r[C];
+    bool ok[C];
+#pragma unroll
+    for (int u = 0; u < C; ++u) {
+      const long long q = q0 + (long long)u * BLOCK + t;
+      ok[u] = q < p.nvec;
+      RedAcc<P, NIN> a;
+      a.ptr = p.in;
+      a.imm = p.imm;
+      a.vstride = no_stride;
+#pragma unroll
+      for (int i = 0; i < NIN; ++i) a.off[i] = (IT)(q * VEC);
+      if (ok[u]) R::template load<VEC>(a, r[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < C; ++u) {
+      if (ok[u]) {
+        Acc lane[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) R::init(lane[j]);
+        R::template accum_lanes<VEC>(lane, r[u]);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) R::comb(acc[(u * DELTA + j) % C], lane[j]);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < C; ++i) {
+    int c = first + i;
+    if (c >= C) c -= C;
+    lds[c][t] = acc[i];
+  }
+  __syncthreads();
+  const int wave = t / THX_WAVE, lane_id = t % THX_WAVE;
+  for (int c = wave; c < C; c += BLOCK / THX_WAVE) {
+    Acc tot = lds[c][lane_id];
+#pragma unroll
+    for (int k = 1; k < BLOCK / THX_WAVE; ++k) R::comb(tot, lds[c][lane_id + k * THX_WAVE]);
+    tot = group_reduce<R, THX_WAVE>(tot);
+    if (lane_id == 0) {
+      if (blockIdx.x == 0) {       // the elements after the last whole vector
+        for (long long e = p.nvec * VEC; e < p.n; ++e) {
+          if ((int)(e % C) != c) continue;
+          typename R::template Regs<1> r1;
+          RedAcc<P, NIN> a;
+          a.ptr = p.in;
+          a.imm = p.imm;
+          a.vstride = no_stride;
+#pragma unroll
+          for (int i = 0; i < NIN; ++i) a.off[i] = (IT)e;
+          R::template load<1>(a, r1);
+          R::template accum<1>(tot, r1);
+        }
+      }
+      if (p.blocks == 1) R::post(p.out, c, tot);
+      else ((Acc*)p.partial)[(long long)blockIdx.x * C + c] = tot;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Second pass: merge the S partial Acc values of every output, slice 0 first.
 // TPO threads per output (1, 64 or BLOCK).
 template <int NOUT, int NEX>

@@ -73,6 +73,8 @@ struct PlanRowS { typedef int IT; enum { NK = 1, VEC = 1, UNR = 1, NACC = 1, BLO
   static constexpr int sclass(int i, int w) { constexpr int m[][2] = {{0, 2}}; return m[i][w]; } };
 struct PlanCol { typedef int IT; enum { NK = 1, VEC = 4, UNR = 4, BLOCK = 256, TX = 64, RR2 = 1, TICKET = 0, GS = 1, UA = 1 }; static constexpr unsigned long long NT = 1ull;
   static constexpr int mode(int i) { constexpr int m[] = {0}; return m[i]; } };
+struct PlanStrip { typedef int IT; enum { VEC = 4, COLS = 3, BLOCK = 256, UA = 1 }; static constexpr unsigned long long NT = 1ull;
+  static constexpr int mode(int i) { constexpr int m[] = {0}; return m[i]; } };
 struct PlanGen { typedef int IT; enum { NK = 3, NR = 3, BLOCK = 256, TPR = 64, GS = 1, UA = 0 }; static constexpr unsigned long long NT = 0ull;
   static constexpr int mode(int i) { constexpr int m[] = {2}; return m[i]; } };
 
@@ -89,5 +91,6 @@ extern "C" __global__ __launch_bounds__(256) void check_ew3(thx::EwParams<3, 3, 
 extern "C" __global__ __launch_bounds__(256) void check_row(thx::RowParams<1, 2, 1, 2, int> p) { thx::red_row_body<CheckR, PlanRow>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_rows(thx::RowParams<1, 2, 1, 1, int> p) { thx::red_row_body<CheckR, PlanRowS>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_col(thx::ColParams<1, 2, 1, 1, int> p) { thx::red_col_body<CheckR, PlanCol>(p); }
+extern "C" __global__ __launch_bounds__(256) void check_strip(thx::StripParams<1, 2, 1> p) { thx::red_strip_body<CheckR, PlanStrip>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_gen(thx::GenParams<1, 2, 1, 3, 3, int> p) { thx::red_gen_body<CheckR, PlanGen>(p); }
 extern "C" __global__ __launch_bounds__(256) void check_fin(thx::FinalParams<2, 1> p) { thx::red_final_body<CheckR, 256, 64>(p); }
