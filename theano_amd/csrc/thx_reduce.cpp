@@ -355,9 +355,10 @@ static int reduce_impl(thx_reduce* r, const thx_array* ins, const uint8_t* reduc
   // generic form is, reads such an array at memory speed: neighbouring results lie next to each other.
   if (form == COL && KD.back().extent < 64 && n_red * 4 <= 256 / std::max<int64_t>(1, std::min<int64_t>(64, KD.back().extent)))
     form = GEN;
-  // Two to four rows of columns that cannot be read as vectors (an odd extent, an unaligned view): 1.2 TB/s in the
-  // column form against 2.6 TB/s with one thread per result for a (3, 22369621) float32 sum over axis 0; with
-  // 16-byte accesses the column form is the faster one from four rows on (3.9 against 2.8 TB/s).
+  // Two to four rows of columns that cannot be read as vectors - an odd extent or an unaligned view, and too few
+  // columns for element-aligned vectors: one thread per result (with 4-byte accesses a (3, 22369621) float32 sum over
+  // axis 0 ran at 1.2 TB/s in the column form against 2.6 TB/s; with 16-byte accesses, aligned or not, the column
+  // form is the faster one: 2.9 TB/s for three rows, 3.9 against 2.8 for four).
   if (form == COL && n_red <= 4) {
     bool vectors = KD.back().extent % 2 == 0;
     for (int i = 0; i < NIN && vectors; ++i) {
