@@ -853,3 +853,54 @@ def test_integer_graph_generator_builds(dry_run):
         got = th.function(ins, outs, on_unused_input="ignore")(*vals)
         assert [g.shape for g in got] == [r.shape for r in ref], seed
         assert [g.dtype for g in got] == [r.dtype for r in ref], seed
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "int8", "float16"])
+def test_random_odd_shapes_and_offsets_through_the_vector_paths(dtype):
+    """Reductions over every axis and an elementwise expression on arrays of random, mostly odd extents whose first
+    element lies anywhere in its buffer: the plans with element-aligned vectors, ragged rows, overlapping last
+    vectors and the strip form against the oracle, integers and the floats' grid of eighths bit for bit
+    (CAReduce.perform / Elemwise.perform, theano/tensor/elemwise.py:1307, 790)."""
+    from theano_amd import hip
+    from theano_amd.hip import HipArray
+    rng = np.random.default_rng({"float32": 11, "int8": 12, "float16": 13}[dtype])
+    draw = (lambda n: rng.integers(-100, 100, n).astype(dtype)) if np.dtype(dtype).kind == "i" else \
+           (lambda n: (rng.integers(-8, 9, n) / 8.0).astype(dtype))
+
+    def same(got, ref, what):       # a repeated or a missed element is off by an eighth at least
+        assert_parity(got, ref, what, tol={"rtol": 2e-3, "atol": 2e-3} if dtype == "float16" else None)
+    seen = set()
+    for nd in (1, 2):
+        x = T.TensorType(dtype, (False,) * nd)("x")
+        y = T.TensorType(dtype, (False,) * nd)("y")
+        exprs = [T.sum(x, axis=ax) for ax in [None] + list(range(nd))] + [T.max(x * y, axis=nd - 1), x * 2 + y]
+        if nd == 2:
+            row = T.TensorType(dtype, (True, False))("row")
+            exprs.append(x - row)
+        fs = [th.function([x, y] + ([row] if nd == 2 else []), [th.Out(e, device=True)], on_unused_input="ignore") for e in exprs]
+        for call in range(8):
+            kind = int(rng.integers(3))
+            shape = ((int(rng.integers(1, 400000)),) if nd == 1 else
+                     (int(rng.integers(1, 30)), int(rng.integers(1, 60000))) if kind == 0 else
+                     (int(rng.integers(5000, 90000)), int(rng.integers(2, 18))) if kind == 1 else
+                     (int(rng.integers(1, 900)), int(rng.integers(1, 900))))
+            n = int(np.prod(shape))
+            vals, views = [], []
+            for extent in (shape, shape) + (((1, shape[1]),) if nd == 2 else ()):
+                m = int(np.prod(extent))
+                lo = int(rng.integers(0, 9))
+                host = draw(m + 16)
+                dev = HipArray.from_numpy(host)
+                strides = [host.itemsize * int(np.prod(extent[i + 1:])) for i in range(len(extent))]
+                views.append(dev.view(list(extent), strides, dev.offset + lo * host.itemsize))
+                vals.append(host[lo:lo + m].reshape(extent))
+            ins = [x, y] + ([row] if nd == 2 else [])
+            for e, f in zip(exprs, fs):
+                got = f(*views)[0].to_numpy()
+                plan = hip.last_plan()
+                seen.add(plan.split("|")[1] + ("|ua" if "|ua" in plan else ""))
+                with np.errstate(all="ignore"):
+                    ref = G.evaluate(ins, [e], vals)[0]
+                same(got, ref, "%s %s [%s]" % (dtype, shape, plan))
+    assert {"rr|ua", "rc|ua", "ew|ua", "rs|ua"} <= seen or {"rr|ua", "rc|ua", "ew|ua", "rs"} <= seen, seen
