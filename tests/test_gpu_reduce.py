@@ -896,6 +896,11 @@ def test_many_rows_of_a_few_columns(dtype):
     got = th.function([c3], out)(vol)
     assert "|rs|" in hip.last_plan(), hip.last_plan()
     assert_parity(got, G.evaluate([c3], [out], [vol])[0], "two row axes %s [%s]" % (dtype, hip.last_plan()), tol=tol)
+    if dtype == "int8":          # few enough vectors for one block, which then writes the results itself
+        small = draw((4096, 16))
+        got = th.function([m], T.sum(m, axis=0))(small)
+        assert "|rs|" in hip.last_plan() and not hip.last_plan().split("|")[-1].startswith("s"), hip.last_plan()
+        assert np.array_equal(got, small.sum(axis=0, dtype="int64"))
     # not for these: positions of the maxima, an operand that is a stepped view
     a = draw((70001, 3))
     val, pos = th.function([m], T.max_and_argmax(m, axis=0))(a)
