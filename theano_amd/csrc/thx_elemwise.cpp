@@ -302,6 +302,22 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
       if (force_tile == 32 || force_tile == 64) tile = force_tile;
       // extents of the tile along T (rows read from the permuted inputs) and along the inner dimension
       int tile_t = tile, tile_i = tile;
+      // More operands walk the inner dimension (the results and the inputs that are not permuted) than are
+      // permuted: 512-byte segments for them and 128-byte rows for the permuted reads - x.T * 2 + y on
+      // (8192, 8192) float32 5.6 TB/s against 4.4 with the square tile, (8191, 8193) 4.4 against 2.8 (rows that do
+      // not start on cache lines waste less of a longer segment), float16 4.9 / 3.2 against 4.8 / 2.4.  With the
+      // permuted reads in the majority (two of them and one result: the (64, 128, 56, 56) case) the square tile
+      // ties with every other shape measured.
+      {
+        int along_inner = 0;
+        for (int o = 0; o < nops; ++o)
+          if (!views[o].imm && slot[o] < 0 && mode[o] != M_BCAST) ++along_inner;
+        if (along_inner > ntr && inner >= 256 && !red_outs && env_int("THX_EW_WIDE_TILE", 1) &&
+            (int64_t)ntr * 128 * (32 + 1) * esz <= 60000) {
+          tile_t = 32;
+          tile_i = 128;
+        }
+      }
       {
         const int ft = env_int("THX_EW_TILE_T", 0), fi = env_int("THX_EW_TILE_I", 0);
         auto pow2 = [](int v) { return v >= 8 && v <= 256 && (v & (v - 1)) == 0; };
