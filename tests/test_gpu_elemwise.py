@@ -1084,3 +1084,27 @@ def test_operands_that_start_off_a_vector_boundary(dtype):
     out4 = cube + plane
     got = th.function([cube, plane], out4)(a3, p3)
     assert_parity(got, G.evaluate([cube, plane], [out4], [a3, p3])[0], "ragged rows of a cube %s [%s]" % (dtype, hip.last_plan()), tol=tol)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "float16", "int64"])
+def test_permuted_reads_with_wide_tiles(dtype):
+    """A permuted operand beside operands in the result's layout goes through 32 x 128 tiles when those are the
+    majority, or when odd extents leave single-element accesses (4-byte elements and wider); square tiles otherwise.
+    Extents that are no multiples of either tile side; values as in Elemwise.perform
+    (theano/tensor/elemwise.py:790), integers and the floats' small integers bit for bit."""
+    rng = np.random.default_rng(8)
+    draw = lambda shape: rng.integers(-20, 21, shape).astype(dtype)
+    # the result's rows are 511, 383, 255 and 300 long: the last would leave a quarter of its wide tiles empty
+    cases = [((511, 300), (1, 0)), ((31, 383, 129), (0, 2, 1)), ((127, 255, 33), (2, 0, 1)), ((300, 513), (1, 0))]
+    wide = 0
+    for shape, perm in cases:
+        tt = T.TensorType(dtype, (False,) * len(shape))
+        x, y = tt("x"), tt("y")
+        a, b = draw(shape), draw(tuple(shape[p] for p in perm))
+        for out, ins, vals in ((x.dimshuffle(*perm) * 2 + y, [x, y], [a, b]), (x.dimshuffle(*perm) + y.dimshuffle(*np.argsort(perm)).dimshuffle(*perm) * 3, [x, y], [a, b])):
+            got = th.function(ins, out)(*vals)
+            wide += "|t32x128|" in hip.last_plan()
+            ref = G.evaluate(ins, [out], vals)[0]
+            assert got.dtype == ref.dtype and np.array_equal(got, ref), "%s %s %s [%s]" % (dtype, shape, perm, hip.last_plan())
+    assert wide >= 3, wide

@@ -312,7 +312,7 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
         int along_inner = 0;
         for (int o = 0; o < nops; ++o)
           if (!views[o].imm && slot[o] < 0 && mode[o] != M_BCAST) ++along_inner;
-        if (along_inner > ntr && inner >= 256 && !red_outs && env_int("THX_EW_WIDE_TILE", 1) &&
+        if (along_inner > ntr && (inner + 127) / 128 * 128 * 100 <= inner * 115 && !red_outs && env_int("THX_EW_WIDE_TILE", 1) &&
             (int64_t)ntr * 128 * (32 + 1) * esz <= 60000) {
           tile_t = 32;
           tile_i = 128;
@@ -348,6 +348,20 @@ static int elemwise_impl(thx_elemwise* e, const thx_array* ins, const thx_array*
       };
       while (!tv_ok(tv)) tv /= 2;
       if (env_int("THX_EW_TV", 0) == 1) tv = 1;
+      // Extents or strides that leave single-element accesses, 4-byte elements and wider: the rows of a tile do
+      // not start on cache lines, and a longer segment along the inner dimension wastes less of them - also when the
+      // permuted reads are not in the minority ((255, 513, 511) float32, one permuted read and one result:
+      // 1.7 - 2.2 TB/s with the square tile, 2.9 with 32 x 128; 2-byte elements lose with it)
+      if (tv == 1 && esz >= 4 && tile_t == tile && tile_i == tile && (inner + 127) / 128 * 128 * 100 <= inner * 115 && !red_outs && env_int("THX_EW_WIDE_TILE", 1) &&
+          !env_int("THX_EW_TILE_T", 0) && (int64_t)ntr * 128 * (32 + 1) * esz <= 60000) {
+        int along_inner = 0;
+        for (int o = 0; o < nops; ++o)
+          if (!views[o].imm && slot[o] < 0 && mode[o] != M_BCAST) ++along_inner;
+        if (along_inner >= ntr) {
+          tile_t = 32;
+          tile_i = 128;
+        }
+      }
       if ((int64_t)ntr * tile_i * (tile_t + 1) * esz <= 60000) {
         const int block = 256;
         // the attached reduction rides along when it keeps exactly the innermost dimension of the results
