@@ -162,6 +162,73 @@ def _rate(nbytes, ms):
     return {"us": round(ms * 1e3, 2), "GB/s": round(gbs, 1), "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4)}
 
 
+def _awkward_shapes(th, hip, steps, warmup):
+    """Reductions and elementwise expressions over shapes that are no whole number of vectors, start off a vector
+    boundary, have very few rows or columns, or mix layouts: GB/s of the bytes each must move (inputs once, results
+    once), with the plan the library chose.  Every case is about 256 MB of input."""
+    import numpy as np
+    from theano_amd import tensor as T
+    from theano_amd.hip import HipArray
+    from theano_amd.tensor import nnet
+    N = 64 * 1024 * 1024
+
+    def arr(shape, dtype):
+        return HipArray.from_numpy(np.ones(shape, dtype))
+
+    def var(dtype, nd, name="x"):
+        return T.TensorType(dtype, (False,) * nd)(name)
+    cases = []
+
+    def reduce_case(name, dtype, shape, axis, op="sum"):
+        x = var(dtype, len(shape))
+        out = (T.sum if op == "sum" else T.max)(x, axis=axis)
+        cases.append((name, [x], out, [arr(shape, dtype)]))
+    sz = {"float32": 4, "float16": 2, "int8": 1}
+    reduce_case("sum of 67108863 float32", "float32", (N - 1,), None)
+    reduce_case("sum of 134217727 float16", "float16", (2 * N - 1,), None)
+    reduce_case("sum of 268435455 int8", "int8", (4 * N - 1,), None)
+    reduce_case("sum (22369621, 3) float32 axis 0", "float32", (N // 3, 3), 0)
+    reduce_case("max (22369621, 3) float32 axis 0", "float32", (N // 3, 3), 0, "max")
+    reduce_case("sum (44739242, 3) float16 axis 0", "float16", (2 * N // 3, 3), 0)
+    reduce_case("sum (2164802, 31) float32 axis 0", "float32", (N // 31, 31), 0)
+    reduce_case("sum (100, 100, 13421) float16 axes (0, 1)", "float16", (100, 100, 2 * N // 10000), (0, 1))
+    reduce_case("sum (2, 33554432) float32 axis 0", "float32", (2, N // 2), 0)
+    reduce_case("sum (3, 22369621) float32 axis 0", "float32", (3, N // 3), 0)
+    reduce_case("sum (1048576, 4, 4, 4) float32 axis 1", "float32", (N // 64, 4, 4, 4), 1)
+    reduce_case("sum (1000, 67107) float32 axis 1", "float32", (1000, N // 1000 - 1), 1)
+    for dtype in ("float32", "float16", "int8"):
+        n = 4 * N // sz[dtype]
+        x, y = var(dtype, 1), var(dtype, 1, "y")
+        a, b = arr(n + 8, dtype), arr(n + 8, dtype)
+        cases.append(("x[1:] * 2 + y %s" % dtype, [x, y], x * 2 + y,
+                      [a.view([n], [sz[dtype]], a.offset + sz[dtype]), b.view([n], [sz[dtype]], b.offset)]))
+        rows = n // 1001
+        m, row = var(dtype, 2, "m"), T.TensorType(dtype, (True, False))("row")
+        cases.append(("(%d, 1001) * 2 + row %s" % (rows, dtype), [m, row], m * 2 + row, [arr((rows, 1001), dtype), arr((1, 1001), dtype)]))
+    for shape in ((8192, 8192), (8191, 8193)):
+        x, y = var("float32", 2), var("float32", 2, "y")
+        cases.append(("x.T * 2 + y %s float32" % (shape,), [x, y], x.T * 2 + y, [arr(shape, "float32"), arr(shape[::-1], "float32")]))
+        cases.append(("tanh(x.T) + 1 %s float32" % (shape,), [x], T.tanh(x.T) + 1, [arr(shape, "float32")]))
+    for dtype, cols in (("float32", 1000), ("float32", 1001), ("float32", 4097), ("float16", 1001)):
+        rows = (2 * N // sz[dtype]) // cols
+        x = var(dtype, 2)
+        cases.append(("softmax (%d, %d) %s" % (rows, cols, dtype), [x], nnet.softmax(x), [arr((rows, cols), dtype)]))
+    out = []
+    for name, ins, expr, vals in cases:
+        f = th.function(ins, [th.Out(expr, device=True)])
+        res = f(*vals)[0]
+        nbytes = sum(int(np.prod(v.shape)) * np.dtype(v.dtype).itemsize for v in vals) + int(np.prod(res.shape)) * np.dtype(res.dtype).itemsize
+        plan = hip.last_plan()
+        del res
+        ms, _ = _time_steps(hip, lambda: f(*vals), steps, warmup)
+        parts = plan.split("|")
+        split = parts[-1][:1] == "s" and parts[-1][1:].isdigit()       # "|s<slices>": a second launch merges them
+        out.append(dict(_rate(nbytes, ms), case=name, bytes=nbytes, plan=plan.split("|", 1)[1],
+                        kernel=_symbol("|".join(parts[:-1]) if split else plan)))
+        print("%-52s %8.1f us %7.0f GB/s  %s" % (name, ms * 1e3, out[-1]["GB/s"], out[-1]["plan"]), file=sys.stderr, flush=True)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -176,6 +243,9 @@ def main():
                     help="also launch a plain streaming kernel (out = -x on the same (8192, 8192) float32 array, "
                          "256 MiB read + 256 MiB written) K times: the known-size kernel that hardware counters "
                          "of the reductions are scaled by")
+    ap.add_argument("--awkward-shapes", action="store_true",
+                    help="instead of the benchmark: time reductions and elementwise expressions over shapes of odd "
+                         "length, alignment and layout (one JSON line of its own)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); got --gpus %d" % args.gpus)
@@ -192,6 +262,12 @@ def main():
     hip.init()
     info = hip.device_info()
     SETTLE_MS[0] = max(0.0, args.settle_ms)
+
+    if args.awkward_shapes:
+        print(json.dumps({"metric": "GB/s of algorithmic bytes over awkward shapes at 1 MI355X", "unit": "GB/s",
+                          "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "data": "synthetic",
+                          "cases": _awkward_shapes(th, hip, args.steps, args.warmup)}))
+        return
 
     # ---- headline: config 2 -----------------------------------------------------------------
     # The four reductions of x share one device array and prod has its own, as the configuration

@@ -465,7 +465,10 @@ def _eligible(node, nd, red):
         return (len(op.scalar_ops) == 1 and op.pre_scalar_op is None and op.post_scalar_op is None and
                 len(node.inputs) == 1 and node.inputs[0].type.ndim == nd and
                 _chain_axes(nd, op.axis) == red and
-                _klass(node.inputs[0], nd, red) == FULL and op.acc_dtypes[0] != "float16")
+                _klass(node.inputs[0], nd, red) == FULL and
+                # float16 accumulators: maxima and minima only, which pick one of the values whatever the
+                # arithmetic's width (the row max of a float16 softmax then stays in the chain's one kernel)
+                (op.acc_dtypes[0] != "float16" or isinstance(op.scalar_ops[0], (scal.Maximum, scal.Minimum))))
     if isinstance(op, HipDimShuffle):
         x = node.inputs[0]
         kept = iter(range(nd - len(red)))
