@@ -1338,3 +1338,23 @@ def test_shared_takes_the_references_arguments(dry_run):
     assert d.get_value().dtype == np.float32
     with pytest.raises(TypeError):
         th.shared(np.zeros(3), colour="red")
+
+
+def test_float16_softmax_and_its_gradient_are_one_row_chain(dry_run):
+    """The row maximum of a float16 softmax has a float16 accumulator; it joins the row chain like the float32 one
+    (a maximum picks one of the values whatever the arithmetic's width), so forward and gradient are one kernel and
+    x is read once.  Sums keep their float32 accumulators (theano/tensor/elemwise.py:1395-1398)."""
+    import numpy as np
+    import theano_amd as th
+    from theano_amd import tensor as T
+    from theano_amd.hip import HipRowChain, HipCAReduce
+    for dtype in ("float16", "float32"):
+        x = T.TensorType(dtype, (False, False))("x")
+        g = T.TensorType(dtype, (False, False))("g")
+        sm = T.nnet.softmax(x)
+        for outs in ([sm], [sm, th.grad(T.sum(sm * g), x)], [x - T.max(x, axis=1, keepdims=True)]):
+            f = th.function([x, g], outs, on_unused_input="ignore")
+            ops = [n.op for n in f.toposort()]
+            assert sum(isinstance(o, HipRowChain) for o in ops) == 1, (dtype, ops)
+            assert not any(isinstance(o, HipCAReduce) for o in ops), (dtype, ops)
+            f(np.ones((8, 1001), dtype), np.ones((8, 1001), dtype))
