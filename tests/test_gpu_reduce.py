@@ -911,3 +911,27 @@ def test_many_rows_of_a_few_columns(dtype):
     got = th.function([m], out)(wide_a)
     assert "|rs|" not in hip.last_plan()
     assert_parity(got, G.evaluate([m], [out], [wide_a])[0], "stepped columns %s" % dtype, tol=tol)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "int8"])
+def test_reductions_over_axes_of_extent_one(dtype):
+    """An axis of extent 1 that is not declared broadcastable: the "reduction" copies every element through the
+    accumulator's type and the epilogue (theano/tensor/elemwise.py:1307); long rows of such results are read and
+    written as vectors (the column form with one row)."""
+    rng = np.random.default_rng(4)
+    draw = (lambda shape: rng.integers(-100, 100, shape).astype(dtype)) if np.dtype(dtype).kind == "i" else \
+           (lambda shape: (rng.integers(-8, 9, shape) / 8.0).astype(dtype))
+    for shape, axis in (((1, 300001), 0), ((300001, 1), 1), ((1, 37, 4099), 0), ((5, 1, 70000), (1,)), ((1, 1, 2048), (0, 1)), ((1, 100), 0)):
+        x = T.TensorType(dtype, (False,) * len(shape))("x")
+        v = draw(shape)
+        for name in ("sum", "max"):
+            out = REDUCERS[name](x, axis)
+            got = th.function([x], out)(v)
+            if v.size >= 65536:
+                assert "|rc|" in hip.last_plan(), hip.last_plan()
+            ref = G.evaluate([x], [out], [v])[0]
+            assert got.dtype == ref.dtype and np.array_equal(got, ref), "%s %s %s %s [%s]" % (name, dtype, shape, axis, hip.last_plan())
+    x = T.TensorType(dtype, (False, False))("x")
+    v = draw((1, 100000))
+    val, pos = th.function([x], T.max_and_argmax(x, axis=0))(v)
+    assert np.array_equal(val, v[0]) and not pos.any()
