@@ -37,6 +37,9 @@ REDUCTIONS = [
     ("float64", (2581110, 13), 0, ["|rc|"]),
     # few columns and few rows: one thread per result
     ("float32", (1048576, 4, 4, 4), 1, ["|rg|", "|t1|"]),
+    # nothing to reduce (the reduced extent is 1): one row of the column form, in vectors
+    ("float32", (1, 67108864), 0, ["|rc|", "|v4|", "|x256|"]),
+    ("float16", (300001, 1), 1, ["|rc|", "|v8|", "|ua|"]),
     # at most 64 bytes of column accumulators per thread
     ("int8", (16384, 16384), 0, ["|rc|", "|v8|"]),
 ]
